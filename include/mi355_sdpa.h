@@ -1,0 +1,190 @@
+/*
+ * mi355_sdpa.h - C ABI of the MI355X (gfx950) fused scaled-dot-product-attention library.
+ *
+ * Every entry point is extern "C", takes plain pointers / sizes / POD structs, never
+ * allocates device memory, never synchronises, launches on the stream it is given
+ * (a hipStream_t passed as void*; NULL = the default stream) and reports failure with a
+ * negative return code plus a thread-local message (mi355_sdpa_last_error).  No C++
+ * exception crosses this boundary.
+ *
+ * Each declaration names the piece of aws-neuron/torch-neuronx it stands in for
+ * (paths relative to that tree).
+ *
+ * Tensor convention: 4-D (batch, heads, sequence, head_dim), sizes and strides in
+ * ELEMENTS.  The fast kernels need unit stride on the last dimension; everything else is
+ * free (the usual (B,S,H,D).transpose(1,2) views are consumed in place).
+ */
+#ifndef MI355_SDPA_H
+#define MI355_SDPA_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355_SDPA_ABI_VERSION 1
+
+/* element types */
+enum mi355_sdpa_dtype {
+  MI355_SDPA_F32 = 0,
+  MI355_SDPA_F16 = 1,
+  MI355_SDPA_BF16 = 2,
+  MI355_SDPA_F64 = 3,       /* descriptors only: validated, then computed as f32 by the host */
+  MI355_SDPA_BOOL = 4,      /* attention mask only: 1 byte, non-zero = attend               */
+  MI355_SDPA_FP8_E4M3 = 5,  /* OCP e4m3fn, decode K/V cache only                            */
+  MI355_SDPA_OTHER = 99
+};
+
+/* return codes */
+enum mi355_sdpa_status {
+  MI355_SDPA_OK = 0,
+  MI355_SDPA_ERR_INVALID = -1,     /* argument breaks the operator contract        */
+  MI355_SDPA_ERR_UNSUPPORTED = -2, /* valid, but no kernel in this library takes it */
+  MI355_SDPA_ERR_LAUNCH = -3       /* HIP reported an error at launch               */
+};
+
+/* backend ids: numerically equal to at::SDPBackend */
+enum mi355_sdpa_backend { MI355_SDPA_BACKEND_MATH = 0, MI355_SDPA_BACKEND_OVERRIDEABLE = 4 };
+
+/* which kernel family a call is served by */
+enum mi355_sdpa_kernel {
+  MI355_SDPA_KERNEL_NONE = 0,
+  MI355_SDPA_KERNEL_GENERIC = 1, /* fp32-accumulate kernel: any head dim, bias, masks, dropout */
+  MI355_SDPA_KERNEL_MFMA = 2     /* bf16/f16 MFMA flash kernel: head dim 64 or 128            */
+};
+
+typedef struct mi355_sdpa_tensor {
+  void* data; /* device pointer; NULL = absent */
+  int64_t size[4];
+  int64_t stride[4];
+} mi355_sdpa_tensor;
+
+/* Shape/dtype description used by the host-logic entry points (no device pointers read). */
+typedef struct mi355_sdpa_desc {
+  int32_t q_dim, k_dim, v_dim;       /* tensor ranks                                  */
+  int64_t q_size[4], k_size[4], v_size[4];
+  int32_t q_dtype, k_dtype, v_dtype; /* enum mi355_sdpa_dtype                         */
+  int32_t on_device;                 /* 1 if all three live on the GPU                */
+  int32_t has_symbolic_shape;        /* 1 if any size is symbolic (tracing)           */
+  int32_t has_attn_bias;             /* a mask / bias tensor is present               */
+  int32_t is_causal;
+  int32_t return_debug_mask;
+  int32_t has_scale;                 /* 0: scale = 1/sqrt(E)                          */
+  float scale;
+  float dropout_p;
+  int32_t requires_lse;
+  int32_t q_last_stride, k_last_stride, v_last_stride; /* stride of head_dim           */
+} mi355_sdpa_desc;
+
+typedef struct mi355_sdpa_fwd_params {
+  mi355_sdpa_tensor q;    /* (B,Hq,L,E)                                               */
+  mi355_sdpa_tensor k;    /* (B,Hkv,S,E)   Hq % Hkv == 0; query head h reads h/(Hq/Hkv) */
+  mi355_sdpa_tensor v;    /* (B,Hkv,S,Dv)                                             */
+  mi355_sdpa_tensor out;  /* (B,Hq,L,Dv)   same dtype as q                            */
+  float* lse;             /* (B,Hq,L) contiguous float32, natural log; may be NULL    */
+  mi355_sdpa_tensor bias; /* optional additive bias or bool keep-mask, sizes (B,Hq,L,S),
+                             stride 0 on broadcast dims                               */
+  int32_t bias_dtype;     /* F32/F16/BF16/BOOL                                        */
+  const int32_t* kv_lens; /* optional (B,): key j of batch b takes part iff j<kv_lens[b] */
+  const uint8_t* dropout_keep; /* optional (B,Hq,L,S) contiguous, 1 = keep            */
+  float dropout_p;
+  int32_t dtype;          /* dtype of q/k/v/out                                       */
+  int32_t is_causal;      /* lower-triangular, anchored top-left (also when L != S)   */
+  float scale;            /* multiplies Q K^T in float32                              */
+  int32_t force_kernel;   /* 0 = library picks; else enum mi355_sdpa_kernel           */
+} mi355_sdpa_fwd_params;
+
+typedef struct mi355_sdpa_bwd_params {
+  mi355_sdpa_tensor grad_out; /* (B,Hq,L,Dv) */
+  mi355_sdpa_tensor q, k, v, out;
+  const float* lse;           /* (B,Hq,L) contiguous float32                          */
+  mi355_sdpa_tensor grad_q;   /* (B,Hq,L,E)                                           */
+  mi355_sdpa_tensor grad_k;   /* (B,Hkv,S,E)   summed over each query-head group      */
+  mi355_sdpa_tensor grad_v;   /* (B,Hkv,S,Dv)                                         */
+  mi355_sdpa_tensor bias;     /* as in forward                                        */
+  int32_t bias_dtype;
+  mi355_sdpa_tensor grad_bias; /* optional (B,Hq,L,S), dtype of q                     */
+  const int32_t* kv_lens;
+  const uint8_t* dropout_keep;
+  float dropout_p;
+  int32_t dtype;
+  int32_t is_causal;
+  float scale;
+  void* workspace;            /* mi355_sdpa_bwd_workspace_bytes() bytes, 256-aligned  */
+  size_t workspace_bytes;
+  int32_t force_kernel;
+} mi355_sdpa_bwd_params;
+
+typedef struct mi355_sdpa_decode_params {
+  mi355_sdpa_tensor q;      /* (B,Hq,Lq,D) bf16/f16/f32, Lq*Hq/Hkv <= 16               */
+  mi355_sdpa_tensor k;      /* (B,Hkv,S,D)  fp8 e4m3fn, 1 byte per element             */
+  mi355_sdpa_tensor v;      /* (B,Hkv,S,D)  fp8 e4m3fn                                 */
+  const float* k_scale;     /* (B,Hkv) contiguous: real K = fp8 value * k_scale        */
+  const float* v_scale;     /* (B,Hkv)                                                 */
+  const int32_t* kv_lens;   /* (B,) or NULL (= S everywhere)                           */
+  mi355_sdpa_tensor out;    /* (B,Hq,Lq,D) dtype of q                                  */
+  float* lse;               /* (B,Hq,Lq) float32 or NULL                               */
+  int32_t q_dtype;
+  float scale;
+  int32_t num_splits;       /* 0 = library picks                                       */
+  void* workspace;          /* mi355_sdpa_decode_workspace_bytes() bytes               */
+  size_t workspace_bytes;
+} mi355_sdpa_decode_params;
+
+/* ---- kernels -------------------------------------------------------------------------- */
+
+/* Fused forward: O = softmax(scale*Q K^T + causal + bias) V and LSE.
+ * Stands in for the device kernel launched at
+ *   torch_neuronx/neuron_dynamo_backend/decompositions.py:2233-2262 (_compute_attention_nki)
+ * and, for inputs the flash kernel refuses, for the math path
+ *   torch_neuronx/_sdpa_math.py:51-95 (compute_attention). */
+int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream);
+
+/* Fused backward: dQ, dK, dV (dK/dV already reduced over each GQA group), optional dBias.
+ * Stands in for decompositions.py:2467-2477 (_compute_attention_backward_nki),
+ * _sdpa_math.py:98-176 (compute_attention_backward) and decompositions.py:2569-2599
+ * (_reduce_gqa_gradients). */
+int mi355_sdpa_bwd(const mi355_sdpa_bwd_params* p, void* stream);
+size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p);
+
+/* Decode-step attention over an fp8 e4m3 K/V cache with per-sequence lengths.
+ * No counterpart in the reference (it has no fp8 attention path); defined as
+ * compute_attention (_sdpa_math.py:51-95) on the dequantised cache with a key-padding bias. */
+int mi355_sdpa_decode_fp8kv(const mi355_sdpa_decode_params* p, void* stream);
+size_t mi355_sdpa_decode_workspace_bytes(const mi355_sdpa_decode_params* p);
+
+/* ---- host logic (no GPU needed) --------------------------------------------------------- */
+
+/* Backend choice for F.scaled_dot_product_attention.  Rules of
+ *   torch_neuronx/csrc/aten/SdpBackendSelection.cpp:14-68 (_fused_sdp_choice_neuron):
+ * overrideable (4) for on-device, 4-D, concrete, non-empty q/k/v; otherwise math (0). */
+int mi355_sdpa_choose_backend(const mi355_sdpa_desc* d);
+
+/* Operator-boundary validation with the reference's messages.  Follows
+ *   torch_neuronx/csrc/core/dispatch/NeuronDispatcher.cpp:2377-2459 (DispatchSdpaFwdImpl).
+ * Returns 0 or MI355_SDPA_ERR_INVALID and writes the message (NUL-terminated) to msg. */
+int mi355_sdpa_validate(const mi355_sdpa_desc* d, char* msg, size_t msg_len);
+
+/* Strides of an output that keeps the dimension order of a reference tensor: the rule of
+ * at::native::alloc_with_matching_layout used at NeuronDispatcher.cpp:2485-2491 and
+ * :2554-2558 (dims sorted by descending stride of ref, dense strides for out_sizes). */
+int mi355_sdpa_out_strides(const int64_t ref_sizes[4], const int64_t ref_strides[4],
+                           const int64_t out_sizes[4], int64_t out_strides[4]);
+
+/* Kernel eligibility: which kernel family serves a forward / backward call.  The analogue
+ * of decompositions.py:2161-2207 (_can_use_nki_flash_attention) and :2371-2424
+ * (_can_use_nki_flash_attention_backward) for this library's own kernels.
+ * Returns an enum mi355_sdpa_kernel. */
+int mi355_sdpa_can_use_fused_fwd(const mi355_sdpa_desc* d);
+int mi355_sdpa_can_use_fused_bwd(const mi355_sdpa_desc* d);
+
+/* Message of the last failing call on this thread ("" if none). */
+const char* mi355_sdpa_last_error(void);
+int mi355_sdpa_abi_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MI355_SDPA_H */

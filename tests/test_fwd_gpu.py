@@ -1,0 +1,197 @@
+"""GPU parity of the forward kernels against the CPU oracle, through the C ABI."""
+
+import math
+
+import pytest
+import torch
+
+from helpers import max_abs, oracle_fwd, qkv, tol_for
+
+pytestmark = pytest.mark.gpu
+
+GENERIC, MFMA = 1, 2
+
+
+@pytest.fixture(scope="module")
+def amd(gpu_device):
+    import torch_neuronx_amd as amd
+
+    return amd
+
+
+def _run(amd, q, k, v, dev, **kw):
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), **kw)
+    torch.cuda.synchronize()
+    return out, lse
+
+
+def test_config1_fp32_noncausal_mha(amd, gpu_device):
+    # BASELINE config 1: B=2,H=4,S=128,D=64 fp32, scale 1/8, max-abs <= 1e-5
+    q, k, v = qkv(2, 4, 4, 128, 128, 64, dtype=torch.float32, seed=1001)
+    out, lse = _run(amd, q, k, v, gpu_device, scale=0.125)
+    ro, rl = oracle_fwd(q, k, v, scale=0.125)
+    assert max_abs(out, ro) <= 1e-5
+    assert max_abs(lse, rl) <= 1e-5
+    assert out.dtype == torch.float32 and lse.dtype == torch.float32 and lse.shape == (2, 4, 128)
+
+
+def test_config2_bf16_causal_mha(amd, gpu_device):
+    # BASELINE config 2: B=4,H=12,S=1024,D=64 bf16 causal; output within 2e-2 of the fp32 oracle
+    q, k, v = qkv(4, 12, 12, 1024, 1024, 64, dtype=torch.bfloat16, seed=1002)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=True, scale=0.125, force_kernel=MFMA)
+    ro, rl = oracle_fwd(q, k, v, is_causal=True, scale=0.125)
+    assert out.dtype == torch.bfloat16
+    assert max_abs(out, ro) <= 2e-2
+    assert max_abs(lse, rl) <= 1e-3
+
+
+def test_config3_llama8b_shape_head_subset(amd, gpu_device):
+    # BASELINE config 3 at full size on the GPU; the oracle checks a subset of heads
+    # (first/last of a group, first/last kv head) to stay within seconds on the CPU.
+    q, k, v = qkv(1, 32, 8, 8192, 8192, 128, dtype=torch.bfloat16, seed=1003)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=True, force_kernel=MFMA)
+    assert lse.shape == (1, 32, 8192) and lse.dtype == torch.float32
+    for h in (0, 3, 13, 31):
+        hk = h // 4
+        ro, rl = oracle_fwd(q[:, h : h + 1], k[:, hk : hk + 1], v[:, hk : hk + 1], is_causal=True)
+        assert max_abs(out[:, h : h + 1], ro) <= 2e-2, f"head {h}"
+        assert max_abs(lse[:, h : h + 1], rl) <= 2e-3, f"head {h}"
+    # size-independent property: under a causal mask row 0 attends to key 0 only
+    torch.testing.assert_close(out[0, :, 0].float().cpu(), v[0].repeat_interleave(4, 0)[:, 0].float(), rtol=0, atol=0)
+    s00 = (q[0, :, 0].float() * k[0].repeat_interleave(4, 0)[:, 0].float()).sum(-1) / math.sqrt(128)
+    assert max_abs(lse[0, :, 0], s00) <= 1e-4
+
+
+SHAPES = [
+    # B, Hq, Hkv, L, S, E, causal   (reference parity matrix + edge cases)
+    (1, 8, 8, 512, 512, 64, False),
+    (1, 24, 6, 512, 512, 64, False),
+    (1, 8, 1, 512, 512, 64, False),
+    (1, 4, 2, 512, 512, 64, True),
+    (1, 2, 1, 577, 577, 64, False),
+    (1, 2, 1, 577, 577, 64, True),
+    (2, 4, 4, 51, 51, 64, True),
+    (2, 4, 2, 13, 51, 128, True),
+    (2, 4, 2, 51, 13, 128, True),
+    (1, 4, 4, 128, 1024, 128, False),
+    (1, 4, 1, 200, 333, 128, True),
+    (2, 8, 2, 1, 257, 128, False),
+    (1, 8, 8, 2048, 2048, 128, True),
+]
+
+
+@pytest.mark.parametrize("shape", SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_forward_matrix(amd, gpu_device, shape, dtype):
+    B, Hq, Hkv, L, S, E, causal = shape
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 7 + S)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=causal, force_kernel=MFMA)
+    ro, rl = oracle_fwd(q, k, v, is_causal=causal)
+    assert max_abs(out, ro) <= 2e-2
+    assert max_abs(lse, rl) <= 2e-3
+
+
+GENERIC_SHAPES = SHAPES[:9] + [
+    (1, 4, 4, 256, 256, 256, False),
+    (1, 4, 2, 512, 512, 256, True),
+    (2, 8, 1, 12, 12, 16, False),
+    (2, 8, 2, 10, 10, 16, True),
+    (1, 4, 4, 6, 6, 12, False),
+    (1, 2, 2, 6, 10, 40, False),
+]
+
+
+@pytest.mark.parametrize("shape", GENERIC_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16, torch.float16])
+def test_generic_forward_matrix(amd, gpu_device, shape, dtype):
+    B, Hq, Hkv, L, S, E, causal = shape
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 5 + S)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=causal, force_kernel=GENERIC)
+    ro, rl = oracle_fwd(q, k, v, is_causal=causal)
+    assert max_abs(out, ro) <= tol_for(dtype)
+    assert max_abs(lse, rl) <= (2e-5 if dtype is torch.float32 else 2e-3)
+
+
+def test_asymmetric_head_dims_generic(amd, gpu_device):
+    # reference: D_qk=192, D_v=128 (MLA-style)
+    q, k, v = qkv(1, 4, 2, 96, 96, 192, Dv=128, dtype=torch.float32, seed=5)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=True)
+    ro, rl = oracle_fwd(q, k, v, is_causal=True)
+    assert out.shape == (1, 4, 96, 128)
+    assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
+
+
+@pytest.mark.parametrize("mask_kind", ["float", "bool", "bool_bcast", "float_bcast"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_masks_and_bias(amd, gpu_device, mask_kind, dtype):
+    B, H, L, S, E = 2, 4, 51, 77, 48
+    q, k, v = qkv(B, H, H, L, S, E, dtype=dtype, seed=77)
+    g = torch.Generator().manual_seed(3)
+    if mask_kind == "float":
+        mask = torch.randn(B, H, L, S, generator=g).to(dtype)
+    elif mask_kind == "float_bcast":
+        mask = torch.randn(1, 1, L, S, generator=g).to(dtype)
+    elif mask_kind == "bool":
+        mask = torch.rand(B, H, L, S, generator=g) > 0.3
+    else:
+        mask = (torch.rand(B, 1, 1, S, generator=g) > 0.3)
+    out, lse = _run(amd, q, k, v, gpu_device, attn_bias=mask.to(gpu_device))
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask if mask.dtype == torch.bool else mask.float())
+    assert max_abs(out, ro) <= tol_for(dtype)
+    assert max_abs(lse, rl) <= (2e-5 if dtype is torch.float32 else 2e-3)
+
+
+def test_fully_masked_rows_give_zero_and_minus_inf(amd, gpu_device):
+    # reference: tests/python_ops/test_scaled_dot_product_attention.py:1003-1064
+    q, k, v = qkv(1, 4, 4, 32, 32, 32, dtype=torch.float32, seed=9)
+    mask = torch.ones(1, 1, 32, 32, dtype=torch.bool)
+    mask[:, :, :10, :] = False
+    out, lse = _run(amd, q, k, v, gpu_device, attn_bias=mask.to(gpu_device))
+    assert torch.equal(out[:, :, :10].cpu(), torch.zeros(1, 4, 10, 32))
+    assert torch.isinf(lse[:, :, :10]).all() and (lse[:, :, :10] < 0).all()
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
+    assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
+
+
+def test_kv_lens_equals_key_padding_mask(amd, gpu_device):
+    q, k, v = qkv(3, 4, 2, 5, 64, 32, dtype=torch.float32, seed=4)
+    lens = torch.tensor([64, 1, 17], dtype=torch.int32)
+    out, lse = _run(amd, q, k, v, gpu_device, kv_lens=lens.to(gpu_device))
+    pad = (torch.arange(64)[None, :] < lens[:, None])[:, None, None, :]
+    ro, rl = oracle_fwd(q, k, v, attn_mask=pad)
+    assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
+
+
+def test_scale_zero_and_explicit_scale(amd, gpu_device):
+    q, k, v = qkv(1, 2, 2, 40, 40, 64, dtype=torch.bfloat16, seed=8)
+    for sc in (0.0, 0.25, 0.5):
+        out, lse = _run(amd, q, k, v, gpu_device, scale=sc)
+        ro, rl = oracle_fwd(q, k, v, scale=sc)
+        assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 2e-3
+
+
+@pytest.mark.parametrize("kernel", [GENERIC, MFMA])
+def test_noncontiguous_inputs_keep_query_layout(amd, gpu_device, kernel):
+    # reference: test_scaled_dot_product_attention.py:943-1000 - (B,L,H,D).transpose(1,2) views,
+    # last-dim chunks of a fused QKV buffer, as_strided with gaps
+    B, H, L, E = 2, 4, 130, 64
+    g = torch.Generator().manual_seed(21)
+    base = torch.randn(B, L, H, 3 * E, generator=g).to(torch.bfloat16).to(gpu_device)
+    q, k, v = (t.transpose(1, 2) for t in base.chunk(3, dim=-1))
+    assert not q.is_contiguous()
+    out, lse = amd.sdpa_forward(q, k, v, is_causal=True, force_kernel=kernel)
+    ro, rl = oracle_fwd(q.cpu(), k.cpu(), v.cpu(), is_causal=True)
+    assert max_abs(out, ro) <= 2e-2
+    expect = torch.empty(B, L, H, E).transpose(1, 2).stride()
+    assert out.stride() == expect
+    assert lse.is_contiguous()
+
+
+def test_expanded_kv_stride0(amd, gpu_device):
+    # reference: test_scaled_dot_product_attention.py:1123-1221 (repeat_kv style expand)
+    q, k, v = qkv(1, 8, 1, 512, 512, 64, dtype=torch.bfloat16, seed=12)
+    ke = k.to(gpu_device).expand(1, 8, 512, 64)
+    ve = v.to(gpu_device).expand(1, 8, 512, 64)
+    out, lse = amd.sdpa_forward(q.to(gpu_device), ke, ve, is_causal=True)
+    ro, rl = oracle_fwd(q, k, v, is_causal=True)
+    assert max_abs(out, ro) <= 2e-2

@@ -1,0 +1,269 @@
+// C ABI of the library: argument checking, kernel selection and the host-side rules of the
+// operator boundary (backend choice, validation messages, output layout).  See
+// include/mi355_sdpa.h for the contract of every entry point.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <algorithm>
+
+#include "common.h"
+
+namespace mi355 {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+int check_launch(const char* what) {
+  hipError_t e = hipGetLastError();
+  if (e != hipSuccess) {
+    set_error("SDPA: launch of %s failed: %s", what, hipGetErrorString(e));
+    return MI355_SDPA_ERR_LAUNCH;
+  }
+  return MI355_SDPA_OK;
+}
+
+static const char* dtype_name(int dt) {
+  switch (dt) {
+    case MI355_SDPA_F32: return "Float";
+    case MI355_SDPA_F16: return "Half";
+    case MI355_SDPA_BF16: return "BFloat16";
+    case MI355_SDPA_F64: return "Double";
+    case MI355_SDPA_BOOL: return "Bool";
+    case MI355_SDPA_FP8_E4M3: return "Float8_e4m3fn";
+  }
+  return "Other";
+}
+
+static int fail(char* msg, size_t n, const char* fmt, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  set_error("%s", buf);
+  if (msg && n) {
+    strncpy(msg, buf, n - 1);
+    msg[n - 1] = 0;
+  }
+  return MI355_SDPA_ERR_INVALID;
+}
+
+static bool tensor_ok(const mi355_sdpa_tensor& t, const char* name) {
+  if (!t.data) {
+    set_error("SDPA: %s is a null pointer", name);
+    return false;
+  }
+  for (int i = 0; i < 4; ++i)
+    if (t.size[i] < 0) {
+      set_error("SDPA: %s has a negative size", name);
+      return false;
+    }
+  return true;
+}
+
+static bool shapes_ok(const mi355_sdpa_tensor& q, const mi355_sdpa_tensor& k,
+                      const mi355_sdpa_tensor& v) {
+  if (q.size[0] != k.size[0] || q.size[0] != v.size[0]) return set_error("SDPA: batch sizes must match"), false;
+  if (k.size[1] != v.size[1]) return set_error("SDPA: key and value must have the same number of heads"), false;
+  if (k.size[2] != v.size[2]) return set_error("SDPA: key and value must have the same sequence length"), false;
+  if (k.size[1] == 0 || q.size[1] % k.size[1] != 0)
+    return set_error("SDPA: Number of heads in key and value must divide the number of heads in query"), false;
+  if (q.size[3] != k.size[3]) return set_error("SDPA: query and key must have the same head dim"), false;
+  return true;
+}
+
+static bool same_shape(const mi355_sdpa_tensor& t, int64_t a, int64_t b, int64_t c, int64_t d) {
+  return t.size[0] == a && t.size[1] == b && t.size[2] == c && t.size[3] == d;
+}
+
+}  // namespace mi355
+
+using namespace mi355;
+
+extern "C" {
+
+int mi355_sdpa_abi_version(void) { return MI355_SDPA_ABI_VERSION; }
+const char* mi355_sdpa_last_error(void) { return g_err; }
+
+int mi355_sdpa_choose_backend(const mi355_sdpa_desc* d) {
+  if (!d || !d->on_device) return MI355_SDPA_BACKEND_MATH;
+  if (d->q_dim != 4 || d->k_dim != 4 || d->v_dim != 4) return MI355_SDPA_BACKEND_MATH;
+  if (d->has_symbolic_shape) return MI355_SDPA_BACKEND_MATH;
+  for (int i = 0; i < 4; ++i)
+    if (d->q_size[i] == 0 || d->k_size[i] == 0 || d->v_size[i] == 0) return MI355_SDPA_BACKEND_MATH;
+  return MI355_SDPA_BACKEND_OVERRIDEABLE;
+}
+
+int mi355_sdpa_validate(const mi355_sdpa_desc* d, char* msg, size_t n) {
+  if (msg && n) msg[0] = 0;
+  if (!d) return fail(msg, n, "SDPA: null descriptor");
+  if (d->return_debug_mask)
+    return fail(msg, n, "return_debug_mask=True is not supported in Neuron SDPA implementation");
+  if (d->has_attn_bias && d->is_causal)
+    return fail(msg, n,
+                "_scaled_dot_product_attention: Explicit attn_mask should not be set when "
+                "is_causal=True");
+  int dt = d->q_dtype;
+  if (dt == MI355_SDPA_F64) dt = MI355_SDPA_F32;  // float64 is computed as float32 by the host
+  if (dt != MI355_SDPA_F32 && dt != MI355_SDPA_F16 && dt != MI355_SDPA_BF16)
+    return fail(msg, n, "SDPA: query dtype must be float32, float16, or bfloat16, got %s",
+                dtype_name(d->q_dtype));
+  if (d->k_dtype != d->q_dtype || d->v_dtype != d->q_dtype)
+    return fail(msg, n, "SDPA: query, key, value must have the same dtype");
+  if (d->q_dim != 4 || d->k_dim != 4 || d->v_dim != 4)
+    return fail(msg, n, "SDPA: query, key, value must be 4D tensors (B, H, S, D)");
+  if (d->q_size[0] != d->k_size[0] || d->q_size[0] != d->v_size[0])
+    return fail(msg, n, "SDPA: batch sizes must match");
+  if (d->k_size[1] != d->v_size[1])
+    return fail(msg, n, "SDPA: key and value must have the same number of heads");
+  if (d->k_size[2] != d->v_size[2])
+    return fail(msg, n, "SDPA: key and value must have the same sequence length");
+  if (d->k_size[1] == 0 || d->q_size[1] % d->k_size[1] != 0)
+    return fail(msg, n,
+                "SDPA: Number of heads in key and value must divide the number of heads in query");
+  if (d->dropout_p < 0.f || d->dropout_p > 1.f)
+    return fail(msg, n, "dropout_p=%g is outside [0, 1]. Pass a value in [0, 1].", (double)d->dropout_p);
+  return MI355_SDPA_OK;
+}
+
+int mi355_sdpa_out_strides(const int64_t ref_sizes[4], const int64_t ref_strides[4],
+                           const int64_t out_sizes[4], int64_t out_strides[4]) {
+  (void)ref_sizes;
+  int order[4] = {0, 1, 2, 3};
+  // outermost first; ties keep the original dimension order
+  std::stable_sort(order, order + 4, [&](int a, int b) { return ref_strides[a] > ref_strides[b]; });
+  int64_t s = 1;
+  for (int i = 3; i >= 0; --i) {
+    out_strides[order[i]] = s;
+    s *= std::max<int64_t>(out_sizes[order[i]], 1);
+  }
+  return MI355_SDPA_OK;
+}
+
+static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
+  if (!d) return MI355_SDPA_KERNEL_NONE;
+  if (d->q_dim != 4 || d->k_dim != 4 || d->v_dim != 4) return MI355_SDPA_KERNEL_NONE;
+  const int64_t B = d->q_size[0], Hq = d->q_size[1], L = d->q_size[2], E = d->q_size[3];
+  const int64_t Hkv = d->k_size[1], S = d->k_size[2], Dv = d->v_size[3];
+  const bool shapes = B > 0 && Hq > 0 && L > 0 && E > 0 && Hkv > 0 && S > 0 && Dv > 0 &&
+                      d->k_size[0] == B && d->v_size[0] == B && d->v_size[1] == Hkv &&
+                      d->v_size[2] == S && d->k_size[3] == E && Hq % Hkv == 0;
+  if (!shapes) return MI355_SDPA_KERNEL_NONE;
+  if (d->q_dtype != d->k_dtype || d->q_dtype != d->v_dtype) return MI355_SDPA_KERNEL_NONE;
+  if (d->q_dtype != MI355_SDPA_F32 && d->q_dtype != MI355_SDPA_F16 && d->q_dtype != MI355_SDPA_BF16)
+    return MI355_SDPA_KERNEL_NONE;
+  if (d->return_debug_mask) return MI355_SDPA_KERNEL_NONE;
+  if (E > 512 || Dv > 512) return MI355_SDPA_KERNEL_NONE;
+  const float scale = d->has_scale ? d->scale : 1.f;
+  const bool fast = d->q_dtype != MI355_SDPA_F32 && E == Dv && (E == 64 || E == 128) &&
+                    !d->has_attn_bias && d->dropout_p == 0.f && scale > 0.f &&
+                    d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;
+  (void)backward;
+  return fast ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
+}
+
+int mi355_sdpa_can_use_fused_fwd(const mi355_sdpa_desc* d) { return kernel_for(d, false); }
+int mi355_sdpa_can_use_fused_bwd(const mi355_sdpa_desc* d) { return kernel_for(d, true); }
+
+int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
+  if (!p) return set_error("SDPA: null params"), MI355_SDPA_ERR_INVALID;
+  if (!tensor_ok(p->q, "query") || !tensor_ok(p->k, "key") || !tensor_ok(p->v, "value") ||
+      !tensor_ok(p->out, "out"))
+    return MI355_SDPA_ERR_INVALID;
+  if (!shapes_ok(p->q, p->k, p->v)) return MI355_SDPA_ERR_INVALID;
+  if (!same_shape(p->out, p->q.size[0], p->q.size[1], p->q.size[2], p->v.size[3]))
+    return set_error("SDPA: out must have shape (B, Hq, L, Dv)"), MI355_SDPA_ERR_INVALID;
+  if (p->bias.data && !same_shape(p->bias, p->q.size[0], p->q.size[1], p->q.size[2], p->k.size[2]))
+    return set_error("SDPA: attn_bias must be expanded to (B, Hq, L, S)"), MI355_SDPA_ERR_INVALID;
+  if (p->dropout_p < 0.f || p->dropout_p > 1.f)
+    return set_error("dropout_p=%g is outside [0, 1]. Pass a value in [0, 1].", (double)p->dropout_p),
+           MI355_SDPA_ERR_INVALID;
+  if (p->dropout_p > 0.f && !p->dropout_keep)
+    return set_error("SDPA: dropout_p > 0 needs a keep mask"), MI355_SDPA_ERR_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  const char* why = "";
+  int kernel = p->force_kernel;
+  if (kernel == 0) kernel = fwd_mfma_supported(*p, &why) ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
+  if (kernel == MI355_SDPA_KERNEL_MFMA) return launch_fwd_mfma(*p, s);
+  if (kernel == MI355_SDPA_KERNEL_GENERIC) return launch_fwd_generic(*p, s);
+  return set_error("SDPA: unknown kernel id %d", kernel), MI355_SDPA_ERR_INVALID;
+}
+
+static bool bwd_args_ok(const mi355_sdpa_bwd_params* p) {
+  if (!p) return set_error("SDPA: null params"), false;
+  if (!tensor_ok(p->grad_out, "grad_out") || !tensor_ok(p->q, "query") || !tensor_ok(p->k, "key") ||
+      !tensor_ok(p->v, "value") || !tensor_ok(p->out, "out") || !tensor_ok(p->grad_q, "grad_query") ||
+      !tensor_ok(p->grad_k, "grad_key") || !tensor_ok(p->grad_v, "grad_value"))
+    return false;
+  if (!p->lse) return set_error("SDPA: logsumexp is a null pointer"), false;
+  if (!shapes_ok(p->q, p->k, p->v)) return false;
+  const int64_t B = p->q.size[0], Hq = p->q.size[1], L = p->q.size[2], E = p->q.size[3];
+  const int64_t Hkv = p->k.size[1], S = p->k.size[2], Dv = p->v.size[3];
+  if (!same_shape(p->out, B, Hq, L, Dv) || !same_shape(p->grad_out, B, Hq, L, Dv))
+    return set_error("SDPA: out and grad_out must have shape (B, Hq, L, Dv)"), false;
+  if (!same_shape(p->grad_q, B, Hq, L, E) || !same_shape(p->grad_k, B, Hkv, S, E) ||
+      !same_shape(p->grad_v, B, Hkv, S, Dv))
+    return set_error("SDPA: gradient buffers must have the shapes of query, key and value"), false;
+  if (p->bias.data && !same_shape(p->bias, B, Hq, L, S))
+    return set_error("SDPA: attn_bias must be expanded to (B, Hq, L, S)"), false;
+  if (p->grad_bias.data && !same_shape(p->grad_bias, B, Hq, L, S))
+    return set_error("SDPA: grad_attn_bias must have shape (B, Hq, L, S)"), false;
+  if (p->dropout_p < 0.f || p->dropout_p > 1.f)
+    return set_error("dropout_p=%g is outside [0, 1]. Pass a value in [0, 1].", (double)p->dropout_p), false;
+  if (p->dropout_p > 0.f && !p->dropout_keep) return set_error("SDPA: dropout_p > 0 needs a keep mask"), false;
+  return true;
+}
+
+static int bwd_kernel_choice(const mi355_sdpa_bwd_params* p) {
+  if (p->force_kernel) return p->force_kernel;
+  const char* why;
+  return bwd_mfma_supported(*p, &why) ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
+}
+
+size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p) {
+  if (!p) return 0;
+  // sized for either kernel so the host can allocate before the choice is visible to it
+  return std::max(bwd_generic_workspace(*p), bwd_mfma_workspace(*p));
+}
+
+int mi355_sdpa_bwd(const mi355_sdpa_bwd_params* p, void* stream) {
+  if (!bwd_args_ok(p)) return MI355_SDPA_ERR_INVALID;
+  const int kernel = bwd_kernel_choice(p);
+  const size_t need = kernel == MI355_SDPA_KERNEL_MFMA ? bwd_mfma_workspace(*p) : bwd_generic_workspace(*p);
+  if (need && (!p->workspace || p->workspace_bytes < need))
+    return set_error("SDPA: backward workspace too small (%zu < %zu bytes)", p->workspace_bytes, need),
+           MI355_SDPA_ERR_INVALID;
+  hipStream_t s = (hipStream_t)stream;
+  if (kernel == MI355_SDPA_KERNEL_MFMA) return launch_bwd_mfma(*p, s);
+  if (kernel == MI355_SDPA_KERNEL_GENERIC) return launch_bwd_generic(*p, s);
+  return set_error("SDPA: unknown kernel id %d", kernel), MI355_SDPA_ERR_INVALID;
+}
+
+size_t mi355_sdpa_decode_workspace_bytes(const mi355_sdpa_decode_params* p) {
+  return p ? decode_workspace(*p) : 0;
+}
+
+int mi355_sdpa_decode_fp8kv(const mi355_sdpa_decode_params* p, void* stream) {
+  if (!p) return set_error("SDPA: null params"), MI355_SDPA_ERR_INVALID;
+  if (!tensor_ok(p->q, "query") || !tensor_ok(p->k, "key") || !tensor_ok(p->v, "value") ||
+      !tensor_ok(p->out, "out"))
+    return MI355_SDPA_ERR_INVALID;
+  if (!p->k_scale || !p->v_scale) return set_error("SDPA decode: k_scale / v_scale missing"), MI355_SDPA_ERR_INVALID;
+  if (!shapes_ok(p->q, p->k, p->v)) return MI355_SDPA_ERR_INVALID;
+  if (!same_shape(p->out, p->q.size[0], p->q.size[1], p->q.size[2], p->v.size[3]))
+    return set_error("SDPA decode: out must have shape (B, Hq, Lq, D)"), MI355_SDPA_ERR_INVALID;
+  const size_t need = decode_workspace(*p);
+  if (need && (!p->workspace || p->workspace_bytes < need))
+    return set_error("SDPA decode: workspace too small (%zu < %zu bytes)", p->workspace_bytes, need),
+           MI355_SDPA_ERR_INVALID;
+  return launch_decode_fp8kv(*p, (hipStream_t)stream);
+}
+
+}  // extern "C"

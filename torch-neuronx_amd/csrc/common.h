@@ -1,0 +1,59 @@
+// Shared device/host helpers for the gfx950 SDPA kernels.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/mi355_sdpa.h"
+
+namespace mi355 {
+
+// host side -------------------------------------------------------------------------------
+void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
+int check_launch(const char* what);
+
+int launch_fwd_generic(const mi355_sdpa_fwd_params& p, hipStream_t s);
+int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s);
+bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why);
+int launch_bwd_generic(const mi355_sdpa_bwd_params& p, hipStream_t s);
+int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s);
+bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why);
+size_t bwd_generic_workspace(const mi355_sdpa_bwd_params& p);
+size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p);
+int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s);
+size_t decode_workspace(const mi355_sdpa_decode_params& p);
+int decode_pick_splits(const mi355_sdpa_decode_params& p);
+
+// device side -----------------------------------------------------------------------------
+typedef __bf16 bf16_t;
+typedef _Float16 f16_t;
+
+struct T4 {  // device view of a 4-D tensor, strides in elements
+  const void* data;
+  int64_t st[4];
+};
+
+static inline T4 view(const mi355_sdpa_tensor& t) {
+  T4 r;
+  r.data = t.data;
+  for (int i = 0; i < 4; ++i) r.st[i] = t.stride[i];
+  return r;
+}
+
+template <typename T>
+__device__ __forceinline__ float to_f32(T x) {
+  return (float)x;
+}
+
+__device__ __forceinline__ float wave_max(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x = fmaxf(x, __shfl_xor(x, o, 64));
+  return x;
+}
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) x += __shfl_xor(x, o, 64);
+  return x;
+}
+
+}  // namespace mi355

@@ -1,0 +1,382 @@
+// Decode-step attention over an fp8 (OCP e4m3) K/V cache for gfx950: split-KV flash decoding
+// on the 16x16x32 fp8 MFMA, streaming K and V straight from HBM into registers (no LDS on
+// the hot path).  Defined as torch_neuronx/_sdpa_math.py:51-95 applied to the dequantised
+// cache with a key-padding bias; the reference itself has no fp8 attention path.
+//
+// Work split: grid = (key chunks, kv heads, batch); a workgroup of 4 wavefronts takes one
+// chunk of one (batch, kv head) and serves all R = Lq * Hq/Hkv query rows that share that kv
+// head, so every K/V byte is read from HBM exactly once.  Chunks at or past kv_lens[b] exit
+// at once: padding is never read.  Each wavefront walks its quarter of the chunk 32 keys at a
+// time with its own running max / sum / output, the four are merged through LDS, and a second
+// small kernel merges the chunks of a sequence.
+//
+// Precision without dequantising the cache: the bf16 query row is scaled by a power of two
+// and split into up to three e4m3 terms (q = q0 + q1 + q2, exact to ~12 bits); the terms
+// occupy separate columns of the 16-wide MFMA N dimension, which would otherwise idle, and
+// are summed after the product.  The probabilities are split the same way before P*V.
+//
+// Per 32 keys a lane loads 64 contiguous K bytes of one key (A operand of S^T = K Q^T, the
+// contraction order is permuted identically for Q) and eight 4-byte pieces of V which are
+// byte-transposed in registers into the A operand of O^T = V^T P^T.
+#include "common.h"
+
+namespace mi355 {
+namespace {
+
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) float f32x2;
+
+constexpr int D = 128;
+constexpr int kWaves = 4;
+constexpr float kLog2e = 1.4426950408889634f;
+constexpr float kLn2 = 0.6931471805599453f;
+constexpr float kPScale = 256.f;  // probabilities are stored as e4m3 of 256*p
+
+struct DecP {
+  const void* q;
+  const uint8_t *k, *v;
+  const float *k_scale, *v_scale;
+  const int32_t* kv_lens;
+  void* out;
+  float* lse;
+  float* ws_o;   // (B,Hkv,chunks,R,128)
+  float* ws_ml;  // (B,Hkv,chunks,R,2)
+  int64_t q_sb, q_sh, q_sl;
+  int64_t k_sb, k_sh, k_sl;
+  int64_t v_sb, v_sh, v_sl;
+  int64_t o_sb, o_sh, o_sl;
+  int B, Hq, Hkv, Lq, S, R;
+  int chunk_keys, chunks;
+  float scale;
+};
+
+__device__ __forceinline__ uint32_t fp8x2(float a, float b) {
+  return (uint32_t)__builtin_amdgcn_cvt_pk_fp8_f32(a, b, 0, false) & 0xffffu;
+}
+__device__ __forceinline__ f32x2 fp8x2_to_f32(uint32_t w) {
+  return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
+}
+
+// e4m3 term `part` of the split x = t0 + t1 + t2 for a pair of values, as two packed bytes
+__device__ __forceinline__ uint32_t split_pair(float a, float b, int part) {
+  uint32_t w = fp8x2(a, b);
+  if (part == 0) return w;
+  f32x2 d = fp8x2_to_f32(w);
+  a -= d[0], b -= d[1];
+  w = fp8x2(a, b);
+  if (part == 1) return w;
+  d = fp8x2_to_f32(w);
+  a -= d[0], b -= d[1];
+  return fp8x2(a, b);
+}
+
+__device__ __forceinline__ long as_long(uint32_t lo, uint32_t hi) {
+  return (long)(((uint64_t)hi << 32) | lo);
+}
+
+struct KVRegs {
+  u32x4 k[2][2];      // [16-key block][16-byte half of the lane's 32 bytes]
+  uint32_t v[2][8];   // [64-wide half of d][key slot]
+};
+
+template <typename TQ, int PARTS>
+__global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
+  constexpr int RS = PARTS == 3 ? 4 : 8;  // column stride between split terms
+  __shared__ float s_o[kWaves][8][D];
+  __shared__ float s_m[kWaves][8], s_l[kWaves][8];
+
+  const int chunk = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+  int len = p.S;
+  if (p.kv_lens) len = min(p.S, max(0, p.kv_lens[b]));
+  const int c_begin = chunk * p.chunk_keys;
+  if (c_begin >= len) return;  // whole workgroup: nothing but padding here
+  const int c_end = min(len, c_begin + p.chunk_keys);
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int n = lane & 15, g = lane >> 4;
+  const int part = n / RS, r = n % RS;
+  const int rep = p.Hq / p.Hkv;
+  const bool col_live = r < p.R && part < PARTS;
+  const int rr = min(r, p.R - 1);
+  const int h = hk * rep + rr % rep, lq = rr / rep;
+
+  // ---- query fragment: B operand of S^T = K Q^T ------------------------------------------
+  // the lane owns d = 32g .. 32g+31 of row r; step ks consumes d = 32g + 8ks .. +7
+  float qv[32];
+  {
+    const TQ* qr = (const TQ*)p.q + b * p.q_sb + h * p.q_sh + lq * p.q_sl + 32 * g;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) qv[i] = to_f32(qr[i]);
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qv[i]));
+  amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+  amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+  // power-of-two pre-scale so the row peaks in [120, 240]: well inside e4m3 and exact
+  const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
+  long qb[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      w[j] = col_live ? split_pair(qv[ks * 8 + 2 * j] * f, qv[ks * 8 + 2 * j + 1] * f, part) : 0u;
+    qb[ks] = as_long(w[0] | (w[1] << 16), w[2] | (w[3] << 16));
+  }
+  const float kscale = p.k_scale[b * p.Hkv + hk];
+  const float c_row = p.scale * kscale / f * kLog2e;  // raw dot -> log2-domain logit
+
+  // ---- this wavefront's key range -----------------------------------------------------------
+  const int wave_keys = p.chunk_keys / kWaves;
+  const int w_begin = c_begin + wave * wave_keys;
+  const int w_end = min(c_end, w_begin + wave_keys);
+  const int steps = w_end > w_begin ? (w_end - w_begin + 31) / 32 : 0;
+
+  const uint8_t* kp = p.k + b * p.k_sb + hk * p.k_sh;
+  const uint8_t* vp = p.v + b * p.v_sb + hk * p.v_sh;
+  const int last = len - 1;
+
+  auto load = [&](KVRegs& R_, int step) {
+    const int base = w_begin + step * 32;
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      const int row = min(base + blk * 16 + n, last);
+      const uint8_t* kr = kp + (int64_t)row * p.k_sl + 32 * g;
+      R_.k[blk][0] = *(const u32x4*)kr;
+      R_.k[blk][1] = *(const u32x4*)(kr + 16);
+    }
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+      const int row = min(base + (s >> 2) * 16 + 4 * g + (s & 3), last);
+      const uint8_t* vr = vp + (int64_t)row * p.v_sl + 4 * n;
+      R_.v[0][s] = *(const uint32_t*)vr;
+      R_.v[1][s] = *(const uint32_t*)(vr + 64);
+    }
+  };
+
+  f32x4 oacc[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+  float m_run = -INFINITY, l_run = 0.f;
+
+  auto compute = [&](const KVRegs& R_, int step) {
+    const int base = w_begin + step * 32;
+    // S^T = K Q^T : rows = 16 keys of a block, columns = (split term, query row)
+    f32x4 sacc[2];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+      sacc[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const u32x4 kk = R_.k[blk][ks >> 1];
+        const long a = as_long(kk[(ks & 1) * 2], kk[(ks & 1) * 2 + 1]);
+        sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, qb[ks], sacc[blk], 0, 0, 0);
+      }
+    }
+    float t[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      float x = sacc[i >> 2][i & 3];
+      if (PARTS == 3) x += __shfl_xor(x, 4, 64);
+      x += __shfl_xor(x, 8, 64);
+      const int key = base + (i >> 2) * 16 + 4 * g + (i & 3);
+      t[i] = key < w_end ? x * c_row : -INFINITY;
+    }
+    float tmax = t[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) tmax = fmaxf(tmax, t[i]);
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+    const float m_new = fmaxf(m_run, tmax);  // finite: every step holds at least one live key
+    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+    m_run = m_new;
+    float pv[8], psum = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      pv[i] = __builtin_amdgcn_exp2f(t[i] - m_new);
+      psum += pv[i];
+    }
+    l_run = l_run * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
+    // P^T (B operand): key slot s of this lane is key (s/4)*16 + 4g + s%4, the order V is loaded in
+    uint32_t pw[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      pw[j] = col_live ? split_pair(pv[2 * j] * kPScale, pv[2 * j + 1] * kPScale, part) : 0u;
+    const long pb = as_long(pw[0] | (pw[1] << 16), pw[2] | (pw[3] << 16));
+    // O^T += V^T P^T : byte-transpose the 4-byte V pieces into rows d = 64*hf + 4n + j
+#pragma unroll
+    for (int hf = 0; hf < 2; ++hf) {
+      uint32_t o_lo[4], o_hi[4];
+#pragma unroll
+      for (int q4 = 0; q4 < 2; ++q4) {
+        const uint32_t w0 = R_.v[hf][q4 * 4 + 0], w1 = R_.v[hf][q4 * 4 + 1];
+        const uint32_t w2 = R_.v[hf][q4 * 4 + 2], w3 = R_.v[hf][q4 * 4 + 3];
+        const uint32_t t0 = __builtin_amdgcn_perm(w1, w0, 0x05010400);
+        const uint32_t t1 = __builtin_amdgcn_perm(w1, w0, 0x07030602);
+        const uint32_t t2 = __builtin_amdgcn_perm(w3, w2, 0x05010400);
+        const uint32_t t3 = __builtin_amdgcn_perm(w3, w2, 0x07030602);
+        uint32_t* o = q4 ? o_hi : o_lo;
+        o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100);
+        o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302);
+        o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100);
+        o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        oacc[hf * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(
+            as_long(o_lo[j], o_hi[j]), pb, oacc[hf * 4 + j], 0, 0, 0);
+    }
+  };
+
+  KVRegs ra, rb;
+  if (steps > 0) load(ra, 0);
+  for (int s = 0; s < steps; s += 2) {
+    if (s + 1 < steps) load(rb, s + 1);
+    compute(ra, s);
+    if (s + 2 < steps) load(ra, s + 2);
+    if (s + 1 < steps) compute(rb, s + 1);
+  }
+
+  // ---- merge split terms, then the four wavefronts, and emit the chunk's partial result ------
+#pragma unroll
+  for (int i = 0; i < 8; ++i)
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      float x = oacc[i][e];
+      if (PARTS == 3) x += __shfl_xor(x, 4, 64);
+      x += __shfl_xor(x, 8, 64);
+      oacc[i][e] = x;
+    }
+  float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+  l_tot += __shfl_xor(l_tot, 32, 64);
+  if (n < p.R) {  // split term 0 lanes of live rows
+    if (g == 0) s_m[wave][n] = m_run, s_l[wave][n] = l_tot;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int e = 0; e < 4; ++e)
+        s_o[wave][n][(i >> 2) * 64 + 16 * g + 4 * e + (i & 3)] = oacc[i][e];
+  }
+  __syncthreads();
+  const float vscale = p.v_scale[b * p.Hkv + hk] * (1.f / kPScale);
+  const int64_t slot = ((int64_t)(b * p.Hkv + hk) * p.chunks + chunk) * p.R;
+  for (int idx = tid; idx < p.R * D; idx += 64 * kWaves) {
+    const int row = idx / D, d = idx % D;
+    float M = s_m[0][row];
+#pragma unroll
+    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, s_m[w][row]);
+    float L = 0.f, O = 0.f;
+#pragma unroll
+    for (int w = 0; w < kWaves; ++w) {
+      const float sc = __builtin_amdgcn_exp2f(s_m[w][row] - M);  // empty wavefront: exp2(-inf) = 0
+      L += s_l[w][row] * sc;
+      O += s_o[w][row][d] * sc;
+    }
+    p.ws_o[(slot + row) * D + d] = O * vscale;
+    if (d == 0) p.ws_ml[(slot + row) * 2] = M, p.ws_ml[(slot + row) * 2 + 1] = L;
+  }
+}
+
+// Merge the chunk partials of one (batch, kv head, query row); 128 threads = 128 output columns.
+template <typename TQ>
+__global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
+  const int row = blockIdx.x % p.R;
+  const int hk = (blockIdx.x / p.R) % p.Hkv;
+  const int b = blockIdx.x / (p.R * p.Hkv);
+  const int d = threadIdx.x;
+  int len = p.S;
+  if (p.kv_lens) len = min(p.S, max(0, p.kv_lens[b]));
+  const int nch = (len + p.chunk_keys - 1) / p.chunk_keys;
+  const int64_t slot0 = (int64_t)(b * p.Hkv + hk) * p.chunks * p.R + row;
+  float M = -INFINITY;
+  for (int c = 0; c < nch; ++c) M = fmaxf(M, p.ws_ml[(slot0 + (int64_t)c * p.R) * 2]);
+  float L = 0.f, O = 0.f;
+  for (int c = 0; c < nch; ++c) {
+    const int64_t s = slot0 + (int64_t)c * p.R;
+    const float sc = __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
+    L += p.ws_ml[s * 2 + 1] * sc;
+    O += p.ws_o[s * D + d] * sc;
+  }
+  const int rep = p.Hq / p.Hkv;
+  const int h = hk * rep + row % rep, lq = row / rep;
+  TQ* o = (TQ*)p.out + b * p.o_sb + h * p.o_sh + lq * p.o_sl;
+  o[d] = (TQ)(L > 0.f ? O / L : 0.f);
+  if (p.lse && d == 0)
+    p.lse[((int64_t)b * p.Hq + h) * p.Lq + lq] = L > 0.f ? (M + __builtin_amdgcn_logf(L)) * kLn2 : -INFINITY;
+}
+
+int chunk_keys_for(const mi355_sdpa_decode_params& p) {
+  const int S = (int)p.k.size[2];
+  int ck = 512;
+  if (p.num_splits > 0) ck = (S + p.num_splits - 1) / p.num_splits;
+  ck = ((ck + 127) / 128) * 128;
+  return ck < 128 ? 128 : ck;
+}
+
+template <typename TQ>
+int launch_t(const DecP& g, hipStream_t s) {
+  dim3 grid(g.chunks, g.Hkv, g.B), block(64 * kWaves);
+  if (g.R <= 4) hipLaunchKernelGGL((decode_kernel<TQ, 3>), grid, block, 0, s, g);
+  else hipLaunchKernelGGL((decode_kernel<TQ, 2>), grid, block, 0, s, g);
+  int rc = check_launch("decode_kernel");
+  if (rc) return rc;
+  hipLaunchKernelGGL((decode_merge_kernel<TQ>), dim3(g.B * g.Hkv * g.R), dim3(D), 0, s, g);
+  return check_launch("decode_merge_kernel");
+}
+
+}  // namespace
+
+int decode_pick_splits(const mi355_sdpa_decode_params& p) {
+  const int S = (int)p.k.size[2], ck = chunk_keys_for(p);
+  return (S + ck - 1) / ck;
+}
+
+size_t decode_workspace(const mi355_sdpa_decode_params& p) {
+  const int64_t rep = p.k.size[1] ? p.q.size[1] / p.k.size[1] : 0;
+  const int64_t R = rep * p.q.size[2];
+  const int64_t slots = p.q.size[0] * p.k.size[1] * decode_pick_splits(p) * R;
+  return (size_t)slots * (D + 2) * sizeof(float);
+}
+
+int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
+  DecP g;
+  g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Lq = (int)p.q.size[2];
+  g.Hkv = (int)p.k.size[1], g.S = (int)p.k.size[2];
+  const int rep = g.Hq / g.Hkv;
+  g.R = rep * g.Lq;
+  if (p.q.size[3] != D || p.v.size[3] != D)
+    return set_error("SDPA decode: head dim must be 128, got %lld/%lld", (long long)p.q.size[3],
+                     (long long)p.v.size[3]), MI355_SDPA_ERR_UNSUPPORTED;
+  if (g.R < 1 || g.R > 8)
+    return set_error("SDPA decode: Lq * Hq/Hkv must be in [1, 8], got %d", g.R), MI355_SDPA_ERR_UNSUPPORTED;
+  if (p.q.stride[3] != 1 || p.k.stride[3] != 1 || p.v.stride[3] != 1 || p.out.stride[3] != 1)
+    return set_error("SDPA decode: head dim must be unit-stride"), MI355_SDPA_ERR_UNSUPPORTED;
+  if (((uintptr_t)p.k.data & 15) || ((uintptr_t)p.v.data & 15) || (p.k.stride[2] & 15) || (p.v.stride[2] & 15) ||
+      (p.k.stride[1] & 15) || (p.v.stride[1] & 15) || (p.k.stride[0] & 15) || (p.v.stride[0] & 15))
+    return set_error("SDPA decode: K/V rows must be 16-byte aligned"), MI355_SDPA_ERR_UNSUPPORTED;
+  if (g.B == 0 || g.S == 0) return set_error("SDPA decode: empty batch or cache"), MI355_SDPA_ERR_UNSUPPORTED;
+  g.q = p.q.data, g.k = (const uint8_t*)p.k.data, g.v = (const uint8_t*)p.v.data;
+  g.k_scale = p.k_scale, g.v_scale = p.v_scale, g.kv_lens = p.kv_lens, g.out = p.out.data, g.lse = p.lse;
+  g.q_sb = p.q.stride[0], g.q_sh = p.q.stride[1], g.q_sl = p.q.stride[2];
+  g.k_sb = p.k.stride[0], g.k_sh = p.k.stride[1], g.k_sl = p.k.stride[2];
+  g.v_sb = p.v.stride[0], g.v_sh = p.v.stride[1], g.v_sl = p.v.stride[2];
+  g.o_sb = p.out.stride[0], g.o_sh = p.out.stride[1], g.o_sl = p.out.stride[2];
+  g.chunk_keys = chunk_keys_for(p);
+  g.chunks = (g.S + g.chunk_keys - 1) / g.chunk_keys;
+  g.scale = p.scale;
+  const int64_t slots = (int64_t)g.B * g.Hkv * g.chunks * g.R;
+  g.ws_o = (float*)p.workspace;
+  g.ws_ml = g.ws_o + slots * D;
+  switch (p.q_dtype) {
+    case MI355_SDPA_BF16: return launch_t<bf16_t>(g, s);
+    case MI355_SDPA_F16: return launch_t<f16_t>(g, s);
+    case MI355_SDPA_F32: return launch_t<float>(g, s);
+  }
+  return set_error("SDPA decode: query dtype must be float32, float16, or bfloat16"), MI355_SDPA_ERR_INVALID;
+}
+
+}  // namespace mi355

@@ -1,0 +1,141 @@
+"""ctypes binding of the C ABI declared in include/mi355_sdpa.h.
+
+The library is loaded from the package's ``lib/`` directory.  There is no fallback: if it is
+missing the import of any op raises, so a GPU run can never silently take another path.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+import torch
+
+from ._build import LIB_PATH
+
+F32, F16, BF16, F64, BOOL, FP8_E4M3, OTHER = 0, 1, 2, 3, 4, 5, 99
+KERNEL_NONE, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+BACKEND_MATH, BACKEND_OVERRIDEABLE = 0, 4
+OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_LAUNCH = 0, -1, -2, -3
+
+_DTYPES = {
+    torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64,
+    torch.bool: BOOL, torch.float8_e4m3fn: FP8_E4M3,
+}
+
+
+def dtype_id(dt: torch.dtype) -> int:
+    return _DTYPES.get(dt, OTHER)
+
+
+class Tensor4(C.Structure):
+    _fields_ = [("data", C.c_void_p), ("size", C.c_int64 * 4), ("stride", C.c_int64 * 4)]
+
+
+class Desc(C.Structure):
+    _fields_ = [
+        ("q_dim", C.c_int32), ("k_dim", C.c_int32), ("v_dim", C.c_int32),
+        ("q_size", C.c_int64 * 4), ("k_size", C.c_int64 * 4), ("v_size", C.c_int64 * 4),
+        ("q_dtype", C.c_int32), ("k_dtype", C.c_int32), ("v_dtype", C.c_int32),
+        ("on_device", C.c_int32), ("has_symbolic_shape", C.c_int32), ("has_attn_bias", C.c_int32),
+        ("is_causal", C.c_int32), ("return_debug_mask", C.c_int32), ("has_scale", C.c_int32),
+        ("scale", C.c_float), ("dropout_p", C.c_float), ("requires_lse", C.c_int32),
+        ("q_last_stride", C.c_int32), ("k_last_stride", C.c_int32), ("v_last_stride", C.c_int32),
+    ]
+
+
+class FwdParams(C.Structure):
+    _fields_ = [
+        ("q", Tensor4), ("k", Tensor4), ("v", Tensor4), ("out", Tensor4),
+        ("lse", C.c_void_p), ("bias", Tensor4), ("bias_dtype", C.c_int32),
+        ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
+        ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
+        ("force_kernel", C.c_int32),
+    ]
+
+
+class BwdParams(C.Structure):
+    _fields_ = [
+        ("grad_out", Tensor4), ("q", Tensor4), ("k", Tensor4), ("v", Tensor4), ("out", Tensor4),
+        ("lse", C.c_void_p), ("grad_q", Tensor4), ("grad_k", Tensor4), ("grad_v", Tensor4),
+        ("bias", Tensor4), ("bias_dtype", C.c_int32), ("grad_bias", Tensor4),
+        ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
+        ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("force_kernel", C.c_int32),
+    ]
+
+
+class DecodeParams(C.Structure):
+    _fields_ = [
+        ("q", Tensor4), ("k", Tensor4), ("v", Tensor4),
+        ("k_scale", C.c_void_p), ("v_scale", C.c_void_p), ("kv_lens", C.c_void_p),
+        ("out", Tensor4), ("lse", C.c_void_p), ("q_dtype", C.c_int32), ("scale", C.c_float),
+        ("num_splits", C.c_int32), ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+    ]
+
+
+EXPORTS = {
+    "mi355_sdpa_fwd": (C.c_int, [C.POINTER(FwdParams), C.c_void_p]),
+    "mi355_sdpa_bwd": (C.c_int, [C.POINTER(BwdParams), C.c_void_p]),
+    "mi355_sdpa_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdParams)]),
+    "mi355_sdpa_decode_fp8kv": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),
+    "mi355_sdpa_decode_workspace_bytes": (C.c_size_t, [C.POINTER(DecodeParams)]),
+    "mi355_sdpa_choose_backend": (C.c_int, [C.POINTER(Desc)]),
+    "mi355_sdpa_validate": (C.c_int, [C.POINTER(Desc), C.c_char_p, C.c_size_t]),
+    "mi355_sdpa_out_strides": (C.c_int, [C.POINTER(C.c_int64), C.POINTER(C.c_int64),
+                                         C.POINTER(C.c_int64), C.POINTER(C.c_int64)]),
+    "mi355_sdpa_can_use_fused_fwd": (C.c_int, [C.POINTER(Desc)]),
+    "mi355_sdpa_can_use_fused_bwd": (C.c_int, [C.POINTER(Desc)]),
+    "mi355_sdpa_last_error": (C.c_char_p, []),
+    "mi355_sdpa_abi_version": (C.c_int, []),
+}
+
+_lib = None
+
+
+def load() -> C.CDLL:
+    """Load the shared library (once).  Raises if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(
+                f"{LIB_PATH} is missing: build the HIP extension first "
+                "(python -m torch_neuronx_amd._build, or __graft_entry__.build()). "
+                "There is no fallback path."
+            )
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in EXPORTS.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _lib = lib
+    return _lib
+
+
+def last_error() -> str:
+    return load().mi355_sdpa_last_error().decode()
+
+
+def tensor4(t) -> Tensor4:
+    r = Tensor4()
+    if t is None:
+        return r
+    assert t.dim() == 4
+    r.data = t.data_ptr()
+    for i in range(4):
+        r.size[i] = t.size(i)
+        r.stride[i] = t.stride(i)
+    return r
+
+
+def current_stream(device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def check(rc: int) -> None:
+    """Turn a status code into the exception type the operator contract asks for."""
+    if rc == OK:
+        return
+    msg = last_error()
+    if rc == ERR_UNSUPPORTED:
+        raise NotImplementedError(msg)
+    raise RuntimeError(msg)

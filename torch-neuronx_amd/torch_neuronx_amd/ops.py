@@ -1,0 +1,219 @@
+"""Host side of the fused attention path: marshals torch tensors into the C ABI.
+
+Everything here is plumbing - allocation of outputs with the layout rules of the operator
+contract, argument normalisation and error mapping.  All arithmetic happens in the HIP
+kernels behind ``libmi355_sdpa.so``.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import math
+
+import torch
+
+from . import _lib
+
+
+def _require_cuda(t: torch.Tensor, name: str) -> None:
+    if t.device.type != "cuda":
+        raise ValueError(f"Expected a GPU tensor for {name}, got {t.device}")
+
+
+def make_desc(query, key, value, attn_bias=None, dropout_p=0.0, is_causal=False,
+              return_debug_mask=False, scale=None, requires_lse=True) -> _lib.Desc:
+    """Shape/dtype descriptor for the host-logic entry points (works for meta/CPU tensors)."""
+    d = _lib.Desc()
+    d.q_dim, d.k_dim, d.v_dim = query.dim(), key.dim(), value.dim()
+    symbolic = False
+    for arr, t in ((d.q_size, query), (d.k_size, key), (d.v_size, value)):
+        for i in range(min(4, t.dim())):
+            s = t.shape[i]
+            if isinstance(s, int):
+                arr[i] = s
+            else:
+                symbolic = True
+                arr[i] = 1
+    d.q_dtype, d.k_dtype, d.v_dtype = (_lib.dtype_id(t.dtype) for t in (query, key, value))
+    d.on_device = int(all(t.device.type == "cuda" for t in (query, key, value)))
+    d.has_symbolic_shape = int(symbolic)
+    d.has_attn_bias = int(attn_bias is not None)
+    d.is_causal = int(bool(is_causal))
+    d.return_debug_mask = int(bool(return_debug_mask))
+    d.has_scale = int(scale is not None)
+    d.scale = float(scale) if scale is not None else 0.0
+    d.dropout_p = float(dropout_p)
+    d.requires_lse = int(requires_lse)
+    strides = []
+    for t in (query, key, value):
+        st = t.stride(-1) if t.dim() > 0 and not symbolic else 1
+        strides.append(int(st) if isinstance(st, int) else 1)
+    d.q_last_stride, d.k_last_stride, d.v_last_stride = strides
+    return d
+
+
+def validate(desc: _lib.Desc) -> None:
+    """Raise RuntimeError with the operator-boundary message if the call breaks the contract."""
+    buf = C.create_string_buffer(512)
+    if _lib.load().mi355_sdpa_validate(C.byref(desc), buf, 512) != 0:
+        raise RuntimeError(buf.value.decode())
+
+
+def choose_backend(desc: _lib.Desc) -> int:
+    return _lib.load().mi355_sdpa_choose_backend(C.byref(desc))
+
+
+def can_use_fused_fwd(desc: _lib.Desc) -> int:
+    return _lib.load().mi355_sdpa_can_use_fused_fwd(C.byref(desc))
+
+
+def can_use_fused_bwd(desc: _lib.Desc) -> int:
+    return _lib.load().mi355_sdpa_can_use_fused_bwd(C.byref(desc))
+
+
+def out_strides(ref_sizes, ref_strides, out_sizes):
+    arr = lambda v: (C.c_int64 * 4)(*[int(x) for x in v])
+    res = (C.c_int64 * 4)()
+    _lib.load().mi355_sdpa_out_strides(arr(ref_sizes), arr(ref_strides), arr(out_sizes), res)
+    return tuple(res)
+
+
+def empty_like_layout(ref: torch.Tensor, shape, dtype=None) -> torch.Tensor:
+    """New tensor of ``shape`` whose dimension order follows ``ref`` (stride-0 dims never alias)."""
+    st = out_strides(ref.shape, ref.stride(), shape)
+    return torch.empty_strided(tuple(shape), st, dtype=dtype or ref.dtype, device=ref.device)
+
+
+def _unit_last(t: torch.Tensor) -> torch.Tensor:
+    return t if t.stride(-1) == 1 or t.size(-1) <= 1 else t.contiguous()
+
+
+def _bias_view(attn_bias, B, Hq, L, S):
+    if attn_bias is None:
+        return None, 0
+    b = attn_bias
+    while b.dim() < 4:
+        b = b.unsqueeze(0)
+    b = b.expand(B, Hq, L, S)
+    return b, _lib.dtype_id(b.dtype)
+
+
+def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None, dropout_p=0.0,
+                 dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0):
+    """Fused forward.  K/V arrive at ``Hkv`` heads.  Returns ``(out, lse)``; ``out`` keeps the
+    dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``."""
+    for t, n in ((query, "query"), (key, "key"), (value, "value")):
+        _require_cuda(t, n)
+    B, Hq, L, E = query.shape
+    S, Dv = key.shape[2], value.shape[3]
+    if scale is None:
+        scale = 1.0 / math.sqrt(E)
+    q, k, v = _unit_last(query), _unit_last(key), _unit_last(value)
+    out = empty_like_layout(query, (B, Hq, L, Dv))
+    if out.stride(-1) != 1 and Dv > 1:
+        out = torch.empty((B, Hq, L, Dv), dtype=query.dtype, device=query.device)
+    lse = torch.empty((B, Hq, L), dtype=torch.float32, device=query.device) if need_lse else None
+    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
+    p = _lib.FwdParams()
+    p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (q, k, v, out))
+    p.lse = lse.data_ptr() if lse is not None else None
+    p.bias, p.bias_dtype = _lib.tensor4(bias), bias_dt
+    if kv_lens is not None:
+        kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
+        p.kv_lens = kv_lens.data_ptr()
+    if dropout_p > 0.0:
+        if dropout_keep is None:
+            raise ValueError("dropout_p > 0 needs dropout_keep")
+        dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
+        p.dropout_keep = dropout_keep.data_ptr()
+    p.dropout_p = float(dropout_p)
+    p.dtype = _lib.dtype_id(query.dtype)
+    p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
+    with torch.cuda.device(query.device):
+        rc = _lib.load().mi355_sdpa_fwd(C.byref(p), _lib.current_stream(query.device))
+    _lib.check(rc)
+    return out, lse
+
+
+def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_causal=False,
+                  scale=None, dropout_p=0.0, dropout_keep=None, kv_lens=None,
+                  want_grad_bias=False, force_kernel=0):
+    """Fused backward.  Returns ``(dq, dk, dv, dbias-or-None)``; each gradient keeps the
+    dimension order of its input, dk/dv come back at ``Hkv`` heads."""
+    for t, n in ((grad_out, "grad_out"), (query, "query"), (key, "key"), (value, "value")):
+        _require_cuda(t, n)
+    B, Hq, L, E = query.shape
+    Hkv, S, Dv = key.shape[1], key.shape[2], value.shape[3]
+    if scale is None:
+        scale = 1.0 / math.sqrt(E)
+    go, q, k, v, o = (_unit_last(t) for t in (grad_out, query, key, value, out))
+    lse = lse.to(torch.float32).contiguous()
+
+    def grad_like(ref, shape):
+        g = empty_like_layout(ref, shape)
+        if g.stride(-1) != 1 and shape[-1] > 1:
+            g = torch.empty(shape, dtype=ref.dtype, device=ref.device)
+        return g
+
+    dq, dk, dv = grad_like(query, (B, Hq, L, E)), grad_like(key, (B, Hkv, S, E)), grad_like(value, (B, Hkv, S, Dv))
+    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
+    dbias = None
+    if want_grad_bias and bias is not None:
+        dbias = torch.empty((B, Hq, L, S), dtype=query.dtype, device=query.device)
+    p = _lib.BwdParams()
+    p.grad_out, p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (go, q, k, v, o))
+    p.lse = lse.data_ptr()
+    p.grad_q, p.grad_k, p.grad_v = (_lib.tensor4(t) for t in (dq, dk, dv))
+    p.bias, p.bias_dtype, p.grad_bias = _lib.tensor4(bias), bias_dt, _lib.tensor4(dbias)
+    if kv_lens is not None:
+        kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
+        p.kv_lens = kv_lens.data_ptr()
+    if dropout_p > 0.0:
+        if dropout_keep is None:
+            raise ValueError("dropout_p > 0 needs dropout_keep")
+        dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
+        p.dropout_keep = dropout_keep.data_ptr()
+    p.dropout_p = float(dropout_p)
+    p.dtype = _lib.dtype_id(query.dtype)
+    p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
+    lib = _lib.load()
+    nbytes = lib.mi355_sdpa_bwd_workspace_bytes(C.byref(p))
+    ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=query.device)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+    with torch.cuda.device(query.device):
+        rc = lib.mi355_sdpa_bwd(C.byref(p), _lib.current_stream(query.device))
+    _lib.check(rc)
+    return dq, dk, dv, dbias
+
+
+def decode_fp8kv(query, k_fp8, v_fp8, k_scale, v_scale, kv_lens=None, scale=None,
+                 num_splits=0, need_lse=True):
+    """Decode-step attention over an fp8 e4m3 K/V cache.  Returns ``(out, lse)``."""
+    for t, n in ((query, "query"), (k_fp8, "key"), (v_fp8, "value")):
+        _require_cuda(t, n)
+    if k_fp8.dtype != torch.float8_e4m3fn or v_fp8.dtype != torch.float8_e4m3fn:
+        raise RuntimeError("decode_fp8kv: key and value must be float8_e4m3fn")
+    B, Hq, Lq, D = query.shape
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    q, k, v = _unit_last(query), _unit_last(k_fp8), _unit_last(v_fp8)
+    out = torch.empty((B, Hq, Lq, v.shape[3]), dtype=query.dtype, device=query.device)
+    lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=query.device) if need_lse else None
+    ks = k_scale.to(device=query.device, dtype=torch.float32).contiguous()
+    vs = v_scale.to(device=query.device, dtype=torch.float32).contiguous()
+    p = _lib.DecodeParams()
+    p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (q, k, v, out))
+    p.k_scale, p.v_scale = ks.data_ptr(), vs.data_ptr()
+    if kv_lens is not None:
+        kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
+        p.kv_lens = kv_lens.data_ptr()
+    p.lse = lse.data_ptr() if lse is not None else None
+    p.q_dtype, p.scale, p.num_splits = _lib.dtype_id(query.dtype), float(scale), int(num_splits)
+    lib = _lib.load()
+    nbytes = lib.mi355_sdpa_decode_workspace_bytes(C.byref(p))
+    ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=query.device)
+    p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
+    with torch.cuda.device(query.device):
+        rc = lib.mi355_sdpa_decode_fp8kv(C.byref(p), _lib.current_stream(query.device))
+    _lib.check(rc)
+    return out, lse
