@@ -47,3 +47,11 @@ def tol_for(dtype, grads=False):
     if dtype is torch.float32:
         return 1e-5 if not grads else 5e-5
     return 5e-2 if grads else 2e-2
+
+
+def rel_err(a, b):
+    """Relative Frobenius error; guards against mistakes that hide under an absolute bound."""
+    a, b = a.double().cpu(), b.double().cpu()
+    finite = torch.isfinite(b)
+    den = b[finite].norm().item()
+    return (a[finite] - b[finite]).norm().item() / max(den, 1e-30)

@@ -1,0 +1,185 @@
+"""GPU parity of the backward kernels against the CPU oracle, through the C ABI."""
+
+import pytest
+import torch
+
+from helpers import max_abs, oracle_bwd, oracle_fwd, qkv, rel_err
+from oracle import sdpa_math as om
+
+pytestmark = pytest.mark.gpu
+
+GENERIC, MFMA = 1, 2
+
+
+@pytest.fixture(scope="module")
+def amd(gpu_device):
+    import torch_neuronx_amd as amd
+
+    return amd
+
+
+def _fwd_bwd(amd, dev, q, k, v, go, kernel, **kw):
+    qd, kd, vd, god = (t.to(dev) for t in (q, k, v, go))
+    out, lse = amd.sdpa_forward(qd, kd, vd, force_kernel=kernel, **kw)
+    dq, dk, dv, db = amd.sdpa_backward(god, qd, kd, vd, out, lse, force_kernel=kernel, **kw)
+    torch.cuda.synchronize()
+    return out, lse, dq, dk, dv, db
+
+
+def _reference(q, k, v, go, attn_mask=None, is_causal=False, scale=None):
+    ro, rl = oracle_fwd(q, k, v, attn_mask=attn_mask, is_causal=is_causal, scale=scale)
+    return (ro, rl) + tuple(oracle_bwd(go, q, k, v, ro, rl, attn_mask=attn_mask, is_causal=is_causal, scale=scale))
+
+
+BWD_SHAPES = [
+    # B, Hq, Hkv, L, S, E, causal
+    (1, 8, 8, 512, 512, 64, False),
+    (1, 24, 6, 512, 512, 64, False),
+    (1, 8, 1, 512, 512, 64, True),
+    (1, 2, 1, 577, 577, 64, True),
+    (2, 4, 2, 51, 51, 128, True),
+    (2, 4, 2, 13, 51, 128, True),
+    (2, 4, 2, 51, 13, 128, True),
+    (1, 4, 4, 128, 1024, 128, False),
+    (1, 4, 1, 200, 333, 128, True),
+    (1, 8, 2, 1024, 1024, 128, True),
+]
+
+
+@pytest.mark.parametrize("shape", BWD_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_backward_matrix(amd, gpu_device, shape, dtype):
+    B, Hq, Hkv, L, S, E, causal = shape
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 3 + S, with_do=True)
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, is_causal=causal)
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, is_causal=causal)
+    assert dk.shape == k.shape and dv.shape == v.shape and dq.dtype == dtype
+    assert max_abs(out, ro) <= 2e-2
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert max_abs(a, r) <= 5e-2, name
+        assert rel_err(a, r) <= 2e-2, name
+
+
+GEN_SHAPES = BWD_SHAPES[:7] + [
+    (1, 4, 4, 64, 64, 256, False),
+    (2, 8, 1, 12, 12, 16, False),
+    (2, 8, 2, 10, 10, 16, True),
+    (1, 4, 4, 6, 6, 12, False),
+    (1, 2, 2, 6, 10, 40, False),
+]
+
+
+@pytest.mark.parametrize("shape", GEN_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_generic_backward_matrix(amd, gpu_device, shape, dtype):
+    B, Hq, Hkv, L, S, E, causal = shape
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 11 + S, with_do=True)
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, GENERIC, is_causal=causal)
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, is_causal=causal)
+    tol = 5e-5 if dtype is torch.float32 else 5e-2
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert max_abs(a, r) <= tol * max(1.0, r.abs().max().item()), name
+        assert rel_err(a, r) <= (1e-5 if dtype is torch.float32 else 2e-2), name
+
+
+def test_config4_full_size_group_subset(amd, gpu_device):
+    # BASELINE config 4: B=2,Hq=32,Hkv=8,S=4096,D=128 bf16 causal fwd+bwd on the GPU at full
+    # size; the oracle checks two whole kv-head groups (4 query heads each) to stay in seconds.
+    q, k, v, go = qkv(2, 32, 8, 4096, 4096, 128, dtype=torch.bfloat16, seed=1004, with_do=True)
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, is_causal=True)
+    assert dq.shape == (2, 32, 4096, 128) and dk.shape == (2, 8, 4096, 128) and dv.shape == (2, 8, 4096, 128)
+    for b, hk in ((0, 0), (1, 7)):
+        hs = slice(hk * 4, hk * 4 + 4)
+        qq, kk, vv, gg = q[b : b + 1, hs], k[b : b + 1, hk : hk + 1], v[b : b + 1, hk : hk + 1], go[b : b + 1, hs]
+        ro, rl, rdq, rdk, rdv = _reference(qq, kk, vv, gg, is_causal=True)
+        assert max_abs(out[b : b + 1, hs], ro) <= 2e-2
+        assert max_abs(lse[b : b + 1, hs], rl) <= 2e-3
+        assert max_abs(dq[b : b + 1, hs], rdq) <= 5e-2
+        assert max_abs(dk[b : b + 1, hk : hk + 1], rdk) <= 5e-2
+        assert max_abs(dv[b : b + 1, hk : hk + 1], rdv) <= 5e-2
+        assert rel_err(dq[b : b + 1, hs], rdq) <= 2e-2
+        assert rel_err(dk[b : b + 1, hk : hk + 1], rdk) <= 2e-2
+        assert rel_err(dv[b : b + 1, hk : hk + 1], rdv) <= 2e-2
+    # size-independent property: with a causal mask the last key only meets the last query, so
+    # dV[last] = sum over the group of P[last,last] * dO[last]
+    p_last = torch.exp((q[:, :, -1].float() * k[:, :, -1].float().repeat_interleave(4, 1)).sum(-1) / 128**0.5
+                       - lse[:, :, -1].float().cpu())
+    expect = (p_last[..., None] * go[:, :, -1].float()).reshape(2, 8, 4, 128).sum(2)
+    assert max_abs(dv[:, :, -1], expect) <= 5e-2
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_backward_with_bias_and_grad_bias(amd, gpu_device, dtype):
+    B, H, L, S, E = 2, 4, 33, 47, 32
+    q, k, v, go = qkv(B, H, H, L, S, E, dtype=dtype, seed=31, with_do=True)
+    bias = torch.randn(B, H, L, S, generator=torch.Generator().manual_seed(2)).to(dtype)
+    dev = gpu_device
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), attn_bias=bias.to(dev))
+    dq, dk, dv, db = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse,
+                                       attn_bias=bias.to(dev), want_grad_bias=True)
+    # oracle with bias, head-expanded call of the reference-shaped backward
+    ro, rl = om.compute_attention(q.float(), k.float(), v.float(), bias.float(), None, E**-0.5, False, 0.0)
+    rdq, rdk, rdv, rdb = om.compute_attention_backward(go.float(), q.float(), k.float(), v.float(), bias.float(),
+                                                       None, ro, rl, E**-0.5, False, 0.0)
+    tol = 5e-5 if dtype is torch.float32 else 5e-2
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv), ("dbias", db, rdb)):
+        assert max_abs(a, r) <= tol * max(1.0, r.abs().max().item()), name
+
+
+def test_backward_fully_masked_rows(amd, gpu_device):
+    # reference: test_scaled_dot_product_attention.py:1067-1120
+    q, k, v, go = qkv(1, 4, 4, 32, 32, 32, dtype=torch.float32, seed=9, with_do=True)
+    mask = torch.ones(1, 1, 32, 32, dtype=torch.bool)
+    mask[:, :, :10, :] = False
+    dev = gpu_device
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), attn_bias=mask.to(dev))
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, attn_bias=mask.to(dev))
+    for g in (dq, dk, dv):
+        assert torch.isfinite(g).all()
+    assert torch.equal(dq[:, :, :10].cpu(), torch.zeros(1, 4, 10, 32))
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, attn_mask=mask)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= 5e-5
+
+
+def test_backward_with_dropout_mask(amd, gpu_device):
+    B, H, L, S, E = 1, 2, 17, 23, 16
+    q, k, v, go = qkv(B, H, H, L, S, E, dtype=torch.float32, seed=13, with_do=True)
+    keep = torch.rand(B, H, L, S, generator=torch.Generator().manual_seed(1)) >= 0.25
+    dev = gpu_device
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), dropout_p=0.25, dropout_keep=keep.to(dev))
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse,
+                                      dropout_p=0.25, dropout_keep=keep.to(dev))
+    ro, rl = om.compute_attention(q, k, v, None, keep, E**-0.5, False, 0.25)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(go, q, k, v, None, keep, ro, rl, E**-0.5, False, 0.25)
+    assert max_abs(out, ro) <= 1e-5
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= 5e-5
+
+
+def test_backward_kv_lens(amd, gpu_device):
+    q, k, v, go = qkv(3, 4, 2, 5, 64, 32, dtype=torch.float32, seed=4, with_do=True)
+    lens = torch.tensor([64, 1, 17], dtype=torch.int32)
+    dev = gpu_device
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), kv_lens=lens.to(dev))
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, kv_lens=lens.to(dev))
+    pad = (torch.arange(64)[None, :] < lens[:, None])[:, None, None, :]
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, attn_mask=pad)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= 5e-5
+
+
+@pytest.mark.parametrize("kernel", [GENERIC, MFMA])
+def test_backward_grad_layouts_follow_inputs(amd, gpu_device, kernel):
+    B, H, L, E = 2, 4, 130, 64
+    g = torch.Generator().manual_seed(21)
+    base = torch.randn(B, L, H, 3 * E, generator=g).to(torch.bfloat16).to(gpu_device)
+    q, k, v = (t.transpose(1, 2) for t in base.chunk(3, dim=-1))
+    go = torch.randn(B, L, H, E, generator=g).to(torch.bfloat16).to(gpu_device).transpose(1, 2)
+    out, lse = amd.sdpa_forward(q, k, v, is_causal=True, force_kernel=kernel)
+    dq, dk, dv, _ = amd.sdpa_backward(go, q, k, v, out, lse, is_causal=True, force_kernel=kernel)
+    expect = torch.empty(B, L, H, E).transpose(1, 2).stride()
+    assert dq.stride() == expect and dk.stride() == expect and dv.stride() == expect
+    ro, rl, rdq, rdk, rdv = _reference(q.cpu(), k.cpu(), v.cpu(), go.cpu(), is_causal=True)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= 5e-2

@@ -1,7 +1,457 @@
-// placeholder until the MFMA backward lands
-#include "common.h"
+// Flash-attention backward for gfx950 on the 32x32x16 bf16/f16 MFMA.  Three kernels, no
+// atomics, deterministic; P is recomputed from the saved log-sum-exp:
+//
+//   bwd_delta_kernel   delta_i = sum_d dO_id O_id  (float32).  This is the whole row term of
+//                      torch_neuronx/_sdpa_math.py:160-163: its two P-dependent parts cancel.
+//   bwd_dkdv_kernel    one workgroup per 128 keys of a (batch, kv head); loops over the query
+//                      heads of the group (the GQA sum of decompositions.py:2595-2598 happens
+//                      in registers) and over 64-row query tiles:
+//                        S = Q K^T, dP = dO V^T      (A = Q / dO tile from LDS, B = K / V in registers)
+//                        P = exp2(c S - lse), dS = P (dP - delta)
+//                        dV^T += dO^T P, dK^T += Q^T dS  (A = transposed tile from LDS, B = P / dS
+//                                                         packed straight from the accumulators)
+//   bwd_dq_kernel      one workgroup per 128 query rows; loops over 64-key tiles:
+//                        S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T
+//
+// In both main kernels the softmax statistics a lane needs are either per-lane scalars or four
+// consecutive floats, and no probability ever goes through LDS.  Row-major tiles are XOR
+// swizzled, transposed tiles are written with byte permutes (see mfma_common.h).  Math follows
+// _sdpa_math.py:98-176: everything accumulates in float32, rows with lse = -inf give zero
+// gradients, scale multiplies dQ and dK once at the end.
+#include "mfma_common.h"
+
 namespace mi355 {
-bool bwd_mfma_supported(const mi355_sdpa_bwd_params&, const char** why) { *why = "not built"; return false; }
-size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params&) { return 0; }
-int launch_bwd_mfma(const mi355_sdpa_bwd_params&, hipStream_t) { set_error("SDPA: MFMA backward not built"); return MI355_SDPA_ERR_UNSUPPORTED; }
+namespace {
+
+struct BwdM {
+  const void *go, *q, *k, *v, *out;
+  const float* lse;
+  void *gq, *gk, *gv;
+  float* delta;
+  int64_t go_sb, go_sh, go_sl, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl;
+  int64_t o_sb, o_sh, o_sl, gq_sb, gq_sh, gq_sl, gk_sb, gk_sh, gk_sl, gv_sb, gv_sh, gv_sl;
+  int B, Hq, Hkv, L, S;
+  int n_qt, n_kt;
+  int causal, xcd_map;
+  float scale;
+};
+
+template <typename T>
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
+  typedef __attribute__((ext_vector_type(8))) T v8;
+  const v8 x = __builtin_bit_cast(v8, a), y = __builtin_bit_cast(v8, b);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s = fmaf((float)x[i], (float)y[i], s);
+  return s;
 }
+
+template <typename T, int D>
+__global__ __launch_bounds__(256) void bwd_delta_kernel(BwdM p) {
+  constexpr int LPR = D / 8, RPB = 256 / LPR;
+  const int64_t row = (int64_t)blockIdx.x * RPB + threadIdx.x / LPR;
+  const int sub = threadIdx.x % LPR;
+  const int64_t rows = (int64_t)p.B * p.Hq * p.L;
+  float s = 0.f;
+  if (row < rows) {
+    const int i = (int)(row % p.L), h = (int)((row / p.L) % p.Hq), b = (int)(row / ((int64_t)p.L * p.Hq));
+    const uint16_t* g = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)i * p.go_sl + sub * 8;
+    const uint16_t* o = (const uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)i * p.o_sl + sub * 8;
+    s = dot8<T>(*(const u32x4*)g, *(const u32x4*)o);
+  }
+#pragma unroll
+  for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
+  if (row < rows && sub == 0) p.delta[row] = s;
+}
+
+// ================================================================================================
+template <typename T, int D>
+__global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
+  constexpr int BQ = 64, BK = 128;
+  constexpr int KS = D / 16, DB = D / 32, NCH = D / 8;
+  constexpr int TP = BQ + 8;            // pitch of the transposed tiles (elements)
+  constexpr int U = 16 * NCH;           // 4-row x 8-d units per tile
+  constexpr int NU = (2 * U) / 256;     // units per thread over the Q and dO tiles
+  __shared__ __attribute__((aligned(16))) uint16_t q_rm[2][BQ * D];
+  __shared__ __attribute__((aligned(16))) uint16_t do_rm[2][BQ * D];
+  __shared__ __attribute__((aligned(16))) uint16_t q_t[2][D * TP];
+  __shared__ __attribute__((aligned(16))) uint16_t do_t[2][D * TP];
+  __shared__ __attribute__((aligned(16))) float lse_s[2][BQ];
+  __shared__ __attribute__((aligned(16))) float dl_s[2][BQ];
+
+  const int streams = p.B * p.Hkv;
+  const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
+  const int st = blockIdx.x % streams;
+  const int b = st / p.Hkv, hk = st % p.Hkv;
+  const int rep = p.Hq / p.Hkv;
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, half = lane >> 5;
+  const int k0 = kt * BK, kw0 = k0 + wave * 32;
+  const int key = kw0 + col;
+
+  // K and V fragments of this lane's key: B operands of S = Q K^T and dP = dO V^T
+  u32x4 kf[KS], vf[KS];
+  {
+    const int kc = min(key, p.S - 1);
+    const uint16_t* kr = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl + half * 8;
+    const uint16_t* vr = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) kf[ks] = *(const u32x4*)(kr + ks * 16), vf[ks] = *(const u32x4*)(vr + ks * 16);
+  }
+
+  const int nqs = (p.L + BQ - 1) / BQ;
+  const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+  const int per_head = nqs - qs_begin;
+  const int n_items = rep * per_head;
+
+  u32x4 stage[NU][4];
+  float lse_r = 0.f, dl_r = 0.f;
+  auto item_head = [&](int it) { return hk * rep + it / per_head; };
+  auto item_q0 = [&](int it) { return (qs_begin + it % per_head) * BQ; };
+  auto load_item = [&](int it) {
+    const int h = item_head(it), q0 = item_q0(it);
+#pragma unroll
+    for (int n = 0; n < NU; ++n) {
+      const int u = tid + n * 256, tile = u / U, uu = u % U, g = uu & 15, dc = uu >> 4;
+      const uint16_t* base = tile ? (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh
+                                  : (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
+      const int64_t sl = tile ? p.go_sl : p.q_sl;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int r = min(q0 + 4 * g + i, p.L - 1);
+        stage[n][i] = *(const u32x4*)(base + (int64_t)r * sl + dc * 8);
+      }
+    }
+    if (tid < BQ) {
+      const int qi = q0 + tid;
+      const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + min(qi, p.L - 1);
+      const float l = p.lse[idx];
+      // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
+      lse_r = (qi < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
+      dl_r = qi < p.L ? p.delta[idx] : 0.f;
+    }
+  };
+  auto store_item = [&](int buf) {
+#pragma unroll
+    for (int n = 0; n < NU; ++n) {
+      const int u = tid + n * 256, tile = u / U, uu = u % U, g = uu & 15, dc = uu >> 4;
+      uint16_t* rm = tile ? do_rm[buf] : q_rm[buf];
+      uint16_t* tt = tile ? do_t[buf] : q_t[buf];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *(u32x4*)(&rm[rm_off<D>(4 * g + i, dc)]) = stage[n][i];
+      tr_store<TP>(tt, stage[n], g, dc * 8);
+    }
+    if (tid < BQ) lse_s[buf][tid] = lse_r, dl_s[buf][tid] = dl_r;
+  };
+
+  f32x16 dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(dkacc[i]), zero(dvacc[i]);
+  const float c = p.scale * kLog2eF;
+
+  if (n_items > 0) {
+    load_item(0);
+    store_item(0);
+    __syncthreads();
+    if (n_items > 1) load_item(1);
+  }
+  for (int it = 0; it < n_items; ++it) {
+    const int buf = it & 1;
+    const int q0 = item_q0(it);
+    const bool active = !p.causal || q0 + BQ - 1 >= kw0;
+    if (active) {
+      const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= p.S);
+      uint32_t pP[2][8], pS[2][8];
+#pragma unroll
+      for (int mq = 0; mq < 2; ++mq) {
+        f32x16 sacc, dpacc;
+        zero(sacc), zero(dpacc);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const u32x4 a = *(const u32x4*)(&q_rm[buf][rm_off<D>(mq * 32 + col, 2 * ks + half)]);
+          sacc = Mma<T>::run(a, kf[ks], sacc);
+          const u32x4 a2 = *(const u32x4*)(&do_rm[buf][rm_off<D>(mq * 32 + col, 2 * ks + half)]);
+          dpacc = Mma<T>::run(a2, vf[ks], dpacc);
+        }
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const f32x4 l4 = *(const f32x4*)(&lse_s[buf][mq * 32 + r4 * 8 + half * 4]);
+          const f32x4 d4 = *(const f32x4*)(&dl_s[buf][mq * 32 + r4 * 8 + half * 4]);
+          float pr[4], ds[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = r4 * 4 + e;
+            pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
+            if (edge) {
+              const int qi = q0 + mq * 32 + r4 * 8 + half * 4 + e;
+              if ((p.causal && key > qi) || key >= p.S) pr[e] = 0.f;
+            }
+            ds[e] = pr[e] * (dpacc[r] - d4[e]);
+          }
+          pP[mq][r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[mq][r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+          pS[mq][r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[mq][r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
+        }
+      }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int mq = ks >> 1, r0 = (ks & 1) * 4;
+        const u32x4 bP = {pP[mq][r0], pP[mq][r0 + 1], pP[mq][r0 + 2], pP[mq][r0 + 3]};
+        const u32x4 bS = {pS[mq][r0], pS[mq][r0 + 1], pS[mq][r0 + 2], pS[mq][r0 + 3]};
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const u32x4 a = *(const u32x4*)(&do_t[buf][(db * 32 + col) * TP + ks * 16 + half * 8]);
+          dvacc[db] = Mma<T>::run(a, bP, dvacc[db]);
+          const u32x4 a2 = *(const u32x4*)(&q_t[buf][(db * 32 + col) * TP + ks * 16 + half * 8]);
+          dkacc[db] = Mma<T>::run(a2, bS, dkacc[db]);
+        }
+      }
+    }
+    if (it + 1 < n_items) store_item(buf ^ 1);
+    __syncthreads();
+    if (it + 2 < n_items) load_item(it + 2);
+  }
+
+  if (key < p.S) {
+    uint16_t* gk = (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
+    uint16_t* gv = (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = Mma<T>::pack(dkacc[db][g * 4] * p.scale, dkacc[db][g * 4 + 1] * p.scale);
+        w[1] = Mma<T>::pack(dkacc[db][g * 4 + 2] * p.scale, dkacc[db][g * 4 + 3] * p.scale);
+        *(u32x2*)(gk + db * 32 + g * 8 + half * 4) = w;
+        w[0] = Mma<T>::pack(dvacc[db][g * 4], dvacc[db][g * 4 + 1]);
+        w[1] = Mma<T>::pack(dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]);
+        *(u32x2*)(gv + db * 32 + g * 8 + half * 4) = w;
+      }
+  }
+}
+
+// ================================================================================================
+template <typename T, int D>
+__global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
+  constexpr int BM = 128, BN = 64;
+  constexpr int KS = D / 16, DB = D / 32, NCH = D / 8;
+  constexpr int TP = BN + 8;
+  constexpr int U = 16 * NCH;               // K units (4 keys x 8 d)
+  constexpr int VLD = (BN * NCH) / 256;     // V chunks per thread
+  __shared__ __attribute__((aligned(16))) uint16_t k_rm[2][BN * D];
+  __shared__ __attribute__((aligned(16))) uint16_t v_rm[2][BN * D];
+  __shared__ __attribute__((aligned(16))) uint16_t k_t[2][D * TP];
+
+  int b, h, qt;
+  {
+    const int bid = blockIdx.x, rep = p.Hq / p.Hkv;
+    if (p.xcd_map) {
+      const int per_xcd = (p.B * p.Hkv) / 8, xcd = bid & 7;
+      int r = bid >> 3;
+      const int hg = r % rep;
+      r /= rep;
+      const int sl = r % per_xcd;
+      r /= per_xcd;
+      qt = p.n_qt - 1 - r;
+      const int stream = sl * 8 + xcd;
+      b = stream / p.Hkv, h = (stream % p.Hkv) * rep + hg;
+    } else {
+      const int heads = p.B * p.Hq;
+      qt = p.n_qt - 1 - bid / heads;
+      b = (bid % heads) / p.Hq, h = (bid % heads) % p.Hq;
+    }
+  }
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, half = lane >> 5;
+  const int q0 = qt * BM, qw0 = q0 + wave * 32, qrow = qw0 + col;
+  const int qc = min(qrow, p.L - 1);
+
+  u32x4 qf[KS], dof[KS];
+  {
+    const uint16_t* qr = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl + half * 8;
+    const uint16_t* gr = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16), dof[ks] = *(const u32x4*)(gr + ks * 16);
+  }
+  float lse2, dl;
+  {
+    const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc;
+    const float l = p.lse[idx];
+    lse2 = (qrow < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
+    dl = p.delta[idx];
+  }
+
+  int nt = (p.S + BN - 1) / BN;
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+
+  const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
+  const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
+  u32x4 kst[4], vst[VLD];
+  const int k_g = tid & 15, k_dc = tid >> 4;
+  const bool k_loader = tid < U;
+  const int v_ch = tid % NCH, v_r0 = tid / NCH;
+  auto load_tile = [&](int t) {
+    const int kv0 = t * BN;
+    if (k_loader) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        kst[i] = *(const u32x4*)(kp + (int64_t)min(kv0 + 4 * k_g + i, p.S - 1) * p.k_sl + k_dc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i)
+      vst[i] = *(const u32x4*)(vp + (int64_t)min(kv0 + v_r0 + i * (256 / NCH), p.S - 1) * p.v_sl + v_ch * 8);
+  };
+  auto store_tile = [&](int buf) {
+    if (k_loader) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) *(u32x4*)(&k_rm[buf][rm_off<D>(4 * k_g + i, k_dc)]) = kst[i];
+      tr_store<TP>(k_t[buf], kst, k_g, k_dc * 8);
+    }
+#pragma unroll
+    for (int i = 0; i < VLD; ++i) *(u32x4*)(&v_rm[buf][rm_off<D>(v_r0 + i * (256 / NCH), v_ch)]) = vst[i];
+  };
+
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(dqacc[i]);
+  const float c = p.scale * kLog2eF;
+
+  load_tile(0);
+  store_tile(0);
+  __syncthreads();
+  if (nt > 1) load_tile(1);
+  for (int t = 0; t < nt; ++t) {
+    const int buf = t & 1, kv0 = t * BN;
+    const bool active = !p.causal || kv0 <= qw0 + 31;
+    if (active) {
+      const bool edge = (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S);
+      const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+      uint32_t pS[2][8];
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+        f32x16 sacc, dpacc;
+        zero(sacc), zero(dpacc);
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+          const u32x4 a = *(const u32x4*)(&k_rm[buf][rm_off<D>(mb * 32 + col, 2 * ks + half)]);
+          sacc = Mma<T>::run(a, qf[ks], sacc);
+          const u32x4 a2 = *(const u32x4*)(&v_rm[buf][rm_off<D>(mb * 32 + col, 2 * ks + half)]);
+          dpacc = Mma<T>::run(a2, dof[ks], dpacc);
+        }
+#pragma unroll
+        for (int r = 0; r < 16; r += 2) {
+          float ds[2];
+#pragma unroll
+          for (int e = 0; e < 2; ++e) {
+            float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+            if (edge) {
+              const int kv = kv0 + mb * 32 + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
+              if (kv > lim) pr = 0.f;
+            }
+            ds[e] = pr * (dpacc[r + e] - dl);
+          }
+          pS[mb][r >> 1] = Mma<T>::pack(ds[0], ds[1]);
+        }
+      }
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) {
+        const int mb = ks >> 1, r0 = (ks & 1) * 4;
+        const u32x4 bS = {pS[mb][r0], pS[mb][r0 + 1], pS[mb][r0 + 2], pS[mb][r0 + 3]};
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+          const u32x4 a = *(const u32x4*)(&k_t[buf][(db * 32 + col) * TP + ks * 16 + half * 8]);
+          dqacc[db] = Mma<T>::run(a, bS, dqacc[db]);
+        }
+      }
+    }
+    if (t + 1 < nt) store_tile(buf ^ 1);
+    __syncthreads();
+    if (t + 2 < nt) load_tile(t + 2);
+  }
+
+  if (qrow < p.L) {
+    uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = Mma<T>::pack(dqacc[db][g * 4] * p.scale, dqacc[db][g * 4 + 1] * p.scale);
+        w[1] = Mma<T>::pack(dqacc[db][g * 4 + 2] * p.scale, dqacc[db][g * 4 + 3] * p.scale);
+        *(u32x2*)(gq + db * 32 + g * 8 + half * 4) = w;
+      }
+  }
+}
+
+template <typename T, int D>
+int launch_td(const BwdM& g, hipStream_t s) {
+  const int64_t rows = (int64_t)g.B * g.Hq * g.L;
+  constexpr int RPB = 256 / (D / 8);
+  hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, s, g);
+  int rc = check_launch("bwd_delta_kernel");
+  if (rc) return rc;
+  hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(256), 0, s, g);
+  rc = check_launch("bwd_dkdv_kernel");
+  if (rc) return rc;
+  hipLaunchKernelGGL((bwd_dq_kernel<T, D>), dim3((unsigned)(g.B * g.Hq * g.n_qt)), dim3(256), 0, s, g);
+  return check_launch("bwd_dq_kernel");
+}
+
+}  // namespace
+
+bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
+  *why = "";
+  const int64_t E = p.q.size[3], Dv = p.v.size[3];
+  if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
+  if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
+  if (p.bias.data || p.grad_bias.data) return *why = "attn_bias present", false;
+  if (p.kv_lens) return *why = "kv_lens present", false;
+  if (p.dropout_p > 0.f) return *why = "dropout", false;
+  if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
+  if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
+  const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
+  for (const mi355_sdpa_tensor* t : ts) {
+    if (t->stride[3] != 1) return *why = "head dim is not unit-stride", false;
+    if (((uintptr_t)t->data & 15) != 0) return *why = "pointer not 16-byte aligned", false;
+    for (int i = 0; i < 3; ++i)
+      if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
+  }
+  if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
+  return true;
+}
+
+size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p) {
+  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * sizeof(float);
+}
+
+int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
+  const char* why;
+  if (!bwd_mfma_supported(p, &why)) {
+    set_error("SDPA: MFMA backward kernel cannot take this call: %s", why);
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  BwdM g;
+  g.go = p.grad_out.data, g.q = p.q.data, g.k = p.k.data, g.v = p.v.data, g.out = p.out.data;
+  g.lse = p.lse, g.gq = p.grad_q.data, g.gk = p.grad_k.data, g.gv = p.grad_v.data;
+  g.delta = (float*)p.workspace;
+#define SET3(dst, src) g.dst##_sb = p.src.stride[0], g.dst##_sh = p.src.stride[1], g.dst##_sl = p.src.stride[2]
+  SET3(go, grad_out);
+  SET3(q, q);
+  SET3(k, k);
+  SET3(v, v);
+  SET3(o, out);
+  SET3(gq, grad_q);
+  SET3(gk, grad_k);
+  SET3(gv, grad_v);
+#undef SET3
+  g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Hkv = (int)p.k.size[1];
+  g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
+  g.n_qt = (g.L + 127) / 128, g.n_kt = (g.S + 127) / 128;
+  g.causal = p.is_causal, g.scale = p.scale;
+  g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
+  const int D = (int)p.q.size[3];
+  if (p.dtype == MI355_SDPA_BF16) return D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
+  return D == 128 ? launch_td<f16_t, 128>(g, s) : launch_td<f16_t, 64>(g, s);
+}
+
+}  // namespace mi355

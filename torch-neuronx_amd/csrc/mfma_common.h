@@ -1,0 +1,94 @@
+// Building blocks shared by the MFMA attention kernels (gfx950, 32x32x16 bf16/f16 MFMA).
+//
+// Operand convention used everywhere: a lane supplies 8 consecutive contraction elements of
+// row/column (lane % 32), taken from offset 8*(lane / 32) of each 16-wide contraction step.
+// In the 32x32 float32 accumulator, register r of a lane is row 8*(r/4) + 4*(lane/32) + r%4
+// and column lane % 32.  Because A and B use the same lane->contraction mapping, the
+// accumulator registers of one product, packed pairwise to 16 bit, ARE the B (or A) operand
+// of a following product that contracts over that product's rows - as long as the other
+// operand presents the rows in the order 8*(r/4) + 4*half + r%4.  Transposed LDS tiles below
+// are stored in that order.
+#pragma once
+
+#include "common.h"
+
+namespace mi355 {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(8))) _Float16 f16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16;
+typedef __attribute__((ext_vector_type(4))) float f32x4;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+
+constexpr float kLog2eF = 1.4426950408889634f;
+
+template <typename T>
+struct Mma;
+template <>
+struct Mma<bf16_t> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8_t, a),
+                                                   __builtin_bit_cast(bf16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) __bf16 v2;
+    v2 r = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, r);
+  }
+};
+template <>
+struct Mma<f16_t> {
+  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
+    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8_t, a),
+                                                  __builtin_bit_cast(f16x8_t, b), c, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 v2;
+    v2 r = {(_Float16)lo, (_Float16)hi};
+    return __builtin_bit_cast(uint32_t, r);
+  }
+};
+
+__device__ __forceinline__ void zero(f32x16& a) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) a[r] = 0.f;
+}
+
+// ---- row-major tile, XOR-swizzled instead of padded ------------------------------------------
+// A row is D 16-bit elements = D/8 chunks of 16 bytes.  Chunk c of row r lives at chunk
+// c ^ swz(r).  swz is a bijection of the low three row bits for fixed high bits (eight
+// consecutive rows reading the same chunk hit eight different 16-byte slots) and also of row
+// bits 2..4 for fixed bits 0..1 (writers that own rows 4g+i hit different slots too).
+__device__ __forceinline__ int swz(int r) {
+  return (r & 4) | ((((r >> 1) ^ (r >> 4)) & 1) << 1) | ((r ^ (r >> 3)) & 1);
+}
+template <int D>
+__device__ __forceinline__ int rm_off(int r, int chunk) {  // element offset in a row-major tile
+  return r * D + ((chunk ^ swz(r)) << 3);
+}
+
+// ---- transposed tile: [d][row], rows in groups of four ------------------------------------------
+// Within every 16 rows the 4-row groups are stored in the order 0,2,1,3, so the eight rows a
+// lane needs for one contraction step (4*half .. +3 and 8 + 4*half .. +3) are one 16-byte read.
+__device__ __forceinline__ int tr_pos(int g) {  // g = row / 4 -> position in 4-row units
+  return (g & ~3) | ((g & 1) << 1) | ((g >> 1) & 1);
+}
+// rows[i][c] = dword c (two consecutive d) of row 4g+i; writes d = d0 .. d0+7 for 4 rows
+template <int PITCH>
+__device__ __forceinline__ void tr_store(uint16_t* tile, const u32x4 rows[4], int g, int d0) {
+  const int pos = tr_pos(g) * 4;
+#pragma unroll
+  for (int c = 0; c < 4; ++c) {
+    const uint32_t a0 = rows[0][c], a1 = rows[1][c], a2 = rows[2][c], a3 = rows[3][c];
+    u32x2 even, odd;
+    even[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100);
+    even[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100);
+    odd[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302);
+    odd[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302);
+    *(u32x2*)(&tile[(d0 + 2 * c) * PITCH + pos]) = even;
+    *(u32x2*)(&tile[(d0 + 2 * c + 1) * PITCH + pos]) = odd;
+  }
+}
+
+}  // namespace mi355
