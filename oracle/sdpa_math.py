@@ -183,6 +183,15 @@ def _head_slices(hq: int, chunk: int):
         yield h0, min(hq, h0 + chunk)
 
 
+def _as_4d(mask):
+    """Masks broadcast from the right: pad leading dimensions up to (B, H, L, S)."""
+    if mask is None:
+        return None
+    while mask.dim() < 4:
+        mask = mask.unsqueeze(0)
+    return mask
+
+
 def _chunk_for(L: int, S: int, budget_bytes: int = 1 << 30) -> int:
     per_head = max(1, L * S * 4)
     return max(1, budget_bytes // per_head)
@@ -200,6 +209,7 @@ def sdpa_forward(query, key, value, attn_mask=None, is_causal=False, scale=None,
     if scale is None:
         scale = 1.0 / math.sqrt(query.shape[-1])
     chunk = head_chunk or _chunk_for(L, S)
+    attn_mask = _as_4d(attn_mask)
     out = torch.empty(B, Hq, L, value.shape[-1], dtype=query.dtype)
     lse = torch.empty(B, Hq, L, dtype=torch.float32)
     for b in range(B):
@@ -237,6 +247,7 @@ def sdpa_backward(
     if scale is None:
         scale = 1.0 / math.sqrt(E)
     chunk = head_chunk or _chunk_for(L, S)
+    attn_mask = _as_4d(attn_mask)
     res_dtype = torch.float32 if reduce_in_fp32 else query.dtype
     dq = torch.empty(B, Hq, L, E, dtype=res_dtype)
     dk = torch.zeros(B, Hkv, S, E, dtype=res_dtype)

@@ -1,0 +1,167 @@
+"""Fused scaled-dot-product attention entry points with the reference's operator surface.
+
+Mirrors, for GPU tensors, what the reference does for its device in
+``torch_neuronx/python_ops/scaled_dot_product_fused_attention.py`` (entry functions :458-508 and
+:710-781, output/grad layout rule :357-358 and :601-603) and in the boxed handlers of
+``torch_neuronx/csrc/core/dispatch/NeuronDispatcher.cpp:2370-2582`` (validation, float64 round
+trip, stride fix-up, ``grad_attn_bias = None`` without a bias).  The arithmetic is in the HIP
+kernels; there is no fallback to a math path here.
+"""
+
+from __future__ import annotations
+
+import math
+import os
+
+import torch
+
+from .. import _lib, ops
+
+
+def _mfma_enabled() -> bool:
+    """Kill switch for the MFMA kernels, the analogue of TORCH_NEURONX_ENABLE_NKI_SDPA
+    (torch_neuronx/neuron_dynamo_backend/decompositions.py:2183)."""
+    return os.environ.get("TORCH_NEURONX_AMD_ENABLE_MFMA_SDPA", "1").lower() not in ("0", "false", "off", "no")
+
+
+def _force_kernel() -> int:
+    return 0 if _mfma_enabled() else _lib.KERNEL_GENERIC
+
+
+def _check_device(query: torch.Tensor) -> None:
+    if query.device.type != "cuda":
+        raise ValueError(f"Expected a ROCm GPU device, got {query.device}")
+
+
+def _empty_rng(device):
+    # inert placeholders when no dropout is applied (reference: decompositions.py:2309-2311)
+    return (torch.empty((0,), dtype=torch.int32, device=device),
+            torch.empty((0,), dtype=torch.int32, device=device))
+
+
+def _dropout_keep(query, S, dropout_p):
+    """Keep-mask drawn on the device; it travels to the backward in the philox_seed slot, the
+    way the reference carries its mask (decompositions.py:2354-2356)."""
+    B, H, L, _ = query.shape
+    if dropout_p >= 1.0:
+        return torch.zeros((B, H, L, S), dtype=torch.uint8, device=query.device)
+    return (torch.rand((B, H, L, S), device=query.device) >= dropout_p).to(torch.uint8)
+
+
+def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale, need_lse=True):
+    _check_device(query)
+    if return_debug_mask:
+        raise NotImplementedError("Debug mask not supported in Neuron implementation.")
+    ops.validate(ops.make_desc(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale))
+    orig_dtype = query.dtype
+    if orig_dtype == torch.float64:  # computed as float32, result restored to the caller's dtype
+        query, key, value = query.float(), key.float(), value.float()
+        if attn_bias is not None and attn_bias.dtype == torch.float64:
+            attn_bias = attn_bias.float()
+    S = key.shape[2]
+    keep = None
+    if dropout_p > 0.0:
+        keep = _dropout_keep(query, S, dropout_p)
+        seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
+    else:
+        seed, offset = _empty_rng(query.device)
+    out, lse = ops.sdpa_forward(query, key, value, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
+                                dropout_p=dropout_p, dropout_keep=keep, need_lse=need_lse,
+                                force_kernel=_force_kernel())
+    if orig_dtype == torch.float64:
+        out = out.to(orig_dtype)
+    return out, lse, seed, offset
+
+
+def scaled_dot_product_fused_attention_overrideable(
+    query, key, value, attn_bias=None, dropout_p=0.0, is_causal=False, return_debug_mask=False, scale=None
+):
+    """``aten::_scaled_dot_product_fused_attention_overrideable``: returns the 9-tuple
+    ``(output, logsumexp, cum_seq_q, cum_seq_k, max_q, max_k, philox_seed, philox_offset,
+    debug_attn_mask)``.  ``logsumexp`` is always a real float32 ``(B,Hq,L)`` tensor."""
+    out, lse, seed, offset = _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale)
+    return out, lse, None, None, query.shape[2], key.shape[2], seed, offset, None
+
+
+def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p, is_causal, philox_seed,
+              scale, want_grad_bias):
+    _check_device(query)
+    orig_dtype = query.dtype
+    if orig_dtype == torch.float64:
+        grad_out, query, key, value, out = (t.float() for t in (grad_out, query, key, value, out))
+        if attn_bias is not None and attn_bias.dtype == torch.float64:
+            attn_bias = attn_bias.float()
+    if grad_out.dtype != query.dtype:
+        grad_out = grad_out.to(query.dtype)
+    keep = None
+    if dropout_p > 0.0:
+        if philox_seed is None or philox_seed.numel() <= 1:
+            dropout_p = 0.0  # a placeholder carries no mask: treated as absent (_sdpa_math.py:42-45)
+        else:
+            keep = philox_seed
+    dq, dk, dv, dbias = ops.sdpa_backward(
+        grad_out, query, key, value, out, logsumexp, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
+        dropout_p=dropout_p, dropout_keep=keep, want_grad_bias=want_grad_bias, force_kernel=_force_kernel())
+    if orig_dtype == torch.float64:
+        dq, dk, dv = dq.to(orig_dtype), dk.to(orig_dtype), dv.to(orig_dtype)
+        dbias = dbias.to(orig_dtype) if dbias is not None else None
+    return dq, dk, dv, dbias
+
+
+def scaled_dot_product_fused_attention_overrideable_backward(
+    grad_out, query, key, value, attn_bias, grad_input_mask, out, logsumexp, cum_seq_q, cum_seq_k,
+    max_q, max_k, dropout_p, is_causal, philox_seed, philox_offset, scale=None
+):
+    """``aten::_scaled_dot_product_fused_attention_overrideable_backward``: ``(dq, dk, dv, dbias)``;
+    ``dbias`` is ``None`` when there is no bias or its gradient is not asked for."""
+    want = attn_bias is not None and len(grad_input_mask) > 3 and bool(grad_input_mask[3])
+    return _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p, is_causal,
+                     philox_seed, scale, want)
+
+
+def scaled_dot_product_flash_attention(
+    query, key, value, dropout_p=0.0, is_causal=False, return_debug_mask=False, scale=None
+):
+    """``aten::_scaled_dot_product_flash_attention``: same 9-tuple, no bias argument."""
+    out, lse, seed, offset = _forward(query, key, value, None, dropout_p, is_causal, return_debug_mask, scale)
+    return out, lse, None, None, query.shape[2], key.shape[2], seed, offset, None
+
+
+def scaled_dot_product_flash_attention_backward(
+    grad_out, query, key, value, out, logsumexp, cum_seq_q, cum_seq_k, max_q, max_k, dropout_p, is_causal,
+    philox_seed, philox_offset, scale=None
+):
+    """``aten::_scaled_dot_product_flash_attention_backward``: ``(dq, dk, dv)``."""
+    return _backward(grad_out, query, key, value, None, out, logsumexp, dropout_p, is_causal,
+                     philox_seed, scale, False)[:3]
+
+
+def scaled_dot_product_efficient_attention(
+    query, key, value, attn_bias, compute_log_sumexp, dropout_p=0.0, is_causal=False, scale=None
+):
+    """``aten::_scaled_dot_product_efficient_attention``: ``(output, log_sumexp, philox_seed,
+    philox_offset)``; the bias-capable route ATen takes when a mask is present."""
+    out, lse, seed, offset = _forward(query, key, value, attn_bias, dropout_p, is_causal, False, scale)
+    if not compute_log_sumexp:
+        lse = torch.empty((query.shape[0], query.shape[1], 0), dtype=torch.float32, device=query.device)
+    return out, lse, seed, offset
+
+
+def scaled_dot_product_efficient_attention_backward(
+    grad_out_, query, key, value, attn_bias, out, logsumexp, philox_seed, philox_offset, dropout_p,
+    grad_input_mask, is_causal=False, scale=None
+):
+    """``aten::_scaled_dot_product_efficient_attention_backward``: ``(dq, dk, dv, dbias)``."""
+    want = attn_bias is not None and len(grad_input_mask) > 3 and bool(grad_input_mask[3])
+    dq, dk, dv, dbias = _backward(grad_out_, query, key, value, attn_bias, out, logsumexp, dropout_p,
+                                  is_causal, philox_seed, scale, want)
+    if dbias is None:
+        dbias = torch.empty((0,), dtype=query.dtype, device=query.device)
+    return dq, dk, dv, dbias
+
+
+def fused_sdp_choice(query, key, value, attn_mask=None, dropout_p=0.0, is_causal=False, scale=None,
+                     enable_gqa=False) -> int:
+    """``aten::_fused_sdp_choice`` for GPU tensors: the rules of
+    ``torch_neuronx/csrc/aten/SdpBackendSelection.cpp:14-68`` evaluated in the C library."""
+    return ops.choose_backend(ops.make_desc(query, key, value, attn_mask, dropout_p, is_causal, False, scale))
