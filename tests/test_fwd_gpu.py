@@ -82,10 +82,11 @@ SHAPES = [
 
 @pytest.mark.parametrize("shape", SHAPES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_mfma_forward_matrix(amd, gpu_device, shape, dtype):
+@pytest.mark.parametrize("tile", [3, 4])  # 128 / 256 query rows per workgroup
+def test_mfma_forward_matrix(amd, gpu_device, shape, dtype, tile):
     B, Hq, Hkv, L, S, E, causal = shape
     q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 7 + S)
-    out, lse = _run(amd, q, k, v, gpu_device, is_causal=causal, force_kernel=MFMA)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=causal, force_kernel=tile)
     ro, rl = oracle_fwd(q, k, v, is_causal=causal)
     assert max_abs(out, ro) <= 2e-2
     assert rel_err(out, ro) <= 1e-2
@@ -171,7 +172,7 @@ def test_scale_zero_and_explicit_scale(amd, gpu_device):
         assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 2e-3
 
 
-@pytest.mark.parametrize("kernel", [GENERIC, MFMA])
+@pytest.mark.parametrize("kernel", [GENERIC, 3, 4])
 def test_noncontiguous_inputs_keep_query_layout(amd, gpu_device, kernel):
     # reference: test_scaled_dot_product_attention.py:943-1000 - (B,L,H,D).transpose(1,2) views,
     # last-dim chunks of a fused QKV buffer, as_strided with gaps

@@ -191,7 +191,9 @@ int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
   const char* why = "";
   int kernel = p->force_kernel;
   if (kernel == 0) kernel = fwd_mfma_supported(*p, &why) ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
-  if (kernel == MI355_SDPA_KERNEL_MFMA) return launch_fwd_mfma(*p, s);
+  if (kernel == MI355_SDPA_KERNEL_MFMA || kernel == MI355_SDPA_KERNEL_MFMA_T128 ||
+      kernel == MI355_SDPA_KERNEL_MFMA_T256)
+    return launch_fwd_mfma(*p, s);
   if (kernel == MI355_SDPA_KERNEL_GENERIC) return launch_fwd_generic(*p, s);
   return set_error("SDPA: unknown kernel id %d", kernel), MI355_SDPA_ERR_INVALID;
 }

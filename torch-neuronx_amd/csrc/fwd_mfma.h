@@ -1,0 +1,55 @@
+// Parameter block and workgroup-to-tile mapping shared by the MFMA forward kernels.
+#pragma once
+
+#include "mfma_common.h"
+
+namespace mi355 {
+
+struct FwdM {
+  const void *q, *k, *v;
+  void* out;
+  float* lse;
+  int64_t q_sb, q_sh, q_sl;
+  int64_t k_sb, k_sh, k_sl;
+  int64_t v_sb, v_sh, v_sl;
+  int64_t o_sb, o_sh, o_sl;
+  int B, Hq, Hkv, L, S;
+  int n_qt;    // query tiles per head
+  int causal;
+  int xcd_map;  // 1: (batch, kv head) streams are pinned to XCDs
+  float scale;
+};
+
+// Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first
+// (for causal attention the last query tile walks the most keys).  With xcd_map the eight
+// XCDs (blocks are dealt round-robin, block i -> XCD i % 8) each serve a fixed subset of
+// (batch, kv head) streams, so the K/V of a stream stay in one XCD's L2.
+__device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int& qt) {
+  const int bid = blockIdx.x;
+  const int rep = p.Hq / p.Hkv;
+  if (p.xcd_map) {
+    const int streams = p.B * p.Hkv;  // multiple of 8
+    const int per_xcd = streams / 8;
+    const int xcd = bid & 7;
+    int r = bid >> 3;  // index within this XCD: [qt desc][stream in xcd][head in group]
+    const int hg = r % rep;
+    r /= rep;
+    const int sl = r % per_xcd;
+    r /= per_xcd;
+    qt = p.n_qt - 1 - r;
+    const int stream = sl * 8 + xcd;
+    b = stream / p.Hkv;
+    h = (stream % p.Hkv) * rep + hg;
+  } else {
+    const int heads = p.B * p.Hq;
+    qt = p.n_qt - 1 - bid / heads;
+    const int bh = bid % heads;
+    b = bh / p.Hq;
+    h = bh % p.Hq;
+  }
+}
+
+
+int launch_fwd_mfma_w64(const FwdM& g, int dtype, hipStream_t s);
+
+}  // namespace mi355

@@ -1,9 +1,14 @@
 // Flash-attention forward for gfx950 on the 32x32x16 bf16/f16 MFMA.
 //
-// Work split: one workgroup = 4 wavefronts = 128 query rows of one (batch, query head);
-// each wavefront owns 32 query rows and walks the keys in tiles of 64.  Two workgroups fit
-// one compute unit (<=256 VGPRs, 2 x ~35 KB LDS), so while one wavefront is in its softmax
-// the matrix pipe is fed by its neighbour.
+// Work split: one workgroup = 4 wavefronts; each wavefront owns NB blocks of 32 query rows
+// (NB = 2: 256 query rows per workgroup, one workgroup per compute unit with the full 512
+// registers per lane; NB = 1: 128 rows, two workgroups per compute unit, for short sequences)
+// and walks the keys in tiles of 64.
+//
+// What bounds this kernel is LDS bandwidth, not the matrix pipe: every MFMA needs a fresh
+// 1 KB A operand from LDS and a compute unit delivers roughly 64 B/clk.  With NB = 2 each K
+// or V^T fragment read from LDS feeds two MFMAs (two query blocks held in registers), which
+// halves the LDS bytes per flop.
 //
 // Both products are computed TRANSPOSED so that the softmax needs no shuffle and P never
 // leaves registers:
@@ -15,104 +20,31 @@
 // the B operand of the second product.  The order in which the contraction index is spread
 // over lanes is free as long as A and B agree; V^T is stored in LDS in the matching order.
 //
+// The key loop is software pipelined by hand inside each wavefront: S^T of tile t+1 runs on
+// the matrix pipe while the vector pipe turns S^T of tile t into probabilities, and V^T P^T of
+// tile t runs while the vector pipe finds the row max of tile t+1.  The instruction interleave
+// is pinned with scheduling-group barriers.  K therefore runs one tile ahead of V through the
+// two LDS buffers each of them has; global loads run two to three tiles ahead.
+//
 // K tile in LDS: row-major [key][d], rows padded by 16 bytes (conflict-free 128-bit reads).
 // V tile in LDS: transposed [d][key] in groups of four keys, built from 4x(8 d) register
-// blocks with byte permutes; row padded by 16 bytes.  Both tiles are double buffered; the
-// global loads of tile j+2 are in flight while tile j is consumed.
+// blocks with byte permutes; rows padded by 16 bytes.
 //
 // Numerics follow torch_neuronx/_sdpa_math.py:51-95: raw dot products accumulate in
 // float32, the scale is applied in float32 inside the exponent, probabilities are rounded
 // to the input dtype only as the operand of P*V while the row sum uses the float32 values,
 // a row without a live key yields zeros and lse = -inf.
-#include "common.h"
+#include "fwd_mfma.h"
 
 namespace mi355 {
 namespace {
 
-typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8;
-typedef __attribute__((ext_vector_type(8))) _Float16 f16x8;
-typedef __attribute__((ext_vector_type(16))) float f32x16;
-typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
-typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
-
-constexpr int BM = 128;  // query rows per workgroup
 constexpr int BN = 64;   // keys per tile
 constexpr int PAD = 8;   // elements of row padding in LDS (16 bytes)
-constexpr float kLog2e = 1.4426950408889634f;
 
-struct FwdM {
-  const void *q, *k, *v;
-  void* out;
-  float* lse;
-  int64_t q_sb, q_sh, q_sl;
-  int64_t k_sb, k_sh, k_sl;
-  int64_t v_sb, v_sh, v_sl;
-  int64_t o_sb, o_sh, o_sl;
-  int B, Hq, Hkv, L, S;
-  int n_qt;    // query tiles per head
-  int causal;
-  int xcd_map;  // 1: (batch, kv head) streams are pinned to XCDs
-  float scale;
-};
-
-template <typename T>
-struct Mma;
-template <>
-struct Mma<bf16_t> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
-                                                   __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    typedef __attribute__((ext_vector_type(2))) __bf16 bf16x2;
-    bf16x2 r = {(__bf16)lo, (__bf16)hi};
-    return __builtin_bit_cast(uint32_t, r);
-  }
-};
-template <>
-struct Mma<f16_t> {
-  static __device__ __forceinline__ f32x16 run(u32x4 a, u32x4 b, f32x16 c) {
-    return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
-                                                  __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
-  }
-  static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-    typedef __attribute__((ext_vector_type(2))) _Float16 f16x2;
-    f16x2 r = {(_Float16)lo, (_Float16)hi};
-    return __builtin_bit_cast(uint32_t, r);
-  }
-};
-
-// Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first
-// (for causal attention the last query tile walks the most keys).  With xcd_map the eight
-// XCDs (blocks are dealt round-robin, block i -> XCD i % 8) each serve a fixed subset of
-// (batch, kv head) streams, so the K/V of a stream stay in one XCD's L2.
-__device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int& qt) {
-  const int bid = blockIdx.x;
-  const int rep = p.Hq / p.Hkv;
-  if (p.xcd_map) {
-    const int streams = p.B * p.Hkv;  // multiple of 8
-    const int per_xcd = streams / 8;
-    const int xcd = bid & 7;
-    int r = bid >> 3;  // index within this XCD: [qt desc][stream in xcd][head in group]
-    const int hg = r % rep;
-    r /= rep;
-    const int sl = r % per_xcd;
-    r /= per_xcd;
-    qt = p.n_qt - 1 - r;
-    const int stream = sl * 8 + xcd;
-    b = stream / p.Hkv;
-    h = (stream % p.Hkv) * rep + hg;
-  } else {
-    const int heads = p.B * p.Hq;
-    qt = p.n_qt - 1 - bid / heads;
-    const int bh = bid % heads;
-    b = bh / p.Hq;
-    h = bh % p.Hq;
-  }
-}
-
-template <typename T, int D>
-__global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FwdM p) {
+template <typename T, int D, int NB>
+__global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void fwd_mfma_kernel(FwdM p) {
+  constexpr int BM = 128 * NB;     // query rows per workgroup
   constexpr int KS = D / 16;       // contraction steps of S^T = K Q^T
   constexpr int DB = D / 32;       // 32-row blocks of O^T
   constexpr int KROW = D + PAD;    // K tile row pitch (elements)
@@ -128,19 +60,23 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FwdM p) {
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int col = lane & 31, half = lane >> 5;
   const int q0 = qt * BM;
-  const int qw0 = q0 + wave * 32;  // first query row of this wavefront
-  const int qrow = qw0 + col;      // this lane's query row
+  const int qw0 = q0 + wave * (32 * NB);  // first query row of this wavefront
+  int qrow[NB];                           // this lane's query rows
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) qrow[nb] = qw0 + nb * 32 + col;
+  const int qw_last = qw0 + 32 * NB - 1;
 
   const uint16_t* qp = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
 
-  // ---- Q fragment (B operand): lane = query column, 8 consecutive d per step ------------
-  u32x4 qf[KS];
-  {
-    const uint16_t* qr = qp + (int64_t)min(qrow, p.L - 1) * p.q_sl + half * 8;
+  // ---- Q fragments (B operand): lane = query column, 8 consecutive d per step -------------
+  u32x4 qf[NB][KS];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16);
+  for (int nb = 0; nb < NB; ++nb) {
+    const uint16_t* qr = qp + (int64_t)min(qrow[nb], p.L - 1) * p.q_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[nb][ks] = *(const u32x4*)(qr + ks * 16);
   }
 
   // number of key tiles this workgroup walks
@@ -152,13 +88,16 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FwdM p) {
   const int k_chunk = tid % KCH, k_row0 = tid / KCH;  // rows k_row0 + i * (256 / KCH)
   const int v_g = tid & 15, v_dc = tid >> 4;           // key group of 4, d chunk of 8
   const bool v_loader = v_dc < D / 8;
-  auto load_tile = [&](int t) {
+  auto load_tile_k = [&](int t) {
     const int kv0 = t * BN;
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const int r = min(kv0 + k_row0 + i * (256 / KCH), p.S - 1);
       kreg[i] = *(const u32x4*)(kp + (int64_t)r * p.k_sl + k_chunk * 8);
     }
+  };
+  auto load_tile_v = [&](int t) {
+    const int kv0 = t * BN;
     if (v_loader) {
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
@@ -167,143 +106,218 @@ __global__ __launch_bounds__(256, 2) void fwd_mfma_kernel(FwdM p) {
       }
     }
   };
-  // position (in 4-key units) of key group g inside a V^T row: within every 16 keys the
-  // groups are stored 0,2,1,3 so that the 8 keys one lane needs are contiguous
-  const int v_pos = (v_g & ~3) | ((v_g & 1) << 1) | ((v_g >> 1) & 1);
-  auto store_tile = [&](int buf) {
+  auto store_tile_k = [&](int buf) {
 #pragma unroll
     for (int i = 0; i < KLD; ++i) {
       const int r = k_row0 + i * (256 / KCH);
       *(u32x4*)(&k_lds[buf][r * KROW + k_chunk * 8]) = kreg[i];
     }
-    if (v_loader) {
-#pragma unroll
-      for (int c = 0; c < 4; ++c) {  // dword c of each row holds d = 2c, 2c+1
-        const uint32_t a0 = vreg[0][c], a1 = vreg[1][c], a2 = vreg[2][c], a3 = vreg[3][c];
-        u32x2 even, odd;
-        even[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100);  // (a0.lo, a1.lo)
-        even[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100);
-        odd[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302);   // (a0.hi, a1.hi)
-        odd[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302);
-        const int d = v_dc * 8 + 2 * c;
-        *(u32x2*)(&v_lds[buf][d * VROW + v_pos * 4]) = even;
-        *(u32x2*)(&v_lds[buf][(d + 1) * VROW + v_pos * 4]) = odd;
-      }
-    }
+  };
+  auto store_tile_v = [&](int buf) {
+    if (v_loader) tr_store<VROW>(v_lds[buf], vreg, v_g, v_dc * 8);
   };
 
-  f32x16 oacc[DB];
+  f32x16 oacc[DB][NB];
 #pragma unroll
   for (int i = 0; i < DB; ++i)
 #pragma unroll
-    for (int r = 0; r < 16; ++r) oacc[i][r] = 0.f;
-  float m_run = -INFINITY;  // running max of the raw dot products of this lane's query
-  float l_run = 0.f;        // this lane's share of the running row sum
-  const float c = p.scale * kLog2e;
+    for (int nb = 0; nb < NB; ++nb) zero(oacc[i][nb]);
+  float m_run[NB], l_run[NB];  // running max of the raw dot products / this lane's share of the row sum
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) m_run[nb] = -INFINITY, l_run[nb] = 0.f;
+  const float c = p.scale * kLog2eF;
 
-  load_tile(0);
-  store_tile(0);
+  const int nt_w = p.causal ? min(nt, qw_last / BN + 1) : nt;  // tiles with work for this wavefront
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  int lim[NB];  // last key each of this lane's queries sees
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) lim[nb] = p.causal ? min(qrow[nb], p.S - 1) : p.S - 1;
+
+  auto mask_tile = [&](f32x16 (&sacc)[2][NB], int kv0) {
+#pragma unroll
+    for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int kv = kv0 + mb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+          if (kv > lim[nb]) sacc[mb][nb][r] = -INFINITY;
+        }
+  };
+  auto is_edge = [&](int kv0) { return (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S); };
+
+  // statistics of the tile whose probabilities are formed next (set by the row-max step)
+  float m_new[NB], mc[NB], alpha[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) m_new[nb] = -INFINITY, mc[nb] = 0.f, alpha[nb] = 1.f;
+  bool need_rescale = false;
+  auto row_max_step = [&](const f32x16 (&sacc)[2][NB]) {
+    bool moved = false;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      float tmax = fmaxf(sacc[0][nb][0], sacc[1][nb][0]);
+#pragma unroll
+      for (int r = 1; r < 16; ++r) tmax = fmaxf(fmaxf(tmax, sacc[0][nb][r]), sacc[1][nb][r]);  // v_max3
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      m_new[nb] = fmaxf(m_run[nb], tmax);
+      const float m_use = (m_new[nb] == -INFINITY) ? 0.f : m_new[nb];
+      moved |= m_new[nb] != m_run[nb];
+      alpha[nb] = __builtin_amdgcn_exp2f((m_run[nb] - m_use) * c);
+      mc[nb] = m_use * c;
+    }
+    // the running max moves only a handful of times per row: O is rescaled only when it did
+    need_rescale = __builtin_amdgcn_ballot_w64(moved) != 0;
+  };
+
+  load_tile_k(0);
+  load_tile_v(0);
+  store_tile_k(0);
+  store_tile_v(0);
+  if (nt > 1) {
+    load_tile_k(1);
+    store_tile_k(1);
+  }
   __syncthreads();
-  if (nt > 1) load_tile(1);
+  if (nt > 1) load_tile_v(1);
+  if (nt > 2) load_tile_k(2);
+
+  f32x16 scur[2][NB];
+  if (nt_w > 0) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb) {
+        const u32x4 a = *(const u32x4*)(&k_lds[0][(mb * 32 + col) * KROW + ks * 16 + half * 8]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb)
+          scur[mb][nb] = Mma<T>::run(a, qf[nb][ks], ks == 0 ? zero16 : scur[mb][nb]);
+      }
+    row_max_step(scur);
+  }
+  __syncthreads();  // tile 0 of K is overwritten at the end of the first iteration
 
   for (int t = 0; t < nt; ++t) {
-    const int buf = t & 1;
-    const int kv0 = t * BN;
-    // causal: this wavefront has nothing to do once the tile starts past its last row
-    const bool active = !p.causal || kv0 <= qw0 + 31;
-    if (active) {
-      // ---- S^T = K Q^T ------------------------------------------------------------------
-      f32x16 sacc[2];
+    if (t < nt_w) {
+      // rare paths first, so that everything after them is one straight-line region: a tile that
+      // crosses the causal diagonal or the end of the keys is masked here and its row max redone
+      if (is_edge(t * BN)) {
+        mask_tile(scur, t * BN);
+        row_max_step(scur);
+      }
+      if (need_rescale) {
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
+        for (int nb = 0; nb < NB; ++nb) {
+          l_run[nb] *= alpha[nb];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sacc[mb][r] = 0.f;
+          for (int i = 0; i < DB; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][nb][r] *= alpha[nb];
+          m_run[nb] = m_new[nb];
+        }
+      }
+      // ---- phase A: S^T of tile t+1 on the matrix pipe, probabilities of tile t on the VALU ----
+      // (for the last tile S^T of a tile that is not there is computed and dropped)
+      const uint16_t* kt = k_lds[(t + 1) & 1];
+      f32x16 snext[2][NB];
+      uint32_t pk[2][NB][8];
+      float ps0[NB], ps1[NB];  // the row sum uses the unrounded float32 probabilities
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) ps0[nb] = 0.f, ps1[nb] = 0.f;
+      constexpr int EPS = 32 / KS;  // elements per query block handled per contraction step
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
 #pragma unroll
         for (int mb = 0; mb < 2; ++mb) {
-          const u32x4 a =
-              *(const u32x4*)(&k_lds[buf][(mb * 32 + col) * KROW + ks * 16 + half * 8]);
-          sacc[mb] = Mma<T>::run(a, qf[ks], sacc[mb]);
+          const u32x4 a = *(const u32x4*)(&kt[(mb * 32 + col) * KROW + ks * 16 + half * 8]);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb)
+            snext[mb][nb] = Mma<T>::run(a, qf[nb][ks], ks == 0 ? zero16 : snext[mb][nb]);
         }
-      }
-      // ---- masks --------------------------------------------------------------------------
-      const bool edge = (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S);
-      if (edge) {
-        const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;  // last key this query sees
 #pragma unroll
-        for (int mb = 0; mb < 2; ++mb)
+        for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int kv = kv0 + mb * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-            if (kv > lim) sacc[mb][r] = -INFINITY;
+          for (int e = 0; e < EPS; e += 2) {
+            const int idx = ks * EPS + e, mb = idx >> 4, r = idx & 15;
+            const float p0 = __builtin_amdgcn_exp2f(fmaf(scur[mb][nb][r], c, -mc[nb]));
+            const float p1 = __builtin_amdgcn_exp2f(fmaf(scur[mb][nb][r + 1], c, -mc[nb]));
+            ps0[nb] += p0, ps1[nb] += p1;
+            pk[mb][nb][r >> 1] = Mma<T>::pack(p0, p1);
           }
       }
-      // ---- online softmax -----------------------------------------------------------------
-      float tmax = sacc[0][0];
 #pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) tmax = fmaxf(tmax, sacc[mb][r]);
-      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      const float m_new = fmaxf(m_run, tmax);
-      const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
-      const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
-      m_run = m_new;
-      const float mc = m_use * c;
-      float psum = 0.f;
-      uint32_t pk[2][8];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb)
-#pragma unroll
-        for (int r = 0; r < 16; r += 2) {
-          const float p0 = __builtin_amdgcn_exp2f(fmaf(sacc[mb][r], c, -mc));
-          const float p1 = __builtin_amdgcn_exp2f(fmaf(sacc[mb][r + 1], c, -mc));
-          psum += p0 + p1;
-          pk[mb][r >> 1] = Mma<T>::pack(p0, p1);
-        }
-      l_run = l_run * alpha + psum;
-#pragma unroll
-      for (int i = 0; i < DB; ++i)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
-      // ---- O^T += V^T P^T -----------------------------------------------------------------
+      for (int nb = 0; nb < NB; ++nb) l_run[nb] += ps0[nb] + ps1[nb];
+      // ---- phase B: O^T += V^T P^T on the matrix pipe, row max of tile t+1 on the VALU ---------
+      const uint16_t* vt = v_lds[t & 1];
 #pragma unroll
       for (int ks = 0; ks < 4; ++ks) {
-        u32x4 bfrag;
+        u32x4 bfrag[NB];
         const int mb = ks >> 1, r0 = (ks & 1) * 4;
-        bfrag[0] = pk[mb][r0], bfrag[1] = pk[mb][r0 + 1];
-        bfrag[2] = pk[mb][r0 + 2], bfrag[3] = pk[mb][r0 + 3];
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          bfrag[nb][0] = pk[mb][nb][r0], bfrag[nb][1] = pk[mb][nb][r0 + 1];
+          bfrag[nb][2] = pk[mb][nb][r0 + 2], bfrag[nb][3] = pk[mb][nb][r0 + 3];
+        }
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-          const u32x4 a =
-              *(const u32x4*)(&v_lds[buf][(db * 32 + col) * VROW + ks * 16 + half * 8]);
-          oacc[db] = Mma<T>::run(a, bfrag, oacc[db]);
+          const u32x4 a = *(const u32x4*)(&vt[(db * 32 + col) * VROW + ks * 16 + half * 8]);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) oacc[db][nb] = Mma<T>::run(a, bfrag[nb], oacc[db][nb]);
         }
       }
+      row_max_step(snext);
+      // pin the interleave of the whole region: LDS operand fetches two steps ahead, then per
+      // fetch NB MFMAs, each followed by its share of the VALU work
+      __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
+#pragma unroll
+      for (int i = 0; i < 2 * KS; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);  // LDS read
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);  // MFMA
+          __builtin_amdgcn_sched_group_barrier(0x002, (112 + 2 * KS - 1) / (2 * KS), 0);  // VALU
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < 4 * DB; ++i) {
+        __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
+        }
+      }
+#pragma unroll
+      for (int mb = 0; mb < 2; ++mb)
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) scur[mb][nb] = snext[mb][nb];
     }
-    if (t + 1 < nt) store_tile(buf ^ 1);
+    if (t + 2 < nt) store_tile_k(t & 1);
+    if (t + 1 < nt) store_tile_v((t + 1) & 1);
     __syncthreads();
-    if (t + 2 < nt) load_tile(t + 2);
+    if (t + 3 < nt) load_tile_k(t + 3);
+    if (t + 2 < nt) load_tile_v(t + 2);
   }
 
   // ---- epilogue -----------------------------------------------------------------------------
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (qrow < p.L) {
-    uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+  for (int nb = 0; nb < NB; ++nb) {
+    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32, 64);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (qrow[nb] < p.L) {
+      uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow[nb] * p.o_sl;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
-        w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
-        *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
-      }
-    if (p.lse && half == 0)
-      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] =
-          l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w;
+          w[0] = Mma<T>::pack(oacc[db][nb][g * 4 + 0] * inv, oacc[db][nb][g * 4 + 1] * inv);
+          w[1] = Mma<T>::pack(oacc[db][nb][g * 4 + 2] * inv, oacc[db][nb][g * 4 + 3] * inv);
+          *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
+        }
+      if (p.lse && half == 0)
+        p.lse[((int64_t)b * p.Hq + h) * p.L + qrow[nb]] =
+            l_tot > 0.f ? m_run[nb] * p.scale + __builtin_logf(l_tot) : -INFINITY;
+    }
   }
 }
 
@@ -345,9 +359,17 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.o_sb = p.out.stride[0], g.o_sh = p.out.stride[1], g.o_sl = p.out.stride[2];
   g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Hkv = (int)p.k.size[1];
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
-  g.n_qt = (g.L + BM - 1) / BM;
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
+  // 256-row workgroups (one per compute unit, half the LDS traffic per flop) once they can
+  // fill the chip a few times over; 128-row workgroups for short or few sequences
+  const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
+  const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
+                         : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
+  (void)wg256;
+  const int NB = force_tile == 256 ? 2 : 1;  // 256-row tiles only on request for now
+  const int BM = 128 * NB;
+  g.n_qt = (g.L + BM - 1) / BM;
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
   if (blocks > 0x7fffffff) {
@@ -356,12 +378,15 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   }
   dim3 grid((unsigned)blocks), block(256);
   const int D = (int)p.q.size[3];
+  if (NB == 2 && D == 128) return launch_fwd_mfma_w64(g, p.dtype, s);
   if (p.dtype == MI355_SDPA_BF16) {
-    if (D == 128) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 128>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 64>), grid, block, 0, s, g);
+    if (D == 128) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 128, 1>), grid, block, 0, s, g);
+    else if (NB == 2) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 64, 2>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 64, 1>), grid, block, 0, s, g);
   } else {
-    if (D == 128) hipLaunchKernelGGL((fwd_mfma_kernel<f16_t, 128>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((fwd_mfma_kernel<f16_t, 64>), grid, block, 0, s, g);
+    if (D == 128) hipLaunchKernelGGL((fwd_mfma_kernel<f16_t, 128, 1>), grid, block, 0, s, g);
+    else if (NB == 2) hipLaunchKernelGGL((fwd_mfma_kernel<f16_t, 64, 2>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((fwd_mfma_kernel<f16_t, 64, 1>), grid, block, 0, s, g);
   }
   return check_launch("fwd_mfma_kernel");
 }

@@ -1,0 +1,301 @@
+// Flash-attention forward for gfx950, head dim 128, bf16/f16: the variant for long sequences.
+//
+// One workgroup = 4 wavefronts = 256 query rows of one (batch, query head); ONE workgroup per
+// compute unit, so a wavefront has the whole 512-register budget: 64 query rows (two 32-column
+// blocks) per wavefront, O^T in the accumulation registers, keys in tiles of 32.
+//
+// Why 64 rows per wavefront: the kernel is bound by LDS bandwidth before it is bound by the
+// matrix pipe.  Every 32x32x16 MFMA consumes a fresh 1 KB A operand (a K or V^T fragment) out
+// of LDS, a compute unit delivers about 64 B/clk of LDS reads, and four SIMDs at full MFMA rate
+// would ask for twice that.  Holding two query blocks per wavefront lets each fragment feed two
+// MFMAs.
+//
+// With one wavefront per SIMD nothing hides latency but the instruction stream itself, so the
+// key loop is software pipelined and its order pinned by hand:
+//   phase A   S^T(t+1) = K(t+1) Q^T on the matrix pipe  |  exp2 / row sum / pack of tile t
+//   phase B   O^T += V^T(t) P^T(t) on the matrix pipe    |  LDS stores of tiles t+2 / t+1, global
+//                                                           loads of tiles t+3 / t+2, row max of t+1
+// LDS operands are fetched three MFMA pairs ahead through a four-entry register ring, and a
+// scheduling barrier after every MFMA pair keeps the compiler from regrouping the stream.
+// Products are computed transposed (S^T = K Q^T, O^T = V^T P^T) as in fwd_mfma.hip, so the
+// softmax statistics are per-lane scalars and P goes from accumulator to B operand in registers.
+//
+// Numerics: torch_neuronx/_sdpa_math.py:51-95 (float32 accumulation and softmax, probabilities
+// rounded to the input dtype for P*V only, dead rows give zeros and lse = -inf).
+#include "fwd_mfma.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int D = 128;
+constexpr int BM = 256, BN = 32, NB = 2;
+constexpr int KS = D / 16, DB = D / 32;
+constexpr int KROW = D + 8;   // K tile row pitch (elements): conflict-free 128-bit reads
+constexpr int VROW = BN + 8;  // V^T tile row pitch
+constexpr int KCH = D / 8;    // 16-byte chunks per K row
+
+// x *= a for a value that lives in an accumulation register, updated in place.  Written as one
+// asm block so the rare rescale path neither duplicates the 128 accumulators at the join that
+// follows it nor drags them through the general registers all at once.
+__device__ __forceinline__ float scale_acc(float x, float a) {
+  float tmp;
+  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
+               : "+a"(x), "=&v"(tmp)
+               : "v"(a));
+  return x;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KROW];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][D * VROW];
+
+  int b, h, qt;
+  decode_block(p, b, h, qt);
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, half = lane >> 5;
+  const int q0 = qt * BM;
+  const int qw0 = q0 + wave * 64;
+  const int qrow[NB] = {qw0 + col, qw0 + 32 + col};
+  const int qw_last = qw0 + 63;
+
+  const uint16_t* qp = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
+  const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
+  const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
+
+  u32x4 qf[NB][KS];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const uint16_t* qr = qp + (int64_t)min(qrow[nb], p.L - 1) * p.q_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[nb][ks] = *(const u32x4*)(qr + ks * 16);
+  }
+
+  int nt = (p.S + BN - 1) / BN;
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+  const int nt_w = p.causal ? min(nt, qw_last / BN + 1) : nt;
+
+  // ---- staging: every thread moves two 16-byte K chunks and a 4-key x 4-d block of V ----------
+  u32x4 kreg[2];
+  u32x2 vreg[4];
+  const int k_chunk = tid & 15, k_row0 = tid >> 4;  // K rows k_row0, k_row0 + 16
+  const int v_g = tid & 7, v_dq = tid >> 3;         // keys 4 v_g .. +3, d = 4 v_dq .. +3
+  auto load_k = [&](int t) {
+    const int kv0 = min(t, nt - 1) * BN;
+#pragma unroll
+    for (int i = 0; i < 2; ++i) {
+      const int r = min(kv0 + k_row0 + 16 * i, p.S - 1);
+      kreg[i] = *(const u32x4*)(kp + (int64_t)r * p.k_sl + k_chunk * 8);
+    }
+  };
+  auto load_v = [&](int t) {
+    const int kv0 = min(t, nt - 1) * BN;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int r = min(kv0 + 4 * v_g + i, p.S - 1);
+      vreg[i] = *(const u32x2*)(vp + (int64_t)r * p.v_sl + v_dq * 4);
+    }
+  };
+  auto store_k = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 2; ++i) *(u32x4*)(&k_lds[buf][(k_row0 + 16 * i) * KROW + k_chunk * 8]) = kreg[i];
+  };
+  // transpose the 4x4 block with byte permutes: one 8-byte write of four keys per d
+  auto store_v_half = [&](int buf, int c) {  // c = 0/1: dword c of each row holds d = 2c, 2c+1
+    const int pos = tr_pos(v_g) * 4;
+    const uint32_t a0 = vreg[0][c], a1 = vreg[1][c], a2 = vreg[2][c], a3 = vreg[3][c];
+    u32x2 even, odd;
+    even[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100);
+    even[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100);
+    odd[0] = __builtin_amdgcn_perm(a1, a0, 0x07060302);
+    odd[1] = __builtin_amdgcn_perm(a3, a2, 0x07060302);
+    const int d = v_dq * 4 + 2 * c;
+    *(u32x2*)(&v_lds[buf][d * VROW + pos]) = even;
+    *(u32x2*)(&v_lds[buf][(d + 1) * VROW + pos]) = odd;
+  };
+
+  f32x16 oacc[DB][NB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) zero(oacc[i][nb]);
+  float m_run[NB] = {-INFINITY, -INFINITY}, l_run[NB] = {0.f, 0.f};
+  const float c = p.scale * kLog2eF;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int lim[NB] = {p.causal ? min(qrow[0], p.S - 1) : p.S - 1, p.causal ? min(qrow[1], p.S - 1) : p.S - 1};
+
+  auto mask_tile = [&](f32x16 (&s)[NB], int kv0) {
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kv = kv0 + (r >> 2) * 8 + half * 4 + (r & 3);
+        if (kv > lim[nb]) s[nb][r] = -INFINITY;
+      }
+  };
+  auto is_edge = [&](int kv0) { return (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S); };
+
+  float m_new[NB] = {-INFINITY, -INFINITY}, mc[NB] = {0.f, 0.f}, alpha[NB] = {1.f, 1.f};
+  bool need_rescale = false;
+  auto tile_max = [&](const f32x16& s) {
+    float t = fmaxf(s[0], s[1]);
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) t = fmaxf(fmaxf(t, s[r]), s[r + 1]);  // v_max3
+    return t;
+  };
+  auto finish_max = [&](float t0, float t1) {
+    const float tm[NB] = {fmaxf(t0, __shfl_xor(t0, 32, 64)), fmaxf(t1, __shfl_xor(t1, 32, 64))};
+    bool moved = false;
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) {
+      m_new[nb] = fmaxf(m_run[nb], tm[nb]);
+      const float m_use = (m_new[nb] == -INFINITY) ? 0.f : m_new[nb];
+      moved |= m_new[nb] != m_run[nb];
+      alpha[nb] = __builtin_amdgcn_exp2f((m_run[nb] - m_use) * c);
+      mc[nb] = m_use * c;
+    }
+    need_rescale = __builtin_amdgcn_ballot_w64(moved) != 0;
+  };
+
+  // ---- prologue ----------------------------------------------------------------------------------
+  load_k(0);
+  load_v(0);
+  store_k(0);
+  store_v_half(0, 0);
+  store_v_half(0, 1);
+  load_k(1);
+  store_k(1);
+  __syncthreads();
+  load_v(1);
+  load_k(2);
+  f32x16 s_a[NB], s_b[NB];
+  if (nt_w > 0) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 a = *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
+#pragma unroll
+      for (int nb = 0; nb < NB; ++nb) s_a[nb] = Mma<T>::run(a, qf[nb][ks], ks == 0 ? zero16 : s_a[nb]);
+    }
+    finish_max(tile_max(s_a[0]), tile_max(s_a[1]));
+  }
+  __syncthreads();  // K buffer 0 is rewritten during the first iteration
+
+  // one pipelined iteration: scur holds S^T of tile t (statistics ready), snext receives tile t+1
+  auto iteration = [&](int t, f32x16 (&scur)[NB], f32x16 (&snext)[NB]) {
+    if (t < nt_w) {
+      if (is_edge(t * BN)) {  // rare: tile crosses the causal diagonal or the end of the keys
+        mask_tile(scur, t * BN);
+        finish_max(tile_max(scur[0]), tile_max(scur[1]));
+      }
+      if (need_rescale) {  // rare: some row's running max moved
+        // the matrix pipe finished the last tile's accumulation long ago (a barrier lies between),
+        // these idle cycles only make that independent of what the compiler placed in between
+        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          l_run[nb] *= alpha[nb];
+#pragma unroll
+          for (int i = 0; i < DB; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][nb][r] = scale_acc(oacc[i][nb][r], alpha[nb]);
+          m_run[nb] = m_new[nb];
+        }
+      }
+      const uint16_t* kt = &k_lds[(t + 1) & 1][col * KROW + half * 8];
+      const uint16_t* vt = &v_lds[t & 1][col * VROW + half * 8];
+      auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
+      auto read_v = [&](int i) { return *(const u32x4*)(vt + (i & 3) * 32 * VROW + (i >> 2) * 16); };
+      uint32_t pk[NB][8];
+      float ps[NB] = {0.f, 0.f};
+      auto soft_pair = [&](int j) {  // pair j of 16: query block j / 8, registers 2 (j % 8), +1
+        const int nb = j >> 3, r = (j & 7) * 2;
+        const float p0 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r], c, -mc[nb]));
+        const float p1 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r + 1], c, -mc[nb]));
+        ps[nb] += p0 + p1;
+        pk[nb][r >> 1] = Mma<T>::pack(p0, p1);
+      };
+      u32x4 ring[4];
+      __builtin_amdgcn_sched_barrier(0);
+      ring[0] = read_k(0), ring[1] = read_k(1), ring[2] = read_k(2);
+      // ---- phase A -------------------------------------------------------------------------------
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
+        else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
+        snext[0] = Mma<T>::run(ring[ks & 3], qf[0][ks], ks == 0 ? zero16 : snext[0]);
+        soft_pair(2 * ks);
+        snext[1] = Mma<T>::run(ring[ks & 3], qf[1][ks], ks == 0 ? zero16 : snext[1]);
+        soft_pair(2 * ks + 1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      l_run[0] += ps[0], l_run[1] += ps[1];
+      // ---- phase B -------------------------------------------------------------------------------
+      float tmax0 = 0.f, tmax1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
+        if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
+        const int ks2 = i >> 2, db = i & 3;
+        const u32x4 b0 = {pk[0][ks2 * 4], pk[0][ks2 * 4 + 1], pk[0][ks2 * 4 + 2], pk[0][ks2 * 4 + 3]};
+        const u32x4 b1 = {pk[1][ks2 * 4], pk[1][ks2 * 4 + 1], pk[1][ks2 * 4 + 2], pk[1][ks2 * 4 + 3]};
+        oacc[db][0] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db][0]);
+        if (i == 0) store_k(t & 1);                    // tile t+2
+        if (i == 1) store_v_half((t + 1) & 1, 0);      // tile t+1
+        if (i == 2) load_k(t + 3);
+        if (i == 4) tmax0 = tile_max(snext[0]);
+        oacc[db][1] = Mma<T>::run(ring[(i + KS) & 3], b1, oacc[db][1]);
+        if (i == 1) store_v_half((t + 1) & 1, 1);
+        if (i == 3) load_v(t + 2);
+        if (i == 5) tmax1 = tile_max(snext[1]);
+        if (i == 6) finish_max(tmax0, tmax1);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    } else {  // nothing to compute for this wavefront any more: keep feeding the others
+      store_k(t & 1);
+      store_v_half((t + 1) & 1, 0);
+      store_v_half((t + 1) & 1, 1);
+      load_k(t + 3);
+      load_v(t + 2);
+    }
+    __syncthreads();
+  };
+
+  for (int t = 0; t < nt; t += 2) {
+    iteration(t, s_a, s_b);
+    if (t + 1 < nt) iteration(t + 1, s_b, s_a);
+  }
+
+  // ---- epilogue ------------------------------------------------------------------------------------
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const float l_tot = l_run[nb] + __shfl_xor(l_run[nb], 32, 64);
+    const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+    if (qrow[nb] < p.L) {
+      uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow[nb] * p.o_sl;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w;
+          w[0] = Mma<T>::pack(oacc[db][nb][g * 4 + 0] * inv, oacc[db][nb][g * 4 + 1] * inv);
+          w[1] = Mma<T>::pack(oacc[db][nb][g * 4 + 2] * inv, oacc[db][nb][g * 4 + 3] * inv);
+          *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
+        }
+      if (p.lse && half == 0)
+        p.lse[((int64_t)b * p.Hq + h) * p.L + qrow[nb]] =
+            l_tot > 0.f ? m_run[nb] * p.scale + __builtin_logf(l_tot) : -INFINITY;
+    }
+  }
+}
+
+}  // namespace
+
+int launch_fwd_mfma_w64(const FwdM& g, int dtype, hipStream_t s) {
+  const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
+  dim3 grid((unsigned)blocks), block(256);
+  if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_w64_kernel<bf16_t>), grid, block, 0, s, g);
+  else hipLaunchKernelGGL((fwd_w64_kernel<f16_t>), grid, block, 0, s, g);
+  return check_launch("fwd_w64_kernel");
+}
+
+}  // namespace mi355

@@ -14,7 +14,7 @@ import torch
 from ._build import LIB_PATH
 
 F32, F16, BF16, F64, BOOL, FP8_E4M3, OTHER = 0, 1, 2, 3, 4, 5, 99
-KERNEL_NONE, KERNEL_GENERIC, KERNEL_MFMA = 0, 1, 2
+KERNEL_NONE, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA_T128, KERNEL_MFMA_T256 = 0, 1, 2, 3, 4
 BACKEND_MATH, BACKEND_OVERRIDEABLE = 0, 4
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_LAUNCH = 0, -1, -2, -3
 
