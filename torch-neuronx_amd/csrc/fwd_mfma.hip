@@ -41,6 +41,7 @@ namespace {
 
 constexpr int BN = 64;   // keys per tile
 constexpr int PAD = 8;   // elements of row padding in LDS (16 bytes)
+constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
 template <typename T, int D, int NB>
 __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void fwd_mfma_kernel(FwdM p) {
@@ -159,9 +160,12 @@ __global__ __launch_bounds__(256, NB == 1 ? 2 : 1) void fwd_mfma_kernel(FwdM p) 
 #pragma unroll
       for (int r = 1; r < 16; ++r) tmax = fmaxf(fmaxf(tmax, sacc[0][nb][r]), sacc[1][nb][r]);  // v_max3
       tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-      m_new[nb] = fmaxf(m_run[nb], tmax);
+      // lazy reference max: raised only when a tile beats it by more than kLazy in the exponent,
+      // so O is rescaled a few times per row; probabilities stay below 2^kLazy (exact arithmetic)
+      const bool up = (tmax - m_run[nb]) * c > kLazy;  // false for NaN (-inf minus -inf)
+      m_new[nb] = up ? tmax : m_run[nb];
       const float m_use = (m_new[nb] == -INFINITY) ? 0.f : m_new[nb];
-      moved |= m_new[nb] != m_run[nb];
+      moved |= up;
       alpha[nb] = __builtin_amdgcn_exp2f((m_run[nb] - m_use) * c);
       mc[nb] = m_use * c;
     }

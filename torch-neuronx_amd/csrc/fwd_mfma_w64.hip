@@ -22,6 +22,8 @@
 //
 // Numerics: torch_neuronx/_sdpa_math.py:51-95 (float32 accumulation and softmax, probabilities
 // rounded to the input dtype for P*V only, dead rows give zeros and lse = -inf).
+#include <type_traits>
+
 #include "fwd_mfma.h"
 
 namespace mi355 {
@@ -33,17 +35,7 @@ constexpr int KS = D / 16, DB = D / 32;
 constexpr int KROW = D + 8;   // K tile row pitch (elements): conflict-free 128-bit reads
 constexpr int VROW = BN + 8;  // V^T tile row pitch
 constexpr int KCH = D / 8;    // 16-byte chunks per K row
-
-// x *= a for a value that lives in an accumulation register, updated in place.  Written as one
-// asm block so the rare rescale path neither duplicates the 128 accumulators at the join that
-// follows it nor drags them through the general registers all at once.
-__device__ __forceinline__ float scale_acc(float x, float a) {
-  float tmp;
-  asm volatile("v_accvgpr_read_b32 %1, %0\n\tv_mul_f32 %1, %1, %2\n\ts_nop 0\n\tv_accvgpr_write_b32 %0, %1"
-               : "+a"(x), "=&v"(tmp)
-               : "v"(a));
-  return x;
-}
+constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
 template <typename T>
 __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
@@ -77,34 +69,37 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   const int nt_w = p.causal ? min(nt, qw_last / BN + 1) : nt;
 
   // ---- staging: every thread moves two 16-byte K chunks and a 4-key x 4-d block of V ----------
-  u32x4 kreg[2];
-  u32x2 vreg[4];
+  // Two staging sets each: a tile is fetched from global memory two iterations before it is
+  // written to LDS, so a fetch has about two tile times to land.
+  u32x4 kreg[2][2];
+  u32x2 vreg[2][4];
   const int k_chunk = tid & 15, k_row0 = tid >> 4;  // K rows k_row0, k_row0 + 16
   const int v_g = tid & 7, v_dq = tid >> 3;         // keys 4 v_g .. +3, d = 4 v_dq .. +3
-  auto load_k = [&](int t) {
+  auto load_k = [&](int set, int t) {
     const int kv0 = min(t, nt - 1) * BN;
 #pragma unroll
     for (int i = 0; i < 2; ++i) {
       const int r = min(kv0 + k_row0 + 16 * i, p.S - 1);
-      kreg[i] = *(const u32x4*)(kp + (int64_t)r * p.k_sl + k_chunk * 8);
+      kreg[set][i] = *(const u32x4*)(kp + (int64_t)r * p.k_sl + k_chunk * 8);
     }
   };
-  auto load_v = [&](int t) {
+  auto load_v = [&](int set, int t) {
     const int kv0 = min(t, nt - 1) * BN;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const int r = min(kv0 + 4 * v_g + i, p.S - 1);
-      vreg[i] = *(const u32x2*)(vp + (int64_t)r * p.v_sl + v_dq * 4);
+      vreg[set][i] = *(const u32x2*)(vp + (int64_t)r * p.v_sl + v_dq * 4);
     }
   };
-  auto store_k = [&](int buf) {
+  auto store_k = [&](int set, int buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) *(u32x4*)(&k_lds[buf][(k_row0 + 16 * i) * KROW + k_chunk * 8]) = kreg[i];
+    for (int i = 0; i < 2; ++i)
+      *(u32x4*)(&k_lds[buf][(k_row0 + 16 * i) * KROW + k_chunk * 8]) = kreg[set][i];
   };
   // transpose the 4x4 block with byte permutes: one 8-byte write of four keys per d
-  auto store_v_half = [&](int buf, int c) {  // c = 0/1: dword c of each row holds d = 2c, 2c+1
+  auto store_v_half = [&](int set, int buf, int c) {  // dword c of each row holds d = 2c, 2c+1
     const int pos = tr_pos(v_g) * 4;
-    const uint32_t a0 = vreg[0][c], a1 = vreg[1][c], a2 = vreg[2][c], a3 = vreg[3][c];
+    const uint32_t a0 = vreg[set][0][c], a1 = vreg[set][1][c], a2 = vreg[set][2][c], a3 = vreg[set][3][c];
     u32x2 even, odd;
     even[0] = __builtin_amdgcn_perm(a1, a0, 0x05040100);
     even[1] = __builtin_amdgcn_perm(a3, a2, 0x05040100);
@@ -149,9 +144,14 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     bool moved = false;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      m_new[nb] = fmaxf(m_run[nb], tm[nb]);
+      // The reference max follows the true row max lazily: it is raised only when a tile beats it
+      // by more than kLazy in the exponent, so probabilities stay below 2^kLazy and the
+      // accumulator is rescaled a few times per row instead of once per tile.  Exact arithmetic:
+      // numerator and row sum carry the same reference.
+      const bool up = (tm[nb] - m_run[nb]) * c > kLazy;  // false for NaN (-inf minus -inf)
+      m_new[nb] = up ? tm[nb] : m_run[nb];
       const float m_use = (m_new[nb] == -INFINITY) ? 0.f : m_new[nb];
-      moved |= m_new[nb] != m_run[nb];
+      moved |= up;
       alpha[nb] = __builtin_amdgcn_exp2f((m_run[nb] - m_use) * c);
       mc[nb] = m_use * c;
     }
@@ -159,16 +159,18 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   };
 
   // ---- prologue ----------------------------------------------------------------------------------
-  load_k(0);
-  load_v(0);
-  store_k(0);
-  store_v_half(0, 0);
-  store_v_half(0, 1);
-  load_k(1);
-  store_k(1);
+  load_k(0, 0);
+  load_v(0, 0);
+  load_k(1, 1);
+  store_k(0, 0);
+  store_v_half(0, 0, 0);
+  store_v_half(0, 0, 1);
+  store_k(1, 1);
   __syncthreads();
-  load_v(1);
-  load_k(2);
+  load_k(0, 2);
+  load_k(1, 3);
+  load_v(1, 1);
+  load_v(0, 2);
   f32x16 s_a[NB], s_b[NB];
   if (nt_w > 0) {
 #pragma unroll
@@ -182,87 +184,107 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   __syncthreads();  // K buffer 0 is rewritten during the first iteration
 
   // one pipelined iteration: scur holds S^T of tile t (statistics ready), snext receives tile t+1
-  auto iteration = [&](int t, f32x16 (&scur)[NB], f32x16 (&snext)[NB]) {
-    if (t < nt_w) {
-      if (is_edge(t * BN)) {  // rare: tile crosses the causal diagonal or the end of the keys
-        mask_tile(scur, t * BN);
-        finish_max(tile_max(scur[0]), tile_max(scur[1]));
-      }
-      if (need_rescale) {  // rare: some row's running max moved
-        // the matrix pipe finished the last tile's accumulation long ago (a barrier lies between),
-        // these idle cycles only make that independent of what the compiler placed in between
-        asm volatile("s_nop 15\n\ts_nop 15" ::: "memory");
+  auto iteration = [&](int t, auto parity, f32x16 (&scur)[NB], f32x16 (&snext)[NB]) {
+    constexpr int par = decltype(parity)::value;  // t & 1, known at compile time
+    if (__builtin_expect(is_edge(t * BN), 0)) {  // rare: tile crosses the causal diagonal or the end of the keys
+      mask_tile(scur, t * BN);
+      finish_max(tile_max(scur[0]), tile_max(scur[1]));
+    }
+    if (__builtin_expect(need_rescale, 0)) {  // rare: some row's reference max moved
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-          l_run[nb] *= alpha[nb];
+      for (int nb = 0; nb < NB; ++nb) {
+        l_run[nb] *= alpha[nb];
 #pragma unroll
-          for (int i = 0; i < DB; ++i)
+        for (int i = 0; i < DB; ++i) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[i][nb][r] = scale_acc(oacc[i][nb][r], alpha[nb]);
-          m_run[nb] = m_new[nb];
+          for (int r = 0; r < 16; ++r) {
+            // read and write-back are pinned to accumulation registers one element at a time; left
+            // to itself the compiler drags all 128 accumulators through the general registers at
+            // once, which evicts the query fragments from them for the whole loop
+            float xv, y;
+            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(xv) : "a"(oacc[i][nb][r]));
+            y = xv * alpha[nb];
+            asm volatile("" : "+a"(y));
+            oacc[i][nb][r] = y;
+          }
+          __builtin_amdgcn_sched_barrier(0);  // one accumulator block at a time
         }
+        m_run[nb] = m_new[nb];
       }
-      const uint16_t* kt = &k_lds[(t + 1) & 1][col * KROW + half * 8];
-      const uint16_t* vt = &v_lds[t & 1][col * VROW + half * 8];
-      auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
-      auto read_v = [&](int i) { return *(const u32x4*)(vt + (i & 3) * 32 * VROW + (i >> 2) * 16); };
-      uint32_t pk[NB][8];
-      float ps[NB] = {0.f, 0.f};
-      auto soft_pair = [&](int j) {  // pair j of 16: query block j / 8, registers 2 (j % 8), +1
-        const int nb = j >> 3, r = (j & 7) * 2;
-        const float p0 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r], c, -mc[nb]));
-        const float p1 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r + 1], c, -mc[nb]));
-        ps[nb] += p0 + p1;
-        pk[nb][r >> 1] = Mma<T>::pack(p0, p1);
-      };
-      u32x4 ring[4];
+    }
+    const uint16_t* kt = &k_lds[par ^ 1][col * KROW + half * 8];
+    const uint16_t* vt = &v_lds[par][col * VROW + half * 8];
+    auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
+    auto read_v = [&](int i) { return *(const u32x4*)(vt + (i & 3) * 32 * VROW + (i >> 2) * 16); };
+    uint32_t pk[NB][8];
+    float ps[NB] = {0.f, 0.f};
+    auto soft_pair = [&](int j) {  // pair j of 16: query block j / 8, registers 2 (j % 8), +1
+      const int nb = j >> 3, r = (j & 7) * 2;
+      const float p0 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r], c, -mc[nb]));
+      const float p1 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r + 1], c, -mc[nb]));
+      ps[nb] += p0 + p1;
+      pk[nb][r >> 1] = Mma<T>::pack(p0, p1);
+    };
+    u32x4 ring[4];
+    __builtin_amdgcn_sched_barrier(0);
+    ring[0] = read_k(0), ring[1] = read_k(1), ring[2] = read_k(2);
+    // ---- phase A -------------------------------------------------------------------------------
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
+      else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
+      snext[0] = Mma<T>::run(ring[ks & 3], qf[0][ks], ks == 0 ? zero16 : snext[0]);
+      soft_pair(2 * ks);
+      snext[1] = Mma<T>::run(ring[ks & 3], qf[1][ks], ks == 0 ? zero16 : snext[1]);
+      soft_pair(2 * ks + 1);
       __builtin_amdgcn_sched_barrier(0);
-      ring[0] = read_k(0), ring[1] = read_k(1), ring[2] = read_k(2);
-      // ---- phase A -------------------------------------------------------------------------------
+    }
+    l_run[0] += ps[0], l_run[1] += ps[1];
+    // ---- phase B -------------------------------------------------------------------------------
+    float tmax0 = 0.f, tmax1 = 0.f;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
-        else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
-        snext[0] = Mma<T>::run(ring[ks & 3], qf[0][ks], ks == 0 ? zero16 : snext[0]);
-        soft_pair(2 * ks);
-        snext[1] = Mma<T>::run(ring[ks & 3], qf[1][ks], ks == 0 ? zero16 : snext[1]);
-        soft_pair(2 * ks + 1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-      l_run[0] += ps[0], l_run[1] += ps[1];
-      // ---- phase B -------------------------------------------------------------------------------
-      float tmax0 = 0.f, tmax1 = 0.f;
-#pragma unroll
-      for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
-        if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
-        const int ks2 = i >> 2, db = i & 3;
-        const u32x4 b0 = {pk[0][ks2 * 4], pk[0][ks2 * 4 + 1], pk[0][ks2 * 4 + 2], pk[0][ks2 * 4 + 3]};
-        const u32x4 b1 = {pk[1][ks2 * 4], pk[1][ks2 * 4 + 1], pk[1][ks2 * 4 + 2], pk[1][ks2 * 4 + 3]};
-        oacc[db][0] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db][0]);
-        if (i == 0) store_k(t & 1);                    // tile t+2
-        if (i == 1) store_v_half((t + 1) & 1, 0);      // tile t+1
-        if (i == 2) load_k(t + 3);
-        if (i == 4) tmax0 = tile_max(snext[0]);
-        oacc[db][1] = Mma<T>::run(ring[(i + KS) & 3], b1, oacc[db][1]);
-        if (i == 1) store_v_half((t + 1) & 1, 1);
-        if (i == 3) load_v(t + 2);
-        if (i == 5) tmax1 = tile_max(snext[1]);
-        if (i == 6) finish_max(tmax0, tmax1);
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    } else {  // nothing to compute for this wavefront any more: keep feeding the others
-      store_k(t & 1);
-      store_v_half((t + 1) & 1, 0);
-      store_v_half((t + 1) & 1, 1);
-      load_k(t + 3);
-      load_v(t + 2);
+    for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
+      if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
+      const int ks2 = i >> 2, db = i & 3;
+      const u32x4 b0 = {pk[0][ks2 * 4], pk[0][ks2 * 4 + 1], pk[0][ks2 * 4 + 2], pk[0][ks2 * 4 + 3]};
+      const u32x4 b1 = {pk[1][ks2 * 4], pk[1][ks2 * 4 + 1], pk[1][ks2 * 4 + 2], pk[1][ks2 * 4 + 3]};
+      oacc[db][0] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db][0]);
+      if (i == 0) store_k(par, par);                  // tile t+2
+      if (i == 1) store_v_half(par ^ 1, par ^ 1, 0);  // tile t+1
+      if (i == 2) load_k(par, t + 4);
+      if (i == 4) tmax0 = tile_max(snext[0]);
+      oacc[db][1] = Mma<T>::run(ring[(i + KS) & 3], b1, oacc[db][1]);
+      if (i == 1) store_v_half(par ^ 1, par ^ 1, 1);
+      if (i == 3) load_v(par ^ 1, t + 3);
+      if (i == 5) tmax1 = tile_max(snext[1]);
+      if (i == 6) finish_max(tmax0, tmax1);
+      __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
   };
+  // a wavefront whose rows lie above the causal diagonal of the remaining tiles only feeds LDS
+  auto idle_step = [&](int t, auto parity) {
+    constexpr int par = decltype(parity)::value;
+    store_k(par, par);
+    store_v_half(par ^ 1, par ^ 1, 0);
+    store_v_half(par ^ 1, par ^ 1, 1);
+    load_k(par, t + 4);
+    load_v(par ^ 1, t + 3);
+    __syncthreads();
+  };
 
-  for (int t = 0; t < nt; t += 2) {
-    iteration(t, s_a, s_b);
-    if (t + 1 < nt) iteration(t + 1, s_b, s_a);
+  int t = 0;
+  for (; t + 1 < nt_w; t += 2) {
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b);
+    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a);
+  }
+  if (t < nt_w) {  // odd count: t is even here
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b);
+    ++t;
+  }
+  for (; t < nt; ++t) {
+    if (t & 1) idle_step(t, std::integral_constant<int, 1>{});
+    else idle_step(t, std::integral_constant<int, 0>{});
   }
 
   // ---- epilogue ------------------------------------------------------------------------------------
