@@ -75,21 +75,23 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   u32x2 vreg[2][4];
   const int k_chunk = tid & 15, k_row0 = tid >> 4;  // K rows k_row0, k_row0 + 16
   const int v_g = tid & 7, v_dq = tid >> 3;         // keys 4 v_g .. +3, d = 4 v_dq .. +3
-  auto load_k = [&](int set, int t) {
-    const int kv0 = min(t, nt - 1) * BN;
+  // per-thread byte offsets inside a tile are fixed; the tile base is wave-uniform, so a load is
+  // one instruction with a scalar base and a 32-bit lane offset.  S is a multiple of BN here
+  // (the launcher guarantees it), so no row needs clamping.
+  uint32_t k_off[2], v_off[4];
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      const int r = min(kv0 + k_row0 + 16 * i, p.S - 1);
-      kreg[set][i] = *(const u32x4*)(kp + (int64_t)r * p.k_sl + k_chunk * 8);
-    }
+  for (int i = 0; i < 2; ++i) k_off[i] = (uint32_t)(((k_row0 + 16 * i) * p.k_sl + k_chunk * 8) * 2);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v_off[i] = (uint32_t)(((4 * v_g + i) * p.v_sl + v_dq * 4) * 2);
+  auto load_k = [&](int set, int t) {
+    const char* base = (const char*)(kp + (int64_t)(min(t, nt - 1) * BN) * p.k_sl);
+#pragma unroll
+    for (int i = 0; i < 2; ++i) kreg[set][i] = *(const u32x4*)(base + k_off[i]);
   };
   auto load_v = [&](int set, int t) {
-    const int kv0 = min(t, nt - 1) * BN;
+    const char* base = (const char*)(vp + (int64_t)(min(t, nt - 1) * BN) * p.v_sl);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int r = min(kv0 + 4 * v_g + i, p.S - 1);
-      vreg[set][i] = *(const u32x2*)(vp + (int64_t)r * p.v_sl + v_dq * 4);
-    }
+    for (int i = 0; i < 4; ++i) vreg[set][i] = *(const u32x2*)(base + v_off[i]);
   };
   auto store_k = [&](int set, int buf) {
 #pragma unroll
@@ -139,15 +141,15 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     for (int r = 2; r < 16; r += 2) t = fmaxf(fmaxf(t, s[r]), s[r + 1]);  // v_max3
     return t;
   };
-  auto finish_max = [&](float t0, float t1) {
-    const float tm[NB] = {fmaxf(t0, __shfl_xor(t0, 32, 64)), fmaxf(t1, __shfl_xor(t1, 32, 64))};
+  // The reference max follows the true row max lazily: it is raised only when a tile beats it by
+  // more than kLazy in the exponent, so probabilities stay below 2^kLazy and the accumulator is
+  // rescaled a few times per row instead of once per tile.  Exact arithmetic: numerator and row
+  // sum carry the same reference.
+  auto finish_max_x = [&](float t0, float t1, float x0, float x1) {  // x = the other half-wave's max
+    const float tm[NB] = {fmaxf(t0, x0), fmaxf(t1, x1)};
     bool moved = false;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
-      // The reference max follows the true row max lazily: it is raised only when a tile beats it
-      // by more than kLazy in the exponent, so probabilities stay below 2^kLazy and the
-      // accumulator is rescaled a few times per row instead of once per tile.  Exact arithmetic:
-      // numerator and row sum carry the same reference.
       const bool up = (tm[nb] - m_run[nb]) * c > kLazy;  // false for NaN (-inf minus -inf)
       m_new[nb] = up ? tm[nb] : m_run[nb];
       const float m_use = (m_new[nb] == -INFINITY) ? 0.f : m_new[nb];
@@ -156,6 +158,9 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
       mc[nb] = m_use * c;
     }
     need_rescale = __builtin_amdgcn_ballot_w64(moved) != 0;
+  };
+  auto finish_max = [&](float t0, float t1) {
+    finish_max_x(t0, t1, __shfl_xor(t0, 32, 64), __shfl_xor(t1, 32, 64));
   };
 
   // ---- prologue ----------------------------------------------------------------------------------
@@ -218,30 +223,57 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     auto read_v = [&](int i) { return *(const u32x4*)(vt + (i & 3) * 32 * VROW + (i >> 2) * 16); };
     uint32_t pk[NB][8];
     float ps[NB] = {0.f, 0.f};
-    auto soft_pair = [&](int j) {  // pair j of 16: query block j / 8, registers 2 (j % 8), +1
+    // The chain read S -> fma -> exp2 -> add/pack of one register pair is strictly dependent, and a
+    // wavefront issues in order, so the three stages of consecutive pairs are staggered by hand:
+    // a slot runs stage 1 of pair j+2, stage 2 of pair j+1 and stage 3 of pair j.
+    float xs[3][2], pv[2][2];
+    auto stage1 = [&](int j) {  // pair j of 16: query block j / 8, registers 2 (j % 8), +1
+      if (j >= 16) return;
       const int nb = j >> 3, r = (j & 7) * 2;
-      const float p0 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r], c, -mc[nb]));
-      const float p1 = __builtin_amdgcn_exp2f(fmaf(scur[nb][r + 1], c, -mc[nb]));
-      ps[nb] += p0 + p1;
-      pk[nb][r >> 1] = Mma<T>::pack(p0, p1);
+      xs[j % 3][0] = fmaf(scur[nb][r], c, -mc[nb]);
+      xs[j % 3][1] = fmaf(scur[nb][r + 1], c, -mc[nb]);
+    };
+    auto stage2 = [&](int j) {
+      if (j >= 16) return;
+      pv[j & 1][0] = __builtin_amdgcn_exp2f(xs[j % 3][0]);
+      pv[j & 1][1] = __builtin_amdgcn_exp2f(xs[j % 3][1]);
+    };
+    auto stage3 = [&](int j) {
+      if (j >= 16) return;
+      const int nb = j >> 3, r = (j & 7) * 2;
+      ps[nb] += pv[j & 1][0] + pv[j & 1][1];
+      pk[nb][r >> 1] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
     };
     u32x4 ring[4];
     __builtin_amdgcn_sched_barrier(0);
+    // the first operand fetches are in flight while the first probabilities are formed
     ring[0] = read_k(0), ring[1] = read_k(1), ring[2] = read_k(2);
+    stage1(0);
+    stage1(1);
+    stage2(0);
+    __builtin_amdgcn_sched_barrier(0);
     // ---- phase A -------------------------------------------------------------------------------
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
       else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
       snext[0] = Mma<T>::run(ring[ks & 3], qf[0][ks], ks == 0 ? zero16 : snext[0]);
-      soft_pair(2 * ks);
+      stage1(2 * ks + 2);
+      stage2(2 * ks + 1);
+      stage3(2 * ks);
       snext[1] = Mma<T>::run(ring[ks & 3], qf[1][ks], ks == 0 ? zero16 : snext[1]);
-      soft_pair(2 * ks + 1);
+      stage1(2 * ks + 3);
+      stage2(2 * ks + 2);
+      stage3(2 * ks + 1);
       __builtin_amdgcn_sched_barrier(0);
     }
     l_run[0] += ps[0], l_run[1] += ps[1];
     // ---- phase B -------------------------------------------------------------------------------
-    float tmax0 = 0.f, tmax1 = 0.f;
+    // VALU / memory work is dealt out slot by slot (two MFMAs per slot):
+    //   0-3  row max of tile t+1, four registers of each query block per slot; K store in slot 0
+    //   4    exchange of the half-wave maxima is issued      5    V transpose + store
+    //   6    global loads of the tiles two ahead, exchange consumed: new reference max
+    float tm0 = -INFINITY, tm1 = -INFINITY, x0 = 0.f, x1 = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
       if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
@@ -249,15 +281,26 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
       const u32x4 b0 = {pk[0][ks2 * 4], pk[0][ks2 * 4 + 1], pk[0][ks2 * 4 + 2], pk[0][ks2 * 4 + 3]};
       const u32x4 b1 = {pk[1][ks2 * 4], pk[1][ks2 * 4 + 1], pk[1][ks2 * 4 + 2], pk[1][ks2 * 4 + 3]};
       oacc[db][0] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db][0]);
-      if (i == 0) store_k(par, par);                  // tile t+2
-      if (i == 1) store_v_half(par ^ 1, par ^ 1, 0);  // tile t+1
-      if (i == 2) load_k(par, t + 4);
-      if (i == 4) tmax0 = tile_max(snext[0]);
+      if (i < 4) {
+        const int r = 4 * i;
+        tm0 = fmaxf(fmaxf(tm0, snext[0][r]), snext[0][r + 1]);
+        tm0 = fmaxf(fmaxf(tm0, snext[0][r + 2]), snext[0][r + 3]);
+      }
+      if (i == 0) store_k(par, par);  // tile t+2
+      if (i == 4) x0 = __shfl_xor(tm0, 32, 64), x1 = __shfl_xor(tm1, 32, 64);
+      if (i == 5) store_v_half(par ^ 1, par ^ 1, 0);  // tile t+1
+      if (i == 6) load_k(par, t + 4);
       oacc[db][1] = Mma<T>::run(ring[(i + KS) & 3], b1, oacc[db][1]);
-      if (i == 1) store_v_half(par ^ 1, par ^ 1, 1);
-      if (i == 3) load_v(par ^ 1, t + 3);
-      if (i == 5) tmax1 = tile_max(snext[1]);
-      if (i == 6) finish_max(tmax0, tmax1);
+      if (i < 4) {
+        const int r = 4 * i;
+        tm1 = fmaxf(fmaxf(tm1, snext[1][r]), snext[1][r + 1]);
+        tm1 = fmaxf(fmaxf(tm1, snext[1][r + 2]), snext[1][r + 3]);
+      }
+      if (i == 5) store_v_half(par ^ 1, par ^ 1, 1);
+      if (i == 6) {
+        load_v(par ^ 1, t + 3);
+        finish_max_x(tm0, tm1, x0, x1);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
