@@ -71,6 +71,40 @@ __device__ __forceinline__ uint32_t split_pair(float a, float b, int part) {
   return fp8x2(a, b);
 }
 
+// x + (x rotated right by N lanes inside each row of 16 lanes): one VALU op with a DPP modifier
+template <int N>
+__device__ __forceinline__ float add_row_ror(float x) {
+  const int r = __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, x), 0x120 | N, 0xf, 0xf, false);
+  return x + __builtin_bit_cast(float, r);
+}
+// sum over the split-term columns n, n+RS, ... of a 16-lane row (all lanes get the total)
+template <int PARTS>
+__device__ __forceinline__ float sum_parts(float x) {
+  if (PARTS == 3) x = add_row_ror<4>(x);
+  return add_row_ror<8>(x);
+}
+
+// 32 consecutive query elements as float, fetched with 16-byte loads
+template <typename TQ>
+__device__ __forceinline__ void load_q32(const TQ* p, float (&out)[32]) {
+  typedef __attribute__((ext_vector_type(8))) TQ v8;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const v8 v = *(const v8*)(p + 8 * i);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) out[8 * i + j] = (float)v[j];
+  }
+}
+template <>
+__device__ __forceinline__ void load_q32<float>(const float* p, float (&out)[32]) {
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const f32x4 v = *(const f32x4*)(p + 4 * i);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) out[4 * i + j] = v[j];
+  }
+}
+
 __device__ __forceinline__ long as_long(uint32_t lo, uint32_t hi) {
   return (long)(((uint64_t)hi << 32) | lo);
 }
@@ -81,7 +115,7 @@ struct KVRegs {
 };
 
 template <typename TQ, int PARTS>
-__global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
+__global__ __launch_bounds__(64 * kWaves, 3) void decode_kernel(DecP p) {
   constexpr int RS = PARTS == 3 ? 4 : 8;  // column stride between split terms
   __shared__ float s_o[kWaves][8][D];
   __shared__ float s_m[kWaves][8], s_l[kWaves][8];
@@ -100,33 +134,6 @@ __global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
   const bool col_live = r < p.R && part < PARTS;
   const int rr = min(r, p.R - 1);
   const int h = hk * rep + rr % rep, lq = rr / rep;
-
-  // ---- query fragment: B operand of S^T = K Q^T ------------------------------------------
-  // the lane owns d = 32g .. 32g+31 of row r; step ks consumes d = 32g + 8ks .. +7
-  float qv[32];
-  {
-    const TQ* qr = (const TQ*)p.q + b * p.q_sb + h * p.q_sh + lq * p.q_sl + 32 * g;
-#pragma unroll
-    for (int i = 0; i < 32; ++i) qv[i] = to_f32(qr[i]);
-  }
-  float amax = 0.f;
-#pragma unroll
-  for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qv[i]));
-  amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-  amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-  // power-of-two pre-scale so the row peaks in [120, 240]: well inside e4m3 and exact
-  const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
-  long qb[4];
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    uint32_t w[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      w[j] = col_live ? split_pair(qv[ks * 8 + 2 * j] * f, qv[ks * 8 + 2 * j + 1] * f, part) : 0u;
-    qb[ks] = as_long(w[0] | (w[1] << 16), w[2] | (w[3] << 16));
-  }
-  const float kscale = p.k_scale[b * p.Hkv + hk];
-  const float c_row = p.scale * kscale / f * kLog2e;  // raw dot -> log2-domain logit
 
   // ---- this wavefront's key range -----------------------------------------------------------
   const int wave_keys = p.chunk_keys / kWaves;
@@ -156,6 +163,32 @@ __global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
     }
   };
 
+  KVRegs ra, rb;
+  if (steps > 0) load(ra, 0);  // in flight while the query fragment is prepared
+
+  // ---- query fragment: B operand of S^T = K Q^T ------------------------------------------
+  // the lane owns d = 32g .. 32g+31 of row r; step ks consumes d = 32g + 8ks .. +7
+  float qv[32];
+  load_q32<TQ>((const TQ*)p.q + b * p.q_sb + h * p.q_sh + lq * p.q_sl + 32 * g, qv);
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qv[i]));
+  amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+  amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+  // power-of-two pre-scale so the row peaks in [120, 240]: well inside e4m3 and exact
+  const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
+  long qb[4];
+#pragma unroll
+  for (int ks = 0; ks < 4; ++ks) {
+    uint32_t w[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      w[j] = col_live ? split_pair(qv[ks * 8 + 2 * j] * f, qv[ks * 8 + 2 * j + 1] * f, part) : 0u;
+    qb[ks] = as_long(w[0] | (w[1] << 16), w[2] | (w[3] << 16));
+  }
+  const float kscale = p.k_scale[b * p.Hkv + hk];
+  const float c_row = p.scale * kscale / f * kLog2e;  // raw dot -> log2-domain logit
+
   f32x4 oacc[8];
 #pragma unroll
   for (int i = 0; i < 8; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
@@ -178,9 +211,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
     float t[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
-      float x = sacc[i >> 2][i & 3];
-      if (PARTS == 3) x += __shfl_xor(x, 4, 64);
-      x += __shfl_xor(x, 8, 64);
+      const float x = sum_parts<PARTS>(sacc[i >> 2][i & 3]);
       const int key = base + (i >> 2) * 16 + 4 * g + (i & 3);
       t[i] = key < w_end ? x * c_row : -INFINITY;
     }
@@ -232,8 +263,6 @@ __global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
     }
   };
 
-  KVRegs ra, rb;
-  if (steps > 0) load(ra, 0);
   for (int s = 0; s < steps; s += 2) {
     if (s + 1 < steps) load(rb, s + 1);
     compute(ra, s);
@@ -246,10 +275,7 @@ __global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
   for (int i = 0; i < 8; ++i)
 #pragma unroll
     for (int e = 0; e < 4; ++e) {
-      float x = oacc[i][e];
-      if (PARTS == 3) x += __shfl_xor(x, 4, 64);
-      x += __shfl_xor(x, 8, 64);
-      oacc[i][e] = x;
+      oacc[i][e] = sum_parts<PARTS>(oacc[i][e]);
     }
   float l_tot = l_run + __shfl_xor(l_run, 16, 64);
   l_tot += __shfl_xor(l_tot, 32, 64);
@@ -282,25 +308,38 @@ __global__ __launch_bounds__(64 * kWaves) void decode_kernel(DecP p) {
 }
 
 // Merge the chunk partials of one (batch, kv head, query row); 128 threads = 128 output columns.
+// The (max, sum) pairs of all chunks are fetched first (one per lane), so the weights are known
+// before the partial outputs stream in and the loads of the outputs are independent.
 template <typename TQ>
 __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
+  __shared__ float s_w[64];
   const int row = blockIdx.x % p.R;
   const int hk = (blockIdx.x / p.R) % p.Hkv;
   const int b = blockIdx.x / (p.R * p.Hkv);
   const int d = threadIdx.x;
   int len = p.S;
   if (p.kv_lens) len = min(p.S, max(0, p.kv_lens[b]));
-  const int nch = (len + p.chunk_keys - 1) / p.chunk_keys;
+  const int nch = (len + p.chunk_keys - 1) / p.chunk_keys;  // <= 64 (checked by the launcher)
   const int64_t slot0 = (int64_t)(b * p.Hkv + hk) * p.chunks * p.R + row;
-  float M = -INFINITY;
-  for (int c = 0; c < nch; ++c) M = fmaxf(M, p.ws_ml[(slot0 + (int64_t)c * p.R) * 2]);
-  float L = 0.f, O = 0.f;
-  for (int c = 0; c < nch; ++c) {
-    const int64_t s = slot0 + (int64_t)c * p.R;
-    const float sc = __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
-    L += p.ws_ml[s * 2 + 1] * sc;
-    O += p.ws_o[s * D + d] * sc;
+  float m = -INFINITY, l = 0.f;
+  if (d < nch) {
+    const int64_t s = slot0 + (int64_t)d * p.R;
+    m = p.ws_ml[s * 2], l = p.ws_ml[s * 2 + 1];
   }
+  float M = m;
+  if (d < 64) M = wave_max(M);
+  const float w = (d < nch) ? __builtin_amdgcn_exp2f(m - M) : 0.f;
+  float L = l * w;
+  if (d < 64) {
+    L = wave_sum(L);
+    s_w[d] = w;
+  }
+  __shared__ float s_ML[2];
+  if (d == 0) s_ML[0] = M, s_ML[1] = L;
+  __syncthreads();
+  M = s_ML[0], L = s_ML[1];
+  float O = 0.f;
+  for (int c = 0; c < nch; ++c) O = fmaf(p.ws_o[(slot0 + (int64_t)c * p.R) * D + d], s_w[c], O);
   const int rep = p.Hq / p.Hkv;
   const int h = hk * rep + row % rep, lq = row / rep;
   TQ* o = (TQ*)p.out + b * p.o_sb + h * p.o_sh + lq * p.o_sl;
@@ -311,10 +350,12 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
 
 int chunk_keys_for(const mi355_sdpa_decode_params& p) {
   const int S = (int)p.k.size[2];
-  int ck = 512;
+  int ck = 1024;
   if (p.num_splits > 0) ck = (S + p.num_splits - 1) / p.num_splits;
   ck = ((ck + 127) / 128) * 128;
-  return ck < 128 ? 128 : ck;
+  if (ck < 128) ck = 128;
+  while ((S + ck - 1) / ck > 64) ck *= 2;  // the merge step handles at most 64 chunks
+  return ck;
 }
 
 template <typename TQ>
@@ -367,6 +408,12 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
   g.o_sb = p.out.stride[0], g.o_sh = p.out.stride[1], g.o_sl = p.out.stride[2];
   g.chunk_keys = chunk_keys_for(p);
   g.chunks = (g.S + g.chunk_keys - 1) / g.chunk_keys;
+  if (g.chunks > 64)
+    return set_error("SDPA decode: at most 64 key chunks per sequence (got %d): lower num_splits", g.chunks),
+           MI355_SDPA_ERR_UNSUPPORTED;
+  const int64_t qes = p.q_dtype == MI355_SDPA_F32 ? 4 : 2;
+  if (((uintptr_t)p.q.data & 15) || (p.q.stride[0] * qes) % 16 || (p.q.stride[1] * qes) % 16 || (p.q.stride[2] * qes) % 16)
+    return set_error("SDPA decode: query rows must be 16-byte aligned"), MI355_SDPA_ERR_UNSUPPORTED;
   g.scale = p.scale;
   const int64_t slots = (int64_t)g.B * g.Hkv * g.chunks * g.R;
   g.ws_o = (float*)p.workspace;
