@@ -3,12 +3,11 @@
 // the hot path).  Defined as torch_neuronx/_sdpa_math.py:51-95 applied to the dequantised
 // cache with a key-padding bias; the reference itself has no fp8 attention path.
 //
-// Work split: grid = (key chunks, kv heads, batch); a workgroup of 4 wavefronts takes one
-// chunk of one (batch, kv head) and serves all R = Lq * Hq/Hkv query rows that share that kv
-// head, so every K/V byte is read from HBM exactly once.  Chunks at or past kv_lens[b] exit
-// at once: padding is never read.  Each wavefront walks its quarter of the chunk 32 keys at a
-// time with its own running max / sum / output, the four are merged through LDS, and a second
-// small kernel merges the chunks of a sequence.
+// Work split: the keys of a (batch, kv head) are cut into chunks; one wavefront takes a chunk and
+// serves all R = Lq * Hq/Hkv query rows that share that kv head, so every K/V byte is read from
+// HBM exactly once, and padding past kv_lens[b] is never read.  A wavefront walks its chunk 32
+// keys at a time with a running max / sum / output, writes the chunk's partial result, and a
+// second small kernel merges the chunks of a sequence.  Wavefronts are persistent (see below).
 //
 // Precision without dequantising the cache: the bf16 query row is scaled by a power of two
 // and split into up to three e4m3 terms (q = q0 + q1 + q2, exact to ~12 bits); the terms
@@ -18,6 +17,8 @@
 // Per 32 keys a lane loads 64 contiguous K bytes of one key (A operand of S^T = K Q^T, the
 // contraction order is permuted identically for Q) and eight 4-byte pieces of V which are
 // byte-transposed in registers into the A operand of O^T = V^T P^T.
+#include <algorithm>
+
 #include "common.h"
 
 namespace mi355 {
@@ -31,6 +32,10 @@ constexpr int D = 128;
 constexpr int kWaves = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
+#ifndef DEC_OCC
+#define DEC_OCC 2
+#endif
+constexpr int kDecOcc = DEC_OCC;  // wavefronts per SIMD the decode kernel is built for
 constexpr float kPScale = 256.f;  // probabilities are stored as e4m3 of 256*p
 
 struct DecP {
@@ -58,17 +63,23 @@ __device__ __forceinline__ f32x2 fp8x2_to_f32(uint32_t w) {
   return __builtin_amdgcn_cvt_pk_f32_fp8((int)w, false);
 }
 
-// e4m3 term `part` of the split x = t0 + t1 + t2 for a pair of values, as two packed bytes
-__device__ __forceinline__ uint32_t split_pair(float a, float b, int part) {
-  uint32_t w = fp8x2(a, b);
-  if (part == 0) return w;
-  f32x2 d = fp8x2_to_f32(w);
+// The split x = t0 + t1 + t2 into e4m3 terms for a pair of values; each lane keeps one term, picked
+// with the lane's masks (0xffff for its own term, 0 elsewhere; all 0 for a dead column).  Written
+// without branches: every lane computes all terms, which costs less than divergent control flow.
+struct PartMask { uint32_t m0, m1, m2; };
+template <int PARTS>
+__device__ __forceinline__ uint32_t split_pair(float a, float b, const PartMask& pm) {
+  const uint32_t w0 = fp8x2(a, b);
+  f32x2 d = fp8x2_to_f32(w0);
   a -= d[0], b -= d[1];
-  w = fp8x2(a, b);
-  if (part == 1) return w;
-  d = fp8x2_to_f32(w);
-  a -= d[0], b -= d[1];
-  return fp8x2(a, b);
+  const uint32_t w1 = fp8x2(a, b);
+  uint32_t w = (w0 & pm.m0) | (w1 & pm.m1);
+  if (PARTS == 3) {
+    d = fp8x2_to_f32(w1);
+    a -= d[0], b -= d[1];
+    w |= fp8x2(a, b) & pm.m2;
+  }
+  return w;
 }
 
 // x + (x rotated right by N lanes inside each row of 16 lanes): one VALU op with a DPP modifier
@@ -84,27 +95,6 @@ __device__ __forceinline__ float sum_parts(float x) {
   return add_row_ror<8>(x);
 }
 
-// 32 consecutive query elements as float, fetched with 16-byte loads
-template <typename TQ>
-__device__ __forceinline__ void load_q32(const TQ* p, float (&out)[32]) {
-  typedef __attribute__((ext_vector_type(8))) TQ v8;
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const v8 v = *(const v8*)(p + 8 * i);
-#pragma unroll
-    for (int j = 0; j < 8; ++j) out[8 * i + j] = (float)v[j];
-  }
-}
-template <>
-__device__ __forceinline__ void load_q32<float>(const float* p, float (&out)[32]) {
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const f32x4 v = *(const f32x4*)(p + 4 * i);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) out[4 * i + j] = v[j];
-  }
-}
-
 __device__ __forceinline__ long as_long(uint32_t lo, uint32_t hi) {
   return (long)(((uint64_t)hi << 32) | lo);
 }
@@ -114,196 +104,286 @@ struct KVRegs {
   uint32_t v[2][8];   // [64-wide half of d][key slot]
 };
 
+// One workgroup = one wavefront, launched once per wavefront slot of the chip and PERSISTENT:
+// wavefront w of W takes work items w, w + W, w + 2W, ...  An item is one chunk of chunk_keys keys
+// of one (batch, kv head), so all items cost the same but for the ragged last chunk of a
+// sequence, and the static deal balances the chip to within one item without atomics.  The item
+// list is never materialised: a wavefront prefix-sums the chunk counts of 64 batches at a time
+// across its lanes and finds the batch of an item with a ballot.
+// While an item streams, the query rows of the next one are already in flight (they wait in
+// registers), and its first K/V tile is requested before the epilogue of the current one, so the
+// memory pipe of a wavefront never drains between items.
 template <typename TQ, int PARTS>
-__global__ __launch_bounds__(64 * kWaves, 3) void decode_kernel(DecP p) {
+__global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   constexpr int RS = PARTS == 3 ? 4 : 8;  // column stride between split terms
-  __shared__ float s_o[kWaves][8][D];
-  __shared__ float s_m[kWaves][8], s_l[kWaves][8];
-
-  const int chunk = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
-  int len = p.S;
-  if (p.kv_lens) len = min(p.S, max(0, p.kv_lens[b]));
-  const int c_begin = chunk * p.chunk_keys;
-  if (c_begin >= len) return;  // whole workgroup: nothing but padding here
-  const int c_end = min(len, c_begin + p.chunk_keys);
-
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  constexpr int QV = sizeof(TQ) == 4 ? 8 : 4;  // 16-byte loads per 32 query elements
+  const int lane = threadIdx.x;
   const int n = lane & 15, g = lane >> 4;
   const int part = n / RS, r = n % RS;
   const int rep = p.Hq / p.Hkv;
   const bool col_live = r < p.R && part < PARTS;
+  const PartMask pm = {col_live && part == 0 ? 0xffffu : 0u, col_live && part == 1 ? 0xffffu : 0u,
+                       col_live && part == 2 ? 0xffffu : 0u};
   const int rr = min(r, p.R - 1);
-  const int h = hk * rep + rr % rep, lq = rr / rep;
+  const int hq_off = rr % rep, lq = rr / rep;
 
-  // ---- this wavefront's key range -----------------------------------------------------------
-  const int wave_keys = p.chunk_keys / kWaves;
-  const int w_begin = c_begin + wave * wave_keys;
-  const int w_end = min(c_end, w_begin + wave_keys);
-  const int steps = w_end > w_begin ? (w_end - w_begin + 31) / 32 : 0;
+  // ---- the item list ------------------------------------------------------------------------------
+  // Batch b owns cnt(b) = ceil(len_b / chunk_keys) chunks; items are numbered batch-major,
+  // then chunk, then kv head.  Lane i of a block of 64 batches holds cnt and its inclusive prefix;
+  // the batch of an item is the first lane whose prefix exceeds the item's chunk number.
+  auto block_counts = [&](int b0, int& len, int& cnt, int& incl) {
+    const int bb = b0 + lane;
+    len = 0;
+    if (bb < p.B) len = p.kv_lens ? min(p.S, max(0, p.kv_lens[bb])) : p.S;
+    cnt = (len + p.chunk_keys - 1) / p.chunk_keys;
+    incl = cnt;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+      const int up = __shfl_up(incl, o, 64);
+      if (lane >= o) incl += up;
+    }
+  };
+  int len0, cnt0, incl0;  // block 0 stays in registers: batches <= 64 never reload
+  block_counts(0, len0, cnt0, incl0);
+  int total_chunks = __builtin_amdgcn_readlane(incl0, 63);
+  for (int b0 = 64; b0 < p.B; b0 += 64) {
+    int l, c, i;
+    block_counts(b0, l, c, i);
+    total_chunks += __builtin_amdgcn_readlane(i, 63);
+  }
+  const int total_items = total_chunks * p.Hkv;
+  const int n_waves = gridDim.x;
 
-  const uint8_t* kp = p.k + b * p.k_sb + hk * p.k_sh;
-  const uint8_t* vp = p.v + b * p.v_sb + hk * p.v_sh;
-  const int last = len - 1;
+  struct Item { int b, hk, begin, end, chunk; float kscale, vscale; };
+  int cur_b0 = 0, cur_pref = 0;  // block cursor: items only move forward
+  auto decode_item = [&](int j) {  // requires j < total_items
+    Item it;
+    it.hk = j % p.Hkv;
+    const int jj = j / p.Hkv;
+    int len = len0, cnt = cnt0, incl = incl0;
+    if (cur_b0 != 0) block_counts(cur_b0, len, cnt, incl);
+    while (jj >= cur_pref + __builtin_amdgcn_readlane(incl, 63) && cur_b0 + 64 < p.B) {
+      cur_pref += __builtin_amdgcn_readlane(incl, 63);
+      cur_b0 += 64;
+      block_counts(cur_b0, len, cnt, incl);
+    }
+    const uint64_t hit = __ballot(cur_pref + incl > jj);
+    const int ln = __builtin_ctzll(hit);
+    it.b = cur_b0 + ln;
+    const int first = cur_pref + __shfl(incl - cnt, ln, 64);
+    it.chunk = jj - first;
+    it.begin = it.chunk * p.chunk_keys;
+    it.end = min(__shfl(len, ln, 64), it.begin + p.chunk_keys);
+    it.b = __builtin_amdgcn_readfirstlane(it.b);
+    it.chunk = __builtin_amdgcn_readfirstlane(it.chunk);
+    it.begin = __builtin_amdgcn_readfirstlane(it.begin);
+    it.end = __builtin_amdgcn_readfirstlane(it.end);
+    // fetched here, ahead of the item's query and tiles, so that their use waits on nothing younger
+    it.kscale = p.k_scale[it.b * p.Hkv + it.hk];
+    it.vscale = p.v_scale[it.b * p.Hkv + it.hk];
+    return it;
+  };
 
-  auto load = [&](KVRegs& R_, int step) {
-    const int base = w_begin + step * 32;
+  typedef __attribute__((ext_vector_type(4))) uint32_t qraw_t;
+  qraw_t qraw[QV];  // the 32 query elements of this lane for the item fetched last, as loaded
+  auto fetch_q = [&](const Item& it) {
+    const TQ* qr = (const TQ*)p.q + it.b * p.q_sb + (it.hk * rep + hq_off) * p.q_sh + lq * p.q_sl + 32 * g;
+#pragma unroll
+    for (int i = 0; i < QV; ++i) qraw[i] = *(const qraw_t*)((const char*)qr + 16 * i);
+  };
+
+  KVRegs ra, rb;
+  auto load = [&](KVRegs& R_, const Item& it, int step) {
+    const uint8_t* kp = p.k + it.b * p.k_sb + it.hk * p.k_sh;
+    const uint8_t* vp = p.v + it.b * p.v_sb + it.hk * p.v_sh;
+    const int base = it.begin + step * 32, last = it.end - 1;
+    const int ksl = (int)p.k_sl, vsl = (int)p.v_sl;  // host checked: a (batch, head) slab spans < 2^31 bytes
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
       const int row = min(base + blk * 16 + n, last);
-      const uint8_t* kr = kp + (int64_t)row * p.k_sl + 32 * g;
+      const uint8_t* kr = kp + (uint32_t)(row * ksl + 32 * g);
       R_.k[blk][0] = *(const u32x4*)kr;
       R_.k[blk][1] = *(const u32x4*)(kr + 16);
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int row = min(base + (s >> 2) * 16 + 4 * g + (s & 3), last);
-      const uint8_t* vr = vp + (int64_t)row * p.v_sl + 4 * n;
+      const uint8_t* vr = vp + (uint32_t)(row * vsl + 4 * n);
       R_.v[0][s] = *(const uint32_t*)vr;
       R_.v[1][s] = *(const uint32_t*)(vr + 64);
     }
   };
 
-  KVRegs ra, rb;
-  if (steps > 0) load(ra, 0);  // in flight while the query fragment is prepared
-
-  // ---- query fragment: B operand of S^T = K Q^T ------------------------------------------
-  // the lane owns d = 32g .. 32g+31 of row r; step ks consumes d = 32g + 8ks .. +7
-  float qv[32];
-  load_q32<TQ>((const TQ*)p.q + b * p.q_sb + h * p.q_sh + lq * p.q_sl + 32 * g, qv);
-  float amax = 0.f;
+  // Query fragment of the item fetched last: B operand of S^T = K Q^T.
+  // The lane owns d = 32g .. 32g+31 of row r; MFMA step ks consumes d = 32g + 8ks .. +7.
+  // Returns the factor that turns a raw fp8 dot product into a log2-domain logit.
+  auto convert_q = [&](const Item& it, long (&qb)[4]) -> float {
+    float qv[32];
+    {
+      typedef __attribute__((ext_vector_type(16 / sizeof(TQ)))) TQ qvec_t;
+      constexpr int PER = 16 / sizeof(TQ);
 #pragma unroll
-  for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qv[i]));
-  amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
-  amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
-  // power-of-two pre-scale so the row peaks in [120, 240]: well inside e4m3 and exact
-  const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
-  long qb[4];
+      for (int i = 0; i < QV; ++i) {
+        const qvec_t v = __builtin_bit_cast(qvec_t, qraw[i]);
 #pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    uint32_t w[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      w[j] = col_live ? split_pair(qv[ks * 8 + 2 * j] * f, qv[ks * 8 + 2 * j + 1] * f, part) : 0u;
-    qb[ks] = as_long(w[0] | (w[1] << 16), w[2] | (w[3] << 16));
-  }
-  const float kscale = p.k_scale[b * p.Hkv + hk];
-  const float c_row = p.scale * kscale / f * kLog2e;  // raw dot -> log2-domain logit
-
-  f32x4 oacc[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
-  float m_run = -INFINITY, l_run = 0.f;
-
-  auto compute = [&](const KVRegs& R_, int step) {
-    const int base = w_begin + step * 32;
-    // S^T = K Q^T : rows = 16 keys of a block, columns = (split term, query row)
-    f32x4 sacc[2];
-#pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-      sacc[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const u32x4 kk = R_.k[blk][ks >> 1];
-        const long a = as_long(kk[(ks & 1) * 2], kk[(ks & 1) * 2 + 1]);
-        sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, qb[ks], sacc[blk], 0, 0, 0);
+        for (int e = 0; e < PER; ++e) qv[i * PER + e] = (float)v[e];
       }
     }
-    float t[8];
+    float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const float x = sum_parts<PARTS>(sacc[i >> 2][i & 3]);
-      const int key = base + (i >> 2) * 16 + 4 * g + (i & 3);
-      t[i] = key < w_end ? x * c_row : -INFINITY;
+    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qv[i]));
+    amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
+    amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
+    // power-of-two pre-scale so the row peaks in [120, 240]: well inside e4m3 and exact
+    const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) {
+      uint32_t w[4];
+#pragma unroll
+      for (int jq = 0; jq < 4; ++jq)
+        w[jq] = split_pair<PARTS>(qv[ks * 8 + 2 * jq] * f, qv[ks * 8 + 2 * jq + 1] * f, pm);
+      qb[ks] = as_long(w[0] | (w[1] << 16), w[2] | (w[3] << 16));
     }
-    float tmax = t[0];
-#pragma unroll
-    for (int i = 1; i < 8; ++i) tmax = fmaxf(tmax, t[i]);
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
-    tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
-    const float m_new = fmaxf(m_run, tmax);  // finite: every step holds at least one live key
-    const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
-    m_run = m_new;
-    float pv[8], psum = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      pv[i] = __builtin_amdgcn_exp2f(t[i] - m_new);
-      psum += pv[i];
-    }
-    l_run = l_run * alpha + psum;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
-    // P^T (B operand): key slot s of this lane is key (s/4)*16 + 4g + s%4, the order V is loaded in
-    uint32_t pw[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      pw[j] = col_live ? split_pair(pv[2 * j] * kPScale, pv[2 * j + 1] * kPScale, part) : 0u;
-    const long pb = as_long(pw[0] | (pw[1] << 16), pw[2] | (pw[3] << 16));
-    // O^T += V^T P^T : byte-transpose the 4-byte V pieces into rows d = 64*hf + 4n + j
-#pragma unroll
-    for (int hf = 0; hf < 2; ++hf) {
-      uint32_t o_lo[4], o_hi[4];
-#pragma unroll
-      for (int q4 = 0; q4 < 2; ++q4) {
-        const uint32_t w0 = R_.v[hf][q4 * 4 + 0], w1 = R_.v[hf][q4 * 4 + 1];
-        const uint32_t w2 = R_.v[hf][q4 * 4 + 2], w3 = R_.v[hf][q4 * 4 + 3];
-        const uint32_t t0 = __builtin_amdgcn_perm(w1, w0, 0x05010400);
-        const uint32_t t1 = __builtin_amdgcn_perm(w1, w0, 0x07030602);
-        const uint32_t t2 = __builtin_amdgcn_perm(w3, w2, 0x05010400);
-        const uint32_t t3 = __builtin_amdgcn_perm(w3, w2, 0x07030602);
-        uint32_t* o = q4 ? o_hi : o_lo;
-        o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100);
-        o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302);
-        o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100);
-        o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        oacc[hf * 4 + j] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(
-            as_long(o_lo[j], o_hi[j]), pb, oacc[hf * 4 + j], 0, 0, 0);
-    }
+    return p.scale * it.kscale / f * kLog2e;
   };
 
-  for (int s = 0; s < steps; s += 2) {
-    if (s + 1 < steps) load(rb, s + 1);
-    compute(ra, s);
-    if (s + 2 < steps) load(ra, s + 2);
-    if (s + 1 < steps) compute(rb, s + 1);
-  }
+  int j = blockIdx.x;
+  if (j >= total_items) return;
+  Item cur = decode_item(j);
+  fetch_q(cur);
+  load(ra, cur, 0);
+  long qb[4];
+  float c_row = convert_q(cur, qb);
 
-  // ---- merge split terms, then the four wavefronts, and emit the chunk's partial result ------
-#pragma unroll
-  for (int i = 0; i < 8; ++i)
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-      oacc[i][e] = sum_parts<PARTS>(oacc[i][e]);
+  while (true) {
+    // the next item: its query rows travel while this one streams
+    const int jn = j + n_waves;
+    const bool more = jn < total_items;
+    Item nxt = cur;
+    if (more) {
+      nxt = decode_item(jn);
+      fetch_q(nxt);
     }
-  float l_tot = l_run + __shfl_xor(l_run, 16, 64);
-  l_tot += __shfl_xor(l_tot, 32, 64);
-  if (n < p.R) {  // split term 0 lanes of live rows
-    if (g == 0) s_m[wave][n] = m_run, s_l[wave][n] = l_tot;
+
+    f32x4 oacc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_run = -INFINITY, l_run = 0.f;
+    const int w_end = cur.end;
+
+    auto compute = [&](const KVRegs& R_, int step) {
+      const int base = cur.begin + step * 32;
+      // S^T = K Q^T : rows = 16 keys of a block, columns = (split term, query row)
+      f32x4 sacc[2];
+#pragma unroll
+      for (int blk = 0; blk < 2; ++blk) {
+        sacc[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int ks = 0; ks < 4; ++ks) {
+          const u32x4 kk = R_.k[blk][ks >> 1];
+          const long a = as_long(kk[(ks & 1) * 2], kk[(ks & 1) * 2 + 1]);
+          sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, qb[ks], sacc[blk], 0, 0, 0);
+        }
+      }
+      float t[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        const float x = sum_parts<PARTS>(sacc[i >> 2][i & 3]);
+        const int key = base + (i >> 2) * 16 + 4 * g + (i & 3);
+        t[i] = key < w_end ? x * c_row : -INFINITY;
+      }
+      float tmax = t[0];
+#pragma unroll
+      for (int i = 1; i < 8; ++i) tmax = fmaxf(tmax, t[i]);
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 16, 64));
+      tmax = fmaxf(tmax, __shfl_xor(tmax, 32, 64));
+      const float m_new = fmaxf(m_run, tmax);  // finite: every step holds at least one live key
+      const float alpha = __builtin_amdgcn_exp2f(m_run - m_new);
+      m_run = m_new;
+      float pv[8], psum = 0.f;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) {
+        pv[i] = __builtin_amdgcn_exp2f(t[i] - m_new);
+        psum += pv[i];
+      }
+      l_run = l_run * alpha + psum;
+#pragma unroll
+      for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
+      // P^T (B operand): key slot s of this lane is key (s/4)*16 + 4g + s%4, the order V is loaded in
+      uint32_t pw[4];
+#pragma unroll
+      for (int jq = 0; jq < 4; ++jq)
+        pw[jq] = split_pair<PARTS>(pv[2 * jq] * kPScale, pv[2 * jq + 1] * kPScale, pm);
+      const long pb = as_long(pw[0] | (pw[1] << 16), pw[2] | (pw[3] << 16));
+      // O^T += V^T P^T : byte-transpose the 4-byte V pieces into rows d = 64*hf + 4n + j
+#pragma unroll
+      for (int hf = 0; hf < 2; ++hf) {
+        uint32_t o_lo[4], o_hi[4];
+#pragma unroll
+        for (int q4 = 0; q4 < 2; ++q4) {
+          const uint32_t w0 = R_.v[hf][q4 * 4 + 0], w1 = R_.v[hf][q4 * 4 + 1];
+          const uint32_t w2 = R_.v[hf][q4 * 4 + 2], w3 = R_.v[hf][q4 * 4 + 3];
+          const uint32_t t0 = __builtin_amdgcn_perm(w1, w0, 0x05010400);
+          const uint32_t t1 = __builtin_amdgcn_perm(w1, w0, 0x07030602);
+          const uint32_t t2 = __builtin_amdgcn_perm(w3, w2, 0x05010400);
+          const uint32_t t3 = __builtin_amdgcn_perm(w3, w2, 0x07030602);
+          uint32_t* o = q4 ? o_hi : o_lo;
+          o[0] = __builtin_amdgcn_perm(t2, t0, 0x05040100);
+          o[1] = __builtin_amdgcn_perm(t2, t0, 0x07060302);
+          o[2] = __builtin_amdgcn_perm(t3, t1, 0x05040100);
+          o[3] = __builtin_amdgcn_perm(t3, t1, 0x07060302);
+        }
+#pragma unroll
+        for (int jq = 0; jq < 4; ++jq)
+          oacc[hf * 4 + jq] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(
+              as_long(o_lo[jq], o_hi[jq]), pb, oacc[hf * 4 + jq], 0, 0, 0);
+      }
+    };
+
+    const int steps = (cur.end - cur.begin + 31) / 32;  // >= 1: an item is never empty
+    // Loads are issued unconditionally (rows past the item's end clamp to its last key, a cache
+    // hit) so that the count of loads in flight at every wait is the same on all paths.
+    int s = 0;
+    do {  // (a do-while: the compiler then knows that a tile was requested after the next query)
+      load(rb, cur, s + 1);
+      __builtin_amdgcn_sched_barrier(0);  // keep every tile's loads ahead of the work they overlap
+      compute(ra, s);
+      __builtin_amdgcn_sched_barrier(0);
+      const bool stay = s + 2 < steps;  // else: the next item's first tile, in flight during the epilogue
+      load(ra, stay ? cur : nxt, stay ? s + 2 : 0);
+      __builtin_amdgcn_sched_barrier(0);
+      if (s + 1 < steps) compute(rb, s + 1);
+      s += 2;
+    } while (s < steps);
+    // all tiles of this item are consumed; what is in flight is the next item's first tile, and
+    // its query rows landed long ago: build its fragment now, ahead of the stores below
+    long qb_next[4];
+    float c_next = 0.f;
+    if (more) c_next = convert_q(nxt, qb_next);
+
+    // ---- merge the split terms and emit this chunk's partial result -------------------------------
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
-      for (int e = 0; e < 4; ++e)
-        s_o[wave][n][(i >> 2) * 64 + 16 * g + 4 * e + (i & 3)] = oacc[i][e];
-  }
-  __syncthreads();
-  const float vscale = p.v_scale[b * p.Hkv + hk] * (1.f / kPScale);
-  const int64_t slot = ((int64_t)(b * p.Hkv + hk) * p.chunks + chunk) * p.R;
-  for (int idx = tid; idx < p.R * D; idx += 64 * kWaves) {
-    const int row = idx / D, d = idx % D;
-    float M = s_m[0][row];
+      for (int e = 0; e < 4; ++e) oacc[i][e] = sum_parts<PARTS>(oacc[i][e]);
+    float l_tot = l_run + __shfl_xor(l_run, 16, 64);
+    l_tot += __shfl_xor(l_tot, 32, 64);
+    if (n < p.R) {  // split term 0 lanes of live rows
+      const float vscale = cur.vscale * (1.f / kPScale);
+      const int64_t slot = ((int64_t)(cur.b * p.Hkv + cur.hk) * p.chunks + cur.chunk) * p.R + n;
+      if (g == 0) p.ws_ml[slot * 2] = m_run, p.ws_ml[slot * 2 + 1] = l_tot;
+      float* dst = p.ws_o + slot * D + 16 * g;
 #pragma unroll
-    for (int w = 1; w < kWaves; ++w) M = fmaxf(M, s_m[w][row]);
-    float L = 0.f, O = 0.f;
+      for (int i = 0; i < 8; ++i)
 #pragma unroll
-    for (int w = 0; w < kWaves; ++w) {
-      const float sc = __builtin_amdgcn_exp2f(s_m[w][row] - M);  // empty wavefront: exp2(-inf) = 0
-      L += s_l[w][row] * sc;
-      O += s_o[w][row][d] * sc;
+        for (int e = 0; e < 4; ++e) dst[(i >> 2) * 64 + 4 * e + (i & 3)] = oacc[i][e] * vscale;
     }
-    p.ws_o[(slot + row) * D + d] = O * vscale;
-    if (d == 0) p.ws_ml[(slot + row) * 2] = M, p.ws_ml[(slot + row) * 2 + 1] = L;
+    if (!more) break;
+    j = jn;
+    cur = nxt;
+    c_row = c_next;
+#pragma unroll
+    for (int ks = 0; ks < 4; ++ks) qb[ks] = qb_next[ks];
   }
 }
 
@@ -350,7 +430,7 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
 
 int chunk_keys_for(const mi355_sdpa_decode_params& p) {
   const int S = (int)p.k.size[2];
-  int ck = 1024;
+  int ck = 256;
   if (p.num_splits > 0) ck = (S + p.num_splits - 1) / p.num_splits;
   ck = ((ck + 127) / 128) * 128;
   if (ck < 128) ck = 128;
@@ -358,11 +438,25 @@ int chunk_keys_for(const mi355_sdpa_decode_params& p) {
   return ck;
 }
 
+int wave_slots() {  // wavefronts of the decode kernel the chip holds at once
+  static int slots = 0;
+  if (!slots) {
+    int dev = 0, cus = 0;
+    if (hipGetDevice(&dev) == hipSuccess &&
+        hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
+      slots = cus * 4 * kDecOcc;
+    else
+      slots = 256 * 4 * kDecOcc;
+  }
+  return slots;
+}
+
 template <typename TQ>
 int launch_t(const DecP& g, hipStream_t s) {
-  dim3 grid(g.chunks, g.Hkv, g.B), block(64 * kWaves);
-  if (g.R <= 4) hipLaunchKernelGGL((decode_kernel<TQ, 3>), grid, block, 0, s, g);
-  else hipLaunchKernelGGL((decode_kernel<TQ, 2>), grid, block, 0, s, g);
+  const int64_t max_items = (int64_t)g.B * g.Hkv * g.chunks;
+  const int waves = (int)std::min<int64_t>(max_items, wave_slots());
+  if (g.R <= 4) hipLaunchKernelGGL((decode_kernel<TQ, 3>), dim3(waves), dim3(64), 0, s, g);
+  else hipLaunchKernelGGL((decode_kernel<TQ, 2>), dim3(waves), dim3(64), 0, s, g);
   int rc = check_launch("decode_kernel");
   if (rc) return rc;
   hipLaunchKernelGGL((decode_merge_kernel<TQ>), dim3(g.B * g.Hkv * g.R), dim3(D), 0, s, g);
