@@ -3,11 +3,12 @@
 // the hot path).  Defined as torch_neuronx/_sdpa_math.py:51-95 applied to the dequantised
 // cache with a key-padding bias; the reference itself has no fp8 attention path.
 //
-// Work split: the keys of a (batch, kv head) are cut into chunks; one wavefront takes a chunk and
-// serves all R = Lq * Hq/Hkv query rows that share that kv head, so every K/V byte is read from
-// HBM exactly once, and padding past kv_lens[b] is never read.  A wavefront walks its chunk 32
-// keys at a time with a running max / sum / output, writes the chunk's partial result, and a
-// second small kernel merges the chunks of a sequence.  Wavefronts are persistent (see below).
+// Work split: the live keys of all (batch, kv head) pairs, in steps of 32 keys, form one long
+// list which is cut into equal contiguous ranges, one per wavefront; the wavefront serves all
+// R = Lq * Hq/Hkv query rows that share a kv head, so every K/V byte is read from HBM exactly
+// once, and padding past kv_lens[b] is never read.  A wavefront walks its range 32 keys at a
+// time with a running max / sum / output, writes one partial result per (batch, kv head) it
+// touched, and a second small kernel merges the partials of a sequence.
 //
 // Precision without dequantising the cache: the bf16 query row is scaled by a power of two
 // and split into up to three e4m3 terms (q = q0 + q1 + q2, exact to ~12 bits); the terms
@@ -29,7 +30,6 @@ typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 
 constexpr int D = 128;
-constexpr int kWaves = 4;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
 #ifndef DEC_OCC
@@ -45,14 +45,16 @@ struct DecP {
   const int32_t* kv_lens;
   void* out;
   float* lse;
-  float* ws_o;   // (B,Hkv,chunks,R,128)
-  float* ws_ml;  // (B,Hkv,chunks,R,2)
+  float* ws_o;        // (slots,R,128) partial outputs; slot = b*Hkv + hk + wavefront index
+  float* ws_ml;       // (slots,R,2)   partial (max, sum)
+  int32_t* ws_steps;  // (B+1) exclusive prefix of the 32-key step counts per batch, then the total
   int64_t q_sb, q_sh, q_sl;
   int64_t k_sb, k_sh, k_sl;
   int64_t v_sb, v_sh, v_sl;
   int64_t o_sb, o_sh, o_sl;
   int B, Hq, Hkv, Lq, S, R;
-  int chunk_keys, chunks;
+  int n_waves;  // wavefronts of the streaming kernel
+  int t_min;    // least number of steps per wavefront
   float scale;
 };
 
@@ -104,12 +106,17 @@ struct KVRegs {
   uint32_t v[2][8];   // [64-wide half of d][key slot]
 };
 
-// One workgroup = one wavefront, launched once per wavefront slot of the chip and PERSISTENT:
-// wavefront w of W takes work items w, w + W, w + 2W, ...  An item is one chunk of chunk_keys keys
-// of one (batch, kv head), so all items cost the same but for the ragged last chunk of a
-// sequence, and the static deal balances the chip to within one item without atomics.  The item
-// list is never materialised: a wavefront prefix-sums the chunk counts of 64 batches at a time
-// across its lanes and finds the batch of an item with a ballot.
+// Steps per wavefront for a work list of `total` steps: equal shares, but not so small that the
+// partial results outweigh the keys read.
+__device__ __forceinline__ int steps_per_wave(int total, int n_waves, int t_min) {
+  return max(t_min, (total + n_waves - 1) / n_waves);
+}
+
+// One workgroup = one wavefront, launched once per wavefront slot of the chip.  The work list is
+// never materialised: step number G = (steps of batches < b) * Hkv + hk * steps(b) + s, so the
+// steps of one (batch, kv head) are contiguous; wavefront w owns [w*T, (w+1)*T).  A wavefront
+// prefix-sums the step counts of 64 batches at a time across its lanes and finds the batch of a
+// step with a ballot.  An item is the part of one (batch, kv head) inside the wavefront's range.
 // While an item streams, the query rows of the next one are already in flight (they wait in
 // registers), and its first K/V tile is requested before the epilogue of the current one, so the
 // memory pipe of a wavefront never drains between items.
@@ -127,15 +134,14 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   const int rr = min(r, p.R - 1);
   const int hq_off = rr % rep, lq = rr / rep;
 
-  // ---- the item list ------------------------------------------------------------------------------
-  // Batch b owns cnt(b) = ceil(len_b / chunk_keys) chunks; items are numbered batch-major,
-  // then chunk, then kv head.  Lane i of a block of 64 batches holds cnt and its inclusive prefix;
-  // the batch of an item is the first lane whose prefix exceeds the item's chunk number.
+  // ---- the work list ------------------------------------------------------------------------------
+  // Lane i of a block of 64 batches holds the batch's length, its step count and the inclusive
+  // prefix of the counts.  Wavefront 0 also leaves the prefix sums for the merge kernel.
   auto block_counts = [&](int b0, int& len, int& cnt, int& incl) {
     const int bb = b0 + lane;
     len = 0;
     if (bb < p.B) len = p.kv_lens ? min(p.S, max(0, p.kv_lens[bb])) : p.S;
-    cnt = (len + p.chunk_keys - 1) / p.chunk_keys;
+    cnt = (len + 31) >> 5;
     incl = cnt;
 #pragma unroll
     for (int o = 1; o < 64; o <<= 1) {
@@ -143,41 +149,47 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       if (lane >= o) incl += up;
     }
   };
+  const bool scribe = blockIdx.x == 0;
   int len0, cnt0, incl0;  // block 0 stays in registers: batches <= 64 never reload
   block_counts(0, len0, cnt0, incl0);
-  int total_chunks = __builtin_amdgcn_readlane(incl0, 63);
+  if (scribe && lane < p.B) p.ws_steps[lane] = incl0 - cnt0;
+  int seq_steps = __builtin_amdgcn_readlane(incl0, 63);
   for (int b0 = 64; b0 < p.B; b0 += 64) {
     int l, c, i;
     block_counts(b0, l, c, i);
-    total_chunks += __builtin_amdgcn_readlane(i, 63);
+    if (scribe && b0 + lane < p.B) p.ws_steps[b0 + lane] = seq_steps + i - c;
+    seq_steps += __builtin_amdgcn_readlane(i, 63);
   }
-  const int total_items = total_chunks * p.Hkv;
-  const int n_waves = gridDim.x;
+  if (scribe && lane == 0) p.ws_steps[p.B] = seq_steps;
+  const int total = seq_steps * p.Hkv;
+  const int T = steps_per_wave(total, p.n_waves, p.t_min);
+  const int g_first = blockIdx.x * T, g_end = min(total, g_first + T);
+  if (g_first >= total) return;
 
-  struct Item { int b, hk, begin, end, chunk; float kscale, vscale; };
+  struct Item { int b, hk, begin, end, steps, slot; float kscale, vscale; };
   int cur_b0 = 0, cur_pref = 0;  // block cursor: items only move forward
-  auto decode_item = [&](int j) {  // requires j < total_items
+  auto decode_item = [&](int G) {  // the item that starts at step G, g_first <= G < g_end
     Item it;
-    it.hk = j % p.Hkv;
-    const int jj = j / p.Hkv;
     int len = len0, cnt = cnt0, incl = incl0;
     if (cur_b0 != 0) block_counts(cur_b0, len, cnt, incl);
-    while (jj >= cur_pref + __builtin_amdgcn_readlane(incl, 63) && cur_b0 + 64 < p.B) {
+    while (G >= (cur_pref + __builtin_amdgcn_readlane(incl, 63)) * p.Hkv && cur_b0 + 64 < p.B) {
       cur_pref += __builtin_amdgcn_readlane(incl, 63);
       cur_b0 += 64;
       block_counts(cur_b0, len, cnt, incl);
     }
-    const uint64_t hit = __ballot(cur_pref + incl > jj);
+    // first batch whose steps end beyond G (a batch without steps never is the first)
+    const uint64_t hit = __ballot((cur_pref + incl) * p.Hkv > G);
     const int ln = __builtin_ctzll(hit);
-    it.b = cur_b0 + ln;
-    const int first = cur_pref + __shfl(incl - cnt, ln, 64);
-    it.chunk = jj - first;
-    it.begin = it.chunk * p.chunk_keys;
-    it.end = min(__shfl(len, ln, 64), it.begin + p.chunk_keys);
-    it.b = __builtin_amdgcn_readfirstlane(it.b);
-    it.chunk = __builtin_amdgcn_readfirstlane(it.chunk);
-    it.begin = __builtin_amdgcn_readfirstlane(it.begin);
-    it.end = __builtin_amdgcn_readfirstlane(it.end);
+    const int nb = __shfl(cnt, ln, 64);                                  // steps of a kv head of this batch
+    const int rem = G - (cur_pref + __shfl(incl - cnt, ln, 64)) * p.Hkv;  // steps into the batch
+    const int hk = rem / nb, s0 = rem - hk * nb;
+    const int ns = max(1, min(nb - s0, g_end - G));  // (never below 1: the walk always advances)
+    it.b = __builtin_amdgcn_readfirstlane(cur_b0 + ln);
+    it.hk = __builtin_amdgcn_readfirstlane(hk);
+    it.steps = __builtin_amdgcn_readfirstlane(ns);
+    it.begin = __builtin_amdgcn_readfirstlane(s0 * 32);
+    it.end = __builtin_amdgcn_readfirstlane(min(__shfl(len, ln, 64), (s0 + ns) * 32));
+    it.slot = it.b * p.Hkv + it.hk + blockIdx.x;
     // fetched here, ahead of the item's query and tiles, so that their use waits on nothing younger
     it.kscale = p.k_scale[it.b * p.Hkv + it.hk];
     it.vscale = p.v_scale[it.b * p.Hkv + it.hk];
@@ -247,9 +259,8 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     return p.scale * it.kscale / f * kLog2e;
   };
 
-  int j = blockIdx.x;
-  if (j >= total_items) return;
-  Item cur = decode_item(j);
+  int G = g_first;
+  Item cur = decode_item(G);
   fetch_q(cur);
   load(ra, cur, 0);
   long qb[4];
@@ -257,11 +268,11 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
 
   while (true) {
     // the next item: its query rows travel while this one streams
-    const int jn = j + n_waves;
-    const bool more = jn < total_items;
+    const int g_next = G + cur.steps;
+    const bool more = g_next < g_end;
     Item nxt = cur;
     if (more) {
-      nxt = decode_item(jn);
+      nxt = decode_item(g_next);
       fetch_q(nxt);
     }
 
@@ -340,7 +351,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       }
     };
 
-    const int steps = (cur.end - cur.begin + 31) / 32;  // >= 1: an item is never empty
+    const int steps = cur.steps;  // >= 1: an item is never empty
     // Loads are issued unconditionally (rows past the item's end clamp to its last key, a cache
     // hit) so that the count of loads in flight at every wait is the same on all paths.
     int s = 0;
@@ -361,7 +372,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     float c_next = 0.f;
     if (more) c_next = convert_q(nxt, qb_next);
 
-    // ---- merge the split terms and emit this chunk's partial result -------------------------------
+    // ---- merge the split terms and emit this item's partial result -------------------------------
 #pragma unroll
     for (int i = 0; i < 8; ++i)
 #pragma unroll
@@ -370,7 +381,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     l_tot += __shfl_xor(l_tot, 32, 64);
     if (n < p.R) {  // split term 0 lanes of live rows
       const float vscale = cur.vscale * (1.f / kPScale);
-      const int64_t slot = ((int64_t)(cur.b * p.Hkv + cur.hk) * p.chunks + cur.chunk) * p.R + n;
+      const int64_t slot = (int64_t)cur.slot * p.R + n;
       if (g == 0) p.ws_ml[slot * 2] = m_run, p.ws_ml[slot * 2 + 1] = l_tot;
       float* dst = p.ws_o + slot * D + 16 * g;
 #pragma unroll
@@ -379,7 +390,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
         for (int e = 0; e < 4; ++e) dst[(i >> 2) * 64 + 4 * e + (i & 3)] = oacc[i][e] * vscale;
     }
     if (!more) break;
-    j = jn;
+    G = g_next;
     cur = nxt;
     c_row = c_next;
 #pragma unroll
@@ -387,39 +398,42 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   }
 }
 
-// Merge the chunk partials of one (batch, kv head, query row); 128 threads = 128 output columns.
-// The (max, sum) pairs of all chunks are fetched first (one per lane), so the weights are known
-// before the partial outputs stream in and the loads of the outputs are independent.
+// Merge the partials of one (batch, kv head, query row); 128 threads = 128 output columns.
+// The wavefronts that touched this (batch, kv head) follow from the step numbering alone, and
+// their partials sit in consecutive slots.
 template <typename TQ>
 __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
-  __shared__ float s_w[64];
+  __shared__ float s_red[2][2];
   const int row = blockIdx.x % p.R;
   const int hk = (blockIdx.x / p.R) % p.Hkv;
   const int b = blockIdx.x / (p.R * p.Hkv);
   const int d = threadIdx.x;
-  int len = p.S;
-  if (p.kv_lens) len = min(p.S, max(0, p.kv_lens[b]));
-  const int nch = (len + p.chunk_keys - 1) / p.chunk_keys;  // <= 64 (checked by the launcher)
-  const int64_t slot0 = (int64_t)(b * p.Hkv + hk) * p.chunks * p.R + row;
-  float m = -INFINITY, l = 0.f;
-  if (d < nch) {
-    const int64_t s = slot0 + (int64_t)d * p.R;
-    m = p.ws_ml[s * 2], l = p.ws_ml[s * 2 + 1];
-  }
-  float M = m;
-  if (d < 64) M = wave_max(M);
-  const float w = (d < nch) ? __builtin_amdgcn_exp2f(m - M) : 0.f;
-  float L = l * w;
-  if (d < 64) {
-    L = wave_sum(L);
-    s_w[d] = w;
-  }
-  __shared__ float s_ML[2];
-  if (d == 0) s_ML[0] = M, s_ML[1] = L;
+  const int pref = p.ws_steps[b], nb = p.ws_steps[b + 1] - pref;
+  const int T = steps_per_wave(p.ws_steps[p.B] * p.Hkv, p.n_waves, p.t_min);
+  const int g0 = pref * p.Hkv + hk * nb;
+  const int w0 = g0 / T;
+  const int npart = nb > 0 ? (g0 + nb - 1) / T - w0 + 1 : 0;
+  const int64_t slot0 = (int64_t)(b * p.Hkv + hk + w0) * p.R + row;  // partial c sits at slot0 + c*R
+  float M = -INFINITY;
+  for (int c = d; c < npart; c += D) M = fmaxf(M, p.ws_ml[(slot0 + (int64_t)c * p.R) * 2]);
+  M = wave_max(M);
+  if ((d & 63) == 0) s_red[0][d >> 6] = M;
   __syncthreads();
-  M = s_ML[0], L = s_ML[1];
+  M = fmaxf(s_red[0][0], s_red[0][1]);
+  float L = 0.f;
+  for (int c = d; c < npart; c += D) {
+    const int64_t s = slot0 + (int64_t)c * p.R;
+    L += p.ws_ml[s * 2 + 1] * __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
+  }
+  L = wave_sum(L);
+  if ((d & 63) == 0) s_red[1][d >> 6] = L;
+  __syncthreads();
+  L = s_red[1][0] + s_red[1][1];
   float O = 0.f;
-  for (int c = 0; c < nch; ++c) O = fmaf(p.ws_o[(slot0 + (int64_t)c * p.R) * D + d], s_w[c], O);
+  for (int c = 0; c < npart; ++c) {
+    const int64_t s = slot0 + (int64_t)c * p.R;
+    O = fmaf(p.ws_o[s * D + d], __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M), O);
+  }
   const int rep = p.Hq / p.Hkv;
   const int h = hk * rep + row % rep, lq = row / rep;
   TQ* o = (TQ*)p.out + b * p.o_sb + h * p.o_sh + lq * p.o_sl;
@@ -428,15 +442,8 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     p.lse[((int64_t)b * p.Hq + h) * p.Lq + lq] = L > 0.f ? (M + __builtin_amdgcn_logf(L)) * kLn2 : -INFINITY;
 }
 
-int chunk_keys_for(const mi355_sdpa_decode_params& p) {
-  const int S = (int)p.k.size[2];
-  int ck = 256;
-  if (p.num_splits > 0) ck = (S + p.num_splits - 1) / p.num_splits;
-  ck = ((ck + 127) / 128) * 128;
-  if (ck < 128) ck = 128;
-  while ((S + ck - 1) / ck > 64) ck *= 2;  // the merge step handles at most 64 chunks
-  return ck;
-}
+constexpr int kMaxWaves = 4096;  // bound on the streaming kernel's grid; sizes the workspace
+constexpr int kMinSteps = 4;     // 128 keys: below this the partial results rival the keys in bytes
 
 int wave_slots() {  // wavefronts of the decode kernel the chip holds at once
   static int slots = 0;
@@ -444,37 +451,46 @@ int wave_slots() {  // wavefronts of the decode kernel the chip holds at once
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
-      slots = cus * 4 * kDecOcc;
+      slots = std::min(cus * 4 * kDecOcc, kMaxWaves);
     else
       slots = 256 * 4 * kDecOcc;
   }
   return slots;
 }
 
+// least steps per wavefront: num_splits > 0 asks for at most about that many pieces per sequence
+int min_steps_for(const mi355_sdpa_decode_params& p) {
+  const int64_t seq_steps = (p.k.size[2] + 31) / 32;
+  int t = kMinSteps;
+  if (p.num_splits > 0) t = (int)std::max<int64_t>(t, (seq_steps + p.num_splits - 1) / p.num_splits);
+  return t;
+}
+
 template <typename TQ>
 int launch_t(const DecP& g, hipStream_t s) {
-  const int64_t max_items = (int64_t)g.B * g.Hkv * g.chunks;
-  const int waves = (int)std::min<int64_t>(max_items, wave_slots());
-  if (g.R <= 4) hipLaunchKernelGGL((decode_kernel<TQ, 3>), dim3(waves), dim3(64), 0, s, g);
-  else hipLaunchKernelGGL((decode_kernel<TQ, 2>), dim3(waves), dim3(64), 0, s, g);
+  if (g.R <= 4) hipLaunchKernelGGL((decode_kernel<TQ, 3>), dim3(g.n_waves), dim3(64), 0, s, g);
+  else hipLaunchKernelGGL((decode_kernel<TQ, 2>), dim3(g.n_waves), dim3(64), 0, s, g);
   int rc = check_launch("decode_kernel");
   if (rc) return rc;
   hipLaunchKernelGGL((decode_merge_kernel<TQ>), dim3(g.B * g.Hkv * g.R), dim3(D), 0, s, g);
   return check_launch("decode_merge_kernel");
 }
 
+int64_t partial_slots(const mi355_sdpa_decode_params& p) { return p.q.size[0] * p.k.size[1] + kMaxWaves; }
+
 }  // namespace
 
 int decode_pick_splits(const mi355_sdpa_decode_params& p) {
-  const int S = (int)p.k.size[2], ck = chunk_keys_for(p);
-  return (S + ck - 1) / ck;
+  const int64_t seq_steps = (p.k.size[2] + 31) / 32;
+  const int t = min_steps_for(p);
+  return (int)((seq_steps + t - 1) / t);
 }
 
+// partial outputs, partial (max, sum) pairs, then the per-batch step prefix sums
 size_t decode_workspace(const mi355_sdpa_decode_params& p) {
   const int64_t rep = p.k.size[1] ? p.q.size[1] / p.k.size[1] : 0;
   const int64_t R = rep * p.q.size[2];
-  const int64_t slots = p.q.size[0] * p.k.size[1] * decode_pick_splits(p) * R;
-  return (size_t)slots * (D + 2) * sizeof(float);
+  return (size_t)(partial_slots(p) * R * (D + 2)) * sizeof(float) + (size_t)(p.q.size[0] + 1) * sizeof(int32_t);
 }
 
 int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
@@ -500,18 +516,20 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
   g.k_sb = p.k.stride[0], g.k_sh = p.k.stride[1], g.k_sl = p.k.stride[2];
   g.v_sb = p.v.stride[0], g.v_sh = p.v.stride[1], g.v_sl = p.v.stride[2];
   g.o_sb = p.out.stride[0], g.o_sh = p.out.stride[1], g.o_sl = p.out.stride[2];
-  g.chunk_keys = chunk_keys_for(p);
-  g.chunks = (g.S + g.chunk_keys - 1) / g.chunk_keys;
-  if (g.chunks > 64)
-    return set_error("SDPA decode: at most 64 key chunks per sequence (got %d): lower num_splits", g.chunks),
-           MI355_SDPA_ERR_UNSUPPORTED;
+  const int64_t max_steps = (int64_t)g.B * g.Hkv * ((g.S + 31) / 32);
+  if (max_steps >= (1ll << 31) || (int64_t)(g.S - 1) * p.k.stride[2] + D >= (1ll << 31) ||
+      (int64_t)(g.S - 1) * p.v.stride[2] + D >= (1ll << 31))
+    return set_error("SDPA decode: cache too large for 32-bit step and row offsets"), MI355_SDPA_ERR_UNSUPPORTED;
+  g.t_min = min_steps_for(p);
+  g.n_waves = (int)std::min<int64_t>(wave_slots(), std::max<int64_t>(1, (max_steps + g.t_min - 1) / g.t_min));
   const int64_t qes = p.q_dtype == MI355_SDPA_F32 ? 4 : 2;
   if (((uintptr_t)p.q.data & 15) || (p.q.stride[0] * qes) % 16 || (p.q.stride[1] * qes) % 16 || (p.q.stride[2] * qes) % 16)
     return set_error("SDPA decode: query rows must be 16-byte aligned"), MI355_SDPA_ERR_UNSUPPORTED;
   g.scale = p.scale;
-  const int64_t slots = (int64_t)g.B * g.Hkv * g.chunks * g.R;
+  const int64_t slots = partial_slots(p) * g.R;
   g.ws_o = (float*)p.workspace;
   g.ws_ml = g.ws_o + slots * D;
+  g.ws_steps = (int32_t*)(g.ws_ml + slots * 2);
   switch (p.q_dtype) {
     case MI355_SDPA_BF16: return launch_t<bf16_t>(g, s);
     case MI355_SDPA_F16: return launch_t<f16_t>(g, s);
