@@ -314,6 +314,9 @@ def decode_fp8kv(query, k_q, v_q, k_scale, v_scale, kv_lens, scale=None, head_ch
     lse = torch.empty(B, Hq, Lq, dtype=torch.float32)
     for b in range(B):
         n = int(kv_lens[b])
+        if n == 0:  # every key padded away: the fully-masked-row rule of compute_attention
+            out[b], lse[b] = 0.0, float("-inf")
+            continue
         kb = dequantize_kv_fp8(k_q[b : b + 1, :, :n], k_scale[b : b + 1])
         vb = dequantize_kv_fp8(v_q[b : b + 1, :, :n], v_scale[b : b + 1])
         heads = torch.arange(Hq)

@@ -73,6 +73,35 @@ def test_decode_fp32_and_fp16_queries(amd, gpu_device):
         _check(amd, gpu_device, _case(2, 8, 2, 1, 300, lens, seed=11, qdtype=dt))
 
 
+def test_decode_many_batches_with_empty_and_short_sequences(amd, gpu_device):
+    # more than 64 batches (the kernel scans lengths 64 at a time), empty sequences between
+    # live ones, and sequences so short that one wavefront's share spans several of them
+    B = 150
+    g = torch.Generator().manual_seed(77)
+    lens = torch.randint(0, 97, (B,), generator=g).to(torch.int32)
+    lens[0] = 0
+    lens[63:66] = 0
+    lens[-1] = 0
+    lens[70] = 300
+    case = _case(B, 8, 2, 1, 300, lens, seed=78)
+    out, lse = _check(amd, gpu_device, case)
+    dead = lens == 0
+    assert torch.equal(out[dead].float().cpu(), torch.zeros(int(dead.sum()), 8, 1, 128))
+    assert torch.isinf(lse[dead]).all()
+    # one piece per sequence at most (plus alignment) gives the same answer
+    out1, _ = _check(amd, gpu_device, case, num_splits=1)
+    assert max_abs(out, out1) <= 4e-3
+
+
+def test_decode_all_sequences_empty(amd, gpu_device):
+    lens = torch.zeros(3, dtype=torch.int32)
+    q, kq, vq, ks, vs, _ = _case(3, 8, 2, 1, 64, lens, seed=9)
+    out, lse = amd.decode_fp8kv(q.to(gpu_device), kq.to(gpu_device), vq.to(gpu_device),
+                                ks.to(gpu_device), vs.to(gpu_device), lens.to(gpu_device))
+    assert torch.equal(out.float().cpu(), torch.zeros(3, 8, 1, 128))
+    assert torch.isinf(lse).all() and (lse < 0).all()
+
+
 def test_config5_full_size(amd, gpu_device):
     # BASELINE config 5: B=64,Hq=32,Hkv=8,D=128,q_len=1, kv_len ~ U[512,8192] padded to 8192
     B, Hq, Hkv, S = 64, 32, 8, 8192

@@ -297,3 +297,18 @@ def test_fp8_quantisation_definition_and_decode():
     o2, l2 = om.sdpa_forward(q.float(), kd, vd, attn_mask=pad)
     torch.testing.assert_close(o2, out, rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(l2, lse, rtol=1e-5, atol=1e-6)
+
+
+def test_decode_empty_sequence_matches_fully_masked_rows():
+    g = torch.Generator().manual_seed(3)
+    B, Hq, Hkv, S, D = 2, 4, 2, 8, 16
+    q = torch.randn(B, Hq, 1, D, generator=g)
+    kq, ks = om.quantize_kv_fp8(torch.randn(B, Hkv, S, D, generator=g))
+    vq, vs = om.quantize_kv_fp8(torch.randn(B, Hkv, S, D, generator=g))
+    lens = torch.tensor([0, 5])
+    out, lse = om.decode_fp8kv(q, kq, vq, ks, vs, lens)
+    pad = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+    o2, l2 = om.sdpa_forward(q, om.dequantize_kv_fp8(kq, ks), om.dequantize_kv_fp8(vq, vs), attn_mask=pad)
+    assert torch.equal(out[0], torch.zeros_like(out[0])) and torch.isinf(lse[0]).all() and (lse[0] < 0).all()
+    torch.testing.assert_close(o2, out, rtol=1e-5, atol=1e-6)
+    torch.testing.assert_close(l2, lse, rtol=1e-5, atol=1e-6)

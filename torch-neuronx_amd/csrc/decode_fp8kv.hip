@@ -414,25 +414,46 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
   const int w0 = g0 / T;
   const int npart = nb > 0 ? (g0 + nb - 1) / T - w0 + 1 : 0;
   const int64_t slot0 = (int64_t)(b * p.Hkv + hk + w0) * p.R + row;  // partial c sits at slot0 + c*R
-  float M = -INFINITY;
-  for (int c = d; c < npart; c += D) M = fmaxf(M, p.ws_ml[(slot0 + (int64_t)c * p.R) * 2]);
-  M = wave_max(M);
-  if ((d & 63) == 0) s_red[0][d >> 6] = M;
-  __syncthreads();
-  M = fmaxf(s_red[0][0], s_red[0][1]);
-  float L = 0.f;
-  for (int c = d; c < npart; c += D) {
-    const int64_t s = slot0 + (int64_t)c * p.R;
-    L += p.ws_ml[s * 2 + 1] * __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
-  }
-  L = wave_sum(L);
-  if ((d & 63) == 0) s_red[1][d >> 6] = L;
-  __syncthreads();
-  L = s_red[1][0] + s_red[1][1];
-  float O = 0.f;
-  for (int c = 0; c < npart; ++c) {
-    const int64_t s = slot0 + (int64_t)c * p.R;
-    O = fmaf(p.ws_o[s * D + d], __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M), O);
+  float M = -INFINITY, L = 0.f, O = 0.f;
+  constexpr int kFew = 8;
+  if (npart <= kFew) {
+    // few partials: fetch every (max, sum) pair and output value at once, then combine; each
+    // thread repeats the scalar part, which costs less than a second round trip to memory
+    float m[kFew], l[kFew], o[kFew];
+#pragma unroll
+    for (int c = 0; c < kFew; ++c) {
+      const int64_t s = slot0 + (int64_t)min(c, max(npart - 1, 0)) * p.R;
+      const bool live = c < npart;
+      m[c] = live ? p.ws_ml[s * 2] : -INFINITY;
+      l[c] = live ? p.ws_ml[s * 2 + 1] : 0.f;
+      o[c] = live ? p.ws_o[s * D + d] : 0.f;
+    }
+#pragma unroll
+    for (int c = 0; c < kFew; ++c) M = fmaxf(M, m[c]);
+#pragma unroll
+    for (int c = 0; c < kFew; ++c) {
+      const float w = c < npart ? __builtin_amdgcn_exp2f(m[c] - M) : 0.f;
+      L = fmaf(l[c], w, L);
+      O = fmaf(o[c], w, O);
+    }
+  } else {
+    for (int c = d; c < npart; c += D) M = fmaxf(M, p.ws_ml[(slot0 + (int64_t)c * p.R) * 2]);
+    M = wave_max(M);
+    if ((d & 63) == 0) s_red[0][d >> 6] = M;
+    __syncthreads();
+    M = fmaxf(s_red[0][0], s_red[0][1]);
+    for (int c = d; c < npart; c += D) {
+      const int64_t s = slot0 + (int64_t)c * p.R;
+      L += p.ws_ml[s * 2 + 1] * __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
+    }
+    L = wave_sum(L);
+    if ((d & 63) == 0) s_red[1][d >> 6] = L;
+    __syncthreads();
+    L = s_red[1][0] + s_red[1][1];
+    for (int c = 0; c < npart; ++c) {
+      const int64_t s = slot0 + (int64_t)c * p.R;
+      O = fmaf(p.ws_o[s * D + d], __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M), O);
+    }
   }
   const int rep = p.Hq / p.Hkv;
   const int h = hk * rep + row % rep, lq = row / rep;
