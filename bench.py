@@ -9,6 +9,9 @@ forward at the Llama-3-8B layer shape (B=1, Hq=32, Hkv=8, S=8192, D=128).  One J
 printed; `roofline` is for the dominant kernel of the workload (kernel time from HIP events on
 the launch stream), `cpu_baseline` is the CPU oracle timed on a bounded sample of the same
 workload on this box's host cores, `extras` carries the other workloads of the metric.
+
+Before the W warmup steps the workload runs untimed for 0.3 s so that the GPU's clocks have
+settled; the K timed steps are bracketed by torch.cuda.synchronize() on both sides.
 """
 
 from __future__ import annotations
@@ -43,8 +46,25 @@ def seeded(shapes, seed, dtype, dev):
     return [torch.randn(s, generator=g).to(dtype).to(dev) for s in shapes]
 
 
+def spin_up(fn, seconds=0.3):
+    """Untimed load before the warmup steps: the GPU's clocks climb over the first tens of
+    milliseconds of work (the same kernel runs ~25 % slower right after idle), and a handful of
+    warmup launches of a sub-millisecond kernel does not get there."""
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < seconds:
+        for _ in range(10):
+            fn()
+        torch.cuda.synchronize()
+
+
+SPIN = True
+
+
 def event_time_ms(fn, steps, warmup):
     """Run warmup + steps launches; returns (wall ms per step, event ms per step)."""
+    if SPIN:
+        spin_up(fn)
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()
@@ -135,8 +155,9 @@ def cpu_baseline_fwd(B, Hq, Hkv, S, D, seed, heads=2):
 
     g = torch.Generator(device="cpu").manual_seed(seed)
     q = torch.randn(B, Hq, S, D, generator=g).to(torch.bfloat16)[:, :heads].float()
-    k = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)[:, :1].float()
-    v = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)[:, :1].float()
+    kvh = max(1, heads * Hkv // Hq)
+    k = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)[:, :kvh].float()
+    v = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)[:, :kvh].float()
     t0 = time.perf_counter()
     om.sdpa_forward(q, k, v, is_causal=True)
     dt = time.perf_counter() - t0
@@ -147,14 +168,80 @@ def cpu_baseline_fwd(B, Hq, Hkv, S, D, seed, heads=2):
                       f"algorithmic (unmasked-pair) FLOPs / wall time; {dt:.2f} s"}
 
 
+def cpu_baseline_fwd_bwd(B, Hq, Hkv, S, D, seed, heads=32):
+    """CPU oracle forward + backward on `heads` query heads of config 4 (one batch element)."""
+    from oracle import sdpa_math as om
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    q = torch.randn(B, Hq, S, D, generator=g).to(torch.bfloat16)[:1, :heads].float()
+    kvh = max(1, heads * Hkv // Hq)
+    k = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)[:1, :kvh].float()
+    v = torch.randn(B, Hkv, S, D, generator=g).to(torch.bfloat16)[:1, :kvh].float()
+    do = torch.randn(B, Hq, S, D, generator=g).to(torch.bfloat16)[:1, :heads].float()
+    t0 = time.perf_counter()
+    out, lse = om.sdpa_forward(q, k, v, is_causal=True)
+    om.sdpa_backward(do, q, k, v, out, lse, is_causal=True)
+    dt = time.perf_counter() - t0
+    flops = 14.0 * heads * D * causal_pairs(S, S)
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+            "kind": "port",
+            "sample": f"{heads} of {B * Hq} (batch, query head) pairs of the same workload, full S={S}, "
+                      f"forward + backward; algorithmic (unmasked-pair) FLOPs / wall time; {dt:.2f} s"}
+
+
+def cpu_baseline_decode(batches=32):
+    """CPU oracle decode on the first `batches` sequences of config 5."""
+    from oracle import sdpa_math as om
+
+    B, Hq, Hkv, S, D = 64, 32, 8, 8192, 128
+    g = torch.Generator(device="cpu").manual_seed(1005)
+    q = torch.randn(B, Hq, 1, D, generator=g).to(torch.bfloat16)[:batches]
+    lens = torch.randint(512, 8193, (B,), generator=g).to(torch.int32)[:batches]
+    kq, ks = om.quantize_kv_fp8(torch.randn(batches, Hkv, S, D, generator=g))
+    vq, vs = om.quantize_kv_fp8(torch.randn(batches, Hkv, S, D, generator=g))
+    t0 = time.perf_counter()
+    om.decode_fp8kv(q, kq, vq, ks, vs, lens)
+    dt = time.perf_counter() - t0
+    nbytes = 2.0 * Hkv * D * int(lens.sum())
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"first {batches} of {B} sequences of the same workload ({int(lens.sum())} live keys); "
+                      f"fp8 K/V bytes of the live keys / wall time (dequantisation included); {dt:.2f} s"}
+
+
+def known_size_copy(dev, mib=256):
+    """One plain device-to-device copy of `mib` MiB: the yardstick that the HBM traffic counters
+    (FETCH_SIZE / WRITE_SIZE) of a profiled run are scaled by."""
+    src = torch.empty(mib << 20, dtype=torch.uint8, device=dev).fill_(1)
+    dst = torch.empty_like(src)
+    torch.cuda.synchronize()
+    dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+    torch.cuda.empty_cache()
+
+
+# HBM bytes per launch of the dominant kernel, from `rocprofv3 --pmc FETCH_SIZE` and
+# `--pmc WRITE_SIZE` runs of this script (--pmc-copy), scaled by the same counters' reading for
+# the known-size copy.  None = not measured for that workload.
+MEASURED_TRAFFIC_BYTES = {
+    "c3_fwd": 213.9e6,      # fwd_w64_kernel: 145.7 MB read + 68.2 MB written (algorithmic 168.8 MB)
+    "c2_fwd": None,
+    "c4_fwd_bwd": 1587.9e6,  # the three backward kernels of one call (algorithmic 337 MB)
+    "c5_decode": 620.6e6,    # decode_kernel + decode_merge_kernel of one call (algorithmic 590.8 MB)
+}
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="c3_fwd", choices=["c3_fwd", "c2_fwd", "c4_fwd_bwd", "c5_decode"])
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-spin", action="store_true", help="skip the untimed clock spin-up (profiled runs)")
+    ap.add_argument("--pmc-copy", action="store_true",
+                    help="also run one 256 MiB device copy (counter yardstick for profiled runs)")
     args = ap.parse_args()
     if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -169,6 +256,10 @@ def main():
     dev = torch.device("cuda:0")
     torch.cuda.set_device(dev)
     extras = {}
+    global SPIN
+    SPIN = not args.no_spin
+    if args.pmc_copy:
+        known_size_copy(dev)
 
     if args.workload in ("c3_fwd", "c2_fwd"):
         if args.workload == "c3_fwd":
@@ -179,13 +270,13 @@ def main():
         value = flops / (wall * 1e-3) / 1e12
         ach = flops / (ev * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "fwd_mfma_kernel",
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "fwd_w64_kernel" if args.workload == "c3_fwd" else "fwd_mfma_kernel",
                 "kernel_ms": ev}
         unit, dtype = "TFLOP/s", "bf16"
         cpu = None
         if not args.no_cpu:
             if args.workload == "c3_fwd":
-                cpu = cpu_baseline_fwd(1, 32, 8, 8192, 128, 1003, heads=2)
+                cpu = cpu_baseline_fwd(1, 32, 8, 8192, 128, 1003, heads=32)
             else:
                 cpu = cpu_baseline_fwd(4, 12, 12, 1024, 64, 1002, heads=12)
     elif args.workload == "c4_fwd_bwd":
@@ -207,16 +298,18 @@ def main():
         cfg = {"workload": "c4_causal_gqa_bf16_fwd_bwd", "B": 2, "Hq": 32, "Hkv": 8, "S": 4096, "D": 128,
                "fwd_tflops": f_fwd / (ev_f * 1e-3) / 1e12, "bwd_tflops": ach,
                "algorithmic_flops": flops}
-        unit, dtype, cpu = "TFLOP/s", "bf16", None
+        unit, dtype = "TFLOP/s", "bf16"
+        cpu = None if args.no_cpu else cpu_baseline_fwd_bwd(2, 32, 8, 4096, 128, 1004, heads=32)
     else:
         step, nbytes, cfg = wl_decode(amd, dev)
         wall, ev = event_time_ms(step, args.steps, args.warmup)
         value = nbytes / (wall * 1e-3) / 1e9
         ach = nbytes / (ev * 1e-3) / 1e9
         roof = {"bound": "hbm", "achieved": ach, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                "frac": ach / PEAK_HBM_GBS, "traffic": None, "kernel": "decode_kernel (+merge)",
+                "frac": ach / PEAK_HBM_GBS, "traffic": None, "kernel": "decode_kernel + decode_merge_kernel (one call)",
                 "kernel_ms": ev}
-        unit, dtype, cpu = "GB/s", "fp8_e4m3 (K/V), bf16 (Q/O), f32 accumulate", None
+        unit, dtype = "GB/s", "fp8_e4m3 (K/V), bf16 (Q/O), f32 accumulate"
+        cpu = None if args.no_cpu else cpu_baseline_decode(batches=32)
 
     if not args.no_extras and args.workload == "c3_fwd":
         try:
@@ -240,6 +333,7 @@ def main():
         except Exception as e:
             extras["c4_fwd_bwd"] = {"error": repr(e)}
 
+    roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
     line = {
         "metric": METRIC, "value": value, "unit": unit, "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": wall, "higher_is_better": True, "scaling": "weak",

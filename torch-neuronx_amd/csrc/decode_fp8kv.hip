@@ -274,6 +274,8 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     if (more) {
       nxt = decode_item(g_next);
       fetch_q(nxt);
+    } else {
+      nxt.begin = cur.end - 1;  // no next item: the unconditional tile request below re-reads one cached row
     }
 
     f32x4 oacc[8];
