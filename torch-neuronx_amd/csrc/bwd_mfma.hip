@@ -18,6 +18,8 @@
 // swizzled, transposed tiles are written with byte permutes (see mfma_common.h).  Math follows
 // _sdpa_math.py:98-176: everything accumulates in float32, rows with lse = -inf give zero
 // gradients, scale multiplies dQ and dK once at the end.
+#include <type_traits>
+
 #include "mfma_common.h"
 
 namespace mi355 {
@@ -158,21 +160,40 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
   for (int it = 0; it < n_items; ++it) {
     const int buf = it & 1;
     const int q0 = item_q0(it);
+    // register classes, stated once per item: the dK / dV accumulators are touched by matrix ops
+    // only and live in accumulation registers; the K / V fragments feed every matrix op as a
+    // source operand and must stay in ordinary vector registers
+#pragma unroll
+    for (int i = 0; i < DB; ++i) {
+      asm volatile("" : "+a"(dkacc[i]));
+      asm volatile("" : "+a"(dvacc[i]));
+    }
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+v"(kf[ks]));
+      asm volatile("" : "+v"(vf[ks]));
+    }
     const bool active = !p.causal || q0 + BQ - 1 >= kw0;
     if (active) {
       const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= p.S);
       uint32_t pP[2][8], pS[2][8];
-#pragma unroll
-      for (int mq = 0; mq < 2; ++mq) {
-        f32x16 sacc, dpacc;
-        zero(sacc), zero(dpacc);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const u32x4 a = *(const u32x4*)(&q_rm[buf][rm_off<D>(mq * 32 + col, 2 * ks + half)]);
-          sacc = Mma<T>::run(a, kf[ks], sacc);
-          const u32x4 a2 = *(const u32x4*)(&do_rm[buf][rm_off<D>(mq * 32 + col, 2 * ks + half)]);
-          dpacc = Mma<T>::run(a2, vf[ks], dpacc);
-        }
+      // A operands stream from LDS through a small register ring, kRing reads ahead of the
+      // matrix op that consumes them: with one wavefront per SIMD nothing else hides LDS latency.
+      constexpr int kRing = 4;
+      u32x4 ring[kRing];
+      // S / dP operand i of query-row block mq: (i even) Q rows for S, (i odd) dO rows for dP
+      auto read_rows = [&](int mq, int i) -> u32x4 {
+        const uint16_t* t = (i & 1) ? do_rm[buf] : q_rm[buf];
+        return *(const u32x4*)(&t[rm_off<D>(mq * 32 + col, 2 * (i >> 1) + half)]);
+      };
+      // dV / dK operand i: step ks = i / (2 DB), d block db, (i even) dO^T for dV, (i odd) Q^T for dK
+      auto read_cols = [&](int i) -> u32x4 {
+        const uint16_t* t = (i & 1) ? q_t[buf] : do_t[buf];
+        const int ks = i / (2 * DB), db = (i >> 1) % DB;
+        return *(const u32x4*)(&t[(db * 32 + col) * TP + ks * 16 + half * 8]);
+      };
+      // P = exp2(c S - lse), dS = P (dP - delta) for 32 query rows x this lane's key
+      auto softmax = [&](int mq, const f32x16& sacc, const f32x16& dpacc, auto edge_c) {
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const f32x4 l4 = *(const f32x4*)(&lse_s[buf][mq * 32 + r4 * 8 + half * 4]);
@@ -182,29 +203,49 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
           for (int e = 0; e < 4; ++e) {
             const int r = r4 * 4 + e;
             pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
-            if (edge) {
+            if (decltype(edge_c)::value) {
               const int qi = q0 + mq * 32 + r4 * 8 + half * 4 + e;
-              if ((p.causal && key > qi) || key >= p.S) pr[e] = 0.f;
+              pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
             }
             ds[e] = pr[e] * (dpacc[r] - d4[e]);
           }
           pP[mq][r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[mq][r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
           pS[mq][r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[mq][r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
         }
-      }
+      };
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int mq = ks >> 1, r0 = (ks & 1) * 4;
-        const u32x4 bP = {pP[mq][r0], pP[mq][r0 + 1], pP[mq][r0 + 2], pP[mq][r0 + 3]};
-        const u32x4 bS = {pS[mq][r0], pS[mq][r0 + 1], pS[mq][r0 + 2], pS[mq][r0 + 3]};
+      for (int i = 0; i < kRing; ++i) ring[i] = read_rows(0, i);
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const u32x4 a = *(const u32x4*)(&do_t[buf][(db * 32 + col) * TP + ks * 16 + half * 8]);
-          dvacc[db] = Mma<T>::run(a, bP, dvacc[db]);
-          const u32x4 a2 = *(const u32x4*)(&q_t[buf][(db * 32 + col) * TP + ks * 16 + half * 8]);
-          dkacc[db] = Mma<T>::run(a2, bS, dkacc[db]);
+      for (int mq = 0; mq < 2; ++mq) {
+        f32x16 sacc, dpacc;
+        zero(sacc), zero(dpacc);
+#pragma unroll
+        for (int i = 0; i < 2 * KS; ++i) {
+          if (i & 1) dpacc = Mma<T>::run(ring[i % kRing], vf[i >> 1], dpacc);
+          else sacc = Mma<T>::run(ring[i % kRing], kf[i >> 1], sacc);
+          if (i + kRing < 2 * KS) ring[i % kRing] = read_rows(mq, i + kRing);
+          else if (mq == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
+          else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (edge) softmax(mq, sacc, dpacc, std::true_type{});
+        else softmax(mq, sacc, dpacc, std::false_type{});
+        __builtin_amdgcn_sched_barrier(0);
       }
+      // dV^T += dO^T P, dK^T += Q^T dS
+#pragma unroll
+      for (int i = 0; i < 8 * DB; ++i) {
+        const int ks = i / (2 * DB), db = (i >> 1) % DB, mq = ks >> 1, r0 = (ks & 1) * 4;
+        if (i & 1) {
+          const u32x4 bS = {pS[mq][r0], pS[mq][r0 + 1], pS[mq][r0 + 2], pS[mq][r0 + 3]};
+          dkacc[db] = Mma<T>::run(ring[i % kRing], bS, dkacc[db]);
+        } else {
+          const u32x4 bP = {pP[mq][r0], pP[mq][r0 + 1], pP[mq][r0 + 2], pP[mq][r0 + 3]};
+          dvacc[db] = Mma<T>::run(ring[i % kRing], bP, dvacc[db]);
+        }
+        if (i + kRing < 8 * DB) ring[i % kRing] = read_cols(i + kRing);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (it + 1 < n_items) store_item(buf ^ 1);
     __syncthreads();
