@@ -364,46 +364,72 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
   for (int t = 0; t < nt; ++t) {
     const int buf = t & 1, kv0 = t * BN;
     const bool active = !p.causal || kv0 <= qw0 + 31;
+    // register classes, stated once per tile (see bwd_dkdv_kernel)
+#pragma unroll
+    for (int i = 0; i < DB; ++i) asm volatile("" : "+a"(dqacc[i]));
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      asm volatile("" : "+v"(qf[ks]));
+      asm volatile("" : "+v"(dof[ks]));
+    }
     if (active) {
       const bool edge = (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S);
       const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
       uint32_t pS[2][8];
-#pragma unroll
-      for (int mb = 0; mb < 2; ++mb) {
-        f32x16 sacc, dpacc;
-        zero(sacc), zero(dpacc);
-#pragma unroll
-        for (int ks = 0; ks < KS; ++ks) {
-          const u32x4 a = *(const u32x4*)(&k_rm[buf][rm_off<D>(mb * 32 + col, 2 * ks + half)]);
-          sacc = Mma<T>::run(a, qf[ks], sacc);
-          const u32x4 a2 = *(const u32x4*)(&v_rm[buf][rm_off<D>(mb * 32 + col, 2 * ks + half)]);
-          dpacc = Mma<T>::run(a2, dof[ks], dpacc);
-        }
+      constexpr int kRing = 4;
+      u32x4 ring[kRing];
+      // S^T / dP^T operand i of key block mb: (i even) K rows, (i odd) V rows
+      auto read_rows = [&](int mb, int i) -> u32x4 {
+        const uint16_t* t_ = (i & 1) ? v_rm[buf] : k_rm[buf];
+        return *(const u32x4*)(&t_[rm_off<D>(mb * 32 + col, 2 * (i >> 1) + half)]);
+      };
+      // dQ^T operand i: step ks = i / DB, d block db = i % DB of K^T
+      auto read_cols = [&](int i) -> u32x4 {
+        return *(const u32x4*)(&k_t[buf][((i % DB) * 32 + col) * TP + (i / DB) * 16 + half * 8]);
+      };
+      auto softmax = [&](int mb, const f32x16& sacc, const f32x16& dpacc, auto edge_c) {
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           float ds[2];
 #pragma unroll
           for (int e = 0; e < 2; ++e) {
             float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
-            if (edge) {
+            if (decltype(edge_c)::value) {
               const int kv = kv0 + mb * 32 + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
-              if (kv > lim) pr = 0.f;
+              pr = kv > lim ? 0.f : pr;
             }
             ds[e] = pr * (dpacc[r + e] - dl);
           }
           pS[mb][r >> 1] = Mma<T>::pack(ds[0], ds[1]);
         }
-      }
+      };
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) {
-        const int mb = ks >> 1, r0 = (ks & 1) * 4;
-        const u32x4 bS = {pS[mb][r0], pS[mb][r0 + 1], pS[mb][r0 + 2], pS[mb][r0 + 3]};
+      for (int i = 0; i < kRing; ++i) ring[i] = read_rows(0, i);
 #pragma unroll
-        for (int db = 0; db < DB; ++db) {
-          const u32x4 a = *(const u32x4*)(&k_t[buf][(db * 32 + col) * TP + ks * 16 + half * 8]);
-          dqacc[db] = Mma<T>::run(a, bS, dqacc[db]);
+      for (int mb = 0; mb < 2; ++mb) {
+        f32x16 sacc, dpacc;
+        zero(sacc), zero(dpacc);
+#pragma unroll
+        for (int i = 0; i < 2 * KS; ++i) {
+          if (i & 1) dpacc = Mma<T>::run(ring[i % kRing], dof[i >> 1], dpacc);
+          else sacc = Mma<T>::run(ring[i % kRing], qf[i >> 1], sacc);
+          if (i + kRing < 2 * KS) ring[i % kRing] = read_rows(mb, i + kRing);
+          else if (mb == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
+          else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
+        __builtin_amdgcn_sched_barrier(0);
+        if (edge) softmax(mb, sacc, dpacc, std::true_type{});
+        else softmax(mb, sacc, dpacc, std::false_type{});
+        __builtin_amdgcn_sched_barrier(0);
       }
+#pragma unroll
+      for (int i = 0; i < 4 * DB; ++i) {
+        const int ks = i / DB, db = i % DB, mb = ks >> 1, r0 = (ks & 1) * 4;
+        const u32x4 bS = {pS[mb][r0], pS[mb][r0 + 1], pS[mb][r0 + 2], pS[mb][r0 + 3]};
+        dqacc[db] = Mma<T>::run(ring[i % kRing], bS, dqacc[db]);
+        if (i + kRing < 4 * DB) ring[i % kRing] = read_cols(i + kRing);
+      }
+      __builtin_amdgcn_sched_barrier(0);
     }
     if (t + 1 < nt) store_tile(buf ^ 1);
     __syncthreads();
