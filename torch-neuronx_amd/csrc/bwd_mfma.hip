@@ -179,7 +179,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
       uint32_t pP[2][8], pS[2][8];
       // A operands stream from LDS through a small register ring, kRing reads ahead of the
       // matrix op that consumes them: with one wavefront per SIMD nothing else hides LDS latency.
-      constexpr int kRing = 4;
+      constexpr int kRing = 8;
       u32x4 ring[kRing];
       // S / dP operand i of query-row block mq: (i even) Q rows for S, (i odd) dO rows for dP
       auto read_rows = [&](int mq, int i) -> u32x4 {
@@ -227,10 +227,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
           else if (mq == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
-        __builtin_amdgcn_sched_barrier(0);
         if (edge) softmax(mq, sacc, dpacc, std::true_type{});
         else softmax(mq, sacc, dpacc, std::false_type{});
-        __builtin_amdgcn_sched_barrier(0);
       }
       // dV^T += dO^T P, dK^T += Q^T dS
 #pragma unroll
@@ -376,7 +374,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
       const bool edge = (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S);
       const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
       uint32_t pS[2][8];
-      constexpr int kRing = 4;
+      constexpr int kRing = 8;
       u32x4 ring[kRing];
       // S^T / dP^T operand i of key block mb: (i even) K rows, (i odd) V rows
       auto read_rows = [&](int mb, int i) -> u32x4 {
@@ -417,10 +415,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
           else if (mb == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
-        __builtin_amdgcn_sched_barrier(0);
         if (edge) softmax(mb, sacc, dpacc, std::true_type{});
         else softmax(mb, sacc, dpacc, std::false_type{});
-        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int i = 0; i < 4 * DB; ++i) {
