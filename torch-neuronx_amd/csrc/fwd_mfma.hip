@@ -372,6 +372,10 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
   int NB = (force_tile == 256 || (force_tile == 0 && wg256 >= 512)) ? 2 : 1;
   if (NB == 2 && p.q.size[3] == 128 && g.S % 32 != 0) NB = 1;  // the 256-row kernel wants whole key tiles
+  // ... and addresses K / V rows with 32-bit byte offsets from the start of a (batch, head)
+  if (NB == 2 && p.q.size[3] == 128 &&
+      ((int64_t)g.S * g.k_sl * 2 >= (1ll << 31) || (int64_t)g.S * g.v_sl * 2 >= (1ll << 31)))
+    NB = 1;
   const int BM = 128 * NB;
   g.n_qt = (g.L + BM - 1) / BM;
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;

@@ -75,23 +75,27 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   u32x2 vreg[2][4];
   const int k_chunk = tid & 15, k_row0 = tid >> 4;  // K rows k_row0, k_row0 + 16
   const int v_g = tid & 7, v_dq = tid >> 3;         // keys 4 v_g .. +3, d = 4 v_dq .. +3
-  // per-thread byte offsets inside a tile are fixed; the tile base is wave-uniform, so a load is
-  // one instruction with a scalar base and a 32-bit lane offset.  S is a multiple of BN here
-  // (the launcher guarantees it), so no row needs clamping.
+  // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
+  // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
+  // instruction with no address arithmetic on the vector unit.  S is a multiple of BN here (the
+  // launcher guarantees it), so no row needs clamping.
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, 0x7fffffff, 0x00020000);
   uint32_t k_off[2], v_off[4];
 #pragma unroll
   for (int i = 0; i < 2; ++i) k_off[i] = (uint32_t)(((k_row0 + 16 * i) * p.k_sl + k_chunk * 8) * 2);
 #pragma unroll
   for (int i = 0; i < 4; ++i) v_off[i] = (uint32_t)(((4 * v_g + i) * p.v_sl + v_dq * 4) * 2);
+  const int k_tile_bytes = (int)(BN * p.k_sl * 2), v_tile_bytes = (int)(BN * p.v_sl * 2);
   auto load_k = [&](int set, int t) {
-    const char* base = (const char*)(kp + (int64_t)(min(t, nt - 1) * BN) * p.k_sl);
+    const int base = min(t, nt - 1) * k_tile_bytes;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) kreg[set][i] = *(const u32x4*)(base + k_off[i]);
+    for (int i = 0; i < 2; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i], base, 0);
   };
   auto load_v = [&](int set, int t) {
-    const char* base = (const char*)(vp + (int64_t)(min(t, nt - 1) * BN) * p.v_sl);
+    const int base = min(t, nt - 1) * v_tile_bytes;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) vreg[set][i] = *(const u32x2*)(base + v_off[i]);
+    for (int i = 0; i < 4; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b64(v_rsrc, v_off[i], base, 0);
   };
   auto store_k = [&](int set, int buf) {
 #pragma unroll
@@ -242,6 +246,7 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
       if (j >= 16) return;
       const int nb = j >> 3, r = (j & 7) * 2;
       ps[nb] += pv[j & 1][0] + pv[j & 1][1];
+      asm volatile("" : "+v"(ps[nb]));  // keeps the add in this slot (left alone it sinks below the loop body)
       pk[nb][r >> 1] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
     };
     u32x4 ring[4];
