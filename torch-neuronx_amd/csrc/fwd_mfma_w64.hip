@@ -11,12 +11,12 @@
 // MFMAs.
 //
 // With one wavefront per SIMD nothing hides latency but the instruction stream itself, so the
-// key loop is software pipelined and its order pinned by hand:
-//   phase A   S^T(t+1) = K(t+1) Q^T on the matrix pipe  |  exp2 / row sum / pack of tile t
-//   phase B   O^T += V^T(t) P^T(t) on the matrix pipe    |  LDS stores of tiles t+2 / t+1, global
-//                                                           loads of tiles t+3 / t+2, row max of t+1
+// key loop is software pipelined and its order pinned by hand (see `iteration` below): the
+// softmax of a tile is split in two halves that ride on the matrix ops of two different phases,
 // LDS operands are fetched three MFMA pairs ahead through a four-entry register ring, and a
-// scheduling barrier after every MFMA pair keeps the compiler from regrouping the stream.
+// scheduling barrier after every MFMA pair keeps the compiler from regrouping the stream.  The
+// vector unit, not the matrix pipe, is the scarce resource (v_exp_f32 alone costs half the
+// matrix time), so the loop carries no row maximum at all: see kTrig.
 // Products are computed transposed (S^T = K Q^T, O^T = V^T P^T) as in fwd_mfma.hip, so the
 // softmax statistics are per-lane scalars and P goes from accumulator to B operand in registers.
 //
@@ -145,12 +145,17 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     for (int r = 2; r < 16; r += 2) t = fmaxf(fmaxf(t, s[r]), s[r + 1]);  // v_max3
     return t;
   };
-  // The reference max follows the true row max lazily: it is raised only when a tile beats it by
-  // more than kLazy in the exponent, so probabilities stay below 2^kLazy and the accumulator is
-  // rescaled a few times per row instead of once per tile.  Exact arithmetic: numerator and row
-  // sum carry the same reference.
-  auto finish_max_x = [&](float t0, float t1, float x0, float x1) {  // x = the other half-wave's max
-    const float tm[NB] = {fmaxf(t0, x0), fmaxf(t1, x1)};
+  // The softmax reference of a row (m_run, folded into mc) is NOT the running maximum.  The fast
+  // path never looks for a maximum at all: probabilities are formed against the current reference
+  // and only their sum is watched.  A lane's sum over its 16 keys above kTrig means that some
+  // probability outgrew 2^kLazy-ish headroom (or that there is no reference yet): then, and only
+  // then, the slow path finds the true tile maximum, raises the reference of every row that beat
+  // it by more than kLazy in the exponent, rescales those rows' accumulators and redoes the
+  // tile's probabilities.  Exact arithmetic: numerator and row sum always carry the same
+  // reference, and lse = reference * scale + ln(sum).
+  constexpr float kTrig = 8192.f;  // 16 probabilities of at most 2^kLazy stay below this
+  auto raise_reference = [&](float t0, float t1) {
+    const float tm[NB] = {fmaxf(t0, __shfl_xor(t0, 32, 64)), fmaxf(t1, __shfl_xor(t1, 32, 64))};
     bool moved = false;
 #pragma unroll
     for (int nb = 0; nb < NB; ++nb) {
@@ -163,9 +168,30 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     }
     need_rescale = __builtin_amdgcn_ballot_w64(moved) != 0;
   };
-  auto finish_max = [&](float t0, float t1) {
-    finish_max_x(t0, t1, __shfl_xor(t0, 32, 64), __shfl_xor(t1, 32, 64));
+
+  // Softmax of one register pair, in three stages so that consecutive pairs can be staggered by
+  // hand (the chain read S -> fma -> exp2 -> add/pack is strictly dependent and a wavefront
+  // issues in order).  Pair j of 16: query block j / 8, accumulator registers 2 (j % 8), +1.
+  float xs[3][2], pv[2][2];
+  auto stage1 = [&](const f32x16 (&sv)[NB], int j, int q) {
+    const int nb = j >> 3, r = (j & 7) * 2;
+    xs[q % 3][0] = fmaf(sv[nb][r], c, -mc[nb]);
+    xs[q % 3][1] = fmaf(sv[nb][r + 1], c, -mc[nb]);
   };
+  auto stage2 = [&](int q) {
+    pv[q & 1][0] = __builtin_amdgcn_exp2f(xs[q % 3][0]);
+    pv[q & 1][1] = __builtin_amdgcn_exp2f(xs[q % 3][1]);
+  };
+  auto stage3 = [&](int j, int q, uint32_t (&pk)[NB][8], float (&ps)[NB]) {
+    const int nb = j >> 3, r = (j & 7) * 2;
+    ps[nb] += pv[q & 1][0] + pv[q & 1][1];
+    asm volatile("" : "+v"(ps[nb]));  // keeps the add in its slot (left alone it sinks below the loop body)
+    pk[nb][r >> 1] = Mma<T>::pack(pv[q & 1][0], pv[q & 1][1]);
+  };
+  // The 16 pairs of a tile are split in two halves by key: pairs whose registers 0..7 hold the
+  // tile's first 16 keys (the first contraction step of P*V) and those of the last 16 keys.
+  auto early_pair = [](int q) { return q < 4 ? q : q + 4; };      // 0..3, 8..11
+  auto late_pair = [](int q) { return q < 4 ? q + 4 : q + 8; };   // 4..7, 12..15
 
   // ---- prologue ----------------------------------------------------------------------------------
   load_k(0, 0);
@@ -181,6 +207,9 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   load_v(1, 1);
   load_v(0, 2);
   f32x16 s_a[NB], s_b[NB];
+  uint32_t pk_a[NB][8], pk_b[NB][8];
+  float ps_a[NB] = {0.f, 0.f}, ps_b[NB] = {0.f, 0.f};
+  bool first = true;  // no reference yet: the first tile goes through the slow path whatever its sums
   if (nt_w > 0) {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -188,73 +217,35 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
 #pragma unroll
       for (int nb = 0; nb < NB; ++nb) s_a[nb] = Mma<T>::run(a, qf[nb][ks], ks == 0 ? zero16 : s_a[nb]);
     }
-    finish_max(tile_max(s_a[0]), tile_max(s_a[1]));
+    if (is_edge(0)) mask_tile(s_a, 0);
+#pragma unroll
+    for (int q = 0; q < 8; ++q) {  // first half of tile 0 (redone by the slow path of iteration 0)
+      stage1(s_a, early_pair(q), q);
+      stage2(q);
+      stage3(early_pair(q), q, pk_a, ps_a);
+    }
   }
   __syncthreads();  // K buffer 0 is rewritten during the first iteration
 
-  // one pipelined iteration: scur holds S^T of tile t (statistics ready), snext receives tile t+1
-  auto iteration = [&](int t, auto parity, f32x16 (&scur)[NB], f32x16 (&snext)[NB]) {
+  // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
+  // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
+  //   phase A   S^T(t+1) = K(t+1) Q^T on the matrix pipe  |  softmax of the last 16 keys of tile t
+  //   check     sums of tile t against kTrig; rare slow path
+  //   phase B   O^T += V^T(t) P^T(t) on the matrix pipe    |  softmax of the first 16 keys of tile
+  //             t+1, LDS stores of tiles t+2 / t+1, fetches of tiles t+4 / t+3
+  auto iteration = [&](int t, auto parity, f32x16 (&scur)[NB], f32x16 (&snext)[NB], uint32_t (&pk)[NB][8],
+                       uint32_t (&pkn)[NB][8], float (&ps)[NB], float (&psn)[NB]) {
     constexpr int par = decltype(parity)::value;  // t & 1, known at compile time
-    if (__builtin_expect(is_edge(t * BN), 0)) {  // rare: tile crosses the causal diagonal or the end of the keys
-      mask_tile(scur, t * BN);
-      finish_max(tile_max(scur[0]), tile_max(scur[1]));
-    }
-    if (__builtin_expect(need_rescale, 0)) {  // rare: some row's reference max moved
-#pragma unroll
-      for (int nb = 0; nb < NB; ++nb) {
-        l_run[nb] *= alpha[nb];
-#pragma unroll
-        for (int i = 0; i < DB; ++i) {
-#pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            // read and write-back are pinned to accumulation registers one element at a time; left
-            // to itself the compiler drags all 128 accumulators through the general registers at
-            // once, which evicts the query fragments from them for the whole loop
-            float xv, y;
-            asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(xv) : "a"(oacc[i][nb][r]));
-            y = xv * alpha[nb];
-            asm volatile("" : "+a"(y));
-            oacc[i][nb][r] = y;
-          }
-          __builtin_amdgcn_sched_barrier(0);  // one accumulator block at a time
-        }
-        m_run[nb] = m_new[nb];
-      }
-    }
     const uint16_t* kt = &k_lds[par ^ 1][col * KROW + half * 8];
     const uint16_t* vt = &v_lds[par][col * VROW + half * 8];
     auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
     auto read_v = [&](int i) { return *(const u32x4*)(vt + (i & 3) * 32 * VROW + (i >> 2) * 16); };
-    uint32_t pk[NB][8];
-    float ps[NB] = {0.f, 0.f};
-    // The chain read S -> fma -> exp2 -> add/pack of one register pair is strictly dependent, and a
-    // wavefront issues in order, so the three stages of consecutive pairs are staggered by hand:
-    // a slot runs stage 1 of pair j+2, stage 2 of pair j+1 and stage 3 of pair j.
-    float xs[3][2], pv[2][2];
-    auto stage1 = [&](int j) {  // pair j of 16: query block j / 8, registers 2 (j % 8), +1
-      if (j >= 16) return;
-      const int nb = j >> 3, r = (j & 7) * 2;
-      xs[j % 3][0] = fmaf(scur[nb][r], c, -mc[nb]);
-      xs[j % 3][1] = fmaf(scur[nb][r + 1], c, -mc[nb]);
-    };
-    auto stage2 = [&](int j) {
-      if (j >= 16) return;
-      pv[j & 1][0] = __builtin_amdgcn_exp2f(xs[j % 3][0]);
-      pv[j & 1][1] = __builtin_amdgcn_exp2f(xs[j % 3][1]);
-    };
-    auto stage3 = [&](int j) {
-      if (j >= 16) return;
-      const int nb = j >> 3, r = (j & 7) * 2;
-      ps[nb] += pv[j & 1][0] + pv[j & 1][1];
-      asm volatile("" : "+v"(ps[nb]));  // keeps the add in this slot (left alone it sinks below the loop body)
-      pk[nb][r >> 1] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
-    };
     u32x4 ring[4];
     __builtin_amdgcn_sched_barrier(0);
     // the first operand fetches are in flight while the first probabilities are formed
     ring[0] = read_k(0), ring[1] = read_k(1), ring[2] = read_k(2);
-    stage1(0);
-    stage1(1);
+    stage1(scur, late_pair(0), 0);
+    stage1(scur, late_pair(1), 1);
     stage2(0);
     __builtin_amdgcn_sched_barrier(0);
     // ---- phase A -------------------------------------------------------------------------------
@@ -263,22 +254,56 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
       if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
       else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
       snext[0] = Mma<T>::run(ring[ks & 3], qf[0][ks], ks == 0 ? zero16 : snext[0]);
-      stage1(2 * ks + 2);
-      stage2(2 * ks + 1);
-      stage3(2 * ks);
+      if (ks + 2 < 8) stage1(scur, late_pair(ks + 2), ks + 2);
+      if (ks + 1 < 8) stage2(ks + 1);
       snext[1] = Mma<T>::run(ring[ks & 3], qf[1][ks], ks == 0 ? zero16 : snext[1]);
-      stage1(2 * ks + 3);
-      stage2(2 * ks + 2);
-      stage3(2 * ks + 1);
+      stage3(late_pair(ks), ks, pk, ps);
       __builtin_amdgcn_sched_barrier(0);
     }
+    // ---- check ---------------------------------------------------------------------------------
+    const bool trig = first || !(ps[0] <= kTrig) || !(ps[1] <= kTrig);  // (NaN also lands here)
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(trig) != 0, 0)) {
+      first = false;
+      raise_reference(tile_max(scur[0]), tile_max(scur[1]));
+      if (need_rescale) {
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          l_run[nb] *= alpha[nb];
+#pragma unroll
+          for (int i = 0; i < DB; ++i) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+              // read and write-back are pinned to accumulation registers one element at a time; left
+              // to itself the compiler drags all 128 accumulators through the general registers at
+              // once, which evicts the query fragments from them for the whole loop
+              float xv, y;
+              asm volatile("v_accvgpr_read_b32 %0, %1" : "=v"(xv) : "a"(oacc[i][nb][r]));
+              y = xv * alpha[nb];
+              asm volatile("" : "+a"(y));
+              oacc[i][nb][r] = y;
+            }
+            __builtin_amdgcn_sched_barrier(0);  // one accumulator block at a time
+          }
+          m_run[nb] = m_new[nb];
+        }
+      }
+      ps[0] = 0.f, ps[1] = 0.f;
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {  // the whole tile again, against the new reference
+        stage1(scur, j, j);
+        stage2(j);
+        stage3(j, j, pk, ps);
+      }
+    }
     l_run[0] += ps[0], l_run[1] += ps[1];
+    if (__builtin_expect(is_edge((t + 1) * BN), 0)) mask_tile(snext, (t + 1) * BN);  // rare
+    psn[0] = 0.f, psn[1] = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+    stage1(snext, early_pair(0), 0);
+    stage1(snext, early_pair(1), 1);
+    stage2(0);
+    __builtin_amdgcn_sched_barrier(0);
     // ---- phase B -------------------------------------------------------------------------------
-    // VALU / memory work is dealt out slot by slot (two MFMAs per slot):
-    //   0-3  row max of tile t+1, four registers of each query block per slot; K store in slot 0
-    //   4    exchange of the half-wave maxima is issued      5    V transpose + store
-    //   6    global loads of the tiles two ahead, exchange consumed: new reference max
-    float tm0 = -INFINITY, tm1 = -INFINITY, x0 = 0.f, x1 = 0.f;
 #pragma unroll
     for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
       if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
@@ -286,26 +311,15 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
       const u32x4 b0 = {pk[0][ks2 * 4], pk[0][ks2 * 4 + 1], pk[0][ks2 * 4 + 2], pk[0][ks2 * 4 + 3]};
       const u32x4 b1 = {pk[1][ks2 * 4], pk[1][ks2 * 4 + 1], pk[1][ks2 * 4 + 2], pk[1][ks2 * 4 + 3]};
       oacc[db][0] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db][0]);
-      if (i < 4) {
-        const int r = 4 * i;
-        tm0 = fmaxf(fmaxf(tm0, snext[0][r]), snext[0][r + 1]);
-        tm0 = fmaxf(fmaxf(tm0, snext[0][r + 2]), snext[0][r + 3]);
-      }
+      if (i + 2 < 8) stage1(snext, early_pair(i + 2), i + 2);
+      if (i + 1 < 8) stage2(i + 1);
       if (i == 0) store_k(par, par);  // tile t+2
-      if (i == 4) x0 = __shfl_xor(tm0, 32, 64), x1 = __shfl_xor(tm1, 32, 64);
-      if (i == 5) store_v_half(par ^ 1, par ^ 1, 0);  // tile t+1
+      if (i == 2) store_v_half(par ^ 1, par ^ 1, 0);  // tile t+1
       if (i == 6) load_k(par, t + 4);
       oacc[db][1] = Mma<T>::run(ring[(i + KS) & 3], b1, oacc[db][1]);
-      if (i < 4) {
-        const int r = 4 * i;
-        tm1 = fmaxf(fmaxf(tm1, snext[1][r]), snext[1][r + 1]);
-        tm1 = fmaxf(fmaxf(tm1, snext[1][r + 2]), snext[1][r + 3]);
-      }
-      if (i == 5) store_v_half(par ^ 1, par ^ 1, 1);
-      if (i == 6) {
-        load_v(par ^ 1, t + 3);
-        finish_max_x(tm0, tm1, x0, x1);
-      }
+      stage3(early_pair(i), i, pkn, psn);
+      if (i == 4) store_v_half(par ^ 1, par ^ 1, 1);
+      if (i == 7) load_v(par ^ 1, t + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
     __syncthreads();
@@ -323,11 +337,11 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
 
   int t = 0;
   for (; t + 1 < nt_w; t += 2) {
-    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b);
-    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a);
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
   }
   if (t < nt_w) {  // odd count: t is even here
-    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b);
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
     ++t;
   }
   for (; t < nt; ++t) {
