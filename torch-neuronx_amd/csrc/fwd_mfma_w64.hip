@@ -37,6 +37,37 @@ constexpr int VROW = BN + 8;  // V^T tile row pitch
 constexpr int KCH = D / 8;    // 16-byte chunks per K row
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
+// S^T = K Q^T with the result in ordinary vector registers.  The compiler picks one register
+// class for the results of ALL matrix ops of a kernel, and here it must be the accumulation
+// registers (O^T alone fills half of the file); but every element of S^T is consumed by the
+// vector unit, which cannot read accumulation registers, so leaving S^T there costs one copy
+// instruction per element per tile.  Written as inline assembly the op is opaque to the
+// compiler's hazard tracking: the caller owes kMfmaToValuNops idle cycles between the last op
+// of a chain and the first vector instruction that touches its result (see phase A).
+template <typename T>
+struct MmaV;
+template <>
+struct MmaV<bf16_t> {
+  static __device__ __forceinline__ void first(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+};
+template <>
+struct MmaV<f16_t> {
+  static __device__ __forceinline__ void first(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+};
+// idle cycles after an 8-pass matrix op before the vector unit may touch its result (the
+// architecture asks for 11; the margin is free)
+__device__ __forceinline__ void mfma_to_valu_gap() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+
 template <typename T>
 __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KROW];
@@ -215,8 +246,12 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     for (int ks = 0; ks < KS; ++ks) {
       const u32x4 a = *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
 #pragma unroll
-      for (int nb = 0; nb < NB; ++nb) s_a[nb] = Mma<T>::run(a, qf[nb][ks], ks == 0 ? zero16 : s_a[nb]);
+      for (int nb = 0; nb < NB; ++nb) {
+        if (ks == 0) MmaV<T>::first(s_a[nb], a, qf[nb][ks]);
+        else MmaV<T>::next(s_a[nb], a, qf[nb][ks]);
+      }
     }
+    mfma_to_valu_gap();
     if (is_edge(0)) mask_tile(s_a, 0);
 #pragma unroll
     for (int q = 0; q < 8; ++q) {  // first half of tile 0 (redone by the slow path of iteration 0)
@@ -253,13 +288,16 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     for (int ks = 0; ks < KS; ++ks) {
       if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
       else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
-      snext[0] = Mma<T>::run(ring[ks & 3], qf[0][ks], ks == 0 ? zero16 : snext[0]);
+      if (ks == 0) MmaV<T>::first(snext[0], ring[ks & 3], qf[0][ks]);
+      else MmaV<T>::next(snext[0], ring[ks & 3], qf[0][ks]);
       if (ks + 2 < 8) stage1(scur, late_pair(ks + 2), ks + 2);
       if (ks + 1 < 8) stage2(ks + 1);
-      snext[1] = Mma<T>::run(ring[ks & 3], qf[1][ks], ks == 0 ? zero16 : snext[1]);
+      if (ks == 0) MmaV<T>::first(snext[1], ring[ks & 3], qf[1][ks]);
+      else MmaV<T>::next(snext[1], ring[ks & 3], qf[1][ks]);
       stage3(late_pair(ks), ks, pk, ps);
       __builtin_amdgcn_sched_barrier(0);
     }
+    mfma_to_valu_gap();  // snext is read (and, on the diagonal, masked) from here on
     // ---- check ---------------------------------------------------------------------------------
     const bool trig = first || !(ps[0] <= kTrig) || !(ps[1] <= kTrig);  // (NaN also lands here)
     if (__builtin_expect(__builtin_amdgcn_ballot_w64(trig) != 0, 0)) {
