@@ -217,16 +217,21 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
       for (int i = 0; i < kRing; ++i) ring[i] = read_rows(0, i);
 #pragma unroll
       for (int mq = 0; mq < 2; ++mq) {
-        f32x16 sacc, dpacc;
-        zero(sacc), zero(dpacc);
+        f32x16 sacc, dpacc;  // written by the matrix ops below into ordinary vector registers
 #pragma unroll
         for (int i = 0; i < 2 * KS; ++i) {
-          if (i & 1) dpacc = Mma<T>::run(ring[i % kRing], vf[i >> 1], dpacc);
-          else sacc = Mma<T>::run(ring[i % kRing], kf[i >> 1], sacc);
+          if (i & 1) {
+            if (i == 1) MmaV<T>::first(dpacc, ring[i % kRing], vf[i >> 1]);
+            else MmaV<T>::next(dpacc, ring[i % kRing], vf[i >> 1]);
+          } else {
+            if (i == 0) MmaV<T>::first(sacc, ring[i % kRing], kf[i >> 1]);
+            else MmaV<T>::next(sacc, ring[i % kRing], kf[i >> 1]);
+          }
           if (i + kRing < 2 * KS) ring[i % kRing] = read_rows(mq, i + kRing);
           else if (mq == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
+        mfma_to_valu_gap();
         if (edge) softmax(mq, sacc, dpacc, std::true_type{});
         else softmax(mq, sacc, dpacc, std::false_type{});
       }
@@ -405,16 +410,21 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
       for (int i = 0; i < kRing; ++i) ring[i] = read_rows(0, i);
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) {
-        f32x16 sacc, dpacc;
-        zero(sacc), zero(dpacc);
+        f32x16 sacc, dpacc;  // written by the matrix ops below into ordinary vector registers
 #pragma unroll
         for (int i = 0; i < 2 * KS; ++i) {
-          if (i & 1) dpacc = Mma<T>::run(ring[i % kRing], dof[i >> 1], dpacc);
-          else sacc = Mma<T>::run(ring[i % kRing], qf[i >> 1], sacc);
+          if (i & 1) {
+            if (i == 1) MmaV<T>::first(dpacc, ring[i % kRing], dof[i >> 1]);
+            else MmaV<T>::next(dpacc, ring[i % kRing], dof[i >> 1]);
+          } else {
+            if (i == 0) MmaV<T>::first(sacc, ring[i % kRing], qf[i >> 1]);
+            else MmaV<T>::next(sacc, ring[i % kRing], qf[i >> 1]);
+          }
           if (i + kRing < 2 * KS) ring[i % kRing] = read_rows(mb, i + kRing);
           else if (mb == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
+        mfma_to_valu_gap();
         if (edge) softmax(mb, sacc, dpacc, std::true_type{});
         else softmax(mb, sacc, dpacc, std::false_type{});
       }

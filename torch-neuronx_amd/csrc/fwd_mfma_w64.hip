@@ -37,37 +37,6 @@ constexpr int VROW = BN + 8;  // V^T tile row pitch
 constexpr int KCH = D / 8;    // 16-byte chunks per K row
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
-// S^T = K Q^T with the result in ordinary vector registers.  The compiler picks one register
-// class for the results of ALL matrix ops of a kernel, and here it must be the accumulation
-// registers (O^T alone fills half of the file); but every element of S^T is consumed by the
-// vector unit, which cannot read accumulation registers, so leaving S^T there costs one copy
-// instruction per element per tile.  Written as inline assembly the op is opaque to the
-// compiler's hazard tracking: the caller owes kMfmaToValuNops idle cycles between the last op
-// of a chain and the first vector instruction that touches its result (see phase A).
-template <typename T>
-struct MmaV;
-template <>
-struct MmaV<bf16_t> {
-  static __device__ __forceinline__ void first(f32x16& d, const u32x4& a, const u32x4& b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
-    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
-  }
-};
-template <>
-struct MmaV<f16_t> {
-  static __device__ __forceinline__ void first(f32x16& d, const u32x4& a, const u32x4& b) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
-  }
-  static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
-    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
-  }
-};
-// idle cycles after an 8-pass matrix op before the vector unit may touch its result (the
-// architecture asks for 11; the margin is free)
-__device__ __forceinline__ void mfma_to_valu_gap() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
-
 template <typename T>
 __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KROW];

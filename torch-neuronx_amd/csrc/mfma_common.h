@@ -50,6 +50,37 @@ struct Mma<f16_t> {
   }
 };
 
+// A matrix op whose result lands in ordinary vector registers.  The compiler picks one register
+// class for the results of ALL matrix ops of a kernel, and in the attention kernels it must be the
+// accumulation registers (the output accumulators alone fill half of the file); but every element
+// of a score tile is consumed by the vector unit, which cannot read accumulation registers, so
+// leaving score tiles there costs one copy instruction per element per tile.  Written as inline assembly the op is opaque to the
+// compiler's hazard tracking: the caller owes kMfmaToValuNops idle cycles between the last op
+// of a chain and the first vector instruction that touches its result (mfma_to_valu_gap).
+template <typename T>
+struct MmaV;
+template <>
+struct MmaV<bf16_t> {
+  static __device__ __forceinline__ void first(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+};
+template <>
+struct MmaV<f16_t> {
+  static __device__ __forceinline__ void first(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+};
+// idle cycles after an 8-pass matrix op before the vector unit may touch its result (the
+// architecture asks for 11; the margin is free)
+__device__ __forceinline__ void mfma_to_valu_gap() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+
 __device__ __forceinline__ void zero(f32x16& a) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) a[r] = 0.f;
