@@ -306,11 +306,9 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
     if (__builtin_expect(is_edge((t + 1) * BN), 0)) mask_tile(snext, (t + 1) * BN);  // rare
     psn[0] = 0.f, psn[1] = 0.f;
     __builtin_amdgcn_sched_barrier(0);
-    stage1(snext, early_pair(0), 0);
-    stage1(snext, early_pair(1), 1);
-    stage2(0);
-    __builtin_amdgcn_sched_barrier(0);
     // ---- phase B -------------------------------------------------------------------------------
+    // (the softmax pipeline of tile t+1 fills and drains under the matrix ops: nothing of it runs
+    // between the phases, where the matrix pipe would sit idle)
 #pragma unroll
     for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
       if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
@@ -318,17 +316,20 @@ __global__ __launch_bounds__(256, 1) void fwd_w64_kernel(FwdM p) {
       const u32x4 b0 = {pk[0][ks2 * 4], pk[0][ks2 * 4 + 1], pk[0][ks2 * 4 + 2], pk[0][ks2 * 4 + 3]};
       const u32x4 b1 = {pk[1][ks2 * 4], pk[1][ks2 * 4 + 1], pk[1][ks2 * 4 + 2], pk[1][ks2 * 4 + 3]};
       oacc[db][0] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db][0]);
-      if (i + 2 < 8) stage1(snext, early_pair(i + 2), i + 2);
-      if (i + 1 < 8) stage2(i + 1);
+      stage1(snext, early_pair(i), i);
+      if (i >= 1) stage2(i - 1);
       if (i == 0) store_k(par, par);  // tile t+2
       if (i == 2) store_v_half(par ^ 1, par ^ 1, 0);  // tile t+1
       if (i == 6) load_k(par, t + 4);
       oacc[db][1] = Mma<T>::run(ring[(i + KS) & 3], b1, oacc[db][1]);
-      stage3(early_pair(i), i, pkn, psn);
+      if (i >= 2) stage3(early_pair(i - 2), i - 2, pkn, psn);
       if (i == 4) store_v_half(par ^ 1, par ^ 1, 1);
       if (i == 7) load_v(par ^ 1, t + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
+    stage2(7);
+    stage3(early_pair(6), 6, pkn, psn);
+    stage3(early_pair(7), 7, pkn, psn);
     __syncthreads();
   };
   // a wavefront whose rows lie above the causal diagonal of the remaining tiles only feeds LDS
