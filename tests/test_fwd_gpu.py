@@ -197,3 +197,40 @@ def test_expanded_kv_stride0(amd, gpu_device):
     out, lse = amd.sdpa_forward(q.to(gpu_device), ke, ve, is_causal=True)
     ro, rl = oracle_fwd(q, k, v, is_causal=True)
     assert max_abs(out, ro) <= 2e-2
+
+
+@pytest.mark.parametrize("tile", [3, 4])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("kind", ["rising", "falling", "spiky", "huge"])
+def test_softmax_reference_tracking_under_stress(amd, gpu_device, kind, causal, tile):
+    """Logit profiles that make the running softmax reference move often, rarely, or violently.
+
+    The long-sequence forward kernel keeps no row maximum in its fast path: it raises its
+    reference only when a tile's probability sums run away.  Rising logits trigger that again and
+    again, falling logits never after the first tile, spikes arrive in the middle of a row, and
+    'huge' logits overflow exp2 against a stale reference.  All must match the oracle.
+    """
+    B, Hq, Hkv, L, S, E = 1, 2, 1, 256, 1024, 128
+    g = torch.Generator().manual_seed({"rising": 1, "falling": 2, "spiky": 3, "huge": 4}[kind])
+    q = torch.randn(B, Hq, L, E, generator=g)
+    k = torch.randn(B, Hkv, S, E, generator=g)
+    v = torch.randn(B, Hkv, S, E, generator=g)
+    u = torch.nn.functional.normalize(torch.randn(E, generator=g), dim=0)
+    q = q + 6.0 * u  # every query has a strong component along u ...
+    ramp = torch.linspace(-1.0, 1.0, S)
+    if kind == "rising":
+        k = k + (9.0 * ramp)[None, None, :, None] * u  # ... so the logit grows with the key index
+    elif kind == "falling":
+        k = k - (9.0 * ramp)[None, None, :, None] * u
+    elif kind == "spiky":
+        spikes = torch.zeros(S)
+        spikes[torch.tensor([37, 300, 301, 640, 1001])] = torch.tensor([4.0, 9.0, 9.5, 14.0, 20.0])
+        k = k + spikes[None, None, :, None] * u
+    else:
+        k = k + (60.0 * ramp)[None, None, :, None] * u  # logits of several hundred: exp2 overflows without care
+    q, k, v = q.to(torch.bfloat16), k.to(torch.bfloat16), v.to(torch.bfloat16)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=causal, force_kernel=tile)
+    ro, rl = oracle_fwd(q, k, v, is_causal=causal)
+    assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
+    assert max_abs(out, ro) <= 2e-2  # bf16 output tolerance of the path
+    assert max_abs(lse, rl) <= 2e-3 * max(1.0, rl.abs().max().item())
