@@ -365,12 +365,13 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
-  // 256-row workgroups (one per compute unit, half the LDS traffic per flop) once they can
-  // fill the chip a few times over; 128-row workgroups for short or few sequences
+  // 256-row workgroups (one per compute unit, half the LDS traffic per flop) once there is one
+  // for every compute unit and the key loop is long enough to amortise their longer prologue;
+  // 128-row workgroups for short or few sequences (measured crossover on MI355X)
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
-  int NB = (force_tile == 256 || (force_tile == 0 && wg256 >= 512)) ? 2 : 1;
+  int NB = (force_tile == 256 || (force_tile == 0 && wg256 >= 256 && g.S >= 2048)) ? 2 : 1;
   if (NB == 2 && p.q.size[3] == 128 && g.S % 32 != 0) NB = 1;  // the 256-row kernel wants whole key tiles
   // ... and addresses K / V rows with 32-bit byte offsets from the start of a (batch, head)
   if (NB == 2 && p.q.size[3] == 128 &&
