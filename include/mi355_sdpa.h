@@ -131,7 +131,8 @@ typedef struct mi355_sdpa_decode_params {
   float* lse;               /* (B,Hq,Lq) float32 or NULL                               */
   int32_t q_dtype;
   float scale;
-  int32_t num_splits;       /* 0 = library picks                                       */
+  int32_t num_splits;       /* 0 = library picks; N > 0: cut a full-length sequence into
+                               about N pieces at most (fewer, larger partial results)  */
   void* workspace;          /* mi355_sdpa_decode_workspace_bytes() bytes               */
   size_t workspace_bytes;
 } mi355_sdpa_decode_params;
