@@ -274,9 +274,13 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
 }
 
 // ================================================================================================
-template <typename T, int D>
+// NB = query-row blocks of 32 per wavefront.  NB = 2 (256 rows per workgroup) lets every K / V /
+// K^T fragment read from LDS feed two matrix ops, which halves the LDS bytes per flop, the bound of
+// this kernel; the Q and dO fragments of 64 rows (128 registers) are then parked in accumulation
+// registers, which the score matrix ops can read directly as their B operand.
+template <typename T, int D, int NB>
 __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
-  constexpr int BM = 128, BN = 64;
+  constexpr int BM = 128 * NB, BN = 64;
   constexpr int KS = D / 16, DB = D / 32, NCH = D / 8;
   constexpr int TP = BN + 8;
   constexpr int U = 16 * NCH;               // K units (4 keys x 8 d)
@@ -288,6 +292,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
   int b, h, qt;
   {
     const int bid = blockIdx.x, rep = p.Hq / p.Hkv;
+    const int n_qt = (p.L + BM - 1) / BM;
     if (p.xcd_map) {
       const int per_xcd = (p.B * p.Hkv) / 8, xcd = bid & 7;
       int r = bid >> 3;
@@ -295,34 +300,35 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
       r /= rep;
       const int sl = r % per_xcd;
       r /= per_xcd;
-      qt = p.n_qt - 1 - r;
+      qt = n_qt - 1 - r;
       const int stream = sl * 8 + xcd;
       b = stream / p.Hkv, h = (stream % p.Hkv) * rep + hg;
     } else {
       const int heads = p.B * p.Hq;
-      qt = p.n_qt - 1 - bid / heads;
+      qt = n_qt - 1 - bid / heads;
       b = (bid % heads) / p.Hq, h = (bid % heads) % p.Hq;
     }
   }
   const int hk = h / (p.Hq / p.Hkv);
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int col = lane & 31, half = lane >> 5;
-  const int q0 = qt * BM, qw0 = q0 + wave * 32, qrow = qw0 + col;
-  const int qc = min(qrow, p.L - 1);
-
-  u32x4 qf[KS], dof[KS];
-  {
-    const uint16_t* qr = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl + half * 8;
-    const uint16_t* gr = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl + half * 8;
+  const int q0 = qt * BM, qw0 = q0 + wave * 32 * NB;
+  int qrow[NB], qc[NB];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16), dof[ks] = *(const u32x4*)(gr + ks * 16);
-  }
-  float lse2, dl;
-  {
-    const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc;
+  for (int nb = 0; nb < NB; ++nb) qrow[nb] = qw0 + 32 * nb + col, qc[nb] = min(qrow[nb], p.L - 1);
+
+  u32x4 qf[NB][KS], dof[NB][KS];
+  float lse2[NB], dl[NB];
+#pragma unroll
+  for (int nb = 0; nb < NB; ++nb) {
+    const uint16_t* qr = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc[nb] * p.q_sl + half * 8;
+    const uint16_t* gr = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc[nb] * p.go_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[nb][ks] = *(const u32x4*)(qr + ks * 16), dof[nb][ks] = *(const u32x4*)(gr + ks * 16);
+    const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc[nb];
     const float l = p.lse[idx];
-    lse2 = (qrow < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
-    dl = p.delta[idx];
+    lse2[nb] = (qrow[nb] < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
+    dl[nb] = p.delta[idx];
   }
 
   int nt = (p.S + BN - 1) / BN;
@@ -355,9 +361,11 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
     for (int i = 0; i < VLD; ++i) *(u32x4*)(&v_rm[buf][rm_off<D>(v_r0 + i * (256 / NCH), v_ch)]) = vst[i];
   };
 
-  f32x16 dqacc[DB];
+  f32x16 dqacc[DB][NB];
 #pragma unroll
-  for (int i = 0; i < DB; ++i) zero(dqacc[i]);
+  for (int i = 0; i < DB; ++i)
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb) zero(dqacc[i][nb]);
   const float c = p.scale * kLog2eF;
 
   load_tile(0);
@@ -366,19 +374,27 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
   if (nt > 1) load_tile(1);
   for (int t = 0; t < nt; ++t) {
     const int buf = t & 1, kv0 = t * BN;
-    const bool active = !p.causal || kv0 <= qw0 + 31;
+    const bool active = !p.causal || kv0 <= qw0 + 32 * NB - 1;
     // register classes, stated once per tile (see bwd_dkdv_kernel)
 #pragma unroll
-    for (int i = 0; i < DB; ++i) asm volatile("" : "+a"(dqacc[i]));
+    for (int i = 0; i < DB; ++i)
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      asm volatile("" : "+v"(qf[ks]));
-      asm volatile("" : "+v"(dof[ks]));
-    }
+      for (int nb = 0; nb < NB; ++nb) asm volatile("" : "+a"(dqacc[i][nb]));
+#pragma unroll
+    for (int nb = 0; nb < NB; ++nb)
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) {
+        if (NB == 2) {
+          asm volatile("" : "+a"(qf[nb][ks]));
+          asm volatile("" : "+a"(dof[nb][ks]));
+        } else {
+          asm volatile("" : "+v"(qf[nb][ks]));
+          asm volatile("" : "+v"(dof[nb][ks]));
+        }
+      }
     if (active) {
       const bool edge = (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S);
-      const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
-      uint32_t pS[2][8];
+      uint32_t pS[NB][2][8];
       constexpr int kRing = 8;
       u32x4 ring[kRing];
       // S^T / dP^T operand i of key block mb: (i even) K rows, (i odd) V rows
@@ -390,49 +406,61 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
       auto read_cols = [&](int i) -> u32x4 {
         return *(const u32x4*)(&k_t[buf][((i % DB) * 32 + col) * TP + (i / DB) * 16 + half * 8]);
       };
-      auto softmax = [&](int mb, const f32x16& sacc, const f32x16& dpacc, auto edge_c) {
+      auto softmax = [&](int nb, int mb, const f32x16& sacc, const f32x16& dpacc, auto edge_c) {
+        const int lim = p.causal ? min(qrow[nb], p.S - 1) : p.S - 1;
 #pragma unroll
         for (int r = 0; r < 16; r += 2) {
           float ds[2];
 #pragma unroll
           for (int e = 0; e < 2; ++e) {
-            float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+            float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2[nb]));
             if (decltype(edge_c)::value) {
               const int kv = kv0 + mb * 32 + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
               pr = kv > lim ? 0.f : pr;
             }
-            ds[e] = pr * (dpacc[r + e] - dl);
+            ds[e] = pr * (dpacc[r + e] - dl[nb]);
           }
-          pS[mb][r >> 1] = Mma<T>::pack(ds[0], ds[1]);
+          pS[nb][mb][r >> 1] = Mma<T>::pack(ds[0], ds[1]);
         }
       };
 #pragma unroll
       for (int i = 0; i < kRing; ++i) ring[i] = read_rows(0, i);
 #pragma unroll
       for (int mb = 0; mb < 2; ++mb) {
-        f32x16 sacc, dpacc;  // written by the matrix ops below into ordinary vector registers
+        f32x16 sacc[NB], dpacc[NB];  // written by the matrix ops below into ordinary vector registers
 #pragma unroll
         for (int i = 0; i < 2 * KS; ++i) {
-          if (i & 1) {
-            if (i == 1) MmaV<T>::first(dpacc, ring[i % kRing], dof[i >> 1]);
-            else MmaV<T>::next(dpacc, ring[i % kRing], dof[i >> 1]);
-          } else {
-            if (i == 0) MmaV<T>::first(sacc, ring[i % kRing], qf[i >> 1]);
-            else MmaV<T>::next(sacc, ring[i % kRing], qf[i >> 1]);
+#pragma unroll
+          for (int nb = 0; nb < NB; ++nb) {
+            f32x16& acc = (i & 1) ? dpacc[nb] : sacc[nb];
+            const u32x4& frag = (i & 1) ? dof[nb][i >> 1] : qf[nb][i >> 1];
+            if (NB == 2) {
+              if (i < 2) MmaV<T>::first_ba(acc, ring[i % kRing], frag);
+              else MmaV<T>::next_ba(acc, ring[i % kRing], frag);
+            } else {
+              if (i < 2) MmaV<T>::first(acc, ring[i % kRing], frag);
+              else MmaV<T>::next(acc, ring[i % kRing], frag);
+            }
           }
           if (i + kRing < 2 * KS) ring[i % kRing] = read_rows(mb, i + kRing);
           else if (mb == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
         mfma_to_valu_gap();
-        if (edge) softmax(mb, sacc, dpacc, std::true_type{});
-        else softmax(mb, sacc, dpacc, std::false_type{});
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          if (edge) softmax(nb, mb, sacc[nb], dpacc[nb], std::true_type{});
+          else softmax(nb, mb, sacc[nb], dpacc[nb], std::false_type{});
+        }
       }
 #pragma unroll
       for (int i = 0; i < 4 * DB; ++i) {
         const int ks = i / DB, db = i % DB, mb = ks >> 1, r0 = (ks & 1) * 4;
-        const u32x4 bS = {pS[mb][r0], pS[mb][r0 + 1], pS[mb][r0 + 2], pS[mb][r0 + 3]};
-        dqacc[db] = Mma<T>::run(ring[i % kRing], bS, dqacc[db]);
+#pragma unroll
+        for (int nb = 0; nb < NB; ++nb) {
+          const u32x4 bS = {pS[nb][mb][r0], pS[nb][mb][r0 + 1], pS[nb][mb][r0 + 2], pS[nb][mb][r0 + 3]};
+          dqacc[db][nb] = Mma<T>::run(ring[i % kRing], bS, dqacc[db][nb]);
+        }
         if (i + kRing < 4 * DB) ring[i % kRing] = read_cols(i + kRing);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -442,17 +470,20 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
     if (t + 2 < nt) load_tile(t + 2);
   }
 
-  if (qrow < p.L) {
-    uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+  for (int nb = 0; nb < NB; ++nb) {
+    if (qrow[nb] < p.L) {
+      uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow[nb] * p.gq_sl;
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = Mma<T>::pack(dqacc[db][g * 4] * p.scale, dqacc[db][g * 4 + 1] * p.scale);
-        w[1] = Mma<T>::pack(dqacc[db][g * 4 + 2] * p.scale, dqacc[db][g * 4 + 3] * p.scale);
-        *(u32x2*)(gq + db * 32 + g * 8 + half * 4) = w;
-      }
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          u32x2 w;
+          w[0] = Mma<T>::pack(dqacc[db][nb][g * 4] * p.scale, dqacc[db][nb][g * 4 + 1] * p.scale);
+          w[1] = Mma<T>::pack(dqacc[db][nb][g * 4 + 2] * p.scale, dqacc[db][nb][g * 4 + 3] * p.scale);
+          *(u32x2*)(gq + db * 32 + g * 8 + half * 4) = w;
+        }
+    }
   }
 }
 
@@ -466,7 +497,13 @@ int launch_td(const BwdM& g, hipStream_t s) {
   hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(256), 0, s, g);
   rc = check_launch("bwd_dkdv_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL((bwd_dq_kernel<T, D>), dim3((unsigned)(g.B * g.Hq * g.n_qt)), dim3(256), 0, s, g);
+  // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
+  const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
+  if (D == 128 && wg256 >= 256) {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
+  } else {
+    hipLaunchKernelGGL((bwd_dq_kernel<T, D, 1>), dim3((unsigned)(g.B * g.Hq * g.n_qt)), dim3(256), 0, s, g);
+  }
   return check_launch("bwd_dq_kernel");
 }
 

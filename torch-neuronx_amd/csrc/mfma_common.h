@@ -67,6 +67,13 @@ struct MmaV<bf16_t> {
   static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
     asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
   }
+  // B operand read from accumulation registers (a long-lived fragment parked there)
+  static __device__ __forceinline__ void first_ba(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  }
+  static __device__ __forceinline__ void next_ba(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_bf16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
+  }
 };
 template <>
 struct MmaV<f16_t> {
@@ -75,6 +82,12 @@ struct MmaV<f16_t> {
   }
   static __device__ __forceinline__ void next(f32x16& d, const u32x4& a, const u32x4& b) {
     asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "v"(b));
+  }
+  static __device__ __forceinline__ void first_ba(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, 0" : "=&v"(d) : "v"(a), "a"(b));
+  }
+  static __device__ __forceinline__ void next_ba(f32x16& d, const u32x4& a, const u32x4& b) {
+    asm volatile("v_mfma_f32_32x32x16_f16 %0, %1, %2, %0" : "+v"(d) : "v"(a), "a"(b));
   }
 };
 // idle cycles after an 8-pass matrix op before the vector unit may touch its result (the
