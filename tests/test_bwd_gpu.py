@@ -43,6 +43,10 @@ BWD_SHAPES = [
     (1, 4, 4, 128, 1024, 128, False),
     (1, 4, 1, 200, 333, 128, True),
     (1, 8, 2, 1024, 1024, 128, True),
+    # enough 256-row query blocks for the 64-rows-per-wavefront dQ kernel, ragged on purpose
+    (4, 16, 4, 1000, 1000, 128, True),
+    (4, 16, 4, 1000, 777, 128, False),
+    (2, 32, 8, 700, 1100, 128, True),
 ]
 
 
