@@ -87,7 +87,7 @@ def test_generic_backward_matrix(amd, gpu_device, shape, dtype):
 
 
 def test_config4_full_size_group_subset(amd, gpu_device):
-    # BASELINE config 4: B=2,Hq=32,Hkv=8,S=4096,D=128 bf16 causal fwd+bwd on the GPU at full
+    # benchmark configuration 4: B=2,Hq=32,Hkv=8,S=4096,D=128 bf16 causal fwd+bwd on the GPU at full
     # size; the oracle checks two whole kv-head groups (4 query heads each) to stay in seconds.
     q, k, v, go = qkv(2, 32, 8, 4096, 4096, 128, dtype=torch.bfloat16, seed=1004, with_do=True)
     out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, is_causal=True)

@@ -103,7 +103,7 @@ def test_decode_all_sequences_empty(amd, gpu_device):
 
 
 def test_config5_full_size(amd, gpu_device):
-    # BASELINE config 5: B=64,Hq=32,Hkv=8,D=128,q_len=1, kv_len ~ U[512,8192] padded to 8192
+    # benchmark configuration 5: B=64,Hq=32,Hkv=8,D=128,q_len=1, kv_len ~ U[512,8192] padded to 8192
     B, Hq, Hkv, S = 64, 32, 8, 8192
     g = torch.Generator().manual_seed(1005)
     q = torch.randn(B, Hq, 1, 128, generator=g).to(torch.bfloat16)

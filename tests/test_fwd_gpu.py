@@ -26,7 +26,7 @@ def _run(amd, q, k, v, dev, **kw):
 
 
 def test_config1_fp32_noncausal_mha(amd, gpu_device):
-    # BASELINE config 1: B=2,H=4,S=128,D=64 fp32, scale 1/8, max-abs <= 1e-5
+    # benchmark configuration 1: B=2,H=4,S=128,D=64 fp32, scale 1/8, max-abs <= 1e-5
     q, k, v = qkv(2, 4, 4, 128, 128, 64, dtype=torch.float32, seed=1001)
     out, lse = _run(amd, q, k, v, gpu_device, scale=0.125)
     ro, rl = oracle_fwd(q, k, v, scale=0.125)
@@ -36,7 +36,7 @@ def test_config1_fp32_noncausal_mha(amd, gpu_device):
 
 
 def test_config2_bf16_causal_mha(amd, gpu_device):
-    # BASELINE config 2: B=4,H=12,S=1024,D=64 bf16 causal; output within 2e-2 of the fp32 oracle
+    # benchmark configuration 2: B=4,H=12,S=1024,D=64 bf16 causal; output within 2e-2 of the fp32 oracle
     q, k, v = qkv(4, 12, 12, 1024, 1024, 64, dtype=torch.bfloat16, seed=1002)
     out, lse = _run(amd, q, k, v, gpu_device, is_causal=True, scale=0.125, force_kernel=MFMA)
     ro, rl = oracle_fwd(q, k, v, is_causal=True, scale=0.125)
@@ -46,7 +46,7 @@ def test_config2_bf16_causal_mha(amd, gpu_device):
 
 
 def test_config3_llama8b_shape_head_subset(amd, gpu_device):
-    # BASELINE config 3 at full size on the GPU; the oracle checks a subset of heads
+    # benchmark configuration 3 at full size on the GPU; the oracle checks a subset of heads
     # (first/last of a group, first/last kv head) to stay within seconds on the CPU.
     q, k, v = qkv(1, 32, 8, 8192, 8192, 128, dtype=torch.bfloat16, seed=1003)
     out, lse = _run(amd, q, k, v, gpu_device, is_causal=True, force_kernel=MFMA)
