@@ -51,5 +51,6 @@ __device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int&
 
 
 int launch_fwd_mfma_w64(const FwdM& g, int dtype, hipStream_t s);
+int launch_fwd_mfma_w32(const FwdM& g, int dtype, int waves, hipStream_t s);
 
 }  // namespace mi355

@@ -369,7 +369,7 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   // for every compute unit and the key loop is long enough to amortise their longer prologue;
   // 128-row workgroups for short or few sequences (measured crossover on MI355X)
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
+  const int force_tile = (p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 || p.force_kernel >= 5) ? 256
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
   int NB = (force_tile == 256 || (force_tile == 0 && wg256 >= 256 && g.S >= 2048)) ? 2 : 1;
   if (NB == 2 && p.q.size[3] == 128 && g.S % 32 != 0) NB = 1;  // the 256-row kernel wants whole key tiles
@@ -387,7 +387,9 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   }
   dim3 grid((unsigned)blocks), block(256);
   const int D = (int)p.q.size[3];
-  if (NB == 2 && D == 128 && g.S % 32 == 0) return launch_fwd_mfma_w64(g, p.dtype, s);
+  if (NB == 2 && D == 128 && g.S % 32 == 0)
+    return p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? launch_fwd_mfma_w64(g, p.dtype, s)
+                                                          : launch_fwd_mfma_w32(g, p.dtype, p.force_kernel == 6 ? 4 : 8, s);
   if (p.dtype == MI355_SDPA_BF16) {
     if (D == 128) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 128, 1>), grid, block, 0, s, g);
     else if (NB == 2) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 64, 2>), grid, block, 0, s, g);

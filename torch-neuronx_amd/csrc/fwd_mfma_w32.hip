@@ -1,0 +1,378 @@
+// Flash-attention forward for gfx950, head dim 128, bf16/f16: the variant for long sequences.
+//
+// One workgroup = 8 wavefronts = 256 query rows of one (batch, query head), ONE workgroup per
+// compute unit: two wavefronts per SIMD, 32 query rows and 256 registers each.
+//
+// Why two wavefronts per SIMD: a wavefront issues at most one instruction every four cycles,
+// whatever the instruction.  A 32x32x16 matrix op keeps the matrix pipe busy for 32 cycles, the
+// softmax of the scores it produces costs about 20 cycles on the vector unit (v_exp_f32 is half
+// rate), and around those sit LDS reads, waits and scalar bookkeeping.  A single wavefront per
+// SIMD runs out of issue slots long before either pipe is full; with two, one wavefront's
+// vector and LDS instructions issue under the other's matrix op.  LDS bandwidth is not a
+// concern (a compute unit reads 256 B/clk with ds_read_b128; this kernel asks for half that).
+//
+// Inside a wavefront the key loop is still software pipelined by hand, because a wavefront
+// issues in order: the softmax of a 32-key tile is split in two halves that ride on the matrix
+// ops of two different phases, LDS operands are fetched three matrix ops ahead through a
+// four-entry register ring, and a scheduling barrier after every matrix op keeps the compiler
+// from regrouping the stream.  The loop carries no row maximum: see kTrig.
+// Products are computed transposed (S^T = K Q^T, O^T = V^T P^T) as in fwd_mfma.hip, so the
+// softmax statistics are per-lane scalars and P goes from accumulator to B operand in registers.
+//
+// Numerics: torch_neuronx/_sdpa_math.py:51-95 (float32 accumulation and softmax, probabilities
+// rounded to the input dtype for P*V only, dead rows give zeros and lse = -inf).
+#include <type_traits>
+
+#include "fwd_mfma.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int D = 128;
+constexpr int BN = 32;
+constexpr int KS = D / 16, DB = D / 32;
+constexpr int KROW = D + 8;   // K tile row pitch (elements): conflict-free 128-bit reads
+constexpr int VP = D + 32;    // V tile row pitch: 320 bytes, conflict-free row writes and transposing reads
+constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
+
+template <typename T, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) {
+  constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
+  constexpr int KLD = 512 / NT;  // 16-byte chunks of K and of V per thread
+  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KROW];
+  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][BN * VP];
+
+  int b, h, qt;
+  decode_block(p, b, h, qt);
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int col = lane & 31, half = lane >> 5;
+  const int q0 = qt * BM;
+  const int qw0 = q0 + wave * 32;
+  const int qrow = qw0 + col;
+  const int qw_last = qw0 + 31;
+
+  const uint16_t* qp = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
+  const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
+  const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
+
+  u32x4 qf[KS];
+  {
+    const uint16_t* qr = qp + (int64_t)min(qrow, p.L - 1) * p.q_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16);
+  }
+
+  int nt = (p.S + BN - 1) / BN;
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+  const int nt_w = p.causal ? min(nt, qw_last / BN + 1) : nt;
+
+  // ---- staging: every thread moves KLD 16-byte chunks of the K tile and of the V tile ------------
+  // Both tiles sit in LDS as they sit in memory, [key][d].  K is the A operand of S^T = K Q^T as it
+  // is; V^T, the A operand of O^T = V^T P^T, is produced by the transposing LDS read
+  // (ds_read_b64_tr_b16), so no transposition is done on the vector unit.
+  // Two staging sets each: a tile is fetched from global memory two iterations before it is
+  // written to LDS, so a fetch has about two tile times to land.
+  u32x4 kreg[2][KLD], vreg[2][KLD];
+  const int k_chunk = tid & 15, k_row = tid >> 4;  // rows k_row + i * NT / 16
+  // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
+  // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
+  // instruction with no address arithmetic on the vector unit.  S is a multiple of BN here (the
+  // launcher guarantees it), so no row needs clamping.
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, 0x7fffffff, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, 0x7fffffff, 0x00020000);
+  uint32_t k_off[KLD], v_off[KLD];
+#pragma unroll
+  for (int i = 0; i < KLD; ++i) {
+    k_off[i] = (uint32_t)(((k_row + i * (NT / 16)) * p.k_sl + k_chunk * 8) * 2);
+    v_off[i] = (uint32_t)(((k_row + i * (NT / 16)) * p.v_sl + k_chunk * 8) * 2);
+  }
+  const int k_tile_bytes = (int)(BN * p.k_sl * 2), v_tile_bytes = (int)(BN * p.v_sl * 2);
+  auto load_k = [&](int set, int t) {
+    const int base = min(t, nt - 1) * k_tile_bytes;
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i], base, 0);
+  };
+  auto load_v = [&](int set, int t) {
+    const int base = min(t, nt - 1) * v_tile_bytes;
+#pragma unroll
+    for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i], base, 0);
+  };
+  auto store_k = [&](int set, int buf) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i)
+      *(u32x4*)(&k_lds[buf][(k_row + i * (NT / 16)) * KROW + k_chunk * 8]) = kreg[set][i];
+  };
+  auto store_v = [&](int set, int buf) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i)
+      *(u32x4*)(&v_lds[buf][(k_row + i * (NT / 16)) * VP + k_chunk * 8]) = vreg[set][i];
+  };
+  // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
+  // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
+  // 8 + i / 4, 12 + i / 4: four keys at d = 4 (i / 4) + i % 4 = i.  A lane of the 32x32x16 A
+  // operand (d row lane % 32, key half lane / 32) takes two such reads: keys 4 half .. +3 and
+  // 8 + 4 half .. +3 of a 16-key step, the order in which the S^T accumulator holds them.
+  const int tr_jj = lane & 15, tr_g = lane >> 4;
+  const int tr_base = ((tr_g >> 1) * 4 + (tr_jj >> 2)) * VP + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  auto tr_read = [&](const uint16_t* ptr) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
+    return __builtin_bit_cast(u32x2, v);
+  };
+
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(oacc[i]);
+  float m_run = -INFINITY, l_run = 0.f;
+  const float c = p.scale * kLog2eF;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+
+  auto mask_tile = [&](f32x16& s, int kv0) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kv = kv0 + (r >> 2) * 8 + half * 4 + (r & 3);
+      if (kv > lim) s[r] = -INFINITY;
+    }
+  };
+  auto is_edge = [&](int kv0) { return (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S); };
+
+  float m_new = -INFINITY, mc = 0.f, alpha = 1.f;
+  bool need_rescale = false;
+  auto tile_max = [&](const f32x16& s) {
+    float t = fmaxf(s[0], s[1]);
+#pragma unroll
+    for (int r = 2; r < 16; r += 2) t = fmaxf(fmaxf(t, s[r]), s[r + 1]);  // v_max3
+    return t;
+  };
+  // The softmax reference of a row (m_run, folded into mc) is NOT the running maximum.  The fast
+  // path never looks for a maximum at all: probabilities are formed against the current reference
+  // and only their sum is watched.  A lane's sum over its 16 keys above kTrig means that some
+  // probability outgrew 2^kLazy-ish headroom (or that there is no reference yet): then, and only
+  // then, the slow path finds the true tile maximum, raises the reference of every row that beat
+  // it by more than kLazy in the exponent, rescales those rows' accumulators and redoes the
+  // tile's probabilities.  Exact arithmetic: numerator and row sum always carry the same
+  // reference, and lse = reference * scale + ln(sum).
+  constexpr float kTrig = 8192.f;  // 16 probabilities of at most 2^kLazy stay below this
+  auto raise_reference = [&](float t0) {
+    const float tm = fmaxf(t0, __shfl_xor(t0, 32, 64));
+    const bool up = (tm - m_run) * c > kLazy;  // false for NaN (-inf minus -inf)
+    m_new = up ? tm : m_run;
+    const float m_use = (m_new == -INFINITY) ? 0.f : m_new;
+    alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+    mc = m_use * c;
+    need_rescale = __builtin_amdgcn_ballot_w64(up) != 0;
+  };
+
+  // Softmax of one register pair, in three stages so that consecutive pairs can be staggered by
+  // hand (the chain read S -> fma -> exp2 -> add/pack is strictly dependent and a wavefront
+  // issues in order).  Pair j of 8: accumulator registers 2 j, 2 j + 1.
+  float xs[2][2], pv[2][2];
+  auto stage1 = [&](const f32x16& sv, int j) {
+    xs[j & 1][0] = fmaf(sv[2 * j], c, -mc);
+    xs[j & 1][1] = fmaf(sv[2 * j + 1], c, -mc);
+  };
+  auto stage2 = [&](int j) {
+    pv[j & 1][0] = __builtin_amdgcn_exp2f(xs[j & 1][0]);
+    pv[j & 1][1] = __builtin_amdgcn_exp2f(xs[j & 1][1]);
+  };
+  auto stage3 = [&](int j, uint32_t (&pk)[8], float& ps) {
+    ps += pv[j & 1][0] + pv[j & 1][1];
+    asm volatile("" : "+v"(ps));  // keeps the add in its slot (left alone it sinks below the loop body)
+    pk[j] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
+  };
+  // Pairs 0..3 hold the tile's first 16 keys (the first contraction step of P*V), pairs 4..7 the
+  // last 16.  Four pairs are spread over the eight matrix ops of a phase:
+  //   slot 2q: exp2 of pair q, scaling of pair q+1     slot 2q+1: sum and packing of pair q
+  auto softmax_slot = [&](const f32x16& sv, int base, int slot, uint32_t (&pk)[8], float& ps) {
+    const int q = slot >> 1;
+    if ((slot & 1) == 0) {
+      stage2(base + q);
+      if (q + 1 < 4) stage1(sv, base + q + 1);
+    } else {
+      stage3(base + q, pk, ps);
+    }
+  };
+
+  // ---- prologue ----------------------------------------------------------------------------------
+  load_k(0, 0);
+  load_v(0, 0);
+  load_k(1, 1);
+  store_k(0, 0);
+  store_v(0, 0);
+  store_k(1, 1);
+  __syncthreads();
+  load_k(0, 2);
+  load_k(1, 3);
+  load_v(1, 1);
+  load_v(0, 2);
+  f32x16 s_a, s_b;
+  uint32_t pk_a[8], pk_b[8];
+  float ps_a = 0.f, ps_b = 0.f;
+  bool first = true;  // no reference yet: the first tile goes through the slow path whatever its sums
+  {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const u32x4 a = *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
+      s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
+    }
+    if (is_edge(0)) mask_tile(s_a, 0);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {  // first half of tile 0 (redone by the slow path of iteration 0)
+      stage1(s_a, j);
+      stage2(j);
+      stage3(j, pk_a, ps_a);
+    }
+  }
+  __syncthreads();  // K buffer 0 is rewritten during the first iteration
+  // LDS operands travel through a four-entry register ring, three matrix ops ahead of their use;
+  // the ring runs across iterations (the first three K fragments of a tile are requested at the
+  // end of the previous iteration, right after the barrier that publishes the tile)
+  u32x4 ring[4];
+#pragma unroll
+  for (int ks = 0; ks < 3; ++ks) ring[ks] = *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
+
+  // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
+  // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
+  //   phase A   S^T(t+1) = K(t+1) Q^T on the matrix pipe  |  softmax of the last 16 keys of tile t
+  //   check     sum of tile t against kTrig; rare slow path
+  //   phase B   O^T += V^T(t) P^T(t) on the matrix pipe    |  softmax of the first 16 keys of tile
+  //             t+1, LDS stores of tiles t+2 / t+1, fetches of tiles t+4 / t+3
+  auto iteration = [&](int t, auto parity, f32x16& scur, f32x16& snext, uint32_t (&pk)[8], uint32_t (&pkn)[8],
+                       float& ps, float& psn) {
+    constexpr int par = decltype(parity)::value;  // t & 1, known at compile time
+    const uint16_t* kt = &k_lds[par ^ 1][col * KROW + half * 8];
+    const uint16_t* kn = &k_lds[par][col * KROW + half * 8];  // tile t+2, stored during this iteration
+    const uint16_t* vt = &v_lds[par][tr_base];
+    auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
+    auto read_v = [&](int i) {  // d block i % 4, 16-key step i / 4
+      const u32x2 lo = tr_read(vt + (i >> 2) * 16 * VP + (i & 3) * 32);
+      const u32x2 hi = tr_read(vt + ((i >> 2) * 16 + 8) * VP + (i & 3) * 32);
+      return u32x4{lo[0], lo[1], hi[0], hi[1]};
+    };
+    __builtin_amdgcn_sched_barrier(0);
+    stage1(scur, 4);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase A -------------------------------------------------------------------------------
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
+      else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
+      snext = Mma<T>::run(ring[ks & 3], qf[ks], ks == 0 ? zero16 : snext);
+      softmax_slot(scur, 4, ks, pk, ps);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    // ---- check ---------------------------------------------------------------------------------
+    const bool trig = first || !(ps <= kTrig);  // (NaN also lands here)
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(trig) != 0, 0)) {
+      first = false;
+      raise_reference(tile_max(scur));
+      if (need_rescale) {
+        l_run *= alpha;
+#pragma unroll
+        for (int i = 0; i < DB; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+        m_run = m_new;
+      }
+      ps = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {  // the whole tile again, against the new reference
+        stage1(scur, j);
+        stage2(j);
+        stage3(j, pk, ps);
+      }
+    }
+    l_run += ps;
+    psn = 0.f;
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase B -------------------------------------------------------------------------------
+    // The first matrix op needs nothing of S^T(t+1): it is issued before anything reads that tile,
+    // so the wait for the last op of phase A is spent on the matrix pipe.  The barrier sits before
+    // slot 6: by then every wavefront has stored its share of tiles t+2 (K) and t+1 (V) and has
+    // issued its last read of V(t); behind it the first K fragments of the next phase A are requested.
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
+      if (i == 6) __syncthreads();
+      if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
+      if (i == 6) ring[0] = *(const u32x4*)(kn), ring[1] = *(const u32x4*)(kn + 16);
+      if (i == 7) ring[2] = *(const u32x4*)(kn + 32);
+      const int ks2 = i >> 2, db = i & 3;
+      const u32x4 b0 = {pk[ks2 * 4], pk[ks2 * 4 + 1], pk[ks2 * 4 + 2], pk[ks2 * 4 + 3]};
+      oacc[db] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db]);
+      if (i == 0) {
+        if (__builtin_expect(is_edge((t + 1) * BN), 0)) mask_tile(snext, (t + 1) * BN);  // rare
+        stage1(snext, 0);
+      } else {
+        softmax_slot(snext, 0, i - 1, pkn, psn);
+      }
+      if (i == 0) store_k(par, par);  // tile t+2
+      if (i == 1) store_v(par ^ 1, par ^ 1);  // tile t+1
+      if (i == 4) load_k(par, t + 4);
+      if (i == 5) load_v(par ^ 1, t + 3);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    softmax_slot(snext, 0, 7, pkn, psn);
+  };
+  // a wavefront whose rows lie above the causal diagonal of the remaining tiles only feeds LDS
+  auto idle_step = [&](int t, auto parity) {
+    constexpr int par = decltype(parity)::value;
+    store_k(par, par);
+    store_v(par ^ 1, par ^ 1);
+    load_k(par, t + 4);
+    load_v(par ^ 1, t + 3);
+    __syncthreads();
+  };
+
+  int t = 0;
+  for (; t + 1 < nt_w; t += 2) {
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
+  }
+  if (t < nt_w) {  // odd count: t is even here
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+    ++t;
+  }
+  for (; t < nt; ++t) {
+    if (t & 1) idle_step(t, std::integral_constant<int, 1>{});
+    else idle_step(t, std::integral_constant<int, 0>{});
+  }
+
+  // ---- epilogue ------------------------------------------------------------------------------------
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (qrow < p.L) {
+    uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
+        w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
+        *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
+      }
+    if (p.lse && half == 0)
+      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+  }
+}
+
+}  // namespace
+
+int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int waves, hipStream_t s) {
+  FwdM g = g0;
+  g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
+  const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
+  dim3 grid((unsigned)blocks), block(64 * waves);
+  if (waves == 8) {
+    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_w32_kernel<bf16_t, 8>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((fwd_w32_kernel<f16_t, 8>), grid, block, 0, s, g);
+  } else {
+    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_w32_kernel<bf16_t, 4>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((fwd_w32_kernel<f16_t, 4>), grid, block, 0, s, g);
+  }
+  return check_launch("fwd_w32_kernel");
+}
+
+}  // namespace mi355
