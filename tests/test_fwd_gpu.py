@@ -93,6 +93,24 @@ def test_mfma_forward_matrix(amd, gpu_device, shape, dtype, tile):
     assert max_abs(lse, rl) <= 2e-3
 
 
+def test_mfma_forward_rows_far_apart(amd, gpu_device):
+    # key / value rows 512 KiB apart: one (batch, head) spans 2 GiB, beyond the 32-bit row
+    # addressing of the head-dim-128 kernels, so the call is served by the 64-bit-address kernel
+    B, Hq, Hkv, L, S, E = 1, 2, 1, 160, 4096, 128
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=torch.bfloat16, seed=77)
+    pitch = 262144
+    assert S * pitch * 2 >= 2**31
+    kd = torch.empty(B, Hkv, S, pitch, dtype=torch.bfloat16, device=gpu_device)[..., :E]
+    vd = torch.empty(B, Hkv, S, pitch, dtype=torch.bfloat16, device=gpu_device)[..., :E]
+    kd.copy_(k)
+    vd.copy_(v)
+    out, lse = amd.sdpa_forward(q.to(gpu_device), kd, vd, is_causal=False, force_kernel=MFMA)
+    torch.cuda.synchronize()
+    ro, rl = oracle_fwd(q, k, v)
+    assert max_abs(out, ro) <= 2e-2
+    assert max_abs(lse, rl) <= 2e-3
+
+
 GENERIC_SHAPES = SHAPES[:9] + [
     (1, 4, 4, 256, 256, 256, False),
     (1, 4, 2, 512, 512, 256, True),

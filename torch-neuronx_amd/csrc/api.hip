@@ -192,7 +192,7 @@ int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
   int kernel = p->force_kernel;
   if (kernel == 0) kernel = fwd_mfma_supported(*p, &why) ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
   if (kernel == MI355_SDPA_KERNEL_MFMA || kernel == MI355_SDPA_KERNEL_MFMA_T128 ||
-      kernel == MI355_SDPA_KERNEL_MFMA_T256 || kernel == 5 || kernel == 6)
+      kernel == MI355_SDPA_KERNEL_MFMA_T256)
     return launch_fwd_mfma(*p, s);
   if (kernel == MI355_SDPA_KERNEL_GENERIC) return launch_fwd_generic(*p, s);
   return set_error("SDPA: unknown kernel id %d", kernel), MI355_SDPA_ERR_INVALID;

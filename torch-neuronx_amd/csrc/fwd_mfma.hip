@@ -3,12 +3,11 @@
 // Work split: one workgroup = 4 wavefronts; each wavefront owns NB blocks of 32 query rows
 // (NB = 2: 256 query rows per workgroup, one workgroup per compute unit with the full 512
 // registers per lane; NB = 1: 128 rows, two workgroups per compute unit, for short sequences)
-// and walks the keys in tiles of 64.
+// and walks the keys in tiles of 64.  This file serves head dim 64, and head dim 128 only
+// when the strides are too large for the 32-bit addressing of fwd_mfma_w32.hip.
 //
-// What bounds this kernel is LDS bandwidth, not the matrix pipe: every MFMA needs a fresh
-// 1 KB A operand from LDS and a compute unit delivers roughly 64 B/clk.  With NB = 2 each K
-// or V^T fragment read from LDS feeds two MFMAs (two query blocks held in registers), which
-// halves the LDS bytes per flop.
+// With NB = 2 each K or V^T fragment read from LDS feeds two MFMAs (two query blocks held in
+// registers), which halves the LDS reads per flop.
 //
 // Both products are computed TRANSPOSED so that the softmax needs no shuffle and P never
 // leaves registers:
@@ -365,18 +364,24 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
-  // 256-row workgroups (one per compute unit, half the LDS traffic per flop) once there is one
-  // for every compute unit and the key loop is long enough to amortise their longer prologue;
-  // 128-row workgroups for short or few sequences (measured crossover on MI355X)
+  const int D = (int)p.q.size[3];
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  const int force_tile = (p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 || p.force_kernel >= 5) ? 256
+  const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
+  // Head dim 128 goes to the kernels of fwd_mfma_w32.hip, which address K / V rows with 32-bit
+  // byte offsets from the start of a (batch, head).  256-row workgroups (one per compute unit)
+  // once every compute unit gets at least one (two when the causal mask makes half of them
+  // light) and the key loop is long; 128-row workgroups (two per compute unit) for short or few
+  // sequences (measured crossovers on MI355X).
+  if (D == 128 && (int64_t)g.S * g.k_sl * 2 < (1ll << 31) && (int64_t)g.S * g.v_sl * 2 < (1ll << 31)) {
+    const bool big = (g.S >= 2048 && wg256 >= (g.causal ? 512 : 256)) || (!g.causal && g.S >= 1024 && wg256 >= 512);
+    const int rows = force_tile ? force_tile : big ? 256 : 128;
+    return launch_fwd_mfma_w32(g, p.dtype, rows / 32, s);
+  }
+  // head dim 64 (and head dim 128 with strides beyond 32-bit offsets): the kernel above, with 256
+  // rows per workgroup under the same conditions
   int NB = (force_tile == 256 || (force_tile == 0 && wg256 >= 256 && g.S >= 2048)) ? 2 : 1;
-  if (NB == 2 && p.q.size[3] == 128 && g.S % 32 != 0) NB = 1;  // the 256-row kernel wants whole key tiles
-  // ... and addresses K / V rows with 32-bit byte offsets from the start of a (batch, head)
-  if (NB == 2 && p.q.size[3] == 128 &&
-      ((int64_t)g.S * g.k_sl * 2 >= (1ll << 31) || (int64_t)g.S * g.v_sl * 2 >= (1ll << 31)))
-    NB = 1;
+  if (D == 128) NB = 1;
   const int BM = 128 * NB;
   g.n_qt = (g.L + BM - 1) / BM;
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
@@ -386,10 +391,6 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   dim3 grid((unsigned)blocks), block(256);
-  const int D = (int)p.q.size[3];
-  if (NB == 2 && D == 128 && g.S % 32 == 0)
-    return p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? launch_fwd_mfma_w64(g, p.dtype, s)
-                                                          : launch_fwd_mfma_w32(g, p.dtype, p.force_kernel == 6 ? 4 : 8, s);
   if (p.dtype == MI355_SDPA_BF16) {
     if (D == 128) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 128, 1>), grid, block, 0, s, g);
     else if (NB == 2) hipLaunchKernelGGL((fwd_mfma_kernel<bf16_t, 64, 2>), grid, block, 0, s, g);

@@ -1,21 +1,26 @@
-// Flash-attention forward for gfx950, head dim 128, bf16/f16: the variant for long sequences.
+// Flash-attention forward for gfx950, head dim 128, bf16/f16.
 //
-// One workgroup = 8 wavefronts = 256 query rows of one (batch, query head), ONE workgroup per
-// compute unit: two wavefronts per SIMD, 32 query rows and 256 registers each.
+// One workgroup = WAVES wavefronts of 32 query rows each, all of one (batch, query head):
+// WAVES = 8 (256 rows, one workgroup per compute unit) for long sequences, WAVES = 4 (128 rows,
+// two workgroups per compute unit) for short or few ones.  Either way a SIMD hosts two
+// wavefronts with 256 registers each.
 //
 // Why two wavefronts per SIMD: a wavefront issues at most one instruction every four cycles,
 // whatever the instruction.  A 32x32x16 matrix op keeps the matrix pipe busy for 32 cycles, the
 // softmax of the scores it produces costs about 20 cycles on the vector unit (v_exp_f32 is half
 // rate), and around those sit LDS reads, waits and scalar bookkeeping.  A single wavefront per
-// SIMD runs out of issue slots long before either pipe is full; with two, one wavefront's
-// vector and LDS instructions issue under the other's matrix op.  LDS bandwidth is not a
-// concern (a compute unit reads 256 B/clk with ds_read_b128; this kernel asks for half that).
+// SIMD (64 query rows, so that every LDS fragment feeds two matrix ops) runs out of issue slots
+// long before either pipe is full; with two, one wavefront's vector and LDS instructions issue
+// under the other's matrix op.  LDS bandwidth does not bind (a compute unit reads about
+// 256 B/clk with ds_read_b128; this kernel asks for a third of that).  What the kernel runs
+// into instead is the power limit: with random operands a pure stream of these matrix ops
+// sustains about 1.7 PFLOP/s on MI355X (2.3 with zeros), and every LDS read, global load and
+// vector op costs some of that.
 //
-// Inside a wavefront the key loop is still software pipelined by hand, because a wavefront
-// issues in order: the softmax of a 32-key tile is split in two halves that ride on the matrix
-// ops of two different phases, LDS operands are fetched three matrix ops ahead through a
-// four-entry register ring, and a scheduling barrier after every matrix op keeps the compiler
-// from regrouping the stream.  The loop carries no row maximum: see kTrig.
+// Inside a wavefront the key loop is software pipelined by hand, because a wavefront issues in
+// order: the softmax of a 32-key tile is split in two halves that ride on the matrix ops of two
+// different phases, and LDS operands are fetched AHEAD matrix ops ahead through a register
+// ring.  The loop carries no row maximum: see kTrig.
 // Products are computed transposed (S^T = K Q^T, O^T = V^T P^T) as in fwd_mfma.hip, so the
 // softmax statistics are per-lane scalars and P goes from accumulator to B operand in registers.
 //
@@ -33,6 +38,7 @@ constexpr int BN = 32;
 constexpr int KS = D / 16, DB = D / 32;
 constexpr int KROW = D + 8;   // K tile row pitch (elements): conflict-free 128-bit reads
 constexpr int VP = D + 32;    // V tile row pitch: 320 bytes, conflict-free row writes and transposing reads
+constexpr int AHEAD = 4;  // LDS operands are requested this many matrix ops ahead (at most 6)
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
 template <typename T, int WAVES>
@@ -45,7 +51,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   int b, h, qt;
   decode_block(p, b, h, qt);
   const int hk = h / (p.Hq / p.Hkv);
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps per-wavefront tests on the scalar unit
   const int col = lane & 31, half = lane >> 5;
   const int q0 = qt * BM;
   const int qw0 = q0 + wave * 32;
@@ -77,10 +84,12 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   const int k_chunk = tid & 15, k_row = tid >> 4;  // rows k_row + i * NT / 16
   // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
   // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
-  // instruction with no address arithmetic on the vector unit.  S is a multiple of BN here (the
-  // launcher guarantees it), so no row needs clamping.
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, 0x7fffffff, 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, 0x7fffffff, 0x00020000);
+  // instruction with no address arithmetic on the vector unit.  The resources end with the last
+  // key row of this (batch, head): rows of a ragged last tile beyond it read as zeros (their
+  // scores are masked, and a zero V row keeps 0 * V finite).
+  const int k_bytes = (int)(((int64_t)(p.S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(p.S - 1) * p.v_sl + D) * 2);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
   uint32_t k_off[KLD], v_off[KLD];
 #pragma unroll
   for (int i = 0; i < KLD; ++i) {
@@ -136,7 +145,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       if (kv > lim) s[r] = -INFINITY;
     }
   };
-  auto is_edge = [&](int kv0) { return (p.causal && kv0 + BN - 1 > qw0) || (kv0 + BN > p.S); };
+  // first tile that needs masking: the one that reaches this wavefront's first row on the causal
+  // diagonal (qw0 is a multiple of BN), or a ragged last tile
+  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (p.S % BN) ? p.S / BN : 0x7fffffff);
 
   float m_new = -INFINITY, mc = 0.f, alpha = 1.f;
   bool need_rescale = false;
@@ -149,7 +160,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   // The softmax reference of a row (m_run, folded into mc) is NOT the running maximum.  The fast
   // path never looks for a maximum at all: probabilities are formed against the current reference
   // and only their sum is watched.  A lane's sum over its 16 keys above kTrig means that some
-  // probability outgrew 2^kLazy-ish headroom (or that there is no reference yet): then, and only
+  // probability outgrew 2^kLazy-ish headroom: then, and only
   // then, the slow path finds the true tile maximum, raises the reference of every row that beat
   // it by more than kLazy in the exponent, rescales those rows' accumulators and redoes the
   // tile's probabilities.  Exact arithmetic: numerator and row sum always carry the same
@@ -210,16 +221,17 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   f32x16 s_a, s_b;
   uint32_t pk_a[8], pk_b[8];
   float ps_a = 0.f, ps_b = 0.f;
-  bool first = true;  // no reference yet: the first tile goes through the slow path whatever its sums
   {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
       const u32x4 a = *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
       s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
     }
-    if (is_edge(0)) mask_tile(s_a, 0);
+    if (t_edge == 0) mask_tile(s_a, 0);
+    raise_reference(tile_max(s_a));  // the first reference is the maximum of the first tile
+    m_run = m_new;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {  // first half of tile 0 (redone by the slow path of iteration 0)
+    for (int j = 0; j < 4; ++j) {  // first half of tile 0
       stage1(s_a, j);
       stage2(j);
       stage3(j, pk_a, ps_a);
@@ -229,9 +241,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   // LDS operands travel through a four-entry register ring, three matrix ops ahead of their use;
   // the ring runs across iterations (the first three K fragments of a tile are requested at the
   // end of the previous iteration, right after the barrier that publishes the tile)
-  u32x4 ring[4];
+  u32x4 ring[8];
 #pragma unroll
-  for (int ks = 0; ks < 3; ++ks) ring[ks] = *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
+  for (int ks = 0; ks < AHEAD; ++ks) ring[ks] = *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
 
   // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
   // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
@@ -257,16 +269,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
     // ---- phase A -------------------------------------------------------------------------------
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      if (ks + 3 < KS) ring[(ks + 3) & 3] = read_k(ks + 3);
-      else ring[(ks + 3) & 3] = read_v(ks + 3 - KS);
-      snext = Mma<T>::run(ring[ks & 3], qf[ks], ks == 0 ? zero16 : snext);
+      if (ks + AHEAD < KS) ring[ks + AHEAD] = read_k(ks + AHEAD);
+      else ring[ks + AHEAD - KS] = read_v(ks + AHEAD - KS);
+      snext = Mma<T>::run(ring[ks], qf[ks], ks == 0 ? zero16 : snext);
       softmax_slot(scur, 4, ks, pk, ps);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- check ---------------------------------------------------------------------------------
-    const bool trig = first || !(ps <= kTrig);  // (NaN also lands here)
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(trig) != 0, 0)) {
-      first = false;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ps <= kTrig)) != 0, 0)) {  // (NaN also lands here)
       raise_reference(tile_max(scur));
       if (need_rescale) {
         l_run *= alpha;
@@ -295,14 +305,20 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
 #pragma unroll
     for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
       if (i == 6) __syncthreads();
-      if (i + 3 < 8) ring[(i + 3 + KS) & 3] = read_v(i + 3);
-      if (i == 6) ring[0] = *(const u32x4*)(kn), ring[1] = *(const u32x4*)(kn + 16);
-      if (i == 7) ring[2] = *(const u32x4*)(kn + 32);
+      if (i + AHEAD < 8) ring[i + AHEAD] = read_v(i + AHEAD);
+      if (i == 6) {
+#pragma unroll
+        for (int j = 0; j < (AHEAD + 1) / 2; ++j) ring[j] = *(const u32x4*)(kn + j * 16);
+      }
+      if (i == 7) {
+#pragma unroll
+        for (int j = (AHEAD + 1) / 2; j < AHEAD; ++j) ring[j] = *(const u32x4*)(kn + j * 16);
+      }
       const int ks2 = i >> 2, db = i & 3;
       const u32x4 b0 = {pk[ks2 * 4], pk[ks2 * 4 + 1], pk[ks2 * 4 + 2], pk[ks2 * 4 + 3]};
-      oacc[db] = Mma<T>::run(ring[(i + KS) & 3], b0, oacc[db]);
+      oacc[db] = Mma<T>::run(ring[i], b0, oacc[db]);
       if (i == 0) {
-        if (__builtin_expect(is_edge((t + 1) * BN), 0)) mask_tile(snext, (t + 1) * BN);  // rare
+        if (__builtin_expect(t + 1 >= t_edge, 0)) mask_tile(snext, (t + 1) * BN);  // rare
         stage1(snext, 0);
       } else {
         softmax_slot(snext, 0, i - 1, pkn, psn);
@@ -364,6 +380,11 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int waves, hipStream_t s) {
   FwdM g = g0;
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
+  if (blocks == 0) return MI355_SDPA_OK;
+  if (blocks > 0x7fffffff) {
+    set_error("SDPA: too many query tiles (%lld)", (long long)blocks);
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
   dim3 grid((unsigned)blocks), block(64 * waves);
   if (waves == 8) {
     if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_w32_kernel<bf16_t, 8>), grid, block, 0, s, g);
