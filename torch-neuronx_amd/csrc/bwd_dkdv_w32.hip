@@ -1,0 +1,293 @@
+// Flash-attention backward, dK and dV, for gfx950, head dim 128, bf16/f16.
+//
+// One workgroup = 8 wavefronts = 128 keys of one (batch, kv head); it loops over the query
+// heads of the group (the GQA sum of decompositions.py:2595-2598 happens in registers) and over
+// 64-row query tiles.  The four matrix products of a tile are split between TWO wavefronts per
+// 32-key block, which sit on the same SIMD:
+//
+//   role A   S = Q K^T            P = exp2(c S - lse)            dV^T += dO^T P
+//   role B   dP = dO V^T          dS = P (dP - delta)            dK^T += Q^T dS
+//
+// so that each wavefront holds one accumulator (64 registers) and one operand (K or V
+// fragments, 32 registers) and fits in 256 registers: with two wavefronts per SIMD the vector
+// work of one issues under the matrix ops of the other (a wavefront issues at most one
+// instruction every four cycles, so a single wavefront per SIMD cannot keep both pipes busy).
+// Role B needs P from role A: A leaves it in LDS (packed to the input dtype, as it is fed to the
+// matrix pipe), and B works ONE TILE BEHIND A, so the only synchronisation is the one barrier
+// per tile that the staging needs anyway.  Three tile buffers are live: the one being staged,
+// A's and B's.
+//
+// Q and dO tiles sit in LDS row-major as they sit in memory; the transposed operands (dO^T, Q^T)
+// come out of the transposing LDS read ds_read_b64_tr_b16, so nothing is transposed on the
+// vector unit.  Math follows torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows
+// with lse = -inf give zero gradients, scale multiplies dK once at the end.
+#include "bwd_mfma.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int D = 128, BQ = 64, BK = 128;
+constexpr int KS = D / 16, DB = D / 32;
+constexpr int RP = D + 8;  // row pitch of the tiles (elements)
+constexpr int TILE = BQ * RP;
+constexpr int kSmemBytes = 2 * 3 * TILE * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
+
+template <typename T>
+__global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
+  uint16_t* const q_t = (uint16_t*)smem;          // [3][TILE]
+  uint16_t* const do_t = q_t + 3 * TILE;          // [3][TILE]
+  uint32_t* const pex = (uint32_t*)(do_t + 3 * TILE);  // [2][4 key blocks][64 lanes][16]
+  float* const lse_s = (float*)(pex + 2 * 4 * 1024);   // [3][BQ]
+  float* const dl_s = lse_s + 3 * BQ;                  // [3][BQ]
+
+  const int streams = p.B * p.Hkv;
+  const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
+  const int st = blockIdx.x % streams;
+  const int b = st / p.Hkv, hk = st % p.Hkv;
+  const int rep = p.Hq / p.Hkv;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int role = wave >> 2, kb = wave & 3;  // wavefronts w and w + 4 share a SIMD and a key block
+  const int col = lane & 31, half = lane >> 5;
+  const int k0 = kt * BK, kw0 = k0 + kb * 32;
+  const int key = kw0 + col;
+
+  // this lane's key as B operand: K fragments for S = Q K^T (role A), V fragments for dP = dO V^T (role B)
+  u32x4 frag[KS];
+  {
+    const int kc = min(key, p.S - 1);
+    const uint16_t* r = role ? (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl
+                             : (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) frag[ks] = *(const u32x4*)(r + half * 8 + ks * 16);
+  }
+
+  const int nqs = (p.L + BQ - 1) / BQ;
+  const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+  const int per_head = nqs - qs_begin;
+  const int n_items = rep * per_head;
+  auto item_head = [&](int it) { return hk * rep + it / per_head; };
+  auto item_q0 = [&](int it) { return (qs_begin + it % per_head) * BQ; };
+
+  // ---- staging: every thread moves two 16-byte chunks of the Q tile and two of the dO tile ------
+  // Buffer resources end with the last row of the batch (the tile offset travels in the vector
+  // offset, which is the part the hardware checks against that bound): rows past L read as zeros
+  // or as another head's rows, and are switched off through lse = +inf.
+  const int64_t q_ext = ((int64_t)(p.Hq - 1) * p.q_sh + (int64_t)(p.L - 1) * p.q_sl + D) * 2;
+  const int64_t go_ext = ((int64_t)(p.Hq - 1) * p.go_sh + (int64_t)(p.L - 1) * p.go_sl + D) * 2;
+  const __amdgpu_buffer_rsrc_t q_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.q + b * p.q_sb), 0, (int)q_ext, 0x00020000);
+  const __amdgpu_buffer_rsrc_t go_rsrc =
+      __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.go + b * p.go_sb), 0, (int)go_ext, 0x00020000);
+  const int s_row = tid >> 4, s_ch = tid & 15;  // rows s_row, s_row + 32
+  uint32_t q_off[2], go_off[2];
+#pragma unroll
+  for (int n = 0; n < 2; ++n) {
+    q_off[n] = (uint32_t)(((s_row + 32 * n) * p.q_sl + s_ch * 8) * 2);
+    go_off[n] = (uint32_t)(((s_row + 32 * n) * p.go_sl + s_ch * 8) * 2);
+  }
+  u32x4 sq[2], sgo[2];
+  float lse_r = 0.f, dl_r = 0.f;
+  auto load_item = [&](int it) {
+    const int h = item_head(it), q0 = item_q0(it);
+    const uint32_t qb = (uint32_t)((h * p.q_sh + (int64_t)q0 * p.q_sl) * 2);
+    const uint32_t gb = (uint32_t)((h * p.go_sh + (int64_t)q0 * p.go_sl) * 2);
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      sq[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, q_off[n] + qb, 0, 0);
+      sgo[n] = __builtin_amdgcn_raw_buffer_load_b128(go_rsrc, go_off[n] + gb, 0, 0);
+    }
+    if (tid < BQ) {
+      const int qi = q0 + tid;
+      const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + min(qi, p.L - 1);
+      const float l = p.lse[idx];
+      // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
+      lse_r = (qi < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
+      dl_r = qi < p.L ? p.delta[idx] : 0.f;
+    }
+  };
+  auto store_item = [&](int buf) {
+#pragma unroll
+    for (int n = 0; n < 2; ++n) {
+      *(u32x4*)(&q_t[buf * TILE + (s_row + 32 * n) * RP + s_ch * 8]) = sq[n];
+      *(u32x4*)(&do_t[buf * TILE + (s_row + 32 * n) * RP + s_ch * 8]) = sgo[n];
+    }
+    if (tid < BQ) lse_s[buf * BQ + tid] = lse_r, dl_s[buf * BQ + tid] = dl_r;
+  };
+
+  // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
+  // row k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
+  // 8 + i / 4, 12 + i / 4: four rows at d = i.  A lane of the 32x32x16 A operand (d row lane % 32,
+  // row half lane / 32) takes two such reads: rows 4 half .. +3 and 8 + 4 half .. +3 of a 16-row
+  // step, the order in which the score accumulators hold them.
+  const int tr_jj = lane & 15, tr_g = lane >> 4;
+  const int tr_base = ((tr_g >> 1) * 4 + (tr_jj >> 2)) * RP + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  auto tr_read = [&](const uint16_t* ptr) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
+    return __builtin_bit_cast(u32x2, v);
+  };
+  // operand i = 4 * (16-row step) + d block of the transposed tile
+  auto read_cols = [&](const uint16_t* tile, int i) {
+    const u32x2 lo = tr_read(tile + tr_base + (i >> 2) * 16 * RP + (i & 3) * 32);
+    const u32x2 hi = tr_read(tile + tr_base + ((i >> 2) * 16 + 8) * RP + (i & 3) * 32);
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+  };
+  // operand i = 8 * (32-row block) + contraction step of the row-major tile
+  auto read_rows = [&](const uint16_t* tile, int i) {
+    return *(const u32x4*)(tile + ((i >> 3) * 32 + col) * RP + (i & 7) * 16 + half * 8);
+  };
+
+  f32x16 acc[DB];  // dV^T (role A) or dK^T (role B): d rows x this lane's key
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(acc[i]);
+  const float c = p.scale * kLog2eF;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  constexpr int AHEAD = 4;
+
+  // scores of the 64 x 32 tile: sc[mq] = rows(tile)[32 mq ..] * frag
+  auto scores = [&](const uint16_t* tile, f32x16 (&sc)[2]) {
+    u32x4 ring[8];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) ring[i] = read_rows(tile, i);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (i + AHEAD < 16) ring[(i + AHEAD) & 7] = read_rows(tile, i + AHEAD);
+      sc[i >> 3] = Mma<T>::run(ring[i & 7], frag[i & 7], (i & 7) == 0 ? zero16 : sc[i >> 3]);
+    }
+  };
+  // acc += cols(tile)^T * pk, pk = the 64 x 32 tile of P or dS packed from the accumulator layout
+  auto accumulate = [&](const uint16_t* tile, const uint32_t (&pk)[2][8]) {
+    u32x4 ring[8];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) ring[i] = read_cols(tile, i);
+#pragma unroll
+    for (int i = 0; i < 16; ++i) {
+      if (i + AHEAD < 16) ring[(i + AHEAD) & 7] = read_cols(tile, i + AHEAD);
+      const int ks4 = i >> 2, db = i & 3, mq = ks4 >> 1, r0 = (ks4 & 1) * 4;
+      const u32x4 bb = {pk[mq][r0], pk[mq][r0 + 1], pk[mq][r0 + 2], pk[mq][r0 + 3]};
+      acc[db] = Mma<T>::run(ring[i & 7], bb, acc[db]);
+    }
+  };
+
+  auto role_a = [&](int it, int tb, int pb) {
+    const int q0 = item_q0(it);
+    if (p.causal && q0 + BQ - 1 < kw0) return;  // every key of this block lies above the diagonal
+    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= p.S);
+    f32x16 sc[2];
+    scores(q_t + tb * TILE, sc);
+    uint32_t pk[2][8];
+#pragma unroll
+    for (int mq = 0; mq < 2; ++mq)
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const f32x4 l4 = *(const f32x4*)(&lse_s[tb * BQ + mq * 32 + r4 * 8 + half * 4]);
+        float pr[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, -l4[e]));
+          if (edge) {
+            const int qi = q0 + mq * 32 + r4 * 8 + half * 4 + e;
+            pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
+          }
+        }
+        pk[mq][r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pk[mq][r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+      }
+    uint32_t* px = pex + ((pb * 4 + kb) * 64 + lane) * 16;
+#pragma unroll
+    for (int mq = 0; mq < 2; ++mq) {
+      *(u32x4*)(px + mq * 8) = u32x4{pk[mq][0], pk[mq][1], pk[mq][2], pk[mq][3]};
+      *(u32x4*)(px + mq * 8 + 4) = u32x4{pk[mq][4], pk[mq][5], pk[mq][6], pk[mq][7]};
+    }
+    accumulate(do_t + tb * TILE, pk);
+  };
+  auto role_b = [&](int it, int tb, int pb) {
+    const int q0 = item_q0(it);
+    if (p.causal && q0 + BQ - 1 < kw0) return;
+    f32x16 dp[2];
+    scores(do_t + tb * TILE, dp);
+    const uint32_t* px = pex + ((pb * 4 + kb) * 64 + lane) * 16;
+    uint32_t pk[2][8];
+#pragma unroll
+    for (int mq = 0; mq < 2; ++mq) {
+      const u32x4 w0 = *(const u32x4*)(px + mq * 8), w1 = *(const u32x4*)(px + mq * 8 + 4);
+      const uint32_t w[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const f32x4 d4 = *(const f32x4*)(&dl_s[tb * BQ + mq * 32 + r4 * 8 + half * 4]);
+        float ds[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const float pr = Mma<T>::unpack(w[r4 * 2 + (e >> 1)], e & 1);
+          ds[e] = pr * (dp[mq][r4 * 4 + e] - d4[e]);
+        }
+        pk[mq][r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pk[mq][r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
+      }
+    }
+    accumulate(q_t + tb * TILE, pk);
+  };
+
+  if (n_items > 0) {
+    load_item(0);
+    store_item(0);
+    __syncthreads();
+    if (n_items > 1) load_item(1);
+  }
+  // iteration `it`: role A works on tile it, role B on tile it - 1; tile it + 1 goes to LDS
+  int tb_a = 0, tb_b = 2;  // tile buffers of A's and B's tiles: it % 3 and (it - 1) % 3
+  for (int it = 0; it <= n_items && n_items > 0; ++it) {
+    if (role == 0) {
+      if (it < n_items) role_a(it, tb_a, it & 1);
+    } else {
+      if (it >= 1) role_b(it - 1, tb_b, (it - 1) & 1);
+    }
+    const int tb_n = tb_a == 2 ? 0 : tb_a + 1;
+    if (it + 1 < n_items) store_item(tb_n);
+    __syncthreads();
+    if (it + 2 < n_items) load_item(it + 2);
+    tb_b = tb_a, tb_a = tb_n;
+  }
+
+  if (key < p.S) {
+    uint16_t* g = role ? (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl
+                       : (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
+    const float sc = role ? p.scale : 1.f;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int gq = 0; gq < 4; ++gq) {
+        u32x2 w;
+        w[0] = Mma<T>::pack(acc[db][gq * 4] * sc, acc[db][gq * 4 + 1] * sc);
+        w[1] = Mma<T>::pack(acc[db][gq * 4 + 2] * sc, acc[db][gq * 4 + 3] * sc);
+        *(u32x2*)(g + db * 32 + gq * 8 + half * 4) = w;
+      }
+  }
+}
+
+template <typename T>
+int launch_t(const BwdM& g, hipStream_t s) {
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+  if (attr != hipSuccess) {
+    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dkdv_w32_kernel: %s", kSmemBytes, hipGetErrorString(attr));
+    return MI355_SDPA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(512), kSmemBytes, s, g);
+  return check_launch("bwd_dkdv_w32_kernel");
+}
+
+}  // namespace
+
+bool bwd_dkdv_w32_fits(const BwdM& g) {
+  // 32-bit byte offsets from the start of a batch for Q and dO
+  const int64_t q_ext = ((int64_t)(g.Hq - 1) * g.q_sh + (int64_t)(g.L + BQ) * g.q_sl + D) * 2;
+  const int64_t go_ext = ((int64_t)(g.Hq - 1) * g.go_sh + (int64_t)(g.L + BQ) * g.go_sl + D) * 2;
+  return q_ext < (1ll << 31) && go_ext < (1ll << 31) && g.q_sh >= 0 && g.q_sl >= 0 && g.go_sh >= 0 && g.go_sl >= 0;
+}
+
+int launch_bwd_dkdv_w32(const BwdM& g, int dtype, hipStream_t s) {
+  return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t>(g, s) : launch_t<f16_t>(g, s);
+}
+
+}  // namespace mi355

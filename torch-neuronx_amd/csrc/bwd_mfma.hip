@@ -20,23 +20,10 @@
 // gradients, scale multiplies dQ and dK once at the end.
 #include <type_traits>
 
-#include "mfma_common.h"
+#include "bwd_mfma.h"
 
 namespace mi355 {
 namespace {
-
-struct BwdM {
-  const void *go, *q, *k, *v, *out;
-  const float* lse;
-  void *gq, *gk, *gv;
-  float* delta;
-  int64_t go_sb, go_sh, go_sl, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl;
-  int64_t o_sb, o_sh, o_sl, gq_sb, gq_sh, gq_sl, gk_sb, gk_sh, gk_sl, gv_sb, gv_sh, gv_sl;
-  int B, Hq, Hkv, L, S;
-  int n_qt, n_kt;
-  int causal, xcd_map;
-  float scale;
-};
 
 template <typename T>
 __device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
@@ -494,8 +481,12 @@ int launch_td(const BwdM& g, hipStream_t s) {
   hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, s, g);
   int rc = check_launch("bwd_delta_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(256), 0, s, g);
-  rc = check_launch("bwd_dkdv_kernel");
+  if (D == 128 && bwd_dkdv_w32_fits(g)) {
+    rc = launch_bwd_dkdv_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
+  } else {
+    hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(256), 0, s, g);
+    rc = check_launch("bwd_dkdv_kernel");
+  }
   if (rc) return rc;
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);

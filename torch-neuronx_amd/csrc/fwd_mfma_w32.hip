@@ -84,9 +84,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   const int k_chunk = tid & 15, k_row = tid >> 4;  // rows k_row + i * NT / 16
   // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
   // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
-  // instruction with no address arithmetic on the vector unit.  The resources end with the last
-  // key row of this (batch, head): rows of a ragged last tile beyond it read as zeros (their
-  // scores are masked, and a zero V row keeps 0 * V finite).
+  // instruction with one addition on the vector unit.  The resources end with the last key row
+  // of this (batch, head), and the whole offset travels in the vector offset, the part the
+  // hardware checks against that bound: rows of a ragged last tile beyond it read as zeros
+  // (their scores are masked, and a zero V row keeps 0 * V finite).
   const int k_bytes = (int)(((int64_t)(p.S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(p.S - 1) * p.v_sl + D) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
@@ -98,14 +99,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   }
   const int k_tile_bytes = (int)(BN * p.k_sl * 2), v_tile_bytes = (int)(BN * p.v_sl * 2);
   auto load_k = [&](int set, int t) {
-    const int base = min(t, nt - 1) * k_tile_bytes;
+    const uint32_t base = (uint32_t)(min(t, nt - 1) * k_tile_bytes);
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i], base, 0);
+    for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i] + base, 0, 0);
   };
   auto load_v = [&](int set, int t) {
-    const int base = min(t, nt - 1) * v_tile_bytes;
+    const uint32_t base = (uint32_t)(min(t, nt - 1) * v_tile_bytes);
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i], base, 0);
+    for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i] + base, 0, 0);
   };
   auto store_k = [&](int set, int buf) {
 #pragma unroll

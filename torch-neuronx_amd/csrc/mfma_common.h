@@ -36,6 +36,9 @@ struct Mma<bf16_t> {
     v2 r = {(__bf16)lo, (__bf16)hi};
     return __builtin_bit_cast(uint32_t, r);
   }
+  static __device__ __forceinline__ float unpack(uint32_t w, int hi) {  // element 0 or 1 of a packed pair
+    return __builtin_bit_cast(float, hi ? (w & 0xffff0000u) : (w << 16));
+  }
 };
 template <>
 struct Mma<f16_t> {
@@ -47,6 +50,11 @@ struct Mma<f16_t> {
     typedef __attribute__((ext_vector_type(2))) _Float16 v2;
     v2 r = {(_Float16)lo, (_Float16)hi};
     return __builtin_bit_cast(uint32_t, r);
+  }
+  static __device__ __forceinline__ float unpack(uint32_t w, int hi) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 v2;
+    const v2 r = __builtin_bit_cast(v2, w);
+    return (float)(hi ? r[1] : r[0]);
   }
 };
 
