@@ -6,16 +6,16 @@
 // 32-key block, which sit on the same SIMD:
 //
 //   role A   S = Q K^T            P = exp2(c S - lse)            dV^T += dO^T P
-//   role B   dP = dO V^T          dS = P (dP - delta)            dK^T += Q^T dS
+//   role B   dS = P (dP - delta)  dK^T += Q^T dS                 dP = dO V^T of the next tile
 //
 // so that each wavefront holds one accumulator (64 registers) and one operand (K or V
 // fragments, 32 registers) and fits in 256 registers: with two wavefronts per SIMD the vector
 // work of one issues under the matrix ops of the other (a wavefront issues at most one
 // instruction every four cycles, so a single wavefront per SIMD cannot keep both pipes busy).
 // Role B needs P from role A: A leaves it in LDS (packed to the input dtype, as it is fed to the
-// matrix pipe), and B works ONE TILE BEHIND A, so the only synchronisation is the one barrier
-// per tile that the staging needs anyway.  Three tile buffers are live: the one being staged,
-// A's and B's.
+// matrix pipe), and B finishes a tile ONE ITERATION BEHIND A, so the only synchronisation is the
+// one barrier per tile that the staging needs anyway; B's vector work then runs under A's first
+// matrix ops and A's under B's.  Three tile buffers are live: the one being staged, A's and B's.
 //
 // Q and dO tiles sit in LDS row-major as they sit in memory; the transposed operands (dO^T, Q^T)
 // come out of the transposing LDS read ds_read_b64_tr_b16, so nothing is transposed on the
@@ -202,11 +202,17 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
     accumulate(do_t + tb * TILE, pk);
   };
+  // Role B splits a tile over two iterations, so that its vector work falls on role A's first
+  // matrix ops and its matrix ops on role A's vector work: dP of tile it at the end of iteration
+  // it, dS and dK of that tile at the start of iteration it + 1.
+  f32x16 dp[2];
+  auto role_b_scores = [&](int it, int tb) {
+    if (p.causal && item_q0(it) + BQ - 1 < kw0) return;
+    scores(do_t + tb * TILE, dp);
+  };
   auto role_b = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
     if (p.causal && q0 + BQ - 1 < kw0) return;
-    f32x16 dp[2];
-    scores(do_t + tb * TILE, dp);
     const uint32_t* px = pex + ((pb * 4 + kb) * 64 + lane) * 16;
     uint32_t pk[2][8];
 #pragma unroll
@@ -235,18 +241,27 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     if (n_items > 1) load_item(1);
   }
   // iteration `it`: role A works on tile it, role B on tile it - 1; tile it + 1 goes to LDS
-  int tb_a = 0, tb_b = 2;  // tile buffers of A's and B's tiles: it % 3 and (it - 1) % 3
-  for (int it = 0; it <= n_items && n_items > 0; ++it) {
-    if (role == 0) {
-      if (it < n_items) role_a(it, tb_a, it & 1);
-    } else {
-      if (it >= 1) role_b(it - 1, tb_b, (it - 1) & 1);
-    }
+  // (one loop per role, with the same barriers: in a shared loop the registers that one role
+  // carries across iterations would count as live in the other role's code)
+  int tb_a = 0, tb_b = 2;  // tile buffers of tiles it and it - 1: it % 3 and (it - 1) % 3
+  auto stage_and_sync = [&](int it) {
     const int tb_n = tb_a == 2 ? 0 : tb_a + 1;
     if (it + 1 < n_items) store_item(tb_n);
     __syncthreads();
     if (it + 2 < n_items) load_item(it + 2);
     tb_b = tb_a, tb_a = tb_n;
+  };
+  if (role == 0) {
+    for (int it = 0; it <= n_items && n_items > 0; ++it) {
+      if (it < n_items) role_a(it, tb_a, it & 1);
+      stage_and_sync(it);
+    }
+  } else {
+    for (int it = 0; it <= n_items && n_items > 0; ++it) {
+      if (it >= 1) role_b(it - 1, tb_b, (it - 1) & 1);
+      if (it < n_items) role_b_scores(it, tb_a);
+      stage_and_sync(it);
+    }
   }
 
   if (key < p.S) {
