@@ -28,9 +28,14 @@ namespace {
 
 constexpr int D = 128, BQ = 64, BK = 128;
 constexpr int KS = D / 16, DB = D / 32;
-constexpr int RP = D + 8;  // row pitch of the tiles (elements)
-constexpr int TILE = BQ * RP;
+constexpr int TILE = BQ * D;  // tiles are XOR swizzled, not padded: see swz16
 constexpr int kSmemBytes = 2 * 3 * TILE * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
+
+// A tile row is 16 chunks of 16 bytes; chunk c of row r lives at chunk c ^ swz16(r).  Both ways
+// of reading a tile are then free of bank conflicts: 16 consecutive rows reading the same chunk
+// (row-major A operand) land in 16 different chunks, and 4 consecutive rows reading the same 4
+// consecutive chunks (one transposing read) land in 4 different 64-byte windows.
+__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
 
 template <typename T>
 __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
@@ -110,8 +115,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   auto store_item = [&](int buf) {
 #pragma unroll
     for (int n = 0; n < 2; ++n) {
-      *(u32x4*)(&q_t[buf * TILE + (s_row + 32 * n) * RP + s_ch * 8]) = sq[n];
-      *(u32x4*)(&do_t[buf * TILE + (s_row + 32 * n) * RP + s_ch * 8]) = sgo[n];
+      // (row s_row + 32 has the swizzle of row s_row)
+      *(u32x4*)(&q_t[buf * TILE + (s_row + 32 * n) * D + ((s_ch ^ swz16(s_row)) << 3)]) = sq[n];
+      *(u32x4*)(&do_t[buf * TILE + (s_row + 32 * n) * D + ((s_ch ^ swz16(s_row)) << 3)]) = sgo[n];
     }
     if (tid < BQ) lse_s[buf * BQ + tid] = lse_r, dl_s[buf * BQ + tid] = dl_r;
   };
@@ -121,8 +127,26 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // 8 + i / 4, 12 + i / 4: four rows at d = i.  A lane of the 32x32x16 A operand (d row lane % 32,
   // row half lane / 32) takes two such reads: rows 4 half .. +3 and 8 + 4 half .. +3 of a 16-row
   // step, the order in which the score accumulators hold them.
+  // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
+  // row k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
+  // 8 + i / 4, 12 + i / 4: four rows at d = i.  A lane of the 32x32x16 A operand (d row lane % 32,
+  // row half lane / 32) takes two such reads: rows 4 half .. +3 and 8 + 4 half .. +3 of a 16-row
+  // step, the order in which the score accumulators hold them.
+  // The element offsets inside a tile depend on the swizzle of the row a lane reads, which is not
+  // additive in the d block / contraction step: one offset register per combination.
   const int tr_jj = lane & 15, tr_g = lane >> 4;
-  const int tr_base = ((tr_g >> 1) * 4 + (tr_jj >> 2)) * RP + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
+  int tr_off[2][DB];  // [second read of a pair][d block], without the 16-row step (a multiple of 16 rows)
+#pragma unroll
+  for (int sec = 0; sec < 2; ++sec)
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int row = 8 * sec + (tr_g >> 1) * 4 + (tr_jj >> 2);  // within the 16-row step
+      const int d = db * 32 + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
+      tr_off[sec][db] = row * D + (((d >> 3) ^ swz16(row)) << 3) + (d & 7);
+    }
+  int row_off[KS];  // [contraction step], without the 32-row block
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ swz16(col)) << 3);
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   auto tr_read = [&](const uint16_t* ptr) {
     const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
@@ -130,13 +154,13 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
   // operand i = 4 * (16-row step) + d block of the transposed tile
   auto read_cols = [&](const uint16_t* tile, int i) {
-    const u32x2 lo = tr_read(tile + tr_base + (i >> 2) * 16 * RP + (i & 3) * 32);
-    const u32x2 hi = tr_read(tile + tr_base + ((i >> 2) * 16 + 8) * RP + (i & 3) * 32);
+    const u32x2 lo = tr_read(tile + tr_off[0][i & 3] + (i >> 2) * 16 * D);
+    const u32x2 hi = tr_read(tile + tr_off[1][i & 3] + (i >> 2) * 16 * D);
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
   // operand i = 8 * (32-row block) + contraction step of the row-major tile
   auto read_rows = [&](const uint16_t* tile, int i) {
-    return *(const u32x4*)(tile + ((i >> 3) * 32 + col) * RP + (i & 7) * 16 + half * 8);
+    return *(const u32x4*)(tile + row_off[i & 7] + (i >> 3) * 32 * D);
   };
 
   f32x16 acc[DB];  // dV^T (role A) or dK^T (role B): d rows x this lane's key
@@ -194,11 +218,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
         }
         pk[mq][r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pk[mq][r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
       }
-    uint32_t* px = pex + ((pb * 4 + kb) * 64 + lane) * 16;
+    uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;  // [4 groups of 4 words][lane][4]
 #pragma unroll
     for (int mq = 0; mq < 2; ++mq) {
-      *(u32x4*)(px + mq * 8) = u32x4{pk[mq][0], pk[mq][1], pk[mq][2], pk[mq][3]};
-      *(u32x4*)(px + mq * 8 + 4) = u32x4{pk[mq][4], pk[mq][5], pk[mq][6], pk[mq][7]};
+      *(u32x4*)(px + (2 * mq) * 256) = u32x4{pk[mq][0], pk[mq][1], pk[mq][2], pk[mq][3]};
+      *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{pk[mq][4], pk[mq][5], pk[mq][6], pk[mq][7]};
     }
     accumulate(do_t + tb * TILE, pk);
   };
@@ -213,11 +237,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   auto role_b = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
     if (p.causal && q0 + BQ - 1 < kw0) return;
-    const uint32_t* px = pex + ((pb * 4 + kb) * 64 + lane) * 16;
+    const uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;
     uint32_t pk[2][8];
 #pragma unroll
     for (int mq = 0; mq < 2; ++mq) {
-      const u32x4 w0 = *(const u32x4*)(px + mq * 8), w1 = *(const u32x4*)(px + mq * 8 + 4);
+      const u32x4 w0 = *(const u32x4*)(px + (2 * mq) * 256), w1 = *(const u32x4*)(px + (2 * mq + 1) * 256);
       const uint32_t w[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
