@@ -1,0 +1,256 @@
+// Flash-attention backward, dQ, for gfx950, head dim 128, bf16/f16.
+//
+// One workgroup = 8 wavefronts of 32 query rows each (256 rows of one (batch, query head)), one
+// workgroup per compute unit, two wavefronts per SIMD with 256 registers each; it walks the keys
+// in tiles of 32:
+//
+//   S^T = K Q^T, dP^T = V dO^T      (A = K / V rows from LDS, B = Q / dO fragments in registers)
+//   P^T = exp2(c S^T - lse), dS^T = P^T (dP^T - delta)
+//   dQ^T += K^T dS^T                (A = K^T from the transposing LDS read, B = dS^T packed
+//                                    straight from the accumulators)
+//
+// The scores of tile t + 1 are issued before the vector work of tile t, so that a wavefront's
+// own matrix ops cover part of it; the rest is covered by the other wavefront of the SIMD (a
+// wavefront issues at most one instruction every four cycles, so one wavefront per SIMD cannot
+// keep the matrix and the vector pipe busy together).
+//
+// K and V tiles sit in LDS row-major and XOR swizzled (see swz16).  Math follows
+// torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows with lse = -inf give zero
+// gradients, scale multiplies dQ once at the end.
+#include "bwd_mfma.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int D = 128, BM = 256, BN = 32;
+constexpr int KS = D / 16, DB = D / 32;
+constexpr int TILE = BN * D;
+constexpr int AHEAD = 4;
+
+// A tile row is 16 chunks of 16 bytes; chunk c of row r lives at chunk c ^ swz16(r).  Both ways
+// of reading a tile are then free of bank conflicts: 16 consecutive rows reading the same chunk
+// (row-major A operand) land in 16 different chunks, and 4 consecutive rows reading the same 4
+// consecutive chunks (one transposing read) land in 4 different 64-byte windows.
+__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
+
+template <typename T>
+__global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
+  __shared__ __attribute__((aligned(16))) uint16_t k_t[3][TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_t[3][TILE];
+
+  int b, h, qt;
+  {
+    const int bid = blockIdx.x, rep = p.Hq / p.Hkv;
+    const int n_qt = (p.L + BM - 1) / BM;
+    if (p.xcd_map) {
+      const int per_xcd = (p.B * p.Hkv) / 8, xcd = bid & 7;
+      int r = bid >> 3;
+      const int hg = r % rep;
+      r /= rep;
+      const int sl = r % per_xcd;
+      r /= per_xcd;
+      qt = n_qt - 1 - r;
+      const int stream = sl * 8 + xcd;
+      b = stream / p.Hkv, h = (stream % p.Hkv) * rep + hg;
+    } else {
+      const int heads = p.B * p.Hq;
+      qt = n_qt - 1 - bid / heads;
+      b = (bid % heads) / p.Hq, h = (bid % heads) % p.Hq;
+    }
+  }
+  const int hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col = lane & 31, half = lane >> 5;
+  const int q0 = qt * BM, qw0 = q0 + wave * 32;
+  const int qrow = qw0 + col, qc = min(qrow, p.L - 1);
+
+  // this lane's query row as B operand of the score products
+  u32x4 qf[KS], dof[KS];
+  float lse2, dl;
+  {
+    const uint16_t* qr = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl + half * 8;
+    const uint16_t* gr = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl + half * 8;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16), dof[ks] = *(const u32x4*)(gr + ks * 16);
+    const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc;
+    const float l = p.lse[idx];
+    // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
+    lse2 = (qrow < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
+    dl = p.delta[idx];
+  }
+
+  int nt = (p.S + BN - 1) / BN;
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BN + 1) : nt;  // tiles with work for this wavefront
+  // first tile that needs masking: the one that reaches this wavefront's first row on the causal
+  // diagonal (qw0 is a multiple of BN), or a ragged last tile
+  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (p.S % BN) ? p.S / BN : 0x7fffffff);
+  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+
+  // ---- staging: every thread moves one 16-byte chunk of the K tile and one of the V tile ----------
+  // Buffer resources end with the last key row of this (batch, head), and the whole offset travels
+  // in the vector offset, the part the hardware checks against that bound: rows of a ragged last
+  // tile beyond it read as zeros (their probabilities are masked to zero).
+  const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
+  const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
+  const int k_bytes = (int)(((int64_t)(p.S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(p.S - 1) * p.v_sl + D) * 2);
+  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
+  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
+  const int s_row = tid >> 4, s_ch = tid & 15;
+  const uint32_t k_off = (uint32_t)((s_row * p.k_sl + s_ch * 8) * 2), v_off = (uint32_t)((s_row * p.v_sl + s_ch * 8) * 2);
+  const uint32_t k_tile_bytes = (uint32_t)(BN * p.k_sl * 2), v_tile_bytes = (uint32_t)(BN * p.v_sl * 2);
+  const int s_lds = s_row * D + ((s_ch ^ swz16(s_row)) << 3);
+  u32x4 kreg, vreg;
+  auto load_tile = [&](int t) {
+    const uint32_t tt = (uint32_t)min(t, nt - 1);
+    kreg = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off + tt * k_tile_bytes, 0, 0);
+    vreg = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off + tt * v_tile_bytes, 0, 0);
+  };
+  auto store_tile = [&](int buf) {
+    *(u32x4*)(&k_t[buf][s_lds]) = kreg;
+    *(u32x4*)(&v_t[buf][s_lds]) = vreg;
+  };
+
+  // element offsets inside a tile (the swizzle is not additive in the d block / contraction step:
+  // one offset register per combination)
+  const int tr_jj = lane & 15, tr_g = lane >> 4;
+  int tr_off[2][DB];  // [second read of a pair][d block], without the 16-key step
+#pragma unroll
+  for (int sec = 0; sec < 2; ++sec)
+#pragma unroll
+    for (int db = 0; db < DB; ++db) {
+      const int row = 8 * sec + (tr_g >> 1) * 4 + (tr_jj >> 2);
+      const int d = db * 32 + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
+      tr_off[sec][db] = row * D + (((d >> 3) ^ swz16(row)) << 3) + (d & 7);
+    }
+  int row_off[KS];
+#pragma unroll
+  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ swz16(col)) << 3);
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
+  // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
+  // 8 + i / 4, 12 + i / 4: four keys at d = i.  A lane of the 32x32x16 A operand (d row lane % 32,
+  // key half lane / 32) takes two such reads: keys 4 half .. +3 and 8 + 4 half .. +3 of a 16-key
+  // step, the order in which the score accumulators hold them.
+  auto tr_read = [&](const uint16_t* ptr) {
+    const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
+    return __builtin_bit_cast(u32x2, v);
+  };
+  // operand i = 4 * (16-key step) + d block of K^T
+  auto read_cols = [&](const uint16_t* tile, int i) {
+    const u32x2 lo = tr_read(tile + tr_off[0][i & 3] + (i >> 2) * 16 * D);
+    const u32x2 hi = tr_read(tile + tr_off[1][i & 3] + (i >> 2) * 16 * D);
+    return u32x4{lo[0], lo[1], hi[0], hi[1]};
+  };
+
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(dqacc[i]);
+  const float c = p.scale * kLog2eF;
+  const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+
+  // S^T and dP^T of the tile in buffer `buf`: operand i = 2 * contraction step + (0: K rows, 1: V rows)
+  auto scores = [&](int buf, f32x16& sacc, f32x16& dpacc) {
+    u32x4 ring[8];
+    auto rd = [&](int i) { return *(const u32x4*)(((i & 1) ? v_t[buf] : k_t[buf]) + row_off[i >> 1]); };
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) ring[i] = rd(i);
+#pragma unroll
+    for (int i = 0; i < 2 * KS; ++i) {
+      if (i + AHEAD < 2 * KS) ring[(i + AHEAD) & 7] = rd(i + AHEAD);
+      if (i & 1) dpacc = Mma<T>::run(ring[i & 7], dof[i >> 1], i == 1 ? zero16 : dpacc);
+      else sacc = Mma<T>::run(ring[i & 7], qf[i >> 1], i == 0 ? zero16 : sacc);
+    }
+  };
+  // dS^T of tile t, packed as the B operand of dQ^T += K^T dS^T
+  auto softmax = [&](int t, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
+    const bool edge = t >= t_edge;
+#pragma unroll
+    for (int r = 0; r < 16; r += 2) {
+      float ds[2];
+#pragma unroll
+      for (int e = 0; e < 2; ++e) {
+        float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+        if (edge) {
+          const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
+          pr = kv > lim ? 0.f : pr;
+        }
+        ds[e] = pr * (dpacc[r + e] - dl);
+      }
+      pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
+    }
+  };
+  auto accumulate = [&](int buf, const uint32_t (&pS)[8]) {
+    u32x4 ring[8];
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) ring[i] = read_cols(k_t[buf], i);
+#pragma unroll
+    for (int i = 0; i < 2 * DB; ++i) {
+      if (i + AHEAD < 2 * DB) ring[(i + AHEAD) & 7] = read_cols(k_t[buf], i + AHEAD);
+      const int r0 = (i >> 2) * 4;
+      const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
+      dqacc[i & 3] = Mma<T>::run(ring[i & 7], bS, dqacc[i & 3]);
+    }
+  };
+
+  // Iteration t: scores of tile t + 1, vector work of tile t, dQ of tile t; tile t + 2 goes to LDS.
+  // Buffers: tile t in t % 3.
+  load_tile(0);
+  store_tile(0);
+  load_tile(1);
+  store_tile(1);
+  __syncthreads();
+  load_tile(2);
+  f32x16 s_a, dp_a, s_b, dp_b;
+  if (nt_w > 0) scores(0, s_a, dp_a);
+  int buf = 0;  // t % 3
+  auto iteration = [&](int t, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
+    const int bn = buf == 2 ? 0 : buf + 1, bnn = bn == 2 ? 0 : bn + 1;
+    if (t < nt_w) {
+      if (t + 1 < nt_w) scores(bn, snext, dpnext);
+      uint32_t pS[8];
+      softmax(t, scur, dpcur, pS);
+      accumulate(buf, pS);
+    }
+    store_tile(bnn);  // tile t + 2 (buffer of tile t - 1, whose last readers passed the previous barrier)
+    __syncthreads();
+    load_tile(t + 3);
+    buf = bn;
+  };
+  int t = 0;
+  for (; t + 1 < nt; t += 2) {
+    iteration(t, s_a, dp_a, s_b, dp_b);
+    iteration(t + 1, s_b, dp_b, s_a, dp_a);
+  }
+  if (t < nt) iteration(t, s_a, dp_a, s_b, dp_b);
+
+  if (qrow < p.L) {
+    uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = Mma<T>::pack(dqacc[db][g * 4] * p.scale, dqacc[db][g * 4 + 1] * p.scale);
+        w[1] = Mma<T>::pack(dqacc[db][g * 4 + 2] * p.scale, dqacc[db][g * 4 + 3] * p.scale);
+        *(u32x2*)(gq + db * 32 + g * 8 + half * 4) = w;
+      }
+  }
+}
+
+}  // namespace
+
+bool bwd_dq_w32_fits(const BwdM& g) {
+  // 32-bit byte offsets from the start of a (batch, kv head) for K and V
+  return (int64_t)(g.S + BN) * g.k_sl * 2 < (1ll << 31) && (int64_t)(g.S + BN) * g.v_sl * 2 < (1ll << 31) && g.k_sl >= 0 && g.v_sl >= 0;
+}
+
+int launch_bwd_dq_w32(const BwdM& g, int dtype, hipStream_t s) {
+  const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
+  if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dq_w32_kernel<bf16_t>), dim3((unsigned)blocks), dim3(512), 0, s, g);
+  else hipLaunchKernelGGL((bwd_dq_w32_kernel<f16_t>), dim3((unsigned)blocks), dim3(512), 0, s, g);
+  return check_launch("bwd_dq_w32_kernel");
+}
+
+}  // namespace mi355

@@ -22,5 +22,8 @@ struct BwdM {
 // tensors do not fit its 32-bit addressing and the caller must use the kernel in bwd_mfma.hip
 bool bwd_dkdv_w32_fits(const BwdM& g);
 int launch_bwd_dkdv_w32(const BwdM& g, int dtype, hipStream_t s);
+// dQ for head dim 128 with two wavefronts per SIMD (bwd_dq_w32.hip), same convention
+bool bwd_dq_w32_fits(const BwdM& g);
+int launch_bwd_dq_w32(const BwdM& g, int dtype, hipStream_t s);
 
 }  // namespace mi355

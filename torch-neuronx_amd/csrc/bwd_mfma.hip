@@ -490,6 +490,8 @@ int launch_td(const BwdM& g, hipStream_t s) {
   if (rc) return rc;
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
+  if (D == 128 && wg256 >= 256 && bwd_dq_w32_fits(g))
+    return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
   if (D == 128 && wg256 >= 256) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
   } else {
