@@ -161,6 +161,75 @@ def test_masks_and_bias(amd, gpu_device, mask_kind, dtype):
     assert max_abs(lse, rl) <= (2e-5 if dtype is torch.float32 else 2e-3)
 
 
+MASKED_MFMA_CASES = [
+    # B, Hq, Hkv, L, S, mask kind, causal
+    (2, 4, 2, 96, 160, "float_same", False),
+    (2, 4, 2, 96, 160, "float32", False),
+    (2, 4, 4, 130, 76, "float_bcast_q", False),     # (B,1,1,S): one bias row for every query
+    (1, 8, 2, 300, 512, "float_bcast_bh", True),    # (1,1,L,S) together with the causal mask
+    (2, 4, 2, 96, 160, "bool", False),
+    (3, 4, 1, 70, 132, "bool_padding", False),      # (B,1,1,S) key-padding mask
+    (1, 4, 4, 257, 1024, "bool_rows_dead", False),  # some query rows see no key at all
+    (2, 8, 2, 512, 2048, "float_same", True),
+]
+
+
+@pytest.mark.parametrize("case", MASKED_MFMA_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("tile", [3, 4])
+def test_mfma_forward_with_bias_and_masks(amd, gpu_device, case, dtype, tile):
+    # additive bias / bool keep-mask inside the head-dim-128 MFMA kernels (forced: a call they
+    # cannot take is an error, not a fallback)
+    B, Hq, Hkv, L, S, kind, causal = case
+    q, k, v = qkv(B, Hq, Hkv, L, S, 128, dtype=dtype, seed=L + 3 * S)
+    g = torch.Generator().manual_seed(L * 31 + S)
+    if kind == "float_same":
+        mask = (2.0 * torch.randn(B, Hq, L, S, generator=g)).to(dtype)
+    elif kind == "float32":
+        mask = 2.0 * torch.randn(B, Hq, L, S, generator=g)
+    elif kind == "float_bcast_q":
+        mask = (2.0 * torch.randn(B, 1, 1, S, generator=g)).to(dtype)
+    elif kind == "float_bcast_bh":
+        mask = (2.0 * torch.randn(1, 1, L, S, generator=g)).to(dtype)
+    elif kind == "bool":
+        mask = torch.rand(B, Hq, L, S, generator=g) > 0.3
+    elif kind == "bool_padding":
+        lens = torch.tensor([S, 5, 67])[:B]
+        mask = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+    else:
+        mask = torch.rand(B, 1, L, S, generator=g) > 0.5
+        mask[:, :, 3:40] = False
+        mask[:, :, L - 1] = False
+    out, lse = _run(amd, q, k, v, gpu_device, attn_bias=mask.to(gpu_device), is_causal=causal, force_kernel=tile)
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask if mask.dtype == torch.bool else mask.float(), is_causal=causal)
+    assert max_abs(out, ro) <= 2e-2
+    assert rel_err(out, ro) <= 1e-2
+    assert max_abs(lse, rl) <= 3e-3
+    if kind == "bool_rows_dead":
+        assert torch.equal(out[:, :, 3:40].float().cpu(), torch.zeros(B, Hq, 37, 128))
+        assert torch.isinf(lse[:, :, 3:40]).all() and (lse[:, :, 3:40] < 0).all()
+
+
+@pytest.mark.parametrize("tile", [3, 4])
+def test_mfma_forward_with_kv_lens(amd, gpu_device, tile):
+    # per-batch key counts inside the MFMA kernels, including an empty and a one-key batch; the
+    # rows of the cache past a batch's count hold NaN and must never reach the output
+    B, Hq, Hkv, L, S = 4, 8, 2, 200, 640
+    q, k, v = qkv(B, Hq, Hkv, L, S, 128, dtype=torch.bfloat16, seed=41)
+    lens = torch.tensor([640, 0, 1, 333], dtype=torch.int32)
+    kd, vd = k.clone(), v.clone()
+    for bi in range(B):
+        kd[bi, :, int(lens[bi]):] = float("nan")
+        vd[bi, :, int(lens[bi]):] = float("nan")
+    out, lse = _run(amd, q, kd, vd, gpu_device, kv_lens=lens.to(gpu_device), force_kernel=tile)
+    pad = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+    ro, rl = oracle_fwd(q, k, v, attn_mask=pad)
+    assert torch.isfinite(out.float()).all()
+    assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 3e-3
+    assert torch.equal(out[1].float().cpu(), torch.zeros(Hq, L, 128))
+    assert torch.isinf(lse[1]).all() and (lse[1] < 0).all()
+
+
 def test_fully_masked_rows_give_zero_and_minus_inf(amd, gpu_device):
     # reference: tests/python_ops/test_scaled_dot_product_attention.py:1003-1064
     q, k, v = qkv(1, 4, 4, 32, 32, 32, dtype=torch.float32, seed=9)

@@ -18,6 +18,12 @@ struct FwdM {
   int causal;
   int xcd_map;  // 1: (batch, kv head) streams are pinned to XCDs
   float scale;
+  // masked calls (fwd_mfma_w32.hip only): additive bias or bool keep-mask with unit stride on the
+  // key dim, strides in elements (0 on broadcast dims), and per-batch key counts
+  const void* bias = nullptr;
+  int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
+  int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int32_t* kv_lens = nullptr;
 };
 
 // Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first

@@ -332,8 +332,26 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
   if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
-  if (p.bias.data) return *why = "attn_bias present", false;
-  if (p.kv_lens) return *why = "kv_lens present", false;
+  // masked calls (bias, bool keep-mask, per-batch key counts): head dim 128 kernels only, with
+  // 32-bit row addressing and a bias whose rows can be read four keys at a time
+  if (p.bias.data || p.kv_lens) {
+    if (E != 128) return *why = "attn_bias / kv_lens with head dim 64", false;
+    if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
+      return *why = "attn_bias / kv_lens with rows beyond 32-bit offsets", false;
+  }
+  if (p.bias.data) {
+    const int esz = p.bias_dtype == MI355_SDPA_F32 ? 4 : p.bias_dtype == MI355_SDPA_BOOL ? 1
+                    : (p.bias_dtype == MI355_SDPA_F16 || p.bias_dtype == MI355_SDPA_BF16) ? 2 : 0;
+    if (!esz) return *why = "attn_bias dtype", false;
+    const int64_t S = p.k.size[2], L = p.q.size[2];
+    const int gran = 4 / esz;  // elements per dword
+    if (S > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
+    if (((uintptr_t)p.bias.data & 3) != 0 || S % gran != 0) return *why = "attn_bias not dword aligned", false;
+    for (int i = 0; i < 3; ++i)
+      if (p.bias.size[i] > 1 && (p.bias.stride[i] % gran) != 0) return *why = "attn_bias stride not dword aligned", false;
+    if ((31 * p.bias.stride[2] + S) * esz >= (1ll << 31)) return *why = "attn_bias rows beyond 32-bit offsets", false;
+    (void)L;
+  }
   if (p.dropout_p > 0.f) return *why = "dropout", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
@@ -364,6 +382,12 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
+  g.kv_lens = p.kv_lens;
+  if (p.bias.data) {
+    g.bias = p.bias.data;
+    g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1], g.bias_sl = p.bias.stride[2];
+    g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
+  }
   const int D = (int)p.q.size[3];
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256

@@ -41,7 +41,9 @@ constexpr int VP = D + 32;    // V tile row pitch: 320 bytes, conflict-free row 
 constexpr int AHEAD = 4;  // LDS operands are requested this many matrix ops ahead (at most 6)
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
-template <typename T, int WAVES>
+// MASK = 1 adds what a masked call brings: per-batch key counts (kv_lens) and an additive bias or
+// boolean keep-mask, folded into the score tile right after the matrix ops that produce it.
+template <typename T, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
   constexpr int KLD = 512 / NT;  // 16-byte chunks of K and of V per thread
@@ -59,6 +61,21 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   const int qrow = qw0 + col;
   const int qw_last = qw0 + 31;
 
+  // keys of this batch that take part
+  int S = p.S;
+  if constexpr (MASK) {
+    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    if (S == 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87)
+      if (qrow < p.L) {
+        uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
+#pragma unroll
+        for (int i = 0; i < D / 16; ++i) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
+        if (p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = -INFINITY;
+      }
+      return;
+    }
+  }
+
   const uint16_t* qp = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
@@ -70,7 +87,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
     for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16);
   }
 
-  int nt = (p.S + BN - 1) / BN;
+  int nt = (S + BN - 1) / BN;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   const int nt_w = p.causal ? min(nt, qw_last / BN + 1) : nt;
 
@@ -88,7 +105,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   // of this (batch, head), and the whole offset travels in the vector offset, the part the
   // hardware checks against that bound: rows of a ragged last tile beyond it read as zeros
   // (their scores are masked, and a zero V row keeps 0 * V finite).
-  const int k_bytes = (int)(((int64_t)(p.S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(p.S - 1) * p.v_sl + D) * 2);
+  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + D) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
   uint32_t k_off[KLD], v_off[KLD];
@@ -137,7 +154,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   float m_run = -INFINITY, l_run = 0.f;
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
 
   auto mask_tile = [&](f32x16& s, int kv0) {
 #pragma unroll
@@ -146,9 +163,68 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       if (kv > lim) s[r] = -INFINITY;
     }
   };
+  // Bias of the score tile: lane = query row, 4 groups of 4 consecutive keys.  The resource starts
+  // at this wavefront's first row of the (batch, head) plane and ends with its last one, so keys
+  // past S read as zero (they are masked anyway).  Folded into the RAW scores, s += bias / scale,
+  // so that everything downstream (reference tracking, lse) is the unbiased code.
+  uint32_t braw[16];
+  float inv_scale = 0.f;
+  __amdgpu_buffer_rsrc_t b_rsrc;
+  uint32_t b_off = 0;
+  const int bkind = MASK ? p.bias_kind : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  if constexpr (MASK) {
+    if (bkind) {
+      const int esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+      const int rows = min(32, p.L - qw0);
+      const char* base = (const char*)p.bias + (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * esz;
+      b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, rows > 0 ? (int)(((rows - 1) * p.bias_sl + p.S) * esz) : 0, 0x00020000);
+      b_off = (uint32_t)((min(col, max(rows - 1, 0)) * p.bias_sl + half * 4) * esz);
+      inv_scale = 1.f / p.scale;
+    }
+  }
+  auto load_bias = [&](int t) {
+    if constexpr (MASK) {
+      if (bkind == 1) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_off + (uint32_t)((t * BN + g * 8) * 4), 0, 0);
+          braw[4 * g] = w[0], braw[4 * g + 1] = w[1], braw[4 * g + 2] = w[2], braw[4 * g + 3] = w[3];
+        }
+      } else if (bkind == 4) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) braw[g] = __builtin_amdgcn_raw_buffer_load_b32(b_rsrc, b_off + (uint32_t)(t * BN + g * 8), 0, 0);
+      } else if (bkind) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, b_off + (uint32_t)((t * BN + g * 8) * 2), 0, 0);
+          braw[2 * g] = w[0], braw[2 * g + 1] = w[1];
+        }
+      }
+    }
+  };
+  auto apply_bias = [&](f32x16& sv) {
+    if constexpr (MASK) {
+      if (bkind == 1) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf(__builtin_bit_cast(float, braw[r]), inv_scale, sv[r]);
+      } else if (bkind == 4) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? sv[r] : -INFINITY;
+      } else if (bkind == 2) {
+        typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf((float)__builtin_bit_cast(h2, braw[r >> 1])[r & 1], inv_scale, sv[r]);
+      } else if (bkind == 3) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+          sv[r] = fmaf(__builtin_bit_cast(float, (r & 1) ? (braw[r >> 1] & 0xffff0000u) : (braw[r >> 1] << 16)), inv_scale, sv[r]);
+      }
+    }
+  };
+
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile
-  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (p.S % BN) ? p.S / BN : 0x7fffffff);
+  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
 
   float m_new = -INFINITY, mc = 0.f, alpha = 1.f;
   bool need_rescale = false;
@@ -208,6 +284,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   };
 
   // ---- prologue ----------------------------------------------------------------------------------
+  load_bias(0);
   load_k(0, 0);
   load_v(0, 0);
   load_k(1, 1);
@@ -228,6 +305,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       const u32x4 a = *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
       s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
     }
+    apply_bias(s_a);
+    load_bias(1);
     if (t_edge == 0) mask_tile(s_a, 0);
     raise_reference(tile_max(s_a));  // the first reference is the maximum of the first tile
     m_run = m_new;
@@ -319,6 +398,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       const u32x4 b0 = {pk[ks2 * 4], pk[ks2 * 4 + 1], pk[ks2 * 4 + 2], pk[ks2 * 4 + 3]};
       oacc[db] = Mma<T>::run(ring[i], b0, oacc[db]);
       if (i == 0) {
+        apply_bias(snext);
+        load_bias(t + 2);
         if (__builtin_expect(t + 1 >= t_edge, 0)) mask_tile(snext, (t + 1) * BN);  // rare
         stage1(snext, 0);
       } else {
@@ -387,13 +468,17 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int waves, hipStream_t s) {
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   dim3 grid((unsigned)blocks), block(64 * waves);
+  const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr;
+  const bool bf = dtype == MI355_SDPA_BF16;
+#define LAUNCH(TT, WW, MM) hipLaunchKernelGGL((fwd_w32_kernel<TT, WW, MM>), grid, block, 0, s, g)
   if (waves == 8) {
-    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_w32_kernel<bf16_t, 8>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((fwd_w32_kernel<f16_t, 8>), grid, block, 0, s, g);
+    if (masked) { if (bf) LAUNCH(bf16_t, 8, 1); else LAUNCH(f16_t, 8, 1); }
+    else { if (bf) LAUNCH(bf16_t, 8, 0); else LAUNCH(f16_t, 8, 0); }
   } else {
-    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_w32_kernel<bf16_t, 4>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((fwd_w32_kernel<f16_t, 4>), grid, block, 0, s, g);
+    if (masked) { if (bf) LAUNCH(bf16_t, 4, 1); else LAUNCH(f16_t, 4, 1); }
+    else { if (bf) LAUNCH(bf16_t, 4, 0); else LAUNCH(f16_t, 4, 0); }
   }
+#undef LAUNCH
   return check_launch("fwd_w32_kernel");
 }
 
