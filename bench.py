@@ -98,6 +98,24 @@ def wl_fwd(amd, dev, B, Hq, Hkv, S, D, seed, name):
     return step, flops, cfg, (q, k, v)
 
 
+def wl_masked_fwd(amd, dev):
+    """Forward with an additive bias shared by batch and heads (relative-position style),
+    B=4 Hq=32 Hkv=8 L=S=4096 D=128 bf16, non-causal: the path the reference leaves to its
+    unfused implementation whenever a mask is present (decompositions.py:2203)."""
+    B, Hq, Hkv, S, D = 4, 32, 8, 4096, 128
+    q, k, v = seeded([(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, D)], 1006, torch.bfloat16, dev)
+    bias = torch.randn(1, 1, S, S, generator=torch.Generator().manual_seed(1007)).to(torch.bfloat16).to(dev)
+    flops = 4.0 * B * Hq * D * S * S
+    nbytes = 2.0 * (2 * B * Hq * S * D + 2 * B * Hkv * S * D) + 4.0 * B * Hq * S + 2.0 * S * S
+
+    def step():
+        amd.sdpa_forward(q, k, v, attn_bias=bias)
+
+    cfg = {"workload": "masked_noncausal_gqa_bf16_fwd_shared_bias", "B": B, "Hq": Hq, "Hkv": Hkv, "S": S, "D": D,
+           "causal": False, "bias": "(1,1,L,S) bf16", "algorithmic_flops": flops, "algorithmic_bytes": nbytes}
+    return step, flops, cfg
+
+
 def wl_fwd_bwd(amd, dev):
     B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
     q, k, v, do = seeded([(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, D), (B, Hq, S, D)], 1004,
@@ -236,7 +254,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3_fwd", choices=["c3_fwd", "c2_fwd", "c4_fwd_bwd", "c5_decode"])
+    ap.add_argument("--workload", default="c3_fwd", choices=["c3_fwd", "c2_fwd", "c4_fwd_bwd", "c5_decode", "masked_fwd"])
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-spin", action="store_true", help="skip the untimed clock spin-up (profiled runs)")
@@ -279,6 +297,16 @@ def main():
                 cpu = cpu_baseline_fwd(1, 32, 8, 8192, 128, 1003, heads=32)
             else:
                 cpu = cpu_baseline_fwd(4, 12, 12, 1024, 64, 1002, heads=12)
+    elif args.workload == "masked_fwd":
+        step, flops, cfg = wl_masked_fwd(amd, dev)
+        wall, ev = event_time_ms(step, args.steps, args.warmup)
+        value = flops / (wall * 1e-3) / 1e12
+        ach = flops / (ev * 1e-3) / 1e12
+        roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "fwd_w32_kernel (masked variant)",
+                "kernel_ms": ev}
+        unit, dtype = "TFLOP/s", "bf16"
+        cpu = None  # the oracle's rate on this shape is the forward baseline of c3_fwd
     elif args.workload == "c4_fwd_bwd":
         sf, sb, f_fwd, f_bwd = wl_fwd_bwd(amd, dev)
         _, ev_f = event_time_ms(sf, args.steps, args.warmup)
@@ -332,6 +360,13 @@ def main():
                                     "bwd_frac_of_bf16_peak": f_bwd / (evb * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
         except Exception as e:
             extras["c4_fwd_bwd"] = {"error": repr(e)}
+        try:
+            stepm, flopsm, cfgm = wl_masked_fwd(amd, dev)
+            _, evm = event_time_ms(stepm, 10, 3)
+            extras["masked_fwd_shared_bias"] = {"TFLOP/s": flopsm / (evm * 1e-3) / 1e12, "kernel_ms": evm,
+                                                "frac_of_bf16_peak": flopsm / (evm * 1e-3) / 1e12 / PEAK_BF16_TFLOPS}
+        except Exception as e:
+            extras["masked_fwd_shared_bias"] = {"error": repr(e)}
 
     roof["traffic"] = MEASURED_TRAFFIC_BYTES.get(args.workload)
     line = {
