@@ -288,7 +288,7 @@ def main():
         value = flops / (wall * 1e-3) / 1e12
         ach = flops / (ev * 1e-3) / 1e12
         roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
-                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "fwd_w32_kernel" if args.workload == "c3_fwd" else "fwd_mfma_kernel",
+                "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "fwd_w32_kernel",
                 "kernel_ms": ev}
         unit, dtype = "TFLOP/s", "bf16"
         cpu = None

@@ -210,6 +210,28 @@ def test_mfma_forward_with_bias_and_masks(amd, gpu_device, case, dtype, tile):
         assert torch.isinf(lse[:, :, 3:40]).all() and (lse[:, :, 3:40] < 0).all()
 
 
+@pytest.mark.parametrize("kind", ["float", "bool", "kv_lens"])
+@pytest.mark.parametrize("tile", [3, 4])
+def test_mfma_forward_masked_head_dim_64(amd, gpu_device, kind, tile):
+    B, Hq, Hkv, L, S = 2, 6, 3, 150, 264
+    q, k, v = qkv(B, Hq, Hkv, L, S, 64, dtype=torch.bfloat16, seed=64)
+    g = torch.Generator().manual_seed(640)
+    kw, mask = {}, None
+    if kind == "float":
+        mask = (2.0 * torch.randn(B, 1, L, S, generator=g)).to(torch.bfloat16)
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "bool":
+        mask = torch.rand(1, Hq, L, S, generator=g) > 0.4
+        kw["attn_bias"] = mask.to(gpu_device)
+    else:
+        lens = torch.tensor([77, 264], dtype=torch.int32)
+        mask = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+        kw["kv_lens"] = lens.to(gpu_device)
+    out, lse = _run(amd, q, k, v, gpu_device, force_kernel=tile, **kw)
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask if mask.dtype == torch.bool else mask.float())
+    assert max_abs(out, ro) <= 2e-2 and rel_err(out, ro) <= 1e-2 and max_abs(lse, rl) <= 3e-3
+
+
 @pytest.mark.parametrize("tile", [3, 4])
 def test_mfma_forward_with_kv_lens(amd, gpu_device, tile):
     # per-batch key counts inside the MFMA kernels, including an empty and a one-key batch; the

@@ -162,9 +162,9 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   if (d->return_debug_mask) return MI355_SDPA_KERNEL_NONE;
   if (E > 512 || Dv > 512) return MI355_SDPA_KERNEL_NONE;
   const float scale = d->has_scale ? d->scale : 1.f;
-  // a bias or mask is taken by the head-dim-128 forward kernels only (its layout is checked again
-  // at the call); the backward of a masked call is the generic kernel's
-  const bool bias_ok = !d->has_attn_bias || (!backward && E == 128);
+  // a bias or mask is taken by the forward kernels only (its layout is checked again at the
+  // call); the backward of a masked call is the generic kernel's
+  const bool bias_ok = !d->has_attn_bias || !backward;
   const bool fast = d->q_dtype != MI355_SDPA_F32 && E == Dv && (E == 64 || E == 128) &&
                     bias_ok && d->dropout_p == 0.f && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;

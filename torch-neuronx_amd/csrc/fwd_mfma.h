@@ -56,7 +56,7 @@ __device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int&
 }
 
 
-// head dim 128; waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup
-int launch_fwd_mfma_w32(const FwdM& g, int dtype, int waves, hipStream_t s);
+// head dim 64 or 128; waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup
+int launch_fwd_mfma_w32(const FwdM& g, int dtype, int head_dim, int waves, hipStream_t s);
 
 }  // namespace mi355

@@ -3,8 +3,8 @@
 // Work split: one workgroup = 4 wavefronts; each wavefront owns NB blocks of 32 query rows
 // (NB = 2: 256 query rows per workgroup, one workgroup per compute unit with the full 512
 // registers per lane; NB = 1: 128 rows, two workgroups per compute unit, for short sequences)
-// and walks the keys in tiles of 64.  This file serves head dim 64, and head dim 128 only
-// when the strides are too large for the 32-bit addressing of fwd_mfma_w32.hip.
+// and walks the keys in tiles of 64.  This is the first generation of the forward kernel; it
+// serves only tensors whose strides are too large for the 32-bit addressing of fwd_mfma_w32.hip.
 //
 // With NB = 2 each K or V^T fragment read from LDS feeds two MFMAs (two query blocks held in
 // registers), which halves the LDS reads per flop.
@@ -332,10 +332,9 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
   if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
-  // masked calls (bias, bool keep-mask, per-batch key counts): head dim 128 kernels only, with
-  // 32-bit row addressing and a bias whose rows can be read four keys at a time
+  // masked calls (bias, bool keep-mask, per-batch key counts): the kernels with 32-bit row
+  // addressing only, and a bias whose rows can be read four keys at a time
   if (p.bias.data || p.kv_lens) {
-    if (E != 128) return *why = "attn_bias / kv_lens with head dim 64", false;
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
       return *why = "attn_bias / kv_lens with rows beyond 32-bit offsets", false;
   }
@@ -392,20 +391,18 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
-  // Head dim 128 goes to the kernels of fwd_mfma_w32.hip, which address K / V rows with 32-bit
-  // byte offsets from the start of a (batch, head).  256-row workgroups (one per compute unit)
-  // once every compute unit gets at least one (two when the causal mask makes half of them
-  // light) and the key loop is long; 128-row workgroups (two per compute unit) for short or few
-  // sequences (measured crossovers on MI355X).
-  if (D == 128 && (int64_t)g.S * g.k_sl * 2 < (1ll << 31) && (int64_t)g.S * g.v_sl * 2 < (1ll << 31)) {
-    const bool big = (g.S >= 2048 && wg256 >= (g.causal ? 512 : 256)) || (!g.causal && g.S >= 1024 && wg256 >= 512);
+  // The kernels of fwd_mfma_w32.hip address K / V rows with 32-bit byte offsets from the start of
+  // a (batch, head).  Head dim 128: 256-row workgroups (one per compute unit) once every compute
+  // unit gets at least one (two when the causal mask makes half of them light) and the key loop
+  // is long, 128-row workgroups (two per compute unit) for short or few sequences.  Head dim 64:
+  // 128-row workgroups always (measured crossovers on MI355X).
+  if ((int64_t)g.S * g.k_sl * 2 < (1ll << 31) && (int64_t)g.S * g.v_sl * 2 < (1ll << 31)) {
+    const bool big = D == 128 && ((g.S >= 2048 && wg256 >= (g.causal ? 512 : 256)) || (!g.causal && g.S >= 1024 && wg256 >= 512));
     const int rows = force_tile ? force_tile : big ? 256 : 128;
-    return launch_fwd_mfma_w32(g, p.dtype, rows / 32, s);
+    return launch_fwd_mfma_w32(g, p.dtype, D, rows / 32, s);
   }
-  // head dim 64 (and head dim 128 with strides beyond 32-bit offsets): the kernel above, with 256
-  // rows per workgroup under the same conditions
-  int NB = (force_tile == 256 || (force_tile == 0 && wg256 >= 256 && g.S >= 2048)) ? 2 : 1;
-  if (D == 128) NB = 1;
+  // strides beyond 32-bit offsets: the kernel above (64-bit addressing)
+  int NB = (D == 64 && (force_tile == 256 || (force_tile == 0 && wg256 >= 256 && g.S >= 2048))) ? 2 : 1;
   const int BM = 128 * NB;
   g.n_qt = (g.L + BM - 1) / BM;
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;

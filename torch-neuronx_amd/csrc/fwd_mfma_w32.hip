@@ -33,20 +33,26 @@
 namespace mi355 {
 namespace {
 
-constexpr int D = 128;
 constexpr int BN = 32;
-constexpr int KS = D / 16, DB = D / 32;
-constexpr int KROW = D + 8;   // K tile row pitch (elements): conflict-free 128-bit reads
-constexpr int VP = D + 32;    // V tile row pitch: 320 bytes, conflict-free row writes and transposing reads
-constexpr int AHEAD = 4;  // LDS operands are requested this many matrix ops ahead (at most 6)
+constexpr int AHEAD = 4;  // LDS operands are requested this many matrix ops ahead
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
 // MASK = 1 adds what a masked call brings: per-batch key counts (kv_lens) and an additive bias or
 // boolean keep-mask, folded into the score tile right after the matrix ops that produce it.
-template <typename T, int WAVES, int MASK>
+template <typename T, int D, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
-  constexpr int KLD = 512 / NT;  // 16-byte chunks of K and of V per thread
+  constexpr int KS = D / 16;      // matrix ops of S^T = K Q^T per tile (phase A)
+  constexpr int DB = D / 32;      // 32-row blocks of O^T
+  constexpr int NPV = 2 * DB;     // matrix ops of O^T += V^T P^T per tile (phase B)
+  constexpr int KROW = D + 8;     // K tile row pitch (elements): conflict-free 128-bit row reads
+  constexpr int VP = D + 32;      // V tile row pitch: four consecutive rows land in four different
+                                  // 64-byte windows, which the transposing reads need
+  constexpr int CH = D / 8;       // 16-byte chunks per row
+  constexpr int TCH = BN * CH;    // ... per tile
+  constexpr bool SPLIT = NT > TCH;  // more threads than chunks: one half stages K, the other V
+  constexpr int KLD = SPLIT ? 1 : TCH / NT;  // chunks of a tile per staging thread
+  static_assert(AHEAD <= KS && AHEAD <= NPV && (KS + NPV) % 8 == 0, "ring layout");
   __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KROW];
   __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][BN * VP];
 
@@ -98,7 +104,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   // Two staging sets each: a tile is fetched from global memory two iterations before it is
   // written to LDS, so a fetch has about two tile times to land.
   u32x4 kreg[2][KLD], vreg[2][KLD];
-  const int k_chunk = tid & 15, k_row = tid >> 4;  // rows k_row + i * NT / 16
+  const bool do_k = !SPLIT || tid < TCH, do_v = !SPLIT || tid >= TCH;  // (uniform per wavefront)
+  const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
+  const int k_chunk = s_idx % CH, k_row = s_idx / CH;  // rows k_row + i * NT / CH
   // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
   // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
   // instruction with one addition on the vector unit.  The resources end with the last key row
@@ -111,29 +119,37 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   uint32_t k_off[KLD], v_off[KLD];
 #pragma unroll
   for (int i = 0; i < KLD; ++i) {
-    k_off[i] = (uint32_t)(((k_row + i * (NT / 16)) * p.k_sl + k_chunk * 8) * 2);
-    v_off[i] = (uint32_t)(((k_row + i * (NT / 16)) * p.v_sl + k_chunk * 8) * 2);
+    k_off[i] = (uint32_t)(((k_row + i * (NT / CH)) * p.k_sl + k_chunk * 8) * 2);
+    v_off[i] = (uint32_t)(((k_row + i * (NT / CH)) * p.v_sl + k_chunk * 8) * 2);
   }
   const int k_tile_bytes = (int)(BN * p.k_sl * 2), v_tile_bytes = (int)(BN * p.v_sl * 2);
   auto load_k = [&](int set, int t) {
     const uint32_t base = (uint32_t)(min(t, nt - 1) * k_tile_bytes);
+    if (do_k) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i] + base, 0, 0);
+      for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i] + base, 0, 0);
+    }
   };
   auto load_v = [&](int set, int t) {
     const uint32_t base = (uint32_t)(min(t, nt - 1) * v_tile_bytes);
+    if (do_v) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i] + base, 0, 0);
+      for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i] + base, 0, 0);
+    }
   };
   auto store_k = [&](int set, int buf) {
+    if (do_k) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i)
-      *(u32x4*)(&k_lds[buf][(k_row + i * (NT / 16)) * KROW + k_chunk * 8]) = kreg[set][i];
+      for (int i = 0; i < KLD; ++i)
+        *(u32x4*)(&k_lds[buf][(k_row + i * (NT / CH)) * KROW + k_chunk * 8]) = kreg[set][i];
+    }
   };
   auto store_v = [&](int set, int buf) {
+    if (do_v) {
 #pragma unroll
-    for (int i = 0; i < KLD; ++i)
-      *(u32x4*)(&v_lds[buf][(k_row + i * (NT / 16)) * VP + k_chunk * 8]) = vreg[set][i];
+      for (int i = 0; i < KLD; ++i)
+        *(u32x4*)(&v_lds[buf][(k_row + i * (NT / CH)) * VP + k_chunk * 8]) = vreg[set][i];
+    }
   };
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
   // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
@@ -338,9 +354,9 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
     const uint16_t* kn = &k_lds[par][col * KROW + half * 8];  // tile t+2, stored during this iteration
     const uint16_t* vt = &v_lds[par][tr_base];
     auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
-    auto read_v = [&](int i) {  // d block i % 4, 16-key step i / 4
-      const u32x2 lo = tr_read(vt + (i >> 2) * 16 * VP + (i & 3) * 32);
-      const u32x2 hi = tr_read(vt + ((i >> 2) * 16 + 8) * VP + (i & 3) * 32);
+    auto read_v = [&](int i) {  // d block i % DB, 16-key step i / DB
+      const u32x2 lo = tr_read(vt + (i / DB) * 16 * VP + (i % DB) * 32);
+      const u32x2 hi = tr_read(vt + ((i / DB) * 16 + 8) * VP + (i % DB) * 32);
       return u32x4{lo[0], lo[1], hi[0], hi[1]};
     };
     __builtin_amdgcn_sched_barrier(0);
@@ -349,10 +365,12 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
     // ---- phase A -------------------------------------------------------------------------------
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      if (ks + AHEAD < KS) ring[ks + AHEAD] = read_k(ks + AHEAD);
-      else ring[ks + AHEAD - KS] = read_v(ks + AHEAD - KS);
-      snext = Mma<T>::run(ring[ks], qf[ks], ks == 0 ? zero16 : snext);
-      softmax_slot(scur, 4, ks, pk, ps);
+      // ring entry = (matrix op number within the tile, K ops first) mod 8
+      if (ks + AHEAD < KS) ring[(ks + AHEAD) & 7] = read_k(ks + AHEAD);
+      else ring[(ks + AHEAD) & 7] = read_v(ks + AHEAD - KS);
+      snext = Mma<T>::run(ring[ks & 7], qf[ks], ks == 0 ? zero16 : snext);
+#pragma unroll
+      for (int hs = 0; hs < 8 / KS; ++hs) softmax_slot(scur, 4, ks * (8 / KS) + hs, pk, ps);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- check ---------------------------------------------------------------------------------
@@ -379,36 +397,39 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
     __builtin_amdgcn_sched_barrier(0);
     // ---- phase B -------------------------------------------------------------------------------
     // The first matrix op needs nothing of S^T(t+1): it is issued before anything reads that tile,
-    // so the wait for the last op of phase A is spent on the matrix pipe.  The barrier sits before
-    // slot 6: by then every wavefront has stored its share of tiles t+2 (K) and t+1 (V) and has
-    // issued its last read of V(t); behind it the first K fragments of the next phase A are requested.
+    // so the wait for the last op of phase A is spent on the matrix pipe.  The barrier sits two
+    // slots before the end: by then every wavefront has stored its share of tiles t+2 (K) and
+    // t+1 (V) and has issued its last read of V(t); behind it the first K fragments of the next
+    // phase A are requested.  The eight half-steps of the softmax are spread over the slots, the
+    // last one trailing the loop.
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {  // i = 4 * (16-key step) + d block
-      if (i == 6) __syncthreads();
-      if (i + AHEAD < 8) ring[i + AHEAD] = read_v(i + AHEAD);
-      if (i == 6) {
+    for (int i = 0; i < NPV; ++i) {  // i = DB * (16-key step) + d block
+      if (i == NPV - 2) __syncthreads();
+      if (i + AHEAD < NPV) ring[(KS + i + AHEAD) & 7] = read_v(i + AHEAD);
+      if (i == NPV - 2) {
 #pragma unroll
         for (int j = 0; j < (AHEAD + 1) / 2; ++j) ring[j] = *(const u32x4*)(kn + j * 16);
       }
-      if (i == 7) {
+      if (i == NPV - 1) {
 #pragma unroll
         for (int j = (AHEAD + 1) / 2; j < AHEAD; ++j) ring[j] = *(const u32x4*)(kn + j * 16);
       }
-      const int ks2 = i >> 2, db = i & 3;
+      const int ks2 = i / DB, db = i % DB;
       const u32x4 b0 = {pk[ks2 * 4], pk[ks2 * 4 + 1], pk[ks2 * 4 + 2], pk[ks2 * 4 + 3]};
-      oacc[db] = Mma<T>::run(ring[i], b0, oacc[db]);
+      oacc[db] = Mma<T>::run(ring[(KS + i) & 7], b0, oacc[db]);
       if (i == 0) {
         apply_bias(snext);
         load_bias(t + 2);
         if (__builtin_expect(t + 1 >= t_edge, 0)) mask_tile(snext, (t + 1) * BN);  // rare
         stage1(snext, 0);
-      } else {
-        softmax_slot(snext, 0, i - 1, pkn, psn);
       }
+      constexpr int HSB = 8 / NPV;
+#pragma unroll
+      for (int hs = (i == 0 ? 0 : i * HSB - 1); hs < (i + 1) * HSB - 1; ++hs) softmax_slot(snext, 0, hs, pkn, psn);
       if (i == 0) store_k(par, par);  // tile t+2
       if (i == 1) store_v(par ^ 1, par ^ 1);  // tile t+1
-      if (i == 4) load_k(par, t + 4);
-      if (i == 5) load_v(par ^ 1, t + 3);
+      if (i == NPV / 2) load_k(par, t + 4);
+      if (i == NPV / 2 + 1) load_v(par ^ 1, t + 3);
       __builtin_amdgcn_sched_barrier(0);
     }
     softmax_slot(snext, 0, 7, pkn, psn);
@@ -458,7 +479,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
 
 }  // namespace
 
-int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int waves, hipStream_t s) {
+int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipStream_t s) {
   FwdM g = g0;
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
@@ -470,14 +491,20 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int waves, hipStream_t s) {
   dim3 grid((unsigned)blocks), block(64 * waves);
   const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr;
   const bool bf = dtype == MI355_SDPA_BF16;
-#define LAUNCH(TT, WW, MM) hipLaunchKernelGGL((fwd_w32_kernel<TT, WW, MM>), grid, block, 0, s, g)
-  if (waves == 8) {
-    if (masked) { if (bf) LAUNCH(bf16_t, 8, 1); else LAUNCH(f16_t, 8, 1); }
-    else { if (bf) LAUNCH(bf16_t, 8, 0); else LAUNCH(f16_t, 8, 0); }
-  } else {
-    if (masked) { if (bf) LAUNCH(bf16_t, 4, 1); else LAUNCH(f16_t, 4, 1); }
-    else { if (bf) LAUNCH(bf16_t, 4, 0); else LAUNCH(f16_t, 4, 0); }
-  }
+#define LAUNCH(TT, DD, WW, MM) hipLaunchKernelGGL((fwd_w32_kernel<TT, DD, WW, MM>), grid, block, 0, s, g)
+#define LAUNCH_D(DD)                                                                    \
+  do {                                                                                  \
+    if (waves == 8) {                                                                   \
+      if (masked) { if (bf) LAUNCH(bf16_t, DD, 8, 1); else LAUNCH(f16_t, DD, 8, 1); }   \
+      else { if (bf) LAUNCH(bf16_t, DD, 8, 0); else LAUNCH(f16_t, DD, 8, 0); }          \
+    } else {                                                                            \
+      if (masked) { if (bf) LAUNCH(bf16_t, DD, 4, 1); else LAUNCH(f16_t, DD, 4, 1); }   \
+      else { if (bf) LAUNCH(bf16_t, DD, 4, 0); else LAUNCH(f16_t, DD, 4, 0); }          \
+    }                                                                                   \
+  } while (0)
+  if (head_dim == 128) LAUNCH_D(128);
+  else LAUNCH_D(64);
+#undef LAUNCH_D
 #undef LAUNCH
   return check_launch("fwd_w32_kernel");
 }
