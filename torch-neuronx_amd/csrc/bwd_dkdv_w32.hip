@@ -1,4 +1,4 @@
-// Flash-attention backward, dK and dV, for gfx950, head dim 128, bf16/f16.
+// Flash-attention backward, dK and dV, for gfx950, head dim 64 or 128, bf16/f16.
 //
 // One workgroup = 8 wavefronts = 128 keys of one (batch, kv head); it loops over the query
 // heads of the group (the GQA sum of decompositions.py:2595-2598 happens in registers) and over
@@ -26,19 +26,17 @@
 namespace mi355 {
 namespace {
 
-constexpr int D = 128, BQ = 64, BK = 128;
-constexpr int KS = D / 16, DB = D / 32;
-constexpr int TILE = BQ * D;  // tiles are XOR swizzled, not padded: see swz16
-constexpr int kSmemBytes = 2 * 3 * TILE * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
+constexpr int BQ = 64, BK = 128;
+template <int D>
+constexpr int smem_bytes() {  // three Q and three dO tiles, two P hand-over buffers, lse / delta rows
+  return 2 * 3 * BQ * D * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
+}
 
-// A tile row is 16 chunks of 16 bytes; chunk c of row r lives at chunk c ^ swz16(r).  Both ways
-// of reading a tile are then free of bank conflicts: 16 consecutive rows reading the same chunk
-// (row-major A operand) land in 16 different chunks, and 4 consecutive rows reading the same 4
-// consecutive chunks (one transposing read) land in 4 different 64-byte windows.
-__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
-
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
+  constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
+  constexpr int TILE = BQ * D;           // tiles are XOR swizzled, not padded: see tile_swz
+  constexpr int NCH = BQ * CH / 512;     // 16-byte chunks of a tile per thread
   extern __shared__ __attribute__((aligned(16))) unsigned char smem[];
   uint16_t* const q_t = (uint16_t*)smem;          // [3][TILE]
   uint16_t* const do_t = q_t + 3 * TILE;          // [3][TILE]
@@ -85,21 +83,21 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.q + b * p.q_sb), 0, (int)q_ext, 0x00020000);
   const __amdgpu_buffer_rsrc_t go_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.go + b * p.go_sb), 0, (int)go_ext, 0x00020000);
-  const int s_row = tid >> 4, s_ch = tid & 15;  // rows s_row, s_row + 32
-  uint32_t q_off[2], go_off[2];
+  const int s_row = tid / CH, s_ch = tid % CH;  // rows s_row + n * 512 / CH
+  uint32_t q_off[NCH], go_off[NCH];
 #pragma unroll
-  for (int n = 0; n < 2; ++n) {
-    q_off[n] = (uint32_t)(((s_row + 32 * n) * p.q_sl + s_ch * 8) * 2);
-    go_off[n] = (uint32_t)(((s_row + 32 * n) * p.go_sl + s_ch * 8) * 2);
+  for (int n = 0; n < NCH; ++n) {
+    q_off[n] = (uint32_t)(((s_row + (512 / CH) * n) * p.q_sl + s_ch * 8) * 2);
+    go_off[n] = (uint32_t)(((s_row + (512 / CH) * n) * p.go_sl + s_ch * 8) * 2);
   }
-  u32x4 sq[2], sgo[2];
+  u32x4 sq[NCH], sgo[NCH];
   float lse_r = 0.f, dl_r = 0.f;
   auto load_item = [&](int it) {
     const int h = item_head(it), q0 = item_q0(it);
     const uint32_t qb = (uint32_t)((h * p.q_sh + (int64_t)q0 * p.q_sl) * 2);
     const uint32_t gb = (uint32_t)((h * p.go_sh + (int64_t)q0 * p.go_sl) * 2);
 #pragma unroll
-    for (int n = 0; n < 2; ++n) {
+    for (int n = 0; n < NCH; ++n) {
       sq[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, q_off[n] + qb, 0, 0);
       sgo[n] = __builtin_amdgcn_raw_buffer_load_b128(go_rsrc, go_off[n] + gb, 0, 0);
     }
@@ -114,19 +112,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
   auto store_item = [&](int buf) {
 #pragma unroll
-    for (int n = 0; n < 2; ++n) {
+    for (int n = 0; n < NCH; ++n) {
       // (row s_row + 32 has the swizzle of row s_row)
-      *(u32x4*)(&q_t[buf * TILE + (s_row + 32 * n) * D + ((s_ch ^ swz16(s_row)) << 3)]) = sq[n];
-      *(u32x4*)(&do_t[buf * TILE + (s_row + 32 * n) * D + ((s_ch ^ swz16(s_row)) << 3)]) = sgo[n];
+      *(u32x4*)(&q_t[buf * TILE + (s_row + (512 / CH) * n) * D + ((s_ch ^ tile_swz<D>(s_row)) << 3)]) = sq[n];
+      *(u32x4*)(&do_t[buf * TILE + (s_row + (512 / CH) * n) * D + ((s_ch ^ tile_swz<D>(s_row)) << 3)]) = sgo[n];
     }
     if (tid < BQ) lse_s[buf * BQ + tid] = lse_r, dl_s[buf * BQ + tid] = dl_r;
   };
 
-  // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
-  // row k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
-  // 8 + i / 4, 12 + i / 4: four rows at d = i.  A lane of the 32x32x16 A operand (d row lane % 32,
-  // row half lane / 32) takes two such reads: rows 4 half .. +3 and 8 + 4 half .. +3 of a 16-row
-  // step, the order in which the score accumulators hold them.
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
   // row k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
   // 8 + i / 4, 12 + i / 4: four rows at d = i.  A lane of the 32x32x16 A operand (d row lane % 32,
@@ -142,25 +135,25 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     for (int db = 0; db < DB; ++db) {
       const int row = 8 * sec + (tr_g >> 1) * 4 + (tr_jj >> 2);  // within the 16-row step
       const int d = db * 32 + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
-      tr_off[sec][db] = row * D + (((d >> 3) ^ swz16(row)) << 3) + (d & 7);
+      tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
     }
   int row_off[KS];  // [contraction step], without the 32-row block
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ swz16(col)) << 3);
+  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   auto tr_read = [&](const uint16_t* ptr) {
     const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
     return __builtin_bit_cast(u32x2, v);
   };
-  // operand i = 4 * (16-row step) + d block of the transposed tile
+  // operand i = DB * (16-row step) + d block of the transposed tile
   auto read_cols = [&](const uint16_t* tile, int i) {
-    const u32x2 lo = tr_read(tile + tr_off[0][i & 3] + (i >> 2) * 16 * D);
-    const u32x2 hi = tr_read(tile + tr_off[1][i & 3] + (i >> 2) * 16 * D);
+    const u32x2 lo = tr_read(tile + tr_off[0][i % DB] + (i / DB) * 16 * D);
+    const u32x2 hi = tr_read(tile + tr_off[1][i % DB] + (i / DB) * 16 * D);
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
-  // operand i = 8 * (32-row block) + contraction step of the row-major tile
+  // operand i = KS * (32-row block) + contraction step of the row-major tile
   auto read_rows = [&](const uint16_t* tile, int i) {
-    return *(const u32x4*)(tile + row_off[i & 7] + (i >> 3) * 32 * D);
+    return *(const u32x4*)(tile + row_off[i % KS] + (i / KS) * 32 * D);
   };
 
   f32x16 acc[DB];  // dV^T (role A) or dK^T (role B): d rows x this lane's key
@@ -176,9 +169,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i) ring[i] = read_rows(tile, i);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if (i + AHEAD < 16) ring[(i + AHEAD) & 7] = read_rows(tile, i + AHEAD);
-      sc[i >> 3] = Mma<T>::run(ring[i & 7], frag[i & 7], (i & 7) == 0 ? zero16 : sc[i >> 3]);
+    for (int i = 0; i < 2 * KS; ++i) {
+      if (i + AHEAD < 2 * KS) ring[(i + AHEAD) & 7] = read_rows(tile, i + AHEAD);
+      sc[i / KS] = Mma<T>::run(ring[i & 7], frag[i % KS], (i % KS) == 0 ? zero16 : sc[i / KS]);
     }
   };
   // acc += cols(tile)^T * pk, pk = the 64 x 32 tile of P or dS packed from the accumulator layout
@@ -187,9 +180,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i) ring[i] = read_cols(tile, i);
 #pragma unroll
-    for (int i = 0; i < 16; ++i) {
-      if (i + AHEAD < 16) ring[(i + AHEAD) & 7] = read_cols(tile, i + AHEAD);
-      const int ks4 = i >> 2, db = i & 3, mq = ks4 >> 1, r0 = (ks4 & 1) * 4;
+    for (int i = 0; i < 4 * DB; ++i) {
+      if (i + AHEAD < 4 * DB) ring[(i + AHEAD) & 7] = read_cols(tile, i + AHEAD);
+      const int ks4 = i / DB, db = i % DB, mq = ks4 >> 1, r0 = (ks4 & 1) * 4;
       const u32x4 bb = {pk[mq][r0], pk[mq][r0 + 1], pk[mq][r0 + 2], pk[mq][r0 + 3]};
       acc[db] = Mma<T>::run(ring[i & 7], bb, acc[db]);
     }
@@ -304,29 +297,31 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   }
 }
 
-template <typename T>
+template <typename T, int D>
 int launch_t(const BwdM& g, hipStream_t s) {
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T>,
+  constexpr int kSmemBytes = smem_bytes<D>();
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dkdv_w32_kernel: %s", kSmemBytes, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(512), kSmemBytes, s, g);
+  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(512), kSmemBytes, s, g);
   return check_launch("bwd_dkdv_w32_kernel");
 }
 
 }  // namespace
 
-bool bwd_dkdv_w32_fits(const BwdM& g) {
+bool bwd_dkdv_w32_fits(const BwdM& g, int head_dim) {
   // 32-bit byte offsets from the start of a batch for Q and dO
-  const int64_t q_ext = ((int64_t)(g.Hq - 1) * g.q_sh + (int64_t)(g.L + BQ) * g.q_sl + D) * 2;
-  const int64_t go_ext = ((int64_t)(g.Hq - 1) * g.go_sh + (int64_t)(g.L + BQ) * g.go_sl + D) * 2;
+  const int64_t q_ext = ((int64_t)(g.Hq - 1) * g.q_sh + (int64_t)(g.L + BQ) * g.q_sl + head_dim) * 2;
+  const int64_t go_ext = ((int64_t)(g.Hq - 1) * g.go_sh + (int64_t)(g.L + BQ) * g.go_sl + head_dim) * 2;
   return q_ext < (1ll << 31) && go_ext < (1ll << 31) && g.q_sh >= 0 && g.q_sl >= 0 && g.go_sh >= 0 && g.go_sl >= 0;
 }
 
-int launch_bwd_dkdv_w32(const BwdM& g, int dtype, hipStream_t s) {
-  return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t>(g, s) : launch_t<f16_t>(g, s);
+int launch_bwd_dkdv_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
+  if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t, 128>(g, s) : launch_t<f16_t, 128>(g, s);
+  return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t, 64>(g, s) : launch_t<f16_t, 64>(g, s);
 }
 
 }  // namespace mi355

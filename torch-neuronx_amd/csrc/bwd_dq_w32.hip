@@ -1,4 +1,4 @@
-// Flash-attention backward, dQ, for gfx950, head dim 128, bf16/f16.
+// Flash-attention backward, dQ, for gfx950, head dim 64 or 128, bf16/f16.
 //
 // One workgroup = 8 wavefronts of 32 query rows each (256 rows of one (batch, query head)), one
 // workgroup per compute unit, two wavefronts per SIMD with 256 registers each; it walks the keys
@@ -14,7 +14,7 @@
 // wavefront issues at most one instruction every four cycles, so one wavefront per SIMD cannot
 // keep the matrix and the vector pipe busy together).
 //
-// K and V tiles sit in LDS row-major and XOR swizzled (see swz16).  Math follows
+// K and V tiles sit in LDS row-major and XOR swizzled (see tile_swz).  Math follows
 // torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows with lse = -inf give zero
 // gradients, scale multiplies dQ once at the end.
 #include "bwd_mfma.h"
@@ -22,19 +22,16 @@
 namespace mi355 {
 namespace {
 
-constexpr int D = 128, BM = 256, BN = 32;
-constexpr int KS = D / 16, DB = D / 32;
-constexpr int TILE = BN * D;
+constexpr int BM = 256, BN = 32;
 constexpr int AHEAD = 4;
 
-// A tile row is 16 chunks of 16 bytes; chunk c of row r lives at chunk c ^ swz16(r).  Both ways
-// of reading a tile are then free of bank conflicts: 16 consecutive rows reading the same chunk
-// (row-major A operand) land in 16 different chunks, and 4 consecutive rows reading the same 4
-// consecutive chunks (one transposing read) land in 4 different 64-byte windows.
-__device__ __forceinline__ int swz16(int r) { return ((r & 3) << 2) | ((r >> 2) & 3); }
-
-template <typename T>
+template <typename T, int D>
 __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
+  constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
+  constexpr int TILE = BN * D;
+  constexpr int TCH = BN * CH;        // 16-byte chunks per tile
+  constexpr bool SPLIT = 512 > TCH;   // more threads than chunks: one half stages K, the other V
+  static_assert(AHEAD <= 2 * DB, "ring");
   __shared__ __attribute__((aligned(16))) uint16_t k_t[3][TILE];
   __shared__ __attribute__((aligned(16))) uint16_t v_t[3][TILE];
 
@@ -97,19 +94,21 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   const int k_bytes = (int)(((int64_t)(p.S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(p.S - 1) * p.v_sl + D) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
-  const int s_row = tid >> 4, s_ch = tid & 15;
+  const bool do_k = !SPLIT || tid < TCH, do_v = !SPLIT || tid >= TCH;  // (uniform per wavefront)
+  const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
+  const int s_row = s_idx / CH, s_ch = s_idx % CH;
   const uint32_t k_off = (uint32_t)((s_row * p.k_sl + s_ch * 8) * 2), v_off = (uint32_t)((s_row * p.v_sl + s_ch * 8) * 2);
   const uint32_t k_tile_bytes = (uint32_t)(BN * p.k_sl * 2), v_tile_bytes = (uint32_t)(BN * p.v_sl * 2);
-  const int s_lds = s_row * D + ((s_ch ^ swz16(s_row)) << 3);
+  const int s_lds = s_row * D + ((s_ch ^ tile_swz<D>(s_row)) << 3);
   u32x4 kreg, vreg;
   auto load_tile = [&](int t) {
     const uint32_t tt = (uint32_t)min(t, nt - 1);
-    kreg = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off + tt * k_tile_bytes, 0, 0);
-    vreg = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off + tt * v_tile_bytes, 0, 0);
+    if (do_k) kreg = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off + tt * k_tile_bytes, 0, 0);
+    if (do_v) vreg = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off + tt * v_tile_bytes, 0, 0);
   };
   auto store_tile = [&](int buf) {
-    *(u32x4*)(&k_t[buf][s_lds]) = kreg;
-    *(u32x4*)(&v_t[buf][s_lds]) = vreg;
+    if (do_k) *(u32x4*)(&k_t[buf][s_lds]) = kreg;
+    if (do_v) *(u32x4*)(&v_t[buf][s_lds]) = vreg;
   };
 
   // element offsets inside a tile (the swizzle is not additive in the d block / contraction step:
@@ -122,11 +121,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     for (int db = 0; db < DB; ++db) {
       const int row = 8 * sec + (tr_g >> 1) * 4 + (tr_jj >> 2);
       const int d = db * 32 + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
-      tr_off[sec][db] = row * D + (((d >> 3) ^ swz16(row)) << 3) + (d & 7);
+      tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
     }
   int row_off[KS];
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ swz16(col)) << 3);
+  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
   // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
@@ -137,10 +136,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
     return __builtin_bit_cast(u32x2, v);
   };
-  // operand i = 4 * (16-key step) + d block of K^T
+  // operand i = DB * (16-key step) + d block of K^T
   auto read_cols = [&](const uint16_t* tile, int i) {
-    const u32x2 lo = tr_read(tile + tr_off[0][i & 3] + (i >> 2) * 16 * D);
-    const u32x2 hi = tr_read(tile + tr_off[1][i & 3] + (i >> 2) * 16 * D);
+    const u32x2 lo = tr_read(tile + tr_off[0][i % DB] + (i / DB) * 16 * D);
+    const u32x2 hi = tr_read(tile + tr_off[1][i % DB] + (i / DB) * 16 * D);
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   };
 
@@ -188,9 +187,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
 #pragma unroll
     for (int i = 0; i < 2 * DB; ++i) {
       if (i + AHEAD < 2 * DB) ring[(i + AHEAD) & 7] = read_cols(k_t[buf], i + AHEAD);
-      const int r0 = (i >> 2) * 4;
+      const int r0 = (i / DB) * 4;
       const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
-      dqacc[i & 3] = Mma<T>::run(ring[i & 7], bS, dqacc[i & 3]);
+      dqacc[i % DB] = Mma<T>::run(ring[i & 7], bS, dqacc[i % DB]);
     }
   };
 
@@ -241,15 +240,22 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
 
 }  // namespace
 
-bool bwd_dq_w32_fits(const BwdM& g) {
+bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
   // 32-bit byte offsets from the start of a (batch, kv head) for K and V
+  (void)head_dim;
   return (int64_t)(g.S + BN) * g.k_sl * 2 < (1ll << 31) && (int64_t)(g.S + BN) * g.v_sl * 2 < (1ll << 31) && g.k_sl >= 0 && g.v_sl >= 0;
 }
 
-int launch_bwd_dq_w32(const BwdM& g, int dtype, hipStream_t s) {
+int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
-  if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dq_w32_kernel<bf16_t>), dim3((unsigned)blocks), dim3(512), 0, s, g);
-  else hipLaunchKernelGGL((bwd_dq_w32_kernel<f16_t>), dim3((unsigned)blocks), dim3(512), 0, s, g);
+  const dim3 grid((unsigned)blocks), block(512);
+  if (head_dim == 128) {
+    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dq_w32_kernel<bf16_t, 128>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((bwd_dq_w32_kernel<f16_t, 128>), grid, block, 0, s, g);
+  } else {
+    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dq_w32_kernel<bf16_t, 64>), grid, block, 0, s, g);
+    else hipLaunchKernelGGL((bwd_dq_w32_kernel<f16_t, 64>), grid, block, 0, s, g);
+  }
   return check_launch("bwd_dq_w32_kernel");
 }
 

@@ -18,12 +18,23 @@ struct BwdM {
   float scale;
 };
 
-// dK / dV for head dim 128 with two wavefronts per SIMD (bwd_dkdv_w32.hip); false when the
-// tensors do not fit its 32-bit addressing and the caller must use the kernel in bwd_mfma.hip
-bool bwd_dkdv_w32_fits(const BwdM& g);
-int launch_bwd_dkdv_w32(const BwdM& g, int dtype, hipStream_t s);
-// dQ for head dim 128 with two wavefronts per SIMD (bwd_dq_w32.hip), same convention
-bool bwd_dq_w32_fits(const BwdM& g);
-int launch_bwd_dq_w32(const BwdM& g, int dtype, hipStream_t s);
+// Swizzle of the row-major LDS tiles of the two-wavefronts-per-SIMD kernels.  A tile row is D/8
+// chunks of 16 bytes; chunk c of row r lives at chunk c ^ tile_swz<D>(r).  Both ways of reading a
+// tile are then free of bank conflicts: 16 consecutive rows reading the same chunk (row-major A
+// operand) land in 16 different 16-byte slots of the 256-byte bank window, and 4 consecutive
+// rows reading the same 4 consecutive chunks (one transposing read) land in 4 different 64-byte
+// windows.  (With D = 64 two rows share a bank window, so the row parity does part of the job.)
+template <int D>
+__device__ __forceinline__ int tile_swz(int r) {
+  return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+}
+
+// dK / dV with two wavefronts per SIMD (bwd_dkdv_w32.hip), head dim 64 or 128; `fits` is false
+// when the tensors do not fit its 32-bit addressing and the caller must use bwd_mfma.hip
+bool bwd_dkdv_w32_fits(const BwdM& g, int head_dim);
+int launch_bwd_dkdv_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s);
+// dQ with two wavefronts per SIMD (bwd_dq_w32.hip), same convention
+bool bwd_dq_w32_fits(const BwdM& g, int head_dim);
+int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s);
 
 }  // namespace mi355

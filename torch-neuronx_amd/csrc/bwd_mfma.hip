@@ -481,8 +481,8 @@ int launch_td(const BwdM& g, hipStream_t s) {
   hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, s, g);
   int rc = check_launch("bwd_delta_kernel");
   if (rc) return rc;
-  if (D == 128 && bwd_dkdv_w32_fits(g)) {
-    rc = launch_bwd_dkdv_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
+  if (bwd_dkdv_w32_fits(g, D)) {
+    rc = launch_bwd_dkdv_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
   } else {
     hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(256), 0, s, g);
     rc = check_launch("bwd_dkdv_kernel");
@@ -490,8 +490,8 @@ int launch_td(const BwdM& g, hipStream_t s) {
   if (rc) return rc;
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  if (D == 128 && wg256 >= 256 && bwd_dq_w32_fits(g))
-    return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
+  if (wg256 >= 256 && bwd_dq_w32_fits(g, D))
+    return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
   if (D == 128 && wg256 >= 256) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
   } else {
