@@ -173,6 +173,61 @@ def test_backward_kv_lens(amd, gpu_device):
         assert max_abs(a, r) <= 5e-5
 
 
+MASKED_BWD_CASES = [
+    # B, Hq, Hkv, L, S, E, mask kind, causal
+    (3, 4, 2, 200, 328, 128, "bool_padding", False),   # (B,1,1,S) key-padding mask
+    (2, 8, 2, 130, 256, 128, "float_key", True),        # (B,H,1,S) additive per-key bias + causal
+    (2, 4, 4, 96, 200, 64, "bool_padding", False),
+    (2, 6, 3, 150, 264, 64, "float_key32", False),      # float32 bias shared by all heads
+    (4, 8, 2, 200, 640, 128, "kv_lens", False),
+    (3, 4, 4, 100, 200, 64, "kv_lens", True),
+]
+
+
+@pytest.mark.parametrize("case", MASKED_BWD_CASES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_backward_with_key_masks(amd, gpu_device, case, dtype):
+    # key-only masks and per-batch key counts inside the MFMA backward kernels (forced: a call
+    # they cannot take is an error, not a fallback); cache rows past a batch's count hold NaN
+    B, Hq, Hkv, L, S, E, kind, causal = case
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 3 + S, with_do=True)
+    go = go.clamp(-1, 1) * 0.1
+    g = torch.Generator().manual_seed(L + 7 * S)
+    kw, mask = {}, None
+    kd, vd = k.clone(), v.clone()
+    if kind == "bool_padding":
+        lens = torch.randint(1, S + 1, (B,), generator=g)
+        lens[0] = S
+        mask = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "float_key":
+        mask = (2.0 * torch.randn(B, Hq, 1, S, generator=g)).to(dtype)
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "float_key32":
+        mask = 2.0 * torch.randn(1, 1, 1, S, generator=g)
+        kw["attn_bias"] = mask.to(gpu_device)
+    else:
+        lens = torch.randint(0, S + 1, (B,), generator=g).to(torch.int32)
+        lens[0], lens[1] = S, 0
+        mask = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+        kw["kv_lens"] = lens.to(gpu_device)
+        for bi in range(B):
+            kd[bi, :, int(lens[bi]):] = float("nan")
+            vd[bi, :, int(lens[bi]):] = float("nan")
+    dev = gpu_device
+    out, lse = amd.sdpa_forward(q.to(dev), kd.to(dev), vd.to(dev), is_causal=causal, force_kernel=MFMA, **kw)
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), kd.to(dev), vd.to(dev), out, lse, is_causal=causal,
+                                      force_kernel=MFMA, **kw)
+    torch.cuda.synchronize()
+    om_mask = mask if mask.dtype == torch.bool else mask.float()
+    ro, rl = oracle_fwd(q, k, v, attn_mask=om_mask, is_causal=causal)
+    rdq, rdk, rdv = oracle_bwd(go, q, k, v, ro, rl, attn_mask=om_mask, is_causal=causal)[:3]
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert torch.isfinite(a.float()).all(), name
+        assert max_abs(a, r) <= 5e-2, name
+        assert rel_err(a, r) <= 2e-2, name
+
+
 @pytest.mark.parametrize("kernel", [GENERIC, MFMA])
 def test_backward_grad_layouts_follow_inputs(amd, gpu_device, kernel):
     B, H, L, E = 2, 4, 130, 64

@@ -32,7 +32,8 @@ constexpr int smem_bytes() {  // three Q and three dO tiles, two P hand-over buf
   return 2 * 3 * BQ * D * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
 }
 
-template <typename T, int D>
+// MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only
+template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
   constexpr int TILE = BQ * D;           // tiles are XOR swizzled, not padded: see tile_swz
@@ -56,10 +57,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int k0 = kt * BK, kw0 = k0 + kb * 32;
   const int key = kw0 + col;
 
+  int S = p.S;  // keys of this batch that take part
+  if constexpr (MASK) {
+    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+  }
   // this lane's key as B operand: K fragments for S = Q K^T (role A), V fragments for dP = dO V^T (role B)
   u32x4 frag[KS];
   {
-    const int kc = min(key, p.S - 1);
+    const int kc = max(min(key, S - 1), 0);  // (a live row: rows past the batch's keys may hold anything)
     const uint16_t* r = role ? (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl
                              : (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl;
 #pragma unroll
@@ -69,7 +74,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int nqs = (p.L + BQ - 1) / BQ;
   const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
   const int per_head = nqs - qs_begin;
-  const int n_items = rep * per_head;
+  const int n_items = (MASK && k0 >= S) ? 0 : rep * per_head;  // no live key in this tile: zeros
   auto item_head = [&](int it) { return hk * rep + it / per_head; };
   auto item_q0 = [&](int it) { return (qs_begin + it % per_head) * BQ; };
 
@@ -190,8 +195,13 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 
   auto role_a = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
-    if (p.causal && q0 + BQ - 1 < kw0) return;  // every key of this block lies above the diagonal
-    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= p.S);
+    if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;  // every key of this block lies above the diagonal / past the keys
+    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S);
+    float bl = 0.f;  // this key's bias in the log2 domain
+    if constexpr (MASK) {
+      if (p.bias_kind)
+        bl = bias_value(p.bias, b * p.bias_sb + item_head(it) * p.bias_sh + min(key, p.S - 1), p.bias_kind) * kLog2eF;
+    }
     f32x16 sc[2];
     scores(q_t + tb * TILE, sc);
     uint32_t pk[2][8];
@@ -203,10 +213,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
         float pr[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, -l4[e]));
+          if constexpr (MASK) pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, bl) - l4[e]);
+          else pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, -l4[e]));
           if (edge) {
             const int qi = q0 + mq * 32 + r4 * 8 + half * 4 + e;
-            pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
+            pr[e] = ((p.causal && key > qi) || key >= S) ? 0.f : pr[e];
           }
         }
         pk[mq][r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pk[mq][r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
@@ -224,12 +235,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // it, dS and dK of that tile at the start of iteration it + 1.
   f32x16 dp[2];
   auto role_b_scores = [&](int it, int tb) {
-    if (p.causal && item_q0(it) + BQ - 1 < kw0) return;
+    if ((p.causal && item_q0(it) + BQ - 1 < kw0) || kw0 >= S) return;
     scores(do_t + tb * TILE, dp);
   };
   auto role_b = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
-    if (p.causal && q0 + BQ - 1 < kw0) return;
+    if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
     const uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;
     uint32_t pk[2][8];
 #pragma unroll
@@ -297,17 +308,21 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   }
 }
 
-template <typename T, int D>
+template <typename T, int D, int MASK>
 int launch_t(const BwdM& g, hipStream_t s) {
   constexpr int kSmemBytes = smem_bytes<D>();
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D, MASK>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dkdv_w32_kernel: %s", kSmemBytes, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(512), kSmemBytes, s, g);
+  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D, MASK>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(512), kSmemBytes, s, g);
   return check_launch("bwd_dkdv_w32_kernel");
+}
+template <typename T, int D>
+int launch_m(const BwdM& g, hipStream_t s) {
+  return (g.bias_kind || g.kv_lens) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
 }
 
 }  // namespace
@@ -320,8 +335,8 @@ bool bwd_dkdv_w32_fits(const BwdM& g, int head_dim) {
 }
 
 int launch_bwd_dkdv_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
-  if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t, 128>(g, s) : launch_t<f16_t, 128>(g, s);
-  return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t, 64>(g, s) : launch_t<f16_t, 64>(g, s);
+  if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 128>(g, s) : launch_m<f16_t, 128>(g, s);
+  return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 64>(g, s) : launch_m<f16_t, 64>(g, s);
 }
 
 }  // namespace mi355

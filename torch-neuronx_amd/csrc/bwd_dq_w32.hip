@@ -25,7 +25,8 @@ namespace {
 constexpr int BM = 256, BN = 32;
 constexpr int AHEAD = 4;
 
-template <typename T, int D>
+// MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only
+template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
   constexpr int TILE = BN * D;
@@ -77,13 +78,25 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     dl = p.delta[idx];
   }
 
-  int nt = (p.S + BN - 1) / BN;
+  int S = p.S;  // keys of this batch that take part
+  if constexpr (MASK) {
+    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    if (S == 0) {  // no live key: zero gradient
+      if (qrow < p.L) {
+        uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
+#pragma unroll
+        for (int i = 0; i < D / 16; ++i) *(u32x4*)(gq + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
+      }
+      return;
+    }
+  }
+  int nt = (S + BN - 1) / BN;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BN + 1) : nt;  // tiles with work for this wavefront
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile
-  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (p.S % BN) ? p.S / BN : 0x7fffffff);
-  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
+  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
 
   // ---- staging: every thread moves one 16-byte chunk of the K tile and one of the V tile ----------
   // Buffer resources end with the last key row of this (batch, head), and the whole offset travels
@@ -91,7 +104,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // tile beyond it read as zeros (their probabilities are masked to zero).
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
-  const int k_bytes = (int)(((int64_t)(p.S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(p.S - 1) * p.v_sl + D) * 2);
+  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + D) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
   const bool do_k = !SPLIT || tid < TCH, do_v = !SPLIT || tid >= TCH;  // (uniform per wavefront)
@@ -162,6 +175,45 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       else sacc = Mma<T>::run(ring[i & 7], qf[i >> 1], i == 0 ? zero16 : sacc);
     }
   };
+  // Bias of a score tile (it depends on the key only): this lane's 16 keys, fetched one tile ahead
+  // as 4 groups of 4 consecutive keys; keys past the row read as zero (they are masked anyway).
+  uint32_t braw[16];
+  const int bkind = MASK ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  // (set up unconditionally, with no records when there is no bias: a resource that is defined on
+  // one path only stops being uniform for the compiler)
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
+      __builtin_amdgcn_readfirstlane(bkind ? p.S * besz : 0), 0x00020000);
+  auto load_bias = [&](int t) {
+    if constexpr (MASK) {
+      const uint32_t off = (uint32_t)((t * BN + half * 4) * besz);
+      if (bkind == 1) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, off + g * 32, 0, 0);
+          braw[4 * g] = w[0], braw[4 * g + 1] = w[1], braw[4 * g + 2] = w[2], braw[4 * g + 3] = w[3];
+        }
+      } else if (bkind == 4) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) braw[g] = __builtin_amdgcn_raw_buffer_load_b32(b_rsrc, off + g * 8, 0, 0);
+      } else if (bkind) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, off + g * 16, 0, 0);
+          braw[2 * g] = w[0], braw[2 * g + 1] = w[1];
+        }
+      }
+    }
+  };
+  auto bias_log2 = [&](int r) -> float {  // bias of accumulator register r, in the log2 domain
+    if (bkind == 1) return __builtin_bit_cast(float, braw[r]) * kLog2eF;
+    if (bkind == 4) return ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? 0.f : -INFINITY;
+    const uint32_t w = braw[r >> 1];
+    if (bkind == 3) return __builtin_bit_cast(float, (r & 1) ? (w & 0xffff0000u) : (w << 16)) * kLog2eF;
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    return (float)__builtin_bit_cast(h2, w)[r & 1] * kLog2eF;
+  };
   // dS^T of tile t, packed as the B operand of dQ^T += K^T dS^T
   auto softmax = [&](int t, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
     const bool edge = t >= t_edge;
@@ -170,7 +222,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       float ds[2];
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
-        float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+        float pr;
+        if (MASK && bkind) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bias_log2(r + e)) - lse2);
+        else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
         if (edge) {
           const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
           pr = kv > lim ? 0.f : pr;
@@ -195,6 +249,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
 
   // Iteration t: scores of tile t + 1, vector work of tile t, dQ of tile t; tile t + 2 goes to LDS.
   // Buffers: tile t in t % 3.
+  load_bias(0);
   load_tile(0);
   store_tile(0);
   load_tile(1);
@@ -202,14 +257,18 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   __syncthreads();
   load_tile(2);
   f32x16 s_a, dp_a, s_b, dp_b;
-  if (nt_w > 0) scores(0, s_a, dp_a);
+  if (!MASK && nt_w > 0) scores(0, s_a, dp_a);
   int buf = 0;  // t % 3
   auto iteration = [&](int t, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
     const int bn = buf == 2 ? 0 : buf + 1, bnn = bn == 2 ? 0 : bn + 1;
     if (t < nt_w) {
-      if (t + 1 < nt_w) scores(bn, snext, dpnext);
+      // (the masked variant has no registers to spare for a second score tile: it computes the
+      // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap)
+      if constexpr (MASK) scores(buf, scur, dpcur);
+      else if (t + 1 < nt_w) scores(bn, snext, dpnext);
       uint32_t pS[8];
       softmax(t, scur, dpcur, pS);
+      load_bias(t + 1);
       accumulate(buf, pS);
     }
     store_tile(bnn);  // tile t + 2 (buffer of tile t - 1, whose last readers passed the previous barrier)
@@ -249,13 +308,17 @@ bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
 int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
-  if (head_dim == 128) {
-    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dq_w32_kernel<bf16_t, 128>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((bwd_dq_w32_kernel<f16_t, 128>), grid, block, 0, s, g);
-  } else {
-    if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dq_w32_kernel<bf16_t, 64>), grid, block, 0, s, g);
-    else hipLaunchKernelGGL((bwd_dq_w32_kernel<f16_t, 64>), grid, block, 0, s, g);
-  }
+  const bool bf = dtype == MI355_SDPA_BF16, masked = g.bias_kind || g.kv_lens;
+#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, 0, s, g)
+#define LAUNCH_D(DD)                                                         \
+  do {                                                                       \
+    if (masked) { if (bf) LAUNCH(bf16_t, DD, 1); else LAUNCH(f16_t, DD, 1); }  \
+    else { if (bf) LAUNCH(bf16_t, DD, 0); else LAUNCH(f16_t, DD, 0); }         \
+  } while (0)
+  if (head_dim == 128) LAUNCH_D(128);
+  else LAUNCH_D(64);
+#undef LAUNCH_D
+#undef LAUNCH
   return check_launch("bwd_dq_w32_kernel");
 }
 

@@ -16,7 +16,23 @@ struct BwdM {
   int n_qt, n_kt;
   int causal, xcd_map;
   float scale;
+  // masked calls (the two-wavefronts-per-SIMD kernels only): a bias or bool keep-mask that does not
+  // depend on the query row (stride 0 over L, unit stride over keys; strides in elements) and
+  // per-batch key counts
+  const void* bias = nullptr;
+  int64_t bias_sb = 0, bias_sh = 0;
+  int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int32_t* kv_lens = nullptr;
 };
+
+// bias element as a float (bool: 0 or -inf)
+__device__ __forceinline__ float bias_value(const void* base, int64_t idx, int kind) {
+  if (kind == 1) return ((const float*)base)[idx];
+  if (kind == 4) return ((const uint8_t*)base)[idx] ? 0.f : -INFINITY;
+  const uint32_t w = ((const uint16_t*)base)[idx];
+  if (kind == 3) return __builtin_bit_cast(float, w << 16);
+  return (float)__builtin_bit_cast(_Float16, (uint16_t)w);
+}
 
 // Swizzle of the row-major LDS tiles of the two-wavefronts-per-SIMD kernels.  A tile row is D/8
 // chunks of 16 bytes; chunk c of row r lives at chunk c ^ tile_swz<D>(r).  Both ways of reading a

@@ -490,7 +490,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   if (rc) return rc;
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  if (wg256 >= 256 && bwd_dq_w32_fits(g, D))
+  if ((wg256 >= 256 || g.bias_kind || g.kv_lens) && bwd_dq_w32_fits(g, D))  // (a masked call has no other kernel)
     return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
   if (D == 128 && wg256 >= 256) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
@@ -502,38 +502,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
 
 }  // namespace
 
-bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
-  *why = "";
-  const int64_t E = p.q.size[3], Dv = p.v.size[3];
-  if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
-  if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
-  if (p.bias.data || p.grad_bias.data) return *why = "attn_bias present", false;
-  if (p.kv_lens) return *why = "kv_lens present", false;
-  if (p.dropout_p > 0.f) return *why = "dropout", false;
-  if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
-  if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
-  const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
-  for (const mi355_sdpa_tensor* t : ts) {
-    if (t->stride[3] != 1) return *why = "head dim is not unit-stride", false;
-    if (((uintptr_t)t->data & 15) != 0) return *why = "pointer not 16-byte aligned", false;
-    for (int i = 0; i < 3; ++i)
-      if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
-  }
-  if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
-  return true;
-}
-
-size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p) {
-  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * sizeof(float);
-}
-
-int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
-  const char* why;
-  if (!bwd_mfma_supported(p, &why)) {
-    set_error("SDPA: MFMA backward kernel cannot take this call: %s", why);
-    return MI355_SDPA_ERR_UNSUPPORTED;
-  }
-  BwdM g;
+static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.go = p.grad_out.data, g.q = p.q.data, g.k = p.k.data, g.v = p.v.data, g.out = p.out.data;
   g.lse = p.lse, g.gq = p.grad_q.data, g.gk = p.grad_k.data, g.gv = p.grad_v.data;
   g.delta = (float*)p.workspace;
@@ -552,6 +521,66 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.n_qt = (g.L + 127) / 128, g.n_kt = (g.S + 127) / 128;
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
+  g.kv_lens = p.kv_lens;
+  if (p.bias.data) {
+    g.bias = p.bias.data;
+    g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1];
+    g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
+  }
+}
+
+bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
+  *why = "";
+  const int64_t E = p.q.size[3], Dv = p.v.size[3];
+  if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
+  if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
+  if (p.grad_bias.data) return *why = "grad_attn_bias requested", false;
+  // masked calls: a bias / bool keep-mask that does not depend on the query row (key-padding
+  // masks, per-key biases) and per-batch key counts, in the kernels with 32-bit addressing
+  if (p.bias.data) {
+    const int esz = p.bias_dtype == MI355_SDPA_F32 ? 4 : p.bias_dtype == MI355_SDPA_BOOL ? 1
+                    : (p.bias_dtype == MI355_SDPA_F16 || p.bias_dtype == MI355_SDPA_BF16) ? 2 : 0;
+    if (!esz) return *why = "attn_bias dtype", false;
+    const int64_t S = p.k.size[2];
+    const int gran = 4 / esz;
+    if (p.q.size[2] > 1 && p.bias.stride[2] != 0) return *why = "attn_bias depends on the query row", false;
+    if (S > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
+    if (((uintptr_t)p.bias.data & 3) != 0 || S % gran != 0) return *why = "attn_bias not dword aligned", false;
+    for (int i = 0; i < 2; ++i)
+      if (p.bias.size[i] > 1 && (p.bias.stride[i] % gran) != 0) return *why = "attn_bias stride not dword aligned", false;
+  }
+  if (p.dropout_p > 0.f) return *why = "dropout", false;
+  if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
+  if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
+  const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
+  for (const mi355_sdpa_tensor* t : ts) {
+    if (t->stride[3] != 1) return *why = "head dim is not unit-stride", false;
+    if (((uintptr_t)t->data & 15) != 0) return *why = "pointer not 16-byte aligned", false;
+    for (int i = 0; i < 3; ++i)
+      if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
+  }
+  if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
+  if (p.bias.data || p.kv_lens) {
+    BwdM g;
+    fill(g, p);
+    const int D = (int)p.q.size[3];
+    if (!bwd_dkdv_w32_fits(g, D) || !bwd_dq_w32_fits(g, D)) return *why = "masked call beyond 32-bit offsets", false;
+  }
+  return true;
+}
+
+size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p) {
+  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * sizeof(float);
+}
+
+int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
+  const char* why;
+  if (!bwd_mfma_supported(p, &why)) {
+    set_error("SDPA: MFMA backward kernel cannot take this call: %s", why);
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  BwdM g;
+  fill(g, p);
   const int D = (int)p.q.size[3];
   if (p.dtype == MI355_SDPA_BF16) return D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
   return D == 128 ? launch_td<f16_t, 128>(g, s) : launch_td<f16_t, 64>(g, s);

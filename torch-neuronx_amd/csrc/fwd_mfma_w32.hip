@@ -185,19 +185,16 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   // so that everything downstream (reference tracking, lse) is the unbiased code.
   uint32_t braw[16];
   float inv_scale = 0.f;
-  __amdgpu_buffer_rsrc_t b_rsrc;
-  uint32_t b_off = 0;
-  const int bkind = MASK ? p.bias_kind : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  if constexpr (MASK) {
-    if (bkind) {
-      const int esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
-      const int rows = min(32, p.L - qw0);
-      const char* base = (const char*)p.bias + (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * esz;
-      b_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)base, 0, rows > 0 ? (int)(((rows - 1) * p.bias_sl + p.S) * esz) : 0, 0x00020000);
-      b_off = (uint32_t)((min(col, max(rows - 1, 0)) * p.bias_sl + half * 4) * esz);
-      inv_scale = 1.f / p.scale;
-    }
-  }
+  const int bkind = MASK ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  // (the resource is set up unconditionally, with no records when there is no bias: defined on one
+  // path only it stops being uniform for the compiler)
+  const int b_esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const int b_rows = min(32, p.L - qw0);
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * b_esz : 0)), 0,
+      __builtin_amdgcn_readfirstlane((bkind && b_rows > 0) ? (int)(((b_rows - 1) * p.bias_sl + p.S) * b_esz) : 0), 0x00020000);
+  const uint32_t b_off = (uint32_t)((min(col, max(b_rows - 1, 0)) * p.bias_sl + half * 4) * b_esz);
+  if (bkind) inv_scale = 1.f / p.scale;
   auto load_bias = [&](int t) {
     if constexpr (MASK) {
       if (bkind == 1) {

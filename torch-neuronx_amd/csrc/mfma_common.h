@@ -23,6 +23,14 @@ typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 
 constexpr float kLog2eF = 1.4426950408889634f;
 
+// A pointer that is the same in every lane, said so to the compiler (which otherwise wraps every
+// buffer access built on it in a loop over the distinct values it might hold).
+__device__ __forceinline__ void* uniform_ptr(const void* p) {
+  const uint64_t a = (uint64_t)p;
+  const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)a), hi = __builtin_amdgcn_readfirstlane((uint32_t)(a >> 32));
+  return (void*)(((uint64_t)hi << 32) | lo);
+}
+
 template <typename T>
 struct Mma;
 template <>
