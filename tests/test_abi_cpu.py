@@ -189,6 +189,8 @@ def test_host_ops_refuse_cpu_tensors(amd):
         amd.sdpa_forward(q, q, q)
     with pytest.raises(ValueError):
         amd.python_ops.scaled_dot_product_fused_attention_overrideable(q, q, q)
+    with pytest.raises(ValueError):
+        amd.native_multi_head_attn_mid(q, q, q)
 
 
 def test_registered_operator_surface(amd):

@@ -191,3 +191,68 @@ def test_llama_style_transposed_views_fwd_bwd(amd, gpu_device):
     assert max_abs(out, ro) <= 2e-2
     for a, r in ((xq.grad, rdq), (xk.grad, rdk), (xv.grad, rdv)):
         assert max_abs(a.transpose(1, 2), r) <= 5e-2 and rel_err(a.transpose(1, 2), r) <= 3e-2
+
+
+# ---- middle stage of native multi-head attention ([B, H, D, S] operands) ---------------------------
+# cases of the reference's tests/python_ops/test_native_multi_head_attn_mid.py, checked against
+# the oracle instead of only for shape and NaNs
+
+@pytest.mark.parametrize("dtype,B,H,D,S,causal", [
+    (torch.float32, 1, 8, 128, 512, False),
+    (torch.float32, 2, 4, 64, 384, True),       # a length the reference sends to its fallback
+    (torch.bfloat16, 1, 8, 128, 2048, False),
+    (torch.bfloat16, 1, 8, 128, 2048, True),
+    (torch.float16, 4, 16, 64, 1024, True),
+])
+def test_native_mha_mid(amd, gpu_device, dtype, B, H, D, S, causal):
+    q, k, v = qkv(B, H, H, S, S, D, dtype=dtype, seed=77)
+    # the op's layout: sequence last
+    qm, km, vm = (t.transpose(-2, -1).contiguous().to(gpu_device) for t in (q, k, v))
+    got = amd.native_multi_head_attn_mid(qm, km, vm, use_causal_mask=causal, dropout_p=0.0, training=False)
+    assert got.shape == (B, H, S, D) and got.device.type == "cuda" and got.dtype == dtype
+    ref, _ = oracle_fwd(q, k, v, is_causal=causal)
+    tol = 1e-5 if dtype is torch.float32 else 2e-2  # fp32 1e-5, half precisions 2e-2 against the fp32 oracle
+    assert max_abs(got, ref) <= tol
+    assert rel_err(got, ref) <= (1e-5 if dtype is torch.float32 else 1e-2)
+
+
+def test_native_mha_mid_gqa_and_value_width(amd, gpu_device):
+    # general form: H_kv key/value heads, value rows of their own width
+    B, Hq, Hkv, D, Dv, Sq, Sk = 2, 8, 2, 64, 32, 96, 160
+    q, k, v = qkv(B, Hq, Hkv, Sq, Sk, D, Dv=Dv, dtype=torch.float32, seed=78)
+    qm, km, vm = (t.transpose(-2, -1).contiguous().to(gpu_device) for t in (q, k, v))
+    got = amd.native_multi_head_attn_mid(qm, km, vm)
+    ref, _ = oracle_fwd(q, k.repeat_interleave(Hq // Hkv, 1), v.repeat_interleave(Hq // Hkv, 1))
+    assert got.shape == (B, Hq, Sq, Dv)
+    assert max_abs(got, ref) <= 1e-5
+
+
+def test_native_mha_mid_out_variant(amd, gpu_device):
+    B, H, D, S = 1, 8, 128, 512
+    q, k, v = qkv(B, H, H, S, S, D, dtype=torch.bfloat16, seed=79)
+    qm, km, vm = (t.transpose(-2, -1).contiguous().to(gpu_device) for t in (q, k, v))
+    out = torch.empty(B, H, S, D, dtype=torch.bfloat16, device=gpu_device)
+    got = amd.native_multi_head_attn_mid(qm, km, vm, out=out)
+    assert got is out
+    ref, _ = oracle_fwd(q, k, v)
+    assert max_abs(out, ref) <= 2e-2
+    with pytest.raises(RuntimeError, match="doesn't match expected shape"):
+        amd.native_multi_head_attn_mid(qm, km, vm, out=torch.empty(B, H, D, S, dtype=torch.bfloat16, device=gpu_device))
+
+
+def test_native_mha_mid_errors(amd, gpu_device):
+    B, H, D, S = 1, 8, 128, 2048
+    mk = lambda *shape: torch.randn(*shape, device=gpu_device)
+    q, k, v = mk(B, H, D, S), mk(B, H, D, S), mk(B, H, D, S)
+    with pytest.raises(RuntimeError):  # key shorter than value
+        amd.native_multi_head_attn_mid(q, mk(B, H, D, S // 2), v)
+    with pytest.raises(RuntimeError):  # value shorter than key
+        amd.native_multi_head_attn_mid(q, k, mk(B, H, D, S // 2))
+    with pytest.raises(RuntimeError):  # value in [B, H, S, D] order
+        amd.native_multi_head_attn_mid(q, k, mk(B, H, S, D))
+    with pytest.raises(RuntimeError, match="do not support empty tensors"):
+        amd.native_multi_head_attn_mid(mk(0, H, D, S), mk(0, H, D, S), mk(0, H, D, S))
+    with pytest.raises(RuntimeError, match="4-dimensional"):
+        amd.native_multi_head_attn_mid(mk(H, D, S), mk(H, D, S), mk(H, D, S))
+    with pytest.raises(ValueError):
+        amd.native_multi_head_attn_mid(q.cpu(), k.cpu(), v.cpu())

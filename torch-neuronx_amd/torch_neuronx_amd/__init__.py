@@ -13,6 +13,7 @@ from .kernels import (  # noqa: F401
     sdpa_decode_fp8kv,
 )
 from .ops import decode_fp8kv, sdpa_backward, sdpa_forward  # noqa: F401
+from .python_ops import native_multi_head_attn_mid  # noqa: F401
 from .registration import register, registered_ops, unregister  # noqa: F401
 
 if _os.environ.get("TORCH_NEURONX_AMD_REGISTER", "1").lower() not in ("0", "false", "off", "no"):
@@ -21,5 +22,5 @@ if _os.environ.get("TORCH_NEURONX_AMD_REGISTER", "1").lower() not in ("0", "fals
 __all__ = [
     "sdpa_forward", "sdpa_backward", "decode_fp8kv", "ops", "kernels", "python_ops", "registration",
     "register", "unregister", "registered_ops", "scaled_dot_product_attention_kernel",
-    "scaled_dot_product_attention_backward_kernel", "sdpa_decode_fp8kv",
+    "scaled_dot_product_attention_backward_kernel", "sdpa_decode_fp8kv", "native_multi_head_attn_mid",
 ]
