@@ -181,14 +181,21 @@ MASKED_BWD_CASES = [
     (2, 6, 3, 150, 264, 64, "float_key32", False),      # float32 bias shared by all heads
     (4, 8, 2, 200, 640, 128, "kv_lens", False),
     (3, 4, 4, 100, 200, 64, "kv_lens", True),
+    # masks with a row per query: one element per score
+    (2, 4, 2, 200, 328, 128, "bool_full", False),       # (B,1,L,S) keep-mask with fully masked rows
+    (2, 8, 2, 130, 256, 128, "float_full", True),        # (B,H,L,S) additive bias in the input dtype + causal
+    (1, 6, 3, 150, 264, 64, "float_full32", False),      # (1,1,L,S) float32 bias shared by batches and heads
+    (2, 4, 4, 96, 200, 64, "bool_window", False),        # sliding-window keep-mask (L,S)
+    (2, 4, 2, 77, 136, 128, "float_full_kv_lens", False),  # a full bias together with per-batch key counts
 ]
 
 
 @pytest.mark.parametrize("case", MASKED_BWD_CASES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_mfma_backward_with_key_masks(amd, gpu_device, case, dtype):
-    # key-only masks and per-batch key counts inside the MFMA backward kernels (forced: a call
-    # they cannot take is an error, not a fallback); cache rows past a batch's count hold NaN
+    # masks (per key or per score) and per-batch key counts inside the MFMA backward kernels
+    # (forced: a call they cannot take is an error, not a fallback); cache rows past a batch's
+    # count hold NaN
     B, Hq, Hkv, L, S, E, kind, causal = case
     q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L * 3 + S, with_do=True)
     go = go.clamp(-1, 1) * 0.1
@@ -206,6 +213,32 @@ def test_mfma_backward_with_key_masks(amd, gpu_device, case, dtype):
     elif kind == "float_key32":
         mask = 2.0 * torch.randn(1, 1, 1, S, generator=g)
         kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "bool_full":
+        mask = torch.rand(B, 1, L, S, generator=g) > 0.4
+        mask[:, :, 5] = False   # rows without a live key: zero gradients
+        mask[:, :, L - 1] = False
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "float_full":
+        mask = (2.0 * torch.randn(B, Hq, L, S, generator=g)).to(dtype)
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "float_full32":
+        mask = 2.0 * torch.randn(1, 1, L, S, generator=g)
+        mask[..., 3, :] = float("-inf")  # a row masked through the additive form
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "bool_window":
+        i, j = torch.arange(L)[:, None], torch.arange(S)[None, :]
+        mask = (j <= i + 40) & (j >= i - 23)
+        kw["attn_bias"] = mask.to(gpu_device)
+    elif kind == "float_full_kv_lens":
+        bias = (torch.randn(B, Hq, L, S, generator=g)).to(dtype)
+        lens = torch.tensor([S, 37], dtype=torch.int32)[:B]
+        pad = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+        mask = bias.float().masked_fill(~pad, float("-inf"))
+        kw["attn_bias"] = bias.to(gpu_device)
+        kw["kv_lens"] = lens.to(gpu_device)
+        for bi in range(B):
+            kd[bi, :, int(lens[bi]):] = float("nan")
+            vd[bi, :, int(lens[bi]):] = float("nan")
     else:
         lens = torch.randint(0, S + 1, (B,), generator=g).to(torch.int32)
         lens[0], lens[1] = S, 0

@@ -210,6 +210,35 @@ def test_mfma_forward_with_bias_and_masks(amd, gpu_device, case, dtype, tile):
         assert torch.isinf(lse[:, :, 3:40]).all() and (lse[:, :, 3:40] < 0).all()
 
 
+@pytest.mark.parametrize("kind", ["window", "left_padding", "late_and_low", "late_and_high"])
+@pytest.mark.parametrize("D", [64, 128])
+@pytest.mark.parametrize("tile", [3, 4])
+def test_mfma_forward_rows_whose_first_keys_are_masked(amd, gpu_device, kind, D, tile):
+    # The MFMA forward takes a row's softmax reference from its first key tile.  Rows whose first
+    # tiles are fully masked have none until a live key arrives; what arrives may lie far below or
+    # far above zero in the exponent.
+    B, Hq, Hkv, L, S = 2, 4, 2, 200, 328
+    q, k, v = qkv(B, Hq, Hkv, L, S, D, dtype=torch.bfloat16, seed=D + 5)
+    i, j = torch.arange(L)[:, None], torch.arange(S)[None, :]
+    if kind == "window":
+        mask = (j <= i + 40) & (j >= i - 23)  # sliding window: row i starts at key i - 23
+    elif kind == "left_padding":
+        start = torch.tensor([0, 150])[:B]
+        mask = (j[None] >= start[:, None, None])[:, None].expand(B, 1, L, S)
+    else:
+        # keys 0..99 masked, the live ones carry a bias of -200 / +60 (log2 domain: -288 / +87):
+        # probabilities against a reference of 0 would underflow / overflow
+        mask = torch.full((1, 1, L, S), float("-inf"))
+        mask[..., 100:] = -200.0 if kind == "late_and_low" else 60.0
+        mask[..., 100:] += torch.randn(L, S - 100, generator=torch.Generator().manual_seed(3))
+    out, lse = _run(amd, q, k, v, gpu_device, attn_bias=mask.to(gpu_device), force_kernel=tile)
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask if mask.dtype == torch.bool else mask.float())
+    assert torch.isfinite(lse).all()
+    assert max_abs(out, ro) <= 2e-2
+    assert rel_err(out, ro) <= 1e-2
+    assert max_abs(lse, rl) <= 3e-3
+
+
 @pytest.mark.parametrize("kind", ["float", "bool", "kv_lens"])
 @pytest.mark.parametrize("tile", [3, 4])
 def test_mfma_forward_masked_head_dim_64(amd, gpu_device, kind, tile):

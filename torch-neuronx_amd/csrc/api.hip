@@ -162,9 +162,10 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   if (d->return_debug_mask) return MI355_SDPA_KERNEL_NONE;
   if (E > 512 || Dv > 512) return MI355_SDPA_KERNEL_NONE;
   const float scale = d->has_scale ? d->scale : 1.f;
-  // a bias or mask is taken by the forward kernels only (its layout is checked again at the
-  // call); the backward of a masked call is the generic kernel's
-  const bool bias_ok = !d->has_attn_bias || !backward;
+  // (the layout of a bias or mask is checked again at the call; a requested bias gradient sends
+  // the backward to the generic kernel there)
+  (void)backward;
+  const bool bias_ok = true;
   const bool fast = d->q_dtype != MI355_SDPA_F32 && E == Dv && (E == 64 || E == 128) &&
                     bias_ok && d->dropout_p == 0.f && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;

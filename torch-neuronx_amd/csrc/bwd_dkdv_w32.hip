@@ -32,7 +32,9 @@ constexpr int smem_bytes() {  // three Q and three dO tiles, two P hand-over buf
   return 2 * 3 * BQ * D * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
 }
 
-// MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only
+// MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only (a lane
+// is a key: one register);  MASK = 2: a bias / keep-mask with a row per query as well (one element
+// per score, fetched by role A ahead of the tile's matrix ops)
 template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -193,17 +195,64 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
   };
 
+  const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const uint32_t b_rowbytes = MASK == 2 ? (uint32_t)(p.bias_sl * besz) : 0u;
+  const uint32_t b_lane = MASK == 2 ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
+  const int b_records = MASK == 2 ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0;
+  // the fetched bias elements of a tile, turned into floats in the log2 domain in place (the
+  // element type is tested once, outside the loops: inside, every element would carry the branch)
+  auto bias_to_log2 = [&](uint32_t (&w)[2][16]) {
+    auto each = [&](auto conv) {
+#pragma unroll
+      for (int mq = 0; mq < 2; ++mq)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) w[mq][r] = __builtin_bit_cast(uint32_t, conv(w[mq][r]));
+    };
+    if (bkind == 1) each([](uint32_t x) { return __builtin_bit_cast(float, x) * kLog2eF; });
+    else if (bkind == 4) each([](uint32_t x) { return x ? 0.f : -INFINITY; });
+    else if (bkind == 3) each([](uint32_t x) { return __builtin_bit_cast(float, x << 16) * kLog2eF; });
+    else each([](uint32_t x) { return (float)__builtin_bit_cast(_Float16, (uint16_t)x) * kLog2eF; });
+  };
+  // MASK = 2: the bias of this lane's key in each of a tile's 64 rows, in the order of the score
+  // accumulators, requested ahead of the tile's first product.  (Requesting it a tile ahead
+  // keeps 32 more registers live across the loop, which spills at head dim 128 and is slower.)
+  // The resource ends with
+  // the last row of the (batch, head): rows past L read as zeros (they are switched off through
+  // lse = +inf), keys past S as a neighbouring element (their probabilities are replaced by zero).
+  uint32_t braw[2][16];
+  auto load_bias_a = [&](int it) {
+    if constexpr (MASK == 2) {
+      const int q0 = item_q0(it);
+      if (it >= n_items || (p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
+      const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          uniform_ptr((const char*)p.bias + (b * p.bias_sb + item_head(it) * p.bias_sh) * besz), 0, b_records, 0x00020000);
+      const uint32_t base = b_lane + (uint32_t)q0 * b_rowbytes;
+      auto each = [&](auto fetch) {
+#pragma unroll
+        for (int mq = 0; mq < 2; ++mq)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            braw[mq][r] = fetch(base + (uint32_t)(mq * 32 + (r >> 2) * 8 + (r & 3)) * b_rowbytes);
+      };
+      if (bkind == 1) each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(b_rsrc, off, 0, 0); });
+      else if (bkind == 4) each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(b_rsrc, off, 0, 0); });
+      else each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(b_rsrc, off, 0, 0); });
+    }
+  };
   auto role_a = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
     if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;  // every key of this block lies above the diagonal / past the keys
     const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S);
+    load_bias_a(it);
     float bl = 0.f;  // this key's bias in the log2 domain
-    if constexpr (MASK) {
+    if constexpr (MASK == 1) {
       if (p.bias_kind)
         bl = bias_value(p.bias, b * p.bias_sb + item_head(it) * p.bias_sh + min(key, p.S - 1), p.bias_kind) * kLog2eF;
     }
     f32x16 sc[2];
     scores(q_t + tb * TILE, sc);
+    if constexpr (MASK == 2) bias_to_log2(braw);
     uint32_t pk[2][8];
 #pragma unroll
     for (int mq = 0; mq < 2; ++mq)
@@ -213,7 +262,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
         float pr[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
-          if constexpr (MASK) pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, bl) - l4[e]);
+          if constexpr (MASK == 2) pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, __builtin_bit_cast(float, braw[mq][r4 * 4 + e])) - l4[e]);
+          else if constexpr (MASK == 1) pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, bl) - l4[e]);
           else pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, -l4[e]));
           if (edge) {
             const int qi = q0 + mq * 32 + r4 * 8 + half * 4 + e;
@@ -322,6 +372,7 @@ int launch_t(const BwdM& g, hipStream_t s) {
 }
 template <typename T, int D>
 int launch_m(const BwdM& g, hipStream_t s) {
+  if (g.bias_kind && g.bias_sl != 0) return launch_t<T, D, 2>(g, s);
   return (g.bias_kind || g.kv_lens) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
 }
 

@@ -25,7 +25,7 @@ namespace {
 constexpr int BM = 256, BN = 32;
 constexpr int AHEAD = 4;
 
-// MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only
+// MASK = 1: per-batch key counts and a bias / bool keep-mask (a lane reads its own row of it)
 template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -175,8 +175,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       else sacc = Mma<T>::run(ring[i & 7], qf[i >> 1], i == 0 ? zero16 : sacc);
     }
   };
-  // Bias of a score tile (it depends on the key only): this lane's 16 keys, fetched one tile ahead
-  // as 4 groups of 4 consecutive keys; keys past the row read as zero (they are masked anyway).
+  // Bias of a score tile: this lane's 16 keys of its query row (row stride 0: a bias per key),
+  // fetched one tile ahead as 4 groups of 4 consecutive keys; keys past the row read the next row
+  // or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
   const int bkind = MASK ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
   const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
@@ -184,10 +185,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // one path only stops being uniform for the compiler)
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
-      __builtin_amdgcn_readfirstlane(bkind ? p.S * besz : 0), 0x00020000);
+      __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
+  const uint32_t b_row = MASK ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
   auto load_bias = [&](int t) {
     if constexpr (MASK) {
-      const uint32_t off = (uint32_t)((t * BN + half * 4) * besz);
+      const uint32_t off = b_row + (uint32_t)(t * BN * besz);
       if (bkind == 1) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -206,24 +208,33 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       }
     }
   };
-  auto bias_log2 = [&](int r) -> float {  // bias of accumulator register r, in the log2 domain
-    if (bkind == 1) return __builtin_bit_cast(float, braw[r]) * kLog2eF;
-    if (bkind == 4) return ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? 0.f : -INFINITY;
-    const uint32_t w = braw[r >> 1];
-    if (bkind == 3) return __builtin_bit_cast(float, (r & 1) ? (w & 0xffff0000u) : (w << 16)) * kLog2eF;
+  // bias of the 16 accumulator registers in the log2 domain (the element type is tested once,
+  // outside the loop: inside, every element would carry the branch)
+  auto bias_log2 = [&](float (&bl)[16]) {
     typedef __attribute__((ext_vector_type(2))) _Float16 h2;
-    return (float)__builtin_bit_cast(h2, w)[r & 1] * kLog2eF;
+    auto each = [&](auto conv) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bl[r] = conv(r);
+    };
+    if (bkind == 1) each([&](int r) { return __builtin_bit_cast(float, braw[r]) * kLog2eF; });
+    else if (bkind == 4) each([&](int r) { return ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? 0.f : -INFINITY; });
+    else if (bkind == 3)
+      each([&](int r) { return __builtin_bit_cast(float, (r & 1) ? (braw[r >> 1] & 0xffff0000u) : (braw[r >> 1] << 16)) * kLog2eF; });
+    else if (bkind == 2) each([&](int r) { return (float)__builtin_bit_cast(h2, braw[r >> 1])[r & 1] * kLog2eF; });
+    else each([](int) { return 0.f; });
   };
   // dS^T of tile t, packed as the B operand of dQ^T += K^T dS^T
   auto softmax = [&](int t, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
     const bool edge = t >= t_edge;
+    float bl[16];
+    if constexpr (MASK) bias_log2(bl);
 #pragma unroll
     for (int r = 0; r < 16; r += 2) {
       float ds[2];
 #pragma unroll
       for (int e = 0; e < 2; ++e) {
         float pr;
-        if (MASK && bkind) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bias_log2(r + e)) - lse2);
+        if constexpr (MASK) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
         else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
         if (edge) {
           const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);

@@ -16,11 +16,11 @@ struct BwdM {
   int n_qt, n_kt;
   int causal, xcd_map;
   float scale;
-  // masked calls (the two-wavefronts-per-SIMD kernels only): a bias or bool keep-mask that does not
-  // depend on the query row (stride 0 over L, unit stride over keys; strides in elements) and
-  // per-batch key counts
+  // masked calls (the two-wavefronts-per-SIMD kernels only): a bias or bool keep-mask (unit stride
+  // over keys; strides in elements; bias_sl = 0 for one that does not depend on the query row)
+  // and per-batch key counts
   const void* bias = nullptr;
-  int64_t bias_sb = 0, bias_sh = 0;
+  int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int32_t* kv_lens = nullptr;
 };

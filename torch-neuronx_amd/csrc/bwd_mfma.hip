@@ -525,6 +525,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   if (p.bias.data) {
     g.bias = p.bias.data;
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1];
+    g.bias_sl = p.q.size[2] > 1 ? p.bias.stride[2] : 0;
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
   }
 }
@@ -535,19 +536,22 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
   if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
   if (p.grad_bias.data) return *why = "grad_attn_bias requested", false;
-  // masked calls: a bias / bool keep-mask that does not depend on the query row (key-padding
-  // masks, per-key biases) and per-batch key counts, in the kernels with 32-bit addressing
+  // masked calls: a bias / bool keep-mask whose rows can be read four keys at a time and that one
+  // (batch, head) addresses with 32 bits, and per-batch key counts, in the kernels with 32-bit
+  // addressing
   if (p.bias.data) {
     const int esz = p.bias_dtype == MI355_SDPA_F32 ? 4 : p.bias_dtype == MI355_SDPA_BOOL ? 1
                     : (p.bias_dtype == MI355_SDPA_F16 || p.bias_dtype == MI355_SDPA_BF16) ? 2 : 0;
     if (!esz) return *why = "attn_bias dtype", false;
     const int64_t S = p.k.size[2];
     const int gran = 4 / esz;
-    if (p.q.size[2] > 1 && p.bias.stride[2] != 0) return *why = "attn_bias depends on the query row", false;
     if (S > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
     if (((uintptr_t)p.bias.data & 3) != 0 || S % gran != 0) return *why = "attn_bias not dword aligned", false;
-    for (int i = 0; i < 2; ++i)
+    for (int i = 0; i < 3; ++i)
       if (p.bias.size[i] > 1 && (p.bias.stride[i] % gran) != 0) return *why = "attn_bias stride not dword aligned", false;
+    if (p.q.size[2] > 1 && p.bias.stride[2] < 0) return *why = "attn_bias row stride is negative", false;
+    if (((p.q.size[2] + 64) * (p.q.size[2] > 1 ? p.bias.stride[2] : 0) + S + 64) * esz >= (1ll << 31))
+      return *why = "attn_bias rows beyond 32-bit offsets", false;
   }
   if (p.dropout_p > 0.f) return *why = "dropout", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;

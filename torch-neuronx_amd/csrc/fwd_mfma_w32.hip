@@ -371,7 +371,13 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- check ---------------------------------------------------------------------------------
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(ps <= kTrig)) != 0, 0)) {  // (NaN also lands here)
+    // (NaN also lands here.)  A row whose keys so far were all masked has no reference yet
+    // (m_run = -inf, probabilities formed against 0): it takes the slow path until a live key
+    // sets one, or sums against 0 would be rescaled from -inf, or underflow, later.  Without a
+    // mask key 0 is live for every row.
+    bool trig = !(ps <= kTrig);
+    if constexpr (MASK) trig |= m_run == -INFINITY;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(trig) != 0, 0)) {
       raise_reference(tile_max(scur));
       if (need_rescale) {
         l_run *= alpha;
