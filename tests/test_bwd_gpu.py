@@ -275,3 +275,37 @@ def test_backward_grad_layouts_follow_inputs(amd, gpu_device, kernel):
     ro, rl, rdq, rdk, rdv = _reference(q.cpu(), k.cpu(), v.cpu(), go.cpu(), is_causal=True)
     for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
         assert max_abs(a, r) <= 5e-2
+
+
+@pytest.mark.parametrize("E", [8, 32, 40, 56, 72, 80, 96, 112, 120])
+@pytest.mark.parametrize("variant", ["plain", "causal_gqa", "bias"])
+def test_mfma_backward_narrow_head_dims(amd, gpu_device, E, variant):
+    # head dims below 64 / 128 (multiples of 8) run in the next wider MFMA kernels, the tail of
+    # every row counting as zeros; the inputs are slices of wider tensors whose tails hold NaN, and
+    # the gradients go into slices of wider tensors whose tails must stay untouched
+    B, Hq, Hkv, L, S = (2, 4, 4, 150, 264) if variant != "causal_gqa" else (2, 8, 2, 200, 200)
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=torch.bfloat16, seed=E + 1, with_do=True)
+    go = go.clamp(-1, 1) * 0.1
+    dev = gpu_device
+
+    def wide(t):
+        w = torch.full(t.shape[:-1] + (E + 8,), float("nan"), dtype=t.dtype, device=dev)
+        w[..., :E] = t.to(dev)
+        return w[..., :E]
+
+    kw, mask = {}, None
+    if variant == "bias":
+        mask = (2.0 * torch.randn(1, Hq, L, S, generator=torch.Generator().manual_seed(E))).to(torch.bfloat16)
+        kw["attn_bias"] = mask.to(dev)
+    causal = variant == "causal_gqa"
+    qd, kd, vd, god = wide(q), wide(k), wide(v), wide(go)
+    out, lse = amd.sdpa_forward(qd, kd, vd, is_causal=causal, force_kernel=MFMA, **kw)
+    dq, dk, dv, _ = amd.sdpa_backward(god, qd, kd, vd, out, lse, is_causal=causal, force_kernel=MFMA, **kw)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+    om_mask = None if mask is None else mask.float()
+    ro, rl = oracle_fwd(q, k, v, attn_mask=om_mask, is_causal=causal)
+    rdq, rdk, rdv = oracle_bwd(go, q, k, v, ro, rl, attn_mask=om_mask, is_causal=causal)[:3]
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert torch.isfinite(a.float()).all(), name
+        assert max_abs(a, r) <= 5e-2, name
+        assert rel_err(a, r) <= 2e-2, name

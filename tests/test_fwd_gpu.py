@@ -372,3 +372,34 @@ def test_softmax_reference_tracking_under_stress(amd, gpu_device, kind, causal, 
     assert torch.isfinite(out.float()).all() and torch.isfinite(lse).all()
     assert max_abs(out, ro) <= 2e-2  # bf16 output tolerance of the path
     assert max_abs(lse, rl) <= 2e-3 * max(1.0, rl.abs().max().item())
+
+
+@pytest.mark.parametrize("E", [8, 32, 40, 56, 72, 80, 96, 112, 120])
+@pytest.mark.parametrize("variant", ["plain", "causal_gqa", "bias"])
+def test_mfma_forward_narrow_head_dims(amd, gpu_device, E, variant):
+    # head dims below 64 / 128 (multiples of 8) run in the next wider MFMA kernel, the tail of every
+    # row counting as zeros; the tensors are slices of wider ones whose tails hold NaN, so a read
+    # past a row's end would show
+    B, Hq, Hkv, L, S = (2, 4, 4, 150, 264) if variant != "causal_gqa" else (2, 8, 2, 200, 200)
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=torch.bfloat16, seed=E)
+    dev = gpu_device
+
+    def wide(t):
+        w = torch.full(t.shape[:-1] + (E + 8,), float("nan"), dtype=t.dtype, device=dev)
+        w[..., :E] = t.to(dev)
+        return w[..., :E]
+
+    kw = {}
+    mask = None
+    if variant == "bias":
+        mask = (2.0 * torch.randn(1, Hq, L, S, generator=torch.Generator().manual_seed(E))).to(torch.bfloat16)
+        kw["attn_bias"] = mask.to(dev)
+    causal = variant == "causal_gqa"
+    for tile in (3, 4):
+        out, lse = amd.sdpa_forward(wide(q), wide(k), wide(v), is_causal=causal, force_kernel=tile, **kw)
+        assert out.shape == (B, Hq, L, E)
+        ro, rl = oracle_fwd(q, k, v, attn_mask=None if mask is None else mask.float(), is_causal=causal)
+        assert torch.isfinite(out.float()).all()
+        assert max_abs(out, ro) <= 2e-2
+        assert rel_err(out, ro) <= 1e-2
+        assert max_abs(lse, rl) <= 3e-3

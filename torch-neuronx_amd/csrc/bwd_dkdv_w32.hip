@@ -32,6 +32,8 @@ constexpr int smem_bytes() {  // three Q and three dO tiles, two P hand-over buf
   return 2 * 3 * BQ * D * 2 + 2 * 4 * 64 * 16 * 4 + 2 * 3 * BQ * 4;
 }
 
+// MASK >= 1 also serves head dims below D (multiples of 8): the missing tail of every row counts
+// as zeros.
 // MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only (a lane
 // is a key: one register);  MASK = 2: a bias / keep-mask with a row per query as well (one element
 // per score, fetched by role A ahead of the tile's matrix ops)
@@ -59,6 +61,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int k0 = kt * BK, kw0 = k0 + kb * 32;
   const int key = kw0 + col;
 
+  const int dr = MASK ? p.d_real : D;  // elements per row that exist
   int S = p.S;  // keys of this batch that take part
   if constexpr (MASK) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
@@ -70,7 +73,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     const uint16_t* r = role ? (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl
                              : (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) frag[ks] = *(const u32x4*)(r + half * 8 + ks * 16);
+    for (int ks = 0; ks < KS; ++ks) {
+      if (!MASK || half * 8 + ks * 16 < dr) frag[ks] = *(const u32x4*)(r + half * 8 + ks * 16);
+      else frag[ks] = u32x4{0u, 0u, 0u, 0u};
+    }
   }
 
   const int nqs = (p.L + BQ - 1) / BQ;
@@ -84,8 +90,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // Buffer resources end with the last row of the batch (the tile offset travels in the vector
   // offset, which is the part the hardware checks against that bound): rows past L read as zeros
   // or as another head's rows, and are switched off through lse = +inf.
-  const int64_t q_ext = ((int64_t)(p.Hq - 1) * p.q_sh + (int64_t)(p.L - 1) * p.q_sl + D) * 2;
-  const int64_t go_ext = ((int64_t)(p.Hq - 1) * p.go_sh + (int64_t)(p.L - 1) * p.go_sl + D) * 2;
+  const int64_t q_ext = ((int64_t)(p.Hq - 1) * p.q_sh + (int64_t)(p.L - 1) * p.q_sl + dr) * 2;
+  const int64_t go_ext = ((int64_t)(p.Hq - 1) * p.go_sh + (int64_t)(p.L - 1) * p.go_sl + dr) * 2;
   const __amdgpu_buffer_rsrc_t q_rsrc =
       __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.q + b * p.q_sb), 0, (int)q_ext, 0x00020000);
   const __amdgpu_buffer_rsrc_t go_rsrc =
@@ -98,6 +104,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     go_off[n] = (uint32_t)(((s_row + (512 / CH) * n) * p.go_sl + s_ch * 8) * 2);
   }
   u32x4 sq[NCH], sgo[NCH];
+  const bool fetch = !MASK || s_ch * 8 < dr;  // chunks past the end of a narrow row stay zero
+#pragma unroll
+  for (int n = 0; n < NCH; ++n) sq[n] = sgo[n] = u32x4{0u, 0u, 0u, 0u};
   float lse_r = 0.f, dl_r = 0.f;
   auto load_item = [&](int it) {
     const int h = item_head(it), q0 = item_q0(it);
@@ -105,8 +114,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     const uint32_t gb = (uint32_t)((h * p.go_sh + (int64_t)q0 * p.go_sl) * 2);
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      sq[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, q_off[n] + qb, 0, 0);
-      sgo[n] = __builtin_amdgcn_raw_buffer_load_b128(go_rsrc, go_off[n] + gb, 0, 0);
+      if (fetch) {
+        sq[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, q_off[n] + qb, 0, 0);
+        sgo[n] = __builtin_amdgcn_raw_buffer_load_b128(go_rsrc, go_off[n] + gb, 0, 0);
+      }
     }
     if (tid < BQ) {
       const int qi = q0 + tid;
@@ -353,7 +364,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
         u32x2 w;
         w[0] = Mma<T>::pack(acc[db][gq * 4] * sc, acc[db][gq * 4 + 1] * sc);
         w[1] = Mma<T>::pack(acc[db][gq * 4 + 2] * sc, acc[db][gq * 4 + 3] * sc);
-        *(u32x2*)(g + db * 32 + gq * 8 + half * 4) = w;
+        if (!MASK || db * 32 + gq * 8 + half * 4 < dr) *(u32x2*)(g + db * 32 + gq * 8 + half * 4) = w;
       }
   }
 }
@@ -373,7 +384,7 @@ int launch_t(const BwdM& g, hipStream_t s) {
 template <typename T, int D>
 int launch_m(const BwdM& g, hipStream_t s) {
   if (g.bias_kind && g.bias_sl != 0) return launch_t<T, D, 2>(g, s);
-  return (g.bias_kind || g.kv_lens) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
+  return (g.bias_kind || g.kv_lens || g.d_real != D) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
 }
 
 }  // namespace

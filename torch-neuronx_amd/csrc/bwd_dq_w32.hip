@@ -25,7 +25,8 @@ namespace {
 constexpr int BM = 256, BN = 32;
 constexpr int AHEAD = 4;
 
-// MASK = 1: per-batch key counts and a bias / bool keep-mask (a lane reads its own row of it)
+// MASK = 1: per-batch key counts and a bias / bool keep-mask (a lane reads its own row of it); also
+// head dims below D (multiples of 8), the missing tail of every row counting as zeros
 template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -63,6 +64,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   const int q0 = qt * BM, qw0 = q0 + wave * 32;
   const int qrow = qw0 + col, qc = min(qrow, p.L - 1);
 
+  const int dr = MASK ? p.d_real : D;  // elements per row that exist
   // this lane's query row as B operand of the score products
   u32x4 qf[KS], dof[KS];
   float lse2, dl;
@@ -70,7 +72,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     const uint16_t* qr = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl + half * 8;
     const uint16_t* gr = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl + half * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16), dof[ks] = *(const u32x4*)(gr + ks * 16);
+    for (int ks = 0; ks < KS; ++ks) {
+      if (!MASK || half * 8 + ks * 16 < dr) qf[ks] = *(const u32x4*)(qr + ks * 16), dof[ks] = *(const u32x4*)(gr + ks * 16);
+      else qf[ks] = dof[ks] = u32x4{0u, 0u, 0u, 0u};
+    }
     const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc;
     const float l = p.lse[idx];
     // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
@@ -85,7 +90,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       if (qrow < p.L) {
         uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
-        for (int i = 0; i < D / 16; ++i) *(u32x4*)(gq + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
+        for (int i = 0; i < D / 16; ++i)
+          if (half * (D / 2) + i * 8 < dr) *(u32x4*)(gq + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
       }
       return;
     }
@@ -104,24 +110,28 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // tile beyond it read as zeros (their probabilities are masked to zero).
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
-  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + D) * 2);
+  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + dr) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + dr) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
-  const bool do_k = !SPLIT || tid < TCH, do_v = !SPLIT || tid >= TCH;  // (uniform per wavefront)
   const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
   const int s_row = s_idx / CH, s_ch = s_idx % CH;
+  // (uniform per wavefront, unless the rows are narrower than D: chunks past their end are never
+  // fetched, and the zeros they start with are what goes to LDS)
+  const bool fetch = !MASK || s_ch * 8 < dr;
+  const bool do_k = (!SPLIT || tid < TCH) && fetch, do_v = (!SPLIT || tid >= TCH) && fetch;
+  const bool put_k = !SPLIT || tid < TCH, put_v = !SPLIT || tid >= TCH;
   const uint32_t k_off = (uint32_t)((s_row * p.k_sl + s_ch * 8) * 2), v_off = (uint32_t)((s_row * p.v_sl + s_ch * 8) * 2);
   const uint32_t k_tile_bytes = (uint32_t)(BN * p.k_sl * 2), v_tile_bytes = (uint32_t)(BN * p.v_sl * 2);
   const int s_lds = s_row * D + ((s_ch ^ tile_swz<D>(s_row)) << 3);
-  u32x4 kreg, vreg;
+  u32x4 kreg = {0u, 0u, 0u, 0u}, vreg = {0u, 0u, 0u, 0u};
   auto load_tile = [&](int t) {
     const uint32_t tt = (uint32_t)min(t, nt - 1);
     if (do_k) kreg = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off + tt * k_tile_bytes, 0, 0);
     if (do_v) vreg = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off + tt * v_tile_bytes, 0, 0);
   };
   auto store_tile = [&](int buf) {
-    if (do_k) *(u32x4*)(&k_t[buf][s_lds]) = kreg;
-    if (do_v) *(u32x4*)(&v_t[buf][s_lds]) = vreg;
+    if (put_k) *(u32x4*)(&k_t[buf][s_lds]) = kreg;
+    if (put_v) *(u32x4*)(&v_t[buf][s_lds]) = vreg;
   };
 
   // element offsets inside a tile (the swizzle is not additive in the d block / contraction step:
@@ -303,7 +313,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
         u32x2 w;
         w[0] = Mma<T>::pack(dqacc[db][g * 4] * p.scale, dqacc[db][g * 4 + 1] * p.scale);
         w[1] = Mma<T>::pack(dqacc[db][g * 4 + 2] * p.scale, dqacc[db][g * 4 + 3] * p.scale);
-        *(u32x2*)(gq + db * 32 + g * 8 + half * 4) = w;
+        if (!MASK || db * 32 + g * 8 + half * 4 < dr) *(u32x2*)(gq + db * 32 + g * 8 + half * 4) = w;
       }
   }
 }
@@ -319,7 +329,7 @@ bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
 int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
-  const bool bf = dtype == MI355_SDPA_BF16, masked = g.bias_kind || g.kv_lens;
+  const bool bf = dtype == MI355_SDPA_BF16, masked = g.bias_kind || g.kv_lens || g.d_real != head_dim;
 #define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, 0, s, g)
 #define LAUNCH_D(DD)                                                         \
   do {                                                                       \

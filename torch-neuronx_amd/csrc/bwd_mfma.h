@@ -23,6 +23,10 @@ struct BwdM {
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int32_t* kv_lens = nullptr;
+  // Elements per row that exist (a multiple of 8).  Below the head dim a kernel is built for, the
+  // masked variants treat the rest of every Q / K / V / dO / O row as zeros and leave it out of
+  // the gradients; 0 means the full width.
+  int d_real = 0;
 };
 
 // bias element as a float (bool: 0 or -inf)

@@ -46,7 +46,7 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(BwdM p) {
     const int i = (int)(row % p.L), h = (int)((row / p.L) % p.Hq), b = (int)(row / ((int64_t)p.L * p.Hq));
     const uint16_t* g = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)i * p.go_sl + sub * 8;
     const uint16_t* o = (const uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)i * p.o_sl + sub * 8;
-    s = dot8<T>(*(const u32x4*)g, *(const u32x4*)o);
+    if (sub * 8 < p.d_real) s = dot8<T>(*(const u32x4*)g, *(const u32x4*)o);
   }
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
@@ -490,7 +490,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   if (rc) return rc;
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  if ((wg256 >= 256 || g.bias_kind || g.kv_lens) && bwd_dq_w32_fits(g, D))  // (a masked call has no other kernel)
+  if ((wg256 >= 256 || g.bias_kind || g.kv_lens || g.d_real != D) && bwd_dq_w32_fits(g, D))  // (a masked call has no other kernel)
     return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
   if (D == 128 && wg256 >= 256) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
@@ -522,6 +522,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
   g.kv_lens = p.kv_lens;
+  g.d_real = (int)p.q.size[3];
   if (p.bias.data) {
     g.bias = p.bias.data;
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1];
@@ -534,7 +535,8 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   *why = "";
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
-  if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
+  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  const bool padded = E != 64 && E != 128;  // served by the next wider kernels' masked variants
   if (p.grad_bias.data) return *why = "grad_attn_bias requested", false;
   // masked calls: a bias / bool keep-mask whose rows can be read four keys at a time and that one
   // (batch, head) addresses with 32 bits, and per-batch key counts, in the kernels with 32-bit
@@ -564,11 +566,11 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
       if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
   }
   if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
-  if (p.bias.data || p.kv_lens) {
+  if (p.bias.data || p.kv_lens || padded) {
     BwdM g;
     fill(g, p);
-    const int D = (int)p.q.size[3];
-    if (!bwd_dkdv_w32_fits(g, D) || !bwd_dq_w32_fits(g, D)) return *why = "masked call beyond 32-bit offsets", false;
+    const int D = E <= 64 ? 64 : 128;
+    if (!bwd_dkdv_w32_fits(g, D) || !bwd_dq_w32_fits(g, D)) return *why = "masked call / padded head dim beyond 32-bit offsets", false;
   }
   return true;
 }
@@ -585,7 +587,7 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   }
   BwdM g;
   fill(g, p);
-  const int D = (int)p.q.size[3];
+  const int D = p.q.size[3] <= 64 ? 64 : 128;  // the kernels' width
   if (p.dtype == MI355_SDPA_BF16) return D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
   return D == 128 ? launch_td<f16_t, 128>(g, s) : launch_td<f16_t, 64>(g, s);
 }

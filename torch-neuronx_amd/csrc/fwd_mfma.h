@@ -24,6 +24,10 @@ struct FwdM {
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int32_t* kv_lens = nullptr;
+  // Elements per row that exist (a multiple of 8).  Below the head dim a kernel is built for, the
+  // masked variant treats the rest of every Q / K / V row as zeros and leaves it out of the output
+  // (head dims 8 .. 56 in the 64 kernel, 72 .. 120 in the 128 kernel); 0 means the full width.
+  int d_real = 0;
 };
 
 // Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first
@@ -56,7 +60,8 @@ __device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int&
 }
 
 
-// head dim 64 or 128; waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup
+// head_dim 64 or 128: the width the kernel is built for (g.d_real: the width of the data);
+// waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup
 int launch_fwd_mfma_w32(const FwdM& g, int dtype, int head_dim, int waves, hipStream_t s);
 
 }  // namespace mi355

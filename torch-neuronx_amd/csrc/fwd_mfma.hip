@@ -331,12 +331,13 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   *why = ok;
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
-  if (E != Dv || (E != 64 && E != 128)) return *why = "head dim is not 64 or 128", false;
-  // masked calls (bias, bool keep-mask, per-batch key counts): the kernels with 32-bit row
-  // addressing only, and a bias whose rows can be read four keys at a time
-  if (p.bias.data || p.kv_lens) {
+  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  const bool padded = E != 64 && E != 128;  // served by the next wider kernel's masked variant
+  // masked calls (bias, bool keep-mask, per-batch key counts) and padded head dims: the kernels
+  // with 32-bit row addressing only, and a bias whose rows can be read four keys at a time
+  if (p.bias.data || p.kv_lens || padded) {
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
-      return *why = "attn_bias / kv_lens with rows beyond 32-bit offsets", false;
+      return *why = "attn_bias / kv_lens / padded head dim with rows beyond 32-bit offsets", false;
   }
   if (p.bias.data) {
     const int esz = p.bias_dtype == MI355_SDPA_F32 ? 4 : p.bias_dtype == MI355_SDPA_BOOL ? 1
@@ -387,7 +388,8 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1], g.bias_sl = p.bias.stride[2];
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
   }
-  const int D = (int)p.q.size[3];
+  g.d_real = (int)p.q.size[3];
+  const int D = g.d_real <= 64 ? 64 : 128;  // the kernel's width
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;

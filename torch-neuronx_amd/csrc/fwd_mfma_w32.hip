@@ -1,4 +1,4 @@
-// Flash-attention forward for gfx950, head dim 128, bf16/f16.
+// Flash-attention forward for gfx950, head dim 64 or 128 (narrower rows: see MASK), bf16/f16.
 //
 // One workgroup = WAVES wavefronts of 32 query rows each, all of one (batch, query head):
 // WAVES = 8 (256 rows, one workgroup per compute unit) for long sequences, WAVES = 4 (128 rows,
@@ -38,7 +38,9 @@ constexpr int AHEAD = 4;  // LDS operands are requested this many matrix ops ahe
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
 // MASK = 1 adds what a masked call brings: per-batch key counts (kv_lens) and an additive bias or
-// boolean keep-mask, folded into the score tile right after the matrix ops that produce it.
+// boolean keep-mask, folded into the score tile right after the matrix ops that produce it.  It
+// also serves head dims below D (multiples of 8): the missing tail of every Q / K / V row counts
+// as zeros, which changes neither the scores nor the live part of the output.
 template <typename T, int D, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
@@ -67,6 +69,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   const int qrow = qw0 + col;
   const int qw_last = qw0 + 31;
 
+  const int dr = MASK ? p.d_real : D;  // elements per row that exist
   // keys of this batch that take part
   int S = p.S;
   if constexpr (MASK) {
@@ -75,7 +78,8 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       if (qrow < p.L) {
         uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
-        for (int i = 0; i < D / 16; ++i) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
+        for (int i = 0; i < D / 16; ++i)
+          if (half * (D / 2) + i * 8 < dr) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
         if (p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = -INFINITY;
       }
       return;
@@ -90,7 +94,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   {
     const uint16_t* qr = qp + (int64_t)min(qrow, p.L - 1) * p.q_sl + half * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) qf[ks] = *(const u32x4*)(qr + ks * 16);
+    for (int ks = 0; ks < KS; ++ks) {
+      if (!MASK || half * 8 + ks * 16 < dr) qf[ks] = *(const u32x4*)(qr + ks * 16);
+      else qf[ks] = u32x4{0u, 0u, 0u, 0u};
+    }
   }
 
   int nt = (S + BN - 1) / BN;
@@ -104,16 +111,25 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   // Two staging sets each: a tile is fetched from global memory two iterations before it is
   // written to LDS, so a fetch has about two tile times to land.
   u32x4 kreg[2][KLD], vreg[2][KLD];
-  const bool do_k = !SPLIT || tid < TCH, do_v = !SPLIT || tid >= TCH;  // (uniform per wavefront)
   const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
   const int k_chunk = s_idx % CH, k_row = s_idx / CH;  // rows k_row + i * NT / CH
+  // (uniform per wavefront, unless the rows are narrower than D: chunks past their end are never
+  // fetched, and the zeros they start with are what goes to LDS)
+  const bool fetch = !MASK || k_chunk * 8 < dr;
+  const bool do_k = (!SPLIT || tid < TCH) && fetch, do_v = (!SPLIT || tid >= TCH) && fetch;
+  const bool put_k = !SPLIT || tid < TCH, put_v = !SPLIT || tid >= TCH;
+  if constexpr (MASK) {
+#pragma unroll
+    for (int i = 0; i < KLD; ++i)
+      kreg[0][i] = kreg[1][i] = vreg[0][i] = vreg[1][i] = u32x4{0u, 0u, 0u, 0u};
+  }
   // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
   // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
   // instruction with one addition on the vector unit.  The resources end with the last key row
   // of this (batch, head), and the whole offset travels in the vector offset, the part the
   // hardware checks against that bound: rows of a ragged last tile beyond it read as zeros
   // (their scores are masked, and a zero V row keeps 0 * V finite).
-  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + D) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + D) * 2);
+  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + dr) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + dr) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
   uint32_t k_off[KLD], v_off[KLD];
@@ -138,14 +154,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
     }
   };
   auto store_k = [&](int set, int buf) {
-    if (do_k) {
+    if (put_k) {
 #pragma unroll
       for (int i = 0; i < KLD; ++i)
         *(u32x4*)(&k_lds[buf][(k_row + i * (NT / CH)) * KROW + k_chunk * 8]) = kreg[set][i];
     }
   };
   auto store_v = [&](int set, int buf) {
-    if (do_v) {
+    if (put_v) {
 #pragma unroll
       for (int i = 0; i < KLD; ++i)
         *(u32x4*)(&v_lds[buf][(k_row + i * (NT / CH)) * VP + k_chunk * 8]) = vreg[set][i];
@@ -473,7 +489,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
         u32x2 w;
         w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
         w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
-        *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
+        if (!MASK || db * 32 + g * 8 + half * 4 < dr) *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
       }
     if (p.lse && half == 0)
       p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
@@ -484,6 +500,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
 
 int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipStream_t s) {
   FwdM g = g0;
+  if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
@@ -492,7 +509,7 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   dim3 grid((unsigned)blocks), block(64 * waves);
-  const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr;
+  const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr || g.d_real != head_dim;
   const bool bf = dtype == MI355_SDPA_BF16;
 #define LAUNCH(TT, DD, WW, MM) hipLaunchKernelGGL((fwd_w32_kernel<TT, DD, WW, MM>), grid, block, 0, s, g)
 #define LAUNCH_D(DD)                                                                    \
