@@ -109,7 +109,8 @@ def compute_attention(query, key, value, attn_bias, dropout_mask, scale, is_caus
 
 
 def compute_attention_backward(
-    grad_out, query, key, value, attn_bias, dropout_mask, out, lse, scale, is_causal, dropout_p
+    grad_out, query, key, value, attn_bias, dropout_mask, out, lse, scale, is_causal, dropout_p,
+    bias_present=None,
 ):
     """Backward for head-expanded operands; returns ``(dQ, dK, dV, dBias-or-None)``.
 
@@ -122,7 +123,8 @@ def compute_attention_backward(
     acc = accumulator_dtype(in_dtype)
     go, q, k, v, o = (t.to(acc) for t in (grad_out, query, key, value, out))
     lse = lse.to(acc)
-    with_bias = _bias_present_bwd(attn_bias)
+    # (bias_present: the decision of a caller that hands in one slice of a larger bias)
+    with_bias = _bias_present_bwd(attn_bias) if bias_present is None else bias_present
     # a one-element bias is a lowering placeholder: ignored here, while the forward
     # (numel > 0) would still add it
     bias = attn_bias.to(acc) if with_bias else None
@@ -265,9 +267,12 @@ def sdpa_backward(
                 if mask.shape[1] > 1:
                     mask = mask[:, h0:h1]
             _, _, bias, _ = normalize_sdpa_args(cast(sel(query)), kb, vb, mask, scale, False)
+            # the one-element-placeholder rule applies to the bias of the whole call, not to the
+            # slice of it that this chunk sees
             gq, gk, gv, _ = compute_attention_backward(
                 cast(sel(grad_out)), cast(sel(query)), kb, vb, bias, None,
                 cast(sel(out)), sel(lse), scale, is_causal, 0.0,
+                bias_present=None if attn_mask is None else _bias_present_bwd(attn_mask),
             )
             dq[b, h0:h1] = gq[0]
             dk[b].index_add_(0, heads // rep, gk[0])

@@ -174,6 +174,24 @@ def test_head_chunking_does_not_change_results():
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
 
 
+@pytest.mark.parametrize("S", [1, 3])
+def test_chunking_keeps_a_per_batch_bias_in_the_backward(S):
+    # A (B,1,1,1) bias has more than one element, so the backward applies it; the wrapper hands the
+    # math one batch at a time, where each slice has a single element and would pass for the
+    # placeholder that the backward ignores.  Checked against autograd of the library routine.
+    B, H, L, E = 2, 2, 4, 8
+    g = torch.Generator().manual_seed(9)
+    q, k, v = [torch.randn(shape, generator=g, dtype=torch.float64).requires_grad_(True)
+               for shape in ((B, H, L, E), (B, H, S, E), (B, H, S, E))]
+    bias = 2 * torch.randn(B, 1, 1, 1, generator=g, dtype=torch.float64)
+    go = torch.randn(B, H, L, E, generator=g, dtype=torch.float64)
+    F.scaled_dot_product_attention(q, k, v, attn_mask=bias).backward(go)
+    out, lse = om.sdpa_forward(q.detach(), k.detach(), v.detach(), attn_mask=bias)
+    dq, dk, dv = om.sdpa_backward(go, q.detach(), k.detach(), v.detach(), out, lse, attn_mask=bias)
+    for a, e in ((dq, q.grad), (dk, k.grad), (dv, v.grad)):
+        torch.testing.assert_close(a, e, rtol=1e-5, atol=1e-6)  # lse is stored in float32
+
+
 def test_reduce_gqa_gradients_with_different_head_dims():
     # reference: test_sdpa_nki_gates.py:142-168
     gk = torch.randn(2, 8, 5, 6)
