@@ -115,20 +115,42 @@ def last_error() -> str:
     return load().mi355_sdpa_last_error().decode()
 
 
+_I64x4 = C.c_int64 * 4
+
+
 def tensor4(t) -> Tensor4:
-    r = Tensor4()
     if t is None:
-        return r
+        return Tensor4()
     assert t.dim() == 4
-    r.data = t.data_ptr()
-    for i in range(4):
-        r.size[i] = t.size(i)
-        r.stride[i] = t.stride(i)
-    return r
+    return Tensor4(t.data_ptr(), _I64x4(*t.shape), _I64x4(*t.stride()))
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 
 
 def current_stream(device) -> int:
+    """Handle of torch's current stream on ``device`` (a hipStream_t as an integer)."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
     return torch.cuda.current_stream(device).cuda_stream
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device(device):
+    """Context that makes ``device`` current for the launch; free when it already is."""
+    if device.index is None or torch.cuda.current_device() == device.index:
+        return _NO_SWITCH
+    return torch.cuda.device(device)
 
 
 def check(rc: int) -> None:

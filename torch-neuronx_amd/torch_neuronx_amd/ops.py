@@ -80,6 +80,8 @@ def out_strides(ref_sizes, ref_strides, out_sizes):
 
 def empty_like_layout(ref: torch.Tensor, shape, dtype=None) -> torch.Tensor:
     """New tensor of ``shape`` whose dimension order follows ``ref`` (stride-0 dims never alias)."""
+    if ref.is_contiguous():  # the common case needs no stride arithmetic
+        return torch.empty(tuple(shape), dtype=dtype or ref.dtype, device=ref.device)
     st = out_strides(ref.shape, ref.stride(), shape)
     return torch.empty_strided(tuple(shape), st, dtype=dtype or ref.dtype, device=ref.device)
 
@@ -129,7 +131,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
-    with torch.cuda.device(query.device):
+    with _lib.on_device(query.device):
         rc = _lib.load().mi355_sdpa_fwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
     return out, lse
@@ -180,7 +182,7 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     nbytes = lib.mi355_sdpa_bwd_workspace_bytes(C.byref(p))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=query.device)
     p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
-    with torch.cuda.device(query.device):
+    with _lib.on_device(query.device):
         rc = lib.mi355_sdpa_bwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
     return dq, dk, dv, dbias
@@ -213,7 +215,7 @@ def decode_fp8kv(query, k_fp8, v_fp8, k_scale, v_scale, kv_lens=None, scale=None
     nbytes = lib.mi355_sdpa_decode_workspace_bytes(C.byref(p))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=query.device)
     p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
-    with torch.cuda.device(query.device):
+    with _lib.on_device(query.device):
         rc = lib.mi355_sdpa_decode_fp8kv(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
     return out, lse

@@ -33,10 +33,33 @@ def _check_device(query: torch.Tensor) -> None:
         raise ValueError(f"Expected a ROCm GPU device, got {query.device}")
 
 
+_rng_placeholders = {}
+
+
 def _empty_rng(device):
-    # inert placeholders when no dropout is applied (reference: decompositions.py:2309-2311)
-    return (torch.empty((0,), dtype=torch.int32, device=device),
-            torch.empty((0,), dtype=torch.int32, device=device))
+    # inert placeholders when no dropout is applied (reference: decompositions.py:2309-2311);
+    # never written, so one pair per device serves every call
+    pair = _rng_placeholders.get(device)
+    if pair is None:
+        pair = (torch.empty((0,), dtype=torch.int32, device=device),
+                torch.empty((0,), dtype=torch.int32, device=device))
+        _rng_placeholders[device] = pair
+    return pair
+
+
+_validated = set()
+
+
+def _validate_once(query, key, value, attn_bias, dropout_p, is_causal, scale):
+    """Boundary checks of the call; a signature that passed is not checked again."""
+    sig = (query.shape, key.shape, value.shape, query.dtype, key.dtype, value.dtype, key.device.type,
+           value.device.type, attn_bias is None, dropout_p, is_causal, scale,
+           query.stride(-1), key.stride(-1), value.stride(-1))
+    if sig in _validated:
+        return
+    ops.validate(ops.make_desc(query, key, value, attn_bias, dropout_p, is_causal, False, scale))
+    if len(_validated) < 4096 and all(isinstance(d, int) for t in (query, key, value) for d in t.shape):
+        _validated.add(sig)
 
 
 def _dropout_keep(query, S, dropout_p):
@@ -52,7 +75,7 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
     _check_device(query)
     if return_debug_mask:
         raise NotImplementedError("Debug mask not supported in Neuron implementation.")
-    ops.validate(ops.make_desc(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale))
+    _validate_once(query, key, value, attn_bias, dropout_p, is_causal, scale)
     orig_dtype = query.dtype
     if orig_dtype == torch.float64:  # computed as float32, result restored to the caller's dtype
         query, key, value = query.float(), key.float(), value.float()
