@@ -309,3 +309,53 @@ def test_mfma_backward_narrow_head_dims(amd, gpu_device, E, variant):
         assert torch.isfinite(a.float()).all(), name
         assert max_abs(a, r) <= 5e-2, name
         assert rel_err(a, r) <= 2e-2, name
+
+
+@pytest.mark.parametrize("case", [
+    # B, Hq, Hkv, L, S, E, bias shape kind, causal, kv_lens
+    (2, 4, 2, 150, 264, 128, "full", False, False),
+    (2, 4, 4, 96, 200, 64, "bcast", False, False),
+    (2, 4, 2, 130, 256, 128, "full", True, False),     # zeros above the diagonal, written by the kernel
+    (3, 2, 1, 77, 136, 96, "full", False, True),       # zeros past each batch's keys; a narrow head dim
+])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_backward_grad_bias(amd, gpu_device, case, dtype):
+    # grad_bias = P (dP - delta) leaves the MFMA dQ kernel in the input dtype (forced: no fallback);
+    # the buffer starts as NaN, so every element must be written
+    B, Hq, Hkv, L, S, E, kind, causal, with_lens = case
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L + S, with_do=True)
+    go = go.clamp(-1, 1) * 0.1
+    g = torch.Generator().manual_seed(S)
+    bias = torch.randn((B, Hq, L, S) if kind == "full" else (1, Hq, L, S), generator=g).to(dtype)
+    dev = gpu_device
+    kw = {"attn_bias": bias.to(dev)}
+    mask = bias.float().expand(B, Hq, L, S)
+    if with_lens:
+        lens = torch.tensor([S, 0, 37], dtype=torch.int32)[:B]
+        kw["kv_lens"] = lens.to(dev)
+        pad = (torch.arange(S)[None, :] < lens[:, None])[:, None, None, :]
+        mask = mask.masked_fill(~pad, float("-inf"))
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), is_causal=causal, force_kernel=MFMA, **kw)
+    import torch_neuronx_amd.ops as ops
+    real_empty = torch.empty
+
+    def nan_empty(*a, **k2):  # poison what the host allocates for the gradients
+        t = real_empty(*a, **k2)
+        return t.fill_(float("nan")) if t.is_floating_point() else t
+
+    torch.empty = nan_empty
+    try:
+        dq, dk, dv, db = ops.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, is_causal=causal,
+                                           want_grad_bias=True, force_kernel=MFMA, **kw)
+    finally:
+        torch.empty = real_empty
+    rep = Hq // Hkv
+    ke, ve = k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1)
+    ro, rl = om.compute_attention(q.float(), ke, ve, mask, None, E**-0.5, causal, 0.0)
+    rdq, _, _, rdb = om.compute_attention_backward(go.float(), q.float(), ke, ve, mask, None, ro, rl, E**-0.5, causal, 0.0)
+    assert db.shape == (B, Hq, L, S) and db.dtype == dtype
+    assert torch.isfinite(db.float()).all()
+    assert max_abs(db, rdb) <= 5e-2 and rel_err(db, rdb) <= 2e-2
+    assert max_abs(dq, rdq) <= 5e-2
+    if causal:
+        assert (db.float().cpu().triu(1) == 0).all()

@@ -83,10 +83,26 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     dl = p.delta[idx];
   }
 
+  uint16_t* gb_row = nullptr;  // this lane's row of the bias gradient, at its first key of a tile
+  if constexpr (MASK) {
+    if (p.gbias && qrow < p.L)
+      gb_row = (uint16_t*)p.gbias + b * p.gbias_sb + h * p.gbias_sh + (int64_t)qrow * p.gbias_sl + half * 4;
+  }
+  auto zero_gbias = [&](int t_from) {  // tiles this wavefront does not visit
+    if constexpr (MASK) {
+      if (gb_row) {
+        for (int t = t_from; t * BN < p.S; ++t)
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            if (t * BN + g * 8 + half * 4 < p.S) *(u32x2*)(gb_row + t * BN + g * 8) = u32x2{0u, 0u};
+      }
+    }
+  };
   int S = p.S;  // keys of this batch that take part
   if constexpr (MASK) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
     if (S == 0) {  // no live key: zero gradient
+      zero_gbias(0);
       if (qrow < p.L) {
         uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
@@ -254,6 +270,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       }
       pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
     }
+    if constexpr (MASK) {
+      // grad_bias = grad_logits (torch_neuronx/_sdpa_math.py:163,169): the packed pairs are its
+      // elements in the input dtype already; four consecutive keys per store
+      if (gb_row) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (t * BN + g * 8 + half * 4 < p.S) *(u32x2*)(gb_row + t * BN + g * 8) = u32x2{pS[2 * g], pS[2 * g + 1]};
+      }
+    }
   };
   auto accumulate = [&](int buf, const uint32_t (&pS)[8]) {
     u32x4 ring[8];
@@ -303,6 +328,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     iteration(t + 1, s_b, dp_b, s_a, dp_a);
   }
   if (t < nt) iteration(t, s_a, dp_a, s_b, dp_b);
+  zero_gbias(nt_w);
 
   if (qrow < p.L) {
     uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
@@ -329,7 +355,7 @@ bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
 int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
-  const bool bf = dtype == MI355_SDPA_BF16, masked = g.bias_kind || g.kv_lens || g.d_real != head_dim;
+  const bool bf = dtype == MI355_SDPA_BF16, masked = g.bias_kind || g.kv_lens || g.gbias || g.d_real != head_dim;
 #define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, 0, s, g)
 #define LAUNCH_D(DD)                                                         \
   do {                                                                       \

@@ -23,6 +23,11 @@ struct BwdM {
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int32_t* kv_lens = nullptr;
+  // gradient of the bias (the dQ kernel writes it): P (dP - delta) in the input dtype, one element
+  // per score, unit stride over keys, rows a whole number of 8-byte words (zeros where a score
+  // takes no part: above the causal diagonal, past a batch's keys)
+  void* gbias = nullptr;
+  int64_t gbias_sb = 0, gbias_sh = 0, gbias_sl = 0;
   // Elements per row that exist (a multiple of 8).  Below the head dim a kernel is built for, the
   // masked variants treat the rest of every Q / K / V / dO / O row as zeros and leave it out of
   // the gradients; 0 means the full width.

@@ -490,7 +490,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   if (rc) return rc;
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  if ((wg256 >= 256 || g.bias_kind || g.kv_lens || g.d_real != D) && bwd_dq_w32_fits(g, D))  // (a masked call has no other kernel)
+  if ((wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D) && bwd_dq_w32_fits(g, D))  // (a masked call has no other kernel)
     return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
   if (D == 128 && wg256 >= 256) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
@@ -523,6 +523,10 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
+  if (p.grad_bias.data) {
+    g.gbias = p.grad_bias.data;
+    g.gbias_sb = p.grad_bias.stride[0], g.gbias_sh = p.grad_bias.stride[1], g.gbias_sl = p.grad_bias.stride[2];
+  }
   if (p.bias.data) {
     g.bias = p.bias.data;
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1];
@@ -537,7 +541,14 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
   const bool padded = E != 64 && E != 128;  // served by the next wider kernels' masked variants
-  if (p.grad_bias.data) return *why = "grad_attn_bias requested", false;
+  if (p.grad_bias.data) {  // written by the dQ kernel four keys (8 bytes) at a time
+    const int64_t S = p.k.size[2];
+    if (!p.bias.data) return *why = "grad_attn_bias without attn_bias", false;
+    if (S % 4 != 0 || (S > 1 && p.grad_bias.stride[3] != 1) || ((uintptr_t)p.grad_bias.data & 7) != 0)
+      return *why = "grad_attn_bias rows are not whole 8-byte words", false;
+    for (int i = 0; i < 3; ++i)
+      if (p.grad_bias.size[i] > 1 && (p.grad_bias.stride[i] % 4) != 0) return *why = "grad_attn_bias stride not 8-byte aligned", false;
+  }
   // masked calls: a bias / bool keep-mask whose rows can be read four keys at a time and that one
   // (batch, head) addresses with 32 bits, and per-batch key counts, in the kernels with 32-bit
   // addressing
