@@ -374,10 +374,10 @@ def test_softmax_reference_tracking_under_stress(amd, gpu_device, kind, causal, 
     assert max_abs(lse, rl) <= 2e-3 * max(1.0, rl.abs().max().item())
 
 
-@pytest.mark.parametrize("E", [8, 32, 40, 56, 72, 80, 96, 112, 120])
+@pytest.mark.parametrize("E", [8, 32, 40, 56, 72, 80, 96, 112, 120, 136, 160, 192, 248, 256])
 @pytest.mark.parametrize("variant", ["plain", "causal_gqa", "bias"])
 def test_mfma_forward_narrow_head_dims(amd, gpu_device, E, variant):
-    # head dims below 64 / 128 (multiples of 8) run in the next wider MFMA kernel, the tail of every
+    # head dims below 64 / 128 / 256 (multiples of 8) run in the next wider MFMA kernel, the tail of every
     # row counting as zeros; the tensors are slices of wider ones whose tails hold NaN, so a read
     # past a row's end would show
     B, Hq, Hkv, L, S = (2, 4, 4, 150, 264) if variant != "causal_gqa" else (2, 8, 2, 200, 200)

@@ -164,9 +164,8 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   const float scale = d->has_scale ? d->scale : 1.f;
   // (the layout of a bias or mask is checked again at the call; a requested bias gradient sends
   // the backward to the generic kernel there)
-  (void)backward;
   const bool bias_ok = true;
-  const bool fast = d->q_dtype != MI355_SDPA_F32 && E == Dv && E % 8 == 0 && E <= 128 &&
+  const bool fast = d->q_dtype != MI355_SDPA_F32 && E == Dv && E % 8 == 0 && E <= (backward ? 128 : 256) &&
                     bias_ok && d->dropout_p == 0.f && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;
   return fast ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;

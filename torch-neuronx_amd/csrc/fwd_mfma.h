@@ -60,8 +60,8 @@ __device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int&
 }
 
 
-// head_dim 64 or 128: the width the kernel is built for (g.d_real: the width of the data);
-// waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup
+// head_dim 64, 128 or 256: the width the kernel is built for (g.d_real: the width of the data);
+// waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup, 4 only at head dim 256
 int launch_fwd_mfma_w32(const FwdM& g, int dtype, int head_dim, int waves, hipStream_t s);
 
 }  // namespace mi355

@@ -331,11 +331,12 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   *why = ok;
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
-  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  const bool padded = E != 64 && E != 128;  // served by the next wider kernel's masked variant
+  if (E != Dv || E < 8 || E > 256 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 256", false;
+  const bool padded = E != 64 && E != 128 && E != 256;  // served by the next wider kernel's masked variant
+  const bool w32_only = padded || E > 128;
   // masked calls (bias, bool keep-mask, per-batch key counts) and padded head dims: the kernels
   // with 32-bit row addressing only, and a bias whose rows can be read four keys at a time
-  if (p.bias.data || p.kv_lens || padded) {
+  if (p.bias.data || p.kv_lens || w32_only) {
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
       return *why = "attn_bias / kv_lens / padded head dim with rows beyond 32-bit offsets", false;
   }
@@ -389,7 +390,7 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
   }
   g.d_real = (int)p.q.size[3];
-  const int D = g.d_real <= 64 ? 64 : 128;  // the kernel's width
+  const int D = g.d_real <= 64 ? 64 : g.d_real <= 128 ? 128 : 256;  // the kernel's width
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
                          : p.force_kernel == MI355_SDPA_KERNEL_MFMA_T128 ? 128 : 0;
@@ -400,7 +401,7 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   // 128-row workgroups always (measured crossovers on MI355X).
   if ((int64_t)g.S * g.k_sl * 2 < (1ll << 31) && (int64_t)g.S * g.v_sl * 2 < (1ll << 31)) {
     const bool big = D == 128 && ((g.S >= 2048 && wg256 >= (g.causal ? 512 : 256)) || (!g.causal && g.S >= 1024 && wg256 >= 512));
-    const int rows = force_tile ? force_tile : big ? 256 : 128;
+    const int rows = D == 256 ? 128 : force_tile ? force_tile : big ? 256 : 128;
     return launch_fwd_mfma_w32(g, p.dtype, D, rows / 32, s);
   }
   // strides beyond 32-bit offsets: the kernel above (64-bit addressing)

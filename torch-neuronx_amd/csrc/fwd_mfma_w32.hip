@@ -42,7 +42,7 @@ constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescale
 // also serves head dims below D (multiples of 8): the missing tail of every Q / K / V row counts
 // as zeros, which changes neither the scores nor the live part of the output.
 template <typename T, int D, int WAVES, int MASK>
-__global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) {
+__global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
   constexpr int KS = D / 16;      // matrix ops of S^T = K Q^T per tile (phase A)
   constexpr int DB = D / 32;      // 32-row blocks of O^T
@@ -55,8 +55,14 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
   constexpr bool SPLIT = NT > TCH;  // more threads than chunks: one half stages K, the other V
   constexpr int KLD = SPLIT ? 1 : TCH / NT;  // chunks of a tile per staging thread
   static_assert(AHEAD <= KS && AHEAD <= NPV && (KS + NPV) % 8 == 0, "ring layout");
-  __shared__ __attribute__((aligned(16))) uint16_t k_lds[2][BN * KROW];
-  __shared__ __attribute__((aligned(16))) uint16_t v_lds[2][BN * VP];
+  // (head dim 256 needs more than the 64 KB of LDS a kernel may declare: it takes the launch's
+  // dynamic LDS instead, and runs one wavefront per SIMD with the 512-register budget)
+  constexpr bool DYN = D > 128;
+  __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : 2 * BN * KROW];
+  __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : 2 * BN * VP];
+  extern __shared__ __attribute__((aligned(16))) uint16_t dyn_lds[];
+  uint16_t (*const k_lds)[BN * KROW] = (uint16_t (*)[BN * KROW])(DYN ? dyn_lds : k_static);
+  uint16_t (*const v_lds)[BN * VP] = (uint16_t (*)[BN * VP])(DYN ? dyn_lds + 2 * BN * KROW : v_static);
 
   int b, h, qt;
   decode_block(p, b, h, qt);
@@ -383,7 +389,7 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
       else ring[(ks + AHEAD) & 7] = read_v(ks + AHEAD - KS);
       snext = Mma<T>::run(ring[ks & 7], qf[ks], ks == 0 ? zero16 : snext);
 #pragma unroll
-      for (int hs = 0; hs < 8 / KS; ++hs) softmax_slot(scur, 4, ks * (8 / KS) + hs, pk, ps);
+      for (int hs = ks * 8 / KS; hs < (ks + 1) * 8 / KS; ++hs) softmax_slot(scur, 4, hs, pk, ps);
       __builtin_amdgcn_sched_barrier(0);
     }
     // ---- check ---------------------------------------------------------------------------------
@@ -442,9 +448,10 @@ __global__ __launch_bounds__(64 * WAVES, 8 / WAVES) void fwd_w32_kernel(FwdM p) 
         if (__builtin_expect(t + 1 >= t_edge, 0)) mask_tile(snext, (t + 1) * BN);  // rare
         stage1(snext, 0);
       }
-      constexpr int HSB = 8 / NPV;
+      // half-steps 0 .. 6 spread over the slots (the last one trails the loop)
 #pragma unroll
-      for (int hs = (i == 0 ? 0 : i * HSB - 1); hs < (i + 1) * HSB - 1; ++hs) softmax_slot(snext, 0, hs, pkn, psn);
+      for (int hs = (i == 0 ? 0 : max((i * 8) / NPV - 1, 0)); hs < max(((i + 1) * 8) / NPV - 1, 0); ++hs)
+        softmax_slot(snext, 0, hs, pkn, psn);
       if (i == 0) store_k(par, par);  // tile t+2
       if (i == 1) store_v(par ^ 1, par ^ 1);  // tile t+1
       if (i == NPV / 2) load_k(par, t + 4);
@@ -522,7 +529,22 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
       else { if (bf) LAUNCH(bf16_t, DD, 4, 0); else LAUNCH(f16_t, DD, 4, 0); }          \
     }                                                                                   \
   } while (0)
-  if (head_dim == 128) LAUNCH_D(128);
+  if (head_dim == 256) {  // 128-row workgroups only, dynamic LDS
+    constexpr int kBytes = (2 * BN * (256 + 8) + 2 * BN * (256 + 32)) * 2;
+#define LAUNCH_256(TT, MM)                                                                                   \
+  do {                                                                                                       \
+    static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<TT, 256, 4, MM>,          \
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);  \
+    if (attr != hipSuccess) {                                                                                \
+      set_error("SDPA: cannot reserve %d bytes of LDS for fwd_w32_kernel: %s", kBytes, hipGetErrorString(attr)); \
+      return MI355_SDPA_ERR_LAUNCH;                                                                          \
+    }                                                                                                        \
+    hipLaunchKernelGGL((fwd_w32_kernel<TT, 256, 4, MM>), grid, block, kBytes, s, g);                         \
+  } while (0)
+    if (masked) { if (bf) LAUNCH_256(bf16_t, 1); else LAUNCH_256(f16_t, 1); }
+    else { if (bf) LAUNCH_256(bf16_t, 0); else LAUNCH_256(f16_t, 0); }
+#undef LAUNCH_256
+  } else if (head_dim == 128) LAUNCH_D(128);
   else LAUNCH_D(64);
 #undef LAUNCH_D
 #undef LAUNCH
