@@ -170,7 +170,8 @@ def test_kernel_gates(amd):
     q100 = _meta(2, 8, 512, 100)
     assert gate(q100, q100, q100) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     q2, k2 = _meta(1, 4, 64, 192), _meta(1, 4, 64, 192)
-    assert gate(q2, k2, _meta(1, 4, 64, 128)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)  # D_qk != D_v
+    assert gate(q2, k2, _meta(1, 4, 64, 128)) == (L.KERNEL_MFMA, L.KERNEL_GENERIC)  # D_qk > D_v: forward only
+    assert gate(_meta(1, 4, 64, 64), _meta(1, 4, 64, 64), _meta(1, 4, 64, 128)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(_meta(1, 4, 64, 640), _meta(1, 4, 64, 640), _meta(1, 4, 64, 640)) == (L.KERNEL_NONE, L.KERNEL_NONE)
     assert gate(q, _meta(1, 3, 8192, 128), _meta(1, 3, 8192, 128)) == (L.KERNEL_NONE, L.KERNEL_NONE)
     assert gate(_meta(1, 4, 0, 64), _meta(1, 4, 16, 64), _meta(1, 4, 16, 64)) == (L.KERNEL_NONE, L.KERNEL_NONE)

@@ -403,3 +403,18 @@ def test_mfma_forward_narrow_head_dims(amd, gpu_device, E, variant):
         assert max_abs(out, ro) <= 2e-2
         assert rel_err(out, ro) <= 1e-2
         assert max_abs(lse, rl) <= 3e-3
+
+
+@pytest.mark.parametrize("E,Dv", [(192, 128), (128, 64), (96, 64), (256, 128), (64, 32)])
+@pytest.mark.parametrize("causal", [False, True])
+def test_mfma_forward_value_rows_narrower_than_keys(amd, gpu_device, E, Dv, causal):
+    # D_qk > D_v (multi-head latent attention: 192 / 128, reference gate cases
+    # tests/neuron_dynamo_backend/unit/test_sdpa_nki_gates.py:52-56) inside the MFMA forward kernel
+    B, Hq, Hkv, L, S = 2, 8, 2, 200, 264
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, Dv=Dv, dtype=torch.bfloat16, seed=E + Dv)
+    out, lse = _run(amd, q, k, v, gpu_device, is_causal=causal, force_kernel=MFMA)
+    assert out.shape == (B, Hq, L, Dv)
+    ro, rl = oracle_fwd(q, k, v, is_causal=causal)
+    assert max_abs(out, ro) <= 2e-2
+    assert rel_err(out, ro) <= 1e-2
+    assert max_abs(lse, rl) <= 3e-3

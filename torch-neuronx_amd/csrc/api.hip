@@ -165,7 +165,8 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   // (the layout of a bias or mask is checked again at the call; a requested bias gradient sends
   // the backward to the generic kernel there)
   const bool bias_ok = true;
-  const bool fast = d->q_dtype != MI355_SDPA_F32 && E == Dv && E % 8 == 0 && E <= (backward ? 128 : 256) &&
+  const bool dims = backward ? (E == Dv && E % 8 == 0 && E <= 128) : (E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E);
+  const bool fast = d->q_dtype != MI355_SDPA_F32 && dims &&
                     bias_ok && d->dropout_p == 0.f && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;
   return fast ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;

@@ -27,7 +27,8 @@ struct FwdM {
   // Elements per row that exist (a multiple of 8).  Below the head dim a kernel is built for, the
   // masked variant treats the rest of every Q / K / V row as zeros and leaves it out of the output
   // (head dims 8 .. 56 in the 64 kernel, 72 .. 120 in the 128 kernel); 0 means the full width.
-  int d_real = 0;
+  // dv_real: the same for V and the output, which may be narrower than Q and K (192 / 128).
+  int d_real = 0, dv_real = 0;
 };
 
 // Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first

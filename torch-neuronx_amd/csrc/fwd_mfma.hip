@@ -331,8 +331,10 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   *why = ok;
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
-  if (E != Dv || E < 8 || E > 256 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 256", false;
-  const bool padded = E != 64 && E != 128 && E != 256;  // served by the next wider kernel's masked variant
+  // (V may be narrower than Q and K, as in multi-head latent attention's 192 / 128)
+  if (E < 8 || E > 256 || E % 8 != 0 || Dv < 8 || Dv > E || Dv % 8 != 0)
+    return *why = "head dims are not multiples of 8 up to 256 with D_v <= D_qk", false;
+  const bool padded = (E != 64 && E != 128 && E != 256) || Dv != E;  // served by the next wider kernel's masked variant
   const bool w32_only = padded || E > 128;
   // masked calls (bias, bool keep-mask, per-batch key counts) and padded head dims: the kernels
   // with 32-bit row addressing only, and a bias whose rows can be read four keys at a time
@@ -389,7 +391,7 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1], g.bias_sl = p.bias.stride[2];
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
   }
-  g.d_real = (int)p.q.size[3];
+  g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   const int D = g.d_real <= 64 ? 64 : g.d_real <= 128 ? 128 : 256;  // the kernel's width
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256

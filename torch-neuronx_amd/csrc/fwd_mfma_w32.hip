@@ -75,7 +75,8 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const int qrow = qw0 + col;
   const int qw_last = qw0 + 31;
 
-  const int dr = MASK ? p.d_real : D;  // elements per row that exist
+  const int dr = MASK ? p.d_real : D;    // elements per row of Q and K that exist
+  const int drv = MASK ? p.dv_real : D;  // ... of V and the output
   // keys of this batch that take part
   int S = p.S;
   if constexpr (MASK) {
@@ -85,7 +86,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
         uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
         for (int i = 0; i < D / 16; ++i)
-          if (half * (D / 2) + i * 8 < dr) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
+          if (half * (D / 2) + i * 8 < drv) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
         if (p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = -INFINITY;
       }
       return;
@@ -121,8 +122,8 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const int k_chunk = s_idx % CH, k_row = s_idx / CH;  // rows k_row + i * NT / CH
   // (uniform per wavefront, unless the rows are narrower than D: chunks past their end are never
   // fetched, and the zeros they start with are what goes to LDS)
-  const bool fetch = !MASK || k_chunk * 8 < dr;
-  const bool do_k = (!SPLIT || tid < TCH) && fetch, do_v = (!SPLIT || tid >= TCH) && fetch;
+  const bool do_k = (!SPLIT || tid < TCH) && (!MASK || k_chunk * 8 < dr);
+  const bool do_v = (!SPLIT || tid >= TCH) && (!MASK || k_chunk * 8 < drv);
   const bool put_k = !SPLIT || tid < TCH, put_v = !SPLIT || tid >= TCH;
   if constexpr (MASK) {
 #pragma unroll
@@ -135,7 +136,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // of this (batch, head), and the whole offset travels in the vector offset, the part the
   // hardware checks against that bound: rows of a ragged last tile beyond it read as zeros
   // (their scores are masked, and a zero V row keeps 0 * V finite).
-  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + dr) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + dr) * 2);
+  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + dr) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + drv) * 2);
   const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
   const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
   uint32_t k_off[KLD], v_off[KLD];
@@ -496,7 +497,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
         u32x2 w;
         w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
         w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
-        if (!MASK || db * 32 + g * 8 + half * 4 < dr) *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
+        if (!MASK || db * 32 + g * 8 + half * 4 < drv) *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
       }
     if (p.lse && half == 0)
       p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
@@ -508,6 +509,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipStream_t s) {
   FwdM g = g0;
   if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
+  if (g.dv_real <= 0 || g.dv_real > head_dim) g.dv_real = g.d_real;
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
@@ -516,7 +518,7 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   dim3 grid((unsigned)blocks), block(64 * waves);
-  const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr || g.d_real != head_dim;
+  const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim;
   const bool bf = dtype == MI355_SDPA_BF16;
 #define LAUNCH(TT, DD, WW, MM) hipLaunchKernelGGL((fwd_w32_kernel<TT, DD, WW, MM>), grid, block, 0, s, g)
 #define LAUNCH_D(DD)                                                                    \
