@@ -256,3 +256,52 @@ def test_native_mha_mid_errors(amd, gpu_device):
         amd.native_multi_head_attn_mid(mk(H, D, S), mk(H, D, S), mk(H, D, S))
     with pytest.raises(ValueError):
         amd.native_multi_head_attn_mid(q.cpu(), k.cpu(), v.cpu())
+
+
+# ---- HIP graph capture -----------------------------------------------------------------------------
+
+def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
+    # The library only launches kernels on the stream it is given (no allocation, no memset, no
+    # synchronisation), so forward, backward and decode can be recorded into one graph.  The graph
+    # is replayed several times on fresh inputs, with eager work and synchronisations in between,
+    # and every replay is checked against the eager result.
+    from oracle import sdpa_math as om
+
+    dev = gpu_device
+    B, Hq, Hkv, L, E = 2, 8, 2, 256, 128
+    g = torch.Generator().manual_seed(404)
+    mk = lambda *s: torch.randn(*s, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v, go = mk(B, Hq, L, E), mk(B, Hkv, L, E), mk(B, Hkv, L, E), mk(B, Hq, L, E)
+    bias = mk(1, Hq, L, L)
+    qd = mk(4, Hq, 1, E)
+    kq, ks = om.quantize_kv_fp8(torch.randn(4, Hkv, 512, E, generator=g))
+    vq, vs = om.quantize_kv_fp8(torch.randn(4, Hkv, 512, E, generator=g))
+    kq, vq, ks, vs = kq.to(dev), vq.to(dev), ks.to(dev), vs.to(dev)
+    lens = torch.tensor([512, 1, 300, 77], dtype=torch.int32, device=dev)
+
+    def work():
+        out, lse = amd.sdpa_forward(q, k, v, is_causal=True)
+        dq, dk, dv, _ = amd.sdpa_backward(go, q, k, v, out, lse, is_causal=True)
+        outb, lseb = amd.sdpa_forward(q, k, v, attn_bias=bias)
+        dqb, dkb, dvb, dbb = amd.sdpa_backward(go, q, k, v, outb, lseb, attn_bias=bias, want_grad_bias=True)
+        od, ld = amd.decode_fp8kv(qd, kq, vq, ks, vs, lens)
+        return [out, lse, dq, dk, dv, outb, dqb, dkb, dvb, dbb, od, ld]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        work()  # warm-up outside the capture (first-launch attribute calls, allocator pools)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = work()
+    for rep in range(3):
+        for t in (q, k, v, go, qd):
+            t.copy_(torch.randn(t.shape, generator=g).to(t.dtype))
+        bias.mul_(0.5)
+        eager = [t.clone() for t in work()]
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for i, (a, b) in enumerate(zip(captured, eager)):
+            assert torch.equal(a, b), (rep, i)
