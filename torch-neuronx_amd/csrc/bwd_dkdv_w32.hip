@@ -21,6 +21,8 @@
 // come out of the transposing LDS read ds_read_b64_tr_b16, so nothing is transposed on the
 // vector unit.  Math follows torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows
 // with lse = -inf give zero gradients, scale multiplies dK once at the end.
+#include <type_traits>
+
 #include "bwd_mfma.h"
 
 namespace mi355 {
@@ -251,45 +253,109 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       else each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(b_rsrc, off, 0, 0); });
     }
   };
-  auto role_a = [&](int it, int tb, int pb) {
-    const int q0 = item_q0(it);
-    if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;  // every key of this block lies above the diagonal / past the keys
-    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S);
+  // One tile of role A, software pipelined by hand (a wavefront issues in order, and left alone
+  // the compiler emits a tile's matrix ops in two solid runs with all of the vector work between
+  // them, which leaves the overlap to the other wavefront of the SIMD alone):
+  //   phase 1  scores of rows 0-31
+  //   phase 2  scores of rows 32-63        | probabilities of rows 0-31
+  //   phase 3  dV from rows 0-31           | probabilities of rows 32-63
+  //   phase 4  dV from rows 32-63
+  // Every matrix op is one slot: the LDS operand of the op AHEAD slots later is requested, the op
+  // is issued, and 16 / KS probabilities are formed.  A tile that crosses the causal diagonal or
+  // the end of the keys (edge) has the scores of its masked positions set to -inf between the
+  // phases, in blocks of their own: tested per element inside the unrolled loops, the compiler
+  // turns the test into selects that every element of every tile pays for.
+  auto role_a_tile = [&](int it, int tb, int pb, bool edge) {
+    constexpr int EPS = 16 / KS;  // probabilities per slot (2 or 4)
+    constexpr int SPG = 4 / EPS;  // slots per group of four consecutive rows
     load_bias_a(it);
     float bl = 0.f;  // this key's bias in the log2 domain
     if constexpr (MASK == 1) {
       if (p.bias_kind)
         bl = bias_value(p.bias, b * p.bias_sb + item_head(it) * p.bias_sh + min(key, p.S - 1), p.bias_kind) * kLog2eF;
     }
-    f32x16 sc[2];
-    scores(q_t + tb * TILE, sc);
-    if constexpr (MASK == 2) bias_to_log2(braw);
-    uint32_t pk[2][8];
-#pragma unroll
-    for (int mq = 0; mq < 2; ++mq)
-#pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const f32x4 l4 = *(const f32x4*)(&lse_s[tb * BQ + mq * 32 + r4 * 8 + half * 4]);
-        float pr[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          if constexpr (MASK == 2) pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, __builtin_bit_cast(float, braw[mq][r4 * 4 + e])) - l4[e]);
-          else if constexpr (MASK == 1) pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, bl) - l4[e]);
-          else pr[e] = __builtin_amdgcn_exp2f(fmaf(sc[mq][r4 * 4 + e], c, -l4[e]));
-          if (edge) {
-            const int qi = q0 + mq * 32 + r4 * 8 + half * 4 + e;
-            pr[e] = ((p.causal && key > qi) || key >= S) ? 0.f : pr[e];
-          }
-        }
-        pk[mq][r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pk[mq][r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
-      }
+    const uint16_t* qt = q_t + tb * TILE;
+    const uint16_t* dot = do_t + tb * TILE;
+    const float* lrow = &lse_s[tb * BQ + half * 4];
     uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;  // [4 groups of 4 words][lane][4]
+    f32x16 sc[2];
+    uint32_t pk[2][8];
+    f32x4 l4[2][4];
+    u32x4 ring[8];
+    auto load_l4 = [&](int mq, int r4) { l4[mq][r4] = *(const f32x4*)(lrow + mq * 32 + r4 * 8); };
+    auto prob = [&](int mq, int r) {
+      const float l = l4[mq][r >> 2][r & 3];
+      float x;
+      if constexpr (MASK == 2) x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, __builtin_bit_cast(float, braw[mq][r])) - l);
+      else if constexpr (MASK == 1) x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, bl) - l);
+      else x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, -l));
+      return x;
+    };
+    auto slot_probs = [&](int mq, int slot) {  // and the row statistics of the group after the next slot's
+      if ((slot + 1) % SPG == 0 && (slot + 1) / SPG < 4) load_l4(mq, (slot + 1) / SPG);
 #pragma unroll
-    for (int mq = 0; mq < 2; ++mq) {
+      for (int k = 0; k < EPS; k += 2) {
+        const int r = slot * EPS + k;
+        const float p0 = prob(mq, r), p1 = prob(mq, r + 1);
+        pk[mq][r >> 1] = Mma<T>::pack(p0, p1);
+      }
+    };
+    auto mask_scores = [&](int mq) {
+      const int q0 = item_q0(it);
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int qi = q0 + mq * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
+        if ((p.causal && key > qi) || key >= S) sc[mq][r] = -INFINITY;
+      }
+    };
+    auto hand_over = [&](int mq) {
       *(u32x4*)(px + (2 * mq) * 256) = u32x4{pk[mq][0], pk[mq][1], pk[mq][2], pk[mq][3]};
       *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{pk[mq][4], pk[mq][5], pk[mq][6], pk[mq][7]};
+    };
+#pragma unroll
+    for (int i = 0; i < AHEAD; ++i) ring[i] = read_rows(qt, i);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase 1
+#pragma unroll
+    for (int i = 0; i < KS; ++i) {
+      ring[(i + AHEAD) & 7] = read_rows(qt, i + AHEAD);
+      sc[0] = Mma<T>::run(ring[i & 7], frag[i], i == 0 ? zero16 : sc[0]);
+      if (i == KS - 1) load_l4(0, 0);
+      __builtin_amdgcn_sched_barrier(0);
     }
-    accumulate(do_t + tb * TILE, pk);
+    if constexpr (MASK == 2) bias_to_log2(braw);
+    if (__builtin_expect(edge, 0)) mask_scores(0);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase 2
+#pragma unroll
+    for (int i = KS; i < 2 * KS; ++i) {
+      const int n = i + AHEAD;  // the operand after next: rows of Q, then columns of dO
+      ring[n & 7] = n < 2 * KS ? read_rows(qt, n) : read_cols(dot, n - 2 * KS);
+      sc[1] = Mma<T>::run(ring[i & 7], frag[i - KS], i == KS ? zero16 : sc[1]);
+      slot_probs(0, i - KS);
+      if (i == 2 * KS - 1) load_l4(1, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    hand_over(0);
+    if (__builtin_expect(edge, 0)) mask_scores(1);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phases 3 and 4: operand j = DB * (16-row step) + d block of dO^T
+#pragma unroll
+    for (int j = 0; j < 4 * DB; ++j) {
+      if (j + AHEAD < 4 * DB) ring[(j + AHEAD) & 7] = read_cols(dot, j + AHEAD);
+      const int ks4 = j / DB, db = j % DB, mq = ks4 >> 1, r0 = (ks4 & 1) * 4;
+      const u32x4 bb = {pk[mq][r0], pk[mq][r0 + 1], pk[mq][r0 + 2], pk[mq][r0 + 3]};
+      acc[db] = Mma<T>::run(ring[j & 7], bb, acc[db]);
+      if (j < 2 * DB) slot_probs(1, j);
+      if (j == 2 * DB - 1) hand_over(1);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto role_a = [&](int it, int tb, int pb) {
+    const int q0 = item_q0(it);
+    if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;  // every key of this block lies above the diagonal / past the keys
+    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S);
+    role_a_tile(it, tb, pb, edge);
   };
   // Role B splits a tile over two iterations, so that its vector work falls on role A's first
   // matrix ops and its matrix ops on role A's vector work: dP of tile it at the end of iteration
@@ -299,28 +365,57 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     if ((p.causal && item_q0(it) + BQ - 1 < kw0) || kw0 >= S) return;
     scores(do_t + tb * TILE, dp);
   };
+  // One tile of role B, pipelined like role A's:
+  //   phase 0  dS of rows 0-31
+  //   phase 1  dK from rows 0-31           | dS of rows 32-63
+  //   phase 2  dK from rows 32-63
   auto role_b = [&](int it, int tb, int pb) {
+    constexpr int EPS = 16 / KS;  // elements per slot (2 or 4)
+    constexpr int SPG = 4 / EPS;  // slots per group of four consecutive rows
     const int q0 = item_q0(it);
     if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
     const uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;
+    const uint16_t* qt = q_t + tb * TILE;
+    const float* drow = &dl_s[tb * BQ + half * 4];
     uint32_t pk[2][8];
+    u32x4 w[2][2];  // P of this lane's key in the tile's 64 rows, packed as role A fed it to the matrix pipe
+    f32x4 d4[2][4];
+    u32x4 ring[8];
+    auto load_d4 = [&](int mq, int r4) { d4[mq][r4] = *(const f32x4*)(drow + mq * 32 + r4 * 8); };
+    auto ds_pair = [&](int mq, int r) {  // elements r, r + 1
+      const uint32_t word = w[mq][r >> 3][(r >> 1) & 3];
+      const float s0 = Mma<T>::unpack(word, 0) * (dp[mq][r] - d4[mq][r >> 2][r & 3]);
+      const float s1 = Mma<T>::unpack(word, 1) * (dp[mq][r + 1] - d4[mq][(r + 1) >> 2][(r + 1) & 3]);
+      pk[mq][r >> 1] = Mma<T>::pack(s0, s1);
+    };
+    w[0][0] = *(const u32x4*)(px), w[0][1] = *(const u32x4*)(px + 256);
+    load_d4(0, 0);
 #pragma unroll
-    for (int mq = 0; mq < 2; ++mq) {
-      const u32x4 w0 = *(const u32x4*)(px + (2 * mq) * 256), w1 = *(const u32x4*)(px + (2 * mq + 1) * 256);
-      const uint32_t w[8] = {w0[0], w0[1], w0[2], w0[3], w1[0], w1[1], w1[2], w1[3]};
+    for (int i = 0; i < AHEAD; ++i) ring[i] = read_cols(qt, i);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phase 0
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const f32x4 d4 = *(const f32x4*)(&dl_s[tb * BQ + mq * 32 + r4 * 8 + half * 4]);
-        float ds[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const float pr = Mma<T>::unpack(w[r4 * 2 + (e >> 1)], e & 1);
-          ds[e] = pr * (dp[mq][r4 * 4 + e] - d4[e]);
-        }
-        pk[mq][r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pk[mq][r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
-      }
+    for (int r4 = 0; r4 < 4; ++r4) {
+      if (r4 + 1 < 4) load_d4(0, r4 + 1);
+      ds_pair(0, r4 * 4), ds_pair(0, r4 * 4 + 2);
     }
-    accumulate(q_t + tb * TILE, pk);
+    w[1][0] = *(const u32x4*)(px + 512), w[1][1] = *(const u32x4*)(px + 768);
+    load_d4(1, 0);
+    __builtin_amdgcn_sched_barrier(0);
+    // ---- phases 1 and 2: operand j = DB * (16-row step) + d block of Q^T
+#pragma unroll
+    for (int j = 0; j < 4 * DB; ++j) {
+      if (j + AHEAD < 4 * DB) ring[(j + AHEAD) & 7] = read_cols(qt, j + AHEAD);
+      const int ks4 = j / DB, db = j % DB, mq = ks4 >> 1, r0 = (ks4 & 1) * 4;
+      const u32x4 bb = {pk[mq][r0], pk[mq][r0 + 1], pk[mq][r0 + 2], pk[mq][r0 + 3]};
+      acc[db] = Mma<T>::run(ring[j & 7], bb, acc[db]);
+      if (j < 2 * DB) {
+        if ((j + 1) % SPG == 0 && (j + 1) / SPG < 4) load_d4(1, (j + 1) / SPG);
+#pragma unroll
+        for (int k = 0; k < EPS; k += 2) ds_pair(1, j * EPS + k);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
   };
 
   if (n_items > 0) {

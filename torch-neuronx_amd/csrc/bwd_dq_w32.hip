@@ -17,6 +17,8 @@
 // K and V tiles sit in LDS row-major and XOR swizzled (see tile_swz).  Math follows
 // torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows with lse = -inf give zero
 // gradients, scale multiplies dQ once at the end.
+#include <type_traits>
+
 #include "bwd_mfma.h"
 
 namespace mi355 {
@@ -254,22 +256,29 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     const bool edge = t >= t_edge;
     float bl[16];
     if constexpr (MASK) bias_log2(bl);
+    // (the test for a tile that needs masking stays outside the unrolled loop: inside, the compiler
+    // turns it into selects that every element of every tile pays for)
+    auto elements = [&](auto edge_c) {
+      constexpr bool EDGE = decltype(edge_c)::value;
 #pragma unroll
-    for (int r = 0; r < 16; r += 2) {
-      float ds[2];
+      for (int r = 0; r < 16; r += 2) {
+        float ds[2];
 #pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        float pr;
-        if constexpr (MASK) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
-        else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
-        if (edge) {
-          const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
-          pr = kv > lim ? 0.f : pr;
+        for (int e = 0; e < 2; ++e) {
+          float pr;
+          if constexpr (MASK) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
+          else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+          if constexpr (EDGE) {
+            const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
+            pr = kv > lim ? 0.f : pr;
+          }
+          ds[e] = pr * (dpacc[r + e] - dl);
         }
-        ds[e] = pr * (dpacc[r + e] - dl);
+        pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
       }
-      pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
-    }
+    };
+    if (__builtin_expect(edge, 0)) elements(std::true_type{});
+    else elements(std::false_type{});
     if constexpr (MASK) {
       // grad_bias = grad_logits (torch_neuronx/_sdpa_math.py:163,169): the packed pairs are its
       // elements in the input dtype already; four consecutive keys per store

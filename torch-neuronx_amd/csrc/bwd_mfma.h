@@ -54,6 +54,20 @@ __device__ __forceinline__ int tile_swz(int r) {
   return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
 
+// Instruction order of a tile, spelled out for the scheduler: a wavefront issues in order, and
+// left alone the compiler emits a tile's matrix ops in solid runs with all of the vector work
+// between them, which leaves the overlap to the other wavefront of the SIMD alone.  A pipeline
+// is GROUPS groups of 1 matrix op + READS LDS reads + VALU vector instructions, in that order.
+template <int GROUPS, int READS, int VALU>
+__device__ __forceinline__ void pipeline() {
+#pragma unroll
+  for (int g = 0; g < GROUPS; ++g) {
+    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+    if constexpr (READS > 0) __builtin_amdgcn_sched_group_barrier(0x100, READS, 0);
+    if constexpr (VALU > 0) __builtin_amdgcn_sched_group_barrier(0x002, VALU, 0);
+  }
+}
+
 // dK / dV with two wavefronts per SIMD (bwd_dkdv_w32.hip), head dim 64 or 128; `fits` is false
 // when the tensors do not fit its 32-bit addressing and the caller must use bwd_mfma.hip
 bool bwd_dkdv_w32_fits(const BwdM& g, int head_dim);
