@@ -25,7 +25,7 @@ namespace mi355 {
 namespace {
 
 constexpr int BM = 256, BN = 32;
-constexpr int AHEAD = 4;
+constexpr int AHEAD = 2;  // LDS operands are requested this many matrix ops ahead (more spills at head dim 128)
 
 // MASK = 1: per-batch key counts and a bias / bool keep-mask (a lane reads its own row of it); also
 // head dims below D (multiples of 8), the missing tail of every row counting as zeros
@@ -319,12 +319,61 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     if (t < nt_w) {
       // (the masked variant has no registers to spare for a second score tile: it computes the
       // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap)
-      if constexpr (MASK) scores(buf, scur, dpcur);
-      else if (t + 1 < nt_w) scores(bn, snext, dpnext);
-      uint32_t pS[8];
-      softmax(t, scur, dpcur, pS);
-      load_bias(t + 1);
-      accumulate(buf, pS);
+      if constexpr (MASK) {
+        scores(buf, scur, dpcur);
+        uint32_t pS[8];
+        softmax(t, scur, dpcur, pS);
+        load_bias(t + 1);
+        accumulate(buf, pS);
+      } else {
+        // Software pipelined by hand (a wavefront issues in order, and left alone the compiler emits
+        // the matrix ops in solid runs with all of the vector work between them): the scores of tile
+        // t + 1 are one matrix op per slot, and each slot forms one element of dS of tile t; the
+        // operands of dQ follow in the same register ring.  A tile that crosses the causal diagonal
+        // or the end of the keys gets the scores of its masked positions set to -inf first, in a
+        // block of its own (tested per element, the test becomes selects that every tile pays for).
+        // (For a wavefront's last tile the scores of the tile after it are computed and dropped.)
+        if (__builtin_expect(t >= t_edge, 0)) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int kv = t * BN + (r >> 2) * 8 + half * 4 + (r & 3);
+            if (kv > lim) scur[r] = -INFINITY;
+          }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        uint32_t pS[8];
+        u32x4 ring[8];
+        const uint16_t* kt = k_t[buf];
+        auto rd = [&](int i) { return *(const u32x4*)(((i & 1) ? v_t[bn] : k_t[bn]) + row_off[i >> 1]); };
+#pragma unroll
+        for (int i = 0; i < AHEAD; ++i) ring[i] = rd(i);
+        __builtin_amdgcn_sched_barrier(0);
+        float ds_even = 0.f;
+#pragma unroll
+        for (int i = 0; i < 2 * KS; ++i) {
+          const int n = i + AHEAD;
+          ring[n & 7] = n < 2 * KS ? rd(n) : read_cols(kt, n - 2 * KS);
+          if (i & 1) dpnext = Mma<T>::run(ring[i & 7], dof[i >> 1], i == 1 ? zero16 : dpnext);
+          else snext = Mma<T>::run(ring[i & 7], qf[i >> 1], i == 0 ? zero16 : snext);
+          // elements of dS: 16 over the 2 * KS slots
+#pragma unroll
+          for (int r = i * 16 / (2 * KS); r < (i + 1) * 16 / (2 * KS); ++r) {
+            const float pr = __builtin_amdgcn_exp2f(fmaf(scur[r], c, -lse2));
+            const float d = pr * (dpcur[r] - dl);
+            if (r & 1) pS[r >> 1] = Mma<T>::pack(ds_even, d);
+            else ds_even = d;
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int j = 0; j < 2 * DB; ++j) {
+          if (j + AHEAD < 2 * DB) ring[(j + AHEAD) & 7] = read_cols(kt, j + AHEAD);
+          const int r0 = (j / DB) * 4;
+          const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
+          dqacc[j % DB] = Mma<T>::run(ring[j & 7], bS, dqacc[j % DB]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+      }
     }
     store_tile(bnn);  // tile t + 2 (buffer of tile t - 1, whose last readers passed the previous barrier)
     __syncthreads();
