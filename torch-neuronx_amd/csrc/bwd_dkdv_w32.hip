@@ -79,6 +79,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       if (!MASK || half * 8 + ks * 16 < dr) frag[ks] = *(const u32x4*)(r + half * 8 + ks * 16);
       else frag[ks] = u32x4{0u, 0u, 0u, 0u};
     }
+    // (the fragments are awaited here, once: left pending, their first use inside the tile loop
+    // becomes a wait for every outstanding load there, the tile loads of the next items included)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(frag[ks]));
   }
 
   const int nqs = (p.L + BQ - 1) / BQ;
@@ -94,50 +98,70 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // or as another head's rows, and are switched off through lse = +inf.
   const int64_t q_ext = ((int64_t)(p.Hq - 1) * p.q_sh + (int64_t)(p.L - 1) * p.q_sl + dr) * 2;
   const int64_t go_ext = ((int64_t)(p.Hq - 1) * p.go_sh + (int64_t)(p.L - 1) * p.go_sl + dr) * 2;
-  const __amdgpu_buffer_rsrc_t q_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.q + b * p.q_sb), 0, (int)q_ext, 0x00020000);
-  const __amdgpu_buffer_rsrc_t go_rsrc =
-      __builtin_amdgcn_make_buffer_rsrc((void*)((const uint16_t*)p.go + b * p.go_sb), 0, (int)go_ext, 0x00020000);
-  const int s_row = tid / CH, s_ch = tid % CH;  // rows s_row + n * 512 / CH
+  auto descriptor = [&](const void* base, int64_t bytes) {  // raw buffer resource, in scalar registers
+    const uint64_t a = (uint64_t)base;
+    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+  };
+  const u32x4 q_rsrc = descriptor((const uint16_t*)p.q + b * p.q_sb, q_ext);
+  const u32x4 go_rsrc = descriptor((const uint16_t*)p.go + b * p.go_sb, go_ext);
+  // row statistics of this batch (written by bwd_delta_kernel): (Hq, L) floats each
+  const u32x4 lse_rsrc = descriptor(p.lse2 + (int64_t)b * p.Hq * p.L, (int64_t)p.Hq * p.L * 4);
+  const u32x4 dl_rsrc = descriptor(p.delta + (int64_t)b * p.Hq * p.L, (int64_t)p.Hq * p.L * 4);
+  // The tiles go from global memory straight into LDS (buffer loads with the LDS bit: no trip
+  // through registers, no LDS store instructions).  The loads are written as inline assembly: the
+  // compiler's own form of them makes it wait for all outstanding loads before the next LDS read
+  // of any address, which would expose the whole memory latency at the top of every iteration.
+  // Their completion is awaited by hand, before the barrier that publishes the tile (wait_tiles).  Such a load writes 64 x 16 contiguous bytes, one
+  // chunk per lane in lane order, at an LDS address that is uniform for the wavefront: 1 KB = 1024 / (2 D)
+  // whole tile rows.  The swizzle is therefore applied on the global side: the lane that owns LDS
+  // chunk position c of row r fetches the row's chunk c ^ tile_swz(r).
+  const int s_row = tid / CH;                       // rows s_row + n * 512 / CH
+  const int s_ch = (tid % CH) ^ tile_swz<D>(s_row);  // (row s_row + 32 has the swizzle of row s_row)
   uint32_t q_off[NCH], go_off[NCH];
 #pragma unroll
   for (int n = 0; n < NCH; ++n) {
     q_off[n] = (uint32_t)(((s_row + (512 / CH) * n) * p.q_sl + s_ch * 8) * 2);
     go_off[n] = (uint32_t)(((s_row + (512 / CH) * n) * p.go_sl + s_ch * 8) * 2);
+    if (MASK && s_ch * 8 >= dr) q_off[n] = go_off[n] = 0x7ffffff0u;  // past the end of a narrow row: reads as zeros
   }
-  u32x4 sq[NCH], sgo[NCH];
-  const bool fetch = !MASK || s_ch * 8 < dr;  // chunks past the end of a narrow row stay zero
-#pragma unroll
-  for (int n = 0; n < NCH; ++n) sq[n] = sgo[n] = u32x4{0u, 0u, 0u, 0u};
-  float lse_r = 0.f, dl_r = 0.f;
-  auto load_item = [&](int it) {
+  typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
+  // LDS byte addresses of this wavefront's 1 KB inside a pass of 512 chunks, for tile buffer 0
+  const uint32_t lds_q = (uint32_t)(uintptr_t)(lds_bytes)q_t + wave * 1024;
+  const uint32_t lds_do = (uint32_t)(uintptr_t)(lds_bytes)do_t + wave * 1024;
+  auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
+    // (m0 holds the LDS address of such a load; nothing else in this kernel uses it)
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+  };
+  const uint32_t lds_lse = (uint32_t)(uintptr_t)(lds_bytes)lse_s, lds_dl = (uint32_t)(uintptr_t)(lds_bytes)dl_s;
+  auto row_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+  };
+  auto wait_tiles = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+  auto load_item = [&](int it, int buf) {  // the tiles of item `it` into tile buffer `buf`
     const int h = item_head(it), q0 = item_q0(it);
     const uint32_t qb = (uint32_t)((h * p.q_sh + (int64_t)q0 * p.q_sl) * 2);
     const uint32_t gb = (uint32_t)((h * p.go_sh + (int64_t)q0 * p.go_sl) * 2);
 #pragma unroll
     for (int n = 0; n < NCH; ++n) {
-      if (fetch) {
-        sq[n] = __builtin_amdgcn_raw_buffer_load_b128(q_rsrc, q_off[n] + qb, 0, 0);
-        sgo[n] = __builtin_amdgcn_raw_buffer_load_b128(go_rsrc, go_off[n] + gb, 0, 0);
-      }
+      tile_load(q_rsrc, q_off[n] + qb, lds_q + (uint32_t)(buf * TILE * 2 + n * 8192));
+      tile_load(go_rsrc, go_off[n] + gb, lds_do + (uint32_t)(buf * TILE * 2 + n * 8192));
     }
-    if (tid < BQ) {
-      const int qi = q0 + tid;
-      const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + min(qi, p.L - 1);
-      const float l = p.lse[idx];
-      // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
-      lse_r = (qi < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
-      dl_r = qi < p.L ? p.delta[idx] : 0.f;
+    if (wave == 0) {  // the 64 rows' statistics: one dword per lane, straight into LDS as well
+      const uint32_t off = (uint32_t)((h * p.L + q0 + lane) * 4);
+      row_load(lse_rsrc, off, lds_lse + (uint32_t)(buf * BQ * 4));
+      row_load(dl_rsrc, off, lds_dl + (uint32_t)(buf * BQ * 4));
     }
   };
-  auto store_item = [&](int buf) {
-#pragma unroll
-    for (int n = 0; n < NCH; ++n) {
-      // (row s_row + 32 has the swizzle of row s_row)
-      *(u32x4*)(&q_t[buf * TILE + (s_row + (512 / CH) * n) * D + ((s_ch ^ tile_swz<D>(s_row)) << 3)]) = sq[n];
-      *(u32x4*)(&do_t[buf * TILE + (s_row + (512 / CH) * n) * D + ((s_ch ^ tile_swz<D>(s_row)) << 3)]) = sgo[n];
-    }
-    if (tid < BQ) lse_s[buf * BQ + tid] = lse_r, dl_s[buf * BQ + tid] = dl_r;
+  // Rows past L of a head's last tile hold another head's rows and statistics (or zeros): they are
+  // switched off through lse = +inf and delta = 0, written over what the loads brought once those
+  // have landed (wait_tiles first).
+  auto finish_item = [&](int it, int buf) {
+    const int q0 = item_q0(it);
+    if (q0 + BQ > p.L && tid < BQ && q0 + tid >= p.L) lse_s[buf * BQ + tid] = INFINITY, dl_s[buf * BQ + tid] = 0.f;
   };
 
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
@@ -419,10 +443,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
 
   if (n_items > 0) {
-    load_item(0);
-    store_item(0);
+    load_item(0, 0);
+    wait_tiles();
+    finish_item(0, 0);
     __syncthreads();
-    if (n_items > 1) load_item(1);
+    if (n_items > 1) load_item(1, 1);
   }
   // iteration `it`: role A works on tile it, role B on tile it - 1; tile it + 1 goes to LDS
   // (one loop per role, with the same barriers: in a shared loop the registers that one role
@@ -430,9 +455,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   int tb_a = 0, tb_b = 2;  // tile buffers of tiles it and it - 1: it % 3 and (it - 1) % 3
   auto stage_and_sync = [&](int it) {
     const int tb_n = tb_a == 2 ? 0 : tb_a + 1;
-    if (it + 1 < n_items) store_item(tb_n);
+    wait_tiles();
+    if (it + 1 < n_items) finish_item(it + 1, tb_n);
     __syncthreads();
-    if (it + 2 < n_items) load_item(it + 2);
+    // (the buffer of tile it - 1: its last reader, role B, passed the barrier above)
+    if (it + 2 < n_items) load_item(it + 2, tb_b);
     tb_b = tb_a, tb_a = tb_n;
   };
   if (role == 0) {

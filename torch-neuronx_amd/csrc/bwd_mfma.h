@@ -9,7 +9,8 @@ struct BwdM {
   const void *go, *q, *k, *v, *out;
   const float* lse;
   void *gq, *gk, *gv;
-  float* delta;
+  float* delta;  // workspace: rowsum(dO * O) per query row (B, Hq, L)
+  float* lse2;   // workspace: the log-sum-exp in the log2 domain, +inf for rows without a live key
   int64_t go_sb, go_sh, go_sl, q_sb, q_sh, q_sl, k_sb, k_sh, k_sl, v_sb, v_sh, v_sl;
   int64_t o_sb, o_sh, o_sl, gq_sb, gq_sh, gq_sl, gk_sb, gk_sh, gk_sl, gv_sb, gv_sh, gv_sl;
   int B, Hq, Hkv, L, S;

@@ -50,7 +50,12 @@ __global__ __launch_bounds__(256) void bwd_delta_kernel(BwdM p) {
   }
 #pragma unroll
   for (int off = LPR / 2; off > 0; off >>= 1) s += __shfl_xor(s, off, 64);
-  if (row < rows && sub == 0) p.delta[row] = s;
+  if (row < rows && sub == 0) {
+    p.delta[row] = s;
+    // (+inf turns exp2(x - lse) into 0 for rows without a live key)
+    const float l = p.lse[row];
+    p.lse2[row] = l != -INFINITY ? l * kLog2eF : INFINITY;
+  }
 }
 
 // ================================================================================================
@@ -506,6 +511,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.go = p.grad_out.data, g.q = p.q.data, g.k = p.k.data, g.v = p.v.data, g.out = p.out.data;
   g.lse = p.lse, g.gq = p.grad_q.data, g.gk = p.grad_k.data, g.gv = p.grad_v.data;
   g.delta = (float*)p.workspace;
+  g.lse2 = g.delta + p.q.size[0] * p.q.size[1] * p.q.size[2];
 #define SET3(dst, src) g.dst##_sb = p.src.stride[0], g.dst##_sh = p.src.stride[1], g.dst##_sl = p.src.stride[2]
   SET3(go, grad_out);
   SET3(q, q);
@@ -587,7 +593,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
 }
 
 size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p) {
-  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * sizeof(float);
+  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float);  // delta and lse2
 }
 
 int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
