@@ -25,7 +25,7 @@ namespace mi355 {
 namespace {
 
 constexpr int BM = 256, BN = 32;
-constexpr int AHEAD = 2;  // LDS operands are requested this many matrix ops ahead (more spills at head dim 128)
+constexpr int AHEAD = 2;  // LDS operands are requested this many matrix ops ahead (3 and 4 measure the same)
 
 // MASK = 1: per-batch key counts and a bias / bool keep-mask (a lane reads its own row of it); also
 // head dims below D (multiples of 8), the missing tail of every row counting as zeros
@@ -36,8 +36,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int TCH = BN * CH;        // 16-byte chunks per tile
   constexpr bool SPLIT = 512 > TCH;   // more threads than chunks: one half stages K, the other V
   static_assert(AHEAD <= 2 * DB, "ring");
-  __shared__ __attribute__((aligned(16))) uint16_t k_t[3][TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t v_t[3][TILE];
+  constexpr int NBUF = 4;  // tile t lives in buffer t % 4
+  __shared__ __attribute__((aligned(16))) uint16_t k_t[NBUF][TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_t[NBUF][TILE];
 
   int b, h, qt;
   {
@@ -78,6 +79,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       if (!MASK || half * 8 + ks * 16 < dr) qf[ks] = *(const u32x4*)(qr + ks * 16), dof[ks] = *(const u32x4*)(gr + ks * 16);
       else qf[ks] = dof[ks] = u32x4{0u, 0u, 0u, 0u};
     }
+    // (the fragments are awaited here, once: left pending, their first use inside the tile loop
+    // becomes a wait for every outstanding load there, the tile loads in flight included)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]), "+v"(dof[ks]));
     const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc;
     const float l = p.lse[idx];
     // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
@@ -122,34 +127,55 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
 
-  // ---- staging: every thread moves one 16-byte chunk of the K tile and one of the V tile ----------
-  // Buffer resources end with the last key row of this (batch, head), and the whole offset travels
-  // in the vector offset, the part the hardware checks against that bound: rows of a ragged last
-  // tile beyond it read as zeros (their probabilities are masked to zero).
+  // ---- staging: K and V tiles go from global memory straight into LDS ---------------------------
+  // (buffer loads with the LDS bit: no trip through registers, no LDS store instructions).  Such a
+  // load writes 64 x 16 contiguous bytes, one chunk per lane in lane order, at an LDS address that is
+  // uniform for the wavefront: 1 KB = 1024 / (2 D) whole tile rows.  The swizzle is therefore
+  // applied on the global side: the lane that owns LDS chunk position c of row r fetches the
+  // row's chunk c ^ tile_swz(r).  The resources end with the last key row of this (batch, head),
+  // and the whole offset travels in the vector offset, the part the hardware checks against that
+  // bound: rows of a ragged last tile beyond it, and chunks past the end of a narrow row, read as
+  // zeros.  The loads are inline assembly (the compiler's own form makes every later LDS read
+  // wait for all outstanding loads); a tile is requested three iterations before its first use and
+  // awaited by hand, with a count that leaves the youngest tile's loads in flight, before the
+  // barrier that publishes it.
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
-  const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + dr) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + dr) * 2);
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
-  const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
-  const int s_row = s_idx / CH, s_ch = s_idx % CH;
-  // (uniform per wavefront, unless the rows are narrower than D: chunks past their end are never
-  // fetched, and the zeros they start with are what goes to LDS)
-  const bool fetch = !MASK || s_ch * 8 < dr;
-  const bool do_k = (!SPLIT || tid < TCH) && fetch, do_v = (!SPLIT || tid >= TCH) && fetch;
-  const bool put_k = !SPLIT || tid < TCH, put_v = !SPLIT || tid >= TCH;
-  const uint32_t k_off = (uint32_t)((s_row * p.k_sl + s_ch * 8) * 2), v_off = (uint32_t)((s_row * p.v_sl + s_ch * 8) * 2);
-  const uint32_t k_tile_bytes = (uint32_t)(BN * p.k_sl * 2), v_tile_bytes = (uint32_t)(BN * p.v_sl * 2);
-  const int s_lds = s_row * D + ((s_ch ^ tile_swz<D>(s_row)) << 3);
-  u32x4 kreg = {0u, 0u, 0u, 0u}, vreg = {0u, 0u, 0u, 0u};
-  auto load_tile = [&](int t) {
-    const uint32_t tt = (uint32_t)min(t, nt - 1);
-    if (do_k) kreg = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off + tt * k_tile_bytes, 0, 0);
-    if (do_v) vreg = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off + tt * v_tile_bytes, 0, 0);
+  const int64_t k_bytes = ((int64_t)(S - 1) * p.k_sl + dr) * 2, v_bytes = ((int64_t)(S - 1) * p.v_sl + dr) * 2;
+  auto descriptor = [&](const void* base, int64_t bytes) {  // raw buffer resource, in scalar registers
+    const uint64_t a = (uint64_t)base;
+    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
   };
-  auto store_tile = [&](int buf) {
-    if (put_k) *(u32x4*)(&k_t[buf][s_lds]) = kreg;
-    if (put_v) *(u32x4*)(&v_t[buf][s_lds]) = vreg;
+  const u32x4 k_rsrc = descriptor(kp, k_bytes), v_rsrc = descriptor(vp, v_bytes);
+  const bool do_k = !SPLIT || wave < TCH / 64, do_v = !SPLIT || wave >= TCH / 64;  // (uniform per wavefront)
+  constexpr int NDMA = SPLIT ? 1 : 2;  // loads per wavefront and tile
+  const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
+  const int s_row = s_idx / CH, s_ch = (s_idx % CH) ^ tile_swz<D>(s_row);
+  uint32_t k_off = (uint32_t)((s_row * p.k_sl + s_ch * 8) * 2), v_off = (uint32_t)((s_row * p.v_sl + s_ch * 8) * 2);
+  if (MASK && s_ch * 8 >= dr) k_off = v_off = 0x7ffffff0u;  // past the end of a narrow row
+  const uint32_t k_tile_bytes = (uint32_t)(BN * p.k_sl * 2), v_tile_bytes = (uint32_t)(BN * p.v_sl * 2);
+  typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
+  // LDS byte address of this wavefront's 1 KB of a tile, for tile buffer 0
+  const uint32_t lds_k = (uint32_t)(uintptr_t)(lds_bytes)&k_t[0][0] + (uint32_t)((SPLIT ? wave % (TCH / 64) : wave) * 1024);
+  const uint32_t lds_v = (uint32_t)(uintptr_t)(lds_bytes)&v_t[0][0] + (uint32_t)((SPLIT ? wave % (TCH / 64) : wave) * 1024);
+  auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
+    // (m0 holds the LDS address of such a load, one wait state after it is written; nothing else in
+    // this kernel uses m0)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+  };
+  auto load_tile = [&](int t) {  // tile t (the last one again past the end) into buffer t % 4
+    const uint32_t tt = (uint32_t)min(t, nt - 1);
+    const uint32_t boff = (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+    if (do_k) tile_load(k_rsrc, k_off + tt * k_tile_bytes, lds_k + boff);
+    if (do_v) tile_load(v_rsrc, v_off + tt * v_tile_bytes, lds_v + boff);
+  };
+  auto wait_all_tiles = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+  auto wait_older_tiles = [&]() {  // all but the tile requested last
+    if constexpr (NDMA == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
   };
 
   // element offsets inside a tile (the swizzle is not additive in the d block / contraction step:
@@ -302,20 +328,22 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     }
   };
 
-  // Iteration t: scores of tile t + 1, vector work of tile t, dQ of tile t; tile t + 2 goes to LDS.
-  // Buffers: tile t in t % 3.
+  // Iteration t: tile t + 3 is requested, scores of tile t + 1, vector work of tile t, dQ of tile t.
+  // Buffers: tile t in t % 4 (the buffer of tile t + 3 is that of tile t - 1, whose last readers
+  // passed the barrier that ended iteration t - 1).
   load_bias(0);
   load_tile(0);
-  store_tile(0);
   load_tile(1);
-  store_tile(1);
+  wait_all_tiles();
   __syncthreads();
   load_tile(2);
   f32x16 s_a, dp_a, s_b, dp_b;
   if (!MASK && nt_w > 0) scores(0, s_a, dp_a);
-  int buf = 0;  // t % 3
   auto iteration = [&](int t, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
-    const int bn = buf == 2 ? 0 : buf + 1, bnn = bn == 2 ? 0 : bn + 1;
+    const int buf = t & (NBUF - 1), bn = (t + 1) & (NBUF - 1);
+    // (the masked variant requests the tile at the end of the iteration instead: its bias loads are
+    // awaited by the compiler with a count that knows nothing of the tile loads, so those had
+    // better be the older ones)
     if (t < nt_w) {
       // (the masked variant has no registers to spare for a second score tile: it computes the
       // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap)
@@ -375,10 +403,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
         }
       }
     }
-    store_tile(bnn);  // tile t + 2 (buffer of tile t - 1, whose last readers passed the previous barrier)
-    __syncthreads();
     load_tile(t + 3);
-    buf = bn;
+    wait_older_tiles();  // tile t + 2, read from the next iteration on
+    __syncthreads();
   };
   int t = 0;
   for (; t + 1 < nt; t += 2) {
