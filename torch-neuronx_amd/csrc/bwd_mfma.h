@@ -44,17 +44,6 @@ __device__ __forceinline__ float bias_value(const void* base, int64_t idx, int k
   return (float)__builtin_bit_cast(_Float16, (uint16_t)w);
 }
 
-// Swizzle of the row-major LDS tiles of the two-wavefronts-per-SIMD kernels.  A tile row is D/8
-// chunks of 16 bytes; chunk c of row r lives at chunk c ^ tile_swz<D>(r).  Both ways of reading a
-// tile are then free of bank conflicts: 16 consecutive rows reading the same chunk (row-major A
-// operand) land in 16 different 16-byte slots of the 256-byte bank window, and 4 consecutive
-// rows reading the same 4 consecutive chunks (one transposing read) land in 4 different 64-byte
-// windows.  (With D = 64 two rows share a bank window, so the row parity does part of the job.)
-template <int D>
-__device__ __forceinline__ int tile_swz(int r) {
-  return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
-}
-
 // Instruction order of a tile, spelled out for the scheduler: a wavefront issues in order, and
 // left alone the compiler emits a tile's matrix ops in solid runs with all of the vector work
 // between them, which leaves the overlap to the other wavefront of the SIMD alone.  A pipeline

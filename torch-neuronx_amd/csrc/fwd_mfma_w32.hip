@@ -58,8 +58,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // (head dim 256 needs more than the 64 KB of LDS a kernel may declare: it takes the launch's
   // dynamic LDS instead, and runs one wavefront per SIMD with the 512-register budget)
   constexpr bool DYN = D > 128;
-  __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : 2 * BN * KROW];
-  __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : 2 * BN * VP];
+  // Unmasked calls at head dim 64 / 128 stage their tiles from global memory straight into LDS
+  // (see the staging section): four unpadded, swizzled buffers per operand, tile t in buffer t % 4.
+  constexpr bool DMA = !MASK && D <= 128;
+  constexpr int NBUF = 4, TILE = BN * D;
+  __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * KROW];
+  __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * VP];
   extern __shared__ __attribute__((aligned(16))) uint16_t dyn_lds[];
   uint16_t (*const k_lds)[BN * KROW] = (uint16_t (*)[BN * KROW])(DYN ? dyn_lds : k_static);
   uint16_t (*const v_lds)[BN * VP] = (uint16_t (*)[BN * VP])(DYN ? dyn_lds + 2 * BN * KROW : v_static);
@@ -104,6 +108,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     for (int ks = 0; ks < KS; ++ks) {
       if (!MASK || half * 8 + ks * 16 < dr) qf[ks] = *(const u32x4*)(qr + ks * 16);
       else qf[ks] = u32x4{0u, 0u, 0u, 0u};
+    }
+    // (awaited here, once: left pending, their first use inside the tile loop would become a wait
+    // for every outstanding load there, the tile loads in flight included)
+    if constexpr (DMA) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
     }
   }
 
@@ -174,6 +184,89 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
         *(u32x4*)(&v_lds[buf][(k_row + i * (NT / CH)) * VP + k_chunk * 8]) = vreg[set][i];
     }
   };
+  // ---- staging, unmasked calls: K and V tiles go from global memory straight into LDS -----------
+  // (buffer loads with the LDS bit: no trip through registers, no LDS store instructions).  Such a
+  // load writes 64 x 16 contiguous bytes, one chunk per lane in lane order, at an LDS address that is
+  // uniform for the wavefront, so the tiles are unpadded and bank conflicts are avoided by a
+  // swizzle applied on the global side: the lane that owns LDS chunk position c of row r fetches
+  // the row's chunk c ^ tile_swz(r).  Rows of a ragged last tile lie beyond the resource's bound
+  // and read as zeros.  The loads are inline assembly (the compiler's own form makes every later
+  // LDS read wait for all outstanding loads) and are awaited by hand.  Tiles travel in pairs,
+  // pair j = K tile j+1 and V tile j, the two that the barrier of iteration j-1 publishes; pair
+  // j is requested right after the barrier of iteration j-4, when the last reads of the buffers
+  // it overwrites are behind every wavefront, so a pair has three iterations to land.
+  constexpr int KL = TCH / 64;             // wavefront loads per tile
+  constexpr bool DSPLIT = KL < WAVES;      // fewer than wavefronts: half of them stage K, half V
+  constexpr int NL = DSPLIT ? 1 : KL / WAVES;  // loads per wavefront and tile
+  constexpr int PL = DSPLIT ? 1 : 2 * NL;      // ... and pair
+  static_assert(!DMA || (DSPLIT ? 2 * KL == WAVES : KL % WAVES == 0), "staging layout");
+  auto descriptor = [&](const void* base, int bytes) {  // raw buffer resource, in scalar registers
+    const uint64_t a = (uint64_t)base;
+    return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+                 (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+                 (uint32_t)__builtin_amdgcn_readfirstlane(bytes), 0x00020000u};
+  };
+  const u32x4 kd_rsrc = descriptor(kp, k_bytes), vd_rsrc = descriptor(vp, v_bytes);
+  const int d_wave = DSPLIT ? wave % KL : wave;  // this wavefront's first 1 KB slice of a tile
+  const bool dma_k = !DSPLIT || wave < KL, dma_v = !DSPLIT || wave >= KL;  // (uniform per wavefront)
+  uint32_t kd_off[NL], vd_off[NL];
+#pragma unroll
+  for (int i = 0; i < NL; ++i) {
+    const int ch = (d_wave + i * WAVES) * 64 + lane, row = ch / CH, gch = (ch % CH) ^ tile_swz<(D <= 128 ? D : 128)>(row);
+    kd_off[i] = (uint32_t)((row * p.k_sl + gch * 8) * 2);
+    vd_off[i] = (uint32_t)((row * p.v_sl + gch * 8) * 2);
+  }
+  typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
+  const uint32_t lds_kd = (uint32_t)(uintptr_t)(lds_bytes)&k_static[0] + (uint32_t)(d_wave * 1024);
+  const uint32_t lds_vd = (uint32_t)(uintptr_t)(lds_bytes)&v_static[0] + (uint32_t)(d_wave * 1024);
+  auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
+    // (m0 holds the LDS address of such a load, one wait state after it is written; nothing else in
+    // this kernel uses m0)
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+  };
+  auto request_k = [&](int t) {  // K tile t (the last one again past the end) into buffer t % 4
+    if constexpr (DMA) {
+      const uint32_t g = (uint32_t)(min(t, nt - 1) * k_tile_bytes), l = lds_kd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+      if (dma_k) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) tile_load(kd_rsrc, kd_off[i] + g, l + i * WAVES * 1024);
+      }
+    }
+  };
+  auto request_v = [&](int t) {
+    if constexpr (DMA) {
+      const uint32_t g = (uint32_t)(min(t, nt - 1) * v_tile_bytes), l = lds_vd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+      if (dma_v) {
+#pragma unroll
+        for (int i = 0; i < NL; ++i) tile_load(vd_rsrc, vd_off[i] + g, l + i * WAVES * 1024);
+      }
+    }
+  };
+  auto request_pair = [&](int j) { request_k(j + 1), request_v(j); };
+  auto wait_all_tiles = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+  auto wait_oldest_pair = [&]() {  // of three in flight
+    static_assert(!DMA || PL == 1 || PL == 2 || PL == 4, "wait count");
+    if constexpr (PL == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else if constexpr (PL == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  };
+  // element offsets of the LDS reads inside a swizzled tile (the swizzle is not additive in the d
+  // block / contraction step: one offset register per combination)
+  int row_off[KS], tr_off[2][DB];  // K row reads; V transposing reads [second read of a pair][d block]
+  if constexpr (DMA) {
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<(D <= 128 ? D : 128)>(col)) << 3);
+#pragma unroll
+    for (int sec = 0; sec < 2; ++sec)
+#pragma unroll
+      for (int db = 0; db < DB; ++db) {
+        const int row = 8 * sec + ((lane >> 5) & 1) * 4 + ((lane & 15) >> 2);
+        const int d = db * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+        tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<(D <= 128 ? D : 128)>(row)) << 3) + (d & 7);
+      }
+  }
+
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
   // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
   // 8 + i / 4, 12 + i / 4: four keys at d = 4 (i / 4) + i % 4 = i.  A lane of the 32x32x16 A
@@ -321,24 +414,33 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 
   // ---- prologue ----------------------------------------------------------------------------------
   load_bias(0);
-  load_k(0, 0);
-  load_v(0, 0);
-  load_k(1, 1);
-  store_k(0, 0);
-  store_v(0, 0);
-  store_k(1, 1);
-  __syncthreads();
-  load_k(0, 2);
-  load_k(1, 3);
-  load_v(1, 1);
-  load_v(0, 2);
+  if constexpr (DMA) {
+    request_k(0);
+    request_pair(0);
+    wait_all_tiles();
+    __syncthreads();
+    request_pair(1);
+    request_pair(2);
+  } else {
+    load_k(0, 0);
+    load_v(0, 0);
+    load_k(1, 1);
+    store_k(0, 0);
+    store_v(0, 0);
+    store_k(1, 1);
+    __syncthreads();
+    load_k(0, 2);
+    load_k(1, 3);
+    load_v(1, 1);
+    load_v(0, 2);
+  }
   f32x16 s_a, s_b;
   uint32_t pk_a[8], pk_b[8];
   float ps_a = 0.f, ps_b = 0.f;
   {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 a = *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
+      const u32x4 a = DMA ? *(const u32x4*)(k_static + row_off[ks]) : *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
       s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
     }
     apply_bias(s_a);
@@ -354,12 +456,14 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   }
   __syncthreads();  // K buffer 0 is rewritten during the first iteration
+  if constexpr (DMA) request_pair(3);
   // LDS operands travel through a four-entry register ring, three matrix ops ahead of their use;
   // the ring runs across iterations (the first three K fragments of a tile are requested at the
   // end of the previous iteration, right after the barrier that publishes the tile)
   u32x4 ring[8];
 #pragma unroll
-  for (int ks = 0; ks < AHEAD; ++ks) ring[ks] = *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
+  for (int ks = 0; ks < AHEAD; ++ks)
+    ring[ks] = DMA ? *(const u32x4*)(k_static + TILE + row_off[ks]) : *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
 
   // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
   // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
@@ -367,16 +471,19 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   //   check     sum of tile t against kTrig; rare slow path
   //   phase B   O^T += V^T(t) P^T(t) on the matrix pipe    |  softmax of the first 16 keys of tile
   //             t+1, LDS stores of tiles t+2 / t+1, fetches of tiles t+4 / t+3
-  auto iteration = [&](int t, auto parity, f32x16& scur, f32x16& snext, uint32_t (&pk)[8], uint32_t (&pkn)[8],
+  auto iteration = [&](int t, auto tile_mod, f32x16& scur, f32x16& snext, uint32_t (&pk)[8], uint32_t (&pkn)[8],
                        float& ps, float& psn) {
-    constexpr int par = decltype(parity)::value;  // t & 1, known at compile time
-    const uint16_t* kt = &k_lds[par ^ 1][col * KROW + half * 8];
-    const uint16_t* kn = &k_lds[par][col * KROW + half * 8];  // tile t+2, stored during this iteration
-    const uint16_t* vt = &v_lds[par][tr_base];
-    auto read_k = [&](int ks) { return *(const u32x4*)(kt + ks * 16); };
+    constexpr int tq = decltype(tile_mod)::value;  // t % 4, known at compile time
+    constexpr int par = tq & 1;
+    // tiles t+1 (K, this iteration's scores), t+2 (K, published by this iteration's barrier), t (V)
+    const uint16_t* kt = DMA ? k_static + ((tq + 1) & 3) * TILE : &k_lds[par ^ 1][col * KROW + half * 8];
+    const uint16_t* kn = DMA ? k_static + ((tq + 2) & 3) * TILE : &k_lds[par][col * KROW + half * 8];
+    const uint16_t* vt = DMA ? v_static + tq * TILE : &v_lds[par][tr_base];
+    auto read_k = [&](int ks) { return DMA ? *(const u32x4*)(kt + row_off[ks]) : *(const u32x4*)(kt + ks * 16); };
+    auto read_kn = [&](int ks) { return DMA ? *(const u32x4*)(kn + row_off[ks]) : *(const u32x4*)(kn + ks * 16); };
     auto read_v = [&](int i) {  // d block i % DB, 16-key step i / DB
-      const u32x2 lo = tr_read(vt + (i / DB) * 16 * VP + (i % DB) * 32);
-      const u32x2 hi = tr_read(vt + ((i / DB) * 16 + 8) * VP + (i % DB) * 32);
+      const u32x2 lo = DMA ? tr_read(vt + tr_off[0][i % DB] + (i / DB) * 16 * D) : tr_read(vt + (i / DB) * 16 * VP + (i % DB) * 32);
+      const u32x2 hi = DMA ? tr_read(vt + tr_off[1][i % DB] + (i / DB) * 16 * D) : tr_read(vt + ((i / DB) * 16 + 8) * VP + (i % DB) * 32);
       return u32x4{lo[0], lo[1], hi[0], hi[1]};
     };
     __builtin_amdgcn_sched_barrier(0);
@@ -435,15 +542,19 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     // last one trailing the loop.
 #pragma unroll
     for (int i = 0; i < NPV; ++i) {  // i = DB * (16-key step) + d block
-      if (i == NPV - 2) __syncthreads();
+      if (i == NPV - 2) {
+        if constexpr (DMA) wait_oldest_pair();
+        __syncthreads();
+      }
       if (i + AHEAD < NPV) ring[(KS + i + AHEAD) & 7] = read_v(i + AHEAD);
       if (i == NPV - 2) {
 #pragma unroll
-        for (int j = 0; j < (AHEAD + 1) / 2; ++j) ring[j] = *(const u32x4*)(kn + j * 16);
+        for (int j = 0; j < (AHEAD + 1) / 2; ++j) ring[j] = read_kn(j);
       }
       if (i == NPV - 1) {
 #pragma unroll
-        for (int j = (AHEAD + 1) / 2; j < AHEAD; ++j) ring[j] = *(const u32x4*)(kn + j * 16);
+        for (int j = (AHEAD + 1) / 2; j < AHEAD; ++j) ring[j] = read_kn(j);
+        if constexpr (DMA) request_pair(t + 4);
       }
       const int ks2 = i / DB, db = i % DB;
       const u32x4 b0 = {pk[ks2 * 4], pk[ks2 * 4 + 1], pk[ks2 * 4 + 2], pk[ks2 * 4 + 3]};
@@ -458,10 +569,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
       for (int hs = (i == 0 ? 0 : max((i * 8) / NPV - 1, 0)); hs < max(((i + 1) * 8) / NPV - 1, 0); ++hs)
         softmax_slot(snext, 0, hs, pkn, psn);
-      if (i == 0) store_k(par, par);  // tile t+2
-      if (i == 1) store_v(par ^ 1, par ^ 1);  // tile t+1
-      if (i == NPV / 2) load_k(par, t + 4);
-      if (i == NPV / 2 + 1) load_v(par ^ 1, t + 3);
+      if constexpr (!DMA) {
+        if (i == 0) store_k(par, par);  // tile t+2
+        if (i == 1) store_v(par ^ 1, par ^ 1);  // tile t+1
+        if (i == NPV / 2) load_k(par, t + 4);
+        if (i == NPV / 2 + 1) load_v(par ^ 1, t + 3);
+      }
       __builtin_amdgcn_sched_barrier(0);
     }
     softmax_slot(snext, 0, 7, pkn, psn);
@@ -469,26 +582,48 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // a wavefront whose rows lie above the causal diagonal of the remaining tiles only feeds LDS
   auto idle_step = [&](int t, auto parity) {
     constexpr int par = decltype(parity)::value;
-    store_k(par, par);
-    store_v(par ^ 1, par ^ 1);
-    load_k(par, t + 4);
-    load_v(par ^ 1, t + 3);
-    __syncthreads();
+    if constexpr (DMA) {
+      wait_oldest_pair();
+      __syncthreads();
+      request_pair(t + 4);
+    } else {
+      store_k(par, par);
+      store_v(par ^ 1, par ^ 1);
+      load_k(par, t + 4);
+      load_v(par ^ 1, t + 3);
+      __syncthreads();
+    }
   };
 
   int t = 0;
-  for (; t + 1 < nt_w; t += 2) {
-    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
-    iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
-  }
-  if (t < nt_w) {  // odd count: t is even here
-    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
-    ++t;
+  if constexpr (DMA) {  // the buffer of a tile is a compile-time constant: four copies of the iteration
+    for (;;) {
+      if (t >= nt_w) break;
+      iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+      if (++t >= nt_w) break;
+      iteration(t, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
+      if (++t >= nt_w) break;
+      iteration(t, std::integral_constant<int, 2>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+      if (++t >= nt_w) break;
+      iteration(t, std::integral_constant<int, 3>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
+      ++t;
+    }
+  } else {
+    for (; t + 1 < nt_w; t += 2) {
+      iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+      iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
+    }
+    if (t < nt_w) {  // odd count: t is even here
+      iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+      ++t;
+    }
   }
   for (; t < nt; ++t) {
     if (t & 1) idle_step(t, std::integral_constant<int, 1>{});
     else idle_step(t, std::integral_constant<int, 0>{});
   }
+  // (no load into LDS may be in flight when the workgroup's LDS is handed to the next one)
+  if constexpr (DMA) wait_all_tiles();
 
   // ---- epilogue ------------------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
