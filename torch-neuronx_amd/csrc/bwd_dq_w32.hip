@@ -339,8 +339,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   load_tile(2);
   f32x16 s_a, dp_a, s_b, dp_b;
   if (!MASK && nt_w > 0) scores(0, s_a, dp_a);
-  auto iteration = [&](int t, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
-    const int buf = t & (NBUF - 1), bn = (t + 1) & (NBUF - 1);
+  auto iteration = [&](int t, auto tile_mod, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
+    // (t % 4 is a compile-time constant, four copies of the iteration: the buffer of a tile then is
+    // an immediate offset of the LDS reads, not an addition on the vector unit per read)
+    constexpr int buf = decltype(tile_mod)::value, bn = (buf + 1) & (NBUF - 1);
     // (the masked variant requests the tile at the end of the iteration instead: its bias loads are
     // awaited by the compiler with a count that knows nothing of the tile loads, so those had
     // better be the older ones)
@@ -411,12 +413,17 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     wait_older_tiles();  // tile t + 2, read from the next iteration on
     __syncthreads();
   };
-  int t = 0;
-  for (; t + 1 < nt; t += 2) {
-    iteration(t, s_a, dp_a, s_b, dp_b);
-    iteration(t + 1, s_b, dp_b, s_a, dp_a);
+  for (int t = 0;;) {
+    if (t >= nt) break;
+    iteration(t, std::integral_constant<int, 0>{}, s_a, dp_a, s_b, dp_b);
+    if (++t >= nt) break;
+    iteration(t, std::integral_constant<int, 1>{}, s_b, dp_b, s_a, dp_a);
+    if (++t >= nt) break;
+    iteration(t, std::integral_constant<int, 2>{}, s_a, dp_a, s_b, dp_b);
+    if (++t >= nt) break;
+    iteration(t, std::integral_constant<int, 3>{}, s_b, dp_b, s_a, dp_a);
+    ++t;
   }
-  if (t < nt) iteration(t, s_a, dp_a, s_b, dp_b);
   zero_gbias(nt_w);
 
   if (qrow < p.L) {
