@@ -60,11 +60,13 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   constexpr bool DYN = D > 128;
   // Unmasked calls at head dim 64 / 128 stage their tiles from global memory straight into LDS
   // (see the staging section): four unpadded, swizzled buffers per operand, tile t in buffer t % 4.
-  constexpr bool DMA = !MASK && D <= 128;
+  constexpr bool DMA = !MASK;
   constexpr int NBUF = 4, TILE = BN * D;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * KROW];
   __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * VP];
   extern __shared__ __attribute__((aligned(16))) uint16_t dyn_lds[];
+  uint16_t* const k_dma = DYN ? dyn_lds : k_static;                // the buffers of the direct staging
+  uint16_t* const v_dma = DYN ? dyn_lds + NBUF * TILE : v_static;
   uint16_t (*const k_lds)[BN * KROW] = (uint16_t (*)[BN * KROW])(DYN ? dyn_lds : k_static);
   uint16_t (*const v_lds)[BN * VP] = (uint16_t (*)[BN * VP])(DYN ? dyn_lds + 2 * BN * KROW : v_static);
 
@@ -212,13 +214,13 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   uint32_t kd_off[NL], vd_off[NL];
 #pragma unroll
   for (int i = 0; i < NL; ++i) {
-    const int ch = (d_wave + i * WAVES) * 64 + lane, row = ch / CH, gch = (ch % CH) ^ tile_swz<(D <= 128 ? D : 128)>(row);
+    const int ch = (d_wave + i * WAVES) * 64 + lane, row = ch / CH, gch = (ch % CH) ^ tile_swz<D>(row);
     kd_off[i] = (uint32_t)((row * p.k_sl + gch * 8) * 2);
     vd_off[i] = (uint32_t)((row * p.v_sl + gch * 8) * 2);
   }
   typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
-  const uint32_t lds_kd = (uint32_t)(uintptr_t)(lds_bytes)&k_static[0] + (uint32_t)(d_wave * 1024);
-  const uint32_t lds_vd = (uint32_t)(uintptr_t)(lds_bytes)&v_static[0] + (uint32_t)(d_wave * 1024);
+  const uint32_t lds_kd = (uint32_t)(uintptr_t)(lds_bytes)k_dma + (uint32_t)(d_wave * 1024);
+  const uint32_t lds_vd = (uint32_t)(uintptr_t)(lds_bytes)v_dma + (uint32_t)(d_wave * 1024);
   auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
     // (m0 holds the LDS address of such a load, one wait state after it is written; nothing else in
     // this kernel uses m0)
@@ -246,24 +248,25 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   auto request_pair = [&](int j) { request_k(j + 1), request_v(j); };
   auto wait_all_tiles = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
   auto wait_oldest_pair = [&]() {  // of three in flight
-    static_assert(!DMA || PL == 1 || PL == 2 || PL == 4, "wait count");
+    static_assert(!DMA || PL == 1 || PL == 2 || PL == 4 || PL == 8, "wait count");
     if constexpr (PL == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
     else if constexpr (PL == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else if constexpr (PL == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   };
   // element offsets of the LDS reads inside a swizzled tile (the swizzle is not additive in the d
   // block / contraction step: one offset register per combination)
   int row_off[KS], tr_off[2][DB];  // K row reads; V transposing reads [second read of a pair][d block]
   if constexpr (DMA) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<(D <= 128 ? D : 128)>(col)) << 3);
+    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
 #pragma unroll
     for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
       for (int db = 0; db < DB; ++db) {
         const int row = 8 * sec + ((lane >> 5) & 1) * 4 + ((lane & 15) >> 2);
         const int d = db * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-        tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<(D <= 128 ? D : 128)>(row)) << 3) + (d & 7);
+        tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
       }
   }
 
@@ -440,7 +443,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 a = DMA ? *(const u32x4*)(k_static + row_off[ks]) : *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
+      const u32x4 a = DMA ? *(const u32x4*)(k_dma + row_off[ks]) : *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
       s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
     }
     apply_bias(s_a);
@@ -463,7 +466,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   u32x4 ring[8];
 #pragma unroll
   for (int ks = 0; ks < AHEAD; ++ks)
-    ring[ks] = DMA ? *(const u32x4*)(k_static + TILE + row_off[ks]) : *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
+    ring[ks] = DMA ? *(const u32x4*)(k_dma + TILE + row_off[ks]) : *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
 
   // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
   // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
@@ -476,9 +479,9 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     constexpr int tq = decltype(tile_mod)::value;  // t % 4, known at compile time
     constexpr int par = tq & 1;
     // tiles t+1 (K, this iteration's scores), t+2 (K, published by this iteration's barrier), t (V)
-    const uint16_t* kt = DMA ? k_static + ((tq + 1) & 3) * TILE : &k_lds[par ^ 1][col * KROW + half * 8];
-    const uint16_t* kn = DMA ? k_static + ((tq + 2) & 3) * TILE : &k_lds[par][col * KROW + half * 8];
-    const uint16_t* vt = DMA ? v_static + tq * TILE : &v_lds[par][tr_base];
+    const uint16_t* kt = DMA ? k_dma + ((tq + 1) & 3) * TILE : &k_lds[par ^ 1][col * KROW + half * 8];
+    const uint16_t* kn = DMA ? k_dma + ((tq + 2) & 3) * TILE : &k_lds[par][col * KROW + half * 8];
+    const uint16_t* vt = DMA ? v_dma + tq * TILE : &v_lds[par][tr_base];
     auto read_k = [&](int ks) { return DMA ? *(const u32x4*)(kt + row_off[ks]) : *(const u32x4*)(kt + ks * 16); };
     auto read_kn = [&](int ks) { return DMA ? *(const u32x4*)(kn + row_off[ks]) : *(const u32x4*)(kn + ks * 16); };
     auto read_v = [&](int i) {  // d block i % DB, 16-key step i / DB
@@ -672,9 +675,10 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     }                                                                                   \
   } while (0)
   if (head_dim == 256) {  // 128-row workgroups only, dynamic LDS
-    constexpr int kBytes = (2 * BN * (256 + 8) + 2 * BN * (256 + 32)) * 2;
+    // (padded double buffers for the masked variant, four plain buffers per operand otherwise)
 #define LAUNCH_256(TT, MM)                                                                                   \
   do {                                                                                                       \
+    constexpr int kBytes = MM ? (2 * BN * (256 + 8) + 2 * BN * (256 + 32)) * 2 : 2 * 4 * BN * 256 * 2;                \
     static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<TT, 256, 4, MM>,          \
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);  \
     if (attr != hipSuccess) {                                                                                \

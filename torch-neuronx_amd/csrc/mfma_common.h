@@ -156,10 +156,11 @@ __device__ __forceinline__ void tr_store(uint16_t* tile, const u32x4 rows[4], in
 // tile are then free of bank conflicts: 16 consecutive rows reading the same chunk (row-major A
 // operand) land in 16 different 16-byte slots of the 256-byte bank window, and 4 consecutive
 // rows reading the same 4 consecutive chunks (one transposing read) land in 4 different 64-byte
-// windows.  (With D = 64 two rows share a bank window, so the row parity does part of the job.)
+// windows.  (With D = 64 two rows share a bank window, so the row parity does part of the job;
+// with D = 256 a row is two windows, and the swizzle stays inside each.)
 template <int D>
 __device__ __forceinline__ int tile_swz(int r) {
-  return D == 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
+  return D >= 128 ? (((r & 3) << 2) | ((r >> 2) & 3)) : ((((r >> 1) & 1) << 2) | ((r >> 2) & 3));
 }
 
 }  // namespace mi355
