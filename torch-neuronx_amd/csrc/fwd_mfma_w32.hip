@@ -37,10 +37,12 @@ constexpr int BN = 32;
 constexpr int AHEAD = 4;  // LDS operands are requested this many matrix ops ahead
 constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescaled
 
-// MASK = 1 adds what a masked call brings: per-batch key counts (kv_lens) and an additive bias or
-// boolean keep-mask, folded into the score tile right after the matrix ops that produce it.  It
-// also serves head dims below D (multiples of 8): the missing tail of every Q / K / V row counts
-// as zeros, which changes neither the scores nor the live part of the output.
+// MASK = 1 adds per-batch key counts (kv_lens) and head dims below D (multiples of 8): the missing
+// tail of every Q / K / V row counts as zeros, which changes neither the scores nor the live part
+// of the output.  MASK = 2 adds an additive bias or boolean keep-mask on top, folded into the
+// score tile right after the matrix ops that produce it; its bias loads are awaited by the
+// compiler, with counts that know nothing of loads written as assembly, so this variant keeps
+// the staging through registers.
 template <typename T, int D, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
@@ -60,7 +62,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   constexpr bool DYN = D > 128;
   // Unmasked calls at head dim 64 / 128 stage their tiles from global memory straight into LDS
   // (see the staging section): four unpadded, swizzled buffers per operand, tile t in buffer t % 4.
-  constexpr bool DMA = !MASK;
+  constexpr bool DMA = MASK != 2;
   constexpr int NBUF = 4, TILE = BN * D;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * KROW];
   __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * VP];
@@ -217,6 +219,10 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     const int ch = (d_wave + i * WAVES) * 64 + lane, row = ch / CH, gch = (ch % CH) ^ tile_swz<D>(row);
     kd_off[i] = (uint32_t)((row * p.k_sl + gch * 8) * 2);
     vd_off[i] = (uint32_t)((row * p.v_sl + gch * 8) * 2);
+    if constexpr (MASK) {  // chunks past the end of a narrow row: an offset beyond any resource reads as zeros
+      if (gch * 8 >= dr) kd_off[i] = 0x7ffffff0u;
+      if (gch * 8 >= drv) vd_off[i] = 0x7ffffff0u;
+    }
   }
   typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
   const uint32_t lds_kd = (uint32_t)(uintptr_t)(lds_bytes)k_dma + (uint32_t)(d_wave * 1024);
@@ -304,7 +310,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // so that everything downstream (reference tracking, lse) is the unbiased code.
   uint32_t braw[16];
   float inv_scale = 0.f;
-  const int bkind = MASK ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   // (the resource is set up unconditionally, with no records when there is no bias: defined on one
   // path only it stops being uniform for the compiler)
   const int b_esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
@@ -315,7 +321,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const uint32_t b_off = (uint32_t)((min(col, max(b_rows - 1, 0)) * p.bias_sl + half * 4) * b_esz);
   if (bkind) inv_scale = 1.f / p.scale;
   auto load_bias = [&](int t) {
-    if constexpr (MASK) {
+    if constexpr (MASK == 2) {
       if (bkind == 1) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -335,7 +341,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   };
   auto apply_bias = [&](f32x16& sv) {
-    if constexpr (MASK) {
+    if constexpr (MASK == 2) {
       if (bkind == 1) {
 #pragma unroll
         for (int r = 0; r < 16; ++r) sv[r] = fmaf(__builtin_bit_cast(float, braw[r]), inv_scale, sv[r]);
@@ -647,12 +653,44 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   }
 }
 
+// one instantiation; head dim 256 needs more than the 64 KB of LDS a kernel may declare
+template <typename T, int D, int WAVES, int MASK>
+int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
+  int bytes = 0;
+  if constexpr (D > 128) {
+    // (padded double buffers with a bias, four plain buffers per operand otherwise)
+    constexpr int kBytes = MASK == 2 ? (2 * BN * (D + 8) + 2 * BN * (D + 32)) * 2 : 2 * 4 * BN * D * 2;
+    static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
+    if (attr != hipSuccess) {
+      set_error("SDPA: cannot reserve %d bytes of LDS for fwd_w32_kernel: %s", kBytes, hipGetErrorString(attr));
+      return MI355_SDPA_ERR_LAUNCH;
+    }
+    bytes = kBytes;
+  }
+  hipLaunchKernelGGL((fwd_w32_kernel<T, D, WAVES, MASK>), grid, dim3(64 * WAVES), bytes, s, g);
+  return MI355_SDPA_OK;
+}
+template <typename T, int D, int WAVES>
+int launch_mask(const FwdM& g, int mask, dim3 grid, hipStream_t s) {
+  if (mask == 2) return launch_one<T, D, WAVES, 2>(g, grid, s);
+  if (mask == 1) return launch_one<T, D, WAVES, 1>(g, grid, s);
+  return launch_one<T, D, WAVES, 0>(g, grid, s);
+}
+template <typename T>
+int launch_dims(const FwdM& g, int head_dim, int waves, int mask, dim3 grid, hipStream_t s) {
+  if (head_dim == 256) return launch_mask<T, 256, 4>(g, mask, grid, s);  // 128-row workgroups only
+  if (head_dim == 128) return waves == 8 ? launch_mask<T, 128, 8>(g, mask, grid, s) : launch_mask<T, 128, 4>(g, mask, grid, s);
+  return waves == 8 ? launch_mask<T, 64, 8>(g, mask, grid, s) : launch_mask<T, 64, 4>(g, mask, grid, s);
+}
+
 }  // namespace
 
 int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipStream_t s) {
   FwdM g = g0;
   if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
   if (g.dv_real <= 0 || g.dv_real > head_dim) g.dv_real = g.d_real;
+  if (head_dim == 256) waves = 4;
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
@@ -660,40 +698,12 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     set_error("SDPA: too many query tiles (%lld)", (long long)blocks);
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  dim3 grid((unsigned)blocks), block(64 * waves);
-  const bool masked = g.bias_kind != 0 || g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim;
-  const bool bf = dtype == MI355_SDPA_BF16;
-#define LAUNCH(TT, DD, WW, MM) hipLaunchKernelGGL((fwd_w32_kernel<TT, DD, WW, MM>), grid, block, 0, s, g)
-#define LAUNCH_D(DD)                                                                    \
-  do {                                                                                  \
-    if (waves == 8) {                                                                   \
-      if (masked) { if (bf) LAUNCH(bf16_t, DD, 8, 1); else LAUNCH(f16_t, DD, 8, 1); }   \
-      else { if (bf) LAUNCH(bf16_t, DD, 8, 0); else LAUNCH(f16_t, DD, 8, 0); }          \
-    } else {                                                                            \
-      if (masked) { if (bf) LAUNCH(bf16_t, DD, 4, 1); else LAUNCH(f16_t, DD, 4, 1); }   \
-      else { if (bf) LAUNCH(bf16_t, DD, 4, 0); else LAUNCH(f16_t, DD, 4, 0); }          \
-    }                                                                                   \
-  } while (0)
-  if (head_dim == 256) {  // 128-row workgroups only, dynamic LDS
-    // (padded double buffers for the masked variant, four plain buffers per operand otherwise)
-#define LAUNCH_256(TT, MM)                                                                                   \
-  do {                                                                                                       \
-    constexpr int kBytes = MM ? (2 * BN * (256 + 8) + 2 * BN * (256 + 32)) * 2 : 2 * 4 * BN * 256 * 2;                \
-    static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<TT, 256, 4, MM>,          \
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);  \
-    if (attr != hipSuccess) {                                                                                \
-      set_error("SDPA: cannot reserve %d bytes of LDS for fwd_w32_kernel: %s", kBytes, hipGetErrorString(attr)); \
-      return MI355_SDPA_ERR_LAUNCH;                                                                          \
-    }                                                                                                        \
-    hipLaunchKernelGGL((fwd_w32_kernel<TT, 256, 4, MM>), grid, block, kBytes, s, g);                         \
-  } while (0)
-    if (masked) { if (bf) LAUNCH_256(bf16_t, 1); else LAUNCH_256(f16_t, 1); }
-    else { if (bf) LAUNCH_256(bf16_t, 0); else LAUNCH_256(f16_t, 0); }
-#undef LAUNCH_256
-  } else if (head_dim == 128) LAUNCH_D(128);
-  else LAUNCH_D(64);
-#undef LAUNCH_D
-#undef LAUNCH
+  const dim3 grid((unsigned)blocks);
+  // kernel variant: 2 with a bias or keep-mask, 1 with key counts or rows narrower than the kernel's head dim
+  const int mask = g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim) ? 1 : 0;
+  const int rc = dtype == MI355_SDPA_BF16 ? launch_dims<bf16_t>(g, head_dim, waves, mask, grid, s)
+                                          : launch_dims<f16_t>(g, head_dim, waves, mask, grid, s);
+  if (rc != MI355_SDPA_OK) return rc;
   return check_launch("fwd_w32_kernel");
 }
 
