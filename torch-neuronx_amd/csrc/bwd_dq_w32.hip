@@ -27,8 +27,9 @@ namespace {
 constexpr int BM = 256, BN = 32;
 constexpr int AHEAD = 2;  // LDS operands are requested this many matrix ops ahead (3 and 4 measure the same)
 
-// MASK = 1: per-batch key counts and a bias / bool keep-mask (a lane reads its own row of it); also
-// head dims below D (multiples of 8), the missing tail of every row counting as zeros
+// MASK = 1: per-batch key counts, and head dims below D (multiples of 8), the missing tail of every
+// row counting as zeros.  MASK = 2: on top, a bias / bool keep-mask (a lane reads its own row of
+// it) and the gradient of the bias.
 template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -91,12 +92,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   }
 
   uint16_t* gb_row = nullptr;  // this lane's row of the bias gradient, at its first key of a tile
-  if constexpr (MASK) {
+  if constexpr (MASK == 2) {
     if (p.gbias && qrow < p.L)
       gb_row = (uint16_t*)p.gbias + b * p.gbias_sb + h * p.gbias_sh + (int64_t)qrow * p.gbias_sl + half * 4;
   }
   auto zero_gbias = [&](int t_from) {  // tiles this wavefront does not visit
-    if constexpr (MASK) {
+    if constexpr (MASK == 2) {
       if (gb_row) {
         for (int t = t_from; t * BN < p.S; ++t)
 #pragma unroll
@@ -233,16 +234,16 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // fetched one tile ahead as 4 groups of 4 consecutive keys; keys past the row read the next row
   // or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
-  const int bkind = MASK ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
   const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   // (set up unconditionally, with no records when there is no bias: a resource that is defined on
   // one path only stops being uniform for the compiler)
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
       __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
-  const uint32_t b_row = MASK ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
+  const uint32_t b_row = MASK == 2 ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
   auto load_bias = [&](int t) {
-    if constexpr (MASK) {
+    if constexpr (MASK == 2) {
       const uint32_t off = b_row + (uint32_t)(t * BN * besz);
       if (bkind == 1) {
 #pragma unroll
@@ -281,7 +282,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   auto softmax = [&](int t, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
     const bool edge = t >= t_edge;
     float bl[16];
-    if constexpr (MASK) bias_log2(bl);
+    if constexpr (MASK == 2) bias_log2(bl);
     // (the test for a tile that needs masking stays outside the unrolled loop: inside, the compiler
     // turns it into selects that every element of every tile pays for)
     auto elements = [&](auto edge_c) {
@@ -292,7 +293,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           float pr;
-          if constexpr (MASK) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
+          if constexpr (MASK == 2) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
           else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
           if constexpr (EDGE) {
             const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
@@ -305,7 +306,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     };
     if (__builtin_expect(edge, 0)) elements(std::true_type{});
     else elements(std::false_type{});
-    if constexpr (MASK) {
+    if constexpr (MASK == 2) {
       // grad_bias = grad_logits (torch_neuronx/_sdpa_math.py:163,169): the packed pairs are its
       // elements in the input dtype already; four consecutive keys per store
       if (gb_row) {
@@ -338,18 +339,18 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   __syncthreads();
   load_tile(2);
   f32x16 s_a, dp_a, s_b, dp_b;
-  if (!MASK && nt_w > 0) scores(0, s_a, dp_a);
+  if (MASK != 2 && nt_w > 0) scores(0, s_a, dp_a);
   auto iteration = [&](int t, auto tile_mod, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
     // (t % 4 is a compile-time constant, four copies of the iteration: the buffer of a tile then is
     // an immediate offset of the LDS reads, not an addition on the vector unit per read)
     constexpr int buf = decltype(tile_mod)::value, bn = (buf + 1) & (NBUF - 1);
-    // (the masked variant requests the tile at the end of the iteration instead: its bias loads are
-    // awaited by the compiler with a count that knows nothing of the tile loads, so those had
-    // better be the older ones)
+    // (the tile is requested at the end of the iteration: the bias loads of the variant that has
+    // them are awaited by the compiler with a count that knows nothing of the tile loads, so those
+    // had better be the older ones)
     if (t < nt_w) {
-      // (the masked variant has no registers to spare for a second score tile: it computes the
+      // (the variant with a bias has no registers to spare for a second score tile: it computes the
       // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap)
-      if constexpr (MASK) {
+      if constexpr (MASK == 2) {
         scores(buf, scur, dpcur);
         uint32_t pS[8];
         softmax(t, scur, dpcur, pS);
@@ -451,16 +452,23 @@ bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
 int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
-  const bool bf = dtype == MI355_SDPA_BF16, masked = g.bias_kind || g.kv_lens || g.gbias || g.d_real != head_dim;
+  const bool bf = dtype == MI355_SDPA_BF16;
+  const int mask = (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim) ? 1 : 0;
 #define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, 0, s, g)
+#define LAUNCH_M(TT, DD)                                                     \
+  do {                                                                       \
+    if (mask == 2) LAUNCH(TT, DD, 2);                                        \
+    else if (mask == 1) LAUNCH(TT, DD, 1);                                   \
+    else LAUNCH(TT, DD, 0);                                                  \
+  } while (0)
 #define LAUNCH_D(DD)                                                         \
   do {                                                                       \
-    if (masked) { if (bf) LAUNCH(bf16_t, DD, 1); else LAUNCH(f16_t, DD, 1); }  \
-    else { if (bf) LAUNCH(bf16_t, DD, 0); else LAUNCH(f16_t, DD, 0); }         \
+    if (bf) LAUNCH_M(bf16_t, DD); else LAUNCH_M(f16_t, DD);                  \
   } while (0)
   if (head_dim == 128) LAUNCH_D(128);
   else LAUNCH_D(64);
 #undef LAUNCH_D
+#undef LAUNCH_M
 #undef LAUNCH
   return check_launch("bwd_dq_w32_kernel");
 }
