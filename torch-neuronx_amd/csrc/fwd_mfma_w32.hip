@@ -1,9 +1,9 @@
-// Flash-attention forward for gfx950, head dim 64 or 128 (narrower rows: see MASK), bf16/f16.
+// Flash-attention forward for gfx950, head dim 64, 128 or 256 (narrower rows: see MASK), bf16/f16.
 //
 // One workgroup = WAVES wavefronts of 32 query rows each, all of one (batch, query head):
 // WAVES = 8 (256 rows, one workgroup per compute unit) for long sequences, WAVES = 4 (128 rows,
 // two workgroups per compute unit) for short or few ones.  Either way a SIMD hosts two
-// wavefronts with 256 registers each.
+// wavefronts with 256 registers each (head dim 256: one wavefront with 512).
 //
 // Why two wavefronts per SIMD: a wavefront issues at most one instruction every four cycles,
 // whatever the instruction.  A 32x32x16 matrix op keeps the matrix pipe busy for 32 cycles, the
@@ -20,7 +20,8 @@
 // Inside a wavefront the key loop is software pipelined by hand, because a wavefront issues in
 // order: the softmax of a 32-key tile is split in two halves that ride on the matrix ops of two
 // different phases, and LDS operands are fetched AHEAD matrix ops ahead through a register
-// ring.  The loop carries no row maximum: see kTrig.
+// ring.  The loop carries no row maximum: see kTrig.  K and V tiles go from global memory
+// straight into LDS, three tiles ahead of their use (with a bias: through registers, two ahead).
 // Products are computed transposed (S^T = K Q^T, O^T = V^T P^T) as in fwd_mfma.hip, so the
 // softmax statistics are per-lane scalars and P goes from accumulator to B operand in registers.
 //
