@@ -638,7 +638,36 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // ---- epilogue ------------------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
-  if (qrow < p.L) {
+  if constexpr (DMA) {
+    // A lane holds its query row in 8-byte pieces, 16 bytes apart: stored as they are, one
+    // instruction writes 32 fragments of 16 bytes, and the stores of a workgroup's last tile,
+    // which nothing overlaps, took 3 % of the kernel.  The tile goes through LDS instead (the
+    // tile buffers are free now; 32 rows x D per wavefront, 16-byte chunks XOR-swizzled by row
+    // against bank conflicts) and leaves as whole rows, 16 bytes per lane.
+    __syncthreads();  // every wavefront is done with the K / V tiles
+    uint16_t* ot = wave < WAVES / 2 ? k_dma + wave * 32 * D : v_dma + (wave - WAVES / 2) * 32 * D;
+    constexpr int SW = CH < 16 ? CH - 1 : 15;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 w;
+        w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
+        w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
+        *(u32x2*)(ot + col * D + (((db * 4 + g) ^ (col & SW)) << 3) + half * 4) = w;
+      }
+    constexpr int RPI = 64 / CH;  // rows per store instruction
+    const int rr = lane / CH, cc = lane % CH;
+    uint16_t* obase = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + cc * 8;
+#pragma unroll
+    for (int i = 0; i < 32 / RPI; ++i) {
+      const int r = i * RPI + rr;
+      const u32x4 w = *(const u32x4*)(ot + r * D + ((cc ^ (r & SW)) << 3));
+      if (qw0 + r < p.L && (!MASK || cc * 8 < drv)) *(u32x4*)(obase + (int64_t)(qw0 + r) * p.o_sl) = w;
+    }
+    if (qrow < p.L && p.lse && half == 0)
+      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+  } else if (qrow < p.L) {
     uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
