@@ -242,9 +242,9 @@ def known_size_copy(dev, mib=256):
 # `--pmc WRITE_SIZE` runs of this script (--pmc-copy), scaled by the same counters' reading for
 # the known-size copy.  None = not measured for that workload.
 MEASURED_TRAFFIC_BYTES = {
-    "c3_fwd": 214.3e6,      # fwd_w32_kernel: 146.1 MB read + 68.2 MB written (algorithmic 168.8 MB)
+    "c3_fwd": 213.8e6,      # fwd_w32_kernel: 145.7 MB read + 68.2 MB written (algorithmic 168.8 MB)
     "c2_fwd": None,
-    "c4_fwd_bwd": 1535.3e6,  # the three backward kernels of one call (algorithmic 337 MB)
+    "c4_fwd_bwd": 1531.1e6,  # the three backward kernels of one call (algorithmic 337 MB)
     "c5_decode": 604.5e6,    # decode_kernel + decode_merge_kernel of one call (algorithmic 590.8 MB)
 }
 
