@@ -302,6 +302,30 @@ def test_kv_lens_equals_key_padding_mask(amd, gpu_device):
     assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
 
 
+@pytest.mark.parametrize("tile", [3, 4])
+@pytest.mark.parametrize("per_head", [False, True])
+def test_mfma_forward_padding_masks_with_holes_and_dead_batches(amd, gpu_device, tile, per_head):
+    # per-key keep-masks (no row stride): the kernel stops at the last kept key of a (batch, head),
+    # skips nothing in front of it, and a row of the mask that keeps no key gives zeros and lse = -inf
+    B, Hq, Hkv, L, S = 4, 4, 2, 200, 328
+    q, k, v = qkv(B, Hq, Hkv, L, S, 128, dtype=torch.bfloat16, seed=77)
+    g = torch.Generator().manual_seed(5)
+    mask = torch.zeros(B, Hq if per_head else 1, 1, S, dtype=torch.bool)
+    mask[0, :, :, :S] = True                      # keeps every key
+    mask[1, :, :, 40:133] = True                  # left and right padding
+    mask[1, :, :, 64:96] = False                  # ... with a whole tile dropped in the middle
+    mask[2] = torch.rand(mask[2].shape, generator=g) > 0.5
+    mask[2, :, :, 300:] = False                   # ragged end inside a tile
+    # batch 3 keeps nothing
+    if per_head: mask[0, 1, :, 7:] = False        # heads of a batch differ
+    out, lse = _run(amd, q, k, v, gpu_device, attn_bias=mask.to(gpu_device), force_kernel=tile)
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
+    assert torch.equal(out[3].cpu().float(), torch.zeros(Hq, L, 128))
+    assert torch.isinf(lse[3]).all() and (lse[3] < 0).all()
+    assert max_abs(out, ro) <= 2e-2
+    assert max_abs(lse[:3], rl[:3]) <= 2e-3
+
+
 def test_scale_zero_and_explicit_scale(amd, gpu_device):
     q, k, v = qkv(1, 2, 2, 40, 40, 64, dtype=torch.bfloat16, seed=8)
     for sc in (0.0, 0.25, 0.5):

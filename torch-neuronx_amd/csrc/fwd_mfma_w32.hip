@@ -90,6 +90,22 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   int S = p.S;
   if constexpr (MASK) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    if constexpr (MASK == 2) {
+      // A keep-mask per key (no row stride: padding masks): the keys behind the last one it keeps are
+      // never visited, as with a key count.  Every wavefront scans the row itself (S bytes, four
+      // per lane and step; rows are whole dwords) and they all arrive at the same count.
+      if (p.bias_kind == 4 && p.bias_sl == 0 && S > 0) {
+        const uint8_t* mrow = (const uint8_t*)p.bias + b * p.bias_sb + h * p.bias_sh;
+        int last = -1;
+        for (int j = lane * 4; j < S; j += 256) {
+          const uint32_t w = *(const uint32_t*)(mrow + j);
+          if (w) last = j + ((31 - __builtin_clz(w)) >> 3);
+        }
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) last = max(last, __shfl_xor(last, off, 64));
+        S = min(S, __builtin_amdgcn_readfirstlane(last) + 1);
+      }
+    }
     if (S == 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87)
       if (qrow < p.L) {
         uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
@@ -347,8 +363,19 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
         for (int r = 0; r < 16; ++r) sv[r] = fmaf(__builtin_bit_cast(float, braw[r]), inv_scale, sv[r]);
       } else if (bkind == 4) {
+        // (a tile that the mask keeps whole - most tiles of a padding or window mask - costs four
+        // compares instead of three instructions per score)
+        const bool whole = braw[0] == 0x01010101u && braw[1] == 0x01010101u && braw[2] == 0x01010101u && braw[3] == 0x01010101u;
+        if (__builtin_amdgcn_ballot_w64(!whole) != 0) {
+          const bool none = (braw[0] | braw[1] | braw[2] | braw[3]) == 0u;  // ... and one that it drops whole, 16 moves
+          if (__builtin_amdgcn_ballot_w64(!none) == 0) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sv[r] = ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? sv[r] : -INFINITY;
+            for (int r = 0; r < 16; ++r) sv[r] = -INFINITY;
+          } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sv[r] = ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? sv[r] : -INFINITY;
+          }
+        }
       } else if (bkind == 2) {
         typedef __attribute__((ext_vector_type(2))) _Float16 h2;
 #pragma unroll
