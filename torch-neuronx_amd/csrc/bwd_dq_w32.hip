@@ -88,7 +88,19 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     const float l = p.lse[idx];
     // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
     lse2 = (qrow < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
-    dl = p.delta[idx];
+    if (p.make_delta) {
+      // delta = rowsum(dO * O) (torch_neuronx/_sdpa_math.py:160-163): dO is in registers already
+      const uint16_t* orow = (const uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qc * p.o_sl + half * 8;
+      float dsum = 0.f;
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks)
+        if (!MASK || half * 8 + ks * 16 < dr) dsum += dot8<T>(dof[ks], *(const u32x4*)(orow + ks * 16));
+      dsum += __shfl_xor(dsum, 32, 64);
+      dl = dsum;
+      if (qrow < p.L && half == 0) p.delta[idx] = dsum, p.lse2[idx] = l != -INFINITY ? l * kLog2eF : INFINITY;
+    } else {
+      dl = p.delta[idx];
+    }
   }
 
   uint16_t* gb_row = nullptr;  // this lane's row of the bias gradient, at its first key of a tile

@@ -33,7 +33,22 @@ struct BwdM {
   // masked variants treat the rest of every Q / K / V / dO / O row as zeros and leave it out of
   // the gradients; 0 means the full width.
   int d_real = 0;
+  // 1: the dQ kernel of bwd_dq_w32.hip computes delta and lse2 itself and writes them to the
+  // workspace for the dK/dV kernel that follows it (bwd_delta_kernel is then not launched)
+  int make_delta = 0;
 };
+
+// dot product of eight packed elements, float32 accumulation
+template <typename T>
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
+  typedef __attribute__((ext_vector_type(8))) T v8;
+  const v8 x = __builtin_bit_cast(v8, a), y = __builtin_bit_cast(v8, b);
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s = fmaf((float)x[i], (float)y[i], s);
+  return s;
+}
+
 
 // bias element as a float (bool: 0 or -inf)
 __device__ __forceinline__ float bias_value(const void* base, int64_t idx, int kind) {

@@ -25,16 +25,6 @@
 namespace mi355 {
 namespace {
 
-template <typename T>
-__device__ __forceinline__ float dot8(u32x4 a, u32x4 b) {
-  typedef __attribute__((ext_vector_type(8))) T v8;
-  const v8 x = __builtin_bit_cast(v8, a), y = __builtin_bit_cast(v8, b);
-  float s = 0.f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) s = fmaf((float)x[i], (float)y[i], s);
-  return s;
-}
-
 template <typename T, int D>
 __global__ __launch_bounds__(256) void bwd_delta_kernel(BwdM p) {
   constexpr int LPR = D / 8, RPB = 256 / LPR;
@@ -483,8 +473,21 @@ template <typename T, int D>
 int launch_td(const BwdM& g, hipStream_t s) {
   const int64_t rows = (int64_t)g.B * g.Hq * g.L;
   constexpr int RPB = 256 / (D / 8);
-  hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, s, g);
-  int rc = check_launch("bwd_delta_kernel");
+  // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
+  const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
+  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
+  int rc;
+  if (dq_w32) {
+    // that kernel holds every row of dO in registers anyway: it goes first and leaves the row
+    // terms (delta, log2-domain LSE) behind for the dK/dV kernel, which saves the pass over dO
+    // and O of bwd_delta_kernel
+    BwdM g2 = g;
+    g2.make_delta = 1;
+    rc = launch_bwd_dq_w32(g2, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
+  } else {
+    hipLaunchKernelGGL((bwd_delta_kernel<T, D>), dim3((unsigned)((rows + RPB - 1) / RPB)), dim3(256), 0, s, g);
+    rc = check_launch("bwd_delta_kernel");
+  }
   if (rc) return rc;
   if (bwd_dkdv_w32_fits(g, D)) {
     rc = launch_bwd_dkdv_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
@@ -492,11 +495,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
     hipLaunchKernelGGL((bwd_dkdv_kernel<T, D>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(256), 0, s, g);
     rc = check_launch("bwd_dkdv_kernel");
   }
-  if (rc) return rc;
-  // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
-  const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  if ((wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D) && bwd_dq_w32_fits(g, D))  // (a masked call has no other kernel)
-    return launch_bwd_dq_w32(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, D, s);
+  if (rc || dq_w32) return rc;
   if (D == 128 && wg256 >= 256) {
     hipLaunchKernelGGL((bwd_dq_kernel<T, D, D == 128 ? 2 : 1>), dim3((unsigned)wg256), dim3(256), 0, s, g);
   } else {
