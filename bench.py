@@ -244,7 +244,7 @@ def known_size_copy(dev, mib=256):
 MEASURED_TRAFFIC_BYTES = {
     "c3_fwd": 213.8e6,      # fwd_w32_kernel: 145.7 MB read + 68.2 MB written (algorithmic 168.8 MB)
     "c2_fwd": None,
-    "c4_fwd_bwd": 1531.1e6,  # the three backward kernels of one call (algorithmic 337 MB)
+    "c4_fwd_bwd": 1471.8e6,  # the two backward kernels of one call (algorithmic 337 MB)
     "c5_decode": 604.5e6,    # decode_kernel + decode_merge_kernel of one call (algorithmic 590.8 MB)
 }
 

@@ -3,6 +3,8 @@
 //
 //   bwd_delta_kernel   delta_i = sum_d dO_id O_id  (float32).  This is the whole row term of
 //                      torch_neuronx/_sdpa_math.py:160-163: its two P-dependent parts cancel.
+//                      (Not launched when the dQ kernel of bwd_dq_w32.hip serves the call: that
+//                      one goes first and leaves the row terms behind itself.)
 //   bwd_dkdv_kernel    one workgroup per 128 keys of a (batch, kv head); loops over the query
 //                      heads of the group (the GQA sum of decompositions.py:2595-2598 happens
 //                      in registers) and over 64-row query tiles:
