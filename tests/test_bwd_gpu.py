@@ -190,6 +190,30 @@ MASKED_BWD_CASES = [
 ]
 
 
+@pytest.mark.parametrize("per_head", [False, True])
+def test_mfma_backward_padding_masks_with_holes_and_dead_batches(amd, gpu_device, per_head):
+    # per-key keep-masks (no row stride) with left and right padding and holes: the keys behind the
+    # last kept one and a batch whose row keeps nothing get zero gradients
+    B, Hq, Hkv, L, S = 4, 4, 2, 200, 392
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, 128, dtype=torch.bfloat16, seed=78, with_do=True)
+    go = go.clamp(-1, 1) * 0.1
+    g = torch.Generator().manual_seed(6)
+    mask = torch.zeros(B, Hq if per_head else 1, 1, S, dtype=torch.bool)
+    mask[0] = True
+    mask[1, :, :, 40:133] = True
+    mask[1, :, :, 64:96] = False
+    mask[2] = torch.rand(mask[2].shape, generator=g) > 0.5
+    mask[2, :, :, 230:] = False  # the last 128-key block and more are dropped whole
+    if per_head: mask[0, 1, :, 7:] = False
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, attn_bias=mask.to(gpu_device))
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, attn_mask=mask)[:5]
+    for a in (dq[3], dk[3], dv[3], dk[2, :, 230:], dv[2, :, 230:]):
+        assert torch.count_nonzero(a.float()).item() == 0
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert bool(torch.isfinite(a.float()).all())
+        assert max_abs(a, r) <= 5e-2 and rel_err(a, r) <= 3e-2
+
+
 @pytest.mark.parametrize("case", MASKED_BWD_CASES)
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_mfma_backward_with_key_masks(amd, gpu_device, case, dtype):
