@@ -135,8 +135,6 @@ def wl_fwd_bwd(amd, dev):
 
 def wl_decode(amd, dev, sets=4):
     """Config 5.  `sets` rotating copies of the cache keep K/V cold in the last-level cache."""
-    from oracle import sdpa_math as om
-
     B, Hq, Hkv, S, D = 64, 32, 8, 8192, 128
     g = torch.Generator(device="cpu").manual_seed(1005)
     q = torch.randn(B, Hq, 1, D, generator=g).to(torch.bfloat16).to(dev)
@@ -167,6 +165,23 @@ def wl_decode(amd, dev, sets=4):
     return step, nbytes, cfg
 
 
+def cpu_model():
+    """Model name of the host CPU the baseline runs on."""
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_threads():
+    """Threads the CPU baseline uses: torch's intra-op pool, which follows OMP_NUM_THREADS (the
+    box's CPU share) rather than the number of cores the machine shows."""
+    return torch.get_num_threads()
+
+
 def cpu_baseline_fwd(B, Hq, Hkv, S, D, seed, heads=2):
     """CPU oracle on a bounded sample: `heads` query heads of the same problem."""
     from oracle import sdpa_math as om
@@ -180,7 +195,7 @@ def cpu_baseline_fwd(B, Hq, Hkv, S, D, seed, heads=2):
     om.sdpa_forward(q, k, v, is_causal=True)
     dt = time.perf_counter() - t0
     flops = 4.0 * B * heads * D * causal_pairs(S, S)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "cpu_model": cpu_model(),
             "kind": "port",
             "sample": f"{heads} of {Hq} query heads of the same workload, full S={S}; "
                       f"algorithmic (unmasked-pair) FLOPs / wall time; {dt:.2f} s"}
@@ -201,7 +216,7 @@ def cpu_baseline_fwd_bwd(B, Hq, Hkv, S, D, seed, heads=32):
     om.sdpa_backward(do, q, k, v, out, lse, is_causal=True)
     dt = time.perf_counter() - t0
     flops = 14.0 * heads * D * causal_pairs(S, S)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(),
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "cpu_model": cpu_model(),
             "kind": "port",
             "sample": f"{heads} of {B * Hq} (batch, query head) pairs of the same workload, full S={S}, "
                       f"forward + backward; algorithmic (unmasked-pair) FLOPs / wall time; {dt:.2f} s"}
@@ -221,7 +236,7 @@ def cpu_baseline_decode(batches=32):
     om.decode_fp8kv(q, kq, vq, ks, vs, lens)
     dt = time.perf_counter() - t0
     nbytes = 2.0 * Hkv * D * int(lens.sum())
-    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": cpu_threads(), "cpu_model": cpu_model(), "kind": "port",
             "sample": f"first {batches} of {B} sequences of the same workload ({int(lens.sum())} live keys); "
                       f"fp8 K/V bytes of the live keys / wall time (dequantisation included); {dt:.2f} s"}
 

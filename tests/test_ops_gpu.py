@@ -134,6 +134,86 @@ def test_zero_size_dims_take_the_math_backend(amd, gpu_device, calls):
     assert torch._fused_sdp_choice(q, kk, kk) == 4
 
 
+def test_zero_size_head_dims_take_the_math_backend(amd, gpu_device, calls):
+    # test_scaled_dot_product_attention.py:1224-1285: D_qk = 0 and D_v = 0 go to the math backend
+    # (SdpBackendSelection.cpp:54-56) and equal the CPU result; gradients keep their inputs' shapes
+    g = torch.Generator().manual_seed(0)
+    for value_dim in (1, 8):
+        for scale in (1.0, None):
+            q = torch.empty((1, 16, 16, 0), device=gpu_device)
+            k = torch.empty((1, 16, 16, 0), device=gpu_device)
+            v = torch.randn((1, 16, 16, value_dim), generator=g).to(gpu_device)
+            assert torch._fused_sdp_choice(q, k, v, scale=scale) == 0
+            out = F.scaled_dot_product_attention(q, k, v, dropout_p=0.0, scale=scale)
+            ref = F.scaled_dot_product_attention(q.cpu(), k.cpu(), v.cpu(), dropout_p=0.0, scale=scale)
+            assert out.shape == (1, 16, 16, value_dim) and out.device.type == "cuda"
+            torch.testing.assert_close(out.cpu(), ref)
+    for qs, ks, vs in (((1, 4, 10, 8), (1, 4, 10, 8), (1, 4, 10, 0)), ((1, 4, 10, 8), (1, 4, 0, 8), (1, 4, 0, 8))):
+        q, k, v = (torch.randn(*s_, generator=g).to(gpu_device).requires_grad_(True) for s_ in (qs, ks, vs))
+        out = F.scaled_dot_product_attention(q, k, v, dropout_p=0.0)
+        assert out.shape == (*qs[:-1], vs[-1])
+        ref = F.scaled_dot_product_attention(q.detach().cpu(), k.detach().cpu(), v.detach().cpu(), dropout_p=0.0)
+        torch.testing.assert_close(out.detach().cpu(), ref)
+        out.sum().backward()
+        assert q.grad.shape == q.shape and k.grad.shape == k.shape and v.grad.shape == v.shape
+    assert calls["fwd"] == 0 and calls["bwd"] == 0
+
+
+@pytest.mark.parametrize("Hq,S,D", [(8, 1280, 256), (8, 512, 64)])
+def test_backward_with_stride0_expanded_kv(amd, gpu_device, calls, Hq, S, D):
+    # test_scaled_dot_product_attention.py:1123-1221: K/V from repeat_kv's expand + reshape (stride 0 on
+    # batch and heads).  The gradients of such views are dense tensors that alias nothing (autograd then
+    # sums them back to the one real head), their leaf strides equal what the CPU gives, and here the
+    # values are also checked against the oracle.
+    def repeat_kv(t, n):
+        b, kv, s, d = t.shape
+        return t[:, :, None, :, :].expand(b, kv, n, s, d).reshape(b, kv * n, s, d)
+
+    q, k, v, go = qkv(1, Hq, 1, S, S, D, dtype=torch.bfloat16, seed=21, with_do=True)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    k_in, v_in = repeat_kv(kd, Hq), repeat_kv(vd, Hq)
+    assert k_in.stride()[:2] == (0, 0) and v_in.stride()[:2] == (0, 0)
+    seen = {}
+    k_in.register_hook(lambda g_: seen.__setitem__("dk", g_))
+    v_in.register_hook(lambda g_: seen.__setitem__("dv", g_))
+    out = F.scaled_dot_product_attention(qd, k_in, v_in, is_causal=True)
+    out.backward(go.to(gpu_device))
+    assert calls["fwd"] == 1 and calls["bwd"] == 1
+    for g_ in (seen["dk"], seen["dv"]):  # dense, one slab per (expanded) head
+        assert g_.shape == (1, Hq, S, D) and g_.stride() == (Hq * S * D, S * D, D, 1)
+    qc, kc, vc = (t.clone().requires_grad_(True) for t in (q, k, v))
+    F.scaled_dot_product_attention(qc, repeat_kv(kc, Hq), repeat_kv(vc, Hq), is_causal=True).backward(go)
+    assert qd.grad.stride() == qc.grad.stride() and kd.grad.stride() == kc.grad.stride()
+    assert vd.grad.stride() == vc.grad.stride() and kd.grad.shape == k.shape
+    ro, rl = oracle_fwd(q, k, v, is_causal=True)
+    rdq, rdk, rdv = oracle_bwd(go, q, k, v, ro, rl, is_causal=True)
+    assert max_abs(out, ro) <= 2e-2
+    assert max_abs(qd.grad, rdq) <= 5e-2 and rel_err(qd.grad, rdq) <= 3e-2
+    # (the leaf gradient is the sum of eight bf16 head gradients: one more rounding per head)
+    for a, r in ((kd.grad, rdk), (vd.grad, rdv)):
+        assert rel_err(a, r) <= 3e-2 and max_abs(a, r) <= 5e-2 + 2e-2 * r.abs().max().item()
+
+
+def test_unregister_brings_the_stock_kernels_back(amd, gpu_device, calls):
+    q, k, v = (t.to(gpu_device) for t in qkv(1, 4, 4, 128, 128, 64, dtype=torch.bfloat16, seed=3))
+    F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert calls["fwd"] == 1
+    names = amd.registered_ops()
+    assert "_scaled_dot_product_flash_attention" in names
+    amd.unregister()
+    try:
+        assert amd.registered_ops() == []
+        out = F.scaled_dot_product_attention(q, k, v, is_causal=True)  # the stock kernel (or its math path)
+        assert calls["fwd"] == 1
+        ro, _ = oracle_fwd(q.cpu(), k.cpu(), v.cpu(), is_causal=True)
+        assert max_abs(out, ro) <= 2e-2
+    finally:
+        amd.register()
+    assert set(amd.registered_ops()) == set(names)
+    F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    assert calls["fwd"] == 2
+
+
 def test_dropout_extremes_and_mask_round_trip(amd, gpu_device):
     q, k, v = (t.to(gpu_device) for t in qkv(1, 2, 2, 32, 32, 32, dtype=torch.float32, seed=8))
     op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
@@ -167,6 +247,16 @@ def test_kernel_level_custom_ops(amd, gpu_device):
     tiled = lse.reshape(2, 8, 2, 128).transpose(-1, -2).contiguous()  # (B,H,128,L/128) form
     dq2, dk2, dv2 = amd.scaled_dot_product_attention_backward_kernel(go, q, k, v, out, tiled, True)
     assert torch.equal(dq, dq2) and torch.equal(dk, dk2)
+    # a tiled buffer filled by the forward op holds row t * 128 + p at [p, t], which is what the
+    # backward op reads from it: forward -> backward round trip through the 4-D form
+    tiled_fwd = torch.empty(2, 8, 128, 2, dtype=torch.float32, device=gpu_device)
+    out3 = amd.scaled_dot_product_attention_kernel(q, k, v, is_causal=True, training=True, lse=tiled_fwd)
+    assert torch.equal(out3, out) and torch.equal(tiled_fwd, tiled)
+    dq3, dk3, dv3 = amd.scaled_dot_product_attention_backward_kernel(go, q, k, v, out3, tiled_fwd, True)
+    assert torch.equal(dq, dq3) and torch.equal(dk, dk3) and torch.equal(dv, dv3)
+    with pytest.raises(ValueError):  # same element count, wrong shape: refused, not reshaped
+        amd.scaled_dot_product_attention_kernel(q, k, v, is_causal=True, training=True,
+                                                lse=torch.empty(2, 8, 2, 128, dtype=torch.float32, device=gpu_device))
     rdq, rdk, rdv = oracle_bwd(go.cpu(), q.cpu(), k.cpu(), v.cpu(), ro, rl, is_causal=True)
     for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
         assert max_abs(a, r) <= 5e-2 and rel_err(a, r) <= 3e-2

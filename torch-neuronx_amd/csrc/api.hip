@@ -115,7 +115,12 @@ int mi355_sdpa_validate(const mi355_sdpa_desc* d, char* msg, size_t n) {
   if (dt != MI355_SDPA_F32 && dt != MI355_SDPA_F16 && dt != MI355_SDPA_BF16)
     return fail(msg, n, "SDPA: query dtype must be float32, float16, or bfloat16, got %s",
                 dtype_name(d->q_dtype));
-  if (d->k_dtype != d->q_dtype || d->v_dtype != d->q_dtype)
+  // (a float64 query makes the reference downcast every float64 operand before it compares the
+  // dtypes, NeuronDispatcher.cpp:2418-2432: float64 query with float32 key / value is accepted)
+  const bool q64 = d->q_dtype == MI355_SDPA_F64;
+  const int kdt = q64 && d->k_dtype == MI355_SDPA_F64 ? MI355_SDPA_F32 : d->k_dtype;
+  const int vdt = q64 && d->v_dtype == MI355_SDPA_F64 ? MI355_SDPA_F32 : d->v_dtype;
+  if (kdt != dt || vdt != dt)
     return fail(msg, n, "SDPA: query, key, value must have the same dtype");
   if (d->q_dim != 4 || d->k_dim != 4 || d->v_dim != 4)
     return fail(msg, n, "SDPA: query, key, value must be 4D tensors (B, H, S, D)");
@@ -133,9 +138,71 @@ int mi355_sdpa_validate(const mi355_sdpa_desc* d, char* msg, size_t n) {
   return MI355_SDPA_OK;
 }
 
+// true if the strides describe a dense block in some dimension order without overlap
+// (c10::TensorImpl::compute_non_overlapping_and_dense)
+static bool non_overlapping_and_dense(const int64_t sizes[4], const int64_t strides[4]) {
+  int perm[4] = {0, 1, 2, 3};
+  // size-1 dims last, the rest by ascending stride
+  std::stable_sort(perm, perm + 4, [&](int a, int b) {
+    if (sizes[a] < 2) return false;
+    if (sizes[b] < 2) return true;
+    return strides[a] < strides[b];
+  });
+  int64_t need = 1;
+  for (int i = 0; i < 4; ++i) {
+    const int d = perm[i];
+    if (sizes[d] < 2) return true;
+    if (strides[d] != need) return false;
+    need *= sizes[d];
+  }
+  return true;
+}
+
+// at::infer_dense_strides: dense strides that keep the dimension order of a strided tensor;
+// dims with stride 0 (expanded) are never moved
+static void infer_dense_strides(const int64_t sizes[4], const int64_t strides[4], int64_t out[4]) {
+  int perm[4] = {3, 2, 1, 0};
+  auto should_swap = [&](int d0, int d1) {
+    const int64_t s0 = strides[d0], s1 = strides[d1];
+    if (s0 == 0 || s1 == 0) return 0;
+    if (s0 < s1) return -1;
+    if (s0 > s1) return 1;
+    return sizes[d0] > sizes[d1] ? 1 : 0;
+  };
+  for (int i = 1; i < 4; ++i) {
+    int dim1 = i;
+    for (int j = 1; j <= i; ++j) {
+      const int dim0 = i - j;
+      const int c = should_swap(perm[dim0], perm[dim1]);
+      if (c > 0) {
+        std::swap(perm[dim0], perm[dim1]);
+        dim1 = dim0;
+      } else if (c < 0) {
+        break;
+      }
+    }
+  }
+  int64_t s = 1;
+  for (int i = 0; i < 4; ++i) {
+    out[perm[i]] = s;
+    if (sizes[perm[i]] > 1) s *= sizes[perm[i]];
+  }
+}
+
 int mi355_sdpa_out_strides(const int64_t ref_sizes[4], const int64_t ref_strides[4],
                            const int64_t out_sizes[4], int64_t out_strides[4]) {
-  (void)ref_sizes;
+  bool same = true;
+  for (int i = 0; i < 4; ++i) same = same && ref_sizes[i] == out_sizes[i];
+  if (same) {
+    // torch.empty_like(ref): the strides themselves when they are dense, else the dense strides
+    // of the same dimension order (an expanded dim becomes a real one)
+    if (non_overlapping_and_dense(ref_sizes, ref_strides)) {
+      for (int i = 0; i < 4; ++i) out_strides[i] = ref_strides[i];
+    } else {
+      infer_dense_strides(ref_sizes, ref_strides, out_strides);
+    }
+    return MI355_SDPA_OK;
+  }
   int order[4] = {0, 1, 2, 3};
   // outermost first; ties keep the original dimension order
   std::stable_sort(order, order + 4, [&](int a, int b) { return ref_strides[a] > ref_strides[b]; });
@@ -162,8 +229,9 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   if (d->return_debug_mask) return MI355_SDPA_KERNEL_NONE;
   if (E > 512 || Dv > 512) return MI355_SDPA_KERNEL_NONE;
   const float scale = d->has_scale ? d->scale : 1.f;
-  // (the layout of a bias or mask is checked again at the call; a requested bias gradient sends
-  // the backward to the generic kernel there)
+  // The descriptor carries no pointers and no bias layout, so this answer is an upper bound: the
+  // call itself still sends to the generic kernel a bias whose rows are not dword-aligned, tensors
+  // that are not 16-byte aligned or whose strides are not multiples of 8 elements.
   const bool bias_ok = true;
   const bool dims = backward ? (E == Dv && E % 8 == 0 && E <= 128) : (E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E);
   const bool fast = d->q_dtype != MI355_SDPA_F32 && dims &&

@@ -131,15 +131,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const uint32_t lds_q = (uint32_t)(uintptr_t)(lds_bytes)q_t + wave * 1024;
   const uint32_t lds_do = (uint32_t)(uintptr_t)(lds_bytes)do_t + wave * 1024;
   auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
-    // (m0 holds the LDS address of such a load, one wait state after it is written; nothing else in
-    // this kernel uses m0)
+    // (m0 holds the LDS address of such a load, one wait state after it is written; it is declared
+    // clobbered, so the compiler keeps no value of its own in m0 across the statement)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   const uint32_t lds_lse = (uint32_t)(uintptr_t)(lds_bytes)lse_s, lds_dl = (uint32_t)(uintptr_t)(lds_bytes)dl_s;
   auto row_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   auto wait_tiles = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
   auto load_item = [&](int it, int buf) {  // the tiles of item `it` into tile buffer `buf`

@@ -174,10 +174,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   const uint32_t lds_k = (uint32_t)(uintptr_t)(lds_bytes)&k_t[0][0] + (uint32_t)((SPLIT ? wave % (TCH / 64) : wave) * 1024);
   const uint32_t lds_v = (uint32_t)(uintptr_t)(lds_bytes)&v_t[0][0] + (uint32_t)((SPLIT ? wave % (TCH / 64) : wave) * 1024);
   auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
-    // (m0 holds the LDS address of such a load, one wait state after it is written; nothing else in
-    // this kernel uses m0)
+    // (m0 holds the LDS address of such a load, one wait state after it is written; it is declared
+    // clobbered, so the compiler keeps no value of its own in m0 across the statement)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   auto load_tile = [&](int t) {  // tile t (the last one again past the end) into buffer t % 4
     const uint32_t tt = (uint32_t)min(t, nt - 1);

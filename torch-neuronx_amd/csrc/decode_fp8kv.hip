@@ -32,10 +32,7 @@ typedef __attribute__((ext_vector_type(2))) float f32x2;
 constexpr int D = 128;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-#ifndef DEC_OCC
-#define DEC_OCC 2
-#endif
-constexpr int kDecOcc = DEC_OCC;  // wavefronts per SIMD the decode kernel is built for
+constexpr int kDecOcc = 2;  // wavefronts per SIMD the decode kernel is built for (three or four spill)
 constexpr float kPScale = 256.f;  // probabilities are stored as e4m3 of 256*p
 
 struct DecP {

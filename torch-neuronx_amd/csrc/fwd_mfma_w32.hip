@@ -245,10 +245,10 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const uint32_t lds_kd = (uint32_t)(uintptr_t)(lds_bytes)k_dma + (uint32_t)(d_wave * 1024);
   const uint32_t lds_vd = (uint32_t)(uintptr_t)(lds_bytes)v_dma + (uint32_t)(d_wave * 1024);
   auto tile_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
-    // (m0 holds the LDS address of such a load, one wait state after it is written; nothing else in
-    // this kernel uses m0)
+    // (m0 holds the LDS address of such a load, one wait state after it is written; it is declared
+    // clobbered, so the compiler keeps no value of its own in m0 across the statement)
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
-                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory");
+                 :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   auto request_k = [&](int t) {  // K tile t (the last one again past the end) into buffer t % 4
     if constexpr (DMA) {

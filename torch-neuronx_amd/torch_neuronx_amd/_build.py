@@ -21,7 +21,10 @@ HIPCC_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # per-kernel register / scratch / LDS figures, kept next to the library (RESOURCE_PATH)
+    "-Rpass-analysis=kernel-resource-usage",
 ]
+RESOURCE_PATH = os.path.join(LIB_DIR, "resource_usage.txt")
 
 
 def _hipcc() -> str:
@@ -31,13 +34,55 @@ def _hipcc() -> str:
     return exe
 
 
+def _resource_lines(stderr: str):
+    """'<mangled kernel name> <key>=<value> ...' per kernel, from the compiler's resource remarks."""
+    out, cur = [], None
+    for line in stderr.splitlines():
+        if "[-Rpass-analysis=kernel-resource-usage]" not in line or "remark:" not in line:
+            continue
+        body = line.split("remark:", 1)[1].rsplit("[-Rpass", 1)[0].strip()
+        key, _, val = body.partition(":")
+        if key.strip() == "Function Name":
+            cur = [val.strip()]
+            out.append(cur)
+        elif cur is not None:
+            cur.append(f"{key.strip().replace(' ', '_')}={val.strip()}")
+    return [" ".join(c) for c in out]
+
+
+def _noise(lines):
+    """Compiler output minus what every build prints: the host pass does not know the packed-fp32
+    feature, the resource remarks (collected separately), and the note that m0, which the LDS-direct
+    loads clobber on purpose, is a reserved register."""
+    keep, skip = [], 0
+    for l in lines:
+        if skip:
+            skip -= 1
+            continue
+        if "packed-fp32-ops" in l:
+            continue
+        if "-Rpass-analysis=kernel-resource-usage" in l:
+            skip = 2 if "Function Name" in l else 0  # the source line and the caret under it
+            continue
+        if "clobber list contains reserved registers: m0" in l:
+            skip = 2
+            continue
+        if "Reserved registers on the clobber list" in l:
+            continue
+        if l.strip() in ("", "^") or l.strip().endswith("warnings generated when compiling for gfx950."):
+            continue
+        keep.append(l)
+    return keep
+
+
 def _run(cmd, verbose):
     proc = subprocess.run(cmd, capture_output=True, text=True)
-    err = "\n".join(l for l in proc.stderr.splitlines() if "packed-fp32-ops" not in l)
+    err = "\n".join(_noise(proc.stderr.splitlines()))
     if proc.returncode != 0:
         raise RuntimeError(f"build step failed: {' '.join(cmd)}\n{proc.stdout}\n{err}")
     if verbose and err.strip():
         print(err, file=sys.stderr)
+    return _resource_lines(proc.stderr)
 
 
 def build(verbose: bool = False, jobs: int = 6) -> str:
@@ -48,11 +93,16 @@ def build(verbose: bool = False, jobs: int = 6) -> str:
     def compile_one(name):
         src = os.path.join(CSRC_DIR, name + ".hip")
         obj = os.path.join(OBJ_DIR, name + ".o")
-        _run([hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj], verbose)
-        return obj
+        return obj, _run([hipcc, *HIPCC_FLAGS, "-c", src, "-o", obj], verbose)
 
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(compile_one, SOURCES))
+        results = list(pool.map(compile_one, SOURCES))
+    objs = [o for o, _ in results]
+    with open(RESOURCE_PATH + ".tmp", "w") as f:
+        for name, (_, lines) in zip(SOURCES, results):
+            for l in lines:
+                f.write(f"{name}.hip {l}\n")
+    os.replace(RESOURCE_PATH + ".tmp", RESOURCE_PATH)
     tmp = LIB_PATH + ".tmp"
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", tmp, *objs], verbose)
     os.replace(tmp, LIB_PATH)

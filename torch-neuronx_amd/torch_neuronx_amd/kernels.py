@@ -27,7 +27,17 @@ def _scaled_dot_product_attention_kernel(
 ) -> torch.Tensor:
     out, lse_ret = ops.sdpa_forward(q, k, v, is_causal=is_causal, scale=scale, need_lse=training)
     if training and lse is not None:
-        lse.copy_(lse_ret.reshape(lse.shape))
+        B, H, L = lse_ret.shape
+        if lse.dim() == 4:  # the tiled (B, H, 128, L // 128) form: row t * 128 + p sits at [p, t]
+            if L % 128 != 0 or tuple(lse.shape) != (B, H, 128, L // 128):
+                raise ValueError(f"a tiled lse buffer must have shape {(B, H, 128, L // 128)} with L divisible by 128, "
+                                 f"got {tuple(lse.shape)}")
+            lse.copy_(lse_ret.reshape(B, H, L // 128, 128).transpose(-1, -2))
+        elif tuple(lse.shape) == (B, H, L):
+            lse.copy_(lse_ret)
+        else:
+            raise ValueError(f"lse buffer must have shape {(B, H, L)} or the tiled {(B, H, 128, 'L // 128')}, "
+                             f"got {tuple(lse.shape)}")
     return out
 
 
@@ -51,8 +61,8 @@ def scaled_dot_product_attention_backward_kernel(
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     B, H, L, _ = q.shape
     if lse.dim() == 4:  # the reference's tiled (B, H, 128, L // 128) form
-        if L % 128 != 0:
-            raise ValueError("a tiled lse needs a query length divisible by 128")
+        if L % 128 != 0 or tuple(lse.shape) != (B, H, 128, L // 128):
+            raise ValueError("a tiled lse needs a query length divisible by 128 and shape (B, H, 128, L // 128)")
         lse = lse.transpose(-1, -2).reshape(B, H, L)
     dq, dk, dv, _ = ops.sdpa_backward(grad_out, q, k, v, out, lse, is_causal=is_causal, scale=scale)
     return dq, dk, dv

@@ -80,7 +80,7 @@ def out_strides(ref_sizes, ref_strides, out_sizes):
 
 def empty_like_layout(ref: torch.Tensor, shape, dtype=None) -> torch.Tensor:
     """New tensor of ``shape`` whose dimension order follows ``ref`` (stride-0 dims never alias)."""
-    if ref.is_contiguous():  # the common case needs no stride arithmetic
+    if ref.is_contiguous() and 0 not in ref.shape:  # the common case needs no stride arithmetic
         return torch.empty(tuple(shape), dtype=dtype or ref.dtype, device=ref.device)
     st = out_strides(ref.shape, ref.stride(), shape)
     return torch.empty_strided(tuple(shape), st, dtype=dtype or ref.dtype, device=ref.device)

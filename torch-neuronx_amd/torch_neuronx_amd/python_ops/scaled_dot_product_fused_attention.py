@@ -71,14 +71,26 @@ def _dropout_keep(query, S, dropout_p):
     return (torch.rand((B, H, L, S), device=query.device) >= dropout_p).to(torch.uint8)
 
 
+def _present(attn_bias):
+    """An empty bias is a lowering placeholder and counts as absent (torch_neuronx/_sdpa_math.py:30)."""
+    return None if attn_bias is None or attn_bias.numel() == 0 else attn_bias
+
+
+def _wants_grad_bias(attn_bias, grad_input_mask) -> bool:
+    """A bias of at most one element gets no gradient (torch_neuronx/_sdpa_math.py:142,169)."""
+    return (attn_bias is not None and attn_bias.numel() > 1 and len(grad_input_mask) > 3
+            and bool(grad_input_mask[3]))
+
+
 def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale, need_lse=True):
     _check_device(query)
+    attn_bias = _present(attn_bias)
     if return_debug_mask:
         raise NotImplementedError("Debug mask not supported in Neuron implementation.")
     _validate_once(query, key, value, attn_bias, dropout_p, is_causal, scale)
     orig_dtype = query.dtype
     if orig_dtype == torch.float64:  # computed as float32, result restored to the caller's dtype
-        query, key, value = query.float(), key.float(), value.float()
+        query, key, value = query.float(), key.float(), value.float()  # (no-ops for float32 key / value)
         if attn_bias is not None and attn_bias.dtype == torch.float64:
             attn_bias = attn_bias.float()
     S = key.shape[2]
@@ -109,6 +121,7 @@ def scaled_dot_product_fused_attention_overrideable(
 def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p, is_causal, philox_seed,
               scale, want_grad_bias):
     _check_device(query)
+    attn_bias = _present(attn_bias)
     orig_dtype = query.dtype
     if orig_dtype == torch.float64:
         grad_out, query, key, value, out = (t.float() for t in (grad_out, query, key, value, out))
@@ -137,7 +150,7 @@ def scaled_dot_product_fused_attention_overrideable_backward(
 ):
     """``aten::_scaled_dot_product_fused_attention_overrideable_backward``: ``(dq, dk, dv, dbias)``;
     ``dbias`` is ``None`` when there is no bias or its gradient is not asked for."""
-    want = attn_bias is not None and len(grad_input_mask) > 3 and bool(grad_input_mask[3])
+    want = _wants_grad_bias(attn_bias, grad_input_mask)
     return _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p, is_causal,
                      philox_seed, scale, want)
 
@@ -175,7 +188,7 @@ def scaled_dot_product_efficient_attention_backward(
     grad_input_mask, is_causal=False, scale=None
 ):
     """``aten::_scaled_dot_product_efficient_attention_backward``: ``(dq, dk, dv, dbias)``."""
-    want = attn_bias is not None and len(grad_input_mask) > 3 and bool(grad_input_mask[3])
+    want = _wants_grad_bias(attn_bias, grad_input_mask)
     dq, dk, dv, dbias = _backward(grad_out_, query, key, value, attn_bias, out, logsumexp, dropout_p,
                                   is_causal, philox_seed, scale, want)
     if dbias is None:
