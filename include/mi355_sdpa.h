@@ -159,6 +159,20 @@ size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p);
 int mi355_sdpa_decode_fp8kv(const mi355_sdpa_decode_params* p, void* stream);
 size_t mi355_sdpa_decode_workspace_bytes(const mi355_sdpa_decode_params* p);
 
+/* The same decode step for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid it).  No counterpart in the reference.
+ * p->workspace and p->workspace_bytes are ignored: partial results and step counts go to a
+ * static device array of MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES that every GPU holds from the
+ * first call on it until the process ends.  A call that would need more scratch than that
+ * (mi355_sdpa_decode_workspace_bytes tells) fails with MI355_SDPA_ERR_UNSUPPORTED.  The entry
+ * point calls no allocating routine; the caller passes inputs and outputs as for
+ * mi355_sdpa_decode_fp8kv, and the results are the same bit for bit.  All calls on one GPU
+ * share the array: calls that overlap there (different streams, different threads) race; keep
+ * them on one stream or order them with events.  The first call on a device looks the array's
+ * address up (hipGetSymbolAddress): make it outside a stream capture. */
+#define MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES (32u << 20)
+int mi355_sdpa_decode_fp8kv_static(const mi355_sdpa_decode_params* p, void* stream);
+
 /* ---- host logic (no GPU needed) --------------------------------------------------------- */
 
 /* Backend choice for F.scaled_dot_product_attention.  Rules of

@@ -323,15 +323,36 @@ size_t mi355_sdpa_decode_workspace_bytes(const mi355_sdpa_decode_params* p) {
   return p ? decode_workspace(*p) : 0;
 }
 
-int mi355_sdpa_decode_fp8kv(const mi355_sdpa_decode_params* p, void* stream) {
-  if (!p) return set_error("SDPA: null params"), MI355_SDPA_ERR_INVALID;
+static bool decode_args_ok(const mi355_sdpa_decode_params* p) {
+  if (!p) return set_error("SDPA: null params"), false;
   if (!tensor_ok(p->q, "query") || !tensor_ok(p->k, "key") || !tensor_ok(p->v, "value") ||
       !tensor_ok(p->out, "out"))
-    return MI355_SDPA_ERR_INVALID;
-  if (!p->k_scale || !p->v_scale) return set_error("SDPA decode: k_scale / v_scale missing"), MI355_SDPA_ERR_INVALID;
-  if (!shapes_ok(p->q, p->k, p->v)) return MI355_SDPA_ERR_INVALID;
+    return false;
+  if (!p->k_scale || !p->v_scale) return set_error("SDPA decode: k_scale / v_scale missing"), false;
+  if (!shapes_ok(p->q, p->k, p->v)) return false;
   if (!same_shape(p->out, p->q.size[0], p->q.size[1], p->q.size[2], p->v.size[3]))
-    return set_error("SDPA decode: out must have shape (B, Hq, Lq, D)"), MI355_SDPA_ERR_INVALID;
+    return set_error("SDPA decode: out must have shape (B, Hq, Lq, D)"), false;
+  return true;
+}
+
+int mi355_sdpa_decode_fp8kv_static(const mi355_sdpa_decode_params* p, void* stream) {
+  if (!decode_args_ok(p)) return MI355_SDPA_ERR_INVALID;
+  const size_t need = decode_workspace(*p);
+  if (need > (size_t)MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES)
+    return set_error("SDPA decode: this call needs %zu bytes of scratch, the static scratch holds %zu; "
+                     "use mi355_sdpa_decode_fp8kv with a workspace", need, (size_t)MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES),
+           MI355_SDPA_ERR_UNSUPPORTED;
+  mi355_sdpa_decode_params q = *p;
+  void* ptr = nullptr;
+  const int rc = decode_static_scratch(&ptr);
+  if (rc != MI355_SDPA_OK) return rc;
+  q.workspace = ptr;
+  q.workspace_bytes = (size_t)MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES;
+  return launch_decode_fp8kv(q, (hipStream_t)stream);
+}
+
+int mi355_sdpa_decode_fp8kv(const mi355_sdpa_decode_params* p, void* stream) {
+  if (!decode_args_ok(p)) return MI355_SDPA_ERR_INVALID;
   const size_t need = decode_workspace(*p);
   if (need && (!p->workspace || p->workspace_bytes < need))
     return set_error("SDPA decode: workspace too small (%zu < %zu bytes)", p->workspace_bytes, need),

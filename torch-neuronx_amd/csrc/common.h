@@ -23,6 +23,7 @@ size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p);
 int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s);
 size_t decode_workspace(const mi355_sdpa_decode_params& p);
 int decode_pick_splits(const mi355_sdpa_decode_params& p);
+int decode_static_scratch(void** device_ptr);
 
 // device side -----------------------------------------------------------------------------
 typedef __bf16 bf16_t;

@@ -19,8 +19,15 @@
 // contraction order is permuted identically for Q) and eight 4-byte pieces of V which are
 // byte-transposed in registers into the A operand of O^T = V^T P^T.
 #include <algorithm>
+#include <atomic>
 
 #include "common.h"
+
+// Scratch of the entry point that allocates nothing (mi355_sdpa_decode_fp8kv_static): partial
+// results and step counts of one decode call.  Every GPU the library runs on holds its own copy
+// until the process ends.  In host code this name is only a handle for hipGetSymbolAddress; the
+// device address it yields, kept per device, is what kernels and copies are given.
+static __device__ __align__(256) unsigned char scratch[MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES];
 
 namespace mi355 {
 namespace {
@@ -511,6 +518,26 @@ size_t decode_workspace(const mi355_sdpa_decode_params& p) {
   const int64_t rep = p.k.size[1] ? p.q.size[1] / p.k.size[1] : 0;
   const int64_t R = rep * p.q.size[2];
   return (size_t)(partial_slots(p) * R * (D + 2)) * sizeof(float) + (size_t)(p.q.size[0] + 1) * sizeof(int32_t);
+}
+
+// Device address of `scratch` on the current device, looked up once per device.
+int decode_static_scratch(void** out) {
+  constexpr int kMaxDevices = 64;
+  static std::atomic<void*> addr[kMaxDevices];
+  int dev = -1;
+  const hipError_t e0 = hipGetDevice(&dev);
+  if (e0 != hipSuccess || dev < 0 || dev >= kMaxDevices)
+    return set_error("SDPA decode: no usable current device (%s)", hipGetErrorString(e0)), MI355_SDPA_ERR_LAUNCH;
+  void* ptr = addr[dev].load(std::memory_order_acquire);
+  if (!ptr) {
+    const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || !ptr)
+      return set_error("SDPA decode: static scratch has no address on device %d (%s)", dev, hipGetErrorString(e)),
+             MI355_SDPA_ERR_LAUNCH;
+    addr[dev].store(ptr, std::memory_order_release);
+  }
+  *out = ptr;
+  return MI355_SDPA_OK;
 }
 
 int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {

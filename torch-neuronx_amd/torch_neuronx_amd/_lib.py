@@ -17,6 +17,7 @@ F32, F16, BF16, F64, BOOL, FP8_E4M3, OTHER = 0, 1, 2, 3, 4, 5, 99
 KERNEL_NONE, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA_T128, KERNEL_MFMA_T256 = 0, 1, 2, 3, 4
 BACKEND_MATH, BACKEND_OVERRIDEABLE = 0, 4
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_LAUNCH = 0, -1, -2, -3
+DECODE_STATIC_SCRATCH_BYTES = 32 << 20
 
 _DTYPES = {
     torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64,
@@ -80,6 +81,7 @@ EXPORTS = {
     "mi355_sdpa_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdParams)]),
     "mi355_sdpa_decode_fp8kv": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),
     "mi355_sdpa_decode_workspace_bytes": (C.c_size_t, [C.POINTER(DecodeParams)]),
+    "mi355_sdpa_decode_fp8kv_static": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),
     "mi355_sdpa_choose_backend": (C.c_int, [C.POINTER(Desc)]),
     "mi355_sdpa_validate": (C.c_int, [C.POINTER(Desc), C.c_char_p, C.c_size_t]),
     "mi355_sdpa_out_strides": (C.c_int, [C.POINTER(C.c_int64), C.POINTER(C.c_int64),

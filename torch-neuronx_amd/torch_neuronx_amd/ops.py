@@ -189,8 +189,13 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
 
 
 def decode_fp8kv(query, k_fp8, v_fp8, k_scale, v_scale, kv_lens=None, scale=None,
-                 num_splits=0, need_lse=True):
-    """Decode-step attention over an fp8 e4m3 K/V cache.  Returns ``(out, lse)``."""
+                 num_splits=0, need_lse=True, out=None, lse=None, static_scratch=False):
+    """Decode-step attention over an fp8 e4m3 K/V cache.  Returns ``(out, lse)``.
+
+    With ``static_scratch=True`` the call goes through ``mi355_sdpa_decode_fp8kv_static``, which
+    allocates nothing: the caller passes ``out`` (and ``lse`` if wanted), ``k_scale`` / ``v_scale`` /
+    ``kv_lens`` must already be contiguous float32 / int32 device tensors, and nothing is allocated
+    here either."""
     for t, n in ((query, "query"), (k_fp8, "key"), (v_fp8, "value")):
         _require_cuda(t, n)
     if k_fp8.dtype != torch.float8_e4m3fn or v_fp8.dtype != torch.float8_e4m3fn:
@@ -198,20 +203,44 @@ def decode_fp8kv(query, k_fp8, v_fp8, k_scale, v_scale, kv_lens=None, scale=None
     B, Hq, Lq, D = query.shape
     if scale is None:
         scale = 1.0 / math.sqrt(D)
-    q, k, v = _unit_last(query), _unit_last(k_fp8), _unit_last(v_fp8)
-    out = torch.empty((B, Hq, Lq, v.shape[3]), dtype=query.dtype, device=query.device)
-    lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=query.device) if need_lse else None
-    ks = k_scale.to(device=query.device, dtype=torch.float32).contiguous()
-    vs = v_scale.to(device=query.device, dtype=torch.float32).contiguous()
+    if static_scratch:
+        if out is None:
+            raise ValueError("decode_fp8kv: static_scratch=True needs a preallocated out")
+        for t, n, dt in ((k_scale, "k_scale", torch.float32), (v_scale, "v_scale", torch.float32),
+                         (kv_lens, "kv_lens", torch.int32)):
+            if t is not None and (t.dtype != dt or not t.is_contiguous() or t.device != query.device):
+                raise ValueError(f"decode_fp8kv: with static_scratch=True {n} must be a contiguous {dt} tensor on the query's device")
+        for t, n in ((query, "query"), (k_fp8, "key"), (v_fp8, "value"), (out, "out")):
+            if t.stride(-1) != 1:
+                raise ValueError(f"decode_fp8kv: with static_scratch=True {n} must have unit stride on the head dim")
+        q, k, v, ks, vs = query, k_fp8, v_fp8, k_scale, v_scale
+    else:
+        q, k, v = _unit_last(query), _unit_last(k_fp8), _unit_last(v_fp8)
+        if out is None:
+            out = torch.empty((B, Hq, Lq, v.shape[3]), dtype=query.dtype, device=query.device)
+        if lse is None and need_lse:
+            lse = torch.empty((B, Hq, Lq), dtype=torch.float32, device=query.device)
+        ks = k_scale.to(device=query.device, dtype=torch.float32).contiguous()
+        vs = v_scale.to(device=query.device, dtype=torch.float32).contiguous()
+        if kv_lens is not None:
+            kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
+    if tuple(out.shape) != (B, Hq, Lq, v.shape[3]) or out.dtype != query.dtype:
+        raise ValueError("decode_fp8kv: out must have shape (B, Hq, Lq, D) and the query's dtype")
+    if lse is not None and (tuple(lse.shape) != (B, Hq, Lq) or lse.dtype != torch.float32 or not lse.is_contiguous()):
+        raise ValueError("decode_fp8kv: lse must be a contiguous float32 (B, Hq, Lq) tensor")
     p = _lib.DecodeParams()
     p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (q, k, v, out))
     p.k_scale, p.v_scale = ks.data_ptr(), vs.data_ptr()
     if kv_lens is not None:
-        kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
         p.kv_lens = kv_lens.data_ptr()
     p.lse = lse.data_ptr() if lse is not None else None
     p.q_dtype, p.scale, p.num_splits = _lib.dtype_id(query.dtype), float(scale), int(num_splits)
     lib = _lib.load()
+    if static_scratch:
+        with _lib.on_device(query.device):
+            rc = lib.mi355_sdpa_decode_fp8kv_static(C.byref(p), _lib.current_stream(query.device))
+        _lib.check(rc)
+        return out, lse
     nbytes = lib.mi355_sdpa_decode_workspace_bytes(C.byref(p))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=query.device)
     p.workspace, p.workspace_bytes = ws.data_ptr(), nbytes
