@@ -15,9 +15,13 @@
 // occupy separate columns of the 16-wide MFMA N dimension, which would otherwise idle, and
 // are summed after the product.  The probabilities are split the same way before P*V.
 //
-// Per 32 keys a lane loads 64 contiguous K bytes of one key (A operand of S^T = K Q^T, the
-// contraction order is permuted identically for Q) and eight 4-byte pieces of V which are
-// byte-transposed in registers into the A operand of O^T = V^T P^T.
+// Per 32 keys a lane loads two 16-byte pieces of each of two keys (A operand of S^T = K Q^T; the
+// contraction order is permuted identically for Q) and eight 8-byte pieces of V, one from each
+// of eight keys, which are byte-transposed in registers into the A operand of O^T = V^T P^T.
+// Every load is non-temporal (the cache is read once) and a V instruction covers four whole
+// 128-byte rows: with plain loads the stream reads 5.8 TB/s whatever the shape, with
+// non-temporal ones 5.8 TB/s when a row is fetched in two instructions and 6.5 TB/s when in one
+// (measured with a memory-only model of this kernel's work split).
 #include <algorithm>
 #include <atomic>
 
@@ -105,9 +109,10 @@ __device__ __forceinline__ long as_long(uint32_t lo, uint32_t hi) {
   return (long)(((uint64_t)hi << 32) | lo);
 }
 
+typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
 struct KVRegs {
-  u32x4 k[2][2];      // [16-key block][16-byte half of the lane's 32 bytes]
-  uint32_t v[2][8];   // [64-wide half of d][key slot]
+  u32x4 k[2][2];  // [16-key block][d = 16g .. +15 | d = 64 + 16g .. +15] of the lane's key
+  u32x2 v[8];     // [key slot s]: d = 8n .. 8n+7 of key 4s + g
 };
 
 // Steps per wavefront for a work list of `total` steps: equal shares, but not so small that the
@@ -203,12 +208,17 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   typedef __attribute__((ext_vector_type(4))) uint32_t qraw_t;
   qraw_t qraw[QV];  // the 32 query elements of this lane for the item fetched last, as loaded
   auto fetch_q = [&](const Item& it) {
-    const TQ* qr = (const TQ*)p.q + it.b * p.q_sb + (it.hk * rep + hq_off) * p.q_sh + lq * p.q_sl + 32 * g;
+    const TQ* qr = (const TQ*)p.q + it.b * p.q_sb + (it.hk * rep + hq_off) * p.q_sh + lq * p.q_sl + 16 * g;
 #pragma unroll
-    for (int i = 0; i < QV; ++i) qraw[i] = *(const qraw_t*)((const char*)qr + 16 * i);
+    for (int i = 0; i < QV; ++i)
+      qraw[i] = *(const qraw_t*)((const char*)(qr + (i >= QV / 2 ? 64 : 0)) + 16 * (i % (QV / 2)));
   };
 
   KVRegs ra, rb;
+  // Which key is which: the score tile of a 16-key block leaves the matrix op with rows 4g .. 4g+3
+  // in lane group g, and the second product wants lane group g to hold the probabilities of the keys
+  // whose V pieces it loaded, 4s + g for s = 0 .. 7.  So row m of block blk is key 16 blk + 4 (m % 4)
+  // + m / 4: accumulator register i of block blk in lane group g is key 16 blk + 4 i + g, slot s = 4 blk + i.
   auto load = [&](KVRegs& R_, const Item& it, int step) {
     const uint8_t* kp = p.k + it.b * p.k_sb + it.hk * p.k_sh;
     const uint8_t* vp = p.v + it.b * p.v_sb + it.hk * p.v_sh;
@@ -216,22 +226,21 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     const int ksl = (int)p.k_sl, vsl = (int)p.v_sl;  // host checked: a (batch, head) slab spans < 2^31 bytes
 #pragma unroll
     for (int blk = 0; blk < 2; ++blk) {
-      const int row = min(base + blk * 16 + n, last);
-      const uint8_t* kr = kp + (uint32_t)(row * ksl + 32 * g);
-      R_.k[blk][0] = *(const u32x4*)kr;
-      R_.k[blk][1] = *(const u32x4*)(kr + 16);
+      const int row = min(base + blk * 16 + 4 * (n & 3) + (n >> 2), last);
+      const uint8_t* kr = kp + (uint32_t)(row * ksl + 16 * g);
+      R_.k[blk][0] = __builtin_nontemporal_load((const u32x4*)kr);
+      R_.k[blk][1] = __builtin_nontemporal_load((const u32x4*)(kr + 64));
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
-      const int row = min(base + (s >> 2) * 16 + 4 * g + (s & 3), last);
-      const uint8_t* vr = vp + (uint32_t)(row * vsl + 4 * n);
-      R_.v[0][s] = *(const uint32_t*)vr;
-      R_.v[1][s] = *(const uint32_t*)(vr + 64);
+      const int row = min(base + 4 * s + g, last);
+      R_.v[s] = __builtin_nontemporal_load((const u32x2*)(vp + (uint32_t)(row * vsl + 8 * n)));
     }
   };
 
   // Query fragment of the item fetched last: B operand of S^T = K Q^T.
-  // The lane owns d = 32g .. 32g+31 of row r; MFMA step ks consumes d = 32g + 8ks .. +7.
+  // The lane owns d = 16g .. 16g+15 and 64+16g .. 64+16g+15 of row r, as for K; MFMA steps 0, 1
+  // consume the first group, steps 2, 3 the second.
   // Returns the factor that turns a raw fp8 dot product into a log2-domain logit.
   auto convert_q = [&](const Item& it, long (&qb)[4]) -> float {
     float qv[32];
@@ -306,7 +315,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) {
         const float x = sum_parts<PARTS>(sacc[i >> 2][i & 3]);
-        const int key = base + (i >> 2) * 16 + 4 * g + (i & 3);
+        const int key = base + (i >> 2) * 16 + 4 * (i & 3) + g;
         t[i] = key < w_end ? x * c_row : -INFINITY;
       }
       float tmax = t[0];
@@ -326,20 +335,21 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       l_run = l_run * alpha + psum;
 #pragma unroll
       for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
-      // P^T (B operand): key slot s of this lane is key (s/4)*16 + 4g + s%4, the order V is loaded in
+      // P^T (B operand): key slot s of this lane is key 4 s + g, the order V is loaded in
       uint32_t pw[4];
 #pragma unroll
       for (int jq = 0; jq < 4; ++jq)
         pw[jq] = split_pair<PARTS>(pv[2 * jq] * kPScale, pv[2 * jq + 1] * kPScale, pm);
       const long pb = as_long(pw[0] | (pw[1] << 16), pw[2] | (pw[3] << 16));
-      // O^T += V^T P^T : byte-transpose the 4-byte V pieces into rows d = 64*hf + 4n + j
+      // O^T += V^T P^T : the lane holds bytes d = 8n + e (e = 0 .. 7) of its eight keys; matrix op e
+      // takes byte e of every key (rows d = 8n + e), an 8 x 8 byte transpose done as four 4 x 4 ones
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {
-        uint32_t o_lo[4], o_hi[4];
+      for (int hf = 0; hf < 2; ++hf) {  // e = 4 hf .. 4 hf + 3: dword hf of every piece
+        uint32_t o_lo[4], o_hi[4];      // [e % 4]: key slots 0 .. 3 / 4 .. 7
 #pragma unroll
         for (int q4 = 0; q4 < 2; ++q4) {
-          const uint32_t w0 = R_.v[hf][q4 * 4 + 0], w1 = R_.v[hf][q4 * 4 + 1];
-          const uint32_t w2 = R_.v[hf][q4 * 4 + 2], w3 = R_.v[hf][q4 * 4 + 3];
+          const uint32_t w0 = R_.v[q4 * 4 + 0][hf], w1 = R_.v[q4 * 4 + 1][hf];
+          const uint32_t w2 = R_.v[q4 * 4 + 2][hf], w3 = R_.v[q4 * 4 + 3][hf];
           const uint32_t t0 = __builtin_amdgcn_perm(w1, w0, 0x05010400);
           const uint32_t t1 = __builtin_amdgcn_perm(w1, w0, 0x07030602);
           const uint32_t t2 = __builtin_amdgcn_perm(w3, w2, 0x05010400);
@@ -389,11 +399,13 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       const float vscale = cur.vscale * (1.f / kPScale);
       const int64_t slot = (int64_t)cur.slot * p.R + n;
       if (g == 0) p.ws_ml[slot * 2] = m_run, p.ws_ml[slot * 2 + 1] = l_tot;
-      float* dst = p.ws_o + slot * D + 16 * g;
+      // (register a of matrix op e is row d = 8 (4g + a) + e of O^T)
+      float* dst = p.ws_o + slot * D + 32 * g;
 #pragma unroll
-      for (int i = 0; i < 8; ++i)
+      for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) dst[(i >> 2) * 64 + 4 * e + (i & 3)] = oacc[i][e] * vscale;
+        for (int e4 = 0; e4 < 2; ++e4)
+          *(f32x4*)(dst + 8 * a + 4 * e4) = f32x4{oacc[4 * e4][a], oacc[4 * e4 + 1][a], oacc[4 * e4 + 2][a], oacc[4 * e4 + 3][a]} * vscale;
     }
     if (!more) break;
     G = g_next;
