@@ -281,6 +281,87 @@ def sdpa_backward(
 
 
 # --------------------------------------------------------------------------------------
+# Mask / score functors: sliding window, sink keys, sink logit.  The reference takes
+# ``sliding_window`` and ``sink`` as arguments of its templated kernel
+# (torch_neuronx/neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:94-117; the sink
+# joins the row maximum :1921-1923 and the exponential sum :2134-2140), but the rendered mask
+# function is not in the tree, so the window's boundary convention here is this build's:
+# a window of ``window`` keys that ends at the query's own position.  PARITY UNPINNED by the
+# reference's tests; pinned by float64 ``F.scaled_dot_product_attention`` on the explicit mask
+# with the sink as one more key of value zero (tests/test_oracle.py).
+# --------------------------------------------------------------------------------------
+
+
+def window_keep_mask(L: int, S: int, window: int, sink_keys: int = 0) -> torch.Tensor:
+    """Boolean ``(L, S)`` keep-mask: causal (top-left), and key ``j`` within the last
+    ``window`` positions of query ``i`` or among the first ``sink_keys`` keys."""
+    row = torch.arange(L).unsqueeze(-1)
+    col = torch.arange(S).unsqueeze(0)
+    keep = col <= row
+    if window and window > 0:
+        keep = keep & ((row - col < window) | (col < sink_keys))
+    return keep
+
+
+def _with_sink(query, key, value, bias, sink_logit):
+    """The sink as one more key: zero key and value rows and a bias column holding the logit."""
+    B, Hq, L, _ = query.shape
+    S = key.shape[2]
+    z = sink_logit.to(torch.float32).reshape(-1, Hq).expand(B, Hq)
+    key = torch.cat([key, key.new_zeros(key.shape[0], key.shape[1], 1, key.shape[3])], dim=2)
+    value = torch.cat([value, value.new_zeros(value.shape[0], value.shape[1], 1, value.shape[3])], dim=2)
+    full = torch.zeros(B, Hq, L, S + 1, dtype=torch.float32)
+    if bias is not None:
+        full[..., :S] = bias
+    full[..., S] = z[:, :, None]
+    return key, value, full
+
+
+def sdpa_forward_functor(query, key, value, is_causal=False, scale=None, window=0, sink_keys=0, sink_logit=None):
+    """Forward with the mask functors; K/V at ``Hkv`` heads.  Returns ``(out, lse)``."""
+    B, Hq, L, E = query.shape
+    S = key.shape[2]
+    rep = Hq // key.shape[1]
+    if scale is None:
+        scale = 1.0 / math.sqrt(E)
+    k = key.repeat_interleave(rep, dim=1)
+    v = value.repeat_interleave(rep, dim=1)
+    bias = None
+    if is_causal or window:
+        keep = window_keep_mask(L, S, window, sink_keys) if window else (torch.arange(S)[None] <= torch.arange(L)[:, None])
+        bias = torch.zeros(L, S, dtype=torch.float32).masked_fill(~keep, NEG_INF)
+    if sink_logit is not None:
+        k, v, bias = _with_sink(query, k, v, bias, sink_logit)
+    return compute_attention(query, k, v, bias, None, scale, False, 0.0)
+
+
+def sdpa_backward_functor(grad_out, query, key, value, out, lse, is_causal=False, scale=None, window=0,
+                          sink_keys=0, sink_logit=None):
+    """Backward with the mask functors: ``(dq, dk, dv, dsink-or-None)`` in float32, dk/dv at ``Hkv`` heads."""
+    B, Hq, L, E = query.shape
+    Hkv, S = key.shape[1], key.shape[2]
+    rep = Hq // Hkv
+    if scale is None:
+        scale = 1.0 / math.sqrt(E)
+    k = key.float().repeat_interleave(rep, dim=1)
+    v = value.float().repeat_interleave(rep, dim=1)
+    bias = None
+    if is_causal or window:
+        keep = window_keep_mask(L, S, window, sink_keys) if window else (torch.arange(S)[None] <= torch.arange(L)[:, None])
+        bias = torch.zeros(1, 1, L, S, dtype=torch.float32).masked_fill(~keep, NEG_INF).expand(B, Hq, L, S)
+    if sink_logit is not None:
+        k, v, bias = _with_sink(query, k, v, None if bias is None else bias, sink_logit)
+    gq, gk, gv, gb = compute_attention_backward(grad_out.float(), query.float(), k, v, bias, None, out.float(), lse,
+                                                scale, False, 0.0, bias_present=bias is not None)
+    dsink = None
+    if sink_logit is not None:
+        dsink = gb[..., S].sum(-1)
+        gk, gv = gk[:, :, :S], gv[:, :, :S]
+    gk, gv = reduce_gqa_gradients(gk, gv, Hkv)
+    return gq, gk, gv, dsink
+
+
+# --------------------------------------------------------------------------------------
 # fp8 key/value cache decode.  No reference counterpart: PARITY UNPINNED (see header).
 # --------------------------------------------------------------------------------------
 

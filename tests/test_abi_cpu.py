@@ -38,7 +38,7 @@ def test_library_exports_every_declared_symbol(amd):
     for n in names:
         assert hasattr(lib, n), n
     assert set(names) == set(amd._lib.EXPORTS)
-    assert lib.mi355_sdpa_abi_version() == 1
+    assert lib.mi355_sdpa_abi_version() == 2
 
 
 def test_ctypes_structs_match_c_layout(amd, tmp_path):
@@ -50,6 +50,8 @@ def test_ctypes_structs_match_c_layout(amd, tmp_path):
         " sizeof(mi355_sdpa_fwd_params), sizeof(mi355_sdpa_bwd_params), sizeof(mi355_sdpa_decode_params));\n"
         'printf("%zu %zu %zu %zu\\n", offsetof(mi355_sdpa_fwd_params, scale), offsetof(mi355_sdpa_bwd_params, workspace),'
         " offsetof(mi355_sdpa_decode_params, workspace), offsetof(mi355_sdpa_desc, q_last_stride));\n"
+        'printf("%zu %zu %zu %zu\\n", sizeof(mi355_sdpa_mask_spec), offsetof(mi355_sdpa_fwd_params, mask),'
+        " offsetof(mi355_sdpa_bwd_params, mask), offsetof(mi355_sdpa_bwd_params, grad_sink_logit));\n"
         "return 0;}\n"
     )
     exe = tmp_path / "sizes"
@@ -58,7 +60,8 @@ def test_ctypes_structs_match_c_layout(amd, tmp_path):
     L = amd._lib
     got = [C.sizeof(L.Tensor4), C.sizeof(L.Desc), C.sizeof(L.FwdParams), C.sizeof(L.BwdParams), C.sizeof(L.DecodeParams),
            L.FwdParams.scale.offset, L.BwdParams.workspace.offset, L.DecodeParams.workspace.offset,
-           L.Desc.q_last_stride.offset]
+           L.Desc.q_last_stride.offset,
+           C.sizeof(L.MaskSpec), L.FwdParams.mask.offset, L.BwdParams.mask.offset, L.BwdParams.grad_sink_logit.offset]
     assert [int(x) for x in out] == got
 
 

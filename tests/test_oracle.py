@@ -330,3 +330,68 @@ def test_decode_empty_sequence_matches_fully_masked_rows():
     assert torch.equal(out[0], torch.zeros_like(out[0])) and torch.isinf(lse[0]).all() and (lse[0] < 0).all()
     torch.testing.assert_close(o2, out, rtol=1e-5, atol=1e-6)
     torch.testing.assert_close(l2, lse, rtol=1e-5, atol=1e-6)
+
+
+# ---- mask functors (sliding window, sink keys, sink logit) ------------------------------------------
+
+
+def _functor_reference(q, k, v, window, sink_keys, sink_logit, scale):
+    """float64 library routine on the explicit mask; the sink is one more key with a zero value
+    whose logit arrives through the bias."""
+    B, Hq, L, E = q.shape
+    S = k.shape[2]
+    rep = Hq // k.shape[1]
+    q64 = q.double().requires_grad_(True)
+    k64 = k.double().requires_grad_(True)
+    v64 = v.double().requires_grad_(True)
+    ke, ve = k64.repeat_interleave(rep, 1), v64.repeat_interleave(rep, 1)
+    row, col = torch.arange(L)[:, None], torch.arange(S)[None]
+    keep = col <= row
+    if window:
+        keep = keep & ((row - col < window) | (col < sink_keys))
+    bias = torch.zeros(B, Hq, L, S, dtype=torch.float64).masked_fill(~keep, float("-inf"))
+    z = None
+    if sink_logit is not None:
+        z = sink_logit.double().reshape(-1, Hq).expand(B, Hq).clone().requires_grad_(True)
+        ke = torch.cat([ke, torch.zeros(B, Hq, 1, E, dtype=torch.float64)], 2)
+        ve = torch.cat([ve, torch.zeros(B, Hq, 1, v.shape[3], dtype=torch.float64)], 2)
+        bias = torch.cat([bias, z[:, :, None, None].expand(B, Hq, L, 1)], 3)
+    out = F.scaled_dot_product_attention(q64, ke, ve, attn_mask=bias, scale=scale)
+    logits = torch.matmul(q64, ke.transpose(-1, -2)) * scale + bias
+    return out, torch.logsumexp(logits, -1), (q64, k64, v64, z)
+
+
+@pytest.mark.parametrize("window,sink_keys,with_sink", [(5, 0, False), (7, 3, False), (0, 0, True), (4, 2, True), (64, 0, True)])
+def test_functor_oracle_matches_float64_library(window, sink_keys, with_sink):
+    g = torch.Generator().manual_seed(window * 7 + sink_keys)
+    B, Hq, Hkv, L, S, E = 2, 4, 2, 19, 19, 16
+    q, k, v, go = (torch.randn(s_, generator=g) for s_ in ((B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, E), (B, Hq, L, E)))
+    z = torch.randn(B, Hq, generator=g) * 2 if with_sink else None
+    scale = 0.3
+    out, lse = om.sdpa_forward_functor(q, k, v, is_causal=True, scale=scale, window=window, sink_keys=sink_keys, sink_logit=z)
+    ro, rl, (q64, k64, v64, z64) = _functor_reference(q, k, v, window, sink_keys, z, scale)
+    assert (out.double() - ro).abs().max() < 1e-5 and (lse.double() - rl).abs().max() < 1e-5
+    dq, dk, dv, dz = om.sdpa_backward_functor(go, q, k, v, out, lse, is_causal=True, scale=scale, window=window,
+                                              sink_keys=sink_keys, sink_logit=z)
+    leaves = [q64, k64, v64] + ([z64] if with_sink else [])
+    grads = torch.autograd.grad(ro, leaves, go.double())
+    for a, r in zip((dq, dk, dv), grads[:3]):
+        assert a.shape == r.shape and (a.double() - r).abs().max() < 1e-4
+    if with_sink:
+        assert (dz.double() - grads[3]).abs().max() < 1e-4
+    else:
+        assert dz is None
+
+
+def test_window_mask_closed_forms():
+    # a window at least as long as the sequence is the causal mask; window 1 keeps the diagonal;
+    # row i keeps min(i + 1, window) keys plus the sink keys that the window does not already hold
+    L = S = 11
+    causal = torch.tril(torch.ones(L, S, dtype=torch.bool))
+    assert torch.equal(om.window_keep_mask(L, S, 11), causal) and torch.equal(om.window_keep_mask(L, S, 0), causal)
+    assert torch.equal(om.window_keep_mask(L, S, 1), torch.eye(L, dtype=torch.bool))
+    m = om.window_keep_mask(L, S, 3, 2)
+    for i in range(L):
+        want = {j for j in range(S) if j <= i and (i - j < 3 or j < 2)}
+        assert {j for j in range(S) if m[i, j]} == want
+    assert om.window_keep_mask(5, 9, 2).sum() == 1 + 2 * 4  # L != S: anchored top-left

@@ -79,6 +79,13 @@ static bool shapes_ok(const mi355_sdpa_tensor& q, const mi355_sdpa_tensor& k,
   return true;
 }
 
+static bool mask_spec_ok(const mi355_sdpa_mask_spec& m, int is_causal) {
+  if (m.window < 0 || m.sink_keys < 0) return set_error("SDPA: window and sink_keys must not be negative"), false;
+  if (m.window > 0 && !is_causal) return set_error("SDPA: a sliding window needs is_causal"), false;
+  if (m.sink_keys > 0 && m.window == 0) return set_error("SDPA: sink_keys needs a sliding window"), false;
+  return true;
+}
+
 static bool same_shape(const mi355_sdpa_tensor& t, int64_t a, int64_t b, int64_t c, int64_t d) {
   return t.size[0] == a && t.size[1] == b && t.size[2] == c && t.size[3] == d;
 }
@@ -258,6 +265,7 @@ int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
            MI355_SDPA_ERR_INVALID;
   if (p->dropout_p > 0.f && !p->dropout_keep)
     return set_error("SDPA: dropout_p > 0 needs a keep mask"), MI355_SDPA_ERR_INVALID;
+  if (!mask_spec_ok(p->mask, p->is_causal)) return MI355_SDPA_ERR_INVALID;
   hipStream_t s = (hipStream_t)stream;
   const char* why = "";
   int kernel = p->force_kernel;
@@ -291,6 +299,9 @@ static bool bwd_args_ok(const mi355_sdpa_bwd_params* p) {
   if (p->dropout_p < 0.f || p->dropout_p > 1.f)
     return set_error("dropout_p=%g is outside [0, 1]. Pass a value in [0, 1].", (double)p->dropout_p), false;
   if (p->dropout_p > 0.f && !p->dropout_keep) return set_error("SDPA: dropout_p > 0 needs a keep mask"), false;
+  if (!mask_spec_ok(p->mask, p->is_causal)) return false;
+  if (p->grad_sink_logit && !p->mask.sink_logit)
+    return set_error("SDPA: grad_sink_logit without a sink_logit"), false;
   return true;
 }
 

@@ -29,6 +29,7 @@ struct BwdG {
   int B, Hq, Hkv, L, S, E, Dv;
   int causal, bias_kind;
   float scale;
+  int window, sink_keys;  // sliding window over the causal pattern: keys i-window+1 .. i and the first sink_keys
 };
 
 template <typename TB>
@@ -101,7 +102,8 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_row_kernel(BwdG p) {
       for (int e = 0; e < p.E; ++e) dot = fmaf(qrow[wave][e], to_f32(kr[e * p.k.st[3]]), dot);
       for (int d = 0; d < p.Dv; ++d) dp = fmaf(dorow[wave][d], to_f32(vr[d * p.v.st[3]]), dp);
       const float s = apply_bias<TB>(dot * p.scale, bias_row, j * p.bias.st[3], p.bias_kind);
-      const float pr = expf(s - lse);
+      float pr = expf(s - lse);
+      if (p.window > 0 && i - j >= p.window && j >= p.sink_keys) pr = 0.f;
       if (keep_row) dp = keep_row[j] ? dp * p.keep_scale : 0.f;
       dlog = pr * (dp - delta);
     }
@@ -168,7 +170,7 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_col_kernel(BwdG p) {
       for (int i0 = i_begin; i0 < p.L; i0 += 64) {
         const int i = i0 + lane;
         float pr = 0.f, ds = 0.f;
-        if (i < p.L && (!p.causal || j <= i)) {
+        if (i < p.L && (!p.causal || j <= i) && (p.window <= 0 || i - j < p.window || j < p.sink_keys)) {
           const float l = lse[i];
           if (l != -INFINITY) {
             const T* qr = qbase + i * p.q.st[2];
@@ -216,6 +218,27 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_col_kernel(BwdG p) {
   }
 }
 
+// Gradient of the sink logit z of one (batch, head): the sink's probability in row i is
+// exp(z - lse_i) and its dP is 0 (it carries no value), so d z = - sum_i exp(z - lse_i) delta_i.
+// One workgroup per (batch, head), summed in a fixed order.
+__global__ __launch_bounds__(256) void sink_grad_kernel(const float* lse, const float* delta, const float* z, float* out, int L) {
+  __shared__ float part[256];
+  const int bh = blockIdx.x;
+  const float zz = z[bh];
+  float s = 0.f;
+  for (int i = threadIdx.x; i < L; i += 256) {
+    const float l = lse[(int64_t)bh * L + i];
+    if (l != -INFINITY && zz != -INFINITY) s -= expf(zz - l) * delta[(int64_t)bh * L + i];
+  }
+  part[threadIdx.x] = s;
+  __syncthreads();
+  for (int o = 128; o > 0; o >>= 1) {
+    if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
+    __syncthreads();
+  }
+  if (threadIdx.x == 0) out[bh] = part[0];
+}
+
 template <typename T, typename TB>
 int launch_tb(const BwdG& g, hipStream_t s) {
   const int64_t qrows = (int64_t)g.B * g.Hq * g.L, krows = (int64_t)g.B * g.Hkv * g.S;
@@ -244,6 +267,13 @@ int launch_t(const BwdG& g, int bias_dtype, hipStream_t s) {
 
 }  // namespace
 
+int launch_sink_grad(const float* lse, const float* delta, const float* sink_logit, float* grad, int64_t heads, int L,
+                     hipStream_t s) {
+  if (heads == 0) return MI355_SDPA_OK;
+  hipLaunchKernelGGL(sink_grad_kernel, dim3((unsigned)heads), dim3(256), 0, s, lse, delta, sink_logit, grad, L);
+  return check_launch("sink_grad_kernel");
+}
+
 size_t bwd_generic_workspace(const mi355_sdpa_bwd_params& p) {
   return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * sizeof(float);
 }
@@ -260,17 +290,23 @@ int launch_bwd_generic(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.Hkv = (int)p.k.size[1], g.S = (int)p.k.size[2], g.Dv = (int)p.v.size[3];
   g.causal = p.is_causal, g.scale = p.scale;
   g.bias_kind = !p.bias.data ? 0 : (p.bias_dtype == MI355_SDPA_BOOL ? 2 : 1);
+  g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
   if (g.E > kMaxHeadDim || g.Dv > kMaxHeadDim) {
     set_error("SDPA: head dim %d/%d exceeds the supported maximum %d", g.E, g.Dv, kMaxHeadDim);
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
+  int rc;
   switch (p.dtype) {
-    case MI355_SDPA_F32: return launch_t<float>(g, p.bias_dtype, s);
-    case MI355_SDPA_F16: return launch_t<f16_t>(g, p.bias_dtype, s);
-    case MI355_SDPA_BF16: return launch_t<bf16_t>(g, p.bias_dtype, s);
+    case MI355_SDPA_F32: rc = launch_t<float>(g, p.bias_dtype, s); break;
+    case MI355_SDPA_F16: rc = launch_t<f16_t>(g, p.bias_dtype, s); break;
+    case MI355_SDPA_BF16: rc = launch_t<bf16_t>(g, p.bias_dtype, s); break;
+    default:
+      set_error("SDPA: query dtype must be float32, float16, or bfloat16, got dtype id %d", p.dtype);
+      return MI355_SDPA_ERR_INVALID;
   }
-  set_error("SDPA: query dtype must be float32, float16, or bfloat16, got dtype id %d", p.dtype);
-  return MI355_SDPA_ERR_INVALID;
+  if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
+    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
+  return rc;
 }
 
 }  // namespace mi355

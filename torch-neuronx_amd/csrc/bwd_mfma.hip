@@ -576,6 +576,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   if (p.dropout_p > 0.f) return *why = "dropout", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
+  if (p.mask.window > 0) return *why = "window functor", false;
   const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
   for (const mi355_sdpa_tensor* t : ts) {
     if (t->stride[3] != 1) return *why = "head dim is not unit-stride", false;
@@ -606,8 +607,14 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   BwdM g;
   fill(g, p);
   const int D = p.q.size[3] <= 64 ? 64 : 128;  // the kernels' width
-  if (p.dtype == MI355_SDPA_BF16) return D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
-  return D == 128 ? launch_td<f16_t, 128>(g, s) : launch_td<f16_t, 64>(g, s);
+  int rc;
+  if (p.dtype == MI355_SDPA_BF16) rc = D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
+  else rc = D == 128 ? launch_td<f16_t, 128>(g, s) : launch_td<f16_t, 64>(g, s);
+  // (a sink logit changes nothing in these kernels: the probabilities come from the saved
+  // log-sum-exp, which includes it; only its own gradient is one more small reduction)
+  if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
+    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
+  return rc;
 }
 
 }  // namespace mi355

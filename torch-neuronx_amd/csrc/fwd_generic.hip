@@ -25,6 +25,8 @@ struct FwdG {
   int B, Hq, Hkv, L, S, E, Dv;
   int causal, bias_kind;  // 0 none, 1 additive, 2 bool
   float scale;
+  int window, sink_keys;    // sliding window over the causal pattern: keys i-window+1 .. i and the first sink_keys
+  const float* sink_logit;  // (B,Hq): a logit without a value that joins every row's softmax
 };
 
 template <typename T, typename TB>
@@ -71,6 +73,7 @@ __global__ __launch_bounds__(64 * kWaves) void fwd_generic_kernel(FwdG p) {
       float dot = 0.f;
       for (int e = 0; e < p.E; ++e) dot = fmaf(qrow[wave][e], to_f32(kr[e * p.k.st[3]]), dot);
       s = dot * p.scale;
+      if (p.window > 0 && i - j >= p.window && j >= p.sink_keys) s = -INFINITY;
       if (p.bias_kind == 1) {
         s += to_f32(bias_row[j * p.bias.st[3]]);
       } else if (p.bias_kind == 2) {
@@ -101,6 +104,17 @@ __global__ __launch_bounds__(64 * kWaves) void fwd_generic_kernel(FwdG p) {
     }
   }
 
+  if (p.sink_logit) {
+    const float z = p.sink_logit[(int64_t)b * p.Hq + h];
+    if (z != -INFINITY) {
+      const float m2 = fmaxf(m, z);
+      const float a = m == -INFINITY ? 0.f : expf(m - m2);
+      l = l * a + expf(z - m2);
+      m = m2;
+#pragma unroll
+      for (int c = 0; c < NV; ++c) acc[c] *= a;
+    }
+  }
   const float inv = l > 0.f ? 1.f / l : 0.f;
   T* o = (T*)p.out.data + b * p.out.st[0] + h * p.out.st[1] + i * p.out.st[2];
 #pragma unroll
@@ -141,6 +155,7 @@ int launch_fwd_generic(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.Hkv = (int)p.k.size[1], g.S = (int)p.k.size[2], g.Dv = (int)p.v.size[3];
   g.causal = p.is_causal, g.scale = p.scale;
   g.bias_kind = !p.bias.data ? 0 : (p.bias_dtype == MI355_SDPA_BOOL ? 2 : 1);
+  g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
   if (g.E > kMaxHeadDim || g.Dv > kMaxHeadDim) {
     set_error("SDPA: head dim %d/%d exceeds the supported maximum %d", g.E, g.Dv, kMaxHeadDim);
     return MI355_SDPA_ERR_UNSUPPORTED;

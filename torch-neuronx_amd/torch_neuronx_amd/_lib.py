@@ -45,13 +45,17 @@ class Desc(C.Structure):
     ]
 
 
+class MaskSpec(C.Structure):
+    _fields_ = [("window", C.c_int32), ("sink_keys", C.c_int32), ("sink_logit", C.c_void_p)]
+
+
 class FwdParams(C.Structure):
     _fields_ = [
         ("q", Tensor4), ("k", Tensor4), ("v", Tensor4), ("out", Tensor4),
         ("lse", C.c_void_p), ("bias", Tensor4), ("bias_dtype", C.c_int32),
         ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
         ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
-        ("force_kernel", C.c_int32),
+        ("force_kernel", C.c_int32), ("mask", MaskSpec),
     ]
 
 
@@ -63,6 +67,7 @@ class BwdParams(C.Structure):
         ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
         ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("force_kernel", C.c_int32),
+        ("mask", MaskSpec), ("grad_sink_logit", C.c_void_p),
     ]
 
 

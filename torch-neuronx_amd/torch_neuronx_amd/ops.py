@@ -100,10 +100,30 @@ def _bias_view(attn_bias, B, Hq, L, S):
     return b, _lib.dtype_id(b.dtype)
 
 
+def _mask_spec(spec, query, window, sink_keys, sink_logit):
+    """Fill the functor part of a parameter block; returns the tensors that must stay alive."""
+    spec.window = int(window or 0)
+    spec.sink_keys = int(sink_keys or 0)
+    if sink_logit is None:
+        return None
+    B, Hq = query.shape[0], query.shape[1]
+    z = sink_logit.to(device=query.device, dtype=torch.float32)
+    if z.numel() == Hq:
+        z = z.reshape(1, Hq)
+    z = z.reshape(-1, Hq).expand(B, Hq).contiguous()
+    spec.sink_logit = z.data_ptr()
+    return z
+
+
 def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None, dropout_p=0.0,
-                 dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0):
+                 dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0,
+                 window=None, sink_keys=0, sink_logit=None):
     """Fused forward.  K/V arrive at ``Hkv`` heads.  Returns ``(out, lse)``; ``out`` keeps the
-    dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``."""
+    dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``.
+
+    ``window`` (with ``is_causal``): query ``i`` sees keys ``i-window+1 .. i`` and the first
+    ``sink_keys`` keys; ``sink_logit`` ``(B,Hq)`` or ``(Hq,)``: one more logit per row that joins
+    the softmax and carries no value."""
     for t, n in ((query, "query"), (key, "key"), (value, "value")):
         _require_cuda(t, n)
     B, Hq, L, E = query.shape
@@ -131,6 +151,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
+    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit)  # noqa: F841 (kept alive over the launch)
     with _lib.on_device(query.device):
         rc = _lib.load().mi355_sdpa_fwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
@@ -139,9 +160,10 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
 
 def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_causal=False,
                   scale=None, dropout_p=0.0, dropout_keep=None, kv_lens=None,
-                  want_grad_bias=False, force_kernel=0):
+                  want_grad_bias=False, force_kernel=0, window=None, sink_keys=0, sink_logit=None):
     """Fused backward.  Returns ``(dq, dk, dv, dbias-or-None)``; each gradient keeps the
-    dimension order of its input, dk/dv come back at ``Hkv`` heads."""
+    dimension order of its input, dk/dv come back at ``Hkv`` heads.  With a ``sink_logit`` a
+    fifth element follows: its gradient, float32 ``(B,Hq)``."""
     for t, n in ((grad_out, "grad_out"), (query, "query"), (key, "key"), (value, "value")):
         _require_cuda(t, n)
     B, Hq, L, E = query.shape
@@ -178,6 +200,11 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
+    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit)
+    dsink = None
+    if _z is not None:
+        dsink = torch.empty((B, Hq), dtype=torch.float32, device=query.device)
+        p.grad_sink_logit = dsink.data_ptr()
     lib = _lib.load()
     nbytes = lib.mi355_sdpa_bwd_workspace_bytes(C.byref(p))
     ws = torch.empty((max(nbytes, 1),), dtype=torch.uint8, device=query.device)
@@ -185,6 +212,8 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     with _lib.on_device(query.device):
         rc = lib.mi355_sdpa_bwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
+    if _z is not None:
+        return dq, dk, dv, dbias, dsink
     return dq, dk, dv, dbias
 
 
