@@ -29,6 +29,11 @@ struct FwdM {
   // (head dims 8 .. 56 in the 64 kernel, 72 .. 120 in the 128 kernel); 0 means the full width.
   // dv_real: the same for V and the output, which may be narrower than Q and K (192 / 128).
   int d_real = 0, dv_real = 0;
+  // mask functors (masked variant without a bias only): with window > 0 (causal calls) query i sees
+  // keys i-window+1 .. i and the first sink_keys keys; sink_logit (B, Hq) is one more logit per row
+  // that joins the softmax and carries no value
+  int window = 0, sink_keys = 0;
+  const float* sink_logit = nullptr;
 };
 
 // Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first

@@ -338,7 +338,7 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const bool w32_only = padded || E > 128;
   // masked calls (bias, bool keep-mask, per-batch key counts) and padded head dims: the kernels
   // with 32-bit row addressing only, and a bias whose rows can be read four keys at a time
-  if (p.bias.data || p.kv_lens || w32_only) {
+  if (p.bias.data || p.kv_lens || w32_only || p.mask.window > 0 || p.mask.sink_logit) {
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
       return *why = "attn_bias / kv_lens / padded head dim with rows beyond 32-bit offsets", false;
   }
@@ -358,7 +358,8 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   if (p.dropout_p > 0.f) return *why = "dropout", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
-  if (p.mask.window > 0 || p.mask.sink_logit) return *why = "window / sink functor", false;
+  if ((p.mask.window > 0 || p.mask.sink_logit) && (p.bias.data || E > 128))
+    return *why = "window / sink functor together with attn_bias or a head dim above 128", false;
   if (p.q.stride[3] != 1 || p.k.stride[3] != 1 || p.v.stride[3] != 1 || p.out.stride[3] != 1)
     return *why = "head dim is not unit-stride", false;
   const mi355_sdpa_tensor* ts[4] = {&p.q, &p.k, &p.v, &p.out};
@@ -393,6 +394,7 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
   }
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
+  g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
   const int D = g.d_real <= 64 ? 64 : g.d_real <= 128 ? 128 : 256;  // the kernel's width
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
@@ -404,7 +406,9 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   // 128-row workgroups always (measured crossovers on MI355X).
   if ((int64_t)g.S * g.k_sl * 2 < (1ll << 31) && (int64_t)g.S * g.v_sl * 2 < (1ll << 31)) {
     const bool big = D == 128 && ((g.S >= 2048 && wg256 >= (g.causal ? 512 : 256)) || (!g.causal && g.S >= 1024 && wg256 >= 512));
-    const int rows = D == 256 ? 128 : force_tile ? force_tile : big ? 256 : 128;
+    // (a short window: the keys a workgroup walks are window + rows, so smaller workgroups waste less)
+    const bool short_window = g.window > 0 && g.window <= 512;
+    const int rows = D == 256 ? 128 : force_tile ? force_tile : (big && !short_window) ? 256 : 128;
     return launch_fwd_mfma_w32(g, p.dtype, D, rows / 32, s);
   }
   // strides beyond 32-bit offsets: the kernel above (64-bit addressing)

@@ -64,6 +64,8 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // Unmasked calls at head dim 64 / 128 stage their tiles from global memory straight into LDS
   // (see the staging section): four unpadded, swizzled buffers per operand, tile t in buffer t % 4.
   constexpr bool DMA = MASK != 2;
+  // mask functors (window, sink keys, sink logit): in the masked variant without a bias, head dim <= 128
+  constexpr bool FUNC = MASK == 1 && D <= 128;
   constexpr int NBUF = 4, TILE = BN * D;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * KROW];
   __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * VP];
@@ -106,13 +108,31 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
         S = min(S, __builtin_amdgcn_readfirstlane(last) + 1);
       }
     }
-    if (S == 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87)
+  }
+  // The key tiles this workgroup walks.  Without a window: 0 .. nt-1.  With one, the tiles below the
+  // lowest window of its rows are dropped whole, except the leading ones that hold sink keys: stream
+  // position u is key tile u + (u >= n_lead ? skip : 0).
+  int nt = (S + BN - 1) / BN;
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+  int n_lead = 0, skip = 0;
+  if constexpr (FUNC) {
+    if (p.window > 0) {
+      const int t_lo = max(q0 - p.window + 1, 0) / BN;
+      n_lead = min(min((p.sink_keys + BN - 1) / BN, t_lo), nt);
+      skip = min(t_lo, nt) - n_lead;
+      nt -= skip;
+    }
+  }
+  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  if constexpr (MASK) {
+    if (nt <= 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87), or the sink logit alone
       if (qrow < p.L) {
         uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
         for (int i = 0; i < D / 16; ++i)
           if (half * (D / 2) + i * 8 < drv) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
-        if (p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = -INFINITY;
+        if (p.lse && half == 0)
+          p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = (FUNC && p.sink_logit) ? p.sink_logit[(int64_t)b * p.Hq + h] : -INFINITY;
       }
       return;
     }
@@ -138,9 +158,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   }
 
-  int nt = (S + BN - 1) / BN;
-  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
-  const int nt_w = p.causal ? min(nt, qw_last / BN + 1) : nt;
+  const int nt_w = p.causal ? min(nt, qw_last / BN + 1 - skip) : nt;
 
   // ---- staging: every thread moves KLD 16-byte chunks of the K tile and of the V tile ------------
   // Both tiles sit in LDS as they sit in memory, [key][d].  K is the A operand of S^T = K Q^T as it
@@ -178,14 +196,14 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   }
   const int k_tile_bytes = (int)(BN * p.k_sl * 2), v_tile_bytes = (int)(BN * p.v_sl * 2);
   auto load_k = [&](int set, int t) {
-    const uint32_t base = (uint32_t)(min(t, nt - 1) * k_tile_bytes);
+    const uint32_t base = (uint32_t)(tile_of(min(t, nt - 1)) * k_tile_bytes);
     if (do_k) {
 #pragma unroll
       for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i] + base, 0, 0);
     }
   };
   auto load_v = [&](int set, int t) {
-    const uint32_t base = (uint32_t)(min(t, nt - 1) * v_tile_bytes);
+    const uint32_t base = (uint32_t)(tile_of(min(t, nt - 1)) * v_tile_bytes);
     if (do_v) {
 #pragma unroll
       for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i] + base, 0, 0);
@@ -252,7 +270,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   };
   auto request_k = [&](int t) {  // K tile t (the last one again past the end) into buffer t % 4
     if constexpr (DMA) {
-      const uint32_t g = (uint32_t)(min(t, nt - 1) * k_tile_bytes), l = lds_kd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+      const uint32_t g = (uint32_t)(tile_of(min(t, nt - 1)) * k_tile_bytes), l = lds_kd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
       if (dma_k) {
 #pragma unroll
         for (int i = 0; i < NL; ++i) tile_load(kd_rsrc, kd_off[i] + g, l + i * WAVES * 1024);
@@ -261,7 +279,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   };
   auto request_v = [&](int t) {
     if constexpr (DMA) {
-      const uint32_t g = (uint32_t)(min(t, nt - 1) * v_tile_bytes), l = lds_vd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+      const uint32_t g = (uint32_t)(tile_of(min(t, nt - 1)) * v_tile_bytes), l = lds_vd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
       if (dma_v) {
 #pragma unroll
         for (int i = 0; i < NL; ++i) tile_load(vd_rsrc, vd_off[i] + g, l + i * WAVES * 1024);
@@ -313,12 +331,15 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  // (window: keys below lo_w are dropped unless they are sink keys)
+  const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
+  const int n_sink = FUNC ? p.sink_keys : 0;
 
   auto mask_tile = [&](f32x16& s, int kv0) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kv = kv0 + (r >> 2) * 8 + half * 4 + (r & 3);
-      if (kv > lim) s[r] = -INFINITY;
+      if (kv > lim || (FUNC && kv < lo_w && kv >= n_sink)) s[r] = -INFINITY;
     }
   };
   // Bias of the score tile: lane = query row, 4 groups of 4 consecutive keys.  The resource starts
@@ -391,6 +412,16 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile
   const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
+  // ... or, with a window, a tile that reaches below the window of this wavefront's last row and
+  // is not made of sink keys alone.  (Stream position -> does the tile need masking.)
+  auto edge = [&](int u) {
+    const int ta = tile_of(u);
+    bool e = ta >= t_edge;
+    if constexpr (FUNC) {
+      if (p.window > 0) e |= ta * BN < qw_last - p.window + 1 && ta * BN + BN > n_sink;
+    }
+    return e;
+  };
 
   float m_new = -INFINITY, mc = 0.f, alpha = 1.f;
   bool need_rescale = false;
@@ -482,7 +513,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
     apply_bias(s_a);
     load_bias(1);
-    if (t_edge == 0) mask_tile(s_a, 0);
+    if (edge(0)) mask_tile(s_a, tile_of(0) * BN);
     raise_reference(tile_max(s_a));  // the first reference is the maximum of the first tile
     m_run = m_new;
 #pragma unroll
@@ -599,7 +630,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       if (i == 0) {
         apply_bias(snext);
         load_bias(t + 2);
-        if (__builtin_expect(t + 1 >= t_edge, 0)) mask_tile(snext, (t + 1) * BN);  // rare
+        if (__builtin_expect(edge(t + 1), 0)) mask_tile(snext, tile_of(t + 1) * BN);  // rare
         stage1(snext, 0);
       }
       // half-steps 0 .. 6 spread over the slots (the last one trails the loop)
@@ -664,7 +695,22 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 
   // ---- epilogue ------------------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  float lse_row = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+  if constexpr (FUNC) {
+    // the sink logit joins the row's maximum and sum (flex_attention.py.jinja:1921-1923, :2134-2140)
+    if (p.sink_logit) {
+      const float z = p.sink_logit[(int64_t)b * p.Hq + h];
+      if (z != -INFINITY) {
+        const float mn = l_tot > 0.f ? m_run * p.scale : -INFINITY;  // the reference, natural-log domain
+        const float mx = fmaxf(mn, z);
+        const float f = l_tot > 0.f ? __expf(mn - mx) : 0.f;
+        const float l2 = l_tot * f + __expf(z - mx);
+        inv = f / l2;
+        lse_row = mx + __builtin_logf(l2);
+      }
+    }
+  }
   if constexpr (DMA) {
     // A lane holds its query row in 8-byte pieces, 16 bytes apart: stored as they are, one
     // instruction writes 32 fragments of 16 bytes, and the stores of a workgroup's last tile,
@@ -692,8 +738,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       const u32x4 w = *(const u32x4*)(ot + r * D + ((cc ^ (r & SW)) << 3));
       if (qw0 + r < p.L && (!MASK || cc * 8 < drv)) *(u32x4*)(obase + (int64_t)(qw0 + r) * p.o_sl) = w;
     }
-    if (qrow < p.L && p.lse && half == 0)
-      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+    if (qrow < p.L && p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
   } else if (qrow < p.L) {
     uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
@@ -705,8 +750,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
         w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
         if (!MASK || db * 32 + g * 8 + half * 4 < drv) *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
       }
-    if (p.lse && half == 0)
-      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+    if (p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
   }
 }
 
@@ -757,7 +801,7 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
   }
   const dim3 grid((unsigned)blocks);
   // kernel variant: 2 with a bias or keep-mask, 1 with key counts or rows narrower than the kernel's head dim
-  const int mask = g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim) ? 1 : 0;
+  const int mask = g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit) ? 1 : 0;
   const int rc = dtype == MI355_SDPA_BF16 ? launch_dims<bf16_t>(g, head_dim, waves, mask, grid, s)
                                           : launch_dims<f16_t>(g, head_dim, waves, mask, grid, s);
   if (rc != MI355_SDPA_OK) return rc;
