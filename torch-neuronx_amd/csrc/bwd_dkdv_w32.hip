@@ -85,9 +85,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(frag[ks]));
   }
 
+  // sliding window (masked variant without a per-score bias): rows past the window of the block's last
+  // key see none of its keys, unless the block holds sink keys
+  constexpr bool FUNC = MASK == 1;
+  const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
   const int nqs = (p.L + BQ - 1) / BQ;
   const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
-  const int per_head = nqs - qs_begin;
+  const int qs_end = (W > 0 && k0 >= n_sink) ? max(min(nqs, (k0 + BK + W - 2) / BQ + 1), qs_begin) : nqs;
+  const int per_head = qs_end - qs_begin;
   const int n_items = (MASK && k0 >= S) ? 0 : rep * per_head;  // no live key in this tile: zeros
   auto item_head = [&](int it) { return hk * rep + it / per_head; };
   auto item_q0 = [&](int it) { return (qs_begin + it % per_head) * BQ; };
@@ -330,7 +335,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int qi = q0 + mq * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        if ((p.causal && key > qi) || key >= S) sc[mq][r] = -INFINITY;
+        if ((p.causal && key > qi) || key >= S || (W > 0 && qi - key >= W && key >= n_sink)) sc[mq][r] = -INFINITY;
       }
     };
     auto hand_over = [&](int mq) {
@@ -376,10 +381,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       __builtin_amdgcn_sched_barrier(0);
     }
   };
+  // every key of this block lies above the diagonal of the tile's rows / past the keys / below their windows
+  auto dead_tile = [&](int q0) {
+    return (p.causal && q0 + BQ - 1 < kw0) || kw0 >= S || (W > 0 && q0 - kw0 - 31 >= W && kw0 >= n_sink);
+  };
   auto role_a = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
-    if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;  // every key of this block lies above the diagonal / past the keys
-    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S);
+    if (dead_tile(q0)) return;
+    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
     role_a_tile(it, tb, pb, edge);
   };
   // Role B splits a tile over two iterations, so that its vector work falls on role A's first
@@ -387,7 +396,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // it, dS and dK of that tile at the start of iteration it + 1.
   f32x16 dp[2];
   auto role_b_scores = [&](int it, int tb) {
-    if ((p.causal && item_q0(it) + BQ - 1 < kw0) || kw0 >= S) return;
+    if (dead_tile(item_q0(it))) return;
     scores(do_t + tb * TILE, dp);
   };
   // One tile of role B, pipelined like role A's:
@@ -398,7 +407,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     constexpr int EPS = 16 / KS;  // elements per slot (2 or 4)
     constexpr int SPG = 4 / EPS;  // slots per group of four consecutive rows
     const int q0 = item_q0(it);
-    if ((p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
+    if (dead_tile(q0)) return;
     const uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;
     const uint16_t* qt = q_t + tb * TILE;
     const float* drow = &dl_s[tb * BQ + half * 4];
@@ -507,7 +516,7 @@ int launch_t(const BwdM& g, hipStream_t s) {
 template <typename T, int D>
 int launch_m(const BwdM& g, hipStream_t s) {
   if (g.bias_kind && g.bias_sl != 0) return launch_t<T, D, 2>(g, s);
-  return (g.bias_kind || g.kv_lens || g.d_real != D) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
+  return (g.bias_kind || g.kv_lens || g.d_real != D || g.window > 0) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
 }
 
 }  // namespace

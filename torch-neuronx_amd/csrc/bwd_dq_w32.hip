@@ -132,13 +132,38 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       return;
     }
   }
+  // The key tiles this workgroup walks.  Without a window: 0 .. nt-1.  With one, the tiles below the
+  // lowest window of its rows are dropped whole, except the leading ones that hold sink keys: stream
+  // position u is key tile u + (u >= n_lead ? skip : 0).
+  constexpr bool FUNC = MASK == 1;
   int nt = (S + BN - 1) / BN;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
-  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BN + 1) : nt;  // tiles with work for this wavefront
+  int n_lead = 0, skip = 0;
+  if constexpr (FUNC) {
+    if (p.window > 0) {
+      const int t_lo = max(q0 - p.window + 1, 0) / BN;
+      n_lead = min(min((p.sink_keys + BN - 1) / BN, t_lo), nt);
+      skip = min(t_lo, nt) - n_lead;
+      nt -= skip;
+    }
+  }
+  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BN + 1 - skip) : nt;  // tiles with work for this wavefront
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
-  // diagonal (qw0 is a multiple of BN), or a ragged last tile
+  // diagonal (qw0 is a multiple of BN), or a ragged last tile; with a window also every tile that
+  // reaches below the window of the wavefront's last row and is not made of sink keys alone
   const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
+  const int n_sink = FUNC ? p.sink_keys : 0;
+  auto edge_tile = [&](int u) {
+    const int ta = tile_of(u);
+    bool e = ta >= t_edge;
+    if constexpr (FUNC) {
+      if (p.window > 0) e |= ta * BN < qw0 + 31 - p.window + 1 && ta * BN + BN > n_sink;
+    }
+    return e;
+  };
 
   // ---- staging: K and V tiles go from global memory straight into LDS ---------------------------
   // (buffer loads with the LDS bit: no trip through registers, no LDS store instructions).  Such a
@@ -180,7 +205,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
                  :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   auto load_tile = [&](int t) {  // tile t (the last one again past the end) into buffer t % 4
-    const uint32_t tt = (uint32_t)min(t, nt - 1);
+    const uint32_t tt = (uint32_t)tile_of(min(t, nt - 1));
     const uint32_t boff = (uint32_t)((t & (NBUF - 1)) * TILE * 2);
     if (do_k) tile_load(k_rsrc, k_off + tt * k_tile_bytes, lds_k + boff);
     if (do_v) tile_load(v_rsrc, v_off + tt * v_tile_bytes, lds_v + boff);
@@ -376,11 +401,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
         // or the end of the keys gets the scores of its masked positions set to -inf first, in a
         // block of its own (tested per element, the test becomes selects that every tile pays for).
         // (For a wavefront's last tile the scores of the tile after it are computed and dropped.)
-        if (__builtin_expect(t >= t_edge, 0)) {
+        if (__builtin_expect(edge_tile(t), 0)) {
+          const int kv0 = tile_of(t) * BN;
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
-            const int kv = t * BN + (r >> 2) * 8 + half * 4 + (r & 3);
-            if (kv > lim) scur[r] = -INFINITY;
+            const int kv = kv0 + (r >> 2) * 8 + half * 4 + (r & 3);
+            if (kv > lim || (FUNC && kv < lo_w && kv >= n_sink)) scur[r] = -INFINITY;
           }
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -465,7 +491,7 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
   const bool bf = dtype == MI355_SDPA_BF16;
-  const int mask = (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim) ? 1 : 0;
+  const int mask = (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
 #define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, 0, s, g)
 #define LAUNCH_M(TT, DD)                                                     \
   do {                                                                       \

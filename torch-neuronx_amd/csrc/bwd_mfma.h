@@ -36,6 +36,9 @@ struct BwdM {
   // 1: the dQ kernel of bwd_dq_w32.hip computes delta and lse2 itself and writes them to the
   // workspace for the dK/dV kernel that follows it (bwd_delta_kernel is then not launched)
   int make_delta = 0;
+  // sliding window (causal calls, masked variants without a per-score bias): query i sees keys
+  // i-window+1 .. i and the first sink_keys keys; tiles that the window drops whole are skipped
+  int window = 0, sink_keys = 0;
 };
 
 // dot product of eight packed elements, float32 accumulation

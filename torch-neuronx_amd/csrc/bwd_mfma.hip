@@ -477,7 +477,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   constexpr int RPB = 256 / (D / 8);
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
+  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D || g.window > 0) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
   int rc;
   if (dq_w32) {
     // that kernel holds every row of dO in registers anyway: it goes first and leaves the row
@@ -530,6 +530,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
+  g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
   if (p.grad_bias.data) {
     g.gbias = p.grad_bias.data;
     g.gbias_sb = p.grad_bias.stride[0], g.gbias_sh = p.grad_bias.stride[1], g.gbias_sl = p.grad_bias.stride[2];
@@ -576,7 +577,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   if (p.dropout_p > 0.f) return *why = "dropout", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
-  if (p.mask.window > 0) return *why = "window functor", false;
+  if (p.mask.window > 0 && p.bias.data) return *why = "window functor together with attn_bias", false;
   const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
   for (const mi355_sdpa_tensor* t : ts) {
     if (t->stride[3] != 1) return *why = "head dim is not unit-stride", false;
@@ -585,7 +586,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
       if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
   }
   if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
-  if (p.bias.data || p.kv_lens || padded) {
+  if (p.bias.data || p.kv_lens || padded || p.mask.window > 0) {
     BwdM g;
     fill(g, p);
     const int D = E <= 64 ? 64 : 128;
