@@ -193,6 +193,17 @@ size_t mi355_sdpa_decode_workspace_bytes(const mi355_sdpa_decode_params* p);
 #define MI355_SDPA_DECODE_STATIC_SCRATCH_BYTES (32u << 20)
 int mi355_sdpa_decode_fp8kv_static(const mi355_sdpa_decode_params* p, void* stream);
 
+/* Row summary of an attention mask (L rows of S keys, unit stride over keys, row_stride in
+ * elements; bool, or float with 0 = keep and -inf = drop): rows_out receives four int32 per row
+ *   { last kept key, number of kept keys (-1 if some value is neither 0 nor -inf), length of the
+ *     kept run starting at key 0, first key of the kept run ending at the last kept key }
+ * from which the host recognises masks that a kernel can generate by itself (causal, sliding
+ * window with sink keys, keep-everything) and calls the unmasked kernels instead.  The run-time
+ * stand-in for the causal-mask recovery of
+ *   torch_neuronx/neuron_dynamo_backend/fx/passes/sdpa_causal_mask.py:162-289 (SdpaCausalMaskRewrite). */
+int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, int64_t S, int64_t row_stride,
+                         int32_t* rows_out, void* stream);
+
 /* ---- host logic (no GPU needed) --------------------------------------------------------- */
 
 /* Backend choice for F.scaled_dot_product_attention.  Rules of

@@ -1,0 +1,231 @@
+"""Recognition of masks that the kernels generate by themselves (causal, sliding window with sink
+keys, keep-everything): the run-time counterpart of the reference's causal-mask recovery
+(fx/passes/sdpa_causal_mask.py:162-289).  The host logic is checked on the CPU against brute force;
+the device row summary, the routing and its effect on results and time are GPU tests."""
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from helpers import max_abs, qkv, rel_err
+from oracle import sdpa_math as om
+
+
+def rows_of(mask: np.ndarray) -> np.ndarray:
+    """Brute-force row summary of a boolean (L, S) mask."""
+    L, S = mask.shape
+    out = np.zeros((L, 4), dtype=np.int32)
+    for i in range(L):
+        kept = np.flatnonzero(mask[i])
+        hi = int(kept[-1]) if kept.size else -1
+        dropped = np.flatnonzero(~mask[i])
+        lead = int(dropped[0]) if dropped.size else S
+        gaps = dropped[dropped < hi]
+        out[i] = (hi, kept.size, lead, int(gaps[-1]) + 1 if gaps.size else 0)
+    return out
+
+
+def pattern(mask_bool: torch.Tensor):
+    from torch_neuronx_amd.mask_patterns import pattern_from_rows
+
+    m = mask_bool.numpy()
+    return pattern_from_rows(rows_of(m), *m.shape)
+
+
+def rebuild(pat, L, S):
+    if pat == ("all",):
+        return torch.ones(L, S, dtype=torch.bool)
+    if pat == ("causal",):
+        return om.window_keep_mask(L, S, 0)
+    return om.window_keep_mask(L, S, pat[1], pat[2])
+
+
+@pytest.mark.parametrize("L,S", [(16, 16), (9, 30), (30, 9), (1, 5), (64, 64)])
+def test_causal_and_full_masks_are_recognised(L, S):
+    assert pattern(torch.ones(L, S, dtype=torch.bool)) == ("all",)
+    tril = torch.tril(torch.ones(L, S, dtype=torch.bool))
+    want = ("all",) if (tril.all()) else ("causal",)
+    assert pattern(tril) == want
+
+
+@pytest.mark.parametrize("L,W,N", [(40, 7, 0), (40, 7, 3), (40, 1, 0), (40, 16, 16), (40, 10, 30), (33, 32, 1), (70, 64, 0)])
+def test_window_masks_are_recognised(L, W, N):
+    m = om.window_keep_mask(L, L, W, N)
+    pat = pattern(m)
+    assert pat is not None and torch.equal(rebuild(pat, L, L), m)  # (N may come back smaller when the window covers it)
+    if N < L - W:
+        assert pat == ("window", W, N)
+
+
+def test_anything_else_is_left_alone():
+    g = torch.Generator().manual_seed(0)
+    L = 48
+    assert pattern(torch.rand(L, L, generator=g) < 0.5) is None
+    tril = torch.tril(torch.ones(L, L, dtype=torch.bool))
+    for (i, j) in [(10, 3), (30, 12), (5, 5), (0, 1), (20, 30)]:  # (a key dropped in the last row only would be a window)
+        m = tril.clone()
+        m[i, j] = not m[i, j]
+        assert pattern(m) is None, (i, j)
+    w = om.window_keep_mask(L, L, 9, 2)
+    for (i, j) in [(30, 1), (30, 22), (30, 5), (47, 39), (12, 2)]:
+        m = w.clone()
+        m[i, j] = not m[i, j]
+        assert pattern(m) is None, (i, j)
+    assert pattern(torch.triu(torch.ones(L, L, dtype=torch.bool))) is None       # upper triangle
+    assert pattern(torch.tril(torch.ones(L, L, dtype=torch.bool), -1)) is None   # strictly lower: row 0 is dead
+    pad = torch.ones(L, L, dtype=torch.bool)
+    pad[:, 40:] = False
+    assert pattern(pad) is None                                                   # key padding
+
+
+def test_recognition_is_sound_on_random_near_patterns():
+    # whatever is recognised rebuilds exactly the mask it came from
+    g = torch.Generator().manual_seed(1)
+    seen = 0
+    for trial in range(300):
+        L = int(torch.randint(2, 40, (1,), generator=g))
+        S = int(torch.randint(2, 40, (1,), generator=g))
+        W = int(torch.randint(0, 12, (1,), generator=g))
+        N = int(torch.randint(0, 6, (1,), generator=g)) if W else 0
+        m = om.window_keep_mask(L, S, W, N)
+        if trial % 3 == 0:
+            i, j = int(torch.randint(0, L, (1,), generator=g)), int(torch.randint(0, S, (1,), generator=g))
+            m[i, j] = not m[i, j]
+        pat = pattern(m)
+        if pat is not None:
+            seen += 1
+            assert torch.equal(rebuild(pat, L, S), m), (L, S, W, N, pat)
+    assert seen > 100
+
+
+# ---- GPU ----------------------------------------------------------------------------------------------
+
+
+@pytest.fixture(scope="module")
+def amd(gpu_device):
+    import torch_neuronx_amd as amd
+
+    return amd
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.bool, torch.float32, torch.bfloat16, torch.float16])
+def test_device_row_summary_matches_brute_force(amd, gpu_device, dtype):
+    import ctypes as C
+
+    from torch_neuronx_amd import _lib
+
+    g = torch.Generator().manual_seed(3)
+    L, S = 37, 203
+    keep = torch.rand(L, S, generator=g) < 0.6
+    keep[5] = False
+    keep[6] = True
+    m = keep if dtype is torch.bool else torch.zeros(L, S, dtype=dtype).masked_fill(~keep, float("-inf"))
+    wide = torch.zeros(L, S + 13, dtype=m.dtype)
+    wide[:, :S] = m
+    md = wide.to(gpu_device)[:, :S]  # row stride != S
+    rows = torch.empty(L, 4, dtype=torch.int32, device=gpu_device)
+    rc = _lib.load().mi355_sdpa_mask_rows(md.data_ptr(), _lib.dtype_id(md.dtype), L, S, md.stride(0), rows.data_ptr(),
+                                          _lib.current_stream(gpu_device))
+    assert rc == 0
+    assert np.array_equal(rows.cpu().numpy(), rows_of(keep.numpy()))
+    if dtype is not torch.bool:  # a real bias value makes the row "not a mask"
+        md2 = md.clone()
+        md2[3, 100] = 0.5
+        _lib.load().mi355_sdpa_mask_rows(md2.data_ptr(), _lib.dtype_id(md2.dtype), L, S, md2.stride(0), rows.data_ptr(),
+                                         _lib.current_stream(gpu_device))
+        got = rows.cpu().numpy()
+        assert got[3, 1] == -1 and (np.delete(got, 3, 0)[:, 1] >= 0).all()
+
+
+def _best_ms(fn, reps=5, inner=10):
+    best = 1e9
+    for _ in range(reps):
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(inner):
+            fn()
+        e1.record()
+        torch.cuda.synchronize()
+        best = min(best, e0.elapsed_time(e1) / inner)
+    return best
+
+
+@pytest.mark.gpu
+def test_tril_mask_takes_the_causal_kernel(amd, gpu_device, monkeypatch):
+    dev = gpu_device
+    L = 4096
+    # (no GQA here: upstream sends a mask together with enable_gqa to its composite math path)
+    q, k, v, go = (t.to(dev) for t in qkv(1, 8, 8, L, L, 128, dtype=torch.bfloat16, seed=2, with_do=True))
+    tril = torch.ones(L, L, dtype=torch.bool, device=dev).tril()[None, None]
+    amd.mask_patterns.clear_cache()
+    seen = []
+    f0 = amd.ops.sdpa_forward
+    monkeypatch.setattr(amd.ops, "sdpa_forward", lambda *a, **kw: (seen.append(kw), f0(*a, **kw))[1])
+    # the reference's own operator, with the mask as the caller made it
+    fused = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    fused_bwd = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    r_m = fused(q, k, v, tril)
+    assert seen[-1]["attn_bias"] is None and seen[-1]["is_causal"] is True
+    r_c = fused(q, k, v, None, 0.0, True)
+    assert torch.equal(r_m[0], r_c[0]) and torch.equal(r_m[1], r_c[1])  # the same kernel, bit for bit
+    g_m = fused_bwd(go, q, k, v, tril, [True, True, True, False], r_m[0], r_m[1], None, None, L, L, 0.0, False, r_m[6], r_m[7])
+    g_c = fused_bwd(go, q, k, v, None, [True, True, True, False], r_c[0], r_c[1], None, None, L, L, 0.0, True, r_c[6], r_c[7])
+    for a, b in zip(g_m[:3], g_c[:3]):
+        assert torch.equal(a, b)
+    # ... and at its speed once the mask has been looked at (the first call reads it and caches the answer)
+    t_mask = _best_ms(lambda: fused(q, k, v, tril))
+    t_causal = _best_ms(lambda: fused(q, k, v, None, 0.0, True))
+    assert t_mask <= 1.10 * t_causal, (t_mask, t_causal)
+    # a mask that changes in place is looked at again
+    tril[0, 0, 100, 3000] = True
+    r_x = fused(q, k, v, tril)
+    assert seen[-1]["attn_bias"] is not None and not torch.equal(r_x[0], r_c[0])
+    tril[0, 0, 100, 3000] = False
+    # the functional API: an additive mask that the caller keeps is recognised (and cached) ...
+    fm = torch.zeros(L, L, device=dev, dtype=torch.bfloat16).masked_fill(~tril[0, 0], float("-inf"))
+    out_f = F.scaled_dot_product_attention(q, k, v, attn_mask=fm)
+    assert seen[-1]["attn_bias"] is None and seen[-1]["is_causal"] is True and torch.equal(out_f, r_c[0])
+    # ... while a boolean one reaches the fused op as a fresh additive tensor on every call: after a
+    # few looks such masks are left to the masked kernel rather than paying a round trip per call
+    amd.mask_patterns.clear_cache()
+    looked0 = amd.mask_patterns.stats["looked"]
+    for _ in range(8):
+        out_b = F.scaled_dot_product_attention(q, k, v, attn_mask=tril)
+    assert amd.mask_patterns.stats["looked"] - looked0 == 3
+    assert seen[-1]["attn_bias"] is not None and max_abs(out_b, r_c[0]) <= 4e-3
+
+
+@pytest.mark.gpu
+def test_sliding_window_mask_takes_the_window_kernel(amd, gpu_device, monkeypatch):
+    dev = gpu_device
+    B, Hq, Hkv, L, D, W = 1, 4, 4, 4096, 128, 1024
+    q, k, v, go = qkv(B, Hq, Hkv, L, L, D, dtype=torch.bfloat16, seed=4, with_do=True)
+    keep = om.window_keep_mask(L, L, W)
+    maskd = keep.to(dev)[None, None]
+    maskd = torch.zeros(L, L, dtype=torch.bfloat16, device=dev).masked_fill(~maskd[0, 0], float("-inf"))  # kept by the caller
+    amd.mask_patterns.clear_cache()
+    seen = []
+    f0 = amd.ops.sdpa_forward
+    monkeypatch.setattr(amd.ops, "sdpa_forward", lambda *a, **kw: (seen.append(kw), f0(*a, **kw))[1])
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    out = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=maskd)
+    out.backward(go.to(dev))
+    assert seen[-1]["attn_bias"] is None and seen[-1]["is_causal"] is True and seen[-1]["window"] == W
+    # parity with the oracle on the explicit mask, forward and backward (head subset: the oracle is a CPU program)
+    hs = slice(0, 2)
+    ro, rl = om.sdpa_forward(q[:, hs].float(), k[:, hs].float(), v[:, hs].float(), attn_mask=keep)
+    assert max_abs(out[:, hs], ro) <= 2e-2
+    rdq, rdk, rdv = om.sdpa_backward(go[:, hs].float(), q[:, hs].float(), k[:, hs].float(), v[:, hs].float(), ro, rl,
+                                     attn_mask=keep, reduce_in_fp32=True)
+    assert max_abs(qd.grad[:, hs], rdq) <= 5e-2 and rel_err(qd.grad[:, hs], rdq) <= 3e-2
+    assert rel_err(kd.grad[:, hs], rdk) <= 3e-2 and rel_err(vd.grad[:, hs], rdv) <= 3e-2
+    # rate on the scores the window keeps
+    Bp = 4
+    qb, kb, vb = (torch.randn(Bp, 32, L, D, device=dev, dtype=torch.bfloat16) for _ in range(3))
+    with torch.no_grad():
+        ms = _best_ms(lambda: F.scaled_dot_product_attention(qb, kb, vb, attn_mask=maskd))
+    live = int(keep.sum())
+    tflops = 4.0 * Bp * 32 * D * live / (ms * 1e-3) / 1e12
+    assert tflops >= 600.0, tflops

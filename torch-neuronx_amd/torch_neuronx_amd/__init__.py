@@ -6,7 +6,7 @@ attention ops for ROCm GPU tensors unless ``TORCH_NEURONX_AMD_REGISTER=0``.
 
 import os as _os
 
-from . import _lib, kernels, ops, python_ops, registration  # noqa: F401
+from . import _lib, kernels, mask_patterns, ops, python_ops, registration  # noqa: F401
 from .kernels import (  # noqa: F401
     scaled_dot_product_attention_backward_kernel,
     scaled_dot_product_attention_kernel,

@@ -1,0 +1,135 @@
+"""Recognise attention masks that a kernel can generate by itself.
+
+The reference recovers causality at trace time: its graph pass proves that an explicit mask is
+lower-triangular and rewrites the call to ``is_causal=True``, so that the fused kernel stays
+eligible (torch_neuronx/neuron_dynamo_backend/fx/passes/sdpa_causal_mask.py:162-289); with a mask
+its fused path is refused (decompositions.py:2203).  Here a mask only exists as a tensor, so it is
+read once on the device (``mi355_sdpa_mask_rows``: four numbers per row) and the decision is cached
+for as long as the tensor is unchanged: a causal mask, a sliding window with sink keys and a
+keep-everything mask are then served by the kernels that generate those patterns from indices,
+skip the tiles they drop and read no mask at all.
+"""
+
+from __future__ import annotations
+
+import ctypes as C
+import os
+from collections import OrderedDict
+
+import numpy as np
+import torch
+
+from . import _lib
+
+_CACHE_ENTRIES = 16
+_cache: "OrderedDict[tuple, tuple]" = OrderedDict()
+# Looking at a mask costs one device-to-host round trip.  A caller that hands in a NEW tensor on
+# every call (upstream's functional API turns a boolean mask into a fresh additive one each time
+# before it reaches the fused op) would pay that on every call and never hit the cache: after
+# _MAX_MISSES misses in a row for one (rows, keys, dtype) signature the masks of that signature
+# are left alone, with another try every _RETRY_EVERY calls.
+_MAX_MISSES = 3
+_RETRY_EVERY = 512
+_misses: dict = {}
+stats = {"looked": 0, "hits": 0, "left_alone": 0}
+
+
+def enabled() -> bool:
+    return os.environ.get("TORCH_NEURONX_AMD_RECOVER_MASKS", "1").lower() not in ("0", "false", "off", "no")
+
+
+def pattern_from_rows(rows: np.ndarray, L: int, S: int):
+    """``rows[i] = (last kept key, kept keys or -1, kept run from key 0, start of the run ending at
+    the last kept key)`` -> ``("all",)``, ``("causal",)``, ``("window", W, N)`` or ``None``.
+
+    Causal is anchored top-left (row ``i`` keeps keys ``0 .. min(i, S-1)``); a window keeps keys
+    ``i-W+1 .. i`` and the first ``N`` keys.  A candidate is accepted only if the summary of every
+    row equals what the pattern would give."""
+    if L == 0 or S == 0 or rows.shape != (L, 4):
+        return None
+    hi, cnt, lead, lo = (rows[:, c].astype(np.int64) for c in range(4))
+    if (cnt < 0).any():
+        return None
+    if (cnt == S).all():
+        return ("all",)
+    i = np.arange(L, dtype=np.int64)
+    hi_c = np.minimum(i, S - 1)
+    if not (hi == hi_c).all():
+        return None
+    lead_full = np.where(hi_c + 1 < S, hi_c + 1, S)
+    if (cnt == hi_c + 1).all():
+        return ("causal",) if (lead == lead_full).all() and (lo == 0).all() else None
+    r = L - 1
+    W = int(hi[r] - lo[r] + 1)
+    N = int(lead[r]) if lead[r] < lo[r] else 0
+    if W <= 0 or lo[r] == 0:
+        return None
+    lo_w = np.maximum(i - W + 1, 0)
+    joined = lo_w <= N  # the window reaches into the sink keys (or to key 0): one run from key 0
+    exp_lo = np.where(joined, 0, lo_w)
+    exp_lead = np.where(joined, lead_full, N)
+    exp_cnt = np.where(joined, hi_c + 1, hi_c - lo_w + 1 + N)
+    if (i - W + 1 > hi_c).any():  # a row whose window lies past the last key is dead: not this pattern
+        return None
+    if (lo == exp_lo).all() and (lead == exp_lead).all() and (cnt == exp_cnt).all():
+        return ("window", W, N)
+    return None
+
+
+def _as_2d(mask: torch.Tensor):
+    """The ``(L, S)`` slice of a mask that does not depend on batch and head, or ``None``."""
+    m = mask
+    while m.dim() > 2:
+        if m.size(0) == 1 or m.stride(0) == 0:
+            m = m[0]
+        else:
+            return None
+    if m.dim() != 2 or (m.size(1) > 1 and m.stride(1) != 1):
+        return None
+    return m
+
+
+def classify(mask: torch.Tensor):
+    """Pattern of a device mask (see ``pattern_from_rows``), or ``None`` if it is none of them, is a
+    real bias, depends on batch or head, or cannot be looked at now (stream capture in progress).
+    The answer is cached while the tensor is unchanged (its version counter included); the cache
+    holds the tensor, so its memory cannot be handed to another mask meanwhile."""
+    if mask.device.type != "cuda" or _lib.dtype_id(mask.dtype) not in (_lib.BOOL, _lib.F32, _lib.F16, _lib.BF16):
+        return None
+    m = _as_2d(mask)
+    if m is None:
+        return None
+    L, S = m.shape
+    if L < 1 or S < 1:
+        return None
+    key = (m.data_ptr(), L, S, m.stride(0), m.dtype, mask._version, mask.device.index)
+    sig = (L, S, m.dtype, mask.device.index)
+    hit = _cache.get(key)
+    if hit is not None:
+        _cache.move_to_end(key)
+        _misses.pop(sig, None)
+        stats["hits"] += 1
+        return hit[0]
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    streak = _misses.get(sig, 0)
+    _misses[sig] = streak + 1
+    if streak >= _MAX_MISSES and (streak - _MAX_MISSES) % _RETRY_EVERY != _RETRY_EVERY - 1:
+        stats["left_alone"] += 1
+        return None
+    stats["looked"] += 1
+    rows = torch.empty((L, 4), dtype=torch.int32, device=mask.device)
+    with _lib.on_device(mask.device):
+        rc = _lib.load().mi355_sdpa_mask_rows(m.data_ptr(), _lib.dtype_id(m.dtype), L, S, m.stride(0), rows.data_ptr(),
+                                              _lib.current_stream(mask.device))
+    _lib.check(rc)
+    pat = pattern_from_rows(rows.cpu().numpy(), L, S)
+    _cache[key] = (pat, mask)
+    while len(_cache) > _CACHE_ENTRIES:
+        _cache.popitem(last=False)
+    return pat
+
+
+def clear_cache() -> None:
+    _cache.clear()
+    _misses.clear()

@@ -15,7 +15,7 @@ import os
 
 import torch
 
-from .. import _lib, ops
+from .. import _lib, mask_patterns, ops
 
 
 def _mfma_enabled() -> bool:
@@ -82,6 +82,23 @@ def _wants_grad_bias(attn_bias, grad_input_mask) -> bool:
             and bool(grad_input_mask[3]))
 
 
+def _recover_pattern(attn_bias, is_causal, want_grad_bias=False):
+    """A mask that is a pattern the kernels generate by themselves (causal, sliding window with sink
+    keys, keep-everything) is dropped in favour of that pattern - the run-time counterpart of the
+    reference's causal-mask recovery (fx/passes/sdpa_causal_mask.py:162-289).
+    Returns ``(attn_bias, is_causal, functor keyword arguments)``."""
+    if attn_bias is None or is_causal or want_grad_bias or not mask_patterns.enabled():
+        return attn_bias, is_causal, {}
+    pat = mask_patterns.classify(attn_bias)
+    if pat is None:
+        return attn_bias, is_causal, {}
+    if pat[0] == "all":
+        return None, False, {}
+    if pat[0] == "causal":
+        return None, True, {}
+    return None, True, {"window": pat[1], "sink_keys": pat[2]}
+
+
 def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale, need_lse=True):
     _check_device(query)
     attn_bias = _present(attn_bias)
@@ -100,9 +117,10 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
         seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
     else:
         seed, offset = _empty_rng(query.device)
+    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal)
     out, lse = ops.sdpa_forward(query, key, value, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
                                 dropout_p=dropout_p, dropout_keep=keep, need_lse=need_lse,
-                                force_kernel=_force_kernel())
+                                force_kernel=_force_kernel(), **functor)
     if orig_dtype == torch.float64:
         out = out.to(orig_dtype)
     return out, lse, seed, offset
@@ -135,9 +153,11 @@ def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p,
             dropout_p = 0.0  # a placeholder carries no mask: treated as absent (_sdpa_math.py:42-45)
         else:
             keep = philox_seed
+    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, want_grad_bias)
     dq, dk, dv, dbias = ops.sdpa_backward(
         grad_out, query, key, value, out, logsumexp, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
-        dropout_p=dropout_p, dropout_keep=keep, want_grad_bias=want_grad_bias, force_kernel=_force_kernel())
+        dropout_p=dropout_p, dropout_keep=keep, want_grad_bias=want_grad_bias, force_kernel=_force_kernel(),
+        **functor)
     if orig_dtype == torch.float64:
         dq, dk, dv = dq.to(orig_dtype), dk.to(orig_dtype), dv.to(orig_dtype)
         dbias = dbias.to(orig_dtype) if dbias is not None else None
