@@ -177,12 +177,12 @@ def test_kernel_gates(amd):
     assert gate(q, k, v, scale=0.25) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q96 = _meta(2, 8, 512, 96)  # narrow head dims (multiples of 8) run padded in the next wider kernel
     assert gate(q96, q96, q96, is_causal=True) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
-    q256 = _meta(2, 8, 512, 256)  # head dims up to 256: forward only
-    assert gate(q256, q256, q256) == (L.KERNEL_MFMA, L.KERNEL_GENERIC)
+    q256 = _meta(2, 8, 512, 256)  # head dims up to 256, forward and backward
+    assert gate(q256, q256, q256) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q100 = _meta(2, 8, 512, 100)
     assert gate(q100, q100, q100) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     q2, k2 = _meta(1, 4, 64, 192), _meta(1, 4, 64, 192)
-    assert gate(q2, k2, _meta(1, 4, 64, 128)) == (L.KERNEL_MFMA, L.KERNEL_GENERIC)  # D_qk > D_v: forward only
+    assert gate(q2, k2, _meta(1, 4, 64, 128)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # D_qk > D_v (192 / 128)
     assert gate(_meta(1, 4, 64, 64), _meta(1, 4, 64, 64), _meta(1, 4, 64, 128)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(_meta(1, 4, 64, 640), _meta(1, 4, 64, 640), _meta(1, 4, 64, 640)) == (L.KERNEL_NONE, L.KERNEL_NONE)
     assert gate(q, _meta(1, 3, 8192, 128), _meta(1, 3, 8192, 128)) == (L.KERNEL_NONE, L.KERNEL_NONE)

@@ -383,3 +383,48 @@ def test_mfma_backward_grad_bias(amd, gpu_device, case, dtype):
     assert max_abs(dq, rdq) <= 5e-2
     if causal:
         assert (db.float().cpu().triu(1) == 0).all()
+
+
+# head dims above 128 and D_qk != D_v (multi-head latent attention's 192 / 128): the reference's fused
+# backward takes them (tests/python_ops/test_scaled_dot_product_attention.py:98-183, tolerances 5e-2 /
+# 1e-2 there; gate cases tests/neuron_dynamo_backend/unit/test_sdpa_nki_gates.py:52-56)
+WIDE_SHAPES = [
+    # B, Hq, Hkv, L, S, E, Dv, causal
+    (1, 24, 24, 512, 512, 192, 128, True),
+    (1, 4, 2, 512, 512, 192, 128, True),
+    (1, 4, 4, 256, 256, 256, 256, False),
+    (1, 4, 2, 512, 512, 256, 256, True),
+    (2, 8, 2, 333, 200, 160, 96, True),
+    (1, 2, 1, 130, 777, 136, 136, False),
+    (1, 4, 4, 64, 64, 256, 8, True),
+    (2, 4, 1, 1280, 1280, 256, 256, True),
+]
+
+
+@pytest.mark.parametrize("shape", WIDE_SHAPES)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_backward_wide_and_asymmetric_head_dims(amd, gpu_device, shape, dtype):
+    B, Hq, Hkv, L, S, E, Dv, causal = shape
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, Dv=Dv, dtype=dtype, seed=E + Dv + L, with_do=True)
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, is_causal=causal)
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, is_causal=causal)
+    assert dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape and dq.dtype == dtype
+    assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 5e-3
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert max_abs(a, r) <= 5e-2, name
+        assert rel_err(a, r) <= 2e-2, name
+
+
+def test_wide_backward_is_what_autograd_reaches(amd, gpu_device):
+    # the functional API lands in the MFMA kernels for 192 / 128 as well, forward and backward
+    import torch.nn.functional as F
+
+    q, k, v, go = qkv(1, 4, 4, 512, 512, 192, Dv=128, dtype=torch.bfloat16, seed=77, with_do=True)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    desc = amd.ops.make_desc(qd, kd, vd, is_causal=True)
+    assert amd.ops.can_use_fused_fwd(desc) == amd._lib.KERNEL_MFMA and amd.ops.can_use_fused_bwd(desc) == amd._lib.KERNEL_MFMA
+    out = torch.ops.aten._scaled_dot_product_fused_attention_overrideable(qd, kd, vd, None, 0.0, True)[0]
+    out.backward(go.to(gpu_device))
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, is_causal=True)
+    for a, r in ((qd.grad, rdq), (kd.grad, rdk), (vd.grad, rdv)):
+        assert max_abs(a, r) <= 5e-2 and rel_err(a, r) <= 2e-2

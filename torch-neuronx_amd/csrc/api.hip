@@ -240,7 +240,9 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   // call itself still sends to the generic kernel a bias whose rows are not dword-aligned, tensors
   // that are not 16-byte aligned or whose strides are not multiples of 8 elements.
   const bool bias_ok = true;
-  const bool dims = backward ? (E == Dv && E % 8 == 0 && E <= 128) : (E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E);
+  // (a mask, bias or key counts send the backward of head dims above 128 and of D_qk != D_v to the
+  // generic kernel at the call)
+  const bool dims = E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E;
   const bool fast = d->q_dtype != MI355_SDPA_F32 && dims &&
                     bias_ok && d->dropout_p == 0.f && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;

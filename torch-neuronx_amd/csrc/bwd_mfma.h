@@ -33,6 +33,8 @@ struct BwdM {
   // masked variants treat the rest of every Q / K / V / dO / O row as zeros and leave it out of
   // the gradients; 0 means the full width.
   int d_real = 0;
+  // ... of V, dO, O and dV when they are narrower than Q and K (bwd_wide.hip only); 0 means d_real
+  int dv_real = 0;
   // 1: the dQ kernel of bwd_dq_w32.hip computes delta and lse2 itself and writes them to the
   // workspace for the dK/dV kernel that follows it (bwd_delta_kernel is then not launched)
   int make_delta = 0;
@@ -83,5 +85,7 @@ int launch_bwd_dkdv_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s);
 // dQ with two wavefronts per SIMD (bwd_dq_w32.hip), same convention
 bool bwd_dq_w32_fits(const BwdM& g, int head_dim);
 int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s);
+// head dims above 128 and D_qk != D_v (D_v <= D_qk <= 256), without masks (bwd_wide.hip)
+int launch_bwd_wide(const BwdM& g, int dtype, hipStream_t s);
 
 }  // namespace mi355

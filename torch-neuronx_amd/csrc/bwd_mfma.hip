@@ -529,7 +529,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.causal = p.is_causal, g.scale = p.scale;
   g.xcd_map = ((g.B * g.Hkv) % 8 == 0) ? 1 : 0;
   g.kv_lens = p.kv_lens;
-  g.d_real = (int)p.q.size[3];
+  g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
   if (p.grad_bias.data) {
     g.gbias = p.grad_bias.data;
@@ -547,7 +547,12 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   *why = "";
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
-  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  if (E < 8 || E > 256 || E % 8 != 0 || Dv < 8 || Dv > E || Dv % 8 != 0)
+    return *why = "head dims are not multiples of 8 up to 256 with D_v <= D_qk", false;
+  // head dims above 128 and D_qk != D_v: the kernels of bwd_wide.hip, which take no mask of any kind
+  const bool wide = E > 128 || Dv != E;
+  if (wide && (p.bias.data || p.grad_bias.data || p.kv_lens || p.mask.window > 0))
+    return *why = "mask, bias or key counts with a head dim above 128 or D_qk != D_v", false;
   const bool padded = E != 64 && E != 128;  // served by the next wider kernels' masked variants
   if (p.grad_bias.data) {  // written by the dQ kernel four keys (8 bytes) at a time
     const int64_t S = p.k.size[2];
@@ -586,7 +591,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
       if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
   }
   if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
-  if (p.bias.data || p.kv_lens || padded || p.mask.window > 0) {
+  if (!wide && (p.bias.data || p.kv_lens || padded || p.mask.window > 0)) {
     BwdM g;
     fill(g, p);
     const int D = E <= 64 ? 64 : 128;
@@ -609,7 +614,8 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   fill(g, p);
   const int D = p.q.size[3] <= 64 ? 64 : 128;  // the kernels' width
   int rc;
-  if (p.dtype == MI355_SDPA_BF16) rc = D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
+  if (p.q.size[3] > 128 || p.v.size[3] != p.q.size[3]) rc = launch_bwd_wide(g, p.dtype, s);
+  else if (p.dtype == MI355_SDPA_BF16) rc = D == 128 ? launch_td<bf16_t, 128>(g, s) : launch_td<bf16_t, 64>(g, s);
   else rc = D == 128 ? launch_td<f16_t, 128>(g, s) : launch_td<f16_t, 64>(g, s);
   // (a sink logit changes nothing in these kernels: the probabilities come from the saved
   // log-sum-exp, which includes it; only its own gradient is one more small reduction)
