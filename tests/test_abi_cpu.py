@@ -260,7 +260,7 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
     # forward instances with a per-score bias at 128 rows per workgroup are known to spill a little
     known = re.compile(r"fwd_w32_kernelIDF16[b_]Li(128|256)ELi4ELi2EE")
     for name, r in rows.items():
-        if r["src"] not in ("fwd_mfma_w32.hip", "bwd_dq_w32.hip", "bwd_dkdv_w32.hip", "decode_fp8kv.hip"):
+        if r["src"] not in ("fwd_mfma_w32.hip", "bwd_dq_w32.hip", "bwd_dkdv_w32.hip", "bwd_wide.hip", "decode_fp8kv.hip"):
             continue
         scratch = int(r["ScratchSize_[bytes/lane]"])
         if known.search(name):

@@ -35,18 +35,29 @@ __device__ __forceinline__ u32x2 tr_read(const uint16_t* ptr) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// A 32-row tile of a (rows, width) matrix into LDS, zero beyond `width` and beyond `rows_left` rows.
-// 256 threads, 16-byte chunks: chunk c of row r at r * PITCH + 8 c.
-__device__ __forceinline__ void stage_tile(uint16_t* lds, const uint16_t* base, int64_t row_stride, int rows_left, int width,
-                                           int tid) {
+// A 32-row tile of a (rows, width) matrix on its way to LDS, zero beyond `width` and beyond
+// `rows_left` rows: fetched into registers one tile ahead (the loads travel under the matrix ops
+// of the current tile) and written to LDS between two barriers.  256 threads, 16-byte chunks:
+// chunk c of row r at r * PITCH + 8 c.
+constexpr int NST = (BT * (DW / 8)) / 256;  // chunks per thread and tile
+struct TileRegs {
+  u32x4 w[NST];
+  __device__ __forceinline__ void fetch(const uint16_t* base, int64_t row_stride, int rows_left, int width, int tid) {
 #pragma unroll
-  for (int n = 0; n < (BT * (DW / 8)) / 256; ++n) {
-    const int u = tid + n * 256, r = u / (DW / 8), ch = u % (DW / 8);
-    u32x4 w = {0u, 0u, 0u, 0u};
-    if (r < rows_left && ch * 8 < width) w = *(const u32x4*)(base + (int64_t)r * row_stride + ch * 8);
-    *(u32x4*)(lds + r * PITCH + ch * 8) = w;
+    for (int n = 0; n < NST; ++n) {
+      const int u = tid + n * 256, r = u / (DW / 8), ch = u % (DW / 8);
+      w[n] = u32x4{0u, 0u, 0u, 0u};
+      if (r < rows_left && ch * 8 < width) w[n] = *(const u32x4*)(base + (int64_t)r * row_stride + ch * 8);
+    }
   }
-}
+  __device__ __forceinline__ void put(uint16_t* lds, int tid) const {
+#pragma unroll
+    for (int n = 0; n < NST; ++n) {
+      const int u = tid + n * 256, r = u / (DW / 8), ch = u % (DW / 8);
+      *(u32x4*)(lds + r * PITCH + ch * 8) = w[n];
+    }
+  }
+};
 
 // element offsets of the transposing reads of a tile, [second read of a pair][d block]
 struct TrOff {
@@ -117,11 +128,16 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;  // tiles with work for this wavefront
   const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
 
+  TileRegs kn, vn;
+  if (nt > 0) kn.fetch(kp, p.k_sl, p.S, er, tid), vn.fetch(vp, p.v_sl, p.S, dvr, tid);
   for (int t = 0; t < nt; ++t) {
     __syncthreads();  // the previous tile has been read by every wavefront
-    stage_tile(k_t, kp + (int64_t)t * BT * p.k_sl, p.k_sl, p.S - t * BT, er, tid);
-    stage_tile(v_t, vp + (int64_t)t * BT * p.v_sl, p.v_sl, p.S - t * BT, dvr, tid);
+    kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
+    if (t + 1 < nt) {
+      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, p.S - (t + 1) * BT, er, tid);
+      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, p.S - (t + 1) * BT, dvr, tid);
+    }
     if (t >= nt_w) continue;
     f32x16 sacc = zero16, dpacc = zero16;
 #pragma unroll
@@ -197,6 +213,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   const int nqs = (p.L + BT - 1) / BT;
   const int qs_begin = p.causal ? min(k0 / BT, nqs) : 0;
 
+  // (no fetch ahead here: the two accumulators and the two fragments fill the register file, and the
+  // 32 registers of a tile in flight spill)
   for (int hg = 0; hg < rep; ++hg) {
     const int h = hk * rep + hg;
     const uint16_t* qb = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
@@ -205,8 +223,13 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     for (int qs = qs_begin; qs < nqs; ++qs) {
       const int q0 = qs * BT;
       __syncthreads();  // the previous tile has been read by every wavefront
-      stage_tile(q_t, qb + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, er, tid);
-      stage_tile(do_t, gb + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, dvr, tid);
+      {
+        TileRegs qn;
+        qn.fetch(qb + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, er, tid);
+        qn.put(q_t, tid);
+        qn.fetch(gb + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, dvr, tid);
+        qn.put(do_t, tid);
+      }
       if (tid < BT) {
         const int qi = q0 + tid;
         // rows past L are switched off through lse = +inf
