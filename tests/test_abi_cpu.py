@@ -168,7 +168,8 @@ def test_kernel_gates(amd):
     q, k, v = _meta(1, 32, 8192, 128), _meta(1, 8, 8192, 128), _meta(1, 8, 8192, 128)
     assert gate(q, k, v, is_causal=True) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q.half(), k.half(), v.half()) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
-    assert gate(q.float(), k.float(), v.float()) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q.float(), k.float(), v.float()) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # float32 matrix op
+    assert gate(q.float(), k.float(), v.float(), attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(q, k, v, attn_bias=_meta(8192, 8192)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # masked calls too
     q64, k64 = _meta(1, 8, 512, 64), _meta(1, 8, 512, 64)
     assert gate(q64, k64, k64, attn_bias=_meta(512, 512)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)

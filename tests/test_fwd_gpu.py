@@ -442,3 +442,55 @@ def test_mfma_forward_value_rows_narrower_than_keys(amd, gpu_device, E, Dv, caus
     assert max_abs(out, ro) <= 2e-2
     assert rel_err(out, ro) <= 1e-2
     assert max_abs(lse, rl) <= 3e-3
+
+
+# ---- float32 inputs on the float32 matrix op --------------------------------------------------------
+# (the reference's fused gate takes float32, decompositions.py:2131-2158; shapes of its accuracy
+# matrix, tests/python_ops/test_scaled_dot_product_attention.py:220-302 and :362-387)
+F32_SHAPES = [
+    # B, Hq, Hkv, L, S, E, causal
+    (2, 4, 4, 128, 128, 64, False),      # config 1
+    (1, 8, 8, 512, 512, 64, False),
+    (1, 24, 6, 512, 512, 64, False),
+    (1, 8, 1, 512, 512, 64, True),
+    (1, 4, 2, 512, 512, 128, True),
+    (2, 4, 2, 51, 51, 48, True),
+    (2, 4, 2, 13, 51, 48, False),
+    (1, 2, 1, 577, 577, 64, True),
+    (1, 4, 4, 6, 6, 8, False),
+    (2, 8, 2, 300, 1100, 128, True),
+    (1, 2, 2, 200, 70, 104, True),
+]
+
+
+@pytest.mark.parametrize("shape", F32_SHAPES)
+def test_float32_matrix_op_forward_and_backward(amd, gpu_device, shape):
+    from helpers import oracle_bwd, rel_err
+
+    B, Hq, Hkv, L, S, E, causal = shape
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=torch.float32, seed=L + S + E, with_do=True)
+    qd, kd, vd, god = (t.to(gpu_device) for t in (q, k, v, go))
+    out, lse = amd.sdpa_forward(qd, kd, vd, is_causal=causal, force_kernel=MFMA)
+    dq, dk, dv, _ = amd.sdpa_backward(god, qd, kd, vd, out, lse, is_causal=causal, force_kernel=MFMA)
+    torch.cuda.synchronize()
+    ro, rl = oracle_fwd(q, k, v, is_causal=causal)
+    rdq, rdk, rdv = oracle_bwd(go, q, k, v, ro, rl, is_causal=causal)
+    assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert a.shape == r.shape and a.dtype == torch.float32
+        assert rel_err(a, r) <= 2e-6 and max_abs(a, r) <= 2e-5 * max(1.0, r.abs().max().item())
+    # the library picks these kernels by itself for such calls, and the generic kernels agree with them
+    out2, lse2 = amd.sdpa_forward(qd, kd, vd, is_causal=causal)
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+    out3, _ = amd.sdpa_forward(qd, kd, vd, is_causal=causal, force_kernel=GENERIC)
+    assert max_abs(out3, out) <= 1e-5
+
+
+def test_float32_matrix_op_refuses_what_it_does_not_serve(amd, gpu_device):
+    q, k, v = (t.to(gpu_device) for t in qkv(1, 2, 2, 64, 64, 64, dtype=torch.float32, seed=1))
+    bias = torch.zeros(64, 64, device=gpu_device)
+    with pytest.raises(NotImplementedError, match="float32 MFMA"):
+        amd.sdpa_forward(q, k, v, attn_bias=bias, force_kernel=MFMA)
+    out, _ = amd.sdpa_forward(q, k, v, attn_bias=bias)  # served by the generic kernel
+    ro, _ = oracle_fwd(q.cpu(), k.cpu(), v.cpu())
+    assert max_abs(out, ro) <= 1e-5

@@ -243,7 +243,9 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   // (a mask, bias or key counts send the backward of head dims above 128 and of D_qk != D_v to the
   // generic kernel at the call)
   const bool dims = E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E;
-  const bool fast = d->q_dtype != MI355_SDPA_F32 && dims &&
+  // (float32: the float32 matrix-op kernels, head dims up to 128 with D_qk = D_v and no mask)
+  const bool f32_ok = d->q_dtype != MI355_SDPA_F32 || (E == Dv && E <= 128 && !d->has_attn_bias);
+  const bool fast = f32_ok && dims &&
                     bias_ok && d->dropout_p == 0.f && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;
   return fast ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
@@ -271,10 +273,13 @@ int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
   hipStream_t s = (hipStream_t)stream;
   const char* why = "";
   int kernel = p->force_kernel;
-  if (kernel == 0) kernel = fwd_mfma_supported(*p, &why) ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
+  const bool f32 = p->dtype == MI355_SDPA_F32;
+  if (kernel == 0)
+    kernel = (f32 ? fwd_f32_mfma_supported(*p, &why) : fwd_mfma_supported(*p, &why)) ? MI355_SDPA_KERNEL_MFMA
+                                                                                     : MI355_SDPA_KERNEL_GENERIC;
   if (kernel == MI355_SDPA_KERNEL_MFMA || kernel == MI355_SDPA_KERNEL_MFMA_T128 ||
       kernel == MI355_SDPA_KERNEL_MFMA_T256)
-    return launch_fwd_mfma(*p, s);
+    return f32 ? launch_fwd_f32_mfma(*p, s) : launch_fwd_mfma(*p, s);
   if (kernel == MI355_SDPA_KERNEL_GENERIC) return launch_fwd_generic(*p, s);
   return set_error("SDPA: unknown kernel id %d", kernel), MI355_SDPA_ERR_INVALID;
 }
@@ -310,24 +315,27 @@ static bool bwd_args_ok(const mi355_sdpa_bwd_params* p) {
 static int bwd_kernel_choice(const mi355_sdpa_bwd_params* p) {
   if (p->force_kernel) return p->force_kernel;
   const char* why;
-  return bwd_mfma_supported(*p, &why) ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
+  const bool ok = p->dtype == MI355_SDPA_F32 ? bwd_f32_mfma_supported(*p, &why) : bwd_mfma_supported(*p, &why);
+  return ok ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
 }
 
 size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p) {
   if (!p) return 0;
   // sized for either kernel so the host can allocate before the choice is visible to it
-  return std::max(bwd_generic_workspace(*p), bwd_mfma_workspace(*p));
+  return std::max(bwd_generic_workspace(*p), std::max(bwd_mfma_workspace(*p), bwd_f32_mfma_workspace(*p)));
 }
 
 int mi355_sdpa_bwd(const mi355_sdpa_bwd_params* p, void* stream) {
   if (!bwd_args_ok(p)) return MI355_SDPA_ERR_INVALID;
   const int kernel = bwd_kernel_choice(p);
-  const size_t need = kernel == MI355_SDPA_KERNEL_MFMA ? bwd_mfma_workspace(*p) : bwd_generic_workspace(*p);
+  const bool f32 = p->dtype == MI355_SDPA_F32;
+  const size_t need = kernel != MI355_SDPA_KERNEL_MFMA ? bwd_generic_workspace(*p)
+                      : f32 ? bwd_f32_mfma_workspace(*p) : bwd_mfma_workspace(*p);
   if (need && (!p->workspace || p->workspace_bytes < need))
     return set_error("SDPA: backward workspace too small (%zu < %zu bytes)", p->workspace_bytes, need),
            MI355_SDPA_ERR_INVALID;
   hipStream_t s = (hipStream_t)stream;
-  if (kernel == MI355_SDPA_KERNEL_MFMA) return launch_bwd_mfma(*p, s);
+  if (kernel == MI355_SDPA_KERNEL_MFMA) return f32 ? launch_bwd_f32_mfma(*p, s) : launch_bwd_mfma(*p, s);
   if (kernel == MI355_SDPA_KERNEL_GENERIC) return launch_bwd_generic(*p, s);
   return set_error("SDPA: unknown kernel id %d", kernel), MI355_SDPA_ERR_INVALID;
 }

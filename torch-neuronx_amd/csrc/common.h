@@ -23,6 +23,12 @@ size_t bwd_generic_workspace(const mi355_sdpa_bwd_params& p);
 int launch_sink_grad(const float* lse, const float* delta, const float* sink_logit, float* grad, int64_t heads, int L,
                      hipStream_t s);
 size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p);
+// float32 inputs on the float32 matrix op (f32_mfma.hip)
+bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why);
+int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s);
+bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why);
+int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s);
+size_t bwd_f32_mfma_workspace(const mi355_sdpa_bwd_params& p);
 int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s);
 size_t decode_workspace(const mi355_sdpa_decode_params& p);
 int decode_pick_splits(const mi355_sdpa_decode_params& p);

@@ -1,0 +1,416 @@
+// Flash attention for float32 inputs on the float32 matrix op (v_mfma_f32_32x32x2_f32), forward and
+// backward, head dims up to 128 (multiples of 8; narrower rows count as zero padded), causal or
+// unmasked.  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
+// stays in float32 as in torch_neuronx/_sdpa_math.py (float32 inputs accumulate in float32, and the
+// probabilities that multiply V are not rounded, :94).
+//
+// Products are computed transposed, as in the half-precision kernels: a query row (forward, dQ)
+// or a key (dK / dV) is a lane, so softmax statistics are per-lane scalars.  With this matrix op a
+// lane supplies ONE element per operand (row / column lane % 32, contraction index lane / 32),
+// so an accumulator register of one product IS the B operand of a step of the next product, and
+// transposed operands are plain 4-byte LDS reads: no packing, no transposing reads.  A 32 x 32 x 2
+// op keeps the matrix pipe busy for 64 cycles, which leaves the compiler's own schedule enough
+// room: these kernels are not pipelined by hand.
+//
+//   fwd_f32_kernel        128 query rows per workgroup (4 wavefronts x 32), 32-key tiles
+//   bwd_f32_dq_kernel     the same shape; also leaves delta = rowsum(dO * O) and the log2-domain
+//                         log-sum-exp in the workspace
+//   bwd_f32_dkdv_kernel   128 keys per workgroup; loops over the query heads of the group (the GQA
+//                         sum of decompositions.py:2569-2599 happens in registers) and 32-row tiles
+#include "bwd_mfma.h"
+#include "fwd_mfma.h"
+
+namespace mi355 {
+namespace {
+
+constexpr int BT = 32;  // rows of a staged tile
+
+__device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
+  return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
+}
+
+// A 32-row tile of a (rows, width) float matrix into LDS, zeros beyond `width` and `rows_left`;
+// 256 threads, 16-byte chunks; row pitch D + 4 floats (16-byte row reads of 16 lanes hit every bank once)
+template <int D>
+__device__ __forceinline__ void stage_f32(float* lds, const float* base, int64_t row_stride, int rows_left, int width, int tid) {
+#pragma unroll
+  for (int n = 0; n < (BT * (D / 4)) / 256; ++n) {
+    const int u = tid + n * 256, r = u / (D / 4), ch = u % (D / 4);
+    f32x4 w = {0.f, 0.f, 0.f, 0.f};
+    if (r < rows_left && ch * 4 < width) w = *(const f32x4*)(base + (int64_t)r * row_stride + ch * 4);
+    *(f32x4*)(lds + r * (D + 4) + ch * 4) = w;
+  }
+}
+
+// this lane's half of a row (elements half * D/2 .. +D/2-1), zeros beyond `width`
+template <int D>
+__device__ __forceinline__ void load_half_row(float (&f)[D / 2], const float* row, int half, int width) {
+#pragma unroll
+  for (int i = 0; i < D / 8; ++i) {
+    const int d = half * (D / 2) + i * 4;
+    const f32x4 w = d < width ? *(const f32x4*)(row + d) : f32x4{0.f, 0.f, 0.f, 0.f};
+    f[i * 4] = w[0], f[i * 4 + 1] = w[1], f[i * 4 + 2] = w[2], f[i * 4 + 3] = w[3];
+  }
+}
+
+// acc = rows(tile)[lane % 32] . f over this lane's half of the head dim (A from LDS, B in registers)
+template <int D>
+__device__ __forceinline__ f32x16 row_product(const float* tile, int col, int half, const float (&f)[D / 2]) {
+  f32x16 acc = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  const float* r = tile + col * (D + 4) + half * (D / 2);
+#pragma unroll
+  for (int i = 0; i < D / 8; ++i) {
+    const f32x4 a = *(const f32x4*)(r + i * 4);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) acc = mma(a[e], f[i * 4 + e], acc);
+  }
+  return acc;
+}
+
+// acc[db] += cols(tile)^T . x : contraction over the tile's 32 rows in the order the accumulators of
+// a row product hold them (register r of lane half h is row 8 (r / 4) + 4 h + r % 4)
+template <int D>
+__device__ __forceinline__ void col_product(f32x16 (&acc)[D / 32], const float* tile, int col, int half, const f32x16& x) {
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const float* row = tile + ((r >> 2) * 8 + half * 4 + (r & 3)) * (D + 4) + col;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db) acc[db] = mma(row[db * 32], x[r], acc[db]);
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 1) void fwd_f32_kernel(FwdM p) {
+  constexpr int DB = D / 32;
+  __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
+  const int qt = p.n_qt - 1 - blockIdx.x / (p.B * p.Hq);  // heavy query tiles first
+  const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
+  const int q0 = qt * 128, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
+  float qf[D / 2];
+  load_half_row<D>(qf, (const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl, half, p.d_real);
+  f32x16 oacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(oacc[i]);
+  float m_run = -INFINITY, l_run = 0.f;  // (l_run: this lane half's keys only; the halves share m_run)
+  const float c = p.scale * kLog2eF;
+  const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
+  const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
+  int nt = (p.S + BT - 1) / BT;
+  if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
+  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  for (int t = 0; t < nt; ++t) {
+    __syncthreads();  // the previous tile has been read by every wavefront
+    stage_f32<D>(k_t, kp + (int64_t)t * BT * p.k_sl, p.k_sl, p.S - t * BT, p.d_real, tid);
+    stage_f32<D>(v_t, vp + (int64_t)t * BT * p.v_sl, p.v_sl, p.S - t * BT, p.d_real, tid);
+    __syncthreads();
+    if (t >= nt_w) continue;
+    f32x16 s = row_product<D>(k_t, col, half, qf);
+    float tm = -INFINITY;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kv = t * BT + (r >> 2) * 8 + half * 4 + (r & 3);
+      if (kv > lim) s[r] = -INFINITY;
+      tm = fmaxf(tm, s[r]);
+    }
+    tm = fmaxf(tm, __shfl_xor(tm, 32, 64));
+    const float m_new = fmaxf(m_run, tm);
+    const float m_use = m_new == -INFINITY ? 0.f : m_new;  // a row without a live key so far
+    const float alpha = __builtin_amdgcn_exp2f((m_run - m_use) * c);
+    m_run = m_new;
+    float psum = 0.f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      s[r] = __builtin_amdgcn_exp2f((s[r] - m_use) * c);
+      psum += s[r];
+    }
+    l_run = l_run * alpha + psum;
+#pragma unroll
+    for (int i = 0; i < DB; ++i)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+    col_product<D>(oacc, v_t, col, half, s);
+  }
+  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if (qrow < p.L) {
+    float* orow = (float*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8 + half * 4;
+        if (d < p.d_real)
+          *(f32x4*)(orow + d) = f32x4{oacc[db][g * 4] * inv, oacc[db][g * 4 + 1] * inv, oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv};
+      }
+    if (p.lse && half == 0)
+      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 1) void bwd_f32_dq_kernel(BwdM p) {
+  constexpr int DB = D / 32;
+  __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
+  const int n_qt = (p.L + 127) / 128;
+  const int qt = n_qt - 1 - blockIdx.x / (p.B * p.Hq);
+  const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
+  const int q0 = qt * 128, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
+  float qf[D / 2], dof[D / 2];
+  load_half_row<D>(qf, (const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl, half, p.d_real);
+  load_half_row<D>(dof, (const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl, half, p.d_real);
+  float lse2, dl;
+  {
+    // delta = rowsum(dO * O) (torch_neuronx/_sdpa_math.py:160-163): dO is in registers already
+    const float* orow = (const float*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qc * p.o_sl;
+    float dsum = 0.f;
+#pragma unroll
+    for (int i = 0; i < D / 8; ++i) {
+      const int d = half * (D / 2) + i * 4;
+      if (d < p.d_real) {
+        const f32x4 o = *(const f32x4*)(orow + d);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) dsum = fmaf(dof[i * 4 + e], o[e], dsum);
+      }
+    }
+    dsum += __shfl_xor(dsum, 32, 64);
+    const int64_t idx = ((int64_t)b * p.Hq + h) * p.L + qc;
+    const float l = p.lse[idx];
+    // +inf turns exp2(x - lse) into 0 for rows past L and for rows without a live key
+    lse2 = (qrow < p.L && l != -INFINITY) ? l * kLog2eF : INFINITY;
+    dl = dsum;
+    if (qrow < p.L && half == 0) p.delta[idx] = dsum, p.lse2[idx] = l != -INFINITY ? l * kLog2eF : INFINITY;
+  }
+  f32x16 dqacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(dqacc[i]);
+  const float c = p.scale * kLog2eF;
+  const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
+  const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
+  int nt = (p.S + BT - 1) / BT;
+  if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
+  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  for (int t = 0; t < nt; ++t) {
+    __syncthreads();
+    stage_f32<D>(k_t, kp + (int64_t)t * BT * p.k_sl, p.k_sl, p.S - t * BT, p.d_real, tid);
+    stage_f32<D>(v_t, vp + (int64_t)t * BT * p.v_sl, p.v_sl, p.S - t * BT, p.d_real, tid);
+    __syncthreads();
+    if (t >= nt_w) continue;
+    const f32x16 s = row_product<D>(k_t, col, half, qf);
+    const f32x16 dp = row_product<D>(v_t, col, half, dof);
+    f32x16 ds;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const int kv = t * BT + (r >> 2) * 8 + half * 4 + (r & 3);
+      float pr = __builtin_amdgcn_exp2f(fmaf(s[r], c, -lse2));
+      pr = kv > lim ? 0.f : pr;
+      ds[r] = pr * (dp[r] - dl);
+    }
+    col_product<D>(dqacc, k_t, col, half, ds);
+  }
+  if (qrow < p.L) {
+    float* gq = (float*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8 + half * 4;
+        if (d < p.d_real)
+          *(f32x4*)(gq + d) = f32x4{dqacc[db][g * 4] * p.scale, dqacc[db][g * 4 + 1] * p.scale, dqacc[db][g * 4 + 2] * p.scale,
+                                    dqacc[db][g * 4 + 3] * p.scale};
+      }
+  }
+}
+
+template <int D>
+__global__ __launch_bounds__(256, 1) void bwd_f32_dkdv_kernel(BwdM p) {
+  constexpr int DB = D / 32;
+  __shared__ __attribute__((aligned(16))) float q_t[BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float do_t[BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float lse_s[BT];
+  __shared__ __attribute__((aligned(16))) float dl_s[BT];
+  const int streams = p.B * p.Hkv;
+  const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
+  const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
+  const int k0 = kt * 128, kw0 = k0 + wave * 32, key = kw0 + col, kc = min(key, p.S - 1);
+  float kf[D / 2], vf[D / 2];
+  load_half_row<D>(kf, (const float*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl, half, p.d_real);
+  load_half_row<D>(vf, (const float*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl, half, p.d_real);
+  f32x16 dkacc[DB], dvacc[DB];
+#pragma unroll
+  for (int i = 0; i < DB; ++i) zero(dkacc[i]), zero(dvacc[i]);
+  const float c = p.scale * kLog2eF;
+  const int nqs = (p.L + BT - 1) / BT;
+  const int qs_begin = p.causal ? min(k0 / BT, nqs) : 0;
+  for (int hg = 0; hg < rep; ++hg) {
+    const int h = hk * rep + hg;
+    const float* qb = (const float*)p.q + b * p.q_sb + h * p.q_sh;
+    const float* gb = (const float*)p.go + b * p.go_sb + h * p.go_sh;
+    const int64_t row0 = ((int64_t)b * p.Hq + h) * p.L;
+    for (int qs = qs_begin; qs < nqs; ++qs) {
+      const int q0 = qs * BT;
+      __syncthreads();
+      stage_f32<D>(q_t, qb + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, p.d_real, tid);
+      stage_f32<D>(do_t, gb + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, p.d_real, tid);
+      if (tid < BT) {
+        const int qi = q0 + tid;
+        // rows past L are switched off through lse = +inf
+        lse_s[tid] = qi < p.L ? p.lse2[row0 + qi] : INFINITY;
+        dl_s[tid] = qi < p.L ? p.delta[row0 + qi] : 0.f;
+      }
+      __syncthreads();
+      if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= p.S) continue;  // (uniform per wavefront)
+      const f32x16 s = row_product<D>(q_t, col, half, kf);
+      const f32x16 dp = row_product<D>(do_t, col, half, vf);
+      f32x16 pr, ds;
+#pragma unroll
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
+        const f32x4 d4 = *(const f32x4*)(&dl_s[r4 * 8 + half * 4]);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
+          float x = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[e]));
+          x = ((p.causal && key > qi) || key >= p.S) ? 0.f : x;
+          pr[r] = x;
+          ds[r] = x * (dp[r] - d4[e]);
+        }
+      }
+      col_product<D>(dvacc, do_t, col, half, pr);
+      col_product<D>(dkacc, q_t, col, half, ds);
+    }
+  }
+  if (key < p.S) {
+    float* gk = (float*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
+    float* gv = (float*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8 + half * 4;
+        if (d < p.d_real) {
+          *(f32x4*)(gk + d) = f32x4{dkacc[db][g * 4] * p.scale, dkacc[db][g * 4 + 1] * p.scale, dkacc[db][g * 4 + 2] * p.scale,
+                                    dkacc[db][g * 4 + 3] * p.scale};
+          *(f32x4*)(gv + d) = f32x4{dvacc[db][g * 4], dvacc[db][g * 4 + 1], dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]};
+        }
+      }
+  }
+}
+
+bool tensors_fit(const mi355_sdpa_tensor* const* ts, int n) {
+  for (int k = 0; k < n; ++k) {
+    const mi355_sdpa_tensor* t = ts[k];
+    if (t->stride[3] != 1 || ((uintptr_t)t->data & 15) != 0) return false;
+    for (int i = 0; i < 3; ++i)
+      if (t->size[i] > 1 && (t->stride[i] % 4) != 0) return false;
+  }
+  return true;
+}
+
+}  // namespace
+
+bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
+  *why = "";
+  const int64_t E = p.q.size[3], Dv = p.v.size[3];
+  if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
+  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  if (p.bias.data || p.kv_lens || p.dropout_p > 0.f || p.mask.window > 0 || p.mask.sink_logit)
+    return *why = "bias, key counts, dropout or mask functors", false;
+  if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
+  if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
+  const mi355_sdpa_tensor* ts[4] = {&p.q, &p.k, &p.v, &p.out};
+  if (!tensors_fit(ts, 4)) return *why = "rows are not unit-stride and 16-byte aligned", false;
+  if (p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
+  return true;
+}
+
+int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
+  const char* why;
+  if (!fwd_f32_mfma_supported(p, &why)) {
+    set_error("SDPA: float32 MFMA forward kernel cannot take this call: %s", why);
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  FwdM g;
+  g.q = p.q.data, g.k = p.k.data, g.v = p.v.data, g.out = p.out.data, g.lse = p.lse;
+  g.q_sb = p.q.stride[0], g.q_sh = p.q.stride[1], g.q_sl = p.q.stride[2];
+  g.k_sb = p.k.stride[0], g.k_sh = p.k.stride[1], g.k_sl = p.k.stride[2];
+  g.v_sb = p.v.stride[0], g.v_sh = p.v.stride[1], g.v_sl = p.v.stride[2];
+  g.o_sb = p.out.stride[0], g.o_sh = p.out.stride[1], g.o_sl = p.out.stride[2];
+  g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Hkv = (int)p.k.size[1];
+  g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
+  g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
+  g.d_real = (int)p.q.size[3];
+  g.n_qt = (g.L + 127) / 128;
+  const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(256);
+  if (g.d_real <= 64) hipLaunchKernelGGL((fwd_f32_kernel<64>), grid, block, 0, s, g);
+  else hipLaunchKernelGGL((fwd_f32_kernel<128>), grid, block, 0, s, g);
+  return check_launch("fwd_f32_kernel");
+}
+
+bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
+  *why = "";
+  const int64_t E = p.q.size[3], Dv = p.v.size[3];
+  if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
+  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  if (p.bias.data || p.grad_bias.data || p.kv_lens || p.dropout_p > 0.f || p.mask.window > 0)
+    return *why = "bias, key counts, dropout or window", false;
+  if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
+  if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
+  const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
+  if (!tensors_fit(ts, 8)) return *why = "rows are not unit-stride and 16-byte aligned", false;
+  if (p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff ||
+      p.k.size[0] * p.k.size[1] * ((p.k.size[2] + 127) / 128) > 0x7fffffff)
+    return *why = "too many tiles", false;
+  return true;
+}
+
+size_t bwd_f32_mfma_workspace(const mi355_sdpa_bwd_params& p) {
+  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float);  // delta and lse2
+}
+
+int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
+  const char* why;
+  if (!bwd_f32_mfma_supported(p, &why)) {
+    set_error("SDPA: float32 MFMA backward kernel cannot take this call: %s", why);
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  BwdM g;
+  g.go = p.grad_out.data, g.q = p.q.data, g.k = p.k.data, g.v = p.v.data, g.out = p.out.data;
+  g.lse = p.lse, g.gq = p.grad_q.data, g.gk = p.grad_k.data, g.gv = p.grad_v.data;
+  g.delta = (float*)p.workspace;
+  g.lse2 = g.delta + p.q.size[0] * p.q.size[1] * p.q.size[2];
+#define SET3(dst, src) g.dst##_sb = p.src.stride[0], g.dst##_sh = p.src.stride[1], g.dst##_sl = p.src.stride[2]
+  SET3(go, grad_out);
+  SET3(q, q);
+  SET3(k, k);
+  SET3(v, v);
+  SET3(o, out);
+  SET3(gq, grad_q);
+  SET3(gk, grad_k);
+  SET3(gv, grad_v);
+#undef SET3
+  g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Hkv = (int)p.k.size[1];
+  g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
+  g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
+  g.d_real = (int)p.q.size[3];
+  const dim3 block(256);
+  const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 127) / 128))), kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 127) / 128)));
+  if (g.d_real <= 64) hipLaunchKernelGGL((bwd_f32_dq_kernel<64>), qgrid, block, 0, s, g);
+  else hipLaunchKernelGGL((bwd_f32_dq_kernel<128>), qgrid, block, 0, s, g);
+  int rc = check_launch("bwd_f32_dq_kernel");
+  if (rc) return rc;
+  if (g.d_real <= 64) hipLaunchKernelGGL((bwd_f32_dkdv_kernel<64>), kgrid, block, 0, s, g);
+  else hipLaunchKernelGGL((bwd_f32_dkdv_kernel<128>), kgrid, block, 0, s, g);
+  rc = check_launch("bwd_f32_dkdv_kernel");
+  if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
+    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
+  return rc;
+}
+
+}  // namespace mi355

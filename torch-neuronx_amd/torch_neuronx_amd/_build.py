@@ -14,7 +14,7 @@ LIB_DIR = os.path.join(PKG_DIR, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libmi355_sdpa.so")
 OBJ_DIR = os.path.join(LIB_DIR, "obj")
 
-SOURCES = ["api", "fwd_generic", "fwd_mfma", "fwd_mfma_w32", "bwd_generic", "bwd_mfma", "bwd_dkdv_w32", "bwd_dq_w32", "bwd_wide", "decode_fp8kv", "mask_rows"]
+SOURCES = ["api", "fwd_generic", "fwd_mfma", "fwd_mfma_w32", "bwd_generic", "bwd_mfma", "bwd_dkdv_w32", "bwd_dq_w32", "bwd_wide", "decode_fp8kv", "mask_rows", "f32_mfma"]
 
 # packed-fp32 VALU ops are switched off for all device code in this library
 HIPCC_FLAGS = [
