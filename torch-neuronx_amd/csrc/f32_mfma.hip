@@ -29,18 +29,30 @@ __device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
 }
 
-// A 32-row tile of a (rows, width) float matrix into LDS, zeros beyond `width` and `rows_left`;
-// 256 threads, 16-byte chunks; row pitch D + 4 floats (16-byte row reads of 16 lanes hit every bank once)
-template <int D>
-__device__ __forceinline__ void stage_f32(float* lds, const float* base, int64_t row_stride, int rows_left, int width, int tid) {
+// A 32-row tile of a (rows, width) float matrix on its way to LDS, zeros beyond `width` and
+// `rows_left`: fetched into registers one tile ahead (the loads travel under the matrix ops of the
+// current tile), written to LDS between two barriers.  NT threads, 16-byte chunks; row pitch D + 4
+// floats (16-byte row reads of 16 lanes hit every bank once)
+template <int D, int NT>
+struct TileF32 {
+  static constexpr int N = (BT * (D / 4)) / NT;
+  f32x4 w[N];
+  __device__ __forceinline__ void fetch(const float* base, int64_t row_stride, int rows_left, int width, int tid) {
 #pragma unroll
-  for (int n = 0; n < (BT * (D / 4)) / 256; ++n) {
-    const int u = tid + n * 256, r = u / (D / 4), ch = u % (D / 4);
-    f32x4 w = {0.f, 0.f, 0.f, 0.f};
-    if (r < rows_left && ch * 4 < width) w = *(const f32x4*)(base + (int64_t)r * row_stride + ch * 4);
-    *(f32x4*)(lds + r * (D + 4) + ch * 4) = w;
+    for (int n = 0; n < N; ++n) {
+      const int u = tid + n * NT, r = u / (D / 4), ch = u % (D / 4);
+      w[n] = f32x4{0.f, 0.f, 0.f, 0.f};
+      if (r < rows_left && ch * 4 < width) w[n] = *(const f32x4*)(base + (int64_t)r * row_stride + ch * 4);
+    }
   }
-}
+  __device__ __forceinline__ void put(float* lds, int tid) const {
+#pragma unroll
+    for (int n = 0; n < N; ++n) {
+      const int u = tid + n * NT, r = u / (D / 4), ch = u % (D / 4);
+      *(f32x4*)(lds + r * (D + 4) + ch * 4) = w[n];
+    }
+  }
+};
 
 // this lane's half of a row (elements half * D/2 .. +D/2-1), zeros beyond `width`
 template <int D>
@@ -79,15 +91,16 @@ __device__ __forceinline__ void col_product(f32x16 (&acc)[D / 32], const float* 
   }
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 1) void fwd_f32_kernel(FwdM p) {
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
   __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
   const int qt = p.n_qt - 1 - blockIdx.x / (p.B * p.Hq);  // heavy query tiles first
   const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
-  const int q0 = qt * 128, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
+  constexpr int BM = 32 * WAVES;  // query rows per workgroup
+  const int q0 = qt * BM, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
   float qf[D / 2];
   load_half_row<D>(qf, (const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl, half, p.d_real);
   f32x16 oacc[DB];
@@ -98,14 +111,19 @@ __global__ __launch_bounds__(256, 1) void fwd_f32_kernel(FwdM p) {
   const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
   const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
   int nt = (p.S + BT - 1) / BT;
-  if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BT + 1);
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
   const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  TileF32<D, 64 * WAVES> kn, vn;
+  if (nt > 0) kn.fetch(kp, p.k_sl, p.S, p.d_real, tid), vn.fetch(vp, p.v_sl, p.S, p.d_real, tid);
   for (int t = 0; t < nt; ++t) {
     __syncthreads();  // the previous tile has been read by every wavefront
-    stage_f32<D>(k_t, kp + (int64_t)t * BT * p.k_sl, p.k_sl, p.S - t * BT, p.d_real, tid);
-    stage_f32<D>(v_t, vp + (int64_t)t * BT * p.v_sl, p.v_sl, p.S - t * BT, p.d_real, tid);
+    kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
+    if (t + 1 < nt) {
+      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, p.S - (t + 1) * BT, p.d_real, tid);
+      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, p.S - (t + 1) * BT, p.d_real, tid);
+    }
     if (t >= nt_w) continue;
     f32x16 s = row_product<D>(k_t, col, half, qf);
     float tm = -INFINITY;
@@ -150,16 +168,17 @@ __global__ __launch_bounds__(256, 1) void fwd_f32_kernel(FwdM p) {
   }
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 1) void bwd_f32_dq_kernel(BwdM p) {
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
   __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
-  const int n_qt = (p.L + 127) / 128;
+  constexpr int BM = 32 * WAVES;  // query rows per workgroup
+  const int n_qt = (p.L + BM - 1) / BM;
   const int qt = n_qt - 1 - blockIdx.x / (p.B * p.Hq);
   const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
-  const int q0 = qt * 128, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
+  const int q0 = qt * BM, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
   float qf[D / 2], dof[D / 2];
   load_half_row<D>(qf, (const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl, half, p.d_real);
   load_half_row<D>(dof, (const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl, half, p.d_real);
@@ -192,14 +211,19 @@ __global__ __launch_bounds__(256, 1) void bwd_f32_dq_kernel(BwdM p) {
   const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
   const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
   int nt = (p.S + BT - 1) / BT;
-  if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
+  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BT + 1);
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
   const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  TileF32<D, 64 * WAVES> kn, vn;
+  if (nt > 0) kn.fetch(kp, p.k_sl, p.S, p.d_real, tid), vn.fetch(vp, p.v_sl, p.S, p.d_real, tid);
   for (int t = 0; t < nt; ++t) {
+    __syncthreads();  // the previous tile has been read by every wavefront
+    kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
-    stage_f32<D>(k_t, kp + (int64_t)t * BT * p.k_sl, p.k_sl, p.S - t * BT, p.d_real, tid);
-    stage_f32<D>(v_t, vp + (int64_t)t * BT * p.v_sl, p.v_sl, p.S - t * BT, p.d_real, tid);
-    __syncthreads();
+    if (t + 1 < nt) {
+      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, p.S - (t + 1) * BT, p.d_real, tid);
+      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, p.S - (t + 1) * BT, p.d_real, tid);
+    }
     if (t >= nt_w) continue;
     const f32x16 s = row_product<D>(k_t, col, half, qf);
     const f32x16 dp = row_product<D>(v_t, col, half, dof);
@@ -227,8 +251,8 @@ __global__ __launch_bounds__(256, 1) void bwd_f32_dq_kernel(BwdM p) {
   }
 }
 
-template <int D>
-__global__ __launch_bounds__(256, 1) void bwd_f32_dkdv_kernel(BwdM p) {
+template <int D, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float q_t[BT * (D + 4)];
   __shared__ __attribute__((aligned(16))) float do_t[BT * (D + 4)];
@@ -238,7 +262,7 @@ __global__ __launch_bounds__(256, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
   const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
-  const int k0 = kt * 128, kw0 = k0 + wave * 32, key = kw0 + col, kc = min(key, p.S - 1);
+  const int k0 = kt * 32 * WAVES, kw0 = k0 + wave * 32, key = kw0 + col, kc = min(key, p.S - 1);
   float kf[D / 2], vf[D / 2];
   load_half_row<D>(kf, (const float*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl, half, p.d_real);
   load_half_row<D>(vf, (const float*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl, half, p.d_real);
@@ -248,23 +272,31 @@ __global__ __launch_bounds__(256, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   const float c = p.scale * kLog2eF;
   const int nqs = (p.L + BT - 1) / BT;
   const int qs_begin = p.causal ? min(k0 / BT, nqs) : 0;
-  for (int hg = 0; hg < rep; ++hg) {
-    const int h = hk * rep + hg;
-    const float* qb = (const float*)p.q + b * p.q_sb + h * p.q_sh;
-    const float* gb = (const float*)p.go + b * p.go_sb + h * p.go_sh;
-    const int64_t row0 = ((int64_t)b * p.Hq + h) * p.L;
-    for (int qs = qs_begin; qs < nqs; ++qs) {
-      const int q0 = qs * BT;
+  // items: (query head of the group, 32-row query tile)
+  const int per_head = nqs - qs_begin, n_items = rep * per_head;
+  TileF32<D, 64 * WAVES> qn, gn;
+  float lse_n = INFINITY, dl_n = 0.f;
+  auto fetch_item = [&](int it) {
+    const int h = hk * rep + it / per_head, q0 = (qs_begin + it % per_head) * BT;
+    qn.fetch((const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, p.d_real, tid);
+    gn.fetch((const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, p.d_real, tid);
+    if (tid < BT) {
+      const int qi = q0 + tid;
+      const int64_t row = ((int64_t)b * p.Hq + h) * p.L + min(qi, p.L - 1);
+      // rows past L are switched off through lse = +inf
+      lse_n = qi < p.L ? p.lse2[row] : INFINITY;
+      dl_n = qi < p.L ? p.delta[row] : 0.f;
+    }
+  };
+  if (n_items > 0) fetch_item(0);
+  {
+    for (int it = 0; it < n_items; ++it) {
+      const int q0 = (qs_begin + it % per_head) * BT;
       __syncthreads();
-      stage_f32<D>(q_t, qb + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, p.d_real, tid);
-      stage_f32<D>(do_t, gb + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, p.d_real, tid);
-      if (tid < BT) {
-        const int qi = q0 + tid;
-        // rows past L are switched off through lse = +inf
-        lse_s[tid] = qi < p.L ? p.lse2[row0 + qi] : INFINITY;
-        dl_s[tid] = qi < p.L ? p.delta[row0 + qi] : 0.f;
-      }
+      qn.put(q_t, tid), gn.put(do_t, tid);
+      if (tid < BT) lse_s[tid] = lse_n, dl_s[tid] = dl_n;
       __syncthreads();
+      if (it + 1 < n_items) fetch_item(it + 1);
       if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= p.S) continue;  // (uniform per wavefront)
       const f32x16 s = row_product<D>(q_t, col, half, kf);
       const f32x16 dp = row_product<D>(do_t, col, half, vf);
@@ -302,6 +334,9 @@ __global__ __launch_bounds__(256, 1) void bwd_f32_dkdv_kernel(BwdM p) {
       }
   }
 }
+
+// wavefronts (32 rows each) per workgroup
+int pick_waves(int64_t, int) { return 4; }
 
 bool tensors_fit(const mi355_sdpa_tensor* const* ts, int n) {
   for (int k = 0; k < n; ++k) {
@@ -346,10 +381,17 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
   g.d_real = (int)p.q.size[3];
-  g.n_qt = (g.L + 127) / 128;
-  const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(256);
-  if (g.d_real <= 64) hipLaunchKernelGGL((fwd_f32_kernel<64>), grid, block, 0, s, g);
-  else hipLaunchKernelGGL((fwd_f32_kernel<128>), grid, block, 0, s, g);
+  // rows per workgroup: 128 (a workgroup is one wavefront per 32 rows; 64- and 32-row workgroups
+  // measured slower even when 128-row ones leave compute units without work)
+  const int waves = pick_waves((int64_t)g.B * g.Hq, g.L);
+  g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
+  const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(64 * waves);
+#define LAUNCH(DD, WW) hipLaunchKernelGGL((fwd_f32_kernel<DD, WW>), grid, block, 0, s, g)
+#define LAUNCH_W(DD) LAUNCH(DD, 4)
+  if (g.d_real <= 64) LAUNCH_W(64);
+  else LAUNCH_W(128);
+#undef LAUNCH_W
+#undef LAUNCH
   return check_launch("fwd_f32_kernel");
 }
 
@@ -399,14 +441,19 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
   g.d_real = (int)p.q.size[3];
-  const dim3 block(256);
-  const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 127) / 128))), kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 127) / 128)));
-  if (g.d_real <= 64) hipLaunchKernelGGL((bwd_f32_dq_kernel<64>), qgrid, block, 0, s, g);
-  else hipLaunchKernelGGL((bwd_f32_dq_kernel<128>), qgrid, block, 0, s, g);
+  const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
+  const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
+  const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw))));
+#define LAUNCH(KK, GRID, DD, WW) hipLaunchKernelGGL((KK<DD, WW>), GRID, dim3(64 * WW), 0, s, g)
+#define LAUNCH_W(KK, GRID, WAVES_, DD) LAUNCH(KK, GRID, DD, 4)
+  if (g.d_real <= 64) LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 64);
+  else LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 128);
   int rc = check_launch("bwd_f32_dq_kernel");
   if (rc) return rc;
-  if (g.d_real <= 64) hipLaunchKernelGGL((bwd_f32_dkdv_kernel<64>), kgrid, block, 0, s, g);
-  else hipLaunchKernelGGL((bwd_f32_dkdv_kernel<128>), kgrid, block, 0, s, g);
+  if (g.d_real <= 64) LAUNCH_W(bwd_f32_dkdv_kernel, kgrid, kw, 64);
+  else LAUNCH_W(bwd_f32_dkdv_kernel, kgrid, kw, 128);
+#undef LAUNCH_W
+#undef LAUNCH
   rc = check_launch("bwd_f32_dkdv_kernel");
   if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
     rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
