@@ -258,14 +258,14 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
     assert len(rows) > 50
     fwd = {n: r for n, r in rows.items() if "fwd_w32_kernel" in n}
     assert len(fwd) >= 30
-    # forward instances with a per-score bias at 128 rows per workgroup are known to spill a little
-    known = re.compile(r"fwd_w32_kernelIDF16[b_]Li(128|256)ELi4ELi2EE")
+    # the head-dim-256 forward with a per-score bias is known to spill (it holds 512 registers as it is)
+    known = re.compile(r"fwd_w32_kernelIDF16[b_]Li256ELi4ELi2EE")
     for name, r in rows.items():
         if r["src"] not in ("fwd_mfma_w32.hip", "bwd_dq_w32.hip", "bwd_dkdv_w32.hip", "bwd_wide.hip", "decode_fp8kv.hip"):
             continue
         scratch = int(r["ScratchSize_[bytes/lane]"])
         if known.search(name):
-            assert scratch <= 64, (name, scratch)
+            assert scratch <= 256, (name, scratch)
             continue
         assert scratch == 0, (name, scratch)
         assert r["Dynamic_Stack"] == "False"

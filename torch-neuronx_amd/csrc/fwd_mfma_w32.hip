@@ -21,7 +21,7 @@
 // order: the softmax of a 32-key tile is split in two halves that ride on the matrix ops of two
 // different phases, and LDS operands are fetched AHEAD matrix ops ahead through a register
 // ring.  The loop carries no row maximum: see kTrig.  K and V tiles go from global memory
-// straight into LDS, three tiles ahead of their use (with a bias: through registers, two ahead).
+// straight into LDS, three tiles ahead of their use; so does a bias, one tile ahead.
 // Products are computed transposed (S^T = K Q^T, O^T = V^T P^T) as in fwd_mfma.hip, so the
 // softmax statistics are per-lane scalars and P goes from accumulator to B operand in registers.
 //
@@ -41,39 +41,34 @@ constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescale
 // MASK = 1 adds per-batch key counts (kv_lens) and head dims below D (multiples of 8): the missing
 // tail of every Q / K / V row counts as zeros, which changes neither the scores nor the live part
 // of the output.  MASK = 2 adds an additive bias or boolean keep-mask on top, folded into the
-// score tile right after the matrix ops that produce it; its bias loads are awaited by the
-// compiler, with counts that know nothing of loads written as assembly, so this variant keeps
-// the staging through registers.
+// score tile right after the matrix ops that produce it.  The bias travels like the tiles: from
+// global memory straight into LDS (lane-private slots), with loads written as assembly and
+// awaited by count, so that nothing in the loop waits on a count the compiler chose.
 template <typename T, int D, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
   constexpr int KS = D / 16;      // matrix ops of S^T = K Q^T per tile (phase A)
   constexpr int DB = D / 32;      // 32-row blocks of O^T
   constexpr int NPV = 2 * DB;     // matrix ops of O^T += V^T P^T per tile (phase B)
-  constexpr int KROW = D + 8;     // K tile row pitch (elements): conflict-free 128-bit row reads
-  constexpr int VP = D + 32;      // V tile row pitch: four consecutive rows land in four different
-                                  // 64-byte windows, which the transposing reads need
   constexpr int CH = D / 8;       // 16-byte chunks per row
   constexpr int TCH = BN * CH;    // ... per tile
-  constexpr bool SPLIT = NT > TCH;  // more threads than chunks: one half stages K, the other V
-  constexpr int KLD = SPLIT ? 1 : TCH / NT;  // chunks of a tile per staging thread
   static_assert(AHEAD <= KS && AHEAD <= NPV && (KS + NPV) % 8 == 0, "ring layout");
-  // (head dim 256 needs more than the 64 KB of LDS a kernel may declare: it takes the launch's
-  // dynamic LDS instead, and runs one wavefront per SIMD with the 512-register budget)
-  constexpr bool DYN = D > 128;
-  // Unmasked calls at head dim 64 / 128 stage their tiles from global memory straight into LDS
-  // (see the staging section): four unpadded, swizzled buffers per operand, tile t in buffer t % 4.
-  constexpr bool DMA = MASK != 2;
+  // (head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare:
+  // they take the launch's dynamic LDS instead; head dim 256 runs one wavefront per SIMD with the
+  // 512-register budget)
+  constexpr bool DYN = D > 128 || MASK == 2;
+  // Tiles go from global memory straight into LDS (see the staging section): four unpadded,
+  // swizzled buffers per operand, tile t in buffer t % 4.
   // mask functors (window, sink keys, sink logit): in the masked variant without a bias, head dim <= 128
   constexpr bool FUNC = MASK == 1 && D <= 128;
   constexpr int NBUF = 4, TILE = BN * D;
-  __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * KROW];
-  __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : DMA ? NBUF * TILE : 2 * BN * VP];
+  __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : NBUF * TILE];
   extern __shared__ __attribute__((aligned(16))) uint16_t dyn_lds[];
-  uint16_t* const k_dma = DYN ? dyn_lds : k_static;                // the buffers of the direct staging
+  uint16_t* const k_dma = DYN ? dyn_lds : k_static;
   uint16_t* const v_dma = DYN ? dyn_lds + NBUF * TILE : v_static;
-  uint16_t (*const k_lds)[BN * KROW] = (uint16_t (*)[BN * KROW])(DYN ? dyn_lds : k_static);
-  uint16_t (*const v_lds)[BN * VP] = (uint16_t (*)[BN * VP])(DYN ? dyn_lds + 2 * BN * KROW : v_static);
+  // bias tiles (MASK = 2): per wavefront two buffers of four 1 KB groups, every lane its own 16 bytes of each
+  uint16_t* const bias_lds = dyn_lds + 2 * NBUF * TILE;
 
   int b, h, qt;
   decode_block(p, b, h, qt);
@@ -152,78 +147,19 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
     // (awaited here, once: left pending, their first use inside the tile loop would become a wait
     // for every outstanding load there, the tile loads in flight included)
-    if constexpr (DMA) {
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
-    }
+    for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
   }
 
   const int nt_w = p.causal ? min(nt, qw_last / BN + 1 - skip) : nt;
 
-  // ---- staging: every thread moves KLD 16-byte chunks of the K tile and of the V tile ------------
-  // Both tiles sit in LDS as they sit in memory, [key][d].  K is the A operand of S^T = K Q^T as it
-  // is; V^T, the A operand of O^T = V^T P^T, is produced by the transposing LDS read
-  // (ds_read_b64_tr_b16), so no transposition is done on the vector unit.
-  // Two staging sets each: a tile is fetched from global memory two iterations before it is
-  // written to LDS, so a fetch has about two tile times to land.
-  u32x4 kreg[2][KLD], vreg[2][KLD];
-  const int s_idx = (SPLIT && tid >= TCH) ? tid - TCH : tid;
-  const int k_chunk = s_idx % CH, k_row = s_idx / CH;  // rows k_row + i * NT / CH
-  // (uniform per wavefront, unless the rows are narrower than D: chunks past their end are never
-  // fetched, and the zeros they start with are what goes to LDS)
-  const bool do_k = (!SPLIT || tid < TCH) && (!MASK || k_chunk * 8 < dr);
-  const bool do_v = (!SPLIT || tid >= TCH) && (!MASK || k_chunk * 8 < drv);
-  const bool put_k = !SPLIT || tid < TCH, put_v = !SPLIT || tid >= TCH;
-  if constexpr (MASK) {
-#pragma unroll
-    for (int i = 0; i < KLD; ++i)
-      kreg[0][i] = kreg[1][i] = vreg[0][i] = vreg[1][i] = u32x4{0u, 0u, 0u, 0u};
-  }
-  // K and V are read through buffer resources: the per-thread byte offset inside a tile is fixed
-  // (one register each, set up once) and the tile offset is a scalar, so a fetch is a single
-  // instruction with one addition on the vector unit.  The resources end with the last key row
-  // of this (batch, head), and the whole offset travels in the vector offset, the part the
-  // hardware checks against that bound: rows of a ragged last tile beyond it read as zeros
-  // (their scores are masked, and a zero V row keeps 0 * V finite).
+  // K and V are read through buffer resources that end with the last key row of this (batch, head);
+  // the whole offset travels in the vector offset, the part the hardware checks against that bound:
+  // rows of a ragged last tile beyond it read as zeros (their scores are masked, and a zero V row
+  // keeps 0 * V finite).
   const int k_bytes = (int)(((int64_t)(S - 1) * p.k_sl + dr) * 2), v_bytes = (int)(((int64_t)(S - 1) * p.v_sl + drv) * 2);
-  const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)kp, 0, k_bytes, 0x00020000);
-  const __amdgpu_buffer_rsrc_t v_rsrc = __builtin_amdgcn_make_buffer_rsrc((void*)vp, 0, v_bytes, 0x00020000);
-  uint32_t k_off[KLD], v_off[KLD];
-#pragma unroll
-  for (int i = 0; i < KLD; ++i) {
-    k_off[i] = (uint32_t)(((k_row + i * (NT / CH)) * p.k_sl + k_chunk * 8) * 2);
-    v_off[i] = (uint32_t)(((k_row + i * (NT / CH)) * p.v_sl + k_chunk * 8) * 2);
-  }
   const int k_tile_bytes = (int)(BN * p.k_sl * 2), v_tile_bytes = (int)(BN * p.v_sl * 2);
-  auto load_k = [&](int set, int t) {
-    const uint32_t base = (uint32_t)(tile_of(min(t, nt - 1)) * k_tile_bytes);
-    if (do_k) {
-#pragma unroll
-      for (int i = 0; i < KLD; ++i) kreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(k_rsrc, k_off[i] + base, 0, 0);
-    }
-  };
-  auto load_v = [&](int set, int t) {
-    const uint32_t base = (uint32_t)(tile_of(min(t, nt - 1)) * v_tile_bytes);
-    if (do_v) {
-#pragma unroll
-      for (int i = 0; i < KLD; ++i) vreg[set][i] = __builtin_amdgcn_raw_buffer_load_b128(v_rsrc, v_off[i] + base, 0, 0);
-    }
-  };
-  auto store_k = [&](int set, int buf) {
-    if (put_k) {
-#pragma unroll
-      for (int i = 0; i < KLD; ++i)
-        *(u32x4*)(&k_lds[buf][(k_row + i * (NT / CH)) * KROW + k_chunk * 8]) = kreg[set][i];
-    }
-  };
-  auto store_v = [&](int set, int buf) {
-    if (put_v) {
-#pragma unroll
-      for (int i = 0; i < KLD; ++i)
-        *(u32x4*)(&v_lds[buf][(k_row + i * (NT / CH)) * VP + k_chunk * 8]) = vreg[set][i];
-    }
-  };
-  // ---- staging, unmasked calls: K and V tiles go from global memory straight into LDS -----------
+  // ---- staging: K and V tiles go from global memory straight into LDS ------------------------------
   // (buffer loads with the LDS bit: no trip through registers, no LDS store instructions).  Such a
   // load writes 64 x 16 contiguous bytes, one chunk per lane in lane order, at an LDS address that is
   // uniform for the wavefront, so the tiles are unpadded and bank conflicts are avoided by a
@@ -238,7 +174,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   constexpr bool DSPLIT = KL < WAVES;      // fewer than wavefronts: half of them stage K, half V
   constexpr int NL = DSPLIT ? 1 : KL / WAVES;  // loads per wavefront and tile
   constexpr int PL = DSPLIT ? 1 : 2 * NL;      // ... and pair
-  static_assert(!DMA || (DSPLIT ? 2 * KL == WAVES : KL % WAVES == 0), "staging layout");
+  static_assert(DSPLIT ? 2 * KL == WAVES : KL % WAVES == 0, "staging layout");
   auto descriptor = [&](const void* base, int bytes) {  // raw buffer resource, in scalar registers
     const uint64_t a = (uint64_t)base;
     return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
@@ -269,27 +205,29 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
                  :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   auto request_k = [&](int t) {  // K tile t (the last one again past the end) into buffer t % 4
-    if constexpr (DMA) {
-      const uint32_t g = (uint32_t)(tile_of(min(t, nt - 1)) * k_tile_bytes), l = lds_kd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
-      if (dma_k) {
+    const uint32_t g = (uint32_t)(tile_of(min(t, nt - 1)) * k_tile_bytes), l = lds_kd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+    if (dma_k) {
 #pragma unroll
-        for (int i = 0; i < NL; ++i) tile_load(kd_rsrc, kd_off[i] + g, l + i * WAVES * 1024);
-      }
+      for (int i = 0; i < NL; ++i) tile_load(kd_rsrc, kd_off[i] + g, l + i * WAVES * 1024);
     }
   };
   auto request_v = [&](int t) {
-    if constexpr (DMA) {
-      const uint32_t g = (uint32_t)(tile_of(min(t, nt - 1)) * v_tile_bytes), l = lds_vd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
-      if (dma_v) {
+    const uint32_t g = (uint32_t)(tile_of(min(t, nt - 1)) * v_tile_bytes), l = lds_vd + (uint32_t)((t & (NBUF - 1)) * TILE * 2);
+    if (dma_v) {
 #pragma unroll
-        for (int i = 0; i < NL; ++i) tile_load(vd_rsrc, vd_off[i] + g, l + i * WAVES * 1024);
-      }
+      for (int i = 0; i < NL; ++i) tile_load(vd_rsrc, vd_off[i] + g, l + i * WAVES * 1024);
     }
   };
   auto request_pair = [&](int j) { request_k(j + 1), request_v(j); };
   auto wait_all_tiles = [&]() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); };
+  auto wait_youngest_pair_only = [&]() {  // everything but the pair requested last has landed
+    if constexpr (PL == 1) asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+    else if constexpr (PL == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+    else if constexpr (PL == 4) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+  };
   auto wait_oldest_pair = [&]() {  // of three in flight
-    static_assert(!DMA || PL == 1 || PL == 2 || PL == 4 || PL == 8, "wait count");
+    static_assert(PL == 1 || PL == 2 || PL == 4 || PL == 8, "wait count");
     if constexpr (PL == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
     else if constexpr (PL == 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
     else if constexpr (PL == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
@@ -298,26 +236,22 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // element offsets of the LDS reads inside a swizzled tile (the swizzle is not additive in the d
   // block / contraction step: one offset register per combination)
   int row_off[KS], tr_off[2][DB];  // K row reads; V transposing reads [second read of a pair][d block]
-  if constexpr (DMA) {
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
+  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
 #pragma unroll
-    for (int sec = 0; sec < 2; ++sec)
+  for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
-        const int row = 8 * sec + ((lane >> 5) & 1) * 4 + ((lane & 15) >> 2);
-        const int d = db * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-        tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
-      }
-  }
+    for (int db = 0; db < DB; ++db) {
+      const int row = 8 * sec + ((lane >> 5) & 1) * 4 + ((lane & 15) >> 2);
+      const int d = db * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
+      tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
+    }
 
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
   // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
   // 8 + i / 4, 12 + i / 4: four keys at d = 4 (i / 4) + i % 4 = i.  A lane of the 32x32x16 A
   // operand (d row lane % 32, key half lane / 32) takes two such reads: keys 4 half .. +3 and
   // 8 + 4 half .. +3 of a 16-key step, the order in which the S^T accumulator holds them.
-  const int tr_jj = lane & 15, tr_g = lane >> 4;
-  const int tr_base = ((tr_g >> 1) * 4 + (tr_jj >> 2)) * VP + 16 * (tr_g & 1) + 4 * (tr_jj & 3);
   typedef short s16x4 __attribute__((ext_vector_type(4)));
   auto tr_read = [&](const uint16_t* ptr) {
     const s16x4 v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((s16x4 __attribute__((address_space(3)))*)(ptr));
@@ -346,44 +280,61 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // at this wavefront's first row of the (batch, head) plane and ends with its last one, so keys
   // past S read as zero (they are masked anyway).  Folded into the RAW scores, s += bias / scale,
   // so that everything downstream (reference tracking, lse) is the unbiased code.
-  uint32_t braw[16];
+  // A wavefront's 32 x 32 tile lands in its own 4 KB of LDS through the same kind of load as the
+  // K / V tiles, 16 bytes per lane and instruction whatever the element size:
+  //   float32     4 loads: load g, lane (row, half) -> keys 8 g + 4 half .. +3, read back by the same lane
+  //   16 bits     2 loads: load i, lane (row, half) -> keys 16 i + 8 half .. +7; group g of lane (row, half)
+  //               is the half-th 8 bytes of what lane (row, g % 2) fetched in load g / 2
+  //   bool        1 load:  lane (row, half) -> keys 16 half .. +15; group g is dword 2 (g % 2) + half of
+  //               what lane (row, g / 2) fetched
+  // One buffer: the tile after next is requested right after this one has been read, and has a
+  // whole iteration to land.  It is awaited by count: when the bias of tile t+1 is needed, the only
+  // younger loads are those of the pair requested at the end of the previous iteration.
+  uint32_t braw[4];
   float inv_scale = 0.f;
   const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  // (the resource is set up unconditionally, with no records when there is no bias: defined on one
-  // path only it stops being uniform for the compiler)
   const int b_esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const int b_rows = min(32, p.L - qw0);
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * b_esz : 0)), 0,
-      __builtin_amdgcn_readfirstlane((bkind && b_rows > 0) ? (int)(((b_rows - 1) * p.bias_sl + p.S) * b_esz) : 0), 0x00020000);
-  const uint32_t b_off = (uint32_t)((min(col, max(b_rows - 1, 0)) * p.bias_sl + half * 4) * b_esz);
+  const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * b_esz : 0),
+                                  (bkind && b_rows > 0) ? (int)(((b_rows - 1) * p.bias_sl + p.S) * b_esz) : 0);
+  const uint32_t b_voff = (uint32_t)((min(col, max(b_rows - 1, 0)) * p.bias_sl + half * (bkind == 1 ? 4 : bkind == 4 ? 16 : 8)) * b_esz);
+  const int b_loads = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const unsigned char* const bias_w = (const unsigned char*)bias_lds + (MASK == 2 ? wave * 4096 : 0);
+  const uint32_t lds_b = (uint32_t)(uintptr_t)(lds_bytes)bias_w;
   if (bkind) inv_scale = 1.f / p.scale;
   auto load_bias = [&](int t) {
     if constexpr (MASK == 2) {
-      if (bkind == 1) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, b_off + (uint32_t)((t * BN + g * 8) * 4), 0, 0);
-          braw[4 * g] = w[0], braw[4 * g + 1] = w[1], braw[4 * g + 2] = w[2], braw[4 * g + 3] = w[3];
-        }
-      } else if (bkind == 4) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) braw[g] = __builtin_amdgcn_raw_buffer_load_b32(b_rsrc, b_off + (uint32_t)(t * BN + g * 8), 0, 0);
-      } else if (bkind) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, b_off + (uint32_t)((t * BN + g * 8) * 2), 0, 0);
-          braw[2 * g] = w[0], braw[2 * g + 1] = w[1];
+      if (bkind) {
+        // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const uint32_t g0 = b_voff + (uint32_t)(t * BN * b_esz);
+        tile_load(b_rsrc, g0, lds_b);
+        if (b_loads > 1) tile_load(b_rsrc, g0 + 32, lds_b + 1024);
+        if (b_loads > 2) {
+          tile_load(b_rsrc, g0 + 64, lds_b + 2048);
+          tile_load(b_rsrc, g0 + 96, lds_b + 3072);
         }
       }
     }
   };
-  auto apply_bias = [&](f32x16& sv) {
+  // (awaited: in the loop.  This wait also covers the pair that the iteration's barrier publishes.)
+  auto apply_bias = [&](f32x16& sv, bool awaited) {
     if constexpr (MASK == 2) {
+      if (awaited) wait_youngest_pair_only();
       if (bkind == 1) {
+        // (head dim 256 has no registers to spare: one group at a time there)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sv[r] = fmaf(__builtin_bit_cast(float, braw[r]), inv_scale, sv[r]);
+        for (int g = 0; g < 4; ++g) {
+          const u32x4 w = *(const u32x4*)(bias_w + g * 1024 + lane * 16);
+          // (vector elements are copied out first: a bit cast applied to the element itself reads element 0)
+          const uint32_t u[4] = {w[0], w[1], w[2], w[3]};
+#pragma unroll
+          for (int r = 0; r < 4; ++r) sv[4 * g + r] = fmaf(__builtin_bit_cast(float, u[r]), inv_scale, sv[4 * g + r]);
+          if constexpr (D > 128) __builtin_amdgcn_sched_barrier(0);
+        }
       } else if (bkind == 4) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) braw[g] = *(const uint32_t*)(bias_w + (col + 32 * (g >> 1)) * 16 + (g & 1) * 8 + half * 4);
         // (a tile that the mask keeps whole - most tiles of a padding or window mask - costs four
         // compares instead of three instructions per score)
         const bool whole = braw[0] == 0x01010101u && braw[1] == 0x01010101u && braw[2] == 0x01010101u && braw[3] == 0x01010101u;
@@ -397,14 +348,20 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
             for (int r = 0; r < 16; ++r) sv[r] = ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? sv[r] : -INFINITY;
           }
         }
-      } else if (bkind == 2) {
+      } else if (bkind) {
         typedef __attribute__((ext_vector_type(2))) _Float16 h2;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) sv[r] = fmaf((float)__builtin_bit_cast(h2, braw[r >> 1])[r & 1], inv_scale, sv[r]);
-      } else if (bkind == 3) {
+        for (int g = 0; g < 4; ++g) {
+          const u32x2 w = *(const u32x2*)(bias_w + (g >> 1) * 1024 + (col + 32 * (g & 1)) * 16 + half * 8);
+          const uint32_t u[2] = {w[0], w[1]};
 #pragma unroll
-        for (int r = 0; r < 16; ++r)
-          sv[r] = fmaf(__builtin_bit_cast(float, (r & 1) ? (braw[r >> 1] & 0xffff0000u) : (braw[r >> 1] << 16)), inv_scale, sv[r]);
+          for (int r = 0; r < 4; ++r) {
+            const uint32_t wide = (r & 1) ? (u[r >> 1] & 0xffff0000u) : (u[r >> 1] << 16);
+            const float f = bkind == 2 ? (float)__builtin_bit_cast(h2, u[r >> 1])[r & 1] : __builtin_bit_cast(float, wide);
+            sv[4 * g + r] = fmaf(f, inv_scale, sv[4 * g + r]);
+          }
+          if constexpr (D > 128) __builtin_amdgcn_sched_barrier(0);
+        }
       }
     }
   };
@@ -482,36 +439,22 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 
   // ---- prologue ----------------------------------------------------------------------------------
   load_bias(0);
-  if constexpr (DMA) {
-    request_k(0);
-    request_pair(0);
-    wait_all_tiles();
-    __syncthreads();
-    request_pair(1);
-    request_pair(2);
-  } else {
-    load_k(0, 0);
-    load_v(0, 0);
-    load_k(1, 1);
-    store_k(0, 0);
-    store_v(0, 0);
-    store_k(1, 1);
-    __syncthreads();
-    load_k(0, 2);
-    load_k(1, 3);
-    load_v(1, 1);
-    load_v(0, 2);
-  }
+  request_k(0);
+  request_pair(0);
+  wait_all_tiles();
+  __syncthreads();
+  request_pair(1);
+  request_pair(2);
   f32x16 s_a, s_b;
   uint32_t pk_a[8], pk_b[8];
   float ps_a = 0.f, ps_b = 0.f;
   {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 a = DMA ? *(const u32x4*)(k_dma + row_off[ks]) : *(const u32x4*)(&k_lds[0][col * KROW + ks * 16 + half * 8]);
+      const u32x4 a = *(const u32x4*)(k_dma + row_off[ks]);
       s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
     }
-    apply_bias(s_a);
+    apply_bias(s_a, false);
     load_bias(1);
     if (edge(0)) mask_tile(s_a, tile_of(0) * BN);
     raise_reference(tile_max(s_a));  // the first reference is the maximum of the first tile
@@ -524,34 +467,33 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   }
   __syncthreads();  // K buffer 0 is rewritten during the first iteration
-  if constexpr (DMA) request_pair(3);
+  request_pair(3);
   // LDS operands travel through a four-entry register ring, three matrix ops ahead of their use;
   // the ring runs across iterations (the first three K fragments of a tile are requested at the
   // end of the previous iteration, right after the barrier that publishes the tile)
   u32x4 ring[8];
 #pragma unroll
   for (int ks = 0; ks < AHEAD; ++ks)
-    ring[ks] = DMA ? *(const u32x4*)(k_dma + TILE + row_off[ks]) : *(const u32x4*)(&k_lds[1][col * KROW + half * 8 + ks * 16]);
+    ring[ks] = *(const u32x4*)(k_dma + TILE + row_off[ks]);
 
   // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
   // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
   //   phase A   S^T(t+1) = K(t+1) Q^T on the matrix pipe  |  softmax of the last 16 keys of tile t
   //   check     sum of tile t against kTrig; rare slow path
   //   phase B   O^T += V^T(t) P^T(t) on the matrix pipe    |  softmax of the first 16 keys of tile
-  //             t+1, LDS stores of tiles t+2 / t+1, fetches of tiles t+4 / t+3
+  //             t+1, request of tiles t+5 (K) and t+4 (V)
   auto iteration = [&](int t, auto tile_mod, f32x16& scur, f32x16& snext, uint32_t (&pk)[8], uint32_t (&pkn)[8],
                        float& ps, float& psn) {
     constexpr int tq = decltype(tile_mod)::value;  // t % 4, known at compile time
-    constexpr int par = tq & 1;
     // tiles t+1 (K, this iteration's scores), t+2 (K, published by this iteration's barrier), t (V)
-    const uint16_t* kt = DMA ? k_dma + ((tq + 1) & 3) * TILE : &k_lds[par ^ 1][col * KROW + half * 8];
-    const uint16_t* kn = DMA ? k_dma + ((tq + 2) & 3) * TILE : &k_lds[par][col * KROW + half * 8];
-    const uint16_t* vt = DMA ? v_dma + tq * TILE : &v_lds[par][tr_base];
-    auto read_k = [&](int ks) { return DMA ? *(const u32x4*)(kt + row_off[ks]) : *(const u32x4*)(kt + ks * 16); };
-    auto read_kn = [&](int ks) { return DMA ? *(const u32x4*)(kn + row_off[ks]) : *(const u32x4*)(kn + ks * 16); };
+    const uint16_t* kt = k_dma + ((tq + 1) & 3) * TILE;
+    const uint16_t* kn = k_dma + ((tq + 2) & 3) * TILE;
+    const uint16_t* vt = v_dma + tq * TILE;
+    auto read_k = [&](int ks) { return *(const u32x4*)(kt + row_off[ks]); };
+    auto read_kn = [&](int ks) { return *(const u32x4*)(kn + row_off[ks]); };
     auto read_v = [&](int i) {  // d block i % DB, 16-key step i / DB
-      const u32x2 lo = DMA ? tr_read(vt + tr_off[0][i % DB] + (i / DB) * 16 * D) : tr_read(vt + (i / DB) * 16 * VP + (i % DB) * 32);
-      const u32x2 hi = DMA ? tr_read(vt + tr_off[1][i % DB] + (i / DB) * 16 * D) : tr_read(vt + ((i / DB) * 16 + 8) * VP + (i % DB) * 32);
+      const u32x2 lo = tr_read(vt + tr_off[0][i % DB] + (i / DB) * 16 * D);
+      const u32x2 hi = tr_read(vt + tr_off[1][i % DB] + (i / DB) * 16 * D);
       return u32x4{lo[0], lo[1], hi[0], hi[1]};
     };
     __builtin_amdgcn_sched_barrier(0);
@@ -611,7 +553,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
     for (int i = 0; i < NPV; ++i) {  // i = DB * (16-key step) + d block
       if (i == NPV - 2) {
-        if constexpr (DMA) wait_oldest_pair();
+        if constexpr (MASK != 2) wait_oldest_pair();  // (with a bias: awaited together with the bias)
         __syncthreads();
       }
       if (i + AHEAD < NPV) ring[(KS + i + AHEAD) & 7] = read_v(i + AHEAD);
@@ -622,13 +564,13 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       if (i == NPV - 1) {
 #pragma unroll
         for (int j = (AHEAD + 1) / 2; j < AHEAD; ++j) ring[j] = read_kn(j);
-        if constexpr (DMA) request_pair(t + 4);
+        request_pair(t + 4);
       }
       const int ks2 = i / DB, db = i % DB;
       const u32x4 b0 = {pk[ks2 * 4], pk[ks2 * 4 + 1], pk[ks2 * 4 + 2], pk[ks2 * 4 + 3]};
       oacc[db] = Mma<T>::run(ring[(KS + i) & 7], b0, oacc[db]);
       if (i == 0) {
-        apply_bias(snext);
+        apply_bias(snext, true);
         load_bias(t + 2);
         if (__builtin_expect(edge(t + 1), 0)) mask_tile(snext, tile_of(t + 1) * BN);  // rare
         stage1(snext, 0);
@@ -637,61 +579,32 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
       for (int hs = (i == 0 ? 0 : max((i * 8) / NPV - 1, 0)); hs < max(((i + 1) * 8) / NPV - 1, 0); ++hs)
         softmax_slot(snext, 0, hs, pkn, psn);
-      if constexpr (!DMA) {
-        if (i == 0) store_k(par, par);  // tile t+2
-        if (i == 1) store_v(par ^ 1, par ^ 1);  // tile t+1
-        if (i == NPV / 2) load_k(par, t + 4);
-        if (i == NPV / 2 + 1) load_v(par ^ 1, t + 3);
-      }
       __builtin_amdgcn_sched_barrier(0);
     }
     softmax_slot(snext, 0, 7, pkn, psn);
   };
   // a wavefront whose rows lie above the causal diagonal of the remaining tiles only feeds LDS
-  auto idle_step = [&](int t, auto parity) {
-    constexpr int par = decltype(parity)::value;
-    if constexpr (DMA) {
-      wait_oldest_pair();
-      __syncthreads();
-      request_pair(t + 4);
-    } else {
-      store_k(par, par);
-      store_v(par ^ 1, par ^ 1);
-      load_k(par, t + 4);
-      load_v(par ^ 1, t + 3);
-      __syncthreads();
-    }
+  auto idle_step = [&](int t) {
+    wait_oldest_pair();
+    __syncthreads();
+    request_pair(t + 4);
   };
 
   int t = 0;
-  if constexpr (DMA) {  // the buffer of a tile is a compile-time constant: four copies of the iteration
-    for (;;) {
-      if (t >= nt_w) break;
-      iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
-      if (++t >= nt_w) break;
-      iteration(t, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
-      if (++t >= nt_w) break;
-      iteration(t, std::integral_constant<int, 2>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
-      if (++t >= nt_w) break;
-      iteration(t, std::integral_constant<int, 3>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
-      ++t;
-    }
-  } else {
-    for (; t + 1 < nt_w; t += 2) {
-      iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
-      iteration(t + 1, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
-    }
-    if (t < nt_w) {  // odd count: t is even here
-      iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
-      ++t;
-    }
+  for (;;) {  // the buffer of a tile is a compile-time constant: four copies of the iteration
+    if (t >= nt_w) break;
+    iteration(t, std::integral_constant<int, 0>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+    if (++t >= nt_w) break;
+    iteration(t, std::integral_constant<int, 1>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
+    if (++t >= nt_w) break;
+    iteration(t, std::integral_constant<int, 2>{}, s_a, s_b, pk_a, pk_b, ps_a, ps_b);
+    if (++t >= nt_w) break;
+    iteration(t, std::integral_constant<int, 3>{}, s_b, s_a, pk_b, pk_a, ps_b, ps_a);
+    ++t;
   }
-  for (; t < nt; ++t) {
-    if (t & 1) idle_step(t, std::integral_constant<int, 1>{});
-    else idle_step(t, std::integral_constant<int, 0>{});
-  }
+  for (; t < nt; ++t) idle_step(t);
   // (no load into LDS may be in flight when the workgroup's LDS is handed to the next one)
-  if constexpr (DMA) wait_all_tiles();
+  wait_all_tiles();
 
   // ---- epilogue ------------------------------------------------------------------------------------
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
@@ -711,56 +624,42 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       }
     }
   }
-  if constexpr (DMA) {
-    // A lane holds its query row in 8-byte pieces, 16 bytes apart: stored as they are, one
-    // instruction writes 32 fragments of 16 bytes, and the stores of a workgroup's last tile,
-    // which nothing overlaps, took 3 % of the kernel.  The tile goes through LDS instead (the
-    // tile buffers are free now; 32 rows x D per wavefront, 16-byte chunks XOR-swizzled by row
-    // against bank conflicts) and leaves as whole rows, 16 bytes per lane.
-    __syncthreads();  // every wavefront is done with the K / V tiles
-    uint16_t* ot = wave < WAVES / 2 ? k_dma + wave * 32 * D : v_dma + (wave - WAVES / 2) * 32 * D;
-    constexpr int SW = CH < 16 ? CH - 1 : 15;
+  // A lane holds its query row in 8-byte pieces, 16 bytes apart: stored as they are, one
+  // instruction writes 32 fragments of 16 bytes, and the stores of a workgroup's last tile,
+  // which nothing overlaps, took 3 % of the kernel.  The tile goes through LDS instead (the
+  // tile buffers are free now; 32 rows x D per wavefront, 16-byte chunks XOR-swizzled by row
+  // against bank conflicts) and leaves as whole rows, 16 bytes per lane.
+  __syncthreads();  // every wavefront is done with the K / V tiles
+  uint16_t* ot = wave < WAVES / 2 ? k_dma + wave * 32 * D : v_dma + (wave - WAVES / 2) * 32 * D;
+  constexpr int SW = CH < 16 ? CH - 1 : 15;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+  for (int db = 0; db < DB; ++db)
 #pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
-        w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
-        *(u32x2*)(ot + col * D + (((db * 4 + g) ^ (col & SW)) << 3) + half * 4) = w;
-      }
-    constexpr int RPI = 64 / CH;  // rows per store instruction
-    const int rr = lane / CH, cc = lane % CH;
-    uint16_t* obase = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + cc * 8;
-#pragma unroll
-    for (int i = 0; i < 32 / RPI; ++i) {
-      const int r = i * RPI + rr;
-      const u32x4 w = *(const u32x4*)(ot + r * D + ((cc ^ (r & SW)) << 3));
-      if (qw0 + r < p.L && (!MASK || cc * 8 < drv)) *(u32x4*)(obase + (int64_t)(qw0 + r) * p.o_sl) = w;
+    for (int g = 0; g < 4; ++g) {
+      u32x2 w;
+      w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
+      w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
+      *(u32x2*)(ot + col * D + (((db * 4 + g) ^ (col & SW)) << 3) + half * 4) = w;
     }
-    if (qrow < p.L && p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
-  } else if (qrow < p.L) {
-    uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
+  constexpr int RPI = 64 / CH;  // rows per store instruction
+  const int rr = lane / CH, cc = lane % CH;
+  uint16_t* obase = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + cc * 8;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
-#pragma unroll
-      for (int g = 0; g < 4; ++g) {
-        u32x2 w;
-        w[0] = Mma<T>::pack(oacc[db][g * 4 + 0] * inv, oacc[db][g * 4 + 1] * inv);
-        w[1] = Mma<T>::pack(oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv);
-        if (!MASK || db * 32 + g * 8 + half * 4 < drv) *(u32x2*)(orow + db * 32 + g * 8 + half * 4) = w;
-      }
-    if (p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
+  for (int i = 0; i < 32 / RPI; ++i) {
+    const int r = i * RPI + rr;
+    const u32x4 w = *(const u32x4*)(ot + r * D + ((cc ^ (r & SW)) << 3));
+    if (qw0 + r < p.L && (!MASK || cc * 8 < drv)) *(u32x4*)(obase + (int64_t)(qw0 + r) * p.o_sl) = w;
   }
+  if (qrow < p.L && p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
 }
 
-// one instantiation; head dim 256 needs more than the 64 KB of LDS a kernel may declare
+// one instantiation; head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare
 template <typename T, int D, int WAVES, int MASK>
 int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
   int bytes = 0;
-  if constexpr (D > 128) {
-    // (padded double buffers with a bias, four plain buffers per operand otherwise)
-    constexpr int kBytes = MASK == 2 ? (2 * BN * (D + 8) + 2 * BN * (D + 32)) * 2 : 2 * 4 * BN * D * 2;
+  if constexpr (D > 128 || MASK == 2) {
+    // (four buffers per operand, and 4 KB of bias tile per wavefront)
+    constexpr int kBytes = 2 * 4 * BN * D * 2 + (MASK == 2 ? WAVES * 4096 : 0);
     static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
     if (attr != hipSuccess) {
