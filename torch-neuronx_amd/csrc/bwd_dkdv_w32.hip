@@ -94,8 +94,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int qs_end = (W > 0 && k0 >= n_sink) ? max(min(nqs, (k0 + BK + W - 2) / BQ + 1), qs_begin) : nqs;
   const int per_head = qs_end - qs_begin;
   const int n_items = (MASK && k0 >= S) ? 0 : rep * per_head;  // no live key in this tile: zeros
-  auto item_head = [&](int it) { return hk * rep + it / per_head; };
-  auto item_q0 = [&](int it) { return (qs_begin + it % per_head) * BQ; };
+  // Items run query tile by query tile from the LAST tile down, the group's heads inside.  The
+  // workgroups of a (batch, kv head) share an XCD, and those that start together - under a causal
+  // mask they need different numbers of tiles, all ending with the last one - then ask for the same
+  // Q / dO tile at about the same time: one of them brings it into the XCD's L2, the others find it
+  // there.  (Head by head and upwards from each block's own first tile, the workgroups are at
+  // different tiles all the time and each streams Q / dO from memory on its own: 1.7 GB of fetches
+  // per call on a (2, 32/8, 4096, 128) problem, against 0.13 GB of Q and dO.)
+  auto item_head = [&](int it) { return hk * rep + it % rep; };
+  auto item_q0 = [&](int it) { return (qs_end - 1 - it / rep) * BQ; };
 
   // ---- staging: every thread moves two 16-byte chunks of the Q tile and two of the dO tile ------
   // Buffer resources end with the last row of the batch (the tile offset travels in the vector
