@@ -215,12 +215,14 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 
   // (no fetch ahead here: the two accumulators and the two fragments fill the register file, and the
   // 32 registers of a tile in flight spill)
-  for (int hg = 0; hg < rep; ++hg) {
-    const int h = hk * rep + hg;
-    const uint16_t* qb = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
-    const uint16_t* gb = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh;
-    const int64_t row0 = ((int64_t)b * p.Hq + h) * p.L;
-    for (int qs = qs_begin; qs < nqs; ++qs) {
+  // Query tile by query tile from the last one down, heads inside: the workgroups of a kv head, which
+  // share an XCD, then want the same Q / dO tile at about the same time and find it in its L2.
+  for (int qs = nqs - 1; qs >= qs_begin; --qs) {
+    for (int hg = 0; hg < rep; ++hg) {
+      const int h = hk * rep + hg;
+      const uint16_t* qb = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
+      const uint16_t* gb = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh;
+      const int64_t row0 = ((int64_t)b * p.Hq + h) * p.L;
       const int q0 = qs * BT;
       __syncthreads();  // the previous tile has been read by every wavefront
       {

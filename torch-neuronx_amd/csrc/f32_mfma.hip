@@ -277,7 +277,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   TileF32<D, 64 * WAVES> qn, gn;
   float lse_n = INFINITY, dl_n = 0.f;
   auto fetch_item = [&](int it) {
-    const int h = hk * rep + it / per_head, q0 = (qs_begin + it % per_head) * BT;
+    // (query tile by query tile from the last one down, heads inside: the workgroups of a kv head, which
+    // share an XCD, then want the same Q / dO tile at about the same time and find it in its L2)
+    const int h = hk * rep + it % rep, q0 = (nqs - 1 - it / rep) * BT;
     qn.fetch((const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, p.d_real, tid);
     gn.fetch((const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, p.d_real, tid);
     if (tid < BT) {
@@ -291,7 +293,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   if (n_items > 0) fetch_item(0);
   {
     for (int it = 0; it < n_items; ++it) {
-      const int q0 = (qs_begin + it % per_head) * BT;
+      const int q0 = (nqs - 1 - it / rep) * BT;
       __syncthreads();
       qn.put(q_t, tid), gn.put(do_t, tid);
       if (tid < BT) lse_s[tid] = lse_n, dl_s[tid] = dl_n;
