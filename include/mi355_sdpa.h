@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MI355_SDPA_ABI_VERSION 2
+#define MI355_SDPA_ABI_VERSION 3
 
 /* element types */
 enum mi355_sdpa_dtype {
@@ -92,11 +92,21 @@ typedef struct mi355_sdpa_desc {
  *   sink_keys    with a window: keys 0 .. sink_keys-1 stay visible to every later query
  *   sink_logit   optional (B,Hq) contiguous float32: one more logit per row that joins the
  *                softmax (maximum and sum) and carries no value: out = sum_j p_j v_j with
- *                p = softmax([scores, sink_logit])[:S]; lse includes it.  Works with any mask. */
+ *                p = softmax([scores, sink_logit])[:S]; lse includes it.  Works with any mask.
+ * Tile skip tables for a mask that only exists as a tensor (the run-time counterpart of the
+ * reference's static tile elimination, flex_attention.py.jinja:15-33), built from the bias /
+ * keep-mask by mi355_sdpa_mask_tiles and valid as long as that tensor is unchanged:
+ *   live_tiles    forward: per (mask batch, mask head, block of 64 query rows) a bitmap of the
+ *                 32-key tiles that hold at least one kept score; a workgroup walks only those
+ *   live_tiles_t  backward (dK/dV): per (mask batch, mask head, block of 128 keys) a bitmap of
+ *                 the 64-row query tiles that hold at least one kept score
+ * Both optional; ignored together with is_causal, a window, or more than 32768 keys. */
 typedef struct mi355_sdpa_mask_spec {
   int32_t window;
   int32_t sink_keys;
   const float* sink_logit;
+  const uint32_t* live_tiles;
+  const uint32_t* live_tiles_t;
 } mi355_sdpa_mask_spec;
 
 typedef struct mi355_sdpa_fwd_params {
@@ -204,6 +214,21 @@ int mi355_sdpa_decode_fp8kv_static(const mi355_sdpa_decode_params* p, void* stre
  *   torch_neuronx/neuron_dynamo_backend/fx/passes/sdpa_causal_mask.py:162-289 (SdpaCausalMaskRewrite). */
 int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, int64_t S, int64_t row_stride,
                          int32_t* rows_out, void* stream);
+
+/* Tile skip tables of a bias / keep-mask (sizes (B,Hq,L,S), stride 0 on broadcast dims, unit stride
+ * over keys, rows and data dword aligned as the MFMA kernels want them; bool, or float where
+ * -inf = dropped): which 64-row x 32-key blocks hold at least one kept score.  The mask's own
+ * batch and head extents count (a broadcast dim has extent 1).  Layouts, in uint32 words:
+ *   live_tiles    [batch][head][ceil(L/64)][W],   W  = ceil(ceil(S/32)/32), bit t of a row block =
+ *                 key tile t (word t/32, bit t%32)
+ *   live_tiles_t  [batch][head][ceil(S/128)][Wt], Wt = ceil(ceil(L/64)/32), bit q of a key block =
+ *                 query tile q
+ * mi355_sdpa_mask_tiles_words returns the two sizes (words = 0: the mask cannot have tables).
+ * No counterpart in the reference as a function: its templated kernel eliminates dropped tiles
+ * when the kernel is rendered (flex_attention.py.jinja:15-33); here the mask is data. */
+int mi355_sdpa_mask_tiles_words(const mi355_sdpa_tensor* bias, int32_t bias_dtype, size_t* words, size_t* words_t);
+int mi355_sdpa_mask_tiles(const mi355_sdpa_tensor* bias, int32_t bias_dtype, uint32_t* live_tiles,
+                          uint32_t* live_tiles_t, void* stream);
 
 /* ---- host logic (no GPU needed) --------------------------------------------------------- */
 

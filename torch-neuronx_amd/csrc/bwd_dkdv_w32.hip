@@ -50,6 +50,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   uint32_t* const pex = (uint32_t*)(do_t + 3 * TILE);  // [2][4 key blocks][64 lanes][16]
   float* const lse_s = (float*)(pex + 2 * 4 * 1024);   // [3][BQ]
   float* const dl_s = lse_s + 3 * BQ;                  // [3][BQ]
+  uint32_t* const live_s = (uint32_t*)(dl_s + 3 * BQ);  // [heads of the group][words]: query tiles with a kept score (skip table)
+  uint16_t* const items_s = (uint16_t*)(live_s + 256);  // [1024] live items, and their count behind them
 
   const int streams = p.B * p.Hkv;
   const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
@@ -89,11 +91,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // key see none of its keys, unless the block holds sink keys
   constexpr bool FUNC = MASK == 1;
   const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
+  const bool listed = MASK == 2 && p.live_t != nullptr;
   const int nqs = (p.L + BQ - 1) / BQ;
   const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
   const int qs_end = (W > 0 && k0 >= n_sink) ? max(min(nqs, (k0 + BK + W - 2) / BQ + 1), qs_begin) : nqs;
   const int per_head = qs_end - qs_begin;
-  const int n_items = (MASK && k0 >= S) ? 0 : rep * per_head;  // no live key in this tile: zeros
+  int n_items = (MASK && k0 >= S) ? 0 : rep * per_head;  // no live key in this tile: zeros
   // Items run query tile by query tile from the LAST tile down, the group's heads inside.  The
   // workgroups of a (batch, kv head) share an XCD, and those that start together - under a causal
   // mask they need different numbers of tiles, all ending with the last one - then ask for the same
@@ -101,8 +104,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // there.  (Head by head and upwards from each block's own first tile, the workgroups are at
   // different tiles all the time and each streams Q / dO from memory on its own: 1.7 GB of fetches
   // per call on a (2, 32/8, 4096, 128) problem, against 0.13 GB of Q and dO.)
-  auto item_head = [&](int it) { return hk * rep + it % rep; };
-  auto item_q0 = [&](int it) { return (qs_end - 1 - it / rep) * BQ; };
+  // (with a skip table: the items whose tile holds a kept score, listed in LDS before the first item)
+  bool compact = false;
+  auto item_id = [&](int it) {
+    if constexpr (MASK == 2) return compact ? __builtin_amdgcn_readfirstlane((int)items_s[it]) : it;
+    else return it;
+  };
+  auto item_head = [&](int it) { return hk * rep + item_id(it) % rep; };
+  auto item_q0 = [&](int it) { return (qs_end - 1 - item_id(it) / rep) * BQ; };
 
   // ---- staging: every thread moves two 16-byte chunks of the Q tile and two of the dO tile ------
   // Buffer resources end with the last row of the batch (the tile offset travels in the vector
@@ -388,13 +397,22 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       __builtin_amdgcn_sched_barrier(0);
     }
   };
-  // every key of this block lies above the diagonal of the tile's rows / past the keys / below their windows
-  auto dead_tile = [&](int q0) {
+  // every key of this block lies above the diagonal of the tile's rows / past the keys / below their
+  // windows, or the mask's skip table says that it keeps no score of the tile's rows and the block's keys
+  auto dead_tile = [&](int it) {
+    const int q0 = item_q0(it);
+    if constexpr (MASK == 2) {
+      if (listed) {
+        const int qt = q0 / BQ;
+        const int hg = item_id(it) % rep;
+        if (!compact && !((__builtin_amdgcn_readfirstlane((int)live_s[hg * p.live_t_words + (qt >> 5)]) >> (qt & 31)) & 1)) return true;
+      }
+    }
     return (p.causal && q0 + BQ - 1 < kw0) || kw0 >= S || (W > 0 && q0 - kw0 - 31 >= W && kw0 >= n_sink);
   };
   auto role_a = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
-    if (dead_tile(q0)) return;
+    if (dead_tile(it)) return;
     const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
     role_a_tile(it, tb, pb, edge);
   };
@@ -403,7 +421,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // it, dS and dK of that tile at the start of iteration it + 1.
   f32x16 dp[2];
   auto role_b_scores = [&](int it, int tb) {
-    if (dead_tile(item_q0(it))) return;
+    if (dead_tile(it)) return;
     scores(do_t + tb * TILE, dp);
   };
   // One tile of role B, pipelined like role A's:
@@ -413,8 +431,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   auto role_b = [&](int it, int tb, int pb) {
     constexpr int EPS = 16 / KS;  // elements per slot (2 or 4)
     constexpr int SPG = 4 / EPS;  // slots per group of four consecutive rows
-    const int q0 = item_q0(it);
-    if (dead_tile(q0)) return;
+    if (dead_tile(it)) return;
     const uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;
     const uint16_t* qt = q_t + tb * TILE;
     const float* drow = &dl_s[tb * BQ + half * 4];
@@ -459,6 +476,32 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
   };
 
+  if constexpr (MASK == 2) {
+    if (listed) {  // this key block's row of the skip table, for every head of the group
+      if (tid < rep * p.live_t_words) {
+        const int hd = hk * rep + tid / p.live_t_words;
+        live_s[tid] = p.live_t[(((int64_t)(p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? hd : 0)) * ((p.S + BK - 1) / BK) + kt) * p.live_t_words +
+                               tid % p.live_t_words];
+      }
+      __syncthreads();
+      if (n_items > 0 && n_items <= 1024) {
+        if (wave == 0) {
+          int cnt = 0;
+          for (int j0 = 0; j0 < n_items; j0 += 64) {
+            const int it = j0 + lane, qt = qs_end - 1 - it / rep;
+            const bool live = it < n_items && ((live_s[(it % rep) * p.live_t_words + (qt >> 5)] >> (qt & 31)) & 1u);
+            const uint64_t m = __builtin_amdgcn_ballot_w64(live);
+            if (live) items_s[cnt + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = (uint16_t)it;
+            cnt += __builtin_popcountll(m);
+          }
+          if (lane == 0) *(int*)(items_s + 1024) = cnt;
+        }
+        __syncthreads();
+        n_items = __builtin_amdgcn_readfirstlane(*(const int*)(items_s + 1024));
+        compact = true;
+      }
+    }
+  }
   if (n_items > 0) {
     load_item(0, 0);
     wait_tiles();
@@ -510,7 +553,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 
 template <typename T, int D, int MASK>
 int launch_t(const BwdM& g, hipStream_t s) {
-  constexpr int kSmemBytes = smem_bytes<D>();
+  constexpr int kSmemBytes = smem_bytes<D>() + (MASK == 2 ? 1024 + 2048 + 16 : 0);  // (with the skip table's row of the key block and the item list)
   static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D, MASK>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (attr != hipSuccess) {

@@ -41,6 +41,11 @@ struct BwdM {
   // sliding window (causal calls, masked variants without a per-score bias): query i sees keys
   // i-window+1 .. i and the first sink_keys keys; tiles that the window drops whole are skipped
   int window = 0, sink_keys = 0;
+  // tile skip table of a per-score bias / keep-mask for the dK/dV kernel: per (mask batch, mask head,
+  // block of 128 keys) a bitmap of the 64-row query tiles with a kept score, live_t_words words each;
+  // live_hm = the mask's own head extent
+  const uint32_t* live_t = nullptr;
+  int live_t_words = 0, live_hm = 1;
 };
 
 // dot product of eight packed elements, float32 accumulation

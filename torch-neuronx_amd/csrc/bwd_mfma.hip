@@ -540,6 +540,11 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1];
     g.bias_sl = p.q.size[2] > 1 ? p.bias.stride[2] : 0;
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
+    const int words_t = ((g.L + 63) / 64 + 31) / 32;
+    if (p.mask.live_tiles_t && !p.is_causal && g.bias_sl != 0 && g.S <= 32768 && (g.Hq / g.Hkv) * words_t <= 256) {
+      g.live_t = p.mask.live_tiles_t;
+      g.live_t_words = words_t, g.live_hm = live_extent(p.bias, 1);
+    }
   }
 }
 

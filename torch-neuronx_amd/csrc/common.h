@@ -43,6 +43,11 @@ struct T4 {  // device view of a 4-D tensor, strides in elements
   int64_t st[4];
 };
 
+// extent of a mask over dim i (batch or head) as far as its data goes: a broadcast dim counts once
+static inline int live_extent(const mi355_sdpa_tensor& t, int i) {
+  return (t.size[i] > 1 && t.stride[i] != 0) ? (int)t.size[i] : 1;
+}
+
 static inline T4 view(const mi355_sdpa_tensor& t) {
   T4 r;
   r.data = t.data;

@@ -34,6 +34,11 @@ struct FwdM {
   // that joins the softmax and carries no value
   int window = 0, sink_keys = 0;
   const float* sink_logit = nullptr;
+  // tile skip table of the bias / keep-mask (variant with a bias, no causal flag): per (mask batch,
+  // mask head, 64-row block) a bitmap of the key tiles with a kept score, live_words words each;
+  // live_hm = the mask's own head extent
+  const uint32_t* live_tiles = nullptr;
+  int live_words = 0, live_hm = 1;
 };
 
 // Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first

@@ -395,6 +395,10 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   }
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
+  if (p.bias.data && p.mask.live_tiles && !p.is_causal && g.S <= 32768 && p.bias.stride[2] != 0) {
+    g.live_tiles = p.mask.live_tiles;
+    g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
+  }
   const int D = g.d_real <= 64 ? 64 : g.d_real <= 128 ? 128 : 256;  // the kernel's width
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
@@ -408,7 +412,10 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     const bool big = D == 128 && ((g.S >= 2048 && wg256 >= (g.causal ? 512 : 256)) || (!g.causal && g.S >= 1024 && wg256 >= 512));
     // (a short window: the keys a workgroup walks are window + rows, so smaller workgroups waste less)
     const bool short_window = g.window > 0 && g.window <= 512;
-    const int rows = D == 256 ? 128 : force_tile ? force_tile : (big && !short_window) ? 256 : 128;
+    // (with a tile skip table at head dim 128: 256 rows, whose LDS has room for the tile list at two
+    // wavefronts per SIMD)
+    const bool listed = g.live_tiles && D == 128;
+    const int rows = D == 256 ? 128 : listed ? 256 : force_tile ? force_tile : (big && !short_window) ? 256 : 128;
     return launch_fwd_mfma_w32(g, p.dtype, D, rows / 32, s);
   }
   // strides beyond 32-bit offsets: the kernel above (64-bit addressing)

@@ -69,6 +69,8 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   uint16_t* const v_dma = DYN ? dyn_lds + NBUF * TILE : v_static;
   // bias tiles (MASK = 2): per wavefront two buffers of four 1 KB groups, every lane its own 16 bytes of each
   uint16_t* const bias_lds = dyn_lds + 2 * NBUF * TILE;
+  // ... and, with a tile skip table, the list of the key tiles this workgroup walks (1024 entries and the count)
+  uint16_t* const tile_list = bias_lds + WAVES * 2048;
 
   int b, h, qt;
   decode_block(p, b, h, qt);
@@ -118,7 +120,42 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       nt -= skip;
     }
   }
-  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  // With a tile skip table (variant with a bias): the tiles in which the mask keeps at least one score
+  // of this workgroup's rows, in ascending order.  The first wavefront ORs the bitmaps of the
+  // workgroup's 64-row blocks and expands the set bits into a list in LDS, 64 tiles per step.
+  bool listed = false;
+  if constexpr (MASK == 2) {
+    if (p.live_tiles && !p.causal) {
+      listed = true;
+      if (wave == 0) {
+        const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
+        const uint32_t* map = p.live_tiles + ((int64_t)((p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? h : 0)) * nrb + rb0) * p.live_words;
+        uint32_t w = 0u;
+        if (lane < p.live_words) {
+#pragma unroll
+          for (int r = 0; r < BM / 64; ++r)
+            if (rb0 + r < nrb) w |= map[r * p.live_words + lane];
+        }
+        int cnt = 0;
+        for (int j0 = 0; j0 < nt; j0 += 64) {
+          const uint32_t ww = __shfl(w, (j0 >> 5) + (lane >> 5), 64);
+          const bool live = j0 + lane < nt && ((ww >> (lane & 31)) & 1u);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(live);
+          if (live) tile_list[cnt + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = (uint16_t)(j0 + lane);
+          cnt += __builtin_popcountll(m);
+        }
+        if (lane == 0) *(int*)(tile_list + 1024) = cnt;
+      }
+      __syncthreads();
+      const int n_live = __builtin_amdgcn_readfirstlane(*(const int*)(tile_list + 1024));
+      listed = n_live < nt;  // (every tile live: the list is the identity)
+      nt = n_live;
+    }
+  }
+  auto tile_of = [&](int u) {
+    if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
+    else return FUNC ? u + (u >= n_lead ? skip : 0) : u;
+  };
   if constexpr (MASK) {
     if (nt <= 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87), or the sink logit alone
       if (qrow < p.L) {
@@ -307,7 +344,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       if (bkind) {
         // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const uint32_t g0 = b_voff + (uint32_t)(t * BN * b_esz);
+        const uint32_t g0 = b_voff + (uint32_t)((listed ? tile_of(min(t, nt - 1)) : t) * BN * b_esz);
         tile_load(b_rsrc, g0, lds_b);
         if (b_loads > 1) tile_load(b_rsrc, g0 + 32, lds_b + 1024);
         if (b_loads > 2) {
@@ -658,15 +695,16 @@ template <typename T, int D, int WAVES, int MASK>
 int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
   int bytes = 0;
   if constexpr (D > 128 || MASK == 2) {
-    // (four buffers per operand, and 4 KB of bias tile per wavefront)
-    constexpr int kBytes = 2 * 4 * BN * D * 2 + (MASK == 2 ? WAVES * 4096 : 0);
+    // (four buffers per operand, 4 KB of bias tile per wavefront, and the tile list of a call with a skip table)
+    constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK == 2 ? WAVES * 4096 : 0);
+    constexpr int kBytes = kBase + (MASK == 2 ? 2048 + 16 : 0);
     static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
     if (attr != hipSuccess) {
       set_error("SDPA: cannot reserve %d bytes of LDS for fwd_w32_kernel: %s", kBytes, hipGetErrorString(attr));
       return MI355_SDPA_ERR_LAUNCH;
     }
-    bytes = kBytes;
+    bytes = (MASK == 2 && g.live_tiles) ? kBytes : kBase;
   }
   hipLaunchKernelGGL((fwd_w32_kernel<T, D, WAVES, MASK>), grid, dim3(64 * WAVES), bytes, s, g);
   return MI355_SDPA_OK;

@@ -88,3 +88,137 @@ extern "C" int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, 
   }
   return check_launch("mask_rows_kernel");
 }
+
+// ---- tile skip tables ------------------------------------------------------------------------------
+// The run-time counterpart of the reference's static tile elimination
+// (torch_neuronx/neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:15-33): there the mask
+// is a function known when the kernel is rendered, here it is a tensor, so one pass over it records
+// which 64-row x 32-key blocks hold at least one kept score.  The forward then walks only those key
+// tiles; the dK/dV kernel, whose lanes are keys, gets the transposed map (128 keys x 64 rows).
+//
+// One workgroup per (mask batch, mask head, 64-row block); a wavefront owns 16 of the rows and reads
+// them a dword per lane (4 bool, 2 half, 1 float elements), 16 rows per column of dwords, so every
+// element of the mask is read once, 256 contiguous bytes per load.
+namespace mi355 {
+namespace {
+
+template <int KIND>  // 1 float32, 2 float16, 3 bfloat16, 4 bool: does the dword hold a kept element?
+__device__ __forceinline__ bool any_kept(uint32_t w) {
+  if constexpr (KIND == 1) return w != 0xff800000u;
+  else if constexpr (KIND == 2) return (w & 0xffffu) != 0xfc00u || (w >> 16) != 0xfc00u;
+  else if constexpr (KIND == 3) return (w & 0xffffu) != 0xff80u || (w >> 16) != 0xff80u;
+  else return w != 0u;
+}
+
+struct TileMapArgs {
+  const uint32_t* mask;       // dword view of the mask
+  int64_t sb, sh, sl;         // strides in dwords
+  int Hm, L, S, nrb, words;   // mask heads, rows, keys, 64-row blocks, words per row block
+  uint32_t* out;
+};
+
+template <int KIND>
+__global__ __launch_bounds__(256) void mask_tiles_kernel(TileMapArgs a) {
+  constexpr int KP = KIND == 1 ? 1 : KIND == 4 ? 4 : 2;  // keys per dword
+  constexpr int LPT = 32 / KP;                           // lanes per 32-key tile
+  constexpr int TPC = 64 / LPT;                          // tiles per 64-dword column chunk
+  __shared__ uint32_t bits[32];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int rb = blockIdx.x % a.nrb, hm = (blockIdx.x / a.nrb) % a.Hm, bm = blockIdx.x / (a.nrb * a.Hm);
+  if (tid < 32) bits[tid] = 0u;
+  __syncthreads();
+  const uint32_t* base = a.mask + bm * a.sb + hm * a.sh;
+  const int row0 = rb * 64 + wave * 16;
+  const int nd = a.S / KP;  // dwords per row
+  for (int c = 0; c * 64 < nd; ++c) {
+    const int d = c * 64 + lane;
+    bool kept = false;
+    if (d < nd) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        if (row0 + r < a.L) kept |= any_kept<KIND>(base[(int64_t)(row0 + r) * a.sl + d]);
+    }
+    const uint64_t m = __builtin_amdgcn_ballot_w64(kept);
+    if (lane < TPC) {
+      const uint64_t part = (m >> (lane * LPT)) & (LPT == 32 ? 0xffffffffull : ((1ull << LPT) - 1));
+      const int tile = c * TPC + lane;
+      if (part && !((bits[tile >> 5] >> (tile & 31)) & 1u)) atomicOr(&bits[tile >> 5], 1u << (tile & 31));
+    }
+  }
+  __syncthreads();
+  if (tid < a.words) a.out[((int64_t)(bm * a.Hm + hm) * a.nrb + rb) * a.words + tid] = bits[tid];
+}
+
+// live_t[(batch, head)][key block of 128][word]: bit q = some key tile of the block is live for row block q
+__global__ __launch_bounds__(256) void mask_tiles_transpose_kernel(const uint32_t* live, uint32_t* live_t, int heads, int nrb,
+                                                                   int words, int nkb, int words_t) {
+  const int64_t idx = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx >= (int64_t)heads * nkb * words_t) return;
+  const int w = (int)(idx % words_t), kb = (int)((idx / words_t) % nkb), bh = (int)(idx / ((int64_t)words_t * nkb));
+  uint32_t r = 0u;
+  for (int q = w * 32; q < min(w * 32 + 32, nrb); ++q) {
+    const uint32_t x = live[((int64_t)bh * nrb + q) * words + (kb >> 3)];
+    if ((x >> ((kb & 7) * 4)) & 0xfu) r |= 1u << (q & 31);
+  }
+  live_t[idx] = r;
+}
+
+// the mask's own extents (a broadcast dim counts once) and what a table needs of its layout
+bool tile_map_shape(const mi355_sdpa_tensor& t, int32_t dtype, int* Bm, int* Hm, int* nrb, int* words, int* nkb, int* words_t) {
+  const int esz = dtype == MI355_SDPA_F32 ? 4 : dtype == MI355_SDPA_BOOL ? 1 : (dtype == MI355_SDPA_F16 || dtype == MI355_SDPA_BF16) ? 2 : 0;
+  if (!esz || !t.data) return false;
+  const int64_t L = t.size[2], S = t.size[3];
+  const int gran = 4 / esz;
+  if (L < 1 || S < 1 || S > 32768 || L > (1 << 24)) return false;
+  if ((S > 1 && t.stride[3] != 1) || ((uintptr_t)t.data & 3) != 0 || S % gran != 0) return false;
+  for (int i = 0; i < 3; ++i)
+    if (t.size[i] > 1 && (t.stride[i] % gran) != 0) return false;
+  if (L > 1 && t.stride[2] == 0) return false;  // a mask per key: nothing to skip by row block
+  *Bm = live_extent(t, 0), *Hm = live_extent(t, 1);
+  *nrb = (int)((L + 63) / 64), *words = (int)(((S + 31) / 32 + 31) / 32);
+  *nkb = (int)((S + 127) / 128), *words_t = (*nrb + 31) / 32;
+  return true;
+}
+
+}  // namespace
+}  // namespace mi355
+
+extern "C" int mi355_sdpa_mask_tiles_words(const mi355_sdpa_tensor* bias, int32_t bias_dtype, size_t* words, size_t* words_t) {
+  if (!bias || !words || !words_t) return set_error("SDPA: mask_tiles_words needs a mask and two outputs"), MI355_SDPA_ERR_INVALID;
+  int Bm, Hm, nrb, w, nkb, wt;
+  *words = *words_t = 0;
+  if (!tile_map_shape(*bias, bias_dtype, &Bm, &Hm, &nrb, &w, &nkb, &wt)) return MI355_SDPA_OK;
+  *words = (size_t)Bm * Hm * nrb * w, *words_t = (size_t)Bm * Hm * nkb * wt;
+  return MI355_SDPA_OK;
+}
+
+extern "C" int mi355_sdpa_mask_tiles(const mi355_sdpa_tensor* bias, int32_t bias_dtype, uint32_t* live_tiles,
+                                     uint32_t* live_tiles_t, void* stream) {
+  if (!bias || !live_tiles) return set_error("SDPA: mask_tiles needs a mask and an output buffer"), MI355_SDPA_ERR_INVALID;
+  int Bm, Hm, nrb, w, nkb, wt;
+  if (!tile_map_shape(*bias, bias_dtype, &Bm, &Hm, &nrb, &w, &nkb, &wt))
+    return set_error("SDPA: mask_tiles: this mask cannot have tile tables (dtype, alignment, a row stride of 0, or more than 32768 keys)"),
+           MI355_SDPA_ERR_UNSUPPORTED;
+  const int esz = bias_dtype == MI355_SDPA_F32 ? 4 : bias_dtype == MI355_SDPA_BOOL ? 1 : 2;
+  const int gran = 4 / esz;
+  TileMapArgs a;
+  a.mask = (const uint32_t*)bias->data;
+  a.sb = Bm > 1 ? bias->stride[0] / gran : 0, a.sh = Hm > 1 ? bias->stride[1] / gran : 0, a.sl = bias->stride[2] / gran;
+  a.Hm = Hm, a.L = (int)bias->size[2], a.S = (int)bias->size[3], a.nrb = nrb, a.words = w, a.out = live_tiles;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)(Bm * Hm * nrb)), block(256);
+  switch (bias_dtype) {
+    case MI355_SDPA_F32: hipLaunchKernelGGL((mask_tiles_kernel<1>), grid, block, 0, s, a); break;
+    case MI355_SDPA_F16: hipLaunchKernelGGL((mask_tiles_kernel<2>), grid, block, 0, s, a); break;
+    case MI355_SDPA_BF16: hipLaunchKernelGGL((mask_tiles_kernel<3>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((mask_tiles_kernel<4>), grid, block, 0, s, a); break;
+  }
+  if (int rc = check_launch("mask_tiles_kernel")) return rc;
+  if (live_tiles_t) {
+    const int64_t n = (int64_t)Bm * Hm * nkb * wt;
+    hipLaunchKernelGGL(mask_tiles_transpose_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, live_tiles, live_tiles_t,
+                       Bm * Hm, nrb, w, nkb, wt);
+    return check_launch("mask_tiles_transpose_kernel");
+  }
+  return MI355_SDPA_OK;
+}

@@ -46,7 +46,8 @@ class Desc(C.Structure):
 
 
 class MaskSpec(C.Structure):
-    _fields_ = [("window", C.c_int32), ("sink_keys", C.c_int32), ("sink_logit", C.c_void_p)]
+    _fields_ = [("window", C.c_int32), ("sink_keys", C.c_int32), ("sink_logit", C.c_void_p),
+                ("live_tiles", C.c_void_p), ("live_tiles_t", C.c_void_p)]
 
 
 class FwdParams(C.Structure):
@@ -88,6 +89,8 @@ EXPORTS = {
     "mi355_sdpa_decode_workspace_bytes": (C.c_size_t, [C.POINTER(DecodeParams)]),
     "mi355_sdpa_decode_fp8kv_static": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),
     "mi355_sdpa_mask_rows": (C.c_int, [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
+    "mi355_sdpa_mask_tiles_words": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "mi355_sdpa_mask_tiles": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi355_sdpa_choose_backend": (C.c_int, [C.POINTER(Desc)]),
     "mi355_sdpa_validate": (C.c_int, [C.POINTER(Desc), C.c_char_p, C.c_size_t]),
     "mi355_sdpa_out_strides": (C.c_int, [C.POINTER(C.c_int64), C.POINTER(C.c_int64),

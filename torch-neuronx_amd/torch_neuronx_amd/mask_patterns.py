@@ -130,6 +130,36 @@ def classify(mask: torch.Tensor):
     return pat
 
 
+_tile_cache: "OrderedDict[tuple, tuple]" = OrderedDict()
+
+
+def tile_maps(mask: torch.Tensor, B: int, Hq: int, L: int, S: int):
+    """Tile skip tables of a mask that is no pattern (``ops.mask_tile_maps``), cached for as long as
+    the tensor is unchanged.  The run-time counterpart of the reference's static tile elimination
+    (neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:15-33): one pass over the mask on
+    the device, no trip to the host.  ``None`` for masks too small to matter, masks per key, and
+    inside a graph capture."""
+    if not enabled() or mask is None or L < 256 or S < 256 or mask.dim() < 2 or mask.shape[-2] == 1:
+        return None
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    from . import ops
+
+    key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask._version, mask.device.index, B, Hq)
+    hit = _tile_cache.get(key)
+    if hit is not None:
+        _tile_cache.move_to_end(key)
+        stats["tile_hits"] = stats.get("tile_hits", 0) + 1
+        return hit[0]
+    maps = ops.mask_tile_maps(mask, B, Hq, L, S)
+    stats["tile_builds"] = stats.get("tile_builds", 0) + 1
+    _tile_cache[key] = (maps, mask)
+    while len(_tile_cache) > _CACHE_ENTRIES:
+        _tile_cache.popitem(last=False)
+    return maps
+
+
 def clear_cache() -> None:
     _cache.clear()
     _misses.clear()
+    _tile_cache.clear()

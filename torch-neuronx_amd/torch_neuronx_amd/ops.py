@@ -100,10 +100,34 @@ def _bias_view(attn_bias, B, Hq, L, S):
     return b, _lib.dtype_id(b.dtype)
 
 
-def _mask_spec(spec, query, window, sink_keys, sink_logit):
+def mask_tile_maps(attn_bias, B, Hq, L, S):
+    """Tile skip tables of a bias / keep-mask (``mi355_sdpa_mask_tiles``): ``(live, live_t)`` int32
+    device tensors, or ``None`` for a mask that cannot have them (a mask per key, more than 32768
+    keys, rows that are not dword aligned).  Valid as long as the mask's contents are unchanged."""
+    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
+    if bias is None:
+        return None
+    lib = _lib.load()
+    t4 = _lib.tensor4(bias)
+    w, wt = C.c_size_t(0), C.c_size_t(0)
+    _lib.check(lib.mi355_sdpa_mask_tiles_words(C.byref(t4), bias_dt, C.byref(w), C.byref(wt)))
+    if w.value == 0:
+        return None
+    live = torch.empty((w.value,), dtype=torch.int32, device=bias.device)
+    live_t = torch.empty((max(wt.value, 1),), dtype=torch.int32, device=bias.device)
+    with _lib.on_device(bias.device):
+        rc = lib.mi355_sdpa_mask_tiles(C.byref(t4), bias_dt, live.data_ptr(), live_t.data_ptr(),
+                                       _lib.current_stream(bias.device))
+    _lib.check(rc)
+    return live, live_t
+
+
+def _mask_spec(spec, query, window, sink_keys, sink_logit, live_tiles=None):
     """Fill the functor part of a parameter block; returns the tensors that must stay alive."""
     spec.window = int(window or 0)
     spec.sink_keys = int(sink_keys or 0)
+    if live_tiles is not None:
+        spec.live_tiles, spec.live_tiles_t = live_tiles[0].data_ptr(), live_tiles[1].data_ptr()
     if sink_logit is None:
         return None
     B, Hq = query.shape[0], query.shape[1]
@@ -117,9 +141,12 @@ def _mask_spec(spec, query, window, sink_keys, sink_logit):
 
 def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None, dropout_p=0.0,
                  dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0,
-                 window=None, sink_keys=0, sink_logit=None):
+                 window=None, sink_keys=0, sink_logit=None, live_tiles=None):
     """Fused forward.  K/V arrive at ``Hkv`` heads.  Returns ``(out, lse)``; ``out`` keeps the
     dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``.
+
+    ``live_tiles``: the ``(live, live_t)`` pair of ``mask_tile_maps`` for this ``attn_bias`` (or
+    ``True`` to build it here): the kernels then skip the tiles that the mask drops whole.
 
     ``window`` (with ``is_causal``): query ``i`` sees keys ``i-window+1 .. i`` and the first
     ``sink_keys`` keys; ``sink_logit`` ``(B,Hq)`` or ``(Hq,)``: one more logit per row that joins
@@ -151,7 +178,9 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
-    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit)  # noqa: F841 (kept alive over the launch)
+    if live_tiles is True:
+        live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
+    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit, live_tiles)  # noqa: F841 (kept alive over the launch)
     with _lib.on_device(query.device):
         rc = _lib.load().mi355_sdpa_fwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
@@ -160,7 +189,8 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
 
 def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_causal=False,
                   scale=None, dropout_p=0.0, dropout_keep=None, kv_lens=None,
-                  want_grad_bias=False, force_kernel=0, window=None, sink_keys=0, sink_logit=None):
+                  want_grad_bias=False, force_kernel=0, window=None, sink_keys=0, sink_logit=None,
+                  live_tiles=None):
     """Fused backward.  Returns ``(dq, dk, dv, dbias-or-None)``; each gradient keeps the
     dimension order of its input, dk/dv come back at ``Hkv`` heads.  With a ``sink_logit`` a
     fifth element follows: its gradient, float32 ``(B,Hq)``."""
@@ -200,7 +230,9 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
-    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit)
+    if live_tiles is True:
+        live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
+    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit, live_tiles)
     dsink = None
     if _z is not None:
         dsink = torch.empty((B, Hq), dtype=torch.float32, device=query.device)

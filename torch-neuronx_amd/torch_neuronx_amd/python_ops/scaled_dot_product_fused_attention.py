@@ -99,6 +99,17 @@ def _recover_pattern(attn_bias, is_causal, want_grad_bias=False):
     return None, True, {"window": pat[1], "sink_keys": pat[2]}
 
 
+def _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key):
+    """A mask that stays a tensor gets tile skip tables (cached per tensor), so that the kernels leave
+    out the tiles it drops whole - the run-time counterpart of the reference's static tile
+    elimination (neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:15-33)."""
+    if attn_bias is not None and not is_causal and dropout_p == 0.0 and query.dtype in (torch.float16, torch.bfloat16):
+        maps = mask_patterns.tile_maps(attn_bias, query.shape[0], query.shape[1], query.shape[2], key.shape[2])
+        if maps is not None:
+            functor = dict(functor, live_tiles=maps)
+    return functor
+
+
 def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale, need_lse=True):
     _check_device(query)
     attn_bias = _present(attn_bias)
@@ -118,6 +129,7 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
     else:
         seed, offset = _empty_rng(query.device)
     attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal)
+    functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     out, lse = ops.sdpa_forward(query, key, value, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
                                 dropout_p=dropout_p, dropout_keep=keep, need_lse=need_lse,
                                 force_kernel=_force_kernel(), **functor)
@@ -154,6 +166,7 @@ def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p,
         else:
             keep = philox_seed
     attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, want_grad_bias)
+    functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     dq, dk, dv, dbias = ops.sdpa_backward(
         grad_out, query, key, value, out, logsumexp, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
         dropout_p=dropout_p, dropout_keep=keep, want_grad_bias=want_grad_bias, force_kernel=_force_kernel(),
