@@ -184,3 +184,10 @@ def test_document_mask_through_the_operator_skips_tiles(amd, gpu_device):
     t_plain = timed(lambda: amd.sdpa_forward(q, k, v, attn_bias=mask, force_kernel=MFMA))
     t_table = timed(lambda: op(q, k, v, attn_bias=mask))
     assert t_table < 0.4 * t_plain, (t_table, t_plain)
+    # ... and so does the backward (dQ walks the live key tiles, dK/dV the live query tiles)
+    go = torch.randn_like(out)
+    lse = op(q, k, v, attn_bias=mask)[1]
+    maps = mask_patterns.tile_maps(mask, B, Hq, n, n)
+    b_plain = timed(lambda: amd.sdpa_backward(go, q, k, v, out, lse, attn_bias=mask, force_kernel=MFMA), 5)
+    b_table = timed(lambda: amd.sdpa_backward(go, q, k, v, out, lse, attn_bias=mask, force_kernel=MFMA, live_tiles=maps), 5)
+    assert b_table < 0.4 * b_plain, (b_table, b_plain)

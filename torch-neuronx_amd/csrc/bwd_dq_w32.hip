@@ -38,8 +38,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr bool SPLIT = 512 > TCH;   // more threads than chunks: one half stages K, the other V
   static_assert(AHEAD <= 2 * DB, "ring");
   constexpr int NBUF = 4;  // tile t lives in buffer t % 4
-  __shared__ __attribute__((aligned(16))) uint16_t k_t[NBUF][TILE];
-  __shared__ __attribute__((aligned(16))) uint16_t v_t[NBUF][TILE];
+  // (the variant with a bias takes the launch's dynamic LDS: behind the tiles it keeps the list of the
+  // key tiles it walks when the call brings a skip table, and a kernel may declare 64 KB at most)
+  constexpr bool DYN = MASK == 2;
+  __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
+  __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : NBUF * TILE];
+  extern __shared__ __attribute__((aligned(16))) uint16_t dyn_lds[];
+  uint16_t (*const k_t)[TILE] = (uint16_t (*)[TILE])(DYN ? dyn_lds : k_static);
+  uint16_t (*const v_t)[TILE] = (uint16_t (*)[TILE])(DYN ? dyn_lds + NBUF * TILE : v_static);
+  uint16_t* const tile_list = dyn_lds + 2 * NBUF * TILE;  // [1024] and the count
 
   int b, h, qt;
   {
@@ -147,7 +154,41 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       nt -= skip;
     }
   }
-  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  // With a skip table (variant with a bias, no bias gradient): the tiles in which the mask keeps at
+  // least one score of this workgroup's rows.  The first wavefront ORs the bitmaps of the
+  // workgroup's 64-row blocks and expands the set bits into a list in LDS, 64 tiles per step.
+  bool listed = false;
+  if constexpr (MASK == 2) {
+    if (p.live_tiles && !p.causal && !p.gbias) {
+      if (wave == 0) {
+        const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
+        const uint32_t* map = p.live_tiles + ((int64_t)((p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? h : 0)) * nrb + rb0) * p.live_words;
+        uint32_t w = 0u;
+        if (lane < p.live_words) {
+#pragma unroll
+          for (int r = 0; r < BM / 64; ++r)
+            if (rb0 + r < nrb) w |= map[r * p.live_words + lane];
+        }
+        int cnt = 0;
+        for (int j0 = 0; j0 < nt; j0 += 64) {
+          const uint32_t ww = __shfl(w, (j0 >> 5) + (lane >> 5), 64);
+          const bool live = j0 + lane < nt && ((ww >> (lane & 31)) & 1u);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(live);
+          if (live) tile_list[cnt + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = (uint16_t)(j0 + lane);
+          cnt += __builtin_popcountll(m);
+        }
+        if (lane == 0) *(int*)(tile_list + 1024) = cnt;
+      }
+      __syncthreads();
+      const int n_live = __builtin_amdgcn_readfirstlane(*(const int*)(tile_list + 1024));
+      listed = n_live < nt;  // (every tile live: the list is the identity)
+      nt = n_live;
+    }
+  }
+  auto tile_of = [&](int u) {
+    if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
+    else return FUNC ? u + (u >= n_lead ? skip : 0) : u;
+  };
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BN + 1 - skip) : nt;  // tiles with work for this wavefront
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile; with a window also every tile that
@@ -281,7 +322,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   const uint32_t b_row = MASK == 2 ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
   auto load_bias = [&](int t) {
     if constexpr (MASK == 2) {
-      const uint32_t off = b_row + (uint32_t)(t * BN * besz);
+      const uint32_t off = b_row + (uint32_t)((listed ? tile_of(min(t, max(nt - 1, 0))) : t) * BN * besz);
       if (bkind == 1) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -316,7 +357,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     else each([](int) { return 0.f; });
   };
   // dS^T of tile t, packed as the B operand of dQ^T += K^T dS^T
-  auto softmax = [&](int t, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
+  auto softmax = [&](int u, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
+    const int t = tile_of(u);  // (stream position -> key tile)
     const bool edge = t >= t_edge;
     float bl[16];
     if constexpr (MASK == 2) bias_log2(bl);
@@ -492,7 +534,18 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const dim3 grid((unsigned)blocks), block(512);
   const bool bf = dtype == MI355_SDPA_BF16;
   const int mask = (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
-#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, 0, s, g)
+  // (the variant with a bias: its tiles, and the tile list of a call with a skip table, in dynamic LDS)
+  const int dyn = mask == 2 ? 2 * 4 * BN * head_dim * 2 + 2048 + 16 : 0;
+  if (mask == 2) {
+    const void* fn = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 2>)
+                                     : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 2>);
+    const hipError_t attr = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, dyn);
+    if (attr != hipSuccess) {
+      set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dq_w32_kernel: %s", dyn, hipGetErrorString(attr));
+      return MI355_SDPA_ERR_LAUNCH;
+    }
+  }
+#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, (MM) == 2 ? dyn : 0, s, g)
 #define LAUNCH_M(TT, DD)                                                     \
   do {                                                                       \
     if (mask == 2) LAUNCH(TT, DD, 2);                                        \

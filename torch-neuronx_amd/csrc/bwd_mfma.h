@@ -46,6 +46,10 @@ struct BwdM {
   // live_hm = the mask's own head extent
   const uint32_t* live_t = nullptr;
   int live_t_words = 0, live_hm = 1;
+  // ... and for the dQ kernel (unless a bias gradient is asked for): per (mask batch, mask head, 64-row
+  // block) a bitmap of the 32-key tiles with a kept score, live_words words each
+  const uint32_t* live_tiles = nullptr;
+  int live_words = 0;
 };
 
 // dot product of eight packed elements, float32 accumulation

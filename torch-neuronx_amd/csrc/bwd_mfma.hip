@@ -545,6 +545,10 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
       g.live_t = p.mask.live_tiles_t;
       g.live_t_words = words_t, g.live_hm = live_extent(p.bias, 1);
     }
+    if (p.mask.live_tiles && !p.is_causal && g.bias_sl != 0 && g.S <= 32768 && !p.grad_bias.data) {
+      g.live_tiles = p.mask.live_tiles;
+      g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
+    }
   }
 }
 
