@@ -1,9 +1,9 @@
 // Flash-attention backward for head dims above 128 and for D_qk != D_v (D_v <= D_qk <= 256,
 // multiples of 8; e.g. 192 / 128 of multi-head latent attention, or 256 / 256), bf16/f16, on the
 // 32x32x16 MFMA.  Two kernels built for the widest case, rows narrower than 256 counting as zero
-// padded; one wavefront per SIMD with the 512-register budget, compiler-scheduled: the point of
-// these kernels is to keep such calls on the matrix pipe (the float32 generic kernels that served
-// them run at 1-2 TFLOP/s), not to match the hand-pipelined kernels for head dims 64 / 128.
+// padded; one wavefront per SIMD with the 512-register budget (the dK/dV kernel holds two 128-register
+// accumulators and two 64-register fragments), LDS operands two or three matrix ops ahead through a
+// register ring in a pinned order.
 //
 //   bwd_wide_dq_kernel    128 query rows per workgroup (4 wavefronts x 32 rows), 32-key tiles:
 //                           S^T = K Q^T, dP^T = V dO^T, dS^T = P^T (dP^T - delta), dQ^T += K^T dS^T
@@ -15,8 +15,8 @@
 //                           S = Q K^T, dP = dO V^T, P = exp2(c S - lse), dS = P (dP - delta)
 //                           dV^T += dO^T P, dK^T += Q^T dS
 //
-// Tiles sit in LDS row-major with a padded pitch; transposed operands come out of the transposing
-// LDS read.  Math follows torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows with
+// Tiles sit in LDS row-major, unpadded and XOR swizzled; transposed operands come out of the
+// transposing LDS read.  Math follows torch_neuronx/_sdpa_math.py:98-176: float32 accumulation, rows with
 // lse = -inf give zero gradients, scale multiplies dQ and dK once at the end.
 #include "bwd_mfma.h"
 
@@ -26,7 +26,6 @@ namespace {
 constexpr int DW = 256;           // the width the kernels are built for
 constexpr int KS = DW / 16;       // contraction steps over the head dim
 constexpr int DB = DW / 32;       // 32-row blocks of a transposed product
-constexpr int PITCH = DW + 8;     // LDS row pitch in elements: 16-byte row reads of 16 lanes hit every bank once
 constexpr int BT = 32;            // rows of a staged tile
 
 typedef short s16x4 __attribute__((ext_vector_type(4)));
@@ -35,53 +34,62 @@ __device__ __forceinline__ u32x2 tr_read(const uint16_t* ptr) {
   return __builtin_bit_cast(u32x2, v);
 }
 
-// A 32-row tile of a (rows, width) matrix on its way to LDS, zero beyond `width` and beyond
-// `rows_left` rows: fetched into registers one tile ahead (the loads travel under the matrix ops
-// of the current tile) and written to LDS between two barriers.  256 threads, 16-byte chunks:
-// chunk c of row r at r * PITCH + 8 c.
-constexpr int NST = (BT * (DW / 8)) / 256;  // chunks per thread and tile
-struct TileRegs {
-  u32x4 w[NST];
-  __device__ __forceinline__ void fetch(const uint16_t* base, int64_t row_stride, int rows_left, int width, int tid) {
-#pragma unroll
-    for (int n = 0; n < NST; ++n) {
-      const int u = tid + n * 256, r = u / (DW / 8), ch = u % (DW / 8);
-      w[n] = u32x4{0u, 0u, 0u, 0u};
-      if (r < rows_left && ch * 8 < width) w[n] = *(const u32x4*)(base + (int64_t)r * row_stride + ch * 8);
-    }
-  }
-  __device__ __forceinline__ void put(uint16_t* lds, int tid) const {
-#pragma unroll
-    for (int n = 0; n < NST; ++n) {
-      const int u = tid + n * 256, r = u / (DW / 8), ch = u % (DW / 8);
-      *(u32x4*)(lds + r * PITCH + ch * 8) = w[n];
-    }
-  }
-};
+// Both kernels stage their 32-row tiles from global memory straight into LDS (buffer loads with the
+// LDS bit, 16 bytes per lane, 1 KB of contiguous LDS per wavefront and instruction), one tile ahead,
+// into two buffers per operand.  The tiles are unpadded and XOR swizzled (tile_swz: the lane that owns
+// LDS chunk position c of row r fetches the row's chunk c ^ tile_swz(r)), which keeps both the row
+// reads and the transposing reads free of bank conflicts (with a padded pitch the transposing reads
+// of four consecutive rows overlap in their banks).  16 loads cover a tile; a chunk past a narrow
+// row's end asks for an offset beyond the buffer and gets zeros, and so do rows past the buffer's end.
+constexpr int TILE_LOADS = BT * (DW / 8) / 64;
+constexpr int TILE_ELEMS = BT * DW;
+constexpr int WIDE_DKDV_LDS = 2 * 2 * TILE_ELEMS * 2 + 2 * 2 * BT * 4;
+constexpr int WIDE_DQ_LDS = 2 * 2 * TILE_ELEMS * 2;
 
-// element offsets of the transposing reads of a tile, [second read of a pair][d block]
-struct TrOff {
+// element offsets of the transposing reads of a swizzled tile, [second read of a pair][d block]
+struct TrOffSwz {
   int off[2][DB];
   __device__ __forceinline__ void init(int lane) {
     const int jj = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
-      for (int db = 0; db < DB; ++db)
-        off[sec][db] = (8 * sec + (g >> 1) * 4 + (jj >> 2)) * PITCH + db * 32 + 16 * (g & 1) + 4 * (jj & 3);
+      for (int db = 0; db < DB; ++db) {
+        const int row = 8 * sec + (g >> 1) * 4 + (jj >> 2), d = db * 32 + 16 * (g & 1) + 4 * (jj & 3);
+        off[sec][db] = row * DW + (((d >> 3) ^ tile_swz<DW>(row)) << 3) + (d & 7);
+      }
   }
-  // operand i = DB * (16-row step) + d block of the transposed tile
+  // operand i = DB * (16-row step) + d block of the transposed tile (rows 16 apart share a swizzle)
   __device__ __forceinline__ u32x4 cols(const uint16_t* tile, int i) const {
-    const u32x2 lo = tr_read(tile + off[0][i % DB] + (i / DB) * 16 * PITCH);
-    const u32x2 hi = tr_read(tile + off[1][i % DB] + (i / DB) * 16 * PITCH);
+    const u32x2 lo = tr_read(tile + off[0][i % DB] + (i / DB) * 16 * DW);
+    const u32x2 hi = tr_read(tile + off[1][i % DB] + (i / DB) * 16 * DW);
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   }
 };
 
+// raw buffer resource, in scalar registers
+__device__ __forceinline__ u32x4 wide_descriptor(const void* base, int64_t bytes) {
+  const uint64_t a = (uint64_t)base;
+  return u32x4{(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)a),
+               (uint32_t)__builtin_amdgcn_readfirstlane((int)((uint32_t)(a >> 32) & 0xffffu)),
+               (uint32_t)__builtin_amdgcn_readfirstlane((int)bytes), 0x00020000u};
+}
+// (m0 holds the LDS address of such a load, one wait state after it is written)
+__device__ __forceinline__ void wide_tile_load(const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
+  asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dwordx4 %1, %2, 0 offen lds"
+               :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
+}
+// byte offset of this lane's chunk of load `ld` inside a tile whose first row is the buffer's base
+__device__ __forceinline__ uint32_t wide_chunk_off(int ld, int lane, int row_stride, int width) {
+  const int pos = ld * 64 + lane, r = pos / (DW / 8), ch = (pos % (DW / 8)) ^ tile_swz<DW>(r);
+  return ch * 8 < width ? (uint32_t)((r * row_stride + ch * 8) * 2) : 0xfffffff0u;
+}
+
 template <typename T>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
-  __shared__ __attribute__((aligned(16))) uint16_t k_t[BT * PITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t v_t[BT * PITCH];
+  extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
+  uint16_t* const k_buf = wide_lds;                    // [2][TILE_ELEMS]
+  uint16_t* const v_buf = wide_lds + 2 * TILE_ELEMS;   // [2][TILE_ELEMS]
   const int n_qt = (p.L + 127) / 128;
   const int qt = n_qt - 1 - blockIdx.x / (p.B * p.Hq);  // heavy query tiles first
   const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
@@ -114,8 +122,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
     dl = dsum;
     if (qrow < p.L && half == 0) p.delta[idx] = dsum, p.lse2[idx] = l != -INFINITY ? l * kLog2eF : INFINITY;
   }
-  TrOff tr;
+  TrOffSwz tr;
   tr.init(lane);
+  const int swz_col = tile_swz<DW>(col);
   f32x16 dqacc[DB];
 #pragma unroll
   for (int i = 0; i < DB; ++i) zero(dqacc[i]);
@@ -128,42 +137,85 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;  // tiles with work for this wavefront
   const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
 
-  TileRegs kn, vn;
-  if (nt > 0) kn.fetch(kp, p.k_sl, p.S, er, tid), vn.fetch(vp, p.v_sl, p.S, dvr, tid);
-  for (int t = 0; t < nt; ++t) {
-    __syncthreads();  // the previous tile has been read by every wavefront
-    kn.put(k_t, tid), vn.put(v_t, tid);
+  // the buffers end with the last key row: rows of a ragged last tile beyond it read as zeros
+  const u32x4 k_rsrc = wide_descriptor(kp, ((int64_t)(p.S - 1) * p.k_sl + er) * 2);
+  const u32x4 v_rsrc = wide_descriptor(vp, ((int64_t)(p.S - 1) * p.v_sl + dvr) * 2);
+  typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
+  const uint32_t lds_k = (uint32_t)(uintptr_t)(lds_bytes)k_buf, lds_v = (uint32_t)(uintptr_t)(lds_bytes)v_buf;
+  uint32_t k_off[TILE_LOADS / 4], v_off[TILE_LOADS / 4];
+#pragma unroll
+  for (int n = 0; n < TILE_LOADS / 4; ++n) {
+    k_off[n] = wide_chunk_off(wave + 4 * n, lane, (int)p.k_sl, er);
+    v_off[n] = wide_chunk_off(wave + 4 * n, lane, (int)p.v_sl, dvr);
+  }
+  auto request_tile = [&](int t) {  // tile t into buffer t % 2
+    const uint32_t kt = (uint32_t)(t * BT * p.k_sl * 2), vt = (uint32_t)(t * BT * p.v_sl * 2);
+    const uint32_t boff = (uint32_t)((t & 1) * TILE_ELEMS * 2);
+#pragma unroll
+    for (int n = 0; n < TILE_LOADS / 4; ++n) {
+      // (an offset that stands for "no such chunk" stays beyond the buffer whatever the tile)
+      wide_tile_load(k_rsrc, k_off[n] >= 0xfffffff0u ? k_off[n] : k_off[n] + kt, lds_k + boff + (wave + 4 * n) * 1024);
+      wide_tile_load(v_rsrc, v_off[n] >= 0xfffffff0u ? v_off[n] : v_off[n] + vt, lds_v + boff + (wave + 4 * n) * 1024);
+    }
+  };
+  auto publish_tile = [&]() {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
-    if (t + 1 < nt) {
-      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, p.S - (t + 1) * BT, er, tid);
-      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, p.S - (t + 1) * BT, dvr, tid);
-    }
-    if (t >= nt_w) continue;
-    f32x16 sacc = zero16, dpacc = zero16;
+  };
+  if (nt > 0) {
+    request_tile(0);
+    publish_tile();
+  }
+  for (int t = 0; t < nt; ++t) {
+    // (the other buffer was last read before the barrier that ended the previous tile)
+    if (t + 1 < nt) request_tile(t + 1);
+    if (t < nt_w) {
+      const uint16_t* k_t = k_buf + (t & 1) * TILE_ELEMS;
+      const uint16_t* v_t = v_buf + (t & 1) * TILE_ELEMS;
+      // The 48 LDS operands of a tile - row fragments of K and V in turns, then the transposed
+      // fragments of K - travel through a register ring, three matrix ops ahead of their use, in an
+      // order pinned by scheduling fences (one wavefront per SIMD has nobody to hide an LDS round trip behind).
+      constexpr int AHEAD = 3;
+      auto operand = [&](int n) {
+        if (n < 2 * KS) return *(const u32x4*)(((n & 1) ? v_t : k_t) + col * DW + (((2 * (n >> 1) + half) ^ swz_col) << 3));
+        return tr.cols(k_t, n - 2 * KS);
+      };
+      u32x4 ring[8];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      sacc = Mma<T>::run(*(const u32x4*)(k_t + col * PITCH + ks * 16 + half * 8), qf[ks], sacc);
-      dpacc = Mma<T>::run(*(const u32x4*)(v_t + col * PITCH + ks * 16 + half * 8), dof[ks], dpacc);
-    }
-    uint32_t pS[8];
+      for (int n = 0; n < AHEAD; ++n) ring[n] = operand(n);
+      f32x16 sacc = zero16, dpacc = zero16;
 #pragma unroll
-    for (int r = 0; r < 16; r += 2) {
-      float ds[2];
-#pragma unroll
-      for (int e = 0; e < 2; ++e) {
-        const int kv = t * BT + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
-        float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
-        pr = kv > lim ? 0.f : pr;
-        ds[e] = pr * (dpacc[r + e] - dl);
+      for (int n = 0; n < 2 * KS; ++n) {
+        ring[(n + AHEAD) & 7] = operand(n + AHEAD);
+        if (n & 1) dpacc = Mma<T>::run(ring[n & 7], dof[n >> 1], dpacc);
+        else sacc = Mma<T>::run(ring[n & 7], qf[n >> 1], sacc);
+        __builtin_amdgcn_sched_barrier(0);
       }
-      pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
-    }
+      uint32_t pS[8];
 #pragma unroll
-    for (int i = 0; i < 2 * DB; ++i) {
-      const int r0 = (i / DB) * 4;
-      const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
-      dqacc[i % DB] = Mma<T>::run(tr.cols(k_t, i), bS, dqacc[i % DB]);
+      for (int r = 0; r < 16; r += 2) {
+        float ds[2];
+#pragma unroll
+        for (int e = 0; e < 2; ++e) {
+          const int kv = t * BT + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
+          float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+          pr = kv > lim ? 0.f : pr;
+          ds[e] = pr * (dpacc[r + e] - dl);
+        }
+        pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int i = 0; i < 2 * DB; ++i) {
+        const int n = 2 * KS + i;
+        if (i + AHEAD < 2 * DB) ring[(n + AHEAD) & 7] = operand(n + AHEAD);
+        const int r0 = (i / DB) * 4;
+        const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
+        dqacc[i % DB] = Mma<T>::run(ring[n & 7], bS, dqacc[i % DB]);
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
+    if (t + 1 < nt) publish_tile();
   }
   if (qrow < p.L) {
     uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
@@ -181,10 +233,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
 
 template <typename T>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
-  __shared__ __attribute__((aligned(16))) uint16_t q_t[BT * PITCH];
-  __shared__ __attribute__((aligned(16))) uint16_t do_t[BT * PITCH];
-  __shared__ __attribute__((aligned(16))) float lse_s[BT];
-  __shared__ __attribute__((aligned(16))) float dl_s[BT];
+  extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
+  uint16_t* const q_buf = wide_lds;                        // [2][TILE_ELEMS]
+  uint16_t* const do_buf = wide_lds + 2 * TILE_ELEMS;      // [2][TILE_ELEMS]
+  float* const lse_buf = (float*)(wide_lds + 4 * TILE_ELEMS);  // [2][BT]
+  float* const dl_buf = lse_buf + 2 * BT;                      // [2][BT]
   const int streams = p.B * p.Hkv;
   const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
   const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
@@ -203,8 +256,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       vf[ks] = half * 8 + ks * 16 < dvr ? *(const u32x4*)(vr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
     }
   }
-  TrOff tr;
+  TrOffSwz tr;
   tr.init(lane);
+  const int swz_col = tile_swz<DW>(col);
   f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
   for (int i = 0; i < DB; ++i) zero(dkacc[i]), zero(dvacc[i]);
@@ -213,33 +267,59 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   const int nqs = (p.L + BT - 1) / BT;
   const int qs_begin = p.causal ? min(k0 / BT, nqs) : 0;
 
-  // (no fetch ahead here: the two accumulators and the two fragments fill the register file, and the
-  // 32 registers of a tile in flight spill)
-  // Query tile by query tile from the last one down, heads inside: the workgroups of a kv head, which
-  // share an XCD, then want the same Q / dO tile at about the same time and find it in its L2.
+  // Items: query tile by query tile from the last one down, heads inside: the workgroups of a kv head,
+  // which share an XCD, then want the same Q / dO tile at about the same time and find it in its L2.
+  const int n_items = (nqs - qs_begin) * rep;
+  typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
+  const uint32_t lds_q = (uint32_t)(uintptr_t)(lds_bytes)q_buf, lds_do = (uint32_t)(uintptr_t)(lds_bytes)do_buf;
+  constexpr int NLD = TILE_LOADS / 4;  // loads per wavefront and tile
+  // item `it` into buffer it % 2; the row statistics travel in two registers of the first 32 threads.
+  // The buffers start at the tile's first row and end with the head's last row: rows past L read as zeros.
+  float lse_n = INFINITY, dl_n = 0.f;
+  auto request_item = [&](int qs, int hg, int buf) {
+    const int h = hk * rep + hg, q0 = qs * BT;
+    if (tid < BT) {  // (ordinary loads, ahead of the tile loads: the compiler's wait for them then waits for nothing else)
+      const int qi = q0 + tid;
+      const int64_t row = ((int64_t)b * p.Hq + h) * p.L + min(qi, p.L - 1);
+      // rows past L are switched off through lse = +inf
+      lse_n = qi < p.L ? p.lse2[row] : INFINITY;
+      dl_n = qi < p.L ? p.delta[row] : 0.f;
+    }
+    const int rows = p.L - q0;  // >= 1
+    const u32x4 q_rsrc = wide_descriptor((const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)q0 * p.q_sl, ((int64_t)(rows - 1) * p.q_sl + er) * 2);
+    const u32x4 go_rsrc = wide_descriptor((const uint16_t*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)q0 * p.go_sl, ((int64_t)(rows - 1) * p.go_sl + dvr) * 2);
+    const uint32_t boff = (uint32_t)(buf * TILE_ELEMS * 2);
+#pragma unroll
+    for (int n = 0; n < NLD; ++n) {
+      const int ld = wave + 4 * n;  // (uniform per wavefront)
+      // (offsets recomputed per item, a handful of vector instructions, rather than held in registers
+      // that this kernel does not have)
+      wide_tile_load(q_rsrc, wide_chunk_off(ld, lane, (int)p.q_sl, er), lds_q + boff + ld * 1024);
+      wide_tile_load(go_rsrc, wide_chunk_off(ld, lane, (int)p.go_sl, dvr), lds_do + boff + ld * 1024);
+    }
+  };
+  auto publish_item = [&](int buf) {  // after this, the item in `buf` may be read by every wavefront
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    if (tid < BT) lse_buf[buf * BT + tid] = lse_n, dl_buf[buf * BT + tid] = dl_n;
+    __syncthreads();
+  };
+  if (n_items > 0) {
+    request_item(nqs - 1, 0, 0);
+    publish_item(0);
+  }
+  int buf = 0;
+  // (two nested loops on purpose: written as one loop over items, the compiler spills the fragments)
   for (int qs = nqs - 1; qs >= qs_begin; --qs) {
     for (int hg = 0; hg < rep; ++hg) {
-      const int h = hk * rep + hg;
-      const uint16_t* qb = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh;
-      const uint16_t* gb = (const uint16_t*)p.go + b * p.go_sb + h * p.go_sh;
-      const int64_t row0 = ((int64_t)b * p.Hq + h) * p.L;
-      const int q0 = qs * BT;
-      __syncthreads();  // the previous tile has been read by every wavefront
-      {
-        TileRegs qn;
-        qn.fetch(qb + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, er, tid);
-        qn.put(q_t, tid);
-        qn.fetch(gb + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, dvr, tid);
-        qn.put(do_t, tid);
-      }
-      if (tid < BT) {
-        const int qi = q0 + tid;
-        // rows past L are switched off through lse = +inf
-        lse_s[tid] = qi < p.L ? p.lse2[row0 + qi] : INFINITY;
-        dl_s[tid] = qi < p.L ? p.delta[row0 + qi] : 0.f;
-      }
-      __syncthreads();
-      if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= p.S) continue;  // (uniform per wavefront)
+    const bool last = qs == qs_begin && hg == rep - 1;
+    // (the other buffer was last read before the barrier that ended the previous item)
+    if (!last) request_item(hg + 1 < rep ? qs : qs - 1, hg + 1 < rep ? hg + 1 : 0, buf ^ 1);
+    const int q0 = qs * BT;
+    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= p.S)) {  // (uniform per wavefront)
+      const uint16_t* q_t = q_buf + buf * TILE_ELEMS;
+      const uint16_t* do_t = do_buf + buf * TILE_ELEMS;
+      const float* lse_s = lse_buf + buf * BT;
+      const float* dl_s = dl_buf + buf * BT;
       // the accumulators are touched by matrix ops only: accumulation registers; the K / V fragments
       // feed every matrix op as a source operand: ordinary vector registers
 #pragma unroll
@@ -247,36 +327,79 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
         asm volatile("" : "+a"(dkacc[i]));
         asm volatile("" : "+a"(dvacc[i]));
       }
-      f32x16 sacc = zero16, dpacc = zero16;
+      // Scores, then dP, through one accumulator (holding both at once is what the register file has
+      // no room for next to the two fragments; dS is formed from the probabilities as they feed the
+      // matrix pipe, rounded to the input dtype).  The 64 LDS operands of an item - 16 row fragments
+      // of Q, 16 of dO, then the transposed fragments of dO and Q in turns - travel through one
+      // register ring, two matrix ops ahead of their use, with the order pinned by scheduling
+      // fences: one wavefront per SIMD has nobody else to hide an LDS round trip behind.
+      constexpr int AHEAD = 2;
+      auto operand = [&](int n) {
+        if (n < KS) return *(const u32x4*)(q_t + col * DW + (((2 * n + half) ^ swz_col) << 3));
+        if (n < 2 * KS) return *(const u32x4*)(do_t + col * DW + (((2 * (n - KS) + half) ^ swz_col) << 3));
+        return ((n - 2 * KS) & 1) ? tr.cols(q_t, (n - 2 * KS) >> 1) : tr.cols(do_t, (n - 2 * KS) >> 1);
+      };
+      u32x4 ring[8];
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        sacc = Mma<T>::run(*(const u32x4*)(q_t + col * PITCH + ks * 16 + half * 8), kf[ks], sacc);
-        dpacc = Mma<T>::run(*(const u32x4*)(do_t + col * PITCH + ks * 16 + half * 8), vf[ks], dpacc);
-      }
+      for (int n = 0; n < AHEAD; ++n) ring[n] = operand(n);
       uint32_t pP[8], pS[8];
+      {
+        f32x16 sacc = zero16;
 #pragma unroll
-      for (int r4 = 0; r4 < 4; ++r4) {
-        const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
-        const f32x4 d4 = *(const f32x4*)(&dl_s[r4 * 8 + half * 4]);
-        float pr[4], ds[4];
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
-          pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
-          pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
-          ds[e] = pr[e] * (dpacc[r] - d4[e]);
+        for (int n = 0; n < KS; ++n) {
+          ring[(n + AHEAD) & 7] = operand(n + AHEAD);
+          sacc = Mma<T>::run(ring[n & 7], kf[n], sacc);
+          __builtin_amdgcn_sched_barrier(0);
         }
-        pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
-        pS[r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
+          float pr[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
+            pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
+            pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
+          }
+          pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      {
+        f32x16 dpacc = zero16;
+#pragma unroll
+        for (int n = KS; n < 2 * KS; ++n) {
+          ring[(n + AHEAD) & 7] = operand(n + AHEAD);
+          dpacc = Mma<T>::run(ring[n & 7], vf[n - KS], dpacc);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const f32x4 d4 = *(const f32x4*)(&dl_s[r4 * 8 + half * 4]);
+          float ds[4];
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            ds[e] = Mma<T>::unpack(pP[r4 * 2 + (e >> 1)], e & 1) * (dpacc[r4 * 4 + e] - d4[e]);
+          pS[r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
-      for (int i = 0; i < 2 * DB; ++i) {
-        const int r0 = (i / DB) * 4;
-        const u32x4 bP = {pP[r0], pP[r0 + 1], pP[r0 + 2], pP[r0 + 3]};
-        const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
-        dvacc[i % DB] = Mma<T>::run(tr.cols(do_t, i), bP, dvacc[i % DB]);
-        dkacc[i % DB] = Mma<T>::run(tr.cols(q_t, i), bS, dkacc[i % DB]);
+      for (int n = 2 * KS; n < 2 * KS + 4 * DB; ++n) {
+        if (n + AHEAD < 2 * KS + 4 * DB) ring[(n + AHEAD) & 7] = operand(n + AHEAD);
+        const int i = (n - 2 * KS) >> 1, r0 = (i / DB) * 4;
+        if ((n - 2 * KS) & 1) {
+          const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
+          dkacc[i % DB] = Mma<T>::run(ring[n & 7], bS, dkacc[i % DB]);
+        } else {
+          const u32x4 bP = {pP[r0], pP[r0 + 1], pP[r0 + 2], pP[r0 + 3]};
+          dvacc[i % DB] = Mma<T>::run(ring[n & 7], bP, dvacc[i % DB]);
+        }
+        __builtin_amdgcn_sched_barrier(0);
       }
+    }
+    buf ^= 1;
+    if (!last) publish_item(buf);
     }
   }
   if (key < p.S) {
@@ -304,10 +427,22 @@ int launch_t(const BwdM& g, hipStream_t s) {
     set_error("SDPA: too many tiles for the wide backward kernels");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  hipLaunchKernelGGL((bwd_wide_dq_kernel<T>), dim3((unsigned)q_blocks), dim3(256), 0, s, g);
+  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T>,
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DQ_LDS);
+  if (attr_q != hipSuccess) {
+    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", WIDE_DQ_LDS, hipGetErrorString(attr_q));
+    return MI355_SDPA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((bwd_wide_dq_kernel<T>), dim3((unsigned)q_blocks), dim3(256), WIDE_DQ_LDS, s, g);
   int rc = check_launch("bwd_wide_dq_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T>), dim3((unsigned)k_blocks), dim3(256), 0, s, g);
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DKDV_LDS);
+  if (attr != hipSuccess) {
+    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", WIDE_DKDV_LDS, hipGetErrorString(attr));
+    return MI355_SDPA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T>), dim3((unsigned)k_blocks), dim3(256), WIDE_DKDV_LDS, s, g);
   return check_launch("bwd_wide_dkdv_kernel");
 }
 
