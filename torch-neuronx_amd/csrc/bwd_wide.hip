@@ -85,8 +85,70 @@ __device__ __forceinline__ uint32_t wide_chunk_off(int ld, int lane, int row_str
   return ch * 8 < width ? (uint32_t)((r * row_stride + ch * 8) * 2) : 0xfffffff0u;
 }
 
-template <typename T>
+// compile-time loop: f(std::integral_constant<int, 0>{}) ... f(std::integral_constant<int, N - 1>{})
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_impl(F&& f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F&& f) {
+  static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+// The kernels are instantiated for the widths they serve, ER for Q / K and DVR for V / dO / O
+// (multiples of 32 up to 256): contraction steps and output blocks that would lie wholly in the
+// zero padding of the 256-wide layout do not exist in the instruction stream, nor do the registers
+// of their fragments and accumulators (192 / 128: 40 matrix ops per item instead of 64 in the
+// dK/dV kernel, 32 instead of 48 in the dQ kernel).  An item's LDS operands in the order of their use:
+struct WideOp {
+  int kind, j;  // dQ kernel: 0 K rows (S), 1 V rows (dP), 2 K^T columns (dQ); dK/dV kernel: 0 Q rows (S), 1 dO rows (dP),
+                // 2 dO^T columns (dV), 3 Q^T columns (dK); j = contraction step, or DB * (16-row step) + d block
+};
+template <int ER, int DVR>
+constexpr WideOp dq_op(int k) {  // S and dP steps in turns, then the columns of K^T
+  constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32;
+  int c = 0;
+  for (int j = 0; j < (KSE > KSV ? KSE : KSV); ++j) {
+    if (j < KSE) {
+      if (c == k) return {0, j};
+      ++c;
+    }
+    if (j < KSV) {
+      if (c == k) return {1, j};
+      ++c;
+    }
+  }
+  return {2, ((k - c) / DBE) * DB + (k - c) % DBE};
+}
+template <int ER, int DVR>
+constexpr WideOp dkdv_op(int k) {  // S steps and dP steps (in turns where both accumulators fit: two
+                                   // independent chains), the columns of dO^T, the columns of Q^T
+  constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32, DBV = DVR / 32;
+  if (k < KSE + KSV) {
+    if constexpr (ER + DVR <= 320) {
+      int c = 0;
+      for (int j = 0; j < (KSE > KSV ? KSE : KSV); ++j) {
+        if (j < KSE) {
+          if (c == k) return {0, j};
+          ++c;
+        }
+        if (j < KSV) {
+          if (c == k) return {1, j};
+          ++c;
+        }
+      }
+    }
+    return k < KSE ? WideOp{0, k} : WideOp{1, k - KSE};
+  }
+  k -= KSE + KSV;
+  if (k < 2 * DBV) return {2, (k / DBV) * DB + k % DBV};
+  k -= 2 * DBV;
+  return {3, (k / DBE) * DB + k % DBE};
+}
+
+template <typename T, int ER, int DVR>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
+  constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const k_buf = wide_lds;                    // [2][TILE_ELEMS]
   uint16_t* const v_buf = wide_lds + 2 * TILE_ELEMS;   // [2][TILE_ELEMS]
@@ -97,7 +159,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   const int q0 = qt * 128, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
   const int er = p.d_real, dvr = p.dv_real;
 
-  u32x4 qf[KS], dof[KS];
+  u32x4 qf[KSE], dof[KSV];
   float lse2, dl;
   {
     const uint16_t* qr = (const uint16_t*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl + half * 8;
@@ -105,8 +167,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
     const uint16_t* orow = (const uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qc * p.o_sl + half * 8;
     float dsum = 0.f;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      qf[ks] = half * 8 + ks * 16 < er ? *(const u32x4*)(qr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
+    for (int ks = 0; ks < KSE; ++ks) qf[ks] = half * 8 + ks * 16 < er ? *(const u32x4*)(qr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int ks = 0; ks < KSV; ++ks) {
       if (half * 8 + ks * 16 < dvr) {
         dof[ks] = *(const u32x4*)(gr + ks * 16);
         dsum += dot8<T>(dof[ks], *(const u32x4*)(orow + ks * 16));
@@ -125,9 +188,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   TrOffSwz tr;
   tr.init(lane);
   const int swz_col = tile_swz<DW>(col);
-  f32x16 dqacc[DB];
+  f32x16 dqacc[DBE];
 #pragma unroll
-  for (int i = 0; i < DB; ++i) zero(dqacc[i]);
+  for (int i = 0; i < DBE; ++i) zero(dqacc[i]);
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
@@ -172,25 +235,26 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
     if (t < nt_w) {
       const uint16_t* k_t = k_buf + (t & 1) * TILE_ELEMS;
       const uint16_t* v_t = v_buf + (t & 1) * TILE_ELEMS;
-      // The 48 LDS operands of a tile - row fragments of K and V in turns, then the transposed
-      // fragments of K - travel through a register ring, three matrix ops ahead of their use, in an
-      // order pinned by scheduling fences (one wavefront per SIMD has nobody to hide an LDS round trip behind).
-      constexpr int AHEAD = 3;
-      auto operand = [&](int n) {
-        if (n < 2 * KS) return *(const u32x4*)(((n & 1) ? v_t : k_t) + col * DW + (((2 * (n >> 1) + half) ^ swz_col) << 3));
-        return tr.cols(k_t, n - 2 * KS);
+      // The LDS operands of a tile - row fragments of K and V in turns, then the transposed fragments
+      // of K - travel through a register ring, three matrix ops ahead of their use, in an order
+      // pinned by scheduling fences (one wavefront per SIMD has nobody to hide an LDS round trip behind).
+      constexpr int AHEAD = 3, NA = KSE + KSV, NOPS = NA + 2 * DBE;
+      auto operand = [&](auto kc) {
+        constexpr WideOp op = dq_op<ER, DVR>(decltype(kc)::value);
+        if constexpr (op.kind == 2) return tr.cols(k_t, op.j);
+        else return *(const u32x4*)((op.kind ? v_t : k_t) + col * DW + (((2 * op.j + half) ^ swz_col) << 3));
       };
       u32x4 ring[8];
-#pragma unroll
-      for (int n = 0; n < AHEAD; ++n) ring[n] = operand(n);
+      static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       f32x16 sacc = zero16, dpacc = zero16;
-#pragma unroll
-      for (int n = 0; n < 2 * KS; ++n) {
-        ring[(n + AHEAD) & 7] = operand(n + AHEAD);
-        if (n & 1) dpacc = Mma<T>::run(ring[n & 7], dof[n >> 1], dpacc);
-        else sacc = Mma<T>::run(ring[n & 7], qf[n >> 1], sacc);
+      static_for<NA>([&](auto kc) {
+        constexpr int k = decltype(kc)::value;
+        constexpr WideOp op = dq_op<ER, DVR>(k);
+        ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
+        if constexpr (op.kind) dpacc = Mma<T>::run(ring[k & 7], dof[op.j], dpacc);
+        else sacc = Mma<T>::run(ring[k & 7], qf[op.j], sacc);
         __builtin_amdgcn_sched_barrier(0);
-      }
+      });
       uint32_t pS[8];
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
@@ -205,22 +269,22 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
       }
       __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-      for (int i = 0; i < 2 * DB; ++i) {
-        const int n = 2 * KS + i;
-        if (i + AHEAD < 2 * DB) ring[(n + AHEAD) & 7] = operand(n + AHEAD);
-        const int r0 = (i / DB) * 4;
+      static_for<2 * DBE>([&](auto ic) {
+        constexpr int k = NA + decltype(ic)::value;
+        constexpr WideOp op = dq_op<ER, DVR>(k);
+        if constexpr (k + AHEAD < NOPS) ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
+        constexpr int r0 = (op.j / DB) * 4;
         const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
-        dqacc[i % DB] = Mma<T>::run(ring[n & 7], bS, dqacc[i % DB]);
+        dqacc[op.j % DB] = Mma<T>::run(ring[k & 7], bS, dqacc[op.j % DB]);
         __builtin_amdgcn_sched_barrier(0);
-      }
+      });
     }
     if (t + 1 < nt) publish_tile();
   }
   if (qrow < p.L) {
     uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int db = 0; db < DBE; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 w;
@@ -231,8 +295,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   }
 }
 
-template <typename T>
+template <typename T, int ER, int DVR>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
+  constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32, DBV = DVR / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const q_buf = wide_lds;                        // [2][TILE_ELEMS]
   uint16_t* const do_buf = wide_lds + 2 * TILE_ELEMS;      // [2][TILE_ELEMS]
@@ -245,23 +310,24 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   const int k0 = kt * 128, kw0 = k0 + wave * 32, key = kw0 + col;
   const int er = p.d_real, dvr = p.dv_real;
 
-  u32x4 kf[KS], vf[KS];
+  u32x4 kf[KSE], vf[KSV];
   {
     const int kc = min(key, p.S - 1);
     const uint16_t* kr = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl + half * 8;
     const uint16_t* vr = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl + half * 8;
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      kf[ks] = half * 8 + ks * 16 < er ? *(const u32x4*)(kr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
-      vf[ks] = half * 8 + ks * 16 < dvr ? *(const u32x4*)(vr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
-    }
+    for (int ks = 0; ks < KSE; ++ks) kf[ks] = half * 8 + ks * 16 < er ? *(const u32x4*)(kr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
+#pragma unroll
+    for (int ks = 0; ks < KSV; ++ks) vf[ks] = half * 8 + ks * 16 < dvr ? *(const u32x4*)(vr + ks * 16) : u32x4{0u, 0u, 0u, 0u};
   }
   TrOffSwz tr;
   tr.init(lane);
   const int swz_col = tile_swz<DW>(col);
-  f32x16 dkacc[DB], dvacc[DB];
+  f32x16 dkacc[DBE], dvacc[DBV];
 #pragma unroll
-  for (int i = 0; i < DB; ++i) zero(dkacc[i]), zero(dvacc[i]);
+  for (int i = 0; i < DBE; ++i) zero(dkacc[i]);
+#pragma unroll
+  for (int i = 0; i < DBV; ++i) zero(dvacc[i]);
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int nqs = (p.L + BT - 1) / BT;
@@ -323,56 +389,57 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       // the accumulators are touched by matrix ops only: accumulation registers; the K / V fragments
       // feed every matrix op as a source operand: ordinary vector registers
 #pragma unroll
-      for (int i = 0; i < DB; ++i) {
-        asm volatile("" : "+a"(dkacc[i]));
-        asm volatile("" : "+a"(dvacc[i]));
-      }
-      // Scores, then dP, through one accumulator (holding both at once is what the register file has
-      // no room for next to the two fragments; dS is formed from the probabilities as they feed the
-      // matrix pipe, rounded to the input dtype).  The 64 LDS operands of an item - 16 row fragments
-      // of Q, 16 of dO, then the transposed fragments of dO and Q in turns - travel through one
-      // register ring, two matrix ops ahead of their use, with the order pinned by scheduling
-      // fences: one wavefront per SIMD has nobody else to hide an LDS round trip behind.
-      constexpr int AHEAD = 2;
-      auto operand = [&](int n) {
-        if (n < KS) return *(const u32x4*)(q_t + col * DW + (((2 * n + half) ^ swz_col) << 3));
-        if (n < 2 * KS) return *(const u32x4*)(do_t + col * DW + (((2 * (n - KS) + half) ^ swz_col) << 3));
-        return ((n - 2 * KS) & 1) ? tr.cols(q_t, (n - 2 * KS) >> 1) : tr.cols(do_t, (n - 2 * KS) >> 1);
+      for (int i = 0; i < DBE; ++i) asm volatile("" : "+a"(dkacc[i]));
+#pragma unroll
+      for (int i = 0; i < DBV; ++i) asm volatile("" : "+a"(dvacc[i]));
+      // The matrix ops of an item in the order S, dP, dV, dK, with the vector work between them placed
+      // where the matrix pipe still has the previous ops to execute: the probabilities are formed
+      // while dP runs, dS (from the probabilities as they feed the matrix pipe, rounded to the input
+      // dtype) while dV runs.  One wavefront per SIMD has nobody else to overlap with.  The LDS
+      // operands - row fragments of Q, then of dO, then the transposed fragments of dO, then of Q -
+      // travel through one register ring, two to four matrix ops ahead of their use, with the order
+      // pinned by scheduling fences.
+      constexpr int AHEAD = ER + DVR <= 320 ? 4 : 2, NOPS = KSE + KSV + 2 * (DBE + DBV);  // (deeper where the widths leave registers)
+      auto operand = [&](auto kc) {
+        constexpr WideOp op = dkdv_op<ER, DVR>(decltype(kc)::value);
+        if constexpr (op.kind >= 2) return tr.cols(op.kind == 3 ? q_t : do_t, op.j);
+        else return *(const u32x4*)((op.kind ? do_t : q_t) + col * DW + (((2 * op.j + half) ^ swz_col) << 3));
       };
       u32x4 ring[8];
-#pragma unroll
-      for (int n = 0; n < AHEAD; ++n) ring[n] = operand(n);
+      static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       uint32_t pP[8], pS[8];
-      {
-        f32x16 sacc = zero16;
-#pragma unroll
-        for (int n = 0; n < KS; ++n) {
-          ring[(n + AHEAD) & 7] = operand(n + AHEAD);
-          sacc = Mma<T>::run(ring[n & 7], kf[n], sacc);
+      // (at full width the register file has no room for the score and the dP accumulator at once next
+      // to the two fragments: there the probabilities are formed before dP is issued, uncovered)
+      constexpr bool BOTH = ER + DVR <= 320;
+      f32x16 sacc = zero16, dpacc = zero16;
+      auto issue = [&](auto first, auto count) {  // ops first .. first + count - 1 of the S / dP part
+        static_for<decltype(count)::value>([&](auto jc) {
+          constexpr int k = decltype(first)::value + decltype(jc)::value;
+          constexpr WideOp op = dkdv_op<ER, DVR>(k);
+          ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
+          if constexpr (op.kind) dpacc = Mma<T>::run(ring[k & 7], vf[op.j], dpacc);
+          else sacc = Mma<T>::run(ring[k & 7], kf[op.j], sacc);
           __builtin_amdgcn_sched_barrier(0);
-        }
+        });
+      };
+      auto issue_dp = [&]() { issue(std::integral_constant<int, KSE>{}, std::integral_constant<int, KSV>{}); };
+      if constexpr (BOTH) issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE + KSV>{});
+      else issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE>{});
 #pragma unroll
-        for (int r4 = 0; r4 < 4; ++r4) {
-          const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
-          float pr[4];
+      for (int r4 = 0; r4 < 4; ++r4) {
+        const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
+        float pr[4];
 #pragma unroll
-          for (int e = 0; e < 4; ++e) {
-            const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
-            pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
-            pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
-          }
-          pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+        for (int e = 0; e < 4; ++e) {
+          const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
+          pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
+          pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
         }
-        __builtin_amdgcn_sched_barrier(0);
+        pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
       }
-      {
-        f32x16 dpacc = zero16;
-#pragma unroll
-        for (int n = KS; n < 2 * KS; ++n) {
-          ring[(n + AHEAD) & 7] = operand(n + AHEAD);
-          dpacc = Mma<T>::run(ring[n & 7], vf[n - KS], dpacc);
-          __builtin_amdgcn_sched_barrier(0);
-        }
+      __builtin_amdgcn_sched_barrier(0);
+      if constexpr (!BOTH) issue_dp();
+      auto form_ds = [&]() {
 #pragma unroll
         for (int r4 = 0; r4 < 4; ++r4) {
           const f32x4 d4 = *(const f32x4*)(&dl_s[r4 * 8 + half * 4]);
@@ -383,20 +450,27 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
           pS[r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
         }
         __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int n = 2 * KS; n < 2 * KS + 4 * DB; ++n) {
-        if (n + AHEAD < 2 * KS + 4 * DB) ring[(n + AHEAD) & 7] = operand(n + AHEAD);
-        const int i = (n - 2 * KS) >> 1, r0 = (i / DB) * 4;
-        if ((n - 2 * KS) & 1) {
-          const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
-          dkacc[i % DB] = Mma<T>::run(ring[n & 7], bS, dkacc[i % DB]);
-        } else {
-          const u32x4 bP = {pP[r0], pP[r0 + 1], pP[r0 + 2], pP[r0 + 3]};
-          dvacc[i % DB] = Mma<T>::run(ring[n & 7], bP, dvacc[i % DB]);
-        }
+      };
+      if constexpr (!BOTH) form_ds();
+      static_for<2 * DBV>([&](auto ic) {
+        constexpr int k = KSE + KSV + decltype(ic)::value;
+        constexpr WideOp op = dkdv_op<ER, DVR>(k);
+        if constexpr (k + AHEAD < NOPS) ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
+        constexpr int r0 = (op.j / DB) * 4;
+        const u32x4 bP = {pP[r0], pP[r0 + 1], pP[r0 + 2], pP[r0 + 3]};
+        dvacc[op.j % DB] = Mma<T>::run(ring[k & 7], bP, dvacc[op.j % DB]);
         __builtin_amdgcn_sched_barrier(0);
-      }
+      });
+      if constexpr (BOTH) form_ds();
+      static_for<2 * DBE>([&](auto ic) {
+        constexpr int k = KSE + KSV + 2 * DBV + decltype(ic)::value;
+        constexpr WideOp op = dkdv_op<ER, DVR>(k);
+        if constexpr (k + AHEAD < NOPS) ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
+        constexpr int r0 = (op.j / DB) * 4;
+        const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
+        dkacc[op.j % DB] = Mma<T>::run(ring[k & 7], bS, dkacc[op.j % DB]);
+        __builtin_amdgcn_sched_barrier(0);
+      });
     }
     buf ^= 1;
     if (!last) publish_item(buf);
@@ -406,50 +480,62 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     uint16_t* gk = (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
     uint16_t* gv = (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
 #pragma unroll
-    for (int db = 0; db < DB; ++db)
+    for (int db = 0; db < DBE; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        u32x2 wk, wv;
+        u32x2 wk;
         wk[0] = Mma<T>::pack(dkacc[db][g * 4] * p.scale, dkacc[db][g * 4 + 1] * p.scale);
         wk[1] = Mma<T>::pack(dkacc[db][g * 4 + 2] * p.scale, dkacc[db][g * 4 + 3] * p.scale);
+        if (db * 32 + g * 8 + half * 4 < er) *(u32x2*)(gk + db * 32 + g * 8 + half * 4) = wk;
+      }
+#pragma unroll
+    for (int db = 0; db < DBV; ++db)
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        u32x2 wv;
         wv[0] = Mma<T>::pack(dvacc[db][g * 4], dvacc[db][g * 4 + 1]);
         wv[1] = Mma<T>::pack(dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]);
-        if (db * 32 + g * 8 + half * 4 < er) *(u32x2*)(gk + db * 32 + g * 8 + half * 4) = wk;
         if (db * 32 + g * 8 + half * 4 < dvr) *(u32x2*)(gv + db * 32 + g * 8 + half * 4) = wv;
       }
   }
 }
 
-template <typename T>
+template <typename T, int ER, int DVR>
 int launch_t(const BwdM& g, hipStream_t s) {
   const int64_t q_blocks = (int64_t)g.B * g.Hq * ((g.L + 127) / 128), k_blocks = (int64_t)g.B * g.Hkv * ((g.S + 127) / 128);
   if (q_blocks > 0x7fffffff || k_blocks > 0x7fffffff) {
     set_error("SDPA: too many tiles for the wide backward kernels");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T>,
+  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DQ_LDS);
   if (attr_q != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", WIDE_DQ_LDS, hipGetErrorString(attr_q));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dq_kernel<T>), dim3((unsigned)q_blocks), dim3(256), WIDE_DQ_LDS, s, g);
+  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR>), dim3((unsigned)q_blocks), dim3(256), WIDE_DQ_LDS, s, g);
   int rc = check_launch("bwd_wide_dq_kernel");
   if (rc) return rc;
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DKDV_LDS);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", WIDE_DKDV_LDS, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T>), dim3((unsigned)k_blocks), dim3(256), WIDE_DKDV_LDS, s, g);
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR>), dim3((unsigned)k_blocks), dim3(256), WIDE_DKDV_LDS, s, g);
   return check_launch("bwd_wide_dkdv_kernel");
+}
+// widths the kernels are instantiated for: 192 / 128 (multi-head latent attention) and the full 256 / 256
+template <typename T>
+int launch_w(const BwdM& g, hipStream_t s) {
+  if (g.d_real <= 192 && g.dv_real <= 128) return launch_t<T, 192, 128>(g, s);
+  return launch_t<T, 256, 256>(g, s);
 }
 
 }  // namespace
 
 int launch_bwd_wide(const BwdM& g, int dtype, hipStream_t s) {
-  return dtype == MI355_SDPA_BF16 ? launch_t<bf16_t>(g, s) : launch_t<f16_t>(g, s);
+  return dtype == MI355_SDPA_BF16 ? launch_w<bf16_t>(g, s) : launch_w<f16_t>(g, s);
 }
 
 }  // namespace mi355
