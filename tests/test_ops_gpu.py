@@ -350,6 +350,29 @@ def test_native_mha_mid_errors(amd, gpu_device):
 
 # ---- HIP graph capture -----------------------------------------------------------------------------
 
+def test_traced_module_reaches_the_library(amd, gpu_device, calls):
+    # a compiled (traced with fake tensors, run with the eager backend) attention block: the registered
+    # operators are what the traced graph calls, forward and backward, and the numbers are the eager ones
+    q, k, v = (t.to(gpu_device).requires_grad_(True) for t in qkv(2, 8, 2, 256, 256, 64, dtype=torch.bfloat16, seed=21))
+
+    def block(q, k, v):
+        return F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True).float().square().sum()
+
+    ref = block(q, k, v)
+    ref.backward()
+    eager = [t.grad.clone() for t in (q, k, v)]
+    for t in (q, k, v):
+        t.grad = None
+    before = dict(calls)
+    torch._dynamo.reset()
+    got = torch.compile(block, backend="aot_eager")(q, k, v)
+    got.backward()
+    assert calls["fwd"] > before["fwd"] and calls["bwd"] > before["bwd"], calls
+    assert torch.equal(got, ref)
+    for t, e in zip((q, k, v), eager):
+        assert torch.equal(t.grad, e)
+
+
 def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
     # The library only launches kernels on the stream it is given (no allocation, no memset, no
     # synchronisation), so forward, backward and decode can be recorded into one graph.  The graph

@@ -110,8 +110,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     if constexpr (MASK == 2) return compact ? __builtin_amdgcn_readfirstlane((int)items_s[it]) : it;
     else return it;
   };
-  auto item_head = [&](int it) { return hk * rep + item_id(it) % rep; };
-  auto item_q0 = [&](int it) { return (qs_end - 1 - item_id(it) / rep) * BQ; };
+  // (item / rep as a multiply-high by ceil(2^32 / rep), exact while item * rep < 2^32: these two are
+  // evaluated many times per item, on the scalar unit, and a division there is twenty instructions)
+  const uint32_t rep_inv = (uint32_t)((0x100000000ull + (uint32_t)rep - 1) / (uint32_t)rep);
+  auto item_tile = [&](int it) { return (int)__umulhi((uint32_t)item_id(it), rep_inv); };
+  auto item_head = [&](int it) { return hk * rep + (item_id(it) - item_tile(it) * rep); };
+  auto item_q0 = [&](int it) { return (qs_end - 1 - item_tile(it)) * BQ; };
 
   // ---- staging: every thread moves two 16-byte chunks of the Q tile and two of the dO tile ------
   // Buffer resources end with the last row of the batch (the tile offset travels in the vector
