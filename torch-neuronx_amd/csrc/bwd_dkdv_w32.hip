@@ -113,7 +113,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // (item / rep as a multiply-high by ceil(2^32 / rep), exact while item * rep < 2^32: these two are
   // evaluated many times per item, on the scalar unit, and a division there is twenty instructions)
   const uint32_t rep_inv = (uint32_t)((0x100000000ull + (uint32_t)rep - 1) / (uint32_t)rep);
-  auto item_tile = [&](int it) { return (int)__umulhi((uint32_t)item_id(it), rep_inv); };
+  auto item_tile = [&](int it) { return rep == 1 ? item_id(it) : (int)__umulhi((uint32_t)item_id(it), rep_inv); };  // (2^32 does not fit)
   auto item_head = [&](int it) { return hk * rep + (item_id(it) - item_tile(it) * rep); };
   auto item_q0 = [&](int it) { return (qs_end - 1 - item_tile(it)) * BQ; };
 
