@@ -131,6 +131,30 @@ def test_forward_and_backward_with_tables(amd, gpu_device, case, dtype):
         assert max_abs(a, r) <= 5e-2
 
 
+@pytest.mark.parametrize("shape", [(2, 4, 2, 700, 1100, 128, "head"), (1, 6, 3, 1100, 700, 64, "batch"), (2, 2, 2, 520, 2080, 128, "one")])
+def test_rectangular_block_sparse_masks_with_tables(amd, gpu_device, shape):
+    # L != S, masks with their own head or batch extent, rows and whole row blocks without a kept score
+    B, Hq, Hkv, L, S, E, extent = shape
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=torch.bfloat16, seed=L + S, with_do=True)
+    g = torch.Generator().manual_seed(L * 3 + S)
+    Bm, Hm = (B, Hq) if extent == "head" else (B, 1) if extent == "batch" else (1, 1)
+    coarse = torch.rand(Bm, Hm, (L + 47) // 48, (S + 79) // 80, generator=g) < 0.25
+    mask = coarse.repeat_interleave(48, 2).repeat_interleave(80, 3)[:, :, :L, :S].contiguous()
+    qd, kd, vd, god, md = (t.to(gpu_device) for t in (q, k, v, go, mask))
+    o0, l0 = amd.sdpa_forward(qd, kd, vd, attn_bias=md, force_kernel=MFMA)
+    o1, l1 = amd.sdpa_forward(qd, kd, vd, attn_bias=md, force_kernel=MFMA, live_tiles=True)
+    g0 = amd.sdpa_backward(god, qd, kd, vd, o0, l0, attn_bias=md, force_kernel=MFMA)
+    g1 = amd.sdpa_backward(god, qd, kd, vd, o0, l0, attn_bias=md, force_kernel=MFMA, live_tiles=True)
+    torch.cuda.synchronize()
+    assert max_abs(o1, o0.cpu()) <= 1e-6 and max_abs(l1, l0.cpu()) <= 1e-5
+    for a, b_ in zip(g1[:3], g0[:3]):
+        assert max_abs(a, b_.cpu()) <= 1e-6
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
+    assert max_abs(o1, ro) <= 2e-2 and max_abs(l1, rl) <= 5e-3
+    for a, r in zip(g1[:3], oracle_bwd(go, q, k, v, ro, rl, attn_mask=mask)[:3]):
+        assert max_abs(a, r) <= 5e-2
+
+
 def test_workgroups_without_a_live_tile(amd, gpu_device):
     # whole 256-row blocks of queries see no key: zeros, lse = -inf, zero gradients
     B, H, n, E = 1, 2, 1024, 128
