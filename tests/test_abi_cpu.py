@@ -258,8 +258,9 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
     assert len(rows) > 50
     fwd = {n: r for n, r in rows.items() if "fwd_w32_kernel" in n}
     assert len(fwd) >= 30
-    # the head-dim-256 forward with a per-score bias is known to spill (it holds 512 registers as it is)
-    known = re.compile(r"fwd_w32_kernelIDF16[b_]Li256ELi4ELi2EE")
+    # the head-dim-256 forward with a per-score bias and the full-width wide backward kernels with a
+    # mask are known to spill (they hold 512 registers as it is)
+    known = re.compile(r"fwd_w32_kernelIDF16[b_]Li256ELi4ELi2EE|bwd_wide_(dq|dkdv)_kernelIDF16[b_]Li256ELi256ELb1EE")
     for name, r in rows.items():
         if r["src"] not in ("fwd_mfma_w32.hip", "bwd_dq_w32.hip", "bwd_dkdv_w32.hip", "bwd_wide.hip", "decode_fp8kv.hip"):
             continue

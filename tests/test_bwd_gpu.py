@@ -415,6 +415,63 @@ def test_mfma_backward_wide_and_asymmetric_head_dims(amd, gpu_device, shape, dty
         assert rel_err(a, r) <= 2e-2, name
 
 
+WIDE_MASKED = [
+    # B, Hq, Hkv, L, S, E, Dv, mask kind, causal
+    (2, 4, 2, 300, 300, 256, 256, "kv_lens", True),
+    (2, 4, 2, 300, 420, 256, 256, "bool_pad", False),
+    (2, 4, 4, 256, 256, 192, 128, "float_full", False),
+    (1, 4, 1, 200, 520, 256, 256, "bool_full", False),
+    (2, 8, 2, 384, 384, 192, 128, "hf_causal_pad", False),
+    (1, 2, 2, 130, 260, 160, 96, "float32_key", True),
+    (3, 2, 1, 96, 200, 256, 256, "kv_lens_dead", False),
+]
+
+
+@pytest.mark.parametrize("case", WIDE_MASKED)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_mfma_backward_wide_head_dims_with_masks(amd, gpu_device, case, dtype):
+    # key counts and bias / keep-masks, per key or per score, in the kernels for head dims above 128
+    # and D_qk != D_v (forced: a call they cannot take is an error, not a fallback)
+    B, Hq, Hkv, L, S, E, Dv, kind, causal = case
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, Dv=Dv, dtype=dtype, seed=E + L + S, with_do=True)
+    g = torch.Generator().manual_seed(L * 5 + S)
+    kw, om = {}, None
+    if kind in ("kv_lens", "kv_lens_dead"):
+        lens = torch.randint(1, S + 1, (B,), generator=g).to(torch.int32)
+        if kind == "kv_lens_dead":
+            lens[1] = 0
+        kw["kv_lens"] = lens.to(gpu_device)
+        om = (torch.arange(S)[None] < lens[:, None])[:, None, None, :]
+    elif kind == "bool_pad":
+        lens = torch.randint(1, S + 1, (B,), generator=g)
+        om = (torch.arange(S)[None] < lens[:, None])[:, None, None, :]
+        kw["attn_bias"] = om.to(gpu_device)
+    elif kind == "float_full":
+        om = (2 * torch.randn(B, Hq, L, S, generator=g)).to(dtype)
+        kw["attn_bias"] = om.to(gpu_device)
+        om = om.float()
+    elif kind == "bool_full":
+        om = torch.rand(1, 1, L, S, generator=g) > 0.4
+        om[:, :, 5] = False
+        kw["attn_bias"] = om.to(gpu_device)
+    elif kind == "hf_causal_pad":  # what model code builds: causal and padding folded into one additive (B,1,L,S) mask
+        lens = torch.tensor([S, S - 100])[:B]
+        keep = torch.tril(torch.ones(L, S, dtype=torch.bool))[None, None] & (torch.arange(S)[None] < lens[:, None])[:, None, None, :]
+        om = torch.where(keep, 0.0, float("-inf")).to(dtype)
+        kw["attn_bias"] = om.to(gpu_device)
+        om = om.float()
+    else:
+        om = 2 * torch.randn(B, 1, 1, S, generator=g)
+        kw["attn_bias"] = om.to(gpu_device)
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, is_causal=causal, **kw)
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, attn_mask=om, is_causal=causal)
+    assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 5e-3
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert bool(torch.isfinite(a.float()).all()), name
+        assert max_abs(a, r) <= 5e-2, name
+        assert rel_err(a, r) <= 2e-2, name
+
+
 def test_wide_backward_is_what_autograd_reaches(amd, gpu_device):
     # the functional API lands in the MFMA kernels for 192 / 128 as well, forward and backward
     import torch.nn.functional as F

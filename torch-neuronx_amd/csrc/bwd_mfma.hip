@@ -558,10 +558,11 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return *why = "dtype is not bf16/f16", false;
   if (E < 8 || E > 256 || E % 8 != 0 || Dv < 8 || Dv > E || Dv % 8 != 0)
     return *why = "head dims are not multiples of 8 up to 256 with D_v <= D_qk", false;
-  // head dims above 128 and D_qk != D_v: the kernels of bwd_wide.hip, which take no mask of any kind
+  // head dims above 128 and D_qk != D_v: the kernels of bwd_wide.hip, which take key counts and a
+  // bias / keep-mask, but no bias gradient and no window
   const bool wide = E > 128 || Dv != E;
-  if (wide && (p.bias.data || p.grad_bias.data || p.kv_lens || p.mask.window > 0))
-    return *why = "mask, bias or key counts with a head dim above 128 or D_qk != D_v", false;
+  if (wide && (p.grad_bias.data || p.mask.window > 0))
+    return *why = "bias gradient or window with a head dim above 128 or D_qk != D_v", false;
   const bool padded = E != 64 && E != 128;  // served by the next wider kernels' masked variants
   if (p.grad_bias.data) {  // written by the dQ kernel four keys (8 bytes) at a time
     const int64_t S = p.k.size[2];

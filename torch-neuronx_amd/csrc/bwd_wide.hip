@@ -146,7 +146,10 @@ constexpr WideOp dkdv_op(int k) {  // S steps and dP steps (in turns where both 
   return {3, (k / DBE) * DB + k % DBE};
 }
 
-template <typename T, int ER, int DVR>
+// MASKED: per-batch key counts and an additive bias / bool keep-mask, per key or per score (a lane is
+// a query row in the dQ kernel and reads its own row of it, a key in the dK/dV kernel and reads one
+// element per score register); no bias gradient here.
+template <typename T, int ER, int DVR, bool MASKED>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
@@ -195,14 +198,64 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
-  int nt = (p.S + BT - 1) / BT;
+  int S = p.S;  // keys of this batch that take part
+  if constexpr (MASKED) {
+    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+  }
+  int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;  // tiles with work for this wavefront
-  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
 
   // the buffers end with the last key row: rows of a ragged last tile beyond it read as zeros
-  const u32x4 k_rsrc = wide_descriptor(kp, ((int64_t)(p.S - 1) * p.k_sl + er) * 2);
-  const u32x4 v_rsrc = wide_descriptor(vp, ((int64_t)(p.S - 1) * p.v_sl + dvr) * 2);
+  const u32x4 k_rsrc = wide_descriptor(kp, S > 0 ? ((int64_t)(S - 1) * p.k_sl + er) * 2 : 0);
+  const u32x4 v_rsrc = wide_descriptor(vp, S > 0 ? ((int64_t)(S - 1) * p.v_sl + dvr) * 2 : 0);
+  // bias of a score tile: this lane's 16 keys of its query row (row stride 0: a bias per key), as 4
+  // groups of 4 consecutive keys, requested ahead of the tile's score products; keys past the row
+  // read the next row or, past the last row, zeros (they are masked anyway)
+  const int bkind = MASKED ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
+      __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
+  const uint32_t b_row = MASKED ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
+  uint32_t braw[16];
+  auto load_bias = [&](int t) {
+    if constexpr (MASKED) {
+      const uint32_t off = b_row + (uint32_t)(t * BT * besz);
+      if (bkind == 1) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, off + g * 32, 0, 0);
+          braw[4 * g] = w[0], braw[4 * g + 1] = w[1], braw[4 * g + 2] = w[2], braw[4 * g + 3] = w[3];
+        }
+      } else if (bkind == 4) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) braw[g] = __builtin_amdgcn_raw_buffer_load_b32(b_rsrc, off + g * 8, 0, 0);
+      } else if (bkind) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, off + g * 16, 0, 0);
+          braw[2 * g] = w[0], braw[2 * g + 1] = w[1];
+        }
+      }
+    }
+  };
+  // ... in the log2 domain (the element type is tested once, outside the loop: inside, every element
+  // would carry the branch)
+  auto bias_log2 = [&](float (&bl)[16]) {
+    typedef __attribute__((ext_vector_type(2))) _Float16 h2;
+    auto each = [&](auto conv) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) bl[r] = conv(r);
+    };
+    if (bkind == 1) each([&](int r) { return __builtin_bit_cast(float, braw[r]) * kLog2eF; });
+    else if (bkind == 4) each([&](int r) { return ((braw[r >> 2] >> (8 * (r & 3))) & 0xffu) ? 0.f : -INFINITY; });
+    else if (bkind == 3)
+      each([&](int r) { return __builtin_bit_cast(float, (r & 1) ? (braw[r >> 1] & 0xffff0000u) : (braw[r >> 1] << 16)) * kLog2eF; });
+    else if (bkind == 2) each([&](int r) { return (float)__builtin_bit_cast(h2, braw[r >> 1])[r & 1] * kLog2eF; });
+    else each([](int) { return 0.f; });
+  };
   typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
   const uint32_t lds_k = (uint32_t)(uintptr_t)(lds_bytes)k_buf, lds_v = (uint32_t)(uintptr_t)(lds_bytes)v_buf;
   uint32_t k_off[TILE_LOADS / 4], v_off[TILE_LOADS / 4];
@@ -244,6 +297,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         if constexpr (op.kind == 2) return tr.cols(k_t, op.j);
         else return *(const u32x4*)((op.kind ? v_t : k_t) + col * DW + (((2 * op.j + half) ^ swz_col) << 3));
       };
+      load_bias(t);
       u32x4 ring[8];
       static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       f32x16 sacc = zero16, dpacc = zero16;
@@ -256,13 +310,17 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         __builtin_amdgcn_sched_barrier(0);
       });
       uint32_t pS[8];
+      float bl[16];
+      if constexpr (MASKED) bias_log2(bl);
 #pragma unroll
       for (int r = 0; r < 16; r += 2) {
         float ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           const int kv = t * BT + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
-          float pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
+          float pr;
+          if constexpr (MASKED) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
+          else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
           pr = kv > lim ? 0.f : pr;
           ds[e] = pr * (dpacc[r + e] - dl);
         }
@@ -295,7 +353,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   }
 }
 
-template <typename T, int ER, int DVR>
+template <typename T, int ER, int DVR, bool MASKED>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32, DBV = DVR / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
@@ -310,9 +368,13 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   const int k0 = kt * 128, kw0 = k0 + wave * 32, key = kw0 + col;
   const int er = p.d_real, dvr = p.dv_real;
 
+  int S = p.S;  // keys of this batch that take part
+  if constexpr (MASKED) {
+    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+  }
   u32x4 kf[KSE], vf[KSV];
   {
-    const int kc = min(key, p.S - 1);
+    const int kc = max(min(key, S - 1), 0);  // (a live row: rows past the batch's keys may hold anything)
     const uint16_t* kr = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl + half * 8;
     const uint16_t* vr = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl + half * 8;
 #pragma unroll
@@ -335,7 +397,42 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 
   // Items: query tile by query tile from the last one down, heads inside: the workgroups of a kv head,
   // which share an XCD, then want the same Q / dO tile at about the same time and find it in its L2.
-  const int n_items = (nqs - qs_begin) * rep;
+  const int n_items = (MASKED && k0 >= S) ? 0 : (nqs - qs_begin) * rep;  // no live key in this block: zeros
+  // bias of this lane's key in the 32 rows of an item, one element per score register, requested
+  // ahead of the item's first product through a resource that ends with the (batch, head)'s last row
+  const int bkind = MASKED ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const uint32_t b_rowbytes = MASKED ? (uint32_t)(p.bias_sl * besz) : 0u;
+  const uint32_t b_lane = MASKED ? (uint32_t)((half * 4 * p.bias_sl + min(key, p.S - 1)) * besz) : 0u;
+  const int b_records = MASKED ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0;
+  uint32_t braw[16];
+  auto load_bias = [&](int hg, int q0) {
+    if constexpr (MASKED) {
+      if (!bkind) return;
+      const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          uniform_ptr((const char*)p.bias + (b * p.bias_sb + (hk * rep + hg) * p.bias_sh) * besz), 0, b_records, 0x00020000);
+      const uint32_t base = b_lane + (uint32_t)q0 * b_rowbytes;
+      auto each = [&](auto fetch) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) braw[r] = fetch(base + (uint32_t)((r >> 2) * 8 + (r & 3)) * b_rowbytes);
+      };
+      if (bkind == 1) each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b32(b_rsrc, off, 0, 0); });
+      else if (bkind == 4) each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(b_rsrc, off, 0, 0); });
+      else each([&](uint32_t off) { return (uint32_t)__builtin_amdgcn_raw_buffer_load_b16(b_rsrc, off, 0, 0); });
+    }
+  };
+  // ... turned into floats in the log2 domain in place (the element type is tested once, outside the loop)
+  auto bias_to_log2 = [&]() {
+    auto each = [&](auto conv) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) braw[r] = __builtin_bit_cast(uint32_t, conv(braw[r]));
+    };
+    if (bkind == 1) each([](uint32_t x) { return __builtin_bit_cast(float, x) * kLog2eF; });
+    else if (bkind == 4) each([](uint32_t x) { return x ? 0.f : -INFINITY; });
+    else if (bkind == 3) each([](uint32_t x) { return __builtin_bit_cast(float, x << 16) * kLog2eF; });
+    else if (bkind == 2) each([](uint32_t x) { return (float)__builtin_bit_cast(_Float16, (uint16_t)x) * kLog2eF; });
+    else each([](uint32_t) { return 0.f; });
+  };
   typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
   const uint32_t lds_q = (uint32_t)(uintptr_t)(lds_bytes)q_buf, lds_do = (uint32_t)(uintptr_t)(lds_bytes)do_buf;
   constexpr int NLD = TILE_LOADS / 4;  // loads per wavefront and tile
@@ -381,7 +478,10 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     // (the other buffer was last read before the barrier that ended the previous item)
     if (!last) request_item(hg + 1 < rep ? qs : qs - 1, hg + 1 < rep ? hg + 1 : 0, buf ^ 1);
     const int q0 = qs * BT;
-    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= p.S)) {  // (uniform per wavefront)
+    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= S)) {  // (uniform per wavefront)
+      // (at full width the bias is requested behind the score products: ahead of them its 16
+      // registers are more than the register file has left)
+      if constexpr (ER + DVR <= 320) load_bias(hg, q0);
       const uint16_t* q_t = q_buf + buf * TILE_ELEMS;
       const uint16_t* do_t = do_buf + buf * TILE_ELEMS;
       const float* lse_s = lse_buf + buf * BT;
@@ -425,6 +525,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       auto issue_dp = [&]() { issue(std::integral_constant<int, KSE>{}, std::integral_constant<int, KSV>{}); };
       if constexpr (BOTH) issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE + KSV>{});
       else issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE>{});
+      if constexpr (!BOTH) load_bias(hg, q0);
+      if constexpr (MASKED) bias_to_log2();
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
@@ -432,8 +534,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
-          pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
-          pr[e] = ((p.causal && key > qi) || key >= p.S) ? 0.f : pr[e];
+          if constexpr (MASKED) pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, __builtin_bit_cast(float, braw[r])) - l4[e]);
+          else pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
+          pr[e] = ((p.causal && key > qi) || key >= S) ? 0.f : pr[e];
         }
         pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
       }
@@ -500,36 +603,37 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   }
 }
 
-template <typename T, int ER, int DVR>
+template <typename T, int ER, int DVR, bool MASKED>
 int launch_t(const BwdM& g, hipStream_t s) {
   const int64_t q_blocks = (int64_t)g.B * g.Hq * ((g.L + 127) / 128), k_blocks = (int64_t)g.B * g.Hkv * ((g.S + 127) / 128);
   if (q_blocks > 0x7fffffff || k_blocks > 0x7fffffff) {
     set_error("SDPA: too many tiles for the wide backward kernels");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR>,
+  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR, MASKED>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DQ_LDS);
   if (attr_q != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", WIDE_DQ_LDS, hipGetErrorString(attr_q));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR>), dim3((unsigned)q_blocks), dim3(256), WIDE_DQ_LDS, s, g);
+  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR, MASKED>), dim3((unsigned)q_blocks), dim3(256), WIDE_DQ_LDS, s, g);
   int rc = check_launch("bwd_wide_dq_kernel");
   if (rc) return rc;
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DKDV_LDS);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", WIDE_DKDV_LDS, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR>), dim3((unsigned)k_blocks), dim3(256), WIDE_DKDV_LDS, s, g);
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>), dim3((unsigned)k_blocks), dim3(256), WIDE_DKDV_LDS, s, g);
   return check_launch("bwd_wide_dkdv_kernel");
 }
 // widths the kernels are instantiated for: 192 / 128 (multi-head latent attention) and the full 256 / 256
 template <typename T>
 int launch_w(const BwdM& g, hipStream_t s) {
-  if (g.d_real <= 192 && g.dv_real <= 128) return launch_t<T, 192, 128>(g, s);
-  return launch_t<T, 256, 256>(g, s);
+  const bool masked = g.bias_kind || g.kv_lens;
+  if (g.d_real <= 192 && g.dv_real <= 128) return masked ? launch_t<T, 192, 128, true>(g, s) : launch_t<T, 192, 128, false>(g, s);
+  return masked ? launch_t<T, 256, 256, true>(g, s) : launch_t<T, 256, 256, false>(g, s);
 }
 
 }  // namespace
