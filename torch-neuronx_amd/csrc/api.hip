@@ -240,7 +240,7 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   // call itself still sends to the generic kernel a bias whose rows are not dword-aligned, tensors
   // that are not 16-byte aligned or whose strides are not multiples of 8 elements.
   const bool bias_ok = true;
-  // (a mask, bias or key counts send the backward of head dims above 128 and of D_qk != D_v to the
+  // (a bias gradient or a window sends the backward of head dims above 128 and of D_qk != D_v to the
   // generic kernel at the call)
   const bool dims = E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E;
   // (float32: the float32 matrix-op kernels, head dims up to 128 with D_qk = D_v and no mask)
