@@ -45,6 +45,8 @@ constexpr int TILE_LOADS = BT * (DW / 8) / 64;
 constexpr int TILE_ELEMS = BT * DW;
 constexpr int WIDE_DKDV_LDS = 2 * 2 * TILE_ELEMS * 2 + 2 * 2 * BT * 4;
 constexpr int WIDE_DQ_LDS = 2 * 2 * TILE_ELEMS * 2;
+constexpr int WIDE_LIST_LDS = 2048 + 16;   // masked dQ instances: the list of live key tiles (1024 entries and the count)
+constexpr int WIDE_LIVE_LDS = 1024;        // masked dK/dV instances: the key block's row of the transposed skip table
 
 // element offsets of the transposing reads of a swizzled tile, [second read of a pair][d block]
 struct TrOffSwz {
@@ -155,6 +157,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const k_buf = wide_lds;                    // [2][TILE_ELEMS]
   uint16_t* const v_buf = wide_lds + 2 * TILE_ELEMS;   // [2][TILE_ELEMS]
+  uint16_t* const tile_list = wide_lds + 4 * TILE_ELEMS;  // (masked instances) [1024] and the count
   const int n_qt = (p.L + 127) / 128;
   const int qt = n_qt - 1 - blockIdx.x / (p.B * p.Hq);  // heavy query tiles first
   const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
@@ -204,6 +207,41 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   }
   int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
+  // With a skip table: the key tiles in which the mask keeps at least one score of this workgroup's
+  // rows (the first wavefront ORs the bitmaps of its two 64-row blocks and expands the set bits into a
+  // list in LDS); stream position u is then key tile tile_of(u).
+  bool listed = false;
+  if constexpr (MASKED) {
+    if (p.live_tiles && !p.causal) {
+      if (wave == 0) {
+        const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
+        const uint32_t* map = p.live_tiles + ((int64_t)((p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? h : 0)) * nrb + rb0) * p.live_words;
+        uint32_t w = 0u;
+        if (lane < p.live_words) {
+#pragma unroll
+          for (int r = 0; r < 2; ++r)
+            if (rb0 + r < nrb) w |= map[r * p.live_words + lane];
+        }
+        int cnt = 0;
+        for (int j0 = 0; j0 < nt; j0 += 64) {
+          const uint32_t ww = __shfl(w, (j0 >> 5) + (lane >> 5), 64);
+          const bool live = j0 + lane < nt && ((ww >> (lane & 31)) & 1u);
+          const uint64_t m = __builtin_amdgcn_ballot_w64(live);
+          if (live) tile_list[cnt + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = (uint16_t)(j0 + lane);
+          cnt += __builtin_popcountll(m);
+        }
+        if (lane == 0) *(int*)(tile_list + 1024) = cnt;
+      }
+      __syncthreads();
+      const int n_live = __builtin_amdgcn_readfirstlane(*(const int*)(tile_list + 1024));
+      listed = n_live < nt;  // (every tile live: the list is the identity)
+      nt = n_live;
+    }
+  }
+  auto tile_of = [&](int u) {
+    if constexpr (MASKED) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
+    else return u;
+  };
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;  // tiles with work for this wavefront
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
 
@@ -264,8 +302,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
     k_off[n] = wide_chunk_off(wave + 4 * n, lane, (int)p.k_sl, er);
     v_off[n] = wide_chunk_off(wave + 4 * n, lane, (int)p.v_sl, dvr);
   }
-  auto request_tile = [&](int t) {  // tile t into buffer t % 2
-    const uint32_t kt = (uint32_t)(t * BT * p.k_sl * 2), vt = (uint32_t)(t * BT * p.v_sl * 2);
+  auto request_tile = [&](int t) {  // the tile at stream position t into buffer t % 2
+    const int ta = tile_of(t);
+    const uint32_t kt = (uint32_t)(ta * BT * p.k_sl * 2), vt = (uint32_t)(ta * BT * p.v_sl * 2);
     const uint32_t boff = (uint32_t)((t & 1) * TILE_ELEMS * 2);
 #pragma unroll
     for (int n = 0; n < TILE_LOADS / 4; ++n) {
@@ -297,7 +336,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         if constexpr (op.kind == 2) return tr.cols(k_t, op.j);
         else return *(const u32x4*)((op.kind ? v_t : k_t) + col * DW + (((2 * op.j + half) ^ swz_col) << 3));
       };
-      load_bias(t);
+      const int ta = tile_of(t);
+      load_bias(ta);
       u32x4 ring[8];
       static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       f32x16 sacc = zero16, dpacc = zero16;
@@ -317,7 +357,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         float ds[2];
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
-          const int kv = t * BT + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
+          const int kv = ta * BT + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
           float pr;
           if constexpr (MASKED) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
           else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
@@ -361,6 +401,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   uint16_t* const do_buf = wide_lds + 2 * TILE_ELEMS;      // [2][TILE_ELEMS]
   float* const lse_buf = (float*)(wide_lds + 4 * TILE_ELEMS);  // [2][BT]
   float* const dl_buf = lse_buf + 2 * BT;                      // [2][BT]
+  uint32_t* const live_s = (uint32_t*)(dl_buf + 2 * BT);       // (masked instances) [heads of the group][words]
   const int streams = p.B * p.Hkv;
   const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
   const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
@@ -436,6 +477,29 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   typedef __attribute__((address_space(3))) unsigned char* lds_bytes;
   const uint32_t lds_q = (uint32_t)(uintptr_t)(lds_bytes)q_buf, lds_do = (uint32_t)(uintptr_t)(lds_bytes)do_buf;
   constexpr int NLD = TILE_LOADS / 4;  // loads per wavefront and tile
+  // With a skip table: an item whose 64-row block holds no kept score for this key block is neither
+  // fetched nor computed.
+  bool listed = false;
+  if constexpr (MASKED) {
+    if (p.live_t && !p.causal && rep * p.live_t_words <= 256) {
+      listed = true;
+      if (tid < rep * p.live_t_words) {
+        const int hd = hk * rep + tid / p.live_t_words;
+        live_s[tid] = p.live_t[(((int64_t)(p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? hd : 0)) * ((p.S + 127) / 128) + kt) * p.live_t_words +
+                               tid % p.live_t_words];
+      }
+      __syncthreads();
+    }
+  }
+  auto item_live = [&](int qs, int hg) {
+    if constexpr (MASKED) {
+      if (listed) {
+        const int qt = qs >> 1;  // 64-row blocks of the table, 32-row items here
+        return ((__builtin_amdgcn_readfirstlane((int)live_s[hg * p.live_t_words + (qt >> 5)]) >> (qt & 31)) & 1) != 0;
+      }
+    }
+    return true;
+  };
   // item `it` into buffer it % 2; the row statistics travel in two registers of the first 32 threads.
   // The buffers start at the tile's first row and end with the head's last row: rows past L read as zeros.
   float lse_n = INFINITY, dl_n = 0.f;
@@ -467,7 +531,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     __syncthreads();
   };
   if (n_items > 0) {
-    request_item(nqs - 1, 0, 0);
+    if (item_live(nqs - 1, 0)) request_item(nqs - 1, 0, 0);
     publish_item(0);
   }
   int buf = 0;
@@ -476,9 +540,10 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     for (int hg = 0; hg < rep; ++hg) {
     const bool last = qs == qs_begin && hg == rep - 1;
     // (the other buffer was last read before the barrier that ended the previous item)
-    if (!last) request_item(hg + 1 < rep ? qs : qs - 1, hg + 1 < rep ? hg + 1 : 0, buf ^ 1);
+    const int qs_n = hg + 1 < rep ? qs : qs - 1, hg_n = hg + 1 < rep ? hg + 1 : 0;
+    if (!last && item_live(qs_n, hg_n)) request_item(qs_n, hg_n, buf ^ 1);
     const int q0 = qs * BT;
-    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= S)) {  // (uniform per wavefront)
+    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= S) && item_live(qs, hg)) {  // (uniform per wavefront)
       // (at full width the bias is requested behind the score products: ahead of them its 16
       // registers are more than the register file has left)
       if constexpr (ER + DVR <= 320) load_bias(hg, q0);
@@ -610,22 +675,23 @@ int launch_t(const BwdM& g, hipStream_t s) {
     set_error("SDPA: too many tiles for the wide backward kernels");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
+  constexpr int kDqLds = WIDE_DQ_LDS + (MASKED ? WIDE_LIST_LDS : 0), kDkdvLds = WIDE_DKDV_LDS + (MASKED ? WIDE_LIVE_LDS : 0);
   static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR, MASKED>,
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DQ_LDS);
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
   if (attr_q != hipSuccess) {
-    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", WIDE_DQ_LDS, hipGetErrorString(attr_q));
+    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", kDqLds, hipGetErrorString(attr_q));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR, MASKED>), dim3((unsigned)q_blocks), dim3(256), WIDE_DQ_LDS, s, g);
+  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR, MASKED>), dim3((unsigned)q_blocks), dim3(256), kDqLds, s, g);
   int rc = check_launch("bwd_wide_dq_kernel");
   if (rc) return rc;
   static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, WIDE_DKDV_LDS);
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDkdvLds);
   if (attr != hipSuccess) {
-    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", WIDE_DKDV_LDS, hipGetErrorString(attr));
+    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", kDkdvLds, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>), dim3((unsigned)k_blocks), dim3(256), WIDE_DKDV_LDS, s, g);
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>), dim3((unsigned)k_blocks), dim3(256), kDkdvLds, s, g);
   return check_launch("bwd_wide_dkdv_kernel");
 }
 // widths the kernels are instantiated for: 192 / 128 (multi-head latent attention) and the full 256 / 256
