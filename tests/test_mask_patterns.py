@@ -102,6 +102,40 @@ def test_recognition_is_sound_on_random_near_patterns():
 # ---- GPU ----------------------------------------------------------------------------------------------
 
 
+def test_padding_masks_become_key_counts():
+    # what model code builds from right padding, with or without causality folded in, per batch
+    from torch_neuronx_amd.mask_patterns import lens_pattern_from_rows
+
+    def rows3(m):
+        return np.stack([rows_of(x.numpy()) for x in m])
+
+    L, S = 12, 20
+    lens = torch.tensor([20, 7, 1, 13])
+    pad = (torch.arange(S)[None] < lens[:, None])[:, None, :].expand(4, L, S)
+    pat = lens_pattern_from_rows(rows3(pad), L, S, rows_broadcast=False)
+    assert pat[0] == "all" and pat[1].tolist() == lens.tolist()
+    pat = lens_pattern_from_rows(rows3(pad[:, :1]), L, S, rows_broadcast=True)
+    assert pat[0] == "all" and pat[1].tolist() == lens.tolist()
+    tril = torch.tril(torch.ones(L, S, dtype=torch.bool))
+    pat = lens_pattern_from_rows(rows3(pad & tril), L, S, rows_broadcast=False)
+    # (a batch whose padding starts behind the last row's diagonal is indistinguishable from no padding)
+    assert pat[0] == "causal" and pat[1].tolist() == [20, 7, 1, 20]
+    for b in range(4):
+        n = int(pat[1][b])
+        assert torch.equal(pad[b] & tril, tril & (torch.arange(S)[None] < min(n, int(lens[b]))))
+    # anything else is left alone: left padding, a hole, a row that keeps a later key
+    left = (torch.arange(S)[None] >= lens[:, None])[:, None, :].expand(4, L, S)
+    assert lens_pattern_from_rows(rows3(left), L, S, rows_broadcast=False) is None
+    holed = (pad & tril).clone()
+    holed[1, 9, 3] = False
+    assert lens_pattern_from_rows(rows3(holed), L, S, rows_broadcast=False) is None
+    late = (pad & tril).clone()
+    late[1, 9, 15] = True
+    assert lens_pattern_from_rows(rows3(late), L, S, rows_broadcast=False) is None
+    one_row_causal = (pad & tril)[:, :1]
+    assert lens_pattern_from_rows(rows3(one_row_causal), L, S, rows_broadcast=True)[0] == "all"  # row 0 keeps key 0 only, everywhere
+
+
 @pytest.fixture(scope="module")
 def amd(gpu_device):
     import torch_neuronx_amd as amd
@@ -229,3 +263,42 @@ def test_sliding_window_mask_takes_the_window_kernel(amd, gpu_device, monkeypatc
     live = int(keep.sum())
     tflops = 4.0 * Bp * 32 * D * live / (ms * 1e-3) / 1e12
     assert tflops >= 600.0, tflops
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D", [128, 256])
+def test_causal_and_padding_mask_becomes_causal_with_key_counts(amd, gpu_device, monkeypatch, D):
+    # the additive (B,1,L,S) mask that model code builds from causality and right padding: served by the
+    # causal kernels with per-batch key counts, no mask read, forward and backward
+    dev = gpu_device
+    B, H, L = 3, 4, 1024
+    q, k, v, go = (t.to(dev) for t in qkv(B, H, H, L, L, D, dtype=torch.bfloat16, seed=4, with_do=True))
+    lens = torch.tensor([L, 600, 131])
+    keep = torch.tril(torch.ones(L, L, dtype=torch.bool))[None, None] & (torch.arange(L)[None] < lens[:, None])[:, None, None, :]
+    mask = torch.where(keep, 0.0, float("-inf")).to(torch.bfloat16).to(dev)
+    amd.mask_patterns.clear_cache()
+    seen = []
+    f0, b0 = amd.ops.sdpa_forward, amd.ops.sdpa_backward
+    monkeypatch.setattr(amd.ops, "sdpa_forward", lambda *a, **kw: (seen.append(kw), f0(*a, **kw))[1])
+    monkeypatch.setattr(amd.ops, "sdpa_backward", lambda *a, **kw: (seen.append(kw), b0(*a, **kw))[1])
+    fused = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    fused_bwd = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    r = fused(q, k, v, mask)
+    assert seen[-1]["attn_bias"] is None and seen[-1]["is_causal"] is True and seen[-1]["kv_lens"].tolist() == [L, 600, 131]
+    g = fused_bwd(go, q, k, v, mask, [True, True, True, False], r[0], r[1], None, None, L, L, 0.0, False, r[6], r[7])
+    assert seen[-1]["attn_bias"] is None and seen[-1]["kv_lens"].tolist() == [L, 600, 131]
+    ro, rl = om.sdpa_forward(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=keep)
+    rg = om.sdpa_backward(go.float().cpu(), q.float().cpu(), k.float().cpu(), v.float().cpu(), ro, rl, attn_mask=keep, reduce_in_fp32=True)
+    assert max_abs(r[0], ro) <= 2e-2 and max_abs(r[1], rl) <= 5e-3
+    for a, b_ in zip(g[:3], rg[:3]):
+        assert max_abs(a, b_) <= 5e-2 and rel_err(a, b_) <= 2e-2
+    # padding alone, as a bool (B,1,1,S) mask: key counts without the causal flag
+    pad = (torch.arange(L)[None] < lens[:, None])[:, None, None, :].to(dev)
+    r2 = fused(q, k, v, pad)
+    assert seen[-1]["attn_bias"] is None and seen[-1]["is_causal"] is False and seen[-1]["kv_lens"].tolist() == [L, 600, 131]
+    ro2, _ = om.sdpa_forward(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=pad.cpu())
+    assert max_abs(r2[0], ro2) <= 2e-2
+    # left padding is no key count: the mask stays a mask
+    left = (torch.arange(L)[None] >= (L - lens)[:, None])[:, None, None, :].to(dev)
+    fused(q, k, v, left)
+    assert seen[-1]["attn_bias"] is not None

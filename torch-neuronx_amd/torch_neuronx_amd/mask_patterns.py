@@ -7,7 +7,8 @@ its fused path is refused (decompositions.py:2203).  Here a mask only exists as 
 read once on the device (``mi355_sdpa_mask_rows``: four numbers per row) and the decision is cached
 for as long as the tensor is unchanged: a causal mask, a sliding window with sink keys and a
 keep-everything mask are then served by the kernels that generate those patterns from indices,
-skip the tiles they drop and read no mask at all.
+skip the tiles they drop and read no mask at all; so are the masks that model code builds from
+right padding, with or without causality folded in (per-batch key counts).
 """
 
 from __future__ import annotations
@@ -76,6 +77,48 @@ def pattern_from_rows(rows: np.ndarray, L: int, S: int):
     return None
 
 
+def lens_pattern_from_rows(rows: np.ndarray, L: int, S: int, rows_broadcast: bool):
+    """Masks that depend on the batch the way padding does: ``rows[b, i]`` as in ``pattern_from_rows``
+    for every batch ``b`` -> ``("all", lens)`` (batch ``b`` keeps keys ``0 .. lens[b]-1`` in every row)
+    or ``("causal", lens)`` (row ``i`` keeps keys ``0 .. min(i, lens[b]-1)``): what model code builds
+    when it folds right padding, and causality, into one mask.  ``rows_broadcast``: the mask has one
+    row per batch, valid for every query.  ``None`` if some row is anything else."""
+    B = rows.shape[0]
+    if B == 0 or S == 0 or rows.ndim != 3 or rows.shape[2] != 4:
+        return None
+    hi, cnt, lead, lo = (rows[:, :, c].astype(np.int64) for c in range(4))
+    if (cnt < 0).any() or (lo != 0).any():
+        return None
+    n = hi[:, -1] + 1  # keys of the batch as its last row sees them
+    if (hi == (n - 1)[:, None]).all() and (cnt == n[:, None]).all():  # every row the same run from key 0
+        return ("all", n.astype(np.int32))
+    if rows_broadcast:
+        return None
+    i = np.arange(rows.shape[1], dtype=np.int64)[None, :]
+    full = hi[:, -1] == min(L - 1, S - 1)  # the last row reaches its diagonal: no key is known to be padding
+    n = np.where(full, S, n)
+    hi_c = np.minimum(np.minimum(i, S - 1), (n - 1)[:, None])
+    if (hi == hi_c).all() and (cnt == hi_c + 1).all():
+        return ("causal", n.astype(np.int32))
+    return None
+
+
+def _as_3d(mask: torch.Tensor):
+    """``(batch, rows, keys)`` view of a mask that does not depend on the head (its row dimension may
+    be 1: one row for every query), or ``None``."""
+    m = mask
+    if m.dim() != 4:
+        return None
+    if not (m.size(1) == 1 or m.stride(1) == 0):
+        return None
+    m = m[:, 0]
+    if m.size(2) > 1 and m.stride(2) != 1:
+        return None
+    if m.size(1) > 1 and m.stride(1) == 0:
+        m = m[:, :1]
+    return m
+
+
 def _as_2d(mask: torch.Tensor):
     """The ``(L, S)`` slice of a mask that does not depend on batch and head, or ``None``."""
     m = mask
@@ -98,7 +141,7 @@ def classify(mask: torch.Tensor):
         return None
     m = _as_2d(mask)
     if m is None:
-        return None
+        return _classify_batched(mask)
     L, S = m.shape
     if L < 1 or S < 1:
         return None
@@ -124,6 +167,54 @@ def classify(mask: torch.Tensor):
                                               _lib.current_stream(mask.device))
     _lib.check(rc)
     pat = pattern_from_rows(rows.cpu().numpy(), L, S)
+    _cache[key] = (pat, mask)
+    while len(_cache) > _CACHE_ENTRIES:
+        _cache.popitem(last=False)
+    return pat
+
+
+_MAX_BATCH = 256
+
+
+def _classify_batched(mask: torch.Tensor):
+    """``classify`` for a mask that depends on the batch (and not on the head): one row summary per
+    batch, then ``lens_pattern_from_rows``.  The key counts come back as an int32 device tensor."""
+    m = _as_3d(mask)
+    if m is None or m.size(0) > _MAX_BATCH:
+        return None
+    B, Lm, S = m.shape
+    if B < 1 or Lm < 1 or S < 1:
+        return None
+    key = (m.data_ptr(), tuple(m.shape), tuple(m.stride()), m.dtype, mask._version, mask.device.index)
+    sig = (B, Lm, S, m.dtype, mask.device.index)
+    hit = _cache.get(key)
+    if hit is not None:
+        _cache.move_to_end(key)
+        _misses.pop(sig, None)
+        stats["hits"] += 1
+        return hit[0]
+    if torch.cuda.is_current_stream_capturing():
+        return None
+    streak = _misses.get(sig, 0)
+    _misses[sig] = streak + 1
+    if streak >= _MAX_MISSES and (streak - _MAX_MISSES) % _RETRY_EVERY != _RETRY_EVERY - 1:
+        stats["left_alone"] += 1
+        return None
+    stats["looked"] += 1
+    rows = torch.empty((B, Lm, 4), dtype=torch.int32, device=mask.device)
+    lib = _lib.load()
+    with _lib.on_device(mask.device):
+        for b in range(B):
+            _lib.check(lib.mi355_sdpa_mask_rows(m[b].data_ptr(), _lib.dtype_id(m.dtype), Lm, S, m.stride(1), rows[b].data_ptr(),
+                                                _lib.current_stream(mask.device)))
+    L = mask.shape[-2]
+    pat = lens_pattern_from_rows(rows.cpu().numpy(), L, S, rows_broadcast=Lm == 1 and L > 1)
+    if pat is not None:
+        lens = pat[1]
+        if (lens == S).all():
+            pat = (pat[0],)  # no padding after all
+        else:
+            pat = (pat[0], torch.from_numpy(lens).to(mask.device))
     _cache[key] = (pat, mask)
     while len(_cache) > _CACHE_ENTRIES:
         _cache.popitem(last=False)

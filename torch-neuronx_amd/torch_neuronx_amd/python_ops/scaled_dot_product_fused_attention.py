@@ -92,10 +92,10 @@ def _recover_pattern(attn_bias, is_causal, want_grad_bias=False):
     pat = mask_patterns.classify(attn_bias)
     if pat is None:
         return attn_bias, is_causal, {}
-    if pat[0] == "all":
-        return None, False, {}
+    if pat[0] == "all":  # (with per-batch key counts when the mask was right padding)
+        return None, False, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
     if pat[0] == "causal":
-        return None, True, {}
+        return None, True, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
     return None, True, {"window": pat[1], "sink_keys": pat[2]}
 
 
