@@ -20,6 +20,15 @@
 // lse = -inf give zero gradients, scale multiplies dQ and dK once at the end.
 #include "bwd_mfma.h"
 
+#ifndef WIDE_DQ_AHEAD
+#define WIDE_DQ_AHEAD 3
+#endif
+#ifndef WIDE_KV_AHEAD_S
+#define WIDE_KV_AHEAD_S 4
+#endif
+#ifndef WIDE_KV_AHEAD_L
+#define WIDE_KV_AHEAD_L 2
+#endif
 namespace mi355 {
 namespace {
 
@@ -48,26 +57,37 @@ constexpr int WIDE_DQ_LDS = 2 * 2 * TILE_ELEMS * 2;
 constexpr int WIDE_LIST_LDS = 2048 + 16;   // masked dQ instances: the list of live key tiles (1024 entries and the count)
 constexpr int WIDE_LIVE_LDS = 1024;        // masked dK/dV instances: the key block's row of the transposed skip table
 
-// element offsets of the transposing reads of a swizzled tile, [second read of a pair][d block]
+// The swizzle moves a chunk inside its 256-byte window of a 512-byte row: the offsets of the reads
+// are not additive in the contraction step / d block within a window (one offset register per
+// combination), and the second window is the first plus 256 bytes, which travels in the read's
+// immediate offset.
+constexpr int WIN = 128;  // elements per window
+
+// element offsets of the transposing reads of a swizzled tile, [second read of a pair][d block of a window]
 struct TrOffSwz {
-  int off[2][DB];
+  int off[2][4];
   __device__ __forceinline__ void init(int lane) {
     const int jj = lane & 15, g = lane >> 4;
 #pragma unroll
     for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
-      for (int db = 0; db < DB; ++db) {
+      for (int db = 0; db < 4; ++db) {
         const int row = 8 * sec + (g >> 1) * 4 + (jj >> 2), d = db * 32 + 16 * (g & 1) + 4 * (jj & 3);
         off[sec][db] = row * DW + (((d >> 3) ^ tile_swz<DW>(row)) << 3) + (d & 7);
       }
   }
   // operand i = DB * (16-row step) + d block of the transposed tile (rows 16 apart share a swizzle)
   __device__ __forceinline__ u32x4 cols(const uint16_t* tile, int i) const {
-    const u32x2 lo = tr_read(tile + off[0][i % DB] + (i / DB) * 16 * DW);
-    const u32x2 hi = tr_read(tile + off[1][i % DB] + (i / DB) * 16 * DW);
+    const int db = i % DB;
+    const u32x2 lo = tr_read(tile + off[0][db % 4] + (db / 4) * WIN + (i / DB) * 16 * DW);
+    const u32x2 hi = tr_read(tile + off[1][db % 4] + (db / 4) * WIN + (i / DB) * 16 * DW);
     return u32x4{lo[0], lo[1], hi[0], hi[1]};
   }
 };
+// element offset of the row read of contraction step j (this lane: row col, 8 elements at 16 j + 8 half)
+__device__ __forceinline__ int wide_row_off(int j, int col, int half, int swz_col) {
+  return col * DW + (((2 * (j % 8) + half) ^ swz_col) << 3) + (j / 8) * WIN;
+}
 
 // raw buffer resource, in scalar registers
 __device__ __forceinline__ u32x4 wide_descriptor(const void* base, int64_t bytes) {
@@ -196,7 +216,10 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   const int swz_col = tile_swz<DW>(col);
   f32x16 dqacc[DBE];
 #pragma unroll
-  for (int i = 0; i < DBE; ++i) zero(dqacc[i]);
+  for (int i = 0; i < DBE; ++i) {
+    zero(dqacc[i]);
+    asm volatile("" : "+a"(dqacc[i]));
+  }
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
@@ -330,17 +353,22 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
       // The LDS operands of a tile - row fragments of K and V in turns, then the transposed fragments
       // of K - travel through a register ring, three matrix ops ahead of their use, in an order
       // pinned by scheduling fences (one wavefront per SIMD has nobody to hide an LDS round trip behind).
-      constexpr int AHEAD = 3, NA = KSE + KSV, NOPS = NA + 2 * DBE;
+      constexpr int AHEAD = WIDE_DQ_AHEAD, NA = KSE + KSV, NOPS = NA + 2 * DBE;
       auto operand = [&](auto kc) {
         constexpr WideOp op = dq_op<ER, DVR>(decltype(kc)::value);
         if constexpr (op.kind == 2) return tr.cols(k_t, op.j);
-        else return *(const u32x4*)((op.kind ? v_t : k_t) + col * DW + (((2 * op.j + half) ^ swz_col) << 3));
+        else return *(const u32x4*)((op.kind ? v_t : k_t) + wide_row_off(op.j, col, half, swz_col));
       };
       const int ta = tile_of(t);
       load_bias(ta);
       u32x4 ring[8];
       static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       f32x16 sacc = zero16, dpacc = zero16;
+      // (the dQ accumulators stay in the accumulation registers across the tile: left to itself the
+      // register allocator keeps part of them in vector registers and copies 16 values in and out
+      // around every matrix op that adds to them)
+#pragma unroll
+      for (int i = 0; i < DBE; ++i) asm volatile("" : "+a"(dqacc[i]));
       static_for<NA>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
         constexpr WideOp op = dq_op<ER, DVR>(k);
@@ -377,6 +405,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         __builtin_amdgcn_sched_barrier(0);
       });
     }
+#pragma unroll
+    for (int i = 0; i < DBE; ++i) asm volatile("" : "+a"(dqacc[i]));
     if (t + 1 < nt) publish_tile();
   }
   if (qrow < p.L) {
@@ -413,6 +443,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   if constexpr (MASKED) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
   }
+  // the first query row that sees this lane's key: the key itself under a causal mask, none for a key
+  // past the batch's count
+  const int first_q = key >= S ? INT_MAX : p.causal ? key : INT_MIN;
   u32x4 kf[KSE], vf[KSV];
   {
     const int kc = max(min(key, S - 1), 0);  // (a live row: rows past the batch's keys may hold anything)
@@ -564,11 +597,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       // operands - row fragments of Q, then of dO, then the transposed fragments of dO, then of Q -
       // travel through one register ring, two to four matrix ops ahead of their use, with the order
       // pinned by scheduling fences.
-      constexpr int AHEAD = ER + DVR <= 320 ? 4 : 2, NOPS = KSE + KSV + 2 * (DBE + DBV);  // (deeper where the widths leave registers)
+      constexpr int AHEAD = ER + DVR <= 320 ? WIDE_KV_AHEAD_S : WIDE_KV_AHEAD_L, NOPS = KSE + KSV + 2 * (DBE + DBV);  // (deeper where the widths leave registers)
       auto operand = [&](auto kc) {
         constexpr WideOp op = dkdv_op<ER, DVR>(decltype(kc)::value);
         if constexpr (op.kind >= 2) return tr.cols(op.kind == 3 ? q_t : do_t, op.j);
-        else return *(const u32x4*)((op.kind ? do_t : q_t) + col * DW + (((2 * op.j + half) ^ swz_col) << 3));
+        else return *(const u32x4*)((op.kind ? do_t : q_t) + wide_row_off(op.j, col, half, swz_col));
       };
       u32x4 ring[8];
       static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
@@ -599,9 +632,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
-          if constexpr (MASKED) pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, __builtin_bit_cast(float, braw[r])) - l4[e]);
-          else pr[e] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -l4[e]));
-          pr[e] = ((p.causal && key > qi) || key >= S) ? 0.f : pr[e];
+          float x;
+          if constexpr (MASKED) x = fmaf(sacc[r], c, __builtin_bit_cast(float, braw[r])) - l4[e];
+          else x = fmaf(sacc[r], c, -l4[e]);
+          // (masked before the exponential: a select around it is compiled into a branch per element)
+          pr[e] = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : x);
         }
         pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
       }

@@ -186,6 +186,13 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     // for every outstanding load there, the tile loads in flight included)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
+    // (one wavefront per SIMD owns both halves of the register file: the Q fragments live in the
+    // accumulation half, where the matrix ops read them directly; left to the allocator they are
+    // parked there anyway and copied back, four moves ahead of every op that uses one)
+    if constexpr (D > 128) {
+#pragma unroll
+      for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qf[ks]));
+    }
   }
 
   const int nt_w = p.causal ? min(nt, qw_last / BN + 1 - skip) : nt;
@@ -270,19 +277,24 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     else if constexpr (PL == 4) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
     else asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
   };
-  // element offsets of the LDS reads inside a swizzled tile (the swizzle is not additive in the d
-  // block / contraction step: one offset register per combination)
-  int row_off[KS], tr_off[2][DB];  // K row reads; V transposing reads [second read of a pair][d block]
+  // element offsets of the LDS reads inside a swizzled tile.  The swizzle is not additive in the d
+  // block / contraction step within a 256-byte window of a row (one offset register per
+  // combination there); the second window of a 512-byte row is the first plus 256 bytes, which
+  // travels in the instruction's immediate offset.
+  constexpr int KSW = KS < 8 ? KS : 8, DBW = DB < 4 ? DB : 4;
+  int row_off_w[KSW], tr_off_w[2][DBW];  // K row reads; V transposing reads [second read of a pair][d block]
 #pragma unroll
-  for (int ks = 0; ks < KS; ++ks) row_off[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
+  for (int ks = 0; ks < KSW; ++ks) row_off_w[ks] = col * D + (((2 * ks + half) ^ tile_swz<D>(col)) << 3);
 #pragma unroll
   for (int sec = 0; sec < 2; ++sec)
 #pragma unroll
-    for (int db = 0; db < DB; ++db) {
+    for (int db = 0; db < DBW; ++db) {
       const int row = 8 * sec + ((lane >> 5) & 1) * 4 + ((lane & 15) >> 2);
       const int d = db * 32 + 16 * ((lane >> 4) & 1) + 4 * (lane & 3);
-      tr_off[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
+      tr_off_w[sec][db] = row * D + (((d >> 3) ^ tile_swz<D>(row)) << 3) + (d & 7);
     }
+  auto row_off_of = [&](int ks) { return row_off_w[ks % KSW] + (ks / KSW) * 128; };
+  auto tr_off_of = [&](int sec, int db) { return tr_off_w[sec][db % DBW] + (db / DBW) * 128; };
 
   // Transposing read: within 16 lanes, lane 4 k + m supplies the address of four consecutive d of
   // key k (d quad m), and lane i receives element i % 4 of the pieces of lanes i / 4, 4 + i / 4,
@@ -488,7 +500,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
-      const u32x4 a = *(const u32x4*)(k_dma + row_off[ks]);
+      const u32x4 a = *(const u32x4*)(k_dma + row_off_of(ks));
       s_a = Mma<T>::run(a, qf[ks], ks == 0 ? zero16 : s_a);
     }
     apply_bias(s_a, false);
@@ -511,7 +523,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   u32x4 ring[8];
 #pragma unroll
   for (int ks = 0; ks < AHEAD; ++ks)
-    ring[ks] = *(const u32x4*)(k_dma + TILE + row_off[ks]);
+    ring[ks] = *(const u32x4*)(k_dma + TILE + row_off_of(ks));
 
   // One pipelined iteration.  On entry scur holds S^T of tile t and pk / ps the probabilities of its
   // first 16 keys; snext receives S^T of tile t+1 and pkn / psn the first half of ITS probabilities.
@@ -526,11 +538,11 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     const uint16_t* kt = k_dma + ((tq + 1) & 3) * TILE;
     const uint16_t* kn = k_dma + ((tq + 2) & 3) * TILE;
     const uint16_t* vt = v_dma + tq * TILE;
-    auto read_k = [&](int ks) { return *(const u32x4*)(kt + row_off[ks]); };
-    auto read_kn = [&](int ks) { return *(const u32x4*)(kn + row_off[ks]); };
+    auto read_k = [&](int ks) { return *(const u32x4*)(kt + row_off_of(ks)); };
+    auto read_kn = [&](int ks) { return *(const u32x4*)(kn + row_off_of(ks)); };
     auto read_v = [&](int i) {  // d block i % DB, 16-key step i / DB
-      const u32x2 lo = tr_read(vt + tr_off[0][i % DB] + (i / DB) * 16 * D);
-      const u32x2 hi = tr_read(vt + tr_off[1][i % DB] + (i / DB) * 16 * D);
+      const u32x2 lo = tr_read(vt + tr_off_of(0, i % DB) + (i / DB) * 16 * D);
+      const u32x2 hi = tr_read(vt + tr_off_of(1, i % DB) + (i / DB) * 16 * D);
       return u32x4{lo[0], lo[1], hi[0], hi[1]};
     };
     __builtin_amdgcn_sched_barrier(0);
