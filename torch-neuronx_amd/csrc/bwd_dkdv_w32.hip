@@ -91,6 +91,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // key see none of its keys, unless the block holds sink keys
   constexpr bool FUNC = MASK == 1;
   const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
+  // the query rows that see this lane's key are first_q .. past_q - 1: from the key itself on under a
+  // causal mask, none for a key past the batch's count, up to the end of the key's window unless it is a sink
+  const int first_q = key >= S ? INT_MAX : p.causal ? key : INT_MIN;
+  const int past_q = (W > 0 && key >= n_sink) ? key + W : INT_MAX;
   const bool listed = MASK == 2 && p.live_t != nullptr;
   const int nqs = (p.L + BQ - 1) / BQ;
   const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
@@ -259,10 +263,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
 
   const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
-  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
   const uint32_t b_rowbytes = MASK == 2 ? (uint32_t)(p.bias_sl * besz) : 0u;
   const uint32_t b_lane = MASK == 2 ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
-  const int b_records = MASK == 2 ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0;
+  const int b_records = MASK == 2 ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
   // the fetched bias elements of a tile, turned into floats in the log2 domain in place (the
   // element type is tested once, outside the loops: inside, every element would carry the branch)
   auto bias_to_log2 = [&](uint32_t (&w)[2][16]) {
@@ -355,7 +359,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 #pragma unroll
       for (int r = 0; r < 16; ++r) {
         const int qi = q0 + mq * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
-        if ((p.causal && key > qi) || key >= S || (W > 0 && qi - key >= W && key >= n_sink)) sc[mq][r] = -INFINITY;
+        // (one compare or two against per-lane bounds: spelled out as the conditions they stand for,
+        // the test is compiled into a cascade of branches per element)
+        const bool dead = FUNC ? (qi < first_q) | (qi >= past_q) : qi < first_q;
+        sc[mq][r] = dead ? -INFINITY : sc[mq][r];
       }
     };
     auto hand_over = [&](int mq) {

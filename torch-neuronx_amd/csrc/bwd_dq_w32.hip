@@ -313,7 +313,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
   const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
-  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
   // (set up unconditionally, with no records when there is no bias: a resource that is defined on
   // one path only stops being uniform for the compiler)
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(

@@ -20,15 +20,6 @@
 // lse = -inf give zero gradients, scale multiplies dQ and dK once at the end.
 #include "bwd_mfma.h"
 
-#ifndef WIDE_DQ_AHEAD
-#define WIDE_DQ_AHEAD 3
-#endif
-#ifndef WIDE_KV_AHEAD_S
-#define WIDE_KV_AHEAD_S 4
-#endif
-#ifndef WIDE_KV_AHEAD_L
-#define WIDE_KV_AHEAD_L 2
-#endif
 namespace mi355 {
 namespace {
 
@@ -127,20 +118,11 @@ struct WideOp {
                 // 2 dO^T columns (dV), 3 Q^T columns (dK); j = contraction step, or DB * (16-row step) + d block
 };
 template <int ER, int DVR>
-constexpr WideOp dq_op(int k) {  // S and dP steps in turns, then the columns of K^T
+constexpr WideOp dq_op(int k) {  // the S steps, the dP steps, then the columns of K^T
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32;
-  int c = 0;
-  for (int j = 0; j < (KSE > KSV ? KSE : KSV); ++j) {
-    if (j < KSE) {
-      if (c == k) return {0, j};
-      ++c;
-    }
-    if (j < KSV) {
-      if (c == k) return {1, j};
-      ++c;
-    }
-  }
-  return {2, ((k - c) / DBE) * DB + (k - c) % DBE};
+  if (k < KSE) return {0, k};
+  if (k < KSE + KSV) return {1, k - KSE};
+  return {2, ((k - KSE - KSV) / DBE) * DB + (k - KSE - KSV) % DBE};
 }
 template <int ER, int DVR>
 constexpr WideOp dkdv_op(int k) {  // S steps and dP steps (in turns where both accumulators fit: two
@@ -275,7 +257,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   // groups of 4 consecutive keys, requested ahead of the tile's score products; keys past the row
   // read the next row or, past the last row, zeros (they are masked anyway)
   const int bkind = MASKED ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
       __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
@@ -353,7 +335,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
       // The LDS operands of a tile - row fragments of K and V in turns, then the transposed fragments
       // of K - travel through a register ring, three matrix ops ahead of their use, in an order
       // pinned by scheduling fences (one wavefront per SIMD has nobody to hide an LDS round trip behind).
-      constexpr int AHEAD = WIDE_DQ_AHEAD, NA = KSE + KSV, NOPS = NA + 2 * DBE;
+      constexpr int AHEAD = 3, NA = KSE + KSV, NOPS = NA + 2 * DBE;
       auto operand = [&](auto kc) {
         constexpr WideOp op = dq_op<ER, DVR>(decltype(kc)::value);
         if constexpr (op.kind == 2) return tr.cols(k_t, op.j);
@@ -369,39 +351,50 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
       // around every matrix op that adds to them)
 #pragma unroll
       for (int i = 0; i < DBE; ++i) asm volatile("" : "+a"(dqacc[i]));
+      // One wavefront per SIMD has nobody to hide its vector work behind, so the tile is scheduled by
+      // hand: the scores first; the probabilities are formed under the dP steps, spread over their
+      // slots; dS of the first 16 keys is the only vector work nothing covers, dS of the other 16 keys
+      // is formed under the dQ ops of the first 16.
+      float bl[16], pr[16];
+      uint32_t pS[8];
+      auto prob = [&](int r) {
+        const int kv = ta * BT + (r >> 2) * 8 + half * 4 + (r & 3);
+        float x;
+        if constexpr (MASKED) x = fmaf(sacc[r], c, bl[r]) - lse2;
+        else x = fmaf(sacc[r], c, -lse2);
+        pr[r] = __builtin_amdgcn_exp2f(kv > lim ? -INFINITY : x);  // (masked before the exponential: no branch)
+      };
+      auto form_ds = [&](int r) {  // elements r, r + 1
+        pS[r >> 1] = Mma<T>::pack(pr[r] * (dpacc[r] - dl), pr[r + 1] * (dpacc[r + 1] - dl));
+      };
       static_for<NA>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
         constexpr WideOp op = dq_op<ER, DVR>(k);
         ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
-        if constexpr (op.kind) dpacc = Mma<T>::run(ring[k & 7], dof[op.j], dpacc);
-        else sacc = Mma<T>::run(ring[k & 7], qf[op.j], sacc);
+        if constexpr (op.kind) {
+          dpacc = Mma<T>::run(ring[k & 7], dof[op.j], dpacc);
+          if constexpr (op.j == 0 && MASKED) bias_log2(bl);
+#pragma unroll
+          for (int r = (op.j * 16) / KSV; r < ((op.j + 1) * 16) / KSV; ++r) prob(r);
+        } else {
+          sacc = Mma<T>::run(ring[k & 7], qf[op.j], sacc);
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
-      uint32_t pS[8];
-      float bl[16];
-      if constexpr (MASKED) bias_log2(bl);
 #pragma unroll
-      for (int r = 0; r < 16; r += 2) {
-        float ds[2];
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-          const int kv = ta * BT + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
-          float pr;
-          if constexpr (MASKED) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
-          else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
-          pr = kv > lim ? 0.f : pr;
-          ds[e] = pr * (dpacc[r + e] - dl);
-        }
-        pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
-      }
+      for (int r = 0; r < 8; r += 2) form_ds(r);
       __builtin_amdgcn_sched_barrier(0);
       static_for<2 * DBE>([&](auto ic) {
-        constexpr int k = NA + decltype(ic)::value;
+        constexpr int i = decltype(ic)::value, k = NA + i;
         constexpr WideOp op = dq_op<ER, DVR>(k);
         if constexpr (k + AHEAD < NOPS) ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
         constexpr int r0 = (op.j / DB) * 4;
         const u32x4 bS = {pS[r0], pS[r0 + 1], pS[r0 + 2], pS[r0 + 3]};
         dqacc[op.j % DB] = Mma<T>::run(ring[k & 7], bS, dqacc[op.j % DB]);
+        if constexpr (i < DBE) {  // the four pairs of the second 16 keys, spread over the first DBE slots
+#pragma unroll
+          for (int q = (i * 4) / DBE; q < ((i + 1) * 4) / DBE; ++q) form_ds(8 + 2 * q);
+        }
         __builtin_amdgcn_sched_barrier(0);
       });
     }
@@ -475,10 +468,10 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   // bias of this lane's key in the 32 rows of an item, one element per score register, requested
   // ahead of the item's first product through a resource that ends with the (batch, head)'s last row
   const int bkind = MASKED ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
   const uint32_t b_rowbytes = MASKED ? (uint32_t)(p.bias_sl * besz) : 0u;
   const uint32_t b_lane = MASKED ? (uint32_t)((half * 4 * p.bias_sl + min(key, p.S - 1)) * besz) : 0u;
-  const int b_records = MASKED ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0;
+  const int b_records = MASKED ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
   uint32_t braw[16];
   auto load_bias = [&](int hg, int q0) {
     if constexpr (MASKED) {
@@ -597,7 +590,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       // operands - row fragments of Q, then of dO, then the transposed fragments of dO, then of Q -
       // travel through one register ring, two to four matrix ops ahead of their use, with the order
       // pinned by scheduling fences.
-      constexpr int AHEAD = ER + DVR <= 320 ? WIDE_KV_AHEAD_S : WIDE_KV_AHEAD_L, NOPS = KSE + KSV + 2 * (DBE + DBV);  // (deeper where the widths leave registers)
+      constexpr int AHEAD = ER + DVR <= 320 ? 4 : 2, NOPS = KSE + KSV + 2 * (DBE + DBV);  // (deeper where the widths leave registers)
       auto operand = [&](auto kc) {
         constexpr WideOp op = dkdv_op<ER, DVR>(decltype(kc)::value);
         if constexpr (op.kind >= 2) return tr.cols(op.kind == 3 ? q_t : do_t, op.j);
