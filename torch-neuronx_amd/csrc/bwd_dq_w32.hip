@@ -448,7 +448,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) {
             const int kv = kv0 + (r >> 2) * 8 + half * 4 + (r & 3);
-            if (kv > lim || (FUNC && kv < lo_w && kv >= n_sink)) scur[r] = -INFINITY;
+            // (bitwise on purpose: with || and && every element gets a cascade of branches)
+            const bool dead = FUNC ? (kv > lim) | ((kv < lo_w) & (kv >= n_sink)) : kv > lim;
+            scur[r] = dead ? -INFINITY : scur[r];
           }
         }
         __builtin_amdgcn_sched_barrier(0);

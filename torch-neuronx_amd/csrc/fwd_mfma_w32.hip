@@ -322,7 +322,9 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kv = kv0 + (r >> 2) * 8 + half * 4 + (r & 3);
-      if (kv > lim || (FUNC && kv < lo_w && kv >= n_sink)) s[r] = -INFINITY;
+      // (bitwise on purpose: with || and && every element gets a cascade of branches)
+      const bool dead = FUNC ? (kv > lim) | ((kv < lo_w) & (kv >= n_sink)) : kv > lim;
+      s[r] = dead ? -INFINITY : s[r];
     }
   };
   // Bias of the score tile: lane = query row, 4 groups of 4 consecutive keys.  The resource starts
