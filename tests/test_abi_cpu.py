@@ -173,13 +173,16 @@ def test_kernel_gates(amd):
     assert gate(q, k, v, attn_bias=_meta(8192, 8192)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # masked calls too
     q64, k64 = _meta(1, 8, 512, 64), _meta(1, 8, 512, 64)
     assert gate(q64, k64, k64, attn_bias=_meta(512, 512)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
-    assert gate(q, k, v, dropout_p=0.1) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q, k, v, dropout_p=0.1) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # dropout: 16-bit, head dims up to 128, no bias
+    assert gate(q, k, v, dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q.float(), k.float(), v.float(), dropout_p=0.1) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(q, k, v, scale=0.0) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(q, k, v, scale=0.25) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q96 = _meta(2, 8, 512, 96)  # narrow head dims (multiples of 8) run padded in the next wider kernel
     assert gate(q96, q96, q96, is_causal=True) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q256 = _meta(2, 8, 512, 256)  # head dims up to 256, forward and backward
     assert gate(q256, q256, q256) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
+    assert gate(q256, q256, q256, dropout_p=0.1) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     q100 = _meta(2, 8, 512, 100)
     assert gate(q100, q100, q100) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     q2, k2 = _meta(1, 4, 64, 192), _meta(1, 4, 64, 192)

@@ -161,6 +161,84 @@ def test_backward_with_dropout_mask(amd, gpu_device):
         assert max_abs(a, r) <= 5e-5
 
 
+DROPOUT_MFMA = [
+    # B, Hq, Hkv, L, S, E, causal, kv_lens, dropout_p
+    (1, 2, 2, 64, 64, 64, False, None, 0.25),
+    (2, 4, 2, 300, 260, 128, True, None, 0.1),
+    (2, 4, 4, 129, 512, 64, False, [512, 77], 0.5),
+    (1, 8, 2, 1030, 1028, 128, True, None, 0.1),
+    (3, 3, 1, 33, 36, 40, False, [36, 1, 20], 0.3),
+    (1, 2, 2, 256, 256, 96, True, None, 1.0),
+    (2, 12, 12, 512, 512, 64, False, [512, 300], 0.1),  # a BERT-base layer with right padding
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", DROPOUT_MFMA, ids=lambda c: "B%d_Hq%d_Hkv%d_L%d_S%d_E%d_c%d_p%s" % (c[:7] + (c[8],)))
+def test_dropout_in_the_matrix_op_kernels(amd, gpu_device, case, dtype):
+    """Forward and backward with a keep-mask through the MFMA kernels (forced: the call fails if they
+    cannot take it), against the oracle's dropout (torch_neuronx/_sdpa_math.py:36-48, :154-158)."""
+    B, Hq, Hkv, L, S, E, causal, lens, pdrop = case
+    dev = gpu_device
+    g = torch.Generator().manual_seed(L * 7 + S)
+    q, k, v, go = (torch.randn(s_, generator=g).to(dtype) for s_ in ((B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, E), (B, Hq, L, E)))
+    go = (go.float() * 0.1).to(dtype)
+    keep = (torch.rand(B, Hq, L, S, generator=g) >= pdrop) if pdrop < 1.0 else torch.zeros(B, Hq, L, S, dtype=torch.bool)
+    kw, mask = {}, None
+    if lens is not None:
+        kw["kv_lens"] = torch.tensor(lens, dtype=torch.int32, device=dev)
+        mask = (torch.arange(S)[None] < torch.tensor(lens)[:, None])[:, None, None, :].expand(B, Hq, L, S)
+    if causal:
+        cm = torch.ones(L, S, dtype=torch.bool).tril()
+        mask = cm[None, None].expand(B, Hq, L, S) if mask is None else (mask & cm)
+    bias = None if mask is None else torch.where(mask, 0.0, float("-inf"))
+    rep = Hq // Hkv
+    kf, vf = k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1)
+    ro, rl = om.compute_attention(q.float(), kf, vf, bias, keep, E**-0.5, False, pdrop)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(go.float(), q.float(), kf, vf, bias, keep, ro, rl, E**-0.5, False, pdrop)
+    rdk, rdv = rdk.view(B, Hkv, rep, S, E).sum(2), rdv.view(B, Hkv, rep, S, E).sum(2)
+    MFMA = amd._lib.KERNEL_MFMA
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), is_causal=causal, dropout_p=pdrop,
+                                dropout_keep=keep.to(dev), force_kernel=MFMA, **kw)
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, is_causal=causal,
+                                      dropout_p=pdrop, dropout_keep=keep.to(dev), force_kernel=MFMA, **kw)
+    tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
+    assert max_abs(out, ro) <= tol
+    live = torch.isfinite(rl)
+    assert max_abs(lse.cpu()[live], rl[live]) <= 2e-3 and torch.equal(torch.isfinite(lse.cpu()), live)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
+def test_dropout_with_a_padding_mask_through_the_operator(amd, gpu_device):
+    """What a BERT layer in training sends: an additive (B,1,1,S) padding mask and dropout_p = 0.1.  The
+    mask becomes key counts, the keep-mask goes into the MFMA kernels, and forward / backward agree
+    with the oracle given the mask that the forward drew."""
+    from torch_neuronx_amd import mask_patterns
+    B, H, S, E = 2, 12, 256, 64
+    dev = gpu_device
+    g = torch.Generator().manual_seed(3)
+    q, k, v, go = (torch.randn(B, H, S, E, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
+    lens = torch.tensor([256, 100])
+    pad = torch.where(torch.arange(S)[None] < lens[:, None], 0.0, float("-inf"))[:, None, None, :].to(torch.bfloat16).to(dev)
+    op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    opb = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    mask_patterns.clear_cache()
+    r = op(q, k, v, pad, 0.1)
+    keep = r[6]
+    assert keep.shape == (B, H, S, S)
+    dq, dk, dv, _ = opb(go, q, k, v, pad, [True, True, True, False], r[0], r[1], None, None, S, S, 0.1, False, keep, r[7])
+    bias = pad.float().cpu().expand(B, H, S, S)
+    qc, kc, vc, gc = (t.float().cpu() for t in (q, k, v, go))
+    ro, rl = om.compute_attention(qc, kc, vc, bias, keep.cpu().bool(), E**-0.5, False, 0.1)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(gc, qc, kc, vc, bias, keep.cpu().bool(), ro, rl, E**-0.5, False, 0.1)
+    assert max_abs(r[0], ro) <= 2e-2 and max_abs(r[1], rl) <= 2e-3
+    for a, b_ in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, b_) <= 1e-2
+    frac = keep.float().mean().item()
+    assert 0.88 < frac < 0.92
+
+
 def test_backward_kv_lens(amd, gpu_device):
     q, k, v, go = qkv(3, 4, 2, 5, 64, 32, dtype=torch.float32, seed=4, with_do=True)
     lens = torch.tensor([64, 1, 17], dtype=torch.int32)

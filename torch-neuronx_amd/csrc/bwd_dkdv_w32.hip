@@ -90,6 +90,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // sliding window (masked variant without a per-score bias): rows past the window of the block's last
   // key see none of its keys, unless the block holds sink keys
   constexpr bool FUNC = MASK == 1;
+  // MASK = 3 is dropout: the (B, Hq, L, S) keep-mask is fetched like a bool bias by the wavefronts that
+  // form the probabilities.  They feed dV with the kept probabilities and hand all of them to the dK
+  // wavefronts, the dropped ones with the sign bit set (a probability is never negative): dP is
+  // multiplied by keep / (1 - p) there (torch_neuronx/_sdpa_math.py:36-48, :154-158).
+  constexpr bool BIASED = MASK >= 2, DROP = MASK == 3;
   const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
   // the query rows that see this lane's key are first_q .. past_q - 1: from the key itself on under a
   // causal mask, none for a key past the batch's count, up to the end of the key's window unless it is a sink
@@ -262,11 +267,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
   };
 
-  const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
   const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
-  const uint32_t b_rowbytes = MASK == 2 ? (uint32_t)(p.bias_sl * besz) : 0u;
-  const uint32_t b_lane = MASK == 2 ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
-  const int b_records = MASK == 2 ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
+  const uint32_t b_rowbytes = BIASED ? (uint32_t)(p.bias_sl * besz) : 0u;
+  const uint32_t b_lane = BIASED ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
+  const int b_records = BIASED ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
   // the fetched bias elements of a tile, turned into floats in the log2 domain in place (the
   // element type is tested once, outside the loops: inside, every element would carry the branch)
   auto bias_to_log2 = [&](uint32_t (&w)[2][16]) {
@@ -289,7 +294,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // lse = +inf), keys past S as a neighbouring element (their probabilities are replaced by zero).
   uint32_t braw[2][16];
   auto load_bias_a = [&](int it) {
-    if constexpr (MASK == 2) {
+    if constexpr (BIASED) {
       const int q0 = item_q0(it);
       if (it >= n_items || (p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
       const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
@@ -334,6 +339,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;  // [4 groups of 4 words][lane][4]
     f32x16 sc[2];
     uint32_t pk[2][8];
+    uint32_t pkx[DROP ? 2 : 1][8];  // (dropout) what the dK wavefronts get: every probability, the dropped ones negative
     f32x4 l4[2][4];
     u32x4 ring[8];
     auto load_l4 = [&](int mq, int r4) { l4[mq][r4] = *(const f32x4*)(lrow + mq * 32 + r4 * 8); };
@@ -351,7 +357,13 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       for (int k = 0; k < EPS; k += 2) {
         const int r = slot * EPS + k;
         const float p0 = prob(mq, r), p1 = prob(mq, r + 1);
-        pk[mq][r >> 1] = Mma<T>::pack(p0, p1);
+        if constexpr (DROP) {
+          const float s0 = braw[mq][r] ? p0 : -p0, s1 = braw[mq][r + 1] ? p1 : -p1;
+          pkx[mq][r >> 1] = Mma<T>::pack(s0, s1);
+          pk[mq][r >> 1] = Mma<T>::pack(fmaxf(s0, 0.f), fmaxf(s1, 0.f));
+        } else {
+          pk[mq][r >> 1] = Mma<T>::pack(p0, p1);
+        }
       }
     };
     auto mask_scores = [&](int mq) {
@@ -366,8 +378,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       }
     };
     auto hand_over = [&](int mq) {
-      *(u32x4*)(px + (2 * mq) * 256) = u32x4{pk[mq][0], pk[mq][1], pk[mq][2], pk[mq][3]};
-      *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{pk[mq][4], pk[mq][5], pk[mq][6], pk[mq][7]};
+      const uint32_t(&w)[8] = DROP ? pkx[DROP ? mq : 0] : pk[mq];
+      *(u32x4*)(px + (2 * mq) * 256) = u32x4{w[0], w[1], w[2], w[3]};
+      *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{w[4], w[5], w[6], w[7]};
     };
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i) ring[i] = read_rows(qt, i);
@@ -453,8 +466,16 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     auto load_d4 = [&](int mq, int r4) { d4[mq][r4] = *(const f32x4*)(drow + mq * 32 + r4 * 8); };
     auto ds_pair = [&](int mq, int r) {  // elements r, r + 1
       const uint32_t word = w[mq][r >> 3][(r >> 1) & 3];
-      const float s0 = Mma<T>::unpack(word, 0) * (dp[mq][r] - d4[mq][r >> 2][r & 3]);
-      const float s1 = Mma<T>::unpack(word, 1) * (dp[mq][r + 1] - d4[mq][(r + 1) >> 2][(r + 1) & 3]);
+      float s0, s1;
+      if constexpr (DROP) {  // a negative probability was dropped: its dP counts as zero
+        const float p0 = Mma<T>::unpack(word, 0), p1 = Mma<T>::unpack(word, 1);
+        const float t0 = p0 < 0.f ? 0.f : dp[mq][r] * p.keep_scale, t1 = p1 < 0.f ? 0.f : dp[mq][r + 1] * p.keep_scale;
+        s0 = fabsf(p0) * (t0 - d4[mq][r >> 2][r & 3]);
+        s1 = fabsf(p1) * (t1 - d4[mq][(r + 1) >> 2][(r + 1) & 3]);
+      } else {
+        s0 = Mma<T>::unpack(word, 0) * (dp[mq][r] - d4[mq][r >> 2][r & 3]);
+        s1 = Mma<T>::unpack(word, 1) * (dp[mq][r + 1] - d4[mq][(r + 1) >> 2][(r + 1) & 3]);
+      }
       pk[mq][r >> 1] = Mma<T>::pack(s0, s1);
     };
     w[0][0] = *(const u32x4*)(px), w[0][1] = *(const u32x4*)(px + 256);
@@ -549,7 +570,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   if (key < p.S) {
     uint16_t* g = role ? (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl
                        : (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
-    const float sc = role ? p.scale : 1.f;
+    const float sc = role ? p.scale : DROP ? p.keep_scale : 1.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -576,6 +597,7 @@ int launch_t(const BwdM& g, hipStream_t s) {
 }
 template <typename T, int D>
 int launch_m(const BwdM& g, hipStream_t s) {
+  if (g.keep_scale != 0.f) return launch_t<T, D, 3>(g, s);
   if (g.bias_kind && g.bias_sl != 0) return launch_t<T, D, 2>(g, s);
   return (g.bias_kind || g.kv_lens || g.d_real != D || g.window > 0) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
 }

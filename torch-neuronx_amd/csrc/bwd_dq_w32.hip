@@ -40,7 +40,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int NBUF = 4;  // tile t lives in buffer t % 4
   // (the variant with a bias takes the launch's dynamic LDS: behind the tiles it keeps the list of the
   // key tiles it walks when the call brings a skip table, and a kernel may declare 64 KB at most)
-  constexpr bool DYN = MASK == 2;
+  // MASK = 3 is dropout: the (B, Hq, L, S) keep-mask is fetched like a bool bias, leaves the scores alone and
+  // multiplies dP, together with 1 / (1 - p) (torch_neuronx/_sdpa_math.py:36-48, :154-158)
+  constexpr bool BIASED = MASK >= 2, DROP = MASK == 3;
+  constexpr bool DYN = BIASED;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
   __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : NBUF * TILE];
   extern __shared__ __attribute__((aligned(16))) uint16_t dyn_lds[];
@@ -312,16 +315,16 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // fetched one tile ahead as 4 groups of 4 consecutive keys; keys past the row read the next row
   // or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
-  const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
   const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
   // (set up unconditionally, with no records when there is no bias: a resource that is defined on
   // one path only stops being uniform for the compiler)
   const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
       uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
       __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
-  const uint32_t b_row = MASK == 2 ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
+  const uint32_t b_row = BIASED ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
   auto load_bias = [&](int t) {
-    if constexpr (MASK == 2) {
+    if constexpr (BIASED) {
       const uint32_t off = b_row + (uint32_t)((listed ? tile_of(min(t, max(nt - 1, 0))) : t) * BN * besz);
       if (bkind == 1) {
 #pragma unroll
@@ -378,7 +381,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
             const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
             pr = kv > lim ? 0.f : pr;
           }
-          ds[e] = pr * (dpacc[r + e] - dl);
+          if constexpr (DROP) {
+            const float keep = (float)((braw[(r + e) >> 2] >> (8 * ((r + e) & 3))) & 0xffu);
+            ds[e] = pr * fmaf(dpacc[r + e] * keep, p.keep_scale, -dl);
+          } else {
+            ds[e] = pr * (dpacc[r + e] - dl);
+          }
         }
         pS[r >> 1] = Mma<T>::pack(ds[0], ds[1]);
       }
@@ -418,7 +426,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   __syncthreads();
   load_tile(2);
   f32x16 s_a, dp_a, s_b, dp_b;
-  if (MASK != 2 && nt_w > 0) scores(0, s_a, dp_a);
+  if (!BIASED && nt_w > 0) scores(0, s_a, dp_a);
   auto iteration = [&](int t, auto tile_mod, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
     // (t % 4 is a compile-time constant, four copies of the iteration: the buffer of a tile then is
     // an immediate offset of the LDS reads, not an addition on the vector unit per read)
@@ -429,7 +437,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     if (t < nt_w) {
       // (the variant with a bias has no registers to spare for a second score tile: it computes the
       // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap)
-      if constexpr (MASK == 2) {
+      if constexpr (BIASED) {
         scores(buf, scur, dpcur);
         uint32_t pS[8];
         softmax(t, scur, dpcur, pS);
@@ -535,22 +543,26 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
   const bool bf = dtype == MI355_SDPA_BF16;
-  const int mask = (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
+  const int mask = g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
   // (the variant with a bias: its tiles, and the tile list of a call with a skip table, in dynamic LDS)
-  const int dyn = mask == 2 ? 2 * 4 * BN * head_dim * 2 + 2048 + 16 : 0;
-  if (mask == 2) {
-    const void* fn = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 2>)
-                                     : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 2>);
+  const int dyn = mask >= 2 ? 2 * 4 * BN * head_dim * 2 + 2048 + 16 : 0;
+  if (mask >= 2) {
+    const void* fn2 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 2>)
+                                      : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 2>);
+    const void* fn3 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 3> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 3>)
+                                      : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 3> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 3>);
+    const void* fn = mask == 3 ? fn3 : fn2;
     const hipError_t attr = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, dyn);
     if (attr != hipSuccess) {
       set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dq_w32_kernel: %s", dyn, hipGetErrorString(attr));
       return MI355_SDPA_ERR_LAUNCH;
     }
   }
-#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, (MM) == 2 ? dyn : 0, s, g)
+#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, (MM) >= 2 ? dyn : 0, s, g)
 #define LAUNCH_M(TT, DD)                                                     \
   do {                                                                       \
-    if (mask == 2) LAUNCH(TT, DD, 2);                                        \
+    if (mask == 3) LAUNCH(TT, DD, 3);                                        \
+    else if (mask == 2) LAUNCH(TT, DD, 2);                                   \
     else if (mask == 1) LAUNCH(TT, DD, 1);                                   \
     else LAUNCH(TT, DD, 0);                                                  \
   } while (0)

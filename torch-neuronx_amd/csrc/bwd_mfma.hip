@@ -550,6 +550,12 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
       g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
     }
   }
+  if (p.dropout_p > 0.f && !p.bias.data) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
+    g.bias = p.dropout_keep;
+    g.bias_sl = g.S, g.bias_sh = (int64_t)g.L * g.S, g.bias_sb = (int64_t)g.Hq * g.bias_sh;
+    g.bias_kind = 4;
+    g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
+  }
 }
 
 bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
@@ -589,7 +595,14 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
     if (((p.q.size[2] + 64) * (p.q.size[2] > 1 ? p.bias.stride[2] : 0) + S + 64) * esz >= (1ll << 31))
       return *why = "attn_bias rows beyond 32-bit offsets", false;
   }
-  if (p.dropout_p > 0.f) return *why = "dropout", false;
+  if (p.dropout_p > 0.f) {
+    // the keep-mask takes the bias's way into the kernels (one dword = four keys of a row)
+    const int64_t S = p.k.size[2];
+    if (p.bias.data || p.grad_bias.data || p.mask.window > 0) return *why = "dropout together with attn_bias or a window functor", false;
+    if (wide) return *why = "dropout with a head dim above 128 or D_qk != D_v", false;
+    if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
+    if ((p.q.size[2] + 64) * S + S + 64 >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
+  }
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
   if (p.mask.window > 0 && p.bias.data) return *why = "window functor together with attn_bias", false;
@@ -601,7 +614,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
       if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
   }
   if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
-  if (!wide && (p.bias.data || p.kv_lens || padded || p.mask.window > 0)) {
+  if (!wide && (p.bias.data || p.kv_lens || padded || p.mask.window > 0 || p.dropout_p > 0.f)) {
     BwdM g;
     fill(g, p);
     const int D = E <= 64 ? 64 : 128;

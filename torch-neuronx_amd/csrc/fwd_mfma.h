@@ -23,6 +23,9 @@ struct FwdM {
   const void* bias = nullptr;
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  // dropout (fwd_mfma_w32.hip, head dims up to 128, no bias): nonzero = 1 / (1 - p) (1 for p = 1), and the
+  // bias fields above describe the (B, Hq, L, S) keep-mask, kind 4
+  float keep_scale = 0.f;
   const int32_t* kv_lens = nullptr;
   // Elements per row that exist (a multiple of 8).  Below the head dim a kernel is built for, the
   // masked variant treats the rest of every Q / K / V row as zeros and leaves it out of the output

@@ -355,7 +355,16 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
     if ((31 * p.bias.stride[2] + S) * esz >= (1ll << 31)) return *why = "attn_bias rows beyond 32-bit offsets", false;
     (void)L;
   }
-  if (p.dropout_p > 0.f) return *why = "dropout", false;
+  if (p.dropout_p > 0.f) {
+    // the keep-mask takes the bias's way into the kernel (one dword = four keys of a row)
+    const int64_t S = p.k.size[2];
+    if (p.bias.data || p.mask.window > 0 || p.mask.sink_logit) return *why = "dropout together with attn_bias or a window / sink functor", false;
+    if (E > 128) return *why = "dropout with a head dim above 128", false;
+    if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
+    if (32 * S >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
+    if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
+      return *why = "dropout with rows beyond 32-bit offsets", false;
+  }
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
   if ((p.mask.window > 0 || p.mask.sink_logit) && (p.bias.data || E > 128))
@@ -392,6 +401,12 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     g.bias = p.bias.data;
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1], g.bias_sl = p.bias.stride[2];
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
+  }
+  if (p.dropout_p > 0.f) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
+    g.bias = p.dropout_keep;
+    g.bias_sl = p.k.size[2], g.bias_sh = p.q.size[2] * g.bias_sl, g.bias_sb = p.q.size[1] * g.bias_sh;
+    g.bias_kind = 4;
+    g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;

@@ -44,6 +44,10 @@ constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescale
 // score tile right after the matrix ops that produce it.  The bias travels like the tiles: from
 // global memory straight into LDS (lane-private slots), with loads written as assembly and
 // awaited by count, so that nothing in the loop waits on a count the compiler chose.
+// MASK = 3 is dropout: the (B, Hq, L, S) keep-mask travels like a boolean bias, but it leaves the
+// scores, the row sums and the lse alone and zeroes the dropped probabilities where they are packed
+// for the second product; 1 / (1 - p) is applied with the final normalisation
+// (torch_neuronx/_sdpa_math.py:36-48: the mask multiplies the normalised probabilities).
 template <typename T, int D, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
@@ -56,7 +60,8 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // (head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare:
   // they take the launch's dynamic LDS instead; head dim 256 runs one wavefront per SIMD with the
   // 512-register budget)
-  constexpr bool DYN = D > 128 || MASK == 2;
+  constexpr bool BIASED = MASK >= 2, DROP = MASK == 3;  // a per-score tensor in LDS; ... that is a dropout keep-mask
+  constexpr bool DYN = D > 128 || BIASED;
   // Tiles go from global memory straight into LDS (see the staging section): four unpadded,
   // swizzled buffers per operand, tile t in buffer t % 4.
   // mask functors (window, sink keys, sink logit): in the masked variant without a bias, head dim <= 128
@@ -343,18 +348,18 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // younger loads are those of the pair requested at the end of the previous iteration.
   uint32_t braw[4];
   float inv_scale = 0.f;
-  const int bkind = MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int b_esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const int b_rows = min(32, p.L - qw0);
   const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * b_esz : 0),
                                   (bkind && b_rows > 0) ? (int)(((b_rows - 1) * p.bias_sl + p.S) * b_esz) : 0);
   const uint32_t b_voff = (uint32_t)((min(col, max(b_rows - 1, 0)) * p.bias_sl + half * (bkind == 1 ? 4 : bkind == 4 ? 16 : 8)) * b_esz);
   const int b_loads = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
-  const unsigned char* const bias_w = (const unsigned char*)bias_lds + (MASK == 2 ? wave * 4096 : 0);
+  const unsigned char* const bias_w = (const unsigned char*)bias_lds + (BIASED ? wave * 4096 : 0);
   const uint32_t lds_b = (uint32_t)(uintptr_t)(lds_bytes)bias_w;
   if (bkind) inv_scale = 1.f / p.scale;
   auto load_bias = [&](int t) {
-    if constexpr (MASK == 2) {
+    if constexpr (BIASED) {
       if (bkind) {
         // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -370,7 +375,11 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   };
   // (awaited: in the loop.  This wait also covers the pair that the iteration's barrier publishes.)
   auto apply_bias = [&](f32x16& sv, bool awaited) {
-    if constexpr (MASK == 2) {
+    if constexpr (DROP) {  // the tile's keep bytes, used where its probabilities are packed
+      if (awaited) wait_youngest_pair_only();
+#pragma unroll
+      for (int g = 0; g < 4; ++g) braw[g] = *(const uint32_t*)(bias_w + (col + 32 * (g >> 1)) * 16 + (g & 1) * 8 + half * 4);
+    } else if constexpr (MASK == 2) {
       if (awaited) wait_youngest_pair_only();
       if (bkind == 1) {
         // (head dim 256 has no registers to spare: one group at a time there)
@@ -473,7 +482,13 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   auto stage3 = [&](int j, uint32_t (&pk)[8], float& ps) {
     ps += pv[j & 1][0] + pv[j & 1][1];
     asm volatile("" : "+v"(ps));  // keeps the add in its slot (left alone it sinks below the loop body)
-    pk[j] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
+    if constexpr (DROP) {  // (the sum above keeps the dropped probabilities)
+      const int r = 2 * j;
+      const float k0 = (float)((braw[r >> 2] >> (8 * (r & 3))) & 0xffu), k1 = (float)((braw[r >> 2] >> (8 * (r & 3) + 8)) & 0xffu);
+      pk[j] = Mma<T>::pack(pv[j & 1][0] * k0, pv[j & 1][1] * k1);
+    } else {
+      pk[j] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
+    }
   };
   // Pairs 0..3 hold the tile's first 16 keys (the first contraction step of P*V), pairs 4..7 the
   // last 16.  Four pairs are spread over the eight matrix ops of a phase:
@@ -604,7 +619,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
     for (int i = 0; i < NPV; ++i) {  // i = DB * (16-key step) + d block
       if (i == NPV - 2) {
-        if constexpr (MASK != 2) wait_oldest_pair();  // (with a bias: awaited together with the bias)
+        if constexpr (!BIASED) wait_oldest_pair();  // (with a bias: awaited together with the bias)
         __syncthreads();
       }
       if (i + AHEAD < NPV) ring[(KS + i + AHEAD) & 7] = read_v(i + AHEAD);
@@ -661,6 +676,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
   float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
   float lse_row = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+  if constexpr (DROP) inv *= p.keep_scale;
   if constexpr (FUNC) {
     // the sink logit joins the row's maximum and sum (flex_attention.py.jinja:1921-1923, :2134-2140)
     if (p.sink_logit) {
@@ -708,9 +724,9 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 template <typename T, int D, int WAVES, int MASK>
 int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
   int bytes = 0;
-  if constexpr (D > 128 || MASK == 2) {
+  if constexpr (D > 128 || MASK >= 2) {
     // (four buffers per operand, 4 KB of bias tile per wavefront, and the tile list of a call with a skip table)
-    constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK == 2 ? WAVES * 4096 : 0);
+    constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK >= 2 ? WAVES * 4096 : 0);
     constexpr int kBytes = kBase + (MASK == 2 ? 2048 + 16 : 0);
     static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
@@ -725,6 +741,9 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
 }
 template <typename T, int D, int WAVES>
 int launch_mask(const FwdM& g, int mask, dim3 grid, hipStream_t s) {
+  if constexpr (D <= 128) {
+    if (mask == 3) return launch_one<T, D, WAVES, 3>(g, grid, s);
+  }
   if (mask == 2) return launch_one<T, D, WAVES, 2>(g, grid, s);
   if (mask == 1) return launch_one<T, D, WAVES, 1>(g, grid, s);
   return launch_one<T, D, WAVES, 0>(g, grid, s);
@@ -752,7 +771,11 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
   }
   const dim3 grid((unsigned)blocks);
   // kernel variant: 2 with a bias or keep-mask, 1 with key counts or rows narrower than the kernel's head dim
-  const int mask = g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit) ? 1 : 0;
+  if (g.keep_scale != 0.f && (head_dim > 128 || g.bias_kind != 4)) {
+    set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128 and the keep-mask in the bias slot");
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  const int mask = g.keep_scale != 0.f ? 3 : g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit) ? 1 : 0;
   const int rc = dtype == MI355_SDPA_BF16 ? launch_dims<bf16_t>(g, head_dim, waves, mask, grid, s)
                                           : launch_dims<f16_t>(g, head_dim, waves, mask, grid, s);
   if (rc != MI355_SDPA_OK) return rc;
