@@ -293,6 +293,24 @@ def extra_wide(amd, dev):
     return r
 
 
+def extra_dropout(amd, dev):
+    """Dropout 0.1 with right padding, a BERT-base layer in training: B=32 H=12 S=512 D=64 bf16, key counts
+    between S/2 and S, the (B,H,S,S) keep-mask drawn once.  Rates count the scores that the padding keeps."""
+    B, H, S, D = 32, 12, 512, 64
+    q, k, v, do = seeded([(B, H, S, D)] * 4, 1012, torch.bfloat16, dev)
+    g = torch.Generator(device="cpu").manual_seed(1012)
+    lens = torch.randint(S // 2, S + 1, (B,), generator=g, dtype=torch.int32)
+    keep = (torch.rand(B, H, S, S, device=dev) >= 0.1).to(torch.uint8)
+    kw = dict(kv_lens=lens.to(dev), dropout_p=0.1, dropout_keep=keep)
+    out, lse = amd.sdpa_forward(q, k, v, **kw)
+    _, evf = event_time_ms(lambda: amd.sdpa_forward(q, k, v, **kw), 10, 3)
+    _, evb = event_time_ms(lambda: amd.sdpa_backward(do, q, k, v, out, lse, **kw), 5, 2)
+    live = float(lens.sum().item()) * S * H  # kept (query, key) pairs over all batches and heads
+    return {"fwd_ms": evf, "bwd_ms": evb, "fwd_TFLOP/s_live": 4.0 * D * live / (evf * 1e-3) / 1e12,
+            "bwd_TFLOP/s_live": 10.0 * D * live / (evb * 1e-3) / 1e12,
+            "shape": "B=32 H=12 S=512 D=64 bf16, dropout 0.1, right padding (key counts)"}
+
+
 def extra_f32(amd, dev):
     """float32 inputs on the float32 matrix op (peak 157.3 TFLOP/s), B=2 Hq=32 Hkv=8 S=4096 D=128 causal."""
     B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
@@ -460,7 +478,8 @@ def main():
         except Exception as e:
             extras["masked_fwd_shared_bias"] = {"error": repr(e)}
         for name, fn in (("window_1024_fwd_bwd", extra_window), ("document_mask_tables_fwd_bwd", extra_documents),
-                         ("head_dim_256_fwd_bwd", extra_wide), ("float32_fwd_bwd", extra_f32)):
+                         ("head_dim_256_fwd_bwd", extra_wide), ("dropout_padding_fwd_bwd", extra_dropout),
+                         ("float32_fwd_bwd", extra_f32)):
             try:
                 extras[name] = fn(amd, dev)
             except Exception as e:
