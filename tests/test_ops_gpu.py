@@ -418,3 +418,33 @@ def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
         torch.cuda.synchronize()
         for i, (a, b) in enumerate(zip(captured, eager)):
             assert torch.equal(a, b), (rep, i)
+
+
+def test_fallback_to_the_generic_kernel_can_be_logged(gpu_device):
+    """MI355_SDPA_LOG_FALLBACK=1: a call that the matrix-op kernels cannot take (head dim 100) says so
+    on stderr, with the reason; a call they take says nothing.  (A child process: the switch is read once.)"""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    code = (
+        "import sys, torch\n"
+        f"sys.path.insert(0, {root!r}); sys.path.insert(0, {os.path.join(root, 'torch-neuronx_amd')!r})\n"
+        "import torch_neuronx_amd as amd\n"
+        "d = torch.device('cuda:0')\n"
+        "q = torch.randn(1, 2, 64, 128, device=d, dtype=torch.bfloat16)\n"
+        "amd.sdpa_forward(q, q, q, is_causal=True)\n"
+        "print('--', file=sys.stderr, flush=True)\n"
+        "q = torch.randn(1, 2, 64, 100, device=d, dtype=torch.bfloat16)\n"
+        "o, l = amd.sdpa_forward(q, q, q)\n"
+        "amd.sdpa_backward(q, q, q, q, o, l)\n"
+        "torch.cuda.synchronize()\n"
+    )
+    env = dict(os.environ, MI355_SDPA_LOG_FALLBACK="1")
+    r = subprocess.run([sys.executable, "-c", code], env=env, capture_output=True, text=True, timeout=300)
+    assert r.returncode == 0, r.stderr
+    before, _, after = r.stderr.partition("--")
+    assert "mi355_sdpa" not in before
+    assert "forward runs in the generic kernel: head dims are not multiples of 8" in after
+    assert "backward runs in the generic kernel" in after

@@ -3,9 +3,11 @@
 // include/mi355_sdpa.h for the contract of every entry point.
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <algorithm>
+#include <atomic>
 
 #include "common.h"
 
@@ -257,6 +259,18 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
 int mi355_sdpa_can_use_fused_fwd(const mi355_sdpa_desc* d) { return kernel_for(d, false); }
 int mi355_sdpa_can_use_fused_bwd(const mi355_sdpa_desc* d) { return kernel_for(d, true); }
 
+// With MI355_SDPA_LOG_FALLBACK set in the environment, the first calls that the matrix-op kernels
+// cannot take say so on stderr, with the reason: the generic kernels are a correctness path two
+// orders of magnitude slower, and nothing else tells a caller that a call went there.
+static void note_fallback(const char* what, const char* why) {
+  static const bool on = [] {
+    const char* e = getenv("MI355_SDPA_LOG_FALLBACK");
+    return e && *e && strcmp(e, "0") != 0;
+  }();
+  static std::atomic<int> left{16};
+  if (on && left.fetch_sub(1) > 0) fprintf(stderr, "mi355_sdpa: %s runs in the generic kernel: %s\n", what, why && *why ? why : "(no reason recorded)");
+}
+
 int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
   if (!p) return set_error("SDPA: null params"), MI355_SDPA_ERR_INVALID;
   if (!tensor_ok(p->q, "query") || !tensor_ok(p->k, "key") || !tensor_ok(p->v, "value") ||
@@ -277,9 +291,11 @@ int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
   const char* why = "";
   int kernel = p->force_kernel;
   const bool f32 = p->dtype == MI355_SDPA_F32;
-  if (kernel == 0)
+  if (kernel == 0) {
     kernel = (f32 ? fwd_f32_mfma_supported(*p, &why) : fwd_mfma_supported(*p, &why)) ? MI355_SDPA_KERNEL_MFMA
                                                                                      : MI355_SDPA_KERNEL_GENERIC;
+    if (kernel == MI355_SDPA_KERNEL_GENERIC) note_fallback("forward", why);
+  }
   if (kernel == MI355_SDPA_KERNEL_MFMA || kernel == MI355_SDPA_KERNEL_MFMA_T128 ||
       kernel == MI355_SDPA_KERNEL_MFMA_T256)
     return f32 ? launch_fwd_f32_mfma(*p, s) : launch_fwd_mfma(*p, s);
@@ -315,10 +331,11 @@ static bool bwd_args_ok(const mi355_sdpa_bwd_params* p) {
   return true;
 }
 
-static int bwd_kernel_choice(const mi355_sdpa_bwd_params* p) {
+static int bwd_kernel_choice(const mi355_sdpa_bwd_params* p, bool log = false) {
   if (p->force_kernel) return p->force_kernel;
-  const char* why;
+  const char* why = "";
   const bool ok = p->dtype == MI355_SDPA_F32 ? bwd_f32_mfma_supported(*p, &why) : bwd_mfma_supported(*p, &why);
+  if (!ok && log) note_fallback("backward", why);
   return ok ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
 }
 
@@ -330,7 +347,7 @@ size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p) {
 
 int mi355_sdpa_bwd(const mi355_sdpa_bwd_params* p, void* stream) {
   if (!bwd_args_ok(p)) return MI355_SDPA_ERR_INVALID;
-  const int kernel = bwd_kernel_choice(p);
+  const int kernel = bwd_kernel_choice(p, true);
   const bool f32 = p->dtype == MI355_SDPA_F32;
   const size_t need = kernel != MI355_SDPA_KERNEL_MFMA ? bwd_generic_workspace(*p)
                       : f32 ? bwd_f32_mfma_workspace(*p) : bwd_mfma_workspace(*p);
