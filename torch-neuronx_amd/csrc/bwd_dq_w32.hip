@@ -311,34 +311,66 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       else sacc = Mma<T>::run(ring[i & 7], qf[i >> 1], i == 0 ? zero16 : sacc);
     }
   };
-  // Bias of a score tile: this lane's 16 keys of its query row (row stride 0: a bias per key),
-  // fetched one tile ahead as 4 groups of 4 consecutive keys; keys past the row read the next row
-  // or, past the last row, zeros (they are masked anyway).
+  // Bias of a score tile (MASK >= 2): this lane's 16 keys of its query row (row stride 0: a bias per
+  // key), as 4 groups of 4 consecutive keys.  It travels like the K / V tiles: from global memory
+  // straight into LDS, 16 bytes per lane and instruction whatever the element size, into 4 KB that
+  // belong to the wavefront -
+  //   float32     4 loads: load g, lane (row, half) -> keys 8 g + 4 half .. +3, read back by the same lane
+  //   16 bits     2 loads: load i, lane (row, half) -> keys 16 i + 8 half .. +7; group g of lane (row, half)
+  //               is the half-th 8 bytes of what lane (row, g % 2) fetched in load g / 2
+  //   bool        1 load:  lane (row, half) -> keys 16 half .. +15; group g is dword 2 (g % 2) + half of
+  //               what lane (row, g / 2) fetched
+  // - with loads written as assembly and awaited by count.  (Fetched into registers with the
+  // compiler's own loads, the wait that it puts in front of their first use covers every load in
+  // flight, the tiles requested three iterations ahead included: the kernel then waits out a trip to
+  // memory per tile.)  One buffer: the bias of tile t + 1 is requested right after that of tile t
+  // has been read back, and is awaited when tile t + 1 needs it, by then the oldest loads in flight.
+  // The resource starts at this wavefront's first row of the (batch, head) plane and ends with its
+  // last one: keys past S read the next row or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
   const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
-  const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
-  // (set up unconditionally, with no records when there is no bias: a resource that is defined on
-  // one path only stops being uniform for the compiler)
-  const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      uniform_ptr((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh) * besz : 0)), 0,
-      __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
-  const uint32_t b_row = BIASED ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
+  const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const int b_rows = min(32, p.L - qw0);
+  const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * besz : 0),
+                                  (bkind && b_rows > 0) ? ((int64_t)(b_rows - 1) * p.bias_sl + p.S) * besz : 0);
+  const uint32_t b_voff = BIASED ? (uint32_t)((min(col, max(b_rows - 1, 0)) * p.bias_sl + half * (bkind == 1 ? 4 : bkind == 4 ? 16 : 8)) * besz) : 0u;
+  const int b_loads = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
+  const unsigned char* const bias_w = (const unsigned char*)(tile_list + 1040) + (BIASED ? wave * 4096 : 0);
+  const uint32_t lds_b = (uint32_t)(uintptr_t)(lds_bytes)bias_w;
   auto load_bias = [&](int t) {
     if constexpr (BIASED) {
-      const uint32_t off = b_row + (uint32_t)((listed ? tile_of(min(t, max(nt - 1, 0))) : t) * BN * besz);
+      if (bkind) {
+        // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        const uint32_t g0 = b_voff + (uint32_t)((listed ? tile_of(min(t, max(nt - 1, 0))) : t) * BN * besz);
+        tile_load(b_rsrc, g0, lds_b);
+        if (b_loads > 1) tile_load(b_rsrc, g0 + 32, lds_b + 1024);
+        if (b_loads > 2) {
+          tile_load(b_rsrc, g0 + 64, lds_b + 2048);
+          tile_load(b_rsrc, g0 + 96, lds_b + 3072);
+        }
+      }
+    }
+  };
+  // the bias of the tile at hand, from LDS into braw (the only younger loads are those of the tile
+  // requested at the end of the previous iteration)
+  auto fetch_bias = [&]() {
+    if constexpr (BIASED) {
+      if constexpr (NDMA == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
+      else asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
       if (bkind == 1) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const u32x4 w = __builtin_amdgcn_raw_buffer_load_b128(b_rsrc, off + g * 32, 0, 0);
+          const u32x4 w = *(const u32x4*)(bias_w + g * 1024 + lane * 16);
           braw[4 * g] = w[0], braw[4 * g + 1] = w[1], braw[4 * g + 2] = w[2], braw[4 * g + 3] = w[3];
         }
       } else if (bkind == 4) {
 #pragma unroll
-        for (int g = 0; g < 4; ++g) braw[g] = __builtin_amdgcn_raw_buffer_load_b32(b_rsrc, off + g * 8, 0, 0);
+        for (int g = 0; g < 4; ++g) braw[g] = *(const uint32_t*)(bias_w + (col + 32 * (g >> 1)) * 16 + (g & 1) * 8 + half * 4);
       } else if (bkind) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-          const u32x2 w = __builtin_amdgcn_raw_buffer_load_b64(b_rsrc, off + g * 16, 0, 0);
+          const u32x2 w = *(const u32x2*)(bias_w + (g >> 1) * 1024 + (col + 32 * (g & 1)) * 16 + half * 8);
           braw[2 * g] = w[0], braw[2 * g + 1] = w[1];
         }
       }
@@ -431,17 +463,17 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     // (t % 4 is a compile-time constant, four copies of the iteration: the buffer of a tile then is
     // an immediate offset of the LDS reads, not an addition on the vector unit per read)
     constexpr int buf = decltype(tile_mod)::value, bn = (buf + 1) & (NBUF - 1);
-    // (the tile is requested at the end of the iteration: the bias loads of the variant that has
-    // them are awaited by the compiler with a count that knows nothing of the tile loads, so those
-    // had better be the older ones)
     if (t < nt_w) {
       // (the variant with a bias has no registers to spare for a second score tile: it computes the
-      // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap)
+      // scores of tile t here, and relies on the other wavefront of the SIMD alone for overlap.  The
+      // dropout variant would have them, but gains nothing from the pipelined form: it runs at the
+      // cost of reading its mask, a byte per score, from memory.)
       if constexpr (BIASED) {
         scores(buf, scur, dpcur);
         uint32_t pS[8];
-        softmax(t, scur, dpcur, pS);
+        fetch_bias();
         load_bias(t + 1);
+        softmax(t, scur, dpcur, pS);
         accumulate(buf, pS);
       } else {
         // Software pipelined by hand (a wavefront issues in order, and left alone the compiler emits
@@ -501,7 +533,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
       }
     }
     load_tile(t + 3);
-    wait_older_tiles();  // tile t + 2, read from the next iteration on
+    // Tile t + 2, read from the next iteration on, has to be whole.  (With a bias the tile read next
+    // is t + 1, and a wavefront with work has seen it land when it awaited this iteration's bias, a
+    // younger load: it leaves the bias of the next tile and the tile requested above in flight.  A
+    // wavefront without work awaits no bias and waits here.)
+    if (!BIASED || t >= nt_w) wait_older_tiles();
     __syncthreads();
   };
   for (int t = 0;;) {
@@ -544,8 +580,8 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const dim3 grid((unsigned)blocks), block(512);
   const bool bf = dtype == MI355_SDPA_BF16;
   const int mask = g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
-  // (the variant with a bias: its tiles, and the tile list of a call with a skip table, in dynamic LDS)
-  const int dyn = mask >= 2 ? 2 * 4 * BN * head_dim * 2 + 2048 + 16 : 0;
+  // (the tiles, the tile list of a call with a skip table, 4 KB of bias tile per wavefront)
+  const int dyn = mask >= 2 ? 2 * 4 * BN * head_dim * 2 + 2080 + 8 * 4096 : 0;
   if (mask >= 2) {
     const void* fn2 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 2>)
                                       : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 2>);
