@@ -266,6 +266,33 @@ def test_sliding_window_mask_takes_the_window_kernel(amd, gpu_device, monkeypatc
 
 
 @pytest.mark.gpu
+def test_sliding_window_mask_at_head_dim_256_stays_a_tensor(amd, gpu_device, monkeypatch):
+    """The kernels for head dims above 128 have no window functor: a recognised window mask is kept as a
+    tensor there (with skip tables) and runs in the matrix-op kernels, forward and backward, instead of
+    becoming a functor that only the generic kernels take."""
+    dev = gpu_device
+    B, H, L, D, W = 1, 2, 1024, 256, 256
+    q, k, v, go = qkv(B, H, H, L, L, D, dtype=torch.bfloat16, seed=6, with_do=True)
+    keep = om.window_keep_mask(L, L, W)
+    maskd = torch.zeros(L, L, dtype=torch.bfloat16, device=dev).masked_fill(~keep.to(dev), float("-inf"))
+    amd.mask_patterns.clear_cache()
+    seen, seen_b = [], []
+    f0, b0 = amd.ops.sdpa_forward, amd.ops.sdpa_backward
+    MFMA = amd._lib.KERNEL_MFMA  # forced: the call fails if the matrix-op kernels cannot take it
+    monkeypatch.setattr(amd.ops, "sdpa_forward", lambda *a, **kw: (seen.append(kw), f0(*a, **{**kw, "force_kernel": MFMA}))[1])
+    monkeypatch.setattr(amd.ops, "sdpa_backward", lambda *a, **kw: (seen_b.append(kw), b0(*a, **{**kw, "force_kernel": MFMA}))[1])
+    qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+    out = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=maskd)
+    out.backward(go.to(dev))
+    for kw in (seen[-1], seen_b[-1]):
+        assert kw["attn_bias"] is not None and not kw.get("window") and kw.get("live_tiles") is not None
+    ro, rl = om.sdpa_forward(q.float(), k.float(), v.float(), attn_mask=keep)
+    assert max_abs(out, ro) <= 2e-2
+    rdq, rdk, rdv = om.sdpa_backward(go.float(), q.float(), k.float(), v.float(), ro, rl, attn_mask=keep, reduce_in_fp32=True)
+    assert rel_err(qd.grad, rdq) <= 3e-2 and rel_err(kd.grad, rdk) <= 3e-2 and rel_err(vd.grad, rdv) <= 3e-2
+
+
+@pytest.mark.gpu
 @pytest.mark.parametrize("D", [128, 256])
 def test_causal_and_padding_mask_becomes_causal_with_key_counts(amd, gpu_device, monkeypatch, D):
     # the additive (B,1,L,S) mask that model code builds from causality and right padding: served by the
