@@ -486,6 +486,32 @@ def test_float32_matrix_op_forward_and_backward(amd, gpu_device, shape):
     assert max_abs(out3, out) <= 1e-5
 
 
+@pytest.mark.parametrize("shape", [(3, 4, 2, 100, 160, 64, False, [160, 1, 77]), (2, 8, 8, 300, 300, 128, True, [300, 130]),
+                                   (2, 2, 2, 64, 96, 40, False, [0, 96])])
+def test_float32_matrix_op_with_key_counts(amd, gpu_device, shape):
+    """Per-batch key counts in the float32 kernels (what a right-padding mask becomes), forward and
+    backward, against the oracle on the equivalent keep-mask; a batch without keys gives zeros."""
+    from helpers import oracle_bwd, rel_err
+
+    B, Hq, Hkv, L, S, E, causal, lens = shape
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=torch.float32, seed=L + S + E, with_do=True)
+    qd, kd, vd, god = (t.to(gpu_device) for t in (q, k, v, go))
+    kl = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+    out, lse = amd.sdpa_forward(qd, kd, vd, is_causal=causal, kv_lens=kl, force_kernel=MFMA)
+    dq, dk, dv, _ = amd.sdpa_backward(god, qd, kd, vd, out, lse, is_causal=causal, kv_lens=kl, force_kernel=MFMA)
+    torch.cuda.synchronize()
+    keep = (torch.arange(S)[None] < torch.tensor(lens)[:, None])[:, None, None, :].expand(B, 1, L, S)
+    if causal:
+        keep = keep & torch.ones(L, S, dtype=torch.bool).tril()
+    ro, rl = oracle_fwd(q, k, v, attn_mask=keep)
+    rdq, rdk, rdv = oracle_bwd(go, q, k, v, ro, rl, attn_mask=keep)
+    assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert torch.isfinite(a).all() and max_abs(a, r) <= 2e-5 * max(1.0, r.abs().max().item())
+    out2, lse2 = amd.sdpa_forward(qd, kd, vd, is_causal=causal, kv_lens=kl)  # chosen by the library itself
+    assert torch.equal(out2, out) and torch.equal(lse2, lse)
+
+
 def test_float32_matrix_op_refuses_what_it_does_not_serve(amd, gpu_device):
     q, k, v = (t.to(gpu_device) for t in qkv(1, 2, 2, 64, 64, 64, dtype=torch.float32, seed=1))
     bias = torch.zeros(64, 64, device=gpu_device)

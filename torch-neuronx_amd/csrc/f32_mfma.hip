@@ -1,6 +1,6 @@
 // Flash attention for float32 inputs on the float32 matrix op (v_mfma_f32_32x32x2_f32), forward and
 // backward, head dims up to 128 (multiples of 8; narrower rows count as zero padded), causal or
-// unmasked.  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
+// unmasked, with per-batch key counts.  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
 // stays in float32 as in torch_neuronx/_sdpa_math.py (float32 inputs accumulate in float32, and the
 // probabilities that multiply V are not rounded, :94).
 //
@@ -110,19 +110,20 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   const float c = p.scale * kLog2eF;
   const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
   const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
-  int nt = (p.S + BT - 1) / BT;
+  const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
+  int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BT + 1);
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
-  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
   TileF32<D, 64 * WAVES> kn, vn;
-  if (nt > 0) kn.fetch(kp, p.k_sl, p.S, p.d_real, tid), vn.fetch(vp, p.v_sl, p.S, p.d_real, tid);
+  if (nt > 0) kn.fetch(kp, p.k_sl, S, p.d_real, tid), vn.fetch(vp, p.v_sl, S, p.d_real, tid);
   for (int t = 0; t < nt; ++t) {
     __syncthreads();  // the previous tile has been read by every wavefront
     kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
     if (t + 1 < nt) {
-      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, p.S - (t + 1) * BT, p.d_real, tid);
-      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, p.S - (t + 1) * BT, p.d_real, tid);
+      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, S - (t + 1) * BT, p.d_real, tid);
+      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, S - (t + 1) * BT, p.d_real, tid);
     }
     if (t >= nt_w) continue;
     f32x16 s = row_product<D>(k_t, col, half, qf);
@@ -210,19 +211,20 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   const float c = p.scale * kLog2eF;
   const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
   const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
-  int nt = (p.S + BT - 1) / BT;
+  const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
+  int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BT + 1);
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
-  const int lim = p.causal ? min(qrow, p.S - 1) : p.S - 1;
+  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
   TileF32<D, 64 * WAVES> kn, vn;
-  if (nt > 0) kn.fetch(kp, p.k_sl, p.S, p.d_real, tid), vn.fetch(vp, p.v_sl, p.S, p.d_real, tid);
+  if (nt > 0) kn.fetch(kp, p.k_sl, S, p.d_real, tid), vn.fetch(vp, p.v_sl, S, p.d_real, tid);
   for (int t = 0; t < nt; ++t) {
     __syncthreads();  // the previous tile has been read by every wavefront
     kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
     if (t + 1 < nt) {
-      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, p.S - (t + 1) * BT, p.d_real, tid);
-      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, p.S - (t + 1) * BT, p.d_real, tid);
+      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, S - (t + 1) * BT, p.d_real, tid);
+      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, S - (t + 1) * BT, p.d_real, tid);
     }
     if (t >= nt_w) continue;
     const f32x16 s = row_product<D>(k_t, col, half, qf);
@@ -263,6 +265,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
   const int k0 = kt * 32 * WAVES, kw0 = k0 + wave * 32, key = kw0 + col, kc = min(key, p.S - 1);
+  const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
+  // the first query row that sees this lane's key: the key itself under a causal mask, none for a key
+  // past the batch's count
+  const int first_q = key >= S ? INT_MAX : p.causal ? key : INT_MIN;
   float kf[D / 2], vf[D / 2];
   load_half_row<D>(kf, (const float*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl, half, p.d_real);
   load_half_row<D>(vf, (const float*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl, half, p.d_real);
@@ -299,7 +305,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
       if (tid < BT) lse_s[tid] = lse_n, dl_s[tid] = dl_n;
       __syncthreads();
       if (it + 1 < n_items) fetch_item(it + 1);
-      if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= p.S) continue;  // (uniform per wavefront)
+      if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= S) continue;  // (uniform per wavefront)
       const f32x16 s = row_product<D>(q_t, col, half, kf);
       const f32x16 dp = row_product<D>(do_t, col, half, vf);
       f32x16 pr, ds;
@@ -310,8 +316,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
-          float x = __builtin_amdgcn_exp2f(fmaf(s[r], c, -l4[e]));
-          x = ((p.causal && key > qi) || key >= p.S) ? 0.f : x;
+          const float x = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : fmaf(s[r], c, -l4[e]));
           pr[r] = x;
           ds[r] = x * (dp[r] - d4[e]);
         }
@@ -357,8 +362,8 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.bias.data || p.kv_lens || p.dropout_p > 0.f || p.mask.window > 0 || p.mask.sink_logit)
-    return *why = "bias, key counts, dropout or mask functors", false;
+  if (p.bias.data || p.dropout_p > 0.f || p.mask.window > 0 || p.mask.sink_logit)
+    return *why = "bias, dropout or mask functors", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
   const mi355_sdpa_tensor* ts[4] = {&p.q, &p.k, &p.v, &p.out};
@@ -382,6 +387,7 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Hkv = (int)p.k.size[1];
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
+  g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
   // rows per workgroup: 128 (a workgroup is one wavefront per 32 rows; 64- and 32-row workgroups
   // measured slower even when 128-row ones leave compute units without work)
@@ -402,8 +408,8 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.bias.data || p.grad_bias.data || p.kv_lens || p.dropout_p > 0.f || p.mask.window > 0)
-    return *why = "bias, key counts, dropout or window", false;
+  if (p.bias.data || p.grad_bias.data || p.dropout_p > 0.f || p.mask.window > 0)
+    return *why = "bias, dropout or window", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
   const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
@@ -442,6 +448,7 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.Hkv = (int)p.k.size[1];
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
+  g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
   const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
   const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
