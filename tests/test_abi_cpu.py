@@ -169,13 +169,14 @@ def test_kernel_gates(amd):
     assert gate(q, k, v, is_causal=True) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q.half(), k.half(), v.half()) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q.float(), k.float(), v.float()) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # float32 matrix op
-    assert gate(q.float(), k.float(), v.float(), attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q.float(), k.float(), v.float(), attn_bias=_meta(8192, 8192)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q, k, v, attn_bias=_meta(8192, 8192)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # masked calls too
     q64, k64 = _meta(1, 8, 512, 64), _meta(1, 8, 512, 64)
     assert gate(q64, k64, k64, attn_bias=_meta(512, 512)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q, k, v, dropout_p=0.1) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # dropout: 16-bit, head dims up to 128, no bias
     assert gate(q, k, v, dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
-    assert gate(q.float(), k.float(), v.float(), dropout_p=0.1) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q.float(), k.float(), v.float(), dropout_p=0.1) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
+    assert gate(q.float(), k.float(), v.float(), dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(q, k, v, scale=0.0) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(q, k, v, scale=0.25) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q96 = _meta(2, 8, 512, 96)  # narrow head dims (multiples of 8) run padded in the next wider kernel

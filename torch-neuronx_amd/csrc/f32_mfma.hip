@@ -1,6 +1,6 @@
 // Flash attention for float32 inputs on the float32 matrix op (v_mfma_f32_32x32x2_f32), forward and
 // backward, head dims up to 128 (multiples of 8; narrower rows count as zero padded), causal or
-// unmasked, with per-batch key counts.  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
+// unmasked, with per-batch key counts; instances with a per-score bias / keep-mask or dropout.  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
 // stays in float32 as in torch_neuronx/_sdpa_math.py (float32 inputs accumulate in float32, and the
 // probabilities that multiply V are not rounded, :94).
 //
@@ -91,7 +91,29 @@ __device__ __forceinline__ void col_product(f32x16 (&acc)[D / 32], const float* 
   }
 }
 
-template <int D, int WAVES>
+// MASKED instances: an additive bias / bool keep-mask per score (any of the bias dtypes, stride 0 on
+// broadcast dimensions) or a dropout keep-mask (bytes, (B, Hq, L, S); the bias fields describe it and
+// keep_scale is nonzero), one element load per score: a lane's 16 scores of a tile are 4 groups of 4
+// consecutive keys of its row (forward, dQ) or 16 rows of its key (dK / dV).  Not both at once.
+// bias elements as floats, the element type tested once (inside the loop every element carries the branch)
+template <typename IDX>
+__device__ __forceinline__ void load_bias16(float (&bl)[16], const void* base, int kind, IDX&& idx) {
+  if (kind == 1) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bl[r] = ((const float*)base)[idx(r)];
+  } else if (kind == 4) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bl[r] = ((const uint8_t*)base)[idx(r)] ? 0.f : -INFINITY;
+  } else if (kind == 3) {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bl[r] = __builtin_bit_cast(float, (uint32_t)((const uint16_t*)base)[idx(r)] << 16);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 16; ++r) bl[r] = (float)((const _Float16*)base)[idx(r)];
+  }
+}
+
+template <int D, int WAVES, bool MASKED>
 __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
@@ -108,6 +130,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   for (int i = 0; i < DB; ++i) zero(oacc[i]);
   float m_run = -INFINITY, l_run = 0.f;  // (l_run: this lane half's keys only; the halves share m_run)
   const float c = p.scale * kLog2eF;
+  const float inv_scale = 1.f / p.scale;
   const float* kp = (const float*)p.k + b * p.k_sb + hk * p.k_sh;
   const float* vp = (const float*)p.v + b * p.v_sb + hk * p.v_sh;
   const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
@@ -127,6 +150,22 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
     }
     if (t >= nt_w) continue;
     f32x16 s = row_product<D>(k_t, col, half, qf);
+    float keepf[MASKED ? 16 : 1];
+    if constexpr (MASKED) {
+      // this lane's row of the bias / keep-mask plane of the (batch, head), keys clamped into the row
+      const int64_t row0 = b * p.bias_sb + h * p.bias_sh + (int64_t)qc * p.bias_sl;
+      auto idx = [&](int r) { return row0 + min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
+      if (p.keep_scale != 0.f) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) keepf[r] = (float)((const uint8_t*)p.bias)[idx(r)];
+      } else {
+        float bl[16];
+        load_bias16(bl, p.bias, p.bias_kind, idx);
+        // folded into the raw scores, s += bias / scale: everything downstream is the unbiased code
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] = fmaf(bl[r], inv_scale, s[r]);
+      }
+    }
     float tm = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
@@ -150,10 +189,19 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
     for (int i = 0; i < DB; ++i)
 #pragma unroll
       for (int r = 0; r < 16; ++r) oacc[i][r] *= alpha;
+    if constexpr (MASKED) {  // dropout: the row sum above keeps the dropped probabilities (torch_neuronx/_sdpa_math.py:36-48)
+      if (p.keep_scale != 0.f) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) s[r] *= keepf[r];
+      }
+    }
     col_product<D>(oacc, v_t, col, half, s);
   }
   const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
-  const float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if constexpr (MASKED) {
+    if (p.keep_scale != 0.f) inv *= p.keep_scale;
+  }
   if (qrow < p.L) {
     float* orow = (float*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
@@ -169,7 +217,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   }
 }
 
-template <int D, int WAVES>
+template <int D, int WAVES, bool MASKED>
 __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
@@ -230,12 +278,30 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
     const f32x16 s = row_product<D>(k_t, col, half, qf);
     const f32x16 dp = row_product<D>(v_t, col, half, dof);
     f32x16 ds;
+    float bl[MASKED ? 16 : 1];  // the bias in the log2 domain, or (dropout) keep / (1 - p)
+    bool drop = false;
+    if constexpr (MASKED) {
+      const int64_t row0 = b * p.bias_sb + h * p.bias_sh + (int64_t)qc * p.bias_sl;
+      auto idx = [&](int r) { return row0 + min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
+      drop = p.keep_scale != 0.f;
+      if (drop) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bl[r] = (float)((const uint8_t*)p.bias)[idx(r)] * p.keep_scale;
+      } else {
+        load_bias16(bl, p.bias, p.bias_kind, idx);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bl[r] *= kLog2eF;
+      }
+    }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kv = t * BT + (r >> 2) * 8 + half * 4 + (r & 3);
-      float pr = __builtin_amdgcn_exp2f(fmaf(s[r], c, -lse2));
-      pr = kv > lim ? 0.f : pr;
-      ds[r] = pr * (dp[r] - dl);
+      float x = fmaf(s[r], c, -lse2);
+      if constexpr (MASKED) x = drop ? x : fmaf(s[r], c, bl[r]) - lse2;
+      const float pr = __builtin_amdgcn_exp2f(kv > lim ? -INFINITY : x);
+      float g = dp[r];
+      if constexpr (MASKED) g = drop ? g * bl[r] : g;
+      ds[r] = pr * (g - dl);
     }
     col_product<D>(dqacc, k_t, col, half, ds);
   }
@@ -253,7 +319,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   }
 }
 
-template <int D, int WAVES>
+template <int D, int WAVES, bool MASKED>
 __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float q_t[BT * (D + 4)];
@@ -309,6 +375,22 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
       const f32x16 s = row_product<D>(q_t, col, half, kf);
       const f32x16 dp = row_product<D>(do_t, col, half, vf);
       f32x16 pr, ds;
+      float bl[MASKED ? 16 : 1];  // the bias in the log2 domain, or (dropout) keep / (1 - p)
+      bool drop = false;
+      if constexpr (MASKED) {
+        const int hq = hk * rep + it % rep;
+        const int64_t col0 = b * p.bias_sb + hq * p.bias_sh + min(key, p.S - 1);
+        auto idx = [&](int r) { return col0 + (int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.bias_sl; };
+        drop = p.keep_scale != 0.f;
+        if (drop) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) bl[r] = (float)((const uint8_t*)p.bias)[idx(r)] * p.keep_scale;
+        } else {
+          load_bias16(bl, p.bias, p.bias_kind, idx);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) bl[r] *= kLog2eF;
+        }
+      }
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
@@ -316,9 +398,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
-          const float x = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : fmaf(s[r], c, -l4[e]));
+          float a = fmaf(s[r], c, -l4[e]);
+          if constexpr (MASKED) a = drop ? a : fmaf(s[r], c, bl[r]) - l4[e];
+          const float x = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : a);
+          float g = dp[r];
           pr[r] = x;
-          ds[r] = x * (dp[r] - d4[e]);
+          if constexpr (MASKED) {
+            if (drop) g *= bl[r], pr[r] = x * bl[r];  // dV from the kept probabilities, scaled; dP masked and scaled
+          }
+          ds[r] = x * (g - d4[e]);
         }
       }
       col_product<D>(dvacc, do_t, col, half, pr);
@@ -345,6 +433,22 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
 // wavefronts (32 rows each) per workgroup
 int pick_waves(int64_t, int) { return 4; }
 
+// the bias / keep-mask fields of a call: an attn_bias as it is (strides in elements), or the dropout
+// keep-mask, (B, Hq, L, S) contiguous bytes with keep_scale = 1 / (1 - p) (1 for p = 1)
+template <typename G, typename P>
+void set_score_mask(G& g, const P& p) {
+  if (p.bias.data) {
+    g.bias = p.bias.data;
+    g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1], g.bias_sl = p.q.size[2] > 1 ? p.bias.stride[2] : 0;
+    g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
+  } else if (p.dropout_p > 0.f) {
+    g.bias = p.dropout_keep;
+    g.bias_sl = p.k.size[2], g.bias_sh = p.q.size[2] * g.bias_sl, g.bias_sb = p.q.size[1] * g.bias_sh;
+    g.bias_kind = 4;
+    g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
+  }
+}
+
 bool tensors_fit(const mi355_sdpa_tensor* const* ts, int n) {
   for (int k = 0; k < n; ++k) {
     const mi355_sdpa_tensor* t = ts[k];
@@ -362,8 +466,12 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.bias.data || p.dropout_p > 0.f || p.mask.window > 0 || p.mask.sink_logit)
-    return *why = "bias, dropout or mask functors", false;
+  if (p.mask.window > 0 || p.mask.sink_logit) return *why = "mask functors", false;
+  if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
+  if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
+  if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
+      p.bias_dtype != MI355_SDPA_BOOL)
+    return *why = "attn_bias dtype", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
   const mi355_sdpa_tensor* ts[4] = {&p.q, &p.k, &p.v, &p.out};
@@ -389,13 +497,19 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
+  set_score_mask(g, p);
+  const bool masked = g.bias != nullptr;
   // rows per workgroup: 128 (a workgroup is one wavefront per 32 rows; 64- and 32-row workgroups
   // measured slower even when 128-row ones leave compute units without work)
   const int waves = pick_waves((int64_t)g.B * g.Hq, g.L);
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(64 * waves);
-#define LAUNCH(DD, WW) hipLaunchKernelGGL((fwd_f32_kernel<DD, WW>), grid, block, 0, s, g)
-#define LAUNCH_W(DD) LAUNCH(DD, 4)
+#define LAUNCH(DD, WW, MM) hipLaunchKernelGGL((fwd_f32_kernel<DD, WW, MM>), grid, block, 0, s, g)
+#define LAUNCH_W(DD)                \
+  do {                              \
+    if (masked) LAUNCH(DD, 4, true); \
+    else LAUNCH(DD, 4, false);      \
+  } while (0)
   if (g.d_real <= 64) LAUNCH_W(64);
   else LAUNCH_W(128);
 #undef LAUNCH_W
@@ -408,8 +522,12 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.bias.data || p.grad_bias.data || p.dropout_p > 0.f || p.mask.window > 0)
-    return *why = "bias, dropout or window", false;
+  if (p.grad_bias.data || p.mask.window > 0) return *why = "bias gradient or window", false;
+  if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
+  if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
+  if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
+      p.bias_dtype != MI355_SDPA_BOOL)
+    return *why = "attn_bias dtype", false;
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
   const mi355_sdpa_tensor* ts[8] = {&p.grad_out, &p.q, &p.k, &p.v, &p.out, &p.grad_q, &p.grad_k, &p.grad_v};
@@ -450,11 +568,17 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
+  set_score_mask(g, p);
+  const bool masked = g.bias != nullptr;
   const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
   const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
   const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw))));
-#define LAUNCH(KK, GRID, DD, WW) hipLaunchKernelGGL((KK<DD, WW>), GRID, dim3(64 * WW), 0, s, g)
-#define LAUNCH_W(KK, GRID, WAVES_, DD) LAUNCH(KK, GRID, DD, 4)
+#define LAUNCH(KK, GRID, DD, WW, MM) hipLaunchKernelGGL((KK<DD, WW, MM>), GRID, dim3(64 * WW), 0, s, g)
+#define LAUNCH_W(KK, GRID, WAVES_, DD)          \
+  do {                                          \
+    if (masked) LAUNCH(KK, GRID, DD, 4, true);  \
+    else LAUNCH(KK, GRID, DD, 4, false);        \
+  } while (0)
   if (g.d_real <= 64) LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 64);
   else LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 128);
   int rc = check_launch("bwd_f32_dq_kernel");
