@@ -444,6 +444,37 @@ def test_mfma_forward_value_rows_narrower_than_keys(amd, gpu_device, E, Dv, caus
     assert max_abs(lse, rl) <= 3e-3
 
 
+# ---- short query sequences under grouped-query attention: the heads of a kv group share a workgroup ----
+GROUPED = [
+    # B, Hq, Hkv, L, S, D, causal, kv_lens
+    (3, 8, 2, 1, 700, 128, False, None),     # a decode step, 4 heads per group
+    (2, 32, 8, 1, 4096, 128, False, [4096, 1000]),
+    (2, 8, 1, 5, 300, 64, False, None),      # 8 heads per group
+    (2, 4, 2, 40, 40, 128, True, None),      # two 32-row blocks per head, causal
+    (1, 16, 4, 32, 513, 64, True, [400]),
+    (2, 8, 4, 64, 200, 256, False, None),    # head dim 256: four wavefronts, two heads x two blocks
+    (1, 6, 2, 17, 90, 96, False, None),      # three heads per group: not grouped, same answers
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", GROUPED, ids=lambda c: "B%d_Hq%d_Hkv%d_L%d_S%d_D%d_c%d" % c[:7])
+def test_short_queries_with_grouped_heads(amd, gpu_device, case, dtype):
+    B, Hq, Hkv, L, S, D, causal, lens = case
+    q, k, v = qkv(B, Hq, Hkv, L, S, D, dtype=dtype, seed=L + S + D)
+    kw, mask = {}, None
+    if lens is not None:
+        kw["kv_lens"] = torch.tensor(lens, dtype=torch.int32, device=gpu_device)
+        mask = (torch.arange(S)[None] < torch.tensor(lens)[:, None])[:, None, None, :].expand(B, 1, L, S)
+    if causal:
+        cm = torch.ones(L, S, dtype=torch.bool).tril()
+        mask = cm[None, None].expand(B, 1, L, S) if mask is None else mask & cm
+    out, lse = amd.sdpa_forward(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), is_causal=causal, force_kernel=MFMA, **kw)
+    ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
+    assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3)
+    assert max_abs(lse, rl) <= 2e-3
+
+
 # ---- float32 inputs on the float32 matrix op --------------------------------------------------------
 # (the reference's fused gate takes float32, decompositions.py:2131-2158; shapes of its accuracy
 # matrix, tests/python_ops/test_scaled_dot_product_attention.py:220-302 and :362-387)

@@ -77,14 +77,21 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // ... and, with a tile skip table, the list of the key tiles this workgroup walks (1024 entries and the count)
   uint16_t* const tile_list = bias_lds + WAVES * 2048;
 
-  int b, h, qt;
-  decode_block(p, b, h, qt);
-  const int hk = h / (p.Hq / p.Hkv);
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps per-wavefront tests on the scalar unit
+  int b, h, qt;
+  int wrow = wave * 32;  // this wavefront's first row within the workgroup's rows
+  if (MASK < 2 && p.grouped) {  // (see FwdM::grouped)
+    const int rep = p.Hq / p.Hkv;
+    b = blockIdx.x / p.Hkv, h = (blockIdx.x % p.Hkv) * rep + wave % rep, qt = 0;
+    wrow = (wave / rep) * 32;
+  } else {
+    decode_block(p, b, h, qt);
+  }
+  const int hk = h / (p.Hq / p.Hkv);
   const int col = lane & 31, half = lane >> 5;
   const int q0 = qt * BM;
-  const int qw0 = q0 + wave * 32;
+  const int qw0 = q0 + wrow;
   const int qrow = qw0 + col;
   const int qw_last = qw0 + 31;
 
@@ -762,8 +769,17 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
   if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
   if (g.dv_real <= 0 || g.dv_real > head_dim) g.dv_real = g.d_real;
   if (head_dim == 256) waves = 4;
-  g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
-  const int64_t blocks = (int64_t)g.B * g.Hq * g.n_qt;
+  // Grouped mode: every head of a kv group in one workgroup when their rows fit its wavefronts (four
+  // wavefronts where they do, eight otherwise) and there is no per-score bias / dropout mask.
+  const int rep = g.Hq / g.Hkv;
+  g.grouped = 0;
+  if (rep > 1 && g.bias_kind == 0 && g.keep_scale == 0.f && !g.live_tiles) {
+    const int blocks32 = (g.L + 31) / 32;  // 32-row blocks per head
+    if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = 1;
+    else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = 1;
+  }
+  g.n_qt = g.grouped ? 1 : (g.L + 32 * waves - 1) / (32 * waves);
+  const int64_t blocks = g.grouped ? (int64_t)g.B * g.Hkv : (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
   if (blocks > 0x7fffffff) {
     set_error("SDPA: too many query tiles (%lld)", (long long)blocks);
