@@ -447,7 +447,7 @@ def test_mfma_forward_value_rows_narrower_than_keys(amd, gpu_device, E, Dv, caus
 # ---- short query sequences under grouped-query attention: the heads of a kv group share a workgroup ----
 GROUPED = [
     # B, Hq, Hkv, L, S, D, causal, kv_lens
-    (3, 8, 2, 1, 700, 128, False, None),     # a decode step, 4 heads per group
+    (3, 8, 2, 1, 704, 128, False, None),     # a decode step, 4 heads per group
     (2, 32, 8, 1, 4096, 128, False, [4096, 1000]),
     (2, 8, 1, 5, 300, 64, False, None),      # 8 heads per group
     (2, 4, 2, 40, 40, 128, True, None),      # two 32-row blocks per head, causal
@@ -473,6 +473,18 @@ def test_short_queries_with_grouped_heads(amd, gpu_device, case, dtype):
     ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
     assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3)
     assert max_abs(lse, rl) <= 2e-3
+    if not causal and lens is None and S % 4 == 0:
+        # a mask that does not depend on the head keeps the heads together: left padding per key
+        # (bool, what a batch of left-padded prompts sends with every decode step), and a per-score bias
+        start = torch.randint(0, S // 2, (B,), generator=torch.Generator().manual_seed(S))
+        lp = (torch.arange(S)[None] >= start[:, None])[:, None, None, :]
+        out, lse = amd.sdpa_forward(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), attn_bias=lp.to(gpu_device), force_kernel=MFMA)
+        ro, rl = oracle_fwd(q, k, v, attn_mask=lp.expand(B, 1, L, S))
+        assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3) and max_abs(lse, rl) <= 2e-3
+        bias = torch.randn(B, 1, L, S, generator=torch.Generator().manual_seed(S + 1)).to(dtype)
+        out, lse = amd.sdpa_forward(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), attn_bias=bias.to(gpu_device), force_kernel=MFMA)
+        ro, rl = oracle_fwd(q, k, v, attn_mask=bias.float())
+        assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3) and max_abs(lse, rl) <= 3e-3
 
 
 # ---- float32 inputs on the float32 matrix op --------------------------------------------------------

@@ -26,7 +26,8 @@ struct FwdM {
   // dropout (fwd_mfma_w32.hip, head dims up to 128, no bias): nonzero = 1 / (1 - p) (1 for p = 1), and the
   // bias fields above describe the (B, Hq, L, S) keep-mask, kind 4
   float keep_scale = 0.f;
-  // Short query sequences under grouped-query attention (fwd_mfma_w32.hip, no per-score bias): one
+  // Short query sequences under grouped-query attention (fwd_mfma_w32.hip; no dropout, no bias that
+  // depends on the head): one
   // workgroup per (batch, kv head) serves every query head of the group, wavefront w the rows
   // 32 * (w / rep) .. +31 of head hk * rep + w % rep, so that a K / V tile is fetched once for all
   // of them (decode-like calls are bound by exactly that traffic).  0 = off.

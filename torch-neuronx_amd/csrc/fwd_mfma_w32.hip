@@ -81,7 +81,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps per-wavefront tests on the scalar unit
   int b, h, qt;
   int wrow = wave * 32;  // this wavefront's first row within the workgroup's rows
-  if (MASK < 2 && p.grouped) {  // (see FwdM::grouped)
+  if (MASK <= 2 && p.grouped) {  // (see FwdM::grouped)
     const int rep = p.Hq / p.Hkv;
     b = blockIdx.x / p.Hkv, h = (blockIdx.x % p.Hkv) * rep + wave % rep, qt = 0;
     wrow = (wave / rep) * 32;
@@ -773,7 +773,9 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
   // wavefronts where they do, eight otherwise) and there is no per-score bias / dropout mask.
   const int rep = g.Hq / g.Hkv;
   g.grouped = 0;
-  if (rep > 1 && g.bias_kind == 0 && g.keep_scale == 0.f && !g.live_tiles) {
+  // (a bias that does not depend on the head is fine: every wavefront of the workgroup then arrives at
+  // the same key count when it trims a keep-mask per key, and so at the same number of tiles)
+  if (rep > 1 && (g.bias_kind == 0 || g.bias_sh == 0) && g.keep_scale == 0.f && !g.live_tiles) {
     const int blocks32 = (g.L + 31) / 32;  // 32-row blocks per head
     if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = 1;
     else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = 1;
