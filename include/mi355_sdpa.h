@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MI355_SDPA_ABI_VERSION 3
+#define MI355_SDPA_ABI_VERSION 4
 
 /* element types */
 enum mi355_sdpa_dtype {
@@ -127,6 +127,11 @@ typedef struct mi355_sdpa_fwd_params {
   float scale;            /* multiplies Q K^T in float32                              */
   int32_t force_kernel;   /* 0 = library picks; else enum mi355_sdpa_kernel           */
   mi355_sdpa_mask_spec mask; /* all zero = none                                       */
+  void* workspace;        /* optional: mi355_sdpa_fwd_workspace_bytes() bytes, 256-aligned.  With it,
+                             a call with few query rows and few (batch, kv head) pairs splits its
+                             keys over more workgroups (partial results here, merged by a second
+                             kernel); without it the same call runs unsplit                    */
+  size_t workspace_bytes;
 } mi355_sdpa_fwd_params;
 
 typedef struct mi355_sdpa_bwd_params {
@@ -177,6 +182,9 @@ typedef struct mi355_sdpa_decode_params {
  * and, for inputs the flash kernel refuses, for the math path
  *   torch_neuronx/_sdpa_math.py:51-95 (compute_attention). */
 int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream);
+/* Bytes of workspace with which this forward call would split its keys (0: it would not).  No
+ * counterpart in the reference; the workspace is optional. */
+size_t mi355_sdpa_fwd_workspace_bytes(const mi355_sdpa_fwd_params* p);
 
 /* Fused backward: dQ, dK, dV (dK/dV already reduced over each GQA group), optional dBias.
  * Stands in for decompositions.py:2467-2477 (_compute_attention_backward_nki),

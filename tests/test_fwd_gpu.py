@@ -454,6 +454,12 @@ GROUPED = [
     (1, 16, 4, 32, 513, 64, True, [400]),
     (2, 8, 4, 64, 200, 256, False, None),    # head dim 256: four wavefronts, two heads x two blocks
     (1, 6, 2, 17, 90, 96, False, None),      # three heads per group: not grouped, same answers
+    # few (batch, kv head) pairs and many keys: the keys are split over workgroups and merged
+    (1, 32, 8, 1, 8192, 128, False, [5000]),
+    (2, 8, 2, 3, 4096, 64, False, [4096, 100]),
+    (1, 16, 4, 8, 3000, 96, False, None),
+    (2, 8, 2, 1, 2048, 128, False, [0, 2048]),  # a batch without keys: zeros and lse = -inf
+    (1, 8, 4, 33, 2500, 128, False, None),
 ]
 
 
@@ -472,7 +478,7 @@ def test_short_queries_with_grouped_heads(amd, gpu_device, case, dtype):
     out, lse = amd.sdpa_forward(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), is_causal=causal, force_kernel=MFMA, **kw)
     ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
     assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3)
-    assert max_abs(lse, rl) <= 2e-3
+    assert max_abs(lse, rl) <= 2e-3 and torch.equal(torch.isfinite(lse.cpu()), torch.isfinite(rl))
     if not causal and lens is None and S % 4 == 0:
         # a mask that does not depend on the head keeps the heads together: left padding per key
         # (bool, what a batch of left-padded prompts sends with every decode step), and a per-score bias
@@ -631,3 +637,38 @@ def test_float32_matrix_op_refuses_what_it_does_not_serve(amd, gpu_device):
     out, _ = amd.sdpa_forward(q, k, v, attn_bias=bias, dropout_p=0.5, dropout_keep=keep)  # served by the generic kernel
     ro, _ = oracle_fwd(q.cpu(), k.cpu(), v.cpu())
     assert max_abs(out, 2.0 * ro) <= 2e-5
+
+
+def test_split_keys_need_the_workspace_and_agree_with_the_unsplit_call(amd, gpu_device):
+    """Through the C ABI: the size query says that a decode-like call would split its keys; with the
+    workspace it does (and merges), without it the same call runs unsplit; both agree with the oracle,
+    and with each other to float32 rounding."""
+    import ctypes as C
+
+    from torch_neuronx_amd import _lib
+
+    B, Hq, Hkv, S, D = 1, 32, 8, 8192, 128
+    q, k, v = (t.to(gpu_device) for t in qkv(B, Hq, Hkv, 1, S, D, dtype=torch.bfloat16, seed=77))
+
+    def call(with_ws):
+        out = torch.empty_like(q)
+        lse = torch.empty(B, Hq, 1, dtype=torch.float32, device=gpu_device)
+        p = _lib.FwdParams()
+        p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (q, k, v, out))
+        p.lse, p.dtype, p.scale, p.force_kernel = lse.data_ptr(), _lib.dtype_id(q.dtype), D**-0.5, MFMA
+        need = _lib.load().mi355_sdpa_fwd_workspace_bytes(C.byref(p))
+        assert need == B * Hq * 32 * 1 * (D + 1) * 4  # 256 tiles in 32 parts of 8
+        ws = torch.empty(need, dtype=torch.uint8, device=gpu_device)
+        if with_ws:
+            p.workspace, p.workspace_bytes = ws.data_ptr(), need
+        with _lib.on_device(q.device):
+            _lib.check(_lib.load().mi355_sdpa_fwd(C.byref(p), _lib.current_stream(q.device)))
+        torch.cuda.synchronize()
+        return out, lse
+
+    o1, l1 = call(True)
+    o0, l0 = call(False)
+    ro, rl = oracle_fwd(q.cpu(), k.cpu(), v.cpu())
+    for o, l in ((o1, l1), (o0, l0)):
+        assert max_abs(o, ro) <= 2e-2 and max_abs(l, rl) <= 2e-3
+    assert max_abs(o1, o0) <= 4e-3 and max_abs(l1, l0) <= 1e-5

@@ -14,6 +14,7 @@ int check_launch(const char* what);
 
 int launch_fwd_generic(const mi355_sdpa_fwd_params& p, hipStream_t s);
 int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s);
+size_t fwd_mfma_workspace(const mi355_sdpa_fwd_params& p);  // with which the call would split its keys (0: it would not)
 bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why);
 int launch_bwd_generic(const mi355_sdpa_bwd_params& p, hipStream_t s);
 int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s);

@@ -32,6 +32,15 @@ struct FwdM {
   // 32 * (w / rep) .. +31 of head hk * rep + w % rep, so that a K / V tile is fetched once for all
   // of them (decode-like calls are bound by exactly that traffic).  0 = off.
   int grouped = 0;
+  // ... and, when that leaves most compute units without a workgroup, the keys are split: n_split
+  // workgroups per (batch, kv head), each over split_tiles 32-key tiles, leave their normalised output
+  // (float32, (B, Hq, n_split, L, dv_real)) and log-sum-exp ((B, Hq, n_split, L)) in the workspace,
+  // and fwd_split_merge_kernel combines them.  Grouped calls without a window, a sink logit or the
+  // causal flag, head dims up to 128.  0 = off.
+  int split_tiles = 0, n_split = 1;
+  float* part_o = nullptr;   // the workspace (part_bytes bytes of it)
+  float* part_lse = nullptr;
+  size_t part_bytes = 0;
   const int32_t* kv_lens = nullptr;
   // Elements per row that exist (a multiple of 8).  Below the head dim a kernel is built for, the
   // masked variant treats the rest of every Q / K / V row as zeros and leaves it out of the output
@@ -83,5 +92,7 @@ __device__ __forceinline__ void decode_block(const FwdM& p, int& b, int& h, int&
 // head_dim 64, 128 or 256: the width the kernel is built for (g.d_real: the width of the data);
 // waves = 4 or 8 wavefronts (128 or 256 query rows) per workgroup, 4 only at head dim 256
 int launch_fwd_mfma_w32(const FwdM& g, int dtype, int head_dim, int waves, hipStream_t s);
+// bytes of workspace with which that launch would split the keys of the call (0: it would not)
+size_t fwd_w32_workspace(const FwdM& g, int head_dim, int waves);
 
 }  // namespace mi355

@@ -380,9 +380,12 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   return true;
 }
 
-int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
+// launches the call, or (ws_only) reports the workspace with which it would split its keys
+static int launch_or_size(const mi355_sdpa_fwd_params& p, hipStream_t s, size_t* ws_only) {
   const char* why;
+  if (ws_only) *ws_only = 0;
   if (!fwd_mfma_supported(p, &why)) {
+    if (ws_only) return MI355_SDPA_OK;
     set_error("SDPA: MFMA forward kernel cannot take this call: %s", why);
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
@@ -414,6 +417,7 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     g.live_tiles = p.mask.live_tiles;
     g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
   }
+  if (p.workspace && ((uintptr_t)p.workspace & 255) == 0) g.part_o = (float*)p.workspace, g.part_bytes = p.workspace_bytes;
   const int D = g.d_real <= 64 ? 64 : g.d_real <= 128 ? 128 : 256;  // the kernel's width
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
   const int force_tile = p.force_kernel == MI355_SDPA_KERNEL_MFMA_T256 ? 256
@@ -431,8 +435,10 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     // wavefronts per SIMD)
     const bool listed = g.live_tiles && D == 128;
     const int rows = D == 256 ? 128 : listed ? 256 : force_tile ? force_tile : (big && !short_window) ? 256 : 128;
+    if (ws_only) return *ws_only = fwd_w32_workspace(g, D, rows / 32), MI355_SDPA_OK;
     return launch_fwd_mfma_w32(g, p.dtype, D, rows / 32, s);
   }
+  if (ws_only) return MI355_SDPA_OK;
   // strides beyond 32-bit offsets: the kernel above (64-bit addressing)
   int NB = (D == 64 && (force_tile == 256 || (force_tile == 0 && wg256 >= 256 && g.S >= 2048))) ? 2 : 1;
   const int BM = 128 * NB;
@@ -454,6 +460,14 @@ int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     else hipLaunchKernelGGL((fwd_mfma_kernel<f16_t, 64, 1>), grid, block, 0, s, g);
   }
   return check_launch("fwd_mfma_kernel");
+}
+
+int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) { return launch_or_size(p, s, nullptr); }
+
+size_t fwd_mfma_workspace(const mi355_sdpa_fwd_params& p) {
+  size_t bytes = 0;
+  launch_or_size(p, nullptr, &bytes);
+  return bytes;
 }
 
 }  // namespace mi355

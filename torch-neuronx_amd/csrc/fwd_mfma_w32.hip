@@ -81,9 +81,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps per-wavefront tests on the scalar unit
   int b, h, qt;
   int wrow = wave * 32;  // this wavefront's first row within the workgroup's rows
+  int split = 0;  // (grouped calls with split keys: which part of them)
   if (MASK <= 2 && p.grouped) {  // (see FwdM::grouped)
     const int rep = p.Hq / p.Hkv;
-    b = blockIdx.x / p.Hkv, h = (blockIdx.x % p.Hkv) * rep + wave % rep, qt = 0;
+    const int bhk = blockIdx.x / p.n_split;
+    split = blockIdx.x % p.n_split;
+    b = bhk / p.Hkv, h = (bhk % p.Hkv) * rep + wave % rep, qt = 0;
     wrow = (wave / rep) * 32;
   } else {
     decode_block(p, b, h, qt);
@@ -131,6 +134,10 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
     }
+    if (p.split_tiles) {  // this workgroup's share of the key tiles (no window then)
+      skip = split * p.split_tiles;
+      nt = max(min(nt - skip, p.split_tiles), 0);
+    }
   }
   // With a tile skip table (variant with a bias): the tiles in which the mask keeps at least one score
   // of this workgroup's rows, in ascending order.  The first wavefront ORs the bitmaps of the
@@ -170,6 +177,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   };
   if constexpr (MASK) {
     if (nt <= 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87), or the sink logit alone
+      if constexpr (FUNC) {
+        if (p.split_tiles) {  // (split keys: a part without keys carries no weight in the merge)
+          if (qrow < p.L && half == 0) p.part_lse[(((int64_t)b * p.Hq + h) * p.n_split + split) * p.L + qrow] = -INFINITY;
+          return;
+        }
+      }
       if (qrow < p.L) {
         uint16_t* orow = (uint16_t*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
@@ -698,6 +711,24 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       }
     }
   }
+  if constexpr (FUNC) {
+    if (p.split_tiles) {  // split keys: this part's normalised rows and their log-sum-exp, in float32, for the merge
+      if (qrow < p.L) {
+        const int64_t prow = (((int64_t)b * p.Hq + h) * p.n_split + split) * p.L + qrow;
+        float* po = p.part_o + prow * drv;
+#pragma unroll
+        for (int db = 0; db < DB; ++db)
+#pragma unroll
+          for (int g = 0; g < 4; ++g) {
+            const int d = db * 32 + g * 8 + half * 4;
+            if (d < drv)
+              *(f32x4*)(po + d) = f32x4{oacc[db][g * 4] * inv, oacc[db][g * 4 + 1] * inv, oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv};
+          }
+        if (half == 0) p.part_lse[prow] = lse_row;
+      }
+      return;
+    }
+  }
   // A lane holds its query row in 8-byte pieces, 16 bytes apart: stored as they are, one
   // instruction writes 32 fragments of 16 bytes, and the stores of a workgroup's last tile,
   // which nothing overlaps, took 3 % of the kernel.  The tile goes through LDS instead (the
@@ -725,6 +756,33 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     if (qw0 + r < p.L && (!MASK || cc * 8 < drv)) *(u32x4*)(obase + (int64_t)(qw0 + r) * p.o_sl) = w;
   }
   if (qrow < p.L && p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
+}
+
+// Merge of the parts of a call whose keys were split: out = sum_s w_s O_s with w_s = exp(lse_s - lse),
+// lse = log sum_s exp(lse_s).  One workgroup per query row, one thread per output element.
+template <typename T>
+__global__ __launch_bounds__(128) void fwd_split_merge_kernel(FwdM p) {
+  const int64_t row = blockIdx.x;  // (b * Hq + h) * L + l
+  const int l = (int)(row % p.L);
+  const int64_t bh = row / p.L;
+  const int b = (int)(bh / p.Hq), h = (int)(bh % p.Hq);
+  const float* pl = p.part_lse + bh * p.n_split * p.L + l;
+  float m = -INFINITY;
+  for (int s = 0; s < p.n_split; ++s) m = fmaxf(m, pl[(int64_t)s * p.L]);
+  float sum = 0.f, acc = 0.f;
+  const int d = threadIdx.x;
+  for (int s = 0; s < p.n_split; ++s) {
+    const float ls = pl[(int64_t)s * p.L];
+    if (ls == -INFINITY) continue;  // (a part without keys: its rows were never written)
+    const float w = __expf(ls - m);
+    sum += w;
+    if (d < p.dv_real) acc = fmaf(w, p.part_o[((bh * p.n_split + s) * p.L + l) * p.dv_real + d], acc);
+  }
+  if (d < p.dv_real) {
+    T* o = (T*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)l * p.o_sl + d;
+    *(uint16_t*)o = (uint16_t)Mma<T>::pack(sum > 0.f ? acc / sum : 0.f, 0.f);
+  }
+  if (d == 0 && p.lse) p.lse[row] = sum > 0.f ? m + __builtin_logf(sum) : -INFINITY;
 }
 
 // one instantiation; head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare
@@ -764,24 +822,51 @@ int launch_dims(const FwdM& g, int head_dim, int waves, int mask, dim3 grid, hip
 
 }  // namespace
 
-int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipStream_t s) {
-  FwdM g = g0;
+// Grouped mode: every head of a kv group in one workgroup when their rows fit its wavefronts (four
+// wavefronts where they do, eight otherwise) and there is no dropout mask and no bias that depends
+// on the head (with one that does not, every wavefront of the workgroup arrives at the same key count
+// when it trims a keep-mask per key, and so at the same number of tiles).  When that leaves most of
+// the 256 compute units without a workgroup and the key loop is long, the keys are split: at least 8
+// tiles per part, about two workgroups per compute unit.
+void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
   if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
   if (g.dv_real <= 0 || g.dv_real > head_dim) g.dv_real = g.d_real;
   if (head_dim == 256) waves = 4;
-  // Grouped mode: every head of a kv group in one workgroup when their rows fit its wavefronts (four
-  // wavefronts where they do, eight otherwise) and there is no per-score bias / dropout mask.
   const int rep = g.Hq / g.Hkv;
-  g.grouped = 0;
-  // (a bias that does not depend on the head is fine: every wavefront of the workgroup then arrives at
-  // the same key count when it trims a keep-mask per key, and so at the same number of tiles)
+  g.grouped = 0, g.split_tiles = 0, g.n_split = 1;
   if (rep > 1 && (g.bias_kind == 0 || g.bias_sh == 0) && g.keep_scale == 0.f && !g.live_tiles) {
     const int blocks32 = (g.L + 31) / 32;  // 32-row blocks per head
     if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = 1;
     else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = 1;
   }
+  if (g.grouped && head_dim <= 128 && g.bias_kind == 0 && !g.causal && g.window == 0 && !g.sink_logit) {
+    const int64_t groups = (int64_t)g.B * g.Hkv;
+    const int nt = (g.S + BN - 1) / BN;
+    const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);
+    if (groups < 256 && want >= 2) {
+      g.split_tiles = (nt + want - 1) / want;
+      g.n_split = (nt + g.split_tiles - 1) / g.split_tiles;
+    }
+  }
   g.n_qt = g.grouped ? 1 : (g.L + 32 * waves - 1) / (32 * waves);
-  const int64_t blocks = g.grouped ? (int64_t)g.B * g.Hkv : (int64_t)g.B * g.Hq * g.n_qt;
+}
+
+size_t fwd_w32_workspace(const FwdM& g0, int head_dim, int waves) {
+  FwdM g = g0;
+  fwd_w32_plan(g, head_dim, waves);
+  if (!g.split_tiles) return 0;
+  return (size_t)g.B * g.Hq * g.n_split * g.L * (g.dv_real + 1) * sizeof(float);
+}
+
+int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipStream_t s) {
+  FwdM g = g0;
+  fwd_w32_plan(g, head_dim, waves);
+  if (g.split_tiles) {  // (the caller's workspace: too small or absent, and the call runs unsplit)
+    const size_t rows = (size_t)g.B * g.Hq * g.n_split * g.L;
+    if (g.part_o && g.part_bytes >= rows * (g.dv_real + 1) * sizeof(float)) g.part_lse = g.part_o + rows * g.dv_real;
+    else g.split_tiles = 0, g.n_split = 1;
+  }
+  const int64_t blocks = g.grouped ? (int64_t)g.B * g.Hkv * g.n_split : (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
   if (blocks > 0x7fffffff) {
     set_error("SDPA: too many query tiles (%lld)", (long long)blocks);
@@ -793,11 +878,16 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128 and the keep-mask in the bias slot");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  const int mask = g.keep_scale != 0.f ? 3 : g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit) ? 1 : 0;
-  const int rc = dtype == MI355_SDPA_BF16 ? launch_dims<bf16_t>(g, head_dim, waves, mask, grid, s)
+  const int mask = g.keep_scale != 0.f ? 3 : g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit || g.split_tiles) ? 1 : 0;
+  int rc = dtype == MI355_SDPA_BF16 ? launch_dims<bf16_t>(g, head_dim, waves, mask, grid, s)
                                           : launch_dims<f16_t>(g, head_dim, waves, mask, grid, s);
   if (rc != MI355_SDPA_OK) return rc;
-  return check_launch("fwd_w32_kernel");
+  rc = check_launch("fwd_w32_kernel");
+  if (rc != MI355_SDPA_OK || !g.split_tiles) return rc;
+  const dim3 rows((unsigned)((int64_t)g.B * g.Hq * g.L));
+  if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((fwd_split_merge_kernel<bf16_t>), rows, dim3(128), 0, s, g);
+  else hipLaunchKernelGGL((fwd_split_merge_kernel<f16_t>), rows, dim3(128), 0, s, g);
+  return check_launch("fwd_split_merge_kernel");
 }
 
 }  // namespace mi355

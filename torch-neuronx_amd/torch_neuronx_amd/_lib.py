@@ -57,6 +57,7 @@ class FwdParams(C.Structure):
         ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
         ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
         ("force_kernel", C.c_int32), ("mask", MaskSpec),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
     ]
 
 
@@ -85,6 +86,7 @@ EXPORTS = {
     "mi355_sdpa_fwd": (C.c_int, [C.POINTER(FwdParams), C.c_void_p]),
     "mi355_sdpa_bwd": (C.c_int, [C.POINTER(BwdParams), C.c_void_p]),
     "mi355_sdpa_bwd_workspace_bytes": (C.c_size_t, [C.POINTER(BwdParams)]),
+    "mi355_sdpa_fwd_workspace_bytes": (C.c_size_t, [C.POINTER(FwdParams)]),
     "mi355_sdpa_decode_fp8kv": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),
     "mi355_sdpa_decode_workspace_bytes": (C.c_size_t, [C.POINTER(DecodeParams)]),
     "mi355_sdpa_decode_fp8kv_static": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),

@@ -181,6 +181,13 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     if live_tiles is True:
         live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
     _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit, live_tiles)  # noqa: F841 (kept alive over the launch)
+    ws = None
+    if L * (Hq // max(key.shape[1], 1)) <= 256 and query.dtype in (torch.float16, torch.bfloat16):
+        # few query rows: the library may want to split the keys over more workgroups
+        need = _lib.load().mi355_sdpa_fwd_workspace_bytes(C.byref(p))
+        if need:
+            ws = torch.empty(need, dtype=torch.uint8, device=query.device)
+            p.workspace, p.workspace_bytes = ws.data_ptr(), need
     with _lib.on_device(query.device):
         rc = _lib.load().mi355_sdpa_fwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
