@@ -460,6 +460,7 @@ GROUPED = [
     (1, 16, 4, 8, 3000, 96, False, None),
     (2, 8, 2, 1, 2048, 128, False, [0, 2048]),  # a batch without keys: zeros and lse = -inf
     (1, 8, 4, 33, 2500, 128, False, None),
+    (2, 12, 12, 1, 4096, 64, False, [4096, 777]),  # one query head per kv head: split all the same
 ]
 
 

@@ -834,7 +834,8 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
   if (head_dim == 256) waves = 4;
   const int rep = g.Hq / g.Hkv;
   g.grouped = 0, g.split_tiles = 0, g.n_split = 1;
-  if (rep > 1 && (g.bias_kind == 0 || g.bias_sh == 0) && g.keep_scale == 0.f && !g.live_tiles) {
+  // (one head per kv head counts too: nothing is shared then, but such a call can split its keys)
+  if ((g.bias_kind == 0 || g.bias_sh == 0) && g.keep_scale == 0.f && !g.live_tiles) {
     const int blocks32 = (g.L + 31) / 32;  // 32-row blocks per head
     if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = 1;
     else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = 1;
