@@ -311,6 +311,24 @@ def extra_dropout(amd, dev):
             "shape": "B=32 H=12 S=512 D=64 bf16, dropout 0.1, right padding (key counts)"}
 
 
+def extra_decode_bf16(amd, dev):
+    """A decode step over a bf16 K/V cache through the ordinary forward (no fp8, no decode entry point):
+    Hq=32 Hkv=8 D=128 L=1, a full batch (the heads of a kv group share a workgroup) and a single
+    sequence (its keys are split over workgroups)."""
+    Hq, Hkv, D = 32, 8, 128
+    r = {}
+    for name, B, S in (("B64_S8192", 64, 8192), ("B1_S32768", 1, 32768)):
+        g = torch.Generator(device=dev).manual_seed(1013)  # (drawn on the device: the cache is 2 x 1 GB)
+        q = torch.randn((B, Hq, 1, D), generator=g, device=dev, dtype=torch.bfloat16)
+        k, v = (torch.randn((B, Hkv, S, D), generator=g, device=dev, dtype=torch.bfloat16) for _ in range(2))
+        amd.sdpa_forward(q, k, v)
+        _, ev = event_time_ms(lambda: amd.sdpa_forward(q, k, v), 20, 5)
+        r[name] = {"ms": ev, "kv_GB/s": 2.0 * B * Hkv * S * D * 2 / (ev * 1e-3) / 1e9}
+        del q, k, v
+    r["shape"] = "Hq=32 Hkv=8 D=128 L=1 bf16 cache"
+    return r
+
+
 def extra_f32(amd, dev):
     """float32 inputs on the float32 matrix op (peak 157.3 TFLOP/s), B=2 Hq=32 Hkv=8 S=4096 D=128 causal."""
     B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
@@ -478,7 +496,7 @@ def main():
         except Exception as e:
             extras["masked_fwd_shared_bias"] = {"error": repr(e)}
         for name, fn in (("window_1024_fwd_bwd", extra_window), ("document_mask_tables_fwd_bwd", extra_documents),
-                         ("head_dim_256_fwd_bwd", extra_wide), ("dropout_padding_fwd_bwd", extra_dropout),
+                         ("head_dim_256_fwd_bwd", extra_wide), ("dropout_padding_fwd_bwd", extra_dropout), ("decode_bf16_cache_fwd", extra_decode_bf16),
                          ("float32_fwd_bwd", extra_f32)):
             try:
                 extras[name] = fn(amd, dev)
