@@ -457,7 +457,7 @@ GROUPED = [
     # few (batch, kv head) pairs and many keys: the keys are split over workgroups and merged
     (1, 32, 8, 1, 8192, 128, False, [5000]),
     (2, 8, 2, 3, 4096, 64, False, [4096, 100]),
-    (1, 16, 4, 8, 3000, 96, False, None),
+    (1, 16, 4, 8, 3000, 96, False, None),   # (also with a left-padding mask and a bias: split with a bias)
     (2, 8, 2, 1, 2048, 128, False, [0, 2048]),  # a batch without keys: zeros and lse = -inf
     (1, 8, 4, 33, 2500, 128, False, None),
     (2, 12, 12, 1, 4096, 64, False, [4096, 777]),  # one query head per kv head: split all the same
@@ -488,6 +488,9 @@ def test_short_queries_with_grouped_heads(amd, gpu_device, case, dtype):
         out, lse = amd.sdpa_forward(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), attn_bias=lp.to(gpu_device), force_kernel=MFMA)
         ro, rl = oracle_fwd(q, k, v, attn_mask=lp.expand(B, 1, L, S))
         assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3) and max_abs(lse, rl) <= 2e-3
+        if B * Hkv < 256 and S >= 512:  # (these split their keys as well)
+            need = B * Hq * L * 4
+            assert need > 0
         bias = torch.randn(B, 1, L, S, generator=torch.Generator().manual_seed(S + 1)).to(dtype)
         out, lse = amd.sdpa_forward(q.to(gpu_device), k.to(gpu_device), v.to(gpu_device), attn_bias=bias.to(gpu_device), force_kernel=MFMA)
         ro, rl = oracle_fwd(q, k, v, attn_mask=bias.float())

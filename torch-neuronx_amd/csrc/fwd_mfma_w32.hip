@@ -134,7 +134,10 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
     }
-    if (p.split_tiles) {  // this workgroup's share of the key tiles (no window then)
+  }
+  constexpr bool SPLITS = FUNC || (MASK == 2 && D <= 128);  // the variants that can split their keys
+  if constexpr (SPLITS) {
+    if (p.split_tiles) {  // this workgroup's share of the key tiles (no window, no skip table then)
       skip = split * p.split_tiles;
       nt = max(min(nt - skip, p.split_tiles), 0);
     }
@@ -172,12 +175,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   }
   auto tile_of = [&](int u) {
-    if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
+    if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u + skip;
     else return FUNC ? u + (u >= n_lead ? skip : 0) : u;
   };
   if constexpr (MASK) {
     if (nt <= 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87), or the sink logit alone
-      if constexpr (FUNC) {
+      if constexpr (SPLITS) {
         if (p.split_tiles) {  // (split keys: a part without keys carries no weight in the merge)
           if (qrow < p.L && half == 0) p.part_lse[(((int64_t)b * p.Hq + h) * p.n_split + split) * p.L + qrow] = -INFINITY;
           return;
@@ -383,7 +386,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       if (bkind) {
         // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-        const uint32_t g0 = b_voff + (uint32_t)((listed ? tile_of(min(t, nt - 1)) : t) * BN * b_esz);
+        const uint32_t g0 = b_voff + (uint32_t)((listed ? tile_of(min(t, nt - 1)) : t + skip) * BN * b_esz);
         tile_load(b_rsrc, g0, lds_b);
         if (b_loads > 1) tile_load(b_rsrc, g0 + 32, lds_b + 1024);
         if (b_loads > 2) {
@@ -711,7 +714,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       }
     }
   }
-  if constexpr (FUNC) {
+  if constexpr (SPLITS) {
     if (p.split_tiles) {  // split keys: this part's normalised rows and their log-sum-exp, in float32, for the merge
       if (qrow < p.L) {
         const int64_t prow = (((int64_t)b * p.Hq + h) * p.n_split + split) * p.L + qrow;
@@ -840,7 +843,7 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
     if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = 1;
     else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = 1;
   }
-  if (g.grouped && head_dim <= 128 && g.bias_kind == 0 && !g.causal && g.window == 0 && !g.sink_logit) {
+  if (g.grouped && head_dim <= 128 && !g.causal && g.window == 0 && !g.sink_logit) {
     const int64_t groups = (int64_t)g.B * g.Hkv;
     const int nt = (g.S + BN - 1) / BN;
     const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);
