@@ -191,6 +191,9 @@ size_t mi355_sdpa_fwd_workspace_bytes(const mi355_sdpa_fwd_params* p);
  * _sdpa_math.py:98-176 (compute_attention_backward) and decompositions.py:2569-2599
  * (_reduce_gqa_gradients). */
 int mi355_sdpa_bwd(const mi355_sdpa_bwd_params* p, void* stream);
+/* Bytes of workspace this backward call needs: the row terms (rowsum(dO * O) and the log-sum-exp in
+ * the log2 domain), and for a call with few key blocks the float32 partial dK / dV rows of the
+ * workgroups that share a key block.  Ask per call: the size depends on every shape. */
 size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p);
 
 /* Decode-step attention over an fp8 e4m3 K/V cache with per-sequence lengths.

@@ -565,3 +565,77 @@ def test_wide_backward_is_what_autograd_reaches(amd, gpu_device):
     ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, is_causal=True)
     for a, r in ((qd.grad, rdq), (kd.grad, rdk), (vd.grad, rdv)):
         assert max_abs(a, r) <= 5e-2 and rel_err(a, r) <= 2e-2
+
+
+# Few key blocks (few kv heads, short keys): the dK/dV kernels deal a key block's query tiles to several
+# workgroups, which leave float32 rows in the workspace for a kernel that adds them up.
+SPLIT_ITEMS = [
+    # B, Hq, Hkv, L, S, E, Dv, causal, mask, splits
+    (1, 8, 1, 512, 512, 128, 128, True, None, True),
+    (2, 14, 2, 300, 333, 64, 64, True, None, True),
+    (1, 4, 4, 2000, 77, 40, 40, False, None, True),
+    (2, 8, 2, 700, 257, 128, 128, False, "kv_lens", True),
+    (1, 4, 1, 512, 384, 64, 64, False, "bias", True),
+    (2, 4, 1, 512, 384, 128, 128, False, "bool", True),
+    (1, 2, 1, 1024, 128, 128, 128, False, "dropout", True),
+    (1, 8, 1, 1000, 1000, 256, 256, True, None, True),
+    (2, 4, 2, 800, 333, 192, 128, True, None, True),
+    (1, 4, 4, 2000, 77, 160, 160, False, None, True),
+    (2, 4, 1, 900, 257, 192, 128, False, "kv_lens", True),
+    (1, 4, 1, 1024, 384, 192, 128, False, "bool", True),
+    # the full-width kernel with a mask does not split; few items do not either
+    (2, 4, 1, 900, 257, 256, 256, False, "kv_lens", False),
+    (1, 2, 2, 512, 512, 64, 64, True, None, False),
+]
+
+
+@pytest.mark.parametrize("case", SPLIT_ITEMS)
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_few_key_blocks_deal_their_query_tiles_to_several_workgroups(amd, gpu_device, monkeypatch, case, dtype):
+    B, Hq, Hkv, L, S, E, Dv, causal, mask, splits = case
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, Dv=Dv, dtype=dtype, seed=L + 7 * S + E, with_do=True)
+    go = (go.float().clamp(-1, 1) * 0.1).to(dtype)
+    g = torch.Generator().manual_seed(L + S)
+    kw, om_mask, keep = {}, None, None
+    if mask == "kv_lens":
+        lens = torch.randint(0, S + 1, (B,), generator=g).to(torch.int32)
+        om_mask = (torch.arange(S)[None] < lens[:, None])[:, None, None, :]
+        kw["kv_lens"] = lens.to(gpu_device)
+    elif mask == "bias":
+        om_mask = torch.randn(1, Hq, L, S, generator=g).to(dtype)
+        kw["attn_bias"] = om_mask.to(gpu_device)
+        om_mask = om_mask.float()
+    elif mask == "bool":
+        om_mask = torch.rand(B, 1, L, S, generator=g) > 0.5
+        om_mask[..., 0] = True
+        kw["attn_bias"], kw["live_tiles"] = om_mask.to(gpu_device), True
+    elif mask == "dropout":
+        keep = torch.rand(B, Hq, L, S, generator=g) >= 0.25
+        kw["dropout_p"], kw["dropout_keep"] = 0.25, keep.to(gpu_device)
+
+    # what the library asks for as workspace tells whether the call splits: the row terms alone, or more
+    lib = amd._lib.load()
+    real, asked = lib.mi355_sdpa_bwd_workspace_bytes, []
+
+    def spy(p):
+        asked.append(real(p))
+        return asked[-1]
+
+    monkeypatch.setattr(lib, "mi355_sdpa_bwd_workspace_bytes", spy)
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, gpu_device, q, k, v, go, MFMA, is_causal=causal, **kw)
+    row_terms = (B * Hq * L * 2 * 4 + 255) // 256 * 256
+    assert (asked[-1] > row_terms) == splits, (asked, row_terms)
+
+    if keep is None:
+        ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, attn_mask=om_mask, is_causal=causal)
+    else:
+        rep = Hq // Hkv
+        kf, vf = k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1)
+        ro, rl = om.compute_attention(q.float(), kf, vf, None, keep, E**-0.5, causal, 0.25)
+        rdq, rdk, rdv, _ = om.compute_attention_backward(go.float(), q.float(), kf, vf, None, keep, ro, rl, E**-0.5, causal, 0.25)
+        rdk, rdv = rdk.view(B, Hkv, rep, S, E).sum(2), rdv.view(B, Hkv, rep, S, Dv).sum(2)
+    assert max_abs(out, ro) <= 2e-2
+    for name, a, r in (("dq", dq, rdq), ("dk", dk, rdk), ("dv", dv, rdv)):
+        assert torch.isfinite(a.float()).all(), name
+        assert max_abs(a, r) <= 5e-2, name
+        assert rel_err(a, r) <= 2e-2, name

@@ -122,8 +122,13 @@ def test_forward_and_backward_with_tables(amd, gpu_device, case, dtype):
     g0 = amd.sdpa_backward(god, qd, kd, vd, o0, l0, attn_bias=md, force_kernel=MFMA)
     g1 = amd.sdpa_backward(god, qd, kd, vd, o0, l0, attn_bias=md, force_kernel=MFMA, live_tiles=True)
     torch.cuda.synchronize()
+    # (dK and dV: a call with few key blocks deals a block's query tiles to several workgroups, and
+    # the tables change which tiles a workgroup adds up before the float32 partial sums meet: one
+    # rounding step of the output dtype at most)
+    step = 2.0**-7 if dtype == torch.bfloat16 else 2.0**-10
     for a, b_ in zip(g1[:3], g0[:3]):
-        assert max_abs(a, b_.cpu()) <= 1e-6
+        a, b_ = a.float().cpu(), b_.float().cpu()
+        assert ((a - b_).abs() <= step * b_.abs() + 1e-6).all()
     bias = mask.expand(B, 1, n, n) if kind == "bool" else m.float().expand(B, 1, n, n)
     rq, rk, rv = oracle_bwd(go, q, k, v, ro, rl, attn_mask=bias)[:3]
     for a, r in zip(g1[:3], (rq, rk, rv)):
@@ -146,8 +151,9 @@ def test_rectangular_block_sparse_masks_with_tables(amd, gpu_device, shape):
     g1 = amd.sdpa_backward(god, qd, kd, vd, o0, l0, attn_bias=md, force_kernel=MFMA, live_tiles=True)
     torch.cuda.synchronize()
     assert max_abs(o1, o0.cpu()) <= 1e-6 and max_abs(l1, l0.cpu()) <= 1e-5
-    for a, b_ in zip(g1[:3], g0[:3]):
-        assert max_abs(a, b_.cpu()) <= 1e-6
+    for a, b_ in zip(g1[:3], g0[:3]):  # (one rounding step where the call splits a key block's query tiles: see above)
+        a, b_ = a.float().cpu(), b_.float().cpu()
+        assert ((a - b_).abs() <= 2.0**-7 * b_.abs() + 1e-6).all()
     ro, rl = oracle_fwd(q, k, v, attn_mask=mask)
     assert max_abs(o1, ro) <= 2e-2 and max_abs(l1, rl) <= 5e-3
     for a, r in zip(g1[:3], oracle_bwd(go, q, k, v, ro, rl, attn_mask=mask)[:3]):

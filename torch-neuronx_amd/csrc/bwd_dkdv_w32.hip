@@ -54,8 +54,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   uint16_t* const items_s = (uint16_t*)(live_s + 256);  // [1024] live items, and their count behind them
 
   const int streams = p.B * p.Hkv;
-  const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
-  const int st = blockIdx.x % streams;
+  // (split items: part by part, so that a (batch, kv head) keeps its place modulo 8 in the launch order)
+  const int part = p.parts > 1 ? blockIdx.x / (streams * p.n_kt) : 0;
+  const int blk = p.parts > 1 ? blockIdx.x - part * (streams * p.n_kt) : blockIdx.x;
+  const int kt = blk / streams;  // low key tiles see the most queries under a causal mask: first
+  const int st = blk % streams;
   const int b = st / p.Hkv, hk = st % p.Hkv;
   const int rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63;
@@ -115,9 +118,10 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // per call on a (2, 32/8, 4096, 128) problem, against 0.13 GB of Q and dO.)
   // (with a skip table: the items whose tile holds a kept score, listed in LDS before the first item)
   bool compact = false;
+  int it0 = 0;  // first item of this workgroup's part
   auto item_id = [&](int it) {
-    if constexpr (MASK == 2) return compact ? __builtin_amdgcn_readfirstlane((int)items_s[it]) : it;
-    else return it;
+    if constexpr (MASK == 2) return compact ? __builtin_amdgcn_readfirstlane((int)items_s[it + it0]) : it + it0;
+    else return it + it0;
   };
   // (item / rep as a multiply-high by ceil(2^32 / rep), exact while item * rep < 2^32: these two are
   // evaluated many times per item, on the scalar unit, and a division there is twenty instructions)
@@ -534,6 +538,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       }
     }
   }
+  if (p.parts > 1) {  // this workgroup's share of the (live) items
+    const int chunk = (n_items + p.parts - 1) / p.parts;
+    it0 = part * chunk;
+    n_items = max(min(n_items - it0, chunk), 0);
+  }
   if (n_items > 0) {
     load_item(0, 0);
     wait_tiles();
@@ -567,10 +576,19 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
   }
 
-  if (key < p.S) {
+  const float sc = role ? p.scale : DROP ? p.keep_scale : 1.f;
+  if (p.parts > 1) {  // float32 rows for bwd_dkdv_merge_kernel, which also applies the factor
+    if (key < p.S) {
+      float* g = (role ? p.part_dk : p.part_dv) + ((((int64_t)part * p.B + b) * p.Hkv + hk) * p.S + key) * dr + half * 4;
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int gq = 0; gq < 4; ++gq)
+          if (!MASK || db * 32 + gq * 8 + half * 4 < dr) *(f32x4*)(g + db * 32 + gq * 8) = f32x4{acc[db][gq * 4], acc[db][gq * 4 + 1], acc[db][gq * 4 + 2], acc[db][gq * 4 + 3]};
+    }
+  } else if (key < p.S) {
     uint16_t* g = role ? (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl
                        : (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
-    const float sc = role ? p.scale : DROP ? p.keep_scale : 1.f;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -583,6 +601,32 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   }
 }
 
+// Sum of the parts' float32 rows, one 64-thread block per key row of a (batch, kv head): four columns
+// per thread, dK's d_real columns first, dV's dv_real behind them.  The factors that the kernels apply
+// when they write dK and dV themselves are applied here: the scale for dK, 1 / (1 - p) of dropout for dV.
+template <typename T>
+__global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
+  const int64_t row = blockIdx.x;  // (b * Hkv + hk) * S + key
+  const int key = (int)(row % p.S);
+  const int hk = (int)((row / p.S) % p.Hkv), b = (int)(row / ((int64_t)p.S * p.Hkv));
+  const int er = p.d_real, dvr = p.dv_real;
+  const int64_t rows = (int64_t)p.B * p.Hkv * p.S;
+  for (int c = threadIdx.x * 4; c < er + dvr; c += 64 * 4) {
+    const bool is_v = c >= er;
+    const int col = is_v ? c - er : c, width = is_v ? dvr : er;
+    const float* src = (is_v ? p.part_dv : p.part_dk) + row * width + col;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < p.parts; ++i) a += *(const f32x4*)(src + i * rows * width);
+    a *= is_v ? (p.keep_scale != 0.f ? p.keep_scale : 1.f) : p.scale;
+    uint16_t* g = is_v ? (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl
+                       : (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
+    u32x2 w;
+    w[0] = Mma<T>::pack(a[0], a[1]);
+    w[1] = Mma<T>::pack(a[2], a[3]);
+    *(u32x2*)(g + col) = w;
+  }
+}
+
 template <typename T, int D, int MASK>
 int launch_t(const BwdM& g, hipStream_t s) {
   constexpr int kSmemBytes = smem_bytes<D>() + (MASK == 2 ? 1024 + 2048 + 16 : 0);  // (with the skip table's row of the key block and the item list)
@@ -592,8 +636,10 @@ int launch_t(const BwdM& g, hipStream_t s) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dkdv_w32_kernel: %s", kSmemBytes, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D, MASK>), dim3((unsigned)(g.B * g.Hkv * g.n_kt)), dim3(512), kSmemBytes, s, g);
-  return check_launch("bwd_dkdv_w32_kernel");
+  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D, MASK>), dim3((unsigned)(g.B * g.Hkv * g.n_kt * g.parts)), dim3(512), kSmemBytes, s, g);
+  const int rc = check_launch("bwd_dkdv_w32_kernel");
+  if (rc != MI355_SDPA_OK || g.parts == 1) return rc;
+  return launch_bwd_dkdv_merge(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
 }
 template <typename T, int D>
 int launch_m(const BwdM& g, hipStream_t s) {
@@ -611,7 +657,28 @@ bool bwd_dkdv_w32_fits(const BwdM& g, int head_dim) {
   return q_ext < (1ll << 31) && go_ext < (1ll << 31) && g.q_sh >= 0 && g.q_sl >= 0 && g.go_sh >= 0 && g.go_sl >= 0;
 }
 
-int launch_bwd_dkdv_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
+// Fewer key blocks than would give every compute unit a workgroup or two: their items are dealt to
+// `parts` workgroups each, at least 8 items a part (an item is a 64-row query tile of one head, about
+// a microsecond) and only from 24 items on: below that the second kernel costs what the split saves.
+int bwd_dkdv_w32_parts(const BwdM& g) {
+  const int64_t wgs = (int64_t)g.B * g.Hkv * g.n_kt;
+  if (wgs >= 384 || wgs <= 0) return 1;
+  const int64_t items = (int64_t)(g.Hq / g.Hkv) * ((g.L + BQ - 1) / BQ);  // of a key block that every query sees
+  if (items < 24) return 1;
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>((768 + wgs - 1) / wgs, items / 8), 16));
+}
+int launch_bwd_dkdv_merge(const BwdM& g, int dtype, hipStream_t s) {
+  const dim3 rows((unsigned)((int64_t)g.B * g.Hkv * g.S));
+  if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dkdv_merge_kernel<bf16_t>), rows, dim3(64), 0, s, g);
+  else hipLaunchKernelGGL((bwd_dkdv_merge_kernel<f16_t>), rows, dim3(64), 0, s, g);
+  return check_launch("bwd_dkdv_merge_kernel");
+}
+
+int launch_bwd_dkdv_w32(const BwdM& g0, int dtype, int head_dim, hipStream_t s) {
+  BwdM g = g0;
+  if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
+  g.dv_real = g.d_real;
+  if (!g.part_dk || !g.part_dv) g.parts = 1;
   if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 128>(g, s) : launch_m<f16_t, 128>(g, s);
   return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 64>(g, s) : launch_m<f16_t, 64>(g, s);
 }

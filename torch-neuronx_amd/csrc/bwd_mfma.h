@@ -53,7 +53,20 @@ struct BwdM {
   // block) a bitmap of the 32-key tiles with a kept score, live_words words each
   const uint32_t* live_tiles = nullptr;
   int live_words = 0;
+  // dK/dV kernel of bwd_dkdv_w32.hip with too few key blocks for the 256 compute units (few kv heads,
+  // short keys): the items of a key block (query tile x head of the group) go to `parts` workgroups,
+  // each of which leaves float32 partial rows in the workspace - part_dk / part_dv, indexed
+  // [part][batch][kv head][key][d_real or dv_real] - and bwd_dkdv_merge_kernel adds them up
+  // (bwd_wide.hip's kernel deals out whole query tiles in the same way)
+  int parts = 1;
+  float *part_dk = nullptr, *part_dv = nullptr;
 };
+
+// parts the dK/dV kernel of bwd_dkdv_w32.hip / of bwd_wide.hip would use for this call
+int bwd_dkdv_w32_parts(const BwdM& g);
+int bwd_wide_parts(const BwdM& g);
+// adds up the parts' rows (g.parts, g.part_dk with d_real columns, g.part_dv with dv_real) into dK and dV
+int launch_bwd_dkdv_merge(const BwdM& g, int dtype, hipStream_t s);
 
 // dot product of eight packed elements, float32 accumulation
 template <typename T>

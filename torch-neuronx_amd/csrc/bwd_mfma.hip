@@ -623,8 +623,24 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   return true;
 }
 
+// delta and lse2, rounded up to 256 bytes, and behind them the partial dK / dV rows of a call whose
+// dK/dV kernel splits its items
+static size_t row_terms_bytes(const mi355_sdpa_bwd_params& p) {
+  return ((size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float) + 255) & ~(size_t)255;
+}
+static int parts_of(const BwdM& g, const mi355_sdpa_bwd_params& p) {
+  if (p.k.size[2] <= 0 || p.k.size[1] <= 0) return 1;
+  if (p.q.size[3] > 128 || p.v.size[3] != p.q.size[3]) return bwd_wide_parts(g);
+  return bwd_dkdv_w32_fits(g, p.q.size[3] <= 64 ? 64 : 128) ? bwd_dkdv_w32_parts(g) : 1;
+}
+static size_t part_rows_bytes(const BwdM& g, int parts) {  // dK rows, then dV rows
+  return parts > 1 ? (size_t)parts * g.B * g.Hkv * g.S * (g.d_real + g.dv_real) * sizeof(float) : 0;
+}
 size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p) {
-  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float);  // delta and lse2
+  if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return row_terms_bytes(p);
+  BwdM g;
+  fill(g, p);
+  return row_terms_bytes(p) + part_rows_bytes(g, parts_of(g, p));
 }
 
 int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
@@ -635,6 +651,12 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   }
   BwdM g;
   fill(g, p);
+  const int parts = parts_of(g, p);
+  if (parts > 1 && p.workspace_bytes >= row_terms_bytes(p) + part_rows_bytes(g, parts)) {
+    g.parts = parts;
+    g.part_dk = (float*)((char*)p.workspace + row_terms_bytes(p));
+    g.part_dv = g.part_dk + (size_t)parts * g.B * g.Hkv * g.S * g.d_real;
+  }
   const int D = p.q.size[3] <= 64 ? 64 : 128;  // the kernels' width
   int rc;
   if (p.q.size[3] > 128 || p.v.size[3] != p.q.size[3]) rc = launch_bwd_wide(g, p.dtype, s);

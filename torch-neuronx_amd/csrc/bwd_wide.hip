@@ -426,8 +426,15 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   float* const dl_buf = lse_buf + 2 * BT;                      // [2][BT]
   uint32_t* const live_s = (uint32_t*)(dl_buf + 2 * BT);       // (masked instances) [heads of the group][words]
   const int streams = p.B * p.Hkv;
-  const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
-  const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
+  // (split query tiles: part by part, so that a (batch, kv head) keeps its place modulo 8 in the launch order)
+  // (not in the masked instance at full width, which has no scalar register left for it)
+  constexpr bool SPLIT = !(MASKED && ER + DVR > 320);
+  // (the part is worked out again where the results are written rather than kept in a register all along)
+  auto parts_of = [&]() { return SPLIT ? p.parts : 1; };
+  auto part_of = [&]() { return parts_of() > 1 ? (int)blockIdx.x / (p.B * p.Hkv * p.n_kt) : 0; };
+  const int blk = parts_of() > 1 ? blockIdx.x - part_of() * (streams * p.n_kt) : blockIdx.x;
+  const int kt = blk / streams;  // low key tiles see the most queries under a causal mask: first
+  const int st = blk % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
   const int k0 = kt * 128, kw0 = k0 + wave * 32, key = kw0 + col;
   const int er = p.d_real, dvr = p.dv_real;
@@ -464,7 +471,12 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 
   // Items: query tile by query tile from the last one down, heads inside: the workgroups of a kv head,
   // which share an XCD, then want the same Q / dO tile at about the same time and find it in its L2.
-  const int n_items = (MASKED && k0 >= S) ? 0 : (nqs - qs_begin) * rep;  // no live key in this block: zeros
+  int qs_hi = nqs, qs_lo = qs_begin;  // this workgroup's query tiles: qs_hi - 1 down to qs_lo
+  if (parts_of() > 1) {
+    const int chunk = (nqs - qs_begin + parts_of() - 1) / parts_of();
+    qs_hi = nqs - part_of() * chunk, qs_lo = max(qs_hi - chunk, qs_begin);
+  }
+  const int n_items = (MASKED && k0 >= S) ? 0 : max(qs_hi - qs_lo, 0) * rep;  // no live key in this block: zeros
   // bias of this lane's key in the 32 rows of an item, one element per score register, requested
   // ahead of the item's first product through a resource that ends with the (batch, head)'s last row
   const int bkind = MASKED ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
@@ -557,14 +569,14 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     __syncthreads();
   };
   if (n_items > 0) {
-    if (item_live(nqs - 1, 0)) request_item(nqs - 1, 0, 0);
+    if (item_live(qs_hi - 1, 0)) request_item(qs_hi - 1, 0, 0);
     publish_item(0);
   }
   int buf = 0;
   // (two nested loops on purpose: written as one loop over items, the compiler spills the fragments)
-  for (int qs = nqs - 1; qs >= qs_begin; --qs) {
+  for (int qs = qs_hi - 1; qs >= qs_lo; --qs) {
     for (int hg = 0; hg < rep; ++hg) {
-    const bool last = qs == qs_begin && hg == rep - 1;
+    const bool last = qs == qs_lo && hg == rep - 1;
     // (the other buffer was last read before the barrier that ended the previous item)
     const int qs_n = hg + 1 < rep ? qs : qs - 1, hg_n = hg + 1 < rep ? hg + 1 : 0;
     if (!last && item_live(qs_n, hg_n)) request_item(qs_n, hg_n, buf ^ 1);
@@ -672,7 +684,23 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     if (!last) publish_item(buf);
     }
   }
-  if (key < p.S) {
+  if (parts_of() > 1) {  // float32 rows for bwd_dkdv_merge_kernel, which also multiplies dK by the scale
+    if (key < p.S) {
+      const int64_t row = (((int64_t)part_of() * p.B + b) * p.Hkv + hk) * p.S + key;
+      float* gk = p.part_dk + row * er + half * 4;
+      float* gv = p.part_dv + row * dvr + half * 4;
+#pragma unroll
+      for (int db = 0; db < DBE; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (db * 32 + g * 8 + half * 4 < er) *(f32x4*)(gk + db * 32 + g * 8) = f32x4{dkacc[db][g * 4], dkacc[db][g * 4 + 1], dkacc[db][g * 4 + 2], dkacc[db][g * 4 + 3]};
+#pragma unroll
+      for (int db = 0; db < DBV; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (db * 32 + g * 8 + half * 4 < dvr) *(f32x4*)(gv + db * 32 + g * 8) = f32x4{dvacc[db][g * 4], dvacc[db][g * 4 + 1], dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]};
+    }
+  } else if (key < p.S) {
     uint16_t* gk = (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
     uint16_t* gv = (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
 #pragma unroll
@@ -719,8 +747,10 @@ int launch_t(const BwdM& g, hipStream_t s) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", kDkdvLds, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>), dim3((unsigned)k_blocks), dim3(256), kDkdvLds, s, g);
-  return check_launch("bwd_wide_dkdv_kernel");
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>), dim3((unsigned)(k_blocks * g.parts)), dim3(256), kDkdvLds, s, g);
+  rc = check_launch("bwd_wide_dkdv_kernel");
+  if (rc || g.parts == 1) return rc;
+  return launch_bwd_dkdv_merge(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
 }
 // widths the kernels are instantiated for: 192 / 128 (multi-head latent attention) and the full 256 / 256
 template <typename T>
@@ -732,7 +762,22 @@ int launch_w(const BwdM& g, hipStream_t s) {
 
 }  // namespace
 
-int launch_bwd_wide(const BwdM& g, int dtype, hipStream_t s) {
+// As in bwd_dkdv_w32.hip: with fewer key blocks than keep the compute units busy, the query tiles of a
+// key block go to `parts` workgroups (every head of the group with each tile), at least 16 items - a
+// 32-row tile of one head here - a part.
+int bwd_wide_parts(const BwdM& g) {
+  const int64_t wgs = (int64_t)g.B * g.Hkv * g.n_kt;
+  if (wgs >= 384 || wgs <= 0) return 1;
+  if ((g.bias_kind || g.kv_lens) && !(g.d_real <= 192 && g.dv_real <= 128)) return 1;  // (that instance does not split)
+  const int64_t tiles = (g.L + BT - 1) / BT;
+  const int64_t items = tiles * (g.Hq / g.Hkv);
+  if (items < 48) return 1;
+  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>((768 + wgs - 1) / wgs, std::min(items / 16, tiles)), 16));
+}
+
+int launch_bwd_wide(const BwdM& g0, int dtype, hipStream_t s) {
+  BwdM g = g0;
+  if (!g.part_dk || !g.part_dv) g.parts = 1;
   return dtype == MI355_SDPA_BF16 ? launch_w<bf16_t>(g, s) : launch_w<f16_t>(g, s);
 }
 
