@@ -163,10 +163,11 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
         out = torch.empty((B, Hq, L, Dv), dtype=query.dtype, device=query.device)
     lse = torch.empty((B, Hq, L), dtype=torch.float32, device=query.device) if need_lse else None
     bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
-    p = _lib.FwdParams()
-    p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (q, k, v, out))
+    p, P = _lib.FwdParams(), _lib.FwdParams
+    for f, t in ((P.q, q), (P.k, k), (P.v, v), (P.out, out), (P.bias, bias)):
+        _lib.put4(p, f, t)
     p.lse = lse.data_ptr() if lse is not None else None
-    p.bias, p.bias_dtype = _lib.tensor4(bias), bias_dt
+    p.bias_dtype = bias_dt
     if kv_lens is not None:
         kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
         p.kv_lens = kv_lens.data_ptr()
@@ -221,11 +222,12 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     dbias = None
     if want_grad_bias and bias is not None:
         dbias = torch.empty((B, Hq, L, S), dtype=query.dtype, device=query.device)
-    p = _lib.BwdParams()
-    p.grad_out, p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (go, q, k, v, o))
+    p, P = _lib.BwdParams(), _lib.BwdParams
+    for f, t in ((P.grad_out, go), (P.q, q), (P.k, k), (P.v, v), (P.out, o), (P.grad_q, dq), (P.grad_k, dk),
+                 (P.grad_v, dv), (P.bias, bias), (P.grad_bias, dbias)):
+        _lib.put4(p, f, t)
     p.lse = lse.data_ptr()
-    p.grad_q, p.grad_k, p.grad_v = (_lib.tensor4(t) for t in (dq, dk, dv))
-    p.bias, p.bias_dtype, p.grad_bias = _lib.tensor4(bias), bias_dt, _lib.tensor4(dbias)
+    p.bias_dtype = bias_dt
     if kv_lens is not None:
         kv_lens = kv_lens.to(device=query.device, dtype=torch.int32).contiguous()
         p.kv_lens = kv_lens.data_ptr()
@@ -296,8 +298,9 @@ def decode_fp8kv(query, k_fp8, v_fp8, k_scale, v_scale, kv_lens=None, scale=None
         raise ValueError("decode_fp8kv: out must have shape (B, Hq, Lq, D) and the query's dtype")
     if lse is not None and (tuple(lse.shape) != (B, Hq, Lq) or lse.dtype != torch.float32 or not lse.is_contiguous()):
         raise ValueError("decode_fp8kv: lse must be a contiguous float32 (B, Hq, Lq) tensor")
-    p = _lib.DecodeParams()
-    p.q, p.k, p.v, p.out = (_lib.tensor4(t) for t in (q, k, v, out))
+    p, P = _lib.DecodeParams(), _lib.DecodeParams
+    for f, t in ((P.q, q), (P.k, k), (P.v, v), (P.out, out)):
+        _lib.put4(p, f, t)
     p.k_scale, p.v_scale = ks.data_ptr(), vs.data_ptr()
     if kv_lens is not None:
         p.kv_lens = kv_lens.data_ptr()
