@@ -329,6 +329,17 @@ def extra_decode_bf16(amd, dev):
     return r
 
 
+def extra_few_kv_heads(amd, dev):
+    """Backward with few key blocks, where the dK/dV kernel deals a block's query tiles to several
+    workgroups: one kv head for 32 query heads (B=2 S=4096) and a 32/8 model at batch 1 (S=2048), D=128 causal."""
+    r = {}
+    for name, B, Hq, Hkv, S in (("mqa_32_1_B2_S4096", 2, 32, 1, 4096), ("gqa_32_8_B1_S2048", 1, 32, 8, 2048)):
+        q, k, v, do = seeded([(B, Hq, S, 128), (B, Hkv, S, 128), (B, Hkv, S, 128), (B, Hq, S, 128)], 1015, torch.bfloat16, dev)
+        r[name] = _fwd_bwd_rates(amd, q, k, v, do, causal_pairs(S, S), 128, 128, is_causal=True)
+    r["shape"] = "D=128 bf16 causal"
+    return r
+
+
 def extra_f32(amd, dev):
     """float32 inputs on the float32 matrix op (peak 157.3 TFLOP/s), B=2 Hq=32 Hkv=8 S=4096 D=128 causal."""
     B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
@@ -497,7 +508,7 @@ def main():
             extras["masked_fwd_shared_bias"] = {"error": repr(e)}
         for name, fn in (("window_1024_fwd_bwd", extra_window), ("document_mask_tables_fwd_bwd", extra_documents),
                          ("head_dim_256_fwd_bwd", extra_wide), ("dropout_padding_fwd_bwd", extra_dropout), ("decode_bf16_cache_fwd", extra_decode_bf16),
-                         ("float32_fwd_bwd", extra_f32)):
+                         ("few_kv_heads_fwd_bwd", extra_few_kv_heads), ("float32_fwd_bwd", extra_f32)):
             try:
                 extras[name] = fn(amd, dev)
             except Exception as e:
