@@ -639,3 +639,33 @@ def test_few_key_blocks_deal_their_query_tiles_to_several_workgroups(amd, gpu_de
         assert torch.isfinite(a.float()).all(), name
         assert max_abs(a, r) <= 5e-2, name
         assert rel_err(a, r) <= 2e-2, name
+
+
+def test_long_causal_sequence_by_its_prefix_and_its_last_row(amd, gpu_device):
+    """S = 65536 is beyond what the oracle finishes in seconds; checked by what a causal mask fixes:
+    the first rows of out, lse and dQ depend on the first keys only (equal to a call on that prefix),
+    the last row is one softmax over all keys (float64 on the host), and dV of the last key is
+    p(last row, last key) * dO(last row) summed over the group's heads."""
+    B, Hq, Hkv, S, D, n = 1, 4, 1, 65536, 128, 2048
+    dev = gpu_device
+    g = torch.Generator(device=dev).manual_seed(65536)
+    q, k, v, do = (torch.randn((B, h, S, D), generator=g, device=dev, dtype=torch.bfloat16) for h in (Hq, Hkv, Hkv, Hq))
+    out, lse = amd.sdpa_forward(q, k, v, is_causal=True, force_kernel=MFMA)
+    dq, dk, dv, _ = amd.sdpa_backward(do, q, k, v, out, lse, is_causal=True, force_kernel=MFMA)
+    qs, ks, vs, dos = (t[:, :, :n].contiguous() for t in (q, k, v, do))
+    o2, l2 = amd.sdpa_forward(qs, ks, vs, is_causal=True, force_kernel=MFMA)
+    dq2 = amd.sdpa_backward(dos, qs, ks, vs, o2, l2, is_causal=True, force_kernel=MFMA)[0]
+    torch.cuda.synchronize()
+    assert max_abs(out[:, :, :n], o2.cpu()) <= 1e-6 and max_abs(lse[:, :, :n], l2.cpu()) <= 1e-5
+    assert max_abs(dq[:, :, :n], dq2.cpu()) <= 2e-3
+    for t in (dq, dk, dv):
+        assert torch.isfinite(t.float()).all()
+    kk, vv = k[0, 0].double().cpu(), v[0, 0].double().cpu()
+    acc = torch.zeros(D, dtype=torch.float64)
+    for h in range(Hq):
+        s_ = (kk @ q[0, h, S - 1].double().cpu()) * D**-0.5
+        lse_ref = torch.logsumexp(s_, 0)
+        assert abs(lse_ref.item() - lse[0, h, S - 1].item()) <= 1e-4
+        assert (torch.softmax(s_, 0) @ vv - out[0, h, S - 1].double().cpu()).abs().max().item() <= 2e-3
+        acc += torch.exp(s_[S - 1] - lse_ref) * do[0, h, S - 1].double().cpu()
+    assert (acc - dv[0, 0, S - 1].double().cpu()).abs().max().item() <= 1e-2 * acc.abs().max().item() + 1e-7
