@@ -391,6 +391,10 @@ def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
     vq, vs = om.quantize_kv_fp8(torch.randn(4, Hkv, 512, E, generator=g))
     kq, vq, ks, vs = kq.to(dev), vq.to(dev), ks.to(dev), vs.to(dev)
     lens = torch.tensor([512, 1, 300, 77], dtype=torch.int32, device=dev)
+    # calls that split their work over more workgroups and add the parts up in a second kernel: a
+    # decode-like forward over long keys, a backward with one kv head
+    q1, kl, vl = mk(1, Hq, 1, E), mk(1, Hkv, 4096, E), mk(1, Hkv, 4096, E)
+    qm, km, vm, gom = mk(1, 8, 512, E), mk(1, 1, 512, E), mk(1, 1, 512, E), mk(1, 8, 512, E)
 
     def work():
         out, lse = amd.sdpa_forward(q, k, v, is_causal=True)
@@ -398,7 +402,10 @@ def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
         outb, lseb = amd.sdpa_forward(q, k, v, attn_bias=bias)
         dqb, dkb, dvb, dbb = amd.sdpa_backward(go, q, k, v, outb, lseb, attn_bias=bias, want_grad_bias=True)
         od, ld = amd.decode_fp8kv(qd, kq, vq, ks, vs, lens)
-        return [out, lse, dq, dk, dv, outb, dqb, dkb, dvb, dbb, od, ld]
+        o1, l1 = amd.sdpa_forward(q1, kl, vl)
+        om_, lm = amd.sdpa_forward(qm, km, vm, is_causal=True)
+        dqm, dkm, dvm, _ = amd.sdpa_backward(gom, qm, km, vm, om_, lm, is_causal=True)
+        return [out, lse, dq, dk, dv, outb, dqb, dkb, dvb, dbb, od, ld, o1, l1, dqm, dkm, dvm]
 
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
@@ -409,7 +416,7 @@ def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
     with torch.cuda.graph(graph):
         captured = work()
     for rep in range(3):
-        for t in (q, k, v, go, qd):
+        for t in (q, k, v, go, qd, q1, kl, qm, km, gom):
             t.copy_(torch.randn(t.shape, generator=g).to(t.dtype))
         bias.mul_(0.5)
         eager = [t.clone() for t in work()]
