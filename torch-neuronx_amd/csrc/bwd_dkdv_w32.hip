@@ -54,13 +54,25 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   uint16_t* const items_s = (uint16_t*)(live_s + 256);  // [1024] live items, and their count behind them
 
   const int streams = p.B * p.Hkv;
-  // (split items: part by part, so that a (batch, kv head) keeps its place modulo 8 in the launch order)
-  const int part = p.parts > 1 ? blockIdx.x / (streams * p.n_kt) : 0;
-  const int blk = p.parts > 1 ? blockIdx.x - part * (streams * p.n_kt) : blockIdx.x;
-  const int kt = blk / streams;  // low key tiles see the most queries under a causal mask: first
-  const int st = blk % streams;
+  // Split items: a key block's heads go to parts_h workgroups, and their query tiles to parts / parts_h.
+  // A (batch, kv head, share of the heads) keeps its place in the launch order modulo the number of
+  // such streams - and with that its XCD, when that number is a multiple of 8 - over all key blocks
+  // and tile shares: the workgroups that walk the same Q / dO tiles meet in one L2.
+  int kt, st, ph = 0, pq = 0;
+  if (p.parts > 1) {
+    const int vstreams = streams * p.parts_h;
+    const int v = blockIdx.x % vstreams, rest = blockIdx.x / vstreams;
+    kt = rest % p.n_kt, pq = rest / p.n_kt;
+    st = v / p.parts_h, ph = v % p.parts_h;
+  } else {
+    kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
+    st = blockIdx.x % streams;
+  }
+  const int part = pq * p.parts_h + ph;  // its rows among the partial results
   const int b = st / p.Hkv, hk = st % p.Hkv;
-  const int rep = p.Hq / p.Hkv;
+  const int rep_all = p.Hq / p.Hkv;
+  const int rep = p.parts > 1 ? rep_all / p.parts_h : rep_all;  // heads of the group that this workgroup walks
+  const int h0 = ph * rep;                                       // the first of them
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int role = wave >> 2, kb = wave & 3;  // wavefronts w and w + 4 share a SIMD and a key block
@@ -127,7 +139,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // evaluated many times per item, on the scalar unit, and a division there is twenty instructions)
   const uint32_t rep_inv = (uint32_t)((0x100000000ull + (uint32_t)rep - 1) / (uint32_t)rep);
   auto item_tile = [&](int it) { return rep == 1 ? item_id(it) : (int)__umulhi((uint32_t)item_id(it), rep_inv); };  // (2^32 does not fit)
-  auto item_head = [&](int it) { return hk * rep + (item_id(it) - item_tile(it) * rep); };
+  auto item_head = [&](int it) { return hk * rep_all + h0 + (item_id(it) - item_tile(it) * rep); };
   auto item_q0 = [&](int it) { return (qs_end - 1 - item_tile(it)) * BQ; };
 
   // ---- staging: every thread moves two 16-byte chunks of the Q tile and two of the dO tile ------
@@ -432,7 +444,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     if constexpr (MASK == 2) {
       if (listed) {
         const int qt = q0 / BQ;
-        const int hg = item_id(it) % rep;
+        const int hg = h0 + item_id(it) % rep;
         if (!compact && !((__builtin_amdgcn_readfirstlane((int)live_s[hg * p.live_t_words + (qt >> 5)]) >> (qt & 31)) & 1)) return true;
       }
     }
@@ -514,8 +526,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 
   if constexpr (MASK == 2) {
     if (listed) {  // this key block's row of the skip table, for every head of the group
-      if (tid < rep * p.live_t_words) {
-        const int hd = hk * rep + tid / p.live_t_words;
+      if (tid < rep_all * p.live_t_words) {
+        const int hd = hk * rep_all + tid / p.live_t_words;
         live_s[tid] = p.live_t[(((int64_t)(p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? hd : 0)) * ((p.S + BK - 1) / BK) + kt) * p.live_t_words +
                                tid % p.live_t_words];
       }
@@ -525,7 +537,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
           int cnt = 0;
           for (int j0 = 0; j0 < n_items; j0 += 64) {
             const int it = j0 + lane, qt = qs_end - 1 - it / rep;
-            const bool live = it < n_items && ((live_s[(it % rep) * p.live_t_words + (qt >> 5)] >> (qt & 31)) & 1u);
+            const bool live = it < n_items && ((live_s[(h0 + it % rep) * p.live_t_words + (qt >> 5)] >> (qt & 31)) & 1u);
             const uint64_t m = __builtin_amdgcn_ballot_w64(live);
             if (live) items_s[cnt + __builtin_amdgcn_mbcnt_hi((uint32_t)(m >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)m, 0u))] = (uint16_t)it;
             cnt += __builtin_popcountll(m);
@@ -539,9 +551,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
   }
   if (p.parts > 1) {  // this workgroup's share of the (live) items
-    const int chunk = (n_items + p.parts - 1) / p.parts;
-    it0 = part * chunk;
+    const bool fixed = p.chunk_items > 0 && !listed;
+    const int parts_q = p.parts / p.parts_h;
+    const int chunk = fixed ? p.chunk_items : (n_items + parts_q - 1) / parts_q;
+    it0 = pq * chunk;
     n_items = max(min(n_items - it0, chunk), 0);
+    // (a share past the key block's items: bwd_dkdv_merge_kernel, which counts them in the same way,
+    // does not read it)
+    if (fixed && n_items == 0 && pq > 0) return;
   }
   if (n_items > 0) {
     load_item(0, 0);
@@ -611,12 +628,23 @@ __global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
   const int hk = (int)((row / p.S) % p.Hkv), b = (int)(row / ((int64_t)p.S * p.Hkv));
   const int er = p.d_real, dvr = p.dv_real;
   const int64_t rows = (int64_t)p.B * p.Hkv * p.S;
+  int parts = p.parts;
+  if (p.chunk_items > 0 && p.live_t == nullptr) {
+    // the parts that bwd_dkdv_w32_kernel filled for this row's key block: its items, counted as there
+    const int k0 = key / BK * BK, nqs = (p.L + BQ - 1) / BQ;
+    int S = p.S;
+    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+    const int qs_end = (p.window > 0 && k0 >= p.sink_keys) ? max(min(nqs, (k0 + BK + p.window - 2) / BQ + 1), qs_begin) : nqs;
+    const int n_items = k0 >= S ? 0 : (p.Hq / p.Hkv / p.parts_h) * (qs_end - qs_begin);
+    parts = min(max((n_items + p.chunk_items - 1) / p.chunk_items, 1), p.parts / p.parts_h) * p.parts_h;
+  }
   for (int c = threadIdx.x * 4; c < er + dvr; c += 64 * 4) {
     const bool is_v = c >= er;
     const int col = is_v ? c - er : c, width = is_v ? dvr : er;
     const float* src = (is_v ? p.part_dv : p.part_dk) + row * width + col;
     f32x4 a = {0.f, 0.f, 0.f, 0.f};
-    for (int i = 0; i < p.parts; ++i) a += *(const f32x4*)(src + i * rows * width);
+    for (int i = 0; i < parts; ++i) a += *(const f32x4*)(src + i * rows * width);
     a *= is_v ? (p.keep_scale != 0.f ? p.keep_scale : 1.f) : p.scale;
     uint16_t* g = is_v ? (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl
                        : (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
@@ -657,16 +685,31 @@ bool bwd_dkdv_w32_fits(const BwdM& g, int head_dim) {
   return q_ext < (1ll << 31) && go_ext < (1ll << 31) && g.q_sh >= 0 && g.q_sl >= 0 && g.go_sh >= 0 && g.go_sl >= 0;
 }
 
-// Fewer key blocks than would give every compute unit a workgroup or two: their items are dealt to
-// `parts` workgroups each, at least 8 items a part (an item is a 64-row query tile of one head, about
-// a microsecond) and only from 24 items on: below that the second kernel costs what the split saves.
-int bwd_dkdv_w32_parts(const BwdM& g) {
+// Fewer key blocks than would give every compute unit a workgroup or two: a key block's items (an
+// item is a 64-row query tile of one head, about a microsecond) are dealt to about 768 workgroups in
+// all.  The heads of the group are divided first (every share walks all query tiles, in the order the
+// other key blocks' workgroups walk them, so that they keep finding the tiles in their XCD's L2),
+// then the query tiles, in shares of chunk_items items: at least 8 items each, and only from 24 items
+// on: below that the second kernel costs what the split saves.
+void bwd_dkdv_w32_plan(const BwdM& g, int& parts_h, int& parts) {
+  parts_h = parts = 1;
   const int64_t wgs = (int64_t)g.B * g.Hkv * g.n_kt;
-  if (wgs >= 384 || wgs <= 0) return 1;
-  const int64_t items = (int64_t)(g.Hq / g.Hkv) * ((g.L + BQ - 1) / BQ);  // of a key block that every query sees
-  if (items < 24) return 1;
-  return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>((768 + wgs - 1) / wgs, items / 8), 16));
+  if (wgs >= 384 || wgs <= 0) return;
+  const int rep = g.Hq / g.Hkv, nqs = (g.L + BQ - 1) / BQ;
+  if ((int64_t)rep * nqs < 24) return;
+  const int64_t want = (768 + wgs - 1) / wgs;
+  for (int d = 1; d <= rep && d <= want; ++d)
+    if (rep % d == 0 && (int64_t)(rep / d) * nqs >= 8) parts_h = d;
+  const int64_t items = (int64_t)(rep / parts_h) * nqs;  // of a workgroup that every query of its heads sees
+  const int64_t parts_q = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>((want + parts_h - 1) / parts_h, items / 8), 32));
+  parts = (int)(parts_h * parts_q);
 }
+int bwd_dkdv_w32_parts(const BwdM& g) {
+  int parts_h, parts;
+  bwd_dkdv_w32_plan(g, parts_h, parts);
+  return parts;
+}
+
 int launch_bwd_dkdv_merge(const BwdM& g, int dtype, hipStream_t s) {
   const dim3 rows((unsigned)((int64_t)g.B * g.Hkv * g.S));
   if (dtype == MI355_SDPA_BF16) hipLaunchKernelGGL((bwd_dkdv_merge_kernel<bf16_t>), rows, dim3(64), 0, s, g);
@@ -678,7 +721,19 @@ int launch_bwd_dkdv_w32(const BwdM& g0, int dtype, int head_dim, hipStream_t s) 
   BwdM g = g0;
   if (g.d_real <= 0 || g.d_real > head_dim) g.d_real = head_dim;
   g.dv_real = g.d_real;
+  g.parts_h = 1, g.chunk_items = 0;
   if (!g.part_dk || !g.part_dv) g.parts = 1;
+  if (g.parts > 1) {
+    int parts;
+    bwd_dkdv_w32_plan(g, g.parts_h, parts);
+    if (parts != g.parts) {
+      set_error("SDPA: bwd_dkdv_w32_kernel was given %d parts where its plan has %d", g.parts, parts);
+      return MI355_SDPA_ERR_INVALID;
+    }
+    // the heaviest workgroup (every query tile of its heads) fills all the tile shares
+    const int parts_q = g.parts / g.parts_h;
+    g.chunk_items = ((g.Hq / g.Hkv / g.parts_h) * ((g.L + BQ - 1) / BQ) + parts_q - 1) / parts_q;
+  }
   if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 128>(g, s) : launch_m<f16_t, 128>(g, s);
   return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 64>(g, s) : launch_m<f16_t, 64>(g, s);
 }

@@ -59,7 +59,12 @@ struct BwdM {
   // [part][batch][kv head][key][d_real or dv_real] - and bwd_dkdv_merge_kernel adds them up
   // (bwd_wide.hip's kernel deals out whole query tiles in the same way)
   int parts = 1;
+  int parts_h = 1;  // bwd_dkdv_w32.hip: of these, shares of the group's heads (a divisor of Hq / Hkv and of parts)
   float *part_dk = nullptr, *part_dv = nullptr;
+  // bwd_dkdv_w32.hip without a skip table: items per part (the same for every key block, so that a
+  // block with fewer items - a causal mask, a window, a batch with fewer keys - fills fewer parts;
+  // the others are neither written nor read).  0: every key block uses all `parts`, in equal shares.
+  int chunk_items = 0;
 };
 
 // parts the dK/dV kernel of bwd_dkdv_w32.hip / of bwd_wide.hip would use for this call
