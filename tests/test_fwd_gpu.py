@@ -453,7 +453,16 @@ GROUPED = [
     (2, 4, 2, 40, 40, 128, True, None),      # two 32-row blocks per head, causal
     (1, 16, 4, 32, 513, 64, True, [400]),
     (2, 8, 4, 64, 200, 256, False, None),    # head dim 256: four wavefronts, two heads x two blocks
-    (1, 6, 2, 17, 90, 96, False, None),      # three heads per group: not grouped, same answers
+    (1, 6, 2, 17, 90, 96, False, None),      # three heads per group: one head per workgroup, same answers
+    # more heads per kv head than wavefronts, or a number that does not divide them: a share of the
+    # group's heads per workgroup (8 of 32, 8 of 16, 2 of 6, 4 of 12; 4 of 8 at head dim 256)
+    (2, 32, 1, 1, 4096, 128, False, [4096, 1234]),
+    (1, 64, 4, 2, 700, 64, False, None),
+    (3, 12, 2, 1, 1000, 128, False, None),
+    (1, 24, 2, 30, 260, 64, True, None),
+    (2, 8, 1, 1, 520, 256, False, [520, 77]),
+    (1, 8, 1, 1, 4096, 256, False, [3000]),  # (head dims above 128 do not split their keys)
+    (2, 4, 4, 2, 2048, 192, False, None),
     # few (batch, kv head) pairs and many keys: the keys are split over workgroups and merged
     (1, 32, 8, 1, 8192, 128, False, [5000]),
     (2, 8, 2, 3, 4096, 64, False, [4096, 100]),

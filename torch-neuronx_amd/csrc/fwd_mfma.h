@@ -27,10 +27,11 @@ struct FwdM {
   // bias fields above describe the (B, Hq, L, S) keep-mask, kind 4
   float keep_scale = 0.f;
   // Short query sequences under grouped-query attention (fwd_mfma_w32.hip; no dropout, no bias that
-  // depends on the head): one
-  // workgroup per (batch, kv head) serves every query head of the group, wavefront w the rows
-  // 32 * (w / rep) .. +31 of head hk * rep + w % rep, so that a K / V tile is fetched once for all
-  // of them (decode-like calls are bound by exactly that traffic).  0 = off.
+  // depends on the head): one workgroup serves `grouped` query heads of a kv group (all Hq / Hkv of
+  // them where they fit its wavefronts; a divisor of that otherwise, with Hq / Hkv / grouped
+  // workgroups per kv head): wavefront w the rows 32 * (w / grouped) .. +31 of the workgroup's head
+  // w % grouped, so that a K / V tile is fetched once for all of them (decode-like calls are bound
+  // by exactly that traffic).  0 = off.
   int grouped = 0;
   // ... and, when that leaves most compute units without a workgroup, the keys are split: n_split
   // workgroups per (batch, kv head), each over split_tiles 32-key tiles, leave their normalised output

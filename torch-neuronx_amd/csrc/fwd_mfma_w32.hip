@@ -83,11 +83,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   int wrow = wave * 32;  // this wavefront's first row within the workgroup's rows
   int split = 0;  // (grouped calls with split keys: which part of them)
   if (MASK <= 2 && p.grouped) {  // (see FwdM::grouped)
-    const int rep = p.Hq / p.Hkv;
-    const int bhk = blockIdx.x / p.n_split;
+    const int rep = p.Hq / p.Hkv, hpw = p.grouped, chunks = rep / hpw;  // heads per workgroup, workgroups per kv head
+    const int bhc = blockIdx.x / p.n_split;
     split = blockIdx.x % p.n_split;
-    b = bhk / p.Hkv, h = (bhk % p.Hkv) * rep + wave % rep, qt = 0;
-    wrow = (wave / rep) * 32;
+    const int bhk = bhc / chunks;
+    b = bhk / p.Hkv, h = (bhk % p.Hkv) * rep + (bhc % chunks) * hpw + wave % hpw, qt = 0;
+    wrow = (wave / hpw) * 32;
   } else {
     decode_block(p, b, h, qt);
   }
@@ -826,7 +827,8 @@ int launch_dims(const FwdM& g, int head_dim, int waves, int mask, dim3 grid, hip
 }  // namespace
 
 // Grouped mode: every head of a kv group in one workgroup when their rows fit its wavefronts (four
-// wavefronts where they do, eight otherwise) and there is no dropout mask and no bias that depends
+// wavefronts where they do, eight otherwise; for up to 32 query rows also a share of the group's
+// heads per workgroup) and there is no dropout mask and no bias that depends
 // on the head (with one that does not, every wavefront of the workgroup arrives at the same key count
 // when it trims a keep-mask per key, and so at the same number of tiles).  When that leaves most of
 // the 256 compute units without a workgroup and the key loop is long, the keys are split: at least 8
@@ -840,11 +842,18 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
   // (one head per kv head counts too: nothing is shared then, but such a call can split its keys)
   if ((g.bias_kind == 0 || g.bias_sh == 0) && g.keep_scale == 0.f && !g.live_tiles) {
     const int blocks32 = (g.L + 31) / 32;  // 32-row blocks per head
-    if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = 1;
-    else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = 1;
+    if (4 % rep == 0 && blocks32 * rep <= 4) waves = 4, g.grouped = rep;
+    else if (head_dim != 256 && 8 % rep == 0 && blocks32 * rep <= 8) waves = 8, g.grouped = rep;
+    else if (blocks32 == 1) {
+      // a decode step with more heads per kv head than wavefronts, or a number of them that does not
+      // divide 8: 8, 4, 2 or 1 of them per workgroup, whichever is the most that divides it
+      int d = head_dim != 256 ? 8 : 4;
+      while (rep % d != 0) d >>= 1;
+      waves = d == 8 ? 8 : 4, g.grouped = d;
+    }
   }
   if (g.grouped && head_dim <= 128 && !g.causal && g.window == 0 && !g.sink_logit) {
-    const int64_t groups = (int64_t)g.B * g.Hkv;
+    const int64_t groups = (int64_t)g.B * g.Hkv * (g.Hq / g.Hkv / g.grouped);
     const int nt = (g.S + BN - 1) / BN;
     const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);
     if (groups < 256 && want >= 2) {
@@ -870,7 +879,7 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     if (g.part_o && g.part_bytes >= rows * (g.dv_real + 1) * sizeof(float)) g.part_lse = g.part_o + rows * g.dv_real;
     else g.split_tiles = 0, g.n_split = 1;
   }
-  const int64_t blocks = g.grouped ? (int64_t)g.B * g.Hkv * g.n_split : (int64_t)g.B * g.Hq * g.n_qt;
+  const int64_t blocks = g.grouped ? (int64_t)g.B * (g.Hq / g.grouped) * g.n_split : (int64_t)g.B * g.Hq * g.n_qt;
   if (blocks == 0) return MI355_SDPA_OK;
   if (blocks > 0x7fffffff) {
     set_error("SDPA: too many query tiles (%lld)", (long long)blocks);
