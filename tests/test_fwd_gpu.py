@@ -461,7 +461,7 @@ GROUPED = [
     (3, 12, 2, 1, 1000, 128, False, None),
     (1, 24, 2, 30, 260, 64, True, None),
     (2, 8, 1, 1, 520, 256, False, [520, 77]),
-    (1, 8, 1, 1, 4096, 256, False, [3000]),  # (head dims above 128 do not split their keys)
+    (1, 8, 1, 1, 4096, 256, False, [3000]),  # ... and split keys at head dim 256 (no bias there)
     (2, 4, 4, 2, 2048, 192, False, None),
     # few (batch, kv head) pairs and many keys: the keys are split over workgroups and merged
     (1, 32, 8, 1, 8192, 128, False, [5000]),

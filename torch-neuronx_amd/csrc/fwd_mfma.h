@@ -34,10 +34,10 @@ struct FwdM {
   // by exactly that traffic).  0 = off.
   int grouped = 0;
   // ... and, when that leaves most compute units without a workgroup, the keys are split: n_split
-  // workgroups per (batch, kv head), each over split_tiles 32-key tiles, leave their normalised output
+  // workgroups per group of heads, each over split_tiles key tiles, leave their normalised output
   // (float32, (B, Hq, n_split, L, dv_real)) and log-sum-exp ((B, Hq, n_split, L)) in the workspace,
   // and fwd_split_merge_kernel combines them.  Grouped calls without a window, a sink logit, a skip
-  // table or the causal flag, head dims up to 128.  0 = off.
+  // table or the causal flag; with a bias, head dims up to 128 only.  0 = off.
   int split_tiles = 0, n_split = 1;
   float* part_o = nullptr;   // the workspace (part_bytes bytes of it)
   float* part_lse = nullptr;

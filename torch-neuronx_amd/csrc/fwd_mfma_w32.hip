@@ -136,7 +136,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       nt -= skip;
     }
   }
-  constexpr bool SPLITS = FUNC || (MASK == 2 && D <= 128);  // the variants that can split their keys
+  constexpr bool SPLITS = MASK == 1 || (MASK == 2 && D <= 128);  // the variants that can split their keys
   if constexpr (SPLITS) {
     if (p.split_tiles) {  // this workgroup's share of the key tiles (no window, no skip table then)
       skip = split * p.split_tiles;
@@ -177,7 +177,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   }
   auto tile_of = [&](int u) {
     if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u + skip;
-    else return FUNC ? u + (u >= n_lead ? skip : 0) : u;
+    else return FUNC ? u + (u >= n_lead ? skip : 0) : SPLITS ? u + skip : u;  // (head dim 256: split keys, no window)
   };
   if constexpr (MASK) {
     if (nt <= 0) {  // no live key: zeros and lse = -inf (torch_neuronx/_sdpa_math.py:85-87), or the sink logit alone
@@ -773,19 +773,24 @@ __global__ __launch_bounds__(128) void fwd_split_merge_kernel(FwdM p) {
   const float* pl = p.part_lse + bh * p.n_split * p.L + l;
   float m = -INFINITY;
   for (int s = 0; s < p.n_split; ++s) m = fmaxf(m, pl[(int64_t)s * p.L]);
-  float sum = 0.f, acc = 0.f;
-  const int d = threadIdx.x;
+  float sum = 0.f, acc[2] = {0.f, 0.f};
+  const int d = threadIdx.x;  // columns d and d + 128 (head dims up to 256)
   for (int s = 0; s < p.n_split; ++s) {
     const float ls = pl[(int64_t)s * p.L];
     if (ls == -INFINITY) continue;  // (a part without keys: its rows were never written)
     const float w = __expf(ls - m);
     sum += w;
-    if (d < p.dv_real) acc = fmaf(w, p.part_o[((bh * p.n_split + s) * p.L + l) * p.dv_real + d], acc);
+    const float* po = p.part_o + ((bh * p.n_split + s) * p.L + l) * p.dv_real;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+      if (d + 128 * i < p.dv_real) acc[i] = fmaf(w, po[d + 128 * i], acc[i]);
   }
-  if (d < p.dv_real) {
-    T* o = (T*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)l * p.o_sl + d;
-    *(uint16_t*)o = (uint16_t)Mma<T>::pack(sum > 0.f ? acc / sum : 0.f, 0.f);
-  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (d + 128 * i < p.dv_real) {
+      T* o = (T*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)l * p.o_sl + d + 128 * i;
+      *(uint16_t*)o = (uint16_t)Mma<T>::pack(sum > 0.f ? acc[i] / sum : 0.f, 0.f);
+    }
   if (d == 0 && p.lse) p.lse[row] = sum > 0.f ? m + __builtin_logf(sum) : -INFINITY;
 }
 
@@ -852,7 +857,8 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
       waves = d == 8 ? 8 : 4, g.grouped = d;
     }
   }
-  if (g.grouped && head_dim <= 128 && !g.causal && g.window == 0 && !g.sink_logit) {
+  // (the variant with a bias splits at head dims up to 128 only)
+  if (g.grouped && (head_dim <= 128 || g.bias_kind == 0) && !g.causal && g.window == 0 && !g.sink_logit) {
     const int64_t groups = (int64_t)g.B * g.Hkv * (g.Hq / g.Hkv / g.grouped);
     const int nt = (g.S + BN - 1) / BN;
     const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);
