@@ -183,7 +183,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
         live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
     _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit, live_tiles)  # noqa: F841 (kept alive over the launch)
     ws = None
-    if L * (Hq // max(key.shape[1], 1)) <= 256 and query.dtype in (torch.float16, torch.bfloat16):
+    if (L <= 32 or L * (Hq // max(key.shape[1], 1)) <= 256) and query.dtype in (torch.float16, torch.bfloat16):
         # few query rows: the library may want to split the keys over more workgroups
         need = _lib.load().mi355_sdpa_fwd_workspace_bytes(C.byref(p))
         if need:
