@@ -211,8 +211,11 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       if (!MASK || half * 8 + ks * 16 < dr) qf[ks] = *(const u32x4*)(qr + ks * 16);
       else qf[ks] = u32x4{0u, 0u, 0u, 0u};
     }
-    // (awaited here, once: left pending, their first use inside the tile loop would become a wait
-    // for every outstanding load there, the tile loads in flight included)
+    // (awaited in the prologue, once, behind the request for the first tiles, so that the two trips
+    // to memory overlap: left pending, their first use inside the tile loop would become a wait for
+    // every outstanding load there, the tile loads in flight included)
+  }
+  auto await_q = [&]() {
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+v"(qf[ks]));
     // (one wavefront per SIMD owns both halves of the register file: the Q fragments live in the
@@ -222,7 +225,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) asm volatile("" : "+a"(qf[ks]));
     }
-  }
+  };
 
   const int nt_w = p.causal ? min(nt, qw_last / BN + 1 - skip) : nt;
 
@@ -531,6 +534,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   load_bias(0);
   request_k(0);
   request_pair(0);
+  await_q();
   wait_all_tiles();
   __syncthreads();
   request_pair(1);
