@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused SDPA hot path on one MI355X.
 
-    python bench.py --gpus 1 --steps K --warmup W [--workload c3_fwd|c4_fwd_bwd|c5_decode|c2_fwd]
+    python bench.py --gpus 1 --steps K --warmup W [--workload c3_fwd|c4_fwd_bwd|c5_decode|c2_fwd|masked_fwd|mqa_fwd_bwd]
 
 A step is one pass of the hot path over one batch of synthetic input that is already resident
 in HBM.  The default workload is the one the headline metric is quoted on: causal GQA bf16
@@ -116,8 +116,8 @@ def wl_masked_fwd(amd, dev):
     return step, flops, cfg
 
 
-def wl_fwd_bwd(amd, dev):
-    B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
+def wl_fwd_bwd(amd, dev, Hkv=8):
+    B, Hq, S, D = 2, 32, 4096, 128
     q, k, v, do = seeded([(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, D), (B, Hq, S, D)], 1004,
                          torch.bfloat16, dev)
     pairs = causal_pairs(S, S)
@@ -393,7 +393,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="c3_fwd", choices=["c3_fwd", "c2_fwd", "c4_fwd_bwd", "c5_decode", "masked_fwd"])
+    ap.add_argument("--workload", default="c3_fwd", choices=["c3_fwd", "c2_fwd", "c4_fwd_bwd", "c5_decode", "masked_fwd", "mqa_fwd_bwd"])
     ap.add_argument("--no-extras", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-spin", action="store_true", help="skip the untimed clock spin-up (profiled runs)")
@@ -446,8 +446,9 @@ def main():
                 "kernel_ms": ev}
         unit, dtype = "TFLOP/s", "bf16"
         cpu = None  # the oracle's rate on this shape is the forward baseline of c3_fwd
-    elif args.workload == "c4_fwd_bwd":
-        sf, sb, f_fwd, f_bwd = wl_fwd_bwd(amd, dev)
+    elif args.workload in ("c4_fwd_bwd", "mqa_fwd_bwd"):  # (mqa: config 4 with one kv head for the 32 query heads)
+        hkv = 8 if args.workload == "c4_fwd_bwd" else 1
+        sf, sb, f_fwd, f_bwd = wl_fwd_bwd(amd, dev, hkv)
         _, ev_f = event_time_ms(sf, args.steps, args.warmup)
 
         def both():
@@ -462,11 +463,11 @@ def main():
         roof = {"bound": "mfma", "achieved": ach, "peak": PEAK_BF16_TFLOPS, "unit": "TFLOP/s",
                 "frac": ach / PEAK_BF16_TFLOPS, "traffic": None, "kernel": "backward (all kernels of one call)",
                 "kernel_ms": ev_b}
-        cfg = {"workload": "c4_causal_gqa_bf16_fwd_bwd", "B": 2, "Hq": 32, "Hkv": 8, "S": 4096, "D": 128,
+        cfg = {"workload": "c4_causal_gqa_bf16_fwd_bwd" if hkv == 8 else "causal_mqa_bf16_fwd_bwd", "B": 2, "Hq": 32, "Hkv": hkv, "S": 4096, "D": 128,
                "fwd_tflops": f_fwd / (ev_f * 1e-3) / 1e12, "bwd_tflops": ach,
                "algorithmic_flops": flops}
         unit, dtype = "TFLOP/s", "bf16"
-        cpu = None if args.no_cpu else cpu_baseline_fwd_bwd(2, 32, 8, 4096, 128, 1004, heads=32)
+        cpu = None if args.no_cpu or hkv != 8 else cpu_baseline_fwd_bwd(2, 32, 8, 4096, 128, 1004, heads=32)
     else:
         step, nbytes, cfg = wl_decode(amd, dev)
         wall, ev = event_time_ms(step, args.steps, args.warmup)
