@@ -583,8 +583,11 @@ SPLIT_ITEMS = [
     (1, 4, 4, 2000, 77, 160, 160, False, None, True),
     (2, 4, 1, 900, 257, 192, 128, False, "kv_lens", True),
     (1, 4, 1, 1024, 384, 192, 128, False, "bool", True),
-    # the full-width kernel with a mask does not split; few items do not either
-    (2, 4, 1, 900, 257, 256, 256, False, "kv_lens", False),
+    # the full-width kernel with a mask splits when it has no skip table to read
+    (2, 4, 1, 900, 257, 256, 256, False, "kv_lens", True),
+    (1, 8, 1, 700, 640, 256, 256, True, "kv_lens", True),
+    (1, 4, 1, 1024, 384, 256, 256, False, "bool", False),
+    # few items do not split
     (1, 2, 2, 512, 512, 64, 64, True, None, False),
 ]
 

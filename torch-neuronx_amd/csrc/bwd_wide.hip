@@ -416,7 +416,10 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   }
 }
 
-template <typename T, int ER, int DVR, bool MASKED>
+// TABLES (masked instances): the tile skip table of a per-score mask is honoured.  At full width the
+// kernel has scalar registers for the table or for the split of a key block's query tiles over
+// workgroups, not for both: one instance of each.
+template <typename T, int ER, int DVR, bool MASKED, bool TABLES>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32, DBV = DVR / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
@@ -427,8 +430,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   uint32_t* const live_s = (uint32_t*)(dl_buf + 2 * BT);       // (masked instances) [heads of the group][words]
   const int streams = p.B * p.Hkv;
   // (split query tiles: part by part, so that a (batch, kv head) keeps its place modulo 8 in the launch order)
-  // (not in the masked instance at full width, which has no scalar register left for it)
-  constexpr bool SPLIT = !(MASKED && ER + DVR > 320);
+  constexpr bool SPLIT = !(TABLES && ER + DVR > 320);
   // (the part is worked out again where the results are written rather than kept in a register all along)
   auto parts_of = [&]() { return SPLIT ? p.parts : 1; };
   auto part_of = [&]() { return parts_of() > 1 ? (int)blockIdx.x / (p.B * p.Hkv * p.n_kt) : 0; };
@@ -518,7 +520,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   // With a skip table: an item whose 64-row block holds no kept score for this key block is neither
   // fetched nor computed.
   bool listed = false;
-  if constexpr (MASKED) {
+  if constexpr (TABLES) {
     if (p.live_t && !p.causal && rep * p.live_t_words <= 256) {
       listed = true;
       if (tid < rep * p.live_t_words) {
@@ -724,14 +726,28 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   }
 }
 
-template <typename T, int ER, int DVR, bool MASKED>
+template <typename T, int ER, int DVR, bool MASKED, bool TABLES>
+int launch_dkdv(const BwdM& g, int64_t k_blocks, hipStream_t s) {
+  constexpr int kDkdvLds = WIDE_DKDV_LDS + (MASKED ? WIDE_LIVE_LDS : 0);
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MASKED, TABLES>,
+                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDkdvLds);
+  if (attr != hipSuccess) {
+    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", kDkdvLds, hipGetErrorString(attr));
+    return MI355_SDPA_ERR_LAUNCH;
+  }
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED, TABLES>), dim3((unsigned)(k_blocks * g.parts)), dim3(256), kDkdvLds, s, g);
+  return check_launch("bwd_wide_dkdv_kernel");
+}
+
+// NO_TABLES: the masked full-width dK/dV instance that splits instead of reading a skip table
+template <typename T, int ER, int DVR, bool MASKED, bool NO_TABLES = false>
 int launch_t(const BwdM& g, hipStream_t s) {
   const int64_t q_blocks = (int64_t)g.B * g.Hq * ((g.L + 127) / 128), k_blocks = (int64_t)g.B * g.Hkv * ((g.S + 127) / 128);
   if (q_blocks > 0x7fffffff || k_blocks > 0x7fffffff) {
     set_error("SDPA: too many tiles for the wide backward kernels");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  constexpr int kDqLds = WIDE_DQ_LDS + (MASKED ? WIDE_LIST_LDS : 0), kDkdvLds = WIDE_DKDV_LDS + (MASKED ? WIDE_LIVE_LDS : 0);
+  constexpr int kDqLds = WIDE_DQ_LDS + (MASKED ? WIDE_LIST_LDS : 0);
   static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR, MASKED>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
   if (attr_q != hipSuccess) {
@@ -741,14 +757,7 @@ int launch_t(const BwdM& g, hipStream_t s) {
   hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR, MASKED>), dim3((unsigned)q_blocks), dim3(256), kDqLds, s, g);
   int rc = check_launch("bwd_wide_dq_kernel");
   if (rc) return rc;
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDkdvLds);
-  if (attr != hipSuccess) {
-    set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", kDkdvLds, hipGetErrorString(attr));
-    return MI355_SDPA_ERR_LAUNCH;
-  }
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED>), dim3((unsigned)(k_blocks * g.parts)), dim3(256), kDkdvLds, s, g);
-  rc = check_launch("bwd_wide_dkdv_kernel");
+  rc = launch_dkdv<T, ER, DVR, MASKED, MASKED && !(NO_TABLES && ER + DVR > 320)>(g, k_blocks, s);
   if (rc || g.parts == 1) return rc;
   return launch_bwd_dkdv_merge(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
 }
@@ -757,6 +766,7 @@ template <typename T>
 int launch_w(const BwdM& g, hipStream_t s) {
   const bool masked = g.bias_kind || g.kv_lens;
   if (g.d_real <= 192 && g.dv_real <= 128) return masked ? launch_t<T, 192, 128, true>(g, s) : launch_t<T, 192, 128, false>(g, s);
+  if (masked && g.parts > 1) return launch_t<T, 256, 256, true, true>(g, s);  // (bwd_wide_parts: no skip table then)
   return masked ? launch_t<T, 256, 256, true>(g, s) : launch_t<T, 256, 256, false>(g, s);
 }
 
@@ -768,7 +778,8 @@ int launch_w(const BwdM& g, hipStream_t s) {
 int bwd_wide_parts(const BwdM& g) {
   const int64_t wgs = (int64_t)g.B * g.Hkv * g.n_kt;
   if (wgs >= 384 || wgs <= 0) return 1;
-  if ((g.bias_kind || g.kv_lens) && !(g.d_real <= 192 && g.dv_real <= 128)) return 1;  // (that instance does not split)
+  // (the masked instance at full width either reads a skip table or splits)
+  if ((g.bias_kind || g.kv_lens) && !(g.d_real <= 192 && g.dv_real <= 128) && g.live_t) return 1;
   const int64_t tiles = (g.L + BT - 1) / BT;
   const int64_t items = tiles * (g.Hq / g.Hkv);
   if (items < 48) return 1;
