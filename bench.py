@@ -195,7 +195,7 @@ def cpu_baseline_fwd(B, Hq, Hkv, S, D, seed, heads=2):
     om.sdpa_forward(q, k, v, is_causal=True)
     dt = time.perf_counter() - t0
     flops = 4.0 * B * heads * D * causal_pairs(S, S)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "cpu_model": cpu_model(),
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "threads": cpu_threads(), "host_cores": os.cpu_count(), "cpu_model": cpu_model(),
             "kind": "port",
             "sample": f"{heads} of {Hq} query heads of the same workload, full S={S}; "
                       f"algorithmic (unmasked-pair) FLOPs / wall time; {dt:.2f} s"}
@@ -216,7 +216,7 @@ def cpu_baseline_fwd_bwd(B, Hq, Hkv, S, D, seed, heads=32):
     om.sdpa_backward(do, q, k, v, out, lse, is_causal=True)
     dt = time.perf_counter() - t0
     flops = 14.0 * heads * D * causal_pairs(S, S)
-    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "cpu_model": cpu_model(),
+    return {"value": flops / dt / 1e12, "unit": "TFLOP/s", "cores": cpu_threads(), "threads": cpu_threads(), "host_cores": os.cpu_count(), "cpu_model": cpu_model(),
             "kind": "port",
             "sample": f"{heads} of {B * Hq} (batch, query head) pairs of the same workload, full S={S}, "
                       f"forward + backward; algorithmic (unmasked-pair) FLOPs / wall time; {dt:.2f} s"}
@@ -236,7 +236,7 @@ def cpu_baseline_decode(batches=32):
     om.decode_fp8kv(q, kq, vq, ks, vs, lens)
     dt = time.perf_counter() - t0
     nbytes = 2.0 * Hkv * D * int(lens.sum())
-    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": cpu_threads(), "cpu_model": cpu_model(), "kind": "port",
+    return {"value": nbytes / dt / 1e9, "unit": "GB/s", "cores": cpu_threads(), "threads": cpu_threads(), "host_cores": os.cpu_count(), "cpu_model": cpu_model(), "kind": "port",
             "sample": f"first {batches} of {B} sequences of the same workload ({int(lens.sum())} live keys); "
                       f"fp8 K/V bytes of the live keys / wall time (dequantisation included); {dt:.2f} s"}
 

@@ -117,7 +117,12 @@ typedef struct mi355_sdpa_fwd_params {
   mi355_sdpa_tensor out;  /* (B,Hq,L,Dv)   same dtype as q                            */
   float* lse;             /* (B,Hq,L) contiguous float32, natural log; may be NULL    */
   mi355_sdpa_tensor bias; /* optional additive bias or bool keep-mask, sizes (B,Hq,L,S),
-                             stride 0 on broadcast dims                               */
+                             stride 0 on broadcast dims.  A BOOL bias (1 byte per score,
+                             non-zero = keep, zero = the score is -inf) is an extension of
+                             this boundary: the reference's operator only ever sees additive
+                             masks, because its caller turns a bool mask into 0 / -inf first
+                             (decompositions.py:2101-2102); here that conversion, a pass over
+                             L*S elements, is left out and the kernels read the bytes        */
   int32_t bias_dtype;     /* F32/F16/BF16/BOOL                                        */
   const int32_t* kv_lens; /* optional (B,): key j of batch b takes part iff j<kv_lens[b] */
   const uint8_t* dropout_keep; /* optional (B,Hq,L,S) contiguous, 1 = keep            */

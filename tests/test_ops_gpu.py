@@ -427,6 +427,111 @@ def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
             assert torch.equal(a, b), (rep, i)
 
 
+def _padding_case(dev, seed=11):
+    B, H, L, E = 3, 4, 512, 64
+    q, k, v = (t.to(dev) for t in qkv(B, H, H, L, L, E, dtype=torch.bfloat16, seed=seed))
+    lens = torch.tensor([L, 300, 77])
+    pad = (torch.arange(L)[None] < lens[:, None])[:, None, None, :]
+    return q, k, v, pad
+
+
+def test_masks_made_under_inference_mode(amd, gpu_device):
+    """Tensors created under torch.inference_mode() have no version counter: their masks are taken as
+    they are (no recognition, no cache, no tables) instead of raising.  Bool and additive masks, a
+    recognisable one (causal) and a padding one, forward only, against the oracle."""
+    from oracle import sdpa_math as om
+
+    dev = gpu_device
+    q, k, v, pad = _padding_case(dev)
+    L = q.shape[2]
+    amd.mask_patterns.clear_cache()
+    with torch.inference_mode():
+        tril = torch.ones(L, L, dtype=torch.bool, device=dev).tril()
+        add = torch.zeros(L, L, dtype=torch.bfloat16, device=dev).masked_fill(~tril, float("-inf"))
+        padd = pad.to(dev)
+        big = torch.ones(1, 1, L, L, dtype=torch.bool, device=dev).tril()  # large enough for skip tables
+        for mask, keep in ((tril, tril.cpu()), (add, tril.cpu()), (padd, pad), (big, tril.cpu())):
+            assert mask.is_inference()
+            out = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+            ro, _ = om.sdpa_forward(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=keep)
+            assert max_abs(out, ro) <= 2e-2
+            r = torch.ops.aten._scaled_dot_product_fused_attention_overrideable(q, k, v, mask)
+            assert max_abs(r[0], ro) <= 2e-2
+    assert len(amd.mask_patterns._cache) == 0 and len(amd.mask_patterns._tile_cache) == 0
+
+
+def test_mask_changed_in_place_between_calls(amd, gpu_device):
+    """A verdict is valid for one version of the tensor: after an in-place write the next call follows
+    the new contents (a padding mask whose lengths change, a causal mask that stops being one)."""
+    from oracle import sdpa_math as om
+
+    dev = gpu_device
+    q, k, v, pad = _padding_case(dev, seed=12)
+    L = q.shape[2]
+    fused = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    ref = lambda keep: om.sdpa_forward(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=keep)[0]
+    amd.mask_patterns.clear_cache()
+    padd = pad.to(dev)
+    for _ in range(2):  # (the second call is served from the cache)
+        assert max_abs(fused(q, k, v, padd)[0], ref(pad)) <= 2e-2
+    pad2 = (torch.arange(L)[None] < torch.tensor([100, L, 9])[:, None])[:, None, None, :]
+    padd.copy_(pad2)
+    assert max_abs(fused(q, k, v, padd)[0], ref(pad2)) <= 2e-2
+    pad3 = pad2.clone()
+    pad3[1, 0, 0, 5] = False  # no longer "keys 0 .. n-1"
+    padd.copy_(pad3)
+    assert max_abs(fused(q, k, v, padd)[0], ref(pad3)) <= 2e-2
+    tril = torch.ones(1, 1, L, L, dtype=torch.bool, device=dev).tril()
+    for _ in range(2):
+        assert max_abs(fused(q, k, v, tril)[0], ref(tril.cpu())) <= 2e-2
+    tril[0, 0, 3, 400] = True
+    assert max_abs(fused(q, k, v, tril)[0], ref(tril.cpu())) <= 2e-2
+    with amd.mask_patterns.left_alone():  # the per-call opt-out: the mask is taken as it is
+        looked = amd.mask_patterns.stats["looked"]
+        assert max_abs(fused(q, k, v, padd)[0], ref(pad3)) <= 2e-2
+        assert amd.mask_patterns.stats["looked"] == looked
+
+
+def test_a_captured_call_reads_its_mask_on_every_replay(amd, gpu_device):
+    """The usual graph contract: warm up with the static mask tensor, capture, then update the mask
+    in place between replays.  A captured call never uses a cached verdict about the mask (that
+    would freeze the old key counts into the graph): every replay follows the tensor's contents."""
+    from oracle import sdpa_math as om
+
+    dev = gpu_device
+    q, k, v, pad = _padding_case(dev, seed=13)
+    L = q.shape[2]
+    padd = pad.to(dev)
+    tril = torch.ones(1, 1, L, L, dtype=torch.bool, device=dev).tril()
+    fused = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    amd.mask_patterns.clear_cache()
+
+    def work():
+        return [fused(q, k, v, padd)[0], fused(q, k, v, tril)[0], F.scaled_dot_product_attention(q, k, v, attn_mask=padd)]
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            work()  # warm-up: the verdicts of both masks are in the cache now
+    torch.cuda.current_stream().wait_stream(side)
+    assert len(amd.mask_patterns._cache) >= 2
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        captured = work()
+    for lens in ([L, 300, 77], [5, L, 200], [L, L, L]):
+        keep = (torch.arange(L)[None] < torch.tensor(lens)[:, None])[:, None, None, :]
+        padd.copy_(keep)
+        tril[0, 0, 7, L - 1] = lens[0] == 5  # the second replay's mask is not causal
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        ro = om.sdpa_forward(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=keep)[0]
+        rt = om.sdpa_forward(q.float().cpu(), k.float().cpu(), v.float().cpu(), attn_mask=tril.cpu())[0]
+        assert max_abs(captured[0], ro) <= 2e-2 and max_abs(captured[2], ro) <= 2e-2, lens
+        assert max_abs(captured[1], rt) <= 2e-2, lens
+
+
 def test_fallback_to_the_generic_kernel_can_be_logged(gpu_device):
     """MI355_SDPA_LOG_FALLBACK=1: a call that the matrix-op kernels cannot take (head dim 100) says so
     on stderr, with the reason; a call they take says nothing.  (A child process: the switch is read once.)"""

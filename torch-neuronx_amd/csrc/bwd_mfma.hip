@@ -215,7 +215,7 @@ __global__ __launch_bounds__(256, 1) void bwd_dkdv_kernel(BwdM p) {
           else if (mq == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
-        mfma_to_valu_gap();
+        mfma_to_valu_gap(sacc, dpacc);
         if (edge) softmax(mq, sacc, dpacc, std::true_type{});
         else softmax(mq, sacc, dpacc, std::false_type{});
       }
@@ -430,7 +430,8 @@ __global__ __launch_bounds__(256, 1) void bwd_dq_kernel(BwdM p) {
           else if (mb == 0) ring[i % kRing] = read_rows(1, i + kRing - 2 * KS);
           else ring[i % kRing] = read_cols(i + kRing - 2 * KS);
         }
-        mfma_to_valu_gap();
+        if constexpr (NB == 2) mfma_to_valu_gap(sacc[0], dpacc[0], sacc[NB - 1], dpacc[NB - 1]);
+        else mfma_to_valu_gap(sacc[0], dpacc[0]);
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
           if (edge) softmax(nb, mb, sacc[nb], dpacc[nb], std::true_type{});

@@ -107,8 +107,16 @@ struct MmaV<f16_t> {
   }
 };
 // idle cycles after an 8-pass matrix op before the vector unit may touch its result (the
-// architecture asks for 11; the margin is free)
-__device__ __forceinline__ void mfma_to_valu_gap() { asm volatile("s_nop 15\n\ts_nop 7" ::: "memory"); }
+// architecture asks for 11; the margin is free).  The accumulators are operands of the statement:
+// the matrix ops that write them are inline assembly, whose hazard the compiler does not know, so
+// nothing else would keep it from placing a read of an accumulator between the last op and the idle
+// cycles.
+__device__ __forceinline__ void mfma_to_valu_gap(f32x16& a, f32x16& b) {
+  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(a), "+v"(b) :: "memory");
+}
+__device__ __forceinline__ void mfma_to_valu_gap(f32x16& a, f32x16& b, f32x16& c, f32x16& d) {
+  asm volatile("s_nop 15\n\ts_nop 7" : "+v"(a), "+v"(b), "+v"(c), "+v"(d) :: "memory");
+}
 
 __device__ __forceinline__ void zero(f32x16& a) {
 #pragma unroll

@@ -13,8 +13,11 @@ right padding, with or without causality folded in (per-batch key counts).
 
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 import os
+import threading
+import weakref
 from collections import OrderedDict
 
 import numpy as np
@@ -23,6 +26,11 @@ import torch
 from . import _lib
 
 _CACHE_ENTRIES = 16
+# key -> (pattern, weak reference to the mask's storage).  The cache never keeps a mask alive: an
+# entry goes when the storage dies (so its memory cannot come back under the same key with other
+# contents; views of one mask, which upstream makes afresh on every call, share the storage and its
+# version counter), and what an entry itself holds is a pattern tuple and at most a (B,) tensor of
+# key counts.
 _cache: "OrderedDict[tuple, tuple]" = OrderedDict()
 # Looking at a mask costs one device-to-host round trip.  A caller that hands in a NEW tensor on
 # every call (upstream's functional API turns a boolean mask into a fresh additive one each time
@@ -35,8 +43,62 @@ _misses: dict = {}
 stats = {"looked": 0, "hits": 0, "left_alone": 0}
 
 
+_switch = threading.local()
+
+
 def enabled() -> bool:
+    if getattr(_switch, "off", 0):
+        return False
     return os.environ.get("TORCH_NEURONX_AMD_RECOVER_MASKS", "1").lower() not in ("0", "false", "off", "no")
+
+
+@contextlib.contextmanager
+def left_alone():
+    """Calls made inside this block (on this thread) take their masks as they are: no look at the
+    tensor, no cache, no skip tables.  For masks that are written by something torch's version
+    counter does not see."""
+    _switch.off = getattr(_switch, "off", 0) + 1
+    try:
+        yield
+    finally:
+        _switch.off -= 1
+
+
+def _version(mask: torch.Tensor):
+    """The tensor's version counter, or ``None`` for a tensor that has none (created under
+    ``torch.inference_mode()``): nothing tells when such a tensor changes, so it is never cached
+    and never looked at - it stays the mask it is."""
+    if mask.is_inference():
+        return None
+    return mask._version
+
+
+def _remember(cache: OrderedDict, key, value, mask: torch.Tensor) -> None:
+    def drop(_ref, cache=cache, key=key):
+        cache.pop(key, None)
+
+    cache[key] = (value, weakref.ref(mask.untyped_storage(), drop))
+    while len(cache) > _CACHE_ENTRIES:
+        cache.popitem(last=False)
+
+
+def _lookup(cache: OrderedDict, key):
+    """``(True, value)`` for a live entry, ``(False, None)`` otherwise."""
+    hit = cache.get(key)
+    if hit is None:
+        return False, None
+    if hit[1]() is None:  # (the storage died and its callback has not run yet)
+        cache.pop(key, None)
+        return False, None
+    cache.move_to_end(key)
+    return True, hit[0]
+
+
+def _back_off(sig) -> bool:
+    """Counts a miss for this signature; True if the mask should be left alone this time."""
+    streak = _misses.get(sig, 0)
+    _misses[sig] = streak + 1
+    return streak >= _MAX_MISSES and (streak - _MAX_MISSES) % _RETRY_EVERY != _RETRY_EVERY - 1
 
 
 def pattern_from_rows(rows: np.ndarray, L: int, S: int):
@@ -134,30 +196,29 @@ def _as_2d(mask: torch.Tensor):
 
 def classify(mask: torch.Tensor):
     """Pattern of a device mask (see ``pattern_from_rows``), or ``None`` if it is none of them, is a
-    real bias, depends on batch or head, or cannot be looked at now (stream capture in progress).
-    The answer is cached while the tensor is unchanged (its version counter included); the cache
-    holds the tensor, so its memory cannot be handed to another mask meanwhile."""
+    real bias, depends on batch or head, or cannot be looked at.  Never during a stream capture, not
+    even from the cache: a captured call must read the mask tensor itself on every replay, because
+    the caller may update it in place between replays.  The answer is cached while the tensor is
+    alive and unchanged (its version counter included)."""
     if mask.device.type != "cuda" or _lib.dtype_id(mask.dtype) not in (_lib.BOOL, _lib.F32, _lib.F16, _lib.BF16):
+        return None
+    version = _version(mask)
+    if version is None or torch.cuda.is_current_stream_capturing():
         return None
     m = _as_2d(mask)
     if m is None:
-        return _classify_batched(mask)
+        return _classify_batched(mask, version)
     L, S = m.shape
     if L < 1 or S < 1:
         return None
-    key = (m.data_ptr(), L, S, m.stride(0), m.dtype, mask._version, mask.device.index)
+    key = (m.data_ptr(), L, S, m.stride(0), m.dtype, version, mask.device.index)
     sig = (L, S, m.dtype, mask.device.index)
-    hit = _cache.get(key)
-    if hit is not None:
-        _cache.move_to_end(key)
+    found, pat = _lookup(_cache, key)
+    if found:
         _misses.pop(sig, None)
         stats["hits"] += 1
-        return hit[0]
-    if torch.cuda.is_current_stream_capturing():
-        return None
-    streak = _misses.get(sig, 0)
-    _misses[sig] = streak + 1
-    if streak >= _MAX_MISSES and (streak - _MAX_MISSES) % _RETRY_EVERY != _RETRY_EVERY - 1:
+        return pat
+    if _back_off(sig):
         stats["left_alone"] += 1
         return None
     stats["looked"] += 1
@@ -167,16 +228,14 @@ def classify(mask: torch.Tensor):
                                               _lib.current_stream(mask.device))
     _lib.check(rc)
     pat = pattern_from_rows(rows.cpu().numpy(), L, S)
-    _cache[key] = (pat, mask)
-    while len(_cache) > _CACHE_ENTRIES:
-        _cache.popitem(last=False)
+    _remember(_cache, key, pat, mask)
     return pat
 
 
 _MAX_BATCH = 256
 
 
-def _classify_batched(mask: torch.Tensor):
+def _classify_batched(mask: torch.Tensor, version: int):
     """``classify`` for a mask that depends on the batch (and not on the head): one row summary per
     batch, then ``lens_pattern_from_rows``.  The key counts come back as an int32 device tensor."""
     m = _as_3d(mask)
@@ -185,19 +244,14 @@ def _classify_batched(mask: torch.Tensor):
     B, Lm, S = m.shape
     if B < 1 or Lm < 1 or S < 1:
         return None
-    key = (m.data_ptr(), tuple(m.shape), tuple(m.stride()), m.dtype, mask._version, mask.device.index)
+    key = (m.data_ptr(), tuple(m.shape), tuple(m.stride()), m.dtype, version, mask.device.index)
     sig = (B, Lm, S, m.dtype, mask.device.index)
-    hit = _cache.get(key)
-    if hit is not None:
-        _cache.move_to_end(key)
+    found, pat = _lookup(_cache, key)
+    if found:
         _misses.pop(sig, None)
         stats["hits"] += 1
-        return hit[0]
-    if torch.cuda.is_current_stream_capturing():
-        return None
-    streak = _misses.get(sig, 0)
-    _misses[sig] = streak + 1
-    if streak >= _MAX_MISSES and (streak - _MAX_MISSES) % _RETRY_EVERY != _RETRY_EVERY - 1:
+        return pat
+    if _back_off(sig):
         stats["left_alone"] += 1
         return None
     stats["looked"] += 1
@@ -215,9 +269,7 @@ def _classify_batched(mask: torch.Tensor):
             pat = (pat[0],)  # no padding after all
         else:
             pat = (pat[0], torch.from_numpy(lens).to(mask.device))
-    _cache[key] = (pat, mask)
-    while len(_cache) > _CACHE_ENTRIES:
-        _cache.popitem(last=False)
+    _remember(_cache, key, pat, mask)
     return pat
 
 
@@ -228,29 +280,39 @@ def tile_maps(mask: torch.Tensor, B: int, Hq: int, L: int, S: int):
     """Tile skip tables of a mask that is no pattern (``ops.mask_tile_maps``), cached for as long as
     the tensor is unchanged.  The run-time counterpart of the reference's static tile elimination
     (neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:15-33): one pass over the mask on
-    the device, no trip to the host.  ``None`` for masks too small to matter, masks per key, and
-    inside a graph capture."""
+    the device, no trip to the host.  ``None`` for masks too small to matter, masks per key, tensors
+    without a version counter, inside a graph capture, and for a caller that brings a new tensor on
+    every call (a relative-position bias computed per step, upstream's per-call conversion of a bool
+    mask): after a few misses in a row for one signature such tensors get no tables - a pass over the
+    tensor per call costs more than the tables save - with another try every ``_RETRY_EVERY`` calls.
+    The cache holds the small tables and a weak reference to the mask's storage, never the mask."""
     if not enabled() or mask is None or L < 256 or S < 256 or mask.dim() < 2 or mask.shape[-2] == 1:
         return None
-    if torch.cuda.is_current_stream_capturing():
+    version = _version(mask)
+    if version is None or torch.cuda.is_current_stream_capturing():
         return None
     from . import ops
 
-    key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask.dtype, mask._version, mask.device.index, B, Hq)
-    hit = _tile_cache.get(key)
-    if hit is not None:
-        _tile_cache.move_to_end(key)
+    key = (mask.data_ptr(), tuple(mask.shape), tuple(mask.stride()), mask.dtype, version, mask.device.index, B, Hq)
+    sig = ("tiles", tuple(mask.shape), mask.dtype, mask.device.index)
+    found, maps = _lookup(_tile_cache, key)
+    if found:
+        _misses.pop(sig, None)
         stats["tile_hits"] = stats.get("tile_hits", 0) + 1
-        return hit[0]
+        return maps
+    if _back_off(sig):
+        stats["tile_left_alone"] = stats.get("tile_left_alone", 0) + 1
+        return None
     maps = ops.mask_tile_maps(mask, B, Hq, L, S)
     stats["tile_builds"] = stats.get("tile_builds", 0) + 1
-    _tile_cache[key] = (maps, mask)
-    while len(_tile_cache) > _CACHE_ENTRIES:
-        _tile_cache.popitem(last=False)
+    _remember(_tile_cache, key, maps, mask)
     return maps
 
 
 def clear_cache() -> None:
+    """Forget every verdict and table.  Needed after a mask was changed by anything that does not
+    bump the tensor's version counter (a kernel launched through its data pointer, a graph replay
+    that writes the buffer): only writes through torch ops are seen."""
     _cache.clear()
     _misses.clear()
     _tile_cache.clear()
