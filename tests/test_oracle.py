@@ -395,3 +395,91 @@ def test_window_mask_closed_forms():
         want = {j for j in range(S) if j <= i and (i - j < 3 or j < 2)}
         assert {j for j in range(S) if m[i, j]} == want
     assert om.window_keep_mask(5, 9, 2).sum() == 1 + 2 * 4  # L != S: anchored top-left
+
+
+# ---- score functors, document ids, several sink logits ---------------------------------------------
+# Pinned by the functor written out element by element on a float64 score matrix (a Python loop over
+# heads, rows and keys), float64 softmax with the sink logits as extra columns, and autograd through
+# all of it: a dropped term, a wrong sign of (j - i), a transposed (h, j) index or a missing
+# derivative fails one of the cases below.
+
+
+def _score_mod_reference(q, k, v, scale, causal, window, z, slopes, cap, kb, kw, doc):
+    B, Hq, L, _ = q.shape
+    S, rep = k.shape[2], q.shape[1] // k.shape[1]
+    q64, k64, v64 = (t.double().requires_grad_(True) for t in (q, k, v))
+    z64 = None if z is None else z.double().requires_grad_(True)
+    kk, vv = k64.repeat_interleave(rep, 1), v64.repeat_interleave(rep, 1)
+    heads = []
+    for b in range(B):
+        for h in range(Hq):
+            rows = []
+            for i in range(L):
+                r = []
+                for j in range(S):
+                    s = (q64[b, h, i] * kk[b, h, j]).sum() * scale
+                    if kw is not None:
+                        s = s * kw[h, j].double()
+                    if kb is not None:
+                        s = s + kb[h, j].double()
+                    if slopes is not None:
+                        s = s + slopes[h].double() * (j - i)
+                    if cap:
+                        s = cap * torch.tanh(s / cap)
+                    dead = (causal and j > i) or (window and i - j >= window) or (doc is not None and doc[b, i] != doc[b, j])
+                    r.append(s * 0 + float("-inf") if dead else s)
+                if z64 is not None:
+                    r += [z64[b, h, n] for n in range(z64.shape[2])]
+                rows.append(torch.stack(r))
+            heads.append(torch.stack(rows))
+    full = torch.stack(heads).reshape(B, Hq, L, -1)
+    out = torch.softmax(full, -1)[..., :S] @ vv
+    return out, torch.logsumexp(full, -1), (q64, k64, v64, z64)
+
+
+@pytest.mark.parametrize("case", ["alibi_causal", "head_bias_document", "soft_cap", "weighted", "all_with_sinks", "window_alibi"])
+def test_score_mod_oracle_matches_float64_element_by_element(case):
+    B, Hq, Hkv, L, E = 2, 4, 2, 20, 8
+    g = torch.Generator().manual_seed(31)
+    q, k, v, go = (torch.randn(B, h, L, E, generator=g) for h in (Hq, Hkv, Hkv, Hq))
+    scale = 0.4
+    slopes = torch.exp2(-(torch.arange(Hq) + 1) * 8.0 / Hq)
+    kb, kw = torch.randn(Hq, L, generator=g), torch.rand(Hq, L, generator=g) + 0.5
+    doc = torch.stack([torch.arange(L) // 7, torch.arange(L) // 5])
+    cfg = {
+        "alibi_causal": dict(causal=True, slopes=slopes),
+        "head_bias_document": dict(kb=kb, doc=doc),
+        "soft_cap": dict(cap=2.0),
+        "weighted": dict(kw=kw),
+        "all_with_sinks": dict(causal=True, slopes=slopes, cap=1.5, kb=kb, kw=kw, doc=doc, z=torch.randn(B, Hq, 3, generator=g)),
+        "window_alibi": dict(causal=True, window=6, slopes=slopes, z=torch.randn(B, Hq, 1, generator=g)),
+    }[case]
+    c = dict(causal=False, window=0, z=None, slopes=None, cap=0.0, kb=None, kw=None, doc=None)
+    c.update(cfg)
+    kwargs = dict(is_causal=c["causal"], scale=scale, window=c["window"], sink_logit=c["z"], alibi_slopes=c["slopes"],
+                  softcap=c["cap"], key_bias=c["kb"], key_weight=c["kw"], doc_ids_q=c["doc"], doc_ids_k=c["doc"])
+    out, lse = om.sdpa_forward_score_mod(q, k, v, **kwargs)
+    ro, rl, (q64, k64, v64, z64) = _score_mod_reference(q, k, v, scale, c["causal"], c["window"], c["z"], c["slopes"], c["cap"],
+                                                        c["kb"], c["kw"], c["doc"])
+    assert (out.double() - ro).abs().max() <= 2e-6 and (lse.double() - rl).abs().max() <= 2e-6
+    dq, dk, dv, dz = om.sdpa_backward_score_mod(go, q, k, v, out, lse, **kwargs)
+    wrt = (q64, k64, v64) + ((z64,) if z64 is not None else ())
+    grads = torch.autograd.grad(ro, wrt, go.double())
+    for a, r in zip((dq, dk, dv), grads[:3]):
+        assert (a.double() - r).abs().max() <= 5e-6
+    if z64 is not None:
+        assert dz.shape == c["z"].shape and (dz.double() - grads[3]).abs().max() <= 5e-6
+
+
+def test_score_mod_oracle_reduces_to_the_plain_functor_path():
+    # no score functor, one sink logit: the explicit restatement equals the older one built on compute_attention
+    g = torch.Generator().manual_seed(5)
+    q, k, v, go = (torch.randn(1, h, 33, 16, generator=g) for h in (4, 2, 2, 4))
+    z = torch.randn(1, 4, generator=g)
+    a, la = om.sdpa_forward_score_mod(q, k, v, is_causal=True, window=9, sink_keys=2, sink_logit=z)
+    b, lb = om.sdpa_forward_functor(q, k, v, is_causal=True, window=9, sink_keys=2, sink_logit=z)
+    assert (a - b).abs().max() <= 1e-6 and (la - lb).abs().max() <= 1e-6
+    ga = om.sdpa_backward_score_mod(go, q, k, v, a, la, is_causal=True, window=9, sink_keys=2, sink_logit=z)
+    gb = om.sdpa_backward_functor(go, q, k, v, b, lb, is_causal=True, window=9, sink_keys=2, sink_logit=z)
+    for x, y in zip(ga, gb):
+        assert (x - y).abs().max() <= 2e-6

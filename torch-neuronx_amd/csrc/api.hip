@@ -85,6 +85,10 @@ static bool mask_spec_ok(const mi355_sdpa_mask_spec& m, int is_causal) {
   if (m.window < 0 || m.sink_keys < 0) return set_error("SDPA: window and sink_keys must not be negative"), false;
   if (m.window > 0 && !is_causal) return set_error("SDPA: a sliding window needs is_causal"), false;
   if (m.sink_keys > 0 && m.window == 0) return set_error("SDPA: sink_keys needs a sliding window"), false;
+  if (m.n_sink_logits < 0) return set_error("SDPA: n_sink_logits must not be negative"), false;
+  if ((m.doc_ids_q == nullptr) != (m.doc_ids_k == nullptr))
+    return set_error("SDPA: doc_ids_q and doc_ids_k come together"), false;
+  if (!(m.softcap >= 0.f)) return set_error("SDPA: softcap must not be negative"), false;
   return true;
 }
 

@@ -38,7 +38,9 @@ constexpr int smem_bytes() {  // three Q and three dO tiles, two P hand-over buf
 // as zeros.
 // MASK = 1: per-batch key counts and a bias / bool keep-mask that depends on the key only (a lane
 // is a key: one register);  MASK = 2: a bias / keep-mask with a row per query as well (one element
-// per score, fetched by role A ahead of the tile's matrix ops)
+// per score, fetched by role A ahead of the tile's matrix ops);  MASK = 4: MASK = 1 plus the score
+// functors and document ids of score_mod.h: role A rewrites its score tile in a block of its own
+// and hands P times the derivative of the functors to role B, which forms dS from it.
 template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -50,7 +52,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   uint32_t* const pex = (uint32_t*)(do_t + 3 * TILE);  // [2][4 key blocks][64 lanes][16]
   float* const lse_s = (float*)(pex + 2 * 4 * 1024);   // [3][BQ]
   float* const dl_s = lse_s + 3 * BQ;                  // [3][BQ]
-  uint32_t* const live_s = (uint32_t*)(dl_s + 3 * BQ);  // [heads of the group][words]: query tiles with a kept score (skip table)
+  int32_t* const doc_s = (int32_t*)(dl_s + 3 * BQ);     // [3][BQ] document ids of the tile's rows (MASK = 4)
+  uint32_t* const live_s = (uint32_t*)(dl_s + 3 * BQ);  // [heads of the group][words]: query tiles with a kept score (skip table; MASK = 2)
   uint16_t* const items_s = (uint16_t*)(live_s + 256);  // [1024] live items, and their count behind them
 
   const int streams = p.B * p.Hkv;
@@ -104,12 +107,13 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
 
   // sliding window (masked variant without a per-score bias): rows past the window of the block's last
   // key see none of its keys, unless the block holds sink keys
-  constexpr bool FUNC = MASK == 1;
+  constexpr bool FUNC = MASK == 1 || MASK == 4;
+  constexpr bool SMOD = MASK == 4;  // score functors, document ids
   // MASK = 3 is dropout: the (B, Hq, L, S) keep-mask is fetched like a bool bias by the wavefronts that
   // form the probabilities.  They feed dV with the kept probabilities and hand all of them to the dK
   // wavefronts, the dropped ones with the sign bit set (a probability is never negative): dP is
   // multiplied by keep / (1 - p) there (torch_neuronx/_sdpa_math.py:36-48, :154-158).
-  constexpr bool BIASED = MASK >= 2, DROP = MASK == 3;
+  constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;
   const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
   // the query rows that see this lane's key are first_q .. past_q - 1: from the key itself on under a
   // causal mask, none for a key past the batch's count, up to the end of the key's window unless it is a sink
@@ -117,8 +121,25 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int past_q = (W > 0 && key >= n_sink) ? key + W : INT_MAX;
   const bool listed = MASK == 2 && p.live_t != nullptr;
   const int nqs = (p.L + BQ - 1) / BQ;
-  const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
-  const int qs_end = (W > 0 && k0 >= n_sink) ? max(min(nqs, (k0 + BK + W - 2) / BQ + 1), qs_begin) : nqs;
+  int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+  int qs_end = (W > 0 && k0 >= n_sink) ? max(min(nqs, (k0 + BK + W - 2) / BQ + 1), qs_begin) : nqs;
+  // document ids (MASK = 4): this lane's key id; with ids sorted along the sequence the rows whose id
+  // lies between the ids of the block's first and last key are one run, found by two searches over
+  // doc_q, and only the query tiles that touch it are walked
+  const bool sm_doc = SMOD && p.sm.doc_q && p.sm.doc_k;
+  const int sm_dk = sm_doc ? p.sm.doc_k[(int64_t)b * p.S + max(min(key, S - 1), 0)] : 0;
+  const int sm_dk_first = __builtin_amdgcn_readlane(sm_dk, 0), sm_dk_last = __builtin_amdgcn_readlane(sm_dk, 31);
+  if constexpr (SMOD) {
+    if (sm_doc && p.sm.doc_sorted && k0 < S) {
+      const int32_t* dqr = p.sm.doc_q + (int64_t)b * p.L;
+      const int32_t* dkr = p.sm.doc_k + (int64_t)b * p.S;
+      const int d_lo = dkr[k0], d_hi = dkr[min(k0 + BK, S) - 1];
+      const int r_lo = wave_lower_bound(dqr, p.L, d_lo, lane);
+      const int r_hi = d_hi == INT_MAX ? p.L : wave_lower_bound(dqr, p.L, d_hi + 1, lane);
+      qs_begin = max(qs_begin, r_lo / BQ);
+      qs_end = r_hi > r_lo ? max(min(qs_end, (r_hi + BQ - 1) / BQ), qs_begin) : qs_begin;
+    }
+  }
   const int per_head = qs_end - qs_begin;
   int n_items = (MASK && k0 >= S) ? 0 : rep * per_head;  // no live key in this tile: zeros
   // Items run query tile by query tile from the LAST tile down, the group's heads inside.  The
@@ -159,6 +180,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // row statistics of this batch (written by bwd_delta_kernel): (Hq, L) floats each
   const u32x4 lse_rsrc = descriptor(p.lse2 + (int64_t)b * p.Hq * p.L, (int64_t)p.Hq * p.L * 4);
   const u32x4 dl_rsrc = descriptor(p.delta + (int64_t)b * p.Hq * p.L, (int64_t)p.Hq * p.L * 4);
+  const u32x4 doc_rsrc = descriptor(sm_doc ? p.sm.doc_q + (int64_t)b * p.L : nullptr, sm_doc ? (int64_t)p.L * 4 : 0);
   // The tiles go from global memory straight into LDS (buffer loads with the LDS bit: no trip
   // through registers, no LDS store instructions).  The loads are written as inline assembly: the
   // compiler's own form of them makes it wait for all outstanding loads before the next LDS read
@@ -187,6 +209,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
                  :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
   };
   const uint32_t lds_lse = (uint32_t)(uintptr_t)(lds_bytes)lse_s, lds_dl = (uint32_t)(uintptr_t)(lds_bytes)dl_s;
+  const uint32_t lds_doc = (uint32_t)(uintptr_t)(lds_bytes)doc_s;
   auto row_load = [&](const u32x4& rsrc, uint32_t voffset, uint32_t lds_addr) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tbuffer_load_dword %1, %2, 0 offen lds"
                  :: "s"(__builtin_amdgcn_readfirstlane((int)lds_addr)), "v"(voffset), "s"(rsrc) : "memory", "m0");
@@ -205,6 +228,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       const uint32_t off = (uint32_t)((h * p.L + q0 + lane) * 4);
       row_load(lse_rsrc, off, lds_lse + (uint32_t)(buf * BQ * 4));
       row_load(dl_rsrc, off, lds_dl + (uint32_t)(buf * BQ * 4));
+      if constexpr (SMOD) {
+        if (sm_doc) row_load(doc_rsrc, (uint32_t)((q0 + lane) * 4), lds_doc + (uint32_t)(buf * BQ * 4));
+      }
     }
   };
   // Rows past L of a head's last tile hold another head's rows and statistics (or zeros): they are
@@ -345,6 +371,17 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     constexpr int SPG = 4 / EPS;  // slots per group of four consecutive rows
     load_bias_a(it);
     float bl = 0.f;  // this key's bias in the log2 domain
+    // score functors of this item (MASK = 4): the head's slope, this key's weight and bias
+    const float sm_inv_scale = SMOD ? 1.f / p.scale : 0.f;
+    const float cap_s = SMOD ? p.sm.softcap * sm_inv_scale : 0.f, icap_s = (SMOD && p.sm.softcap > 0.f) ? p.scale / p.sm.softcap : 0.f;
+    float sm_slope = 0.f, sm_w = 1.f, sm_kb = 0.f;
+    if constexpr (SMOD) {
+      const int hh = item_head(it);
+      if (p.sm.alibi) sm_slope = p.sm.alibi[hh] * sm_inv_scale;
+      if (p.sm.key_weight) sm_w = p.sm.key_weight[(int64_t)hh * p.S + min(key, p.S - 1)];
+      if (p.sm.key_bias) sm_kb = p.sm.key_bias[(int64_t)hh * p.S + min(key, p.S - 1)] * sm_inv_scale;
+    }
+    const bool need_dfac = SMOD && (p.sm.key_weight != nullptr || p.sm.softcap > 0.f);
     if constexpr (MASK == 1) {
       if (p.bias_kind)
         bl = bias_value(p.bias, b * p.bias_sb + item_head(it) * p.bias_sh + min(key, p.S - 1), p.bias_kind) * kLog2eF;
@@ -355,7 +392,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;  // [4 groups of 4 words][lane][4]
     f32x16 sc[2];
     uint32_t pk[2][8];
-    uint32_t pkx[DROP ? 2 : 1][8];  // (dropout) what the dK wavefronts get: every probability, the dropped ones negative
+    // what the dK wavefronts get.  Dropout: every probability, the dropped ones negative; score
+    // functors with a derivative other than one: the probability times that derivative
+    uint32_t pkx[(DROP || SMOD) ? 2 : 1][8];
     f32x4 l4[2][4];
     u32x4 ring[8];
     auto load_l4 = [&](int mq, int r4) { l4[mq][r4] = *(const f32x4*)(lrow + mq * 32 + r4 * 8); };
@@ -379,6 +418,37 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
           pk[mq][r >> 1] = Mma<T>::pack(fmaxf(s0, 0.f), fmaxf(s1, 0.f));
         } else {
           pk[mq][r >> 1] = Mma<T>::pack(p0, p1);
+          if constexpr (SMOD) {
+            if (need_dfac) {
+              // the derivative of the functors, from the modified score: 1 - tanh^2 = 1 - (s' / cap)^2
+              // (a masked score, -inf, is clamped to a derivative of 0), times the key's weight
+              const float t0 = __builtin_amdgcn_fmed3f(sc[mq][r] * icap_s, -1.f, 1.f), t1 = __builtin_amdgcn_fmed3f(sc[mq][r + 1] * icap_s, -1.f, 1.f);
+              pkx[mq][r >> 1] = Mma<T>::pack(p0 * (fmaf(-t0, t0, 1.f) * sm_w), p1 * (fmaf(-t1, t1, 1.f) * sm_w));
+            }
+          }
+        }
+      }
+    };
+    // score functors: the raw score tile s becomes mod(scale * s) / scale (lane = key, element r =
+    // row 32 mq + 8 (r / 4) + 4 half + r % 4 of the tile), one block per functor behind a uniform test
+    auto smod_scores = [&](int mq) {
+      if constexpr (SMOD) {
+        if (p.sm.key_weight) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[mq][r] *= sm_w;
+        }
+        if (p.sm.key_bias) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[mq][r] += sm_kb;
+        }
+        if (p.sm.alibi) {
+          const float base = (float)(key - item_q0(it) - mq * 32 - half * 4);
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[mq][r] = fmaf(sm_slope, base - (float)((r >> 2) * 8 + (r & 3)), sc[mq][r]);
+        }
+        if (p.sm.softcap > 0.f) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sc[mq][r] = cap_s * tanh_fast(sc[mq][r] * icap_s);
         }
       }
     };
@@ -389,12 +459,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
         const int qi = q0 + mq * 32 + (r >> 2) * 8 + half * 4 + (r & 3);
         // (one compare or two against per-lane bounds: spelled out as the conditions they stand for,
         // the test is compiled into a cascade of branches per element)
-        const bool dead = FUNC ? (qi < first_q) | (qi >= past_q) : qi < first_q;
+        bool dead = FUNC ? (qi < first_q) | (qi >= past_q) : qi < first_q;
+        if constexpr (SMOD) {
+          if (sm_doc) dead |= doc_s[tb * BQ + mq * 32 + (r >> 2) * 8 + half * 4 + (r & 3)] != sm_dk;
+        }
         sc[mq][r] = dead ? -INFINITY : sc[mq][r];
       }
     };
     auto hand_over = [&](int mq) {
-      const uint32_t(&w)[8] = DROP ? pkx[DROP ? mq : 0] : pk[mq];
+      const uint32_t(&w)[8] = (DROP || (SMOD && need_dfac)) ? pkx[(DROP || SMOD) ? mq : 0] : pk[mq];
       *(u32x4*)(px + (2 * mq) * 256) = u32x4{w[0], w[1], w[2], w[3]};
       *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{w[4], w[5], w[6], w[7]};
     };
@@ -410,6 +483,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     if constexpr (MASK == 2) bias_to_log2(braw);
+    smod_scores(0);
     if (__builtin_expect(edge, 0)) mask_scores(0);
     __builtin_amdgcn_sched_barrier(0);
     // ---- phase 2
@@ -423,6 +497,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       __builtin_amdgcn_sched_barrier(0);
     }
     hand_over(0);
+    smod_scores(1);
     if (__builtin_expect(edge, 0)) mask_scores(1);
     __builtin_amdgcn_sched_barrier(0);
     // ---- phases 3 and 4: operand j = DB * (16-row step) + d block of dO^T
@@ -439,8 +514,21 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
   // every key of this block lies above the diagonal of the tile's rows / past the keys / below their
   // windows, or the mask's skip table says that it keeps no score of the tile's rows and the block's keys
-  auto dead_tile = [&](int it) {
+  // document ids of a tile's first and last row, from the tile's row of ids in LDS
+  auto doc_rows = [&](int it, int tb, int& d_first, int& d_last) {
     const int q0 = item_q0(it);
+    d_first = __builtin_amdgcn_readfirstlane(doc_s[tb * BQ]);
+    d_last = __builtin_amdgcn_readfirstlane(doc_s[tb * BQ + min(BQ, p.L - q0) - 1]);
+  };
+  auto dead_tile = [&](int it, int tb) {
+    const int q0 = item_q0(it);
+    if constexpr (SMOD) {
+      if (sm_doc && p.sm.doc_sorted) {  // the rows' ids and this wavefront's keys' ids do not overlap
+        int d_first, d_last;
+        doc_rows(it, tb, d_first, d_last);
+        if (d_last < sm_dk_first || d_first > sm_dk_last) return true;
+      }
+    }
     if constexpr (MASK == 2) {
       if (listed) {
         const int qt = q0 / BQ;
@@ -452,8 +540,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
   auto role_a = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
-    if (dead_tile(it)) return;
-    const bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
+    if (dead_tile(it, tb)) return;
+    bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
+    if constexpr (SMOD) {
+      if (sm_doc) {  // every score compared, unless the tile's rows and the wavefront's keys all carry one id
+        int d_first = 0, d_last = 1;
+        if (p.sm.doc_sorted) doc_rows(it, tb, d_first, d_last);
+        edge |= !(d_first == d_last && sm_dk_first == sm_dk_last && d_first == sm_dk_first);
+      }
+    }
     role_a_tile(it, tb, pb, edge);
   };
   // Role B splits a tile over two iterations, so that its vector work falls on role A's first
@@ -461,7 +556,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // it, dS and dK of that tile at the start of iteration it + 1.
   f32x16 dp[2];
   auto role_b_scores = [&](int it, int tb) {
-    if (dead_tile(it)) return;
+    if (dead_tile(it, tb)) return;
     scores(do_t + tb * TILE, dp);
   };
   // One tile of role B, pipelined like role A's:
@@ -471,7 +566,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   auto role_b = [&](int it, int tb, int pb) {
     constexpr int EPS = 16 / KS;  // elements per slot (2 or 4)
     constexpr int SPG = 4 / EPS;  // slots per group of four consecutive rows
-    if (dead_tile(it)) return;
+    if (dead_tile(it, tb)) return;
     const uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;
     const uint16_t* qt = q_t + tb * TILE;
     const float* drow = &dl_s[tb * BQ + half * 4];
@@ -657,7 +752,8 @@ __global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
 
 template <typename T, int D, int MASK>
 int launch_t(const BwdM& g, hipStream_t s) {
-  constexpr int kSmemBytes = smem_bytes<D>() + (MASK == 2 ? 1024 + 2048 + 16 : 0);  // (with the skip table's row of the key block and the item list)
+  // (MASK = 2: with the skip table's row of the key block and the item list; MASK = 4: with the document ids of three tiles' rows)
+  constexpr int kSmemBytes = smem_bytes<D>() + (MASK == 2 ? 1024 + 2048 + 16 : MASK == 4 ? 3 * BQ * 4 : 0);
   static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D, MASK>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (attr != hipSuccess) {
@@ -671,6 +767,13 @@ int launch_t(const BwdM& g, hipStream_t s) {
 }
 template <typename T, int D>
 int launch_m(const BwdM& g, hipStream_t s) {
+  if (g.sm.any) {
+    if (g.keep_scale != 0.f || g.bias_kind) {
+      set_error("SDPA: score functors in bwd_dkdv_w32_kernel need a call without bias and dropout");
+      return MI355_SDPA_ERR_UNSUPPORTED;
+    }
+    return launch_t<T, D, 4>(g, s);
+  }
   if (g.keep_scale != 0.f) return launch_t<T, D, 3>(g, s);
   if (g.bias_kind && g.bias_sl != 0) return launch_t<T, D, 2>(g, s);
   return (g.bias_kind || g.kv_lens || g.d_real != D || g.window > 0) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
@@ -733,6 +836,9 @@ int launch_bwd_dkdv_w32(const BwdM& g0, int dtype, int head_dim, hipStream_t s) 
     // the heaviest workgroup (every query tile of its heads) fills all the tile shares
     const int parts_q = g.parts / g.parts_h;
     g.chunk_items = ((g.Hq / g.Hkv / g.parts_h) * ((g.L + BQ - 1) / BQ) + parts_q - 1) / parts_q;
+    // (sorted document ids bound a key block's query tiles in a way that bwd_dkdv_merge_kernel does not
+    // count: every key block then deals its items to all the parts in equal shares)
+    if (g.sm.doc_sorted) g.chunk_items = 0;
   }
   if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 128>(g, s) : launch_m<f16_t, 128>(g, s);
   return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 64>(g, s) : launch_m<f16_t, 64>(g, s);

@@ -29,7 +29,9 @@ constexpr int AHEAD = 2;  // LDS operands are requested this many matrix ops ahe
 
 // MASK = 1: per-batch key counts, and head dims below D (multiples of 8), the missing tail of every
 // row counting as zeros.  MASK = 2: on top, a bias / bool keep-mask (a lane reads its own row of
-// it) and the gradient of the bias.
+// it) and the gradient of the bias.  MASK = 4: MASK = 1 plus the score functors and document ids
+// of score_mod.h, applied to the score tile (and their derivative to dP - delta) in a block of its
+// own ahead of the tile's vector work.
 template <typename T, int D, int MASK>
 __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
@@ -42,7 +44,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // key tiles it walks when the call brings a skip table, and a kernel may declare 64 KB at most)
   // MASK = 3 is dropout: the (B, Hq, L, S) keep-mask is fetched like a bool bias, leaves the scores alone and
   // multiplies dP, together with 1 / (1 - p) (torch_neuronx/_sdpa_math.py:36-48, :154-158)
-  constexpr bool BIASED = MASK >= 2, DROP = MASK == 3;
+  constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;
   constexpr bool DYN = BIASED;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
   __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : NBUF * TILE];
@@ -131,30 +133,55 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   int S = p.S;  // keys of this batch that take part
   if constexpr (MASK) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
-    if (S == 0) {  // no live key: zero gradient
-      zero_gbias(0);
-      if (qrow < p.L) {
-        uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
+  }
+  auto zero_row = [&]() {  // no live key: zero gradient
+    zero_gbias(0);
+    if (qrow < p.L) {
+      uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
-        for (int i = 0; i < D / 16; ++i)
-          if (half * (D / 2) + i * 8 < dr) *(u32x4*)(gq + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
-      }
+      for (int i = 0; i < D / 16; ++i)
+        if (half * (D / 2) + i * 8 < dr) *(u32x4*)(gq + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
+    }
+  };
+  if constexpr (MASK) {
+    if (S == 0) {
+      zero_row();
       return;
     }
   }
   // The key tiles this workgroup walks.  Without a window: 0 .. nt-1.  With one, the tiles below the
   // lowest window of its rows are dropped whole, except the leading ones that hold sink keys: stream
   // position u is key tile u + (u >= n_lead ? skip : 0).
-  constexpr bool FUNC = MASK == 1;
+  constexpr bool FUNC = MASK == 1 || MASK == 4;
+  constexpr bool SMOD = MASK == 4;  // score functors, document ids
   int nt = (S + BN - 1) / BN;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   int n_lead = 0, skip = 0;
   if constexpr (FUNC) {
-    if (p.window > 0) {
-      const int t_lo = max(q0 - p.window + 1, 0) / BN;
-      n_lead = min(min((p.sink_keys + BN - 1) / BN, t_lo), nt);
+    int t_lo = p.window > 0 ? max(q0 - p.window + 1, 0) / BN : 0;
+    if constexpr (SMOD) {
+      // document ids sorted along the sequence: only the run of keys whose id lies between the ids of
+      // this workgroup's first and last row can hold a kept score
+      if (p.sm.doc_sorted) {
+        const int32_t* dqr = p.sm.doc_q + (int64_t)b * p.L;
+        const int32_t* dkr = p.sm.doc_k + (int64_t)b * p.S;
+        const int d_lo = dqr[min(q0, p.L - 1)], d_hi = dqr[min(q0 + BM, p.L) - 1];
+        const int k_lo = wave_lower_bound(dkr, S, d_lo, lane);
+        const int k_hi = d_hi == INT_MAX ? S : wave_lower_bound(dkr, S, d_hi + 1, lane);
+        nt = k_hi > k_lo ? min(nt, (k_hi + BN - 1) / BN) : 0;
+        t_lo = max(t_lo, k_lo / BN);
+      }
+    }
+    if (t_lo > 0) {
+      n_lead = min(min(p.window > 0 ? (p.sink_keys + BN - 1) / BN : 0, t_lo), nt);
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
+    }
+    if constexpr (SMOD) {
+      if (nt <= 0) {  // (the document ids leave this workgroup's rows without a key)
+        zero_row();
+        return;
+      }
     }
   }
   // With a skip table (variant with a bias, no bias gradient): the tiles in which the mask keeps at
@@ -298,6 +325,73 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
 
+  // Score functors and document ids (MASK = 4): the raw score tile s becomes mod(scale * s) / scale
+  // and dP becomes delta + (dP - delta) * mod'(scale * s), so that the common code behind them forms
+  // P from the modified score and dS = P (dP - delta) mod'.  Lane = query row, element r = key
+  // 8 (r / 4) + 4 half + r % 4 of the tile; one block per functor behind a uniform test.
+  const float sm_inv_scale = SMOD ? 1.f / p.scale : 0.f;
+  const float sm_slope = (SMOD && p.sm.alibi) ? p.sm.alibi[h] * sm_inv_scale : 0.f;
+  const float* const sm_kb = (SMOD && p.sm.key_bias) ? p.sm.key_bias + (int64_t)h * p.S : nullptr;
+  const float* const sm_kw = (SMOD && p.sm.key_weight) ? p.sm.key_weight + (int64_t)h * p.S : nullptr;
+  const int32_t* const sm_dk = (SMOD && p.sm.doc_q && p.sm.doc_k) ? p.sm.doc_k + (int64_t)b * p.S : nullptr;
+  // (this row's id is read again where a tile is compared element by element, rather than kept in a
+  // register across the loop: such tiles are the few that straddle a document boundary)
+  auto my_doc = [&]() { return sm_dk ? p.sm.doc_q[(int64_t)b * p.L + qc] : 0; };
+  const int sm_dq0 = __builtin_amdgcn_readfirstlane(my_doc());
+  const bool sm_dq_uniform = SMOD && p.sm.doc_sorted && __builtin_amdgcn_ballot_w64(my_doc() != sm_dq0) == 0;
+  auto apply_smod = [&](f32x16& sv, f32x16& dpv, int ta) {
+    if constexpr (SMOD) {
+      const int kvb = ta * BN + half * 4;
+      // this lane's 16 values of a vector per key (a tile that ends within the keys reads them at
+      // constant offsets from one address; a ragged last tile clamps every index)
+      auto load_keys = [&](const auto* row, auto (&val)[16]) {
+        if (ta * BN + BN <= p.S) {
+          const auto* at = row + kvb;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) val[r] = at[(r >> 2) * 8 + (r & 3)];
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) val[r] = row[min(kvb + (r >> 2) * 8 + (r & 3), p.S - 1)];
+        }
+      };
+      if (sm_kw) {
+        float w[16];
+        load_keys(sm_kw, w);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] *= w[r], dpv[r] = fmaf(dpv[r] - dl, w[r], dl);
+      }
+      if (sm_kb) {
+        float kb[16];
+        load_keys(sm_kb, kb);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf(kb[r], sm_inv_scale, sv[r]);
+      }
+      if (p.sm.alibi) {
+        const float base = (float)(kvb - qrow);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf(sm_slope, base + (float)((r >> 2) * 8 + (r & 3)), sv[r]);
+      }
+      if (p.sm.softcap > 0.f) {
+        const float cap_s = p.sm.softcap * sm_inv_scale, icap_s = p.scale / p.sm.softcap;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float th = tanh_fast(sv[r] * icap_s);
+          sv[r] = cap_s * th, dpv[r] = fmaf(dpv[r] - dl, fmaf(-th, th, 1.f), dl);
+        }
+      }
+      if (sm_dk) {
+        const bool whole = sm_dq_uniform && sm_dk[min(ta * BN, p.S - 1)] == sm_dq0 && sm_dk[min(ta * BN + BN - 1, p.S - 1)] == sm_dq0;
+        if (!whole) {
+          int id[16];
+          load_keys(sm_dk, id);
+          const int mine = my_doc();
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sv[r] = id[r] != mine ? -INFINITY : sv[r];
+        }
+      }
+    }
+  };
+
   // S^T and dP^T of the tile in buffer `buf`: operand i = 2 * contraction step + (0: K rows, 1: V rows)
   auto scores = [&](int buf, f32x16& sacc, f32x16& dpacc) {
     u32x4 ring[8];
@@ -394,7 +488,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // dS^T of tile t, packed as the B operand of dQ^T += K^T dS^T
   auto softmax = [&](int u, const f32x16& sacc, const f32x16& dpacc, uint32_t (&pS)[8]) {
     const int t = tile_of(u);  // (stream position -> key tile)
-    const bool edge = t >= t_edge;
+    const bool edge = SMOD ? edge_tile(u) : t >= t_edge;
     float bl[16];
     if constexpr (MASK == 2) bias_log2(bl);
     // (the test for a tile that needs masking stays outside the unrolled loop: inside, the compiler
@@ -411,7 +505,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
           else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
           if constexpr (EDGE) {
             const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
-            pr = kv > lim ? 0.f : pr;
+            // (bitwise on purpose: with || and && every element gets a cascade of branches)
+            const bool dead = SMOD ? (kv > lim) | ((kv < lo_w) & (kv >= n_sink)) : kv > lim;
+            pr = dead ? 0.f : pr;
           }
           if constexpr (DROP) {
             const float keep = (float)((braw[(r + e) >> 2] >> (8 * ((r + e) & 3))) & 0xffu);
@@ -458,7 +554,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   __syncthreads();
   load_tile(2);
   f32x16 s_a, dp_a, s_b, dp_b;
-  if (!BIASED && nt_w > 0) scores(0, s_a, dp_a);
+  if (!BIASED && !SMOD && nt_w > 0) scores(0, s_a, dp_a);
   auto iteration = [&](int t, auto tile_mod, f32x16& scur, f32x16& dpcur, f32x16& snext, f32x16& dpnext) {
     // (t % 4 is a compile-time constant, four copies of the iteration: the buffer of a tile then is
     // an immediate offset of the LDS reads, not an addition on the vector unit per read)
@@ -473,6 +569,14 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
         uint32_t pS[8];
         fetch_bias();
         load_bias(t + 1);
+        softmax(t, scur, dpcur, pS);
+        accumulate(buf, pS);
+      } else if constexpr (SMOD) {
+        // (the functor variant keeps one score tile, like the variant with a bias: a second one does
+        // not fit next to the functors' operands at head dim 128)
+        scores(buf, scur, dpcur);
+        apply_smod(scur, dpcur, tile_of(t));
+        uint32_t pS[8];
         softmax(t, scur, dpcur, pS);
         accumulate(buf, pS);
       } else {
@@ -579,10 +683,14 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
   const dim3 grid((unsigned)blocks), block(512);
   const bool bf = dtype == MI355_SDPA_BF16;
-  const int mask = g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
+  if (g.sm.any && (g.keep_scale != 0.f || g.bias_kind || g.gbias)) {
+    set_error("SDPA: score functors in bwd_dq_w32_kernel need a call without bias and dropout");
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  const int mask = g.sm.any ? 4 : g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
   // (the tiles, the tile list of a call with a skip table, 4 KB of bias tile per wavefront)
-  const int dyn = mask >= 2 ? 2 * 4 * BN * head_dim * 2 + 2080 + 8 * 4096 : 0;
-  if (mask >= 2) {
+  const int dyn = (mask == 2 || mask == 3) ? 2 * 4 * BN * head_dim * 2 + 2080 + 8 * 4096 : 0;
+  if (mask == 2 || mask == 3) {
     const void* fn2 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 2>)
                                       : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 2>);
     const void* fn3 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 3> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 3>)
@@ -594,10 +702,11 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
       return MI355_SDPA_ERR_LAUNCH;
     }
   }
-#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, (MM) >= 2 ? dyn : 0, s, g)
+#define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, ((MM) == 2 || (MM) == 3) ? dyn : 0, s, g)
 #define LAUNCH_M(TT, DD)                                                     \
   do {                                                                       \
-    if (mask == 3) LAUNCH(TT, DD, 3);                                        \
+    if (mask == 4) LAUNCH(TT, DD, 4);                                        \
+    else if (mask == 3) LAUNCH(TT, DD, 3);                                   \
     else if (mask == 2) LAUNCH(TT, DD, 2);                                   \
     else if (mask == 1) LAUNCH(TT, DD, 1);                                   \
     else LAUNCH(TT, DD, 0);                                                  \

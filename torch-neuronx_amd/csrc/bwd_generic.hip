@@ -11,6 +11,7 @@
 // `out` (the two P-dependent parts cancel), so delta is taken from the `out` that is passed.
 // A query row with lse = -inf contributes nothing; keys at or past kv_lens[b] get zero grads.
 #include "common.h"
+#include "score_mod.h"
 
 namespace mi355 {
 namespace {
@@ -30,7 +31,28 @@ struct BwdG {
   int causal, bias_kind;
   float scale;
   int window, sink_keys;  // sliding window over the causal pattern: keys i-window+1 .. i and the first sink_keys
+  ScoreMod sm;            // score functors and document ids
 };
+
+// score functors on s = scale * q.k of (head h, query i, key j); `dfac` receives the derivative of
+// the chain with respect to s, which multiplies the gradient of the scores; a score that the
+// document ids drop comes back as -inf
+__device__ __forceinline__ float score_mod_generic(const BwdG& p, float s, int b, int h, int i, int j, float& dfac) {
+  dfac = 1.f;
+  if (!p.sm.any) return s;
+  if (p.sm.key_weight) {
+    const float w = p.sm.key_weight[(int64_t)h * p.S + j];
+    s *= w, dfac = w;
+  }
+  if (p.sm.key_bias) s += p.sm.key_bias[(int64_t)h * p.S + j];
+  if (p.sm.alibi) s = fmaf(p.sm.alibi[h], (float)(j - i), s);
+  if (p.sm.softcap > 0.f) {
+    const float th = tanhf(s / p.sm.softcap);
+    s = p.sm.softcap * th, dfac *= 1.f - th * th;
+  }
+  if (p.sm.doc_q && p.sm.doc_k && p.sm.doc_q[(int64_t)b * p.L + i] != p.sm.doc_k[(int64_t)b * p.S + j]) s = -INFINITY;
+  return s;
+}
 
 template <typename TB>
 __device__ __forceinline__ float apply_bias(float s, const TB* row, int64_t off, int kind) {
@@ -94,25 +116,28 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_row_kernel(BwdG p) {
 
   for (int j0 = 0; j0 < p.S; j0 += 64) {
     const int j = j0 + lane;
-    float dlog = 0.f;
+    float dlog = 0.f, dmod = 1.f;  // gradient of the modified score; derivative of the score functors
     if (j < s_end) {
       const T* kr = kbase + j * p.k.st[2];
       const T* vr = vbase + j * p.v.st[2];
       float dot = 0.f, dp = 0.f;
       for (int e = 0; e < p.E; ++e) dot = fmaf(qrow[wave][e], to_f32(kr[e * p.k.st[3]]), dot);
       for (int d = 0; d < p.Dv; ++d) dp = fmaf(dorow[wave][d], to_f32(vr[d * p.v.st[3]]), dp);
-      const float s = apply_bias<TB>(dot * p.scale, bias_row, j * p.bias.st[3], p.bias_kind);
+      float dfac;
+      const float sm = score_mod_generic(p, dot * p.scale, b, h, i, j, dfac);
+      const float s = apply_bias<TB>(sm, bias_row, j * p.bias.st[3], p.bias_kind);
       float pr = expf(s - lse);
       if (p.window > 0 && i - j >= p.window && j >= p.sink_keys) pr = 0.f;
       if (keep_row) dp = keep_row[j] ? dp * p.keep_scale : 0.f;
       dlog = pr * (dp - delta);
+      dmod = dfac;
     }
     if (gb_row && j < p.S) gb_row[j * p.gbias.st[3]] = (T)dlog;
     if (j0 >= s_end) {
       if (!gb_row) break;
       continue;
     }
-    const float ds = dlog * p.scale;
+    const float ds = dlog * dmod * p.scale;
     const int jn = min(64, s_end - j0);
     for (int jj = 0; jj < jn; ++jj) {
       const float dj = __shfl(ds, jj, 64);
@@ -178,7 +203,8 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_col_kernel(BwdG p) {
             float dot = 0.f, dp = 0.f;
             for (int e = 0; e < p.E; ++e) dot = fmaf(krow[wave][e], to_f32(qr[e * p.q.st[3]]), dot);
             for (int d = 0; d < p.Dv; ++d) dp = fmaf(vrow[wave][d], to_f32(gr[d * p.go.st[3]]), dp);
-            float s = dot * p.scale;
+            float dfac;
+            float s = score_mod_generic(p, dot * p.scale, b, h, i, j, dfac);
             if (p.bias_kind) {
               const TB* brow = (const TB*)p.bias.data + b * p.bias.st[0] + h * p.bias.st[1] + i * p.bias.st[2];
               s = apply_bias<TB>(s, brow, j * p.bias.st[3], p.bias_kind);
@@ -187,7 +213,7 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_col_kernel(BwdG p) {
             float keepf = 1.f;
             if (p.keep)
               keepf = p.keep[(((int64_t)b * p.Hq + h) * p.L + i) * (int64_t)p.S + j] ? p.keep_scale : 0.f;
-            ds = pr * (dp * keepf - delta[i]) * p.scale;
+            ds = pr * (dp * keepf - delta[i]) * dfac * p.scale;
             pr *= keepf;
           }
         }
@@ -221,10 +247,10 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_col_kernel(BwdG p) {
 // Gradient of the sink logit z of one (batch, head): the sink's probability in row i is
 // exp(z - lse_i) and its dP is 0 (it carries no value), so d z = - sum_i exp(z - lse_i) delta_i.
 // One workgroup per (batch, head), summed in a fixed order.
-__global__ __launch_bounds__(256) void sink_grad_kernel(const float* lse, const float* delta, const float* z, float* out, int L) {
+__global__ __launch_bounds__(256) void sink_grad_kernel(const float* lse, const float* delta, const float* z, float* out, int L, int n_sinks) {
   __shared__ float part[256];
-  const int bh = blockIdx.x;
-  const float zz = z[bh];
+  const int bh = blockIdx.x / n_sinks;  // (one workgroup per sink logit: each has its own probability exp(z_n - lse_i))
+  const float zz = z[blockIdx.x];
   float s = 0.f;
   for (int i = threadIdx.x; i < L; i += 256) {
     const float l = lse[(int64_t)bh * L + i];
@@ -236,7 +262,7 @@ __global__ __launch_bounds__(256) void sink_grad_kernel(const float* lse, const 
     if ((int)threadIdx.x < o) part[threadIdx.x] += part[threadIdx.x + o];
     __syncthreads();
   }
-  if (threadIdx.x == 0) out[bh] = part[0];
+  if (threadIdx.x == 0) out[blockIdx.x] = part[0];
 }
 
 template <typename T, typename TB>
@@ -268,9 +294,10 @@ int launch_t(const BwdG& g, int bias_dtype, hipStream_t s) {
 }  // namespace
 
 int launch_sink_grad(const float* lse, const float* delta, const float* sink_logit, float* grad, int64_t heads, int L,
-                     hipStream_t s) {
+                     int n_sinks, hipStream_t s) {
   if (heads == 0) return MI355_SDPA_OK;
-  hipLaunchKernelGGL(sink_grad_kernel, dim3((unsigned)heads), dim3(256), 0, s, lse, delta, sink_logit, grad, L);
+  n_sinks = n_sinks > 0 ? n_sinks : 1;
+  hipLaunchKernelGGL(sink_grad_kernel, dim3((unsigned)(heads * n_sinks)), dim3(256), 0, s, lse, delta, sink_logit, grad, L, n_sinks);
   return check_launch("sink_grad_kernel");
 }
 
@@ -291,6 +318,7 @@ int launch_bwd_generic(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.causal = p.is_causal, g.scale = p.scale;
   g.bias_kind = !p.bias.data ? 0 : (p.bias_dtype == MI355_SDPA_BOOL ? 2 : 1);
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
+  g.sm = score_mod_of(p.mask);
   if (g.E > kMaxHeadDim || g.Dv > kMaxHeadDim) {
     set_error("SDPA: head dim %d/%d exceeds the supported maximum %d", g.E, g.Dv, kMaxHeadDim);
     return MI355_SDPA_ERR_UNSUPPORTED;
@@ -305,7 +333,7 @@ int launch_bwd_generic(const mi355_sdpa_bwd_params& p, hipStream_t s) {
       return MI355_SDPA_ERR_INVALID;
   }
   if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
-    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
+    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, p.mask.n_sink_logits, s);
   return rc;
 }
 

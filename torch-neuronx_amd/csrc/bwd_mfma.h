@@ -2,6 +2,7 @@
 #pragma once
 
 #include "mfma_common.h"
+#include "score_mod.h"
 
 namespace mi355 {
 
@@ -44,6 +45,8 @@ struct BwdM {
   // sliding window (causal calls, masked variants without a per-score bias): query i sees keys
   // i-window+1 .. i and the first sink_keys keys; tiles that the window drops whole are skipped
   int window = 0, sink_keys = 0;
+  // score functors and document ids (the functor variants of bwd_dq_w32.hip and bwd_dkdv_w32.hip)
+  ScoreMod sm;
   // tile skip table of a per-score bias / keep-mask for the dK/dV kernel: per (mask batch, mask head,
   // block of 128 keys) a bitmap of the 64-row query tiles with a kept score, live_t_words words each;
   // live_hm = the mask's own head extent

@@ -478,7 +478,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   constexpr int RPB = 256 / (D / 8);
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D || g.window > 0) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
+  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D || g.window > 0 || g.sm.any) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
   int rc;
   if (dq_w32) {
     // that kernel holds every row of dO in registers anyway: it goes first and leaves the row
@@ -532,6 +532,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
+  g.sm = score_mod_of(p.mask);
   if (p.grad_bias.data) {
     g.gbias = p.grad_bias.data;
     g.gbias_sb = p.grad_bias.stride[0], g.gbias_sh = p.grad_bias.stride[1], g.gbias_sl = p.grad_bias.stride[2];
@@ -568,8 +569,11 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   // head dims above 128 and D_qk != D_v: the kernels of bwd_wide.hip, which take key counts and a
   // bias / keep-mask, but no bias gradient and no window
   const bool wide = E > 128 || Dv != E;
-  if (wide && (p.grad_bias.data || p.mask.window > 0))
-    return *why = "bias gradient or window with a head dim above 128 or D_qk != D_v", false;
+  const bool smod = score_mod_of(p.mask).any;
+  if (wide && (p.grad_bias.data || p.mask.window > 0 || smod))
+    return *why = "bias gradient, window or score functor with a head dim above 128 or D_qk != D_v", false;
+  if (smod && (p.bias.data || p.grad_bias.data || p.dropout_p > 0.f))
+    return *why = "score functor together with attn_bias or dropout", false;
   const bool padded = E != 64 && E != 128;  // served by the next wider kernels' masked variants
   if (p.grad_bias.data) {  // written by the dQ kernel four keys (8 bytes) at a time
     const int64_t S = p.k.size[2];
@@ -615,7 +619,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
       if (t->size[i] > 1 && (t->stride[i] % 8) != 0) return *why = "stride not a multiple of 8 elements", false;
   }
   if ((int64_t)p.q.size[0] * p.q.size[1] * ((p.q.size[2] + 127) / 128) > 0x7fffffff) return *why = "too many tiles", false;
-  if (!wide && (p.bias.data || p.kv_lens || padded || p.mask.window > 0 || p.dropout_p > 0.f)) {
+  if (!wide && (p.bias.data || p.kv_lens || padded || p.mask.window > 0 || p.dropout_p > 0.f || smod)) {
     BwdM g;
     fill(g, p);
     const int D = E <= 64 ? 64 : 128;
@@ -666,7 +670,7 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   // (a sink logit changes nothing in these kernels: the probabilities come from the saved
   // log-sum-exp, which includes it; only its own gradient is one more small reduction)
   if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
-    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
+    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, p.mask.n_sink_logits, s);
   return rc;
 }
 

@@ -21,8 +21,9 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s);
 bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why);
 size_t bwd_generic_workspace(const mi355_sdpa_bwd_params& p);
 // d sink_logit = - sum_i exp(sink_logit - lse_i) delta_i per (batch, head); lse natural log, delta = rowsum(dO * O)
+// (n_sinks logits per head, each with a gradient of its own)
 int launch_sink_grad(const float* lse, const float* delta, const float* sink_logit, float* grad, int64_t heads, int L,
-                     hipStream_t s);
+                     int n_sinks, hipStream_t s);
 size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p);
 // float32 inputs on the float32 matrix op (f32_mfma.hip)
 bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why);

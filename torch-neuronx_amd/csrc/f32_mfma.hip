@@ -466,7 +466,7 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.mask.window > 0 || p.mask.sink_logit) return *why = "mask functors", false;
+  if (p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "mask / score functors", false;
   if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
   if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
@@ -522,7 +522,7 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.grad_bias.data || p.mask.window > 0) return *why = "bias gradient or window", false;
+  if (p.grad_bias.data || p.mask.window > 0 || score_mod_of(p.mask).any) return *why = "bias gradient, window or score functor", false;
   if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
   if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
@@ -589,7 +589,7 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
 #undef LAUNCH
   rc = check_launch("bwd_f32_dkdv_kernel");
   if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
-    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, s);
+    rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, p.mask.n_sink_logits, s);
   return rc;
 }
 

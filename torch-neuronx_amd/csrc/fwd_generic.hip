@@ -9,6 +9,7 @@
 // with no live key gives a zero output row and lse = -inf, and for half-precision inputs
 // the probabilities are rounded to the input dtype before they multiply V.
 #include "common.h"
+#include "score_mod.h"
 
 namespace mi355 {
 namespace {
@@ -26,7 +27,9 @@ struct FwdG {
   int causal, bias_kind;  // 0 none, 1 additive, 2 bool
   float scale;
   int window, sink_keys;    // sliding window over the causal pattern: keys i-window+1 .. i and the first sink_keys
-  const float* sink_logit;  // (B,Hq): a logit without a value that joins every row's softmax
+  const float* sink_logit;  // (B,Hq,n_sinks): logits without a value that join every row's softmax
+  int n_sinks;
+  ScoreMod sm;  // score functors and document ids
 };
 
 template <typename T, typename TB>
@@ -73,6 +76,13 @@ __global__ __launch_bounds__(64 * kWaves) void fwd_generic_kernel(FwdG p) {
       float dot = 0.f;
       for (int e = 0; e < p.E; ++e) dot = fmaf(qrow[wave][e], to_f32(kr[e * p.k.st[3]]), dot);
       s = dot * p.scale;
+      if (p.sm.any) {
+        if (p.sm.key_weight) s *= p.sm.key_weight[(int64_t)h * p.S + j];
+        if (p.sm.key_bias) s += p.sm.key_bias[(int64_t)h * p.S + j];
+        if (p.sm.alibi) s = fmaf(p.sm.alibi[h], (float)(j - i), s);
+        if (p.sm.softcap > 0.f) s = p.sm.softcap * tanhf(s / p.sm.softcap);
+        if (p.sm.doc_q && p.sm.doc_k && p.sm.doc_q[(int64_t)b * p.L + i] != p.sm.doc_k[(int64_t)b * p.S + j]) s = -INFINITY;
+      }
       if (p.window > 0 && i - j >= p.window && j >= p.sink_keys) s = -INFINITY;
       if (p.bias_kind == 1) {
         s += to_f32(bias_row[j * p.bias.st[3]]);
@@ -105,7 +115,12 @@ __global__ __launch_bounds__(64 * kWaves) void fwd_generic_kernel(FwdG p) {
   }
 
   if (p.sink_logit) {
-    const float z = p.sink_logit[(int64_t)b * p.Hq + h];
+    // (several sink logits act as one: the logarithm of the sum of their exponentials)
+    const float* zs = p.sink_logit + ((int64_t)b * p.Hq + h) * p.n_sinks;
+    float zm = -INFINITY, zl = 0.f;
+    for (int n = 0; n < p.n_sinks; ++n) zm = fmaxf(zm, zs[n]);
+    for (int n = 0; n < p.n_sinks; ++n) zl += zm == -INFINITY ? 0.f : expf(zs[n] - zm);
+    const float z = zm == -INFINITY ? -INFINITY : zm + logf(zl);
     if (z != -INFINITY) {
       const float m2 = fmaxf(m, z);
       const float a = m == -INFINITY ? 0.f : expf(m - m2);
@@ -156,6 +171,8 @@ int launch_fwd_generic(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.causal = p.is_causal, g.scale = p.scale;
   g.bias_kind = !p.bias.data ? 0 : (p.bias_dtype == MI355_SDPA_BOOL ? 2 : 1);
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
+  g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
+  g.sm = score_mod_of(p.mask);
   if (g.E > kMaxHeadDim || g.Dv > kMaxHeadDim) {
     set_error("SDPA: head dim %d/%d exceeds the supported maximum %d", g.E, g.Dv, kMaxHeadDim);
     return MI355_SDPA_ERR_UNSUPPORTED;

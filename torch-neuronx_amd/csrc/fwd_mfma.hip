@@ -338,7 +338,7 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const bool w32_only = padded || E > 128;
   // masked calls (bias, bool keep-mask, per-batch key counts) and padded head dims: the kernels
   // with 32-bit row addressing only, and a bias whose rows can be read four keys at a time
-  if (p.bias.data || p.kv_lens || w32_only || p.mask.window > 0 || p.mask.sink_logit) {
+  if (p.bias.data || p.kv_lens || w32_only || p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) {
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
       return *why = "attn_bias / kv_lens / padded head dim with rows beyond 32-bit offsets", false;
   }
@@ -358,7 +358,7 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   if (p.dropout_p > 0.f) {
     // the keep-mask takes the bias's way into the kernel (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
-    if (p.bias.data || p.mask.window > 0 || p.mask.sink_logit) return *why = "dropout together with attn_bias or a window / sink functor", false;
+    if (p.bias.data || p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "dropout together with attn_bias or a functor", false;
     if (E > 128) return *why = "dropout with a head dim above 128", false;
     if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
     if (32 * S >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
@@ -367,8 +367,8 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   }
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
-  if ((p.mask.window > 0 || p.mask.sink_logit) && (p.bias.data || E > 128))
-    return *why = "window / sink functor together with attn_bias or a head dim above 128", false;
+  if ((p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) && (p.bias.data || E > 128))
+    return *why = "window / sink / score functor together with attn_bias or a head dim above 128", false;
   if (p.q.stride[3] != 1 || p.k.stride[3] != 1 || p.v.stride[3] != 1 || p.out.stride[3] != 1)
     return *why = "head dim is not unit-stride", false;
   const mi355_sdpa_tensor* ts[4] = {&p.q, &p.k, &p.v, &p.out};
@@ -413,6 +413,8 @@ static int launch_or_size(const mi355_sdpa_fwd_params& p, hipStream_t s, size_t*
   }
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
+  g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
+  g.sm = score_mod_of(p.mask);
   if (p.bias.data && p.mask.live_tiles && !p.is_causal && g.S <= 32768 && p.bias.stride[2] != 0) {
     g.live_tiles = p.mask.live_tiles;
     g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);

@@ -48,6 +48,9 @@ constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescale
 // scores, the row sums and the lse alone and zeroes the dropped probabilities where they are packed
 // for the second product; 1 / (1 - p) is applied with the final normalisation
 // (torch_neuronx/_sdpa_math.py:36-48: the mask multiplies the normalised probabilities).
+// MASK = 4 is MASK = 1 plus the score functors and document ids of score_mod.h (head dims up to 128):
+// they rewrite the raw score tile in a block of its own right after the matrix ops that produce it,
+// where the bias of MASK = 2 is folded in, so the softmax behind them is the common code.
 template <typename T, int D, int WAVES, int MASK>
 __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
@@ -60,12 +63,13 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // (head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare:
   // they take the launch's dynamic LDS instead; head dim 256 runs one wavefront per SIMD with the
   // 512-register budget)
-  constexpr bool BIASED = MASK >= 2, DROP = MASK == 3;  // a per-score tensor in LDS; ... that is a dropout keep-mask
+  constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;  // a per-score tensor in LDS; ... that is a dropout keep-mask
   constexpr bool DYN = D > 128 || BIASED;
   // Tiles go from global memory straight into LDS (see the staging section): four unpadded,
   // swizzled buffers per operand, tile t in buffer t % 4.
   // mask functors (window, sink keys, sink logit): in the masked variant without a bias, head dim <= 128
-  constexpr bool FUNC = MASK == 1 && D <= 128;
+  constexpr bool FUNC = (MASK == 1 || MASK == 4) && D <= 128;
+  constexpr bool SMOD = MASK == 4;  // score functors, document ids
   constexpr int NBUF = 4, TILE = BN * D;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
   __shared__ __attribute__((aligned(16))) uint16_t v_static[DYN ? 8 : NBUF * TILE];
@@ -82,7 +86,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   int b, h, qt;
   int wrow = wave * 32;  // this wavefront's first row within the workgroup's rows
   int split = 0;  // (grouped calls with split keys: which part of them)
-  if (MASK <= 2 && p.grouped) {  // (see FwdM::grouped)
+  if (MASK != 3 && p.grouped) {  // (see FwdM::grouped)
     const int rep = p.Hq / p.Hkv, hpw = p.grouped, chunks = rep / hpw;  // heads per workgroup, workgroups per kv head
     const int bhc = blockIdx.x / p.n_split;
     split = blockIdx.x % p.n_split;
@@ -129,9 +133,23 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   int n_lead = 0, skip = 0;
   if constexpr (FUNC) {
-    if (p.window > 0) {
-      const int t_lo = max(q0 - p.window + 1, 0) / BN;
-      n_lead = min(min((p.sink_keys + BN - 1) / BN, t_lo), nt);
+    int t_lo = p.window > 0 ? max(q0 - p.window + 1, 0) / BN : 0;
+    if constexpr (SMOD) {
+      // Document ids that are sorted along the sequence: the keys whose id lies between the ids of
+      // this workgroup's first and last row are one run, found by two searches over doc_k; the tiles
+      // outside it hold no kept score and are not walked.
+      if (p.sm.doc_sorted) {
+        const int32_t* dqr = p.sm.doc_q + (int64_t)b * p.L;
+        const int32_t* dkr = p.sm.doc_k + (int64_t)b * p.S;
+        const int d_lo = dqr[min(q0, p.L - 1)], d_hi = dqr[min(q0 + BM, p.L) - 1];
+        const int k_lo = wave_lower_bound(dkr, S, d_lo, lane);
+        const int k_hi = d_hi == INT_MAX ? S : wave_lower_bound(dkr, S, d_hi + 1, lane);
+        nt = k_hi > k_lo ? min(nt, (k_hi + BN - 1) / BN) : 0;
+        t_lo = max(t_lo, k_lo / BN);
+      }
+    }
+    if (t_lo > 0) {
+      n_lead = min(min(p.window > 0 ? (p.sink_keys + BN - 1) / BN : 0, t_lo), nt);
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
     }
@@ -175,6 +193,15 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       nt = n_live;
     }
   }
+  // the sink logits of this (batch, head) as one: the logarithm of the sum of their exponentials
+  auto sink_lse = [&]() {
+    const float* zs = p.sink_logit + ((int64_t)b * p.Hq + h) * p.n_sinks;
+    float zm = -INFINITY, zl = 0.f;
+    for (int n = 0; n < p.n_sinks; ++n) zm = fmaxf(zm, zs[n]);
+    if (zm == -INFINITY) return -INFINITY;
+    for (int n = 0; n < p.n_sinks; ++n) zl += __expf(zs[n] - zm);
+    return zm + __builtin_logf(zl);
+  };
   auto tile_of = [&](int u) {
     if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u + skip;
     else return FUNC ? u + (u >= n_lead ? skip : 0) : SPLITS ? u + skip : u;  // (head dim 256: split keys, no window)
@@ -193,7 +220,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
         for (int i = 0; i < D / 16; ++i)
           if (half * (D / 2) + i * 8 < drv) *(u32x4*)(orow + half * (D / 2) + i * 8) = u32x4{0u, 0u, 0u, 0u};
         if (p.lse && half == 0)
-          p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = (FUNC && p.sink_logit) ? p.sink_logit[(int64_t)b * p.Hq + h] : -INFINITY;
+          p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = (FUNC && p.sink_logit) ? sink_lse() : -INFINITY;
       }
       return;
     }
@@ -453,6 +480,73 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   };
 
+  // Score functors and document ids (MASK = 4): the raw score tile s (lane = query row, element r =
+  // key 8 (r / 4) + 4 half + r % 4 of the tile) becomes mod(scale * s) / scale, so that everything
+  // behind it - reference tracking, exp2 with the scale folded in, lse - is the common code.  Each
+  // functor is a block of its own behind a uniform test.  The captured vectors are read with plain
+  // loads (the wait in front of their use also covers the tile loads in flight: the price of a
+  // functor that needs a vector per key); a document mask over sorted ids tests a whole tile with two
+  // loads and compares element by element only in the tiles that straddle a document boundary.
+  const float sm_inv_scale = SMOD ? 1.f / p.scale : 0.f;
+  const float sm_slope = (SMOD && p.sm.alibi) ? p.sm.alibi[h] * sm_inv_scale : 0.f;
+  const float* const sm_kb = (SMOD && p.sm.key_bias) ? p.sm.key_bias + (int64_t)h * p.S : nullptr;
+  const float* const sm_kw = (SMOD && p.sm.key_weight) ? p.sm.key_weight + (int64_t)h * p.S : nullptr;
+  const int32_t* const sm_dk = (SMOD && p.sm.doc_q && p.sm.doc_k) ? p.sm.doc_k + (int64_t)b * p.S : nullptr;
+  // (this row's id is read again where a tile is compared element by element, rather than kept in a
+  // register across the loop: such tiles are the few that straddle a document boundary)
+  auto my_doc = [&]() { return sm_dk ? p.sm.doc_q[(int64_t)b * p.L + min(qrow, p.L - 1)] : 0; };
+  const int sm_dq0 = __builtin_amdgcn_readfirstlane(my_doc());
+  const bool sm_dq_uniform = SMOD && p.sm.doc_sorted && __builtin_amdgcn_ballot_w64(my_doc() != sm_dq0) == 0;
+  auto apply_smod = [&](f32x16& sv, int ta) {
+    if constexpr (SMOD) {
+      const int kvb = ta * BN + half * 4;
+      // this lane's 16 values of a vector per key (a tile that ends within the keys reads them at
+      // constant offsets from one address; a ragged last tile clamps every index)
+      auto load_keys = [&](const auto* row, auto (&val)[16]) {
+        if (ta * BN + BN <= p.S) {
+          const auto* at = row + kvb;
+#pragma unroll
+          for (int r = 0; r < 16; ++r) val[r] = at[(r >> 2) * 8 + (r & 3)];
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) val[r] = row[min(kvb + (r >> 2) * 8 + (r & 3), p.S - 1)];
+        }
+      };
+      if (sm_kw) {
+        float w[16];
+        load_keys(sm_kw, w);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] *= w[r];
+      }
+      if (sm_kb) {
+        float kb[16];
+        load_keys(sm_kb, kb);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf(kb[r], sm_inv_scale, sv[r]);
+      }
+      if (p.sm.alibi) {
+        const float base = (float)(kvb - qrow);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf(sm_slope, base + (float)((r >> 2) * 8 + (r & 3)), sv[r]);
+      }
+      if (p.sm.softcap > 0.f) {
+        const float cap_s = p.sm.softcap * sm_inv_scale, icap_s = p.scale / p.sm.softcap;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = cap_s * tanh_fast(sv[r] * icap_s);
+      }
+      if (sm_dk) {
+        const bool whole = sm_dq_uniform && sm_dk[min(ta * BN, p.S - 1)] == sm_dq0 && sm_dk[min(ta * BN + BN - 1, p.S - 1)] == sm_dq0;
+        if (!whole) {
+          int id[16];
+          load_keys(sm_dk, id);
+          const int mine = my_doc();
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sv[r] = id[r] != mine ? -INFINITY : sv[r];
+        }
+      }
+    }
+  };
+
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile
   const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
@@ -550,6 +644,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
     apply_bias(s_a, false);
     load_bias(1);
+    apply_smod(s_a, tile_of(0));
     if (edge(0)) mask_tile(s_a, tile_of(0) * BN);
     raise_reference(tile_max(s_a));  // the first reference is the maximum of the first tile
     m_run = m_new;
@@ -666,6 +761,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
       if (i == 0) {
         apply_bias(snext, true);
         load_bias(t + 2);
+        apply_smod(snext, tile_of(t + 1));
         if (__builtin_expect(edge(t + 1), 0)) mask_tile(snext, tile_of(t + 1) * BN);  // rare
         stage1(snext, 0);
       }
@@ -708,7 +804,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   if constexpr (FUNC) {
     // the sink logit joins the row's maximum and sum (flex_attention.py.jinja:1921-1923, :2134-2140)
     if (p.sink_logit) {
-      const float z = p.sink_logit[(int64_t)b * p.Hq + h];
+      const float z = sink_lse();
       if (z != -INFINITY) {
         const float mn = l_tot > 0.f ? m_run * p.scale : -INFINITY;  // the reference, natural-log domain
         const float mx = fmaxf(mn, z);
@@ -802,7 +898,7 @@ __global__ __launch_bounds__(128) void fwd_split_merge_kernel(FwdM p) {
 template <typename T, int D, int WAVES, int MASK>
 int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
   int bytes = 0;
-  if constexpr (D > 128 || MASK >= 2) {
+  if constexpr (D > 128 || MASK == 2 || MASK == 3) {
     // (four buffers per operand, 4 KB of bias tile per wavefront, and the tile list of a call with a skip table)
     constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK >= 2 ? WAVES * 4096 : 0);
     constexpr int kBytes = kBase + (MASK == 2 ? 2048 + 16 : 0);
@@ -820,6 +916,7 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
 template <typename T, int D, int WAVES>
 int launch_mask(const FwdM& g, int mask, dim3 grid, hipStream_t s) {
   if constexpr (D <= 128) {
+    if (mask == 4) return launch_one<T, D, WAVES, 4>(g, grid, s);
     if (mask == 3) return launch_one<T, D, WAVES, 3>(g, grid, s);
   }
   if (mask == 2) return launch_one<T, D, WAVES, 2>(g, grid, s);
@@ -862,7 +959,7 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
     }
   }
   // (the variant with a bias splits at head dims up to 128 only)
-  if (g.grouped && (head_dim <= 128 || g.bias_kind == 0) && !g.causal && g.window == 0 && !g.sink_logit) {
+  if (g.grouped && (head_dim <= 128 || g.bias_kind == 0) && !g.causal && g.window == 0 && !g.sink_logit && !g.sm.any) {
     const int64_t groups = (int64_t)g.B * g.Hkv * (g.Hq / g.Hkv / g.grouped);
     const int nt = (g.S + BN - 1) / BN;
     const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);
@@ -901,7 +998,11 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128 and the keep-mask in the bias slot");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  const int mask = g.keep_scale != 0.f ? 3 : g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit || g.split_tiles) ? 1 : 0;
+  if (g.sm.any && (head_dim > 128 || g.bias_kind != 0 || g.keep_scale != 0.f)) {
+    set_error("SDPA: score functors in fwd_w32_kernel need a head dim up to 128, no bias and no dropout");
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  const int mask = g.sm.any ? 4 : g.keep_scale != 0.f ? 3 : g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit || g.split_tiles) ? 1 : 0;
   int rc = dtype == MI355_SDPA_BF16 ? launch_dims<bf16_t>(g, head_dim, waves, mask, grid, s)
                                           : launch_dims<f16_t>(g, head_dim, waves, mask, grid, s);
   if (rc != MI355_SDPA_OK) return rc;

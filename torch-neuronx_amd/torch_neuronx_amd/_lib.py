@@ -48,7 +48,10 @@ class Desc(C.Structure):
 
 class MaskSpec(C.Structure):
     _fields_ = [("window", C.c_int32), ("sink_keys", C.c_int32), ("sink_logit", C.c_void_p),
-                ("live_tiles", C.c_void_p), ("live_tiles_t", C.c_void_p)]
+                ("live_tiles", C.c_void_p), ("live_tiles_t", C.c_void_p),
+                ("n_sink_logits", C.c_int32), ("softcap", C.c_float), ("alibi_slopes", C.c_void_p),
+                ("key_bias", C.c_void_p), ("key_weight", C.c_void_p), ("doc_ids_q", C.c_void_p),
+                ("doc_ids_k", C.c_void_p), ("doc_ids_sorted", C.c_int32)]
 
 
 class FwdParams(C.Structure):

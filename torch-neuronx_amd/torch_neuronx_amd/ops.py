@@ -122,26 +122,79 @@ def mask_tile_maps(attn_bias, B, Hq, L, S):
     return live, live_t
 
 
-def _mask_spec(spec, query, window, sink_keys, sink_logit, live_tiles=None):
-    """Fill the functor part of a parameter block; returns the tensors that must stay alive."""
+def _mask_spec(spec, query, S, window, sink_keys, sink_logit, live_tiles=None, score_mods=None):
+    """Fill the functor part of a parameter block; returns ``(sink logits as passed to the library or
+    None, the tensors that must stay alive over the launch)``."""
     spec.window = int(window or 0)
     spec.sink_keys = int(sink_keys or 0)
     if live_tiles is not None:
         spec.live_tiles, spec.live_tiles_t = live_tiles[0].data_ptr(), live_tiles[1].data_ptr()
-    if sink_logit is None:
-        return None
-    B, Hq = query.shape[0], query.shape[1]
-    z = sink_logit.to(device=query.device, dtype=torch.float32)
-    if z.numel() == Hq:
-        z = z.reshape(1, Hq)
-    z = z.reshape(-1, Hq).expand(B, Hq).contiguous()
-    spec.sink_logit = z.data_ptr()
-    return z
+    B, Hq, L = query.shape[0], query.shape[1], query.shape[2]
+    keep = []
+    z = None
+    if sink_logit is not None:
+        # (Hq,), (B, Hq) or (B, Hq, n): n logits per head (flex_attention_bwd.py.jinja:103)
+        z = sink_logit.to(device=query.device, dtype=torch.float32)
+        if z.dim() <= 1 or (z.dim() == 2 and z.numel() == Hq):
+            z = z.reshape(1, Hq)
+        if z.dim() == 2:
+            z = z.expand(B, Hq).contiguous()
+        else:
+            z = z.expand(B, Hq, z.shape[2]).contiguous()
+            spec.n_sink_logits = int(z.shape[2])
+        spec.sink_logit = z.data_ptr()
+    if score_mods:
+        f32 = lambda t, shape, name: _fixed(t, torch.float32, shape, name, query.device)
+        i32 = lambda t, shape, name: _fixed(t, torch.int32, shape, name, query.device)
+        m = score_mods
+        if m.get("softcap"):
+            spec.softcap = float(m["softcap"])
+        if m.get("alibi_slopes") is not None:
+            keep.append(f32(m["alibi_slopes"], (Hq,), "alibi_slopes"))
+            spec.alibi_slopes = keep[-1].data_ptr()
+        if m.get("key_bias") is not None:
+            keep.append(f32(m["key_bias"], (Hq, S), "key_bias"))
+            spec.key_bias = keep[-1].data_ptr()
+        if m.get("key_weight") is not None:
+            keep.append(f32(m["key_weight"], (Hq, S), "key_weight"))
+            spec.key_weight = keep[-1].data_ptr()
+        dq_, dk_ = m.get("doc_ids_q"), m.get("doc_ids_k")
+        if (dq_ is None) != (dk_ is None):
+            raise ValueError("doc_ids_q and doc_ids_k come together")
+        if dq_ is not None:
+            keep.append(i32(dq_, (B, L), "doc_ids_q"))
+            spec.doc_ids_q = keep[-1].data_ptr()
+            keep.append(i32(dk_, (B, S), "doc_ids_k"))
+            spec.doc_ids_k = keep[-1].data_ptr()
+            spec.doc_ids_sorted = int(bool(m.get("doc_ids_sorted")))
+    return z, keep
+
+
+def _fixed(t, dtype, shape, name, device):
+    """``t`` as a contiguous device tensor of ``dtype`` and ``shape`` (a leading dim of 1, or a
+    missing one, is broadcast)."""
+    t = torch.as_tensor(t).to(device=device, dtype=dtype)
+    while t.dim() < len(shape):
+        t = t.unsqueeze(0)
+    if t.dim() != len(shape) or any(a != b and a != 1 for a, b in zip(t.shape, shape)):
+        raise ValueError(f"{name} must have shape {tuple(shape)}, got {tuple(t.shape)}")
+    return t.expand(*shape).contiguous()
+
+
+_SCORE_MOD_KEYS = ("alibi_slopes", "softcap", "key_bias", "key_weight", "doc_ids_q", "doc_ids_k", "doc_ids_sorted")
+
+
+def _score_mods(kw):
+    m = {k: kw.pop(k) for k in _SCORE_MOD_KEYS if k in kw}
+    if kw:
+        raise TypeError(f"unexpected arguments: {sorted(kw)}")
+    live = any(m.get(k) is not None for k in _SCORE_MOD_KEYS if k not in ("softcap", "doc_ids_sorted"))
+    return m if live or (m.get("softcap") or 0) > 0 else None
 
 
 def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None, dropout_p=0.0,
                  dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0,
-                 window=None, sink_keys=0, sink_logit=None, live_tiles=None):
+                 window=None, sink_keys=0, sink_logit=None, live_tiles=None, **score_mods):
     """Fused forward.  K/V arrive at ``Hkv`` heads.  Returns ``(out, lse)``; ``out`` keeps the
     dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``.
 
@@ -149,8 +202,16 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     ``True`` to build it here): the kernels then skip the tiles that the mask drops whole.
 
     ``window`` (with ``is_causal``): query ``i`` sees keys ``i-window+1 .. i`` and the first
-    ``sink_keys`` keys; ``sink_logit`` ``(B,Hq)`` or ``(Hq,)``: one more logit per row that joins
-    the softmax and carries no value."""
+    ``sink_keys`` keys; ``sink_logit`` ``(B,Hq)``, ``(Hq,)`` or ``(B,Hq,n)``: logits that join every
+    row's softmax and carry no value.
+
+    Score functors (keyword only), applied to ``s = scale * q.k`` in this order: ``key_weight``
+    ``(Hq,S)`` multiplies, ``key_bias`` ``(Hq,S)`` is added, ``alibi_slopes`` ``(Hq,)`` adds
+    ``slope[h] * (j - i)``, ``softcap`` turns ``s`` into ``softcap * tanh(s / softcap)``;
+    ``doc_ids_q`` ``(B,L)`` / ``doc_ids_k`` ``(B,S)`` keep a score iff the two ids are equal
+    (``doc_ids_sorted=True``: the caller's promise that both are non-decreasing along the sequence,
+    which lets the kernels skip the key tiles of other documents)."""
+    score_mods = _score_mods(score_mods)
     for t, n in ((query, "query"), (key, "key"), (value, "value")):
         _require_cuda(t, n)
     B, Hq, L, E = query.shape
@@ -181,7 +242,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
     if live_tiles is True:
         live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
-    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit, live_tiles)  # noqa: F841 (kept alive over the launch)
+    _z = _mask_spec(p.mask, query, S, window, sink_keys, sink_logit, live_tiles, score_mods)  # noqa: F841 (kept alive over the launch)
     ws = None
     if (L <= 32 or L * (Hq // max(key.shape[1], 1)) <= 256) and query.dtype in (torch.float16, torch.bfloat16):
         # few query rows: the library may want to split the keys over more workgroups
@@ -198,10 +259,13 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
 def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_causal=False,
                   scale=None, dropout_p=0.0, dropout_keep=None, kv_lens=None,
                   want_grad_bias=False, force_kernel=0, window=None, sink_keys=0, sink_logit=None,
-                  live_tiles=None):
+                  live_tiles=None, **score_mods):
     """Fused backward.  Returns ``(dq, dk, dv, dbias-or-None)``; each gradient keeps the
     dimension order of its input, dk/dv come back at ``Hkv`` heads.  With a ``sink_logit`` a
-    fifth element follows: its gradient, float32 ``(B,Hq)``."""
+    fifth element follows: its gradient, float32 ``(B,Hq)`` or ``(B,Hq,n)``.  Score functors as in
+    ``sdpa_forward``: their derivative multiplies the gradient of the scores; the captured vectors
+    get no gradient of their own."""
+    score_mods = _score_mods(score_mods)
     for t, n in ((grad_out, "grad_out"), (query, "query"), (key, "key"), (value, "value")):
         _require_cuda(t, n)
     B, Hq, L, E = query.shape
@@ -241,10 +305,10 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
     if live_tiles is True:
         live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
-    _z = _mask_spec(p.mask, query, window, sink_keys, sink_logit, live_tiles)
+    _z, _keep = _mask_spec(p.mask, query, S, window, sink_keys, sink_logit, live_tiles, score_mods)
     dsink = None
     if _z is not None:
-        dsink = torch.empty((B, Hq), dtype=torch.float32, device=query.device)
+        dsink = torch.empty(_z.shape, dtype=torch.float32, device=query.device)
         p.grad_sink_logit = dsink.data_ptr()
     lib = _lib.load()
     nbytes = lib.mi355_sdpa_bwd_workspace_bytes(C.byref(p))
