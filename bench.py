@@ -284,6 +284,29 @@ def extra_documents(amd, dev):
     return r
 
 
+def extra_alibi(amd, dev):
+    """ALiBi under the causal mask, as a score functor (a slope per head, no bias tensor):
+    B=2 Hq=32 Hkv=8 S=4096 D=128 bf16."""
+    B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
+    q, k, v, do = seeded([(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, D), (B, Hq, S, D)], 1013, torch.bfloat16, dev)
+    slopes = torch.exp2(-(torch.arange(Hq, device=dev, dtype=torch.float32) + 1) * 8.0 / Hq)
+    r = _fwd_bwd_rates(amd, q, k, v, do, causal_pairs(S, S), D, D, is_causal=True, alibi_slopes=slopes)
+    r["shape"] = "B=2 Hq=32 Hkv=8 S=4096 D=128 bf16, causal + ALiBi slopes"
+    return r
+
+
+def extra_document_ids(amd, dev):
+    """Packed sequences (eight documents of 512 keys, each causal) given as document ids: no mask
+    tensor; the kernels find the key tiles of a row block's documents by themselves."""
+    B, Hq, Hkv, S, D = 2, 32, 8, 4096, 128
+    q, k, v, do = seeded([(B, Hq, S, D), (B, Hkv, S, D), (B, Hkv, S, D), (B, Hq, S, D)], 1009, torch.bfloat16, dev)
+    doc = (torch.arange(S, device=dev) // 512).to(torch.int32)[None].expand(B, S).contiguous()
+    live = 8 * causal_pairs(512, 512)
+    r = _fwd_bwd_rates(amd, q, k, v, do, live, D, D, is_causal=True, doc_ids_q=doc, doc_ids_k=doc, doc_ids_sorted=True)
+    r["shape"] = "B=2 Hq=32 Hkv=8 S=4096 D=128 bf16, causal + (B,S) document ids, 8 documents of 512"
+    return r
+
+
 def extra_wide(amd, dev):
     """Head dim 256, causal MHA, B=2 H=16 S=4096 bf16."""
     B, H, S, D = 2, 16, 4096, 256
@@ -508,6 +531,7 @@ def main():
         except Exception as e:
             extras["masked_fwd_shared_bias"] = {"error": repr(e)}
         for name, fn in (("window_1024_fwd_bwd", extra_window), ("document_mask_tables_fwd_bwd", extra_documents),
+                         ("alibi_causal_fwd_bwd", extra_alibi), ("document_ids_fwd_bwd", extra_document_ids),
                          ("head_dim_256_fwd_bwd", extra_wide), ("dropout_padding_fwd_bwd", extra_dropout), ("decode_bf16_cache_fwd", extra_decode_bf16),
                          ("few_kv_heads_fwd_bwd", extra_few_kv_heads), ("float32_fwd_bwd", extra_f32)):
             try:

@@ -73,6 +73,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   }
   const int part = pq * p.parts_h + ph;  // its rows among the partial results
   const int b = st / p.Hkv, hk = st % p.Hkv;
+  if constexpr (MASK == 4) {
+    if (p.kt_order) kt = p.kt_order[b * p.n_kt + kt];  // (the batch's key blocks, heaviest first)
+  }
   const int rep_all = p.Hq / p.Hkv;
   const int rep = p.parts > 1 ? rep_all / p.parts_h : rep_all;  // heads of the group that this workgroup walks
   const int h0 = ph * rep;                                       // the first of them
@@ -127,17 +130,25 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   // lies between the ids of the block's first and last key are one run, found by two searches over
   // doc_q, and only the query tiles that touch it are walked
   const bool sm_doc = SMOD && p.sm.doc_q && p.sm.doc_k;
+  // (every load of the searches' first round goes out before anything waits: one trip to memory)
+  const bool sm_runs = SMOD && sm_doc && p.sm.doc_sorted && k0 < S;
+  int sm_first = 0, sm_d_lo = 0, sm_d_hi = 0;
+  if constexpr (SMOD) {
+    if (sm_runs) {
+      sm_first = doc_first_samples(p.sm.doc_q + (int64_t)b * p.L, p.L, lane);
+      sm_d_lo = p.sm.doc_k[(int64_t)b * p.S + k0], sm_d_hi = p.sm.doc_k[(int64_t)b * p.S + min(k0 + BK, S) - 1];
+    }
+  }
   const int sm_dk = sm_doc ? p.sm.doc_k[(int64_t)b * p.S + max(min(key, S - 1), 0)] : 0;
   const int sm_dk_first = __builtin_amdgcn_readlane(sm_dk, 0), sm_dk_last = __builtin_amdgcn_readlane(sm_dk, 31);
+  // (the rows that this wavefront's 32 keys can see: the run of doc_q with their ids)
+  int doc_run_w[2] = {0, 0x7fffffff};
   if constexpr (SMOD) {
-    if (sm_doc && p.sm.doc_sorted && k0 < S) {
-      const int32_t* dqr = p.sm.doc_q + (int64_t)b * p.L;
-      const int32_t* dkr = p.sm.doc_k + (int64_t)b * p.S;
-      const int d_lo = dkr[k0], d_hi = dkr[min(k0 + BK, S) - 1];
-      const int r_lo = wave_lower_bound(dqr, p.L, d_lo, lane);
-      const int r_hi = d_hi == INT_MAX ? p.L : wave_lower_bound(dqr, p.L, d_hi + 1, lane);
-      qs_begin = max(qs_begin, r_lo / BQ);
-      qs_end = r_hi > r_lo ? max(min(qs_end, (r_hi + BQ - 1) / BQ), qs_begin) : qs_begin;
+    if (sm_runs) {
+      int run[2];
+      doc_runs(p.sm.doc_q + (int64_t)b * p.L, p.L, sm_d_lo, sm_d_hi, sm_dk_first, sm_dk_last, run, doc_run_w, lane, sm_first);
+      qs_begin = max(qs_begin, run[0] / BQ);
+      qs_end = run[1] > run[0] ? max(min(qs_end, (run[1] + BQ - 1) / BQ), qs_begin) : qs_begin;
     }
   }
   const int per_head = qs_end - qs_begin;
@@ -381,6 +392,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       if (p.sm.key_weight) sm_w = p.sm.key_weight[(int64_t)hh * p.S + min(key, p.S - 1)];
       if (p.sm.key_bias) sm_kb = p.sm.key_bias[(int64_t)hh * p.S + min(key, p.S - 1)] * sm_inv_scale;
     }
+    // (the functors' derivative differs from one: the dK wavefronts get P times it, see hand_over)
     const bool need_dfac = SMOD && (p.sm.key_weight != nullptr || p.sm.softcap > 0.f);
     if constexpr (MASK == 1) {
       if (p.bias_kind)
@@ -392,9 +404,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     uint32_t* px = pex + (pb * 4 + kb) * 1024 + lane * 4;  // [4 groups of 4 words][lane][4]
     f32x16 sc[2];
     uint32_t pk[2][8];
-    // what the dK wavefronts get.  Dropout: every probability, the dropped ones negative; score
-    // functors with a derivative other than one: the probability times that derivative
-    uint32_t pkx[(DROP || SMOD) ? 2 : 1][8];
+    uint32_t pkx[DROP ? 2 : 1][8];  // (dropout) what the dK wavefronts get: every probability, the dropped ones negative
     f32x4 l4[2][4];
     u32x4 ring[8];
     auto load_l4 = [&](int mq, int r4) { l4[mq][r4] = *(const f32x4*)(lrow + mq * 32 + r4 * 8); };
@@ -418,21 +428,15 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
           pk[mq][r >> 1] = Mma<T>::pack(fmaxf(s0, 0.f), fmaxf(s1, 0.f));
         } else {
           pk[mq][r >> 1] = Mma<T>::pack(p0, p1);
-          if constexpr (SMOD) {
-            if (need_dfac) {
-              // the derivative of the functors, from the modified score: 1 - tanh^2 = 1 - (s' / cap)^2
-              // (a masked score, -inf, is clamped to a derivative of 0), times the key's weight
-              const float t0 = __builtin_amdgcn_fmed3f(sc[mq][r] * icap_s, -1.f, 1.f), t1 = __builtin_amdgcn_fmed3f(sc[mq][r + 1] * icap_s, -1.f, 1.f);
-              pkx[mq][r >> 1] = Mma<T>::pack(p0 * (fmaf(-t0, t0, 1.f) * sm_w), p1 * (fmaf(-t1, t1, 1.f) * sm_w));
-            }
-          }
         }
       }
     };
     // score functors: the raw score tile s becomes mod(scale * s) / scale (lane = key, element r =
     // row 32 mq + 8 (r / 4) + 4 half + r % 4 of the tile), one block per functor behind a uniform test
+    const int sm_on = SMOD ? __builtin_amdgcn_readfirstlane((p.sm.key_weight ? 1 : 0) | (p.sm.key_bias ? 2 : 0) | (p.sm.alibi ? 4 : 0) | (p.sm.softcap > 0.f ? 8 : 0)) : 0;
     auto smod_scores = [&](int mq) {
       if constexpr (SMOD) {
+        if (sm_on == 0) return;  // (document ids alone: nothing to rewrite)
         if (p.sm.key_weight) {
 #pragma unroll
           for (int r = 0; r < 16; ++r) sc[mq][r] *= sm_w;
@@ -467,9 +471,24 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
       }
     };
     auto hand_over = [&](int mq) {
-      const uint32_t(&w)[8] = (DROP || (SMOD && need_dfac)) ? pkx[(DROP || SMOD) ? mq : 0] : pk[mq];
-      *(u32x4*)(px + (2 * mq) * 256) = u32x4{w[0], w[1], w[2], w[3]};
-      *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{w[4], w[5], w[6], w[7]};
+      if (SMOD && need_dfac) {
+        // Score functors whose derivative differs from one: the dK wavefronts get P times that
+        // derivative, formed here from the packed probabilities and the modified scores
+        // (1 - tanh^2 = 1 - (s' / cap)^2, a masked score's -inf clamped to a derivative of 0, times
+        // the key's weight) - outside the slots, which carry neither a branch nor a register for it.
+        uint32_t w[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const float t0 = __builtin_amdgcn_fmed3f(sc[mq][2 * j] * icap_s, -1.f, 1.f), t1 = __builtin_amdgcn_fmed3f(sc[mq][2 * j + 1] * icap_s, -1.f, 1.f);
+          w[j] = Mma<T>::pack(Mma<T>::unpack(pk[mq][j], 0) * (fmaf(-t0, t0, 1.f) * sm_w), Mma<T>::unpack(pk[mq][j], 1) * (fmaf(-t1, t1, 1.f) * sm_w));
+        }
+        *(u32x4*)(px + (2 * mq) * 256) = u32x4{w[0], w[1], w[2], w[3]};
+        *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{w[4], w[5], w[6], w[7]};
+      } else {
+        const uint32_t(&w)[8] = DROP ? pkx[DROP ? mq : 0] : pk[mq];
+        *(u32x4*)(px + (2 * mq) * 256) = u32x4{w[0], w[1], w[2], w[3]};
+        *(u32x4*)(px + (2 * mq + 1) * 256) = u32x4{w[4], w[5], w[6], w[7]};
+      }
     };
 #pragma unroll
     for (int i = 0; i < AHEAD; ++i) ring[i] = read_rows(qt, i);
@@ -514,20 +533,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   };
   // every key of this block lies above the diagonal of the tile's rows / past the keys / below their
   // windows, or the mask's skip table says that it keeps no score of the tile's rows and the block's keys
-  // document ids of a tile's first and last row, from the tile's row of ids in LDS
-  auto doc_rows = [&](int it, int tb, int& d_first, int& d_last) {
-    const int q0 = item_q0(it);
-    d_first = __builtin_amdgcn_readfirstlane(doc_s[tb * BQ]);
-    d_last = __builtin_amdgcn_readfirstlane(doc_s[tb * BQ + min(BQ, p.L - q0) - 1]);
-  };
   auto dead_tile = [&](int it, int tb) {
     const int q0 = item_q0(it);
     if constexpr (SMOD) {
-      if (sm_doc && p.sm.doc_sorted) {  // the rows' ids and this wavefront's keys' ids do not overlap
-        int d_first, d_last;
-        doc_rows(it, tb, d_first, d_last);
-        if (d_last < sm_dk_first || d_first > sm_dk_last) return true;
-      }
+      // (sorted ids: the tile's rows lie outside the run of rows with this wavefront's keys' ids)
+      if (sm_doc && p.sm.doc_sorted && (min(q0 + BQ, p.L) <= doc_run_w[0] || q0 >= doc_run_w[1])) return true;
     }
     if constexpr (MASK == 2) {
       if (listed) {
@@ -543,11 +553,9 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     if (dead_tile(it, tb)) return;
     bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
     if constexpr (SMOD) {
-      if (sm_doc) {  // every score compared, unless the tile's rows and the wavefront's keys all carry one id
-        int d_first = 0, d_last = 1;
-        if (p.sm.doc_sorted) doc_rows(it, tb, d_first, d_last);
-        edge |= !(d_first == d_last && sm_dk_first == sm_dk_last && d_first == sm_dk_first);
-      }
+      // every score compared, unless (sorted ids) the wavefront's keys carry one id and the tile's rows lie
+      // inside the run of rows with that id
+      if (sm_doc) edge |= !(p.sm.doc_sorted && sm_dk_first == sm_dk_last && q0 >= doc_run_w[0] && min(q0 + BQ, p.L) <= doc_run_w[1]);
     }
     role_a_tile(it, tb, pb, edge);
   };
@@ -750,6 +758,51 @@ __global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
   }
 }
 
+// Launch order of the key blocks for a call with sorted document ids.  Workgroups are dispatched in
+// order, one per compute unit at a time, so the heaviest should go first; without documents that is
+// the order of the key blocks under a causal mask, with them the weight of a block is the number of
+// query tiles between itself and the end of its documents, which only the ids tell.  One workgroup
+// per batch counts every key block's query tiles the way bwd_dkdv_w32_kernel does and ranks them.
+__global__ __launch_bounds__(256) void bwd_key_order_kernel(BwdM p) {
+  __shared__ int weight[1024];
+  const int b = blockIdx.x, n_kt = p.n_kt;
+  const int32_t* dqr = p.sm.doc_q + (int64_t)b * p.L;
+  const int32_t* dkr = p.sm.doc_k + (int64_t)b * p.S;
+  int S = p.S;
+  if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+  const int nqs = (p.L + BQ - 1) / BQ;
+  auto lower_bound = [&](int x) {  // first row whose id is >= x
+    int lo = 0, hi = p.L;
+    while (lo < hi) {
+      const int mid = (lo + hi) >> 1;
+      if (dqr[mid] < x) lo = mid + 1;
+      else hi = mid;
+    }
+    return lo;
+  };
+  for (int kt = threadIdx.x; kt < n_kt; kt += 256) {
+    const int k0 = kt * BK;
+    int items = 0;
+    if (k0 < S) {
+      const int d_lo = dkr[k0], d_hi = dkr[min(k0 + BK, S) - 1];
+      const int r_lo = lower_bound(d_lo), r_hi = d_hi == INT_MAX ? p.L : lower_bound(d_hi + 1);
+      int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+      int qs_end = (p.window > 0 && k0 >= p.sink_keys) ? max(min(nqs, (k0 + BK + p.window - 2) / BQ + 1), qs_begin) : nqs;
+      qs_begin = max(qs_begin, r_lo / BQ);
+      qs_end = r_hi > r_lo ? max(min(qs_end, (r_hi + BQ - 1) / BQ), qs_begin) : qs_begin;
+      items = qs_end - qs_begin;
+    }
+    weight[kt] = items;
+  }
+  __syncthreads();
+  for (int kt = threadIdx.x; kt < n_kt; kt += 256) {  // rank = blocks that are heavier, or as heavy and earlier
+    const int w = weight[kt];
+    int rank = 0;
+    for (int j = 0; j < n_kt; ++j) rank += (weight[j] > w) | ((weight[j] == w) & (j < kt));
+    p.kt_order[b * n_kt + rank] = kt;
+  }
+}
+
 template <typename T, int D, int MASK>
 int launch_t(const BwdM& g, hipStream_t s) {
   // (MASK = 2: with the skip table's row of the key block and the item list; MASK = 4: with the document ids of three tiles' rows)
@@ -771,6 +824,11 @@ int launch_m(const BwdM& g, hipStream_t s) {
     if (g.keep_scale != 0.f || g.bias_kind) {
       set_error("SDPA: score functors in bwd_dkdv_w32_kernel need a call without bias and dropout");
       return MI355_SDPA_ERR_UNSUPPORTED;
+    }
+    if (g.kt_order) {
+      hipLaunchKernelGGL(bwd_key_order_kernel, dim3((unsigned)g.B), dim3(256), 0, s, g);
+      const int rc = check_launch("bwd_key_order_kernel");
+      if (rc != MI355_SDPA_OK) return rc;
     }
     return launch_t<T, D, 4>(g, s);
   }
@@ -840,6 +898,7 @@ int launch_bwd_dkdv_w32(const BwdM& g0, int dtype, int head_dim, hipStream_t s) 
     // count: every key block then deals its items to all the parts in equal shares)
     if (g.sm.doc_sorted) g.chunk_items = 0;
   }
+  if (!g.sm.doc_sorted || g.n_kt > 1024) g.kt_order = nullptr;  // (the ranking kernel holds 1024 weights)
   if (head_dim == 128) return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 128>(g, s) : launch_m<f16_t, 128>(g, s);
   return dtype == MI355_SDPA_BF16 ? launch_m<bf16_t, 64>(g, s) : launch_m<f16_t, 64>(g, s);
 }

@@ -157,19 +157,27 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   int nt = (S + BN - 1) / BN;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   int n_lead = 0, skip = 0;
+  // (document ids sorted along the sequence: the keys that this wavefront's rows can see, and whether
+  // those rows all belong to one document)
+  int doc_run_w[2] = {0, 0x7fffffff};
+  bool doc_one_w = false;
   if constexpr (FUNC) {
     int t_lo = p.window > 0 ? max(q0 - p.window + 1, 0) / BN : 0;
     if constexpr (SMOD) {
       // document ids sorted along the sequence: only the run of keys whose id lies between the ids of
-      // this workgroup's first and last row can hold a kept score
+      // this workgroup's first and last row can hold a kept score; the same for this wavefront's own
+      // rows, inside whose run a tile needs no comparison when the rows belong to one document
       if (p.sm.doc_sorted) {
         const int32_t* dqr = p.sm.doc_q + (int64_t)b * p.L;
         const int32_t* dkr = p.sm.doc_k + (int64_t)b * p.S;
+        const int first = doc_first_samples(dkr, S, lane);  // (requested ahead of the ids below: one trip for both)
         const int d_lo = dqr[min(q0, p.L - 1)], d_hi = dqr[min(q0 + BM, p.L) - 1];
-        const int k_lo = wave_lower_bound(dkr, S, d_lo, lane);
-        const int k_hi = d_hi == INT_MAX ? S : wave_lower_bound(dkr, S, d_hi + 1, lane);
-        nt = k_hi > k_lo ? min(nt, (k_hi + BN - 1) / BN) : 0;
-        t_lo = max(t_lo, k_lo / BN);
+        const int w_lo = dqr[min(qw0, p.L - 1)], w_hi = dqr[min(qw0 + 32, p.L) - 1];
+        int run[2];
+        doc_runs(dkr, S, d_lo, d_hi, w_lo, w_hi, run, doc_run_w, lane, first);
+        doc_one_w = w_lo == w_hi;
+        nt = run[1] > run[0] ? min(nt, (run[1] + BN - 1) / BN) : 0;
+        t_lo = max(t_lo, run[0] / BN);
       }
     }
     if (t_lo > 0) {
@@ -337,11 +345,22 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // (this row's id is read again where a tile is compared element by element, rather than kept in a
   // register across the loop: such tiles are the few that straddle a document boundary)
   auto my_doc = [&]() { return sm_dk ? p.sm.doc_q[(int64_t)b * p.L + qc] : 0; };
-  const int sm_dq0 = __builtin_amdgcn_readfirstlane(my_doc());
-  const bool sm_dq_uniform = SMOD && p.sm.doc_sorted && __builtin_amdgcn_ballot_w64(my_doc() != sm_dq0) == 0;
+  // (which functors are on, as one scalar: the common cases - no functor at work in this tile, ALiBi
+  // alone - then cost one or two taken branches per tile instead of one per functor)
+  const int sm_on = SMOD ? __builtin_amdgcn_readfirstlane((sm_kw ? 1 : 0) | (sm_kb ? 2 : 0) | (p.sm.alibi ? 4 : 0) | (p.sm.softcap > 0.f ? 8 : 0)) : 0;
   auto apply_smod = [&](f32x16& sv, f32x16& dpv, int ta) {
     if constexpr (SMOD) {
       const int kvb = ta * BN + half * 4;
+      // (sorted ids: a tile inside the key run of this wavefront's one document keeps everything,
+      // a tile outside the run of its rows' documents keeps nothing - no load either way)
+      const bool doc_whole = doc_one_w && ta * BN >= doc_run_w[0] && ta * BN + BN <= doc_run_w[1];
+      if (sm_on == 0 && (sm_dk == nullptr || doc_whole)) return;
+      if (sm_on == 4 && (sm_dk == nullptr || doc_whole)) {
+        const float base = (float)(kvb - qrow);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) sv[r] = fmaf(sm_slope, base + (float)((r >> 2) * 8 + (r & 3)), sv[r]);
+        return;
+      }
       // this lane's 16 values of a vector per key (a tile that ends within the keys reads them at
       // constant offsets from one address; a ragged last tile clamps every index)
       auto load_keys = [&](const auto* row, auto (&val)[16]) {
@@ -380,8 +399,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
         }
       }
       if (sm_dk) {
-        const bool whole = sm_dq_uniform && sm_dk[min(ta * BN, p.S - 1)] == sm_dq0 && sm_dk[min(ta * BN + BN - 1, p.S - 1)] == sm_dq0;
-        if (!whole) {
+        const bool none = p.sm.doc_sorted && (ta * BN >= doc_run_w[1] || ta * BN + BN <= doc_run_w[0]);
+        if (none) {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sv[r] = -INFINITY;
+        } else if (!doc_whole) {
           int id[16];
           load_keys(sm_dk, id);
           const int mine = my_doc();

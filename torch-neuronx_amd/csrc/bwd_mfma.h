@@ -47,6 +47,9 @@ struct BwdM {
   int window = 0, sink_keys = 0;
   // score functors and document ids (the functor variants of bwd_dq_w32.hip and bwd_dkdv_w32.hip)
   ScoreMod sm;
+  // sorted document ids: workspace for the order in which the dK/dV kernel takes the key blocks of a
+  // batch, heaviest first ((B, n_kt) ints, written by bwd_key_order_kernel ahead of it); nullptr: 0, 1, 2 ...
+  int32_t* kt_order = nullptr;
   // tile skip table of a per-score bias / keep-mask for the dK/dV kernel: per (mask batch, mask head,
   // block of 128 keys) a bitmap of the 64-row query tiles with a kept score, live_t_words words each;
   // live_hm = the mask's own head extent

@@ -630,9 +630,16 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
 
 // delta and lse2, rounded up to 256 bytes, and behind them the partial dK / dV rows of a call whose
 // dK/dV kernel splits its items
-static size_t row_terms_bytes(const mi355_sdpa_bwd_params& p) {
+static size_t row_stats_bytes(const mi355_sdpa_bwd_params& p) {
   return ((size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float) + 255) & ~(size_t)255;
 }
+// (behind them, for a call with sorted document ids: the order in which the dK/dV kernel takes the key
+// blocks of each batch, one int per block)
+static size_t key_order_bytes(const mi355_sdpa_bwd_params& p) {
+  if (!p.mask.doc_ids_sorted || !p.mask.doc_ids_q || !p.mask.doc_ids_k) return 0;
+  return ((size_t)p.q.size[0] * ((p.k.size[2] + 127) / 128) * sizeof(int32_t) + 255) & ~(size_t)255;
+}
+static size_t row_terms_bytes(const mi355_sdpa_bwd_params& p) { return row_stats_bytes(p) + key_order_bytes(p); }
 static int parts_of(const BwdM& g, const mi355_sdpa_bwd_params& p) {
   if (p.k.size[2] <= 0 || p.k.size[1] <= 0) return 1;
   if (p.q.size[3] > 128 || p.v.size[3] != p.q.size[3]) return bwd_wide_parts(g);
@@ -662,6 +669,7 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
     g.part_dk = (float*)((char*)p.workspace + row_terms_bytes(p));
     g.part_dv = g.part_dk + (size_t)parts * g.B * g.Hkv * g.S * g.d_real;
   }
+  if (key_order_bytes(p) && p.workspace_bytes >= row_terms_bytes(p)) g.kt_order = (int32_t*)((char*)p.workspace + row_stats_bytes(p));
   const int D = p.q.size[3] <= 64 ? 64 : 128;  // the kernels' width
   int rc;
   if (p.q.size[3] > 128 || p.v.size[3] != p.q.size[3]) rc = launch_bwd_wide(g, p.dtype, s);

@@ -7,6 +7,7 @@
 // then the masks (causal, window, document ids).
 #pragma once
 
+#include <limits.h>
 #include <stdint.h>
 
 #include "../../include/mi355_sdpa.h"
@@ -43,20 +44,63 @@ __device__ __forceinline__ float tanh_fast(float x) {
 }
 
 // First index of the sorted array a[0 .. n) whose value is >= x (n if none), found by a whole
-// wavefront: every round samples 64 evenly spaced positions and keeps the interval between the last
-// sample below x and the first one at or above it, so 4096 elements take two rounds of one load each.
-__device__ __forceinline__ int wave_lower_bound(const int32_t* a, int n, int x, int lane) {
-  int lo = 0, len = n;
-  while (len > 0) {
-    const int step = (len + 63) >> 6;
-    const int idx = lo + (lane + 1) * step - 1;
-    const bool below = idx < lo + len && a[idx] < x;
-    const int cnt = __builtin_popcountll(__builtin_amdgcn_ballot_w64(below));
-    const int end = lo + len;
-    lo += cnt * step;
-    len = min(step - 1, end - lo);
+// wavefront, for N values of x at once: every round samples 64 evenly spaced positions per search
+// (all the loads of a round go out together) and keeps the interval between the last sample below x
+// and the first one at or above it, so 4096 elements take two trips to memory whatever N is.
+// The first round's samples do not depend on x: a caller fetches them (doc_first_samples) together
+// with whatever tells it x, which saves one of the trips.
+__device__ __forceinline__ int doc_first_samples(const int32_t* a, int n, int lane) {
+  const int idx = (lane + 1) * ((n + 63) >> 6) - 1;
+  return (n > 0 && idx < n) ? a[idx] : INT_MAX;
+}
+template <int N>
+__device__ __forceinline__ void wave_lower_bounds(const int32_t* a, int n, const int (&x)[N], int (&out)[N], int lane, int first) {
+  int lo[N], len[N];
+  {  // round one, on the samples the caller brought
+    const int step = (n + 63) >> 6;
+    const int idx = (lane + 1) * step - 1;
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const bool below = n > 0 && idx < n && first < x[i];
+      const int cnt = __builtin_popcountll(__builtin_amdgcn_ballot_w64(below));
+      lo[i] = cnt * step;
+      len[i] = max(min(step - 1, n - lo[i]), 0);
+    }
   }
-  return __builtin_amdgcn_readfirstlane(lo);
+  for (;;) {
+    int left = 0;
+#pragma unroll
+    for (int i = 0; i < N; ++i) left |= len[i];
+    if (left <= 0) break;  // (uniform: every lane holds the same intervals)
+    int v[N], step[N];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      step[i] = (len[i] + 63) >> 6;
+      const int idx = lo[i] + (lane + 1) * step[i] - 1;
+      v[i] = (len[i] > 0 && idx < lo[i] + len[i]) ? a[idx] : INT_MAX;
+    }
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      const int idx = lo[i] + (lane + 1) * step[i] - 1;
+      const bool below = len[i] > 0 && idx < lo[i] + len[i] && v[i] < x[i];
+      const int cnt = __builtin_popcountll(__builtin_amdgcn_ballot_w64(below));
+      const int end = lo[i] + len[i];
+      lo[i] += cnt * step[i];
+      len[i] = max(min(step[i] - 1, end - lo[i]), 0);
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < N; ++i) out[i] = __builtin_amdgcn_readfirstlane(lo[i]);
+}
+// The run [first, past) of the sorted ids a[0 .. n) whose value lies in [id_lo, id_hi], for two such
+// id ranges at once (a workgroup's rows and a wavefront's rows, say).
+__device__ __forceinline__ void doc_runs(const int32_t* a, int n, int lo0, int hi0, int lo1, int hi1, int (&run0)[2], int (&run1)[2],
+                                         int lane, int first) {
+  const int x[4] = {lo0, hi0 == INT_MAX ? INT_MAX : hi0 + 1, lo1, hi1 == INT_MAX ? INT_MAX : hi1 + 1};
+  int r[4];
+  wave_lower_bounds<4>(a, n, x, r, lane, first);
+  run0[0] = r[0], run0[1] = hi0 == INT_MAX ? n : r[1];
+  run1[0] = r[2], run1[1] = hi1 == INT_MAX ? n : r[3];
 }
 #endif
 
