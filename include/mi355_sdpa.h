@@ -196,7 +196,9 @@ typedef struct mi355_sdpa_bwd_params {
 } mi355_sdpa_bwd_params;
 
 typedef struct mi355_sdpa_decode_params {
-  mi355_sdpa_tensor q;      /* (B,Hq,Lq,D) bf16/f16/f32, D = 128, Lq*Hq/Hkv <= 8       */
+  mi355_sdpa_tensor q;      /* (B,Hq,Lq,D) bf16/f16/f32, D = 128, Lq*Hq/Hkv <= 16.  The
+                               query is carried exactly (bf16), with 12 to 16 significant
+                               bits (f16) or with 16 (f32): see decode_fp8kv.hip           */
   mi355_sdpa_tensor k;      /* (B,Hkv,S,D)  fp8 e4m3fn, 1 byte per element             */
   mi355_sdpa_tensor v;      /* (B,Hkv,S,D)  fp8 e4m3fn                                 */
   const float* k_scale;     /* (B,Hkv) contiguous: real K = fp8 value * k_scale        */

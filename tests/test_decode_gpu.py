@@ -37,7 +37,8 @@ def _check(amd, dev, case, tol=2e-2, **kw):
                                 None if lens is None else lens.to(dev), **kw)
     torch.cuda.synchronize()
     S = kq.shape[2]
-    ro, rl = om.decode_fp8kv(q, kq, vq, ks, vs, lens if lens is not None else torch.full((q.shape[0],), S))
+    ro, rl = om.decode_fp8kv(q, kq, vq, ks, vs, lens if lens is not None else torch.full((q.shape[0],), S),
+                             scale=kw.get("scale"))
     assert out.dtype == q.dtype
     assert max_abs(out, ro) <= tol
     assert max_abs(lse, rl) <= 5e-3
@@ -118,3 +119,69 @@ def test_config5_full_size(amd, gpu_device):
         kq[b : b + 1], ks[b : b + 1] = om.quantize_kv_fp8(kb)
         vq[b : b + 1], vs[b : b + 1] = om.quantize_kv_fp8(vb)
     _check(amd, gpu_device, (q, kq, vq, ks, vs, lens))
+
+
+# Queries that are not bf16 carry more significant bits than two or three e4m3 terms hold (float16: 11,
+# float32: 24).  The configurations below - float16 / float32 queries at scales 0.2 and 1.0 on N(0,1)
+# data, logits of +-10 and more, one key up to 2048 - are the ones a randomised sweep found outside
+# 2e-2 / 5e-3 when such queries were cut to 8 or 12 bits; the kernel now gives them 12 to 16.
+_SHARP = [
+    # (dtype, B, Hq, Hkv, Lq, S, lens, scale, splits)
+    (torch.float32, 130, 4, 2, 4, 1, "short", 0.2, 1),
+    (torch.float32, 2, 16, 8, 4, 31, "none", 1.0, 0),
+    (torch.float16, 2, 16, 8, 3, 2048, "none", 1.0, 0),
+    (torch.float32, 1, 12, 2, 1, 31, "full", 1.0, 0),
+    (torch.float16, 2, 3, 1, 2, 100, "rand", 1.0, 1),
+    (torch.float32, 3, 2, 1, 4, 500, "none", 1.0, 0),
+    (torch.float32, 1, 8, 1, 1, 500, "rand", 1.0, 7),
+    (torch.float32, 2, 2, 1, 3, 33, "short", 1.0, 2),
+    (torch.float32, 5, 2, 1, 3, 32, "short", 1.0, 0),
+    (torch.float16, 17, 48, 8, 1, 1, "rand", 1.0, 7),
+    (torch.float16, 130, 48, 8, 1, 576, "rand", 0.2, 7),
+    (torch.float16, 2, 16, 8, 4, 2048, "full", 1.0, 7),
+    (torch.float16, 2, 16, 8, 3, 1000, "short", 1.0, 7),
+    (torch.float16, 5, 16, 8, 3, 32, "rand", 1.0, 0),
+    (torch.float16, 5, 24, 8, 2, 128, "short", 1.0, 0),
+    (torch.float32, 64, 64, 8, 1, 32, "none", 1.0, 0),
+    (torch.float16, 5, 48, 8, 1, 500, "none", 1.0, 1),
+    (torch.float32, 5, 48, 8, 1, 1000, "rand", 1.0, 0),
+    (torch.float16, 2, 64, 8, 1, 128, "short", 1.0, 2),
+    (torch.float32, 5, 6, 2, 2, 32, "none", 1.0, 7),
+    (torch.float16, 1, 2, 1, 3, 2048, "full", 1.0, 7),
+    (torch.float32, 64, 8, 1, 1, 128, "rand", 1.0, 7),
+    (torch.float16, 5, 6, 2, 2, 2048, "none", 1.0, 1),
+]
+
+
+@pytest.mark.parametrize("cfg", _SHARP, ids=lambda c: f"{str(c[0])[6:]}-B{c[1]}-{c[2]}x{c[3]}-Lq{c[4]}-S{c[5]}-{c[6]}-{c[7]}")
+def test_decode_keeps_the_precision_of_float16_and_float32_queries(amd, gpu_device, cfg):
+    dt, B, Hq, Hkv, Lq, S, mode, scale, splits = cfg
+    g = torch.Generator().manual_seed(B * 1000 + S)
+    lens = {"rand": torch.randint(0, S + 1, (B,), generator=g), "full": torch.full((B,), S), "none": None,
+            "short": torch.randint(0, min(S, 40) + 1, (B,), generator=g)}[mode]
+    lens = None if lens is None else lens.to(torch.int32)
+    _check(amd, gpu_device, _case(B, Hq, Hkv, Lq, S, lens, seed=S + Hq, qdtype=dt), scale=scale, num_splits=splits)
+
+
+def test_decode_float32_query_with_one_key(amd, gpu_device):
+    # one key: the output is that key's value row and lse is the logit itself, so its error is the
+    # error of the query's representation alone (8 bits would give about 6e-3 here)
+    dev = gpu_device
+    q, kq, vq, ks, vs, _ = _case(130, 4, 2, 4, 1, None, seed=5, qdtype=torch.float32)
+    out, lse = amd.decode_fp8kv(q.to(dev), kq.to(dev), vq.to(dev), ks.to(dev), vs.to(dev), None, scale=0.2)
+    ro, rl = om.decode_fp8kv(q, kq, vq, ks, vs, torch.full((130,), 1), scale=0.2)
+    assert max_abs(lse, rl) <= 1e-3 and max_abs(out, ro) <= 1e-3
+
+
+@pytest.mark.parametrize("qdtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("Hq,Hkv,Lq", [(12, 1, 1), (16, 1, 1), (8, 2, 4), (24, 2, 1), (3, 1, 5)])
+def test_decode_up_to_sixteen_query_rows_per_kv_head(amd, gpu_device, qdtype, Hq, Hkv, Lq):
+    lens = torch.tensor([700, 1, 33, 0], dtype=torch.int32)
+    _check(amd, gpu_device, _case(4, Hq, Hkv, Lq, 700, lens, seed=Hq + Lq, qdtype=qdtype))
+
+
+def test_decode_refuses_more_than_sixteen_rows(amd, gpu_device):
+    dev = gpu_device
+    q, kq, vq, ks, vs, _ = _case(1, 17, 1, 1, 64, None, seed=1)
+    with pytest.raises(RuntimeError, match=r"\[1, 16\]"):
+        amd.decode_fp8kv(q.to(dev), kq.to(dev), vq.to(dev), ks.to(dev), vs.to(dev), None)

@@ -10,10 +10,15 @@
 // time with a running max / sum / output, writes one partial result per (batch, kv head) it
 // touched, and a second small kernel merges the partials of a sequence.
 //
-// Precision without dequantising the cache: the bf16 query row is scaled by a power of two
-// and split into up to three e4m3 terms (q = q0 + q1 + q2, exact to ~12 bits); the terms
-// occupy separate columns of the 16-wide MFMA N dimension, which would otherwise idle, and
-// are summed after the product.  The probabilities are split the same way before P*V.
+// Precision without dequantising the cache: the query row is scaled by a power of two and split
+// into e4m3 terms (q = q0 + q1 + ..., four significant bits each).  Up to four terms occupy
+// separate columns of the 16-wide MFMA N dimension, which would otherwise idle, and are summed after
+// the product; when the query rows of a kv head leave no room for that many (more than 4 rows: two
+// terms per matrix op, more than 8: one), the remaining terms go through the matrix ops a second
+// (third, fourth) time into the same accumulators - the pipe is a fraction busy in this kernel.  A
+// bf16 query (8 significant bits) is exact in two terms and gets two or three, a float16 query (11)
+// gets three or four, a float32 query four (16 bits).  The probabilities are split the same way
+// before P*V.
 //
 // Per 32 keys a lane loads two 16-byte pieces of each of two keys (A operand of S^T = K Q^T; the
 // contraction order is permuted identically for Q) and eight 8-byte pieces of V, one from each
@@ -24,6 +29,7 @@
 // (measured with a memory-only model of this kernel's work split).
 #include <algorithm>
 #include <atomic>
+#include <type_traits>
 
 #include "common.h"
 
@@ -76,20 +82,23 @@ __device__ __forceinline__ f32x2 fp8x2_to_f32(uint32_t w) {
 // The split x = t0 + t1 + t2 into e4m3 terms for a pair of values; each lane keeps one term, picked
 // with the lane's masks (0xffff for its own term, 0 elsewhere; all 0 for a dead column).  Written
 // without branches: every lane computes all terms, which costs less than divergent control flow.
-struct PartMask { uint32_t m0, m1, m2; };
-template <int PARTS>
-__device__ __forceinline__ uint32_t split_pair(float a, float b, const PartMask& pm) {
-  const uint32_t w0 = fp8x2(a, b);
-  f32x2 d = fp8x2_to_f32(w0);
-  a -= d[0], b -= d[1];
-  const uint32_t w1 = fp8x2(a, b);
-  uint32_t w = (w0 & pm.m0) | (w1 & pm.m1);
-  if (PARTS == 3) {
-    d = fp8x2_to_f32(w1);
-    a -= d[0], b -= d[1];
-    w |= fp8x2(a, b) & pm.m2;
+// Term number PARTS * pass + j goes to the lanes of column group j in pass `pass`.
+struct PartMask { uint32_t m[4]; };
+template <int PARTS, int PASSES>
+__device__ __forceinline__ void split_pair(float a, float b, const PartMask& pm, uint32_t (&w)[PASSES]) {
+#pragma unroll
+  for (int ps = 0; ps < PASSES; ++ps) {
+    w[ps] = 0u;
+#pragma unroll
+    for (int j = 0; j < PARTS; ++j) {
+      const uint32_t t = fp8x2(a, b);
+      w[ps] |= t & pm.m[j];
+      if (ps * PARTS + j + 1 < PARTS * PASSES) {
+        const f32x2 d = fp8x2_to_f32(t);
+        a -= d[0], b -= d[1];
+      }
+    }
   }
-  return w;
 }
 
 // x + (x rotated right by N lanes inside each row of 16 lanes): one VALU op with a DPP modifier
@@ -101,7 +110,8 @@ __device__ __forceinline__ float add_row_ror(float x) {
 // sum over the split-term columns n, n+RS, ... of a 16-lane row (all lanes get the total)
 template <int PARTS>
 __device__ __forceinline__ float sum_parts(float x) {
-  if (PARTS == 3) x = add_row_ror<4>(x);
+  if (PARTS == 1) return x;
+  if (PARTS >= 3) x = add_row_ror<4>(x);  // (three terms: the fourth column group is dead and adds zeros)
   return add_row_ror<8>(x);
 }
 
@@ -129,17 +139,17 @@ __device__ __forceinline__ int steps_per_wave(int total, int n_waves, int t_min)
 // While an item streams, the query rows of the next one are already in flight (they wait in
 // registers), and its first K/V tile is requested before the epilogue of the current one, so the
 // memory pipe of a wavefront never drains between items.
-template <typename TQ, int PARTS>
+template <typename TQ, int PARTS, int PASSES>
 __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
-  constexpr int RS = PARTS == 3 ? 4 : 8;  // column stride between split terms
+  constexpr int RS = PARTS >= 3 ? 4 : PARTS == 2 ? 8 : 16;  // column stride between split terms
   constexpr int QV = sizeof(TQ) == 4 ? 8 : 4;  // 16-byte loads per 32 query elements
   const int lane = threadIdx.x;
   const int n = lane & 15, g = lane >> 4;
   const int part = n / RS, r = n % RS;
   const int rep = p.Hq / p.Hkv;
   const bool col_live = r < p.R && part < PARTS;
-  const PartMask pm = {col_live && part == 0 ? 0xffffu : 0u, col_live && part == 1 ? 0xffffu : 0u,
-                       col_live && part == 2 ? 0xffffu : 0u};
+  const PartMask pm = {{col_live && part == 0 ? 0xffffu : 0u, col_live && part == 1 ? 0xffffu : 0u,
+                        col_live && part == 2 ? 0xffffu : 0u, col_live && part == 3 ? 0xffffu : 0u}};
   const int rr = min(r, p.R - 1);
   const int hq_off = rr % rep, lq = rr / rep;
 
@@ -242,7 +252,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   // The lane owns d = 16g .. 16g+15 and 64+16g .. 64+16g+15 of row r, as for K; MFMA steps 0, 1
   // consume the first group, steps 2, 3 the second.
   // Returns the factor that turns a raw fp8 dot product into a log2-domain logit.
-  auto convert_q = [&](const Item& it, long (&qb)[4]) -> float {
+  auto convert_q = [&](const Item& it, long (&qb)[PASSES][4]) -> float {
     float qv[32];
     {
       typedef __attribute__((ext_vector_type(16 / sizeof(TQ)))) TQ qvec_t;
@@ -263,11 +273,12 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
 #pragma unroll
     for (int ks = 0; ks < 4; ++ks) {
-      uint32_t w[4];
+      uint32_t w[4][PASSES];
 #pragma unroll
       for (int jq = 0; jq < 4; ++jq)
-        w[jq] = split_pair<PARTS>(qv[ks * 8 + 2 * jq] * f, qv[ks * 8 + 2 * jq + 1] * f, pm);
-      qb[ks] = as_long(w[0] | (w[1] << 16), w[2] | (w[3] << 16));
+        split_pair<PARTS, PASSES>(qv[ks * 8 + 2 * jq] * f, qv[ks * 8 + 2 * jq + 1] * f, pm, w[jq]);
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) qb[ps][ks] = as_long(w[0][ps] | (w[1][ps] << 16), w[2][ps] | (w[3][ps] << 16));
     }
     return p.scale * it.kscale / f * kLog2e;
   };
@@ -276,7 +287,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   Item cur = decode_item(G);
   fetch_q(cur);
   load(ra, cur, 0);
-  long qb[4];
+  long qb[PASSES][4];
   float c_row = convert_q(cur, qb);
 
   while (true) {
@@ -308,7 +319,8 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
         for (int ks = 0; ks < 4; ++ks) {
           const u32x4 kk = R_.k[blk][ks >> 1];
           const long a = as_long(kk[(ks & 1) * 2], kk[(ks & 1) * 2 + 1]);
-          sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, qb[ks], sacc[blk], 0, 0, 0);
+#pragma unroll
+          for (int ps = 0; ps < PASSES; ++ps) sacc[blk] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, qb[ps][ks], sacc[blk], 0, 0, 0);
         }
       }
       float t[8];
@@ -336,11 +348,13 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
 #pragma unroll
       for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
       // P^T (B operand): key slot s of this lane is key 4 s + g, the order V is loaded in
-      uint32_t pw[4];
+      uint32_t pw[4][PASSES];
 #pragma unroll
       for (int jq = 0; jq < 4; ++jq)
-        pw[jq] = split_pair<PARTS>(pv[2 * jq] * kPScale, pv[2 * jq + 1] * kPScale, pm);
-      const long pb = as_long(pw[0] | (pw[1] << 16), pw[2] | (pw[3] << 16));
+        split_pair<PARTS, PASSES>(pv[2 * jq] * kPScale, pv[2 * jq + 1] * kPScale, pm, pw[jq]);
+      long pb[PASSES];
+#pragma unroll
+      for (int ps = 0; ps < PASSES; ++ps) pb[ps] = as_long(pw[0][ps] | (pw[1][ps] << 16), pw[2][ps] | (pw[3][ps] << 16));
       // O^T += V^T P^T : the lane holds bytes d = 8n + e (e = 0 .. 7) of its eight keys; matrix op e
       // takes byte e of every key (rows d = 8n + e), an 8 x 8 byte transpose done as four 4 x 4 ones
 #pragma unroll
@@ -362,8 +376,10 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
         }
 #pragma unroll
         for (int jq = 0; jq < 4; ++jq)
-          oacc[hf * 4 + jq] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(
-              as_long(o_lo[jq], o_hi[jq]), pb, oacc[hf * 4 + jq], 0, 0, 0);
+#pragma unroll
+          for (int ps = 0; ps < PASSES; ++ps)
+            oacc[hf * 4 + jq] = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(
+                as_long(o_lo[jq], o_hi[jq]), pb[ps], oacc[hf * 4 + jq], 0, 0, 0);
       }
     };
 
@@ -384,7 +400,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     } while (s < steps);
     // all tiles of this item are consumed; what is in flight is the next item's first tile, and
     // its query rows landed long ago: build its fragment now, ahead of the stores below
-    long qb_next[4];
+    long qb_next[PASSES][4];
     float c_next = 0.f;
     if (more) c_next = convert_q(nxt, qb_next);
 
@@ -412,7 +428,9 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     cur = nxt;
     c_row = c_next;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) qb[ks] = qb_next[ks];
+    for (int ps = 0; ps < PASSES; ++ps)
+#pragma unroll
+      for (int ks = 0; ks < 4; ++ks) qb[ps][ks] = qb_next[ps][ks];
   }
 }
 
@@ -505,10 +523,26 @@ int min_steps_for(const mi355_sdpa_decode_params& p) {
   return t;
 }
 
+// Terms per query element (and per probability): enough for the query's significant bits at four bits
+// a term - bf16 two (three where the columns are free anyway), float16 three or four, float32 four -
+// laid out as PARTS column groups per matrix op times PASSES trips through the matrix ops, by the
+// number of query rows R that share the 16 columns.
 template <typename TQ>
 int launch_t(const DecP& g, hipStream_t s) {
-  if (g.R <= 4) hipLaunchKernelGGL((decode_kernel<TQ, 3>), dim3(g.n_waves), dim3(64), 0, s, g);
-  else hipLaunchKernelGGL((decode_kernel<TQ, 2>), dim3(g.n_waves), dim3(64), 0, s, g);
+  constexpr bool BF = std::is_same<TQ, bf16_t>::value, F32 = sizeof(TQ) == 4;
+#define DECODE(PARTS, PASSES) hipLaunchKernelGGL((decode_kernel<TQ, PARTS, PASSES>), dim3(g.n_waves), dim3(64), 0, s, g)
+  if (g.R <= 4) {
+    if constexpr (F32) DECODE(4, 1);
+    else DECODE(3, 1);
+  } else if (g.R <= 8) {
+    if constexpr (BF) DECODE(2, 1);
+    else DECODE(2, 2);
+  } else {
+    if constexpr (BF) DECODE(1, 2);
+    else if constexpr (F32) DECODE(1, 4);
+    else DECODE(1, 3);
+  }
+#undef DECODE
   int rc = check_launch("decode_kernel");
   if (rc) return rc;
   hipLaunchKernelGGL((decode_merge_kernel<TQ>), dim3(g.B * g.Hkv * g.R), dim3(D), 0, s, g);
@@ -561,8 +595,8 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
   if (p.q.size[3] != D || p.v.size[3] != D)
     return set_error("SDPA decode: head dim must be 128, got %lld/%lld", (long long)p.q.size[3],
                      (long long)p.v.size[3]), MI355_SDPA_ERR_UNSUPPORTED;
-  if (g.R < 1 || g.R > 8)
-    return set_error("SDPA decode: Lq * Hq/Hkv must be in [1, 8], got %d", g.R), MI355_SDPA_ERR_UNSUPPORTED;
+  if (g.R < 1 || g.R > 16)
+    return set_error("SDPA decode: Lq * Hq/Hkv must be in [1, 16], got %d", g.R), MI355_SDPA_ERR_UNSUPPORTED;
   if (p.q.stride[3] != 1 || p.k.stride[3] != 1 || p.v.stride[3] != 1 || p.out.stride[3] != 1)
     return set_error("SDPA decode: head dim must be unit-stride"), MI355_SDPA_ERR_UNSUPPORTED;
   if (((uintptr_t)p.k.data & 15) || ((uintptr_t)p.v.data & 15) || (p.k.stride[2] & 15) || (p.v.stride[2] & 15) ||
