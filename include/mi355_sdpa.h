@@ -141,6 +141,12 @@ typedef struct mi355_sdpa_mask_spec {
   const int32_t* doc_ids_q;
   const int32_t* doc_ids_k;
   int32_t doc_ids_sorted;
+  const int32_t* mask_verdict; /* optional, with a bias / keep-mask: what mi355_sdpa_mask_verdict wrote
+                                  about that tensor.  The matrix-op kernels for 16-bit inputs at head
+                                  dims up to 128 read it in their prologue and, when the mask is the
+                                  keep-everything or the causal pattern (with or without right padding),
+                                  run as if is_causal / kv_lens had been given and never read the mask;
+                                  every other kernel, and every other verdict, uses the mask itself   */
 } mi355_sdpa_mask_spec;
 
 typedef struct mi355_sdpa_fwd_params {
@@ -266,6 +272,20 @@ int mi355_sdpa_decode_fp8kv_static(const mi355_sdpa_decode_params* p, void* stre
  *   torch_neuronx/neuron_dynamo_backend/fx/passes/sdpa_causal_mask.py:162-289 (SdpaCausalMaskRewrite). */
 int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, int64_t S, int64_t row_stride,
                          int32_t* rows_out, void* stream);
+
+/* The same decision taken on the device, with no trip to the host: row summaries of every (mask
+ * batch, row) and a verdict, in `verdict` (mi355_sdpa_mask_verdict_words(mask) int32 of device
+ * memory; 0 = this mask cannot have one: it depends on the head, its keys are not unit-stride):
+ *   verdict[0] kind: 0 not a pattern, 1 keep-everything, 2 causal, 3 sliding window with sink keys
+ *   verdict[1] window, verdict[2] sink keys, verdict[3] 1 if some batch keeps fewer than S keys
+ *   verdict[8 + b] keys of batch b that take part (right padding under kinds 1 and 2)
+ * `mask` is the bias / keep-mask expanded to (B,Hq,L,S), stride 0 on broadcast dims.  Nothing
+ * synchronises: the call records into a HIP graph in front of the attention call that is given
+ * the verdict (mi355_sdpa_mask_spec.mask_verdict), and then follows a mask that is updated in place
+ * between replays.  Stand-in, like mi355_sdpa_mask_rows, for
+ *   torch_neuronx/neuron_dynamo_backend/fx/passes/sdpa_causal_mask.py:162-289. */
+size_t mi355_sdpa_mask_verdict_words(const mi355_sdpa_tensor* mask, int32_t dtype);
+int mi355_sdpa_mask_verdict(const mi355_sdpa_tensor* mask, int32_t dtype, int32_t* verdict, void* stream);
 
 /* Tile skip tables of a bias / keep-mask (sizes (B,Hq,L,S), stride 0 on broadcast dims, unit stride
  * over keys, rows and data dword aligned as the MFMA kernels want them; bool, or float where

@@ -278,5 +278,5 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
         assert scratch == 0, (name, scratch)
         assert r["Dynamic_Stack"] == "False"
     for name, r in fwd.items():
-        d = int(re.search(r"Li(\d+)ELi\d+ELi\d+EE", name).group(1))
+        d = int(re.search(r"Li(\d+)ELi\d+ELi\d+E(?:Lb[01]E)?E", name).group(1))
         assert int(r["Occupancy_[waves/SIMD]"]) >= (1 if d > 128 else 2), name

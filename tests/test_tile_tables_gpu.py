@@ -191,9 +191,13 @@ def test_document_mask_through_the_operator_skips_tiles(amd, gpu_device):
     mask_patterns.clear_cache()
     before = dict(mask_patterns.stats)
     op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
-    out = op(q, k, v, attn_bias=mask)[0]
+    first = op(q, k, v, attn_bias=mask)[0]  # first sight: nothing is known about the mask yet, it is taken as it is
+    torch.cuda.synchronize()
+    assert mask_patterns.stats.get("tile_builds", 0) == before.get("tile_builds", 0)
+    out = op(q, k, v, attn_bias=mask)[0]  # known to be no pattern by now: tables
     out2 = op(q, k, v, attn_bias=mask)[0]
     torch.cuda.synchronize()
+    assert max_abs(first, out) <= 1e-6
     assert mask_patterns.stats.get("tile_builds", 0) - before.get("tile_builds", 0) == 1
     assert mask_patterns.stats.get("tile_hits", 0) - before.get("tile_hits", 0) == 1
     ref, _ = amd.sdpa_forward(q, k, v, attn_bias=mask, force_kernel=MFMA)

@@ -42,7 +42,7 @@ constexpr int smem_bytes() {  // three Q and three dO tiles, two P hand-over buf
 // functors and document ids of score_mod.h: role A rewrites its score tile in a block of its own
 // and hands P times the derivative of the functors to role B, which forms dS from it.
 template <typename T, int D, int MASK>
-__global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
+__device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs ma) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
   constexpr int TILE = BQ * D;           // tiles are XOR swizzled, not padded: see tile_swz
   constexpr int NCH = BQ * CH / 512;     // 16-byte chunks of a tile per thread
@@ -89,7 +89,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int dr = MASK ? p.d_real : D;  // elements per row that exist
   int S = p.S;  // keys of this batch that take part
   if constexpr (MASK) {
-    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
   }
   // this lane's key as B operand: K fragments for S = Q K^T (role A), V fragments for dP = dO V^T (role B)
   u32x4 frag[KS];
@@ -120,11 +120,11 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
   // the query rows that see this lane's key are first_q .. past_q - 1: from the key itself on under a
   // causal mask, none for a key past the batch's count, up to the end of the key's window unless it is a sink
-  const int first_q = key >= S ? INT_MAX : p.causal ? key : INT_MIN;
+  const int first_q = key >= S ? INT_MAX : ma.causal ? key : INT_MIN;
   const int past_q = (W > 0 && key >= n_sink) ? key + W : INT_MAX;
   const bool listed = MASK == 2 && p.live_t != nullptr;
   const int nqs = (p.L + BQ - 1) / BQ;
-  int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+  int qs_begin = ma.causal ? min(k0 / BQ, nqs) : 0;
   int qs_end = (W > 0 && k0 >= n_sink) ? max(min(nqs, (k0 + BK + W - 2) / BQ + 1), qs_begin) : nqs;
   // document ids (MASK = 4): this lane's key id; with ids sorted along the sequence the rows whose id
   // lies between the ids of the block's first and last key are one run, found by two searches over
@@ -320,7 +320,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     }
   };
 
-  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;
   const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
   const uint32_t b_rowbytes = BIASED ? (uint32_t)(p.bias_sl * besz) : 0u;
   const uint32_t b_lane = BIASED ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   auto load_bias_a = [&](int it) {
     if constexpr (BIASED) {
       const int q0 = item_q0(it);
-      if (it >= n_items || (p.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
+      if (it >= n_items || (ma.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
       const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
           uniform_ptr((const char*)p.bias + (b * p.bias_sb + item_head(it) * p.bias_sh) * besz), 0, b_records, 0x00020000);
       const uint32_t base = b_lane + (uint32_t)q0 * b_rowbytes;
@@ -395,8 +395,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
     // (the functors' derivative differs from one: the dK wavefronts get P times it, see hand_over)
     const bool need_dfac = SMOD && (p.sm.key_weight != nullptr || p.sm.softcap > 0.f);
     if constexpr (MASK == 1) {
-      if (p.bias_kind)
-        bl = bias_value(p.bias, b * p.bias_sb + item_head(it) * p.bias_sh + min(key, p.S - 1), p.bias_kind) * kLog2eF;
+      if (ma.bias_kind)
+        bl = bias_value(p.bias, b * p.bias_sb + item_head(it) * p.bias_sh + min(key, p.S - 1), ma.bias_kind) * kLog2eF;
     }
     const uint16_t* qt = q_t + tb * TILE;
     const uint16_t* dot = do_t + tb * TILE;
@@ -546,12 +546,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
         if (!compact && !((__builtin_amdgcn_readfirstlane((int)live_s[hg * p.live_t_words + (qt >> 5)]) >> (qt & 31)) & 1)) return true;
       }
     }
-    return (p.causal && q0 + BQ - 1 < kw0) || kw0 >= S || (W > 0 && q0 - kw0 - 31 >= W && kw0 >= n_sink);
+    return (ma.causal && q0 + BQ - 1 < kw0) || kw0 >= S || (W > 0 && q0 - kw0 - 31 >= W && kw0 >= n_sink);
   };
   auto role_a = [&](int it, int tb, int pb) {
     const int q0 = item_q0(it);
     if (dead_tile(it, tb)) return;
-    bool edge = (p.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
+    bool edge = (ma.causal && q0 < kw0 + 31) || (kw0 + 31 >= S) || (W > 0 && q0 + BQ - 1 - kw0 >= W && kw0 + 31 >= n_sink);
     if constexpr (SMOD) {
       // every score compared, unless (sorted ids) the wavefront's keys carry one id and the tile's rows lie
       // inside the run of rows with that id
@@ -721,11 +721,26 @@ __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
   }
 }
 
+// The kernel of a variant.  A call whose bias comes with a verdict about it (see MaskArgs) is launched
+// twice: as the variant with a bias (MASK = 2), and as the variant with key counts marked PATTERN; the
+// verdict lets one of them run.
+template <typename T, int D, int MASK, bool PATTERN = false>
+__global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
+  static_assert(!PATTERN || MASK == 1, "the pattern kernel is the variant with key counts");
+  MaskArgs ma = mask_args_of(p);
+  if constexpr (MASK == 2 || PATTERN) {
+    if (verdict_pattern(p, ma) != PATTERN) return;
+  }
+  bwd_dkdv_w32_body<T, D, MASK>(p, ma);
+}
+
 // Sum of the parts' float32 rows, one 64-thread block per key row of a (batch, kv head): four columns
 // per thread, dK's d_real columns first, dV's dv_real behind them.  The factors that the kernels apply
 // when they write dK and dV themselves are applied here: the scale for dK, 1 / (1 - p) of dropout for dV.
 template <typename T>
 __global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
+  MaskArgs ma = mask_args_of(p);
+  verdict_pattern(p, ma);  // (the item counts below are those of the kernel that filled the parts)
   const int64_t row = blockIdx.x;  // (b * Hkv + hk) * S + key
   const int key = (int)(row % p.S);
   const int hk = (int)((row / p.S) % p.Hkv), b = (int)(row / ((int64_t)p.S * p.Hkv));
@@ -736,8 +751,8 @@ __global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
     // the parts that bwd_dkdv_w32_kernel filled for this row's key block: its items, counted as there
     const int k0 = key / BK * BK, nqs = (p.L + BQ - 1) / BQ;
     int S = p.S;
-    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
-    const int qs_begin = p.causal ? min(k0 / BQ, nqs) : 0;
+    if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
+    const int qs_begin = ma.causal ? min(k0 / BQ, nqs) : 0;
     const int qs_end = (p.window > 0 && k0 >= p.sink_keys) ? max(min(nqs, (k0 + BK + p.window - 2) / BQ + 1), qs_begin) : nqs;
     const int n_items = k0 >= S ? 0 : (p.Hq / p.Hkv / p.parts_h) * (qs_end - qs_begin);
     parts = min(max((n_items + p.chunk_items - 1) / p.chunk_items, 1), p.parts / p.parts_h) * p.parts_h;
@@ -803,19 +818,19 @@ __global__ __launch_bounds__(256) void bwd_key_order_kernel(BwdM p) {
   }
 }
 
-template <typename T, int D, int MASK>
+template <typename T, int D, int MASK, bool PATTERN = false>
 int launch_t(const BwdM& g, hipStream_t s) {
   // (MASK = 2: with the skip table's row of the key block and the item list; MASK = 4: with the document ids of three tiles' rows)
   constexpr int kSmemBytes = smem_bytes<D>() + (MASK == 2 ? 1024 + 2048 + 16 : MASK == 4 ? 3 * BQ * 4 : 0);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D, MASK>,
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D, MASK, PATTERN>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dkdv_w32_kernel: %s", kSmemBytes, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D, MASK>), dim3((unsigned)(g.B * g.Hkv * g.n_kt * g.parts)), dim3(512), kSmemBytes, s, g);
+  hipLaunchKernelGGL((bwd_dkdv_w32_kernel<T, D, MASK, PATTERN>), dim3((unsigned)(g.B * g.Hkv * g.n_kt * g.parts)), dim3(512), kSmemBytes, s, g);
   const int rc = check_launch("bwd_dkdv_w32_kernel");
-  if (rc != MI355_SDPA_OK || g.parts == 1) return rc;
+  if (rc != MI355_SDPA_OK || g.parts == 1 || PATTERN) return rc;  // (the parts are added up once, behind the other kernel of the pair)
   return launch_bwd_dkdv_merge(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
 }
 template <typename T, int D>
@@ -833,7 +848,12 @@ int launch_m(const BwdM& g, hipStream_t s) {
     return launch_t<T, D, 4>(g, s);
   }
   if (g.keep_scale != 0.f) return launch_t<T, D, 3>(g, s);
-  if (g.bias_kind && g.bias_sl != 0) return launch_t<T, D, 2>(g, s);
+  if (g.bias_kind && g.bias_sl != 0) {
+    if (g.verdict) {  // (see bwd_dkdv_w32_kernel)
+      if (int rc = launch_t<T, D, 1, true>(g, s)) return rc;
+    }
+    return launch_t<T, D, 2>(g, s);
+  }
   return (g.bias_kind || g.kv_lens || g.d_real != D || g.window > 0) ? launch_t<T, D, 1>(g, s) : launch_t<T, D, 0>(g, s);
 }
 

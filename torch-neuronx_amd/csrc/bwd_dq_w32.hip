@@ -33,7 +33,7 @@ constexpr int AHEAD = 2;  // LDS operands are requested this many matrix ops ahe
 // of score_mod.h, applied to the score tile (and their derivative to dP - delta) in a block of its
 // own ahead of the tile's vector work.
 template <typename T, int D, int MASK>
-__global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
+__device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma) {
   constexpr int KS = D / 16, DB = D / 32, CH = D / 8;
   constexpr int TILE = BN * D;
   constexpr int TCH = BN * CH;        // 16-byte chunks per tile
@@ -132,7 +132,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   };
   int S = p.S;  // keys of this batch that take part
   if constexpr (MASK) {
-    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
   }
   auto zero_row = [&]() {  // no live key: zero gradient
     zero_gbias(0);
@@ -155,7 +155,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   constexpr bool FUNC = MASK == 1 || MASK == 4;
   constexpr bool SMOD = MASK == 4;  // score functors, document ids
   int nt = (S + BN - 1) / BN;
-  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+  if (ma.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   int n_lead = 0, skip = 0;
   // (document ids sorted along the sequence: the keys that this wavefront's rows can see, and whether
   // those rows all belong to one document)
@@ -197,7 +197,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // workgroup's 64-row blocks and expands the set bits into a list in LDS, 64 tiles per step.
   bool listed = false;
   if constexpr (MASK == 2) {
-    if (p.live_tiles && !p.causal && !p.gbias) {
+    if (p.live_tiles && !ma.causal && !p.gbias) {
       if (wave == 0) {
         const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
         const uint32_t* map = p.live_tiles + ((int64_t)((p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? h : 0)) * nrb + rb0) * p.live_words;
@@ -227,12 +227,12 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
     if constexpr (MASK == 2) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
     else return FUNC ? u + (u >= n_lead ? skip : 0) : u;
   };
-  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BN + 1 - skip) : nt;  // tiles with work for this wavefront
+  const int nt_w = ma.causal ? min(nt, (qw0 + 31) / BN + 1 - skip) : nt;  // tiles with work for this wavefront
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile; with a window also every tile that
   // reaches below the window of the wavefront's last row and is not made of sink keys alone
-  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
-  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  const int t_edge = min(ma.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
+  const int lim = ma.causal ? min(qrow, S - 1) : S - 1;
   const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
   const int n_sink = FUNC ? p.sink_keys : 0;
   auto edge_tile = [&](int u) {
@@ -444,7 +444,7 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   // The resource starts at this wavefront's first row of the (batch, head) plane and ends with its
   // last one: keys past S read the next row or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
-  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;
+  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;
   const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const int b_rows = min(32, p.L - qw0);
   const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * besz : 0),
@@ -693,6 +693,19 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   }
 }
 
+// The kernel of a variant.  A call whose bias comes with a verdict about it (see MaskArgs) is launched
+// twice: as the variant with a bias (MASK = 2), and as the variant with key counts marked PATTERN; the
+// verdict lets one of them run.
+template <typename T, int D, int MASK, bool PATTERN = false>
+__global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
+  static_assert(!PATTERN || MASK == 1, "the pattern kernel is the variant with key counts");
+  MaskArgs ma = mask_args_of(p);
+  if constexpr (MASK == 2 || PATTERN) {
+    if (verdict_pattern(p, ma) != PATTERN) return;
+  }
+  bwd_dq_w32_body<T, D, MASK>(p, ma);
+}
+
 }  // namespace
 
 bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
@@ -727,6 +740,8 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
 #define LAUNCH(TT, DD, MM) hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, MM>), grid, block, ((MM) == 2 || (MM) == 3) ? dyn : 0, s, g)
 #define LAUNCH_M(TT, DD)                                                     \
   do {                                                                       \
+    if (mask == 2 && g.verdict) /* (see bwd_dq_w32_kernel) */                \
+      hipLaunchKernelGGL((bwd_dq_w32_kernel<TT, DD, 1, true>), grid, block, 0, s, g); \
     if (mask == 4) LAUNCH(TT, DD, 4);                                        \
     else if (mask == 3) LAUNCH(TT, DD, 3);                                   \
     else if (mask == 2) LAUNCH(TT, DD, 2);                                   \

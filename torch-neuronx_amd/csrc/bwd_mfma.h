@@ -71,6 +71,9 @@ struct BwdM {
   // block with fewer items - a causal mask, a window, a batch with fewer keys - fills fewer parts;
   // the others are neither written nor read).  0: every key block uses all `parts`, in equal shares.
   int chunk_items = 0;
+  // a verdict about the bias (mask_rows.hip), read by the variants with a per-score bias in their
+  // prologue: see apply_verdict
+  const int32_t* verdict = nullptr;
 };
 
 // parts the dK/dV kernel of bwd_dkdv_w32.hip / of bwd_wide.hip would use for this call

@@ -62,6 +62,9 @@ struct FwdM {
   // live_hm = the mask's own head extent
   const uint32_t* live_tiles = nullptr;
   int live_words = 0, live_hm = 1;
+  // a verdict about the bias (mask_rows.hip), read by the variants with a per-score bias in their
+  // prologue: see apply_verdict
+  const int32_t* verdict = nullptr;
 };
 
 // Decode blockIdx.x -> (batch, query head, query tile).  Tiles are issued heaviest first

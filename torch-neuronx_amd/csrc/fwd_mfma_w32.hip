@@ -52,7 +52,7 @@ constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescale
 // they rewrite the raw score tile in a block of its own right after the matrix ops that produce it,
 // where the bias of MASK = 2 is folded in, so the softmax behind them is the common code.
 template <typename T, int D, int WAVES, int MASK>
-__global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
+__device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   constexpr int BM = 32 * WAVES, NT = 64 * WAVES;
   constexpr int KS = D / 16;      // matrix ops of S^T = K Q^T per tile (phase A)
   constexpr int DB = D / 32;      // 32-row blocks of O^T
@@ -108,12 +108,12 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // keys of this batch that take part
   int S = p.S;
   if constexpr (MASK) {
-    if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
+    if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
     if constexpr (MASK == 2) {
       // A keep-mask per key (no row stride: padding masks): the keys behind the last one it keeps are
       // never visited, as with a key count.  Every wavefront scans the row itself (S bytes, four
       // per lane and step; rows are whole dwords) and they all arrive at the same count.
-      if (p.bias_kind == 4 && p.bias_sl == 0 && S > 0) {
+      if (ma.bias_kind == 4 && p.bias_sl == 0 && S > 0) {
         const uint8_t* mrow = (const uint8_t*)p.bias + b * p.bias_sb + h * p.bias_sh;
         int last = -1;
         for (int j = lane * 4; j < S; j += 256) {
@@ -130,7 +130,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // lowest window of its rows are dropped whole, except the leading ones that hold sink keys: stream
   // position u is key tile u + (u >= n_lead ? skip : 0).
   int nt = (S + BN - 1) / BN;
-  if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
+  if (ma.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BN + 1);
   int n_lead = 0, skip = 0;
   // (document ids sorted along the sequence: the keys that this wavefront's rows can see, and whether
   // those rows all belong to one document)
@@ -174,7 +174,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // workgroup's 64-row blocks and expands the set bits into a list in LDS, 64 tiles per step.
   bool listed = false;
   if constexpr (MASK == 2) {
-    if (p.live_tiles && !p.causal) {
+    if (p.live_tiles && !ma.causal) {
       listed = true;
       if (wave == 0) {
         const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
@@ -262,7 +262,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
     }
   };
 
-  const int nt_w = p.causal ? min(nt, qw_last / BN + 1 - skip) : nt;
+  const int nt_w = ma.causal ? min(nt, qw_last / BN + 1 - skip) : nt;
 
   // K and V are read through buffer resources that end with the last key row of this (batch, head);
   // the whole offset travels in the vector offset, the part the hardware checks against that bound:
@@ -380,7 +380,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   float m_run = -INFINITY, l_run = 0.f;
   const float c = p.scale * kLog2eF;
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
-  const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  const int lim = ma.causal ? min(qrow, S - 1) : S - 1;
   // (window: keys below lo_w are dropped unless they are sink keys)
   const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
   const int n_sink = FUNC ? p.sink_keys : 0;
@@ -410,7 +410,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   // younger loads are those of the pair requested at the end of the previous iteration.
   uint32_t braw[4];
   float inv_scale = 0.f;
-  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int b_esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const int b_rows = min(32, p.L - qw0);
   const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * b_esz : 0),
@@ -571,7 +571,7 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 
   // first tile that needs masking: the one that reaches this wavefront's first row on the causal
   // diagonal (qw0 is a multiple of BN), or a ragged last tile
-  const int t_edge = min(p.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
+  const int t_edge = min(ma.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
   // ... or, with a window, a tile that reaches below the window of this wavefront's last row and
   // is not made of sink keys alone.  (Stream position -> does the tile need masking.)
   auto edge = [&](int u) {
@@ -884,6 +884,23 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   if (qrow < p.L && p.lse && half == 0) p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
 }
 
+// The kernel of a variant.  A call whose bias comes with a verdict about it (see MaskArgs) is launched
+// twice: as the variant with a bias (MASK = 2), and as the variant with key counts marked PATTERN.  The
+// verdict lets one of them run: a bias that is the keep-everything or the causal pattern, with or
+// without right padding, is never read - the PATTERN kernel generates it, at the speed of a call that
+// was made with the causal flag - and any other bias leaves that kernel's workgroups nothing to do.
+// (Two kernels rather than one that branches: both variants in one kernel need more scalar registers
+// than there are, and the variant with a bias pays for its bias slot even when the slot is empty.)
+template <typename T, int D, int WAVES, int MASK, bool PATTERN = false>
+__global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_kernel(FwdM p) {
+  static_assert(!PATTERN || MASK == 1, "the pattern kernel is the variant with key counts");
+  MaskArgs ma = mask_args_of(p);
+  if constexpr (MASK == 2 || PATTERN) {
+    if (verdict_pattern(p, ma) != PATTERN) return;
+  }
+  fwd_w32_body<T, D, WAVES, MASK>(p, ma);
+}
+
 // Merge of the parts of a call whose keys were split: out = sum_s w_s O_s with w_s = exp(lse_s - lse),
 // lse = log sum_s exp(lse_s).  One workgroup per query row, one thread per output element.
 template <typename T>
@@ -917,14 +934,14 @@ __global__ __launch_bounds__(128) void fwd_split_merge_kernel(FwdM p) {
 }
 
 // one instantiation; head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare
-template <typename T, int D, int WAVES, int MASK>
+template <typename T, int D, int WAVES, int MASK, bool PATTERN = false>
 int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
   int bytes = 0;
   if constexpr (D > 128 || MASK == 2 || MASK == 3) {
     // (four buffers per operand, 4 KB of bias tile per wavefront, and the tile list of a call with a skip table)
     constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK >= 2 ? WAVES * 4096 : 0);
     constexpr int kBytes = kBase + (MASK == 2 ? 2048 + 16 : 0);
-    static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK>,
+    static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK, PATTERN>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
     if (attr != hipSuccess) {
       set_error("SDPA: cannot reserve %d bytes of LDS for fwd_w32_kernel: %s", kBytes, hipGetErrorString(attr));
@@ -932,7 +949,7 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
     }
     bytes = (MASK == 2 && g.live_tiles) ? kBytes : kBase;
   }
-  hipLaunchKernelGGL((fwd_w32_kernel<T, D, WAVES, MASK>), grid, dim3(64 * WAVES), bytes, s, g);
+  hipLaunchKernelGGL((fwd_w32_kernel<T, D, WAVES, MASK, PATTERN>), grid, dim3(64 * WAVES), bytes, s, g);
   return MI355_SDPA_OK;
 }
 template <typename T, int D, int WAVES>
@@ -941,7 +958,12 @@ int launch_mask(const FwdM& g, int mask, dim3 grid, hipStream_t s) {
     if (mask == 4) return launch_one<T, D, WAVES, 4>(g, grid, s);
     if (mask == 3) return launch_one<T, D, WAVES, 3>(g, grid, s);
   }
-  if (mask == 2) return launch_one<T, D, WAVES, 2>(g, grid, s);
+  if (mask == 2) {
+    if (g.verdict) {  // (see fwd_w32_kernel)
+      if (int rc = launch_one<T, D, WAVES, 1, true>(g, grid, s)) return rc;
+    }
+    return launch_one<T, D, WAVES, 2>(g, grid, s);
+  }
   if (mask == 1) return launch_one<T, D, WAVES, 1>(g, grid, s);
   return launch_one<T, D, WAVES, 0>(g, grid, s);
 }
@@ -991,6 +1013,7 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
     }
   }
   g.n_qt = g.grouped ? 1 : (g.L + 32 * waves - 1) / (32 * waves);
+  if (g.grouped) g.verdict = nullptr;  // (few rows: the mask is taken as it is)
 }
 
 size_t fwd_w32_workspace(const FwdM& g0, int head_dim, int waves) {

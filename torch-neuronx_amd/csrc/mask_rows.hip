@@ -89,6 +89,184 @@ extern "C" int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, 
   return check_launch("mask_rows_kernel");
 }
 
+// ---- the verdict, on the device -------------------------------------------------------------------
+// The same decision without a trip to the host: a row summary of every (mask batch, row), and one
+// workgroup that holds the summaries against the patterns.  The verdict stays in device memory, where
+// the masked variants of the forward and backward kernels read it in their prologue and, for a mask
+// that is a pattern, drop the mask in favour of the causal flag and per-batch key counts.  Nothing
+// here synchronises, so the whole sequence records into a HIP graph and follows a mask that is
+// updated in place between replays.
+//   verdict[0] kind: 0 not a pattern, 1 keep-everything, 2 causal, 3 sliding window with sink keys
+//   verdict[1] window   verdict[2] sink keys   verdict[3] 1 if some batch keeps fewer than S keys
+//   verdict[8 + b] keys of batch b that take part (kinds 1 and 2: right padding becomes a key count)
+// and behind them the row summaries, four ints per (mask batch, row).
+namespace mi355 {
+namespace {
+
+struct VerdictArgs {
+  const void* mask;
+  int64_t sb, sl;  // strides of the mask's batch and row dims in elements (0: broadcast)
+  int B, Bm, L, Lm, S;
+  int32_t* verdict;
+  int32_t* rows;
+};
+
+template <typename T>
+__global__ __launch_bounds__(256) void mask_rows_batched_kernel(VerdictArgs a) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= (int64_t)a.Bm * a.Lm) return;
+  const int bm = (int)(row / a.Lm), l = (int)(row % a.Lm);
+  const T* m = (const T*)a.mask + bm * a.sb + l * a.sl;
+  const int S = a.S;
+  // (elements are read sixteen bytes at a time where the row allows it)
+  constexpr int E = 16 / (int)sizeof(T);
+  const bool wide = ((uintptr_t)m & 15) == 0 && S % E == 0;
+  int hi = -1, cnt = 0, lead = S, bad = 0;
+  auto scan = [&](auto&& visit) {
+    if (wide) {
+      for (int j = lane * E; j < S; j += 64 * E) {
+        const uint4 w = *(const uint4*)(m + j);
+        T e[E];
+        __builtin_memcpy(e, &w, 16);
+#pragma unroll
+        for (int i = 0; i < E; ++i) visit(j + i, classify<T>(e[i]));
+      }
+    } else {
+      for (int j = lane; j < S; j += 64) visit(j, classify<T>(m[j]));
+    }
+  };
+  scan([&](int j, int c) {
+    if (c < 0) bad = 1;
+    if (c == 1) hi = max(hi, j), ++cnt;
+    else lead = min(lead, j);
+  });
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) {
+    hi = max(hi, __shfl_xor(hi, o, 64));
+    cnt += __shfl_xor(cnt, o, 64);
+    lead = min(lead, __shfl_xor(lead, o, 64));
+    bad |= __shfl_xor(bad, o, 64);
+  }
+  int gap = -1;  // last dropped key below the last kept one
+  if (cnt != hi + 1) {  // (a row that is one run from key 0 has none)
+    scan([&](int j, int c) {
+      if (j < hi && c != 1) gap = max(gap, j);
+    });
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) gap = max(gap, __shfl_xor(gap, o, 64));
+  }
+  if (lane == 0) {
+    int32_t* out = a.rows + row * 4;
+    out[0] = hi, out[1] = bad ? -1 : cnt, out[2] = lead, out[3] = gap + 1;
+  }
+}
+
+// One workgroup: the rules of mask_patterns.py (pattern_from_rows, lens_pattern_from_rows), held
+// against the row summaries of every mask batch.
+__global__ __launch_bounds__(1024) void mask_verdict_kernel(VerdictArgs a) {
+  const int tid = threadIdx.x;
+  const int L = a.L, Lm = a.Lm, S = a.S;
+  const bool per_row = Lm == L;  // (otherwise one row stands for every query: no causal, no window)
+  int ok_all = 1, ok_causal = per_row && L > 1, ok_mask = 1;
+  for (int bm = 0; bm < a.Bm; ++bm) {
+    const int32_t* rows = a.rows + (int64_t)bm * Lm * 4;
+    const int hi_last = rows[(Lm - 1) * 4];
+    const int n_all = hi_last + 1;
+    const int n_causal = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;  // the last row reaches its diagonal: no key is known to be padding
+    for (int i = tid; i < Lm; i += 1024) {
+      const int hi = rows[i * 4], cnt = rows[i * 4 + 1], lo = rows[i * 4 + 3];
+      if (cnt < 0) ok_mask = 0;
+      if (lo != 0 || hi != n_all - 1 || cnt != n_all) ok_all = 0;
+      const int hc = min(min(i, S - 1), n_causal - 1);
+      if (lo != 0 || hi != hc || cnt != hc + 1) ok_causal = 0;
+    }
+  }
+  ok_mask = __syncthreads_and(ok_mask);
+  ok_all = __syncthreads_and(ok_all) && ok_mask;
+  ok_causal = __syncthreads_and(ok_causal) && ok_mask;
+  int kind = ok_all ? 1 : ok_causal ? 2 : 0, window = 0, sinks = 0;
+  if (!kind && ok_mask && a.Bm == 1 && per_row && L > 1) {
+    // sliding window with sink keys: query i keeps keys i-W+1 .. i and the first N keys
+    const int32_t* rows = a.rows;
+    const int r = L - 1;
+    const int hi_r = rows[r * 4], lead_r = rows[r * 4 + 2], lo_r = rows[r * 4 + 3];
+    const int W = hi_r - lo_r + 1, N = lead_r < lo_r ? lead_r : 0;
+    int ok = W > 0 && lo_r != 0;
+    for (int i = tid; i < L && ok; i += 1024) {
+      const int hi = rows[i * 4], cnt = rows[i * 4 + 1], lead = rows[i * 4 + 2], lo = rows[i * 4 + 3];
+      const int hc = min(i, S - 1), lead_full = hc + 1 < S ? hc + 1 : S;
+      const int lo_w = max(i - W + 1, 0);
+      const bool joined = lo_w <= N;  // the window reaches into the sink keys (or to key 0): one run from key 0
+      if (hi != hc || i - W + 1 > hc) ok = 0;
+      if (lo != (joined ? 0 : lo_w) || lead != (joined ? lead_full : N) || cnt != (joined ? hc + 1 : hc - lo_w + 1 + N)) ok = 0;
+    }
+    if (__syncthreads_and(ok)) kind = 3, window = W, sinks = N;
+  }
+  // key counts per batch (a mask without a batch dim counts for every batch)
+  int short_any = 0;
+  for (int b = tid; b < a.B; b += 1024) {
+    const int bm = a.Bm > 1 ? b : 0;
+    const int hi_last = a.rows[((int64_t)bm * Lm + Lm - 1) * 4];
+    int n = S;
+    if (kind == 1) n = hi_last + 1;
+    else if (kind == 2) n = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;
+    a.verdict[8 + b] = n;
+    short_any |= n != S;
+  }
+  short_any = __syncthreads_or(short_any);
+  if (tid == 0) {
+    a.verdict[0] = kind, a.verdict[1] = window, a.verdict[2] = sinks, a.verdict[3] = short_any;
+    a.verdict[4] = a.verdict[5] = a.verdict[6] = a.verdict[7] = 0;
+  }
+}
+
+// what a verdict needs of the mask: no dependence on the head, unit stride over keys, a known dtype
+bool verdict_shape(const mi355_sdpa_tensor& t, int32_t dtype, int* Bm, int* Lm) {
+  if (!t.data) return false;
+  if (dtype != MI355_SDPA_BOOL && dtype != MI355_SDPA_F32 && dtype != MI355_SDPA_F16 && dtype != MI355_SDPA_BF16) return false;
+  const int64_t B = t.size[0], L = t.size[2], S = t.size[3];
+  if (B < 1 || L < 1 || S < 1 || B > (1 << 20) || L > (1 << 24) || S > 0x7fffffff) return false;
+  if (t.size[1] > 1 && t.stride[1] != 0) return false;
+  if (S > 1 && t.stride[3] != 1) return false;
+  *Bm = live_extent(t, 0);
+  *Lm = (L > 1 && t.stride[2] == 0) ? 1 : (int)L;
+  return (int64_t)*Bm * *Lm * 4 < 0x7fffffff;
+}
+
+}  // namespace
+}  // namespace mi355
+
+extern "C" size_t mi355_sdpa_mask_verdict_words(const mi355_sdpa_tensor* mask, int32_t dtype) {
+  int Bm, Lm;
+  if (!mask || !verdict_shape(*mask, dtype, &Bm, &Lm)) return 0;
+  return (size_t)8 + (size_t)mask->size[0] + (size_t)Bm * Lm * 4;
+}
+
+extern "C" int mi355_sdpa_mask_verdict(const mi355_sdpa_tensor* mask, int32_t dtype, int32_t* verdict, void* stream) {
+  int Bm, Lm;
+  if (!mask || !verdict) return set_error("SDPA: mask_verdict needs a mask and an output buffer"), MI355_SDPA_ERR_INVALID;
+  if (!verdict_shape(*mask, dtype, &Bm, &Lm))
+    return set_error("SDPA: mask_verdict: this mask cannot have a verdict (it depends on the head, its keys are not unit-stride, or its dtype)"),
+           MI355_SDPA_ERR_UNSUPPORTED;
+  VerdictArgs a;
+  a.mask = mask->data;
+  a.sb = Bm > 1 ? mask->stride[0] : 0, a.sl = Lm > 1 ? mask->stride[2] : 0;
+  a.B = (int)mask->size[0], a.Bm = Bm, a.L = (int)mask->size[2], a.Lm = Lm, a.S = (int)mask->size[3];
+  a.verdict = verdict, a.rows = verdict + 8 + a.B;
+  hipStream_t s = (hipStream_t)stream;
+  const dim3 grid((unsigned)(((int64_t)Bm * Lm + 3) / 4)), block(256);
+  switch (dtype) {
+    case MI355_SDPA_BOOL: hipLaunchKernelGGL((mask_rows_batched_kernel<uint8_t>), grid, block, 0, s, a); break;
+    case MI355_SDPA_F32: hipLaunchKernelGGL((mask_rows_batched_kernel<float>), grid, block, 0, s, a); break;
+    case MI355_SDPA_F16: hipLaunchKernelGGL((mask_rows_batched_kernel<f16_t>), grid, block, 0, s, a); break;
+    default: hipLaunchKernelGGL((mask_rows_batched_kernel<bf16_t>), grid, block, 0, s, a); break;
+  }
+  if (int rc = check_launch("mask_rows_batched_kernel")) return rc;
+  hipLaunchKernelGGL(mask_verdict_kernel, dim3(1), dim3(1024), 0, s, a);
+  return check_launch("mask_verdict_kernel");
+}
+
 // ---- tile skip tables ------------------------------------------------------------------------------
 // The run-time counterpart of the reference's static tile elimination
 // (torch_neuronx/neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:15-33): there the mask

@@ -51,7 +51,8 @@ class MaskSpec(C.Structure):
                 ("live_tiles", C.c_void_p), ("live_tiles_t", C.c_void_p),
                 ("n_sink_logits", C.c_int32), ("softcap", C.c_float), ("alibi_slopes", C.c_void_p),
                 ("key_bias", C.c_void_p), ("key_weight", C.c_void_p), ("doc_ids_q", C.c_void_p),
-                ("doc_ids_k", C.c_void_p), ("doc_ids_sorted", C.c_int32)]
+                ("doc_ids_k", C.c_void_p), ("doc_ids_sorted", C.c_int32),
+                ("mask_verdict", C.c_void_p)]
 
 
 class FwdParams(C.Structure):
@@ -96,6 +97,8 @@ EXPORTS = {
     "mi355_sdpa_decode_fp8kv_static": (C.c_int, [C.POINTER(DecodeParams), C.c_void_p]),
     "mi355_sdpa_mask_rows": (C.c_int, [C.c_void_p, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_void_p, C.c_void_p]),
     "mi355_sdpa_mask_tiles_words": (C.c_int, [C.c_void_p, C.c_int32, C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]),
+    "mi355_sdpa_mask_verdict_words": (C.c_size_t, [C.c_void_p, C.c_int32]),
+    "mi355_sdpa_mask_verdict": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p]),
     "mi355_sdpa_mask_tiles": (C.c_int, [C.c_void_p, C.c_int32, C.c_void_p, C.c_void_p, C.c_void_p]),
     "mi355_sdpa_choose_backend": (C.c_int, [C.POINTER(Desc)]),
     "mi355_sdpa_validate": (C.c_int, [C.POINTER(Desc), C.c_char_p, C.c_size_t]),

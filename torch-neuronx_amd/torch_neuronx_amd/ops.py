@@ -122,6 +122,25 @@ def mask_tile_maps(attn_bias, B, Hq, L, S):
     return live, live_t
 
 
+def mask_verdict(attn_bias, B, Hq, L, S):
+    """The device-side verdict about a bias / keep-mask (``mi355_sdpa_mask_verdict``): an int32 device
+    tensor for ``sdpa_forward(..., mask_verdict=)``, or ``None`` for a mask that cannot have one.
+    ``[0]`` kind (0 no pattern, 1 keep-everything, 2 causal, 3 sliding window), ``[1]`` window,
+    ``[2]`` sink keys, ``[3]`` 1 if a batch keeps fewer than ``S`` keys, ``[8 + b]`` keys of batch ``b``."""
+    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
+    if bias is None:
+        return None
+    lib = _lib.load()
+    t4 = _lib.tensor4(bias)
+    words = lib.mi355_sdpa_mask_verdict_words(C.byref(t4), bias_dt)
+    if words == 0:
+        return None
+    verdict = torch.empty((words,), dtype=torch.int32, device=bias.device)
+    with _lib.on_device(bias.device):
+        _lib.check(lib.mi355_sdpa_mask_verdict(C.byref(t4), bias_dt, verdict.data_ptr(), _lib.current_stream(bias.device)))
+    return verdict
+
+
 def _mask_spec(spec, query, S, window, sink_keys, sink_logit, live_tiles=None, score_mods=None):
     """Fill the functor part of a parameter block; returns ``(sink logits as passed to the library or
     None, the tensors that must stay alive over the launch)``."""
@@ -194,12 +213,14 @@ def _score_mods(kw):
 
 def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None, dropout_p=0.0,
                  dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0,
-                 window=None, sink_keys=0, sink_logit=None, live_tiles=None, **score_mods):
+                 window=None, sink_keys=0, sink_logit=None, live_tiles=None, mask_verdict=None, **score_mods):
     """Fused forward.  K/V arrive at ``Hkv`` heads.  Returns ``(out, lse)``; ``out`` keeps the
     dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``.
 
     ``live_tiles``: the ``(live, live_t)`` pair of ``mask_tile_maps`` for this ``attn_bias`` (or
     ``True`` to build it here): the kernels then skip the tiles that the mask drops whole.
+    ``mask_verdict``: what ``mask_verdict`` below wrote about this ``attn_bias``: where the verdict
+    names the causal or the keep-everything pattern, the kernels generate it and read no mask.
 
     ``window`` (with ``is_causal``): query ``i`` sees keys ``i-window+1 .. i`` and the first
     ``sink_keys`` keys; ``sink_logit`` ``(B,Hq)``, ``(Hq,)`` or ``(B,Hq,n)``: logits that join every
@@ -243,6 +264,8 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     if live_tiles is True:
         live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
     _z = _mask_spec(p.mask, query, S, window, sink_keys, sink_logit, live_tiles, score_mods)  # noqa: F841 (kept alive over the launch)
+    if mask_verdict is not None:
+        p.mask.mask_verdict = mask_verdict.data_ptr()
     ws = None
     if (L <= 32 or L * (Hq // max(key.shape[1], 1)) <= 256) and query.dtype in (torch.float16, torch.bfloat16):
         # few query rows: the library may want to split the keys over more workgroups
@@ -259,7 +282,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
 def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_causal=False,
                   scale=None, dropout_p=0.0, dropout_keep=None, kv_lens=None,
                   want_grad_bias=False, force_kernel=0, window=None, sink_keys=0, sink_logit=None,
-                  live_tiles=None, **score_mods):
+                  live_tiles=None, mask_verdict=None, **score_mods):
     """Fused backward.  Returns ``(dq, dk, dv, dbias-or-None)``; each gradient keeps the
     dimension order of its input, dk/dv come back at ``Hkv`` heads.  With a ``sink_logit`` a
     fifth element follows: its gradient, float32 ``(B,Hq)`` or ``(B,Hq,n)``.  Score functors as in
@@ -306,6 +329,8 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     if live_tiles is True:
         live_tiles = mask_tile_maps(attn_bias, B, Hq, L, S)
     _z, _keep = _mask_spec(p.mask, query, S, window, sink_keys, sink_logit, live_tiles, score_mods)
+    if mask_verdict is not None:
+        p.mask.mask_verdict = mask_verdict.data_ptr()
     dsink = None
     if _z is not None:
         dsink = torch.empty(_z.shape, dtype=torch.float32, device=query.device)

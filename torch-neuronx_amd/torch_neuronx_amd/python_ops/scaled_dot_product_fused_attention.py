@@ -88,15 +88,19 @@ def _is_wide(query, value) -> bool:
     return query.shape[-1] > 128 or value.shape[-1] != query.shape[-1]
 
 
-def _recover_pattern(attn_bias, is_causal, want_grad_bias=False, wide=False):
+def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, wide=False, dropout_p=0.0):
     """A mask that is a pattern the kernels generate by themselves (causal, sliding window with sink
-    keys, keep-everything) is dropped in favour of that pattern - the run-time counterpart of the
-    reference's causal-mask recovery (fx/passes/sdpa_causal_mask.py:162-289).
-    Returns ``(attn_bias, is_causal, functor keyword arguments)``."""
+    keys, keep-everything, either of the first two with right padding) is dropped in favour of that
+    pattern - the run-time counterpart of the reference's causal-mask recovery
+    (fx/passes/sdpa_causal_mask.py:162-289).  A mask about which the host knows nothing yet travels on
+    with its verdict (``mask_verdict``, an int32 device tensor): the kernels then take the decision
+    where the verdict is.  Returns ``(attn_bias, is_causal, functor keyword arguments)``."""
     if attn_bias is None or is_causal or want_grad_bias or not mask_patterns.enabled():
         return attn_bias, is_causal, {}
-    pat = mask_patterns.classify(attn_bias)
+    pat, verdict = mask_patterns.look(attn_bias, query.shape[0], query.shape[1], query.shape[2], key.shape[2])
     if pat is None:
+        if verdict is not None and dropout_p == 0.0 and query.dtype in (torch.float16, torch.bfloat16):
+            return attn_bias, is_causal, {"mask_verdict": verdict}
         return attn_bias, is_causal, {}
     if pat[0] == "all":  # (with per-batch key counts when the mask was right padding)
         return None, False, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
@@ -114,6 +118,8 @@ def _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key):
     """A mask that stays a tensor gets tile skip tables (cached per tensor), so that the kernels leave
     out the tiles it drops whole - the run-time counterpart of the reference's static tile
     elimination (neuron_dynamo_backend/flex_attention/flex_attention.py.jinja:15-33)."""
+    if "mask_verdict" in functor:  # (nothing is known about the mask yet: tables are for masks known to be no pattern)
+        return functor
     if attn_bias is not None and not is_causal and dropout_p == 0.0 and query.dtype in (torch.float16, torch.bfloat16):
         maps = mask_patterns.tile_maps(attn_bias, query.shape[0], query.shape[1], query.shape[2], key.shape[2])
         if maps is not None:
@@ -139,7 +145,8 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
         seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
     else:
         seed, offset = _empty_rng(query.device)
-    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, wide=_is_wide(query, value))
+    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, wide=_is_wide(query, value),
+                                                     dropout_p=dropout_p)
     functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     out, lse = ops.sdpa_forward(query, key, value, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
                                 dropout_p=dropout_p, dropout_keep=keep, need_lse=need_lse,
@@ -176,7 +183,8 @@ def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p,
             dropout_p = 0.0  # a placeholder carries no mask: treated as absent (_sdpa_math.py:42-45)
         else:
             keep = philox_seed
-    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, want_grad_bias, wide=_is_wide(query, value))
+    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias,
+                                                     wide=_is_wide(query, value), dropout_p=dropout_p)
     functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     dq, dk, dv, dbias = ops.sdpa_backward(
         grad_out, query, key, value, out, logsumexp, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
