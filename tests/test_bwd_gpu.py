@@ -422,7 +422,7 @@ def test_mfma_backward_narrow_head_dims(amd, gpu_device, E, variant):
     (2, 4, 2, 130, 256, 128, "full", True, False),     # zeros above the diagonal, written by the kernel
     (3, 2, 1, 77, 136, 96, "full", False, True),       # zeros past each batch's keys; a narrow head dim
 ])
-@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16, torch.float32])
 def test_mfma_backward_grad_bias(amd, gpu_device, case, dtype):
     # grad_bias = P (dP - delta) leaves the MFMA dQ kernel in the input dtype (forced: no fallback);
     # the buffer starts as NaN, so every element must be written
@@ -459,6 +459,8 @@ def test_mfma_backward_grad_bias(amd, gpu_device, case, dtype):
     rdq, _, _, rdb = om.compute_attention_backward(go.float(), q.float(), ke, ve, mask, None, ro, rl, E**-0.5, causal, 0.0)
     assert db.shape == (B, Hq, L, S) and db.dtype == dtype
     assert torch.isfinite(db.float()).all()
+    if dtype is torch.float32:  # (the float32 matrix-op kernels: the float32 bar)
+        assert max_abs(db, rdb) <= 1e-5 and rel_err(db, rdb) <= 1e-5 and max_abs(dq, rdq) <= 1e-5
     assert max_abs(db, rdb) <= 5e-2 and rel_err(db, rdb) <= 2e-2
     assert max_abs(dq, rdq) <= 5e-2
     if causal:

@@ -52,6 +52,18 @@ def test_functors_float32(amd, gpu_device, window, sink_keys, with_sink):
     _run(amd, gpu_device, 2, 4, 2, 77, 32, torch.float32, window, sink_keys, with_sink, seed=window + 3)
 
 
+@pytest.mark.parametrize("L,E,window,sink_keys,with_sink", [
+    (77, 32, 5, 0, False),
+    (300, 64, 40, 3, True),
+    (512, 128, 100, 40, True),    # several tiles below the window are dropped whole, the sink tiles are not
+    (260, 96, 0, 0, True),        # sink logit alone, a narrow head dim
+    (130, 16, 1000, 0, False),    # window longer than the sequence
+])
+def test_functors_float32_in_the_matrix_op_kernels(amd, gpu_device, L, E, window, sink_keys, with_sink):
+    # (forced: the call fails if the float32 matrix-op kernels refuse it)
+    _run(amd, gpu_device, 2, 4, 2, L, E, torch.float32, window, sink_keys, with_sink, seed=L + window, force=amd._lib.KERNEL_MFMA)
+
+
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 @pytest.mark.parametrize("L,E,window,sink_keys,with_sink", [
     (512, 128, 128, 0, False),

@@ -267,12 +267,14 @@ int mi355_sdpa_can_use_fused_bwd(const mi355_sdpa_desc* d) { return kernel_for(d
 // cannot take say so on stderr, with the reason: the generic kernels are a correctness path two
 // orders of magnitude slower, and nothing else tells a caller that a call went there.
 static void note_fallback(const char* what, const char* why) {
-  static const bool on = [] {
+  // (MI355_SDPA_LOG_FALLBACK=1: the first 16 such calls; a larger number: that many)
+  static const int budget = [] {
     const char* e = getenv("MI355_SDPA_LOG_FALLBACK");
-    return e && *e && strcmp(e, "0") != 0;
+    const int n = e && *e ? atoi(e) : 0;
+    return n <= 0 ? 0 : n == 1 ? 16 : n;
   }();
-  static std::atomic<int> left{16};
-  if (on && left.fetch_sub(1) > 0) fprintf(stderr, "mi355_sdpa: %s runs in the generic kernel: %s\n", what, why && *why ? why : "(no reason recorded)");
+  static std::atomic<int> left{budget};
+  if (budget && left.fetch_sub(1) > 0) fprintf(stderr, "mi355_sdpa: %s runs in the generic kernel: %s\n", what, why && *why ? why : "(no reason recorded)");
 }
 
 int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {

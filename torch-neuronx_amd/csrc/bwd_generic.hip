@@ -34,24 +34,8 @@ struct BwdG {
   ScoreMod sm;            // score functors and document ids
 };
 
-// score functors on s = scale * q.k of (head h, query i, key j); `dfac` receives the derivative of
-// the chain with respect to s, which multiplies the gradient of the scores; a score that the
-// document ids drop comes back as -inf
 __device__ __forceinline__ float score_mod_generic(const BwdG& p, float s, int b, int h, int i, int j, float& dfac) {
-  dfac = 1.f;
-  if (!p.sm.any) return s;
-  if (p.sm.key_weight) {
-    const float w = p.sm.key_weight[(int64_t)h * p.S + j];
-    s *= w, dfac = w;
-  }
-  if (p.sm.key_bias) s += p.sm.key_bias[(int64_t)h * p.S + j];
-  if (p.sm.alibi) s = fmaf(p.sm.alibi[h], (float)(j - i), s);
-  if (p.sm.softcap > 0.f) {
-    const float th = tanhf(s / p.sm.softcap);
-    s = p.sm.softcap * th, dfac *= 1.f - th * th;
-  }
-  if (p.sm.doc_q && p.sm.doc_k && p.sm.doc_q[(int64_t)b * p.L + i] != p.sm.doc_k[(int64_t)b * p.S + j]) s = -INFINITY;
-  return s;
+  return score_mod_at(p.sm, s, b, h, i, j, p.L, p.S, dfac);
 }
 
 template <typename TB>

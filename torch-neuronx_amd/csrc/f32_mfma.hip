@@ -1,6 +1,8 @@
 // Flash attention for float32 inputs on the float32 matrix op (v_mfma_f32_32x32x2_f32), forward and
 // backward, head dims up to 128 (multiples of 8; narrower rows count as zero padded), causal or
-// unmasked, with per-batch key counts; instances with a per-score bias / keep-mask or dropout.  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
+// unmasked, with per-batch key counts; instances with a per-score bias / keep-mask (and its gradient)
+// or dropout, and instances with the mask and score functors (sliding window with sink keys, sink
+// logits, the functors and document ids of score_mod.h, element by element).  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
 // stays in float32 as in torch_neuronx/_sdpa_math.py (float32 inputs accumulate in float32, and the
 // probabilities that multiply V are not rounded, :94).
 //
@@ -113,8 +115,9 @@ __device__ __forceinline__ void load_bias16(float (&bl)[16], const void* base, i
   }
 }
 
-template <int D, int WAVES, bool MASKED>
+template <int D, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
+  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // a per-score tensor | window, sinks, score functors
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
   __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
@@ -136,20 +139,45 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
   int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BT + 1);
-  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  // sliding window: the tiles below the lowest window of the workgroup's rows are dropped whole, except
+  // the leading ones that hold sink keys: stream position u is key tile u + (u >= n_lead ? skip : 0)
+  int n_lead = 0, skip = 0;
+  if constexpr (FUNC) {
+    if (p.window > 0) {
+      const int t_lo = max(q0 - p.window + 1, 0) / BT;
+      n_lead = min(min((p.sink_keys + BT - 1) / BT, t_lo), nt);
+      skip = min(t_lo, nt) - n_lead;
+      nt -= skip;
+    }
+  }
+  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1 - skip) : nt;
   TileF32<D, 64 * WAVES> kn, vn;
-  if (nt > 0) kn.fetch(kp, p.k_sl, S, p.d_real, tid), vn.fetch(vp, p.v_sl, S, p.d_real, tid);
-  for (int t = 0; t < nt; ++t) {
+  auto fetch = [&](int u) {
+    const int t = tile_of(u);
+    kn.fetch(kp + (int64_t)t * BT * p.k_sl, p.k_sl, S - t * BT, p.d_real, tid);
+    vn.fetch(vp + (int64_t)t * BT * p.v_sl, p.v_sl, S - t * BT, p.d_real, tid);
+  };
+  if (nt > 0) fetch(0);
+  for (int u = 0; u < nt; ++u) {
     __syncthreads();  // the previous tile has been read by every wavefront
     kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
-    if (t + 1 < nt) {
-      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, S - (t + 1) * BT, p.d_real, tid);
-      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, S - (t + 1) * BT, p.d_real, tid);
-    }
-    if (t >= nt_w) continue;
+    if (u + 1 < nt) fetch(u + 1);
+    if (u >= nt_w) continue;
+    const int t = tile_of(u);
     f32x16 s = row_product<D>(k_t, col, half, qf);
+    if constexpr (FUNC) {
+      // each score through the functors, s = mod(scale * s) / scale: everything downstream is the common code
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kv = t * BT + (r >> 2) * 8 + half * 4 + (r & 3);
+        float dfac;
+        s[r] = score_mod_at(p.sm, s[r] * p.scale, b, h, qc, min(kv, p.S - 1), p.L, p.S, dfac) * inv_scale;
+        if (p.window > 0 && qrow - kv >= p.window && kv >= p.sink_keys) s[r] = -INFINITY;
+      }
+    }
     float keepf[MASKED ? 16 : 1];
     if constexpr (MASKED) {
       // this lane's row of the bias / keep-mask plane of the (batch, head), keys clamped into the row
@@ -197,8 +225,26 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
     }
     col_product<D>(oacc, v_t, col, half, s);
   }
-  const float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  float l_tot = l_run + __shfl_xor(l_run, 32, 64);
+  float lse_row = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
   float inv = l_tot > 0.f ? 1.f / l_tot : 0.f;
+  if constexpr (FUNC) {
+    if (p.sink_logit) {
+      // the sink logits of this (batch, head) join the row's softmax as one more column without a value
+      // (several act as one: the logarithm of the sum of their exponentials)
+      const float* zs = p.sink_logit + ((int64_t)b * p.Hq + h) * p.n_sinks;
+      float zm = -INFINITY, zl = 0.f;
+      for (int n = 0; n < p.n_sinks; ++n) zm = fmaxf(zm, zs[n]);
+      for (int n = 0; n < p.n_sinks; ++n) zl += zm == -INFINITY ? 0.f : __expf(zs[n] - zm);
+      if (zm != -INFINITY) {
+        const float z = zm + __builtin_logf(zl);
+        const float top = fmaxf(lse_row, z);
+        const float both = __expf(lse_row - top) + __expf(z - top);  // (exp(-inf) = 0 for a row without a live key)
+        inv *= __expf(lse_row - top) / both;
+        lse_row = top + __builtin_logf(both);
+      }
+    }
+  }
   if constexpr (MASKED) {
     if (p.keep_scale != 0.f) inv *= p.keep_scale;
   }
@@ -213,12 +259,13 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
           *(f32x4*)(orow + d) = f32x4{oacc[db][g * 4] * inv, oacc[db][g * 4 + 1] * inv, oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv};
       }
     if (p.lse && half == 0)
-      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = l_tot > 0.f ? m_run * p.scale + __builtin_logf(l_tot) : -INFINITY;
+      p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
   }
 }
 
-template <int D, int WAVES, bool MASKED>
+template <int D, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
+  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // a per-score tensor | window, sink keys, score functors
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
   __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
@@ -262,22 +309,48 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
   int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + BM, p.L) - 1) / BT + 1);
-  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  int n_lead = 0, skip = 0;  // (sliding window: the tiles that it drops whole, as in the forward)
+  if constexpr (FUNC) {
+    if (p.window > 0) {
+      const int t_lo = max(q0 - p.window + 1, 0) / BT;
+      n_lead = min(min((p.sink_keys + BT - 1) / BT, t_lo), nt);
+      skip = min(t_lo, nt) - n_lead;
+      nt -= skip;
+    }
+  }
+  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1 - skip) : nt;
+  // gradient of the bias: P (dP - delta) per score, this lane's row; zeros where a score takes no part
+  float* const gb_row = (MASKED && p.gbias && qrow < p.L)
+                            ? (float*)p.gbias + b * p.gbias_sb + h * p.gbias_sh + (int64_t)qrow * p.gbias_sl : nullptr;
   TileF32<D, 64 * WAVES> kn, vn;
-  if (nt > 0) kn.fetch(kp, p.k_sl, S, p.d_real, tid), vn.fetch(vp, p.v_sl, S, p.d_real, tid);
-  for (int t = 0; t < nt; ++t) {
+  auto fetch = [&](int u) {
+    const int t = tile_of(u);
+    kn.fetch(kp + (int64_t)t * BT * p.k_sl, p.k_sl, S - t * BT, p.d_real, tid);
+    vn.fetch(vp + (int64_t)t * BT * p.v_sl, p.v_sl, S - t * BT, p.d_real, tid);
+  };
+  if (nt > 0) fetch(0);
+  for (int u = 0; u < nt; ++u) {
     __syncthreads();  // the previous tile has been read by every wavefront
     kn.put(k_t, tid), vn.put(v_t, tid);
     __syncthreads();
-    if (t + 1 < nt) {
-      kn.fetch(kp + (int64_t)(t + 1) * BT * p.k_sl, p.k_sl, S - (t + 1) * BT, p.d_real, tid);
-      vn.fetch(vp + (int64_t)(t + 1) * BT * p.v_sl, p.v_sl, S - (t + 1) * BT, p.d_real, tid);
-    }
-    if (t >= nt_w) continue;
-    const f32x16 s = row_product<D>(k_t, col, half, qf);
+    if (u + 1 < nt) fetch(u + 1);
+    if (u >= nt_w) continue;
+    const int t = tile_of(u);
+    f32x16 s = row_product<D>(k_t, col, half, qf);
     const f32x16 dp = row_product<D>(v_t, col, half, dof);
     f32x16 ds;
+    float dfac[FUNC ? 16 : 1];  // derivative of the functors, the factor on the gradient of the scores
+    if constexpr (FUNC) {
+      const float inv_scale = 1.f / p.scale;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int kv = t * BT + (r >> 2) * 8 + half * 4 + (r & 3);
+        s[r] = score_mod_at(p.sm, s[r] * p.scale, b, h, qc, min(kv, p.S - 1), p.L, p.S, dfac[r]) * inv_scale;
+        if (p.window > 0 && qrow - kv >= p.window && kv >= p.sink_keys) s[r] = -INFINITY;
+      }
+    }
     float bl[MASKED ? 16 : 1];  // the bias in the log2 domain, or (dropout) keep / (1 - p)
     bool drop = false;
     if constexpr (MASKED) {
@@ -302,8 +375,20 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
       float g = dp[r];
       if constexpr (MASKED) g = drop ? g * bl[r] : g;
       ds[r] = pr * (g - dl);
+      if constexpr (MASKED) {
+        if (gb_row && kv < p.S) gb_row[kv] = ds[r];
+      }
+      if constexpr (FUNC) ds[r] *= dfac[r];
     }
     col_product<D>(dqacc, k_t, col, half, ds);
+  }
+  if constexpr (MASKED) {
+    if (gb_row) {  // the tiles this wavefront did not walk: above the diagonal, past the batch's keys
+      for (int kv = min(nt_w, nt) * BT + half * 4; kv < p.S; kv += 8)
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+          if (kv + e < p.S) gb_row[kv + e] = 0.f;
+    }
   }
   if (qrow < p.L) {
     float* gq = (float*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
@@ -319,8 +404,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   }
 }
 
-template <int D, int WAVES, bool MASKED>
+template <int D, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
+  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // a per-score tensor | window, sink keys, score functors
   constexpr int DB = D / 32;
   __shared__ __attribute__((aligned(16))) float q_t[BT * (D + 4)];
   __shared__ __attribute__((aligned(16))) float do_t[BT * (D + 4)];
@@ -372,9 +458,23 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
       __syncthreads();
       if (it + 1 < n_items) fetch_item(it + 1);
       if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= S) continue;  // (uniform per wavefront)
-      const f32x16 s = row_product<D>(q_t, col, half, kf);
+      if constexpr (FUNC) {  // every row of the tile lies past the window of every key of this wavefront, none of them a sink
+        if (p.window > 0 && q0 - (kw0 + 31) >= p.window && kw0 >= p.sink_keys) continue;
+      }
+      f32x16 s = row_product<D>(q_t, col, half, kf);
       const f32x16 dp = row_product<D>(do_t, col, half, vf);
       f32x16 pr, ds;
+      float dfac[FUNC ? 16 : 1];  // derivative of the functors, the factor on the gradient of the scores
+      if constexpr (FUNC) {
+        const int hq = hk * rep + it % rep;
+        const float inv_scale = 1.f / p.scale;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int qi = q0 + (r >> 2) * 8 + half * 4 + (r & 3);
+          s[r] = score_mod_at(p.sm, s[r] * p.scale, b, hq, min(qi, p.L - 1), kc, p.L, p.S, dfac[r]) * inv_scale;
+          if (p.window > 0 && qi - key >= p.window && key >= p.sink_keys) s[r] = -INFINITY;
+        }
+      }
       float bl[MASKED ? 16 : 1];  // the bias in the log2 domain, or (dropout) keep / (1 - p)
       bool drop = false;
       if constexpr (MASKED) {
@@ -407,6 +507,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
             if (drop) g *= bl[r], pr[r] = x * bl[r];  // dV from the kept probabilities, scaled; dP masked and scaled
           }
           ds[r] = x * (g - d4[e]);
+          if constexpr (FUNC) ds[r] *= dfac[r];
         }
       }
       col_product<D>(dvacc, do_t, col, half, pr);
@@ -466,7 +567,8 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "mask / score functors", false;
+  if ((p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) && (p.bias.data || p.dropout_p > 0.f))
+    return *why = "window / sink / score functor together with attn_bias or dropout", false;
   if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
   if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
@@ -498,17 +600,21 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
   set_score_mask(g, p);
-  const bool masked = g.bias != nullptr;
+  g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
+  g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
+  g.sm = score_mod_of(p.mask);
+  const int mode = g.bias != nullptr ? 1 : (g.window > 0 || g.sink_logit || g.sm.any) ? 2 : 0;
   // rows per workgroup: 128 (a workgroup is one wavefront per 32 rows; 64- and 32-row workgroups
   // measured slower even when 128-row ones leave compute units without work)
   const int waves = pick_waves((int64_t)g.B * g.Hq, g.L);
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(64 * waves);
 #define LAUNCH(DD, WW, MM) hipLaunchKernelGGL((fwd_f32_kernel<DD, WW, MM>), grid, block, 0, s, g)
-#define LAUNCH_W(DD)                \
-  do {                              \
-    if (masked) LAUNCH(DD, 4, true); \
-    else LAUNCH(DD, 4, false);      \
+#define LAUNCH_W(DD)                   \
+  do {                                 \
+    if (mode == 1) LAUNCH(DD, 4, 1);   \
+    else if (mode == 2) LAUNCH(DD, 4, 2); \
+    else LAUNCH(DD, 4, 0);             \
   } while (0)
   if (g.d_real <= 64) LAUNCH_W(64);
   else LAUNCH_W(128);
@@ -522,7 +628,10 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
-  if (p.grad_bias.data || p.mask.window > 0 || score_mod_of(p.mask).any) return *why = "bias gradient, window or score functor", false;
+  if ((p.mask.window > 0 || score_mod_of(p.mask).any) && (p.bias.data || p.dropout_p > 0.f))
+    return *why = "window or score functor together with attn_bias or dropout", false;
+  if (p.grad_bias.data && (!p.bias.data || (p.k.size[2] > 1 && p.grad_bias.stride[3] != 1)))
+    return *why = "grad_attn_bias without attn_bias, or its keys are not unit-stride", false;
   if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
   if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
@@ -569,15 +678,22 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.kv_lens = p.kv_lens;
   g.d_real = (int)p.q.size[3];
   set_score_mask(g, p);
-  const bool masked = g.bias != nullptr;
+  g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
+  g.sm = score_mod_of(p.mask);
+  if (p.grad_bias.data) {
+    g.gbias = p.grad_bias.data;
+    g.gbias_sb = p.grad_bias.stride[0], g.gbias_sh = p.grad_bias.stride[1], g.gbias_sl = p.grad_bias.stride[2];
+  }
+  const int mode = g.bias != nullptr ? 1 : (g.window > 0 || g.sm.any) ? 2 : 0;
   const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
   const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
   const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw))));
 #define LAUNCH(KK, GRID, DD, WW, MM) hipLaunchKernelGGL((KK<DD, WW, MM>), GRID, dim3(64 * WW), 0, s, g)
-#define LAUNCH_W(KK, GRID, WAVES_, DD)          \
-  do {                                          \
-    if (masked) LAUNCH(KK, GRID, DD, 4, true);  \
-    else LAUNCH(KK, GRID, DD, 4, false);        \
+#define LAUNCH_W(KK, GRID, WAVES_, DD)                 \
+  do {                                                 \
+    if (mode == 1) LAUNCH(KK, GRID, DD, 4, 1);         \
+    else if (mode == 2) LAUNCH(KK, GRID, DD, 4, 2);    \
+    else LAUNCH(KK, GRID, DD, 4, 0);                   \
   } while (0)
   if (g.d_real <= 64) LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 64);
   else LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 128);

@@ -43,6 +43,27 @@ __device__ __forceinline__ float tanh_fast(float x) {
   return 1.f - 2.f * __builtin_amdgcn_rcpf(e + 1.f);
 }
 
+// One score through the functors, element by element (the generic and the float32 kernels):
+// x = scale * q.k of (batch b, head h, query i, key j); L and S are the row lengths of the id and
+// per-key vectors.  `dfac` receives d mod / d x, which multiplies the gradient of the score; a score
+// that the document ids drop comes back as -inf.
+__device__ __forceinline__ float score_mod_at(const ScoreMod& sm, float x, int b, int h, int i, int j, int L, int S, float& dfac) {
+  dfac = 1.f;
+  if (!sm.any) return x;
+  if (sm.key_weight) {
+    const float w = sm.key_weight[(int64_t)h * S + j];
+    x *= w, dfac = w;
+  }
+  if (sm.key_bias) x += sm.key_bias[(int64_t)h * S + j];
+  if (sm.alibi) x = fmaf(sm.alibi[h], (float)(j - i), x);
+  if (sm.softcap > 0.f) {
+    const float th = tanhf(x / sm.softcap);
+    x = sm.softcap * th, dfac *= 1.f - th * th;
+  }
+  if (sm.doc_q && sm.doc_k && sm.doc_q[(int64_t)b * L + i] != sm.doc_k[(int64_t)b * S + j]) x = -INFINITY;
+  return x;
+}
+
 // First index of the sorted array a[0 .. n) whose value is >= x (n if none), found by a whole
 // wavefront, for N values of x at once: every round samples 64 evenly spaced positions per search
 // (all the loads of a round go out together) and keeps the interval between the last sample below x
