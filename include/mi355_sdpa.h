@@ -187,7 +187,10 @@ typedef struct mi355_sdpa_bwd_params {
   mi355_sdpa_tensor grad_v;   /* (B,Hkv,S,Dv)                                         */
   mi355_sdpa_tensor bias;     /* as in forward                                        */
   int32_t bias_dtype;
-  mi355_sdpa_tensor grad_bias; /* optional (B,Hq,L,S), dtype of q                     */
+  mi355_sdpa_tensor grad_bias; /* optional (B,Hq,L,S), dtype of q.  The matrix-op kernels for 16-bit
+                                  inputs write it four keys at a time: S a multiple of 4, or rows
+                                  padded to one (a row stride >= S rounded up to 4 is the caller's
+                                  word that every row, the last included, has that room)       */
   const int32_t* kv_lens;
   const uint8_t* dropout_keep;
   float dropout_p;

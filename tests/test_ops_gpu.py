@@ -8,7 +8,7 @@ import pytest
 import torch
 import torch.nn.functional as F
 
-from helpers import max_abs, oracle_bwd, oracle_fwd, qkv, rel_err
+from helpers import max_abs, oracle_bwd, oracle_fwd, qkv, rel_err, seeded
 
 pytestmark = pytest.mark.gpu
 
@@ -560,3 +560,55 @@ def test_fallback_to_the_generic_kernel_can_be_logged(gpu_device):
     assert "mi355_sdpa" not in before
     assert "forward runs in the generic kernel: head dims are not multiples of 8" in after
     assert "backward runs in the generic kernel" in after
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("kind", ["odd_keys_16bit", "odd_keys_bool", "offset_slice", "odd_row_stride", "odd_keys_grad"])
+def test_biases_that_are_not_dword_aligned_still_run_in_the_matrix_op_kernels(amd, gpu_device, dtype, kind):
+    # the host repacks such a bias once (over its own extents) rather than letting the call leave the
+    # matrix-op kernels; forced, so the call fails if they refuse it.  Forward, backward and - for the
+    # last kind - the gradient of the bias over a number of keys that is no multiple of four.
+    from oracle import sdpa_math as om
+
+    dev = gpu_device
+    B, Hq, Hkv, L, E = 2, 4, 2, 130, 64
+    S = 150 if kind == "odd_keys_grad" else 77 if kind.startswith("odd_keys") else 96
+    q, k, v, go = seeded([(B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, E), (B, Hq, L, E)], len(kind), dtype)
+    g = torch.Generator().manual_seed(S)
+    if kind == "odd_keys_bool":
+        bias = torch.rand(B, 1, L, S, generator=g) < 0.7
+        bias[..., 0] = True
+    elif kind == "offset_slice":
+        bias = torch.randn(1, Hq, L, S + 1, generator=g).to(dtype)[..., 1:]   # rows start at an odd element
+    elif kind == "odd_row_stride":
+        bias = torch.randn(1, Hq, L, S + 3, generator=g).to(dtype)[..., :S]   # rows are an odd number of elements apart
+    else:
+        bias = torch.randn(B, Hq, L, S, generator=g).to(dtype)
+    bd = bias.to(dev)
+    if kind == "offset_slice":
+        bd = torch.randn(1, Hq, L, S + 1, device=dev).to(dtype)
+        bd[..., 1:] = bias.to(dev)
+        bd = bd[..., 1:]
+    elif kind == "odd_row_stride":
+        bd = torch.zeros(1, Hq, L, S + 3, device=dev, dtype=dtype)
+        bd[..., :S] = bias.to(dev)
+        bd = bd[..., :S]
+    MFMA = amd._lib.KERNEL_MFMA
+    qd, kd, vd, god = (t.to(dev) for t in (q, k, v, go))
+    want_gb = kind == "odd_keys_grad"
+    out, lse = amd.sdpa_forward(qd, kd, vd, attn_bias=bd, force_kernel=MFMA)
+    res = amd.sdpa_backward(god, qd, kd, vd, out, lse, attn_bias=bd, want_grad_bias=want_gb, force_kernel=MFMA)
+    mask = bias if bias.dtype == torch.bool else bias.float()
+    ro, rl = om.sdpa_forward(q.float(), k.float(), v.float(), attn_mask=mask)
+    assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 5e-3
+    rg = om.sdpa_backward(go.float(), q.float(), k.float(), v.float(), ro, rl, attn_mask=mask, reduce_in_fp32=True)
+    for a, r in zip(res[:3], rg[:3]):
+        assert max_abs(a, r) <= 5e-2 and rel_err(a, r) <= 3e-2
+    if want_gb:
+        rep = Hq // Hkv
+        ke, ve = k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1)
+        co, cl = om.compute_attention(q.float(), ke, ve, mask, None, E**-0.5, False, 0.0)
+        rdb = om.compute_attention_backward(go.float(), q.float(), ke, ve, mask, None, co, cl, E**-0.5, False, 0.0)[3]
+        db = res[3]
+        assert db.shape == (B, Hq, L, S) and db.is_contiguous()
+        assert max_abs(db, rdb) <= 5e-2 and rel_err(db, rdb) <= 2e-2

@@ -582,7 +582,10 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   if (p.grad_bias.data) {  // written by the dQ kernel four keys (8 bytes) at a time
     const int64_t S = p.k.size[2];
     if (!p.bias.data) return *why = "grad_attn_bias without attn_bias", false;
-    if (S % 4 != 0 || (S > 1 && p.grad_bias.stride[3] != 1) || ((uintptr_t)p.grad_bias.data & 7) != 0)
+    // (a row stride of at least S rounded up to four says that every row - the last one of the tensor
+    // included - has room for whole words: the words that cross the end of a row then land in its padding)
+    const bool room = S % 4 == 0 || (p.q.size[2] > 1 && p.grad_bias.stride[2] >= ((S + 3) & ~(int64_t)3));
+    if (!room || (S > 1 && p.grad_bias.stride[3] != 1) || ((uintptr_t)p.grad_bias.data & 7) != 0)
       return *why = "grad_attn_bias rows are not whole 8-byte words", false;
     for (int i = 0; i < 3; ++i)
       if (p.grad_bias.size[i] > 1 && (p.grad_bias.stride[i] % 4) != 0) return *why = "grad_attn_bias stride not 8-byte aligned", false;

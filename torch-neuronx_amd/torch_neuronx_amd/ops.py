@@ -90,14 +90,43 @@ def _unit_last(t: torch.Tensor) -> torch.Tensor:
     return t if t.stride(-1) == 1 or t.size(-1) <= 1 else t.contiguous()
 
 
-def _bias_view(attn_bias, B, Hq, L, S):
+def _bias_view(attn_bias, B, Hq, L, S, repack_for=None):
+    """``attn_bias`` expanded to ``(B,Hq,L,S)`` (stride 0 on broadcast dims) and its dtype id.
+
+    ``repack_for``: the dtype of the query, for calls that may run in the matrix-op kernels.  Those read
+    the bias a dword at a time: a bias whose rows do not start on dwords or are not whole dwords (a
+    16-bit bias over an odd number of keys, a slice that starts at an odd element, a bool mask over a
+    number of keys that is no multiple of four) is copied once, over its own extents - broadcast dims
+    stay broadcast - into a layout they take: the same dtype where that can be aligned, float32
+    otherwise (an additive 0 / -inf tensor for a bool mask).  One pass over the bias, against a call
+    that would otherwise leave the matrix-op kernels altogether."""
     if attn_bias is None:
         return None, 0
     b = attn_bias
     while b.dim() < 4:
         b = b.unsqueeze(0)
     b = b.expand(B, Hq, L, S)
+    if repack_for is not None and not _dword_rows(b, S):
+        own = b[tuple(slice(0, 1) if (b.stride(i) == 0 and b.size(i) > 1) else slice(None) for i in range(4))]
+        if own.dtype == torch.bool:
+            tgt = repack_for if (S % 2 == 0 and repack_for in (torch.float16, torch.bfloat16)) else torch.float32
+            own = torch.zeros(own.shape, dtype=tgt, device=own.device).masked_fill_(~own, float("-inf"))
+        else:
+            gran = max(4 // own.element_size(), 1)
+            own = own.contiguous() if S % gran == 0 else own.to(torch.float32).contiguous()
+        b = own.expand(B, Hq, L, S)
     return b, _lib.dtype_id(b.dtype)
+
+
+def _dword_rows(b, S) -> bool:
+    if b.dtype not in (torch.bool, torch.float16, torch.bfloat16, torch.float32):
+        return True  # (not a dtype the matrix-op kernels take: nothing to gain)
+    gran = max(4 // b.element_size(), 1)
+    if S > 1 and b.stride(3) != 1:
+        return False
+    if b.data_ptr() % 4 != 0 or S % gran != 0:
+        return False
+    return all(b.size(i) <= 1 or b.stride(i) % gran == 0 for i in range(3))
 
 
 def mask_tile_maps(attn_bias, B, Hq, L, S):
@@ -244,7 +273,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     if out.stride(-1) != 1 and Dv > 1:
         out = torch.empty((B, Hq, L, Dv), dtype=query.dtype, device=query.device)
     lse = torch.empty((B, Hq, L), dtype=torch.float32, device=query.device) if need_lse else None
-    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
+    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S, repack_for=None if force_kernel == _lib.KERNEL_GENERIC else query.dtype)
     p, P = _lib.FwdParams(), _lib.FwdParams
     for f, t in ((P.q, q), (P.k, k), (P.v, v), (P.out, out), (P.bias, bias)):
         _lib.put4(p, f, t)
@@ -305,10 +334,12 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
         return g
 
     dq, dk, dv = grad_like(query, (B, Hq, L, E)), grad_like(key, (B, Hkv, S, E)), grad_like(value, (B, Hkv, S, Dv))
-    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S)
+    bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S, repack_for=None if force_kernel == _lib.KERNEL_GENERIC else query.dtype)
     dbias = None
     if want_grad_bias and bias is not None:
-        dbias = torch.empty((B, Hq, L, S), dtype=query.dtype, device=query.device)
+        # (the matrix-op kernels for 16-bit inputs write the gradient four keys at a time: rows padded to that)
+        S4 = S if query.dtype == torch.float32 or L == 1 else (S + 3) // 4 * 4
+        dbias = torch.empty((B, Hq, L, S4), dtype=query.dtype, device=query.device)[..., :S]
     p, P = _lib.BwdParams(), _lib.BwdParams
     for f, t in ((P.grad_out, go), (P.q, q), (P.k, k), (P.v, v), (P.out, o), (P.grad_q, dq), (P.grad_k, dk),
                  (P.grad_v, dv), (P.bias, bias), (P.grad_bias, dbias)):
@@ -342,6 +373,8 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     with _lib.on_device(query.device):
         rc = lib.mi355_sdpa_bwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
+    if dbias is not None and dbias.stride(2) != S and L > 1:
+        dbias = dbias.contiguous()  # (rows were padded for the kernel)
     if _z is not None:
         return dq, dk, dv, dbias, dsink
     return dq, dk, dv, dbias
