@@ -78,6 +78,17 @@ def test_functors_half_precision(amd, gpu_device, dtype, L, E, window, sink_keys
     _run(amd, gpu_device, 2, 8, 2, L, E, dtype, window, sink_keys, with_sink, seed=L + window)
 
 
+@pytest.mark.parametrize("L,E,window,sink_keys,with_sink", [
+    (1024, 256, 256, 0, False),   # several tiles below the window dropped whole in every kernel
+    (777, 256, 100, 40, True),    # sink keys, a sink logit, ragged tiles
+    (640, 192, 130, 33, True),    # a head dim between 128 and 256
+    (300, 256, 1000, 0, False),   # window longer than the sequence: plain causal
+])
+def test_functors_at_head_dims_above_128(amd, gpu_device, L, E, window, sink_keys, with_sink):
+    # the forward's functor variant at width 256 and the wide backward kernels' functor mode, forced
+    _run(amd, gpu_device, 2, 4, 2, L, E, torch.bfloat16, window, sink_keys, with_sink, seed=L + window, force=amd._lib.KERNEL_MFMA)
+
+
 def test_window_equals_the_same_mask_as_a_tensor(amd, gpu_device):
     # the functor and the explicit boolean mask of the same pattern give the same result
     dev = gpu_device

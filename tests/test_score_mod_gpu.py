@@ -44,8 +44,9 @@ def _functors(pattern, B, Hq, L, S, seed):
     }[pattern]
 
 
-def _check(amd, dev, B, Hq, Hkv, L, S, E, dtype, pattern, seed, force=0, scale=None):
-    q, k, v, go = seeded([(B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, E), (B, Hq, L, E)], seed, dtype)
+def _check(amd, dev, B, Hq, Hkv, L, S, E, dtype, pattern, seed, force=0, scale=None, Dv=None):
+    Dv = Dv or E
+    q, k, v, go = seeded([(B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, Dv), (B, Hq, L, Dv)], seed, dtype)
     kw = _functors(pattern, B, Hq, L, S, seed + 1)
     dkw = {n: (t.to(dev) if torch.is_tensor(t) else t) for n, t in kw.items()}
     qd, kd, vd, god = (t.to(dev) for t in (q, k, v, go))
@@ -101,6 +102,18 @@ def test_reference_cases_in_the_matrix_op_kernels(amd, gpu_device, dtype, patter
 ])
 def test_functor_kernels_at_size(amd, gpu_device, pattern, B, Hq, Hkv, L, S, E):
     _check(amd, gpu_device, B, Hq, Hkv, L, S, E, torch.bfloat16, pattern, seed=L + S, force=amd._lib.KERNEL_MFMA)
+
+
+@pytest.mark.parametrize("pattern", PATTERNS)
+@pytest.mark.parametrize("B,Hq,Hkv,L,S,E,Dv", [
+    (1, 4, 2, 512, 512, 256, 256),   # head dim 256 (one wavefront per SIMD in every kernel)
+    (2, 4, 1, 300, 500, 192, 128),   # D_qk != D_v, L != S, ragged tiles
+    (1, 2, 2, 777, 777, 160, 160),   # a head dim between 128 and 256
+])
+def test_functor_kernels_at_wide_head_dims(amd, gpu_device, pattern, B, Hq, Hkv, L, S, E, Dv):
+    # head dims above 128 and D_qk != D_v: the forward's functor variant at width 256 and the wide backward
+    # kernels' functor mode, forced (the call fails if the matrix-op kernels refuse it)
+    _check(amd, gpu_device, B, Hq, Hkv, L, S, E, torch.bfloat16, pattern, seed=L + E, force=amd._lib.KERNEL_MFMA, Dv=Dv)
 
 
 def test_document_ids_equal_the_same_mask_as_a_tensor(amd, gpu_device):

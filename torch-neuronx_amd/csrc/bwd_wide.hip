@@ -150,11 +150,15 @@ constexpr WideOp dkdv_op(int k) {  // S steps and dP steps (in turns where both 
   return {3, (k / DBE) * DB + k % DBE};
 }
 
-// MASKED: per-batch key counts and an additive bias / bool keep-mask, per key or per score (a lane is
-// a query row in the dQ kernel and reads its own row of it, a key in the dK/dV kernel and reads one
-// element per score register); no bias gradient here.
-template <typename T, int ER, int DVR, bool MASKED>
+// MODE 1 (MASKED): per-batch key counts and an additive bias / bool keep-mask, per key or per score (a
+// lane is a query row in the dQ kernel and reads its own row of it, a key in the dK/dV kernel and reads
+// one element per score register); no bias gradient here.
+// MODE 2 (FUNC): per-batch key counts, a sliding window with sink keys (the tiles it drops whole are not
+// walked) and the score functors and document ids of score_mod.h, each score through score_mod_at where
+// its probability is formed; the derivative of the functors multiplies the gradient of the scores.
+template <typename T, int ER, int DVR, int MODE>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
+  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const k_buf = wide_lds;                    // [2][TILE_ELEMS]
@@ -207,11 +211,22 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   const uint16_t* kp = (const uint16_t*)p.k + b * p.k_sb + hk * p.k_sh;
   const uint16_t* vp = (const uint16_t*)p.v + b * p.v_sb + hk * p.v_sh;
   int S = p.S;  // keys of this batch that take part
-  if constexpr (MASKED) {
+  if constexpr (MODE != 0) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
   }
   int nt = (S + BT - 1) / BT;
   if (p.causal) nt = min(nt, (min(q0 + 128, p.L) - 1) / BT + 1);
+  // sliding window: the tiles below the lowest window of the workgroup's rows are dropped whole, except
+  // the leading ones that hold sink keys: stream position u is key tile u + (u >= n_lead ? skip : 0)
+  int n_lead = 0, skip = 0;
+  if constexpr (FUNC) {
+    if (p.window > 0) {
+      const int t_lo = max(q0 - p.window + 1, 0) / BT;
+      n_lead = min(min((p.sink_keys + BT - 1) / BT, t_lo), nt);
+      skip = min(t_lo, nt) - n_lead;
+      nt -= skip;
+    }
+  }
   // With a skip table: the key tiles in which the mask keeps at least one score of this workgroup's
   // rows (the first wavefront ORs the bitmaps of its two 64-row blocks and expands the set bits into a
   // list in LDS); stream position u is then key tile tile_of(u).
@@ -245,10 +260,18 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   }
   auto tile_of = [&](int u) {
     if constexpr (MASKED) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
+    else if constexpr (FUNC) return u + (u >= n_lead ? skip : 0);
     else return u;
   };
-  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1) : nt;  // tiles with work for this wavefront
+  const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1 - skip) : nt;  // tiles with work for this wavefront
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  // (FUNC) the window of this lane's row, and what the derivative of the functors needs
+  const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
+  const int n_sink = FUNC ? p.sink_keys : 0;
+  const float inv_scale = FUNC ? 1.f / p.scale : 0.f;
+  const float icap = (FUNC && p.sm.softcap > 0.f) ? p.scale / p.sm.softcap : 0.f;
+  const float* const f_kw = (FUNC && p.sm.key_weight) ? p.sm.key_weight + (int64_t)h * p.S : nullptr;
+  const bool need_dfac = FUNC && (p.sm.softcap > 0.f || p.sm.key_weight != nullptr);
 
   // the buffers end with the last key row: rows of a ragged last tile beyond it read as zeros
   const u32x4 k_rsrc = wide_descriptor(kp, S > 0 ? ((int64_t)(S - 1) * p.k_sl + er) * 2 : 0);
@@ -329,7 +352,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   for (int t = 0; t < nt; ++t) {
     // (the other buffer was last read before the barrier that ended the previous tile)
     if (t + 1 < nt) request_tile(t + 1);
-    if (t < nt_w) {
+    // (FUNC: GENERAL is the tile as the functors, a window's edge or the diagonal need it; a tile inside
+    // the window of every row of a call without score functors is the plain tile, at the plain speed: tests
+    // per score, even uniform ones, cost this kernel a third of its time)
+    auto tile = [&](auto general_c) {
+      constexpr bool GENERAL = decltype(general_c)::value;
       const uint16_t* k_t = k_buf + (t & 1) * TILE_ELEMS;
       const uint16_t* v_t = v_buf + (t & 1) * TILE_ELEMS;
       // The LDS operands of a tile - row fragments of K and V in turns, then the transposed fragments
@@ -357,9 +384,27 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
       // is formed under the dQ ops of the first 16.
       float bl[16], pr[16];
       uint32_t pS[8];
+      if constexpr (FUNC && GENERAL) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bl[r] = 1.f;
+      }
       auto prob = [&](int r) {
         const int kv = ta * BT + (r >> 2) * 8 + half * 4 + (r & 3);
         float x;
+        if constexpr (FUNC && GENERAL) {
+          // (the scores went through the functors in a block of their own, see below; only dS is formed
+          // from this probability, so the functors' derivative rides on it: 1 - tanh^2 of the soft cap,
+          // recovered from the capped score, times the key's weight)
+          const bool dead = (kv > lim) | ((kv < lo_w) & (kv >= n_sink));
+          const float e = __builtin_amdgcn_exp2f(dead ? -INFINITY : fmaf(sacc[r], c, -lse2));
+          const float th = sacc[r] * icap;
+          pr[r] = e == 0.f ? 0.f : e * fmaf(-th, th, 1.f) * bl[r];  // (a dropped score may carry any derivative)
+          return;
+        }
+        if constexpr (FUNC) {  // (a tile that no mask touches)
+          pr[r] = __builtin_amdgcn_exp2f(fmaf(sacc[r], c, -lse2));
+          return;
+        }
         if constexpr (MASKED) x = fmaf(sacc[r], c, bl[r]) - lse2;
         else x = fmaf(sacc[r], c, -lse2);
         pr[r] = __builtin_amdgcn_exp2f(kv > lim ? -INFINITY : x);  // (masked before the exponential: no branch)
@@ -374,6 +419,19 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         if constexpr (op.kind) {
           dpacc = Mma<T>::run(ring[k & 7], dof[op.j], dpacc);
           if constexpr (op.j == 0 && MASKED) bias_log2(bl);
+          if constexpr (op.j == 0 && FUNC && GENERAL) {
+            // every score through the functors, in one block behind one test: s = mod(scale * s) / scale,
+            // so that the code around it is the common one (a call with a window alone skips the block)
+            if (p.sm.any) {
+#pragma unroll
+              for (int r = 0; r < 16; ++r) {
+                const int kv = min(ta * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1);
+                float dfac;
+                sacc[r] = score_mod_at(p.sm, sacc[r] * p.scale, b, h, qc, kv, p.L, p.S, dfac) * inv_scale;
+                if (f_kw) bl[r] = f_kw[kv];  // (the key's weight is the part of the derivative that the score does not tell)
+              }
+            }
+          }
 #pragma unroll
           for (int r = (op.j * 16) / KSV; r < ((op.j + 1) * 16) / KSV; ++r) prob(r);
         } else {
@@ -397,6 +455,17 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         }
         __builtin_amdgcn_sched_barrier(0);
       });
+    };
+    if (t < nt_w) {
+      if constexpr (FUNC) {
+        // does the tile cross the diagonal, the end of the keys or the edge of a window of this wavefront's rows?
+        const int k_lo = tile_of(t) * BT, k_hi = k_lo + BT - 1;
+        const bool edge_t = k_hi >= S || (p.causal && k_hi > qw0) || (p.window > 0 && k_lo < qw0 + 31 - p.window + 1 && k_hi >= p.sink_keys);
+        if (edge_t || need_dfac || p.sm.any) tile(std::true_type{});
+        else tile(std::false_type{});
+      } else {
+        tile(std::true_type{});
+      }
     }
 #pragma unroll
     for (int i = 0; i < DBE; ++i) asm volatile("" : "+a"(dqacc[i]));
@@ -419,8 +488,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
 // TABLES (masked instances): the tile skip table of a per-score mask is honoured.  At full width the
 // kernel has scalar registers for the table or for the split of a key block's query tiles over
 // workgroups, not for both: one instance of each.
-template <typename T, int ER, int DVR, bool MASKED, bool TABLES>
+template <typename T, int ER, int DVR, int MODE, bool TABLES>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
+  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // (see bwd_wide_dq_kernel)
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32, DBV = DVR / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const q_buf = wide_lds;                        // [2][TILE_ELEMS]
@@ -442,12 +512,16 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   const int er = p.d_real, dvr = p.dv_real;
 
   int S = p.S;  // keys of this batch that take part
-  if constexpr (MASKED) {
+  if constexpr (MODE != 0) {
     if (p.kv_lens) S = min(S, max(p.kv_lens[b], 0));
   }
   // the first query row that sees this lane's key: the key itself under a causal mask, none for a key
   // past the batch's count
   const int first_q = key >= S ? INT_MAX : p.causal ? key : INT_MIN;
+  // (FUNC) ... and the first row past its window, unless it is a sink key; what the functors' derivative needs
+  const int past_q = (FUNC && p.window > 0 && key >= p.sink_keys) ? key + p.window : INT_MAX;
+  const float inv_scale = FUNC ? 1.f / p.scale : 0.f;
+  const float icap = (FUNC && p.sm.softcap > 0.f) ? p.scale / p.sm.softcap : 0.f;
   u32x4 kf[KSE], vf[KSV];
   {
     const int kc = max(min(key, S - 1), 0);  // (a live row: rows past the batch's keys may hold anything)
@@ -473,12 +547,17 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 
   // Items: query tile by query tile from the last one down, heads inside: the workgroups of a kv head,
   // which share an XCD, then want the same Q / dO tile at about the same time and find it in its L2.
-  int qs_hi = nqs, qs_lo = qs_begin;  // this workgroup's query tiles: qs_hi - 1 down to qs_lo
-  if (parts_of() > 1) {
-    const int chunk = (nqs - qs_begin + parts_of() - 1) / parts_of();
-    qs_hi = nqs - part_of() * chunk, qs_lo = max(qs_hi - chunk, qs_begin);
+  // (sliding window: rows past the window of the block's last key see none of its keys, unless it holds sink keys)
+  int qs_top = nqs;
+  if constexpr (FUNC) {
+    if (p.window > 0 && k0 >= p.sink_keys) qs_top = max(min(nqs, (k0 + 128 + p.window - 2) / BT + 1), qs_begin);
   }
-  const int n_items = (MASKED && k0 >= S) ? 0 : max(qs_hi - qs_lo, 0) * rep;  // no live key in this block: zeros
+  int qs_hi = qs_top, qs_lo = qs_begin;  // this workgroup's query tiles: qs_hi - 1 down to qs_lo
+  if (parts_of() > 1) {
+    const int chunk = (qs_top - qs_begin + parts_of() - 1) / parts_of();
+    qs_hi = qs_top - part_of() * chunk, qs_lo = max(qs_hi - chunk, qs_begin);
+  }
+  const int n_items = (MODE != 0 && k0 >= S) ? 0 : max(qs_hi - qs_lo, 0) * rep;  // no live key in this block: zeros
   // bias of this lane's key in the 32 rows of an item, one element per score register, requested
   // ahead of the item's first product through a resource that ends with the (batch, head)'s last row
   const int bkind = MASKED ? __builtin_amdgcn_readfirstlane(p.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
@@ -583,7 +662,12 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     const int qs_n = hg + 1 < rep ? qs : qs - 1, hg_n = hg + 1 < rep ? hg + 1 : 0;
     if (!last && item_live(qs_n, hg_n)) request_item(qs_n, hg_n, buf ^ 1);
     const int q0 = qs * BT;
-    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= S) && item_live(qs, hg)) {  // (uniform per wavefront)
+    // (FUNC: every row of the tile past the window of every key of this wavefront, none of them a sink key)
+    const bool past_window = FUNC && p.window > 0 && q0 - (kw0 + 31) >= p.window && kw0 >= p.sink_keys;
+    if (!((p.causal && q0 + BT - 1 < kw0) || kw0 >= S || past_window) && item_live(qs, hg)) {  // (uniform per wavefront)
+      // (written in place, not as a lambda with a plain and a general variant as in the dQ kernel: wrapped,
+      // the full-width instances spill more, and the items of a window's inside gain little)
+      constexpr bool GENERAL = true;
       // (at full width the bias is requested behind the score products: ahead of them its 16
       // registers are more than the register file has left)
       if constexpr (ER + DVR <= 320) load_bias(hg, q0);
@@ -613,6 +697,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       u32x4 ring[8];
       static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       uint32_t pP[8], pS[8];
+      uint32_t pF[FUNC && GENERAL ? 8 : 1];  // (FUNC) the probabilities times the derivative of the functors, for dS
       // (at full width the register file has no room for the score and the dP accumulator at once next
       // to the two fragments: there the probabilities are formed before dP is issued, uncovered)
       constexpr bool BOTH = ER + DVR <= 320;
@@ -632,20 +717,59 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       else issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE>{});
       if constexpr (!BOTH) load_bias(hg, q0);
       if constexpr (MASKED) bias_to_log2();
+      // (FUNC) what the functors take from this lane's key, for the item's head
+      float f_w = 1.f;
+      if constexpr (FUNC && GENERAL) {
+        // every score through the functors, in one block behind one test: s = mod(scale * s) / scale, so
+        // that the code below is the common one (a call with a window alone skips the block)
+        if (p.sm.any) {
+          const int hq = hk * rep + hg, kc = max(min(key, p.S - 1), 0);
+          float f_kb = 0.f, f_slope = 0.f;
+          int f_doc = 0;
+          if (p.sm.key_weight) f_w = p.sm.key_weight[(int64_t)hq * p.S + kc];
+          if (p.sm.key_bias) f_kb = p.sm.key_bias[(int64_t)hq * p.S + kc];
+          if (p.sm.alibi) f_slope = p.sm.alibi[hq];
+          const bool docs = p.sm.doc_q && p.sm.doc_k;
+          if (docs) f_doc = p.sm.doc_k[(int64_t)b * p.S + kc];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            const int qi = q0 + (r >> 2) * 8 + half * 4 + (r & 3);
+            float u = fmaf(sacc[r] * p.scale, f_w, f_kb) + f_slope * (float)(key - qi);
+            if (p.sm.softcap > 0.f) u = p.sm.softcap * tanh_fast(u / p.sm.softcap);
+            if (docs && p.sm.doc_q[(int64_t)b * p.L + min(qi, p.L - 1)] != f_doc) u = -INFINITY;
+            sacc[r] = u * inv_scale;
+          }
+        }
+      }
 #pragma unroll
       for (int r4 = 0; r4 < 4; ++r4) {
         const f32x4 l4 = *(const f32x4*)(&lse_s[r4 * 8 + half * 4]);
         float pr[4];
+        float df[FUNC && GENERAL ? 4 : 1];
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
           const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
           float x;
-          if constexpr (MASKED) x = fmaf(sacc[r], c, __builtin_bit_cast(float, braw[r])) - l4[e];
-          else x = fmaf(sacc[r], c, -l4[e]);
+          if constexpr (FUNC && GENERAL) {
+            // (the scores went through the functors in a block of their own, see above; the derivative:
+            // 1 - tanh^2 of the soft cap, recovered from the capped score, times this key's weight)
+            x = qi >= past_q ? -INFINITY : fmaf(sacc[r], c, -l4[e]);
+            const float th = sacc[r] * icap;
+            df[e] = fmaf(-th, th, 1.f) * f_w;
+          } else if constexpr (MASKED) {
+            x = fmaf(sacc[r], c, __builtin_bit_cast(float, braw[r])) - l4[e];
+          } else {
+            x = fmaf(sacc[r], c, -l4[e]);
+          }
           // (masked before the exponential: a select around it is compiled into a branch per element)
           pr[e] = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : x);
         }
         pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+        if constexpr (FUNC && GENERAL) {  // (a dropped score may carry any derivative)
+#pragma unroll
+          for (int e = 0; e < 4; ++e) df[e] = pr[e] == 0.f ? 0.f : pr[e] * df[e];
+          pF[r4 * 2] = Mma<T>::pack(df[0], df[1]), pF[r4 * 2 + 1] = Mma<T>::pack(df[2], df[3]);
+        }
       }
       __builtin_amdgcn_sched_barrier(0);
       if constexpr (!BOTH) issue_dp();
@@ -656,7 +780,12 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
           float ds[4];
 #pragma unroll
           for (int e = 0; e < 4; ++e)
-            ds[e] = Mma<T>::unpack(pP[r4 * 2 + (e >> 1)], e & 1) * (dpacc[r4 * 4 + e] - d4[e]);
+          {
+            uint32_t w;
+            if constexpr (FUNC && GENERAL) w = pF[r4 * 2 + (e >> 1)];
+            else w = pP[r4 * 2 + (e >> 1)];
+            ds[e] = Mma<T>::unpack(w, e & 1) * (dpacc[r4 * 4 + e] - d4[e]);
+          }
           pS[r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
         }
         __builtin_amdgcn_sched_barrier(0);
@@ -692,21 +821,25 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       float* gk = p.part_dk + row * er + half * 4;
       float* gv = p.part_dv + row * dvr + half * 4;
 #pragma unroll
-      for (int db = 0; db < DBE; ++db)
+      for (int db = 0; db < DBE; ++db) {  // (block by block: left alone, every accumulator is read out before the first store)
 #pragma unroll
         for (int g = 0; g < 4; ++g)
           if (db * 32 + g * 8 + half * 4 < er) *(f32x4*)(gk + db * 32 + g * 8) = f32x4{dkacc[db][g * 4], dkacc[db][g * 4 + 1], dkacc[db][g * 4 + 2], dkacc[db][g * 4 + 3]};
+        __builtin_amdgcn_sched_barrier(0);
+      }
 #pragma unroll
-      for (int db = 0; db < DBV; ++db)
+      for (int db = 0; db < DBV; ++db) {
 #pragma unroll
         for (int g = 0; g < 4; ++g)
           if (db * 32 + g * 8 + half * 4 < dvr) *(f32x4*)(gv + db * 32 + g * 8) = f32x4{dvacc[db][g * 4], dvacc[db][g * 4 + 1], dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]};
+        __builtin_amdgcn_sched_barrier(0);
+      }
     }
   } else if (key < p.S) {
     uint16_t* gk = (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
     uint16_t* gv = (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
 #pragma unroll
-    for (int db = 0; db < DBE; ++db)
+    for (int db = 0; db < DBE; ++db) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 wk;
@@ -714,8 +847,10 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
         wk[1] = Mma<T>::pack(dkacc[db][g * 4 + 2] * p.scale, dkacc[db][g * 4 + 3] * p.scale);
         if (db * 32 + g * 8 + half * 4 < er) *(u32x2*)(gk + db * 32 + g * 8 + half * 4) = wk;
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
-    for (int db = 0; db < DBV; ++db)
+    for (int db = 0; db < DBV; ++db) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         u32x2 wv;
@@ -723,51 +858,56 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
         wv[1] = Mma<T>::pack(dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]);
         if (db * 32 + g * 8 + half * 4 < dvr) *(u32x2*)(gv + db * 32 + g * 8 + half * 4) = wv;
       }
+      __builtin_amdgcn_sched_barrier(0);
+    }
   }
 }
 
-template <typename T, int ER, int DVR, bool MASKED, bool TABLES>
+template <typename T, int ER, int DVR, int MODE, bool TABLES>
 int launch_dkdv(const BwdM& g, int64_t k_blocks, hipStream_t s) {
-  constexpr int kDkdvLds = WIDE_DKDV_LDS + (MASKED ? WIDE_LIVE_LDS : 0);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MASKED, TABLES>,
+  constexpr int kDkdvLds = WIDE_DKDV_LDS + (MODE == 1 ? WIDE_LIVE_LDS : 0);
+  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MODE, TABLES>,
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, kDkdvLds);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", kDkdvLds, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MASKED, TABLES>), dim3((unsigned)(k_blocks * g.parts)), dim3(256), kDkdvLds, s, g);
+  hipLaunchKernelGGL((bwd_wide_dkdv_kernel<T, ER, DVR, MODE, TABLES>), dim3((unsigned)(k_blocks * g.parts)), dim3(256), kDkdvLds, s, g);
   return check_launch("bwd_wide_dkdv_kernel");
 }
 
 // NO_TABLES: the masked full-width dK/dV instance that splits instead of reading a skip table
-template <typename T, int ER, int DVR, bool MASKED, bool NO_TABLES = false>
+template <typename T, int ER, int DVR, int MODE, bool NO_TABLES = false>
 int launch_t(const BwdM& g, hipStream_t s) {
   const int64_t q_blocks = (int64_t)g.B * g.Hq * ((g.L + 127) / 128), k_blocks = (int64_t)g.B * g.Hkv * ((g.S + 127) / 128);
   if (q_blocks > 0x7fffffff || k_blocks > 0x7fffffff) {
     set_error("SDPA: too many tiles for the wide backward kernels");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  constexpr int kDqLds = WIDE_DQ_LDS + (MASKED ? WIDE_LIST_LDS : 0);
-  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR, MASKED>,
+  constexpr int kDqLds = WIDE_DQ_LDS + (MODE == 1 ? WIDE_LIST_LDS : 0);
+  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR, MODE>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
   if (attr_q != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", kDqLds, hipGetErrorString(attr_q));
     return MI355_SDPA_ERR_LAUNCH;
   }
-  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR, MASKED>), dim3((unsigned)q_blocks), dim3(256), kDqLds, s, g);
+  hipLaunchKernelGGL((bwd_wide_dq_kernel<T, ER, DVR, MODE>), dim3((unsigned)q_blocks), dim3(256), kDqLds, s, g);
   int rc = check_launch("bwd_wide_dq_kernel");
   if (rc) return rc;
-  rc = launch_dkdv<T, ER, DVR, MASKED, MASKED && !(NO_TABLES && ER + DVR > 320)>(g, k_blocks, s);
+  rc = launch_dkdv<T, ER, DVR, MODE, MODE == 1 && !(NO_TABLES && ER + DVR > 320)>(g, k_blocks, s);
   if (rc || g.parts == 1) return rc;
   return launch_bwd_dkdv_merge(g, std::is_same<T, bf16_t>::value ? MI355_SDPA_BF16 : MI355_SDPA_F16, s);
 }
 // widths the kernels are instantiated for: 192 / 128 (multi-head latent attention) and the full 256 / 256
 template <typename T>
 int launch_w(const BwdM& g, hipStream_t s) {
+  const bool func = g.window > 0 || g.sm.any;  // (never together with a bias: refused before)
   const bool masked = g.bias_kind || g.kv_lens;
-  if (g.d_real <= 192 && g.dv_real <= 128) return masked ? launch_t<T, 192, 128, true>(g, s) : launch_t<T, 192, 128, false>(g, s);
-  if (masked && g.parts > 1) return launch_t<T, 256, 256, true, true>(g, s);  // (bwd_wide_parts: no skip table then)
-  return masked ? launch_t<T, 256, 256, true>(g, s) : launch_t<T, 256, 256, false>(g, s);
+  if (g.d_real <= 192 && g.dv_real <= 128)
+    return func ? launch_t<T, 192, 128, 2>(g, s) : masked ? launch_t<T, 192, 128, 1>(g, s) : launch_t<T, 192, 128, 0>(g, s);
+  if (func) return launch_t<T, 256, 256, 2>(g, s);
+  if (masked && g.parts > 1) return launch_t<T, 256, 256, 1, true>(g, s);  // (bwd_wide_parts: no skip table then)
+  return masked ? launch_t<T, 256, 256, 1>(g, s) : launch_t<T, 256, 256, 0>(g, s);
 }
 
 }  // namespace

@@ -55,7 +55,7 @@ struct FwdM {
   int window = 0, sink_keys = 0;
   const float* sink_logit = nullptr;
   int n_sinks = 1;  // logits per (batch, head) behind sink_logit
-  // score functors and document ids (fwd_mfma_w32.hip, the functor variant: head dims up to 128, no bias)
+  // score functors and document ids (fwd_mfma_w32.hip, the functor variant: no bias)
   ScoreMod sm;
   // tile skip table of the bias / keep-mask (variant with a bias, no causal flag): per (mask batch,
   // mask head, 64-row block) a bitmap of the key tiles with a kept score, live_words words each;

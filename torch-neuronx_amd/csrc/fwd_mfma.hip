@@ -367,8 +367,8 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   }
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;
   if (p.q.size[2] < 1 || p.k.size[2] < 1) return *why = "empty sequence", false;
-  if ((p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) && (p.bias.data || E > 128))
-    return *why = "window / sink / score functor together with attn_bias or a head dim above 128", false;
+  if ((p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) && p.bias.data)
+    return *why = "window / sink / score functor together with attn_bias", false;
   if (p.q.stride[3] != 1 || p.k.stride[3] != 1 || p.v.stride[3] != 1 || p.out.stride[3] != 1)
     return *why = "head dim is not unit-stride", false;
   const mi355_sdpa_tensor* ts[4] = {&p.q, &p.k, &p.v, &p.out};

@@ -48,7 +48,7 @@ constexpr float kLazy = 8.f;  // log2 headroom before the accumulator is rescale
 // scores, the row sums and the lse alone and zeroes the dropped probabilities where they are packed
 // for the second product; 1 / (1 - p) is applied with the final normalisation
 // (torch_neuronx/_sdpa_math.py:36-48: the mask multiplies the normalised probabilities).
-// MASK = 4 is MASK = 1 plus the score functors and document ids of score_mod.h (head dims up to 128):
+// MASK = 4 is MASK = 1 plus the score functors and document ids of score_mod.h:
 // they rewrite the raw score tile in a block of its own right after the matrix ops that produce it,
 // where the bias of MASK = 2 is folded in, so the softmax behind them is the common code.
 template <typename T, int D, int WAVES, int MASK>
@@ -67,8 +67,8 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   constexpr bool DYN = D > 128 || BIASED;
   // Tiles go from global memory straight into LDS (see the staging section): four unpadded,
   // swizzled buffers per operand, tile t in buffer t % 4.
-  // mask functors (window, sink keys, sink logit): in the masked variant without a bias, head dim <= 128
-  constexpr bool FUNC = (MASK == 1 || MASK == 4) && D <= 128;
+  // mask functors (window, sink keys, sink logit): in the masked variant without a bias
+  constexpr bool FUNC = MASK == 1 || MASK == 4;
   constexpr bool SMOD = MASK == 4;  // score functors, document ids
   constexpr int NBUF = 4, TILE = BN * D;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
@@ -954,8 +954,8 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
 }
 template <typename T, int D, int WAVES>
 int launch_mask(const FwdM& g, int mask, dim3 grid, hipStream_t s) {
+  if (mask == 4) return launch_one<T, D, WAVES, 4>(g, grid, s);
   if constexpr (D <= 128) {
-    if (mask == 4) return launch_one<T, D, WAVES, 4>(g, grid, s);
     if (mask == 3) return launch_one<T, D, WAVES, 3>(g, grid, s);
   }
   if (mask == 2) {
@@ -1043,8 +1043,8 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128 and the keep-mask in the bias slot");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  if (g.sm.any && (head_dim > 128 || g.bias_kind != 0 || g.keep_scale != 0.f)) {
-    set_error("SDPA: score functors in fwd_w32_kernel need a head dim up to 128, no bias and no dropout");
+  if (g.sm.any && (g.bias_kind != 0 || g.keep_scale != 0.f)) {
+    set_error("SDPA: score functors in fwd_w32_kernel go with no bias and no dropout");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   const int mask = g.sm.any ? 4 : g.keep_scale != 0.f ? 3 : g.bias_kind != 0 ? 2 : (g.kv_lens != nullptr || g.d_real != head_dim || g.dv_real != head_dim || g.window > 0 || g.sink_logit || g.split_tiles) ? 1 : 0;
