@@ -452,10 +452,10 @@ def test_sliding_window_mask_takes_the_window_kernel(amd, gpu_device, monkeypatc
 
 
 @pytest.mark.gpu
-def test_sliding_window_mask_at_head_dim_256_stays_a_tensor(amd, gpu_device, monkeypatch):
-    """The kernels for head dims above 128 have no window functor: a recognised window mask is kept as a
-    tensor there (with skip tables) and runs in the matrix-op kernels, forward and backward, instead of
-    becoming a functor that only the generic kernels take."""
+def test_sliding_window_mask_at_head_dim_256_takes_the_window_kernels(amd, gpu_device, monkeypatch):
+    """Head dims above 128 have the window functor in their matrix-op kernels too (the forward's functor
+    variant at width 256, the wide backward kernels' functor mode): a recognised window mask becomes the
+    functor there as well, forward and backward, and never reaches the generic kernels."""
     dev = gpu_device
     B, H, L, D, W = 1, 2, 1024, 256, 256
     q, k, v, go = qkv(B, H, H, L, L, D, dtype=torch.bfloat16, seed=6, with_do=True)
@@ -475,7 +475,7 @@ def test_sliding_window_mask_at_head_dim_256_stays_a_tensor(amd, gpu_device, mon
     out = F.scaled_dot_product_attention(qd, kd, vd, attn_mask=maskd)
     out.backward(go.to(dev))
     for kw in (seen[-1], seen_b[-1]):
-        assert kw["attn_bias"] is not None and not kw.get("window") and kw.get("live_tiles") is not None
+        assert kw["attn_bias"] is None and kw["is_causal"] is True and kw["window"] == W
     ro, rl = om.sdpa_forward(q.float(), k.float(), v.float(), attn_mask=keep)
     assert max_abs(out, ro) <= 2e-2
     rdq, rdk, rdv = om.sdpa_backward(go.float(), q.float(), k.float(), v.float(), ro, rl, attn_mask=keep, reduce_in_fp32=True)

@@ -84,11 +84,7 @@ def _wants_grad_bias(attn_bias, grad_input_mask) -> bool:
             and bool(grad_input_mask[3]))
 
 
-def _is_wide(query, value) -> bool:
-    return query.shape[-1] > 128 or value.shape[-1] != query.shape[-1]
-
-
-def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, wide=False, dropout_p=0.0):
+def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, dropout_p=0.0):
     """A mask that is a pattern the kernels generate by themselves (causal, sliding window with sink
     keys, keep-everything, either of the first two with right padding) is dropped in favour of that
     pattern - the run-time counterpart of the reference's causal-mask recovery
@@ -106,11 +102,6 @@ def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, wid
         return None, False, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
     if pat[0] == "causal":
         return None, True, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
-    if wide:
-        # head dims above 128 and D_qk != D_v have no window in their matrix-op kernels: there the mask
-        # stays a tensor (with its skip tables), which those kernels take, instead of a functor that
-        # only the generic kernels would
-        return attn_bias, is_causal, {}
     return None, True, {"window": pat[1], "sink_keys": pat[2]}
 
 
@@ -145,8 +136,7 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
         seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
     else:
         seed, offset = _empty_rng(query.device)
-    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, wide=_is_wide(query, value),
-                                                     dropout_p=dropout_p)
+    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, dropout_p=dropout_p)
     functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     out, lse = ops.sdpa_forward(query, key, value, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
                                 dropout_p=dropout_p, dropout_keep=keep, need_lse=need_lse,
@@ -183,8 +173,7 @@ def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p,
             dropout_p = 0.0  # a placeholder carries no mask: treated as absent (_sdpa_math.py:42-45)
         else:
             keep = philox_seed
-    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias,
-                                                     wide=_is_wide(query, value), dropout_p=dropout_p)
+    attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias, dropout_p=dropout_p)
     functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     dq, dk, dv, dbias = ops.sdpa_backward(
         grad_out, query, key, value, out, logsumexp, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
