@@ -316,6 +316,36 @@ def extra_wide(amd, dev):
     return r
 
 
+def extra_wide_window_softcap(amd, dev):
+    """Head dim 256 with a sliding window of 1024 keys and a tanh soft cap of 50 on the scores (the attention
+    of a Gemma-2 layer), both as functors: B=2 H=16 S=4096 bf16.  Rates count the scores the window keeps."""
+    B, H, S, D, W = 2, 16, 4096, 256, 1024
+    q, k, v, do = seeded([(B, H, S, D)] * 4, 1014, torch.bfloat16, dev)
+    live = sum(min(i + 1, W) for i in range(S))
+    r = _fwd_bwd_rates(amd, q, k, v, do, live, D, D, is_causal=True, window=W, softcap=50.0)
+    r["shape"] = "B=2 H=16 S=4096 D=256 bf16, causal window 1024 + soft cap 50"
+    return r
+
+
+def extra_fresh_bool_mask(amd, dev):
+    """F.scaled_dot_product_attention(attn_mask=bool lower triangle): upstream hands the op a NEW additive
+    tensor on every call, so no per-tensor cache can know it; the verdict about the mask is taken on the
+    device in front of the call (two small kernels), and the attention kernels follow it.  Forward time per
+    call over ten calls in a row, against is_causal=True: B=4 H=32 S=4096 D=128 bf16."""
+    import torch.nn.functional as F
+
+    B, H, S, D = 4, 32, 4096, 128
+    q, k, v = seeded([(B, H, S, D)] * 3, 1015, torch.bfloat16, dev)
+    tril = torch.ones(S, S, dtype=torch.bool, device=dev).tril()
+    amd.mask_patterns.clear_cache()
+    with torch.no_grad():
+        _, ev_m = event_time_ms(lambda: F.scaled_dot_product_attention(q, k, v, attn_mask=tril), 10, 3)
+        _, ev_c = event_time_ms(lambda: F.scaled_dot_product_attention(q, k, v, is_causal=True), 10, 3)
+    flops = 4.0 * B * H * D * causal_pairs(S, S)
+    return {"bool_mask_ms": ev_m, "is_causal_ms": ev_c, "ratio": ev_m / ev_c, "TFLOP/s_live": flops / (ev_m * 1e-3) / 1e12,
+            "shape": "B=4 H=32 S=4096 D=128 bf16, F.scaled_dot_product_attention(attn_mask=tril bool)"}
+
+
 def extra_dropout(amd, dev):
     """Dropout 0.1 with right padding, a BERT-base layer in training: B=32 H=12 S=512 D=64 bf16, key counts
     between S/2 and S, the (B,H,S,S) keep-mask drawn once.  Rates count the scores that the padding keeps."""
@@ -532,7 +562,8 @@ def main():
             extras["masked_fwd_shared_bias"] = {"error": repr(e)}
         for name, fn in (("window_1024_fwd_bwd", extra_window), ("document_mask_tables_fwd_bwd", extra_documents),
                          ("alibi_causal_fwd_bwd", extra_alibi), ("document_ids_fwd_bwd", extra_document_ids),
-                         ("head_dim_256_fwd_bwd", extra_wide), ("dropout_padding_fwd_bwd", extra_dropout), ("decode_bf16_cache_fwd", extra_decode_bf16),
+                         ("head_dim_256_fwd_bwd", extra_wide), ("head_dim_256_window_softcap_fwd_bwd", extra_wide_window_softcap),
+                         ("fresh_bool_mask_fwd", extra_fresh_bool_mask), ("dropout_padding_fwd_bwd", extra_dropout), ("decode_bf16_cache_fwd", extra_decode_bf16),
                          ("few_kv_heads_fwd_bwd", extra_few_kv_heads), ("float32_fwd_bwd", extra_f32)):
             try:
                 extras[name] = fn(amd, dev)

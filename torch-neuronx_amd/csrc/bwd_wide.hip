@@ -815,37 +815,56 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     if (!last) publish_item(buf);
     }
   }
+  // Results leave through buffer stores whose offset is pushed past the buffer's end where a lane has
+  // nothing to write (a key past S, columns past the real width): the hardware drops such a store, and
+  // the write-out is one straight run of stores (as tests per store it is a chain of 64 branches around
+  // which the compiler parks accumulators in scratch).
+  constexpr uint32_t kDrop = 0xfffffff0u;
+  const bool live_key = key < p.S;
   if (parts_of() > 1) {  // float32 rows for bwd_dkdv_merge_kernel, which also multiplies dK by the scale
-    if (key < p.S) {
-      const int64_t row = (((int64_t)part_of() * p.B + b) * p.Hkv + hk) * p.S + key;
-      float* gk = p.part_dk + row * er + half * 4;
-      float* gv = p.part_dv + row * dvr + half * 4;
-#pragma unroll
-      for (int db = 0; db < DBE; ++db) {  // (block by block: left alone, every accumulator is read out before the first store)
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-          if (db * 32 + g * 8 + half * 4 < er) *(f32x4*)(gk + db * 32 + g * 8) = f32x4{dkacc[db][g * 4], dkacc[db][g * 4 + 1], dkacc[db][g * 4 + 2], dkacc[db][g * 4 + 3]};
-        __builtin_amdgcn_sched_barrier(0);
-      }
-#pragma unroll
-      for (int db = 0; db < DBV; ++db) {
-#pragma unroll
-        for (int g = 0; g < 4; ++g)
-          if (db * 32 + g * 8 + half * 4 < dvr) *(f32x4*)(gv + db * 32 + g * 8) = f32x4{dvacc[db][g * 4], dvacc[db][g * 4 + 1], dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]};
-        __builtin_amdgcn_sched_barrier(0);
-      }
-    }
-  } else if (key < p.S) {
-    uint16_t* gk = (uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
-    uint16_t* gv = (uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
+    const int64_t row0 = (((int64_t)part_of() * p.B + b) * p.Hkv + hk) * p.S;
+    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr((char*)(p.part_dk + row0 * er)), 0,
+                                                                       __builtin_amdgcn_readfirstlane((int)((int64_t)p.S * er * 4)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(uniform_ptr((char*)(p.part_dv + row0 * dvr)), 0,
+                                                                       __builtin_amdgcn_readfirstlane((int)((int64_t)p.S * dvr * 4)), 0x00020000);
+    const uint32_t ok = (uint32_t)((key * er + half * 4) * 4), ov = (uint32_t)((key * dvr + half * 4) * 4);
 #pragma unroll
     for (int db = 0; db < DBE; ++db) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8;
+        const f32x4 w = {dkacc[db][g * 4], dkacc[db][g * 4 + 1], dkacc[db][g * 4 + 2], dkacc[db][g * 4 + 3]};
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, w), rk, (live_key && d + half * 4 < er) ? ok + d * 4 : kDrop, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);  // (block by block: left alone, every accumulator is read out before the first store)
+    }
+#pragma unroll
+    for (int db = 0; db < DBV; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8;
+        const f32x4 w = {dvacc[db][g * 4], dvacc[db][g * 4 + 1], dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]};
+        __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(u32x4, w), rv, (live_key && d + half * 4 < dvr) ? ov + d * 4 : kDrop, 0, 0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  } else {
+    const __amdgpu_buffer_rsrc_t rk = __builtin_amdgcn_make_buffer_rsrc(
+        uniform_ptr((char*)((uint16_t*)p.gk + b * p.gk_sb + hk * p.gk_sh)), 0,
+        __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.S - 1) * p.gk_sl + er) * 2)), 0x00020000);
+    const __amdgpu_buffer_rsrc_t rv = __builtin_amdgcn_make_buffer_rsrc(
+        uniform_ptr((char*)((uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh)), 0,
+        __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.S - 1) * p.gv_sl + dvr) * 2)), 0x00020000);
+    const uint32_t ok = (uint32_t)(((int64_t)key * p.gk_sl + half * 4) * 2), ov = (uint32_t)(((int64_t)key * p.gv_sl + half * 4) * 2);
+#pragma unroll
+    for (int db = 0; db < DBE; ++db) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8;
         u32x2 wk;
         wk[0] = Mma<T>::pack(dkacc[db][g * 4] * p.scale, dkacc[db][g * 4 + 1] * p.scale);
         wk[1] = Mma<T>::pack(dkacc[db][g * 4 + 2] * p.scale, dkacc[db][g * 4 + 3] * p.scale);
-        if (db * 32 + g * 8 + half * 4 < er) *(u32x2*)(gk + db * 32 + g * 8 + half * 4) = wk;
+        __builtin_amdgcn_raw_buffer_store_b64(wk, rk, (live_key && d + half * 4 < er) ? ok + d * 2 : kDrop, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
@@ -853,10 +872,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
     for (int db = 0; db < DBV; ++db) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
+        const int d = db * 32 + g * 8;
         u32x2 wv;
         wv[0] = Mma<T>::pack(dvacc[db][g * 4], dvacc[db][g * 4 + 1]);
         wv[1] = Mma<T>::pack(dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]);
-        if (db * 32 + g * 8 + half * 4 < dvr) *(u32x2*)(gv + db * 32 + g * 8 + half * 4) = wv;
+        __builtin_amdgcn_raw_buffer_store_b64(wv, rv, (live_key && d + half * 4 < dvr) ? ov + d * 2 : kDrop, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
     }
