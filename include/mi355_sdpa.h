@@ -142,11 +142,13 @@ typedef struct mi355_sdpa_mask_spec {
   const int32_t* doc_ids_k;
   int32_t doc_ids_sorted;
   const int32_t* mask_verdict; /* optional, with a bias / keep-mask: what mi355_sdpa_mask_verdict wrote
-                                  about that tensor.  The matrix-op kernels for 16-bit inputs at head
-                                  dims up to 128 read it in their prologue and, when the mask is the
-                                  keep-everything or the causal pattern (with or without right padding),
-                                  run as if is_causal / kv_lens had been given and never read the mask;
-                                  every other kernel, and every other verdict, uses the mask itself   */
+                                  about that tensor.  The call is then put on the stream as a pair of
+                                  kernels - with the mask, and with the causal flag and key counts -
+                                  whose first instructions read the verdict: a mask that is the
+                                  keep-everything or the causal pattern (with or without right padding)
+                                  is never read.  Matrix-op kernels for 16-bit inputs, head dims up to
+                                  128 (the forward: up to 256), a mask with a row per query, nothing else
+                                  shaping the scores; every other call uses the mask itself           */
 } mi355_sdpa_mask_spec;
 
 typedef struct mi355_sdpa_fwd_params {
