@@ -54,7 +54,7 @@ enum mi355_sdpa_kernel {
   MI355_SDPA_KERNEL_GENERIC = 1, /* fp32-accumulate kernel: any head dim, bias, masks, dropout */
   MI355_SDPA_KERNEL_MFMA = 2,    /* matrix-op flash kernels: bf16/f16 (head dims up to 256, masks,
                                     functors; dropout up to head dim 128 without a bias) and float32
-                                    (head dims up to 128; masks, key counts, dropout) */
+                                    (head dims up to 128; masks, key counts, dropout, functors) */
   /* forward only, for tests and tuning: pin the query rows per workgroup of the MFMA kernel */
   MI355_SDPA_KERNEL_MFMA_T128 = 3,
   MI355_SDPA_KERNEL_MFMA_T256 = 4
@@ -117,8 +117,9 @@ typedef struct mi355_sdpa_desc {
  *                rows, the range of key tiles that can hold an equal id and walk only those, and
  *                test whole tiles with two loads.  Without the promise every tile is walked and
  *                every score compared: same results, no skipping.
- * Score functors and document ids run in the matrix-op kernels for bf16 / f16, head dims up to 128
- * with D_qk = D_v, without attn_bias and dropout; other calls take the generic kernels.
+ * Score functors and document ids run in the matrix-op kernels for bf16 / f16 at every head dim up
+ * to 256 (D_v <= D_qk) and for float32 up to 128, without attn_bias and dropout; other calls take
+ * the generic kernels.
  * Tile skip tables for a mask that only exists as a tensor (the run-time counterpart of the
  * reference's static tile elimination, flex_attention.py.jinja:15-33), built from the bias /
  * keep-mask by mi355_sdpa_mask_tiles and valid as long as that tensor is unchanged:
@@ -207,9 +208,10 @@ typedef struct mi355_sdpa_bwd_params {
 } mi355_sdpa_bwd_params;
 
 typedef struct mi355_sdpa_decode_params {
-  mi355_sdpa_tensor q;      /* (B,Hq,Lq,D) bf16/f16/f32, D = 128, Lq*Hq/Hkv <= 16.  The
-                               query is carried exactly (bf16), with 12 to 16 significant
-                               bits (f16) or with 16 (f32): see decode_fp8kv.hip           */
+  mi355_sdpa_tensor q;      /* (B,Hq,Lq,D) bf16/f16/f32, D = 64, 128 or 256, Lq*Hq/Hkv <= 16.
+                               The query is carried exactly (bf16), with 12 to 16 significant
+                               bits (f16) or with 16 (f32; 12 at D = 256 with more than 8
+                               rows per kv head): see decode_fp8kv.hip                     */
   mi355_sdpa_tensor k;      /* (B,Hkv,S,D)  fp8 e4m3fn, 1 byte per element             */
   mi355_sdpa_tensor v;      /* (B,Hkv,S,D)  fp8 e4m3fn                                 */
   const float* k_scale;     /* (B,Hkv) contiguous: real K = fp8 value * k_scale        */

@@ -21,11 +21,11 @@ def amd(gpu_device):
     return amd
 
 
-def _case(B, Hq, Hkv, Lq, S, lens, seed, qdtype=torch.bfloat16):
+def _case(B, Hq, Hkv, Lq, S, lens, seed, qdtype=torch.bfloat16, D=128):
     g = torch.Generator().manual_seed(seed)
-    q = torch.randn(B, Hq, Lq, 128, generator=g).to(qdtype)
-    k = torch.randn(B, Hkv, S, 128, generator=g)
-    v = torch.randn(B, Hkv, S, 128, generator=g)
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(qdtype)
+    k = torch.randn(B, Hkv, S, D, generator=g)
+    v = torch.randn(B, Hkv, S, D, generator=g)
     kq, ks = om.quantize_kv_fp8(k)
     vq, vs = om.quantize_kv_fp8(v)
     return q, kq, vq, ks, vs, lens
@@ -178,6 +178,34 @@ def test_decode_float32_query_with_one_key(amd, gpu_device):
 def test_decode_up_to_sixteen_query_rows_per_kv_head(amd, gpu_device, qdtype, Hq, Hkv, Lq):
     lens = torch.tensor([700, 1, 33, 0], dtype=torch.int32)
     _check(amd, gpu_device, _case(4, Hq, Hkv, Lq, 700, lens, seed=Hq + Lq, qdtype=qdtype))
+
+
+@pytest.mark.parametrize("D", [64, 256])
+@pytest.mark.parametrize("qdtype", [torch.bfloat16, torch.float16, torch.float32])
+@pytest.mark.parametrize("Hq,Hkv,Lq", [(32, 8, 1), (8, 8, 1), (8, 1, 1), (16, 1, 1), (4, 2, 3)])
+def test_decode_head_dims_64_and_256(amd, gpu_device, D, qdtype, Hq, Hkv, Lq):
+    # the same kernel laid out for 64- and 256-byte cache rows, every group size (terms x passes) of each query dtype
+    lens = torch.tensor([700, 1, 33, 0, 513], dtype=torch.int32)
+    case = _case(5, Hq, Hkv, Lq, 700, lens, seed=D + Hq + Lq, qdtype=qdtype, D=D)
+    out, _ = _check(amd, gpu_device, case)
+    assert torch.equal(out[3].float().cpu(), torch.zeros(Hq, Lq, D))  # the empty sequence
+    _check(amd, gpu_device, case, scale=0.3)  # larger logits (the default scale at 256 is 1/16)
+
+
+def test_decode_head_dims_64_and_256_long_and_split(amd, gpu_device):
+    # sequences that several wavefronts share, with and without a cap on the pieces per sequence
+    for D in (64, 256):
+        case = _case(2, 32, 8, 1, 4096, torch.tensor([4096, 3001], dtype=torch.int32), seed=D, D=D)
+        a, _ = _check(amd, gpu_device, case)
+        b, _ = _check(amd, gpu_device, case, num_splits=1)
+        assert max_abs(a, b) <= 4e-3
+
+
+def test_decode_refuses_other_head_dims(amd, gpu_device):
+    dev = gpu_device
+    q, kq, vq, ks, vs, _ = _case(1, 8, 8, 1, 64, None, seed=1, D=96)
+    with pytest.raises(RuntimeError, match="64, 128 or 256"):
+        amd.decode_fp8kv(q.to(dev), kq.to(dev), vq.to(dev), ks.to(dev), vs.to(dev), None)
 
 
 def test_decode_refuses_more_than_sixteen_rows(amd, gpu_device):

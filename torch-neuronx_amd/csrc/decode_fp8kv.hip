@@ -20,9 +20,11 @@
 // gets three or four, a float32 query four (16 bits).  The probabilities are split the same way
 // before P*V.
 //
+// Head dims 64, 128 and 256 are instances of one kernel; the description is for 128.
 // Per 32 keys a lane loads two 16-byte pieces of each of two keys (A operand of S^T = K Q^T; the
 // contraction order is permuted identically for Q) and eight 8-byte pieces of V, one from each
-// of eight keys, which are byte-transposed in registers into the A operand of O^T = V^T P^T.
+// of eight keys, which are byte-transposed in registers into the A operand of O^T = V^T P^T
+// (head dim 64: one piece per key and 4-byte pieces of V; 256: four and 16-byte pieces).
 // Every load is non-temporal (the cache is read once) and a V instruction covers four whole
 // 128-byte rows: with plain loads the stream reads 5.8 TB/s whatever the shape, with
 // non-temporal ones 5.8 TB/s when a row is fetched in two instructions and 6.5 TB/s when in one
@@ -46,10 +48,11 @@ typedef __attribute__((ext_vector_type(4))) float f32x4;
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;
 typedef __attribute__((ext_vector_type(2))) float f32x2;
 
-constexpr int D = 128;
 constexpr float kLog2e = 1.4426950408889634f;
 constexpr float kLn2 = 0.6931471805599453f;
-constexpr int kDecOcc = 2;  // wavefronts per SIMD the decode kernel is built for (three or four spill)
+// wavefronts per SIMD the decode kernel is built for (at head dims up to 128 three or four spill; at 256
+// the two K/V tiles in flight and the output accumulators alone take 190 registers: one)
+constexpr int dec_occ(int D) { return D > 128 ? 1 : 2; }
 constexpr float kPScale = 256.f;  // probabilities are stored as e4m3 of 256*p
 
 struct DecP {
@@ -59,7 +62,7 @@ struct DecP {
   const int32_t* kv_lens;
   void* out;
   float* lse;
-  float* ws_o;        // (slots,R,128) partial outputs; slot = b*Hkv + hk + wavefront index
+  float* ws_o;        // (slots,R,D) partial outputs; slot = b*Hkv + hk + wavefront index
   float* ws_ml;       // (slots,R,2)   partial (max, sum)
   int32_t* ws_steps;  // (B+1) exclusive prefix of the 32-key step counts per batch, then the total
   int64_t q_sb, q_sh, q_sl;
@@ -120,9 +123,12 @@ __device__ __forceinline__ long as_long(uint32_t lo, uint32_t hi) {
 }
 
 typedef __attribute__((ext_vector_type(2))) uint32_t u32x2;
+// Head dims 64, 128 and 256: a K row is D/64 pieces of 64 bytes, of which lane group g takes 16 each
+// (two contraction steps of 32 per piece); a V row is 16 pieces of D/16 bytes, one per lane n.
+template <int D>
 struct KVRegs {
-  u32x4 k[2][2];  // [16-key block][d = 16g .. +15 | d = 64 + 16g .. +15] of the lane's key
-  u32x2 v[8];     // [key slot s]: d = 8n .. 8n+7 of key 4s + g
+  u32x4 k[2][D / 64];     // [16-key block][piece pc]: d = 64 pc + 16g .. +15 of the lane's key
+  uint32_t v[8][D / 64];  // [key slot s]: d = (D/16) n .. +D/16-1 of key 4s + g, as dwords
 };
 
 // Steps per wavefront for a work list of `total` steps: equal shares, but not so small that the
@@ -139,10 +145,14 @@ __device__ __forceinline__ int steps_per_wave(int total, int n_waves, int t_min)
 // While an item streams, the query rows of the next one are already in flight (they wait in
 // registers), and its first K/V tile is requested before the epilogue of the current one, so the
 // memory pipe of a wavefront never drains between items.
-template <typename TQ, int PARTS, int PASSES>
-__global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
+template <typename TQ, int D, int PARTS, int PASSES>
+__global__ __launch_bounds__(64, dec_occ(D)) void decode_kernel(DecP p) {
   constexpr int RS = PARTS >= 3 ? 4 : PARTS == 2 ? 8 : 16;  // column stride between split terms
-  constexpr int QV = sizeof(TQ) == 4 ? 8 : 4;  // 16-byte loads per 32 query elements
+  constexpr int NPC = D / 64;               // 64-byte pieces of a K row = dwords of a lane's V piece
+  constexpr int KST = D / 32;               // contraction steps of S^T = K Q^T
+  constexpr int PB = D / 16;                // bytes of a lane's V piece = output rows per lane n
+  constexpr int LPP = (int)sizeof(TQ);      // 16-byte loads per 16 query elements (one piece of the lane)
+  constexpr int QV = NPC * LPP;             // 16-byte loads of the lane's D/4 query elements
   const int lane = threadIdx.x;
   const int n = lane & 15, g = lane >> 4;
   const int part = n / RS, r = n % RS;
@@ -221,15 +231,15 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     const TQ* qr = (const TQ*)p.q + it.b * p.q_sb + (it.hk * rep + hq_off) * p.q_sh + lq * p.q_sl + 16 * g;
 #pragma unroll
     for (int i = 0; i < QV; ++i)
-      qraw[i] = *(const qraw_t*)((const char*)(qr + (i >= QV / 2 ? 64 : 0)) + 16 * (i % (QV / 2)));
+      qraw[i] = *(const qraw_t*)((const char*)(qr + 64 * (i / LPP)) + 16 * (i % LPP));
   };
 
-  KVRegs ra, rb;
+  KVRegs<D> ra, rb;
   // Which key is which: the score tile of a 16-key block leaves the matrix op with rows 4g .. 4g+3
   // in lane group g, and the second product wants lane group g to hold the probabilities of the keys
   // whose V pieces it loaded, 4s + g for s = 0 .. 7.  So row m of block blk is key 16 blk + 4 (m % 4)
   // + m / 4: accumulator register i of block blk in lane group g is key 16 blk + 4 i + g, slot s = 4 blk + i.
-  auto load = [&](KVRegs& R_, const Item& it, int step) {
+  auto load = [&](KVRegs<D>& R_, const Item& it, int step) {
     const uint8_t* kp = p.k + it.b * p.k_sb + it.hk * p.k_sh;
     const uint8_t* vp = p.v + it.b * p.v_sb + it.hk * p.v_sh;
     const int base = it.begin + step * 32, last = it.end - 1;
@@ -238,22 +248,31 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     for (int blk = 0; blk < 2; ++blk) {
       const int row = min(base + blk * 16 + 4 * (n & 3) + (n >> 2), last);
       const uint8_t* kr = kp + (uint32_t)(row * ksl + 16 * g);
-      R_.k[blk][0] = __builtin_nontemporal_load((const u32x4*)kr);
-      R_.k[blk][1] = __builtin_nontemporal_load((const u32x4*)(kr + 64));
+#pragma unroll
+      for (int pc = 0; pc < NPC; ++pc) R_.k[blk][pc] = __builtin_nontemporal_load((const u32x4*)(kr + 64 * pc));
     }
 #pragma unroll
     for (int s = 0; s < 8; ++s) {
       const int row = min(base + 4 * s + g, last);
-      R_.v[s] = __builtin_nontemporal_load((const u32x2*)(vp + (uint32_t)(row * vsl + 8 * n)));
+      const uint8_t* vr = vp + (uint32_t)(row * vsl + PB * n);
+      if constexpr (NPC == 1) {
+        R_.v[s][0] = __builtin_nontemporal_load((const uint32_t*)vr);
+      } else if constexpr (NPC == 2) {
+        const u32x2 w = __builtin_nontemporal_load((const u32x2*)vr);
+        R_.v[s][0] = w[0], R_.v[s][1] = w[1];
+      } else {
+        const u32x4 w = __builtin_nontemporal_load((const u32x4*)vr);
+        R_.v[s][0] = w[0], R_.v[s][1] = w[1], R_.v[s][2] = w[2], R_.v[s][3] = w[3];
+      }
     }
   };
 
   // Query fragment of the item fetched last: B operand of S^T = K Q^T.
-  // The lane owns d = 16g .. 16g+15 and 64+16g .. 64+16g+15 of row r, as for K; MFMA steps 0, 1
-  // consume the first group, steps 2, 3 the second.
+  // The lane owns d = 64 pc + 16g .. +15 of row r for every piece pc, as for K; MFMA steps 2 pc and
+  // 2 pc + 1 consume piece pc.
   // Returns the factor that turns a raw fp8 dot product into a log2-domain logit.
-  auto convert_q = [&](const Item& it, long (&qb)[PASSES][4]) -> float {
-    float qv[32];
+  auto convert_q = [&](const Item& it, long (&qb)[PASSES][KST]) -> float {
+    float qv[D / 4];
     {
       typedef __attribute__((ext_vector_type(16 / sizeof(TQ)))) TQ qvec_t;
       constexpr int PER = 16 / sizeof(TQ);
@@ -266,13 +285,13 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     }
     float amax = 0.f;
 #pragma unroll
-    for (int i = 0; i < 32; ++i) amax = fmaxf(amax, fabsf(qv[i]));
+    for (int i = 0; i < D / 4; ++i) amax = fmaxf(amax, fabsf(qv[i]));
     amax = fmaxf(amax, __shfl_xor(amax, 16, 64));
     amax = fmaxf(amax, __shfl_xor(amax, 32, 64));
     // power-of-two pre-scale so the row peaks in [120, 240]: well inside e4m3 and exact
     const float f = amax > 0.f ? __builtin_amdgcn_exp2f(floorf(__builtin_amdgcn_logf(240.f / amax))) : 1.f;
 #pragma unroll
-    for (int ks = 0; ks < 4; ++ks) {
+    for (int ks = 0; ks < KST; ++ks) {
       uint32_t w[4][PASSES];
 #pragma unroll
       for (int jq = 0; jq < 4; ++jq)
@@ -287,7 +306,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
   Item cur = decode_item(G);
   fetch_q(cur);
   load(ra, cur, 0);
-  long qb[PASSES][4];
+  long qb[PASSES][KST];
   float c_row = convert_q(cur, qb);
 
   while (true) {
@@ -302,13 +321,13 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       nxt.begin = cur.end - 1;  // no next item: the unconditional tile request below re-reads one cached row
     }
 
-    f32x4 oacc[8];
+    f32x4 oacc[PB];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < PB; ++i) oacc[i] = f32x4{0.f, 0.f, 0.f, 0.f};
     float m_run = -INFINITY, l_run = 0.f;
     const int w_end = cur.end;
 
-    auto compute = [&](const KVRegs& R_, int step) {
+    auto compute = [&](const KVRegs<D>& R_, int step) {
       const int base = cur.begin + step * 32;
       // S^T = K Q^T : rows = 16 keys of a block, columns = (split term, query row)
       f32x4 sacc[2];
@@ -316,7 +335,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       for (int blk = 0; blk < 2; ++blk) {
         sacc[blk] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int ks = 0; ks < 4; ++ks) {
+        for (int ks = 0; ks < KST; ++ks) {
           const u32x4 kk = R_.k[blk][ks >> 1];
           const long a = as_long(kk[(ks & 1) * 2], kk[(ks & 1) * 2 + 1]);
 #pragma unroll
@@ -346,7 +365,7 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       }
       l_run = l_run * alpha + psum;
 #pragma unroll
-      for (int i = 0; i < 8; ++i) oacc[i] *= alpha;
+      for (int i = 0; i < PB; ++i) oacc[i] *= alpha;
       // P^T (B operand): key slot s of this lane is key 4 s + g, the order V is loaded in
       uint32_t pw[4][PASSES];
 #pragma unroll
@@ -355,10 +374,10 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       long pb[PASSES];
 #pragma unroll
       for (int ps = 0; ps < PASSES; ++ps) pb[ps] = as_long(pw[0][ps] | (pw[1][ps] << 16), pw[2][ps] | (pw[3][ps] << 16));
-      // O^T += V^T P^T : the lane holds bytes d = 8n + e (e = 0 .. 7) of its eight keys; matrix op e
-      // takes byte e of every key (rows d = 8n + e), an 8 x 8 byte transpose done as four 4 x 4 ones
+      // O^T += V^T P^T : the lane holds bytes d = PB n + e (e = 0 .. PB-1) of its eight keys; matrix op e
+      // takes byte e of every key (rows d = PB n + e), an 8 x PB byte transpose done as 4 x 4 ones
 #pragma unroll
-      for (int hf = 0; hf < 2; ++hf) {  // e = 4 hf .. 4 hf + 3: dword hf of every piece
+      for (int hf = 0; hf < NPC; ++hf) {  // e = 4 hf .. 4 hf + 3: dword hf of every piece
         uint32_t o_lo[4], o_hi[4];      // [e % 4]: key slots 0 .. 3 / 4 .. 7
 #pragma unroll
         for (int q4 = 0; q4 < 2; ++q4) {
@@ -400,13 +419,13 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
     } while (s < steps);
     // all tiles of this item are consumed; what is in flight is the next item's first tile, and
     // its query rows landed long ago: build its fragment now, ahead of the stores below
-    long qb_next[PASSES][4];
+    long qb_next[PASSES][KST];
     float c_next = 0.f;
     if (more) c_next = convert_q(nxt, qb_next);
 
     // ---- merge the split terms and emit this item's partial result -------------------------------
 #pragma unroll
-    for (int i = 0; i < 8; ++i)
+    for (int i = 0; i < PB; ++i)
 #pragma unroll
       for (int e = 0; e < 4; ++e) oacc[i][e] = sum_parts<PARTS>(oacc[i][e]);
     float l_tot = l_run + __shfl_xor(l_run, 16, 64);
@@ -415,13 +434,13 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
       const float vscale = cur.vscale * (1.f / kPScale);
       const int64_t slot = (int64_t)cur.slot * p.R + n;
       if (g == 0) p.ws_ml[slot * 2] = m_run, p.ws_ml[slot * 2 + 1] = l_tot;
-      // (register a of matrix op e is row d = 8 (4g + a) + e of O^T)
-      float* dst = p.ws_o + slot * D + 32 * g;
+      // (register a of matrix op e is row d = PB (4g + a) + e of O^T)
+      float* dst = p.ws_o + slot * D + 4 * PB * g;
 #pragma unroll
       for (int a = 0; a < 4; ++a)
 #pragma unroll
-        for (int e4 = 0; e4 < 2; ++e4)
-          *(f32x4*)(dst + 8 * a + 4 * e4) = f32x4{oacc[4 * e4][a], oacc[4 * e4 + 1][a], oacc[4 * e4 + 2][a], oacc[4 * e4 + 3][a]} * vscale;
+        for (int e4 = 0; e4 < NPC; ++e4)
+          *(f32x4*)(dst + PB * a + 4 * e4) = f32x4{oacc[4 * e4][a], oacc[4 * e4 + 1][a], oacc[4 * e4 + 2][a], oacc[4 * e4 + 3][a]} * vscale;
     }
     if (!more) break;
     G = g_next;
@@ -430,16 +449,17 @@ __global__ __launch_bounds__(64, kDecOcc) void decode_kernel(DecP p) {
 #pragma unroll
     for (int ps = 0; ps < PASSES; ++ps)
 #pragma unroll
-      for (int ks = 0; ks < 4; ++ks) qb[ps][ks] = qb_next[ps][ks];
+      for (int ks = 0; ks < KST; ++ks) qb[ps][ks] = qb_next[ps][ks];
   }
 }
 
-// Merge the partials of one (batch, kv head, query row); 128 threads = 128 output columns.
+// Merge the partials of one (batch, kv head, query row); D threads = D output columns.
 // The wavefronts that touched this (batch, kv head) follow from the step numbering alone, and
 // their partials sit in consecutive slots.
-template <typename TQ>
+template <typename TQ, int D>
 __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
-  __shared__ float s_red[2][2];
+  constexpr int NW = D / 64;  // wavefronts of the workgroup
+  __shared__ float s_red[2][4];
   const int row = blockIdx.x % p.R;
   const int hk = (blockIdx.x / p.R) % p.Hkv;
   const int b = blockIdx.x / (p.R * p.Hkv);
@@ -477,7 +497,9 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     M = wave_max(M);
     if ((d & 63) == 0) s_red[0][d >> 6] = M;
     __syncthreads();
-    M = fmaxf(s_red[0][0], s_red[0][1]);
+    M = s_red[0][0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) M = fmaxf(M, s_red[0][w]);
     for (int c = d; c < npart; c += D) {
       const int64_t s = slot0 + (int64_t)c * p.R;
       L += p.ws_ml[s * 2 + 1] * __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
@@ -485,7 +507,9 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     L = wave_sum(L);
     if ((d & 63) == 0) s_red[1][d >> 6] = L;
     __syncthreads();
-    L = s_red[1][0] + s_red[1][1];
+    L = s_red[1][0];
+#pragma unroll
+    for (int w = 1; w < NW; ++w) L += s_red[1][w];
     for (int c = 0; c < npart; ++c) {
       const int64_t s = slot0 + (int64_t)c * p.R;
       O = fmaf(p.ws_o[s * D + d], __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M), O);
@@ -502,17 +526,17 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
 constexpr int kMaxWaves = 4096;  // bound on the streaming kernel's grid; sizes the workspace
 constexpr int kMinSteps = 4;     // 128 keys: below this the partial results rival the keys in bytes
 
-int wave_slots() {  // wavefronts of the decode kernel the chip holds at once
-  static int slots = 0;
-  if (!slots) {
+int wave_slots(int head_dim) {  // wavefronts of the decode kernel the chip holds at once
+  static int simds = 0;
+  if (!simds) {
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) == hipSuccess &&
         hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && cus > 0)
-      slots = std::min(cus * 4 * kDecOcc, kMaxWaves);
+      simds = cus * 4;
     else
-      slots = 256 * 4 * kDecOcc;
+      simds = 256 * 4;
   }
-  return slots;
+  return std::min(simds * dec_occ(head_dim), kMaxWaves);
 }
 
 // least steps per wavefront: num_splits > 0 asks for at most about that many pieces per sequence
@@ -527,10 +551,10 @@ int min_steps_for(const mi355_sdpa_decode_params& p) {
 // a term - bf16 two (three where the columns are free anyway), float16 three or four, float32 four -
 // laid out as PARTS column groups per matrix op times PASSES trips through the matrix ops, by the
 // number of query rows R that share the 16 columns.
-template <typename TQ>
-int launch_t(const DecP& g, hipStream_t s) {
+template <typename TQ, int D>
+int launch_td(const DecP& g, hipStream_t s) {
   constexpr bool BF = std::is_same<TQ, bf16_t>::value, F32 = sizeof(TQ) == 4;
-#define DECODE(PARTS, PASSES) hipLaunchKernelGGL((decode_kernel<TQ, PARTS, PASSES>), dim3(g.n_waves), dim3(64), 0, s, g)
+#define DECODE(PARTS, PASSES) hipLaunchKernelGGL((decode_kernel<TQ, D, PARTS, PASSES>), dim3(g.n_waves), dim3(64), 0, s, g)
   if (g.R <= 4) {
     if constexpr (F32) DECODE(4, 1);
     else DECODE(3, 1);
@@ -539,14 +563,18 @@ int launch_t(const DecP& g, hipStream_t s) {
     else DECODE(2, 2);
   } else {
     if constexpr (BF) DECODE(1, 2);
-    else if constexpr (F32) DECODE(1, 4);
-    else DECODE(1, 3);
+    else if constexpr (F32 && D <= 128) DECODE(1, 4);
+    else DECODE(1, 3);  // (float32 at head dim 256: three terms, 12 bits - a fourth pass spills)
   }
 #undef DECODE
   int rc = check_launch("decode_kernel");
   if (rc) return rc;
-  hipLaunchKernelGGL((decode_merge_kernel<TQ>), dim3(g.B * g.Hkv * g.R), dim3(D), 0, s, g);
+  hipLaunchKernelGGL((decode_merge_kernel<TQ, D>), dim3(g.B * g.Hkv * g.R), dim3(D), 0, s, g);
   return check_launch("decode_merge_kernel");
+}
+template <typename TQ>
+int launch_t(const DecP& g, int head_dim, hipStream_t s) {
+  return head_dim == 64 ? launch_td<TQ, 64>(g, s) : head_dim == 128 ? launch_td<TQ, 128>(g, s) : launch_td<TQ, 256>(g, s);
 }
 
 int64_t partial_slots(const mi355_sdpa_decode_params& p) { return p.q.size[0] * p.k.size[1] + kMaxWaves; }
@@ -563,6 +591,7 @@ int decode_pick_splits(const mi355_sdpa_decode_params& p) {
 size_t decode_workspace(const mi355_sdpa_decode_params& p) {
   const int64_t rep = p.k.size[1] ? p.q.size[1] / p.k.size[1] : 0;
   const int64_t R = rep * p.q.size[2];
+  const int64_t D = p.q.size[3];
   return (size_t)(partial_slots(p) * R * (D + 2)) * sizeof(float) + (size_t)(p.q.size[0] + 1) * sizeof(int32_t);
 }
 
@@ -592,9 +621,10 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
   g.Hkv = (int)p.k.size[1], g.S = (int)p.k.size[2];
   const int rep = g.Hq / g.Hkv;
   g.R = rep * g.Lq;
-  if (p.q.size[3] != D || p.v.size[3] != D)
-    return set_error("SDPA decode: head dim must be 128, got %lld/%lld", (long long)p.q.size[3],
-                     (long long)p.v.size[3]), MI355_SDPA_ERR_UNSUPPORTED;
+  const int D = (int)p.q.size[3];
+  if ((D != 64 && D != 128 && D != 256) || p.v.size[3] != D || p.k.size[3] != D)
+    return set_error("SDPA decode: head dim must be 64, 128 or 256 (the same for q, k and v), got %lld/%lld/%lld", (long long)p.q.size[3],
+                     (long long)p.k.size[3], (long long)p.v.size[3]), MI355_SDPA_ERR_UNSUPPORTED;
   if (g.R < 1 || g.R > 16)
     return set_error("SDPA decode: Lq * Hq/Hkv must be in [1, 16], got %d", g.R), MI355_SDPA_ERR_UNSUPPORTED;
   if (p.q.stride[3] != 1 || p.k.stride[3] != 1 || p.v.stride[3] != 1 || p.out.stride[3] != 1)
@@ -614,7 +644,7 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
       (int64_t)(g.S - 1) * p.v.stride[2] + D >= (1ll << 31))
     return set_error("SDPA decode: cache too large for 32-bit step and row offsets"), MI355_SDPA_ERR_UNSUPPORTED;
   g.t_min = min_steps_for(p);
-  g.n_waves = (int)std::min<int64_t>(wave_slots(), std::max<int64_t>(1, (max_steps + g.t_min - 1) / g.t_min));
+  g.n_waves = (int)std::min<int64_t>(wave_slots(D), std::max<int64_t>(1, (max_steps + g.t_min - 1) / g.t_min));
   const int64_t qes = p.q_dtype == MI355_SDPA_F32 ? 4 : 2;
   if (((uintptr_t)p.q.data & 15) || (p.q.stride[0] * qes) % 16 || (p.q.stride[1] * qes) % 16 || (p.q.stride[2] * qes) % 16)
     return set_error("SDPA decode: query rows must be 16-byte aligned"), MI355_SDPA_ERR_UNSUPPORTED;
@@ -624,9 +654,9 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
   g.ws_ml = g.ws_o + slots * D;
   g.ws_steps = (int32_t*)(g.ws_ml + slots * 2);
   switch (p.q_dtype) {
-    case MI355_SDPA_BF16: return launch_t<bf16_t>(g, s);
-    case MI355_SDPA_F16: return launch_t<f16_t>(g, s);
-    case MI355_SDPA_F32: return launch_t<float>(g, s);
+    case MI355_SDPA_BF16: return launch_t<bf16_t>(g, D, s);
+    case MI355_SDPA_F16: return launch_t<f16_t>(g, D, s);
+    case MI355_SDPA_F32: return launch_t<float>(g, D, s);
   }
   return set_error("SDPA decode: query dtype must be float32, float16, or bfloat16"), MI355_SDPA_ERR_INVALID;
 }
