@@ -574,7 +574,6 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   // bias / keep-mask, but no bias gradient and no window
   const bool wide = E > 128 || Dv != E;
   const bool smod = score_mod_of(p.mask).any;
-  if (wide && p.grad_bias.data) return *why = "bias gradient with a head dim above 128 or D_qk != D_v", false;
   if (smod && (p.bias.data || p.grad_bias.data || p.dropout_p > 0.f))
     return *why = "score functor together with attn_bias or dropout", false;
   const bool padded = E != 64 && E != 128;  // served by the next wider kernels' masked variants

@@ -152,7 +152,8 @@ constexpr WideOp dkdv_op(int k) {  // S steps and dP steps (in turns where both 
 
 // MODE 1 (MASKED): per-batch key counts and an additive bias / bool keep-mask, per key or per score (a
 // lane is a query row in the dQ kernel and reads its own row of it, a key in the dK/dV kernel and reads
-// one element per score register); no bias gradient here.
+// one element per score register); the gradient of the bias, P (dP - delta) in the input dtype, leaves
+// the dQ kernel four keys at a time: the packed dS pairs it feeds to the matrix pipe are its elements.
 // MODE 2 (FUNC): per-batch key counts, a sliding window with sink keys (the tiles it drops whole are not
 // walked) and the score functors and document ids of score_mod.h, each score through score_mod_at where
 // its probability is formed; the derivative of the functors multiplies the gradient of the scores.
@@ -232,7 +233,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   // list in LDS); stream position u is then key tile tile_of(u).
   bool listed = false;
   if constexpr (MASKED) {
-    if (p.live_tiles && !p.causal) {
+    if (p.live_tiles && !p.causal && !p.gbias) {  // (with a bias gradient every tile is walked: its zeros are written there)
       if (wave == 0) {
         const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
         const uint32_t* map = p.live_tiles + ((int64_t)((p.bias_sb ? b : 0) * p.live_hm + (p.bias_sh ? h : 0)) * nrb + rb0) * p.live_words;
@@ -265,6 +266,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   };
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1 - skip) : nt;  // tiles with work for this wavefront
   const int lim = p.causal ? min(qrow, S - 1) : S - 1;
+  // (MASKED) this lane's row of the bias gradient, at its first key of a tile
+  uint16_t* const gb_row = (MASKED && p.gbias && qrow < p.L)
+                               ? (uint16_t*)p.gbias + b * p.gbias_sb + h * p.gbias_sh + (int64_t)qrow * p.gbias_sl + half * 4 : nullptr;
   // (FUNC) the window of this lane's row, and what the derivative of the functors needs
   const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
   const int n_sink = FUNC ? p.sink_keys : 0;
@@ -455,6 +459,13 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         }
         __builtin_amdgcn_sched_barrier(0);
       });
+      if constexpr (MASKED) {
+        if (gb_row) {
+#pragma unroll
+          for (int g = 0; g < 4; ++g)
+            if (ta * BT + g * 8 + half * 4 < p.S) *(u32x2*)(gb_row + ta * BT + g * 8) = u32x2{pS[2 * g], pS[2 * g + 1]};
+        }
+      }
     };
     if (t < nt_w) {
       if constexpr (FUNC) {
@@ -470,6 +481,14 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
 #pragma unroll
     for (int i = 0; i < DBE; ++i) asm volatile("" : "+a"(dqacc[i]));
     if (t + 1 < nt) publish_tile();
+  }
+  if constexpr (MASKED) {
+    if (gb_row) {  // the tiles this wavefront did not walk: above the diagonal, past the batch's keys
+      for (int t = min(nt_w, nt); t * BT < p.S; ++t)
+#pragma unroll
+        for (int g = 0; g < 4; ++g)
+          if (t * BT + g * 8 + half * 4 < p.S) *(u32x2*)(gb_row + t * BT + g * 8) = u32x2{0u, 0u};
+    }
   }
   if (qrow < p.L) {
     uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
@@ -922,7 +941,7 @@ int launch_t(const BwdM& g, hipStream_t s) {
 template <typename T>
 int launch_w(const BwdM& g, hipStream_t s) {
   const bool func = g.window > 0 || g.sm.any;  // (never together with a bias: refused before)
-  const bool masked = g.bias_kind || g.kv_lens;
+  const bool masked = g.bias_kind || g.kv_lens;  // (a bias gradient comes with a bias)
   if (g.d_real <= 192 && g.dv_real <= 128)
     return func ? launch_t<T, 192, 128, 2>(g, s) : masked ? launch_t<T, 192, 128, 1>(g, s) : launch_t<T, 192, 128, 0>(g, s);
   if (func) return launch_t<T, 256, 256, 2>(g, s);
