@@ -167,3 +167,35 @@ def test_score_functor_argument_errors(amd, gpu_device):
     with pytest.raises(RuntimeError, match="functor"):
         amd.sdpa_forward(q, k, v, softcap=2.0, attn_bias=torch.zeros(1, 1, 64, 64, device=dev, dtype=torch.bfloat16),
                          force_kernel=amd._lib.KERNEL_MFMA)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_prefix_length_mask_mod_is_a_key_count(amd, gpu_device, dtype):
+    # the reference's mask_mod with an external buffer (test_flex_attention_legalization.py:783-800):
+    # kv_idx <= prefix_length[b], a per-batch prefix of the keys - here the call's kv_lens = prefix_length + 1,
+    # which the matrix-op kernels take without a mask tensor (tiles past the prefix are never read)
+    dev = gpu_device
+    B, H, L, S, E = 2, 2, 8, 8, 16
+    q, k, v, go = seeded([(B, H, L, E), (B, H, S, E), (B, H, S, E), (B, H, L, E)], 5, dtype)
+    prefix_length = torch.tensor([4, 6], dtype=torch.int32)
+    keep = (torch.arange(S)[None] <= prefix_length[:, None])[:, None, None, :]
+    lens = (prefix_length + 1).to(dev)
+    MFMA = amd._lib.KERNEL_MFMA
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), kv_lens=lens, force_kernel=MFMA)
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, kv_lens=lens, force_kernel=MFMA)
+    ro, rl = om.sdpa_forward(q.float(), k.float(), v.float(), attn_mask=keep)
+    rg = om.sdpa_backward(go.float(), q.float(), k.float(), v.float(), ro, rl, attn_mask=keep, reduce_in_fp32=True)
+    half = dtype is not torch.float32
+    assert max_abs(out, ro) <= (2e-2 if half else 1e-5) and max_abs(lse, rl) <= (5e-3 if half else 1e-5)
+    for a, r in zip((dq, dk, dv), rg):
+        assert max_abs(a, r) <= (5e-2 if half else 1e-5)
+    # ... and the same mask as a tensor is recognised as that key count by the operator
+    fused = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    mask = keep.expand(B, 1, L, S).contiguous().to(dev)
+    amd.mask_patterns.clear_cache()
+    fused(q.to(dev), k.to(dev), v.to(dev), mask)
+    torch.cuda.synchronize()
+    pat = amd.mask_patterns.classify(mask)
+    assert pat[0] == "all" and pat[1].tolist() == [5, 7]
+    r = fused(q.to(dev), k.to(dev), v.to(dev), mask)
+    assert max_abs(r[0], ro) <= (2e-2 if half else 1e-5)
