@@ -361,6 +361,35 @@ def test_fresh_bool_masks_run_at_the_speed_of_the_causal_flag(amd, gpu_device):
 
 
 @pytest.mark.gpu
+def test_training_steps_with_a_mask_that_is_new_every_step(amd, gpu_device, monkeypatch):
+    # forward and backward through autograd with a bool mask: upstream makes a new additive tensor per
+    # step, the forward takes its verdict on the device, and the backward of the same step finds that
+    # verdict again instead of reading the mask a second time; after a few steps no copy to the host either
+    dev = gpu_device
+    B, H, L, D = 2, 8, 1024, 64
+    q, k, v, go = (t.to(dev) for t in qkv(B, H, H, L, L, D, dtype=torch.bfloat16, seed=9, with_do=True))
+    tril = torch.ones(L, L, dtype=torch.bool, device=dev).tril()
+    seen_b = []
+    b0 = amd.ops.sdpa_backward
+    monkeypatch.setattr(amd.ops, "sdpa_backward", lambda *a, **kw: (seen_b.append(kw), b0(*a, **kw))[1])
+    qc, kc, vc = (t.clone().requires_grad_(True) for t in (q, k, v))
+    F.scaled_dot_product_attention(qc, kc, vc, is_causal=True).backward(go)
+    amd.mask_patterns.clear_cache()
+    looked0, launched = amd.mask_patterns.stats["looked"], []
+    real = amd.mask_patterns._launch_verdict
+    monkeypatch.setattr(amd.mask_patterns, "_launch_verdict", lambda *a: (launched.append(1), real(*a))[1])
+    for step in range(6):
+        qm, km, vm = (t.clone().requires_grad_(True) for t in (q, k, v))
+        F.scaled_dot_product_attention(qm, km, vm, attn_mask=tril).backward(go)
+        kw = seen_b[-1]  # (the verdict on the device, or - its copy has arrived meanwhile - the pattern itself)
+        assert kw.get("mask_verdict") is not None or (kw["attn_bias"] is None and kw["is_causal"])
+        for a, b in ((qm.grad, qc.grad), (km.grad, kc.grad), (vm.grad, vc.grad)):
+            assert max_abs(a, b) <= 2e-2 and rel_err(a, b) <= 5e-3
+    assert len(launched) == 6  # one verdict per step: the backward reuses the forward's
+    assert amd.mask_patterns.stats["looked"] - looked0 == 3  # ... and a copy to the host for the first three only
+
+
+@pytest.mark.gpu
 def test_a_captured_call_takes_its_verdict_on_every_replay(amd, gpu_device):
     # inside a stream capture nothing is cached and nothing waits: the verdict is part of the graph, so a
     # replay follows the mask as it then is - causal at the causal kernel's speed, anything else as a mask

@@ -178,7 +178,7 @@ _MIN_SCORES_ON_DEVICE = 256 * 256
 
 
 class _Pending:
-    """A verdict whose copy to the host is under way."""
+    """A verdict on the device whose copy to the host is under way (or was not asked for)."""
 
     __slots__ = ("verdict", "host", "event", "B")
 
@@ -186,7 +186,7 @@ class _Pending:
         self.verdict, self.host, self.event, self.B = verdict, host, event, B
 
     def settled(self) -> bool:
-        return self.event.query()
+        return self.event is not None and self.event.query()
 
     def pattern(self):
         """``("all" | "causal" [, key counts]) | ("window", W, N) | None`` from the host copy."""
@@ -247,14 +247,17 @@ def look(mask: torch.Tensor, B: int, Hq: int, L: int, S: int):
     sig = (B, L, S, mask.dtype, mask.device.index)
     found, entry = _lookup(_cache, key)
     if found:
-        _misses.pop(sig, None)
         if isinstance(entry, _Pending):
             if not entry.settled():
+                # (the backward of the step that made the entry, typically: no sign that the tensor lives on)
                 stats["pending"] = stats.get("pending", 0) + 1
                 return None, (entry.verdict if on_device else None)
+            # (still possibly the backward of the step that made the entry: the miss streak stands)
             pat = entry.pattern()
             _remember(_cache, key, ("known", pat), mask)
             entry = ("known", pat)
+        else:
+            _misses.pop(sig, None)  # (found again after its pattern was known: the caller keeps its masks)
         stats["hits"] += 1
         return entry[1], None
     # A caller that hands in a NEW tensor on every call never finds its entry again: after a few such
@@ -262,7 +265,12 @@ def look(mask: torch.Tensor, B: int, Hq: int, L: int, S: int):
     # that signature; the verdict on the device still is, where the mask is large enough to matter.
     if _back_off(sig):
         stats["left_alone"] += 1
-        return None, (_launch_verdict(view, dtype_id, words) if on_device else None)
+        if not on_device:
+            return None, None
+        # (remembered without a copy to the host: the backward of the same step finds it here)
+        verdict = _launch_verdict(view, dtype_id, words)
+        _remember(_cache, key, _Pending(verdict, None, None, B), mask)
+        return None, verdict
     stats["looked"] += 1
     verdict = _launch_verdict(view, dtype_id, words)
     host = torch.empty((8 + B,), dtype=torch.int32, pin_memory=True)
