@@ -174,9 +174,9 @@ def test_kernel_gates(amd):
     q64, k64 = _meta(1, 8, 512, 64), _meta(1, 8, 512, 64)
     assert gate(q64, k64, k64, attn_bias=_meta(512, 512)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q, k, v, dropout_p=0.1) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # dropout: 16-bit, head dims up to 128, no bias
-    assert gate(q, k, v, dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q, k, v, dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # ... with a bias too
     assert gate(q.float(), k.float(), v.float(), dropout_p=0.1) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
-    assert gate(q.float(), k.float(), v.float(), dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q.float(), k.float(), v.float(), dropout_p=0.1, attn_bias=_meta(8192, 8192)) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     assert gate(q, k, v, scale=0.0) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     assert gate(q, k, v, scale=0.25) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q96 = _meta(2, 8, 512, 96)  # narrow head dims (multiples of 8) run padded in the next wider kernel
@@ -274,6 +274,12 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
         scratch = int(r["ScratchSize_[bytes/lane]"])
         if "decode_kernelIfLi256ELi1ELi3EE" in name:  # float32 queries at head dim 256, 9-16 rows: a dozen bytes, no counted waits there
             assert scratch <= 16, (name, scratch)
+            continue
+        if re.search(r"bwd_dkdv_w32_kernelIDF16[b_]Li128ELi5E", name):
+            # dropout together with a bias at head dim 128: 32 bias elements and 32 keep bytes of a tile in
+            # flight at once; the counted waits of that file stay valid under extra scratch traffic (a
+            # wait that allows N loads in flight covers everything older, whatever the N youngest are)
+            assert scratch <= 112, (name, scratch)
             continue
         m = known.search(name)
         if m:

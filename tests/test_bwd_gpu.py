@@ -210,6 +210,62 @@ def test_dropout_in_the_matrix_op_kernels(amd, gpu_device, case, dtype):
         assert max_abs(a, r) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
 
 
+DROPOUT_BIAS = [
+    # B, Hq, Hkv, L, S, E, causal, bias dtype, bias shape (broadcast dims as 1), dropout_p, grad_bias
+    (2, 4, 2, 128, 128, 64, False, torch.float32, (2, 4, 128, 128), 0.25, False),
+    (2, 4, 4, 300, 260, 128, True, torch.bfloat16, (1, 1, 300, 260), 0.1, False),
+    (1, 6, 2, 129, 516, 64, False, torch.bool, (1, 6, 129, 516), 0.5, False),
+    (2, 4, 4, 96, 200, 128, False, torch.bool, (2, 1, 1, 200), 0.3, False),     # a padding mask per key
+    (2, 8, 2, 130, 256, 128, True, torch.float16, (2, 8, 1, 256), 0.1, False),  # a bias per key, causal
+    (1, 2, 2, 200, 136, 64, False, torch.float32, (1, 2, 200, 136), 0.25, True),
+    (2, 2, 2, 256, 256, 128, True, None, (2, 2, 256, 256), 0.1, True),           # (the bias in the calls' dtype)
+    (1, 3, 1, 40, 72, 40, False, torch.float32, (1, 3, 40, 72), 0.3, False),    # head dim padded to 64
+]
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+@pytest.mark.parametrize("case", DROPOUT_BIAS, ids=lambda c: "B%d_Hq%d_Hkv%d_L%d_S%d_E%d_c%d_%s_p%s_g%d" % (c[:7] + (str(c[7]).replace("torch.", ""), c[9], c[10])))
+def test_dropout_together_with_a_bias_in_the_matrix_op_kernels(amd, gpu_device, case, dtype):
+    """A keep-mask and an attn_bias of every dtype and broadcast in one call (forced: the call fails if
+    the MFMA kernels cannot take it): the bias shapes the scores, the keep-mask the probabilities
+    behind the softmax, as in torch_neuronx/_sdpa_math.py:15-48, :154-169; grad_bias = grad_logits."""
+    B, Hq, Hkv, L, S, E, causal, bdt, bshape, pdrop, want_gb = case
+    dev = gpu_device
+    bdt = dtype if bdt is None else bdt
+    g = torch.Generator().manual_seed(L * 5 + S + E)
+    q, k, v, go = (torch.randn(s_, generator=g).to(dtype) for s_ in ((B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, E), (B, Hq, L, E)))
+    go = (go.float() * 0.1).to(dtype)
+    keep = torch.rand(B, Hq, L, S, generator=g) >= pdrop
+    if bdt == torch.bool:
+        bias = torch.rand(bshape, generator=g) > 0.3
+        bias[..., 0] = True  # (no row without a key)
+        bf = torch.where(bias, 0.0, float("-inf"))
+    else:
+        bias = torch.randn(bshape, generator=g).to(bdt)
+        bf = bias.float()
+    bf = bf.expand(B, Hq, L, S)
+    if causal:
+        bf = bf + torch.where(torch.ones(L, S, dtype=torch.bool).tril(), 0.0, float("-inf"))
+    rep = Hq // Hkv
+    kf, vf = k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1)
+    ro, rl = om.compute_attention(q.float(), kf, vf, bf, keep, E**-0.5, False, pdrop)
+    rdq, rdk, rdv, rdb = om.compute_attention_backward(go.float(), q.float(), kf, vf, bf, keep, ro, rl, E**-0.5, False, pdrop)
+    rdk, rdv = rdk.view(B, Hkv, rep, S, E).sum(2), rdv.view(B, Hkv, rep, S, E).sum(2)
+    MFMA = amd._lib.KERNEL_MFMA
+    kw = dict(attn_bias=bias.to(dev), is_causal=causal, dropout_p=pdrop, dropout_keep=keep.to(dev), force_kernel=MFMA)
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), **kw)
+    dq, dk, dv, db = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, want_grad_bias=want_gb, **kw)
+    tol = 2e-2 if dtype == torch.bfloat16 else 4e-3
+    assert max_abs(out, ro) <= tol
+    live = torch.isfinite(rl)
+    assert max_abs(lse.cpu()[live], rl[live]) <= 2e-3 and torch.equal(torch.isfinite(lse.cpu()), live)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+    if want_gb:
+        # (delta comes from the rounded output: a row with one live key has dS = O(ulp of out) instead of 0)
+        assert db.shape == (B, Hq, L, S) and max_abs(db, rdb) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
 def test_dropout_with_a_padding_mask_through_the_operator(amd, gpu_device):
     """What a BERT layer in training sends: an additive (B,1,1,S) padding mask and dropout_p = 0.1.  The
     mask becomes key counts, the keep-mask goes into the MFMA kernels, and forward / backward agree
@@ -239,6 +295,33 @@ def test_dropout_with_a_padding_mask_through_the_operator(amd, gpu_device):
         assert max_abs(a, b_) <= 1e-2
     frac = keep.float().mean().item()
     assert 0.88 < frac < 0.92
+
+
+def test_dropout_with_a_relative_position_bias_through_the_operator(amd, gpu_device, monkeypatch):
+    """An additive (1,H,S,S) bias that is no pattern, with dropout_p = 0.1, through the registered
+    operators: forward and backward run in the MFMA kernels (forced here: the calls would fail
+    otherwise) and agree with the oracle given the mask that the forward drew."""
+    from torch_neuronx_amd.python_ops import scaled_dot_product_fused_attention as impl
+    monkeypatch.setattr(impl, "_force_kernel", lambda: amd._lib.KERNEL_MFMA)
+    B, H, S, E = 2, 4, 256, 64
+    dev = gpu_device
+    g = torch.Generator().manual_seed(5)
+    q, k, v, go = (torch.randn(B, H, S, E, generator=g).to(torch.bfloat16).to(dev) for _ in range(4))
+    go = (go.float() * 0.1).to(torch.bfloat16)
+    bias = torch.randn(1, H, S, S, generator=g).to(torch.bfloat16).to(dev)
+    torch.manual_seed(13)
+    op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    opb = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    r = op(q, k, v, bias, 0.1)
+    keep = r[6]
+    dq, dk, dv, _ = opb(go, q, k, v, bias, [True, True, True, False], r[0], r[1], None, None, S, S, 0.1, False, keep, r[7])
+    bf = bias.float().cpu().expand(B, H, S, S)
+    qc, kc, vc, gc = (t.float().cpu() for t in (q, k, v, go))
+    ro, rl = om.compute_attention(qc, kc, vc, bf, keep.cpu().bool(), E**-0.5, False, 0.1)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(gc, qc, kc, vc, bf, keep.cpu().bool(), ro, rl, E**-0.5, False, 0.1)
+    assert max_abs(r[0], ro) <= 2e-2 and max_abs(r[1], rl) <= 2e-3
+    for a, b_ in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, b_) <= 1e-2
 
 
 def test_backward_kv_lens(amd, gpu_device):

@@ -583,6 +583,9 @@ F32_MASKED = [
     (2, 4, 2, 64, 64, 64, True, "dropout", None),
     (2, 6, 6, 200, 130, 128, False, "dropout", [130, 77]),
     (1, 2, 2, 128, 128, 32, False, "dropout_all", None),
+    (2, 4, 2, 100, 160, 64, False, "f32_full+dropout", None),
+    (1, 8, 2, 300, 300, 128, True, "bool_full+dropout", None),
+    (3, 2, 2, 33, 70, 40, False, "f16_key+dropout", [70, 5, 33]),
 ]
 
 
@@ -597,6 +600,10 @@ def test_float32_matrix_op_with_a_bias_or_dropout(amd, gpu_device, case):
     g = torch.Generator().manual_seed(L * 3 + S)
     q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=torch.float32, seed=L + S + E, with_do=True)
     kw, bias, keep, pdrop = {}, None, None, 0.0
+    kind, _, both = kind.partition("+")
+    if both:
+        pdrop = 0.3
+        keep = torch.rand(B, Hq, L, S, generator=g) >= pdrop
     if kind == "f32_full":
         bias = torch.randn(B, Hq, L, S, generator=g)
     elif kind == "bf16_b1":
@@ -643,12 +650,11 @@ def test_float32_matrix_op_with_a_bias_or_dropout(amd, gpu_device, case):
 
 def test_float32_matrix_op_refuses_what_it_does_not_serve(amd, gpu_device):
     q, k, v = (t.to(gpu_device) for t in qkv(1, 2, 2, 64, 64, 64, dtype=torch.float32, seed=1))
-    bias = torch.zeros(64, 64, device=gpu_device)
     keep = torch.ones(1, 2, 64, 64, dtype=torch.uint8, device=gpu_device)
-    with pytest.raises(NotImplementedError, match="float32 MFMA"):  # dropout together with a bias
-        amd.sdpa_forward(q, k, v, attn_bias=bias, dropout_p=0.5, dropout_keep=keep, force_kernel=MFMA)
-    out, _ = amd.sdpa_forward(q, k, v, attn_bias=bias, dropout_p=0.5, dropout_keep=keep)  # served by the generic kernel
-    ro, _ = oracle_fwd(q.cpu(), k.cpu(), v.cpu())
+    with pytest.raises(NotImplementedError, match="float32 MFMA"):  # dropout together with a functor
+        amd.sdpa_forward(q, k, v, window=16, is_causal=True, dropout_p=0.5, dropout_keep=keep, force_kernel=MFMA)
+    out, _ = amd.sdpa_forward(q, k, v, window=64, is_causal=True, dropout_p=0.5, dropout_keep=keep)  # served by the generic kernel
+    ro, _ = oracle_fwd(q.cpu(), k.cpu(), v.cpu(), is_causal=True)
     assert max_abs(out, 2.0 * ro) <= 2e-5
 
 

@@ -112,11 +112,14 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
   // key see none of its keys, unless the block holds sink keys
   constexpr bool FUNC = MASK == 1 || MASK == 4;
   constexpr bool SMOD = MASK == 4;  // score functors, document ids
-  // MASK = 3 is dropout: the (B, Hq, L, S) keep-mask is fetched like a bool bias by the wavefronts that
-  // form the probabilities.  They feed dV with the kept probabilities and hand all of them to the dK
+  // MASK = 3 is dropout, MASK = 5 dropout with a bias (an instance of its own: the bias and the keep
+  // bytes of a tile together are more than the registers hold at head dim 128, and a call without a
+  // bias need not pay for that): the (B, Hq, L, S) keep-mask is fetched like a bool bias, beside the
+  // bias, by the wavefronts that form the probabilities.  They feed dV with the kept probabilities and hand all of them to the dK
   // wavefronts, the dropped ones with the sign bit set (a probability is never negative): dP is
   // multiplied by keep / (1 - p) there (torch_neuronx/_sdpa_math.py:36-48, :154-158).
-  constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;
+  constexpr bool HASB = MASK == 2 || MASK == 5, DROP = MASK == 3 || MASK == 5;  // a bias per score; a keep-mask
+  constexpr bool BIASED = HASB || DROP;
   const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
   // the query rows that see this lane's key are first_q .. past_q - 1: from the key itself on under a
   // causal mask, none for a key past the batch's count, up to the end of the key's window unless it is a sink
@@ -320,11 +323,11 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
     }
   };
 
-  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;
+  const int bkind = HASB ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;
   const int besz = __builtin_amdgcn_readfirstlane(bkind == 1 ? 4 : bkind == 4 ? 1 : 2);  // (in a scalar register: a descriptor built from a vector register is looked up lane by lane)
-  const uint32_t b_rowbytes = BIASED ? (uint32_t)(p.bias_sl * besz) : 0u;
-  const uint32_t b_lane = BIASED ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
-  const int b_records = BIASED ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
+  const uint32_t b_rowbytes = HASB ? (uint32_t)(p.bias_sl * besz) : 0u;
+  const uint32_t b_lane = HASB ? (uint32_t)((half * 4 * p.bias_sl + key) * besz) : 0u;
+  const int b_records = HASB ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
   // the fetched bias elements of a tile, turned into floats in the log2 domain in place (the
   // element type is tested once, outside the loops: inside, every element would carry the branch)
   auto bias_to_log2 = [&](uint32_t (&w)[2][16]) {
@@ -346,10 +349,23 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
   // the last row of the (batch, head): rows past L read as zeros (they are switched off through
   // lse = +inf), keys past S as a neighbouring element (their probabilities are replaced by zero).
   uint32_t braw[2][16];
+  uint32_t kraw[DROP ? 2 : 1][16];  // (dropout) the keep bytes of the same scores
   auto load_bias_a = [&](int it) {
     if constexpr (BIASED) {
       const int q0 = item_q0(it);
       if (it >= n_items || (ma.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
+      if constexpr (DROP) {
+        const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+            uniform_ptr((const char*)p.keep + ((int64_t)b * p.Hq + item_head(it)) * p.L * p.S), 0,
+            __builtin_amdgcn_readfirstlane((int)((int64_t)p.L * p.S)), 0x00020000);
+        const uint32_t kbase = (uint32_t)((q0 + half * 4) * p.S + key);
+#pragma unroll
+        for (int mq = 0; mq < 2; ++mq)
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            kraw[mq][r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(k_rsrc, kbase + (uint32_t)((mq * 32 + (r >> 2) * 8 + (r & 3)) * p.S), 0, 0);
+      }
+      if constexpr (!HASB) return;
       const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(
           uniform_ptr((const char*)p.bias + (b * p.bias_sb + item_head(it) * p.bias_sh) * besz), 0, b_records, 0x00020000);
       const uint32_t base = b_lane + (uint32_t)q0 * b_rowbytes;
@@ -411,7 +427,7 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
     auto prob = [&](int mq, int r) {
       const float l = l4[mq][r >> 2][r & 3];
       float x;
-      if constexpr (MASK == 2) x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, __builtin_bit_cast(float, braw[mq][r])) - l);
+      if constexpr (HASB) x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, __builtin_bit_cast(float, braw[mq][r])) - l);
       else if constexpr (MASK == 1) x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, bl) - l);
       else x = __builtin_amdgcn_exp2f(fmaf(sc[mq][r], c, -l));
       return x;
@@ -423,7 +439,7 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
         const int r = slot * EPS + k;
         const float p0 = prob(mq, r), p1 = prob(mq, r + 1);
         if constexpr (DROP) {
-          const float s0 = braw[mq][r] ? p0 : -p0, s1 = braw[mq][r + 1] ? p1 : -p1;
+          const float s0 = kraw[mq][r] ? p0 : -p0, s1 = kraw[mq][r + 1] ? p1 : -p1;
           pkx[mq][r >> 1] = Mma<T>::pack(s0, s1);
           pk[mq][r >> 1] = Mma<T>::pack(fmaxf(s0, 0.f), fmaxf(s1, 0.f));
         } else {
@@ -501,7 +517,7 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
       if (i == KS - 1) load_l4(0, 0);
       __builtin_amdgcn_sched_barrier(0);
     }
-    if constexpr (MASK == 2) bias_to_log2(braw);
+    if constexpr (HASB) bias_to_log2(braw);
     smod_scores(0);
     if (__builtin_expect(edge, 0)) mask_scores(0);
     __builtin_amdgcn_sched_barrier(0);
@@ -847,7 +863,13 @@ int launch_m(const BwdM& g, hipStream_t s) {
     }
     return launch_t<T, D, 4>(g, s);
   }
-  if (g.keep_scale != 0.f) return launch_t<T, D, 3>(g, s);
+  if (g.keep_scale != 0.f) {
+    if (!g.keep || g.live_t) {
+      set_error("SDPA: dropout in bwd_dkdv_w32_kernel needs a keep-mask and no tile table");
+      return MI355_SDPA_ERR_UNSUPPORTED;
+    }
+    return g.bias_kind ? launch_t<T, D, 5>(g, s) : launch_t<T, D, 3>(g, s);
+  }
   if (g.bias_kind && g.bias_sl != 0) {
     if (g.verdict) {  // (see bwd_dkdv_w32_kernel)
       if (int rc = launch_t<T, D, 1, true>(g, s)) return rc;

@@ -42,8 +42,9 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   constexpr int NBUF = 4;  // tile t lives in buffer t % 4
   // (the variant with a bias takes the launch's dynamic LDS: behind the tiles it keeps the list of the
   // key tiles it walks when the call brings a skip table, and a kernel may declare 64 KB at most)
-  // MASK = 3 is dropout: the (B, Hq, L, S) keep-mask is fetched like a bool bias, leaves the scores alone and
-  // multiplies dP, together with 1 / (1 - p) (torch_neuronx/_sdpa_math.py:36-48, :154-158)
+  // MASK = 3 is dropout, with a bias or without: the (B, Hq, L, S) keep-mask is fetched like a bool bias into
+  // LDS of its own, leaves the scores alone and multiplies dP, together with 1 / (1 - p)
+  // (torch_neuronx/_sdpa_math.py:36-48, :154-158)
   constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;
   constexpr bool DYN = BIASED;
   __shared__ __attribute__((aligned(16))) uint16_t k_static[DYN ? 8 : NBUF * TILE];
@@ -116,12 +117,12 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   }
 
   uint16_t* gb_row = nullptr;  // this lane's row of the bias gradient, at its first key of a tile
-  if constexpr (MASK == 2) {
+  if constexpr (BIASED) {
     if (p.gbias && qrow < p.L)
       gb_row = (uint16_t*)p.gbias + b * p.gbias_sb + h * p.gbias_sh + (int64_t)qrow * p.gbias_sl + half * 4;
   }
   auto zero_gbias = [&](int t_from) {  // tiles this wavefront does not visit
-    if constexpr (MASK == 2) {
+    if constexpr (BIASED) {
       if (gb_row) {
         for (int t = t_from; t * BN < p.S; ++t)
 #pragma unroll
@@ -444,7 +445,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   // The resource starts at this wavefront's first row of the (batch, head) plane and ends with its
   // last one: keys past S read the next row or, past the last row, zeros (they are masked anyway).
   uint32_t braw[16];
-  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;
+  const int bkind = BIASED ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;
   const int besz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const int b_rows = min(32, p.L - qw0);
   const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * besz : 0),
@@ -453,11 +454,21 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   const int b_loads = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const unsigned char* const bias_w = (const unsigned char*)(tile_list + 1040) + (BIASED ? wave * 4096 : 0);
   const uint32_t lds_b = (uint32_t)(uintptr_t)(lds_bytes)bias_w;
+  // the keep bytes of a dropout call: one load, lane (row, half) -> keys 16 half .. +15, 1 KB per wavefront behind the bias tiles
+  const u32x4 kp_rsrc = descriptor((const char*)p.keep + (DROP ? (((int64_t)b * p.Hq + h) * p.L + qw0) * p.S : 0),
+                                   (DROP && b_rows > 0) ? (int64_t)b_rows * p.S : 0);
+  const uint32_t kp_voff = DROP ? (uint32_t)(min(col, max(b_rows - 1, 0)) * p.S + half * 16) : 0u;
+  const unsigned char* const keep_w = (const unsigned char*)(tile_list + 1040) + (DROP ? 8 * 4096 + wave * 1024 : 0);
+  const uint32_t lds_kp = (uint32_t)(uintptr_t)(lds_bytes)keep_w;
+  uint32_t kraw[4];
   auto load_bias = [&](int t) {
     if constexpr (BIASED) {
-      if (bkind) {
+      if (bkind || DROP) {
         // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      if constexpr (DROP) tile_load(kp_rsrc, kp_voff + (uint32_t)(t * BN), lds_kp);
+      if (bkind) {
         const uint32_t g0 = b_voff + (uint32_t)((listed ? tile_of(min(t, max(nt - 1, 0))) : t) * BN * besz);
         tile_load(b_rsrc, g0, lds_b);
         if (b_loads > 1) tile_load(b_rsrc, g0 + 32, lds_b + 1024);
@@ -474,6 +485,10 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
     if constexpr (BIASED) {
       if constexpr (NDMA == 2) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
       else asm volatile("s_waitcnt vmcnt(1)" ::: "memory");
+      if constexpr (DROP) {
+#pragma unroll
+        for (int g = 0; g < 4; ++g) kraw[g] = *(const uint32_t*)(keep_w + (col + 32 * (g >> 1)) * 16 + (g & 1) * 8 + half * 4);
+      }
       if (bkind == 1) {
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
@@ -512,7 +527,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
     const int t = tile_of(u);  // (stream position -> key tile)
     const bool edge = SMOD ? edge_tile(u) : t >= t_edge;
     float bl[16];
-    if constexpr (MASK == 2) bias_log2(bl);
+    if constexpr (BIASED) bias_log2(bl);
     // (the test for a tile that needs masking stays outside the unrolled loop: inside, the compiler
     // turns it into selects that every element of every tile pays for)
     auto elements = [&](auto edge_c) {
@@ -523,7 +538,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
 #pragma unroll
         for (int e = 0; e < 2; ++e) {
           float pr;
-          if constexpr (MASK == 2) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
+          if constexpr (BIASED) pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, bl[r + e]) - lse2);
           else pr = __builtin_amdgcn_exp2f(fmaf(sacc[r + e], c, -lse2));
           if constexpr (EDGE) {
             const int kv = t * BN + ((r + e) >> 2) * 8 + half * 4 + ((r + e) & 3);
@@ -532,7 +547,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
             pr = dead ? 0.f : pr;
           }
           if constexpr (DROP) {
-            const float keep = (float)((braw[(r + e) >> 2] >> (8 * ((r + e) & 3))) & 0xffu);
+            const float keep = (float)((kraw[(r + e) >> 2] >> (8 * ((r + e) & 3))) & 0xffu);
             ds[e] = pr * fmaf(dpacc[r + e] * keep, p.keep_scale, -dl);
           } else {
             ds[e] = pr * (dpacc[r + e] - dl);
@@ -543,7 +558,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
     };
     if (__builtin_expect(edge, 0)) elements(std::true_type{});
     else elements(std::false_type{});
-    if constexpr (MASK == 2) {
+    if constexpr (BIASED) {
       // grad_bias = grad_logits (torch_neuronx/_sdpa_math.py:163,169): the packed pairs are its
       // elements in the input dtype already; four consecutive keys per store
       if (gb_row) {
@@ -722,9 +737,13 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
     set_error("SDPA: score functors in bwd_dq_w32_kernel need a call without bias and dropout");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
+  if (g.keep_scale != 0.f && (!g.keep || g.live_tiles)) {
+    set_error("SDPA: dropout in bwd_dq_w32_kernel needs a keep-mask and no tile table");
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
   const int mask = g.sm.any ? 4 : g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
   // (the tiles, the tile list of a call with a skip table, 4 KB of bias tile per wavefront)
-  const int dyn = (mask == 2 || mask == 3) ? 2 * 4 * BN * head_dim * 2 + 2080 + 8 * 4096 : 0;
+  const int dyn = (mask == 2 || mask == 3) ? 2 * 4 * BN * head_dim * 2 + 2080 + 8 * 4096 + (mask == 3 ? 8 * 1024 : 0) : 0;
   if (mask == 2 || mask == 3) {
     const void* fn2 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 2>)
                                       : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 2> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 2>);

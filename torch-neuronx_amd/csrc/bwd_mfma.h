@@ -24,9 +24,10 @@ struct BwdM {
   const void* bias = nullptr;
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  // dropout (head dims up to 128, no bias): nonzero = 1 / (1 - p) (1 for p = 1), and the bias fields
-  // above describe the (B, Hq, L, S) keep-mask, kind 4
+  // dropout (head dims up to 128; with or without a bias): nonzero = 1 / (1 - p) (1 for p = 1), and the
+  // (B, Hq, L, S) contiguous keep bytes
   float keep_scale = 0.f;
+  const void* keep = nullptr;
   const int32_t* kv_lens = nullptr;
   // gradient of the bias (the dQ kernel writes it): P (dP - delta) in the input dtype, one element
   // per score, unit stride over keys, rows a whole number of 8-byte words (zeros where a score

@@ -478,7 +478,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   constexpr int RPB = 256 / (D / 8);
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.kv_lens || g.gbias || g.d_real != D || g.window > 0 || g.sm.any) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
+  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.keep_scale != 0.f || g.kv_lens || g.gbias || g.d_real != D || g.window > 0 || g.sm.any) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
   int rc;
   if (dq_w32) {
     // that kernel holds every row of dO in registers anyway: it goes first and leaves the row
@@ -543,11 +543,11 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
     g.bias_sl = p.q.size[2] > 1 ? p.bias.stride[2] : 0;
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
     const int words_t = ((g.L + 63) / 64 + 31) / 32;
-    if (p.mask.live_tiles_t && !p.is_causal && g.bias_sl != 0 && g.S <= 32768 && (g.Hq / g.Hkv) * words_t <= 256) {
+    if (p.mask.live_tiles_t && !p.is_causal && g.bias_sl != 0 && g.S <= 32768 && (g.Hq / g.Hkv) * words_t <= 256 && p.dropout_p == 0.f) {
       g.live_t = p.mask.live_tiles_t;
       g.live_t_words = words_t, g.live_hm = live_extent(p.bias, 1);
     }
-    if (p.mask.live_tiles && !p.is_causal && g.bias_sl != 0 && g.S <= 32768 && !p.grad_bias.data) {
+    if (p.mask.live_tiles && !p.is_causal && g.bias_sl != 0 && g.S <= 32768 && !p.grad_bias.data && p.dropout_p == 0.f) {
       g.live_tiles = p.mask.live_tiles;
       g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
     }
@@ -556,10 +556,8 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
   if (p.mask.mask_verdict && g.bias_kind && g.bias_sl != 0 && !p.is_causal && !p.kv_lens && p.dropout_p == 0.f && !g.live_t &&
       !g.live_tiles && !g.gbias && g.window == 0 && !g.sm.any && p.q.size[3] <= 128 && p.v.size[3] == p.q.size[3])
     g.verdict = p.mask.mask_verdict;
-  if (p.dropout_p > 0.f && !p.bias.data) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
-    g.bias = p.dropout_keep;
-    g.bias_sl = g.S, g.bias_sh = (int64_t)g.L * g.S, g.bias_sb = (int64_t)g.Hq * g.bias_sh;
-    g.bias_kind = 4;
+  if (p.dropout_p > 0.f) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
+    g.keep = p.dropout_keep;
     g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
 }
@@ -606,9 +604,9 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
       return *why = "attn_bias rows beyond 32-bit offsets", false;
   }
   if (p.dropout_p > 0.f) {
-    // the keep-mask takes the bias's way into the kernels (one dword = four keys of a row)
+    // the keep-mask takes a bool bias's way into the kernels (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
-    if (p.bias.data || p.grad_bias.data || p.mask.window > 0) return *why = "dropout together with attn_bias or a window functor", false;
+    if (p.mask.window > 0) return *why = "dropout together with a window functor", false;
     if (wide) return *why = "dropout with a head dim above 128 or D_qk != D_v", false;
     if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
     if ((p.q.size[2] + 64) * S + S + 64 >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;

@@ -94,9 +94,9 @@ __device__ __forceinline__ void col_product(f32x16 (&acc)[D / 32], const float* 
 }
 
 // MASKED instances: an additive bias / bool keep-mask per score (any of the bias dtypes, stride 0 on
-// broadcast dimensions) or a dropout keep-mask (bytes, (B, Hq, L, S); the bias fields describe it and
-// keep_scale is nonzero), one element load per score: a lane's 16 scores of a tile are 4 groups of 4
-// consecutive keys of its row (forward, dQ) or 16 rows of its key (dK / dV).  Not both at once.
+// broadcast dimensions) and / or a dropout keep-mask (bytes, (B, Hq, L, S) contiguous, with a nonzero
+// keep_scale), one element load per score: a lane's 16 scores of a tile are 4 groups of 4
+// consecutive keys of its row (forward, dQ) or 16 rows of its key (dK / dV).
 // bias elements as floats, the element type tested once (inside the loop every element carries the branch)
 template <typename IDX>
 __device__ __forceinline__ void load_bias16(float (&bl)[16], const void* base, int kind, IDX&& idx) {
@@ -184,9 +184,11 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
       const int64_t row0 = b * p.bias_sb + h * p.bias_sh + (int64_t)qc * p.bias_sl;
       auto idx = [&](int r) { return row0 + min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
       if (p.keep_scale != 0.f) {
+        const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.S;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) keepf[r] = (float)((const uint8_t*)p.bias)[idx(r)];
-      } else {
+        for (int r = 0; r < 16; ++r) keepf[r] = (float)krow[min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1)];
+      }
+      if (p.bias_kind) {
         float bl[16];
         load_bias16(bl, p.bias, p.bias_kind, idx);
         // folded into the raw scores, s += bias / scale: everything downstream is the unbiased code
@@ -351,29 +353,35 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
         if (p.window > 0 && qrow - kv >= p.window && kv >= p.sink_keys) s[r] = -INFINITY;
       }
     }
-    float bl[MASKED ? 16 : 1];  // the bias in the log2 domain, or (dropout) keep / (1 - p)
+    float bl[MASKED ? 16 : 1];  // the bias in the log2 domain
+    float kf[MASKED ? 16 : 1];  // (dropout) keep / (1 - p)
     bool drop = false;
     if constexpr (MASKED) {
       const int64_t row0 = b * p.bias_sb + h * p.bias_sh + (int64_t)qc * p.bias_sl;
       auto idx = [&](int r) { return row0 + min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
       drop = p.keep_scale != 0.f;
       if (drop) {
+        const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.S;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) bl[r] = (float)((const uint8_t*)p.bias)[idx(r)] * p.keep_scale;
-      } else {
+        for (int r = 0; r < 16; ++r) kf[r] = (float)krow[min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1)] * p.keep_scale;
+      }
+      if (p.bias_kind) {
         load_bias16(bl, p.bias, p.bias_kind, idx);
 #pragma unroll
         for (int r = 0; r < 16; ++r) bl[r] *= kLog2eF;
+      } else {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) bl[r] = 0.f;
       }
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
       const int kv = t * BT + (r >> 2) * 8 + half * 4 + (r & 3);
       float x = fmaf(s[r], c, -lse2);
-      if constexpr (MASKED) x = drop ? x : fmaf(s[r], c, bl[r]) - lse2;
+      if constexpr (MASKED) x = fmaf(s[r], c, bl[r]) - lse2;
       const float pr = __builtin_amdgcn_exp2f(kv > lim ? -INFINITY : x);
       float g = dp[r];
-      if constexpr (MASKED) g = drop ? g * bl[r] : g;
+      if constexpr (MASKED) g = drop ? g * kf[r] : g;
       ds[r] = pr * (g - dl);
       if constexpr (MASKED) {
         if (gb_row && kv < p.S) gb_row[kv] = ds[r];
@@ -475,7 +483,8 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
           if (p.window > 0 && qi - key >= p.window && key >= p.sink_keys) s[r] = -INFINITY;
         }
       }
-      float bl[MASKED ? 16 : 1];  // the bias in the log2 domain, or (dropout) keep / (1 - p)
+      float bl[MASKED ? 16 : 1];  // the bias in the log2 domain
+      float kf[MASKED ? 16 : 1];  // (dropout) keep / (1 - p)
       bool drop = false;
       if constexpr (MASKED) {
         const int hq = hk * rep + it % rep;
@@ -483,12 +492,17 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
         auto idx = [&](int r) { return col0 + (int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.bias_sl; };
         drop = p.keep_scale != 0.f;
         if (drop) {
+          const uint8_t* kcol = (const uint8_t*)p.keep + ((int64_t)b * p.Hq + hq) * p.L * p.S + min(key, p.S - 1);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) bl[r] = (float)((const uint8_t*)p.bias)[idx(r)] * p.keep_scale;
-        } else {
+          for (int r = 0; r < 16; ++r) kf[r] = (float)kcol[(int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.S] * p.keep_scale;
+        }
+        if (p.bias_kind) {
           load_bias16(bl, p.bias, p.bias_kind, idx);
 #pragma unroll
           for (int r = 0; r < 16; ++r) bl[r] *= kLog2eF;
+        } else {
+#pragma unroll
+          for (int r = 0; r < 16; ++r) bl[r] = 0.f;
         }
       }
 #pragma unroll
@@ -499,12 +513,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
         for (int e = 0; e < 4; ++e) {
           const int r = r4 * 4 + e, qi = q0 + r4 * 8 + half * 4 + e;
           float a = fmaf(s[r], c, -l4[e]);
-          if constexpr (MASKED) a = drop ? a : fmaf(s[r], c, bl[r]) - l4[e];
+          if constexpr (MASKED) a = fmaf(s[r], c, bl[r]) - l4[e];
           const float x = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : a);
           float g = dp[r];
           pr[r] = x;
           if constexpr (MASKED) {
-            if (drop) g *= bl[r], pr[r] = x * bl[r];  // dV from the kept probabilities, scaled; dP masked and scaled
+            if (drop) g *= kf[r], pr[r] = x * kf[r];  // dV from the kept probabilities, scaled; dP masked and scaled
           }
           ds[r] = x * (g - d4[e]);
           if constexpr (FUNC) ds[r] *= dfac[r];
@@ -534,7 +548,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
 // wavefronts (32 rows each) per workgroup
 int pick_waves(int64_t, int) { return 4; }
 
-// the bias / keep-mask fields of a call: an attn_bias as it is (strides in elements), or the dropout
+// the bias / keep-mask fields of a call: an attn_bias as it is (strides in elements), and the dropout
 // keep-mask, (B, Hq, L, S) contiguous bytes with keep_scale = 1 / (1 - p) (1 for p = 1)
 template <typename G, typename P>
 void set_score_mask(G& g, const P& p) {
@@ -542,10 +556,9 @@ void set_score_mask(G& g, const P& p) {
     g.bias = p.bias.data;
     g.bias_sb = p.bias.stride[0], g.bias_sh = p.bias.stride[1], g.bias_sl = p.q.size[2] > 1 ? p.bias.stride[2] : 0;
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
-  } else if (p.dropout_p > 0.f) {
-    g.bias = p.dropout_keep;
-    g.bias_sl = p.k.size[2], g.bias_sh = p.q.size[2] * g.bias_sl, g.bias_sb = p.q.size[1] * g.bias_sh;
-    g.bias_kind = 4;
+  }
+  if (p.dropout_p > 0.f) {
+    g.keep = p.dropout_keep;
     g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
 }
@@ -569,7 +582,6 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
   if ((p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) && (p.bias.data || p.dropout_p > 0.f))
     return *why = "window / sink / score functor together with attn_bias or dropout", false;
-  if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
   if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
       p.bias_dtype != MI355_SDPA_BOOL)
@@ -603,7 +615,7 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
   g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
   g.sm = score_mod_of(p.mask);
-  const int mode = g.bias != nullptr ? 1 : (g.window > 0 || g.sink_logit || g.sm.any) ? 2 : 0;
+  const int mode = (g.bias != nullptr || g.keep_scale != 0.f) ? 1 : (g.window > 0 || g.sink_logit || g.sm.any) ? 2 : 0;
   // rows per workgroup: 128 (a workgroup is one wavefront per 32 rows; 64- and 32-row workgroups
   // measured slower even when 128-row ones leave compute units without work)
   const int waves = pick_waves((int64_t)g.B * g.Hq, g.L);
@@ -632,7 +644,6 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
     return *why = "window or score functor together with attn_bias or dropout", false;
   if (p.grad_bias.data && (!p.bias.data || (p.k.size[2] > 1 && p.grad_bias.stride[3] != 1)))
     return *why = "grad_attn_bias without attn_bias, or its keys are not unit-stride", false;
-  if (p.bias.data && p.dropout_p > 0.f) return *why = "dropout together with attn_bias", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
   if (p.bias.data && p.bias_dtype != MI355_SDPA_F32 && p.bias_dtype != MI355_SDPA_F16 && p.bias_dtype != MI355_SDPA_BF16 &&
       p.bias_dtype != MI355_SDPA_BOOL)
@@ -684,7 +695,7 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
     g.gbias = p.grad_bias.data;
     g.gbias_sb = p.grad_bias.stride[0], g.gbias_sh = p.grad_bias.stride[1], g.gbias_sl = p.grad_bias.stride[2];
   }
-  const int mode = g.bias != nullptr ? 1 : (g.window > 0 || g.sm.any) ? 2 : 0;
+  const int mode = (g.bias != nullptr || g.keep_scale != 0.f) ? 1 : (g.window > 0 || g.sm.any) ? 2 : 0;
   const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
   const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
   const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw))));

@@ -24,9 +24,10 @@ struct FwdM {
   const void* bias = nullptr;
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  // dropout (fwd_mfma_w32.hip, head dims up to 128, no bias): nonzero = 1 / (1 - p) (1 for p = 1), and the
-  // bias fields above describe the (B, Hq, L, S) keep-mask, kind 4
+  // dropout (fwd_mfma_w32.hip, head dims up to 128; with or without a bias): nonzero = 1 / (1 - p)
+  // (1 for p = 1), and the (B, Hq, L, S) contiguous keep bytes
   float keep_scale = 0.f;
+  const void* keep = nullptr;
   // Short query sequences under grouped-query attention (fwd_mfma_w32.hip; no dropout, no bias that
   // depends on the head): one workgroup serves `grouped` query heads of a kv group (all Hq / Hkv of
   // them where they fit its wavefronts; a divisor of that otherwise, with Hq / Hkv / grouped

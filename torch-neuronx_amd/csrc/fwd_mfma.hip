@@ -356,9 +356,9 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
     (void)L;
   }
   if (p.dropout_p > 0.f) {
-    // the keep-mask takes the bias's way into the kernel (one dword = four keys of a row)
+    // the keep-mask takes a bool bias's way into the kernel (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
-    if (p.bias.data || p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "dropout together with attn_bias or a functor", false;
+    if (p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "dropout together with a functor", false;
     if (E > 128) return *why = "dropout with a head dim above 128", false;
     if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
     if (32 * S >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
@@ -406,16 +406,14 @@ static int launch_or_size(const mi355_sdpa_fwd_params& p, hipStream_t s, size_t*
     g.bias_kind = p.bias_dtype == MI355_SDPA_F32 ? 1 : p.bias_dtype == MI355_SDPA_F16 ? 2 : p.bias_dtype == MI355_SDPA_BF16 ? 3 : 4;
   }
   if (p.dropout_p > 0.f) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
-    g.bias = p.dropout_keep;
-    g.bias_sl = p.k.size[2], g.bias_sh = p.q.size[2] * g.bias_sl, g.bias_sb = p.q.size[1] * g.bias_sh;
-    g.bias_kind = 4;
+    g.keep = p.dropout_keep;
     g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
   g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
   g.sm = score_mod_of(p.mask);
-  if (p.bias.data && p.mask.live_tiles && !p.is_causal && g.S <= 32768 && p.bias.stride[2] != 0) {
+  if (p.bias.data && p.mask.live_tiles && !p.is_causal && g.S <= 32768 && p.bias.stride[2] != 0 && p.dropout_p == 0.f) {
     g.live_tiles = p.mask.live_tiles;
     g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
   }

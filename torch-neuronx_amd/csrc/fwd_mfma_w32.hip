@@ -63,7 +63,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   // (head dim 256 and the variant with a bias need more than the 64 KB of LDS a kernel may declare:
   // they take the launch's dynamic LDS instead; head dim 256 runs one wavefront per SIMD with the
   // 512-register budget)
-  constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;  // a per-score tensor in LDS; ... that is a dropout keep-mask
+  constexpr bool BIASED = MASK == 2 || MASK == 3, DROP = MASK == 3;  // a bias tile in LDS; ... and the tile of a dropout keep-mask beside it
   constexpr bool DYN = D > 128 || BIASED;
   // Tiles go from global memory straight into LDS (see the staging section): four unpadded,
   // swizzled buffers per operand, tile t in buffer t % 4.
@@ -80,6 +80,8 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   uint16_t* const bias_lds = dyn_lds + 2 * NBUF * TILE;
   // ... and, with a tile skip table, the list of the key tiles this workgroup walks (1024 entries and the count)
   uint16_t* const tile_list = bias_lds + WAVES * 2048;
+  // (dropout, which never comes with a table, has a wavefront's 1 KB of keep bytes there)
+  const unsigned char* const keep_lds = (const unsigned char*)(bias_lds + WAVES * 2048);
 
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // uniform: keeps per-wavefront tests on the scalar unit
@@ -109,7 +111,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   int S = p.S;
   if constexpr (MASK) {
     if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
-    if constexpr (MASK == 2) {
+    if constexpr (BIASED) {
       // A keep-mask per key (no row stride: padding masks): the keys behind the last one it keeps are
       // never visited, as with a key count.  Every wavefront scans the row itself (S bytes, four
       // per lane and step; rows are whole dwords) and they all arrive at the same count.
@@ -410,7 +412,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   // younger loads are those of the pair requested at the end of the previous iteration.
   uint32_t braw[4];
   float inv_scale = 0.f;
-  const int bkind = DROP ? 4 : MASK == 2 ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
+  const int bkind = BIASED ? __builtin_amdgcn_readfirstlane(ma.bias_kind) : 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
   const int b_esz = bkind == 1 ? 4 : bkind == 4 ? 1 : 2;
   const int b_rows = min(32, p.L - qw0);
   const u32x4 b_rsrc = descriptor((const char*)p.bias + (bkind ? (b * p.bias_sb + h * p.bias_sh + (int64_t)qw0 * p.bias_sl) * b_esz : 0),
@@ -420,11 +422,21 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   const unsigned char* const bias_w = (const unsigned char*)bias_lds + (BIASED ? wave * 4096 : 0);
   const uint32_t lds_b = (uint32_t)(uintptr_t)(lds_bytes)bias_w;
   if (bkind) inv_scale = 1.f / p.scale;
+  // Dropout: the keep bytes of the tile, (B, Hq, L, S) contiguous, travel the way a bool bias does -
+  // one load, lane (row, half) -> keys 16 half .. +15 - into 1 KB of the wavefront's own, beside the bias.
+  const u32x4 kp_rsrc = descriptor((const char*)p.keep + (DROP ? (((int64_t)b * p.Hq + h) * p.L + qw0) * p.S : 0),
+                                   (DROP && b_rows > 0) ? (int)((int64_t)b_rows * p.S) : 0);
+  const uint32_t kp_voff = DROP ? (uint32_t)(min(col, max(b_rows - 1, 0)) * p.S + half * 16) : 0u;
+  const unsigned char* const keep_w = keep_lds + (DROP ? wave * 1024 : 0);
+  const uint32_t lds_kp = (uint32_t)(uintptr_t)(lds_bytes)keep_w;
+  uint32_t kraw[4];
   auto load_bias = [&](int t) {
     if constexpr (BIASED) {
-      if (bkind) {
+      if (bkind || DROP) {
         // (the reads of the tile before are behind this wavefront before its buffer is rewritten)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+      }
+      if (bkind) {
         const uint32_t g0 = b_voff + (uint32_t)((listed ? tile_of(min(t, nt - 1)) : t + skip) * BN * b_esz);
         tile_load(b_rsrc, g0, lds_b);
         if (b_loads > 1) tile_load(b_rsrc, g0 + 32, lds_b + 1024);
@@ -433,16 +445,17 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
           tile_load(b_rsrc, g0 + 96, lds_b + 3072);
         }
       }
+      if constexpr (DROP) tile_load(kp_rsrc, kp_voff + (uint32_t)((t + skip) * BN), lds_kp);
     }
   };
   // (awaited: in the loop.  This wait also covers the pair that the iteration's barrier publishes.)
   auto apply_bias = [&](f32x16& sv, bool awaited) {
-    if constexpr (DROP) {  // the tile's keep bytes, used where its probabilities are packed
+    if constexpr (BIASED) {
       if (awaited) wait_youngest_pair_only();
+      if constexpr (DROP) {  // the tile's keep bytes, used where its probabilities are packed
 #pragma unroll
-      for (int g = 0; g < 4; ++g) braw[g] = *(const uint32_t*)(bias_w + (col + 32 * (g >> 1)) * 16 + (g & 1) * 8 + half * 4);
-    } else if constexpr (MASK == 2) {
-      if (awaited) wait_youngest_pair_only();
+        for (int g = 0; g < 4; ++g) kraw[g] = *(const uint32_t*)(keep_w + (col + 32 * (g >> 1)) * 16 + (g & 1) * 8 + half * 4);
+      }
       if (bkind == 1) {
         // (head dim 256 has no registers to spare: one group at a time there)
 #pragma unroll
@@ -627,7 +640,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
     asm volatile("" : "+v"(ps));  // keeps the add in its slot (left alone it sinks below the loop body)
     if constexpr (DROP) {  // (the sum above keeps the dropped probabilities)
       const int r = 2 * j;
-      const float k0 = (float)((braw[r >> 2] >> (8 * (r & 3))) & 0xffu), k1 = (float)((braw[r >> 2] >> (8 * (r & 3) + 8)) & 0xffu);
+      const float k0 = (float)((kraw[r >> 2] >> (8 * (r & 3))) & 0xffu), k1 = (float)((kraw[r >> 2] >> (8 * (r & 3) + 8)) & 0xffu);
       pk[j] = Mma<T>::pack(pv[j & 1][0] * k0, pv[j & 1][1] * k1);
     } else {
       pk[j] = Mma<T>::pack(pv[j & 1][0], pv[j & 1][1]);
@@ -939,7 +952,7 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
   int bytes = 0;
   if constexpr (D > 128 || MASK == 2 || MASK == 3) {
     // (four buffers per operand, 4 KB of bias tile per wavefront, and the tile list of a call with a skip table)
-    constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK >= 2 ? WAVES * 4096 : 0);
+    constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK >= 2 ? WAVES * 4096 : 0) + (MASK == 3 ? WAVES * 1024 : 0);
     constexpr int kBytes = kBase + (MASK == 2 ? 2048 + 16 : 0);
     static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK, PATTERN>,
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
@@ -1038,9 +1051,9 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   const dim3 grid((unsigned)blocks);
-  // kernel variant: 2 with a bias or keep-mask, 1 with key counts or rows narrower than the kernel's head dim
-  if (g.keep_scale != 0.f && (head_dim > 128 || g.bias_kind != 4)) {
-    set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128 and the keep-mask in the bias slot");
+  // kernel variant: 3 with a keep-mask (and a bias or none), 2 with a bias, 1 with key counts or rows narrower than the kernel's head dim
+  if (g.keep_scale != 0.f && (head_dim > 128 || !g.keep || g.live_tiles)) {
+    set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128, a keep-mask and no tile table");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   if (g.sm.any && (g.bias_kind != 0 || g.keep_scale != 0.f)) {
