@@ -915,27 +915,63 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
 }
 
 // Merge of the parts of a call whose keys were split: out = sum_s w_s O_s with w_s = exp(lse_s - lse),
-// lse = log sum_s exp(lse_s).  One workgroup per query row, one thread per output element.
+// lse = log sum_s exp(lse_s).  One workgroup per query row, one thread per output element.  The parts'
+// lse are read side by side (a thread per part) and their weights left in LDS; the rows of the parts
+// are then requested eight at a time: read one after the other, each of the two passes was a chain of
+// trips to the L2, and a call with 64 parts spent as long here as in the attention kernel.
 template <typename T>
 __global__ __launch_bounds__(128) void fwd_split_merge_kernel(FwdM p) {
+  constexpr int MAXP = 512;  // (fwd_w32_plan never makes more parts)
+  __shared__ float w_s[MAXP];
+  __shared__ float red_s[4];
   const int64_t row = blockIdx.x;  // (b * Hq + h) * L + l
   const int l = (int)(row % p.L);
   const int64_t bh = row / p.L;
   const int b = (int)(bh / p.Hq), h = (int)(bh % p.Hq);
   const float* pl = p.part_lse + bh * p.n_split * p.L + l;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float ls[MAXP / 128];
   float m = -INFINITY;
-  for (int s = 0; s < p.n_split; ++s) m = fmaxf(m, pl[(int64_t)s * p.L]);
-  float sum = 0.f, acc[2] = {0.f, 0.f};
-  const int d = threadIdx.x;  // columns d and d + 128 (head dims up to 256)
-  for (int s = 0; s < p.n_split; ++s) {
-    const float ls = pl[(int64_t)s * p.L];
-    if (ls == -INFINITY) continue;  // (a part without keys: its rows were never written)
-    const float w = __expf(ls - m);
-    sum += w;
-    const float* po = p.part_o + ((bh * p.n_split + s) * p.L + l) * p.dv_real;
 #pragma unroll
-    for (int i = 0; i < 2; ++i)
-      if (d + 128 * i < p.dv_real) acc[i] = fmaf(w, po[d + 128 * i], acc[i]);
+  for (int i = 0; i < MAXP / 128; ++i) {
+    const int sp = tid + 128 * i;
+    ls[i] = sp < p.n_split ? pl[(int64_t)sp * p.L] : -INFINITY;
+    m = fmaxf(m, ls[i]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  if (lane == 0) red_s[wave] = m;
+  __syncthreads();
+  m = fmaxf(red_s[0], red_s[1]);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXP / 128; ++i) {
+    const int sp = tid + 128 * i;
+    const float w = ls[i] == -INFINITY ? 0.f : __expf(ls[i] - m);  // (a part without keys: weight 0, its rows were never written)
+    if (sp < p.n_split) w_s[sp] = w;
+    sum += w;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  if (lane == 0) red_s[2 + wave] = sum;
+  __syncthreads();
+  sum = red_s[2] + red_s[3];
+  float acc[2] = {0.f, 0.f};
+  const int d = tid;  // columns d and d + 128 (head dims up to 256)
+  const float* po = p.part_o + (bh * p.n_split * p.L + l) * p.dv_real;
+  const int64_t part_stride = (int64_t)p.L * p.dv_real;
+  for (int s0 = 0; s0 < p.n_split; s0 += 8) {
+    float x[2][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool on = s0 + j < p.n_split && w_s[min(s0 + j, MAXP - 1)] > 0.f;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) x[i][j] = (on && d + 128 * i < p.dv_real) ? po[(s0 + j) * part_stride + d + 128 * i] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[i] = fmaf(w_s[min(s0 + j, MAXP - 1)], x[i][j], acc[i]);
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
