@@ -390,6 +390,29 @@ def test_training_steps_with_a_mask_that_is_new_every_step(amd, gpu_device, monk
 
 
 @pytest.mark.gpu
+def test_a_verdict_found_from_another_stream_is_waited_for(amd, gpu_device):
+    # two independent calls with one mask tensor on two streams: the second finds the first one's
+    # verdict still on its way and must not read it before the first stream has written it
+    dev = gpu_device
+    B, H, L, D = 1, 8, 1024, 64
+    q, k, v = (t.to(dev) for t in qkv(B, H, H, L, L, D, dtype=torch.bfloat16, seed=21))
+    ref = F.scaled_dot_product_attention(q, k, v, is_causal=True)
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    for make in (lambda: torch.ones(L, L, dtype=torch.bool, device=dev).tril(),                                  # the host copy is made
+                 lambda: torch.where(torch.ones(L, L, dtype=torch.bool, device=dev).tril(), 0.0, float("-inf")).to(torch.bfloat16)):  # ... and when it is not
+        for rounds in range(5 if make().dtype != torch.bool else 1):  # (the float mask: until its signature is left without a host copy)
+            mask = make()
+            torch.cuda.synchronize()
+            with torch.cuda.stream(s1):
+                o1 = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+            with torch.cuda.stream(s2):
+                o2 = F.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+            torch.cuda.synchronize()
+            assert max_abs(o1, ref) <= 1e-6 and max_abs(o2, ref) <= 1e-6
+
+
+@pytest.mark.gpu
 def test_a_captured_call_takes_its_verdict_on_every_replay(amd, gpu_device):
     # inside a stream capture nothing is cached and nothing waits: the verdict is part of the graph, so a
     # replay follows the mask as it then is - causal at the causal kernel's speed, anything else as a mask

@@ -180,10 +180,20 @@ _MIN_SCORES_ON_DEVICE = 256 * 256
 class _Pending:
     """A verdict on the device whose copy to the host is under way (or was not asked for)."""
 
-    __slots__ = ("verdict", "host", "event", "B")
+    __slots__ = ("verdict", "host", "event", "B", "stream")
 
-    def __init__(self, verdict, host, event, B):
-        self.verdict, self.host, self.event, self.B = verdict, host, event, B
+    def __init__(self, verdict, host, event, B, stream):
+        self.verdict, self.host, self.event, self.B, self.stream = verdict, host, event, B, stream
+
+    def usable_on(self, stream) -> bool:
+        """The verdict was computed on ``self.stream``: work on another stream has to wait for it
+        (through the event, where one was recorded)."""
+        if stream == self.stream:
+            return True
+        if self.event is None:
+            return False
+        stream.wait_event(self.event)
+        return True
 
     def settled(self) -> bool:
         return self.event is not None and self.event.query()
@@ -251,6 +261,8 @@ def look(mask: torch.Tensor, B: int, Hq: int, L: int, S: int):
             if not entry.settled():
                 # (the backward of the step that made the entry, typically: no sign that the tensor lives on)
                 stats["pending"] = stats.get("pending", 0) + 1
+                if on_device and not entry.usable_on(torch.cuda.current_stream(mask.device)):
+                    return None, _launch_verdict(view, dtype_id, words)
                 return None, (entry.verdict if on_device else None)
             # (still possibly the backward of the step that made the entry: the miss streak stands)
             pat = entry.pattern()
@@ -269,15 +281,16 @@ def look(mask: torch.Tensor, B: int, Hq: int, L: int, S: int):
             return None, None
         # (remembered without a copy to the host: the backward of the same step finds it here)
         verdict = _launch_verdict(view, dtype_id, words)
-        _remember(_cache, key, _Pending(verdict, None, None, B), mask)
+        _remember(_cache, key, _Pending(verdict, None, None, B, torch.cuda.current_stream(mask.device)), mask)
         return None, verdict
     stats["looked"] += 1
     verdict = _launch_verdict(view, dtype_id, words)
     host = torch.empty((8 + B,), dtype=torch.int32, pin_memory=True)
     host.copy_(verdict[:8 + B], non_blocking=True)
     event = torch.cuda.Event()
-    event.record(torch.cuda.current_stream(mask.device))
-    _remember(_cache, key, _Pending(verdict, host, event, B), mask)
+    stream = torch.cuda.current_stream(mask.device)
+    event.record(stream)
+    _remember(_cache, key, _Pending(verdict, host, event, B, stream), mask)
     return None, (verdict if on_device else None)
 
 
