@@ -53,7 +53,7 @@ enum mi355_sdpa_kernel {
   MI355_SDPA_KERNEL_NONE = 0,
   MI355_SDPA_KERNEL_GENERIC = 1, /* fp32-accumulate kernel: any head dim, bias, masks, dropout */
   MI355_SDPA_KERNEL_MFMA = 2,    /* matrix-op flash kernels: bf16/f16 (head dims up to 256, masks,
-                                    functors; dropout up to head dim 128) and float32
+                                    functors, dropout) and float32
                                     (head dims up to 128; masks, key counts, dropout, functors) */
   /* forward only, for tests and tuning: pin the query rows per workgroup of the MFMA kernel */
   MI355_SDPA_KERNEL_MFMA_T128 = 3,

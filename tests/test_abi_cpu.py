@@ -183,7 +183,7 @@ def test_kernel_gates(amd):
     assert gate(q96, q96, q96, is_causal=True) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
     q256 = _meta(2, 8, 512, 256)  # head dims up to 256, forward and backward
     assert gate(q256, q256, q256) == (L.KERNEL_MFMA, L.KERNEL_MFMA)
-    assert gate(q256, q256, q256, dropout_p=0.1) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
+    assert gate(q256, q256, q256, dropout_p=0.1) == (L.KERNEL_MFMA, L.KERNEL_MFMA)  # dropout at every width
     q100 = _meta(2, 8, 512, 100)
     assert gate(q100, q100, q100) == (L.KERNEL_GENERIC, L.KERNEL_GENERIC)
     q2, k2 = _meta(1, 4, 64, 192), _meta(1, 4, 64, 192)
@@ -267,7 +267,7 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
     # results out, after the loops (seen in the generated code: no scratch access before the last barrier);
     # its functor mode keeps a second packed copy of the probabilities and spills more.  That file
     # waits for every load at once (no counted waits), so a spill there costs time, not correctness.
-    known = re.compile(r"bwd_wide_dkdv_kernelIDF16[b_]Li256ELi256ELi([012])ELb([01])EE")
+    known = re.compile(r"bwd_wide_dkdv_kernelIDF16[b_]Li256ELi256ELi([0123])ELb([01])EE")
     for name, r in rows.items():
         if r["src"] not in ("fwd_mfma_w32.hip", "bwd_dq_w32.hip", "bwd_dkdv_w32.hip", "bwd_wide.hip", "decode_fp8kv.hip"):
             continue
@@ -286,7 +286,8 @@ def test_hot_kernels_use_no_scratch_and_keep_their_occupancy():
             # (masked with skip tables and no split: the spill in the loop alone; the instances that
             # split: the write-out's as well)
             mode, tables = int(m.group(1)), int(m.group(2))
-            assert scratch <= (288 if mode == 2 else 64 if (mode == 1 and tables == 1) else 96), (name, scratch)
+            # (functor and dropout modes: a second packed copy of the probabilities, the functors' operands or the keep bits)
+            assert scratch <= (288 if mode >= 2 else 64 if (mode == 1 and tables == 1) else 96), (name, scratch)
             continue
         assert scratch == 0, (name, scratch)
         assert r["Dynamic_Stack"] == "False"

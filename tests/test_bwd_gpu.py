@@ -170,6 +170,9 @@ DROPOUT_MFMA = [
     (3, 3, 1, 33, 36, 40, False, [36, 1, 20], 0.3),
     (1, 2, 2, 256, 256, 96, True, None, 1.0),
     (2, 12, 12, 512, 512, 64, False, [512, 300], 0.1),  # a BERT-base layer with right padding
+    (1, 4, 2, 300, 260, 256, True, None, 0.1),            # head dims above 128: the wide backward kernels
+    (2, 2, 2, 129, 512, 192, False, [512, 77], 0.25),
+    (1, 2, 1, 64, 64, 160, True, None, 0.5),
 ]
 
 
@@ -220,6 +223,9 @@ DROPOUT_BIAS = [
     (1, 2, 2, 200, 136, 64, False, torch.float32, (1, 2, 200, 136), 0.25, True),
     (2, 2, 2, 256, 256, 128, True, None, (2, 2, 256, 256), 0.1, True),           # (the bias in the calls' dtype)
     (1, 3, 1, 40, 72, 40, False, torch.float32, (1, 3, 40, 72), 0.3, False),    # head dim padded to 64
+    (1, 4, 2, 200, 136, 256, True, torch.bfloat16, (1, 4, 200, 136), 0.25, True),  # head dims above 128
+    (2, 2, 2, 128, 128, 160, False, torch.bool, (2, 1, 1, 128), 0.3, False),
+    (1, 2, 2, 96, 260, 256, False, torch.float32, (1, 1, 96, 260), 0.1, False),
 ]
 
 
@@ -264,6 +270,33 @@ def test_dropout_together_with_a_bias_in_the_matrix_op_kernels(amd, gpu_device, 
     if want_gb:
         # (delta comes from the rounded output: a row with one live key has dS = O(ulp of out) instead of 0)
         assert db.shape == (B, Hq, L, S) and max_abs(db, rdb) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
+def test_dropout_at_unequal_head_dims(amd, gpu_device, dtype):
+    """D_qk = 192, D_v = 128 (the multi-head-latent-attention shape) with dropout and key counts, causal,
+    forced into the MFMA kernels, against the oracle."""
+    B, Hq, Hkv, L, S, E, Dv, pdrop = 2, 4, 2, 160, 192, 192, 128, 0.2
+    dev = gpu_device
+    g = torch.Generator().manual_seed(17)
+    q, k, v, go = (torch.randn(s_, generator=g).to(dtype) for s_ in ((B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, Dv), (B, Hq, L, Dv)))
+    go = (go.float() * 0.1).to(dtype)
+    keep = torch.rand(B, Hq, L, S, generator=g) >= pdrop
+    lens = [192, 100]
+    mask = (torch.arange(S)[None] < torch.tensor(lens)[:, None])[:, None, None, :].expand(B, Hq, L, S) & torch.ones(L, S, dtype=torch.bool).tril()
+    bias = torch.where(mask, 0.0, float("-inf"))
+    rep = Hq // Hkv
+    kf, vf = k.float().repeat_interleave(rep, 1), v.float().repeat_interleave(rep, 1)
+    ro, rl = om.compute_attention(q.float(), kf, vf, bias, keep, E**-0.5, False, pdrop)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(go.float(), q.float(), kf, vf, bias, keep, ro, rl, E**-0.5, False, pdrop)
+    rdk, rdv = rdk.view(B, Hkv, rep, S, E).sum(2), rdv.view(B, Hkv, rep, S, Dv).sum(2)
+    kw = dict(is_causal=True, dropout_p=pdrop, dropout_keep=keep.to(dev), kv_lens=torch.tensor(lens, dtype=torch.int32, device=dev),
+              force_kernel=amd._lib.KERNEL_MFMA)
+    out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), **kw)
+    dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, **kw)
+    assert max_abs(out, ro) <= (2e-2 if dtype == torch.bfloat16 else 4e-3) and max_abs(lse, rl) <= 2e-3
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= (1e-2 if dtype == torch.bfloat16 else 2e-3)
 
 
 def test_dropout_with_a_padding_mask_through_the_operator(amd, gpu_device):

@@ -24,7 +24,7 @@ struct BwdM {
   const void* bias = nullptr;
   int64_t bias_sb = 0, bias_sh = 0, bias_sl = 0;
   int bias_kind = 0;  // 0 none, 1 float32, 2 float16, 3 bfloat16, 4 bool
-  // dropout (head dims up to 128; with or without a bias): nonzero = 1 / (1 - p) (1 for p = 1), and the
+  // dropout (with or without a bias): nonzero = 1 / (1 - p) (1 for p = 1), and the
   // (B, Hq, L, S) contiguous keep bytes
   float keep_scale = 0.f;
   const void* keep = nullptr;

@@ -607,7 +607,6 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
     // the keep-mask takes a bool bias's way into the kernels (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
     if (p.mask.window > 0) return *why = "dropout together with a window functor", false;
-    if (wide) return *why = "dropout with a head dim above 128 or D_qk != D_v", false;
     if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
     if ((p.q.size[2] + 64) * S + S + 64 >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
   }

@@ -154,12 +154,16 @@ constexpr WideOp dkdv_op(int k) {  // S steps and dP steps (in turns where both 
 // lane is a query row in the dQ kernel and reads its own row of it, a key in the dK/dV kernel and reads
 // one element per score register); the gradient of the bias, P (dP - delta) in the input dtype, leaves
 // the dQ kernel four keys at a time: the packed dS pairs it feeds to the matrix pipe are its elements.
+// MODE 3 (DROP): MODE 1 without the skip tables, and a dropout keep-mask beside the bias (bytes,
+// (B, Hq, L, S) contiguous, read the way a bool mask per score is): it leaves the scores alone, feeds dV
+// with the kept probabilities and multiplies dP, together with 1 / (1 - p)
+// (torch_neuronx/_sdpa_math.py:36-48, :154-158).
 // MODE 2 (FUNC): per-batch key counts, a sliding window with sink keys (the tiles it drops whole are not
 // walked) and the score functors and document ids of score_mod.h, each score through score_mod_at where
 // its probability is formed; the derivative of the functors multiplies the gradient of the scores.
 template <typename T, int ER, int DVR, int MODE>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
-  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;
+  constexpr bool MASKED = MODE == 1 || MODE == 3, FUNC = MODE == 2, DROP = MODE == 3;
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const k_buf = wide_lds;                    // [2][TILE_ELEMS]
@@ -232,7 +236,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   // rows (the first wavefront ORs the bitmaps of its two 64-row blocks and expands the set bits into a
   // list in LDS); stream position u is then key tile tile_of(u).
   bool listed = false;
-  if constexpr (MASKED) {
+  if constexpr (MODE == 1) {
     if (p.live_tiles && !p.causal && !p.gbias) {  // (with a bias gradient every tile is walked: its zeros are written there)
       if (wave == 0) {
         const int nrb = (p.L + 63) / 64, rb0 = q0 / 64;
@@ -260,7 +264,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
     }
   }
   auto tile_of = [&](int u) {
-    if constexpr (MASKED) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
+    if constexpr (MODE == 1) return listed ? __builtin_amdgcn_readfirstlane((int)tile_list[u]) : u;
     else if constexpr (FUNC) return u + (u >= n_lead ? skip : 0);
     else return u;
   };
@@ -290,7 +294,17 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
       __builtin_amdgcn_readfirstlane(bkind ? (int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz) : 0), 0x00020000);
   const uint32_t b_row = MASKED ? (uint32_t)(((int64_t)qc * p.bias_sl + half * 4) * besz) : 0u;
   uint32_t braw[16];
+  // (DROP) the keep bytes of the same 16 keys, four dwords
+  const __amdgpu_buffer_rsrc_t kp_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+      uniform_ptr((const char*)p.keep + (DROP ? ((int64_t)b * p.Hq + h) * p.L * p.S : 0)), 0,
+      __builtin_amdgcn_readfirstlane(DROP ? (int)((int64_t)p.L * p.S) : 0), 0x00020000);
+  const uint32_t kp_row = DROP ? (uint32_t)((int64_t)qc * p.S + half * 4) : 0u;
+  uint32_t kraw[DROP ? 4 : 1];
   auto load_bias = [&](int t) {
+    if constexpr (DROP) {
+#pragma unroll
+      for (int g = 0; g < 4; ++g) kraw[g] = __builtin_amdgcn_raw_buffer_load_b32(kp_rsrc, kp_row + (uint32_t)(t * BT + g * 8), 0, 0);
+    }
     if constexpr (MASKED) {
       const uint32_t off = b_row + (uint32_t)(t * BT * besz);
       if (bkind == 1) {
@@ -414,7 +428,12 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
         pr[r] = __builtin_amdgcn_exp2f(kv > lim ? -INFINITY : x);  // (masked before the exponential: no branch)
       };
       auto form_ds = [&](int r) {  // elements r, r + 1
-        pS[r >> 1] = Mma<T>::pack(pr[r] * (dpacc[r] - dl), pr[r + 1] * (dpacc[r + 1] - dl));
+        if constexpr (DROP) {
+          const float k0 = (float)((kraw[r >> 2] >> (8 * (r & 3))) & 0xffu), k1 = (float)((kraw[r >> 2] >> (8 * (r & 3) + 8)) & 0xffu);
+          pS[r >> 1] = Mma<T>::pack(pr[r] * fmaf(dpacc[r] * k0, p.keep_scale, -dl), pr[r + 1] * fmaf(dpacc[r + 1] * k1, p.keep_scale, -dl));
+        } else {
+          pS[r >> 1] = Mma<T>::pack(pr[r] * (dpacc[r] - dl), pr[r + 1] * (dpacc[r + 1] - dl));
+        }
       };
       static_for<NA>([&](auto kc) {
         constexpr int k = decltype(kc)::value;
@@ -509,7 +528,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
 // workgroups, not for both: one instance of each.
 template <typename T, int ER, int DVR, int MODE, bool TABLES>
 __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
-  constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // (see bwd_wide_dq_kernel)
+  constexpr bool MASKED = MODE == 1 || MODE == 3, FUNC = MODE == 2, DROP = MODE == 3;  // (see bwd_wide_dq_kernel)
   constexpr int KSE = ER / 16, KSV = DVR / 16, DBE = ER / 32, DBV = DVR / 32;
   extern __shared__ __attribute__((aligned(16))) uint16_t wide_lds[];
   uint16_t* const q_buf = wide_lds;                        // [2][TILE_ELEMS]
@@ -585,6 +604,26 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   const uint32_t b_lane = MASKED ? (uint32_t)((half * 4 * p.bias_sl + min(key, p.S - 1)) * besz) : 0u;
   const int b_records = MASKED ? __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.L - 1) * p.bias_sl + p.S) * besz)) : 0;
   uint32_t braw[16];
+  // (DROP) the keep bytes of the same 16 scores, requested with the bias; then one bit each: bit r says
+  // that the score of accumulator register r is kept
+  uint32_t kbits = 0u;
+  auto request_keep = [&](int hg, int q0, uint32_t (&kb)[DROP ? 16 : 1]) {
+    if constexpr (DROP) {
+      const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
+          uniform_ptr((const char*)p.keep + ((int64_t)b * p.Hq + hk * rep + hg) * p.L * p.S), 0,
+          __builtin_amdgcn_readfirstlane((int)((int64_t)p.L * p.S)), 0x00020000);
+      const uint32_t base = (uint32_t)((q0 + half * 4) * p.S + min(key, p.S - 1));
+#pragma unroll
+      for (int r = 0; r < 16; ++r) kb[r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(k_rsrc, base + (uint32_t)(((r >> 2) * 8 + (r & 3)) * p.S), 0, 0);
+    }
+  };
+  auto pack_keep = [&](const uint32_t (&kb)[DROP ? 16 : 1]) {
+    if constexpr (DROP) {
+      kbits = 0u;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) kbits |= min(kb[r], 1u) << r;
+    }
+  };
   auto load_bias = [&](int hg, int q0) {
     if constexpr (MASKED) {
       if (!bkind) return;
@@ -689,7 +728,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       constexpr bool GENERAL = true;
       // (at full width the bias is requested behind the score products: ahead of them its 16
       // registers are more than the register file has left)
-      if constexpr (ER + DVR <= 320) load_bias(hg, q0);
+      uint32_t kb[DROP ? 16 : 1];
+      if constexpr (ER + DVR <= 320) load_bias(hg, q0), request_keep(hg, q0, kb);
       const uint16_t* q_t = q_buf + buf * TILE_ELEMS;
       const uint16_t* do_t = do_buf + buf * TILE_ELEMS;
       const float* lse_s = lse_buf + buf * BT;
@@ -717,6 +757,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       static_for<AHEAD>([&](auto kc) { ring[decltype(kc)::value] = operand(kc); });
       uint32_t pP[8], pS[8];
       uint32_t pF[FUNC && GENERAL ? 8 : 1];  // (FUNC) the probabilities times the derivative of the functors, for dS
+      uint32_t pM[DROP ? 8 : 1];             // (DROP) the kept probabilities, for dV
       // (at full width the register file has no room for the score and the dP accumulator at once next
       // to the two fragments: there the probabilities are formed before dP is issued, uncovered)
       constexpr bool BOTH = ER + DVR <= 320;
@@ -734,8 +775,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       auto issue_dp = [&]() { issue(std::integral_constant<int, KSE>{}, std::integral_constant<int, KSV>{}); };
       if constexpr (BOTH) issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE + KSV>{});
       else issue(std::integral_constant<int, 0>{}, std::integral_constant<int, KSE>{});
-      if constexpr (!BOTH) load_bias(hg, q0);
+      if constexpr (!BOTH) load_bias(hg, q0), request_keep(hg, q0, kb);
       if constexpr (MASKED) bias_to_log2();
+      pack_keep(kb);
       // (FUNC) what the functors take from this lane's key, for the item's head
       float f_w = 1.f;
       if constexpr (FUNC && GENERAL) {
@@ -784,6 +826,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
           pr[e] = __builtin_amdgcn_exp2f(qi < first_q ? -INFINITY : x);
         }
         pP[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pP[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+        if constexpr (DROP) {  // dV gets the kept probabilities, dS all of them
+#pragma unroll
+          for (int e = 0; e < 4; ++e) pr[e] = ((kbits >> (r4 * 4 + e)) & 1u) ? pr[e] : 0.f;
+          pM[r4 * 2] = Mma<T>::pack(pr[0], pr[1]), pM[r4 * 2 + 1] = Mma<T>::pack(pr[2], pr[3]);
+        }
         if constexpr (FUNC && GENERAL) {  // (a dropped score may carry any derivative)
 #pragma unroll
           for (int e = 0; e < 4; ++e) df[e] = pr[e] == 0.f ? 0.f : pr[e] * df[e];
@@ -803,7 +850,12 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
             uint32_t w;
             if constexpr (FUNC && GENERAL) w = pF[r4 * 2 + (e >> 1)];
             else w = pP[r4 * 2 + (e >> 1)];
-            ds[e] = Mma<T>::unpack(w, e & 1) * (dpacc[r4 * 4 + e] - d4[e]);
+            if constexpr (DROP) {
+              const float kf = ((kbits >> (r4 * 4 + e)) & 1u) ? p.keep_scale : 0.f;
+              ds[e] = Mma<T>::unpack(w, e & 1) * fmaf(dpacc[r4 * 4 + e], kf, -d4[e]);
+            } else {
+              ds[e] = Mma<T>::unpack(w, e & 1) * (dpacc[r4 * 4 + e] - d4[e]);
+            }
           }
           pS[r4 * 2] = Mma<T>::pack(ds[0], ds[1]), pS[r4 * 2 + 1] = Mma<T>::pack(ds[2], ds[3]);
         }
@@ -815,7 +867,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
         constexpr WideOp op = dkdv_op<ER, DVR>(k);
         if constexpr (k + AHEAD < NOPS) ring[(k + AHEAD) & 7] = operand(std::integral_constant<int, k + AHEAD>{});
         constexpr int r0 = (op.j / DB) * 4;
-        const u32x4 bP = {pP[r0], pP[r0 + 1], pP[r0 + 2], pP[r0 + 3]};
+        u32x4 bP;
+        if constexpr (DROP) bP = u32x4{pM[r0], pM[r0 + 1], pM[r0 + 2], pM[r0 + 3]};
+        else bP = u32x4{pP[r0], pP[r0 + 1], pP[r0 + 2], pP[r0 + 3]};
         dvacc[op.j % DB] = Mma<T>::run(ring[k & 7], bP, dvacc[op.j % DB]);
         __builtin_amdgcn_sched_barrier(0);
       });
@@ -875,6 +929,7 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
         uniform_ptr((char*)((uint16_t*)p.gv + b * p.gv_sb + hk * p.gv_sh)), 0,
         __builtin_amdgcn_readfirstlane((int)(((int64_t)(p.S - 1) * p.gv_sl + dvr) * 2)), 0x00020000);
     const uint32_t ok = (uint32_t)(((int64_t)key * p.gk_sl + half * 4) * 2), ov = (uint32_t)(((int64_t)key * p.gv_sl + half * 4) * 2);
+    const float v_scale = DROP ? p.keep_scale : 1.f;  // (dropout's 1 / (1 - p) on the kept probabilities)
 #pragma unroll
     for (int db = 0; db < DBE; ++db) {
 #pragma unroll
@@ -893,8 +948,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
       for (int g = 0; g < 4; ++g) {
         const int d = db * 32 + g * 8;
         u32x2 wv;
-        wv[0] = Mma<T>::pack(dvacc[db][g * 4], dvacc[db][g * 4 + 1]);
-        wv[1] = Mma<T>::pack(dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]);
+        wv[0] = Mma<T>::pack(dvacc[db][g * 4] * v_scale, dvacc[db][g * 4 + 1] * v_scale);
+        wv[1] = Mma<T>::pack(dvacc[db][g * 4 + 2] * v_scale, dvacc[db][g * 4 + 3] * v_scale);
         __builtin_amdgcn_raw_buffer_store_b64(wv, rv, (live_key && d + half * 4 < dvr) ? ov + d * 2 : kDrop, 0, 0);
       }
       __builtin_amdgcn_sched_barrier(0);
@@ -942,8 +997,15 @@ template <typename T>
 int launch_w(const BwdM& g, hipStream_t s) {
   const bool func = g.window > 0 || g.sm.any;  // (never together with a bias: refused before)
   const bool masked = g.bias_kind || g.kv_lens;  // (a bias gradient comes with a bias)
+  const bool drop = g.keep_scale != 0.f;          // (never together with a functor or a skip table: refused before)
+  if (drop && (!g.keep || func || g.live_t || g.live_tiles)) {
+    set_error("SDPA: dropout in the wide backward kernels needs a keep-mask, no functor and no tile table");
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
   if (g.d_real <= 192 && g.dv_real <= 128)
-    return func ? launch_t<T, 192, 128, 2>(g, s) : masked ? launch_t<T, 192, 128, 1>(g, s) : launch_t<T, 192, 128, 0>(g, s);
+    return drop ? launch_t<T, 192, 128, 3>(g, s)
+           : func ? launch_t<T, 192, 128, 2>(g, s) : masked ? launch_t<T, 192, 128, 1>(g, s) : launch_t<T, 192, 128, 0>(g, s);
+  if (drop) return launch_t<T, 256, 256, 3>(g, s);
   if (func) return launch_t<T, 256, 256, 2>(g, s);
   if (masked && g.parts > 1) return launch_t<T, 256, 256, 1, true>(g, s);  // (bwd_wide_parts: no skip table then)
   return masked ? launch_t<T, 256, 256, 1>(g, s) : launch_t<T, 256, 256, 0>(g, s);

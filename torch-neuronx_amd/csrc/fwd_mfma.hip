@@ -359,7 +359,6 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
     // the keep-mask takes a bool bias's way into the kernel (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
     if (p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "dropout together with a functor", false;
-    if (E > 128) return *why = "dropout with a head dim above 128", false;
     if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
     if (32 * S >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))

@@ -1004,9 +1004,7 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
 template <typename T, int D, int WAVES>
 int launch_mask(const FwdM& g, int mask, dim3 grid, hipStream_t s) {
   if (mask == 4) return launch_one<T, D, WAVES, 4>(g, grid, s);
-  if constexpr (D <= 128) {
-    if (mask == 3) return launch_one<T, D, WAVES, 3>(g, grid, s);
-  }
+  if (mask == 3) return launch_one<T, D, WAVES, 3>(g, grid, s);
   if (mask == 2) {
     if (g.verdict) {  // (see fwd_w32_kernel)
       if (int rc = launch_one<T, D, WAVES, 1, true>(g, grid, s)) return rc;
@@ -1055,7 +1053,7 @@ void fwd_w32_plan(FwdM& g, int head_dim, int& waves) {
   if (g.grouped && (head_dim <= 128 || g.bias_kind == 0) && !g.causal && g.window == 0 && !g.sink_logit && !g.sm.any) {
     const int64_t groups = (int64_t)g.B * g.Hkv * (g.Hq / g.Hkv / g.grouped);
     const int nt = (g.S + BN - 1) / BN;
-    const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);
+    const int want = (int)std::min<int64_t>((512 + groups - 1) / groups, nt / 8);  // (at most 512 parts: fwd_split_merge_kernel's limit)
     if (groups < 256 && want >= 2) {
       g.split_tiles = (nt + want - 1) / want;
       g.n_split = (nt + g.split_tiles - 1) / g.split_tiles;
@@ -1077,7 +1075,7 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
   fwd_w32_plan(g, head_dim, waves);
   if (g.split_tiles) {  // (the caller's workspace: too small or absent, and the call runs unsplit)
     const size_t rows = (size_t)g.B * g.Hq * g.n_split * g.L;
-    if (g.part_o && g.part_bytes >= rows * (g.dv_real + 1) * sizeof(float)) g.part_lse = g.part_o + rows * g.dv_real;
+    if (g.part_o && g.n_split <= 512 && g.part_bytes >= rows * (g.dv_real + 1) * sizeof(float)) g.part_lse = g.part_o + rows * g.dv_real;
     else g.split_tiles = 0, g.n_split = 1;
   }
   const int64_t blocks = g.grouped ? (int64_t)g.B * (g.Hq / g.grouped) * g.n_split : (int64_t)g.B * g.Hq * g.n_qt;
@@ -1088,8 +1086,8 @@ int launch_fwd_mfma_w32(const FwdM& g0, int dtype, int head_dim, int waves, hipS
   }
   const dim3 grid((unsigned)blocks);
   // kernel variant: 3 with a keep-mask (and a bias or none), 2 with a bias, 1 with key counts or rows narrower than the kernel's head dim
-  if (g.keep_scale != 0.f && (head_dim > 128 || !g.keep || g.live_tiles)) {
-    set_error("SDPA: dropout in fwd_w32_kernel needs a head dim up to 128, a keep-mask and no tile table");
+  if (g.keep_scale != 0.f && (!g.keep || g.live_tiles)) {
+    set_error("SDPA: dropout in fwd_w32_kernel needs a keep-mask and no tile table");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   if (g.sm.any && (g.bias_kind != 0 || g.keep_scale != 0.f)) {
