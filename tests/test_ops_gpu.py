@@ -214,6 +214,22 @@ def test_unregister_brings_the_stock_kernels_back(amd, gpu_device, calls):
     assert calls["fwd"] == 2
 
 
+def test_a_keep_mask_of_one_element_is_a_placeholder(amd, gpu_device):
+    """The reference treats a dropout mask of one element as absent (torch_neuronx/_sdpa_math.py:42-45):
+    so do the forward and the backward here, whatever the byte says and whatever dropout_p is."""
+    from oracle import sdpa_math as om
+    dev = gpu_device
+    q, k, v, go = (t.to(dev) for t in qkv(1, 1, 1, 1, 1, 64, dtype=torch.float32, seed=3, with_do=True))
+    keep = torch.zeros(1, 1, 1, 1, dtype=torch.bool, device=dev)
+    out, lse = amd.sdpa_forward(q, k, v, dropout_p=0.9, dropout_keep=keep)
+    dq, dk, dv, _ = amd.sdpa_backward(go, q, k, v, out, lse, dropout_p=0.9, dropout_keep=keep)
+    ro, rl = om.compute_attention(q.cpu(), k.cpu(), v.cpu(), None, keep.cpu(), 64**-0.5, False, 0.9)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(go.cpu(), q.cpu(), k.cpu(), v.cpu(), None, keep.cpu(), ro, rl, 64**-0.5, False, 0.9)
+    assert max_abs(out, ro) <= 1e-6 and max_abs(out, v) <= 1e-6  # (one key: the output is its value row, undropped and unscaled)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, r) <= 1e-6
+
+
 def test_dropout_extremes_and_mask_round_trip(amd, gpu_device):
     q, k, v = (t.to(gpu_device) for t in qkv(1, 2, 2, 32, 32, 32, dtype=torch.float32, seed=8))
     op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable

@@ -285,8 +285,13 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     if dropout_p > 0.0:
         if dropout_keep is None:
             raise ValueError("dropout_p > 0 needs dropout_keep")
-        dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
-        p.dropout_keep = dropout_keep.data_ptr()
+        if not 0.0 <= dropout_p <= 1.0:
+            raise ValueError(f"dropout_p={dropout_p} is outside [0, 1]. Pass a value in [0, 1].")
+        if dropout_keep.numel() <= 1:
+            dropout_p = 0.0  # a mask of one element is the reference's placeholder for none (torch_neuronx/_sdpa_math.py:42-45)
+        else:
+            dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
+            p.dropout_keep = dropout_keep.data_ptr()
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
@@ -352,8 +357,13 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     if dropout_p > 0.0:
         if dropout_keep is None:
             raise ValueError("dropout_p > 0 needs dropout_keep")
-        dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
-        p.dropout_keep = dropout_keep.data_ptr()
+        if not 0.0 <= dropout_p <= 1.0:
+            raise ValueError(f"dropout_p={dropout_p} is outside [0, 1]. Pass a value in [0, 1].")
+        if dropout_keep.numel() <= 1:
+            dropout_p = 0.0  # a mask of one element is the reference's placeholder for none (torch_neuronx/_sdpa_math.py:42-45)
+        else:
+            dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
+            p.dropout_keep = dropout_keep.data_ptr()
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
