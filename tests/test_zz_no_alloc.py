@@ -15,11 +15,11 @@ from oracle import sdpa_math as om
 pytestmark = pytest.mark.gpu
 
 
-def _inputs(dev, B, Hq, Hkv, Lq, S, lens, seed):
+def _inputs(dev, B, Hq, Hkv, Lq, S, lens, seed, D=128):
     g = torch.Generator().manual_seed(seed)
-    q = torch.randn(B, Hq, Lq, 128, generator=g).to(torch.bfloat16)
-    kq, ks = om.quantize_kv_fp8(torch.randn(B, Hkv, S, 128, generator=g))
-    vq, vs = om.quantize_kv_fp8(torch.randn(B, Hkv, S, 128, generator=g))
+    q = torch.randn(B, Hq, Lq, D, generator=g).to(torch.bfloat16)
+    kq, ks = om.quantize_kv_fp8(torch.randn(B, Hkv, S, D, generator=g))
+    vq, vs = om.quantize_kv_fp8(torch.randn(B, Hkv, S, D, generator=g))
     cpu = (q, kq, vq, ks, vs, lens)
     gpu = tuple(None if t is None else t.to(dev) for t in (q, kq, vq, ks.float().contiguous(), vs.float().contiguous(), lens))
     return cpu, gpu
@@ -31,7 +31,8 @@ def test_static_scratch_decode_matches_the_workspace_entry_point(gpu_device):
     dev = gpu_device
     big_lens = torch.tensor([2048, 517, 1, 1999, 1024, 33, 777, 1500], dtype=torch.int32)
     small_lens = torch.tensor([300, 64, 5], dtype=torch.int32)
-    cases = [_inputs(dev, 8, 32, 8, 1, 2048, big_lens, 11), _inputs(dev, 3, 8, 2, 2, 320, small_lens, 12)]
+    cases = [_inputs(dev, 8, 32, 8, 1, 2048, big_lens, 11), _inputs(dev, 3, 8, 2, 2, 320, small_lens, 12),
+             _inputs(dev, 3, 16, 2, 1, 320, small_lens, 13, D=256), _inputs(dev, 3, 8, 8, 1, 320, small_lens, 14, D=64)]  # (the other head dims)
     # outputs are the caller's: allocated here, before the calls under test
     outs = [(torch.empty(c[1][0].shape, dtype=torch.bfloat16, device=dev),
              torch.empty(c[1][0].shape[:3], dtype=torch.float32, device=dev)) for c in cases]

@@ -523,7 +523,7 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     p.lse[((int64_t)b * p.Hq + h) * p.Lq + lq] = L > 0.f ? (M + __builtin_amdgcn_logf(L)) * kLn2 : -INFINITY;
 }
 
-constexpr int kMaxWaves = 4096;  // bound on the streaming kernel's grid; sizes the workspace
+constexpr int kMaxSimds = 1024;  // bound on the streaming kernel's grid: wavefronts per SIMD it is built for x this; sizes the workspace
 constexpr int kMinSteps = 4;     // 128 keys: below this the partial results rival the keys in bytes
 
 int wave_slots(int head_dim) {  // wavefronts of the decode kernel the chip holds at once
@@ -536,7 +536,7 @@ int wave_slots(int head_dim) {  // wavefronts of the decode kernel the chip hold
     else
       simds = 256 * 4;
   }
-  return std::min(simds * dec_occ(head_dim), kMaxWaves);
+  return std::min(simds, kMaxSimds) * dec_occ(head_dim);
 }
 
 // least steps per wavefront: num_splits > 0 asks for at most about that many pieces per sequence
@@ -577,7 +577,10 @@ int launch_t(const DecP& g, int head_dim, hipStream_t s) {
   return head_dim == 64 ? launch_td<TQ, 64>(g, s) : head_dim == 128 ? launch_td<TQ, 128>(g, s) : launch_td<TQ, 256>(g, s);
 }
 
-int64_t partial_slots(const mi355_sdpa_decode_params& p) { return p.q.size[0] * p.k.size[1] + kMaxWaves; }
+// (the same on every device: the size query and the call need not run with the same device current)
+int64_t partial_slots(const mi355_sdpa_decode_params& p) {
+  return p.q.size[0] * p.k.size[1] + kMaxSimds * dec_occ((int)p.q.size[3]);
+}
 
 }  // namespace
 
