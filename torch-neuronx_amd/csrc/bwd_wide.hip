@@ -445,14 +445,42 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
           if constexpr (op.j == 0 && FUNC && GENERAL) {
             // every score through the functors, in one block behind one test: s = mod(scale * s) / scale,
             // so that the code around it is the common one (a call with a window alone skips the block)
+            // (one loop per functor behind one test each: tested per score, even a uniform test costs this
+            // kernel more than the functor; the soft cap through one exponential and one reciprocal)
             if (p.sm.any) {
+              auto kv_of = [&](int r) { return min(ta * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
 #pragma unroll
-              for (int r = 0; r < 16; ++r) {
-                const int kv = min(ta * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1);
-                float dfac;
-                sacc[r] = score_mod_at(p.sm, sacc[r] * p.scale, b, h, qc, kv, p.L, p.S, dfac) * inv_scale;
-                if (f_kw) bl[r] = f_kw[kv];  // (the key's weight is the part of the derivative that the score does not tell)
+              for (int r = 0; r < 16; ++r) sacc[r] *= p.scale;
+              if (f_kw) {
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                  bl[r] = f_kw[kv_of(r)];  // (the key's weight is the part of the derivative that the score does not tell)
+                  sacc[r] *= bl[r];
+                }
               }
+              if (p.sm.key_bias) {
+                const float* kb = p.sm.key_bias + (int64_t)h * p.S;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[r] += kb[kv_of(r)];
+              }
+              if (p.sm.alibi) {
+                const float slope = p.sm.alibi[h], base = (float)(ta * BT + half * 4 - qc);  // (keys past S are masked whatever they get)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[r] = fmaf(slope, base + (float)((r >> 2) * 8 + (r & 3)), sacc[r]);
+              }
+              if (p.sm.softcap > 0.f) {
+                const float cap = p.sm.softcap, inv_cap = 1.f / p.sm.softcap;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[r] = cap * tanh_fast(sacc[r] * inv_cap);
+              }
+              if (p.sm.doc_q && p.sm.doc_k) {
+                const int32_t mine = p.sm.doc_q[(int64_t)b * p.L + qc];
+                const int32_t* dk = p.sm.doc_k + (int64_t)b * p.S;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sacc[r] = dk[kv_of(r)] != mine ? -INFINITY : sacc[r];
+              }
+#pragma unroll
+              for (int r = 0; r < 16; ++r) sacc[r] *= inv_scale;
             }
           }
 #pragma unroll
@@ -792,14 +820,27 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
           if (p.sm.alibi) f_slope = p.sm.alibi[hq];
           const bool docs = p.sm.doc_q && p.sm.doc_k;
           if (docs) f_doc = p.sm.doc_k[(int64_t)b * p.S + kc];
+          // (one loop per functor behind one test each, as in the dQ kernel)
+          const float sw = p.scale * f_w;
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int qi = q0 + (r >> 2) * 8 + half * 4 + (r & 3);
-            float u = fmaf(sacc[r] * p.scale, f_w, f_kb) + f_slope * (float)(key - qi);
-            if (p.sm.softcap > 0.f) u = p.sm.softcap * tanh_fast(u / p.sm.softcap);
-            if (docs && p.sm.doc_q[(int64_t)b * p.L + min(qi, p.L - 1)] != f_doc) u = -INFINITY;
-            sacc[r] = u * inv_scale;
+          for (int r = 0; r < 16; ++r) sacc[r] = fmaf(sacc[r], sw, f_kb);
+          if (p.sm.alibi) {
+            const float base = (float)(key - q0 - half * 4);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] = fmaf(f_slope, base - (float)((r >> 2) * 8 + (r & 3)), sacc[r]);
           }
+          if (p.sm.softcap > 0.f) {
+            const float cap = p.sm.softcap, inv_cap = 1.f / p.sm.softcap;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] = cap * tanh_fast(sacc[r] * inv_cap);
+          }
+          if (docs) {
+            const int32_t* dq = p.sm.doc_q + (int64_t)b * p.L;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) sacc[r] = dq[min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1)] != f_doc ? -INFINITY : sacc[r];
+          }
+#pragma unroll
+          for (int r = 0; r < 16; ++r) sacc[r] *= inv_scale;
         }
       }
 #pragma unroll
