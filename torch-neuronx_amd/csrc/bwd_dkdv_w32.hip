@@ -838,8 +838,8 @@ template <typename T, int D, int MASK, bool PATTERN = false>
 int launch_t(const BwdM& g, hipStream_t s) {
   // (MASK = 2: with the skip table's row of the key block and the item list; MASK = 4: with the document ids of three tiles' rows)
   constexpr int kSmemBytes = smem_bytes<D>() + (MASK == 2 ? 1024 + 2048 + 16 : MASK == 4 ? 3 * BQ * 4 : 0);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_dkdv_w32_kernel<T, D, MASK, PATTERN>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kSmemBytes);
+  static LdsOnce once;
+  const hipError_t attr = reserve_lds(once, (const void*)bwd_dkdv_w32_kernel<T, D, MASK, PATTERN>, kSmemBytes);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dkdv_w32_kernel: %s", kSmemBytes, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;

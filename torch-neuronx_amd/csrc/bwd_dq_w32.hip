@@ -750,7 +750,8 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
     const void* fn3 = head_dim == 128 ? (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 128, 3> : (const void*)bwd_dq_w32_kernel<f16_t, 128, 3>)
                                       : (bf ? (const void*)bwd_dq_w32_kernel<bf16_t, 64, 3> : (const void*)bwd_dq_w32_kernel<f16_t, 64, 3>);
     const void* fn = mask == 3 ? fn3 : fn2;
-    const hipError_t attr = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, dyn);
+    static LdsOnce once[8];  // (one per instance with dynamic LDS)
+    const hipError_t attr = reserve_lds(once[(head_dim == 128 ? 4 : 0) + (bf ? 2 : 0) + (mask == 3 ? 1 : 0)], fn, dyn);
     if (attr != hipSuccess) {
       set_error("SDPA: cannot reserve %d bytes of LDS for bwd_dq_w32_kernel: %s", dyn, hipGetErrorString(attr));
       return MI355_SDPA_ERR_LAUNCH;

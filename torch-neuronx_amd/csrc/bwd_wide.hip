@@ -1001,8 +1001,8 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
 template <typename T, int ER, int DVR, int MODE, bool TABLES>
 int launch_dkdv(const BwdM& g, int64_t k_blocks, hipStream_t s) {
   constexpr int kDkdvLds = WIDE_DKDV_LDS + (MODE == 1 ? WIDE_LIVE_LDS : 0);
-  static const hipError_t attr = hipFuncSetAttribute((const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MODE, TABLES>,
-                                                     hipFuncAttributeMaxDynamicSharedMemorySize, kDkdvLds);
+  static LdsOnce once;
+  const hipError_t attr = reserve_lds(once, (const void*)bwd_wide_dkdv_kernel<T, ER, DVR, MODE, TABLES>, kDkdvLds);
   if (attr != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dkdv_kernel: %s", kDkdvLds, hipGetErrorString(attr));
     return MI355_SDPA_ERR_LAUNCH;
@@ -1020,8 +1020,8 @@ int launch_t(const BwdM& g, hipStream_t s) {
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
   constexpr int kDqLds = WIDE_DQ_LDS + (MODE == 1 ? WIDE_LIST_LDS : 0);
-  static const hipError_t attr_q = hipFuncSetAttribute((const void*)bwd_wide_dq_kernel<T, ER, DVR, MODE>,
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kDqLds);
+  static LdsOnce once_q;
+  const hipError_t attr_q = reserve_lds(once_q, (const void*)bwd_wide_dq_kernel<T, ER, DVR, MODE>, kDqLds);
   if (attr_q != hipSuccess) {
     set_error("SDPA: cannot reserve %d bytes of LDS for bwd_wide_dq_kernel: %s", kDqLds, hipGetErrorString(attr_q));
     return MI355_SDPA_ERR_LAUNCH;

@@ -4,6 +4,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/mi355_sdpa.h"
 
 namespace mi355 {
@@ -11,6 +13,19 @@ namespace mi355 {
 // host side -------------------------------------------------------------------------------
 void set_error(const char* fmt, ...) __attribute__((format(printf, 1, 2)));
 int check_launch(const char* what);
+// The dynamic-LDS limit of a kernel, raised once per device and call site: the attribute belongs to a
+// device's copy of the kernel, so a process that drives several GPUs sets it on each of them.
+struct LdsOnce {
+  std::atomic<uint64_t> done{0};  // bit d: set on device d
+};
+inline hipError_t reserve_lds(LdsOnce& once, const void* kernel, int bytes) {
+  int dev = -1;
+  const bool known = hipGetDevice(&dev) == hipSuccess && dev >= 0 && dev < 64;
+  if (known && (once.done.load(std::memory_order_acquire) >> dev & 1ull)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (e == hipSuccess && known) once.done.fetch_or(1ull << dev, std::memory_order_release);
+  return e;
+}
 
 int launch_fwd_generic(const mi355_sdpa_fwd_params& p, hipStream_t s);
 int launch_fwd_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s);

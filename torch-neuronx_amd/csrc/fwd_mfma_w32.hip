@@ -990,8 +990,8 @@ int launch_one(const FwdM& g, dim3 grid, hipStream_t s) {
     // (four buffers per operand, 4 KB of bias tile per wavefront, and the tile list of a call with a skip table)
     constexpr int kBase = 2 * 4 * BN * D * 2 + (MASK >= 2 ? WAVES * 4096 : 0) + (MASK == 3 ? WAVES * 1024 : 0);
     constexpr int kBytes = kBase + (MASK == 2 ? 2048 + 16 : 0);
-    static const hipError_t attr = hipFuncSetAttribute((const void*)fwd_w32_kernel<T, D, WAVES, MASK, PATTERN>,
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, kBytes);
+    static LdsOnce once;
+    const hipError_t attr = reserve_lds(once, (const void*)fwd_w32_kernel<T, D, WAVES, MASK, PATTERN>, kBytes);
     if (attr != hipSuccess) {
       set_error("SDPA: cannot reserve %d bytes of LDS for fwd_w32_kernel: %s", kBytes, hipGetErrorString(attr));
       return MI355_SDPA_ERR_LAUNCH;
