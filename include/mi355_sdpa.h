@@ -54,7 +54,7 @@ enum mi355_sdpa_kernel {
   MI355_SDPA_KERNEL_GENERIC = 1, /* fp32-accumulate kernel: any head dim, bias, masks, dropout */
   MI355_SDPA_KERNEL_MFMA = 2,    /* matrix-op flash kernels: bf16/f16 (head dims up to 256, masks,
                                     functors, dropout) and float32
-                                    (head dims up to 128; masks, key counts, dropout, functors) */
+                                    (the same head dims; masks, key counts, dropout, functors) */
   /* forward only, for tests and tuning: pin the query rows per workgroup of the MFMA kernel */
   MI355_SDPA_KERNEL_MFMA_T128 = 3,
   MI355_SDPA_KERNEL_MFMA_T256 = 4
@@ -118,7 +118,7 @@ typedef struct mi355_sdpa_desc {
  *                test whole tiles with two loads.  Without the promise every tile is walked and
  *                every score compared: same results, no skipping.
  * Score functors and document ids run in the matrix-op kernels for bf16 / f16 at every head dim up
- * to 256 (D_v <= D_qk) and for float32 up to 128, without attn_bias and dropout; other calls take
+ * to 256 (D_v <= D_qk), and for float32 at the same head dims, without attn_bias and dropout; other calls take
  * the generic kernels.
  * Tile skip tables for a mask that only exists as a tensor (the run-time counterpart of the
  * reference's static tile elimination, flex_attention.py.jinja:15-33), built from the bias /

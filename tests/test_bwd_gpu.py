@@ -546,8 +546,6 @@ def test_mfma_backward_grad_bias(amd, gpu_device, case, dtype):
     # grad_bias = P (dP - delta) leaves the MFMA dQ kernel in the input dtype (forced: no fallback);
     # the buffer starts as NaN, so every element must be written
     B, Hq, Hkv, L, S, E, kind, causal, with_lens = case
-    if dtype is torch.float32 and E > 128:
-        pytest.skip("float32 above head dim 128 is served by the generic kernels")
     q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L + S, with_do=True)
     go = go.clamp(-1, 1) * 0.1
     g = torch.Generator().manual_seed(S)

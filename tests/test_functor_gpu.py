@@ -58,6 +58,7 @@ def test_functors_float32(amd, gpu_device, window, sink_keys, with_sink):
     (512, 128, 100, 40, True),    # several tiles below the window are dropped whole, the sink tiles are not
     (260, 96, 0, 0, True),        # sink logit alone, a narrow head dim
     (130, 16, 1000, 0, False),    # window longer than the sequence
+    (200, 256, 70, 5, True),      # the width-256 instances
 ])
 def test_functors_float32_in_the_matrix_op_kernels(amd, gpu_device, L, E, window, sink_keys, with_sink):
     # (forced: the call fails if the float32 matrix-op kernels refuse it)

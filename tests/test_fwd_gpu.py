@@ -522,6 +522,9 @@ F32_SHAPES = [
     (1, 4, 4, 6, 6, 8, False),
     (2, 8, 2, 300, 1100, 128, True),
     (1, 2, 2, 200, 70, 104, True),
+    (1, 4, 2, 512, 512, 256, True),      # (:362-387) head dim 256: width-256 instances, two dK/dV workgroups per key block
+    (2, 2, 1, 100, 160, 160, False),
+    (1, 3, 3, 40, 300, 136, True),
 ]
 
 
@@ -546,6 +549,32 @@ def test_float32_matrix_op_forward_and_backward(amd, gpu_device, shape):
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
     out3, _ = amd.sdpa_forward(qd, kd, vd, is_causal=causal, force_kernel=GENERIC)
     assert max_abs(out3, out) <= 1e-5
+
+
+def test_float32_matrix_op_at_unequal_head_dims(amd, gpu_device):
+    """D_qk = 192, D_v = 128 and D_qk = 128, D_v = 64 in float32 (forced into the float32 matrix-op kernels),
+    causal with key counts, forward and backward against the oracle."""
+    from oracle import sdpa_math as om
+
+    dev = gpu_device
+    for B, Hq, Hkv, L, S, E, Dv in ((2, 4, 2, 160, 192, 192, 128), (1, 4, 4, 100, 100, 128, 64), (1, 2, 1, 70, 130, 256, 8)):
+        g = torch.Generator().manual_seed(E + Dv)
+        q, k, v, go = (torch.randn(s_, generator=g) for s_ in ((B, Hq, L, E), (B, Hkv, S, E), (B, Hkv, S, Dv), (B, Hq, L, Dv)))
+        lens = torch.randint(1, S + 1, (B,), generator=g).to(torch.int32)
+        mask = (torch.arange(S)[None] < lens[:, None])[:, None, None, :].expand(B, Hq, L, S) & torch.ones(L, S, dtype=torch.bool).tril()
+        bias = torch.where(mask, 0.0, float("-inf"))
+        rep = Hq // Hkv
+        kf, vf = k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1)
+        ro, rl = om.compute_attention(q, kf, vf, bias, None, E**-0.5, False, 0.0)
+        rdq, rdk, rdv, _ = om.compute_attention_backward(go, q, kf, vf, bias, None, ro, rl, E**-0.5, False, 0.0)
+        rdk, rdv = rdk.view(B, Hkv, rep, S, E).sum(2), rdv.view(B, Hkv, rep, S, Dv).sum(2)
+        kw = dict(is_causal=True, kv_lens=lens.to(dev), force_kernel=MFMA)
+        out, lse = amd.sdpa_forward(q.to(dev), k.to(dev), v.to(dev), **kw)
+        dq, dk, dv, _ = amd.sdpa_backward(go.to(dev), q.to(dev), k.to(dev), v.to(dev), out, lse, **kw)
+        assert out.shape == (B, Hq, L, Dv) and dv.shape == (B, Hkv, S, Dv) and dk.shape == (B, Hkv, S, E)
+        assert max_abs(out, ro) <= 1e-5 and max_abs(lse, rl) <= 1e-5
+        for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+            assert max_abs(a, r) <= 3e-5 * max(1.0, r.abs().max().item())
 
 
 @pytest.mark.parametrize("shape", [(3, 4, 2, 100, 160, 64, False, [160, 1, 77]), (2, 8, 8, 300, 300, 128, True, [300, 130]),
@@ -586,6 +615,8 @@ F32_MASKED = [
     (2, 4, 2, 100, 160, 64, False, "f32_full+dropout", None),
     (1, 8, 2, 300, 300, 128, True, "bool_full+dropout", None),
     (3, 2, 2, 33, 70, 40, False, "f16_key+dropout", [70, 5, 33]),
+    (1, 2, 2, 100, 160, 256, True, "f32_full+dropout", None),   # width 256
+    (2, 2, 1, 70, 96, 192, False, "bool_full", [96, 40]),
 ]
 
 

@@ -81,7 +81,8 @@ def test_reference_cases_float32(amd, gpu_device, pattern, L):
 
 
 @pytest.mark.parametrize("pattern", PATTERNS)
-@pytest.mark.parametrize("B,Hq,Hkv,L,S,E", [(1, 4, 2, 256, 256, 16), (2, 4, 1, 300, 500, 96), (1, 2, 2, 200, 200, 128)])
+@pytest.mark.parametrize("B,Hq,Hkv,L,S,E", [(1, 4, 2, 256, 256, 16), (2, 4, 1, 300, 500, 96), (1, 2, 2, 200, 200, 128),
+                                            (1, 2, 1, 160, 200, 256)])  # (... and the width-256 instances)
 def test_float32_in_the_matrix_op_kernels(amd, gpu_device, pattern, B, Hq, Hkv, L, S, E):
     # float32 inputs on the float32 matrix op, forced (the call fails if those kernels refuse it)
     _check(amd, gpu_device, B, Hq, Hkv, L, S, E, torch.float32, pattern, seed=L + E, force=amd._lib.KERNEL_MFMA)

@@ -249,8 +249,8 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   // (a bias gradient or a window sends the backward of head dims above 128 and of D_qk != D_v to the
   // generic kernel at the call)
   const bool dims = E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E;
-  // (float32: the float32 matrix-op kernels, head dims up to 128 with D_qk = D_v)
-  const bool f32_ok = d->q_dtype != MI355_SDPA_F32 || (E == Dv && E <= 128);
+  // (float32: the float32 matrix-op kernels take the same head dims)
+  const bool f32_ok = true;
   // (dropout, 16-bit dtypes: keep-mask rows that are whole dwords)
   const bool drop_ok = d->dropout_p == 0.f || d->q_dtype == MI355_SDPA_F32 || S % 4 == 0;
   const bool fast = f32_ok && dims &&

@@ -1,7 +1,8 @@
 // Flash attention for float32 inputs on the float32 matrix op (v_mfma_f32_32x32x2_f32), forward and
-// backward, head dims up to 128 (multiples of 8; narrower rows count as zero padded), causal or
+// backward, head dims up to 256 with D_v <= D_qk (multiples of 8; narrower rows count as zero padded:
+// instances of width 64, 128 and 256), causal or
 // unmasked, with per-batch key counts; instances with a per-score bias / keep-mask (and its gradient)
-// or dropout, and instances with the mask and score functors (sliding window with sink keys, sink
+// and / or dropout, and instances with the mask and score functors (sliding window with sink keys, sink
 // logits, the functors and document ids of score_mod.h, element by element).  The reference's fused gate takes float32 (decompositions.py:2131-2158); everything
 // stays in float32 as in torch_neuronx/_sdpa_math.py (float32 inputs accumulate in float32, and the
 // probabilities that multiply V are not rounded, :94).
@@ -26,6 +27,13 @@ namespace mi355 {
 namespace {
 
 constexpr int BT = 32;  // rows of a staged tile
+// Width 256 (head dims above 128, D_v <= D_qk): the two tiles of a kernel are more than the 64 KB of
+// LDS that a kernel may declare, so they live in the launch's dynamic LDS; and the register file has
+// no room for a tile on its way next to the row fragments and accumulators, so a tile is fetched
+// where it is stored (FetchAhead false).
+extern __shared__ __attribute__((aligned(16))) float wide_f32_lds[];
+template <int D> constexpr bool kFetchAhead = D <= 128;
+template <int D> constexpr int kTileFloats = BT * (D + 4);
 
 __device__ __forceinline__ f32x16 mma(float a, float b, f32x16 c) {
   return __builtin_amdgcn_mfma_f32_32x32x2f32(a, b, c, 0, 0, 0);
@@ -83,13 +91,14 @@ __device__ __forceinline__ f32x16 row_product(const float* tile, int col, int ha
 
 // acc[db] += cols(tile)^T . x : contraction over the tile's 32 rows in the order the accumulators of
 // a row product hold them (register r of lane half h is row 8 (r / 4) + 4 h + r % 4)
-template <int D>
-__device__ __forceinline__ void col_product(f32x16 (&acc)[D / 32], const float* tile, int col, int half, const f32x16& x) {
+// (NB column blocks of 32, from the column that `tile` points at: the whole width, or the share of one pass)
+template <int D, int NB = D / 32>
+__device__ __forceinline__ void col_product(f32x16 (&acc)[NB], const float* tile, int col, int half, const f32x16& x) {
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const float* row = tile + ((r >> 2) * 8 + half * 4 + (r & 3)) * (D + 4) + col;
 #pragma unroll
-    for (int db = 0; db < D / 32; ++db) acc[db] = mma(row[db * 32], x[r], acc[db]);
+    for (int db = 0; db < NB; ++db) acc[db] = mma(row[db * 32], x[r], acc[db]);
   }
 }
 
@@ -119,8 +128,10 @@ template <int D, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // a per-score tensor | window, sinks, score functors
   constexpr int DB = D / 32;
-  __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
-  __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float k_st[D > 128 ? 4 : BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float v_st[D > 128 ? 4 : BT * (D + 4)];
+  float* const k_t = D > 128 ? wide_f32_lds : k_st;
+  float* const v_t = D > 128 ? wide_f32_lds + kTileFloats<D> : v_st;
   const int qt = p.n_qt - 1 - blockIdx.x / (p.B * p.Hq);  // heavy query tiles first
   const int bh = blockIdx.x % (p.B * p.Hq), b = bh / p.Hq, h = bh % p.Hq, hk = h / (p.Hq / p.Hkv);
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
@@ -157,14 +168,18 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
   auto fetch = [&](int u) {
     const int t = tile_of(u);
     kn.fetch(kp + (int64_t)t * BT * p.k_sl, p.k_sl, S - t * BT, p.d_real, tid);
-    vn.fetch(vp + (int64_t)t * BT * p.v_sl, p.v_sl, S - t * BT, p.d_real, tid);
+    if constexpr (!kFetchAhead<D>) kn.put(k_t, tid);  // (one tile's registers serve both operands)
+    auto& v_regs = kFetchAhead<D> ? vn : kn;
+    v_regs.fetch(vp + (int64_t)t * BT * p.v_sl, p.v_sl, S - t * BT, p.dv_real, tid);
+    if constexpr (!kFetchAhead<D>) v_regs.put(v_t, tid);
   };
-  if (nt > 0) fetch(0);
+  if (kFetchAhead<D> && nt > 0) fetch(0);
   for (int u = 0; u < nt; ++u) {
     __syncthreads();  // the previous tile has been read by every wavefront
-    kn.put(k_t, tid), vn.put(v_t, tid);
+    if constexpr (kFetchAhead<D>) kn.put(k_t, tid), vn.put(v_t, tid);
+    else fetch(u);
     __syncthreads();
-    if (u + 1 < nt) fetch(u + 1);
+    if (kFetchAhead<D> && u + 1 < nt) fetch(u + 1);
     if (u >= nt_w) continue;
     const int t = tile_of(u);
     f32x16 s = row_product<D>(k_t, col, half, qf);
@@ -257,7 +272,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         const int d = db * 32 + g * 8 + half * 4;
-        if (d < p.d_real)
+        if (d < p.dv_real)
           *(f32x4*)(orow + d) = f32x4{oacc[db][g * 4] * inv, oacc[db][g * 4 + 1] * inv, oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv};
       }
     if (p.lse && half == 0)
@@ -269,8 +284,10 @@ template <int D, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // a per-score tensor | window, sink keys, score functors
   constexpr int DB = D / 32;
-  __shared__ __attribute__((aligned(16))) float k_t[BT * (D + 4)];
-  __shared__ __attribute__((aligned(16))) float v_t[BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float k_st[D > 128 ? 4 : BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float v_st[D > 128 ? 4 : BT * (D + 4)];
+  float* const k_t = D > 128 ? wide_f32_lds : k_st;
+  float* const v_t = D > 128 ? wide_f32_lds + kTileFloats<D> : v_st;
   constexpr int BM = 32 * WAVES;  // query rows per workgroup
   const int n_qt = (p.L + BM - 1) / BM;
   const int qt = n_qt - 1 - blockIdx.x / (p.B * p.Hq);
@@ -279,7 +296,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   const int q0 = qt * BM, qw0 = q0 + wave * 32, qrow = qw0 + col, qc = min(qrow, p.L - 1);
   float qf[D / 2], dof[D / 2];
   load_half_row<D>(qf, (const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)qc * p.q_sl, half, p.d_real);
-  load_half_row<D>(dof, (const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl, half, p.d_real);
+  load_half_row<D>(dof, (const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)qc * p.go_sl, half, p.dv_real);
   float lse2, dl;
   {
     // delta = rowsum(dO * O) (torch_neuronx/_sdpa_math.py:160-163): dO is in registers already
@@ -288,7 +305,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
 #pragma unroll
     for (int i = 0; i < D / 8; ++i) {
       const int d = half * (D / 2) + i * 4;
-      if (d < p.d_real) {
+      if (d < p.dv_real) {
         const f32x4 o = *(const f32x4*)(orow + d);
 #pragma unroll
         for (int e = 0; e < 4; ++e) dsum = fmaf(dof[i * 4 + e], o[e], dsum);
@@ -330,14 +347,18 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
   auto fetch = [&](int u) {
     const int t = tile_of(u);
     kn.fetch(kp + (int64_t)t * BT * p.k_sl, p.k_sl, S - t * BT, p.d_real, tid);
-    vn.fetch(vp + (int64_t)t * BT * p.v_sl, p.v_sl, S - t * BT, p.d_real, tid);
+    if constexpr (!kFetchAhead<D>) kn.put(k_t, tid);  // (one tile's registers serve both operands)
+    auto& v_regs = kFetchAhead<D> ? vn : kn;
+    v_regs.fetch(vp + (int64_t)t * BT * p.v_sl, p.v_sl, S - t * BT, p.dv_real, tid);
+    if constexpr (!kFetchAhead<D>) v_regs.put(v_t, tid);
   };
-  if (nt > 0) fetch(0);
+  if (kFetchAhead<D> && nt > 0) fetch(0);
   for (int u = 0; u < nt; ++u) {
     __syncthreads();  // the previous tile has been read by every wavefront
-    kn.put(k_t, tid), vn.put(v_t, tid);
+    if constexpr (kFetchAhead<D>) kn.put(k_t, tid), vn.put(v_t, tid);
+    else fetch(u);
     __syncthreads();
-    if (u + 1 < nt) fetch(u + 1);
+    if (kFetchAhead<D> && u + 1 < nt) fetch(u + 1);
     if (u >= nt_w) continue;
     const int t = tile_of(u);
     f32x16 s = row_product<D>(k_t, col, half, qf);
@@ -354,7 +375,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
       }
     }
     float bl[MASKED ? 16 : 1];  // the bias in the log2 domain
-    float kf[MASKED ? 16 : 1];  // (dropout) keep / (1 - p)
+    float kpf[MASKED ? 16 : 1];  // (dropout) keep / (1 - p)
     bool drop = false;
     if constexpr (MASKED) {
       const int64_t row0 = b * p.bias_sb + h * p.bias_sh + (int64_t)qc * p.bias_sl;
@@ -363,7 +384,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
       if (drop) {
         const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.S;
 #pragma unroll
-        for (int r = 0; r < 16; ++r) kf[r] = (float)krow[min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1)] * p.keep_scale;
+        for (int r = 0; r < 16; ++r) kpf[r] = (float)krow[min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1)] * p.keep_scale;
       }
       if (p.bias_kind) {
         load_bias16(bl, p.bias, p.bias_kind, idx);
@@ -381,7 +402,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
       if constexpr (MASKED) x = fmaf(s[r], c, bl[r]) - lse2;
       const float pr = __builtin_amdgcn_exp2f(kv > lim ? -INFINITY : x);
       float g = dp[r];
-      if constexpr (MASKED) g = drop ? g * kf[r] : g;
+      if constexpr (MASKED) g = drop ? g * kpf[r] : g;
       ds[r] = pr * (g - dl);
       if constexpr (MASKED) {
         if (gb_row && kv < p.S) gb_row[kv] = ds[r];
@@ -415,14 +436,21 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
 template <int D, int WAVES, int MODE>
 __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   constexpr bool MASKED = MODE == 1, FUNC = MODE == 2;  // a per-score tensor | window, sink keys, score functors
-  constexpr int DB = D / 32;
-  __shared__ __attribute__((aligned(16))) float q_t[BT * (D + 4)];
-  __shared__ __attribute__((aligned(16))) float do_t[BT * (D + 4)];
+  // Width 256: the K and V fragments of a key are 256 registers, so the accumulators of a workgroup
+  // are half of the columns of dK and dV (128 registers) and a key block is visited by two workgroups,
+  // one per half; both form every score and every dP.
+  constexpr int NP = D > 128 ? 2 : 1;  // passes = workgroups per key block
+  constexpr int DB = D / 32 / NP;      // 32-column blocks of dK / dV per pass
+  __shared__ __attribute__((aligned(16))) float q_st[D > 128 ? 4 : BT * (D + 4)];
+  __shared__ __attribute__((aligned(16))) float do_st[D > 128 ? 4 : BT * (D + 4)];
+  float* const q_t = D > 128 ? wide_f32_lds : q_st;
+  float* const do_t = D > 128 ? wide_f32_lds + kTileFloats<D> : do_st;
   __shared__ __attribute__((aligned(16))) float lse_s[BT];
   __shared__ __attribute__((aligned(16))) float dl_s[BT];
   const int streams = p.B * p.Hkv;
-  const int kt = blockIdx.x / streams;  // low key tiles see the most queries under a causal mask: first
-  const int st = blockIdx.x % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
+  const int pass = blockIdx.x % NP, c0 = pass * DB * 32;  // this pass's first column
+  const int kt = blockIdx.x / NP / streams;  // low key tiles see the most queries under a causal mask: first
+  const int st = blockIdx.x / NP % streams, b = st / p.Hkv, hk = st % p.Hkv, rep = p.Hq / p.Hkv;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6, col = lane & 31, half = lane >> 5;
   const int k0 = kt * 32 * WAVES, kw0 = k0 + wave * 32, key = kw0 + col, kc = min(key, p.S - 1);
   const int S = p.kv_lens ? min(p.S, max(p.kv_lens[b], 0)) : p.S;  // keys of this batch that take part
@@ -431,7 +459,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   const int first_q = key >= S ? INT_MAX : p.causal ? key : INT_MIN;
   float kf[D / 2], vf[D / 2];
   load_half_row<D>(kf, (const float*)p.k + b * p.k_sb + hk * p.k_sh + (int64_t)kc * p.k_sl, half, p.d_real);
-  load_half_row<D>(vf, (const float*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl, half, p.d_real);
+  load_half_row<D>(vf, (const float*)p.v + b * p.v_sb + hk * p.v_sh + (int64_t)kc * p.v_sl, half, p.dv_real);
   f32x16 dkacc[DB], dvacc[DB];
 #pragma unroll
   for (int i = 0; i < DB; ++i) zero(dkacc[i]), zero(dvacc[i]);
@@ -447,7 +475,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
     // share an XCD, then want the same Q / dO tile at about the same time and find it in its L2)
     const int h = hk * rep + it % rep, q0 = (nqs - 1 - it / rep) * BT;
     qn.fetch((const float*)p.q + b * p.q_sb + h * p.q_sh + (int64_t)q0 * p.q_sl, p.q_sl, p.L - q0, p.d_real, tid);
-    gn.fetch((const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, p.d_real, tid);
+    if constexpr (!kFetchAhead<D>) qn.put(q_t, tid);  // (one tile's registers serve both operands)
+    auto& g_regs = kFetchAhead<D> ? gn : qn;
+    g_regs.fetch((const float*)p.go + b * p.go_sb + h * p.go_sh + (int64_t)q0 * p.go_sl, p.go_sl, p.L - q0, p.dv_real, tid);
+    if constexpr (!kFetchAhead<D>) g_regs.put(do_t, tid);
     if (tid < BT) {
       const int qi = q0 + tid;
       const int64_t row = ((int64_t)b * p.Hq + h) * p.L + min(qi, p.L - 1);
@@ -456,15 +487,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
       dl_n = qi < p.L ? p.delta[row] : 0.f;
     }
   };
-  if (n_items > 0) fetch_item(0);
+  if (kFetchAhead<D> && n_items > 0) fetch_item(0);
   {
     for (int it = 0; it < n_items; ++it) {
       const int q0 = (nqs - 1 - it / rep) * BT;
       __syncthreads();
-      qn.put(q_t, tid), gn.put(do_t, tid);
+      if constexpr (kFetchAhead<D>) qn.put(q_t, tid), gn.put(do_t, tid);
+      else fetch_item(it);
       if (tid < BT) lse_s[tid] = lse_n, dl_s[tid] = dl_n;
       __syncthreads();
-      if (it + 1 < n_items) fetch_item(it + 1);
+      if (kFetchAhead<D> && it + 1 < n_items) fetch_item(it + 1);
       if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= S) continue;  // (uniform per wavefront)
       if constexpr (FUNC) {  // every row of the tile lies past the window of every key of this wavefront, none of them a sink
         if (p.window > 0 && q0 - (kw0 + 31) >= p.window && kw0 >= p.sink_keys) continue;
@@ -484,7 +516,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
         }
       }
       float bl[MASKED ? 16 : 1];  // the bias in the log2 domain
-      float kf[MASKED ? 16 : 1];  // (dropout) keep / (1 - p)
+      float kpf[MASKED ? 16 : 1];  // (dropout) keep / (1 - p)
       bool drop = false;
       if constexpr (MASKED) {
         const int hq = hk * rep + it % rep;
@@ -494,7 +526,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
         if (drop) {
           const uint8_t* kcol = (const uint8_t*)p.keep + ((int64_t)b * p.Hq + hq) * p.L * p.S + min(key, p.S - 1);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) kf[r] = (float)kcol[(int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.S] * p.keep_scale;
+          for (int r = 0; r < 16; ++r) kpf[r] = (float)kcol[(int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.S] * p.keep_scale;
         }
         if (p.bias_kind) {
           load_bias16(bl, p.bias, p.bias_kind, idx);
@@ -518,14 +550,14 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
           float g = dp[r];
           pr[r] = x;
           if constexpr (MASKED) {
-            if (drop) g *= kf[r], pr[r] = x * kf[r];  // dV from the kept probabilities, scaled; dP masked and scaled
+            if (drop) g *= kpf[r], pr[r] = x * kpf[r];  // dV from the kept probabilities, scaled; dP masked and scaled
           }
           ds[r] = x * (g - d4[e]);
           if constexpr (FUNC) ds[r] *= dfac[r];
         }
       }
-      col_product<D>(dvacc, do_t, col, half, pr);
-      col_product<D>(dkacc, q_t, col, half, ds);
+      col_product<D, DB>(dvacc, do_t + c0, col, half, pr);
+      col_product<D, DB>(dkacc, q_t + c0, col, half, ds);
     }
   }
   if (key < p.S) {
@@ -535,12 +567,12 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
     for (int db = 0; db < DB; ++db)
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
-        const int d = db * 32 + g * 8 + half * 4;
-        if (d < p.d_real) {
+        const int d = c0 + db * 32 + g * 8 + half * 4;
+        if (d < p.d_real)
           *(f32x4*)(gk + d) = f32x4{dkacc[db][g * 4] * p.scale, dkacc[db][g * 4 + 1] * p.scale, dkacc[db][g * 4 + 2] * p.scale,
                                     dkacc[db][g * 4 + 3] * p.scale};
+        if (d < p.dv_real)
           *(f32x4*)(gv + d) = f32x4{dvacc[db][g * 4], dvacc[db][g * 4 + 1], dvacc[db][g * 4 + 2], dvacc[db][g * 4 + 3]};
-        }
       }
   }
 }
@@ -579,7 +611,7 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   *why = "";
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
-  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  if (E < 8 || E > 256 || E % 8 != 0 || Dv < 8 || Dv > E || Dv % 8 != 0) return *why = "head dims are not multiples of 8 up to 256 with D_v <= D_qk", false;
   if ((p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) && (p.bias.data || p.dropout_p > 0.f))
     return *why = "window / sink / score functor together with attn_bias or dropout", false;
   if (p.bias.data && p.k.size[2] > 1 && p.bias.stride[3] != 1) return *why = "attn_bias keys are not unit-stride", false;
@@ -610,7 +642,7 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
   g.kv_lens = p.kv_lens;
-  g.d_real = (int)p.q.size[3];
+  g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   set_score_mask(g, p);
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
   g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
@@ -621,7 +653,20 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   const int waves = pick_waves((int64_t)g.B * g.Hq, g.L);
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
   const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(64 * waves);
-#define LAUNCH(DD, WW, MM) hipLaunchKernelGGL((fwd_f32_kernel<DD, WW, MM>), grid, block, 0, s, g)
+  // (width 256: both tiles in the launch's dynamic LDS)
+#define LAUNCH(DD, WW, MM)                                                                                       \
+  do {                                                                                                           \
+    constexpr int kLds = DD > 128 ? 2 * kTileFloats<DD> * (int)sizeof(float) : 0;                                \
+    if (kLds) {                                                                                                  \
+      static LdsOnce once;                                                                                       \
+      const hipError_t e = reserve_lds(once, (const void*)fwd_f32_kernel<DD, WW, MM>, kLds);                     \
+      if (e != hipSuccess) {                                                                                     \
+        set_error("SDPA: cannot reserve %d bytes of LDS for fwd_f32_kernel: %s", kLds, hipGetErrorString(e));   \
+        return MI355_SDPA_ERR_LAUNCH;                                                                            \
+      }                                                                                                          \
+    }                                                                                                            \
+    hipLaunchKernelGGL((fwd_f32_kernel<DD, WW, MM>), grid, block, kLds, s, g);                                   \
+  } while (0)
 #define LAUNCH_W(DD)                   \
   do {                                 \
     if (mode == 1) LAUNCH(DD, 4, 1);   \
@@ -629,7 +674,8 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
     else LAUNCH(DD, 4, 0);             \
   } while (0)
   if (g.d_real <= 64) LAUNCH_W(64);
-  else LAUNCH_W(128);
+  else if (g.d_real <= 128) LAUNCH_W(128);
+  else LAUNCH_W(256);
 #undef LAUNCH_W
 #undef LAUNCH
   return check_launch("fwd_f32_kernel");
@@ -639,7 +685,7 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   *why = "";
   const int64_t E = p.q.size[3], Dv = p.v.size[3];
   if (p.dtype != MI355_SDPA_F32) return *why = "dtype is not float32", false;
-  if (E != Dv || E < 8 || E > 128 || E % 8 != 0) return *why = "head dim is not a multiple of 8 up to 128", false;
+  if (E < 8 || E > 256 || E % 8 != 0 || Dv < 8 || Dv > E || Dv % 8 != 0) return *why = "head dims are not multiples of 8 up to 256 with D_v <= D_qk", false;
   if ((p.mask.window > 0 || score_mod_of(p.mask).any) && (p.bias.data || p.dropout_p > 0.f))
     return *why = "window or score functor together with attn_bias or dropout", false;
   if (p.grad_bias.data && (!p.bias.data || (p.k.size[2] > 1 && p.grad_bias.stride[3] != 1)))
@@ -687,7 +733,7 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.L = (int)p.q.size[2], g.S = (int)p.k.size[2];
   g.causal = p.is_causal, g.scale = p.scale, g.xcd_map = 0;
   g.kv_lens = p.kv_lens;
-  g.d_real = (int)p.q.size[3];
+  g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];
   set_score_mask(g, p);
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys;
   g.sm = score_mod_of(p.mask);
@@ -698,8 +744,21 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   const int mode = (g.bias != nullptr || g.keep_scale != 0.f) ? 1 : (g.window > 0 || g.sm.any) ? 2 : 0;
   const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
   const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
-  const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw))));
-#define LAUNCH(KK, GRID, DD, WW, MM) hipLaunchKernelGGL((KK<DD, WW, MM>), GRID, dim3(64 * WW), 0, s, g)
+  // (width 256: two workgroups per key block, one per half of the columns of dK / dV)
+  const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw)) * (g.d_real > 128 ? 2 : 1)));
+#define LAUNCH(KK, GRID, DD, WW, MM)                                                                             \
+  do {                                                                                                           \
+    constexpr int kLds = DD > 128 ? 2 * kTileFloats<DD> * (int)sizeof(float) : 0;                                \
+    if (kLds) {                                                                                                  \
+      static LdsOnce once;                                                                                       \
+      const hipError_t e = reserve_lds(once, (const void*)KK<DD, WW, MM>, kLds);                                 \
+      if (e != hipSuccess) {                                                                                     \
+        set_error("SDPA: cannot reserve %d bytes of LDS for " #KK ": %s", kLds, hipGetErrorString(e));          \
+        return MI355_SDPA_ERR_LAUNCH;                                                                            \
+      }                                                                                                          \
+    }                                                                                                            \
+    hipLaunchKernelGGL((KK<DD, WW, MM>), GRID, dim3(64 * WW), kLds, s, g);                                       \
+  } while (0)
 #define LAUNCH_W(KK, GRID, WAVES_, DD)                 \
   do {                                                 \
     if (mode == 1) LAUNCH(KK, GRID, DD, 4, 1);         \
@@ -707,11 +766,13 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
     else LAUNCH(KK, GRID, DD, 4, 0);                   \
   } while (0)
   if (g.d_real <= 64) LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 64);
-  else LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 128);
+  else if (g.d_real <= 128) LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 128);
+  else LAUNCH_W(bwd_f32_dq_kernel, qgrid, qw, 256);
   int rc = check_launch("bwd_f32_dq_kernel");
   if (rc) return rc;
   if (g.d_real <= 64) LAUNCH_W(bwd_f32_dkdv_kernel, kgrid, kw, 64);
-  else LAUNCH_W(bwd_f32_dkdv_kernel, kgrid, kw, 128);
+  else if (g.d_real <= 128) LAUNCH_W(bwd_f32_dkdv_kernel, kgrid, kw, 128);
+  else LAUNCH_W(bwd_f32_dkdv_kernel, kgrid, kw, 256);
 #undef LAUNCH_W
 #undef LAUNCH
   rc = check_launch("bwd_f32_dkdv_kernel");
