@@ -214,6 +214,40 @@ def test_unregister_brings_the_stock_kernels_back(amd, gpu_device, calls):
     assert calls["fwd"] == 2
 
 
+@pytest.mark.parametrize("shape,dtype,causal,with_bias", [
+    ((1, 4, 4, 256, 64), torch.bfloat16, False, False),
+    ((1, 4, 2, 512, 64), torch.float32, True, False),
+    ((1, 4, 4, 256, 256), torch.bfloat16, False, True),
+    ((1, 4, 2, 512, 256), torch.float32, True, False),
+    ((1, 2, 1, 577, 64), torch.bfloat16, False, False),
+])
+def test_reference_accuracy_cases_run_in_the_matrix_op_kernels(amd, gpu_device, monkeypatch, shape, dtype, causal, with_bias):
+    """The five cases of the reference's accuracy test (tests/python_ops/test_scaled_dot_product_attention.py:
+    362-387) through F.scaled_dot_product_attention and autograd, at its tolerances (forward 5e-2 / 1e-2,
+    backward 5e-2 / 5e-2) against the CPU; forced into the MFMA kernels, so that none of them can pass
+    through the generic ones."""
+    from torch_neuronx_amd.python_ops import scaled_dot_product_fused_attention as impl
+    monkeypatch.setattr(impl, "_force_kernel", lambda: amd._lib.KERNEL_MFMA)
+    B, Hq, Hkv, S, D = shape
+    q, k, v = qkv(B, Hq, Hkv, S, S, D, dtype=dtype, seed=S + D)
+    bias = torch.randn(B, Hq, S, S, generator=torch.Generator().manual_seed(1)).to(dtype) if with_bias else None
+    go = (torch.randn(B, Hq, S, D, generator=torch.Generator().manual_seed(2)).clamp(-1, 1) * 0.1).to(dtype)
+    rep = Hq // Hkv
+
+    def run(dev):
+        qd, kd, vd = (t.to(dev).requires_grad_(True) for t in (q, k, v))
+        kk, vv = (kd.repeat_interleave(rep, 1), vd.repeat_interleave(rep, 1)) if dev == "cpu" else (kd, vd)
+        out = F.scaled_dot_product_attention(qd, kk, vv, attn_mask=None if bias is None else bias.to(dev), is_causal=causal,
+                                             enable_gqa=(dev != "cpu" and rep > 1))
+        out.backward(go.to(dev))
+        return out.detach().cpu(), qd.grad.cpu(), kd.grad.cpu(), vd.grad.cpu()
+
+    got, ref = run(gpu_device), run("cpu")
+    torch.testing.assert_close(got[0].float(), ref[0].float(), atol=5e-2, rtol=1e-2)
+    for a, b_ in zip(got[1:], ref[1:]):
+        torch.testing.assert_close(a.float(), b_.float(), atol=5e-2, rtol=5e-2)
+
+
 def test_a_keep_mask_of_one_element_is_a_placeholder(amd, gpu_device):
     """The reference treats a dropout mask of one element as absent (torch_neuronx/_sdpa_math.py:42-45):
     so do the forward and the backward here, whatever the byte says and whatever dropout_p is."""
