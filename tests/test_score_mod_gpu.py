@@ -41,6 +41,8 @@ def _functors(pattern, B, Hq, L, S, seed):
         "window_alibi_cap": dict(is_causal=True, window=64, alibi_slopes=slopes, softcap=3.0),
         # (causal ALiBi walks its key tiles from the diagonal down in the forward: with vectors per key beside it)
         "alibi_key_vectors": dict(is_causal=True, alibi_slopes=slopes, key_bias=bias, key_weight=weight),
+        # (... a head with a slope that is not positive walks upwards)
+        "alibi_signs": dict(is_causal=True, alibi_slopes=slopes * torch.tensor([1.0, -1.0, 0.0, 1.0]).repeat((Hq + 3) // 4)[:Hq]),
         "everything": dict(is_causal=True, alibi_slopes=slopes, softcap=2.5, key_bias=bias, key_weight=weight,
                            sink_logit=torch.randn(B, Hq, 3, generator=g), **docs),
     }[pattern]
@@ -72,7 +74,7 @@ def _check(amd, dev, B, Hq, Hkv, L, S, E, dtype, pattern, seed, force=0, scale=N
 
 
 PATTERNS = ["alibi", "document", "document_unsorted_promise", "causal_document", "head_bias", "head_bias_document",
-            "soft_cap", "weighted", "window_alibi_cap", "alibi_key_vectors", "everything"]
+            "soft_cap", "weighted", "window_alibi_cap", "alibi_key_vectors", "alibi_signs", "everything"]
 
 
 @pytest.mark.parametrize("pattern", PATTERNS)

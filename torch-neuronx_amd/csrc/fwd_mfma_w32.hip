@@ -171,8 +171,9 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   // calls walk their tiles from the diagonal down instead: the first tiles set the reference, and
   // what follows only falls.  Every wavefront then walks all of the workgroup's tiles (the ones above
   // its own diagonal come first and are masked whole: rows without a live key yet, see the check).
+  // (a head whose slope is not positive keeps the upward walk: its bias falls towards the diagonal)
   const bool backwards = SMOD && ma.causal && p.sm.alibi != nullptr && p.window == 0 && n_lead == 0 && skip == 0 &&
-                         !(p.sm.doc_q && p.sm.doc_k);
+                         !(p.sm.doc_q && p.sm.doc_k) && p.sm.alibi[h] > 0.f;
   constexpr bool SPLITS = MASK == 1 || (MASK == 2 && D <= 128);  // the variants that can split their keys
   if constexpr (SPLITS) {
     if (p.split_tiles) {  // this workgroup's share of the key tiles (no window, no skip table then)
