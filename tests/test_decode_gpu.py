@@ -201,6 +201,16 @@ def test_decode_head_dims_64_and_256_long_and_split(amd, gpu_device):
         assert max_abs(a, b) <= 4e-3
 
 
+@pytest.mark.parametrize("D", [64, 128, 256])
+def test_decode_of_one_long_sequence(amd, gpu_device, D):
+    # a single sequence is cut into one piece per wavefront slot: more than a hundred partials per (batch,
+    # kv head), which the merge reads a thread each and eight rows at a time
+    case = _case(1, 8, 2, 1, 20000, torch.tensor([19977], dtype=torch.int32), seed=D + 1, D=D)
+    a, la = _check(amd, gpu_device, case)
+    b, lb = _check(amd, gpu_device, case, num_splits=4)  # ... against a few long pieces
+    assert max_abs(a, b) <= 4e-3 and max_abs(la, lb) <= 1e-3
+
+
 def test_decode_refuses_other_head_dims(amd, gpu_device):
     dev = gpu_device
     q, kq, vq, ks, vs, _ = _case(1, 8, 8, 1, 64, None, seed=1, D=96)

@@ -53,6 +53,7 @@ constexpr float kLn2 = 0.6931471805599453f;
 // wavefronts per SIMD the decode kernel is built for (at head dims up to 128 three or four spill; at 256
 // the two K/V tiles in flight and the output accumulators alone take 190 registers: one)
 constexpr int dec_occ(int D) { return D > 128 ? 1 : 2; }
+constexpr int kMaxSimds = 1024;  // bound on the streaming kernel's grid: wavefronts per SIMD it is built for x this; sizes the workspace
 constexpr float kPScale = 256.f;  // probabilities are stored as e4m3 of 256*p
 
 struct DecP {
@@ -460,6 +461,7 @@ template <typename TQ, int D>
 __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
   constexpr int NW = D / 64;  // wavefronts of the workgroup
   __shared__ float s_red[2][4];
+  __shared__ float w_s[kMaxSimds * 2];  // weights of the partials (at most one per wavefront of the streaming kernel)
   const int row = blockIdx.x % p.R;
   const int hk = (blockIdx.x / p.R) % p.Hkv;
   const int b = blockIdx.x / (p.R * p.Hkv);
@@ -493,6 +495,10 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
       O = fmaf(o[c], w, O);
     }
   } else {
+    // many partials (a long sequence in a small batch: up to one per wavefront of the chip): their
+    // (max, sum) pairs a thread each, the weights left in LDS, and the partial outputs requested eight
+    // at a time - read one after the other, 256 partials were 256 trips to the L2 in a row, and a
+    // single sequence of 32768 keys spent two thirds of its decode step here
     for (int c = d; c < npart; c += D) M = fmaxf(M, p.ws_ml[(slot0 + (int64_t)c * p.R) * 2]);
     M = wave_max(M);
     if ((d & 63) == 0) s_red[0][d >> 6] = M;
@@ -502,7 +508,9 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     for (int w = 1; w < NW; ++w) M = fmaxf(M, s_red[0][w]);
     for (int c = d; c < npart; c += D) {
       const int64_t s = slot0 + (int64_t)c * p.R;
-      L += p.ws_ml[s * 2 + 1] * __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
+      const float w = __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M);
+      w_s[c] = w;
+      L += p.ws_ml[s * 2 + 1] * w;
     }
     L = wave_sum(L);
     if ((d & 63) == 0) s_red[1][d >> 6] = L;
@@ -510,9 +518,14 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     L = s_red[1][0];
 #pragma unroll
     for (int w = 1; w < NW; ++w) L += s_red[1][w];
-    for (int c = 0; c < npart; ++c) {
-      const int64_t s = slot0 + (int64_t)c * p.R;
-      O = fmaf(p.ws_o[s * D + d], __builtin_amdgcn_exp2f(p.ws_ml[s * 2] - M), O);
+    const float* po = p.ws_o + slot0 * D + d;
+    const int64_t stride = (int64_t)p.R * D;
+    for (int c0 = 0; c0 < npart; c0 += 8) {
+      float o[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) o[j] = c0 + j < npart ? po[(c0 + j) * stride] : 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) O = fmaf(o[j], c0 + j < npart ? w_s[c0 + j] : 0.f, O);
     }
   }
   const int rep = p.Hq / p.Hkv;
@@ -523,7 +536,6 @@ __global__ __launch_bounds__(D) void decode_merge_kernel(DecP p) {
     p.lse[((int64_t)b * p.Hq + h) * p.Lq + lq] = L > 0.f ? (M + __builtin_amdgcn_logf(L)) * kLn2 : -INFINITY;
 }
 
-constexpr int kMaxSimds = 1024;  // bound on the streaming kernel's grid: wavefronts per SIMD it is built for x this; sizes the workspace
 constexpr int kMinSteps = 4;     // 128 keys: below this the partial results rival the keys in bytes
 
 int wave_slots(int head_dim) {  // wavefronts of the decode kernel the chip holds at once
@@ -647,7 +659,13 @@ int launch_decode_fp8kv(const mi355_sdpa_decode_params& p, hipStream_t s) {
       (int64_t)(g.S - 1) * p.v.stride[2] + D >= (1ll << 31))
     return set_error("SDPA decode: cache too large for 32-bit step and row offsets"), MI355_SDPA_ERR_UNSUPPORTED;
   g.t_min = min_steps_for(p);
-  g.n_waves = (int)std::min<int64_t>(wave_slots(D), std::max<int64_t>(1, (max_steps + g.t_min - 1) / g.t_min));
+  // (one or a few long sequences do better with one wavefront per SIMD and longer pieces than with two
+  // and half the keys each: every (batch, kv head) is then cut into a hundred pieces and more, and what a
+  // wavefront costs beyond its keys, and the partials to merge, weigh more than the second wavefront
+  // hides.  8 kv heads, B=1: S=32768 35 -> 26 us, S=131072 64 -> 54; with more sequences, or more keys
+  // in all, the other way round)
+  const int slots_now = ((int64_t)g.B * g.Hkv <= 32 && max_steps <= 40 * 1024) ? std::min(wave_slots(D), kMaxSimds) : wave_slots(D);
+  g.n_waves = (int)std::min<int64_t>(slots_now, std::max<int64_t>(1, (max_steps + g.t_min - 1) / g.t_min));
   const int64_t qes = p.q_dtype == MI355_SDPA_F32 ? 4 : 2;
   if (((uintptr_t)p.q.data & 15) || (p.q.stride[0] * qes) % 16 || (p.q.stride[1] * qes) % 16 || (p.q.stride[2] * qes) % 16)
     return set_error("SDPA decode: query rows must be 16-byte aligned"), MI355_SDPA_ERR_UNSUPPORTED;
