@@ -382,6 +382,24 @@ def extra_decode_bf16(amd, dev):
     return r
 
 
+def extra_decode_fp8_one_sequence(amd, dev):
+    """The fp8-cache decode entry point on one long sequence (interactive serving): Hq=32 Hkv=8 D=128 L=1,
+    B=1 at 32768 and 131072 keys - every (batch, kv head) is cut into a hundred pieces and more."""
+    Hq, Hkv, D = 32, 8, 128
+    r = {}
+    for name, B, S in (("B1_S32768", 1, 32768), ("B1_S131072", 1, 131072)):
+        g = torch.Generator(device=dev).manual_seed(1017)
+        q = torch.randn((B, Hq, 1, D), generator=g, device=dev, dtype=torch.bfloat16)
+        kq, vq = (torch.randn((B, Hkv, S, D), generator=g, device=dev).to(torch.float8_e4m3fn) for _ in range(2))
+        sc = torch.ones(B, Hkv, device=dev)
+        amd.decode_fp8kv(q, kq, vq, sc, sc, None)
+        _, ev = event_time_ms(lambda: amd.decode_fp8kv(q, kq, vq, sc, sc, None), 30, 5)
+        r[name] = {"ms": ev, "kv_GB/s": 2.0 * B * Hkv * S * D / (ev * 1e-3) / 1e9}
+        del q, kq, vq
+    r["shape"] = "Hq=32 Hkv=8 D=128 L=1 fp8 e4m3 cache"
+    return r
+
+
 def extra_few_kv_heads(amd, dev):
     """Backward with few key blocks, where the dK/dV kernel deals a block's query tiles to several
     workgroups: one kv head for 32 query heads (B=2 S=4096) and a 32/8 model at batch 1 (S=2048), D=128 causal."""
@@ -564,6 +582,7 @@ def main():
                          ("alibi_causal_fwd_bwd", extra_alibi), ("document_ids_fwd_bwd", extra_document_ids),
                          ("head_dim_256_fwd_bwd", extra_wide), ("head_dim_256_window_softcap_fwd_bwd", extra_wide_window_softcap),
                          ("fresh_bool_mask_fwd", extra_fresh_bool_mask), ("dropout_padding_fwd_bwd", extra_dropout), ("decode_bf16_cache_fwd", extra_decode_bf16),
+                         ("decode_fp8_one_sequence", extra_decode_fp8_one_sequence),
                          ("few_kv_heads_fwd_bwd", extra_few_kv_heads), ("float32_fwd_bwd", extra_f32)):
             try:
                 extras[name] = fn(amd, dev)
