@@ -357,6 +357,35 @@ def test_dropout_with_a_relative_position_bias_through_the_operator(amd, gpu_dev
         assert max_abs(a, b_) <= 1e-2
 
 
+@pytest.mark.parametrize("D,dtype", [(256, torch.bfloat16), (192, torch.float16), (256, torch.float32)])
+def test_dropout_at_wide_head_dims_through_the_operator(amd, gpu_device, monkeypatch, D, dtype):
+    """dropout_p = 0.1 at head dims above 128 through the registered operators, causal: the keep-mask that the
+    forward drew goes to the wide kernels (forced: the calls would fail otherwise), and forward and backward
+    agree with the oracle given that mask."""
+    from torch_neuronx_amd.python_ops import scaled_dot_product_fused_attention as impl
+    monkeypatch.setattr(impl, "_force_kernel", lambda: amd._lib.KERNEL_MFMA)
+    B, H, S = 2, 4, 260
+    dev = gpu_device
+    g = torch.Generator().manual_seed(D)
+    q, k, v, go = (torch.randn(B, H, S, D, generator=g).to(dtype).to(dev) for _ in range(4))
+    go = (go.float() * 0.1).to(dtype)
+    torch.manual_seed(17)
+    op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    opb = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    r = op(q, k, v, None, 0.1, True)
+    keep = r[6]
+    assert keep.shape == (B, H, S, S)
+    dq, dk, dv, _ = opb(go, q, k, v, None, [True, True, True, False], r[0], r[1], None, None, S, S, 0.1, True, keep, r[7])
+    qc, kc, vc, gc = (t.float().cpu() for t in (q, k, v, go))
+    ro, rl = om.compute_attention(qc, kc, vc, None, keep.cpu().bool(), D**-0.5, True, 0.1)
+    rdq, rdk, rdv, _ = om.compute_attention_backward(gc, qc, kc, vc, None, keep.cpu().bool(), ro, rl, D**-0.5, True, 0.1)
+    half = dtype is not torch.float32
+    assert max_abs(r[0], ro) <= (2e-2 if half else 2e-5) and max_abs(r[1], rl) <= (2e-3 if half else 2e-5)
+    for a, b_ in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert max_abs(a, b_) <= (1e-2 if half else 3e-5)
+    assert 0.88 < keep.float().mean().item() < 0.92
+
+
 def test_backward_kv_lens(amd, gpu_device):
     q, k, v, go = qkv(3, 4, 2, 5, 64, 32, dtype=torch.float32, seed=4, with_do=True)
     lens = torch.tensor([64, 1, 17], dtype=torch.int32)
