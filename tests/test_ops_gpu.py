@@ -423,6 +423,94 @@ def test_traced_module_reaches_the_library(amd, gpu_device, calls):
         assert torch.equal(t.grad, e)
 
 
+@pytest.mark.parametrize("case", ["causal_gqa", "padding_mask", "bias_with_gradient", "float32"])
+def test_compiled_module_with_the_default_backend(amd, gpu_device, calls, case):
+    """torch.compile's default backend calls the attention operators as they are and asserts, in the code it
+    generates, that their outputs have the sizes and strides upstream's operators promise (output laid out
+    like the query for the flash operator and (B,L,H,Dv) for the memory-efficient one, 0-dim int64 seed and
+    offset, gradients (B,L,H,D), the bias gradient a view of rows padded to 16 keys).  The replacements
+    registered here keep those promises: the compiled block runs and gives the eager numbers."""
+    dev = gpu_device
+    g = torch.Generator().manual_seed(31)
+    mk = lambda *shape, dtype=torch.bfloat16: torch.randn(*shape, generator=g).to(dtype).to(dev).requires_grad_(True)
+    if case == "causal_gqa":
+        args = (mk(2, 8, 256, 64), mk(2, 2, 256, 64), mk(2, 2, 256, 64))
+        block = lambda q, k, v: (F.scaled_dot_product_attention(q * 1.0, k, v, is_causal=True, enable_gqa=True).float() * 2).square().sum()
+    elif case == "padding_mask":
+        args = (mk(2, 4, 128, 64), mk(2, 4, 128, 64), mk(2, 4, 128, 64))
+        pad = torch.ones(2, 1, 1, 128, dtype=torch.bool, device=dev)
+        pad[1, ..., 100:] = False
+        block = lambda q, k, v: F.scaled_dot_product_attention(q, k, v, attn_mask=pad).float().square().sum()
+    elif case == "bias_with_gradient":
+        args = (mk(2, 4, 128, 64), mk(2, 4, 128, 64), mk(2, 4, 128, 64), mk(1, 4, 128, 120))
+        block = lambda q, k, v, b: F.scaled_dot_product_attention(q, k[:, :, :120], v[:, :, :120], attn_mask=b).float().square().sum()
+    else:
+        args = (mk(2, 4, 128, 64, dtype=torch.float32),)
+        block = lambda q: F.scaled_dot_product_attention(q, q, q, is_causal=True).square().sum()
+    ref = block(*args)
+    ref.backward()
+    eager = [t.grad.clone() for t in args]
+    for t in args:
+        t.grad = None
+    before = dict(calls)
+    torch._dynamo.reset()
+    got = torch.compile(block)(*args)
+    got.backward()
+    assert calls["fwd"] > before["fwd"] and calls["bwd"] > before["bwd"], calls
+    assert torch.allclose(got, ref, rtol=1e-5)
+    for t, e in zip(args, eager):
+        assert max_abs(t.grad, e) <= 1e-6 * max(1.0, float(e.abs().max()))
+    torch._dynamo.reset()
+
+
+def test_replaced_upstream_operators_keep_upstream_layouts_and_redraw_the_dropout_mask(amd, gpu_device):
+    """The flash and memory-efficient operators called directly with dropout: outputs in upstream's shapes
+    and layouts; seed and offset are the generator's state before the draw, the backward draws the same
+    keep-mask from them (the mask does not travel), and forward and backward agree with the oracle given
+    that mask."""
+    from oracle import sdpa_math as om
+    from torch_neuronx_amd.python_ops import scaled_dot_product_fused_attention as impl
+
+    dev = gpu_device
+    B, H, L, S, D, p = 2, 4, 128, 120, 64, 0.2
+    g = torch.Generator().manual_seed(77)
+    mk = lambda *shape: torch.randn(*shape, generator=g).to(torch.bfloat16).to(dev)
+    q, k, v, go, bias = mk(B, H, L, D), mk(B, H, S, D), mk(B, H, S, D), mk(B, H, L, D), mk(B, H, L, S)
+    qc, kc, vc, gc, bc = (t.float().cpu() for t in (q, k, v, go, bias))
+    torch.cuda.manual_seed(5)
+    r = torch.ops.aten._scaled_dot_product_efficient_attention(q, k, v, bias, True, p, False)
+    out, lse, seed, offset = r
+    assert out.shape == (B, H, L, D) and out.stride() == (L * H * D, D, H * D, 1)
+    assert lse.shape == (B, H, L) and lse.dtype == torch.float32
+    for t in (seed, offset):
+        assert t.dim() == 0 and t.dtype == torch.int64 and t.device.type == "cpu"
+    assert int(seed) == 5
+    keep = impl._keep_again(q, S, p, seed, offset).cpu().bool()
+    assert 0.75 < keep.float().mean().item() < 0.85
+    ro, rl = om.compute_attention(qc, kc, vc, bc, keep, D**-0.5, False, p)
+    assert max_abs(out, ro) <= 2e-2 and max_abs(lse, rl) <= 2e-3
+    dq, dk, dv, db = torch.ops.aten._scaled_dot_product_efficient_attention_backward(
+        go, q, k, v, bias, out, lse, seed, offset, p, [True, True, True, True])
+    for t, n in ((dq, L), (dk, S), (dv, S)):
+        assert t.stride() == (n * H * D, D, H * D, 1)
+    assert db.shape == (B, H, L, S) and db.stride() == (H * L * 128, L * 128, 128, 1)
+    rdq, rdk, rdv, rdb = om.compute_attention_backward(gc, qc, kc, vc, bc, keep, ro, rl, D**-0.5, False, p)
+    for a, b_ in ((dq, rdq), (dk, rdk), (dv, rdv), (db, rdb)):
+        assert max_abs(a, b_) <= 5e-2 * max(1.0, float(b_.abs().max()))
+    # the next call draws at a later offset, hence another mask
+    r2 = torch.ops.aten._scaled_dot_product_flash_attention(q, k, v, p, False)
+    assert int(r2[6]) == 5 and int(r2[7]) > int(offset)
+    assert r2[6].dim() == 0 and r2[7].dim() == 0 and r2[8].numel() == 0
+    keep2 = impl._keep_again(q, S, p, r2[6], r2[7]).cpu().bool()
+    assert not torch.equal(keep2, keep)
+    ro2, rl2 = om.compute_attention(qc, kc, vc, None, keep2, D**-0.5, False, p)
+    assert max_abs(r2[0], ro2) <= 2e-2
+    g3 = torch.ops.aten._scaled_dot_product_flash_attention_backward(go, q, k, v, r2[0], r2[1], None, None, L, S, p, False, r2[6], r2[7])
+    r3 = om.compute_attention_backward(gc, qc, kc, vc, None, keep2, ro2, rl2, D**-0.5, False, p)
+    for a, b_ in zip(g3, r3[:3]):
+        assert max_abs(a, b_) <= 5e-2 * max(1.0, float(b_.abs().max()))
+
+
 def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):
     # The library only launches kernels on the stream it is given (no allocation, no memset, no
     # synchronisation), so forward, backward and decode can be recorded into one graph.  The graph

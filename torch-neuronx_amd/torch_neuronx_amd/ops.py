@@ -242,7 +242,8 @@ def _score_mods(kw):
 
 def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None, dropout_p=0.0,
                  dropout_keep=None, kv_lens=None, need_lse=True, force_kernel=0,
-                 window=None, sink_keys=0, sink_logit=None, live_tiles=None, mask_verdict=None, **score_mods):
+                 window=None, sink_keys=0, sink_logit=None, live_tiles=None, mask_verdict=None,
+                 seq_major_out=False, **score_mods):
     """Fused forward.  K/V arrive at ``Hkv`` heads.  Returns ``(out, lse)``; ``out`` keeps the
     dimension order of ``query`` and ``lse`` is contiguous float32 ``(B,Hq,L)``.
 
@@ -260,7 +261,10 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     ``slope[h] * (j - i)``, ``softcap`` turns ``s`` into ``softcap * tanh(s / softcap)``;
     ``doc_ids_q`` ``(B,L)`` / ``doc_ids_k`` ``(B,S)`` keep a score iff the two ids are equal
     (``doc_ids_sorted=True``: the caller's promise that both are non-decreasing along the sequence,
-    which lets the kernels skip the key tiles of other documents)."""
+    which lets the kernels skip the key tiles of other documents).
+
+    ``seq_major_out``: ``out`` is laid out ``(B,L,Hq,Dv)`` in memory whatever the query's layout, which
+    is what upstream's memory-efficient operator promises its callers."""
     score_mods = _score_mods(score_mods)
     for t, n in ((query, "query"), (key, "key"), (value, "value")):
         _require_cuda(t, n)
@@ -269,9 +273,12 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     if scale is None:
         scale = 1.0 / math.sqrt(E)
     q, k, v = _unit_last(query), _unit_last(key), _unit_last(value)
-    out = empty_like_layout(query, (B, Hq, L, Dv))
-    if out.stride(-1) != 1 and Dv > 1:
-        out = torch.empty((B, Hq, L, Dv), dtype=query.dtype, device=query.device)
+    if seq_major_out:
+        out = torch.empty((B, L, Hq, Dv), dtype=query.dtype, device=query.device).transpose(1, 2)
+    else:
+        out = empty_like_layout(query, (B, Hq, L, Dv))
+        if out.stride(-1) != 1 and Dv > 1:
+            out = torch.empty((B, Hq, L, Dv), dtype=query.dtype, device=query.device)
     lse = torch.empty((B, Hq, L), dtype=torch.float32, device=query.device) if need_lse else None
     bias, bias_dt = _bias_view(attn_bias, B, Hq, L, S, repack_for=None if force_kernel == _lib.KERNEL_GENERIC else query.dtype)
     p, P = _lib.FwdParams(), _lib.FwdParams
@@ -316,12 +323,16 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
 def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_causal=False,
                   scale=None, dropout_p=0.0, dropout_keep=None, kv_lens=None,
                   want_grad_bias=False, force_kernel=0, window=None, sink_keys=0, sink_logit=None,
-                  live_tiles=None, mask_verdict=None, **score_mods):
+                  live_tiles=None, mask_verdict=None, seq_major_grads=False, grad_bias_row_pad=4, **score_mods):
     """Fused backward.  Returns ``(dq, dk, dv, dbias-or-None)``; each gradient keeps the
     dimension order of its input, dk/dv come back at ``Hkv`` heads.  With a ``sink_logit`` a
     fifth element follows: its gradient, float32 ``(B,Hq)`` or ``(B,Hq,n)``.  Score functors as in
     ``sdpa_forward``: their derivative multiplies the gradient of the scores; the captured vectors
-    get no gradient of their own."""
+    get no gradient of their own.
+
+    ``seq_major_grads``: dq, dk and dv are laid out ``(B,L,H,D)`` in memory whatever the inputs' layouts,
+    and ``grad_bias_row_pad = 16`` leaves the bias gradient as a view of rows padded to 16 keys: the
+    layouts upstream's memory-efficient backward promises its callers."""
     score_mods = _score_mods(score_mods)
     for t, n in ((grad_out, "grad_out"), (query, "query"), (key, "key"), (value, "value")):
         _require_cuda(t, n)
@@ -333,6 +344,8 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     lse = lse.to(torch.float32).contiguous()
 
     def grad_like(ref, shape):
+        if seq_major_grads:
+            return torch.empty((shape[0], shape[2], shape[1], shape[3]), dtype=ref.dtype, device=ref.device).transpose(1, 2)
         g = empty_like_layout(ref, shape)
         if g.stride(-1) != 1 and shape[-1] > 1:
             g = torch.empty(shape, dtype=ref.dtype, device=ref.device)
@@ -343,7 +356,7 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     dbias = None
     if want_grad_bias and bias is not None:
         # (the matrix-op kernels for 16-bit inputs write the gradient four keys at a time: rows padded to that)
-        S4 = S if query.dtype == torch.float32 or L == 1 else (S + 3) // 4 * 4
+        S4 = S if (query.dtype == torch.float32 or L == 1) and grad_bias_row_pad <= 4 else -(-S // grad_bias_row_pad) * grad_bias_row_pad
         dbias = torch.empty((B, Hq, L, S4), dtype=query.dtype, device=query.device)[..., :S]
     p, P = _lib.BwdParams(), _lib.BwdParams
     for f, t in ((P.grad_out, go), (P.q, q), (P.k, k), (P.v, v), (P.out, o), (P.grad_q, dq), (P.grad_k, dk),
@@ -383,7 +396,7 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
     with _lib.on_device(query.device):
         rc = lib.mi355_sdpa_bwd(C.byref(p), _lib.current_stream(query.device))
     _lib.check(rc)
-    if dbias is not None and dbias.stride(2) != S and L > 1:
+    if dbias is not None and dbias.stride(2) != S and L > 1 and grad_bias_row_pad <= 4:
         dbias = dbias.contiguous()  # (rows were padded for the kernel)
     if _z is not None:
         return dq, dk, dv, dbias, dsink

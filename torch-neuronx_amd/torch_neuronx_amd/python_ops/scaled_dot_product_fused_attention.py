@@ -73,6 +73,44 @@ def _dropout_keep(query, S, dropout_p):
     return torch.empty((B, H, L, S), dtype=torch.uint8, device=query.device).bernoulli_(1.0 - dropout_p)
 
 
+_scalar_rng_pair = None
+
+
+def _scalar_rng():
+    """What upstream's flash and memory-efficient operators return for seed and offset on ROCm: 0-dim
+    int64 host tensors (torch/_meta_registrations.py, "Note [Seed and Offset]"); zeros when no dropout
+    is applied."""
+    global _scalar_rng_pair
+    if _scalar_rng_pair is None:
+        _scalar_rng_pair = (torch.zeros((), dtype=torch.int64), torch.zeros((), dtype=torch.int64))
+    return _scalar_rng_pair
+
+
+def _seeded_keep(query, S, dropout_p):
+    """Keep-mask from the device's default generator together with the (seed, offset) it was drawn at,
+    as 0-dim int64 host tensors: the backward draws the same mask again from the pair, so the mask
+    itself (``B*H*L*S`` bytes) does not have to stay alive between the two, and the operator's outputs
+    have the shapes upstream's operators promise (a compiled graph checks them)."""
+    index = query.device.index if query.device.index is not None else torch.cuda.current_device()
+    gen = torch.cuda.default_generators[index]
+    seed, offset = gen.initial_seed(), gen.get_offset()
+    keep = _dropout_keep(query, S, dropout_p)
+    if seed >= 1 << 63:
+        seed -= 1 << 64  # (a 64-bit seed in an int64 tensor)
+    return keep, torch.tensor(seed, dtype=torch.int64), torch.tensor(offset, dtype=torch.int64)
+
+
+def _keep_again(query, S, dropout_p, philox_seed, philox_offset):
+    """The mask ``_seeded_keep`` drew at ``(philox_seed, philox_offset)``."""
+    B, H, L, _ = query.shape
+    if dropout_p >= 1.0:
+        return torch.zeros((B, H, L, S), dtype=torch.uint8, device=query.device)
+    gen = torch.Generator(device=query.device)
+    gen.manual_seed(int(philox_seed) % (1 << 64))
+    gen.set_offset(int(philox_offset))
+    return torch.empty((B, H, L, S), dtype=torch.uint8, device=query.device).bernoulli_(1.0 - dropout_p, generator=gen)
+
+
 def _present(attn_bias):
     """An empty bias is a lowering placeholder and counts as absent (torch_neuronx/_sdpa_math.py:30)."""
     return None if attn_bias is None or attn_bias.numel() == 0 else attn_bias
@@ -118,7 +156,12 @@ def _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key):
     return functor
 
 
-def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale, need_lse=True):
+def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_mask, scale, need_lse=True,
+             upstream=None):
+    """``upstream``: None for the reference's operator (outputs in the query's layout, the keep-mask in
+    the seed slot); "flash" / "efficient" for the two upstream operators this package replaces, whose
+    callers - a compiled graph asserts it - expect upstream's output shapes and layouts: seed and offset
+    0-dim int64, and for "efficient" the output laid out ``(B,L,H,Dv)`` in memory."""
     _check_device(query)
     attn_bias = _present(attn_bias)
     if return_debug_mask:
@@ -132,15 +175,18 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
     S = key.shape[2]
     keep = None
     if dropout_p > 0.0:
-        keep = _dropout_keep(query, S, dropout_p)
-        seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
+        if upstream is not None and not torch.cuda.is_current_stream_capturing():
+            keep, seed, offset = _seeded_keep(query, S, dropout_p)
+        else:  # (under capture a seed read on the host would be frozen into the graph: the mask travels)
+            keep = _dropout_keep(query, S, dropout_p)
+            seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
     else:
-        seed, offset = _empty_rng(query.device)
+        seed, offset = _empty_rng(query.device) if upstream is None else _scalar_rng()
     attn_bias, is_causal, functor = _recover_pattern(attn_bias, is_causal, query, key, dropout_p=dropout_p)
     functor = _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key)
     out, lse = ops.sdpa_forward(query, key, value, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
                                 dropout_p=dropout_p, dropout_keep=keep, need_lse=need_lse,
-                                force_kernel=_force_kernel(), **functor)
+                                force_kernel=_force_kernel(), seq_major_out=upstream == "efficient", **functor)
     if orig_dtype == torch.float64:
         out = out.to(orig_dtype)
     return out, lse, seed, offset
@@ -157,7 +203,7 @@ def scaled_dot_product_fused_attention_overrideable(
 
 
 def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p, is_causal, philox_seed,
-              scale, want_grad_bias):
+              scale, want_grad_bias, philox_offset=None, upstream=None):
     _check_device(query)
     attn_bias = _present(attn_bias)
     orig_dtype = query.dtype
@@ -169,7 +215,9 @@ def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p,
         grad_out = grad_out.to(query.dtype)
     keep = None
     if dropout_p > 0.0:
-        if philox_seed is None or philox_seed.numel() <= 1:
+        if upstream is not None and philox_seed is not None and philox_seed.dim() == 0:
+            keep = _keep_again(query, key.shape[2], dropout_p, philox_seed, philox_offset)
+        elif philox_seed is None or philox_seed.numel() <= 1:
             dropout_p = 0.0  # a placeholder carries no mask: treated as absent (_sdpa_math.py:42-45)
         else:
             keep = philox_seed
@@ -178,7 +226,7 @@ def _backward(grad_out, query, key, value, attn_bias, out, logsumexp, dropout_p,
     dq, dk, dv, dbias = ops.sdpa_backward(
         grad_out, query, key, value, out, logsumexp, attn_bias=attn_bias, is_causal=is_causal, scale=scale,
         dropout_p=dropout_p, dropout_keep=keep, want_grad_bias=want_grad_bias, force_kernel=_force_kernel(),
-        **functor)
+        seq_major_grads=upstream == "efficient", grad_bias_row_pad=16 if upstream == "efficient" else 4, **functor)
     if orig_dtype == torch.float64:
         dq, dk, dv = dq.to(orig_dtype), dk.to(orig_dtype), dv.to(orig_dtype)
         dbias = dbias.to(orig_dtype) if dbias is not None else None
@@ -199,9 +247,12 @@ def scaled_dot_product_fused_attention_overrideable_backward(
 def scaled_dot_product_flash_attention(
     query, key, value, dropout_p=0.0, is_causal=False, return_debug_mask=False, scale=None
 ):
-    """``aten::_scaled_dot_product_flash_attention``: same 9-tuple, no bias argument."""
-    out, lse, seed, offset = _forward(query, key, value, None, dropout_p, is_causal, return_debug_mask, scale)
-    return out, lse, None, None, query.shape[2], key.shape[2], seed, offset, None
+    """``aten::_scaled_dot_product_flash_attention``: same 9-tuple, no bias argument; seed, offset and
+    the (empty) debug mask as upstream's operator returns them."""
+    out, lse, seed, offset = _forward(query, key, value, None, dropout_p, is_causal, return_debug_mask, scale,
+                                      upstream="flash")
+    return (out, lse, None, None, query.shape[2], key.shape[2], seed, offset,
+            torch.empty((0,), dtype=query.dtype, device=query.device))
 
 
 def scaled_dot_product_flash_attention_backward(
@@ -210,15 +261,17 @@ def scaled_dot_product_flash_attention_backward(
 ):
     """``aten::_scaled_dot_product_flash_attention_backward``: ``(dq, dk, dv)``."""
     return _backward(grad_out, query, key, value, None, out, logsumexp, dropout_p, is_causal,
-                     philox_seed, scale, False)[:3]
+                     philox_seed, scale, False, philox_offset, "flash")[:3]
 
 
 def scaled_dot_product_efficient_attention(
     query, key, value, attn_bias, compute_log_sumexp, dropout_p=0.0, is_causal=False, scale=None
 ):
     """``aten::_scaled_dot_product_efficient_attention``: ``(output, log_sumexp, philox_seed,
-    philox_offset)``; the bias-capable route ATen takes when a mask is present."""
-    out, lse, seed, offset = _forward(query, key, value, attn_bias, dropout_p, is_causal, False, scale)
+    philox_offset)``; the bias-capable route ATen takes when a mask is present.  The output is laid out
+    ``(B,L,H,Dv)`` in memory, as upstream's."""
+    out, lse, seed, offset = _forward(query, key, value, attn_bias, dropout_p, is_causal, False, scale,
+                                      upstream="efficient")
     if not compute_log_sumexp:
         lse = torch.empty((query.shape[0], query.shape[1], 0), dtype=torch.float32, device=query.device)
     return out, lse, seed, offset
@@ -231,7 +284,7 @@ def scaled_dot_product_efficient_attention_backward(
     """``aten::_scaled_dot_product_efficient_attention_backward``: ``(dq, dk, dv, dbias)``."""
     want = _wants_grad_bias(attn_bias, grad_input_mask)
     dq, dk, dv, dbias = _backward(grad_out_, query, key, value, attn_bias, out, logsumexp, dropout_p,
-                                  is_causal, philox_seed, scale, want)
+                                  is_causal, philox_seed, scale, want, philox_offset, "efficient")
     if dbias is None:
         dbias = torch.empty((0,), dtype=query.dtype, device=query.device)
     return dq, dk, dv, dbias
