@@ -1,0 +1,160 @@
+"""Whole models on the drop-in path: small random-init ``transformers`` models with
+``attn_implementation="sdpa"`` run one training step (loss and every parameter gradient) and a greedy
+generation with the stock attention kernels of this PyTorch build and again with this package
+registered.  The models reach the operators the way real callers do: ``is_causal`` without a mask,
+additive padding + causal masks built by the model code, sliding-window masks, grouped heads with
+``enable_gqa``, head dim 256, bidirectional padding masks, 197-token images.  Not a parity test against
+the oracle (those are the kernel and operator tests): it checks that nothing between the model code and
+the kernels - mask recognition, layouts, autograd, the KV-cache decode steps - changes the numbers.
+"""
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+transformers = pytest.importorskip("transformers")
+
+
+@pytest.fixture(scope="module")
+def amd(gpu_device):
+    import torch_neuronx_amd as amd
+
+    return amd
+
+
+def _llama(**kw):
+    cfg = dict(vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=2,
+               num_attention_heads=8, num_key_value_heads=2, attn_implementation="sdpa")
+    cfg.update(kw)
+    return transformers.LlamaForCausalLM(transformers.LlamaConfig(**cfg))
+
+
+def _mistral():
+    return transformers.MistralForCausalLM(transformers.MistralConfig(
+        vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=8,
+        num_key_value_heads=2, sliding_window=64, attn_implementation="sdpa"))
+
+
+def _gemma2():
+    return transformers.Gemma2ForCausalLM(transformers.Gemma2Config(
+        vocab_size=1000, hidden_size=512, intermediate_size=1024, num_hidden_layers=2, num_attention_heads=4,
+        num_key_value_heads=2, head_dim=256, sliding_window=64, attn_implementation="sdpa"))
+
+
+def _gpt2():
+    return transformers.GPT2LMHeadModel(transformers.GPT2Config(
+        vocab_size=1000, n_embd=384, n_layer=2, n_head=6, n_positions=512, attn_pdrop=0.0, resid_pdrop=0.0,
+        embd_pdrop=0.0, bos_token_id=0, eos_token_id=0, attn_implementation="sdpa"))
+
+
+def _bert():
+    return transformers.BertForMaskedLM(transformers.BertConfig(
+        vocab_size=1000, hidden_size=384, num_hidden_layers=2, num_attention_heads=6, intermediate_size=768,
+        hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, attn_implementation="sdpa"))
+
+
+def _vit():
+    return transformers.ViTModel(transformers.ViTConfig(
+        hidden_size=384, num_hidden_layers=2, num_attention_heads=6, intermediate_size=768,
+        hidden_dropout_prob=0.0, attention_probs_dropout_prob=0.0, attn_implementation="sdpa"))
+
+
+CASES = {
+    "llama_gqa_no_mask": (_llama, False, torch.bfloat16),
+    "llama_gqa_padding": (_llama, True, torch.bfloat16),
+    "llama_gqa_padding_float32": (_llama, True, torch.float32),
+    "mistral_sliding_window": (_mistral, True, torch.bfloat16),
+    "gemma2_head_dim_256": (_gemma2, True, torch.bfloat16),
+    "gpt2_float32": (_gpt2, True, torch.float32),
+    "bert_padding": (_bert, True, torch.bfloat16),
+    "bert_padding_float32": (_bert, True, torch.float32),
+    "vit_197_tokens": (_vit, None, torch.bfloat16),
+}
+
+
+def _step(model, inputs):
+    model.zero_grad()
+    out = model(**inputs)
+    loss = out.loss if getattr(out, "loss", None) is not None else out[0].float().square().mean()
+    loss.backward()
+    return loss.detach().float(), torch.cat([p.grad.float().flatten() for p in model.parameters() if p.grad is not None])
+
+
+@pytest.fixture
+def library_calls(amd, monkeypatch):
+    seen = {"fwd": 0, "bwd": 0}
+    f0, b0 = amd.ops.sdpa_forward, amd.ops.sdpa_backward
+
+    def f(*a, **k):
+        seen["fwd"] += 1
+        return f0(*a, **k)
+
+    def b(*a, **k):
+        seen["bwd"] += 1
+        return b0(*a, **k)
+
+    monkeypatch.setattr(amd.ops, "sdpa_forward", f)
+    monkeypatch.setattr(amd.ops, "sdpa_backward", b)
+    return seen
+
+
+@pytest.mark.parametrize("name", list(CASES))
+def test_training_step_of_a_model_matches_the_stock_kernels(amd, gpu_device, library_calls, name):
+    make, padded, dtype = CASES[name]
+    dev = gpu_device
+    torch.manual_seed(1)
+    model = make().to(dev).to(dtype).train()
+    B, S = 4, 256
+    if padded is None:
+        inputs = dict(pixel_values=torch.randn(B, 3, 224, 224, device=dev, dtype=dtype))
+    else:
+        ids = torch.randint(1, 1000, (B, S), device=dev)
+        inputs = dict(input_ids=ids, labels=ids)
+        if padded:
+            am = torch.ones(B, S, dtype=torch.long, device=dev)
+            am[1, 200:] = 0
+            am[3, 100:] = 0
+            inputs["attention_mask"] = am
+    try:
+        amd.unregister()
+        l0, g0 = _step(model, inputs)
+        assert library_calls == {"fwd": 0, "bwd": 0}
+    finally:
+        amd.register()
+    l1, g1 = _step(model, inputs)
+    assert library_calls["fwd"] == 2 and library_calls["bwd"] == 2, library_calls  # (one call per layer)
+    rel = float((g1 - g0).norm() / g0.norm())
+    if dtype is torch.float32:
+        assert abs(float(l1 - l0)) <= 1e-5 and rel <= 1e-5, (float(l0), float(l1), rel)
+    else:  # two bf16 implementations: each rounds the output and the gradients once per layer
+        assert abs(float(l1 - l0)) <= 2e-3 and rel <= 2e-2, (float(l0), float(l1), rel)
+
+
+@pytest.mark.parametrize("left_padding", [False, True])
+def test_greedy_generation_with_a_kv_cache_matches_the_stock_kernels(amd, gpu_device, library_calls, left_padding):
+    """Prefill, then 24 decode steps of one query row against the growing cache; float32 with grouped
+    heads, which upstream's backend choice sends to its unfused path - routed to the library by
+    ``route_functional``, the reference's backend choice.  The tokens are the stock ones."""
+    dev = gpu_device
+    torch.manual_seed(1)
+    model = _llama().to(dev).eval()
+    ids = torch.randint(1, 1000, (4, 32), device=dev)
+    am = torch.ones_like(ids)
+    if left_padding:
+        am[1, :7] = 0
+        am[2, :20] = 0
+    try:
+        amd.unregister()
+        with torch.no_grad():
+            want = model.generate(ids, attention_mask=am, max_new_tokens=24, do_sample=False)
+    finally:
+        amd.register()
+    amd.route_functional(True)
+    try:
+        with torch.no_grad():
+            got = model.generate(ids, attention_mask=am, max_new_tokens=24, do_sample=False)
+    finally:
+        amd.route_functional(False)
+    assert library_calls["fwd"] == 48, library_calls
+    assert torch.equal(got, want)

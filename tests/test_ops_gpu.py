@@ -463,6 +463,38 @@ def test_compiled_module_with_the_default_backend(amd, gpu_device, calls, case):
     torch._dynamo.reset()
 
 
+def test_functional_call_routed_by_the_reference_rules(amd, gpu_device, calls):
+    """float32 with grouped heads: upstream's compiled-in backend choice for GPUs has no fused kernel for
+    it and takes the unfused path (no call reaches the library); with ``route_functional`` the choice is
+    the reference's (SdpBackendSelection.cpp:14-68: the fused operator for every plain 4-D call), forward
+    and backward run in the library and agree with the oracle; switching it off restores the stock function."""
+    stock = F.scaled_dot_product_attention
+    q, k, v, go = qkv(2, 8, 2, 200, 200, 64, dtype=torch.float32, seed=3, with_do=True)
+    qd, kd, vd = (t.to(gpu_device).requires_grad_(True) for t in (q, k, v))
+    before = dict(calls)
+    F.scaled_dot_product_attention(qd, kd, vd, is_causal=True, enable_gqa=True)
+    assert calls == before
+    amd.route_functional(True)
+    try:
+        assert F.scaled_dot_product_attention is not stock
+        out = F.scaled_dot_product_attention(qd, kd, vd, is_causal=True, enable_gqa=True)
+        out.backward(go.to(gpu_device))
+        assert calls["fwd"] == before["fwd"] + 1 and calls["bwd"] == before["bwd"] + 1
+        ro, rl = oracle_fwd(q, k, v, is_causal=True)
+        rdq, rdk, rdv = oracle_bwd(go, q, k, v, ro, rl, is_causal=True)[:3]
+        assert max_abs(out, ro) <= 2e-5
+        for a, b_ in ((qd.grad, rdq), (kd.grad, rdk), (vd.grad, rdv)):
+            assert max_abs(a, b_) <= 5e-5
+        # what is no plain 4-D GPU call keeps upstream's route
+        cpu = F.scaled_dot_product_attention(q, k, v, is_causal=True, enable_gqa=True)
+        assert max_abs(cpu, ro) <= 2e-5
+        with pytest.raises(RuntimeError):
+            F.scaled_dot_product_attention(qd, kd, vd, is_causal=True)  # (heads differ and no enable_gqa: upstream's error)
+    finally:
+        amd.route_functional(False)
+    assert F.scaled_dot_product_attention is stock
+
+
 def test_replaced_upstream_operators_keep_upstream_layouts_and_redraw_the_dropout_mask(amd, gpu_device):
     """The flash and memory-efficient operators called directly with dropout: outputs in upstream's shapes
     and layouts; seed and offset are the generator's state before the draw, the backward draws the same
