@@ -144,10 +144,10 @@ typedef struct mi355_sdpa_mask_spec {
   int32_t doc_ids_sorted;
   const int32_t* mask_verdict; /* optional, with a bias / keep-mask: what mi355_sdpa_mask_verdict wrote
                                   about that tensor.  The call is then put on the stream as a pair of
-                                  kernels - with the mask, and with the causal flag and key counts -
-                                  whose first instructions read the verdict: a mask that is the
-                                  keep-everything or the causal pattern (with or without right padding)
-                                  is never read.  Matrix-op kernels for 16-bit inputs, head dims up to
+                                  kernels - with the mask, and with the causal flag, the window and
+                                  key counts - whose first instructions read the verdict: a mask that is
+                                  the keep-everything or the causal pattern or a sliding window with
+                                  sink keys (each with or without right padding) is never read.  Matrix-op kernels for 16-bit inputs, head dims up to
                                   128 (the forward: up to 256), a mask with a row per query, nothing else
                                   shaping the scores; every other call uses the mask itself           */
 } mi355_sdpa_mask_spec;
@@ -285,7 +285,7 @@ int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, int64_t S, 
  * memory; 0 = this mask cannot have one: it depends on the head, its keys are not unit-stride):
  *   verdict[0] kind: 0 not a pattern, 1 keep-everything, 2 causal, 3 sliding window with sink keys
  *   verdict[1] window, verdict[2] sink keys, verdict[3] 1 if some batch keeps fewer than S keys
- *   verdict[8 + b] keys of batch b that take part (right padding under kinds 1 and 2)
+ *   verdict[8 + b] keys of batch b that take part (right padding becomes a key count under every kind)
  * `mask` is the bias / keep-mask expanded to (B,Hq,L,S), stride 0 on broadcast dims.  Nothing
  * synchronises: the call records into a HIP graph in front of the attention call that is given
  * the verdict (mi355_sdpa_mask_spec.mask_verdict), and then follows a mask that is updated in place

@@ -99,6 +99,46 @@ def test_recognition_is_sound_on_random_near_patterns():
     assert seen > 100
 
 
+def test_window_masks_with_right_padding_are_recognised():
+    # what model code builds for a sliding-window model from a padded batch: window & causal & key < len[b]
+    from torch_neuronx_amd.mask_patterns import window_lens_pattern_from_rows
+
+    def rows3(m):
+        return np.stack([rows_of(x.numpy()) for x in m])
+
+    def rebuild3(pat, L, S):
+        W, N, lens = pat[1], pat[2], pat[3]
+        return torch.stack([om.window_keep_mask(L, S, W, N) & (torch.arange(S)[None] < int(n)) for n in lens])
+
+    g = torch.Generator().manual_seed(5)
+    seen = exact = 0
+    for trial in range(300):
+        L = int(torch.randint(2, 40, (1,), generator=g))
+        S = L if trial % 2 else int(torch.randint(2, 40, (1,), generator=g))
+        W = int(torch.randint(1, 12, (1,), generator=g))
+        N = int(torch.randint(0, 5, (1,), generator=g))
+        B = int(torch.randint(1, 5, (1,), generator=g))
+        lens = torch.randint(0, S + 1, (B,), generator=g)
+        m = om.window_keep_mask(L, S, W, N)[None] & (torch.arange(S)[None] < lens[:, None])[:, None, :]
+        if trial % 3 == 0:
+            b, i, j = (int(torch.randint(0, n, (1,), generator=g)) for n in (B, L, S))
+            m[b, i, j] = not m[b, i, j]
+        pat = window_lens_pattern_from_rows(rows3(m), L, S)
+        if pat is not None:  # whatever is recognised rebuilds exactly the mask it came from
+            seen += 1
+            assert torch.equal(rebuild3(pat, L, S), m), (L, S, W, N, lens.tolist(), pat)
+        elif trial % 3 and min(L, int(lens.max())) > W + N:  # an unperturbed mask in which the window shows is recognised
+            raise AssertionError((L, S, W, N, lens.tolist()))
+        exact += trial % 3 != 0
+    assert seen > 100
+    # left padding and a causal mask with padding are other patterns
+    L = S = 24
+    left = om.window_keep_mask(L, S, 5, 0)[None] & (torch.arange(S)[None] >= torch.tensor([0, 4])[:, None])[:, None, :]
+    assert window_lens_pattern_from_rows(rows3(left), L, S) is None
+    tril = torch.tril(torch.ones(L, S, dtype=torch.bool))[None]
+    assert window_lens_pattern_from_rows(rows3(tril), L, S) is None
+
+
 # ---- GPU ----------------------------------------------------------------------------------------------
 
 
@@ -253,6 +293,15 @@ def test_tril_mask_takes_the_causal_kernel(amd, gpu_device, monkeypatch):
     assert max_abs(out_b, r_c[0]) <= 4e-3
 
 
+def _holed(keep3, b):
+    """One kept score dropped in batch ``b``: the middle one of the row that keeps the most."""
+    keep3 = keep3.clone()
+    i = int(keep3[b].sum(-1).argmax())
+    kept = torch.nonzero(keep3[b, i]).flatten()
+    keep3[b, i, kept[kept.numel() // 2]] = False
+    return keep3
+
+
 def _keep_masks(L, S, B):
     """Boolean (Bm, Lm, S) masks by name: the patterns, near misses, and masks that are none."""
     g = torch.Generator().manual_seed(L + S)
@@ -270,6 +319,9 @@ def _keep_masks(L, S, B):
         "causal_padding": tril[None] & pad,
         "window": om.window_keep_mask(L, S, max(L // 4, 1), 0)[None],
         "window_sinks": om.window_keep_mask(L, S, max(L // 4, 2), 2)[None],
+        "window_padding": om.window_keep_mask(L, S, max(L // 4, 1), 0)[None] & pad,
+        "window_sinks_padding": om.window_keep_mask(L, S, max(L // 5, 2), 3)[None] & pad,
+        "window_padding_holed": _holed(om.window_keep_mask(L, S, max(L // 4, 1), 0)[None] & pad, B - 1),
         "left_padding": (torch.arange(S)[None] >= (S - lens)[:, None])[:, None, :].expand(B, L, S),
         "random": (torch.rand(1, L, S, generator=g) < 0.5),
         "holed": holed,
@@ -280,7 +332,7 @@ def _keep_masks(L, S, B):
 
 def _expected_verdict(keep3: torch.Tensor, B: int, L: int):
     """(kind, window, sink keys, lens) by the host rules on brute-force row summaries."""
-    from torch_neuronx_amd.mask_patterns import lens_pattern_from_rows, pattern_from_rows
+    from torch_neuronx_amd.mask_patterns import lens_pattern_from_rows, window_lens_pattern_from_rows
 
     Bm, Lm, S = keep3.shape
     rows = np.stack([rows_of(m.numpy()) for m in keep3])
@@ -288,10 +340,11 @@ def _expected_verdict(keep3: torch.Tensor, B: int, L: int):
     if pat is not None:
         lens = np.broadcast_to(pat[1], (B,)) if Bm == 1 else pat[1]
         return (1 if pat[0] == "all" else 2), 0, 0, [int(x) for x in lens]
-    if Bm == 1 and Lm == L:
-        pat = pattern_from_rows(rows[0], L, S)
-        if pat is not None and pat[0] == "window":
-            return 3, pat[1], pat[2], [S] * B
+    if Lm == L and L > 1 and (rows[:, :, 1] >= 0).all():
+        pat = window_lens_pattern_from_rows(rows, L, S)
+        if pat is not None:
+            lens = np.broadcast_to(pat[3], (B,)) if Bm == 1 else pat[3]
+            return 3, pat[1], pat[2], [int(x) for x in lens]
     return 0, 0, 0, [S] * B
 
 
@@ -321,7 +374,8 @@ def test_device_verdict_follows_the_host_rules(amd, gpu_device, dtype, L, S):
 
 @pytest.mark.gpu
 @pytest.mark.parametrize("D", [64, 128])
-@pytest.mark.parametrize("name", ["causal", "causal_padding", "padding", "all", "random", "window", "holed"])
+@pytest.mark.parametrize("name", ["causal", "causal_padding", "padding", "all", "random", "window", "holed",
+                                  "window_sinks", "window_padding", "window_sinks_padding", "window_padding_holed"])
 def test_calls_with_a_verdict_equal_the_calls_they_stand_for(amd, gpu_device, name, D):
     # forward and backward through the C ABI with mask + verdict, against the same call with the flag and
     # key counts (for a pattern) or with the mask alone (for anything else): the same kernels, bit for bit
@@ -331,11 +385,14 @@ def test_calls_with_a_verdict_equal_the_calls_they_stand_for(amd, gpu_device, na
     keep = _keep_masks(L, L, B)[name]
     md = keep.to(dev)[:, None]
     verdict = amd.ops.mask_verdict(md, B, Hq, L, L)
-    kind, _, _, lens = _expected_verdict(keep, B, L)
+    kind, window, sinks, lens = _expected_verdict(keep, B, L)
+    assert (kind == 3) == (name.startswith("window") and not name.endswith("holed"))
     out, lse = amd.sdpa_forward(q, k, v, attn_bias=md, mask_verdict=verdict, force_kernel=amd._lib.KERNEL_MFMA)
     grads = amd.sdpa_backward(go, q, k, v, out, lse, attn_bias=md, mask_verdict=verdict, force_kernel=amd._lib.KERNEL_MFMA)[:3]
     if kind in (1, 2):
         kw = dict(is_causal=kind == 2, kv_lens=torch.tensor(lens, dtype=torch.int32, device=dev))
+    elif kind == 3:
+        kw = dict(is_causal=True, window=window, sink_keys=sinks, kv_lens=torch.tensor(lens, dtype=torch.int32, device=dev))
     else:
         kw = dict(attn_bias=md)
     ro, rl = amd.sdpa_forward(q, k, v, **kw)
@@ -541,6 +598,76 @@ def test_sliding_window_mask_at_head_dim_256_takes_the_window_kernels(amd, gpu_d
     assert max_abs(out, ro) <= 2e-2
     rdq, rdk, rdv = om.sdpa_backward(go.float(), q.float(), k.float(), v.float(), ro, rl, attn_mask=keep, reduce_in_fp32=True)
     assert rel_err(qd.grad, rdq) <= 3e-2 and rel_err(kd.grad, rdk) <= 3e-2 and rel_err(vd.grad, rdv) <= 3e-2
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("D", [128, 256])
+def test_sliding_window_and_padding_mask_becomes_the_window_with_key_counts(amd, gpu_device, monkeypatch, D):
+    """The (B,1,L,S) mask that the code of a sliding-window model builds from a right-padded batch
+    (causal & window & key < len[b]).  A new tensor per call, as that code makes them: the calls carry the
+    verdict and run the window kernels with key counts (within 1.25x of the functor call's time at head
+    dim 128, where a bias would take more than twice as long).  A tensor the caller keeps: once the
+    verdict has reached the host, the functor call itself, forward and backward.  Both against the oracle
+    on the explicit mask."""
+    dev = gpu_device
+    B, H, L, W = 3, 4, 2048, 256
+    q, k, v, go = (t.to(dev) for t in qkv(B, H, H, L, L, D, dtype=torch.bfloat16, seed=8, with_do=True))
+    lens = torch.tensor([L, 1300, 77])
+    keep = om.window_keep_mask(L, L, W)[None, None] & (torch.arange(L)[None] < lens[:, None])[:, None, None, :]
+    amd.mask_patterns.clear_cache()
+    seen = []
+    f0, b0 = amd.ops.sdpa_forward, amd.ops.sdpa_backward
+    MFMA = amd._lib.KERNEL_MFMA  # forced: the call fails if the matrix-op kernels cannot take it
+    monkeypatch.setattr(amd.ops, "sdpa_forward", lambda *a, **kw: (seen.append(kw), f0(*a, **{**kw, "force_kernel": MFMA}))[1])
+    monkeypatch.setattr(amd.ops, "sdpa_backward", lambda *a, **kw: (seen.append(kw), b0(*a, **{**kw, "force_kernel": MFMA}))[1])
+    fused = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    fused_bwd = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    qc, kc, vc, gc = (t.float().cpu() for t in (q, k, v, go))
+    ro, rl = om.sdpa_forward(qc, kc, vc, attn_mask=keep)
+    rg = om.sdpa_backward(gc, qc, kc, vc, ro, rl, attn_mask=keep, reduce_in_fp32=True)
+
+    def check(r, grads):
+        assert max_abs(r[0], ro) <= 2e-2 and max_abs(r[1], rl) <= 5e-3
+        for a, b_ in zip(grads[:3], rg):
+            assert rel_err(a, b_) <= 3e-2 and max_abs(a, b_) <= 5e-2 * max(1.0, float(b_.abs().max()))
+
+    fresh = lambda: torch.where(keep, 0.0, float("-inf")).to(torch.bfloat16).to(dev)
+    if D == 128:  # (the verdict on the device serves head dims up to 128 in the backward)
+        mask = fresh()
+        r = fused(q, k, v, mask)
+        grads = fused_bwd(go, q, k, v, mask, [True, True, True, False], r[0], r[1], None, None, L, L, 0.0, False, r[6], r[7])
+        assert seen[0]["attn_bias"] is not None and seen[0].get("mask_verdict") is not None
+        # (the backward carries the verdict too, unless its copy has reached the host by then)
+        assert seen[1].get("mask_verdict") is not None or (seen[1]["attn_bias"] is None and seen[1]["window"] == W)
+        v0 = seen[0]["mask_verdict"].cpu().tolist()
+        assert v0[:4] == [3, W, 0, 1] and v0[8:8 + B] == lens.tolist()
+        check(r, grads)
+        # time, at a size where the kernels and not the host set it: new masks against the functor call
+        Bt, Ht, Lt, Wt = 4, 16, 4096, 512
+        qt, kt, vt = (torch.randn(Bt, Ht, Lt, D, device=dev, dtype=torch.bfloat16) for _ in range(3))
+        lens_t = torch.tensor([Lt, 3000, 2000, 500])
+        keep_t = (om.window_keep_mask(Lt, Lt, Wt)[None, None] & (torch.arange(Lt)[None] < lens_t[:, None])[:, None, None, :]).to(dev)
+        masks = [torch.where(keep_t, 0.0, float("-inf")).to(torch.bfloat16) for _ in range(10)]
+        kv = lens_t.to(torch.int32).to(dev)
+        turn = iter(range(10**9))
+        with torch.no_grad():
+            ok, seen_t = _within(lambda: fused(qt, kt, vt, masks[next(turn) % 10]),
+                                 lambda: amd.sdpa_forward(qt, kt, vt, is_causal=True, window=Wt, kv_lens=kv), 1.25)
+        assert ok, seen_t
+    # a mask the caller keeps: the host learns the pattern and makes the functor call
+    mask = fresh()
+    amd.mask_patterns.clear_cache()
+    with torch.no_grad():
+        fused(q, k, v, mask)
+    torch.cuda.synchronize()
+    pat = amd.mask_patterns.classify(mask)
+    assert pat[:3] == ("window", W, 0) and pat[3].cpu().tolist() == lens.tolist()
+    del seen[:]
+    r = fused(q, k, v, mask)
+    grads = fused_bwd(go, q, k, v, mask, [True, True, True, False], r[0], r[1], None, None, L, L, 0.0, False, r[6], r[7])
+    for kw in seen:
+        assert kw["attn_bias"] is None and kw["is_causal"] is True and kw["window"] == W and kw["kv_lens"].cpu().tolist() == lens.tolist()
+    check(r, grads)
 
 
 @pytest.mark.gpu

@@ -541,6 +541,26 @@ def test_replaced_upstream_operators_keep_upstream_layouts_and_redraw_the_dropou
     r3 = om.compute_attention_backward(gc, qc, kc, vc, None, keep2, ro2, rl2, D**-0.5, False, p)
     for a, b_ in zip(g3, r3[:3]):
         assert max_abs(a, b_) <= 5e-2 * max(1.0, float(b_.abs().max()))
+    # through autograd the forward keeps its mask for the backward, which takes it; a backward that does
+    # not find it (evicted from the bounded store) draws it again: the same gradients, bit for bit
+    qr, kr, vr = (t.clone().requires_grad_(True) for t in (q, k, v))
+    impl._kept.clear()
+    grads = []
+    for lose_it in (False, True):
+        torch.cuda.manual_seed(9)
+        out = F.scaled_dot_product_attention(qr, kr, vr, dropout_p=p)
+        assert len(impl._kept) == 1
+        if lose_it:
+            impl._kept.clear()
+        out.backward(go)
+        assert len(impl._kept) == 0
+        grads.append([t.grad.clone() for t in (qr, kr, vr)])
+        qr.grad = kr.grad = vr.grad = None
+    for a, b_ in zip(*grads):
+        assert torch.equal(a, b_)
+    with torch.no_grad():  # (no backward can follow: nothing is kept)
+        F.scaled_dot_product_attention(qr, kr, vr, dropout_p=p)
+    assert len(impl._kept) == 0
 
 
 def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):

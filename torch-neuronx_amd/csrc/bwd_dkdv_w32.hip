@@ -120,7 +120,7 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
   // multiplied by keep / (1 - p) there (torch_neuronx/_sdpa_math.py:36-48, :154-158).
   constexpr bool HASB = MASK == 2 || MASK == 5, DROP = MASK == 3 || MASK == 5;  // a bias per score; a keep-mask
   constexpr bool BIASED = HASB || DROP;
-  const int W = FUNC ? p.window : 0, n_sink = FUNC ? p.sink_keys : 0;
+  const int W = FUNC ? ma.window : 0, n_sink = FUNC ? ma.sink_keys : 0;
   // the query rows that see this lane's key are first_q .. past_q - 1: from the key itself on under a
   // causal mask, none for a key past the batch's count, up to the end of the key's window unless it is a sink
   const int first_q = key >= S ? INT_MAX : ma.causal ? key : INT_MIN;
@@ -769,7 +769,7 @@ __global__ __launch_bounds__(64) void bwd_dkdv_merge_kernel(BwdM p) {
     int S = p.S;
     if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
     const int qs_begin = ma.causal ? min(k0 / BQ, nqs) : 0;
-    const int qs_end = (p.window > 0 && k0 >= p.sink_keys) ? max(min(nqs, (k0 + BK + p.window - 2) / BQ + 1), qs_begin) : nqs;
+    const int qs_end = (ma.window > 0 && k0 >= ma.sink_keys) ? max(min(nqs, (k0 + BK + ma.window - 2) / BQ + 1), qs_begin) : nqs;
     const int n_items = k0 >= S ? 0 : (p.Hq / p.Hkv / p.parts_h) * (qs_end - qs_begin);
     parts = min(max((n_items + p.chunk_items - 1) / p.chunk_items, 1), p.parts / p.parts_h) * p.parts_h;
   }

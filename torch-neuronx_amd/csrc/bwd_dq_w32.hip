@@ -163,7 +163,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   int doc_run_w[2] = {0, 0x7fffffff};
   bool doc_one_w = false;
   if constexpr (FUNC) {
-    int t_lo = p.window > 0 ? max(q0 - p.window + 1, 0) / BN : 0;
+    int t_lo = ma.window > 0 ? max(q0 - ma.window + 1, 0) / BN : 0;
     if constexpr (SMOD) {
       // document ids sorted along the sequence: only the run of keys whose id lies between the ids of
       // this workgroup's first and last row can hold a kept score; the same for this wavefront's own
@@ -182,7 +182,7 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
       }
     }
     if (t_lo > 0) {
-      n_lead = min(min(p.window > 0 ? (p.sink_keys + BN - 1) / BN : 0, t_lo), nt);
+      n_lead = min(min(ma.window > 0 ? (ma.sink_keys + BN - 1) / BN : 0, t_lo), nt);
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
     }
@@ -234,13 +234,13 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   // reaches below the window of the wavefront's last row and is not made of sink keys alone
   const int t_edge = min(ma.causal ? qw0 / BN : 0x7fffffff, (S % BN) ? S / BN : 0x7fffffff);
   const int lim = ma.causal ? min(qrow, S - 1) : S - 1;
-  const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
-  const int n_sink = FUNC ? p.sink_keys : 0;
+  const int lo_w = (FUNC && ma.window > 0) ? qrow - ma.window + 1 : (int)0x80000000;
+  const int n_sink = FUNC ? ma.sink_keys : 0;
   auto edge_tile = [&](int u) {
     const int ta = tile_of(u);
     bool e = ta >= t_edge;
     if constexpr (FUNC) {
-      if (p.window > 0) e |= ta * BN < qw0 + 31 - p.window + 1 && ta * BN + BN > n_sink;
+      if (ma.window > 0) e |= ta * BN < qw0 + 31 - ma.window + 1 && ta * BN + BN > n_sink;
     }
     return e;
   };

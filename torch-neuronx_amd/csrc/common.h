@@ -74,26 +74,28 @@ static inline T4 view(const mi355_sdpa_tensor& t) {
 
 // The mask arguments of a call as a kernel body sees them: the parameter block's own, or what a
 // verdict about the call's bias (written by mi355_sdpa_mask_verdict) puts in their place.  A verdict
-// that names the keep-everything or the causal pattern, with or without right padding, turns the call
-// into one with the causal flag and per-batch key counts and no bias (verdict_pattern returns true),
-// and the kernel goes on in its variant for such calls.  Uniform scalar loads, ahead of everything
+// that names the keep-everything or the causal pattern, or a sliding window with sink keys, each with
+// or without right padding, turns the call into one with the causal flag, the window and per-batch key
+// counts and no bias (verdict_pattern returns true), and the kernel goes on in its variant for such calls.  Uniform scalar loads, ahead of everything
 // else; every kernel of a call applies the same rule to the same block, so they agree.  (Passed
 // beside the block rather than written into it: a kernel that modifies its parameter block keeps
 // all of it in registers.)
 struct MaskArgs {
   int causal, bias_kind;
   const int32_t* kv_lens;
+  int window, sink_keys;
 };
 template <typename P>
 __device__ __forceinline__ MaskArgs mask_args_of(const P& p) {
-  return MaskArgs{p.causal, p.bias_kind, p.kv_lens};
+  return MaskArgs{p.causal, p.bias_kind, p.kv_lens, p.window, p.sink_keys};
 }
 template <typename P>
 __device__ __forceinline__ bool verdict_pattern(const P& p, MaskArgs& m) {
   if (!p.verdict) return false;
   const int kind = p.verdict[0];
-  if (kind != 1 && kind != 2) return false;
-  m.causal = kind == 2, m.bias_kind = 0, m.kv_lens = p.verdict + 8;
+  if (kind < 1 || kind > 3) return false;
+  m.causal = kind >= 2, m.bias_kind = 0, m.kv_lens = p.verdict + 8;
+  if (kind == 3) m.window = p.verdict[1], m.sink_keys = p.verdict[2];
   return true;
 }
 

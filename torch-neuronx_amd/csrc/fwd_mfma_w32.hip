@@ -139,7 +139,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   int doc_run_w[2] = {0, 0x7fffffff};
   bool doc_one_w = false;
   if constexpr (FUNC) {
-    int t_lo = p.window > 0 ? max(q0 - p.window + 1, 0) / BN : 0;
+    int t_lo = ma.window > 0 ? max(q0 - ma.window + 1, 0) / BN : 0;
     if constexpr (SMOD) {
       // Document ids that are sorted along the sequence: the keys whose id lies between the ids of
       // this workgroup's first and last row are one run of doc_k; the tiles outside it hold no kept
@@ -159,7 +159,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
       }
     }
     if (t_lo > 0) {
-      n_lead = min(min(p.window > 0 ? (p.sink_keys + BN - 1) / BN : 0, t_lo), nt);
+      n_lead = min(min(ma.window > 0 ? (ma.sink_keys + BN - 1) / BN : 0, t_lo), nt);
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
     }
@@ -172,7 +172,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   // what follows only falls.  Every wavefront then walks all of the workgroup's tiles (the ones above
   // its own diagonal come first and are masked whole: rows without a live key yet, see the check).
   // (a head whose slope is not positive keeps the upward walk: its bias falls towards the diagonal)
-  const bool backwards = SMOD && ma.causal && p.sm.alibi != nullptr && p.window == 0 && n_lead == 0 && skip == 0 &&
+  const bool backwards = SMOD && ma.causal && p.sm.alibi != nullptr && ma.window == 0 && n_lead == 0 && skip == 0 &&
                          !(p.sm.doc_q && p.sm.doc_k) && p.sm.alibi[h] > 0.f;
   constexpr bool SPLITS = MASK == 1 || (MASK == 2 && D <= 128);  // the variants that can split their keys
   if constexpr (SPLITS) {
@@ -397,8 +397,8 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   const f32x16 zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   const int lim = ma.causal ? min(qrow, S - 1) : S - 1;
   // (window: keys below lo_w are dropped unless they are sink keys)
-  const int lo_w = (FUNC && p.window > 0) ? qrow - p.window + 1 : (int)0x80000000;
-  const int n_sink = FUNC ? p.sink_keys : 0;
+  const int lo_w = (FUNC && ma.window > 0) ? qrow - ma.window + 1 : (int)0x80000000;
+  const int n_sink = FUNC ? ma.sink_keys : 0;
 
   auto mask_tile = [&](f32x16& s, int kv0) {
 #pragma unroll
@@ -604,7 +604,7 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
     const int ta = tile_of(u);
     bool e = ta >= t_edge;
     if constexpr (FUNC) {
-      if (p.window > 0) e |= ta * BN < qw_last - p.window + 1 && ta * BN + BN > n_sink;
+      if (ma.window > 0) e |= ta * BN < qw_last - ma.window + 1 && ta * BN + BN > n_sink;
     }
     return e;
   };

@@ -98,8 +98,9 @@ extern "C" int mi355_sdpa_mask_rows(const void* mask, int32_t dtype, int64_t L, 
 // updated in place between replays.
 //   verdict[0] kind: 0 not a pattern, 1 keep-everything, 2 causal, 3 sliding window with sink keys
 //   verdict[1] window   verdict[2] sink keys   verdict[3] 1 if some batch keeps fewer than S keys
-//   verdict[8 + b] keys of batch b that take part (kinds 1 and 2: right padding becomes a key count)
-// and behind them the row summaries, four ints per (mask batch, row).
+//   verdict[8 + b] keys of batch b that take part (right padding becomes a key count)
+// and behind them the row summaries, four ints per (mask batch, row), and one int per mask batch (the
+// key count that a window pattern would have there).
 namespace mi355 {
 namespace {
 
@@ -109,6 +110,7 @@ struct VerdictArgs {
   int B, Bm, L, Lm, S;
   int32_t* verdict;
   int32_t* rows;
+  int32_t* n_win;  // per mask batch
 };
 
 template <typename T>
@@ -162,44 +164,107 @@ __global__ __launch_bounds__(256) void mask_rows_batched_kernel(VerdictArgs a) {
   }
 }
 
-// One workgroup: the rules of mask_patterns.py (pattern_from_rows, lens_pattern_from_rows), held
-// against the row summaries of every mask batch.
+// One workgroup: the rules of mask_patterns.py (lens_pattern_from_rows, window_lens_pattern_from_rows),
+// held against the row summaries of every mask batch.  Its threads share out the (mask batch, row)
+// pairs as one range, so the time does not grow with the batch size on its own.
 __global__ __launch_bounds__(1024) void mask_verdict_kernel(VerdictArgs a) {
   const int tid = threadIdx.x;
   const int L = a.L, Lm = a.Lm, S = a.S;
   const bool per_row = Lm == L;  // (otherwise one row stands for every query: no causal, no window)
-  int ok_all = 1, ok_causal = per_row && L > 1, ok_mask = 1;
-  for (int bm = 0; bm < a.Bm; ++bm) {
-    const int32_t* rows = a.rows + (int64_t)bm * Lm * 4;
-    const int hi_last = rows[(Lm - 1) * 4];
-    const int n_all = hi_last + 1;
-    const int n_causal = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;  // the last row reaches its diagonal: no key is known to be padding
-    for (int i = tid; i < Lm; i += 1024) {
-      const int hi = rows[i * 4], cnt = rows[i * 4 + 1], lo = rows[i * 4 + 3];
+  const bool windows = per_row && L > 1;
+  const int64_t pairs = (int64_t)a.Bm * Lm;
+  __shared__ int red_s[16];
+  auto block_max = [&](int v) {  // (called by every thread)
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = max(v, __shfl_xor(v, o, 64));
+    __syncthreads();
+    if ((tid & 63) == 0) red_s[tid >> 6] = v;
+    __syncthreads();
+    int r = red_s[0];
+#pragma unroll
+    for (int w = 1; w < 16; ++w) r = max(r, red_s[w]);
+    return r;
+  };
+  if (windows) {
+    for (int bm = tid; bm < a.Bm; bm += 1024) a.n_win[bm] = -1;
+    __syncthreads();
+  }
+  int ok_all = 1, ok_causal = windows, ok_mask = 1;
+  for (int64_t base = 0; base < pairs; base += 1024) {  // (every thread makes every trip: the wavefront votes below)
+    const int64_t idx = base + tid;
+    const bool valid = idx < pairs;
+    int bm = -1, top = -1;
+    if (valid) {
+      bm = (int)(idx / Lm);
+      const int i = (int)(idx - (int64_t)bm * Lm);
+      const int hi_last = a.rows[((int64_t)bm * Lm + Lm - 1) * 4];
+      const int n_all = hi_last + 1;
+      const int n_causal = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;  // the last row reaches its diagonal: no key is known to be padding
+      const int32_t* row = a.rows + idx * 4;
+      const int hi = row[0], cnt = row[1], lo = row[3];
       if (cnt < 0) ok_mask = 0;
       if (lo != 0 || hi != n_all - 1 || cnt != n_all) ok_all = 0;
       const int hc = min(min(i, S - 1), n_causal - 1);
       if (lo != 0 || hi != hc || cnt != hc + 1) ok_causal = 0;
+      top = hi;
+    }
+    // (for the window pattern below: the keys of a batch are those up to the last one any of its rows
+    // keeps; a wavefront whose rows belong to one batch, the usual case, adds its maximum once)
+    if (windows) {
+      const int bm0 = __builtin_amdgcn_readfirstlane(bm);
+      if (__builtin_amdgcn_ballot_w64(bm == bm0) == ~0ull) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) top = max(top, __shfl_xor(top, o, 64));
+        if ((tid & 63) == 0 && bm0 >= 0 && top >= 0) atomicMax(&a.n_win[bm0], top);
+      } else if (valid && top >= 0) {
+        atomicMax(&a.n_win[bm], top);
+      }
     }
   }
   ok_mask = __syncthreads_and(ok_mask);
   ok_all = __syncthreads_and(ok_all) && ok_mask;
   ok_causal = __syncthreads_and(ok_causal) && ok_mask;
   int kind = ok_all ? 1 : ok_causal ? 2 : 0, window = 0, sinks = 0;
-  if (!kind && ok_mask && a.Bm == 1 && per_row && L > 1) {
-    // sliding window with sink keys: query i keeps keys i-W+1 .. i and the first N keys
-    const int32_t* rows = a.rows;
-    const int r = L - 1;
-    const int hi_r = rows[r * 4], lead_r = rows[r * 4 + 2], lo_r = rows[r * 4 + 3];
-    const int W = hi_r - lo_r + 1, N = lead_r < lo_r ? lead_r : 0;
-    int ok = W > 0 && lo_r != 0;
-    for (int i = tid; i < L && ok; i += 1024) {
-      const int hi = rows[i * 4], cnt = rows[i * 4 + 1], lead = rows[i * 4 + 2], lo = rows[i * 4 + 3];
-      const int hc = min(i, S - 1), lead_full = hc + 1 < S ? hc + 1 : S;
-      const int lo_w = max(i - W + 1, 0);
-      const bool joined = lo_w <= N;  // the window reaches into the sink keys (or to key 0): one run from key 0
-      if (hi != hc || i - W + 1 > hc) ok = 0;
-      if (lo != (joined ? 0 : lo_w) || lead != (joined ? lead_full : N) || cnt != (joined ? hc + 1 : hc - lo_w + 1 + N)) ok = 0;
+  if (!kind && ok_mask && windows) {
+    // Sliding window with sink keys, with or without right padding: query i of a batch with n keys
+    // keeps the keys of i-W+1 .. i and of the first N that lie below n (all S keys when some row reaches
+    // the last diagonal element).  W and N are read where they show: in the last row that has keys of
+    // its own, in the (first) batch with the most keys.
+    int n_mine = 0;
+    for (int bm = tid; bm < a.Bm; bm += 1024) {
+      const int top = a.n_win[bm];
+      const int n = top == min(L - 1, S - 1) ? S : top + 1;
+      a.n_win[bm] = n;
+      n_mine = max(n_mine, n);
+    }
+    const int n_max = block_max(n_mine);  // (its barriers also publish n_win)
+    int b_mine = -0x7fffffff;
+    for (int bm = tid; bm < a.Bm; bm += 1024)
+      if (a.n_win[bm] == n_max) b_mine = max(b_mine, -bm);
+    const int b_sel = -block_max(b_mine);
+    int W = 0, N = 0, ok = n_max > 0;
+    if (ok) {
+      const int32_t* row = a.rows + ((int64_t)b_sel * Lm + min(n_max, L) - 1) * 4;
+      const int hi_r = row[0], lead_r = row[2], lo_r = row[3];
+      W = hi_r - lo_r + 1, N = lead_r < lo_r ? lead_r : 0;
+      ok = W > 0 && lo_r != 0;
+    }
+    for (int64_t idx = tid; idx < pairs && ok; idx += 1024) {
+      const int bm = (int)(idx / Lm), i = (int)(idx - (int64_t)bm * Lm);
+      const int n = a.n_win[bm];
+      const int32_t* row = a.rows + idx * 4;
+      const int hi = row[0], cnt = row[1], lead = row[2], lo = row[3];
+      const int top = min(min(i, S - 1), n - 1), lo_w = max(i - W + 1, 0);
+      int e_hi, e_cnt, e_lead, e_lo = 0;
+      if (lo_w > top) {  // the window lies behind the batch's keys: the sink keys below n are what is left
+        const int m = max(min(N, top + 1), 0);
+        e_hi = m - 1, e_cnt = m, e_lead = m;
+      } else if (lo_w <= N) {  // the window reaches into the sink keys (or to key 0): one run from key 0
+        e_hi = top, e_cnt = top + 1, e_lead = top + 1;
+      } else {
+        e_hi = top, e_cnt = top - lo_w + 1 + N, e_lead = N, e_lo = lo_w;
+      }
+      if (hi != e_hi || cnt != e_cnt || lead != e_lead || lo != e_lo) ok = 0;
     }
     if (__syncthreads_and(ok)) kind = 3, window = W, sinks = N;
   }
@@ -211,6 +276,7 @@ __global__ __launch_bounds__(1024) void mask_verdict_kernel(VerdictArgs a) {
     int n = S;
     if (kind == 1) n = hi_last + 1;
     else if (kind == 2) n = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;
+    else if (kind == 3) n = a.n_win[bm];
     a.verdict[8 + b] = n;
     short_any |= n != S;
   }
@@ -240,7 +306,7 @@ bool verdict_shape(const mi355_sdpa_tensor& t, int32_t dtype, int* Bm, int* Lm) 
 extern "C" size_t mi355_sdpa_mask_verdict_words(const mi355_sdpa_tensor* mask, int32_t dtype) {
   int Bm, Lm;
   if (!mask || !verdict_shape(*mask, dtype, &Bm, &Lm)) return 0;
-  return (size_t)8 + (size_t)mask->size[0] + (size_t)Bm * Lm * 4;
+  return (size_t)8 + (size_t)mask->size[0] + (size_t)Bm * Lm * 4 + (size_t)Bm;
 }
 
 extern "C" int mi355_sdpa_mask_verdict(const mi355_sdpa_tensor* mask, int32_t dtype, int32_t* verdict, void* stream) {
@@ -253,7 +319,7 @@ extern "C" int mi355_sdpa_mask_verdict(const mi355_sdpa_tensor* mask, int32_t dt
   a.mask = mask->data;
   a.sb = Bm > 1 ? mask->stride[0] : 0, a.sl = Lm > 1 ? mask->stride[2] : 0;
   a.B = (int)mask->size[0], a.Bm = Bm, a.L = (int)mask->size[2], a.Lm = Lm, a.S = (int)mask->size[3];
-  a.verdict = verdict, a.rows = verdict + 8 + a.B;
+  a.verdict = verdict, a.rows = verdict + 8 + a.B, a.n_win = a.rows + (int64_t)Bm * Lm * 4;
   hipStream_t s = (hipStream_t)stream;
   const dim3 grid((unsigned)(((int64_t)Bm * Lm + 3) / 4)), block(256);
   switch (dtype) {

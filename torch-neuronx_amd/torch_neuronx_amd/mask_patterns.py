@@ -14,8 +14,8 @@ A copy of the verdict travels to the host on the side.  Once it has arrived (a l
 that out with a query, never a wait) the decision is cached for as long as the tensor is
 unchanged: a causal mask, a sliding window with sink keys and a keep-everything mask are then
 served by the kernels that generate those patterns from indices and read no mask at all; so are
-the masks that model code builds from right padding, with or without causality folded in
-(per-batch key counts).
+the masks that model code builds from right padding, with or without causality or a sliding window
+folded in (per-batch key counts).
 """
 
 from __future__ import annotations
@@ -172,6 +172,43 @@ def lens_pattern_from_rows(rows: np.ndarray, L: int, S: int, rows_broadcast: boo
     return None
 
 
+def window_lens_pattern_from_rows(rows: np.ndarray, L: int, S: int):
+    """A sliding window with sink keys, with or without right padding, per batch: ``rows[b, i]`` as in
+    ``pattern_from_rows`` -> ``("window", W, N, lens)`` (row ``i`` of batch ``b`` keeps those of the keys
+    ``i-W+1 .. i`` and of the first ``N`` keys that lie below ``lens[b]``; a row whose window lies behind
+    its batch's keys keeps the sink keys or nothing) or ``None``.  The keys of a batch are those up to
+    the last one any of its rows keeps - all ``S`` when a row reaches the last diagonal element; ``W``
+    and ``N`` are read in the last row with keys of its own of the batch with the most keys."""
+    if rows.ndim != 3 or rows.shape[0] == 0 or rows.shape[1] != L or rows.shape[2] != 4 or L < 2 or S < 1:
+        return None
+    hi, cnt, lead, lo = (rows[:, :, c].astype(np.int64) for c in range(4))
+    if (cnt < 0).any():
+        return None
+    top_b = hi.max(axis=1)
+    n = np.where(top_b == min(L - 1, S - 1), S, top_b + 1)
+    b_sel = int(np.argmax(n))
+    if n[b_sel] <= 0:
+        return None
+    r = min(int(n[b_sel]), L) - 1
+    W = int(hi[b_sel, r] - lo[b_sel, r] + 1)
+    N = int(lead[b_sel, r]) if lead[b_sel, r] < lo[b_sel, r] else 0
+    if W <= 0 or lo[b_sel, r] == 0:
+        return None
+    i = np.arange(L, dtype=np.int64)[None, :]
+    top = np.minimum(np.minimum(i, S - 1), (n - 1)[:, None])
+    lo_w = np.maximum(i - W + 1, 0)
+    behind = lo_w > top
+    joined = ~behind & (lo_w <= N)
+    m = np.maximum(np.minimum(N, top + 1), 0)
+    e_hi = np.where(behind, m - 1, top)
+    e_cnt = np.where(behind, m, np.where(joined, top + 1, top - lo_w + 1 + N))
+    e_lead = np.where(behind, m, np.where(joined, top + 1, N))
+    e_lo = np.where(behind | joined, 0, lo_w)
+    if (hi == e_hi).all() and (cnt == e_cnt).all() and (lead == e_lead).all() and (lo == e_lo).all():
+        return ("window", W, N, n.astype(np.int32))
+    return None
+
+
 # A verdict is put to use on the device only where the mask's traffic matters; below, the mask is as
 # cheap as the two extra launches (the copy to the host is still made, for the calls that follow).
 _MIN_SCORES_ON_DEVICE = 256 * 256
@@ -199,7 +236,7 @@ class _Pending:
         return self.event is not None and self.event.query()
 
     def pattern(self):
-        """``("all" | "causal" [, key counts]) | ("window", W, N) | None`` from the host copy."""
+        """``("all" | "causal" [, key counts]) | ("window", W, N [, key counts]) | None`` from the host copy."""
         h = self.host
         kind, window, sinks, short = (int(x) for x in h[:4])
         if kind in (1, 2):
@@ -207,7 +244,7 @@ class _Pending:
             # (the key counts are used where they are: behind the verdict's header, on the device)
             return (name, self.verdict[8:8 + self.B]) if short else (name,)
         if kind == 3:
-            return ("window", window, sinks)
+            return ("window", window, sinks, self.verdict[8:8 + self.B]) if short else ("window", window, sinks)
         return None
 
 

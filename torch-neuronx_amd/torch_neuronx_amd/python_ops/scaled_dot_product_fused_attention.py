@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import math
 import os
+from collections import OrderedDict
 
 import torch
 
@@ -86,28 +87,48 @@ def _scalar_rng():
     return _scalar_rng_pair
 
 
-def _seeded_keep(query, S, dropout_p):
+# Masks of forwards whose backward is still to come, by (device, seed, offset, shape, p): the backward
+# takes its mask from here and draws it again only when it is gone (evicted, taken by an earlier
+# backward of the same graph, a forward that ran in another process).  Bounded in bytes and entries.
+_kept: "OrderedDict[tuple, torch.Tensor]" = OrderedDict()
+_KEPT_MAX_BYTES = 2 << 30
+_KEPT_MAX_ENTRIES = 256
+
+
+def _seeded_keep(query, S, dropout_p, remember):
     """Keep-mask from the device's default generator together with the (seed, offset) it was drawn at,
-    as 0-dim int64 host tensors: the backward draws the same mask again from the pair, so the mask
-    itself (``B*H*L*S`` bytes) does not have to stay alive between the two, and the operator's outputs
-    have the shapes upstream's operators promise (a compiled graph checks them)."""
+    as 0-dim int64 host tensors: the operator's outputs then have the shapes upstream's operators
+    promise (a compiled graph checks them), and the backward can draw the same mask again from the
+    pair.  ``remember``: a backward may follow - the mask is kept for it (``_kept``)."""
     index = query.device.index if query.device.index is not None else torch.cuda.current_device()
     gen = torch.cuda.default_generators[index]
     seed, offset = gen.initial_seed(), gen.get_offset()
     keep = _dropout_keep(query, S, dropout_p)
+    if remember:
+        _kept[(index, seed, offset, tuple(keep.shape), dropout_p)] = keep
+        held = sum(t.numel() for t in _kept.values())
+        while len(_kept) > 1 and (held > _KEPT_MAX_BYTES or len(_kept) > _KEPT_MAX_ENTRIES):
+            held -= _kept.popitem(last=False)[1].numel()
     if seed >= 1 << 63:
         seed -= 1 << 64  # (a 64-bit seed in an int64 tensor)
     return keep, torch.tensor(seed, dtype=torch.int64), torch.tensor(offset, dtype=torch.int64)
 
 
-def _keep_again(query, S, dropout_p, philox_seed, philox_offset):
-    """The mask ``_seeded_keep`` drew at ``(philox_seed, philox_offset)``."""
+def _keep_again(query, S, dropout_p, philox_seed, philox_offset, take=True):
+    """The mask ``_seeded_keep`` drew at ``(philox_seed, philox_offset)``: the one kept for this
+    backward (``take``: removed from the store), or drawn again from the pair."""
     B, H, L, _ = query.shape
+    index = query.device.index if query.device.index is not None else torch.cuda.current_device()
+    seed, offset = int(philox_seed) % (1 << 64), int(philox_offset)
+    key = (index, seed, offset, (B, H, L, S), dropout_p)
+    keep = _kept.pop(key, None) if take else _kept.get(key)
+    if keep is not None:
+        return keep
     if dropout_p >= 1.0:
         return torch.zeros((B, H, L, S), dtype=torch.uint8, device=query.device)
     gen = torch.Generator(device=query.device)
-    gen.manual_seed(int(philox_seed) % (1 << 64))
-    gen.set_offset(int(philox_offset))
+    gen.manual_seed(seed)
+    gen.set_offset(offset)
     return torch.empty((B, H, L, S), dtype=torch.uint8, device=query.device).bernoulli_(1.0 - dropout_p, generator=gen)
 
 
@@ -124,7 +145,7 @@ def _wants_grad_bias(attn_bias, grad_input_mask) -> bool:
 
 def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, dropout_p=0.0):
     """A mask that is a pattern the kernels generate by themselves (causal, sliding window with sink
-    keys, keep-everything, either of the first two with right padding) is dropped in favour of that
+    keys, keep-everything, each of them with right padding) is dropped in favour of that
     pattern - the run-time counterpart of the reference's causal-mask recovery
     (fx/passes/sdpa_causal_mask.py:162-289).  A mask about which the host knows nothing yet travels on
     with its verdict (``mask_verdict``, an int32 device tensor): the kernels then take the decision
@@ -140,7 +161,10 @@ def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, dro
         return None, False, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
     if pat[0] == "causal":
         return None, True, ({"kv_lens": pat[1]} if len(pat) > 1 else {})
-    return None, True, {"window": pat[1], "sink_keys": pat[2]}
+    functor = {"window": pat[1], "sink_keys": pat[2]}
+    if len(pat) > 3:
+        functor["kv_lens"] = pat[3]
+    return None, True, functor
 
 
 def _skip_tables(functor, attn_bias, is_causal, dropout_p, query, key):
@@ -176,7 +200,8 @@ def _forward(query, key, value, attn_bias, dropout_p, is_causal, return_debug_ma
     keep = None
     if dropout_p > 0.0:
         if upstream is not None and not torch.cuda.is_current_stream_capturing():
-            keep, seed, offset = _seeded_keep(query, S, dropout_p)
+            remember = torch.is_grad_enabled() and (query.requires_grad or key.requires_grad or value.requires_grad)
+            keep, seed, offset = _seeded_keep(query, S, dropout_p, remember)
         else:  # (under capture a seed read on the host would be frozen into the graph: the mask travels)
             keep = _dropout_keep(query, S, dropout_p)
             seed, offset = keep, torch.empty((0,), dtype=torch.int32, device=query.device)
