@@ -158,3 +158,56 @@ def test_greedy_generation_with_a_kv_cache_matches_the_stock_kernels(amd, gpu_de
         amd.route_functional(False)
     assert library_calls["fwd"] == 48, library_calls
     assert torch.equal(got, want)
+
+
+@pytest.mark.parametrize("case", ["no_mask", "key_padding", "causal_flag", "causal_and_padding", "eval_fast_path",
+                                  "encoder_padding", "decoder_layer"])
+def test_torch_nn_attention_modules_match_the_stock_kernels(amd, gpu_device, library_calls, case):
+    """``nn.MultiheadAttention`` / ``nn.TransformerEncoder`` / ``nn.TransformerDecoderLayer`` in float32:
+    the masks these modules merge (key padding expanded per head, a causal mask with the flag, both) and
+    the inference fast path reach the library and give the stock numbers, outputs and gradients."""
+    import torch.nn as nn
+
+    dev = gpu_device
+    B, S, E, H = 8, 200, 384, 6
+    torch.manual_seed(0)
+    x = torch.randn(B, S, E, device=dev)
+    pad = torch.zeros(B, S, dtype=torch.bool, device=dev)
+    pad[1, 150:] = True
+    pad[5, 60:] = True
+    causal = nn.Transformer.generate_square_subsequent_mask(S, device=dev)
+    if case == "encoder_padding":
+        mod, args, kw, calls = nn.TransformerEncoder(nn.TransformerEncoderLayer(E, H, 768, dropout=0.0, batch_first=True), 2), (x,), dict(src_key_padding_mask=pad), 2
+    elif case == "decoder_layer":
+        mod, args, calls = nn.TransformerDecoderLayer(E, H, 768, dropout=0.0, batch_first=True), (x, x), 2
+        kw = dict(tgt_mask=causal, tgt_is_causal=True, memory_key_padding_mask=pad)
+    else:
+        mod, args, calls = nn.MultiheadAttention(E, H, batch_first=True, dropout=0.0), (x, x, x), 1
+        kw = {"no_mask": {}, "eval_fast_path": {}, "key_padding": dict(key_padding_mask=pad),
+              "causal_flag": dict(attn_mask=causal, is_causal=True),
+              "causal_and_padding": dict(attn_mask=causal, key_padding_mask=pad.float().masked_fill(pad, float("-inf")))}[case]
+        kw["need_weights"] = False
+    mod = mod.to(dev)
+    train = case != "eval_fast_path"
+
+    def run():
+        mod.train(train)
+        mod.zero_grad()
+        with torch.set_grad_enabled(train):
+            out = mod(*args, **kw)
+            out = out[0] if isinstance(out, tuple) else out
+            if train:
+                out.square().mean().backward()
+        return out.detach(), (torch.cat([p.grad.flatten() for p in mod.parameters()]) if train else None)
+
+    try:
+        amd.unregister()
+        o0, g0 = run()
+        assert library_calls == {"fwd": 0, "bwd": 0}
+    finally:
+        amd.register()
+    o1, g1 = run()
+    assert library_calls["fwd"] == calls and library_calls["bwd"] == (calls if train else 0), library_calls
+    assert float((o1 - o0).abs().max()) <= 1e-5 * max(1.0, float(o0.abs().max()))
+    if train:
+        assert float((g1 - g0).norm() / g0.norm()) <= 1e-5
