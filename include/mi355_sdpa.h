@@ -24,7 +24,7 @@
 extern "C" {
 #endif
 
-#define MI355_SDPA_ABI_VERSION 5
+#define MI355_SDPA_ABI_VERSION 6
 
 /* element types */
 enum mi355_sdpa_dtype {
@@ -167,7 +167,8 @@ typedef struct mi355_sdpa_fwd_params {
                              L*S elements, is left out and the kernels read the bytes        */
   int32_t bias_dtype;     /* F32/F16/BF16/BOOL                                        */
   const int32_t* kv_lens; /* optional (B,): key j of batch b takes part iff j<kv_lens[b] */
-  const uint8_t* dropout_keep; /* optional (B,Hq,L,S) contiguous, 1 = keep            */
+  const uint8_t* dropout_keep; /* optional (B,Hq,L,S), 1 = keep: contiguous, or with rows
+                                  dropout_keep_ld bytes apart (below)                  */
   float dropout_p;
   int32_t dtype;          /* dtype of q/k/v/out                                       */
   int32_t is_causal;      /* lower-triangular, anchored top-left (also when L != S)   */
@@ -179,6 +180,12 @@ typedef struct mi355_sdpa_fwd_params {
                              keys over more workgroups (partial results here, merged by a second
                              kernel); without it the same call runs unsplit                    */
   size_t workspace_bytes;
+  int64_t dropout_keep_ld; /* 0, or the bytes from one row of dropout_keep to the next (>= S; the
+                              (B,Hq,L) rows stay densely packed at that pitch, the last row
+                              included).  The matrix-op kernels for 16-bit inputs read the bytes a
+                              dword at a time and need rows that start on dwords: a caller whose S
+                              is no multiple of 4 pads the rows to one, or the call runs in the
+                              generic kernels                                                */
 } mi355_sdpa_fwd_params;
 
 typedef struct mi355_sdpa_bwd_params {
@@ -205,6 +212,7 @@ typedef struct mi355_sdpa_bwd_params {
   int32_t force_kernel;
   mi355_sdpa_mask_spec mask;  /* as in forward                                          */
   float* grad_sink_logit;     /* optional, shape of mask.sink_logit: its gradient       */
+  int64_t dropout_keep_ld;    /* as in forward                                          */
 } mi355_sdpa_bwd_params;
 
 typedef struct mi355_sdpa_decode_params {

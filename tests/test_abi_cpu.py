@@ -38,7 +38,7 @@ def test_library_exports_every_declared_symbol(amd):
     for n in names:
         assert hasattr(lib, n), n
     assert set(names) == set(amd._lib.EXPORTS)
-    assert lib.mi355_sdpa_abi_version() == 5
+    assert lib.mi355_sdpa_abi_version() == 6
 
 
 def test_ctypes_structs_match_c_layout(amd, tmp_path):

@@ -173,6 +173,12 @@ DROPOUT_MFMA = [
     (1, 4, 2, 300, 260, 256, True, None, 0.1),            # head dims above 128: the wide backward kernels
     (2, 2, 2, 129, 512, 192, False, [512, 77], 0.25),
     (1, 2, 1, 64, 64, 160, True, None, 0.5),
+    # numbers of keys that are no multiple of four (a batch padded to its longest sequence, 197 image
+    # patches): the mask is copied once into rows that start on dwords
+    (2, 6, 6, 197, 197, 64, False, None, 0.1),
+    (2, 4, 2, 301, 259, 128, True, None, 0.25),
+    (1, 2, 2, 70, 131, 256, False, [90], 0.3),
+    (1, 4, 1, 1, 77, 64, False, None, 0.5),
 ]
 
 
@@ -384,6 +390,38 @@ def test_dropout_at_wide_head_dims_through_the_operator(amd, gpu_device, monkeyp
     for a, b_ in ((dq, rdq), (dk, rdk), (dv, rdv)):
         assert max_abs(a, b_) <= (1e-2 if half else 3e-5)
     assert 0.88 < keep.float().mean().item() < 0.92
+
+
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_dropout_over_197_keys_through_the_operators(amd, gpu_device, monkeypatch, dtype):
+    """A ViT-sized layer with attention dropout through the registered operators: the keep-mask is drawn
+    into rows padded to dwords (no copy), the matrix-op kernels take it (forced), the mask that travels to
+    the backward is the (B,H,L,S) view of those rows, and both directions agree with the oracle given it -
+    also together with an additive bias whose rows need the same treatment."""
+    from torch_neuronx_amd.python_ops import scaled_dot_product_fused_attention as impl
+    monkeypatch.setattr(impl, "_force_kernel", lambda: amd._lib.KERNEL_MFMA)
+    B, H, S, D, p = 4, 6, 197, 64, 0.1
+    dev = gpu_device
+    g = torch.Generator().manual_seed(197)
+    q, k, v, go = (torch.randn(B, H, S, D, generator=g).to(dtype).to(dev) for _ in range(4))
+    go = (go.float() * 0.1).to(dtype)
+    bias = torch.randn(1, H, S, S, generator=g).to(dtype).to(dev)
+    op = torch.ops.aten._scaled_dot_product_fused_attention_overrideable
+    opb = torch.ops.aten._scaled_dot_product_fused_attention_overrideable_backward
+    half = dtype is not torch.float32
+    for b_ in (None, bias):
+        r = op(q, k, v, b_, p, False)
+        keep = r[6]
+        assert keep.shape == (B, H, S, S) and keep.stride() == (H * S * 200, S * 200, 200, 1)
+        assert 0.88 < keep.float().mean().item() < 0.92
+        dq, dk, dv, _ = opb(go, q, k, v, b_, [True, True, True, False], r[0], r[1], None, None, S, S, p, False, keep, r[7])
+        qc, kc, vc, gc = (t.float().cpu() for t in (q, k, v, go))
+        bc = None if b_ is None else b_.float().cpu()
+        ro, rl = om.compute_attention(qc, kc, vc, bc, keep.cpu().bool(), D**-0.5, False, p)
+        rdq, rdk, rdv, _ = om.compute_attention_backward(gc, qc, kc, vc, bc, keep.cpu().bool(), ro, rl, D**-0.5, False, p)
+        assert max_abs(r[0], ro) <= (2e-2 if half else 2e-5) and max_abs(r[1], rl) <= (2e-3 if half else 2e-5)
+        for a, c in ((dq, rdq), (dk, rdk), (dv, rdv)):
+            assert max_abs(a, c) <= (1e-2 if half else 3e-5)
 
 
 def test_backward_kv_lens(amd, gpu_device):

@@ -251,10 +251,10 @@ static int kernel_for(const mi355_sdpa_desc* d, bool backward) {
   const bool dims = E % 8 == 0 && E <= 256 && Dv % 8 == 0 && Dv <= E;
   // (float32: the float32 matrix-op kernels take the same head dims)
   const bool f32_ok = true;
-  // (dropout, 16-bit dtypes: keep-mask rows that are whole dwords)
-  const bool drop_ok = d->dropout_p == 0.f || d->q_dtype == MI355_SDPA_F32 || S % 4 == 0;
+  // (dropout, 16-bit dtypes: the call itself sends keep-mask rows that do not start on dwords to the
+  // generic kernel - a caller whose S is no multiple of 4 pads the rows, see dropout_keep_ld)
   const bool fast = f32_ok && dims &&
-                    bias_ok && drop_ok && scale > 0.f &&
+                    bias_ok && scale > 0.f &&
                     d->q_last_stride == 1 && d->k_last_stride == 1 && d->v_last_stride == 1;
   return fast ? MI355_SDPA_KERNEL_MFMA : MI355_SDPA_KERNEL_GENERIC;
 }

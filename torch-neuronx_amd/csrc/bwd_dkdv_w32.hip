@@ -356,14 +356,14 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
       if (it >= n_items || (ma.causal && q0 + BQ - 1 < kw0) || kw0 >= S) return;
       if constexpr (DROP) {
         const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-            uniform_ptr((const char*)p.keep + ((int64_t)b * p.Hq + item_head(it)) * p.L * p.S), 0,
-            __builtin_amdgcn_readfirstlane((int)((int64_t)p.L * p.S)), 0x00020000);
-        const uint32_t kbase = (uint32_t)((q0 + half * 4) * p.S + key);
+            uniform_ptr((const char*)p.keep + ((int64_t)b * p.Hq + item_head(it)) * p.L * p.keep_ld), 0,
+            __builtin_amdgcn_readfirstlane((int)((int64_t)(p.L - 1) * p.keep_ld + p.S)), 0x00020000);
+        const uint32_t kbase = (uint32_t)((q0 + half * 4) * p.keep_ld + key);
 #pragma unroll
         for (int mq = 0; mq < 2; ++mq)
 #pragma unroll
           for (int r = 0; r < 16; ++r)
-            kraw[mq][r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(k_rsrc, kbase + (uint32_t)((mq * 32 + (r >> 2) * 8 + (r & 3)) * p.S), 0, 0);
+            kraw[mq][r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(k_rsrc, kbase + (uint32_t)((mq * 32 + (r >> 2) * 8 + (r & 3)) * p.keep_ld), 0, 0);
       }
       if constexpr (!HASB) return;
       const __amdgpu_buffer_rsrc_t b_rsrc = __builtin_amdgcn_make_buffer_rsrc(

@@ -455,9 +455,9 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   const unsigned char* const bias_w = (const unsigned char*)(tile_list + 1040) + (BIASED ? wave * 4096 : 0);
   const uint32_t lds_b = (uint32_t)(uintptr_t)(lds_bytes)bias_w;
   // the keep bytes of a dropout call: one load, lane (row, half) -> keys 16 half .. +15, 1 KB per wavefront behind the bias tiles
-  const u32x4 kp_rsrc = descriptor((const char*)p.keep + (DROP ? (((int64_t)b * p.Hq + h) * p.L + qw0) * p.S : 0),
-                                   (DROP && b_rows > 0) ? (int64_t)b_rows * p.S : 0);
-  const uint32_t kp_voff = DROP ? (uint32_t)(min(col, max(b_rows - 1, 0)) * p.S + half * 16) : 0u;
+  const u32x4 kp_rsrc = descriptor((const char*)p.keep + (DROP ? (((int64_t)b * p.Hq + h) * p.L + qw0) * p.keep_ld : 0),
+                                   (DROP && b_rows > 0) ? (int64_t)b_rows * p.keep_ld : 0);  // (whole rows: a dword that reaches past the records reads as zero)
+  const uint32_t kp_voff = DROP ? (uint32_t)(min(col, max(b_rows - 1, 0)) * p.keep_ld + half * 16) : 0u;
   const unsigned char* const keep_w = (const unsigned char*)(tile_list + 1040) + (DROP ? 8 * 4096 + wave * 1024 : 0);
   const uint32_t lds_kp = (uint32_t)(uintptr_t)(lds_bytes)keep_w;
   uint32_t kraw[4];

@@ -26,6 +26,7 @@ struct BwdG {
   float* delta;  // workspace (B,Hq,L)
   const int32_t* kv_lens;
   const uint8_t* keep;
+  int64_t keep_ld;  // bytes from one row of keep bytes to the next
   float keep_scale;
   int B, Hq, Hkv, L, S, E, Dv;
   int causal, bias_kind;
@@ -92,7 +93,7 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_row_kernel(BwdG p) {
   if (p.gbias.data)
     gb_row = (T*)p.gbias.data + b * p.gbias.st[0] + h * p.gbias.st[1] + i * p.gbias.st[2];
   const uint8_t* keep_row =
-      p.keep ? p.keep + (((int64_t)b * p.Hq + h) * p.L + i) * (int64_t)p.S : nullptr;
+      p.keep ? p.keep + (((int64_t)b * p.Hq + h) * p.L + i) * p.keep_ld : nullptr;
 
   float acc[NV];
 #pragma unroll
@@ -196,7 +197,7 @@ __global__ __launch_bounds__(64 * kWaves) void bwd_col_kernel(BwdG p) {
             pr = expf(s - l);
             float keepf = 1.f;
             if (p.keep)
-              keepf = p.keep[(((int64_t)b * p.Hq + h) * p.L + i) * (int64_t)p.S + j] ? p.keep_scale : 0.f;
+              keepf = p.keep[(((int64_t)b * p.Hq + h) * p.L + i) * p.keep_ld + j] ? p.keep_scale : 0.f;
             ds = pr * (dp * keepf - delta[i]) * dfac * p.scale;
             pr *= keepf;
           }
@@ -296,6 +297,7 @@ int launch_bwd_generic(const mi355_sdpa_bwd_params& p, hipStream_t s) {
   g.bias = view(p.bias), g.gbias = view(p.grad_bias);
   g.lse = p.lse, g.delta = (float*)p.workspace, g.kv_lens = p.kv_lens;
   g.keep = p.dropout_p > 0.f ? p.dropout_keep : nullptr;
+  g.keep_ld = (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]);
   g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.L = (int)p.q.size[2], g.E = (int)p.q.size[3];
   g.Hkv = (int)p.k.size[1], g.S = (int)p.k.size[2], g.Dv = (int)p.v.size[3];

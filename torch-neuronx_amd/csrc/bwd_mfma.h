@@ -28,6 +28,7 @@ struct BwdM {
   // (B, Hq, L, S) contiguous keep bytes
   float keep_scale = 0.f;
   const void* keep = nullptr;
+  int64_t keep_ld = 0;  // bytes from one row of keep bytes to the next (S, or more where the caller padded the rows)
   const int32_t* kv_lens = nullptr;
   // gradient of the bias (the dQ kernel writes it): P (dP - delta) in the input dtype, one element
   // per score, unit stride over keys, rows a whole number of 8-byte words (zeros where a score

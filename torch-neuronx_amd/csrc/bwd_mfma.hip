@@ -558,6 +558,7 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
     g.verdict = p.mask.mask_verdict;
   if (p.dropout_p > 0.f) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
     g.keep = p.dropout_keep;
+    g.keep_ld = (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]);
     g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
 }
@@ -607,7 +608,7 @@ bool bwd_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
     // the keep-mask takes a bool bias's way into the kernels (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
     if (p.mask.window > 0) return *why = "dropout together with a window functor", false;
-    if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
+    if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]) % 4 != 0) return *why = "dropout keep-mask rows do not start on dwords", false;
     if ((p.q.size[2] + 64) * S + S + 64 >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
   }
   if (!(p.scale > 0.f)) return *why = "scale <= 0", false;

@@ -296,9 +296,9 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dq_kernel(BwdM p) {
   uint32_t braw[16];
   // (DROP) the keep bytes of the same 16 keys, four dwords
   const __amdgpu_buffer_rsrc_t kp_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-      uniform_ptr((const char*)p.keep + (DROP ? ((int64_t)b * p.Hq + h) * p.L * p.S : 0)), 0,
-      __builtin_amdgcn_readfirstlane(DROP ? (int)((int64_t)p.L * p.S) : 0), 0x00020000);
-  const uint32_t kp_row = DROP ? (uint32_t)((int64_t)qc * p.S + half * 4) : 0u;
+      uniform_ptr((const char*)p.keep + (DROP ? ((int64_t)b * p.Hq + h) * p.L * p.keep_ld : 0)), 0,
+      __builtin_amdgcn_readfirstlane(DROP ? (int)((int64_t)p.L * p.keep_ld) : 0), 0x00020000);  // (whole rows: dword loads)
+  const uint32_t kp_row = DROP ? (uint32_t)((int64_t)qc * p.keep_ld + half * 4) : 0u;
   uint32_t kraw[DROP ? 4 : 1];
   auto load_bias = [&](int t) {
     if constexpr (DROP) {
@@ -638,11 +638,11 @@ __global__ __launch_bounds__(256, 1) void bwd_wide_dkdv_kernel(BwdM p) {
   auto request_keep = [&](int hg, int q0, uint32_t (&kb)[DROP ? 16 : 1]) {
     if constexpr (DROP) {
       const __amdgpu_buffer_rsrc_t k_rsrc = __builtin_amdgcn_make_buffer_rsrc(
-          uniform_ptr((const char*)p.keep + ((int64_t)b * p.Hq + hk * rep + hg) * p.L * p.S), 0,
-          __builtin_amdgcn_readfirstlane((int)((int64_t)p.L * p.S)), 0x00020000);
-      const uint32_t base = (uint32_t)((q0 + half * 4) * p.S + min(key, p.S - 1));
+          uniform_ptr((const char*)p.keep + ((int64_t)b * p.Hq + hk * rep + hg) * p.L * p.keep_ld), 0,
+          __builtin_amdgcn_readfirstlane((int)((int64_t)(p.L - 1) * p.keep_ld + p.S)), 0x00020000);
+      const uint32_t base = (uint32_t)((q0 + half * 4) * p.keep_ld + min(key, p.S - 1));
 #pragma unroll
-      for (int r = 0; r < 16; ++r) kb[r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(k_rsrc, base + (uint32_t)(((r >> 2) * 8 + (r & 3)) * p.S), 0, 0);
+      for (int r = 0; r < 16; ++r) kb[r] = (uint32_t)__builtin_amdgcn_raw_buffer_load_b8(k_rsrc, base + (uint32_t)(((r >> 2) * 8 + (r & 3)) * p.keep_ld), 0, 0);
     }
   };
   auto pack_keep = [&](const uint32_t (&kb)[DROP ? 16 : 1]) {

@@ -199,7 +199,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
       const int64_t row0 = b * p.bias_sb + h * p.bias_sh + (int64_t)qc * p.bias_sl;
       auto idx = [&](int r) { return row0 + min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
       if (p.keep_scale != 0.f) {
-        const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.S;
+        const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.keep_ld;
 #pragma unroll
         for (int r = 0; r < 16; ++r) keepf[r] = (float)krow[min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1)];
       }
@@ -382,7 +382,7 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dq_kernel(BwdM p) {
       auto idx = [&](int r) { return row0 + min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1); };
       drop = p.keep_scale != 0.f;
       if (drop) {
-        const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.S;
+        const uint8_t* krow = (const uint8_t*)p.keep + (((int64_t)b * p.Hq + h) * p.L + qc) * p.keep_ld;
 #pragma unroll
         for (int r = 0; r < 16; ++r) kpf[r] = (float)krow[min(t * BT + (r >> 2) * 8 + half * 4 + (r & 3), p.S - 1)] * p.keep_scale;
       }
@@ -524,9 +524,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
         auto idx = [&](int r) { return col0 + (int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.bias_sl; };
         drop = p.keep_scale != 0.f;
         if (drop) {
-          const uint8_t* kcol = (const uint8_t*)p.keep + ((int64_t)b * p.Hq + hq) * p.L * p.S + min(key, p.S - 1);
+          const uint8_t* kcol = (const uint8_t*)p.keep + ((int64_t)b * p.Hq + hq) * p.L * p.keep_ld + min(key, p.S - 1);
 #pragma unroll
-          for (int r = 0; r < 16; ++r) kpf[r] = (float)kcol[(int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.S] * p.keep_scale;
+          for (int r = 0; r < 16; ++r) kpf[r] = (float)kcol[(int64_t)min(q0 + (r >> 2) * 8 + half * 4 + (r & 3), p.L - 1) * p.keep_ld] * p.keep_scale;
         }
         if (p.bias_kind) {
           load_bias16(bl, p.bias, p.bias_kind, idx);
@@ -591,6 +591,7 @@ void set_score_mask(G& g, const P& p) {
   }
   if (p.dropout_p > 0.f) {
     g.keep = p.dropout_keep;
+    g.keep_ld = (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]);
     g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
 }

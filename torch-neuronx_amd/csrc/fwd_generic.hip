@@ -22,6 +22,7 @@ struct FwdG {
   float* lse;
   const int32_t* kv_lens;
   const uint8_t* keep;
+  int64_t keep_ld;  // bytes from one row of keep bytes to the next
   float keep_scale;  // 1/(1-p), or 1 when p == 1 (the mask alone zeroes everything)
   int B, Hq, Hkv, L, S, E, Dv;
   int causal, bias_kind;  // 0 none, 1 additive, 2 bool
@@ -66,7 +67,7 @@ __global__ __launch_bounds__(64 * kWaves) void fwd_generic_kernel(FwdG p) {
   if (p.bias_kind)
     bias_row = (const TB*)p.bias.data + b * p.bias.st[0] + h * p.bias.st[1] + i * p.bias.st[2];
   const uint8_t* keep_row =
-      p.keep ? p.keep + (((int64_t)b * p.Hq + h) * p.L + i) * (int64_t)p.S : nullptr;
+      p.keep ? p.keep + (((int64_t)b * p.Hq + h) * p.L + i) * p.keep_ld : nullptr;
 
   for (int j0 = 0; j0 < s_end; j0 += 64) {
     const int j = j0 + lane;
@@ -165,6 +166,7 @@ int launch_fwd_generic(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   FwdG g;
   g.q = view(p.q), g.k = view(p.k), g.v = view(p.v), g.out = view(p.out), g.bias = view(p.bias);
   g.lse = p.lse, g.kv_lens = p.kv_lens, g.keep = p.dropout_p > 0.f ? p.dropout_keep : nullptr;
+  g.keep_ld = (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]);
   g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   g.B = (int)p.q.size[0], g.Hq = (int)p.q.size[1], g.L = (int)p.q.size[2], g.E = (int)p.q.size[3];
   g.Hkv = (int)p.k.size[1], g.S = (int)p.k.size[2], g.Dv = (int)p.v.size[3];

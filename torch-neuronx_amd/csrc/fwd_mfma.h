@@ -28,6 +28,7 @@ struct FwdM {
   // (1 for p = 1), and the (B, Hq, L, S) contiguous keep bytes
   float keep_scale = 0.f;
   const void* keep = nullptr;
+  int64_t keep_ld = 0;  // bytes from one row of keep bytes to the next (S, or more where the caller padded the rows)
   // Short query sequences under grouped-query attention (fwd_mfma_w32.hip; no dropout, no bias that
   // depends on the head): one workgroup serves `grouped` query heads of a kv group (all Hq / Hkv of
   // them where they fit its wavefronts; a divisor of that otherwise, with Hq / Hkv / grouped

@@ -359,7 +359,7 @@ bool fwd_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
     // the keep-mask takes a bool bias's way into the kernel (one dword = four keys of a row)
     const int64_t S = p.k.size[2];
     if (p.mask.window > 0 || p.mask.sink_logit || score_mod_of(p.mask).any) return *why = "dropout together with a functor", false;
-    if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || S % 4 != 0) return *why = "dropout keep-mask rows are not whole dwords", false;
+    if (!p.dropout_keep || ((uintptr_t)p.dropout_keep & 3) != 0 || (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]) % 4 != 0) return *why = "dropout keep-mask rows do not start on dwords", false;
     if (32 * S >= (1ll << 31)) return *why = "dropout keep-mask rows beyond 32-bit offsets", false;
     if ((int64_t)p.k.size[2] * p.k.stride[2] * 2 >= (1ll << 31) || (int64_t)p.k.size[2] * p.v.stride[2] * 2 >= (1ll << 31))
       return *why = "dropout with rows beyond 32-bit offsets", false;
@@ -406,6 +406,7 @@ static int launch_or_size(const mi355_sdpa_fwd_params& p, hipStream_t s, size_t*
   }
   if (p.dropout_p > 0.f) {  // (B, Hq, L, S) contiguous bytes, 1 = keep
     g.keep = p.dropout_keep;
+    g.keep_ld = (p.dropout_keep_ld > 0 ? p.dropout_keep_ld : p.k.size[2]);
     g.keep_scale = p.dropout_p < 1.f ? 1.f / (1.f - p.dropout_p) : 1.f;
   }
   g.d_real = (int)p.q.size[3], g.dv_real = (int)p.v.size[3];

@@ -437,9 +437,9 @@ __device__ __forceinline__ void fwd_w32_body(const FwdM& p, const MaskArgs ma) {
   if (bkind) inv_scale = 1.f / p.scale;
   // Dropout: the keep bytes of the tile, (B, Hq, L, S) contiguous, travel the way a bool bias does -
   // one load, lane (row, half) -> keys 16 half .. +15 - into 1 KB of the wavefront's own, beside the bias.
-  const u32x4 kp_rsrc = descriptor((const char*)p.keep + (DROP ? (((int64_t)b * p.Hq + h) * p.L + qw0) * p.S : 0),
-                                   (DROP && b_rows > 0) ? (int)((int64_t)b_rows * p.S) : 0);
-  const uint32_t kp_voff = DROP ? (uint32_t)(min(col, max(b_rows - 1, 0)) * p.S + half * 16) : 0u;
+  const u32x4 kp_rsrc = descriptor((const char*)p.keep + (DROP ? (((int64_t)b * p.Hq + h) * p.L + qw0) * p.keep_ld : 0),
+                                   (DROP && b_rows > 0) ? (int)((int64_t)b_rows * p.keep_ld) : 0);  // (whole rows: a dword that reaches past the records reads as zero)
+  const uint32_t kp_voff = DROP ? (uint32_t)(min(col, max(b_rows - 1, 0)) * p.keep_ld + half * 16) : 0u;
   const unsigned char* const keep_w = keep_lds + (DROP ? wave * 1024 : 0);
   const uint32_t lds_kp = (uint32_t)(uintptr_t)(lds_bytes)keep_w;
   uint32_t kraw[4];

@@ -19,6 +19,7 @@ KERNEL_NONE, KERNEL_GENERIC, KERNEL_MFMA, KERNEL_MFMA_T128, KERNEL_MFMA_T256 = 0
 BACKEND_MATH, BACKEND_OVERRIDEABLE = 0, 4
 OK, ERR_INVALID, ERR_UNSUPPORTED, ERR_LAUNCH = 0, -1, -2, -3
 DECODE_STATIC_SCRATCH_BYTES = 32 << 20
+ABI_VERSION = 6  # MI355_SDPA_ABI_VERSION of include/mi355_sdpa.h that the structures below follow
 
 _DTYPES = {
     torch.float32: F32, torch.float16: F16, torch.bfloat16: BF16, torch.float64: F64,
@@ -62,7 +63,7 @@ class FwdParams(C.Structure):
         ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
         ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
         ("force_kernel", C.c_int32), ("mask", MaskSpec),
-        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t),
+        ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("dropout_keep_ld", C.c_int64),
     ]
 
 
@@ -74,7 +75,7 @@ class BwdParams(C.Structure):
         ("kv_lens", C.c_void_p), ("dropout_keep", C.c_void_p), ("dropout_p", C.c_float),
         ("dtype", C.c_int32), ("is_causal", C.c_int32), ("scale", C.c_float),
         ("workspace", C.c_void_p), ("workspace_bytes", C.c_size_t), ("force_kernel", C.c_int32),
-        ("mask", MaskSpec), ("grad_sink_logit", C.c_void_p),
+        ("mask", MaskSpec), ("grad_sink_logit", C.c_void_p), ("dropout_keep_ld", C.c_int64),
     ]
 
 
@@ -127,6 +128,10 @@ def load() -> C.CDLL:
         for name, (res, args) in EXPORTS.items():
             fn = getattr(lib, name)
             fn.restype, fn.argtypes = res, args
+        if lib.mi355_sdpa_abi_version() != ABI_VERSION:
+            raise RuntimeError(
+                f"{LIB_PATH} has ABI version {lib.mi355_sdpa_abi_version()}, this binding is for {ABI_VERSION}: "
+                "rebuild the HIP extension (python -m torch_neuronx_amd._build)")
         _lib = lib
     return _lib
 

@@ -118,6 +118,34 @@ def _bias_view(attn_bias, B, Hq, L, S, repack_for=None):
     return b, _lib.dtype_id(b.dtype)
 
 
+def padded_keep_mask(B, Hq, L, S, device, dtype=torch.uint8):
+    """An uninitialised ``(B,Hq,L,S)`` keep-mask whose rows start on dwords (a view of rows padded to a
+    multiple of four bytes where ``S`` is none): the layout that every kernel takes as it is."""
+    S4 = -(-S // 4) * 4
+    return torch.empty((B, Hq, L, S4), dtype=dtype, device=device)[..., :S]
+
+
+def _keep_rows(keep, B, Hq, L, S, dtype):
+    """The dropout keep-mask as bytes in a layout the kernels take: ``(B,Hq,L)`` rows densely packed at
+    one pitch.  The matrix-op kernels for 16-bit inputs read the bytes a dword at a time, so for them a
+    mask whose rows do not start on dwords (``S`` no multiple of four: 197 image patches, a batch padded
+    to its longest sequence) is copied once into rows padded to one - against a call that would
+    otherwise run in the generic kernels, a hundred times slower.  ``padded_keep_mask`` makes masks
+    that need no copy."""
+    keep = keep.expand(B, Hq, L, S)
+    if keep.dtype != torch.uint8:
+        keep = keep.to(torch.uint8)
+    ld = keep.stride(2) if L > 1 else max(keep.stride(2), S)
+    packed = (keep.stride(3) == 1 or S == 1) and ld >= S and keep.stride(1) == L * ld and keep.stride(0) == Hq * L * ld
+    if packed and (dtype == torch.float32 or (ld % 4 == 0 and keep.data_ptr() % 4 == 0)):
+        return keep if L > 1 or keep.stride(2) == ld else keep.as_strided(keep.shape, (Hq * L * ld, L * ld, ld, 1))
+    if dtype == torch.float32 or S % 4 == 0:
+        return keep.contiguous()
+    out = padded_keep_mask(B, Hq, L, S, keep.device)
+    out.copy_(keep)
+    return out
+
+
 def _dword_rows(b, S) -> bool:
     if b.dtype not in (torch.bool, torch.float16, torch.bfloat16, torch.float32):
         return True  # (not a dtype the matrix-op kernels take: nothing to gain)
@@ -297,8 +325,8 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
         if dropout_keep.numel() <= 1:
             dropout_p = 0.0  # a mask of one element is the reference's placeholder for none (torch_neuronx/_sdpa_math.py:42-45)
         else:
-            dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
-            p.dropout_keep = dropout_keep.data_ptr()
+            dropout_keep = _keep_rows(dropout_keep, B, Hq, L, S, query.dtype)
+            p.dropout_keep, p.dropout_keep_ld = dropout_keep.data_ptr(), dropout_keep.stride(2)
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)
@@ -375,8 +403,8 @@ def sdpa_backward(grad_out, query, key, value, out, lse, attn_bias=None, is_caus
         if dropout_keep.numel() <= 1:
             dropout_p = 0.0  # a mask of one element is the reference's placeholder for none (torch_neuronx/_sdpa_math.py:42-45)
         else:
-            dropout_keep = dropout_keep.expand(B, Hq, L, S).to(torch.uint8).contiguous()
-            p.dropout_keep = dropout_keep.data_ptr()
+            dropout_keep = _keep_rows(dropout_keep, B, Hq, L, S, query.dtype)
+            p.dropout_keep, p.dropout_keep_ld = dropout_keep.data_ptr(), dropout_keep.stride(2)
     p.dropout_p = float(dropout_p)
     p.dtype = _lib.dtype_id(query.dtype)
     p.is_causal, p.scale, p.force_kernel = int(bool(is_causal)), float(scale), int(force_kernel)

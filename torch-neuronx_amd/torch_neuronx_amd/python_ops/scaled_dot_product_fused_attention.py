@@ -67,11 +67,13 @@ def _dropout_keep(query, S, dropout_p):
     """Keep-mask drawn on the device; it travels to the backward in the philox_seed slot, the
     way the reference carries its mask (decompositions.py:2354-2356)."""
     B, H, L, _ = query.shape
+    # (rows that start on dwords, padded where S is no multiple of four: the layout the kernels take as it is)
+    keep = ops.padded_keep_mask(B, H, L, S, query.device)
     if dropout_p >= 1.0:
-        return torch.zeros((B, H, L, S), dtype=torch.uint8, device=query.device)
+        return keep.zero_()
     # (drawn as bytes in place: a float draw, a compare and a cast take five times as long, more than
     # the attention of a short-sequence layer itself)
-    return torch.empty((B, H, L, S), dtype=torch.uint8, device=query.device).bernoulli_(1.0 - dropout_p)
+    return keep.bernoulli_(1.0 - dropout_p)
 
 
 _scalar_rng_pair = None
@@ -124,12 +126,13 @@ def _keep_again(query, S, dropout_p, philox_seed, philox_offset, take=True):
     keep = _kept.pop(key, None) if take else _kept.get(key)
     if keep is not None:
         return keep
+    keep = ops.padded_keep_mask(B, H, L, S, query.device)  # (the layout of _dropout_keep: the same draw)
     if dropout_p >= 1.0:
-        return torch.zeros((B, H, L, S), dtype=torch.uint8, device=query.device)
+        return keep.zero_()
     gen = torch.Generator(device=query.device)
     gen.manual_seed(seed)
     gen.set_offset(offset)
-    return torch.empty((B, H, L, S), dtype=torch.uint8, device=query.device).bernoulli_(1.0 - dropout_p, generator=gen)
+    return keep.bernoulli_(1.0 - dropout_p, generator=gen)
 
 
 def _present(attn_bias):
