@@ -410,6 +410,56 @@ def test_calls_with_a_verdict_equal_the_calls_they_stand_for(amd, gpu_device, na
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("pdrop", [0.0, 0.2])
+@pytest.mark.parametrize("name", ["padding_one_row", "padding", "causal_padding", "all", "random", "window_padding"])
+def test_verdicts_for_masks_per_key_and_for_calls_with_dropout(amd, gpu_device, name, pdrop):
+    """A `(B,1,1,S)` key-padding mask (one row for every query) takes its verdict too, and so do calls with
+    dropout: forward and backward with mask + verdict (+ keep-mask) equal the calls with key counts (for
+    keep-everything and causal patterns; a window has no dropout variant and stays a mask) and agree with
+    the oracle on the explicit mask."""
+    dev = gpu_device
+    B, Hq, Hkv, L, D = 3, 4, 2, 640, 64
+    q, k, v, go = (t.to(dev) for t in qkv(B, Hq, Hkv, L, L, D, dtype=torch.bfloat16, seed=len(name) + 3, with_do=True))
+    keep = _keep_masks(L, L, B)[name]  # (Bm, Lm, S)
+    md = torch.where(keep, 0.0, float("-inf")).to(torch.bfloat16).to(dev)[:, None]
+    verdict = amd.ops.mask_verdict(md, B, Hq, L, L)
+    kind, _, _, lens = _expected_verdict(keep, B, L)
+    MFMA = amd._lib.KERNEL_MFMA
+    drop = {}
+    dk_cpu = None
+    if pdrop:
+        dk_cpu = torch.rand(B, Hq, L, L, generator=torch.Generator().manual_seed(5)) >= pdrop
+        drop = dict(dropout_p=pdrop, dropout_keep=dk_cpu.to(dev))
+    out, lse = amd.sdpa_forward(q, k, v, attn_bias=md, mask_verdict=verdict, force_kernel=MFMA, **drop)
+    grads = amd.sdpa_backward(go, q, k, v, out, lse, attn_bias=md, mask_verdict=verdict, force_kernel=MFMA, **drop)[:3]
+    if kind in (1, 2):
+        kw = dict(is_causal=kind == 2, kv_lens=torch.tensor(lens, dtype=torch.int32, device=dev))
+    else:
+        assert kind == 0 or (kind == 3 and name == "window_padding")
+        kw = dict(attn_bias=md)
+    ro, rl = amd.sdpa_forward(q, k, v, force_kernel=MFMA, **kw, **drop)
+    rg = amd.sdpa_backward(go, q, k, v, ro, rl, force_kernel=MFMA, **kw, **drop)[:3]
+    if kind == 3 and not pdrop:  # (without dropout the window verdict is used: compared with the functor call elsewhere)
+        pass
+    else:
+        assert max_abs(out, ro) <= 1e-6 and max_abs(lse, rl) <= 1e-6, name
+        for a, b_ in zip(grads, rg):
+            assert max_abs(a, b_) <= 8e-3 * max(1.0, b_.abs().max().item()) and rel_err(a, b_) <= 2e-3, name
+    keep4 = keep[:, None].expand(keep.shape[0], 1, keep.shape[1], L).expand(B, 1, keep.shape[1], L).expand(B, Hq, L, L)
+    bias = torch.where(keep4, 0.0, float("-inf"))
+    rep = Hq // Hkv
+    qc, gc = q.float().cpu(), go.float().cpu()
+    kc, vc = k.float().cpu().repeat_interleave(rep, 1), v.float().cpu().repeat_interleave(rep, 1)
+    oo, ol = om.compute_attention(qc, kc, vc, bias, dk_cpu, D**-0.5, False, pdrop)
+    live = torch.isfinite(ol)
+    assert max_abs(out, oo) <= 2e-2 and max_abs(lse.cpu()[live], ol[live]) <= 5e-3
+    odq, odk, odv, _ = om.compute_attention_backward(gc, qc, kc, vc, bias, dk_cpu, oo, ol, D**-0.5, False, pdrop)
+    odk, odv = odk.view(B, Hkv, rep, L, D).sum(2), odv.view(B, Hkv, rep, L, D).sum(2)
+    for a, b_ in zip(grads, (odq, odk, odv)):
+        assert max_abs(a, b_) <= 5e-2 * max(1.0, b_.abs().max().item()) and rel_err(a, b_) <= 3e-2, name
+
+
+@pytest.mark.gpu
 def test_fresh_bool_masks_run_at_the_speed_of_the_causal_flag(amd, gpu_device):
     # F.scaled_dot_product_attention(attn_mask=bool) hands the op a new additive tensor on every call: no
     # cache can know it, the verdict on the device does.  Ten calls in a row, against is_causal=True.

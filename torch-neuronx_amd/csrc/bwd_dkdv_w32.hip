@@ -742,10 +742,12 @@ __device__ __forceinline__ void bwd_dkdv_w32_body(const BwdM& p, const MaskArgs 
 // verdict lets one of them run.
 template <typename T, int D, int MASK, bool PATTERN = false>
 __global__ __launch_bounds__(512, 1) void bwd_dkdv_w32_kernel(BwdM p) {
-  static_assert(!PATTERN || MASK == 1, "the pattern kernel is the variant with key counts");
+  static_assert(!PATTERN || MASK == 1 || MASK == 3, "the pattern kernels are the variants with key counts, without and with dropout");
   MaskArgs ma = mask_args_of(p);
-  if constexpr (MASK == 2 || PATTERN) {
+  if constexpr (MASK == 2 || MASK == 5 || PATTERN) {
     if (verdict_pattern(p, ma) != PATTERN) return;
+  } else if constexpr (MASK == 1) {
+    verdict_pattern(p, ma);  // (a bias per key that comes with a verdict: this variant takes the bias or the key counts)
   }
   bwd_dkdv_w32_body<T, D, MASK>(p, ma);
 }
@@ -868,7 +870,11 @@ int launch_m(const BwdM& g, hipStream_t s) {
       set_error("SDPA: dropout in bwd_dkdv_w32_kernel needs a keep-mask and no tile table");
       return MI355_SDPA_ERR_UNSUPPORTED;
     }
-    return g.bias_kind ? launch_t<T, D, 5>(g, s) : launch_t<T, D, 3>(g, s);
+    if (!g.bias_kind) return launch_t<T, D, 3>(g, s);
+    if (g.verdict) {  // (see bwd_dkdv_w32_kernel: the pair with dropout)
+      if (int rc = launch_t<T, D, 3, true>(g, s)) return rc;
+    }
+    return launch_t<T, D, 5>(g, s);
   }
   if (g.bias_kind && g.bias_sl != 0) {
     if (g.verdict) {  // (see bwd_dkdv_w32_kernel)

@@ -717,6 +717,8 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   MaskArgs ma = mask_args_of(p);
   if constexpr (MASK == 2 || PATTERN) {
     if (verdict_pattern(p, ma) != PATTERN) return;
+  } else if constexpr (MASK == 3) {
+    verdict_pattern(p, ma);  // (dropout: one variant takes a bias or none, so the verdict is applied in place)
   }
   bwd_dq_w32_body<T, D, MASK>(p, ma);
 }

@@ -552,8 +552,8 @@ static void fill(BwdM& g, const mi355_sdpa_bwd_params& p) {
       g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
     }
   }
-  // (a verdict about the bias is for the variants with a per-score bias, where nothing else shapes the scores)
-  if (p.mask.mask_verdict && g.bias_kind && g.bias_sl != 0 && !p.is_causal && !p.kv_lens && p.dropout_p == 0.f && !g.live_t &&
+  // (a verdict about the bias is for calls in which nothing else shapes the scores; dropout may come on top)
+  if (p.mask.mask_verdict && g.bias_kind && p.q.size[2] > 1 && !p.is_causal && !p.kv_lens && !g.live_t &&
       !g.live_tiles && !g.gbias && g.window == 0 && !g.sm.any && p.q.size[3] <= 128 && p.v.size[3] == p.q.size[3])
     g.verdict = p.mask.mask_verdict;
   if (p.dropout_p > 0.f) {  // (B, Hq, L, S) contiguous bytes, 1 = keep

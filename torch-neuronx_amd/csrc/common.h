@@ -93,7 +93,9 @@ template <typename P>
 __device__ __forceinline__ bool verdict_pattern(const P& p, MaskArgs& m) {
   if (!p.verdict) return false;
   const int kind = p.verdict[0];
-  if (kind < 1 || kind > 3) return false;
+  // (the variants with dropout have no window: such a mask stays a mask there - one rule for every
+  // kernel of a call, the merge kernels included)
+  if (kind < 1 || kind > (p.keep_scale != 0.f ? 2 : 3)) return false;
   m.causal = kind >= 2, m.bias_kind = 0, m.kv_lens = p.verdict + 8;
   if (kind == 3) m.window = p.verdict[1], m.sink_keys = p.verdict[2];
   return true;

@@ -417,8 +417,8 @@ static int launch_or_size(const mi355_sdpa_fwd_params& p, hipStream_t s, size_t*
     g.live_tiles = p.mask.live_tiles;
     g.live_words = ((g.S + 31) / 32 + 31) / 32, g.live_hm = live_extent(p.bias, 1);
   }
-  // (a verdict about the bias is for the variant with a per-score bias, where nothing else shapes the scores)
-  if (p.mask.mask_verdict && p.bias.data && p.bias.stride[2] != 0 && g.L > 1 && !p.is_causal && !p.kv_lens && p.dropout_p == 0.f &&
+  // (a verdict about the bias is for calls in which nothing else shapes the scores; dropout may come on top)
+  if (p.mask.mask_verdict && p.bias.data && g.L > 1 && !p.is_causal && !p.kv_lens &&
       !g.live_tiles && !g.sink_logit && g.window == 0 && !g.sm.any)
     g.verdict = p.mask.mask_verdict;
   if (p.workspace && ((uintptr_t)p.workspace & 255) == 0) g.part_o = (float*)p.workspace, g.part_bytes = p.workspace_bytes;

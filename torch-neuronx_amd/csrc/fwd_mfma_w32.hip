@@ -923,6 +923,8 @@ __global__ __launch_bounds__(64 * WAVES, D > 128 ? 1 : 8 / WAVES) void fwd_w32_k
   MaskArgs ma = mask_args_of(p);
   if constexpr (MASK == 2 || PATTERN) {
     if (verdict_pattern(p, ma) != PATTERN) return;
+  } else if constexpr (MASK == 3) {
+    verdict_pattern(p, ma);  // (dropout: one variant takes a bias or none, so the verdict is applied in place)
   }
   fwd_w32_body<T, D, WAVES, MASK>(p, ma);
 }

@@ -157,7 +157,7 @@ def _recover_pattern(attn_bias, is_causal, query, key, want_grad_bias=False, dro
         return attn_bias, is_causal, {}
     pat, verdict = mask_patterns.look(attn_bias, query.shape[0], query.shape[1], query.shape[2], key.shape[2])
     if pat is None:
-        if verdict is not None and dropout_p == 0.0 and query.dtype in (torch.float16, torch.bfloat16):
+        if verdict is not None and query.dtype in (torch.float16, torch.bfloat16):
             return attn_bias, is_causal, {"mask_verdict": verdict}
         return attn_bias, is_causal, {}
     if pat[0] == "all":  # (with per-batch key counts when the mask was right padding)
