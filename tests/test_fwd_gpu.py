@@ -603,6 +603,78 @@ def test_float32_matrix_op_with_key_counts(amd, gpu_device, shape):
     assert torch.equal(out2, out) and torch.equal(lse2, lse)
 
 
+F32_FEW_ROWS = [
+    # B, Hq, Hkv, L, S, E, extras
+    (8, 32, 8, 1, 1023, 128, ""),            # a decode step: the heads of a kv group as rows, keys split
+    (1, 32, 8, 1, 8192, 128, ""),
+    (2, 8, 8, 1, 700, 64, ""),               # no group: keys split only
+    (1, 4, 4, 100, 2000, 64, ""),            # a hundred rows against many keys
+    (3, 16, 4, 1, 1500, 128, "lens"),
+    (2, 16, 4, 1, 1100, 64, "key_bias"),     # a (B,1,1,S) additive padding mask
+    (2, 8, 2, 1, 900, 128, "head_bias"),     # a bias per head: the heads stay heads
+    (2, 8, 2, 1, 900, 128, "dropout"),
+    (1, 8, 2, 1, 3000, 256, ""),             # width 256
+    (2, 6, 3, 1, 40, 64, ""),                # few keys: grouped, not split
+    (8, 32, 8, 4, 1024, 128, ""),            # four rows per head: sixteen rows per kv head
+    (2, 8, 2, 5, 600, 64, "key_bias"),
+    (2, 8, 2, 5, 600, 64, "rows_first"),     # q laid out (B,L,H,E): the heads stay heads
+    (8, 32, 32, 1, 1024, 64, ""),
+]
+
+
+@pytest.mark.parametrize("case", F32_FEW_ROWS, ids=lambda c: "B%d_Hq%d_Hkv%d_L%d_S%d_E%d_%s" % c)
+def test_float32_few_query_rows(amd, gpu_device, case):
+    """Float32 with one query row per head (a decode step) or few rows against many keys: the heads of a kv
+    group run as the rows of one head and the key tiles are split over workgroups into the workspace.
+    Against the oracle, with and without the workspace (the same call unsplit)."""
+    from oracle import sdpa_math as om
+
+    B, Hq, Hkv, L, S, E, extra = case
+    dev = gpu_device
+    MFMA = amd._lib.KERNEL_MFMA
+    g = torch.Generator().manual_seed(S + E)
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=torch.float32, seed=S + E)
+    kw, bias, keep, pdrop = {}, None, None, 0.0
+    if extra == "lens":
+        lens = torch.tensor([S, 1, 777][:B])
+        kw["kv_lens"] = lens.to(torch.int32).to(dev)
+        bias = torch.where((torch.arange(S)[None] < lens[:, None])[:, None, None, :], 0.0, float("-inf")).expand(B, Hq, L, S)
+    elif extra == "key_bias":
+        bias = torch.randn(B, 1, 1, S, generator=g)
+        bias[1, ..., S // 2:] = float("-inf")
+        kw["attn_bias"] = bias.to(dev)
+    elif extra == "head_bias":
+        bias = torch.randn(1, Hq, 1, S, generator=g)
+        kw["attn_bias"] = bias.to(dev)
+    elif extra == "dropout":
+        pdrop = 0.25
+        keep = torch.rand(B, Hq, L, S, generator=g) >= pdrop
+        kw.update(dropout_p=pdrop, dropout_keep=keep.to(dev))
+    rep = Hq // Hkv
+    ro, rl = om.compute_attention(q, k.repeat_interleave(rep, 1), v.repeat_interleave(rep, 1),
+                                  None if bias is None else bias.expand(B, Hq, L, S), keep, E**-0.5, False, pdrop)
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    if extra == "rows_first":
+        qd = qd.transpose(1, 2).contiguous().transpose(1, 2)
+    out, lse = amd.sdpa_forward(qd, kd, vd, force_kernel=MFMA, **kw)
+    assert max_abs(out, ro) <= 2e-5 and max_abs(lse, rl) <= 2e-5
+    # the same call through the C ABI without a workspace: unsplit, the same numbers up to the order of the sums
+    lib = amd._lib.load()
+    real = lib.mi355_sdpa_fwd_workspace_bytes
+    need = []
+    try:
+        class _NoWorkspace:
+            def __call__(self, p):
+                need.append(real(p))
+                return 0
+        lib.mi355_sdpa_fwd_workspace_bytes = _NoWorkspace()
+        out2, lse2 = amd.sdpa_forward(qd, kd, vd, force_kernel=MFMA, **kw)
+    finally:
+        lib.mi355_sdpa_fwd_workspace_bytes = real
+    assert (need[0] > 0) == (S >= 512), need
+    assert max_abs(out2, out) <= 1e-5 and max_abs(lse2, lse) <= 1e-5
+
+
 F32_MASKED = [
     # B, Hq, Hkv, L, S, E, causal, kind of mask, kv_lens
     (2, 4, 2, 100, 160, 64, False, "f32_full", None),

@@ -310,10 +310,10 @@ int mi355_sdpa_fwd(const mi355_sdpa_fwd_params* p, void* stream) {
 
 size_t mi355_sdpa_fwd_workspace_bytes(const mi355_sdpa_fwd_params* p) {
   if (!p || p->force_kernel == MI355_SDPA_KERNEL_GENERIC) return 0;
-  if (p->dtype != MI355_SDPA_F16 && p->dtype != MI355_SDPA_BF16) return 0;
+  if (p->dtype != MI355_SDPA_F16 && p->dtype != MI355_SDPA_BF16 && p->dtype != MI355_SDPA_F32) return 0;
   if (!tensor_ok(p->q, "query") || !tensor_ok(p->k, "key") || !tensor_ok(p->v, "value") || !tensor_ok(p->out, "out")) return 0;
   if (!shapes_ok(p->q, p->k, p->v)) return 0;
-  return fwd_mfma_workspace(*p);
+  return p->dtype == MI355_SDPA_F32 ? fwd_f32_mfma_workspace(*p) : fwd_mfma_workspace(*p);
 }
 
 static bool bwd_args_ok(const mi355_sdpa_bwd_params* p) {

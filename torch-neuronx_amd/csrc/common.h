@@ -43,6 +43,7 @@ size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p);
 // float32 inputs on the float32 matrix op (f32_mfma.hip)
 bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why);
 int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s);
+size_t fwd_f32_mfma_workspace(const mi355_sdpa_fwd_params& p);  // with which the call would split its keys (0: it would not)
 bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why);
 int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s);
 size_t bwd_f32_mfma_workspace(const mi355_sdpa_bwd_params& p);

@@ -162,7 +162,15 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
       nt -= skip;
     }
   }
-  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u; };
+  // (few rows against many keys: the key tiles are split over blockIdx.y, each part leaves its normalised
+  // rows and their log-sum-exp in the workspace for fwd_f32_merge_kernel; no causal flag, no window then)
+  const int split = p.split_tiles ? blockIdx.y : 0;
+  int t_first = 0;
+  if (!FUNC && p.split_tiles) {
+    t_first = split * p.split_tiles;
+    nt = max(min(nt - t_first, p.split_tiles), 0);
+  }
+  auto tile_of = [&](int u) { return FUNC ? u + (u >= n_lead ? skip : 0) : u + t_first; };
   const int nt_w = p.causal ? min(nt, (qw0 + 31) / BT + 1 - skip) : nt;
   TileF32<D, 64 * WAVES> kn, vn;
   auto fetch = [&](int u) {
@@ -266,7 +274,9 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
     if (p.keep_scale != 0.f) inv *= p.keep_scale;
   }
   if (qrow < p.L) {
-    float* orow = (float*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
+    const int64_t prow = (((int64_t)b * p.Hq + h) * p.n_split + split) * p.L + qrow;  // (split keys: this part's row)
+    const bool part = !FUNC && p.split_tiles != 0;
+    float* orow = part ? p.part_o + prow * p.dv_real : (float*)p.out + b * p.o_sb + h * p.o_sh + (int64_t)qrow * p.o_sl;
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -275,9 +285,76 @@ __global__ __launch_bounds__(64 * WAVES, 1) void fwd_f32_kernel(FwdM p) {
         if (d < p.dv_real)
           *(f32x4*)(orow + d) = f32x4{oacc[db][g * 4] * inv, oacc[db][g * 4 + 1] * inv, oacc[db][g * 4 + 2] * inv, oacc[db][g * 4 + 3] * inv};
       }
-    if (p.lse && half == 0)
+    if (part) {
+      if (half == 0) p.part_lse[prow] = lse_row;
+    } else if (p.lse && half == 0) {
       p.lse[((int64_t)b * p.Hq + h) * p.L + qrow] = lse_row;
+    }
   }
+}
+
+// Merge of the parts of a call whose keys were split: out = sum_s w_s O_s with w_s = exp(lse_s - lse),
+// lse = log sum_s exp(lse_s).  One workgroup per query row, a thread per output column (two at widths
+// above 128); the parts' lse are read side by side and their weights left in LDS, the parts' rows are
+// requested eight at a time.
+__global__ __launch_bounds__(128) void fwd_f32_merge_kernel(FwdM p) {
+  constexpr int MAXP = 512;  // (fwd_f32_plan never makes more parts)
+  __shared__ float w_s[MAXP];
+  __shared__ float red_s[4];
+  const int64_t row = blockIdx.x;  // (b * Hq + h) * L + l
+  const int l = (int)(row % p.L);
+  const int64_t bh = row / p.L;
+  const int b = (int)(bh / p.Hq), h = (int)(bh % p.Hq);
+  const float* pl = p.part_lse + bh * p.n_split * p.L + l;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  float ls[MAXP / 128];
+  float m = -INFINITY;
+#pragma unroll
+  for (int i = 0; i < MAXP / 128; ++i) {
+    const int sp = tid + 128 * i;
+    ls[i] = sp < p.n_split ? pl[(int64_t)sp * p.L] : -INFINITY;
+    m = fmaxf(m, ls[i]);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off, 64));
+  if (lane == 0) red_s[wave] = m;
+  __syncthreads();
+  m = fmaxf(red_s[0], red_s[1]);
+  float sum = 0.f;
+#pragma unroll
+  for (int i = 0; i < MAXP / 128; ++i) {
+    const int sp = tid + 128 * i;
+    const float w = ls[i] == -INFINITY ? 0.f : __expf(ls[i] - m);  // (a part without live keys: weight 0)
+    if (sp < p.n_split) w_s[sp] = w;
+    sum += w;
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off, 64);
+  if (lane == 0) red_s[2 + wave] = sum;
+  __syncthreads();
+  sum = red_s[2] + red_s[3];
+  float acc[2] = {0.f, 0.f};
+  const int d = tid;
+  const float* po = p.part_o + (bh * p.n_split * p.L + l) * p.dv_real;
+  const int64_t part_stride = (int64_t)p.L * p.dv_real;
+  for (int s0 = 0; s0 < p.n_split; s0 += 8) {
+    float x[2][8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      const bool on = s0 + j < p.n_split && w_s[min(s0 + j, MAXP - 1)] > 0.f;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) x[i][j] = (on && d + 128 * i < p.dv_real) ? po[(s0 + j) * part_stride + d + 128 * i] : 0.f;
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+#pragma unroll
+      for (int i = 0; i < 2; ++i) acc[i] = fmaf(w_s[min(s0 + j, MAXP - 1)], x[i][j], acc[i]);
+  }
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+    if (d + 128 * i < p.dv_real)
+      ((float*)p.out)[b * p.o_sb + h * p.o_sh + (int64_t)l * p.o_sl + d + 128 * i] = sum > 0.f ? acc[i] / sum : 0.f;
+  if (d == 0 && p.lse) p.lse[row] = sum > 0.f ? m + __builtin_logf(sum) : -INFINITY;
 }
 
 template <int D, int WAVES, int MODE>
@@ -627,13 +704,38 @@ bool fwd_f32_mfma_supported(const mi355_sdpa_fwd_params& p, const char** why) {
   return true;
 }
 
-int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
-  const char* why;
-  if (!fwd_f32_mfma_supported(p, &why)) {
-    set_error("SDPA: float32 MFMA forward kernel cannot take this call: %s", why);
-    return MI355_SDPA_ERR_UNSUPPORTED;
+namespace {
+
+// Few query rows against many keys (a decode step in float32).  A single query row per head leaves 31 of
+// a wavefront's 32 rows empty and one workgroup per head walking every key: the heads of a kv group
+// become the rows of one head (they read the same K and V; a view of q, out and the log-sum-exp, nothing
+// moves) where no causal flag, functor or per-head bias tells the heads apart, and where that still
+// leaves compute units short of workgroups the key tiles are split over blockIdx.y, at least 4
+// tiles (128 keys) per part, into the caller's workspace (fwd_f32_merge_kernel adds the parts up).
+void fwd_f32_plan(FwdM& g, const mi355_sdpa_fwd_params& p, int mode) {
+  g.split_tiles = 0, g.n_split = 1;
+  const int rep = g.Hq / g.Hkv;
+  const bool plain = !g.causal && mode != 2;
+  // (several rows per head: the rows of a group's heads are one run of rows where q and out are laid
+  // out head by head, row by row; a bias must then be one per key)
+  const bool one_row = g.L == 1, runs = g.q_sh == (int64_t)g.L * g.q_sl && g.o_sh == (int64_t)g.L * g.o_sl;
+  if (plain && rep > 1 && (int64_t)rep * g.L <= 128 && (one_row || runs) && (!g.bias || (g.bias_sh == 0 && g.bias_sl == 0))) {
+    if (one_row) g.q_sl = g.q_sh, g.o_sl = g.o_sh;
+    g.q_sh *= rep, g.o_sh *= rep;
+    g.Hq = g.Hkv, g.L *= rep;
   }
-  FwdM g;
+  const int nt = (g.S + BT - 1) / BT;
+  const int64_t groups = (int64_t)g.B * g.Hq;
+  if (plain && g.L <= 128 && groups < 1024 && nt >= 16) {  // (up to about four workgroups per compute unit)
+    const int want = (int)std::min<int64_t>(std::min<int64_t>((1024 + groups - 1) / groups, 512), nt / 4);
+    if (want > 1) {
+      g.split_tiles = (nt + want - 1) / want;
+      g.n_split = (nt + g.split_tiles - 1) / g.split_tiles;
+    }
+  }
+}
+
+void fwd_f32_fill(FwdM& g, const mi355_sdpa_fwd_params& p, int& mode) {
   g.q = p.q.data, g.k = p.k.data, g.v = p.v.data, g.out = p.out.data, g.lse = p.lse;
   g.q_sb = p.q.stride[0], g.q_sh = p.q.stride[1], g.q_sl = p.q.stride[2];
   g.k_sb = p.k.stride[0], g.k_sh = p.k.stride[1], g.k_sl = p.k.stride[2];
@@ -648,12 +750,43 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   g.window = p.mask.window, g.sink_keys = p.mask.sink_keys, g.sink_logit = p.mask.sink_logit;
   g.n_sinks = p.mask.n_sink_logits > 0 ? p.mask.n_sink_logits : 1;
   g.sm = score_mod_of(p.mask);
-  const int mode = (g.bias != nullptr || g.keep_scale != 0.f) ? 1 : (g.window > 0 || g.sink_logit || g.sm.any) ? 2 : 0;
+  mode = (g.bias != nullptr || g.keep_scale != 0.f) ? 1 : (g.window > 0 || g.sink_logit || g.sm.any) ? 2 : 0;
+  fwd_f32_plan(g, p, mode);
+}
+
+}  // namespace
+
+size_t fwd_f32_mfma_workspace(const mi355_sdpa_fwd_params& p) {
+  const char* why;
+  if (!fwd_f32_mfma_supported(p, &why)) return 0;
+  FwdM g;
+  int mode;
+  fwd_f32_fill(g, p, mode);
+  if (!g.split_tiles) return 0;
+  return (size_t)g.B * g.Hq * g.n_split * g.L * (g.dv_real + 1) * sizeof(float);
+}
+
+int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
+  const char* why;
+  if (!fwd_f32_mfma_supported(p, &why)) {
+    set_error("SDPA: float32 MFMA forward kernel cannot take this call: %s", why);
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
+  FwdM g;
+  int mode;
+  fwd_f32_fill(g, p, mode);
+  if (g.split_tiles) {  // (the caller's workspace: too small, misaligned or absent, and the call runs unsplit)
+    const size_t rows = (size_t)g.B * g.Hq * g.n_split * g.L;
+    if (p.workspace && ((uintptr_t)p.workspace & 255) == 0 && g.n_split <= 512 && p.workspace_bytes >= rows * (g.dv_real + 1) * sizeof(float))
+      g.part_o = (float*)p.workspace, g.part_lse = g.part_o + rows * g.dv_real;
+    else
+      g.split_tiles = 0, g.n_split = 1;
+  }
   // rows per workgroup: 128 (a workgroup is one wavefront per 32 rows; 64- and 32-row workgroups
   // measured slower even when 128-row ones leave compute units without work)
   const int waves = pick_waves((int64_t)g.B * g.Hq, g.L);
   g.n_qt = (g.L + 32 * waves - 1) / (32 * waves);
-  const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt)), block(64 * waves);
+  const dim3 grid((unsigned)((int64_t)g.B * g.Hq * g.n_qt), (unsigned)g.n_split), block(64 * waves);
   // (width 256: both tiles in the launch's dynamic LDS)
 #define LAUNCH(DD, WW, MM)                                                                                       \
   do {                                                                                                           \
@@ -679,7 +812,10 @@ int launch_fwd_f32_mfma(const mi355_sdpa_fwd_params& p, hipStream_t s) {
   else LAUNCH_W(256);
 #undef LAUNCH_W
 #undef LAUNCH
-  return check_launch("fwd_f32_kernel");
+  const int rc = check_launch("fwd_f32_kernel");
+  if (rc != MI355_SDPA_OK || !g.split_tiles) return rc;
+  hipLaunchKernelGGL(fwd_f32_merge_kernel, dim3((unsigned)((int64_t)g.B * g.Hq * g.L)), dim3(128), 0, s, g);
+  return check_launch("fwd_f32_merge_kernel");
 }
 
 bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
