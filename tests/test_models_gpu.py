@@ -211,3 +211,26 @@ def test_torch_nn_attention_modules_match_the_stock_kernels(amd, gpu_device, lib
     assert float((o1 - o0).abs().max()) <= 1e-5 * max(1.0, float(o0.abs().max()))
     if train:
         assert float((g1 - g0).norm() / g0.norm()) <= 1e-5
+
+
+def test_a_compiled_model_reaches_the_library_and_matches_eager(amd, gpu_device, library_calls):
+    """A whole model under ``torch.compile`` (default backend), float32, padded batch: the generated code
+    calls the registered operators - it asserts their output shapes and strides on the way - once per layer
+    and direction, and loss and gradients are the eager ones."""
+    dev = gpu_device
+    torch.manual_seed(1)
+    model = _llama().to(dev).train()
+    ids = torch.randint(1, 1000, (4, 256), device=dev)
+    am = torch.ones_like(ids)
+    am[1, 200:] = 0
+    am[3, 100:] = 0
+    inputs = dict(input_ids=ids, labels=ids, attention_mask=am)
+    l0, g0 = _step(model, inputs)
+    before = dict(library_calls)
+    torch._dynamo.reset()
+    try:
+        l1, g1 = _step(torch.compile(model), inputs)
+    finally:
+        torch._dynamo.reset()
+    assert library_calls["fwd"] - before["fwd"] == 2 and library_calls["bwd"] - before["bwd"] == 2, library_calls
+    assert abs(float(l1 - l0)) <= 1e-5 and float((g1 - g0).norm() / g0.norm()) <= 1e-5
