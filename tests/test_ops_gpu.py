@@ -561,6 +561,12 @@ def test_replaced_upstream_operators_keep_upstream_layouts_and_redraw_the_dropou
     with torch.no_grad():  # (no backward can follow: nothing is kept)
         F.scaled_dot_product_attention(qr, kr, vr, dropout_p=p)
     assert len(impl._kept) == 0
+    out = F.scaled_dot_product_attention(qr, kr, vr, dropout_p=p)  # a forward whose backward never comes ...
+    assert len(impl._kept) == 1
+    del out  # ... gives its mask back when its graph goes
+    import gc
+    gc.collect()
+    assert len(impl._kept) == 0
 
 
 def test_calls_can_be_captured_in_a_graph_and_replayed(amd, gpu_device):

@@ -12,6 +12,7 @@ from __future__ import annotations
 
 import math
 import os
+import weakref
 from collections import OrderedDict
 
 import torch
@@ -106,14 +107,17 @@ def _seeded_keep(query, S, dropout_p, remember):
     gen = torch.cuda.default_generators[index]
     seed, offset = gen.initial_seed(), gen.get_offset()
     keep = _dropout_keep(query, S, dropout_p)
+    seed_t = torch.tensor(seed - (1 << 64) if seed >= 1 << 63 else seed, dtype=torch.int64)  # (a 64-bit seed in an int64 tensor)
     if remember:
-        _kept[(index, seed, offset, tuple(keep.shape), dropout_p)] = keep
+        key = (index, seed, offset, tuple(keep.shape), dropout_p)
+        _kept[key] = keep
+        # (the seed tensor lives as long as the graph that saved it: a forward whose backward never comes
+        # gives its mask back when its graph goes)
+        weakref.finalize(seed_t, _kept.pop, key, None)
         held = sum(t.numel() for t in _kept.values())
         while len(_kept) > 1 and (held > _KEPT_MAX_BYTES or len(_kept) > _KEPT_MAX_ENTRIES):
             held -= _kept.popitem(last=False)[1].numel()
-    if seed >= 1 << 63:
-        seed -= 1 << 64  # (a 64-bit seed in an int64 tensor)
-    return keep, torch.tensor(seed, dtype=torch.int64), torch.tensor(offset, dtype=torch.int64)
+    return keep, seed_t, torch.tensor(offset, dtype=torch.int64)
 
 
 def _keep_again(query, S, dropout_p, philox_seed, philox_offset, take=True):
