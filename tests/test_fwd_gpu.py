@@ -675,6 +675,31 @@ def test_float32_few_query_rows(amd, gpu_device, case):
     assert max_abs(out2, out) <= 1e-5 and max_abs(lse2, lse) <= 1e-5
 
 
+@pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float32])
+def test_split_key_merge_ignores_what_earlier_kernels_left_in_lds(amd, gpu_device, dtype):
+    """The merge of a call with split keys keeps the parts' weights in LDS and adds the parts eight at a
+    time: the slots past the last part must count as zero whatever an earlier kernel left there (a NaN
+    times the zero of an absent part is a NaN).  Reductions over NaN tensors run first, on every compute
+    unit; few parts (four), so that most of the eight slots are unused."""
+    dev = gpu_device
+    B, Hq, Hkv, L, S, E = 2, 96, 8, 32, 1100, 256
+    if dtype is torch.float32:
+        B, Hq, Hkv, L, S, E = 8, 32, 8, 1, 520, 128
+    q, k, v = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=11)
+    lens = torch.tensor(([546, 1064] if dtype is torch.bfloat16 else [520] * B), dtype=torch.int32)
+    keep = (torch.arange(S)[None] < lens[:, None])[:, None, None, :].expand(B, 1, L, S)
+    ro, rl = oracle_fwd(q, k, v, attn_mask=keep)
+    qd, kd, vd, ld = q.to(dev), k.to(dev), v.to(dev), lens.to(dev)
+    poison = torch.full((1 << 24,), float("nan"), device=dev)
+    for _ in range(5):
+        poison.view(4096, -1).sum(1)
+        torch.softmax(poison.view(8192, -1), dim=1)
+        torch.cumsum(poison.view(16384, -1), dim=1)
+        out, lse = amd.sdpa_forward(qd, kd, vd, kv_lens=ld, force_kernel=amd._lib.KERNEL_MFMA)
+        assert torch.isfinite(out.float()).all()
+        assert max_abs(out, ro) <= (2e-2 if dtype is torch.bfloat16 else 2e-5) and max_abs(lse, rl) <= 2e-3
+
+
 F32_MASKED = [
     # B, Hq, Hkv, L, S, E, causal, kind of mask, kv_lens
     (2, 4, 2, 100, 160, 64, False, "f32_full", None),

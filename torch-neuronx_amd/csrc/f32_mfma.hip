@@ -325,7 +325,7 @@ __global__ __launch_bounds__(128) void fwd_f32_merge_kernel(FwdM p) {
   for (int i = 0; i < MAXP / 128; ++i) {
     const int sp = tid + 128 * i;
     const float w = ls[i] == -INFINITY ? 0.f : __expf(ls[i] - m);  // (a part without live keys: weight 0)
-    if (sp < p.n_split) w_s[sp] = w;
+    w_s[sp] = w;  // (every slot: the loop below multiplies the slots past the last part by a zero, which a stale NaN would survive)
     sum += w;
   }
 #pragma unroll
@@ -348,7 +348,7 @@ __global__ __launch_bounds__(128) void fwd_f32_merge_kernel(FwdM p) {
 #pragma unroll
     for (int j = 0; j < 8; ++j)
 #pragma unroll
-      for (int i = 0; i < 2; ++i) acc[i] = fmaf(w_s[min(s0 + j, MAXP - 1)], x[i][j], acc[i]);
+      for (int i = 0; i < 2; ++i) acc[i] = fmaf(s0 + j < p.n_split ? w_s[min(s0 + j, MAXP - 1)] : 0.f, x[i][j], acc[i]);
   }
 #pragma unroll
   for (int i = 0; i < 2; ++i)
