@@ -185,41 +185,19 @@ __global__ __launch_bounds__(1024) void mask_verdict_kernel(VerdictArgs a) {
     for (int w = 1; w < 16; ++w) r = max(r, red_s[w]);
     return r;
   };
-  if (windows) {
-    for (int bm = tid; bm < a.Bm; bm += 1024) a.n_win[bm] = -1;
-    __syncthreads();
-  }
   int ok_all = 1, ok_causal = windows, ok_mask = 1;
-  for (int64_t base = 0; base < pairs; base += 1024) {  // (every thread makes every trip: the wavefront votes below)
-    const int64_t idx = base + tid;
-    const bool valid = idx < pairs;
-    int bm = -1, top = -1;
-    if (valid) {
-      bm = (int)(idx / Lm);
-      const int i = (int)(idx - (int64_t)bm * Lm);
-      const int hi_last = a.rows[((int64_t)bm * Lm + Lm - 1) * 4];
-      const int n_all = hi_last + 1;
-      const int n_causal = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;  // the last row reaches its diagonal: no key is known to be padding
-      const int32_t* row = a.rows + idx * 4;
-      const int hi = row[0], cnt = row[1], lo = row[3];
-      if (cnt < 0) ok_mask = 0;
-      if (lo != 0 || hi != n_all - 1 || cnt != n_all) ok_all = 0;
-      const int hc = min(min(i, S - 1), n_causal - 1);
-      if (lo != 0 || hi != hc || cnt != hc + 1) ok_causal = 0;
-      top = hi;
-    }
-    // (for the window pattern below: the keys of a batch are those up to the last one any of its rows
-    // keeps; a wavefront whose rows belong to one batch, the usual case, adds its maximum once)
-    if (windows) {
-      const int bm0 = __builtin_amdgcn_readfirstlane(bm);
-      if (__builtin_amdgcn_ballot_w64(bm == bm0) == ~0ull) {
-#pragma unroll
-        for (int o = 32; o > 0; o >>= 1) top = max(top, __shfl_xor(top, o, 64));
-        if ((tid & 63) == 0 && bm0 >= 0 && top >= 0) atomicMax(&a.n_win[bm0], top);
-      } else if (valid && top >= 0) {
-        atomicMax(&a.n_win[bm], top);
-      }
-    }
+  const int npairs = (int)pairs;  // (verdict_shape keeps it below 2^29)
+  for (int idx = tid; idx < npairs; idx += 1024) {
+    const int bm = (int)((unsigned)idx / (unsigned)Lm), i = idx - bm * Lm;
+    const int hi_last = a.rows[((int64_t)bm * Lm + Lm - 1) * 4];
+    const int n_all = hi_last + 1;
+    const int n_causal = hi_last == min(L - 1, S - 1) ? S : hi_last + 1;  // the last row reaches its diagonal: no key is known to be padding
+    const int32_t* row = a.rows + (int64_t)idx * 4;
+    const int hi = row[0], cnt = row[1], lo = row[3];
+    if (cnt < 0) ok_mask = 0;
+    if (lo != 0 || hi != n_all - 1 || cnt != n_all) ok_all = 0;
+    const int hc = min(min(i, S - 1), n_causal - 1);
+    if (lo != 0 || hi != hc || cnt != hc + 1) ok_causal = 0;
   }
   ok_mask = __syncthreads_and(ok_mask);
   ok_all = __syncthreads_and(ok_all) && ok_mask;
@@ -230,6 +208,24 @@ __global__ __launch_bounds__(1024) void mask_verdict_kernel(VerdictArgs a) {
     // keeps the keys of i-W+1 .. i and of the first N that lie below n (all S keys when some row reaches
     // the last diagonal element).  W and N are read where they show: in the last row that has keys of
     // its own, in the (first) batch with the most keys.
+    // (the keys of a batch are those up to the last one any of its rows keeps: a maximum per batch, for
+    // which a wavefront whose rows belong to one batch, the usual case, adds its own once)
+    for (int bm = tid; bm < a.Bm; bm += 1024) a.n_win[bm] = -1;
+    __syncthreads();
+    for (int base = 0; base < npairs; base += 1024) {  // (every thread makes every trip: the wavefront votes)
+      const int idx = base + tid;
+      const int bm = idx < npairs ? (int)((unsigned)idx / (unsigned)Lm) : -1;
+      int top = idx < npairs ? a.rows[(int64_t)idx * 4] : -1;
+      const int bm0 = __builtin_amdgcn_readfirstlane(bm);
+      if (__builtin_amdgcn_ballot_w64(bm == bm0) == ~0ull) {
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) top = max(top, __shfl_xor(top, o, 64));
+        if ((tid & 63) == 0 && bm0 >= 0 && top >= 0) atomicMax(&a.n_win[bm0], top);
+      } else if (bm >= 0 && top >= 0) {
+        atomicMax(&a.n_win[bm], top);
+      }
+    }
+    __syncthreads();
     int n_mine = 0;
     for (int bm = tid; bm < a.Bm; bm += 1024) {
       const int top = a.n_win[bm];
@@ -249,10 +245,10 @@ __global__ __launch_bounds__(1024) void mask_verdict_kernel(VerdictArgs a) {
       W = hi_r - lo_r + 1, N = lead_r < lo_r ? lead_r : 0;
       ok = W > 0 && lo_r != 0;
     }
-    for (int64_t idx = tid; idx < pairs && ok; idx += 1024) {
-      const int bm = (int)(idx / Lm), i = (int)(idx - (int64_t)bm * Lm);
+    for (int idx = tid; idx < npairs && ok; idx += 1024) {
+      const int bm = (int)((unsigned)idx / (unsigned)Lm), i = idx - bm * Lm;
       const int n = a.n_win[bm];
-      const int32_t* row = a.rows + idx * 4;
+      const int32_t* row = a.rows + (int64_t)idx * 4;
       const int hi = row[0], cnt = row[1], lead = row[2], lo = row[3];
       const int top = min(min(i, S - 1), n - 1), lo_w = max(i - W + 1, 0);
       int e_hi, e_cnt, e_lead, e_lo = 0;
