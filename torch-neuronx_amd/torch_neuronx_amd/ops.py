@@ -336,7 +336,7 @@ def sdpa_forward(query, key, value, attn_bias=None, is_causal=False, scale=None,
     if mask_verdict is not None:
         p.mask.mask_verdict = mask_verdict.data_ptr()
     ws = None
-    if L <= 32 or L * (Hq // max(key.shape[1], 1)) <= 256:
+    if L <= 128:
         # few query rows: the library may want to split the keys over more workgroups
         need = _lib.load().mi355_sdpa_fwd_workspace_bytes(C.byref(p))
         if need:
