@@ -355,7 +355,8 @@ static int bwd_kernel_choice(const mi355_sdpa_bwd_params* p, bool log = false) {
 size_t mi355_sdpa_bwd_workspace_bytes(const mi355_sdpa_bwd_params* p) {
   if (!p) return 0;
   // sized for either kernel so the host can allocate before the choice is visible to it
-  return std::max(bwd_generic_workspace(*p), std::max(bwd_mfma_workspace(*p), bwd_f32_mfma_workspace(*p)));
+  const size_t mfma = p->dtype == MI355_SDPA_F32 ? bwd_f32_mfma_workspace(*p) : bwd_mfma_workspace(*p);
+  return std::max(bwd_generic_workspace(*p), mfma);
 }
 
 int mi355_sdpa_bwd(const mi355_sdpa_bwd_params* p, void* stream) {

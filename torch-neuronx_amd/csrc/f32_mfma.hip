@@ -545,6 +545,13 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   const int qs_begin = p.causal ? min(k0 / BT, nqs) : 0;
   // items: (query head of the group, 32-row query tile)
   const int per_head = nqs - qs_begin, n_items = rep * per_head;
+  // (few key blocks: the items of a key block are shared out over p.parts workgroups, blockIdx.y, which
+  // leave their rows in the workspace for bwd_f32_dkdv_merge_kernel)
+  int it0 = 0, it1 = n_items;
+  if (p.parts > 1) {
+    const int chunk = (n_items + p.parts - 1) / p.parts;
+    it0 = min((int)blockIdx.y * chunk, n_items), it1 = min(it0 + chunk, n_items);
+  }
   TileF32<D, 64 * WAVES> qn, gn;
   float lse_n = INFINITY, dl_n = 0.f;
   auto fetch_item = [&](int it) {
@@ -564,16 +571,16 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
       dl_n = qi < p.L ? p.delta[row] : 0.f;
     }
   };
-  if (kFetchAhead<D> && n_items > 0) fetch_item(0);
+  if (kFetchAhead<D> && it1 > it0) fetch_item(it0);
   {
-    for (int it = 0; it < n_items; ++it) {
+    for (int it = it0; it < it1; ++it) {
       const int q0 = (nqs - 1 - it / rep) * BT;
       __syncthreads();
       if constexpr (kFetchAhead<D>) qn.put(q_t, tid), gn.put(do_t, tid);
       else fetch_item(it);
       if (tid < BT) lse_s[tid] = lse_n, dl_s[tid] = dl_n;
       __syncthreads();
-      if (kFetchAhead<D> && it + 1 < n_items) fetch_item(it + 1);
+      if (kFetchAhead<D> && it + 1 < it1) fetch_item(it + 1);
       if ((p.causal && q0 + BT - 1 < kw0) || kw0 >= S) continue;  // (uniform per wavefront)
       if constexpr (FUNC) {  // every row of the tile lies past the window of every key of this wavefront, none of them a sink
         if (p.window > 0 && q0 - (kw0 + 31) >= p.window && kw0 >= p.sink_keys) continue;
@@ -640,6 +647,10 @@ __global__ __launch_bounds__(64 * WAVES, 1) void bwd_f32_dkdv_kernel(BwdM p) {
   if (key < p.S) {
     float* gk = (float*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
     float* gv = (float*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl;
+    if (p.parts > 1) {  // (this part's rows: (part, batch, kv head, key) x real columns, every part written)
+      const int64_t row = (int64_t)blockIdx.y * p.B * p.Hkv * p.S + ((int64_t)b * p.Hkv + hk) * p.S + key;
+      gk = p.part_dk + row * p.d_real, gv = p.part_dv + row * p.dv_real;
+    }
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
@@ -841,8 +852,48 @@ bool bwd_f32_mfma_supported(const mi355_sdpa_bwd_params& p, const char** why) {
   return true;
 }
 
+namespace {
+
+// dK and dV of a call whose key blocks were shared out over several workgroups: the sum of the parts'
+// rows, one 64-thread block per key row of a (batch, kv head), four columns per thread.
+__global__ __launch_bounds__(64) void bwd_f32_dkdv_merge_kernel(BwdM p) {
+  const int64_t row = blockIdx.x;  // (b * Hkv + hk) * S + key
+  const int key = (int)(row % p.S), hk = (int)((row / p.S) % p.Hkv), b = (int)(row / ((int64_t)p.S * p.Hkv));
+  const int64_t rows = (int64_t)p.B * p.Hkv * p.S;
+  for (int c = threadIdx.x * 4; c < p.d_real + p.dv_real; c += 64 * 4) {
+    const bool is_v = c >= p.d_real;
+    const int col = is_v ? c - p.d_real : c, width = is_v ? p.dv_real : p.d_real;
+    const float* src = (is_v ? p.part_dv : p.part_dk) + row * width + col;
+    f32x4 a = {0.f, 0.f, 0.f, 0.f};
+    for (int i = 0; i < p.parts; ++i) a += *(const f32x4*)(src + i * rows * width);
+    float* g = is_v ? (float*)p.gv + b * p.gv_sb + hk * p.gv_sh + (int64_t)key * p.gv_sl
+                    : (float*)p.gk + b * p.gk_sb + hk * p.gk_sh + (int64_t)key * p.gk_sl;
+    *(f32x4*)(g + col) = a;
+  }
+}
+
+// Few key blocks (one or a few kv heads, a small batch, short keys) leave most compute units without a
+// workgroup of the dK/dV kernel while each one walks every query head of its group: the items of a key
+// block (query head x 32-row tile) are then shared out over several workgroups, at least four items
+// each, about four workgroups per compute unit in all (a compute unit holds one at a time: the
+// later ones even out what a causal mask leaves uneven).
+int bwd_f32_parts(const mi355_sdpa_bwd_params& p) {
+  const int64_t B = p.q.size[0], Hq = p.q.size[1], L = p.q.size[2], Hkv = p.k.size[1], S = p.k.size[2];
+  const int64_t kgrid = B * Hkv * ((S + 127) / 128) * (p.q.size[3] > 128 ? 2 : 1);
+  const int64_t items = (Hq / Hkv) * ((L + BT - 1) / BT);
+  if (kgrid >= 512 || items < 8) return 1;
+  return (int)std::max<int64_t>(std::min<int64_t>(std::min<int64_t>((1024 + kgrid - 1) / kgrid, items / 4), 32), 1);
+}
+
+}  // namespace
+
 size_t bwd_f32_mfma_workspace(const mi355_sdpa_bwd_params& p) {
-  return (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float);  // delta and lse2
+  size_t bytes = (size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float);  // delta and lse2
+  bytes = (bytes + 255) & ~(size_t)255;
+  const int parts = bwd_f32_parts(p);
+  if (parts > 1)  // the parts' float32 rows of dK and dV
+    bytes += (size_t)parts * p.k.size[0] * p.k.size[1] * p.k.size[2] * (p.q.size[3] + p.v.size[3]) * sizeof(float);
+  return bytes;
 }
 
 int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
@@ -879,10 +930,20 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
     g.gbias_sb = p.grad_bias.stride[0], g.gbias_sh = p.grad_bias.stride[1], g.gbias_sl = p.grad_bias.stride[2];
   }
   const int mode = (g.bias != nullptr || g.keep_scale != 0.f) ? 1 : (g.window > 0 || g.sm.any) ? 2 : 0;
+  g.parts = bwd_f32_parts(p);
+  if (g.parts > 1) {  // (the parts' rows lie behind the two row vectors, 256-byte aligned)
+    const size_t head = ((size_t)(p.q.size[0] * p.q.size[1] * p.q.size[2]) * 2 * sizeof(float) + 255) & ~(size_t)255;
+    if (p.workspace_bytes < bwd_f32_mfma_workspace(p)) {
+      g.parts = 1;
+    } else {
+      g.part_dk = (float*)((char*)p.workspace + head);
+      g.part_dv = g.part_dk + (size_t)g.parts * g.B * g.Hkv * g.S * g.d_real;
+    }
+  }
   const int qw = pick_waves((int64_t)g.B * g.Hq, g.L), kw = pick_waves((int64_t)g.B * g.Hkv, g.S);
   const dim3 qgrid((unsigned)((int64_t)g.B * g.Hq * ((g.L + 32 * qw - 1) / (32 * qw))));
   // (width 256: two workgroups per key block, one per half of the columns of dK / dV)
-  const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw)) * (g.d_real > 128 ? 2 : 1)));
+  const dim3 kgrid((unsigned)((int64_t)g.B * g.Hkv * ((g.S + 32 * kw - 1) / (32 * kw)) * (g.d_real > 128 ? 2 : 1)), (unsigned)g.parts);
 #define LAUNCH(KK, GRID, DD, WW, MM)                                                                             \
   do {                                                                                                           \
     constexpr int kLds = DD > 128 ? 2 * kTileFloats<DD> * (int)sizeof(float) : 0;                                \
@@ -913,6 +974,10 @@ int launch_bwd_f32_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
 #undef LAUNCH_W
 #undef LAUNCH
   rc = check_launch("bwd_f32_dkdv_kernel");
+  if (rc == MI355_SDPA_OK && g.parts > 1) {
+    hipLaunchKernelGGL(bwd_f32_dkdv_merge_kernel, dim3((unsigned)((int64_t)g.B * g.Hkv * g.S)), dim3(64), 0, s, g);
+    rc = check_launch("bwd_f32_dkdv_merge_kernel");
+  }
   if (rc == MI355_SDPA_OK && p.grad_sink_logit && p.mask.sink_logit)
     rc = launch_sink_grad(p.lse, g.delta, p.mask.sink_logit, p.grad_sink_logit, (int64_t)g.B * g.Hq, g.L, p.mask.n_sink_logits, s);
   return rc;
