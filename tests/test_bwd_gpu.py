@@ -424,6 +424,41 @@ def test_dropout_over_197_keys_through_the_operators(amd, gpu_device, monkeypatc
             assert max_abs(a, c) <= (1e-2 if half else 3e-5)
 
 
+DQ_SPLITS = [
+    # B, Hq, Hkv, L, S, E, causal, kv_lens
+    (1, 16, 16, 128, 8192, 128, False, None),
+    (2, 8, 8, 100, 20000, 32, False, None),      # a hundred object queries over an image's tokens
+    (4, 16, 4, 64, 4096, 64, False, [4096, 100, 2049, 0]),
+    (1, 4, 2, 300, 6000, 128, True, None),       # causal, top-left: the parts behind the diagonal are empty
+    (1, 32, 8, 64, 8192, 128, False, None),
+]
+
+
+@pytest.mark.parametrize("case", DQ_SPLITS, ids=lambda c: "B%d_Hq%d_Hkv%d_L%d_S%d_E%d_c%d" % c[:7])
+def test_few_query_rows_against_many_keys_split_the_keys_of_the_dq_kernel(amd, gpu_device, monkeypatch, case):
+    """Cross attention over a long memory in the backward: the dQ kernel's few workgroups split their keys
+    into parts (float32 rows in the workspace, added up by a second kernel).  Against the oracle."""
+    B, Hq, Hkv, L, S, E, causal, lens = case
+    dev = gpu_device
+    dtype = torch.bfloat16
+    q, k, v, go = qkv(B, Hq, Hkv, L, S, E, dtype=dtype, seed=L + S, with_do=True)
+    go = (go.float().clamp(-1, 1) * 0.1).to(dtype)
+    kw, om_mask = {}, None
+    if lens is not None:
+        kw["kv_lens"] = torch.tensor(lens, dtype=torch.int32, device=dev)
+        om_mask = (torch.arange(S)[None] < torch.tensor(lens)[:, None])[:, None, None, :]
+    lib = amd._lib.load()
+    real, asked = lib.mi355_sdpa_bwd_workspace_bytes, []
+    monkeypatch.setattr(lib, "mi355_sdpa_bwd_workspace_bytes", lambda p: (asked.append(real(p)), asked[-1])[1])
+    out, lse, dq, dk, dv, _ = _fwd_bwd(amd, dev, q, k, v, go, MFMA, is_causal=causal, **kw)
+    row_terms = (B * Hq * L * 2 * 4 + 255) // 256 * 256
+    assert asked[-1] >= row_terms + 2 * B * Hq * L * E * 4, (asked, row_terms)  # (at least two parts of dQ rows)
+    ro, rl, rdq, rdk, rdv = _reference(q, k, v, go, attn_mask=om_mask, is_causal=causal)
+    for a, r in ((dq, rdq), (dk, rdk), (dv, rdv)):
+        assert torch.isfinite(a.float()).all()
+        assert max_abs(a, r) <= 2e-2 * max(1.0, r.abs().max().item()) and rel_err(a, r) <= 2e-2
+
+
 def test_backward_kv_lens(amd, gpu_device):
     q, k, v, go = qkv(3, 4, 2, 5, 64, 32, dtype=torch.float32, seed=4, with_do=True)
     lens = torch.tensor([64, 1, 17], dtype=torch.int32)

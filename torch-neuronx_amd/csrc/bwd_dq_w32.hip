@@ -135,8 +135,20 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   if constexpr (MASK) {
     if (ma.kv_lens) S = min(S, max(ma.kv_lens[b], 0));
   }
+  // (split keys, variant with key counts only: this workgroup's part and its rows in the workspace)
+  const bool parted = MASK == 1 && p.dq_split_tiles != 0;
+  const int split = parted ? (int)blockIdx.y : 0;
+  float* const part_row = parted ? p.part_dq + (((int64_t)split * p.B * p.Hq + (int64_t)b * p.Hq + h) * p.L + qc) * dr : nullptr;
   auto zero_row = [&]() {  // no live key: zero gradient
     zero_gbias(0);
+    if (parted) {  // (every part writes its rows: the merge adds them all)
+      if (qrow < p.L) {
+#pragma unroll
+        for (int i = 0; i < D / 8; ++i)
+          if (half * (D / 2) + i * 4 < dr) *(f32x4*)(part_row + half * (D / 2) + i * 4) = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+      return;
+    }
     if (qrow < p.L) {
       uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
@@ -181,10 +193,18 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
         t_lo = max(t_lo, run[0] / BN);
       }
     }
+    if (parted) t_lo = split * p.dq_split_tiles;  // (no window in such a call: the part's first tile)
     if (t_lo > 0) {
       n_lead = min(min(ma.window > 0 ? (ma.sink_keys + BN - 1) / BN : 0, t_lo), nt);
       skip = min(t_lo, nt) - n_lead;
       nt -= skip;
+    }
+    if (parted) {
+      nt = min(nt, p.dq_split_tiles);
+      if (nt <= 0) {  // (a part behind the keys of this batch, or above the causal diagonal of these rows)
+        zero_row();
+        return;
+      }
     }
     if constexpr (SMOD) {
       if (nt <= 0) {  // (the document ids leave this workgroup's rows without a key)
@@ -694,6 +714,20 @@ __device__ __forceinline__ void bwd_dq_w32_body(const BwdM& p, const MaskArgs ma
   }
   zero_gbias(nt_w);
 
+  if (parted) {
+    if (qrow < p.L) {
+#pragma unroll
+      for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const int d = db * 32 + g * 8 + half * 4;
+          if (d < dr)
+            *(f32x4*)(part_row + d) = f32x4{dqacc[db][g * 4] * p.scale, dqacc[db][g * 4 + 1] * p.scale, dqacc[db][g * 4 + 2] * p.scale,
+                                            dqacc[db][g * 4 + 3] * p.scale};
+        }
+    }
+    return;
+  }
   if (qrow < p.L) {
     uint16_t* gq = (uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)qrow * p.gq_sl;
 #pragma unroll
@@ -723,6 +757,24 @@ __global__ __launch_bounds__(512, 1) void bwd_dq_w32_kernel(BwdM p) {
   bwd_dq_w32_body<T, D, MASK>(p, ma);
 }
 
+// dQ of a call whose keys were split: the sum of the parts' float32 rows, rounded once.  One 64-thread
+// block per query row, four columns per thread.
+template <typename T>
+__global__ __launch_bounds__(64) void bwd_dq_merge_kernel(BwdM p) {
+  const int64_t row = blockIdx.x;  // (b * Hq + h) * L + l
+  const int l = (int)(row % p.L), h = (int)((row / p.L) % p.Hq), b = (int)(row / ((int64_t)p.L * p.Hq));
+  const int64_t rows = (int64_t)p.B * p.Hq * p.L;
+  const int c = threadIdx.x * 4;
+  if (c >= p.d_real) return;
+  const float* src = p.part_dq + row * p.d_real + c;
+  f32x4 a = {0.f, 0.f, 0.f, 0.f};
+  for (int i = 0; i < p.dq_n_split; ++i) a += *(const f32x4*)(src + i * rows * p.d_real);
+  u32x2 w;
+  w[0] = Mma<T>::pack(a[0], a[1]);
+  w[1] = Mma<T>::pack(a[2], a[3]);
+  *(u32x2*)((uint16_t*)p.gq + b * p.gq_sb + h * p.gq_sh + (int64_t)l * p.gq_sl + c) = w;
+}
+
 }  // namespace
 
 bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
@@ -733,7 +785,7 @@ bool bwd_dq_w32_fits(const BwdM& g, int head_dim) {
 
 int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
   const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + BM - 1) / BM);
-  const dim3 grid((unsigned)blocks), block(512);
+  const dim3 grid((unsigned)blocks, (unsigned)(g.dq_split_tiles ? g.dq_n_split : 1)), block(512);
   const bool bf = dtype == MI355_SDPA_BF16;
   if (g.sm.any && (g.keep_scale != 0.f || g.bias_kind || g.gbias)) {
     set_error("SDPA: score functors in bwd_dq_w32_kernel need a call without bias and dropout");
@@ -743,7 +795,11 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
     set_error("SDPA: dropout in bwd_dq_w32_kernel needs a keep-mask and no tile table");
     return MI355_SDPA_ERR_UNSUPPORTED;
   }
-  const int mask = g.sm.any ? 4 : g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0) ? 1 : 0;
+  const int mask = g.sm.any ? 4 : g.keep_scale != 0.f ? 3 : (g.bias_kind || g.gbias) ? 2 : (g.kv_lens || g.d_real != head_dim || g.window > 0 || g.dq_split_tiles) ? 1 : 0;
+  if (g.dq_split_tiles && (mask != 1 || g.window > 0 || !g.part_dq)) {
+    set_error("SDPA: split keys in bwd_dq_w32_kernel need a call without bias, dropout, functors and window, and a workspace");
+    return MI355_SDPA_ERR_UNSUPPORTED;
+  }
   // (the tiles, the tile list of a call with a skip table, 4 KB of bias tile per wavefront)
   const int dyn = (mask == 2 || mask == 3) ? 2 * 4 * BN * head_dim * 2 + 2080 + 8 * 4096 + (mask == 3 ? 8 * 1024 : 0) : 0;
   if (mask == 2 || mask == 3) {
@@ -779,7 +835,12 @@ int launch_bwd_dq_w32(const BwdM& g, int dtype, int head_dim, hipStream_t s) {
 #undef LAUNCH_D
 #undef LAUNCH_M
 #undef LAUNCH
-  return check_launch("bwd_dq_w32_kernel");
+  const int rc = check_launch("bwd_dq_w32_kernel");
+  if (rc != MI355_SDPA_OK || !g.dq_split_tiles) return rc;
+  const dim3 rows((unsigned)((int64_t)g.B * g.Hq * g.L));
+  if (bf) hipLaunchKernelGGL((bwd_dq_merge_kernel<bf16_t>), rows, dim3(64), 0, s, g);
+  else hipLaunchKernelGGL((bwd_dq_merge_kernel<f16_t>), rows, dim3(64), 0, s, g);
+  return check_launch("bwd_dq_merge_kernel");
 }
 
 }  // namespace mi355

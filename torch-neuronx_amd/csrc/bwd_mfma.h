@@ -73,6 +73,12 @@ struct BwdM {
   // block with fewer items - a causal mask, a window, a batch with fewer keys - fills fewer parts;
   // the others are neither written nor read).  0: every key block uses all `parts`, in equal shares.
   int chunk_items = 0;
+  // The dQ kernel of bwd_dq_w32.hip for few query rows against many keys (cross attention over a long
+  // memory): its workgroups are (batch, head, 256 rows), too few to fill the GPU, each walking every
+  // key.  The key tiles are then split over blockIdx.y, dq_split_tiles tiles of 32 keys per part, the
+  // parts leave float32 rows (dq_n_split, B, Hq, L, d_real) in part_dq and a second kernel adds them.
+  int dq_split_tiles = 0, dq_n_split = 1;
+  float* part_dq = nullptr;
   // a verdict about the bias (mask_rows.hip), read by the variants with a per-score bias in their
   // prologue: see apply_verdict
   const int32_t* verdict = nullptr;

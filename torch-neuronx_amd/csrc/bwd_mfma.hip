@@ -478,7 +478,7 @@ int launch_td(const BwdM& g, hipStream_t s) {
   constexpr int RPB = 256 / (D / 8);
   // dQ: 256-row workgroups when D = 128 and there is at least one for every compute unit
   const int64_t wg256 = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
-  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.keep_scale != 0.f || g.kv_lens || g.gbias || g.d_real != D || g.window > 0 || g.sm.any) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
+  const bool dq_w32 = (wg256 >= 256 || g.bias_kind || g.keep_scale != 0.f || g.kv_lens || g.gbias || g.d_real != D || g.window > 0 || g.sm.any || g.dq_split_tiles) && bwd_dq_w32_fits(g, D);  // (a masked call has no other kernel)
   int rc;
   if (dq_w32) {
     // that kernel holds every row of dO in registers anyway: it goes first and leaves the row
@@ -649,13 +649,36 @@ static int parts_of(const BwdM& g, const mi355_sdpa_bwd_params& p) {
   return bwd_dkdv_w32_fits(g, p.q.size[3] <= 64 ? 64 : 128) ? bwd_dkdv_w32_parts(g) : 1;
 }
 static size_t part_rows_bytes(const BwdM& g, int parts) {  // dK rows, then dV rows
-  return parts > 1 ? (size_t)parts * g.B * g.Hkv * g.S * (g.d_real + g.dv_real) * sizeof(float) : 0;
+  const size_t bytes = parts > 1 ? (size_t)parts * g.B * g.Hkv * g.S * (g.d_real + g.dv_real) * sizeof(float) : 0;
+  return (bytes + 255) & ~(size_t)255;
+}
+// Few query rows against many keys (cross attention over a long memory): parts into which the dQ
+// kernel of bwd_dq_w32.hip splits its keys - at least 1024 keys each, about two workgroups per compute
+// unit in all - and the tiles of 32 keys per part.  1: no split (and for every call with a bias, dropout,
+// a functor, a window or a verdict, which that kernel's variant for split keys does not take).
+static int dq_splits(const BwdM& g, const mi355_sdpa_bwd_params& p, int* split_tiles) {
+  *split_tiles = 0;
+  if (p.q.size[3] > 128 || p.v.size[3] != p.q.size[3] || g.bias_kind || g.gbias || g.keep_scale != 0.f || g.sm.any ||
+      g.window > 0 || g.verdict || g.live_tiles || g.live_t || p.force_kernel == MI355_SDPA_KERNEL_GENERIC)
+    return 1;
+  if (!bwd_dq_w32_fits(g, p.q.size[3] <= 64 ? 64 : 128)) return 1;
+  const int64_t blocks = (int64_t)g.B * g.Hq * ((g.L + 255) / 256);
+  const int nt = (g.S + 31) / 32;
+  if (blocks >= 128 || nt < 64) return 1;
+  const int want = (int)std::min<int64_t>(std::min<int64_t>((512 + blocks - 1) / blocks, nt / 32), 64);
+  if (want <= 1) return 1;
+  *split_tiles = (nt + want - 1) / want;
+  return (nt + *split_tiles - 1) / *split_tiles;
+}
+static size_t dq_part_bytes(const BwdM& g, int n_split) {
+  return n_split > 1 ? (size_t)n_split * g.B * g.Hq * g.L * g.d_real * sizeof(float) : 0;
 }
 size_t bwd_mfma_workspace(const mi355_sdpa_bwd_params& p) {
   if (p.dtype != MI355_SDPA_BF16 && p.dtype != MI355_SDPA_F16) return row_terms_bytes(p);
   BwdM g;
   fill(g, p);
-  return row_terms_bytes(p) + part_rows_bytes(g, parts_of(g, p));
+  int split_tiles;
+  return row_terms_bytes(p) + part_rows_bytes(g, parts_of(g, p)) + dq_part_bytes(g, dq_splits(g, p, &split_tiles));
 }
 
 int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
@@ -671,6 +694,13 @@ int launch_bwd_mfma(const mi355_sdpa_bwd_params& p, hipStream_t s) {
     g.parts = parts;
     g.part_dk = (float*)((char*)p.workspace + row_terms_bytes(p));
     g.part_dv = g.part_dk + (size_t)parts * g.B * g.Hkv * g.S * g.d_real;
+  }
+  {
+    int split_tiles;
+    const int n_split = dq_splits(g, p, &split_tiles);
+    const size_t at = row_terms_bytes(p) + part_rows_bytes(g, parts);
+    if (n_split > 1 && p.workspace_bytes >= at + dq_part_bytes(g, n_split))
+      g.dq_split_tiles = split_tiles, g.dq_n_split = n_split, g.part_dq = (float*)((char*)p.workspace + at);
   }
   if (key_order_bytes(p) && p.workspace_bytes >= row_terms_bytes(p)) g.kt_order = (int32_t*)((char*)p.workspace + row_stats_bytes(p));
   const int D = p.q.size[3] <= 64 ? 64 : 128;  // the kernels' width
